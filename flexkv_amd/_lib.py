@@ -1,0 +1,185 @@
+"""ctypes binding of libfkv_hip.so (the C ABI in include/fkv_transfer.h).
+
+The library must have been built (``make -C flexkv_amd/csrc`` or
+``python -c "import __graft_entry__ as g; g.build()"``).  There is no fallback:
+if the shared object is missing or cannot be loaded the import of the package's
+operator module fails.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import (POINTER, Structure, c_char_p, c_double, c_float, c_int32, c_int64,
+                    c_size_t, c_uint64, c_void_p)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libfkv_hip.so")
+
+FKV_OK = 0
+FKV_ERR_INVALID_ARG = 1
+FKV_ERR_RUNTIME = 2
+FKV_ERR_UNSUPPORTED = 3
+
+FKV_PATH_KERNEL = 100
+CE_PATH_NAMES = {-1: "PER_BLOCK", 0: "CONTIG_DIRECT", 1: "SEGMENT_DIRECT",
+                 2: "SEGMENT_SCATTER", 3: "GATHER_SCATTER", 4: "GATHER_DIRECT",
+                 FKV_PATH_KERNEL: "KERNEL"}
+
+NOTIFY_HOSTFUNC = 0
+NOTIFY_POLLING = 1
+
+
+class CEConfig(Structure):
+    _fields_ = [("segment_threshold", c_int64), ("path_opt_enabled", c_int32),
+                ("force_path", c_int32), ("enable_memcpy2d", c_int32),
+                ("is_blockfirst", c_int32), ("num_kv_heads", c_int32),
+                ("gather_threads", c_int32), ("gather_nt", c_int32), ("reserved", c_int32)]
+
+
+class TransferDesc(Structure):
+    _fields_ = [("backend", c_int32), ("num_layers_total", c_int32),
+                ("gpu_tensor_ptrs", c_void_p), ("num_gpu_tensor_ptrs", c_int32),
+                ("device", c_int32),
+                ("gpu_kv_stride", c_int64), ("gpu_block_stride", c_int64),
+                ("gpu_layer_stride", c_int64), ("gpu_startoff_inside_chunks", c_int64),
+                ("cpu_ptr", c_void_p),
+                ("cpu_kv_stride", c_int64), ("cpu_layer_stride", c_int64),
+                ("cpu_block_stride", c_int64), ("cpu_startoff_inside_chunks", c_int64),
+                ("chunk_size", c_int64),
+                ("start_layer_id", c_int32), ("num_layers", c_int32),
+                ("kv_dim", c_int32), ("num_blocks", c_int32),
+                ("gpu_block_ids", c_void_p), ("cpu_block_ids", c_void_p),
+                ("is_host_to_device", c_int32), ("use_ce_transfer", c_int32),
+                ("transfer_num_cta", c_int32), ("sync", c_int32),
+                ("enable_trace", c_int32), ("reserved", c_int32),
+                ("ce", CEConfig)]
+
+
+class CEAnalysis(Structure):
+    _fields_ = [("gpu_log_contig", c_int32), ("cpu_log_contig", c_int32),
+                ("cpu_phys_contig", c_int32), ("gpu_phys_contig", c_int32),
+                ("num_segments", c_int32), ("reserved", c_int32)]
+
+
+class CESegment(Structure):
+    _fields_ = [("start_k", c_int32), ("nr_blocks", c_int32)]
+
+
+class TPRankPlan(Structure):
+    _fields_ = [("active", c_int32), ("start_layer", c_int32), ("num_layers", c_int32),
+                ("reserved", c_int32), ("cpu_startoff", c_int64), ("gpu_startoff", c_int64),
+                ("chunk_size", c_int64)]
+
+
+class TPGroupParams(Structure):
+    _fields_ = [("num_gpus", c_int32), ("num_tensors_per_gpu", c_int32),
+                ("gpu_block_ptrs_flat", c_void_p), ("cpu_blocks_ptr", c_void_p),
+                ("num_layers", c_int32), ("reserved", c_int32),
+                ("gpu_kv_strides", c_void_p), ("gpu_block_strides", c_void_p),
+                ("gpu_layer_strides", c_void_p), ("gpu_chunk_sizes", c_void_p),
+                ("gpu_device_ids", c_void_p), ("ce", CEConfig)]
+
+
+class LayerwiseParams(Structure):
+    _fields_ = [("num_gpus", c_int32), ("num_tensors_per_gpu", c_int32),
+                ("gpu_block_ptrs_flat", c_void_p), ("cpu_blocks_ptr", c_void_p),
+                ("num_layers", c_int32), ("tp_size", c_int32),
+                ("gpu_kv_strides", c_void_p), ("gpu_block_strides", c_void_p),
+                ("gpu_layer_strides", c_void_p), ("gpu_chunk_sizes", c_void_p),
+                ("gpu_device_ids", c_void_p), ("layer_eventfds", c_void_p),
+                ("num_layer_eventfds", c_int32), ("reserved", c_int32), ("ce", CEConfig)]
+
+
+class Stats(Structure):
+    _fields_ = [("calls", c_uint64), ("bytes_h2d", c_uint64), ("bytes_d2h", c_uint64),
+                ("kernel_launches", c_uint64), ("dma_copies", c_uint64),
+                ("staging_bytes_device", c_uint64), ("staging_bytes_host", c_uint64),
+                ("reserved", c_uint64)]
+
+
+# name -> (restype, argtypes); the complete export list of include/fkv_transfer.h
+SIGNATURES = {
+    "fkv_abi_version": (c_int32, []),
+    "fkv_last_error": (c_char_p, []),
+    "fkv_last_path": (c_int32, []),
+    "fkv_ce_config_default": (None, [POINTER(CEConfig)]),
+    "fkv_transfer_kv_blocks": (c_int32, [POINTER(TransferDesc), c_void_p]),
+    "fkv_ce_analyze": (c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int64,
+                                 POINTER(CEAnalysis), c_void_p, c_int32]),
+    "fkv_ce_choose_path": (c_int32, [POINTER(CEAnalysis), POINTER(CEConfig), c_int64,
+                                     c_int32, c_int32]),
+    "fkv_tp_rank_plan_compute": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_char_p,
+                                           c_int32, c_int32, c_int32, c_int32, c_int32,
+                                           c_int64, c_int64, c_int64, POINTER(TPRankPlan)]),
+    "fkv_tp_group_create": (c_int32, [POINTER(TPGroupParams), POINTER(c_void_p)]),
+    "fkv_tp_group_update_gpu_block_ptrs": (c_int32, [c_void_p, c_void_p, c_int64]),
+    "fkv_tp_group_transfer": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32,
+                                        c_int64, c_int64, c_int64, c_int64,
+                                        c_int32, c_int32, c_int32, c_int32, c_int32,
+                                        c_int32, c_int32, c_char_p, c_int32]),
+    "fkv_tp_group_destroy": (None, [c_void_p]),
+    "fkv_layerwise_create": (c_int32, [POINTER(LayerwiseParams), POINTER(c_void_p)]),
+    "fkv_layerwise_transfer": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32,
+                                         c_int64, c_int64, c_int64, c_int64,
+                                         c_int32, c_int32, c_int32, c_int32, c_int32,
+                                         c_int32, c_int32, c_char_p, c_int32, c_int32]),
+    "fkv_layerwise_wait_layer": (c_int32, [c_void_p, c_int32, c_int32, c_void_p]),
+    "fkv_layerwise_synchronize": (c_int32, [c_void_p]),
+    "fkv_layerwise_batch_times_ms": (c_int32, [c_void_p, POINTER(c_float), c_int32,
+                                               POINTER(c_int32)]),
+    "fkv_layerwise_destroy": (None, [c_void_p]),
+    "fkv_host_alloc": (c_int32, [c_size_t, POINTER(c_void_p)]),
+    "fkv_host_free": (c_int32, [c_void_p]),
+    "fkv_host_register": (c_int32, [c_void_p, c_size_t, c_size_t]),
+    "fkv_host_unregister": (c_int32, [c_void_p, c_size_t, c_size_t]),
+    "fkv_host_register_plan": (c_int64, [c_size_t, c_size_t, c_void_p, c_void_p, c_int64]),
+    "fkv_host_chunk_bytes_from_gb": (c_size_t, [c_double]),
+    "fkv_get_stats": (None, [POINTER(Stats)]),
+    "fkv_reset_stats": (None, []),
+    "fkv_measure_link_peak": (c_int32, [c_int32, c_size_t, c_int32, c_int32,
+                                        POINTER(c_double), POINTER(c_double)]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load libfkv_hip.so and attach the prototypes.  Raises if it is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} not found: build the HIP library first "
+            "(make -C flexkv_amd/csrc); there is no CPU fallback for the transfer path")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    if lib.fkv_abi_version() != 1:
+        raise ImportError(f"{LIB_PATH}: ABI version {lib.fkv_abi_version()} != 1")
+    _lib = lib
+    return lib
+
+
+def last_error() -> str:
+    return (load().fkv_last_error() or b"").decode(errors="replace")
+
+
+def check(status: int) -> None:
+    """Map a status code to the exception class the reference's pybind module
+    would have raised (std::invalid_argument -> ValueError, everything else ->
+    RuntimeError)."""
+    if status == FKV_OK:
+        return
+    msg = last_error()
+    if status == FKV_ERR_INVALID_ARG:
+        raise ValueError(msg)
+    raise RuntimeError(msg)
+
+
+def default_ce_config() -> CEConfig:
+    cfg = CEConfig()
+    load().fkv_ce_config_default(ctypes.byref(cfg))
+    return cfg

@@ -1,0 +1,388 @@
+"""Operator module with the hot-path names of FlexKV's ``flexkv.c_ext``.
+
+``transfer_kv_blocks``, ``TPTransferThreadGroup`` and ``LayerwiseTransferGroup``
+take the same positional order, keyword names, defaults and error behaviour as
+the pybind definitions in the reference (``csrc/bindings.cpp:439-459``,
+``:761-830``, ``:471-545`` and ``:657-691``), so FlexKV's transfer workers
+(``flexkv/transfer/worker.py:1002-1059, 1218-1236, 1484-1499``;
+``flexkv/transfer/layerwise.py:647-664, 952-1001``) can import this module in
+place of ``flexkv.c_ext`` for the GPU<->CPU path.
+
+Everything here is a thin adapter: it pulls raw addresses and sizes out of
+torch tensors, takes the current HIP stream from torch, and calls the C ABI of
+``libfkv_hip.so``.  No copy is ever done in Python and there is no fallback
+when the library is missing.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from . import _lib
+from ._lib import (CEConfig, LayerwiseParams, TPGroupParams, TransferDesc, check,
+                   NOTIFY_HOSTFUNC, NOTIFY_POLLING)
+
+_L = _lib.load()
+
+__all__ = ["transfer_kv_blocks", "TPTransferThreadGroup", "LayerwiseTransferGroup",
+           "last_transfer_path", "get_stats", "reset_stats"]
+
+
+def _ids(t: torch.Tensor, name: str) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if t.device.type != "cpu":
+        raise ValueError(f"{name} must live in host memory")
+    if t.dtype != torch.int64:
+        raise TypeError(f"{name} must be int64, got {t.dtype}")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _current_stream_handle() -> int:
+    return int(torch.cuda.current_stream().cuda_stream)
+
+
+def _ce_config(segment_threshold, path_opt, force_path, enable_memcpy2d, is_blockfirst,
+               num_kv_heads, gather_threads, gather_nt) -> CEConfig:
+    cfg = CEConfig()
+    cfg.segment_threshold = int(segment_threshold)
+    cfg.path_opt_enabled = int(bool(path_opt))
+    cfg.force_path = int(force_path)
+    cfg.enable_memcpy2d = int(bool(enable_memcpy2d))
+    cfg.is_blockfirst = int(bool(is_blockfirst))
+    cfg.num_kv_heads = int(num_kv_heads)
+    cfg.gather_threads = int(gather_threads)
+    cfg.gather_nt = int(bool(gather_nt))
+    return cfg
+
+
+def transfer_kv_blocks(
+        gpu_block_id_tensor: torch.Tensor, gpu_tensor_ptrs_tensor: torch.Tensor,
+        gpu_kv_stride_in_bytes: int, gpu_block_stride_in_bytes: int,
+        gpu_layer_stride_in_bytes: int, cpu_block_id_tensor: torch.Tensor,
+        cpu_tensor: torch.Tensor, cpu_kv_stride_in_bytes: int,
+        cpu_layer_stride_in_bytes: int, cpu_block_stride_in_bytes: int,
+        chunk_size_in_bytes: int, start_layer_id: int, num_layers: int,
+        transfer_num_cta: int = 4, is_host_to_device: bool = True,
+        use_ce_transfer: bool = False, kv_dim: int = 2, num_kv_heads: int = 1,
+        gpu_block_type: int = 0, sync: bool = True, ce_path_opt: bool = False,
+        ce_segment_threshold: int = 8, ce_force_path: int = -1,
+        ce_enable_memcpy2d: bool = False, is_blockfirst: bool = False,
+        ce_gather_threads: int = 4, ce_gather_nt: bool = True,
+        enable_transfer_trace: bool = False) -> None:
+    """Transfer multi-layer KV-cache between CPU and GPU on the current stream
+    (``csrc/bindings.cpp:54-151``).
+
+    ``gpu_tensor_ptrs_tensor`` is an int64 host tensor of device addresses: L
+    entries for vLLM (``gpu_block_type`` 0), one for TRT-LLM (1), K₀..K_{L-1},
+    V₀..V_{L-1} for SGLang (2).
+    """
+    gpu_ids = _ids(gpu_block_id_tensor, "gpu_block_id_tensor")
+    cpu_ids = _ids(cpu_block_id_tensor, "cpu_block_id_tensor")
+    if gpu_ids.numel() != cpu_ids.numel():
+        raise ValueError("gpu_block_id_tensor and cpu_block_id_tensor differ in length")
+    ptrs = _ids(gpu_tensor_ptrs_tensor, "gpu_tensor_ptrs_tensor")
+    if cpu_tensor.device.type != "cpu":
+        raise ValueError("cpu_tensor must live in host memory")
+
+    d = TransferDesc()
+    d.backend = int(gpu_block_type)
+    # The reference builds its GTensorHandler with the num_layers of the call
+    # (csrc/bindings.cpp:108-111), which indexes SGLang's K-then-V pointer table
+    # correctly only for whole-model calls; take the true layer count from the
+    # table itself so partial-layer calls address V tensors correctly too.
+    d.num_layers_total = ptrs.numel() // 2 if int(gpu_block_type) == 2 else int(num_layers)
+    d.gpu_tensor_ptrs = ptrs.data_ptr()
+    d.num_gpu_tensor_ptrs = ptrs.numel()
+    d.device = -1
+    d.gpu_kv_stride = int(gpu_kv_stride_in_bytes)
+    d.gpu_block_stride = int(gpu_block_stride_in_bytes)
+    d.gpu_layer_stride = int(gpu_layer_stride_in_bytes)
+    d.gpu_startoff_inside_chunks = 0
+    d.cpu_ptr = cpu_tensor.data_ptr()
+    d.cpu_kv_stride = int(cpu_kv_stride_in_bytes)
+    d.cpu_layer_stride = int(cpu_layer_stride_in_bytes)
+    d.cpu_block_stride = int(cpu_block_stride_in_bytes)
+    d.cpu_startoff_inside_chunks = 0
+    d.chunk_size = int(chunk_size_in_bytes)
+    d.start_layer_id = int(start_layer_id)
+    d.num_layers = int(num_layers)
+    d.kv_dim = int(kv_dim)
+    d.num_blocks = gpu_ids.numel()
+    d.gpu_block_ids = gpu_ids.data_ptr()
+    d.cpu_block_ids = cpu_ids.data_ptr()
+    d.is_host_to_device = int(bool(is_host_to_device))
+    d.use_ce_transfer = int(bool(use_ce_transfer))
+    d.transfer_num_cta = int(transfer_num_cta)
+    d.sync = int(bool(sync))
+    d.enable_trace = int(bool(enable_transfer_trace))
+    d.ce = _ce_config(ce_segment_threshold, ce_path_opt, ce_force_path, ce_enable_memcpy2d,
+                      is_blockfirst, num_kv_heads, ce_gather_threads, ce_gather_nt)
+    check(_L.fkv_transfer_kv_blocks(ctypes.byref(d), _current_stream_handle()))
+
+
+def last_transfer_path() -> str:
+    """Name of the path the last transfer issued by this thread took: KERNEL or
+    one of the copy-engine strategies."""
+    return _lib.CE_PATH_NAMES.get(int(_L.fkv_last_path()), "UNKNOWN")
+
+
+def get_stats() -> Dict[str, int]:
+    s = _lib.Stats()
+    _L.fkv_get_stats(ctypes.byref(s))
+    return {name: int(getattr(s, name)) for name, _ in s._fields_ if name != "reserved"}
+
+
+def reset_stats() -> None:
+    _L.fkv_reset_stats()
+
+
+def _i64_array(values: Sequence[int], name: str, expect: Optional[int] = None) -> np.ndarray:
+    arr = np.ascontiguousarray(np.asarray(list(values), dtype=np.int64))
+    if expect is not None and arr.size != expect:
+        raise ValueError(f"{name} must have {expect} entries, got {arr.size}")
+    return arr
+
+
+class TPTransferThreadGroup:
+    """One transfer thread + stream per GPU of a tensor-parallel group
+    (``csrc/bindings.cpp:761-830``, ``csrc/tp_transfer_thread_group.cpp``)."""
+
+    def __init__(self, num_gpus: int, gpu_block_ptrs_flat: Sequence[int],
+                 num_tensors_per_gpu: int, cpu_blocks_ptr: int, num_layers: int,
+                 gpu_kv_strides_in_bytes: Sequence[int],
+                 gpu_block_strides_in_bytes: Sequence[int],
+                 gpu_layer_strides_in_bytes: Sequence[int],
+                 gpu_chunk_sizes_in_bytes: Sequence[int],
+                 gpu_device_ids: Sequence[int],
+                 enable_nvcomp: bool = False, nvcomp_batch_size: int = 0,
+                 nvcomp_data_type: int = 0, ce_segment_threshold: int = 8,
+                 ce_path_opt: bool = True, ce_force_path: int = -1,
+                 ce_enable_memcpy2d: bool = False, is_blockfirst: bool = False,
+                 num_kv_heads: int = 1, ce_gather_threads: int = 4,
+                 ce_gather_nt: bool = True) -> None:
+        self._h = ctypes.c_void_p()
+        if enable_nvcomp:
+            raise RuntimeError("nvcomp compressed transfer is not part of this library")
+        ptrs = np.ascontiguousarray(np.asarray(list(gpu_block_ptrs_flat), dtype=np.uint64))
+        if ptrs.size != num_gpus * num_tensors_per_gpu:
+            raise ValueError("gpu_block_ptrs_flat must hold num_gpus * num_tensors_per_gpu pointers")
+        kvs = _i64_array(gpu_kv_strides_in_bytes, "gpu_kv_strides_in_bytes", num_gpus)
+        bs = _i64_array(gpu_block_strides_in_bytes, "gpu_block_strides_in_bytes", num_gpus)
+        ls = _i64_array(gpu_layer_strides_in_bytes, "gpu_layer_strides_in_bytes", num_gpus)
+        cs = _i64_array(gpu_chunk_sizes_in_bytes, "gpu_chunk_sizes_in_bytes", num_gpus)
+        dev = _i64_array(gpu_device_ids, "gpu_device_ids", num_gpus)
+        p = TPGroupParams()
+        p.num_gpus = int(num_gpus)
+        p.num_tensors_per_gpu = int(num_tensors_per_gpu)
+        p.gpu_block_ptrs_flat = ptrs.ctypes.data
+        p.cpu_blocks_ptr = int(cpu_blocks_ptr)
+        p.num_layers = int(num_layers)
+        p.gpu_kv_strides = kvs.ctypes.data
+        p.gpu_block_strides = bs.ctypes.data
+        p.gpu_layer_strides = ls.ctypes.data
+        p.gpu_chunk_sizes = cs.ctypes.data
+        p.gpu_device_ids = dev.ctypes.data
+        p.ce = _ce_config(ce_segment_threshold, ce_path_opt, ce_force_path, ce_enable_memcpy2d,
+                          is_blockfirst, num_kv_heads, ce_gather_threads, ce_gather_nt)
+        self._num_ptrs = int(ptrs.size)
+        check(_L.fkv_tp_group_create(ctypes.byref(p), ctypes.byref(self._h)))
+
+    def update_gpu_block_ptrs(self, gpu_block_ptrs_flat: Sequence[int]) -> None:
+        ptrs = np.ascontiguousarray(np.asarray(list(gpu_block_ptrs_flat), dtype=np.uint64))
+        check(_L.fkv_tp_group_update_gpu_block_ptrs(self._h, ptrs.ctypes.data, int(ptrs.size)))
+
+    def tp_group_transfer(self, gpu_block_id_tensor: torch.Tensor,
+                          cpu_block_id_tensor: torch.Tensor, cpu_kv_stride_in_bytes: int,
+                          cpu_layer_stride_in_bytes: int, cpu_block_stride_in_bytes: int,
+                          cpu_tp_stride_in_bytes: int, transfer_num_cta: int,
+                          is_host_to_device: bool, use_ce_transfer: bool, layer_id: int,
+                          layer_granularity: int, kv_dim: int, num_kv_heads: int,
+                          kv_shared_across_ranks_mode: str = "sharded",
+                          designated_rank: int = 0) -> None:
+        gpu_ids = _ids(gpu_block_id_tensor, "gpu_block_id_tensor")
+        cpu_ids = _ids(cpu_block_id_tensor, "cpu_block_id_tensor")
+        if gpu_ids.numel() != cpu_ids.numel():
+            raise ValueError("gpu_block_id_tensor and cpu_block_id_tensor differ in length")
+        check(_L.fkv_tp_group_transfer(
+            self._h, gpu_ids.data_ptr(), cpu_ids.data_ptr(), gpu_ids.numel(),
+            int(cpu_kv_stride_in_bytes), int(cpu_layer_stride_in_bytes),
+            int(cpu_block_stride_in_bytes), int(cpu_tp_stride_in_bytes),
+            int(transfer_num_cta), int(bool(is_host_to_device)), int(bool(use_ce_transfer)),
+            int(layer_id), int(layer_granularity), int(kv_dim), int(num_kv_heads),
+            str(kv_shared_across_ranks_mode).encode(), int(designated_rank)))
+
+    def close(self) -> None:
+        if getattr(self, "_h", None) is not None and self._h.value:
+            _L.fkv_tp_group_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self) -> None:
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+_NOTIFY = {"hostfunc": NOTIFY_HOSTFUNC, "polling": NOTIFY_POLLING}
+
+
+def _numel(t) -> int:
+    return int(t.numel()) if isinstance(t, torch.Tensor) else len(t)
+
+
+class LayerwiseTransferGroup:
+    """Per-layer host->GPU restore with completion signalling
+    (``csrc/bindings.cpp:471-545, 657-691``, ``csrc/layerwise.cpp``).
+
+    Only the single-group, main-KV form is provided.  SSD pre-load, SWA
+    sidecars and the multi-group constructor raise ``RuntimeError``.
+    """
+
+    def __init__(self, num_gpus: int = None, gpu_blocks: List[List[torch.Tensor]] = None,
+                 cpu_blocks: torch.Tensor = None, ssd_files: dict = None,
+                 num_layers: int = None, gpu_kv_strides_tensor: torch.Tensor = None,
+                 gpu_block_strides_tensor: torch.Tensor = None,
+                 gpu_layer_strides_tensor: torch.Tensor = None,
+                 gpu_chunk_sizes_tensor: torch.Tensor = None, iouring_entries: int = 0,
+                 iouring_flags: int = 0, layer_eventfds_tensor: torch.Tensor = None,
+                 tp_size: int = 1, has_swa: bool = False, swa_gpu_blocks=(),
+                 swa_cpu_blocks=None, swa_ssd_files=None,
+                 swa_gpu_kv_strides_tensor=None, swa_gpu_block_strides_tensor=None,
+                 swa_gpu_layer_strides_tensor=None, swa_gpu_chunk_sizes_tensor=None,
+                 ce_segment_threshold: int = 8, ce_path_opt: bool = True,
+                 ce_force_path: int = -1, ce_enable_memcpy2d: bool = False,
+                 is_blockfirst: bool = False, num_kv_heads: int = 1,
+                 ce_gather_threads: int = 4, ce_gather_nt: bool = True,
+                 ssd_io_opt: bool = True, **multi_group_kwargs) -> None:
+        self._h = ctypes.c_void_p()
+        if multi_group_kwargs:
+            raise RuntimeError(
+                "the multi-group LayerwiseTransferGroup constructor "
+                f"({sorted(multi_group_kwargs)[0]}, ...) is not part of this library")
+        if ssd_files:
+            raise RuntimeError("SSD->CPU pre-load is not part of this library (ssd_files must be empty)")
+        if has_swa or len(swa_gpu_blocks or ()) > 0:
+            raise RuntimeError("SWA sidecar transfer is not part of this library")
+        if gpu_blocks is None or len(gpu_blocks) != num_gpus:
+            raise ValueError("gpu_blocks must hold one tensor list per GPU")
+        per_gpu = len(gpu_blocks[0])
+        ptrs, devs = [], []
+        for g, tensors in enumerate(gpu_blocks):
+            if len(tensors) != per_gpu:
+                raise ValueError("every GPU must bring the same number of KV tensors")
+            for t in tensors:
+                if t.device.type != "cuda":
+                    raise ValueError("gpu_blocks must be device tensors")
+                ptrs.append(t.data_ptr())
+            devs.append(tensors[0].device.index)
+        ptr_arr = np.ascontiguousarray(np.asarray(ptrs, dtype=np.uint64))
+        kvs = _i64_array(gpu_kv_strides_tensor.tolist(), "gpu_kv_strides_tensor", num_gpus)
+        bs = _i64_array(gpu_block_strides_tensor.tolist(), "gpu_block_strides_tensor", num_gpus)
+        ls = _i64_array(gpu_layer_strides_tensor.tolist(), "gpu_layer_strides_tensor", num_gpus)
+        cs = _i64_array(gpu_chunk_sizes_tensor.tolist(), "gpu_chunk_sizes_tensor", num_gpus)
+        dev = _i64_array(devs, "gpu_device_ids", num_gpus)
+        fds = None
+        if layer_eventfds_tensor is not None and layer_eventfds_tensor.numel() > 0:
+            if layer_eventfds_tensor.dtype != torch.int32:
+                raise TypeError("layer_eventfds_tensor must be int32")
+            fds = np.ascontiguousarray(layer_eventfds_tensor.cpu().numpy().reshape(-1))
+        p = LayerwiseParams()
+        p.num_gpus = int(num_gpus)
+        p.num_tensors_per_gpu = per_gpu
+        p.gpu_block_ptrs_flat = ptr_arr.ctypes.data
+        p.cpu_blocks_ptr = cpu_blocks.data_ptr()
+        p.num_layers = int(num_layers)
+        p.tp_size = int(tp_size)
+        p.gpu_kv_strides = kvs.ctypes.data
+        p.gpu_block_strides = bs.ctypes.data
+        p.gpu_layer_strides = ls.ctypes.data
+        p.gpu_chunk_sizes = cs.ctypes.data
+        p.gpu_device_ids = dev.ctypes.data
+        p.layer_eventfds = fds.ctypes.data if fds is not None else None
+        p.num_layer_eventfds = int(fds.size) if fds is not None else 0
+        p.ce = _ce_config(ce_segment_threshold, ce_path_opt, ce_force_path, ce_enable_memcpy2d,
+                          is_blockfirst, num_kv_heads, ce_gather_threads, ce_gather_nt)
+        # the library keeps raw addresses only: hold the tensors for its lifetime
+        self._keepalive = (gpu_blocks, cpu_blocks)
+        self._num_layers = int(num_layers)
+        check(_L.fkv_layerwise_create(ctypes.byref(p), ctypes.byref(self._h)))
+
+    def init_swa_multi_group(self, *args, **kwargs) -> None:
+        raise RuntimeError("SWA sidecar transfer is not part of this library")
+
+    def layerwise_transfer_multi_group(self, *args, **kwargs) -> None:
+        # csrc/layerwise.cpp:1335-1339
+        raise RuntimeError(
+            "[LayerwiseTransferGroup] layerwise_transfer_multi_group() invoked on a "
+            "single-group instance; use layerwise_transfer() instead.")
+
+    def layerwise_transfer(
+            self, ssd_block_ids, cpu_block_ids_d2h, ssd_layer_stride_in_bytes: int,
+            ssd_kv_stride_in_bytes: int, num_blocks_per_file: int, round_robin: int,
+            num_threads_per_device: int, gpu_block_id_tensor: torch.Tensor,
+            cpu_block_id_tensor: torch.Tensor, cpu_kv_stride_in_bytes: int,
+            cpu_layer_stride_in_bytes: int, cpu_block_stride_in_bytes: int,
+            cpu_chunk_size_in_bytes: int, h2d_cpu_kv_stride_in_bytes: int,
+            h2d_cpu_layer_stride_in_bytes: int, cpu_tp_stride_in_bytes: int,
+            transfer_cta_num: int, use_ce_transfer: bool, num_layers: int,
+            layer_granularity: int, kv_dim: int, num_kv_heads: int, counter_id: int = 0,
+            swa_h2d_src=None, swa_h2d_dst=None, swa_disk2h_src=None, swa_disk2h_dst=None,
+            swa_cpu_kv_stride_in_bytes: int = 0, swa_cpu_layer_stride_in_bytes: int = 0,
+            swa_cpu_block_stride_in_bytes: int = 0, swa_cpu_chunk_size_in_bytes: int = 0,
+            swa_h2d_cpu_kv_stride_in_bytes: int = 0,
+            swa_h2d_cpu_layer_stride_in_bytes: int = 0, swa_cpu_tp_stride_in_bytes: int = 0,
+            swa_ssd_layer_stride_in_bytes: int = 0, swa_ssd_kv_stride_in_bytes: int = 0,
+            swa_num_blocks_per_file: int = 0, kv_shared_across_ranks_mode: str = "sharded",
+            notify_mode: str = "hostfunc", enable_trace: bool = False) -> None:
+        if ssd_block_ids is not None and _numel(ssd_block_ids) > 0:
+            raise RuntimeError("SSD->CPU pre-load is not part of this library")
+        for name, t in (("swa_h2d_src", swa_h2d_src), ("swa_h2d_dst", swa_h2d_dst),
+                        ("swa_disk2h_src", swa_disk2h_src), ("swa_disk2h_dst", swa_disk2h_dst)):
+            if t is not None and _numel(t) > 0:
+                raise RuntimeError(f"SWA sidecar transfer is not part of this library ({name})")
+        gpu_ids = _ids(gpu_block_id_tensor, "gpu_block_id_tensor")
+        cpu_ids = _ids(cpu_block_id_tensor, "cpu_block_id_tensor")
+        if gpu_ids.numel() != cpu_ids.numel():
+            raise ValueError("gpu_block_id_tensor and cpu_block_id_tensor differ in length")
+        # any string but "polling" selects the host-function mode, csrc/layerwise.cpp:987-988
+        mode = NOTIFY_POLLING if notify_mode == "polling" else NOTIFY_HOSTFUNC
+        check(_L.fkv_layerwise_transfer(
+            self._h, gpu_ids.data_ptr(), cpu_ids.data_ptr(), gpu_ids.numel(),
+            int(cpu_block_stride_in_bytes), int(h2d_cpu_kv_stride_in_bytes),
+            int(h2d_cpu_layer_stride_in_bytes), int(cpu_tp_stride_in_bytes),
+            int(transfer_cta_num), int(bool(use_ce_transfer)), int(num_layers),
+            int(layer_granularity), int(kv_dim), int(num_kv_heads), int(counter_id),
+            str(kv_shared_across_ranks_mode).encode(), mode, int(bool(enable_trace))))
+
+    # ---- additions for consumers in the same process -------------------------
+    def wait_layer(self, layer: int, stream: Optional["torch.cuda.Stream"] = None,
+                   gpu_index: int = 0) -> None:
+        """Make ``stream`` (default: torch's current stream) wait until ``layer``
+        of the last ``layerwise_transfer`` has landed."""
+        handle = int((stream or torch.cuda.current_stream()).cuda_stream)
+        check(_L.fkv_layerwise_wait_layer(self._h, int(gpu_index), int(layer), handle))
+
+    def synchronize(self) -> None:
+        check(_L.fkv_layerwise_synchronize(self._h))
+
+    def batch_times_ms(self) -> List[float]:
+        n = ctypes.c_int32(0)
+        cap = max(1, self._num_layers)
+        buf = (ctypes.c_float * cap)()
+        check(_L.fkv_layerwise_batch_times_ms(self._h, buf, cap, ctypes.byref(n)))
+        return [float(buf[i]) for i in range(min(cap, n.value))]
+
+    def close(self) -> None:
+        if getattr(self, "_h", None) is not None and self._h.value:
+            _L.fkv_layerwise_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self) -> None:
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,669 @@
+// Copy-engine path: block-id analysis, strategy choice and the strategies.
+//
+// Replaces csrc/ce_transfer.cu of the reference.  The DMA work is
+// hipMemcpyAsync / hipMemcpy2DAsync on the caller's stream; the device-side row
+// gather/scatter that the reference delegates to ATen index_select /
+// index_copy_ is the library's own copy kernel (fkv_kernels.hip) run with a
+// full-chip grid, because that pass is HBM-bound, not link-bound.
+//
+// Differences from the reference that do not change which bytes move:
+//   * the direct strategies (PER_BLOCK, CONTIG_DIRECT, SEGMENT_DIRECT,
+//     GATHER_DIRECT, and the 2-D copy branches) never block the host: they
+//     only enqueue work, so `sync == 0` callers (layerwise restore) stay
+//     asynchronous.  The staging strategies still run host copies and therefore
+//     return with their stream drained, as in the reference.
+//   * GATHER_DIRECT bounds its device staging buffer and walks the block list
+//     in groups instead of staging the whole transfer at once.
+//   * host->GPU staging is double-buffered like GPU->host.
+#include "fkv_host_copy.h"
+#include "fkv_internal.h"
+
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <unordered_map>
+
+namespace fkv {
+namespace {
+
+struct Analysis {
+  fkv_ce_analysis a{};
+  std::vector<fkv_ce_segment> segs;
+};
+
+void analyze(const int64_t *gpu_ids, const int64_t *cpu_ids, int n, int64_t cpu_block_stride,
+             int64_t chunk, int64_t gpu_block_stride, Analysis &out) {
+  out.a.gpu_log_contig = 1;
+  out.a.cpu_log_contig = 1;
+  out.a.cpu_phys_contig = cpu_block_stride == chunk;
+  out.a.gpu_phys_contig = gpu_block_stride == 0 || gpu_block_stride == chunk;
+  out.a.num_segments = 0;
+  out.a.reserved = 0;
+  out.segs.clear();
+  if (n <= 0)
+    return;
+  int run_start = 0;
+  for (int k = 1; k < n; ++k) {
+    const bool g_next = gpu_ids[k] == gpu_ids[k - 1] + 1;
+    const bool c_next = cpu_ids[k] == cpu_ids[k - 1] + 1;
+    out.a.gpu_log_contig &= (int)g_next;
+    out.a.cpu_log_contig &= (int)c_next;
+    if (!(g_next && c_next)) {
+      out.segs.push_back({run_start, k - run_start});
+      run_start = k;
+    }
+  }
+  out.segs.push_back({run_start, n - run_start});
+  out.a.num_segments = (int)out.segs.size();
+}
+
+int choose(const fkv_ce_analysis &a, const fkv_ce_config &cfg, int64_t chunk, bool h2d,
+           bool full_block) {
+  // strategies that view a chunk as int64 rows in the reference need chunk % 8 == 0
+  const bool odd_chunk = chunk > 0 && (chunk % 8) != 0;
+  const int many = odd_chunk ? FKV_CE_SEGMENT_SCATTER : FKV_CE_GATHER_SCATTER;
+  if (cfg.is_blockfirst && !a.cpu_phys_contig && a.gpu_phys_contig) {
+    if (!h2d && cfg.num_kv_heads == 1) {
+      if (a.num_segments > cfg.segment_threshold)
+        return many;
+      if (!full_block)
+        return FKV_CE_SEGMENT_SCATTER;
+    }
+    return FKV_CE_GATHER_DIRECT;
+  }
+  if (a.gpu_log_contig && a.cpu_log_contig && a.cpu_phys_contig && a.gpu_phys_contig)
+    return FKV_CE_CONTIG_DIRECT;
+  if (!a.gpu_phys_contig)
+    return FKV_CE_GATHER_SCATTER;
+  if (a.num_segments <= cfg.segment_threshold)
+    return a.cpu_phys_contig ? FKV_CE_SEGMENT_DIRECT : FKV_CE_SEGMENT_SCATTER;
+  return many;
+}
+
+// ---- cached staging memory, one set per (calling thread, device) ----------
+struct DeviceStage {
+  uint8_t *buf = nullptr;
+  size_t cap = 0;
+  hipEvent_t last_use = nullptr; // recorded after the last enqueued user
+};
+struct HostStage {
+  uint8_t *buf = nullptr;
+  size_t cap = 0;
+};
+struct StageSet {
+  DeviceStage dev[2];
+  HostStage host;
+  hipEvent_t pingpong[2] = {nullptr, nullptr};
+  ~StageSet() {
+    // Best effort: the thread is ending; errors (including a runtime that is
+    // already shutting down) are ignored.
+    for (auto &d : dev) {
+      if (d.buf)
+        (void)hipFree(d.buf);
+      if (d.last_use)
+        (void)hipEventDestroy(d.last_use);
+    }
+    if (host.buf)
+      (void)hipHostFree(host.buf);
+    for (auto &e : pingpong)
+      if (e)
+        (void)hipEventDestroy(e);
+    (void)hipGetLastError();
+  }
+};
+StageSet &stage_set(int device) {
+  thread_local std::unordered_map<int, StageSet> sets;
+  return sets[device];
+}
+
+// Device staging of at least `bytes`; nullptr when HBM is exhausted (callers
+// fall back to PER_BLOCK like the reference, csrc/ce_transfer.cu:149-169).
+// Work already enqueued on other streams that still uses the buffer is ordered
+// before `stream`.
+uint8_t *device_stage(int device, int slot, size_t bytes, hipStream_t stream) {
+  DeviceStage &s = stage_set(device).dev[slot];
+  if (!s.last_use) {
+    if (hipEventCreateWithFlags(&s.last_use, hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      s.last_use = nullptr;
+      return nullptr;
+    }
+  }
+  if (bytes > s.cap) {
+    if (s.buf) {
+      (void)hipEventSynchronize(s.last_use);
+      (void)hipFree(s.buf);
+      s.buf = nullptr;
+      s.cap = 0;
+    }
+    void *p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    s.buf = static_cast<uint8_t *>(p);
+    s.cap = bytes;
+  } else {
+    (void)hipStreamWaitEvent(stream, s.last_use, 0);
+  }
+  return s.buf;
+}
+void device_stage_mark(int device, int slot, hipStream_t stream) {
+  DeviceStage &s = stage_set(device).dev[slot];
+  if (s.last_use)
+    (void)hipEventRecord(s.last_use, stream);
+}
+
+uint8_t *host_stage(int device, size_t bytes) {
+  HostStage &s = stage_set(device).host;
+  if (bytes > s.cap) {
+    if (s.buf)
+      (void)hipHostFree(s.buf);
+    s.buf = nullptr;
+    s.cap = 0;
+    void *p = nullptr;
+    if (hipHostMalloc(&p, bytes, hipHostMallocPortable) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    s.buf = static_cast<uint8_t *>(p);
+    s.cap = bytes;
+  }
+  return s.buf;
+}
+hipEvent_t *pingpong_events(int device) {
+  StageSet &s = stage_set(device);
+  for (auto &e : s.pingpong)
+    if (!e && hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      e = nullptr;
+      return nullptr;
+    }
+  return s.pingpong;
+}
+
+size_t staging_cap_bytes() {
+  static const size_t cap = [] {
+    const char *v = std::getenv("FKV_CE_STAGING_MB");
+    long mb = (v && *v) ? std::atol(v) : 1024;
+    if (mb < 1)
+      mb = 1;
+    return (size_t)mb << 20;
+  }();
+  return cap;
+}
+
+// ---- one transfer's state ------------------------------------------------
+struct Job {
+  const fkv_transfer_desc &d;
+  hipStream_t stream;
+  int device;
+  bool h2d;
+  hipMemcpyKind kind;
+  Analysis an;
+
+  uint8_t *gpu(int layer_local, int kv, int64_t block) const {
+    return reinterpret_cast<uint8_t *>(
+        (uintptr_t)gpu_chunk_addr(d, (int64_t)d.start_layer_id + layer_local, kv, block));
+  }
+  uint8_t *cpu(int layer_local, int kv, int64_t block) const {
+    return cpu_chunk_ptr(d, (int64_t)d.start_layer_id + layer_local, kv, block);
+  }
+  int dma(void *dst, const void *src, size_t bytes, hipMemcpyKind k) const {
+    stats().dma_copies.fetch_add(1, std::memory_order_relaxed);
+    FKV_HIP_TRY(hipMemcpyAsync(dst, src, bytes, k, stream));
+    return FKV_OK;
+  }
+  // gpu <-> cpu copy in the direction of the transfer
+  int dma_dir(uint8_t *gpu_p, uint8_t *cpu_p, size_t bytes) const {
+    return h2d ? dma(gpu_p, cpu_p, bytes, kind) : dma(cpu_p, gpu_p, bytes, kind);
+  }
+  int dma2d(void *dst, size_t dpitch, const void *src, size_t spitch, size_t width,
+            size_t height, hipMemcpyKind k) const {
+    stats().dma_copies.fetch_add(1, std::memory_order_relaxed);
+    FKV_HIP_TRY(hipMemcpy2DAsync(dst, dpitch, src, spitch, width, height, k, stream));
+    return FKV_OK;
+  }
+};
+
+// csrc/ce_transfer.cu:196-229
+int per_block(const Job &j) {
+  const auto &d = j.d;
+  for (int i = 0; i < d.num_layers; ++i)
+    for (int kv = 0; kv < d.kv_dim; ++kv)
+      for (int b = 0; b < d.num_blocks; ++b)
+        FKV_TRY(j.dma_dir(j.gpu(i, kv, d.gpu_block_ids[b]), j.cpu(i, kv, d.cpu_block_ids[b]),
+                          (size_t)d.chunk_size));
+  return FKV_OK;
+}
+
+// csrc/ce_transfer.cu:235-267
+int contig_direct(const Job &j) {
+  const auto &d = j.d;
+  const size_t run = (size_t)d.chunk_size * (size_t)d.num_blocks;
+  for (int i = 0; i < d.num_layers; ++i)
+    for (int kv = 0; kv < d.kv_dim; ++kv)
+      FKV_TRY(j.dma_dir(j.gpu(i, kv, d.gpu_block_ids[0]), j.cpu(i, kv, d.cpu_block_ids[0]),
+                        run));
+  return FKV_OK;
+}
+
+// csrc/ce_transfer.cu:271-309
+int segment_direct(const Job &j) {
+  const auto &d = j.d;
+  for (int i = 0; i < d.num_layers; ++i)
+    for (int kv = 0; kv < d.kv_dim; ++kv)
+      for (const auto &s : j.an.segs)
+        FKV_TRY(j.dma_dir(j.gpu(i, kv, d.gpu_block_ids[s.start_k]),
+                          j.cpu(i, kv, d.cpu_block_ids[s.start_k]),
+                          (size_t)s.nr_blocks * (size_t)d.chunk_size));
+  return FKV_OK;
+}
+
+bool use_memcpy2d(const Job &j) {
+  return j.d.ce.enable_memcpy2d && j.an.a.num_segments <= j.d.ce.segment_threshold;
+}
+
+// Host rows of (layer, kv): base of block 0 including all offsets.
+uint8_t *cpu_row_base(const Job &j, int layer_local, int kv) { return j.cpu(layer_local, kv, 0); }
+
+void rows_to_from_cpu(const Job &j, uint8_t *staging, int layer_local, int kv, bool to_cpu) {
+  const auto &d = j.d;
+  host_rows_copy(staging, cpu_row_base(j, layer_local, kv), d.cpu_block_ids, d.num_blocks,
+                 d.cpu_block_stride, d.chunk_size, to_cpu, j.an.a.cpu_phys_contig != 0,
+                 d.ce.gather_threads, d.ce.gather_nt != 0);
+}
+
+// Runs `produce(it, buf)` (enqueue the GPU->host DMA of iteration `it` into
+// pinned buffer `buf`) and the host scatter of the previous iteration in
+// alternation, so the scatter of (layer, kv) overlaps the DMA of the next one
+// (csrc/ce_transfer.cu:713-810, 1023-1143).
+template <typename Produce>
+int d2h_pingpong(const Job &j, Produce produce) {
+  const auto &d = j.d;
+  const size_t layer_bytes = (size_t)d.num_blocks * (size_t)d.chunk_size;
+  uint8_t *base = host_stage(j.device, 2 * layer_bytes);
+  hipEvent_t *ev = pingpong_events(j.device);
+  if (!base || !ev)
+    return fail(FKV_ERR_RUNTIME, "cannot allocate %zu B of pinned staging", 2 * layer_bytes);
+  stats().staging_bytes_host.fetch_add((uint64_t)layer_bytes * d.num_layers * d.kv_dim);
+  uint8_t *bufs[2] = {base, base + layer_bytes};
+  const int iters = d.num_layers * d.kv_dim;
+  for (int it = 0; it <= iters; ++it) {
+    if (it < iters) {
+      FKV_TRY(produce(it, bufs[it & 1]));
+      FKV_HIP_TRY(hipEventRecord(ev[it & 1], j.stream));
+    }
+    if (it >= 1) {
+      const int p = it - 1;
+      FKV_HIP_TRY(hipEventSynchronize(ev[p & 1]));
+      rows_to_from_cpu(j, bufs[p & 1], p / d.kv_dim, p % d.kv_dim, /*to_cpu=*/true);
+    }
+  }
+  return FKV_OK;
+}
+
+// Host->GPU mirror image: gather (layer, kv) rows into one of two pinned
+// buffers, `consume(it, buf)` enqueues the DMA(s) out of it; a buffer is reused
+// only after the DMA that read it has finished.  Returns with the stream idle
+// with respect to the staging buffers.
+template <typename Consume>
+int h2d_pingpong(const Job &j, Consume consume) {
+  const auto &d = j.d;
+  const size_t layer_bytes = (size_t)d.num_blocks * (size_t)d.chunk_size;
+  uint8_t *base = host_stage(j.device, 2 * layer_bytes);
+  hipEvent_t *ev = pingpong_events(j.device);
+  if (!base || !ev)
+    return fail(FKV_ERR_RUNTIME, "cannot allocate %zu B of pinned staging", 2 * layer_bytes);
+  stats().staging_bytes_host.fetch_add((uint64_t)layer_bytes * d.num_layers * d.kv_dim);
+  uint8_t *bufs[2] = {base, base + layer_bytes};
+  const int iters = d.num_layers * d.kv_dim;
+  for (int it = 0; it < iters; ++it) {
+    if (it >= 2)
+      FKV_HIP_TRY(hipEventSynchronize(ev[it & 1]));
+    rows_to_from_cpu(j, bufs[it & 1], it / d.kv_dim, it % d.kv_dim, /*to_cpu=*/false);
+    FKV_TRY(consume(it, bufs[it & 1]));
+    FKV_HIP_TRY(hipEventRecord(ev[it & 1], j.stream));
+  }
+  for (int k = 0; k < 2 && k < iters; ++k)
+    FKV_HIP_TRY(hipEventSynchronize(ev[k]));
+  return FKV_OK;
+}
+
+// csrc/ce_transfer.cu:645-812
+int segment_scatter(const Job &j) {
+  const auto &d = j.d;
+  if (use_memcpy2d(j)) {
+    // one strided 2-D copy per (layer, kv, segment): rows = blocks of the segment
+    for (int i = 0; i < d.num_layers; ++i)
+      for (int kv = 0; kv < d.kv_dim; ++kv)
+        for (const auto &s : j.an.segs) {
+          uint8_t *g = j.gpu(i, kv, d.gpu_block_ids[s.start_k]);
+          uint8_t *c = j.cpu(i, kv, d.cpu_block_ids[s.start_k]);
+          if (j.h2d)
+            FKV_TRY(j.dma2d(g, (size_t)d.gpu_block_stride, c, (size_t)d.cpu_block_stride,
+                            (size_t)d.chunk_size, (size_t)s.nr_blocks, j.kind));
+          else
+            FKV_TRY(j.dma2d(c, (size_t)d.cpu_block_stride, g, (size_t)d.gpu_block_stride,
+                            (size_t)d.chunk_size, (size_t)s.nr_blocks, j.kind));
+        }
+    return FKV_OK;
+  }
+  if (!j.h2d) {
+    return d2h_pingpong(j, [&](int it, uint8_t *buf) {
+      size_t off = 0;
+      for (const auto &s : j.an.segs) {
+        const size_t n = (size_t)s.nr_blocks * (size_t)d.chunk_size;
+        FKV_TRY(j.dma(buf + off, j.gpu(it / d.kv_dim, it % d.kv_dim, d.gpu_block_ids[s.start_k]),
+                      n, hipMemcpyDeviceToHost));
+        off += n;
+      }
+      return (int)FKV_OK;
+    });
+  }
+  return h2d_pingpong(j, [&](int it, uint8_t *buf) {
+    size_t off = 0;
+    for (const auto &s : j.an.segs) {
+      const size_t n = (size_t)s.nr_blocks * (size_t)d.chunk_size;
+      FKV_TRY(j.dma(j.gpu(it / d.kv_dim, it % d.kv_dim, d.gpu_block_ids[s.start_k]), buf + off, n,
+                    hipMemcpyHostToDevice));
+      off += n;
+    }
+    return (int)FKV_OK;
+  });
+}
+
+} // namespace
+
+// Device-side compaction.  `it` numbers the (layer, kv) pairs of the call:
+// it = layer_local * kv_dim + kv.  Moves the chunks of pairs [it0, it0+nit) x
+// block positions [p0, p0+np) between the engine's KV tensors and a packed
+// device buffer laid out [np][nit][chunk] (blockfirst) or [nit][np][chunk].
+int device_staging_copy(const fkv_transfer_desc &d, int it0, int nit, int p0, int np,
+                        uint8_t *staging, bool blockfirst, bool to_staging,
+                        hipStream_t stream) {
+  static const int kStagingWorkgroups = [] {
+    const char *v = std::getenv("FKV_STAGING_WORKGROUPS");
+    int n = (v && *v) ? std::atoi(v) : 2048;
+    return n > 0 ? n : 2048;
+  }();
+  int device = 0;
+  FKV_HIP_TRY(hipGetDevice(&device));
+  for (int b0 = 0; b0 < nit; b0 += kCopyMaxLK) {
+    const int lk = std::min(kCopyMaxLK, nit - b0);
+    const size_t tab = (size_t)lk * 8, ids = (size_t)np * 8;
+    PlanSlot *slot = plan_acquire(device, 2 * tab + ids);
+    if (!slot)
+      return FKV_ERR_RUNTIME;
+    uint8_t *h = plan_host(slot);
+    uint64_t *gbase = reinterpret_cast<uint64_t *>(h);
+    uint64_t *sbase = reinterpret_cast<uint64_t *>(h + tab);
+    const int64_t stg_stride = blockfirst ? (int64_t)nit * d.chunk_size : d.chunk_size;
+    uint64_t acc = (uint64_t)d.chunk_size | (uint64_t)d.gpu_block_stride | (uint64_t)stg_stride;
+    for (int i = 0; i < lk; ++i) {
+      const int it = it0 + b0 + i;
+      gbase[i] = gpu_chunk_addr(d, (int64_t)d.start_layer_id + it / d.kv_dim, it % d.kv_dim, 0);
+      const uint64_t slot_in_stage = (uint64_t)(b0 + i);
+      sbase[i] = (uint64_t)(uintptr_t)staging +
+                 (blockfirst ? slot_in_stage * (uint64_t)d.chunk_size
+                             : slot_in_stage * (uint64_t)np * (uint64_t)d.chunk_size);
+      acc |= gbase[i] | sbase[i];
+    }
+    std::memcpy(h + 2 * tab, d.gpu_block_ids + p0, ids);
+    uint8_t *dv = nullptr;
+    int rc = plan_publish(slot, 2 * tab + ids, /*mirror=*/true, stream, &dv);
+    if (rc == FKV_OK) {
+      CopyKernelArgs a{};
+      const uint64_t *dg = reinterpret_cast<const uint64_t *>(dv);
+      const uint64_t *ds = reinterpret_cast<const uint64_t *>(dv + tab);
+      const int64_t *dids = reinterpret_cast<const int64_t *>(dv + 2 * tab);
+      a.base_src = to_staging ? dg : ds;
+      a.base_dst = to_staging ? ds : dg;
+      a.ids_src = to_staging ? dids : nullptr;
+      a.ids_dst = to_staging ? nullptr : dids;
+      a.stride_src = to_staging ? d.gpu_block_stride : stg_stride;
+      a.stride_dst = to_staging ? stg_stride : d.gpu_block_stride;
+      a.chunk_bytes = d.chunk_size;
+      a.num_blocks = np;
+      a.lk = lk;
+      a.vec = common_vector_width(&acc, 1);
+      rc = launch_copy_kernel(a, kStagingWorkgroups, stream);
+    }
+    plan_release(slot, stream, false);
+    if (rc != FKV_OK)
+      return rc;
+  }
+  stats().staging_bytes_device.fetch_add((uint64_t)nit * (uint64_t)np * (uint64_t)d.chunk_size);
+  return FKV_OK;
+}
+
+namespace {
+
+// csrc/ce_transfer.cu:816-1179
+int gather_scatter(const Job &j) {
+  const auto &d = j.d;
+  const bool gpu_run = j.an.a.gpu_log_contig && j.an.a.gpu_phys_contig; // one linear GPU run
+  const bool cpu_run = j.an.a.cpu_log_contig && j.an.a.cpu_phys_contig; // one linear host run
+  const size_t layer_bytes = (size_t)d.num_blocks * (size_t)d.chunk_size;
+  uint8_t *dev[2] = {nullptr, nullptr};
+  if (!gpu_run) {
+    for (int k = 0; k < 2; ++k) {
+      dev[k] = device_stage(j.device, k, layer_bytes, j.stream);
+      if (!dev[k])
+        return per_block(j); // HBM exhausted, csrc/ce_transfer.cu:859
+    }
+  }
+  auto mark_dev = [&] {
+    if (!gpu_run)
+      for (int k = 0; k < 2; ++k)
+        device_stage_mark(j.device, k, j.stream);
+  };
+  const int iters = d.num_layers * d.kv_dim;
+  auto pack = [&](int it, bool to_staging) {
+    return device_staging_copy(d, it, 1, 0, d.num_blocks, dev[it & 1], false, to_staging,
+                               j.stream);
+  };
+
+  if (use_memcpy2d(j)) {
+    // device compaction + one strided 2-D DMA per segment, no host staging
+    // (csrc/ce_transfer.cu:933-1018)
+    int rc = FKV_OK;
+    for (int it = 0; it < iters && rc == FKV_OK; ++it) {
+      const int i = it / d.kv_dim, kv = it % d.kv_dim;
+      uint8_t *packed = gpu_run ? j.gpu(i, kv, d.gpu_block_ids[0]) : dev[it & 1];
+      const size_t pitch = gpu_run ? (size_t)d.gpu_block_stride : (size_t)d.chunk_size;
+      if (!j.h2d && !gpu_run)
+        rc = pack(it, true);
+      for (size_t si = 0; si < j.an.segs.size() && rc == FKV_OK; ++si) {
+        const auto &s = j.an.segs[si];
+        uint8_t *c = j.cpu(i, kv, d.cpu_block_ids[s.start_k]);
+        uint8_t *p = packed + (size_t)s.start_k * pitch;
+        rc = j.h2d ? j.dma2d(p, pitch, c, (size_t)d.cpu_block_stride, (size_t)d.chunk_size,
+                             (size_t)s.nr_blocks, j.kind)
+                   : j.dma2d(c, (size_t)d.cpu_block_stride, p, pitch, (size_t)d.chunk_size,
+                             (size_t)s.nr_blocks, j.kind);
+      }
+      if (rc == FKV_OK && j.h2d && !gpu_run)
+        rc = pack(it, false);
+    }
+    mark_dev();
+    return rc;
+  }
+
+  int rc = FKV_OK;
+  if (!j.h2d) {
+    auto produce = [&](int it, uint8_t *host_dst) {
+      const uint8_t *src = dev[it & 1];
+      if (gpu_run)
+        src = j.gpu(it / d.kv_dim, it % d.kv_dim, d.gpu_block_ids[0]);
+      else
+        FKV_TRY(pack(it, true));
+      return j.dma(host_dst, src, layer_bytes, hipMemcpyDeviceToHost);
+    };
+    if (cpu_run) {
+      // destination rows are one linear run: DMA straight into place
+      for (int it = 0; it < iters && rc == FKV_OK; ++it)
+        rc = produce(it, j.cpu(it / d.kv_dim, it % d.kv_dim, d.cpu_block_ids[0]));
+    } else {
+      rc = d2h_pingpong(j, produce);
+    }
+  } else {
+    auto consume = [&](int it, uint8_t *host_src) {
+      if (gpu_run)
+        return j.dma(j.gpu(it / d.kv_dim, it % d.kv_dim, d.gpu_block_ids[0]), host_src,
+                     layer_bytes, hipMemcpyHostToDevice);
+      FKV_TRY(j.dma(dev[it & 1], host_src, layer_bytes, hipMemcpyHostToDevice));
+      return pack(it, false);
+    };
+    if (cpu_run) {
+      for (int it = 0; it < iters && rc == FKV_OK; ++it)
+        rc = consume(it, j.cpu(it / d.kv_dim, it % d.kv_dim, d.cpu_block_ids[0]));
+    } else {
+      rc = h2d_pingpong(j, consume);
+    }
+  }
+  mark_dev();
+  return rc;
+}
+
+// csrc/ce_transfer.cu:1183-1400.  Device staging holds whole host blocks
+// ([block][layer*kv][chunk] == the block-first host layout), so every DMA moves
+// at least one complete block and cpu-adjacent blocks merge into one DMA.
+int gather_direct(const Job &j) {
+  const auto &d = j.d;
+  const int lk = d.num_layers * d.kv_dim;
+  const bool dense = (d.kv_dim == 1 || d.cpu_kv_stride == d.chunk_size) &&
+                     (d.num_layers == 1 || d.cpu_layer_stride == (int64_t)d.kv_dim * d.chunk_size);
+  if (!dense)
+    return gather_scatter(j); // host chunks of a block are not adjacent: stage per (layer, kv)
+  const size_t block_bytes = (size_t)lk * (size_t)d.chunk_size;
+  const bool full_block = (int64_t)block_bytes == d.cpu_block_stride;
+  const int group =
+      (int)std::min<size_t>((size_t)d.num_blocks, std::max<size_t>(1, staging_cap_bytes() / block_bytes));
+  uint8_t *stage = device_stage(j.device, 0, (size_t)group * block_bytes, j.stream);
+  if (!stage)
+    return per_block(j);
+  int rc = FKV_OK;
+  size_t seg_i = 0;
+  for (int p0 = 0; p0 < d.num_blocks && rc == FKV_OK; p0 += group) {
+    const int np = std::min(group, d.num_blocks - p0);
+    if (!j.h2d)
+      rc = device_staging_copy(d, 0, lk, p0, np, stage, true, true, j.stream);
+    // segments (cpu- and gpu-adjacent runs) clipped to this group
+    while (seg_i < j.an.segs.size() && rc == FKV_OK) {
+      const auto &s = j.an.segs[seg_i];
+      const int b = std::max(s.start_k, p0);
+      const int e = std::min(s.start_k + s.nr_blocks, p0 + np);
+      if (b < e) {
+        uint8_t *c = j.cpu(0, 0, d.cpu_block_ids[b]);
+        uint8_t *g = stage + (size_t)(b - p0) * block_bytes;
+        const size_t rows = (size_t)(e - b);
+        if (full_block) {
+          rc = j.dma_dir(g, c, rows * block_bytes);
+        } else if (d.ce.enable_memcpy2d) {
+          rc = j.h2d ? j.dma2d(g, block_bytes, c, (size_t)d.cpu_block_stride, block_bytes, rows,
+                               j.kind)
+                     : j.dma2d(c, (size_t)d.cpu_block_stride, g, block_bytes, block_bytes, rows,
+                               j.kind);
+        } else {
+          for (size_t r = 0; r < rows && rc == FKV_OK; ++r)
+            rc = j.dma_dir(g + r * block_bytes, c + r * (size_t)d.cpu_block_stride, block_bytes);
+        }
+      }
+      if (s.start_k + s.nr_blocks > p0 + np)
+        break; // the rest of this segment belongs to the next group
+      ++seg_i;
+    }
+    if (rc == FKV_OK && j.h2d)
+      rc = device_staging_copy(d, 0, lk, p0, np, stage, true, false, j.stream);
+  }
+  device_stage_mark(j.device, 0, j.stream);
+  return rc;
+}
+
+const char *path_name(int p) {
+  switch (p) {
+  case FKV_CE_CONTIG_DIRECT: return "CONTIG_DIRECT";
+  case FKV_CE_SEGMENT_DIRECT: return "SEGMENT_DIRECT";
+  case FKV_CE_SEGMENT_SCATTER: return "SEGMENT_SCATTER";
+  case FKV_CE_GATHER_SCATTER: return "GATHER_SCATTER";
+  case FKV_CE_GATHER_DIRECT: return "GATHER_DIRECT";
+  default: return "PER_BLOCK";
+  }
+}
+
+} // namespace
+
+int run_ce_path(const fkv_transfer_desc &d, hipStream_t stream) {
+  int device = 0;
+  FKV_HIP_TRY(hipGetDevice(&device));
+  Job j{d, stream, device, d.is_host_to_device != 0,
+        d.is_host_to_device ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost, {}};
+  analyze(d.gpu_block_ids, d.cpu_block_ids, d.num_blocks, d.cpu_block_stride, d.chunk_size,
+          d.gpu_block_stride, j.an);
+  if (!d.ce.path_opt_enabled) { // csrc/transfer.cu:201-208
+    set_last_path(FKV_CE_PER_BLOCK);
+    return per_block(j);
+  }
+  int path;
+  const auto &a = j.an.a;
+  if (d.ce.force_path >= 0) {
+    if (d.ce.force_path > 4) // csrc/transfer.cu:213-214
+      return fail(FKV_ERR_RUNTIME, "force_path out of range [0,4]: %d", d.ce.force_path);
+    path = d.ce.force_path;
+    // A forced strategy whose layout assumptions do not hold would copy the
+    // wrong addresses; refuse instead.
+    const bool ok =
+        (path == FKV_CE_CONTIG_DIRECT)
+            ? (a.gpu_log_contig && a.cpu_log_contig && a.cpu_phys_contig && a.gpu_phys_contig)
+        : (path == FKV_CE_SEGMENT_DIRECT) ? (a.cpu_phys_contig && a.gpu_phys_contig)
+        : (path == FKV_CE_SEGMENT_SCATTER) ? (a.gpu_phys_contig || use_memcpy2d(j))
+                                           : true;
+    if (!ok)
+      return fail(FKV_ERR_INVALID_ARG,
+                  "forced copy-engine strategy %s does not fit this transfer "
+                  "(gpu_log=%d cpu_log=%d cpu_phys=%d gpu_phys=%d)",
+                  path_name(path), a.gpu_log_contig, a.cpu_log_contig, a.cpu_phys_contig,
+                  a.gpu_phys_contig);
+  } else {
+    const bool full_block = // csrc/transfer.cu:219-220
+        (int64_t)d.num_layers * d.kv_dim * d.chunk_size == d.cpu_block_stride;
+    path = choose(a, d.ce, d.chunk_size, j.h2d, full_block);
+  }
+  set_last_path(path);
+  switch (path) {
+  case FKV_CE_CONTIG_DIRECT: return contig_direct(j);
+  case FKV_CE_SEGMENT_DIRECT: return segment_direct(j);
+  case FKV_CE_SEGMENT_SCATTER: return segment_scatter(j);
+  case FKV_CE_GATHER_SCATTER: return gather_scatter(j);
+  default: return gather_direct(j);
+  }
+}
+
+} // namespace fkv
+
+extern "C" {
+
+int fkv_ce_analyze(const int64_t *gpu_block_ids, const int64_t *cpu_block_ids,
+                   int32_t num_blocks, int64_t cpu_block_stride, int64_t chunk_size,
+                   int64_t gpu_block_stride, fkv_ce_analysis *out, fkv_ce_segment *segments,
+                   int32_t segment_capacity) {
+  fkv::clear_error();
+  if (!out || num_blocks < 0 || (num_blocks > 0 && (!gpu_block_ids || !cpu_block_ids)))
+    return fkv::fail(FKV_ERR_INVALID_ARG, "fkv_ce_analyze: bad arguments");
+  fkv::Analysis an;
+  fkv::analyze(gpu_block_ids, cpu_block_ids, num_blocks, cpu_block_stride, chunk_size,
+               gpu_block_stride, an);
+  *out = an.a;
+  if (segments)
+    for (int i = 0; i < (int)an.segs.size() && i < segment_capacity; ++i)
+      segments[i] = an.segs[i];
+  return FKV_OK;
+}
+
+int fkv_ce_choose_path(const fkv_ce_analysis *analysis, const fkv_ce_config *cfg,
+                       int64_t chunk_size, int32_t is_host_to_device, int32_t is_full_block) {
+  return fkv::choose(*analysis, *cfg, chunk_size, is_host_to_device != 0, is_full_block != 0);
+}
+
+} // extern "C"

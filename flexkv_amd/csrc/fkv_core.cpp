@@ -1,0 +1,422 @@
+// Errors, counters, plan memory and the dispatcher of fkv_transfer_kv_blocks.
+//
+// Host side of what csrc/transfer.cu:164-313 does in the reference: pick the
+// kernel path or the copy-engine path, enqueue it on the caller's stream,
+// optionally wait and trace.
+#include "fkv_internal.h"
+
+#include <chrono>
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+#include <mutex>
+
+namespace fkv {
+
+// ---- errors -------------------------------------------------------------
+namespace {
+thread_local std::string t_last_error;
+thread_local int t_last_path = FKV_PATH_KERNEL;
+} // namespace
+
+int fail(int code, const char *fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  t_last_error = buf;
+  return code;
+}
+void clear_error() { t_last_error.clear(); }
+void set_last_path(int path) { t_last_path = path; }
+
+Stats &stats() {
+  static Stats s;
+  return s;
+}
+
+DeviceGuard::DeviceGuard(int device) : device_(device) {
+  if (hipGetDevice(&prev_) != hipSuccess) {
+    (void)hipGetLastError();
+    ok_ = false;
+    return;
+  }
+  if (device < 0) {
+    device_ = prev_;
+    return;
+  }
+  if (device != prev_) {
+    if (hipSetDevice(device) != hipSuccess) {
+      (void)hipGetLastError();
+      ok_ = false;
+      return;
+    }
+    switched_ = true;
+  }
+}
+DeviceGuard::~DeviceGuard() {
+  if (switched_)
+    (void)hipSetDevice(prev_);
+}
+
+// ---- plan memory ---------------------------------------------------------
+struct PlanSlot {
+  uint8_t *host = nullptr;
+  uint8_t *dev = nullptr;
+  size_t cap = 0;
+  hipEvent_t done = nullptr;
+  bool busy = false;          // handed out, not yet released
+  bool event_pending = false; // released behind an event that may not have fired
+  int device = 0;
+};
+
+namespace {
+struct PlanPool {
+  std::mutex mu;
+  // Slots are never freed: the pool outlives every stream that may still read
+  // them, and tearing HIP objects down from a static destructor is unsafe.
+  std::vector<PlanSlot *> slots;
+};
+PlanPool &pool() {
+  static PlanPool *p = new PlanPool();
+  return *p;
+}
+constexpr size_t kPlanMinBytes = 64 * 1024;
+
+bool slot_grow(PlanSlot *s, size_t bytes) {
+  if (s->cap >= bytes)
+    return true;
+  size_t cap = kPlanMinBytes;
+  while (cap < bytes)
+    cap *= 2;
+  if (s->host)
+    (void)hipHostFree(s->host);
+  if (s->dev)
+    (void)hipFree(s->dev);
+  s->host = s->dev = nullptr;
+  s->cap = 0;
+  void *h = nullptr, *d = nullptr;
+  if (hipHostMalloc(&h, cap, hipHostMallocPortable | hipHostMallocMapped) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  if (hipMalloc(&d, cap) != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipHostFree(h);
+    return false;
+  }
+  s->host = static_cast<uint8_t *>(h);
+  s->dev = static_cast<uint8_t *>(d);
+  s->cap = cap;
+  return true;
+}
+} // namespace
+
+PlanSlot *plan_acquire(int device, size_t bytes) {
+  PlanPool &p = pool();
+  PlanSlot *pick = nullptr;
+  PlanSlot *waitable = nullptr;
+  {
+    std::lock_guard<std::mutex> lk(p.mu);
+    for (PlanSlot *s : p.slots) {
+      if (s->busy || s->device != device)
+        continue;
+      if (s->event_pending) {
+        hipError_t q = hipEventQuery(s->done);
+        if (q == hipSuccess) {
+          s->event_pending = false;
+        } else {
+          (void)hipGetLastError();
+          if (!waitable)
+            waitable = s;
+          continue;
+        }
+      }
+      if (!pick || (pick->cap < bytes && s->cap > pick->cap))
+        pick = s;
+      if (pick->cap >= bytes)
+        break;
+    }
+    if (!pick && waitable && p.slots.size() >= 256) {
+      pick = waitable; // pool is large enough: wait for the oldest user instead
+    }
+    if (!pick) {
+      pick = new PlanSlot();
+      pick->device = device;
+      if (hipEventCreateWithFlags(&pick->done, hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError();
+        delete pick;
+        fail(FKV_ERR_RUNTIME, "plan memory: hipEventCreate failed");
+        return nullptr;
+      }
+      p.slots.push_back(pick);
+    }
+    pick->busy = true;
+  }
+  if (pick->event_pending) {
+    (void)hipEventSynchronize(pick->done);
+    pick->event_pending = false;
+  }
+  if (!slot_grow(pick, bytes)) {
+    std::lock_guard<std::mutex> lk(p.mu);
+    pick->busy = false;
+    fail(FKV_ERR_RUNTIME, "plan memory: cannot allocate %zu bytes of pinned/device memory",
+         bytes);
+    return nullptr;
+  }
+  return pick;
+}
+
+uint8_t *plan_host(PlanSlot *s) { return s->host; }
+
+int plan_publish(PlanSlot *s, size_t bytes, bool mirror, hipStream_t stream,
+                 uint8_t **device_visible) {
+  if (!mirror) {
+    *device_visible = s->host; // hipHostMalloc memory: same address on the device
+    return FKV_OK;
+  }
+  FKV_HIP_TRY(hipMemcpyAsync(s->dev, s->host, bytes, hipMemcpyHostToDevice, stream));
+  *device_visible = s->dev;
+  return FKV_OK;
+}
+
+void plan_release(PlanSlot *s, hipStream_t stream, bool drained) {
+  if (!s)
+    return;
+  bool pending = false;
+  if (!drained) {
+    if (hipEventRecord(s->done, stream) == hipSuccess) {
+      pending = true;
+    } else {
+      (void)hipGetLastError();
+      (void)hipStreamSynchronize(stream);
+    }
+  }
+  std::lock_guard<std::mutex> lk(pool().mu);
+  s->event_pending = pending;
+  s->busy = false;
+}
+
+// ---- kernel path ---------------------------------------------------------
+namespace {
+int env_int(const char *name, int fallback) {
+  const char *v = std::getenv(name);
+  if (!v || !*v)
+    return fallback;
+  return std::atoi(v);
+}
+} // namespace
+
+int default_num_cta(bool is_h2d) {
+  static const int h2d = env_int("FKV_NUM_CTA_H2D", 8);
+  static const int d2h = env_int("FKV_NUM_CTA_D2H", 8);
+  return is_h2d ? h2d : d2h;
+}
+
+int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream) {
+  set_last_path(FKV_PATH_KERNEL);
+  // Device-visible alias of the host pool.  hipHostMalloc / torch pinned memory
+  // map to the same address; hipHostRegister-ed memory may not.
+  void *cpu_dev = nullptr;
+  hipError_t e = hipHostGetDevicePointer(&cpu_dev, d.cpu_ptr, 0);
+  if (e != hipSuccess || !cpu_dev) {
+    (void)hipGetLastError();
+    return fail(FKV_ERR_INVALID_ARG,
+                "cpu_tensor at %p is not device-visible (allocate it pinned or register it "
+                "before a kernel transfer): %s",
+                d.cpu_ptr, hipGetErrorString(e));
+  }
+  const bool h2d = d.is_host_to_device != 0;
+  static const bool mirror_plan = env_int("FKV_PLAN_MIRROR", 1) != 0;
+  int num_cta = d.transfer_num_cta > 0 ? d.transfer_num_cta : default_num_cta(h2d);
+
+  // Layers go out in groups whose (layer, kv) base tables fit the kernel's LDS.
+  const int layers_per_launch = kCopyMaxLK / d.kv_dim;
+  if (layers_per_launch < 1)
+    return fail(FKV_ERR_INVALID_ARG, "kv_dim %d too large", d.kv_dim);
+  for (int l0 = 0; l0 < d.num_layers; l0 += layers_per_launch) {
+    const int nl = std::min(layers_per_launch, d.num_layers - l0);
+    const int lk = nl * d.kv_dim;
+    const size_t tab_bytes = (size_t)lk * 8;
+    const size_t ids_bytes = (size_t)d.num_blocks * 8;
+    const size_t plan_bytes = 2 * tab_bytes + 2 * ids_bytes;
+    PlanSlot *slot = plan_acquire(DeviceGuard(-1).device(), plan_bytes);
+    if (!slot)
+      return FKV_ERR_RUNTIME;
+    uint8_t *h = plan_host(slot);
+    uint64_t *gbase = reinterpret_cast<uint64_t *>(h);
+    uint64_t *cbase = reinterpret_cast<uint64_t *>(h + tab_bytes);
+    int64_t *gids = reinterpret_cast<int64_t *>(h + 2 * tab_bytes);
+    int64_t *cids = reinterpret_cast<int64_t *>(h + 2 * tab_bytes + ids_bytes);
+    uint64_t align_bits[8] = {(uint64_t)d.chunk_size, (uint64_t)d.gpu_block_stride,
+                              (uint64_t)d.cpu_block_stride, 0, 0, 0, 0, 0};
+    uint64_t acc = 0;
+    for (int li = 0; li < nl; ++li) {
+      const int64_t layer = (int64_t)d.start_layer_id + l0 + li;
+      for (int kv = 0; kv < d.kv_dim; ++kv) {
+        const uint64_t g = gpu_chunk_addr(d, layer, kv, 0);
+        const uint64_t c = (uint64_t)(uintptr_t)cpu_dev +
+                           (uint64_t)(layer * d.cpu_layer_stride + kv * d.cpu_kv_stride +
+                                      d.cpu_startoff_inside_chunks);
+        gbase[li * d.kv_dim + kv] = g;
+        cbase[li * d.kv_dim + kv] = c;
+        acc |= g | c;
+      }
+    }
+    align_bits[3] = acc;
+    std::memcpy(gids, d.gpu_block_ids, ids_bytes);
+    std::memcpy(cids, d.cpu_block_ids, ids_bytes);
+
+    uint8_t *dv = nullptr;
+    int rc = plan_publish(slot, plan_bytes, mirror_plan, stream, &dv);
+    if (rc != FKV_OK) {
+      plan_release(slot, stream, false);
+      return rc;
+    }
+    CopyKernelArgs a{};
+    const uint64_t *dv_gbase = reinterpret_cast<const uint64_t *>(dv);
+    const uint64_t *dv_cbase = reinterpret_cast<const uint64_t *>(dv + tab_bytes);
+    const int64_t *dv_gids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes);
+    const int64_t *dv_cids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes + ids_bytes);
+    a.base_src = h2d ? dv_cbase : dv_gbase;
+    a.base_dst = h2d ? dv_gbase : dv_cbase;
+    a.ids_src = h2d ? dv_cids : dv_gids;
+    a.ids_dst = h2d ? dv_gids : dv_cids;
+    a.stride_src = h2d ? d.cpu_block_stride : d.gpu_block_stride;
+    a.stride_dst = h2d ? d.gpu_block_stride : d.cpu_block_stride;
+    a.chunk_bytes = d.chunk_size;
+    a.num_blocks = d.num_blocks;
+    a.lk = lk;
+    a.vec = common_vector_width(align_bits, 4);
+    rc = launch_copy_kernel(a, num_cta, stream);
+    plan_release(slot, stream, false);
+    if (rc != FKV_OK)
+      return rc;
+  }
+  return FKV_OK;
+}
+
+namespace {
+int validate(const fkv_transfer_desc &d) {
+  if (d.backend != FKV_BACKEND_VLLM && d.backend != FKV_BACKEND_TRTLLM &&
+      d.backend != FKV_BACKEND_SGLANG)
+    return fail(FKV_ERR_RUNTIME, "Unsupported gpu_block_type: %d", d.backend);
+  if (d.num_blocks < 0 || d.num_layers < 0 || d.start_layer_id < 0 || d.kv_dim < 1)
+    return fail(FKV_ERR_INVALID_ARG,
+                "bad transfer extents: num_blocks=%d start_layer=%d num_layers=%d kv_dim=%d",
+                d.num_blocks, d.start_layer_id, d.num_layers, d.kv_dim);
+  if (d.chunk_size <= 0)
+    return fail(FKV_ERR_INVALID_ARG, "chunk_size_in_bytes must be positive, got %lld",
+                (long long)d.chunk_size);
+  if (d.num_blocks == 0 || d.num_layers == 0)
+    return FKV_OK;
+  if (!d.gpu_tensor_ptrs || !d.cpu_ptr || !d.gpu_block_ids || !d.cpu_block_ids)
+    return fail(FKV_ERR_INVALID_ARG, "null pointer in transfer descriptor");
+  // highest tensor-pointer index the addressing mode will touch
+  const int64_t last_layer = (int64_t)d.start_layer_id + d.num_layers - 1;
+  int64_t need = 1;
+  if (d.backend == FKV_BACKEND_VLLM)
+    need = last_layer + 1;
+  else if (d.backend == FKV_BACKEND_SGLANG)
+    need = (int64_t)(d.kv_dim - 1) * d.num_layers_total + last_layer + 1;
+  if (d.num_gpu_tensor_ptrs > 0 && need > d.num_gpu_tensor_ptrs)
+    return fail(FKV_ERR_INVALID_ARG,
+                "layer range [%d, %lld] with kv_dim %d needs %lld GPU tensor pointers, %d given",
+                d.start_layer_id, (long long)last_layer, d.kv_dim, (long long)need,
+                d.num_gpu_tensor_ptrs);
+  for (int i = 0; i < d.num_blocks; ++i)
+    if (d.gpu_block_ids[i] < 0 || d.cpu_block_ids[i] < 0)
+      return fail(FKV_ERR_INVALID_ARG, "negative block id at position %d", i);
+  return FKV_OK;
+}
+} // namespace
+
+} // namespace fkv
+
+extern "C" {
+
+int fkv_abi_version(void) { return FKV_ABI_VERSION; }
+const char *fkv_last_error(void) { return fkv::t_last_error.c_str(); }
+int fkv_last_path(void) { return fkv::t_last_path; }
+
+void fkv_ce_config_default(fkv_ce_config *cfg) {
+  if (!cfg)
+    return;
+  std::memset(cfg, 0, sizeof(*cfg));
+  cfg->segment_threshold = 8;
+  cfg->path_opt_enabled = 1;
+  cfg->force_path = -1;
+  cfg->enable_memcpy2d = 0;
+  cfg->is_blockfirst = 0;
+  cfg->num_kv_heads = 1;
+  cfg->gather_threads = 4;
+  cfg->gather_nt = 1;
+}
+
+void fkv_get_stats(fkv_stats *out) {
+  if (!out)
+    return;
+  fkv::Stats &s = fkv::stats();
+  out->calls = s.calls.load();
+  out->bytes_h2d = s.bytes_h2d.load();
+  out->bytes_d2h = s.bytes_d2h.load();
+  out->kernel_launches = s.kernel_launches.load();
+  out->dma_copies = s.dma_copies.load();
+  out->staging_bytes_device = s.staging_bytes_device.load();
+  out->staging_bytes_host = s.staging_bytes_host.load();
+  out->reserved = 0;
+}
+void fkv_reset_stats(void) {
+  fkv::Stats &s = fkv::stats();
+  s.calls = 0;
+  s.bytes_h2d = 0;
+  s.bytes_d2h = 0;
+  s.kernel_launches = 0;
+  s.dma_copies = 0;
+  s.staging_bytes_device = 0;
+  s.staging_bytes_host = 0;
+}
+
+int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream_v) {
+  using namespace fkv;
+  clear_error();
+  if (!desc)
+    return fail(FKV_ERR_INVALID_ARG, "null descriptor");
+  const fkv_transfer_desc &d = *desc;
+  FKV_TRY(validate(d));
+  hipStream_t stream = static_cast<hipStream_t>(stream_v);
+  stats().calls.fetch_add(1, std::memory_order_relaxed);
+  if (d.num_blocks == 0 || d.num_layers == 0)
+    return FKV_OK;
+  DeviceGuard guard(d.device);
+  if (!guard.ok())
+    return fail(FKV_ERR_RUNTIME, "cannot select HIP device %d", d.device);
+
+  const uint64_t bytes =
+      (uint64_t)d.num_blocks * d.num_layers * d.kv_dim * (uint64_t)d.chunk_size;
+  int rc = d.use_ce_transfer ? run_ce_path(d, stream) : run_kernel_path(d, stream);
+  if (rc != FKV_OK)
+    return rc;
+  (d.is_host_to_device ? stats().bytes_h2d : stats().bytes_d2h)
+      .fetch_add(bytes, std::memory_order_relaxed);
+
+  if (d.sync) {
+    auto t0 = std::chrono::steady_clock::now();
+    FKV_HIP_TRY(hipStreamSynchronize(stream));
+    if (d.enable_trace) {
+      double ms = std::chrono::duration<double, std::milli>(
+                      std::chrono::steady_clock::now() - t0)
+                      .count();
+      // same fields as the reference's trace line, csrc/transfer.cu:304-311
+      fprintf(stderr, "[XFER] type=%s blocks=%d sync_ms=%.3f\n",
+              d.is_host_to_device ? "H2D" : "D2H", d.num_blocks, ms);
+    }
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return fail(FKV_ERR_RUNTIME, "%s", hipGetErrorString(e));
+  return FKV_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,151 @@
+// Internal declarations shared by the translation units of libfkv_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+#include "fkv_transfer.h"
+
+namespace fkv {
+
+// ---- errors -------------------------------------------------------------
+// Records the message for fkv_last_error() on this thread and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+#define FKV_HIP_TRY(expr)                                                      \
+  do {                                                                         \
+    hipError_t fkv_e_ = (expr);                                                \
+    if (fkv_e_ != hipSuccess) {                                                \
+      (void)hipGetLastError();                                                 \
+      return ::fkv::fail(FKV_ERR_RUNTIME, "%s: %s", #expr,                     \
+                         hipGetErrorString(fkv_e_));                           \
+    }                                                                          \
+  } while (0)
+
+#define FKV_TRY(expr)                                                          \
+  do {                                                                         \
+    int fkv_rc_ = (expr);                                                      \
+    if (fkv_rc_ != FKV_OK)                                                     \
+      return fkv_rc_;                                                          \
+  } while (0)
+
+// ---- counters -----------------------------------------------------------
+struct Stats {
+  std::atomic<uint64_t> calls{0}, bytes_h2d{0}, bytes_d2h{0}, kernel_launches{0},
+      dma_copies{0}, staging_bytes_device{0}, staging_bytes_host{0};
+};
+Stats &stats();
+
+void set_last_path(int path);
+
+// Makes `device` current for the lifetime of the object (no-op for -1) and
+// restores the previous device afterwards.
+class DeviceGuard {
+public:
+  explicit DeviceGuard(int device);
+  ~DeviceGuard();
+  int device() const { return device_; }
+  bool ok() const { return ok_; }
+
+private:
+  int prev_ = -1;
+  int device_ = -1;
+  bool switched_ = false;
+  bool ok_ = true;
+};
+
+// ---- GPU chunk addressing ----------------------------------------------
+// Device address of chunk (layer, kv, block) before the in-chunk offset.
+// Restates ptr_at<> of the reference (csrc/gtensor_handler.cuh:43-67) in bytes.
+inline uint64_t gpu_chunk_addr(int backend, const uint64_t *ptrs,
+                               int64_t num_layers_total, int64_t kv_stride,
+                               int64_t block_stride, int64_t layer_stride,
+                               int64_t layer, int64_t kv, int64_t block) {
+  switch (backend) {
+  case FKV_BACKEND_VLLM:
+    return ptrs[layer] + (uint64_t)(kv * kv_stride) + (uint64_t)(block * block_stride);
+  case FKV_BACKEND_TRTLLM:
+    return ptrs[0] + (uint64_t)(block * block_stride) +
+           (uint64_t)(layer * layer_stride) + (uint64_t)(kv * kv_stride);
+  default: // FKV_BACKEND_SGLANG
+    return ptrs[kv * num_layers_total + layer] + (uint64_t)(block * block_stride);
+  }
+}
+inline uint64_t gpu_chunk_addr(const fkv_transfer_desc &d, int64_t layer, int64_t kv,
+                               int64_t block) {
+  return gpu_chunk_addr(d.backend, d.gpu_tensor_ptrs, d.num_layers_total,
+                        d.gpu_kv_stride, d.gpu_block_stride, d.gpu_layer_stride, layer,
+                        kv, block) +
+         (uint64_t)d.gpu_startoff_inside_chunks;
+}
+// Host address of chunk (layer, kv, block) including the in-chunk offset
+// (csrc/transfer.cu:124-130).
+inline uint8_t *cpu_chunk_ptr(const fkv_transfer_desc &d, int64_t layer, int64_t kv,
+                              int64_t block) {
+  return static_cast<uint8_t *>(d.cpu_ptr) + layer * d.cpu_layer_stride +
+         kv * d.cpu_kv_stride + block * d.cpu_block_stride +
+         d.cpu_startoff_inside_chunks;
+}
+
+// ---- the gather/scatter kernel -----------------------------------------
+// One launch copies `num_blocks * lk` chunks of `chunk_bytes`:
+//   for pos, i:  src = base_src[i] + ids_src[pos]*stride_src
+//                dst = base_dst[i] + ids_dst[pos]*stride_dst
+// (ids == nullptr means ids[pos] == pos).  All four arrays live in memory the
+// device can read.  `lk` = layers-in-call * kv_dim.
+struct CopyKernelArgs {
+  const uint64_t *base_src;
+  const uint64_t *base_dst;
+  const int64_t *ids_src;
+  const int64_t *ids_dst;
+  int64_t stride_src;
+  int64_t stride_dst;
+  int64_t chunk_bytes;
+  int32_t num_blocks;
+  int32_t lk;
+  int32_t slices_per_chunk;
+  int32_t vec; // 16, 8, 4, 2 or 1: widest access all addresses allow
+};
+constexpr int kCopyBlockThreads = 1024;  // 16 wavefronts, one CU
+constexpr int kCopyUnroll = 8;           // vector accesses in flight per lane
+constexpr int kCopyMaxLK = 1024;         // base-table entries staged in LDS
+constexpr int kCopyIdTile = 1024;        // block positions staged in LDS at a time
+int launch_copy_kernel(CopyKernelArgs args, int num_workgroups, hipStream_t stream);
+// Widest vector width (bytes) that divides every value in `vals`.
+int common_vector_width(const uint64_t *vals, int n);
+
+// ---- plan memory ---------------------------------------------------------
+// A plan is the small table (base addresses + block ids) one launch reads.
+// Slots are pinned host buffers with a device mirror, recycled once the event
+// recorded behind their last user has completed.
+struct PlanSlot;
+// Returns nullptr (and sets the error) on allocation failure.
+PlanSlot *plan_acquire(int device, size_t bytes);
+uint8_t *plan_host(PlanSlot *s);
+// Publishes the first `bytes` of the slot to the device on `stream` and returns
+// the address kernels must use (the device mirror, or the pinned buffer itself
+// when `mirror` is false).
+int plan_publish(PlanSlot *s, size_t bytes, bool mirror, hipStream_t stream,
+                 uint8_t **device_visible);
+// `drained`: the stream has been synchronised, the slot is reusable at once.
+void plan_release(PlanSlot *s, hipStream_t stream, bool drained);
+
+// ---- paths ----------------------------------------------------------------
+int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream);
+int run_ce_path(const fkv_transfer_desc &d, hipStream_t stream);
+// Device-side compaction between the engine's KV tensors and a packed device
+// buffer; see fkv_ce.cpp.
+int device_staging_copy(const fkv_transfer_desc &d, int it0, int nit, int p0, int np,
+                        uint8_t *staging, bool blockfirst, bool to_staging,
+                        hipStream_t stream);
+
+int default_num_cta(bool is_h2d);
+
+} // namespace fkv

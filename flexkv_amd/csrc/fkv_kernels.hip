@@ -1,0 +1,185 @@
+// Gather/scatter kernel of the GPU<->CPU KV-block transfer path (gfx950).
+//
+// Replaces transfer_kv_blocks_kernel / transfer_kv_blocks_kernel_8b of the
+// reference (csrc/transfer.cu:45-158) and the ATen index_select / index_copy_
+// device kernels its copy-engine strategies call (csrc/ce_transfer.cu:1051,
+// 1135, 1257-1259, 1389-1391).  One kernel serves all of them: it copies
+// num_blocks * lk chunks, where both endpoints of chunk (pos, i) are
+//     base[i] + ids[pos] * stride.
+// The host resolves the engine-specific addressing (vLLM / TRT-LLM / SGLang)
+// into the two `base` tables, so the device code has no per-engine variant.
+//
+// Work decomposition.  A chunk is cut into slices of 64 lanes x kCopyUnroll
+// vector accesses (8 KiB for 16-byte vectors).  Slices are numbered
+// position-major, then (layer, kv), then slice-in-chunk: that is ascending
+// address order inside a block-first host block.  Each workgroup owns one
+// contiguous run of slice numbers, hence a contiguous run of block positions
+// whose ids it stages in LDS (premultiplied by the block strides) together
+// with the two base tables; its 16 wavefronts take slices round-robin, so the
+// requests a workgroup has in flight target neighbouring addresses.  A
+// wavefront issues all kCopyUnroll loads of a slice before the first store, which
+// is what keeps enough reads outstanding to cover the host-link latency in
+// the host->GPU direction.
+//
+// Data moves as raw integer vectors with nontemporal loads and stores: KV
+// bytes are not reused by this kernel, and integer types cannot canonicalise
+// NaN payloads of fp8/bf16 data.
+#include "fkv_internal.h"
+
+namespace fkv {
+namespace {
+
+constexpr int kWave = 64;
+
+template <int VEC> struct VecType;
+template <> struct VecType<16> { typedef unsigned int type __attribute__((ext_vector_type(4))); };
+template <> struct VecType<8>  { typedef unsigned int type __attribute__((ext_vector_type(2))); };
+template <> struct VecType<4>  { typedef unsigned int type; };
+template <> struct VecType<2>  { typedef unsigned short type; };
+template <> struct VecType<1>  { typedef unsigned char type; };
+
+template <int VEC>
+__device__ __forceinline__ void copy_slice(const uint8_t *__restrict__ src,
+                                           uint8_t *__restrict__ dst,
+                                           int64_t bytes_in_slice, int lane) {
+  using V = typename VecType<VEC>::type;
+  constexpr int64_t kSliceBytes = (int64_t)kWave * kCopyUnroll * VEC;
+  const V *__restrict__ s = reinterpret_cast<const V *>(src) + lane;
+  V *__restrict__ d = reinterpret_cast<V *>(dst) + lane;
+  if (bytes_in_slice == kSliceBytes) {
+    V r[kCopyUnroll];
+#pragma unroll
+    for (int u = 0; u < kCopyUnroll; ++u)
+      r[u] = __builtin_nontemporal_load(s + u * kWave);
+#pragma unroll
+    for (int u = 0; u < kCopyUnroll; ++u)
+      __builtin_nontemporal_store(r[u], d + u * kWave);
+  } else {
+    const int64_t nvec = bytes_in_slice / VEC;
+    for (int64_t i = lane; i < nvec; i += kWave)
+      __builtin_nontemporal_store(__builtin_nontemporal_load(s + (i - lane)),
+                                  d + (i - lane));
+  }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
+    CopyKernelArgs a) {
+  extern __shared__ uint64_t lds[];
+  uint64_t *s_base_src = lds;
+  uint64_t *s_base_dst = lds + a.lk;
+  int64_t *s_off_src = reinterpret_cast<int64_t *>(lds + 2 * a.lk);
+  int64_t *s_off_dst = s_off_src + kCopyIdTile;
+
+  constexpr int64_t kSliceBytes = (int64_t)kWave * kCopyUnroll * VEC;
+  const uint32_t slices = (uint32_t)a.slices_per_chunk;
+  const uint32_t spp = (uint32_t)a.lk * slices; // slices per block position
+  const uint64_t total = (uint64_t)a.num_blocks * spp;
+  const uint64_t s0 = total * blockIdx.x / gridDim.x;
+  const uint64_t s1 = total * (blockIdx.x + 1) / gridDim.x;
+  if (s0 >= s1)
+    return; // whole workgroup leaves together
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const int nwaves = blockDim.x / kWave;
+
+  for (int i = tid; i < a.lk; i += blockDim.x) {
+    s_base_src[i] = a.base_src[i];
+    s_base_dst[i] = a.base_dst[i];
+  }
+
+  const uint32_t pos_lo = (uint32_t)(s0 / spp);
+  const uint32_t pos_hi = (uint32_t)((s1 - 1) / spp);
+  for (uint32_t tile = pos_lo; tile <= pos_hi; tile += kCopyIdTile) {
+    const uint32_t n = min((uint32_t)kCopyIdTile, pos_hi - tile + 1);
+    __syncthreads(); // previous tile fully consumed; base tables visible
+    for (uint32_t i = tid; i < n; i += blockDim.x) {
+      const int64_t p = (int64_t)tile + i;
+      s_off_src[i] = (a.ids_src ? a.ids_src[p] : p) * a.stride_src;
+      s_off_dst[i] = (a.ids_dst ? a.ids_dst[p] : p) * a.stride_dst;
+    }
+    __syncthreads();
+    const uint64_t tile_s0 = (uint64_t)tile * spp;
+    const uint64_t t0 = s0 > tile_s0 ? s0 : tile_s0;
+    const uint64_t tile_s1 = tile_s0 + (uint64_t)n * spp;
+    const uint64_t t1 = s1 < tile_s1 ? s1 : tile_s1;
+    for (uint64_t s = t0 + wave; s < t1; s += nwaves) {
+      const uint32_t rel = (uint32_t)(s - tile_s0); // < kCopyIdTile * spp, checked on host
+      const uint32_t p = rel / spp;
+      const uint32_t r = rel - p * spp;
+      const uint32_t i = r / slices;
+      const uint32_t sl = r - i * slices;
+      const int64_t off = (int64_t)sl * kSliceBytes;
+      const int64_t left = a.chunk_bytes - off;
+      const uint8_t *src =
+          reinterpret_cast<const uint8_t *>(s_base_src[i] + (uint64_t)s_off_src[p]) + off;
+      uint8_t *dst = reinterpret_cast<uint8_t *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + off;
+      copy_slice<VEC>(src, dst, left < kSliceBytes ? left : kSliceBytes, lane);
+    }
+  }
+}
+
+template <int VEC>
+int launch_vec(const CopyKernelArgs &a, int grid, size_t lds_bytes, hipStream_t stream) {
+  hipLaunchKernelGGL(fkv_copy_chunks_kernel<VEC>, dim3(grid), dim3(kCopyBlockThreads),
+                     lds_bytes, stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return fail(FKV_ERR_RUNTIME, "copy kernel launch failed: %s", hipGetErrorString(e));
+  return FKV_OK;
+}
+
+} // namespace
+
+int common_vector_width(const uint64_t *vals, int n) {
+  uint64_t acc = 0;
+  for (int i = 0; i < n; ++i)
+    acc |= vals[i];
+  for (int v = 16; v > 1; v >>= 1)
+    if ((acc & (uint64_t)(v - 1)) == 0)
+      return v;
+  return 1;
+}
+
+int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, hipStream_t stream) {
+  if (a.num_blocks <= 0 || a.lk <= 0 || a.chunk_bytes <= 0)
+    return FKV_OK;
+  if (a.lk > kCopyMaxLK)
+    return fail(FKV_ERR_RUNTIME, "copy kernel: %d (layer,kv) pairs exceed the LDS table (%d)",
+                a.lk, kCopyMaxLK);
+  if (a.vec != 16 && a.vec != 8 && a.vec != 4 && a.vec != 2 && a.vec != 1)
+    return fail(FKV_ERR_RUNTIME, "copy kernel: bad vector width %d", a.vec);
+  if (a.chunk_bytes % a.vec)
+    return fail(FKV_ERR_RUNTIME, "copy kernel: chunk %lld not a multiple of vector width %d",
+                (long long)a.chunk_bytes, a.vec);
+  const int64_t slice_bytes = (int64_t)kWave * kCopyUnroll * a.vec;
+  const int64_t slices = (a.chunk_bytes + slice_bytes - 1) / slice_bytes;
+  const int64_t spp = slices * a.lk;
+  // The kernel indexes slices inside an id tile with 32 bits.
+  if (slices > INT32_MAX || spp * kCopyIdTile > (int64_t)UINT32_MAX)
+    return fail(FKV_ERR_RUNTIME,
+                "copy kernel: chunk of %lld B x %d (layer,kv) pairs is too large for one launch",
+                (long long)a.chunk_bytes, a.lk);
+  a.slices_per_chunk = (int32_t)slices;
+  const int64_t total = spp * a.num_blocks;
+  const int waves_per_wg = kCopyBlockThreads / kWave;
+  int64_t grid = num_workgroups > 0 ? num_workgroups : 1;
+  const int64_t useful = (total + waves_per_wg - 1) / waves_per_wg;
+  if (grid > useful)
+    grid = useful;
+  if (grid < 1)
+    grid = 1;
+  const size_t lds_bytes = (size_t)(2 * a.lk + 2 * kCopyIdTile) * sizeof(uint64_t);
+  stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);
+  switch (a.vec) {
+  case 16: return launch_vec<16>(a, (int)grid, lds_bytes, stream);
+  case 8:  return launch_vec<8>(a, (int)grid, lds_bytes, stream);
+  case 4:  return launch_vec<4>(a, (int)grid, lds_bytes, stream);
+  case 2:  return launch_vec<2>(a, (int)grid, lds_bytes, stream);
+  default: return launch_vec<1>(a, (int)grid, lds_bytes, stream);
+  }
+}
+
+} // namespace fkv

@@ -1,0 +1,325 @@
+/*
+ * fkv_transfer.h — C ABI of libfkv_hip.so: GPU<->CPU KV-cache block transfer for
+ * AMD Instinct MI355X (gfx950).
+ *
+ * Every entry point is `extern "C"`, takes plain pointers / integers only and
+ * returns an int status (FKV_OK == 0).  On failure the text of the error is kept
+ * per calling thread and returned by fkv_last_error().  No C++ exception and no
+ * torch type crosses this boundary.
+ *
+ * The functions replace, one for one, the hot-path part of FlexKV's pybind
+ * module `flexkv.c_ext`.  Each declaration cites the reference interface it
+ * stands in for (paths relative to the FlexKV source tree).
+ *
+ * Conventions
+ *   - all strides, offsets and sizes are BYTES (the reference converts bytes to
+ *     int64 units internally, csrc/transfer.cu:179-187; here bytes are kept);
+ *   - a "chunk" is the contiguous byte run of one (layer, k-or-v, block);
+ *   - `gpu_tensor_ptrs` is a HOST array of device addresses (the reference
+ *     keeps the same table in pinned memory and lets the kernel dereference it,
+ *     csrc/gtensor_handler.cuh:47; here the host resolves it per call);
+ *   - block-id arrays are HOST arrays of int64 and need not be pinned: they are
+ *     copied into library-owned, device-visible plan memory before the call
+ *     returns, so the caller may free them immediately, also when sync == 0;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ */
+#ifndef FKV_TRANSFER_H
+#define FKV_TRANSFER_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FKV_ABI_VERSION 1
+
+/* status codes */
+#define FKV_OK 0
+#define FKV_ERR_INVALID_ARG 1 /* maps to ValueError / std::invalid_argument */
+#define FKV_ERR_RUNTIME 2     /* HIP failure or internal error -> RuntimeError */
+#define FKV_ERR_UNSUPPORTED 3 /* feature outside this library -> RuntimeError */
+
+/* GPU tensor addressing, csrc/gtensor_handler.cuh:8 (enum BackendType) and
+ * csrc/bindings.cpp:85-94 (gpu_block_type 0/1/2). */
+#define FKV_BACKEND_VLLM 0   /* one tensor per layer:  ptrs[l] + kv*Ks + b*Bs          */
+#define FKV_BACKEND_TRTLLM 1 /* one tensor in all:     ptrs[0] + b*Bs + l*Ls + kv*Ks   */
+#define FKV_BACKEND_SGLANG 2 /* K then V per layer:    ptrs[kv*Ltot + l] + b*Bs        */
+
+/* Copy-engine strategies, csrc/ce_transfer.h:42-49 (enum CEPath). */
+#define FKV_CE_PER_BLOCK (-1)
+#define FKV_CE_CONTIG_DIRECT 0
+#define FKV_CE_SEGMENT_DIRECT 1
+#define FKV_CE_SEGMENT_SCATTER 2
+#define FKV_CE_GATHER_SCATTER 3
+#define FKV_CE_GATHER_DIRECT 4
+/* value reported by fkv_last_path() when the gather/scatter kernel ran */
+#define FKV_PATH_KERNEL 100
+
+/* csrc/ce_transfer.h:18-41 (struct CETransferConfig), same defaults when
+ * zero-initialised fields are filled by fkv_ce_config_default(). */
+typedef struct fkv_ce_config {
+  int64_t segment_threshold; /* 8 */
+  int32_t path_opt_enabled;  /* 1: adaptive strategies, 0: PER_BLOCK */
+  int32_t force_path;        /* -1 auto, 0..4 force */
+  int32_t enable_memcpy2d;   /* 0 */
+  int32_t is_blockfirst;     /* host layout is [block, layer, kv, chunk] */
+  int32_t num_kv_heads;      /* 1 = KV identical on all TP ranks (MLA) */
+  int32_t gather_threads;    /* 4; host scatter/gather worker threads, 0 = caller only */
+  int32_t gather_nt;         /* 1; streaming stores in the host scatter/gather */
+  int32_t reserved;
+} fkv_ce_config;
+
+void fkv_ce_config_default(fkv_ce_config *cfg);
+
+/* One transfer.  Replaces flexkv::transfer_kv_blocks<Type>()
+ * (csrc/transfer.cuh:27-37, csrc/transfer.cu:164-313) together with the
+ * GTensorHandler it receives (csrc/gtensor_handler.cuh:11-33). */
+typedef struct fkv_transfer_desc {
+  /* GPU side */
+  int32_t backend;              /* FKV_BACKEND_* */
+  int32_t num_layers_total;     /* GTensorHandler::num_layers (SGLang ptr index) */
+  const uint64_t *gpu_tensor_ptrs; /* host array of device addresses */
+  int32_t num_gpu_tensor_ptrs;  /* entries in gpu_tensor_ptrs (bounds check) */
+  int32_t device;               /* HIP device ordinal of the GPU tensors, -1 = current */
+  int64_t gpu_kv_stride;
+  int64_t gpu_block_stride;
+  int64_t gpu_layer_stride;
+  int64_t gpu_startoff_inside_chunks;
+  /* host side */
+  void *cpu_ptr;
+  int64_t cpu_kv_stride;
+  int64_t cpu_layer_stride;
+  int64_t cpu_block_stride;
+  int64_t cpu_startoff_inside_chunks;
+  /* what to move */
+  int64_t chunk_size;
+  int32_t start_layer_id;
+  int32_t num_layers;
+  int32_t kv_dim;
+  int32_t num_blocks;
+  const int64_t *gpu_block_ids; /* host, num_blocks entries */
+  const int64_t *cpu_block_ids; /* host, num_blocks entries */
+  /* how */
+  int32_t is_host_to_device;
+  int32_t use_ce_transfer;
+  int32_t transfer_num_cta; /* workgroups of 1024 lanes; <= 0 = library default */
+  int32_t sync;             /* 1: hipStreamSynchronize before returning */
+  int32_t enable_trace;     /* 1: print an "[XFER]" line per call to stderr */
+  int32_t reserved;
+  fkv_ce_config ce;
+} fkv_transfer_desc;
+
+/* csrc/bindings.cpp:54-151, 439-459 (`c_ext.transfer_kv_blocks`) and every
+ * internal call of flexkv::transfer_kv_blocks<Type>. */
+int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream);
+
+/* Thread-local text of the last failure on this thread ("" if none).
+ * Stands in for the C++ exceptions of csrc/bindings.cpp:91-94, 147-150. */
+const char *fkv_last_error(void);
+int fkv_abi_version(void);
+
+/* Path taken by the last fkv_transfer_kv_blocks on this thread:
+ * FKV_PATH_KERNEL or one of FKV_CE_*.  The reference cannot report this
+ * (tests/test_kv_transfer_correctness.py:1697-1705 wishes it could). */
+int fkv_last_path(void);
+
+/* ---- copy-engine analysis (pure host functions, usable without a GPU) ---- */
+
+/* csrc/ce_transfer.h:53-65 */
+typedef struct fkv_ce_segment {
+  int32_t start_k;
+  int32_t nr_blocks;
+} fkv_ce_segment;
+
+typedef struct fkv_ce_analysis {
+  int32_t gpu_log_contig;
+  int32_t cpu_log_contig;
+  int32_t cpu_phys_contig;
+  int32_t gpu_phys_contig;
+  int32_t num_segments;
+  int32_t reserved;
+} fkv_ce_analysis;
+
+/* csrc/ce_transfer.cu:37-66 (analyze_ce_transfer).  `segments` may be NULL;
+ * otherwise at most `segment_capacity` entries are written.  */
+int fkv_ce_analyze(const int64_t *gpu_block_ids, const int64_t *cpu_block_ids,
+                   int32_t num_blocks, int64_t cpu_block_stride,
+                   int64_t chunk_size, int64_t gpu_block_stride,
+                   fkv_ce_analysis *out, fkv_ce_segment *segments,
+                   int32_t segment_capacity);
+
+/* csrc/ce_transfer.cu:71-104 (choose_path).  Returns an FKV_CE_* value. */
+int fkv_ce_choose_path(const fkv_ce_analysis *analysis, const fkv_ce_config *cfg,
+                       int64_t chunk_size, int32_t is_host_to_device,
+                       int32_t is_full_block);
+
+/* ---- per-rank placement for tensor-parallel groups (pure host function) ---- */
+
+typedef struct fkv_tp_rank_plan {
+  int32_t active;          /* 0: this rank moves nothing in this call */
+  int32_t start_layer;
+  int32_t num_layers;
+  int32_t reserved;
+  int64_t cpu_startoff;
+  int64_t gpu_startoff;
+  int64_t chunk_size;
+} fkv_tp_rank_plan;
+
+/* csrc/tp_transfer_thread_group.cpp:222-323 (offset / layer-range rules of
+ * tp_group_transfer).  `mode` is the kv_shared_across_ranks_mode string;
+ * `rotate_counter` is the value of the round-robin counter for rank_rotate.
+ * Returns FKV_ERR_INVALID_ARG for the sharded/indivisible case (:237-247). */
+int fkv_tp_rank_plan_compute(int32_t rank, int32_t num_gpus, int32_t num_kv_heads,
+                             int32_t is_host_to_device, const char *mode,
+                             int32_t designated_rank, int32_t rotate_counter,
+                             int32_t layer_id, int32_t layer_granularity,
+                             int32_t num_blocks, int64_t gpu_chunk_size,
+                             int64_t cpu_block_stride, int64_t cpu_tp_stride,
+                             fkv_tp_rank_plan *out);
+
+/* ---- TPTransferThreadGroup: csrc/tp_transfer_thread_group.h:42-133,
+ *      csrc/bindings.cpp:761-830 ---- */
+
+typedef struct fkv_tp_group fkv_tp_group;
+
+typedef struct fkv_tp_group_params {
+  int32_t num_gpus;
+  int32_t num_tensors_per_gpu;
+  const uint64_t *gpu_block_ptrs_flat; /* num_gpus * num_tensors_per_gpu */
+  void *cpu_blocks_ptr;
+  int32_t num_layers;
+  int32_t reserved;
+  const int64_t *gpu_kv_strides;    /* num_gpus entries each */
+  const int64_t *gpu_block_strides;
+  const int64_t *gpu_layer_strides;
+  const int64_t *gpu_chunk_sizes;
+  const int64_t *gpu_device_ids;
+  fkv_ce_config ce;
+} fkv_tp_group_params;
+
+/* ctor, csrc/tp_transfer_thread_group.cpp:30-138 */
+int fkv_tp_group_create(const fkv_tp_group_params *params, fkv_tp_group **out);
+/* csrc/tp_transfer_thread_group.cpp:140-162 */
+int fkv_tp_group_update_gpu_block_ptrs(fkv_tp_group *g, const uint64_t *ptrs_flat,
+                                       int64_t count);
+/* csrc/tp_transfer_thread_group.cpp:199-381 */
+int fkv_tp_group_transfer(fkv_tp_group *g, const int64_t *gpu_block_ids,
+                          const int64_t *cpu_block_ids, int32_t num_blocks,
+                          int64_t cpu_kv_stride, int64_t cpu_layer_stride,
+                          int64_t cpu_block_stride, int64_t cpu_tp_stride,
+                          int32_t transfer_num_cta, int32_t is_host_to_device,
+                          int32_t use_ce_transfer, int32_t layer_id,
+                          int32_t layer_granularity, int32_t kv_dim,
+                          int32_t num_kv_heads, const char *mode,
+                          int32_t designated_rank);
+/* dtor, csrc/tp_transfer_thread_group.cpp:164-185 */
+void fkv_tp_group_destroy(fkv_tp_group *g);
+
+/* ---- LayerwiseTransferGroup (single group, main KV):
+ *      csrc/layerwise.h:59-362, csrc/bindings.cpp:471-545, 657-691 ---- */
+
+typedef struct fkv_layerwise fkv_layerwise;
+
+typedef struct fkv_layerwise_params {
+  int32_t num_gpus;
+  int32_t num_tensors_per_gpu;
+  const uint64_t *gpu_block_ptrs_flat; /* num_gpus * num_tensors_per_gpu */
+  void *cpu_blocks_ptr;
+  int32_t num_layers;
+  int32_t tp_size;
+  const int64_t *gpu_kv_strides; /* num_gpus entries each */
+  const int64_t *gpu_block_strides;
+  const int64_t *gpu_layer_strides;
+  const int64_t *gpu_chunk_sizes;
+  const int64_t *gpu_device_ids;
+  const int32_t *layer_eventfds; /* [num_counters, tp_size, num_layers] or NULL */
+  int32_t num_layer_eventfds;    /* total entries, 0 = eventfd notification off */
+  int32_t reserved;
+  fkv_ce_config ce;
+} fkv_layerwise_params;
+
+#define FKV_NOTIFY_HOSTFUNC 0
+#define FKV_NOTIFY_POLLING 1
+
+/* ctor, csrc/layerwise.cpp:507-646 (SSD and SWA arguments are outside this
+ * library; the Python shim rejects non-empty ones). */
+int fkv_layerwise_create(const fkv_layerwise_params *params, fkv_layerwise **out);
+
+/* csrc/layerwise.cpp:944-1311, host->GPU restore in batches of
+ * `layer_granularity` layers.  HOSTFUNC returns after every stream has
+ * drained (:1249-1256); POLLING returns right after the launches (:1240-1247).
+ * `mode` is kv_shared_across_ranks_mode (:1112-1166). */
+int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
+                           const int64_t *cpu_block_ids, int32_t num_blocks,
+                           int64_t cpu_block_stride, int64_t h2d_cpu_kv_stride,
+                           int64_t h2d_cpu_layer_stride, int64_t cpu_tp_stride,
+                           int32_t transfer_cta_num, int32_t use_ce_transfer,
+                           int32_t num_layers, int32_t layer_granularity,
+                           int32_t kv_dim, int32_t num_kv_heads, int32_t counter_id,
+                           const char *mode, int32_t notify_mode,
+                           int32_t enable_trace);
+
+/* Make `consumer_stream` (a hipStream_t on GPU `gpu_index` of the group) wait
+ * until `layer` of the most recent fkv_layerwise_transfer has landed.  This is
+ * the in-process counterpart of the eventfd a consumer in another process
+ * blocks on (flexkv/integration/sglang/comm.py:705-744); the reference has no
+ * such call. */
+int fkv_layerwise_wait_layer(fkv_layerwise *g, int32_t gpu_index, int32_t layer,
+                             void *consumer_stream);
+/* Block the host until the most recent transfer has finished on all GPUs and
+ * every notification has been written. */
+int fkv_layerwise_synchronize(fkv_layerwise *g);
+/* Milliseconds between the start of the most recent transfer and the
+ * completion of each layer batch, as seen by the transfer stream of GPU 0.
+ * Writes min(capacity, num_batches) values and returns the count via
+ * `num_batches`. Valid after fkv_layerwise_synchronize. */
+int fkv_layerwise_batch_times_ms(fkv_layerwise *g, float *out_ms, int32_t capacity,
+                                 int32_t *num_batches);
+/* dtor, csrc/layerwise.cpp:840-905 */
+void fkv_layerwise_destroy(fkv_layerwise *g);
+
+/* ---- host memory: flexkv/transfer/host_buffer.py:66-118, 180-202 ---- */
+
+/* hipHostMalloc(Portable|Mapped) — alloc_mapped_host_tensor (:180-202). */
+int fkv_host_alloc(size_t bytes, void **out);
+int fkv_host_free(void *ptr);
+/* Chunked hipHostRegister(Portable|Mapped) with rollback on failure —
+ * cudaHostRegister (:66-98).  chunk_bytes == 0 registers in one call. */
+int fkv_host_register(void *ptr, size_t bytes, size_t chunk_bytes);
+/* Reverse of fkv_host_register with the same chunking (:101-118). */
+int fkv_host_unregister(void *ptr, size_t bytes, size_t chunk_bytes);
+/* The (offset, size) pieces fkv_host_register would issue; pure arithmetic.
+ * Returns the number of pieces (also when it exceeds `capacity`). */
+int64_t fkv_host_register_plan(size_t bytes, size_t chunk_bytes, size_t *offsets,
+                               size_t *sizes, int64_t capacity);
+/* FLEXKV_CUDAHOST_CHUNK_SIZE_GB -> chunk bytes, host_buffer.py:57-63. */
+size_t fkv_host_chunk_bytes_from_gb(double chunk_gb);
+
+/* ---- counters (the reference's FLEXKV_GPU_CPU_TRANSFER metric hook is a
+ *      no-op unless monitoring is compiled in, csrc/ce_transfer.cu:29-31) ---- */
+typedef struct fkv_stats {
+  uint64_t calls;
+  uint64_t bytes_h2d;
+  uint64_t bytes_d2h;
+  uint64_t kernel_launches;
+  uint64_t dma_copies;
+  uint64_t staging_bytes_device;
+  uint64_t staging_bytes_host;
+  uint64_t reserved;
+} fkv_stats;
+void fkv_get_stats(fkv_stats *out);
+void fkv_reset_stats(void);
+
+/* Host-link reference rate: `reps` plain hipMemcpyAsync copies of `bytes`
+ * between a pinned host buffer and a device buffer (both owned by the call),
+ * timed with hip events.  direction: 0 = D2H, 1 = H2D.  Result in GB/s
+ * (1e9 B/s) of the best repetition.  No counterpart in the reference. */
+int fkv_measure_link_peak(int32_t device, size_t bytes, int32_t reps,
+                          int32_t direction, double *best_gbps, double *median_gbps);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FKV_TRANSFER_H */

@@ -1,0 +1,244 @@
+"""Python side of the CPU oracle.  TEST INFRASTRUCTURE ONLY.
+
+Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` may import this module; the shipped package never does.
+
+Three things live here:
+
+* a ctypes loader for ``libfkv_oracle.so`` (the C restatement in
+  ``fkv_oracle.c``) with thin numpy wrappers;
+* an independent *index* formulation of the same transfer,
+  ``host.view(N, L, kv, chunk)[cpu_ids, l, kv] = gpu(l, kv)[gpu_ids]`` written
+  with numpy strided views and fancy indexing.  It is the row gather/scatter
+  the reference's own copy-engine path performs with ATen ``index_select`` /
+  ``index_copy_`` (csrc/ce_transfer.cu:1051, 1135);
+* ``torch_index_gather`` / ``torch_index_scatter``: the "reference CPU path"
+  (torch index-gather of the selected blocks into the host cache layout) that
+  the benchmark times as its CPU baseline.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from typing import List, Optional, Sequence
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libfkv_oracle.so")
+_lib: Optional[ctypes.CDLL] = None
+
+BACKEND_VLLM, BACKEND_TRTLLM, BACKEND_SGLANG = 0, 1, 2
+CE_NAMES = {-1: "PER_BLOCK", 0: "CONTIG_DIRECT", 1: "SEGMENT_DIRECT",
+            2: "SEGMENT_SCATTER", 3: "GATHER_SCATTER", 4: "GATHER_DIRECT"}
+
+
+def build(force: bool = False) -> str:
+    """Compile fkv_oracle.c with gcc into libfkv_oracle.so next to it."""
+    src = os.path.join(_HERE, "fkv_oracle.c")
+    if force or not os.path.exists(_LIB_PATH) or \
+            os.path.getmtime(_LIB_PATH) < os.path.getmtime(src):
+        subprocess.check_call(
+            ["gcc", "-O2", "-std=c11", "-Wall", "-Wextra", "-fPIC", "-shared",
+             "-o", _LIB_PATH, src])
+    return _LIB_PATH
+
+
+class Analysis(ctypes.Structure):
+    _fields_ = [("gpu_log_contig", ctypes.c_int32),
+                ("cpu_log_contig", ctypes.c_int32),
+                ("cpu_phys_contig", ctypes.c_int32),
+                ("gpu_phys_contig", ctypes.c_int32),
+                ("num_segments", ctypes.c_int32),
+                ("reserved", ctypes.c_int32)]
+
+
+class Segment(ctypes.Structure):
+    _fields_ = [("start_k", ctypes.c_int32), ("nr_blocks", ctypes.c_int32)]
+
+
+class RankPlan(ctypes.Structure):
+    _fields_ = [("active", ctypes.c_int32), ("start_layer", ctypes.c_int32),
+                ("num_layers", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("cpu_startoff", ctypes.c_int64), ("gpu_startoff", ctypes.c_int64),
+                ("chunk_size", ctypes.c_int64)]
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        i64, i32, u64, vp = ctypes.c_int64, ctypes.c_int, ctypes.c_uint64, ctypes.c_void_p
+        L.fkv_oracle_units_ok.argtypes = [i64] * 9
+        L.fkv_oracle_units_ok.restype = i32
+        L.fkv_oracle_chunk_addr.argtypes = [i32, vp, i64, i64, i64, i64, i64, i64, i64]
+        L.fkv_oracle_chunk_addr.restype = u64
+        L.fkv_oracle_transfer.argtypes = [
+            i32, vp, i64, i64, i64, i64, i64, vp, i64, i64, i64, i64, i64,
+            i32, i32, i32, i32, vp, vp, i32]
+        L.fkv_oracle_transfer.restype = i32
+        L.fkv_oracle_ce_analyze.argtypes = [vp, vp, i32, i64, i64, i64,
+                                            ctypes.POINTER(Analysis), vp, i32]
+        L.fkv_oracle_ce_analyze.restype = None
+        L.fkv_oracle_ce_choose_path.argtypes = [ctypes.POINTER(Analysis), i32, i32,
+                                                i64, i64, i32, i32]
+        L.fkv_oracle_ce_choose_path.restype = i32
+        L.fkv_oracle_is_full_block.argtypes = [i32, i32, i64, i64]
+        L.fkv_oracle_is_full_block.restype = i32
+        L.fkv_oracle_tp_rank_plan.argtypes = [
+            i32, i32, i32, i32, ctypes.c_char_p, i32, i32, i32, i32, i32,
+            i64, i64, i64, ctypes.POINTER(RankPlan)]
+        L.fkv_oracle_tp_rank_plan.restype = i32
+        L.fkv_oracle_layerwise_cpu_startoff.argtypes = [i32, i32, ctypes.c_char_p,
+                                                        i32, i64, i64]
+        L.fkv_oracle_layerwise_cpu_startoff.restype = i64
+        L.fkv_oracle_host_scatter.argtypes = [vp, vp, vp, i32, i64, i64, i64, i32,
+                                              i32, i64, i64, i32]
+        L.fkv_oracle_host_scatter.restype = None
+        L.fkv_oracle_eventfd_index.argtypes = [i32] * 5
+        L.fkv_oracle_eventfd_index.restype = i64
+        L.fkv_oracle_host_chunk_bytes.argtypes = [ctypes.c_double]
+        L.fkv_oracle_host_chunk_bytes.restype = u64
+        _lib = L
+    return _lib
+
+
+def _i64(a) -> np.ndarray:
+    return np.ascontiguousarray(np.asarray(a, dtype=np.int64))
+
+
+def _ptr(a: np.ndarray) -> int:
+    return a.ctypes.data
+
+
+def transfer_c(backend: int, tensor_ptrs: Sequence[int], num_layers_total: int,
+               gpu_kv_stride: int, gpu_block_stride: int, gpu_layer_stride: int,
+               gpu_off: int, cpu_ptr: int, cpu_kv_stride: int, cpu_layer_stride: int,
+               cpu_block_stride: int, cpu_off: int, chunk: int, start_layer: int,
+               num_layers: int, kv_dim: int, gpu_ids, cpu_ids,
+               is_host_to_device: bool) -> None:
+    """Run the C restatement.  All pointers are HOST addresses (ints)."""
+    ptrs = np.ascontiguousarray(np.asarray(tensor_ptrs, dtype=np.uint64))
+    g = _i64(gpu_ids)
+    c = _i64(cpu_ids)
+    assert g.shape == c.shape
+    rc = lib().fkv_oracle_transfer(
+        backend, _ptr(ptrs), num_layers_total, gpu_kv_stride, gpu_block_stride,
+        gpu_layer_stride, gpu_off, cpu_ptr, cpu_kv_stride, cpu_layer_stride,
+        cpu_block_stride, cpu_off, chunk, start_layer, num_layers, kv_dim,
+        int(g.size), _ptr(g), _ptr(c), int(bool(is_host_to_device)))
+    if rc != 0:
+        raise ValueError(f"oracle transfer rejected backend {backend}")
+
+
+def chunk_addr(backend, tensor_ptrs, num_layers_total, kvs, bs, ls, layer, kv, block) -> int:
+    ptrs = np.ascontiguousarray(np.asarray(tensor_ptrs, dtype=np.uint64))
+    return int(lib().fkv_oracle_chunk_addr(backend, _ptr(ptrs), num_layers_total,
+                                           kvs, bs, ls, layer, kv, block))
+
+
+def ce_analyze(gpu_ids, cpu_ids, cpu_block_stride, chunk, gpu_block_stride):
+    g, c = _i64(gpu_ids), _i64(cpu_ids)
+    n = int(g.size)
+    out = Analysis()
+    segs = (Segment * max(n, 1))()
+    lib().fkv_oracle_ce_analyze(_ptr(g), _ptr(c), n, cpu_block_stride, chunk,
+                                gpu_block_stride, ctypes.byref(out),
+                                ctypes.cast(segs, ctypes.c_void_p), max(n, 1))
+    seg_list = [(segs[i].start_k, segs[i].nr_blocks) for i in range(out.num_segments)]
+    return out, seg_list
+
+
+def ce_choose_path(analysis: Analysis, is_blockfirst: bool, num_kv_heads: int,
+                   segment_threshold: int, chunk: int, is_host_to_device: bool,
+                   is_full_block: bool) -> int:
+    return int(lib().fkv_oracle_ce_choose_path(
+        ctypes.byref(analysis), int(is_blockfirst), num_kv_heads, segment_threshold,
+        chunk, int(is_host_to_device), int(is_full_block)))
+
+
+def tp_rank_plan(rank, num_gpus, num_kv_heads, is_h2d, mode, designated_rank,
+                 rotate_counter, layer_id, layer_granularity, num_blocks,
+                 gpu_chunk_size, cpu_block_stride, cpu_tp_stride):
+    out = RankPlan()
+    rc = lib().fkv_oracle_tp_rank_plan(
+        rank, num_gpus, num_kv_heads, int(is_h2d), mode.encode(), designated_rank,
+        rotate_counter, layer_id, layer_granularity, num_blocks, gpu_chunk_size,
+        cpu_block_stride, cpu_tp_stride, ctypes.byref(out))
+    if rc != 0:
+        raise ValueError("sharded D2H needs gpu_chunk_size divisible by num_gpus")
+    return out
+
+
+# ---------------------------------------------------------------------------
+# Independent index formulation (numpy strided views + fancy indexing)
+# ---------------------------------------------------------------------------
+
+def _view(base: np.ndarray, offset: int, shape, strides) -> np.ndarray:
+    """uint8 strided view into ``base`` starting at byte ``offset``; bounds are
+    checked so a wrong stride raises instead of reading outside ``base``."""
+    last = offset + sum((s - 1) * st for s, st in zip(shape, strides) if s > 0)
+    if offset < 0 or (all(s > 0 for s in shape) and last >= base.size):
+        raise IndexError(f"strided view [{offset}, {last}] outside buffer of {base.size} B")
+    return np.lib.stride_tricks.as_strided(base[offset:], shape=shape, strides=strides)
+
+
+def transfer_index(backend: int, gpu_buffers: List[np.ndarray], num_layers_total: int,
+                   gpu_kv_stride: int, gpu_block_stride: int, gpu_layer_stride: int,
+                   gpu_off: int, host: np.ndarray, cpu_kv_stride: int,
+                   cpu_layer_stride: int, cpu_block_stride: int, cpu_off: int,
+                   chunk: int, start_layer: int, num_layers: int, kv_dim: int,
+                   gpu_ids, cpu_ids, is_host_to_device: bool) -> None:
+    """Row gather/scatter with numpy fancy indexing.
+
+    ``gpu_buffers`` are flat uint8 arrays, one per engine tensor (1 for
+    TRT-LLM, L for vLLM, 2L for SGLang); ``host`` is the flat uint8 host pool.
+    """
+    g, c = _i64(gpu_ids), _i64(cpu_ids)
+    if g.size == 0:
+        return
+    for l in range(start_layer, start_layer + num_layers):
+        for kv in range(kv_dim):
+            if backend == BACKEND_VLLM:
+                buf, off = gpu_buffers[l], kv * gpu_kv_stride
+            elif backend == BACKEND_TRTLLM:
+                buf, off = gpu_buffers[0], l * gpu_layer_stride + kv * gpu_kv_stride
+            elif backend == BACKEND_SGLANG:
+                buf, off = gpu_buffers[kv * num_layers_total + l], 0
+            else:
+                raise ValueError(backend)
+            rows_g = _view(buf, off + gpu_off, (int(g.max()) + 1, chunk),
+                           (gpu_block_stride, 1))
+            rows_c = _view(host, l * cpu_layer_stride + kv * cpu_kv_stride + cpu_off,
+                           (int(c.max()) + 1, chunk), (cpu_block_stride, 1))
+            if is_host_to_device:
+                rows_g[g] = rows_c[c]
+            else:
+                rows_c[c] = rows_g[g]
+
+
+# ---------------------------------------------------------------------------
+# "Reference CPU path": torch index-gather into the host cache layout.
+# ---------------------------------------------------------------------------
+
+def torch_index_gather(layers, host_cache, gpu_ids, cpu_ids) -> None:
+    """vLLM-shaped tensors resident in host RAM -> BLOCKFIRST host cache.
+
+    ``layers[l]`` is ``[kv, N, T, H, D]``; ``host_cache`` is
+    ``[NH, L, kv, T, H, D]``.  host_cache[cpu_ids, l] = layers[l][:, gpu_ids]
+    (block axis moved first)."""
+    import torch
+    for l, layer in enumerate(layers):
+        picked = torch.index_select(layer, 1, gpu_ids)          # [kv, n, T, H, D]
+        host_cache[:, l].index_copy_(0, cpu_ids, picked.transpose(0, 1))
+
+
+def torch_index_scatter(layers, host_cache, gpu_ids, cpu_ids) -> None:
+    """Inverse of torch_index_gather: layers[l][:, gpu_ids] = host_cache[cpu_ids, l]."""
+    import torch
+    for l, layer in enumerate(layers):
+        picked = torch.index_select(host_cache[:, l], 0, cpu_ids)  # [n, kv, T, H, D]
+        layer.index_copy_(1, gpu_ids, picked.transpose(0, 1))
