@@ -1,0 +1,540 @@
+#!/usr/bin/env python3
+"""Benchmark of the GPU<->CPU KV-block transfer path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c0..c4]
+
+A step is one pass of the hot path over one batch of block ids: a GPU->host
+gather of the selected blocks into the host cache followed by the host->GPU
+scatter of the same blocks (c0, c1, c2), one layer-by-layer restore (c3), or
+one burst of 64 concurrent requests (c4).  Inputs are resident in HBM / pinned
+host memory before the timed region starts.  One JSON line is printed.
+
+Configurations (BASELINE.json "configs"):
+  c0  Llama-3-8B, vLLM layout, bf16: 32 x [2,4096,16,8,128]; 256 random blocks
+  c1  SGLang token-major, bf16, page 64: 64 x [262144,8,128]; 1024 pages
+      (64 runs of 8 + 512 isolated)                      <- default, the metric's config
+  c2  TRT-LLM layout, fp8 e4m3: [4096,80,2,8,32,128]; 2048 random blocks
+  c3  DeepSeek-V3 MLA, bf16: 61 x [16384,64,576]; layerwise restore of 512 blocks
+  c4  64 concurrent requests on the c0 shape with a 32768-block pool
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import threading
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+METRIC = "KV block transfer GB/s (D2H, H2D) on 1 GPU; % of measured host-link peak"
+
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs of this script scaled by a plain copy kernel of known size;
+# see the summaries under profiles/.  None where no such run has been made.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def _median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+# ---------------------------------------------------------------------------
+# workloads
+# ---------------------------------------------------------------------------
+class Workload:
+    """GPU tensors, pinned host cache, ids and strides of one configuration."""
+
+    def __init__(self, name, torch, device, scale=1.0):
+        self.name, self.torch, self.device = name, torch, device
+        t = torch
+        g = lambda seed: t.Generator().manual_seed(seed)
+        if name in ("c0", "c4"):
+            L, N, T, H, D = 32, (4096 if name == "c0" else 32768), 16, 8, 128
+            self.desc = ("Llama-3-8B vLLM layout bf16: 32 x [2,%d,16,8,128], host [NH,32,2,16,8,128]"
+                         % N)
+            self.backend, self.kv_dim, self.L = 0, 2, L
+            self.chunk = T * H * D * 2
+            gen = t.Generator(device=device).manual_seed(0)
+            self.tensors = [t.randn(2, N, T, H, D, device=device, dtype=t.bfloat16, generator=gen)
+                            for _ in range(L)]
+            self.gks, self.gbs, self.gls = N * self.chunk, self.chunk, 2 * N * self.chunk
+            self.num_gpu_blocks = N
+            if name == "c0":
+                gg = g(1)
+                n = 256
+                self.NH = 1024
+                self.gpu_ids = t.randperm(N, generator=gg)[:n].to(t.int64)
+                self.cpu_ids = t.randperm(self.NH, generator=gg)[:n].to(t.int64)
+            else:
+                # 64 requests, sizes min(512, Geometric(p=1/48)), disjoint random ids
+                gg = g(5)
+                sizes = t.empty(64).geometric_(1.0 / 48, generator=gg).clamp(1, 512).to(t.int64)
+                total = int(sizes.sum())
+                self.NH = total
+                perm_g = t.randperm(N, generator=gg)[:total].to(t.int64)
+                perm_c = t.randperm(self.NH, generator=gg)[:total].to(t.int64)
+                offs = [0] + list(t.cumsum(sizes, 0).tolist())
+                self.requests = [(perm_g[offs[i]:offs[i + 1]].contiguous(),
+                                  perm_c[offs[i]:offs[i + 1]].contiguous()) for i in range(64)]
+                self.gpu_ids, self.cpu_ids = perm_g, perm_c
+        elif name == "c1":
+            L, tokens, H, D, page = 32, 262144, 8, 128, 64
+            self.desc = ("SGLang token-major bf16 page 64: 64 x [262144,8,128] (K then V, 32 layers), "
+                         "1024 pages = 64 runs of 8 + 512 isolated, host [1024,32,2,64,8,128]")
+            self.backend, self.kv_dim, self.L = 2, 2, L
+            self.chunk = page * H * D * 2
+            gen = t.Generator(device=device).manual_seed(2)
+            self.tensors = [t.randn(tokens, H, D, device=device, dtype=t.bfloat16, generator=gen)
+                            for _ in range(2 * L)]
+            N = tokens // page
+            self.num_gpu_blocks = N
+            self.gks, self.gbs, self.gls = 0, self.chunk, N * self.chunk
+            self.NH = 1024
+            self.gpu_ids = sglang_page_ids(t, N, seed=2)
+            self.cpu_ids = t.arange(self.NH, dtype=t.int64)
+        elif name == "c2":
+            N, L, H, T, D = 4096, 80, 8, 32, 128
+            self.desc = ("TRT-LLM layout fp8 e4m3: one [4096,80,2,8,32,128] tensor, 2048 random "
+                         "blocks, host [2048,80,2,8,32,128]")
+            self.backend, self.kv_dim, self.L = 1, 2, L
+            self.chunk = H * T * D
+            gen = t.Generator(device=device).manual_seed(3)
+            codes = t.randint(0, 254, (N, L, 2, H, T, D), device=device, dtype=t.uint8,
+                              generator=gen)
+            codes += (codes >= 0x7F).to(t.uint8)  # skip 0x7F; 0xFF is never produced
+            self.tensors = [codes]
+            self.num_gpu_blocks = N
+            self.gks, self.gls, self.gbs = self.chunk, 2 * self.chunk, L * 2 * self.chunk
+            self.NH = 2048
+            gg = g(3)
+            self.gpu_ids = t.randperm(N, generator=gg)[:2048].to(t.int64)
+            self.gpu_ids_reload = t.randperm(N, generator=gg)[:2048].to(t.int64)
+            self.cpu_ids = t.arange(2048, dtype=t.int64)
+        elif name == "c3":
+            L, N, T, D = 61, 16384, 64, 576
+            self.desc = ("DeepSeek-V3 MLA latent KV bf16: 61 x [16384,64,576], layerwise restore of "
+                         "512 blocks, host [512,61,1,64,1,576]")
+            self.backend, self.kv_dim, self.L = 0, 1, L
+            self.chunk = T * D * 2
+            gen = t.Generator(device=device).manual_seed(4)
+            self.tensors = [(t.randn(N, T, D, device=device, dtype=t.bfloat16, generator=gen) * 0.5)
+                            for _ in range(L)]
+            self.num_gpu_blocks = N
+            self.gks, self.gbs, self.gls = N * self.chunk, self.chunk, N * self.chunk
+            self.NH = 512
+            gg = g(4)
+            self.gpu_ids = t.randperm(N, generator=gg)[:512].to(t.int64)
+            self.cpu_ids = t.randperm(self.NH, generator=gg)[:512].to(t.int64)
+        else:
+            raise ValueError(name)
+        # host cache, block-first: [NH, L, kv, chunk]
+        self.cks = self.chunk
+        self.cls = self.kv_dim * self.chunk
+        self.cbs = self.L * self.kv_dim * self.chunk
+        self.host = t.empty(self.NH * self.cbs, dtype=t.uint8, pin_memory=True)
+        self.ptrs = t.tensor([x.data_ptr() for x in self.tensors], dtype=t.int64).pin_memory()
+        self.num_blocks = int(self.gpu_ids.numel())
+        self.bytes_per_direction = self.num_blocks * self.L * self.kv_dim * self.chunk
+
+    def transfer(self, gpu_ids, cpu_ids, h2d, **kw):
+        from flexkv_amd.c_ext import transfer_kv_blocks
+        kw.setdefault("sync", False)
+        transfer_kv_blocks(gpu_ids, self.ptrs, self.gks, self.gbs, self.gls, cpu_ids, self.host,
+                           self.cks, self.cls, self.cbs, self.chunk, 0, self.L,
+                           is_host_to_device=h2d, kv_dim=self.kv_dim, gpu_block_type=self.backend,
+                           is_blockfirst=True, **kw)
+
+    # block rows of one (layer, kv) as a [N, chunk] uint8 view of the engine tensor
+    def gpu_rows(self, layer, kv):
+        t = self.torch
+        if self.backend == 0:
+            x = self.tensors[layer]
+            x = x[kv] if self.kv_dim == 2 else x
+            return x.reshape(self.num_gpu_blocks, -1).view(t.uint8)
+        if self.backend == 2:
+            return self.tensors[kv * self.L + layer].view(self.num_gpu_blocks, -1).view(t.uint8)
+        return self.tensors[0][:, layer, kv].reshape(self.num_gpu_blocks, -1)  # strided view
+
+    def host_rows(self, layer, kv):
+        return self.host.view(self.NH, self.L, self.kv_dim, self.chunk)[:, layer, kv]
+
+    def verify_host_image(self, gpu_ids, cpu_ids):
+        """host[cpu_ids, l, kv] == engine rows [gpu_ids], compared on the GPU
+        against torch's own index_select."""
+        t = self.torch
+        gi, ci = gpu_ids.to(self.device), cpu_ids
+        for l in range(self.L):
+            for kv in range(self.kv_dim):
+                want = self.gpu_rows(l, kv).index_select(0, gi)
+                got = self.host_rows(l, kv).index_select(0, ci).to(self.device)
+                if not t.equal(want, got):
+                    return False
+        return True
+
+
+def sglang_page_ids(t, num_pages, seed, runs=64, run_len=8, isolated=512):
+    """64 non-overlapping runs of 8 consecutive pages + 512 isolated pages not
+    adjacent to any chosen page, order shuffled; everything from one generator."""
+    g = t.Generator().manual_seed(seed)
+    taken = t.zeros(num_pages + 2, dtype=t.bool)  # index shifted by one, guards at both ends
+    pieces = []
+    while len(pieces) < runs:
+        s = int(t.randint(0, num_pages - run_len + 1, (1,), generator=g))
+        if not taken[s:s + run_len + 2].any():   # the run and one page on either side are free
+            taken[s + 1:s + 1 + run_len] = True
+            pieces.append(t.arange(s, s + run_len, dtype=t.int64))
+    singles = 0
+    while singles < isolated:
+        s = int(t.randint(0, num_pages, (1,), generator=g))
+        if not taken[s:s + 3].any():
+            taken[s + 1] = True
+            pieces.append(t.tensor([s], dtype=t.int64))
+            singles += 1
+    order = t.randperm(len(pieces), generator=g).tolist()
+    return t.cat([pieces[i] for i in order]).contiguous()
+
+
+# ---------------------------------------------------------------------------
+# measurements
+# ---------------------------------------------------------------------------
+def measure_link(device_index=0, nbytes=1 << 30, reps=10):
+    from flexkv_amd import _lib
+    L = _lib.load()
+    out = {}
+    for name, direction in (("d2h", 0), ("h2d", 1)):
+        best, med = ctypes.c_double(), ctypes.c_double()
+        _lib.check(L.fkv_measure_link_peak(device_index, nbytes, reps, direction,
+                                           ctypes.byref(best), ctypes.byref(med)))
+        out[name] = best.value
+    return out
+
+
+def run_gather_scatter(w, torch, steps, warmup, num_cta, use_ce):
+    """c0 / c1 / c2: D2H gather then H2D scatter per step."""
+    st = torch.cuda.Stream()
+    kw = dict(transfer_num_cta=num_cta, use_ce_transfer=use_ce, ce_path_opt=True)
+    reload_ids = getattr(w, "gpu_ids_reload", w.gpu_ids)
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    d2h_ms, h2d_ms = [], []
+    with torch.cuda.stream(st):
+        for _ in range(warmup):
+            w.transfer(w.gpu_ids, w.cpu_ids, False, **kw)
+            w.transfer(reload_ids, w.cpu_ids, True, **kw)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        marks = []
+        for _ in range(steps):
+            a, b, c = ev(), ev(), ev()
+            a.record(st)
+            w.transfer(w.gpu_ids, w.cpu_ids, False, **kw)
+            b.record(st)
+            w.transfer(reload_ids, w.cpu_ids, True, **kw)
+            c.record(st)
+            marks.append((a, b, c))
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    for a, b, c in marks:
+        d2h_ms.append(a.elapsed_time(b))
+        h2d_ms.append(b.elapsed_time(c))
+    return wall, d2h_ms, h2d_ms
+
+
+def verify_round_trip(w, torch, num_cta):
+    """Bit-exactness at full size through size-independent properties:
+    (1) the host image equals torch's own index_select of the engine tensors;
+    (2) gather -> erase the blocks on the GPU -> scatter restores every byte."""
+    from flexkv_amd.c_ext import transfer_kv_blocks  # noqa: F401
+    w.host.zero_()
+    w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=num_cta, sync=True)
+    ok = w.verify_host_image(w.gpu_ids, w.cpu_ids)
+    gi = w.gpu_ids.to(w.device)
+    saved = [[w.gpu_rows(l, kv).index_select(0, gi) for kv in range(w.kv_dim)] for l in range(w.L)]
+    for l in range(w.L):
+        for kv in range(w.kv_dim):
+            w.gpu_rows(l, kv).index_fill_(0, gi, 0)
+    w.transfer(w.gpu_ids, w.cpu_ids, True, transfer_num_cta=num_cta, sync=True)
+    for l in range(w.L):
+        for kv in range(w.kv_dim):
+            ok = ok and torch.equal(w.gpu_rows(l, kv).index_select(0, gi), saved[l][kv])
+    return bool(ok)
+
+
+def run_layerwise(w, torch, steps, warmup, num_cta, notify):
+    """c3: per-layer restore with a dummy per-layer compute kernel on a second
+    stream gated on each layer's event."""
+    from flexkv_amd.c_ext import LayerwiseTransferGroup
+    i64 = lambda v: torch.tensor([v], dtype=torch.int64)
+    grp = LayerwiseTransferGroup(
+        num_gpus=1, gpu_blocks=[w.tensors], cpu_blocks=w.host, ssd_files={}, num_layers=w.L,
+        gpu_kv_strides_tensor=i64(w.gks), gpu_block_strides_tensor=i64(w.gbs),
+        gpu_layer_strides_tensor=i64(w.gls), gpu_chunk_sizes_tensor=i64(w.chunk),
+        iouring_entries=0, iouring_flags=0,
+        layer_eventfds_tensor=torch.empty(0, dtype=torch.int32), tp_size=1, is_blockfirst=True)
+    empty = torch.empty(0, dtype=torch.int64)
+
+    def restore():
+        grp.layerwise_transfer(
+            empty, empty, 0, 0, 0, 0, 0, w.gpu_ids, w.cpu_ids, w.cks, w.cls, w.cbs, w.chunk,
+            w.cks, w.cls, w.cbs, num_cta, False, w.L, 1, w.kv_dim, 1, counter_id=0,
+            kv_shared_across_ranks_mode="sharded", notify_mode=notify)
+
+    layer_bytes = w.num_blocks * w.kv_dim * w.chunk
+    # dummy compute: square matmuls on a side stream, sized to about one layer's copy time
+    comp = torch.cuda.Stream()
+    n = 2048
+    a = torch.randn(n, n, device=w.device, dtype=torch.bfloat16)
+    b = torch.randn(n, n, device=w.device, dtype=torch.bfloat16)
+    c = torch.empty(n, n, device=w.device, dtype=torch.bfloat16)
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+
+    def compute_only(reps):
+        with torch.cuda.stream(comp):
+            s, e = ev(), ev()
+            s.record(comp)
+            for _ in range(w.L):
+                for _ in range(reps):
+                    torch.matmul(a, b, out=c)
+            e.record(comp)
+        e.synchronize()
+        return s.elapsed_time(e)
+
+    compute_only(1)
+    target_ms = layer_bytes / 55e9 * 1e3
+    per_mm = compute_only(4) / (4 * w.L)
+    reps = max(1, int(round(target_ms / per_mm)))
+    compute_ms = _median([compute_only(reps) for _ in range(3)])
+
+    totals, restores, firsts = [], [], []
+    for it in range(warmup + steps):
+        torch.cuda.synchronize()
+        s, e = ev(), ev()
+        t0 = time.perf_counter()
+        with torch.cuda.stream(comp):
+            s.record(comp)
+        restore()  # polling: returns right after the launches
+        with torch.cuda.stream(comp):
+            for l in range(w.L):
+                grp.wait_layer(l, comp)
+                for _ in range(reps):
+                    torch.matmul(a, b, out=c)
+            e.record(comp)
+        e.synchronize()
+        grp.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3
+        if it >= warmup:
+            bt = grp.batch_times_ms()
+            totals.append(s.elapsed_time(e))
+            restores.append(bt[-1])
+            firsts.append(bt[0])
+            _ = wall
+    grp.close()
+    return dict(total_ms=_median(totals), restore_ms=_median(restores),
+                first_layer_ms=_median(firsts), compute_ms=compute_ms,
+                compute_reps_per_layer=reps, layer_bytes=layer_bytes)
+
+
+def run_concurrent(w, torch, steps, warmup, num_cta):
+    """c4: 32 D2H puts and 32 H2D gets issued at once from 64 threads, one
+    stream each."""
+    reqs = w.requests
+    streams = [torch.cuda.Stream() for _ in reqs]
+    lat = [[] for _ in reqs]
+    walls = []
+    w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=num_cta, sync=True)  # fill the host cache
+
+    def worker(i, barrier, record):
+        gi, ci = reqs[i]
+        with torch.cuda.stream(streams[i]):
+            barrier.wait()
+            t0 = time.perf_counter()
+            w.transfer(gi, ci, h2d=(i % 2 == 1), transfer_num_cta=num_cta, sync=True)
+            if record:
+                lat[i].append((time.perf_counter() - t0) * 1e3)
+
+    for it in range(warmup + steps):
+        barrier = threading.Barrier(len(reqs) + 1)
+        threads = [threading.Thread(target=worker, args=(i, barrier, it >= warmup))
+                   for i in range(len(reqs))]
+        for th in threads:
+            th.start()
+        torch.cuda.synchronize()
+        barrier.wait()
+        t0 = time.perf_counter()
+        for th in threads:
+            th.join()
+        if it >= warmup:
+            walls.append(time.perf_counter() - t0)
+    all_lat = sorted(x for l in lat for x in l)
+    p99 = all_lat[min(len(all_lat) - 1, int(0.99 * len(all_lat)))]
+    total_bytes = sum(int(g.numel()) for g, _ in reqs) * w.L * w.kv_dim * w.chunk
+    return dict(walls=walls, p99_ms=p99, p50_ms=_median(all_lat), total_bytes=total_bytes,
+                blocks=[int(g.numel()) for g, _ in reqs])
+
+
+# ---------------------------------------------------------------------------
+# CPU baseline: the reference's CPU path (torch index-gather into the host
+# cache layout), timed on this machine's host cores on a bounded sample.
+# ---------------------------------------------------------------------------
+def cpu_baseline(cfg, budget_s=20.0):
+    import torch
+    from oracle import fkv_oracle as O
+    T, H, D = (64, 8, 128) if cfg == "c1" else (16, 8, 128)
+    L, N, n, NH = 4, 4096, (1024 if cfg == "c1" else 256), 1024
+    # vLLM-shaped [kv, N, T, H, D] tensors in host RAM; for the SGLang config a
+    # page is the same 64x8x128 row block, K and V planes of a layer stacked.
+    layers = [torch.empty(2, N, T, H, D, dtype=torch.bfloat16) for _ in range(L)]
+    for i, x in enumerate(layers):
+        x.view(torch.int16).copy_(
+            (torch.arange(x.numel(), dtype=torch.int32) * (2 * i + 3)).to(torch.int16).view(x.shape))
+    host = torch.zeros(NH, L, 2, T, H, D, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(7)
+    gi = torch.randperm(N, generator=g)[:n]
+    ci = torch.randperm(NH, generator=g)[:n]
+    nbytes = 2 * n * L * 2 * T * H * D * 2  # gather + scatter
+    O.torch_index_gather(layers, host, gi, ci)
+    O.torch_index_scatter(layers, host, gi, ci)
+    t_start, reps, best = time.perf_counter(), 0, float("inf")
+    while True:
+        t0 = time.perf_counter()
+        O.torch_index_gather(layers, host, gi, ci)
+        O.torch_index_scatter(layers, host, gi, ci)
+        dt = time.perf_counter() - t0
+        best = min(best, dt)
+        reps += 1
+        if time.perf_counter() - t_start > budget_s or reps >= 200:
+            break
+    elapsed = time.perf_counter() - t_start
+    return {"value": round(nbytes * reps / elapsed / 1e9, 3), "best": round(nbytes / best / 1e9, 3),
+            "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": (f"{L} of 32 layers, {n} blocks of {T}x{H}x{D} bf16 K+V out of a {N}-block "
+                       f"pool, torch index_select/index_copy_ gather into the block-first host "
+                       f"cache then scatter back, {reps} repetitions ({elapsed:.1f} s), "
+                       f"os.cpu_count()={os.cpu_count()}")}
+
+
+# ---------------------------------------------------------------------------
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4"])
+    ap.add_argument("--num-cta", type=int, default=4,
+                    help="transfer_num_cta (reference default FLEXKV_TRANSFER_NUM_CTA_*=4)")
+    ap.add_argument("--use-ce", action="store_true", help="copy-engine path instead of the kernel")
+    ap.add_argument("--notify", default="polling", choices=["polling", "hostfunc"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-verify", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the transfer path crosses one host "
+              "link per GPU and has no cross-GPU step); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import flexkv_amd.c_ext as c_ext  # fails loudly if libfkv_hip.so is missing
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    device = "cuda:0"
+    torch.cuda.set_device(0)
+
+    link = measure_link()
+    w = Workload(args.config, torch, device)
+    B = w.bytes_per_direction
+    out = {"metric": METRIC, "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "u8", "data": "synthetic"}
+    path_name = "copy-engine" if args.use_ce else "kernel"
+    config = {"workload": f"{args.config}: {w.desc}", "path": path_name,
+              "transfer_num_cta": args.num_cta, "blocks": w.num_blocks,
+              "bytes_per_direction": B}
+
+    if args.config in ("c0", "c1", "c2"):
+        wall, d2h_ms, h2d_ms = run_gather_scatter(w, torch, args.steps, args.warmup, args.num_cta,
+                                                  args.use_ce)
+        taken = c_ext.last_transfer_path()
+        d2h = B / (sum(d2h_ms) / len(d2h_ms) * 1e-3) / 1e9
+        h2d = B / (sum(h2d_ms) / len(h2d_ms) * 1e-3) / 1e9
+        out.update(value=round(2 * B * args.steps / wall / 1e9, 3),
+                   ms_per_step=round(wall / args.steps * 1e3, 3),
+                   d2h_GBps=round(d2h, 3), h2d_GBps=round(h2d, 3),
+                   d2h_frac_of_link=round(d2h / link["d2h"], 4),
+                   h2d_frac_of_link=round(h2d / link["h2d"], 4))
+        # dominant kernel: the gather/scatter kernel; one launch per direction moves B bytes
+        avg_ms = (sum(d2h_ms) + sum(h2d_ms)) / (len(d2h_ms) + len(h2d_ms))
+        achieved = B / (avg_ms * 1e-3) / 1e9
+        kernel = "fkv_copy_chunks_kernel<16>" if not args.use_ce else taken
+        out["roofline"] = {"bound": "hbm", "achieved": round(achieved, 3), "peak": HBM_PEAK_GBPS,
+                           "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 5),
+                           "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, path_name)),
+                           "kernel": kernel, "algorithmic_bytes_per_launch": B,
+                           "avg_launch_ms": round(avg_ms, 4),
+                           "limited_by": "host link (PCIe), not HBM",
+                           "link_peak_GBps": round((link["d2h"] + link["h2d"]) / 2, 3),
+                           "frac_of_link_peak": round(
+                               achieved / ((link["d2h"] + link["h2d"]) / 2), 4)}
+        config["path_taken"] = taken
+        if not args.no_verify:
+            out["bit_exact"] = verify_round_trip(w, torch, args.num_cta)
+    elif args.config == "c3":
+        # fill the host cache with the blocks to restore, then erase them on the GPU
+        w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=args.num_cta, sync=True)
+        gi = w.gpu_ids.to(device)
+        saved = [w.gpu_rows(l, 0).index_select(0, gi) for l in range(w.L)]
+        for l in range(w.L):
+            w.gpu_rows(l, 0).index_fill_(0, gi, 0)
+        r = run_layerwise(w, torch, args.steps, args.warmup, args.num_cta, args.notify)
+        exposed = r["total_ms"] - r["compute_ms"]
+        restore = B / (r["restore_ms"] * 1e-3) / 1e9
+        out.update(value=round(restore, 3), ms_per_step=round(r["total_ms"], 3),
+                   h2d_GBps=round(restore, 3), h2d_frac_of_link=round(restore / link["h2d"], 4),
+                   layerwise={"notify": args.notify, "restore_ms": round(r["restore_ms"], 3),
+                              "first_layer_ms": round(r["first_layer_ms"], 3),
+                              "compute_only_ms": round(r["compute_ms"], 3),
+                              "restore_plus_compute_ms": round(r["total_ms"], 3),
+                              "exposed_ms": round(exposed, 3),
+                              "overlap_frac_beyond_first_layer": round(
+                                  1.0 - max(0.0, exposed - r["first_layer_ms"]) /
+                                  max(1e-9, r["restore_ms"] - r["first_layer_ms"]), 4)})
+        if not args.no_verify:
+            out["bit_exact"] = all(
+                torch.equal(w.gpu_rows(l, 0).index_select(0, gi), saved[l]) for l in range(w.L))
+        achieved = restore
+        out["roofline"] = {"bound": "hbm", "achieved": round(achieved, 3), "peak": HBM_PEAK_GBPS,
+                           "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 5),
+                           "traffic": None, "kernel": "fkv_copy_chunks_kernel<16>",
+                           "algorithmic_bytes_per_launch": r["layer_bytes"],
+                           "limited_by": "host link (PCIe), not HBM",
+                           "link_peak_GBps": round(link["h2d"], 3),
+                           "frac_of_link_peak": round(achieved / link["h2d"], 4)}
+    else:  # c4
+        r = run_concurrent(w, torch, args.steps, args.warmup, args.num_cta)
+        agg = r["total_bytes"] / _median(r["walls"]) / 1e9
+        out.update(value=round(agg, 3), ms_per_step=round(_median(r["walls"]) * 1e3, 3),
+                   concurrent={"requests": 64, "total_blocks": sum(r["blocks"]),
+                               "aggregate_bytes": r["total_bytes"],
+                               "p50_latency_ms": round(r["p50_ms"], 3),
+                               "p99_latency_ms": round(r["p99_ms"], 3),
+                               "frac_of_bidir_link": round(agg / (link["d2h"] + link["h2d"]), 4)})
+        out["roofline"] = {"bound": "hbm", "achieved": round(agg, 3), "peak": HBM_PEAK_GBPS,
+                           "unit": "GB/s", "frac": round(agg / HBM_PEAK_GBPS, 5), "traffic": None,
+                           "kernel": "fkv_copy_chunks_kernel<16>",
+                           "limited_by": "host link (PCIe), both directions at once"}
+    out["link_peak"] = {"d2h_GBps": round(link["d2h"], 3), "h2d_GBps": round(link["h2d"], 3),
+                        "method": "1 GiB pinned hipMemcpyAsync x10, best, same run"}
+    out["config"] = config
+    if not args.no_cpu_baseline:
+        del w
+        torch.cuda.empty_cache()
+        out["cpu_baseline"] = cpu_baseline(args.config)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -209,8 +209,9 @@ int env_int(const char *name, int fallback) {
 } // namespace
 
 int default_num_cta(bool is_h2d) {
-  static const int h2d = env_int("FKV_NUM_CTA_H2D", 8);
-  static const int d2h = env_int("FKV_NUM_CTA_D2H", 8);
+  // same default as FLEXKV_TRANSFER_NUM_CTA_{H2D,D2H} (flexkv/common/config.py:779-780)
+  static const int h2d = env_int("FKV_NUM_CTA_H2D", 4);
+  static const int d2h = env_int("FKV_NUM_CTA_D2H", 4);
   return is_h2d ? h2d : d2h;
 }
 
@@ -229,7 +230,12 @@ int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream) {
   }
   const bool h2d = d.is_host_to_device != 0;
   static const bool mirror_plan = env_int("FKV_PLAN_MIRROR", 1) != 0;
-  int num_cta = d.transfer_num_cta > 0 ? d.transfer_num_cta : default_num_cta(h2d);
+  // A CTA of the reference is 1024 threads = 32 warps (csrc/transfer.cu:176).  A
+  // workgroup here is 1024 lanes = 16 wavefronts, so each requested CTA becomes
+  // kWorkgroupsPerCta workgroups: the same number of independent instruction
+  // streams, which is what bounds the reads a CU keeps in flight over the link.
+  const int num_cta = (d.transfer_num_cta > 0 ? d.transfer_num_cta : default_num_cta(h2d)) *
+                      kWorkgroupsPerCta;
 
   // Layers go out in groups whose (layer, kv) base tables fit the kernel's LDS.
   const int layers_per_launch = kCopyMaxLK / d.kv_dim;

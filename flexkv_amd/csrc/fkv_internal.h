@@ -114,6 +114,7 @@ struct CopyKernelArgs {
   int32_t vec; // 16, 8, 4, 2 or 1: widest access all addresses allow
 };
 constexpr int kCopyBlockThreads = 1024;  // 16 wavefronts, one CU
+constexpr int kWorkgroupsPerCta = 2;      // workgroups launched per requested CTA
 constexpr int kCopyUnroll = 8;           // vector accesses in flight per lane
 constexpr int kCopyMaxLK = 1024;         // base-table entries staged in LDS
 constexpr int kCopyIdTile = 1024;        // block positions staged in LDS at a time

@@ -104,7 +104,8 @@ typedef struct fkv_transfer_desc {
   /* how */
   int32_t is_host_to_device;
   int32_t use_ce_transfer;
-  int32_t transfer_num_cta; /* workgroups of 1024 lanes; <= 0 = library default */
+  int32_t transfer_num_cta; /* CTAs in the reference's unit (32 warps); each becomes two
+                               16-wavefront workgroups; <= 0 = library default (4) */
   int32_t sync;             /* 1: hipStreamSynchronize before returning */
   int32_t enable_trace;     /* 1: print an "[XFER]" line per call to stderr */
   int32_t reserved;
