@@ -42,6 +42,10 @@ def _ids(t: torch.Tensor, name: str) -> torch.Tensor:
 
 
 def _current_stream_handle() -> int:
+    # Without a GPU the null stream is passed on: descriptor validation still runs
+    # in the library, and the first device call there fails with a RuntimeError.
+    if not torch.cuda.is_available():
+        return 0
     return int(torch.cuda.current_stream().cuda_stream)
 
 

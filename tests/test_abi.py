@@ -1,0 +1,136 @@
+"""The C-ABI library loads without a GPU, exports every function the header
+declares, and rejects bad descriptors with the reference's exception classes
+before touching the device."""
+import ctypes
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+import torch
+
+from flexkv_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "fkv_transfer.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fkv_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    lib = _lib.load()
+    names = declared_functions()
+    assert len(names) >= 25
+    dyn = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], capture_output=True,
+                         text=True, check=True).stdout
+    exported = set(re.findall(r" T (fkv_\w+)", dyn))
+    for n in names:
+        assert n in exported, f"{n} declared in the header but not exported"
+        assert hasattr(lib, n)
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes prototype"
+    assert exported == set(names), "exports that the header does not declare"
+
+
+def test_header_compiles_as_c_and_struct_sizes_match():
+    src = r'''
+#include "fkv_transfer.h"
+#include <stdio.h>
+int main(void){ printf("%zu %zu %zu %zu %zu %zu %zu\n", sizeof(fkv_ce_config),
+  sizeof(fkv_transfer_desc), sizeof(fkv_ce_analysis), sizeof(fkv_tp_rank_plan),
+  sizeof(fkv_tp_group_params), sizeof(fkv_layerwise_params), sizeof(fkv_stats)); return 0; }
+'''
+    import tempfile
+    with tempfile.TemporaryDirectory() as d:
+        c = os.path.join(d, "t.c")
+        open(c, "w").write(src)
+        exe = os.path.join(d, "t")
+        subprocess.check_call(["gcc", "-std=c11", "-Wall", "-Werror", "-I",
+                               os.path.join(ROOT, "include"), c, "-o", exe])
+        sizes = list(map(int, subprocess.check_output([exe]).split()))
+    want = [ctypes.sizeof(x) for x in (_lib.CEConfig, _lib.TransferDesc, _lib.CEAnalysis,
+                                       _lib.TPRankPlan, _lib.TPGroupParams, _lib.LayerwiseParams,
+                                       _lib.Stats)]
+    assert sizes == want
+
+
+def test_defaults_of_ce_config():
+    cfg = _lib.default_ce_config()   # csrc/ce_transfer.h:18-41
+    assert (cfg.segment_threshold, cfg.path_opt_enabled, cfg.force_path, cfg.enable_memcpy2d,
+            cfg.is_blockfirst, cfg.num_kv_heads, cfg.gather_threads, cfg.gather_nt) == \
+        (8, 1, -1, 0, 0, 1, 4, 1)
+
+
+def _call(**over):
+    from flexkv_amd.c_ext import transfer_kv_blocks
+    ids = torch.arange(2, dtype=torch.int64)
+    args = dict(gpu_block_id_tensor=ids, gpu_tensor_ptrs_tensor=torch.zeros(4, dtype=torch.int64),
+                gpu_kv_stride_in_bytes=64, gpu_block_stride_in_bytes=16,
+                gpu_layer_stride_in_bytes=128, cpu_block_id_tensor=ids,
+                cpu_tensor=torch.zeros(1024, dtype=torch.uint8), cpu_kv_stride_in_bytes=16,
+                cpu_layer_stride_in_bytes=32, cpu_block_stride_in_bytes=128,
+                chunk_size_in_bytes=16, start_layer_id=0, num_layers=4)
+    args.update(over)
+    transfer_kv_blocks(**args)
+
+
+def test_bad_descriptors_are_rejected_on_the_host():
+    with pytest.raises(RuntimeError, match="Unsupported gpu_block_type: 7"):  # bindings.cpp:91-94
+        _call(gpu_block_type=7)
+    with pytest.raises(ValueError, match="differ in length"):
+        _call(cpu_block_id_tensor=torch.arange(3, dtype=torch.int64))
+    with pytest.raises(TypeError):
+        _call(gpu_block_id_tensor=torch.arange(2, dtype=torch.int32))
+    with pytest.raises(ValueError, match="negative block id"):
+        _call(gpu_block_id_tensor=torch.tensor([0, -1], dtype=torch.int64))
+    with pytest.raises(ValueError, match="GPU tensor pointers"):
+        _call(num_layers=5)                                   # vLLM needs 5 pointers, 4 given
+    with pytest.raises(ValueError, match="GPU tensor pointers"):
+        _call(gpu_block_type=2, num_layers=4, kv_dim=2)       # SGLang needs K and V tables
+    with pytest.raises(ValueError, match="chunk_size_in_bytes"):
+        _call(chunk_size_in_bytes=0)
+
+
+def test_empty_transfer_is_a_no_op_without_a_gpu():
+    empty = torch.empty(0, dtype=torch.int64)
+    _call(gpu_block_id_tensor=empty, cpu_block_id_tensor=empty)   # no device call is made
+    _call(num_layers=0)
+
+
+def test_status_codes_map_to_exception_classes():
+    lib = _lib.load()
+    out = _lib.TPRankPlan()
+    rc = lib.fkv_tp_rank_plan_compute(5, 4, 1, 0, b"sharded", 0, 0, 0, 1, 1, 64, 64, 16,
+                                      ctypes.byref(out))
+    assert rc == _lib.FKV_ERR_INVALID_ARG and "bad rank" in _lib.last_error()
+    with pytest.raises(ValueError):
+        _lib.check(rc)
+    with pytest.raises(RuntimeError):
+        _lib.check(_lib.FKV_ERR_RUNTIME)
+
+
+def test_host_registration_chunking():
+    """flexkv/transfer/host_buffer.py:57-98: chunk size from GiB with a 4 KiB
+    margin rounded down to a page; pieces cover the buffer exactly once."""
+    lib = _lib.load()
+    from oracle import fkv_oracle as O
+    for gb in (0, -1, 0.5, 1, 2.5, 0.001):
+        assert lib.fkv_host_chunk_bytes_from_gb(gb) == O.lib().fkv_oracle_host_chunk_bytes(gb)
+    assert lib.fkv_host_chunk_bytes_from_gb(1.0) == (1 << 30) - 4096
+    assert lib.fkv_host_chunk_bytes_from_gb(0.0) == 0
+    for total, chunk in ((10 << 20, 0), (10 << 20, 16 << 20), (10 << 20, 3 << 20), (4096, 4096),
+                         ((3 << 20) * 4, 3 << 20), (1, 4096)):
+        n = lib.fkv_host_register_plan(total, chunk, None, None, 0)
+        off = np.zeros(n, dtype=np.uint64)
+        sz = np.zeros(n, dtype=np.uint64)
+        assert lib.fkv_host_register_plan(total, chunk, off.ctypes.data, sz.ctypes.data, n) == n
+        want_off = list(range(0, total, chunk)) if chunk and total > chunk else [0]
+        assert off.tolist() == want_off               # range(0, total, chunk) of the reference
+        assert int(sz.sum()) == total and (sz > 0).all()
+        assert all(int(o + s) == int(o2) for o, s, o2 in zip(off, sz, off[1:]))
+        if chunk and total > chunk:
+            assert (sz[:-1] == chunk).all() and sz[-1] <= chunk
