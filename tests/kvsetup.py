@@ -123,6 +123,40 @@ class DeviceSide:
             start_layer, nl, is_host_to_device=is_h2d, kv_dim=s.kv_dim,
             gpu_block_type=s.backend, **kw)
 
+    def transfer_raw(self, gpu_ids, cpu_ids, is_h2d: bool, start_layer: int = 0,
+                     num_layers: Optional[int] = None, gpu_off: int = 0, cpu_off: int = 0,
+                     chunk: Optional[int] = None, use_ce: bool = False, num_cta: int = 4,
+                     sync: bool = True, stream: int = 0, ce: Optional[dict] = None) -> int:
+        """Straight through the C ABI (fkv_transfer_kv_blocks), including the
+        in-chunk offsets the Python operator does not expose.  Returns the status."""
+        import ctypes
+        from flexkv_amd import _lib
+        s = self.s
+        L = _lib.load()
+        g = np.ascontiguousarray(gpu_ids, dtype=np.int64)
+        c = np.ascontiguousarray(cpu_ids, dtype=np.int64)
+        ptrs = np.ascontiguousarray([t.data_ptr() for t in self.gpu], dtype=np.uint64)
+        d = _lib.TransferDesc()
+        d.backend, d.num_layers_total = s.backend, s.num_layers_total
+        d.gpu_tensor_ptrs, d.num_gpu_tensor_ptrs, d.device = ptrs.ctypes.data, ptrs.size, -1
+        d.gpu_kv_stride, d.gpu_block_stride = s.gpu_kv_stride, s.gpu_block_stride
+        d.gpu_layer_stride, d.gpu_startoff_inside_chunks = s.gpu_layer_stride, gpu_off
+        d.cpu_ptr = self.host.data_ptr()
+        d.cpu_kv_stride, d.cpu_layer_stride = s.cpu_kv_stride, s.cpu_layer_stride
+        d.cpu_block_stride, d.cpu_startoff_inside_chunks = s.cpu_block_stride, cpu_off
+        d.chunk_size = s.chunk if chunk is None else chunk
+        d.start_layer_id = start_layer
+        d.num_layers = s.num_layers - start_layer if num_layers is None else num_layers
+        d.kv_dim, d.num_blocks = s.kv_dim, g.size
+        d.gpu_block_ids, d.cpu_block_ids = g.ctypes.data, c.ctypes.data
+        d.is_host_to_device, d.use_ce_transfer = int(is_h2d), int(use_ce)
+        d.transfer_num_cta, d.sync = num_cta, int(sync)
+        d.ce = _lib.default_ce_config()
+        d.ce.is_blockfirst = int(s.cpu_layout == "BLOCKFIRST")
+        for k, v in (ce or {}).items():
+            setattr(d.ce, k, v)
+        return int(L.fkv_transfer_kv_blocks(ctypes.byref(d), stream))
+
     def gpu_bytes(self) -> List[np.ndarray]:
         return [t.cpu().numpy() for t in self.gpu]
 

@@ -1,0 +1,159 @@
+"""Copy-engine strategies vs the CPU oracle (bit-exact), and the strategy that
+actually ran vs the oracle's choose_path."""
+import numpy as np
+import pytest
+
+from kvsetup import KVSetup, VLLM, TRTLLM, SGLANG, block_ids
+from oracle import fkv_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+PATHS = {"CONTIG_DIRECT": 0, "SEGMENT_DIRECT": 1, "SEGMENT_SCATTER": 2, "GATHER_SCATTER": 3,
+         "GATHER_DIRECT": 4}
+
+
+def expected_path(s, gids, cids, heads, thr, h2d, num_layers):
+    an, _ = O.ce_analyze(gids, cids, s.cpu_block_stride, s.chunk, s.gpu_block_stride)
+    full = num_layers * s.kv_dim * s.chunk == s.cpu_block_stride
+    return O.CE_NAMES[O.ce_choose_path(an, s.cpu_layout == "BLOCKFIRST", heads, thr, s.chunk,
+                                       h2d, full)]
+
+
+SHAPES = [
+    pytest.param(VLLM, 4, 2, 64, 64, 4096, "BLOCKFIRST", "LAYERFIRST", id="vllm-bf-kv2"),
+    pytest.param(VLLM, 4, 2, 64, 64, 4096, "LAYERFIRST", "LAYERFIRST", id="vllm-lf-kv2"),
+    pytest.param(VLLM, 4, 1, 64, 64, 9216, "BLOCKFIRST", "LAYERFIRST", id="mla-bf"),
+    pytest.param(VLLM, 4, 1, 64, 64, 9216, "LAYERFIRST", "LAYERFIRST", id="mla-lf"),
+    pytest.param(VLLM, 3, 2, 64, 64, 2048, "BLOCKFIRST", "LAYERBLOCK", id="vllm-layerblock"),
+    pytest.param(TRTLLM, 5, 2, 64, 64, 4096, "BLOCKFIRST", "LAYERFIRST", id="trtllm-bf"),
+    pytest.param(SGLANG, 4, 2, 64, 64, 8192, "BLOCKFIRST", "LAYERFIRST", id="sglang-bf"),
+    pytest.param(SGLANG, 4, 2, 64, 64, 8192, "LAYERFIRST", "LAYERFIRST", id="sglang-lf"),
+]
+
+
+@pytest.mark.parametrize("backend,L,K,N,NH,chunk,cpu_layout,gpu_layout", SHAPES)
+@pytest.mark.parametrize("pattern", ["contiguous", "few_seg", "scattered"])
+@pytest.mark.parametrize("heads", [1, 8])
+@pytest.mark.parametrize("memcpy2d", [False, True], ids=["no2d", "2d"])
+def test_auto_strategy_matches_oracle(gpu_device, backend, L, K, N, NH, chunk, cpu_layout,
+                                      gpu_layout, pattern, heads, memcpy2d):
+    from flexkv_amd.c_ext import last_transfer_path
+    s = KVSetup(backend, L, K, N, NH, chunk, cpu_layout, gpu_layout, seed=31)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(7)
+    n = 32
+    if pattern == "scattered":
+        gids, cids = block_ids(rng, N, n), block_ids(rng, NH, n)
+    else:  # the same shape on both sides so that runs line up
+        gids = block_ids(rng, N, n, pattern)
+        cids = gids - gids.min() + int(rng.integers(0, NH - n + 1))
+        if pattern == "few_seg":
+            cids = block_ids(np.random.default_rng(1), NH, n, "few_seg")
+            gids = cids - cids.min() + int(gids.min())
+    for thr in (8, 2):
+        for h2d in (False, True):
+            want = expected_path(s, gids, cids, heads, thr, h2d, L)
+            print(f"case {pattern} heads={heads} thr={thr} h2d={h2d} 2d={memcpy2d} -> {want}",
+                  flush=True)
+            dev.transfer(gids, cids, is_h2d=h2d, use_ce_transfer=True, ce_path_opt=True,
+                         ce_segment_threshold=thr, num_kv_heads=heads,
+                         ce_enable_memcpy2d=memcpy2d)
+            assert last_transfer_path() == want
+            s.oracle_transfer(gids, cids, h2d)
+            dev.assert_matches_reference(f"{want} h2d={h2d}")
+
+
+@pytest.mark.parametrize("backend,L,K,N,NH,chunk,cpu_layout,gpu_layout", SHAPES)
+def test_per_block_baseline(gpu_device, backend, L, K, N, NH, chunk, cpu_layout, gpu_layout):
+    from flexkv_amd.c_ext import last_transfer_path
+    s = KVSetup(backend, L, K, N, NH, chunk, cpu_layout, gpu_layout, seed=32)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(8)
+    gids, cids = block_ids(rng, N, 12), block_ids(rng, NH, 12)
+    for h2d in (False, True):
+        dev.transfer(gids, cids, is_h2d=h2d, use_ce_transfer=True, ce_path_opt=False)
+        assert last_transfer_path() == "PER_BLOCK"
+        s.oracle_transfer(gids, cids, h2d)
+        dev.assert_matches_reference(f"PER_BLOCK h2d={h2d}")
+
+
+@pytest.mark.parametrize("force", ["SEGMENT_SCATTER", "GATHER_SCATTER", "GATHER_DIRECT"])
+@pytest.mark.parametrize("backend,L,K,N,NH,chunk,cpu_layout,gpu_layout", SHAPES)
+@pytest.mark.parametrize("memcpy2d", [False, True], ids=["no2d", "2d"])
+def test_forced_general_strategies(gpu_device, force, backend, L, K, N, NH, chunk, cpu_layout,
+                                   gpu_layout, memcpy2d):
+    """The three strategies that cope with any id pattern, forced on every shape
+    (kernel path == every copy-engine path on the same inputs)."""
+    from flexkv_amd.c_ext import last_transfer_path
+    s = KVSetup(backend, L, K, N, NH, chunk, cpu_layout, gpu_layout, seed=33)
+    gpu_rows_adjacent = s.gpu_block_stride == s.chunk
+    if force == "SEGMENT_SCATTER" and not gpu_rows_adjacent and not memcpy2d:
+        pytest.skip("segment DMA needs adjacent GPU blocks (checked in test_forced_misfit)")
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(9)
+    for pattern in ("scattered", "few_seg"):
+        cids = block_ids(rng, NH, 24, pattern)
+        gids = block_ids(rng, N, 24, "scattered") if pattern == "scattered" else \
+            cids - cids.min() + 3
+        if force == "SEGMENT_SCATTER" and not gpu_rows_adjacent and pattern == "scattered":
+            continue  # 24 segments exceed the 2-D copy threshold; the staging branch needs adjacency
+        for h2d in (False, True):
+            print(f"case force={force} {pattern} h2d={h2d} 2d={memcpy2d}", flush=True)
+            dev.transfer(gids, cids, is_h2d=h2d, use_ce_transfer=True, ce_path_opt=True,
+                         ce_force_path=PATHS[force], ce_enable_memcpy2d=memcpy2d,
+                         ce_gather_threads=3)
+            assert last_transfer_path() == force
+            s.oracle_transfer(gids, cids, h2d)
+            dev.assert_matches_reference(f"forced {force} {pattern} h2d={h2d}")
+
+
+def test_forced_direct_strategies_on_fitting_input(gpu_device):
+    from flexkv_amd.c_ext import last_transfer_path
+    s = KVSetup(VLLM, 3, 1, 40, 40, 4096, "LAYERFIRST", seed=34)   # adjacent blocks on both sides
+    dev = s.to_device(gpu_device)
+    run_g, run_c = np.arange(5, 25, dtype=np.int64), np.arange(11, 31, dtype=np.int64)
+    for h2d in (False, True):
+        dev.transfer(run_g, run_c, is_h2d=h2d, use_ce_transfer=True, ce_path_opt=True, ce_force_path=0)
+        assert last_transfer_path() == "CONTIG_DIRECT"
+        s.oracle_transfer(run_g, run_c, h2d)
+        dev.assert_matches_reference("CONTIG_DIRECT")
+    seg_g = np.array([0, 1, 2, 10, 11, 30, 20, 21], dtype=np.int64)
+    seg_c = np.array([5, 6, 7, 20, 21, 0, 33, 34], dtype=np.int64)
+    for h2d in (False, True):
+        dev.transfer(seg_g, seg_c, is_h2d=h2d, use_ce_transfer=True, ce_path_opt=True, ce_force_path=1)
+        assert last_transfer_path() == "SEGMENT_DIRECT"
+        s.oracle_transfer(seg_g, seg_c, h2d)
+        dev.assert_matches_reference("SEGMENT_DIRECT")
+
+
+def test_forced_misfit_and_out_of_range(gpu_device):
+    s = KVSetup(VLLM, 2, 2, 16, 16, 1024, "BLOCKFIRST", seed=35)
+    dev = s.to_device(gpu_device)
+    ids = np.array([3, 9, 1], dtype=np.int64)
+    with pytest.raises(RuntimeError, match=r"force_path out of range \[0,4\]: 5"):  # transfer.cu:213
+        dev.transfer(ids, ids, is_h2d=False, use_ce_transfer=True, ce_path_opt=True, ce_force_path=5)
+    # a strategy that assumes adjacent host blocks must not be run on a block-first pool
+    with pytest.raises(ValueError, match="does not fit"):
+        dev.transfer(ids, ids, is_h2d=False, use_ce_transfer=True, ce_path_opt=True, ce_force_path=0)
+    with pytest.raises(ValueError, match="does not fit"):
+        dev.transfer(ids, ids, is_h2d=False, use_ce_transfer=True, ce_path_opt=True, ce_force_path=1)
+    dev.assert_matches_reference("refused calls moved nothing")
+
+
+def test_gather_direct_groups_and_partial_layers(gpu_device, monkeypatch):
+    """Layer batches (host block only partly covered) take the per-block / 2-D
+    branch of GATHER_DIRECT; the result equals the whole-block branch."""
+    from flexkv_amd.c_ext import last_transfer_path
+    s = KVSetup(VLLM, 6, 2, 48, 48, 2048, "BLOCKFIRST", seed=36)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(10)
+    gids, cids = block_ids(rng, 48, 20), block_ids(rng, 48, 20, "few_seg")
+    for memcpy2d in (False, True):
+        for l0 in (0, 2, 4):
+            for h2d in (False, True):
+                dev.transfer(gids, cids, is_h2d=h2d, start_layer=l0, num_layers=2,
+                             use_ce_transfer=True, ce_path_opt=True, ce_force_path=4,
+                             ce_enable_memcpy2d=memcpy2d, num_kv_heads=8)
+                assert last_transfer_path() == "GATHER_DIRECT"
+                s.oracle_transfer(gids, cids, h2d, start_layer=l0, num_layers=2)
+                dev.assert_matches_reference(f"GATHER_DIRECT layers {l0}..{l0 + 1} h2d={h2d}")

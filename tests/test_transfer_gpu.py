@@ -37,3 +37,143 @@ def test_kernel_d2h_then_h2d_matches_oracle(gpu_device, backend, L, K, N, NH, ch
     dev.transfer(gids2, cids, is_h2d=True)
     s.oracle_transfer(gids2, cids, is_h2d=True)
     dev.assert_matches_reference("after H2D")
+
+
+# ---- alignment fallbacks, offsets, edge shapes (straight through the C ABI) ----
+
+@pytest.mark.parametrize("chunk,gpu_off,cpu_off,sub", [
+    (4680 * 8, 4680, 4680, 4680),   # 8-aligned shard of a 16-aligned chunk (the reference's 8-byte kernel)
+    (40, 0, 0, 40),                  # chunk % 16 == 8
+    (48, 8, 24, 16),                 # offsets differ on the two sides
+    (20, 0, 0, 20),                  # 4-byte granularity (outside the reference's domain)
+    (6, 2, 2, 4),
+    (7, 0, 0, 7),                    # odd bytes
+    (3 * 8192 + 48, 0, 0, 3 * 8192 + 48),  # several full slices and a short tail
+])
+@pytest.mark.parametrize("backend", [VLLM, TRTLLM, SGLANG])
+def test_offsets_and_narrow_alignment(gpu_device, backend, chunk, gpu_off, cpu_off, sub):
+    s = KVSetup(backend, 3, 2, 20, 16, chunk, "BLOCKFIRST", seed=21)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(2)
+    gids, cids = block_ids(rng, 20, 9), block_ids(rng, 16, 9)
+    print(f"case backend={backend} chunk={chunk} offs=({gpu_off},{cpu_off}) sub={sub}", flush=True)
+    for h2d in (False, True):
+        assert dev.transfer_raw(gids, cids, h2d, gpu_off=gpu_off, cpu_off=cpu_off, chunk=sub) == 0
+        s.oracle_transfer(gids, cids, h2d, gpu_off=gpu_off, cpu_off=cpu_off, chunk=sub)
+        dev.assert_matches_reference(f"h2d={h2d}")
+        gids = block_ids(rng, 20, 9)
+
+
+def test_padded_gpu_blocks_and_partial_layer_range(gpu_device):
+    s = KVSetup(VLLM, 6, 2, 24, 24, 2048, "LAYERFIRST", seed=5, gpu_block_pad=256)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(3)
+    gids, cids = block_ids(rng, 24, 10), block_ids(rng, 24, 10)
+    dev.transfer(gids, cids, is_h2d=False, start_layer=2, num_layers=3)
+    s.oracle_transfer(gids, cids, False, start_layer=2, num_layers=3)
+    dev.assert_matches_reference("layers 2..4 D2H")
+    dev.transfer(cids, gids, is_h2d=True, start_layer=4, num_layers=2)
+    s.oracle_transfer(cids, gids, True, start_layer=4, num_layers=2)
+    dev.assert_matches_reference("layers 4..5 H2D")
+
+
+def test_sglang_partial_layers_address_v_tensors(gpu_device):
+    """A call that covers only some layers must still find V_l at ptrs[L + l]."""
+    s = KVSetup(SGLANG, 5, 2, 12, 12, 512, "BLOCKFIRST", seed=6)
+    dev = s.to_device(gpu_device)
+    ids = np.array([3, 9, 1], dtype=np.int64)
+    dev.transfer(ids, ids, is_h2d=False, start_layer=3, num_layers=2)
+    s.oracle_transfer(ids, ids, False, start_layer=3, num_layers=2)
+    dev.assert_matches_reference("sglang layers 3..4")
+
+
+def test_empty_single_and_duplicate_ids(gpu_device):
+    s = KVSetup(VLLM, 2, 2, 8, 8, 1024, "BLOCKFIRST", seed=7)
+    dev = s.to_device(gpu_device)
+    none = np.empty(0, dtype=np.int64)
+    dev.transfer(none, none, is_h2d=False)
+    dev.transfer(none, none, is_h2d=True, use_ce_transfer=True, ce_path_opt=True)
+    dev.assert_matches_reference("empty transfer must not touch anything")
+    one = np.array([5], dtype=np.int64)
+    dev.transfer(one, np.array([2], dtype=np.int64), is_h2d=False)
+    s.oracle_transfer(one, np.array([2], dtype=np.int64), False)
+    dev.assert_matches_reference("single block")
+    # one GPU block fanned out to two host blocks (duplicate source ids are legal)
+    dup, dst = np.array([6, 6, 1], dtype=np.int64), np.array([0, 7, 3], dtype=np.int64)
+    dev.transfer(dup, dst, is_h2d=False)
+    s.oracle_transfer(dup, dst, False)
+    dev.assert_matches_reference("duplicate source ids")
+
+
+def test_many_blocks_cross_id_tiles(gpu_device):
+    """More block positions than one LDS id tile holds, few bytes each."""
+    s = KVSetup(VLLM, 2, 2, 5000, 5000, 64, "BLOCKFIRST", seed=8)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(4)
+    gids, cids = block_ids(rng, 5000, 4500), block_ids(rng, 5000, 4500)
+    for cta in (1, 4, 64):
+        assert dev.transfer_raw(gids, cids, False, num_cta=cta) == 0
+    s.oracle_transfer(gids, cids, False)
+    dev.assert_matches_reference("4500 blocks D2H")
+    assert dev.transfer_raw(cids, gids, True, num_cta=3) == 0
+    s.oracle_transfer(cids, gids, True)
+    dev.assert_matches_reference("4500 blocks H2D")
+
+
+def test_more_layer_kv_pairs_than_one_launch_holds(gpu_device):
+    """700 layers x 2 = 1400 (layer, kv) pairs: split over two launches."""
+    s = KVSetup(VLLM, 700, 2, 6, 6, 32, "BLOCKFIRST", seed=9)
+    dev = s.to_device(gpu_device)
+    ids = np.array([4, 0, 5, 2], dtype=np.int64)
+    dev.transfer(ids, ids[::-1].copy(), is_h2d=False)
+    s.oracle_transfer(ids, ids[::-1].copy(), False)
+    dev.assert_matches_reference("1400 pairs D2H")
+    dev.transfer(ids[::-1].copy(), ids, is_h2d=True, use_ce_transfer=True, ce_path_opt=True)
+    s.oracle_transfer(ids[::-1].copy(), ids, True)
+    dev.assert_matches_reference("1400 pairs H2D via copy engine")
+
+
+def test_async_call_owns_its_id_arrays(gpu_device):
+    """sync=False returns before the copy runs; the caller may reuse its id
+    tensors at once (they are copied into library-owned plan memory)."""
+    import torch
+    from flexkv_amd.c_ext import transfer_kv_blocks
+    s = KVSetup(VLLM, 8, 2, 256, 256, 32768, "BLOCKFIRST", seed=10)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(6)
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        for rep in range(6):
+            gids, cids = block_ids(rng, 256, 200), block_ids(rng, 256, 200)
+            g, c = torch.from_numpy(gids.copy()), torch.from_numpy(cids.copy())
+            h2d = bool(rep % 2)
+            transfer_kv_blocks(g, dev.ptrs, s.gpu_kv_stride, s.gpu_block_stride, s.gpu_layer_stride,
+                               c, dev.host, s.cpu_kv_stride, s.cpu_layer_stride,
+                               s.cpu_block_stride, s.chunk, 0, 8, is_host_to_device=h2d,
+                               sync=False, is_blockfirst=True)
+            g.fill_(255)   # scribble over the caller's arrays while the copy is in flight
+            c.fill_(255)
+            s.oracle_transfer(gids, cids, h2d)
+    st.synchronize()
+    dev.assert_matches_reference("six back-to-back async transfers")
+
+
+def test_pageable_host_tensor_is_refused_by_the_kernel_path(gpu_device):
+    import torch
+    from flexkv_amd.c_ext import transfer_kv_blocks
+    s = KVSetup(VLLM, 2, 2, 8, 8, 1024, "BLOCKFIRST", seed=11)
+    dev = s.to_device(gpu_device)
+    pageable = torch.zeros(s.host_bytes, dtype=torch.uint8)
+    ids = torch.arange(4, dtype=torch.int64)
+    with pytest.raises(ValueError, match="not device-visible"):
+        transfer_kv_blocks(ids, dev.ptrs, s.gpu_kv_stride, s.gpu_block_stride, s.gpu_layer_stride,
+                           ids, pageable, s.cpu_kv_stride, s.cpu_layer_stride, s.cpu_block_stride,
+                           s.chunk, 0, 2, is_host_to_device=False)
+    # the copy-engine path reads ids and data through the runtime and accepts pageable memory
+    transfer_kv_blocks(ids, dev.ptrs, s.gpu_kv_stride, s.gpu_block_stride, s.gpu_layer_stride,
+                       ids, pageable, s.cpu_kv_stride, s.cpu_layer_stride, s.cpu_block_stride,
+                       s.chunk, 0, 2, is_host_to_device=False, use_ce_transfer=True)
+    torch.cuda.synchronize()
+    s.host_ref[:] = 0
+    s.oracle_transfer(ids.numpy(), ids.numpy(), False)
+    np.testing.assert_array_equal(pageable.numpy(), s.host_ref)
