@@ -1,0 +1,444 @@
+"""TPTransferThreadGroup and LayerwiseTransferGroup on one GPU: round trips in
+the shape of the reference's own tests, host images vs the oracle, rank
+placement with several "ranks" sharing device 0, notification contract."""
+import ctypes
+import os
+import struct
+
+import numpy as np
+import pytest
+import torch
+
+from flexkv_amd.layout import KVCacheLayout, KVCacheLayoutType
+from oracle import fkv_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DTYPE = torch.float16
+ES = 2
+
+
+def make_layouts(L, N, T, H, D, cpu_name, kv_dim, heads, cpu_blocks=None):
+    gpu = KVCacheLayout(KVCacheLayoutType.LAYERFIRST, L, N, T, H, D, kv_dim=kv_dim, num_kv_heads=heads)
+    cpu = KVCacheLayout(KVCacheLayoutType[cpu_name], L, cpu_blocks or N, T, H, D, kv_dim=kv_dim,
+                        num_kv_heads=heads)
+    return gpu, cpu
+
+
+def make_gpu_tensors(L, N, T, H, D, kv_dim, device):
+    full = torch.zeros((L, kv_dim, N, T, H, D), dtype=DTYPE, device=device)
+    return [full[i] for i in range(L)]
+
+
+def fill_gpu(tensors, gpu_id, L, N, T, H, D, kv_dim):
+    """Deterministic fill of the reference's tests (test_kv_transfer_correctness.py:262-272)."""
+    for layer in range(L):
+        dev = tensors[layer].device
+        kv = torch.arange(kv_dim, device=dev).view(kv_dim, 1, 1, 1, 1)
+        blk = torch.arange(N, device=dev).view(1, N, 1, 1, 1)
+        tok = torch.arange(T, device=dev).view(1, 1, T, 1, 1)
+        h = torch.arange(D, device=dev).view(1, 1, 1, 1, D)
+        vals = (gpu_id * 100000 + kv * 500000 + layer * 10000 + blk * 1000 + tok * 10 + h) % 997
+        tensors[layer][:] = (vals / 997.0).to(DTYPE)
+
+
+def expected_val(gpu_id, layer, block, token, d, kv):
+    return float(((gpu_id * 100000 + kv * 500000 + layer * 10000 + block * 1000 + token * 10 + d)
+                  % 997) / 997.0)
+
+
+def tp_group(cpu, all_gpu, gpu_layout, L, devices, **kw):
+    from flexkv_amd.c_ext import TPTransferThreadGroup
+    n = len(all_gpu)
+    ptrs = [t.data_ptr() for g in all_gpu for t in g]
+    return TPTransferThreadGroup(
+        num_gpus=n, gpu_block_ptrs_flat=ptrs, num_tensors_per_gpu=L, cpu_blocks_ptr=cpu.data_ptr(),
+        num_layers=L, gpu_kv_strides_in_bytes=[gpu_layout.get_kv_stride() * ES] * n,
+        gpu_block_strides_in_bytes=[gpu_layout.get_block_stride() * ES] * n,
+        gpu_layer_strides_in_bytes=[gpu_layout.get_layer_stride() * ES] * n,
+        gpu_chunk_sizes_in_bytes=[gpu_layout.get_chunk_size() * ES] * n,
+        gpu_device_ids=devices, enable_nvcomp=False, nvcomp_batch_size=0, nvcomp_data_type=0, **kw)
+
+
+TP1_CONFIGS = [  # test_kv_transfer_correctness.py:715-721
+    pytest.param((4, 8, 16, 1, 512, 1, 1), id="mla_packed"),
+    pytest.param((4, 8, 16, 1, 512, 2, 1), id="mla_kv_sep"),
+    pytest.param((4, 8, 16, 8, 128, 1, 8), id="mha_packed"),
+    pytest.param((4, 8, 16, 8, 128, 2, 8), id="mha_plain"),
+]
+
+
+@pytest.mark.parametrize("cfg", TP1_CONFIGS)
+@pytest.mark.parametrize("cpu_name", ["LAYERFIRST", "BLOCKFIRST"])
+@pytest.mark.parametrize("use_ce", [False, True], ids=["kernel", "ce"])
+def test_tp1_roundtrip(gpu_device, cfg, cpu_name, use_ce):
+    """Shape of the reference's test_tp1_roundtrip (:739-800): D2H, clear, H2D,
+    spot-check the fill formula; plus byte equality with the original."""
+    L, N, T, H, D, kv_dim, heads = cfg
+    gl, cl = make_layouts(L, N, T, H, D, cpu_name, kv_dim, heads)
+    gpu = make_gpu_tensors(L, N, T, H, D, kv_dim, gpu_device)
+    fill_gpu(gpu, 0, L, N, T, H, D, kv_dim)
+    orig = [t.clone() for t in gpu]
+    cpu = torch.zeros(cl.kv_shape, dtype=DTYPE, pin_memory=True)
+    ids = torch.arange(N, dtype=torch.int64)
+    strides = dict(cpu_kv_stride_in_bytes=cl.get_kv_stride() * ES,
+                   cpu_layer_stride_in_bytes=cl.get_layer_stride() * ES,
+                   cpu_block_stride_in_bytes=cl.get_block_stride() * ES,
+                   cpu_tp_stride_in_bytes=cl.get_block_stride() * ES)
+    tp = tp_group(cpu, [gpu], gl, L, [0], is_blockfirst=(cpu_name == "BLOCKFIRST"),
+                  num_kv_heads=heads)
+    common = dict(transfer_num_cta=4, use_ce_transfer=use_ce, layer_id=0, layer_granularity=L,
+                  kv_dim=kv_dim, num_kv_heads=heads, kv_shared_across_ranks_mode="sharded")
+    tp.tp_group_transfer(gpu_block_id_tensor=ids, cpu_block_id_tensor=ids, is_host_to_device=False,
+                         **strides, **common)
+    # host image: element [b, l, kv, ...] (block-first) or [l, kv, b, ...] equals the fill formula
+    for layer in (0, L - 1):
+        for block in (0, N - 1):
+            for kv in range(kv_dim):
+                for d in (0, D - 1):
+                    got = (cpu[block, layer, kv, 0, 0, d] if cpu_name == "BLOCKFIRST"
+                           else cpu[layer, kv, block, 0, 0, d]).item()
+                    assert abs(got - expected_val(0, layer, block, 0, d, kv)) < 1e-3
+    for t in gpu:
+        t.zero_()
+    torch.cuda.synchronize()
+    tp.tp_group_transfer(gpu_block_id_tensor=ids, cpu_block_id_tensor=ids, is_host_to_device=True,
+                         **strides, **common)
+    for a, b in zip(gpu, orig):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    tp.close()
+
+
+def _oracle_tp(all_ref, host_ref, gl, cl_strides, ids_g, ids_c, n, heads, h2d, mode, designated,
+               rotate, layer_id, gran, kv_dim):
+    """What N ranks must leave on the host / in the 'GPU' buffers, computed rank
+    by rank with the oracle's placement rule and byte loop."""
+    ckv, clayer, cblock, ctp = cl_strides
+    chunk = gl.get_chunk_size() * ES
+    for r in range(n):
+        p = O.tp_rank_plan(r, n, heads, h2d, mode, designated, rotate, layer_id, gran, len(ids_g),
+                           chunk, cblock, ctp)
+        if not p.active:
+            continue
+        O.transfer_c(0, [a.ctypes.data for a in all_ref[r]], gl.num_layer,
+                     gl.get_kv_stride() * ES, gl.get_block_stride() * ES,
+                     gl.get_layer_stride() * ES, p.gpu_startoff, host_ref.ctypes.data, ckv, clayer,
+                     cblock, p.cpu_startoff, p.chunk_size, p.start_layer, p.num_layers, kv_dim,
+                     ids_g, ids_c, h2d)
+
+
+@pytest.mark.parametrize("mode", ["sharded", "all_write", "rank0_only", "layer_parallel",
+                                  "rank_rotate"])
+@pytest.mark.parametrize("cpu_name", ["LAYERFIRST", "BLOCKFIRST"])
+@pytest.mark.parametrize("use_ce", [False, True], ids=["kernel", "ce"])
+def test_shared_kv_modes_with_four_ranks_on_one_device(gpu_device, mode, cpu_name, use_ce):
+    """Four ranks that hold identical MLA KV, all placed on device 0: the host
+    image after a put and the GPU bytes after a get equal the oracle's."""
+    n, L, N, T, H, D, kv_dim, heads = 4, 5, 12, 16, 1, 64, 1, 1
+    copies = n if mode == "all_write" else 1
+    gl, cl = make_layouts(L, N, T, H, D, cpu_name, kv_dim, heads, cpu_blocks=N * copies)
+    rng = np.random.default_rng(12)
+    nbytes = L * kv_dim * N * T * H * D * ES
+    base = rng.integers(0, 256, size=nbytes, dtype=np.uint8)
+    layer_bytes = nbytes // L
+    all_ref = [[base[l * layer_bytes:(l + 1) * layer_bytes].copy() for l in range(L)]
+               for _ in range(n)]
+    all_gpu = [[torch.from_numpy(a.copy()).to(gpu_device) for a in rank] for rank in all_ref]
+    host_ref = rng.integers(0, 256, size=cl.get_total_elements() * ES, dtype=np.uint8)
+    cpu = torch.empty(host_ref.size, dtype=torch.uint8, pin_memory=True)
+    cpu.copy_(torch.from_numpy(host_ref))
+    cl_strides = (cl.get_kv_stride() * ES, cl.get_layer_stride() * ES, cl.get_block_stride() * ES,
+                  cl.get_block_stride() * ES // n)
+    ids_g = rng.permutation(N)[:7].astype(np.int64)
+    ids_c = rng.permutation(N)[:7].astype(np.int64)
+    if mode == "all_write":
+        # rank r's region starts r * num_blocks blocks further on, so the host ids of
+        # one transfer must stay below num_blocks or the regions would overlap
+        ids_c = rng.permutation(7).astype(np.int64)
+    tp = tp_group(cpu, all_gpu, gl, L, [0] * n, is_blockfirst=(cpu_name == "BLOCKFIRST"),
+                  num_kv_heads=heads)
+    kw = dict(cpu_kv_stride_in_bytes=cl_strides[0], cpu_layer_stride_in_bytes=cl_strides[1],
+              cpu_block_stride_in_bytes=cl_strides[2], cpu_tp_stride_in_bytes=cl_strides[3],
+              transfer_num_cta=2, use_ce_transfer=use_ce, layer_id=0, layer_granularity=L,
+              kv_dim=kv_dim, num_kv_heads=heads, kv_shared_across_ranks_mode=mode,
+              designated_rank=2)
+    g, c = torch.from_numpy(ids_g), torch.from_numpy(ids_c)
+    for call in range(2):  # two puts: rank_rotate moves on to the next writer
+        print(f"case mode={mode} {cpu_name} ce={use_ce} put#{call}", flush=True)
+        tp.tp_group_transfer(g, c, is_host_to_device=False, **kw)
+        _oracle_tp(all_ref, host_ref, gl, cl_strides, ids_g, ids_c, n, heads, False, mode, 2,
+                   call % n, 0, L, kv_dim)
+        np.testing.assert_array_equal(cpu.numpy(), host_ref)
+    if mode in ("sharded", "all_write", "rank0_only"):  # the get side of these modes
+        ids_g2 = rng.permutation(N)[:7].astype(np.int64)
+        tp.tp_group_transfer(torch.from_numpy(ids_g2), c, is_host_to_device=True, **kw)
+        _oracle_tp(all_ref, host_ref, gl, cl_strides, ids_g2, ids_c, n, heads, True, mode, 2, 0, 0,
+                   L, kv_dim)
+        for r in range(n):
+            for l in range(L):
+                np.testing.assert_array_equal(all_gpu[r][l].cpu().numpy(), all_ref[r][l])
+    tp.close()
+
+
+def test_multi_head_ranks_write_head_slices(gpu_device):
+    """Two ranks with half the heads each fill one host block-first pool."""
+    n, L, N, T, H, D, kv_dim = 2, 3, 8, 4, 4, 16, 2
+    gl = KVCacheLayout(KVCacheLayoutType.LAYERFIRST, L, N, T, H // n, D, kv_dim=kv_dim, num_kv_heads=H)
+    cl = KVCacheLayout(KVCacheLayoutType.BLOCKFIRST, L, N, T, H, D, kv_dim=kv_dim, num_kv_heads=H)
+    cl_tp = cl.div_head(n)
+    rng = np.random.default_rng(13)
+    per_layer = kv_dim * N * T * (H // n) * D * ES
+    all_ref = [[rng.integers(0, 256, size=per_layer, dtype=np.uint8) for _ in range(L)]
+               for _ in range(n)]
+    all_gpu = [[torch.from_numpy(a.copy()).to(gpu_device) for a in rank] for rank in all_ref]
+    host_ref = np.zeros(cl.get_total_elements() * ES, dtype=np.uint8)
+    cpu = torch.zeros(host_ref.size, dtype=torch.uint8, pin_memory=True)
+    strides = (cl_tp.get_kv_stride() * ES, cl_tp.get_layer_stride() * ES,
+               cl.get_block_stride() * ES, cl.get_block_stride() * ES // n)
+    ids = np.array([5, 2, 7], dtype=np.int64)
+    tp = tp_group(cpu, all_gpu, gl, L, [0, 0], is_blockfirst=True, num_kv_heads=H)
+    tp.tp_group_transfer(torch.from_numpy(ids), torch.from_numpy(ids), strides[0], strides[1],
+                         strides[2], strides[3], 4, False, False, 0, L, kv_dim, H)
+    _oracle_tp(all_ref, host_ref, gl, strides, ids, ids, n, H, False, "sharded", 0, 0, 0, L, kv_dim)
+    np.testing.assert_array_equal(cpu.numpy(), host_ref)
+    # every byte of the three host blocks was written exactly by one of the two ranks
+    blk = cl.get_block_stride() * ES
+    for b in ids:
+        assert cpu.numpy()[b * blk:(b + 1) * blk].any()
+    tp.close()
+
+
+def test_tp_group_errors_and_pointer_update(gpu_device):
+    from flexkv_amd.c_ext import TPTransferThreadGroup
+    L, N, T, H, D = 2, 4, 4, 1, 32
+    gl, cl = make_layouts(L, N, T, H, D, "BLOCKFIRST", 1, 1)
+    gpu_a = make_gpu_tensors(L, N, T, H, D, 1, gpu_device)
+    gpu_b = make_gpu_tensors(L, N, T, H, D, 1, gpu_device)
+    fill_gpu(gpu_a, 0, L, N, T, H, D, 1)
+    fill_gpu(gpu_b, 1, L, N, T, H, D, 1)
+    cpu = torch.zeros(cl.kv_shape, dtype=DTYPE, pin_memory=True)
+    with pytest.raises(RuntimeError, match="Unsupported GPU block type: 3"):
+        TPTransferThreadGroup(1, [1, 2, 3], 3, cpu.data_ptr(), 2, [8], [8], [8], [8], [0])
+    with pytest.raises(RuntimeError, match="nvcomp"):
+        tp_group(cpu, [gpu_a], gl, L, [0]).__class__(1, [1, 2], 2, cpu.data_ptr(), 2, [8], [8], [8],
+                                                     [8], [0], enable_nvcomp=True)
+    tp = tp_group(cpu, [gpu_a], gl, L, [0], is_blockfirst=True)
+    ids = torch.arange(N, dtype=torch.int64)
+    args = (cl.get_kv_stride() * ES, cl.get_layer_stride() * ES, cl.get_block_stride() * ES,
+            cl.get_block_stride() * ES, 4, False, False, 0, L, 1, 1)
+    tp.tp_group_transfer(ids, ids, *args)
+    assert abs(cpu[1, 1, 0, 0, 0, 3].item() - expected_val(0, 1, 1, 0, 3, 0)) < 1e-3
+    with pytest.raises(ValueError, match="GPU pointer count does not match"):
+        tp.update_gpu_block_ptrs([gpu_b[0].data_ptr()])          # tp_transfer_thread_group.cpp:144-146
+    tp.update_gpu_block_ptrs([t.data_ptr() for t in gpu_b])      # "resume" with new mappings
+    tp.tp_group_transfer(ids, ids, *args)
+    assert abs(cpu[1, 1, 0, 0, 0, 3].item() - expected_val(1, 1, 1, 0, 3, 0)) < 1e-3
+    tp.close()
+
+
+# ---------------------------------------------------------------------------
+# LayerwiseTransferGroup
+# ---------------------------------------------------------------------------
+_libc = ctypes.CDLL("libc.so.6", use_errno=True)
+EFD_SEMAPHORE, EFD_NONBLOCK = 0x1, 0o4000
+
+
+def make_eventfds(counters, tp, L):
+    fds = [_libc.eventfd(0, EFD_SEMAPHORE | EFD_NONBLOCK) for _ in range(counters * tp * L)]
+    assert all(fd >= 0 for fd in fds)
+    return torch.tensor(fds, dtype=torch.int32).view(counters, tp, L), fds
+
+
+def drain(fd):
+    total = 0
+    while True:
+        try:
+            total += struct.unpack("Q", os.read(fd, 8))[0]
+        except BlockingIOError:
+            return total
+
+
+def layerwise_group(cpu, all_gpu, gl, L, eventfds=None, tp_size=None, **kw):
+    from flexkv_amd.c_ext import LayerwiseTransferGroup
+    n = len(all_gpu)
+    st = lambda v: torch.tensor([v * ES] * n, dtype=torch.int64)
+    empty = torch.empty(0)
+    return LayerwiseTransferGroup(
+        num_gpus=n, gpu_blocks=all_gpu, cpu_blocks=cpu, ssd_files={}, num_layers=L,
+        gpu_kv_strides_tensor=st(gl.get_kv_stride()), gpu_block_strides_tensor=st(gl.get_block_stride()),
+        gpu_layer_strides_tensor=st(gl.get_layer_stride()),
+        gpu_chunk_sizes_tensor=st(gl.get_chunk_size()), iouring_entries=0, iouring_flags=0,
+        layer_eventfds_tensor=eventfds if eventfds is not None else torch.empty(0, dtype=torch.int32),
+        tp_size=tp_size or n, has_swa=False, swa_gpu_blocks=[], swa_cpu_blocks=empty,
+        swa_ssd_files={}, swa_gpu_kv_strides_tensor=empty, swa_gpu_block_strides_tensor=empty,
+        swa_gpu_layer_strides_tensor=empty, swa_gpu_chunk_sizes_tensor=empty, **kw)
+
+
+def run_layerwise(lw, gids, cids, cl, chunk_bytes, L, kv_dim, heads, use_ce, gran, notify,
+                  counter_id=0, mode="sharded", tp_stride=None):
+    e = torch.empty(0, dtype=torch.int64)
+    lw.layerwise_transfer(
+        e, e, 0, 0, 0, 0, 0, gids, cids, cl.get_kv_stride() * ES, cl.get_layer_stride() * ES,
+        cl.get_block_stride() * ES, chunk_bytes, cl.get_kv_stride() * ES,
+        cl.get_layer_stride() * ES, tp_stride or cl.get_block_stride() * ES, 4, use_ce, L, gran,
+        kv_dim, heads, counter_id=counter_id, swa_h2d_src=e, swa_h2d_dst=e, swa_disk2h_src=e,
+        swa_disk2h_dst=e, kv_shared_across_ranks_mode=mode, notify_mode=notify)
+
+
+@pytest.mark.parametrize("kv_dim", [1, 2], ids=["mla", "kv_sep_1h"])
+@pytest.mark.parametrize("use_ce", [False, True], ids=["kernel", "ce"])
+@pytest.mark.parametrize("notify", ["hostfunc", "polling"])
+@pytest.mark.parametrize("gran", [1, 3, 4])
+def test_layerwise_restore_roundtrip(gpu_device, kv_dim, use_ce, notify, gran):
+    """Shape of test_layerwise_h2d_notify_modes (:808-895): put with the TP group,
+    clear, restore layer by layer, compare every byte."""
+    L, N, T, H, D, heads = 4, 8, 16, 1, 512, 1
+    gl, cl = make_layouts(L, N, T, H, D, "BLOCKFIRST", kv_dim, heads)
+    gpu = make_gpu_tensors(L, N, T, H, D, kv_dim, gpu_device)
+    fill_gpu(gpu, 0, L, N, T, H, D, kv_dim)
+    orig = [t.clone() for t in gpu]
+    cpu = torch.zeros(cl.kv_shape, dtype=DTYPE, pin_memory=True)
+    gids = torch.tensor([5, 0, 7, 2, 3], dtype=torch.int64)
+    cids = torch.tensor([1, 6, 2, 0, 4], dtype=torch.int64)
+    tp = tp_group(cpu, [gpu], gl, L, [0], is_blockfirst=True, num_kv_heads=heads)
+    tp.tp_group_transfer(gids, cids, cl.get_kv_stride() * ES, cl.get_layer_stride() * ES,
+                         cl.get_block_stride() * ES, cl.get_block_stride() * ES, 4, False, use_ce,
+                         0, L, kv_dim, heads)
+    tp.close()
+    for t in gpu:
+        t.zero_()
+    torch.cuda.synchronize()
+    fds_t, fds = make_eventfds(3, 1, L)
+    lw = layerwise_group(cpu, [gpu], gl, L, eventfds=fds_t, is_blockfirst=True, num_kv_heads=heads)
+    run_layerwise(lw, gids, cids, cl, gl.get_chunk_size() * ES, L, kv_dim, heads, use_ce, gran,
+                  notify, counter_id=1)
+    lw.synchronize()
+    for l in range(L):
+        got, want = gpu[l][:, gids.to(gpu_device)], orig[l][:, gids.to(gpu_device)]
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+        mask = torch.ones(N, dtype=torch.bool)
+        mask[gids] = False
+        assert not gpu[l][:, mask.to(gpu_device)].view(torch.int16).any()  # other blocks untouched
+    # exactly one unit per layer on the selected counter, nothing elsewhere
+    units = np.array([drain(fd) for fd in fds]).reshape(3, 1, L)
+    assert units[1].tolist() == [[1] * L] and not units[0].any() and not units[2].any()
+    lw.close()
+    for fd in fds:
+        os.close(fd)
+
+
+def test_layerwise_notifications(gpu_device):
+    """One write(1) per (layer, tp_rank) per transfer, also for an empty block
+    list and for repeated transfers; negative fds are skipped
+    (csrc/layerwise.cpp:15-34, 105-123)."""
+    L, N, T, H, D = 6, 8, 4, 1, 64
+    gl, cl = make_layouts(L, N, T, H, D, "BLOCKFIRST", 1, 1)
+    gpu = make_gpu_tensors(L, N, T, H, D, 1, gpu_device)
+    cpu = torch.zeros(cl.kv_shape, dtype=DTYPE, pin_memory=True)
+    fds_t, fds = make_eventfds(2, 2, L)        # tp_size 2 consumers listen to one transfer GPU
+    fds_t[0, 1, 3] = -1
+    lw = layerwise_group(cpu, [gpu], gl, L, eventfds=fds_t, tp_size=2, is_blockfirst=True)
+    ids = torch.arange(4, dtype=torch.int64)
+    none = torch.empty(0, dtype=torch.int64)
+    for notify in ("hostfunc", "polling"):
+        for blocks in (ids, none):
+            run_layerwise(lw, blocks, blocks, cl, gl.get_chunk_size() * ES, L, 1, 1, False, 2,
+                          notify, counter_id=0)
+            lw.synchronize()
+            units = np.array([drain(fd) for fd in fds]).reshape(2, 2, L)
+            want = np.ones((2, L), dtype=int)
+            want[1, 3] = 0                     # its table entry is -1; the fd itself stays idle
+            assert units[0].tolist() == want.tolist(), (notify, blocks.numel())
+            assert not units[1].any()
+    # a restore of the first layers only announces only those layers
+    run_layerwise(lw, ids, ids, cl, gl.get_chunk_size() * ES, 3, 1, 1, False, 1, "polling",
+                  counter_id=1)
+    lw.synchronize()
+    units = np.array([drain(fd) for fd in fds]).reshape(2, 2, L)
+    assert units[1].tolist() == [[1, 1, 1, 0, 0, 0]] * 2 and not units[0].any()
+    with pytest.raises(ValueError, match="counter_id"):
+        run_layerwise(lw, ids, ids, cl, gl.get_chunk_size() * ES, L, 1, 1, False, 1, "polling",
+                      counter_id=2)
+    lw.close()
+    for fd in fds:
+        os.close(fd)
+
+
+def test_layerwise_wait_layer_orders_a_consumer_stream(gpu_device):
+    """A consumer stream gated on wait_layer(l) sees layer l restored."""
+    L, N, T, H, D = 8, 64, 16, 1, 512
+    gl, cl = make_layouts(L, N, T, H, D, "BLOCKFIRST", 1, 1)
+    gpu = make_gpu_tensors(L, N, T, H, D, 1, gpu_device)
+    g = torch.Generator().manual_seed(3)
+    cpu = torch.empty(cl.kv_shape, dtype=DTYPE, pin_memory=True)
+    cpu.view(torch.int16).copy_(torch.randint(-2 ** 15, 2 ** 15, cl.kv_shape, generator=g,
+                                              dtype=torch.int16))
+    ids = torch.randperm(N, generator=g).to(torch.int64)
+    lw = layerwise_group(cpu, [gpu], gl, L, is_blockfirst=True)
+    consumer = torch.cuda.Stream()
+    snaps = []
+    for notify in ("polling", "hostfunc"):
+        for t in gpu:
+            t.zero_()
+        torch.cuda.synchronize()
+        run_layerwise(lw, ids, ids, cl, gl.get_chunk_size() * ES, L, 1, 1, False, 1, notify)
+        with torch.cuda.stream(consumer):
+            for l in range(L):
+                lw.wait_layer(l, consumer)
+                snaps.append(gpu[l].clone())
+        consumer.synchronize()
+        lw.synchronize()
+        for l in range(L):
+            want = cpu[:, l].transpose(0, 1).to(gpu_device)        # [kv, N, T, H, D] by host block
+            got = snaps[-L + l][:, ids.to(gpu_device)]
+            assert torch.equal(got.view(torch.int16), want[:, ids.to(gpu_device)].view(torch.int16))
+    times = lw.batch_times_ms()
+    assert len(times) == L and all(b >= a for a, b in zip(times, times[1:]))
+    with pytest.raises(ValueError, match="not part of the last transfer"):
+        lw.wait_layer(L, consumer)
+    lw.close()
+
+
+def test_layerwise_all_write_offsets_two_ranks(gpu_device):
+    """all_write restore: rank r reads its own region of the host pool
+    (csrc/layerwise.cpp:1155-1162)."""
+    n, L, N, T, H, D = 2, 3, 6, 4, 1, 64
+    gl, cl = make_layouts(L, N, T, H, D, "BLOCKFIRST", 1, 1, cpu_blocks=N * n)
+    all_gpu = [make_gpu_tensors(L, N, T, H, D, 1, gpu_device) for _ in range(n)]
+    g = torch.Generator().manual_seed(4)
+    cpu = torch.empty(cl.kv_shape, dtype=DTYPE, pin_memory=True)
+    cpu.view(torch.int16).copy_(torch.randint(-2 ** 15, 2 ** 15, cl.kv_shape, generator=g,
+                                              dtype=torch.int16))
+    ids = torch.tensor([4, 1, 3], dtype=torch.int64)
+    cids = torch.tensor([0, 2, 1], dtype=torch.int64)
+    lw = layerwise_group(cpu, all_gpu, gl, L, is_blockfirst=True)
+    run_layerwise(lw, ids, cids, cl, gl.get_chunk_size() * ES, L, 1, 1, False, 1, "hostfunc",
+                  mode="all_write")
+    region_blocks = ids.numel()                 # rank r's blocks start r * num_blocks further on
+    for r in range(n):
+        for l in range(L):
+            want = cpu[cids + r * region_blocks, l, 0].to(gpu_device)
+            assert torch.equal(all_gpu[r][l][0, ids.to(gpu_device)].view(torch.int16),
+                               want.view(torch.int16))
+    lw.close()
+
+
+def test_layerwise_rejects_what_it_does_not_provide(gpu_device):
+    from flexkv_amd.c_ext import LayerwiseTransferGroup
+    L, N, T, H, D = 2, 4, 4, 1, 32
+    gl, cl = make_layouts(L, N, T, H, D, "BLOCKFIRST", 1, 1)
+    gpu = make_gpu_tensors(L, N, T, H, D, 1, gpu_device)
+    cpu = torch.zeros(cl.kv_shape, dtype=DTYPE, pin_memory=True)
+    with pytest.raises(RuntimeError, match="multi-group"):
+        LayerwiseTransferGroup(num_gpus=1, gpu_blocks_per_group=[[gpu]], cpu_blocks=cpu)
+    st = torch.tensor([8], dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="SSD"):
+        LayerwiseTransferGroup(1, [gpu], cpu, {0: ["/tmp/x"]}, L, st, st, st, st, 0, 0,
+                               torch.empty(0, dtype=torch.int32), 1)
+    with pytest.raises(RuntimeError, match="Unsupported GPU block type: 3"):
+        LayerwiseTransferGroup(1, [gpu + [gpu[0]]], cpu, {}, L, st, st, st, st, 0, 0,
+                               torch.empty(0, dtype=torch.int32), 1)
+    lw = layerwise_group(cpu, [gpu], gl, L)
+    with pytest.raises(RuntimeError, match="single-group instance"):
+        lw.layerwise_transfer_multi_group()
+    lw.close()
