@@ -266,7 +266,7 @@ def verify_round_trip(w, torch, num_cta):
     return bool(ok)
 
 
-def run_layerwise(w, torch, steps, warmup, num_cta, notify):
+def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy):
     """c3: per-layer restore with a dummy per-layer compute kernel on a second
     stream gated on each layer's event."""
     from flexkv_amd.c_ext import LayerwiseTransferGroup
@@ -286,57 +286,76 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify):
             kv_shared_across_ranks_mode="sharded", notify_mode=notify)
 
     layer_bytes = w.num_blocks * w.kv_dim * w.chunk
-    # dummy compute: square matmuls on a side stream, sized to about one layer's copy time
+    # Dummy per-layer compute on a second stream, sized to about one layer's copy
+    # time: fused attention (default; what a restored layer feeds), a 2048^3 GEMM
+    # chain, or a streaming elementwise kernel.
     comp = torch.cuda.Stream()
-    n = 2048
-    a = torch.randn(n, n, device=w.device, dtype=torch.bfloat16)
-    b = torch.randn(n, n, device=w.device, dtype=torch.bfloat16)
-    c = torch.empty(n, n, device=w.device, dtype=torch.bfloat16)
     ev = lambda: torch.cuda.Event(enable_timing=True)
+    target_ms = layer_bytes / 55e9 * 1e3
+    if dummy == "sdpa":
+        q = torch.randn(1, 32, 2048, 128, device=w.device, dtype=torch.bfloat16)
+        unit = lambda: torch.nn.functional.scaled_dot_product_attention(q, q, q)
+    elif dummy == "gemm":
+        n = 2048
+        a = torch.randn(n, n, device=w.device, dtype=torch.bfloat16)
+        b = torch.randn(n, n, device=w.device, dtype=torch.bfloat16)
+        c = torch.empty(n, n, device=w.device, dtype=torch.bfloat16)
+        unit = lambda: torch.matmul(a, b, out=c)
+    else:
+        x = torch.randn(16 << 20, device=w.device)
+        unit = lambda: x.mul_(1.0001)
+
+    def layer_compute(reps):
+        for _ in range(reps):
+            unit()
 
     def compute_only(reps):
         with torch.cuda.stream(comp):
             s, e = ev(), ev()
             s.record(comp)
             for _ in range(w.L):
-                for _ in range(reps):
-                    torch.matmul(a, b, out=c)
+                layer_compute(reps)
             e.record(comp)
         e.synchronize()
         return s.elapsed_time(e)
 
     compute_only(1)
-    target_ms = layer_bytes / 55e9 * 1e3
-    per_mm = compute_only(4) / (4 * w.L)
-    reps = max(1, int(round(target_ms / per_mm)))
+    per_unit = compute_only(4) / (4 * w.L)
+    reps = max(1, int(round(target_ms / per_unit)))
     compute_ms = _median([compute_only(reps) for _ in range(3)])
 
-    totals, restores, firsts = [], [], []
+    totals, restores, firsts, stalls, busy = [], [], [], [], []
     for it in range(warmup + steps):
         torch.cuda.synchronize()
         s, e = ev(), ev()
-        t0 = time.perf_counter()
+        spans = []
         with torch.cuda.stream(comp):
             s.record(comp)
         restore()  # polling: returns right after the launches
         with torch.cuda.stream(comp):
             for l in range(w.L):
                 grp.wait_layer(l, comp)
-                for _ in range(reps):
-                    torch.matmul(a, b, out=c)
+                a0, a1 = ev(), ev()
+                a0.record(comp)        # stamped once layer l has landed
+                layer_compute(reps)
+                a1.record(comp)
+                spans.append((a0, a1))
             e.record(comp)
         e.synchronize()
         grp.synchronize()
-        wall = (time.perf_counter() - t0) * 1e3
         if it >= warmup:
             bt = grp.batch_times_ms()
-            totals.append(s.elapsed_time(e))
+            total = s.elapsed_time(e)
+            computing = sum(x.elapsed_time(y) for x, y in spans)
+            totals.append(total)
             restores.append(bt[-1])
             firsts.append(bt[0])
-            _ = wall
+            busy.append(computing)
+            stalls.append(total - computing)  # compute stream idle, waiting for a layer
     grp.close()
     return dict(total_ms=_median(totals), restore_ms=_median(restores),
                 first_layer_ms=_median(firsts), compute_ms=compute_ms,
+                compute_overlapped_ms=_median(busy), stall_ms=_median(stalls),
                 compute_reps_per_layer=reps, layer_bytes=layer_bytes)
 
 
@@ -425,11 +444,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4"])
+    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal"])
     ap.add_argument("--num-cta", type=int, default=4,
                     help="transfer_num_cta (reference default FLEXKV_TRANSFER_NUM_CTA_*=4)")
     ap.add_argument("--use-ce", action="store_true", help="copy-engine path instead of the kernel")
     ap.add_argument("--notify", default="polling", choices=["polling", "hostfunc"])
+    ap.add_argument("--dummy", default="sdpa", choices=["sdpa", "gemm", "elementwise"],
+                    help="c3: the per-layer compute kernel the restore is overlapped with")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     args = ap.parse_args()
@@ -444,6 +465,19 @@ def main():
     device = "cuda:0"
     torch.cuda.set_device(0)
 
+    if args.config == "copycal":
+        # Plain device-to-device copies of a known size: the yardstick the
+        # FETCH_SIZE / WRITE_SIZE counters of the transfer kernel are scaled by.
+        n = 1 << 30
+        src = torch.randint(0, 256, (n,), device=device, dtype=torch.uint8)
+        dst = torch.empty_like(src)
+        for _ in range(max(1, args.steps)):
+            dst.copy_(src)                         # runtime blit kernel
+            torch.bitwise_or(src, 0, out=dst)      # elementwise kernel, reads n and writes n bytes
+        torch.cuda.synchronize()
+        print(json.dumps({"config": {"workload": "copycal"}, "copy_bytes": n,
+                          "copies_of_each_kind": max(1, args.steps)}))
+        return
     link = measure_link()
     w = Workload(args.config, torch, device)
     B = w.bytes_per_direction
@@ -489,18 +523,24 @@ def main():
         saved = [w.gpu_rows(l, 0).index_select(0, gi) for l in range(w.L)]
         for l in range(w.L):
             w.gpu_rows(l, 0).index_fill_(0, gi, 0)
-        r = run_layerwise(w, torch, args.steps, args.warmup, args.num_cta, args.notify)
-        exposed = r["total_ms"] - r["compute_ms"]
+        r = run_layerwise(w, torch, args.steps, args.warmup, args.num_cta, args.notify, args.dummy)
         restore = B / (r["restore_ms"] * 1e-3) / 1e9
+        stall_beyond_first = max(0.0, r["stall_ms"] - r["first_layer_ms"])
         out.update(value=round(restore, 3), ms_per_step=round(r["total_ms"], 3),
                    h2d_GBps=round(restore, 3), h2d_frac_of_link=round(restore / link["h2d"], 4),
-                   layerwise={"notify": args.notify, "restore_ms": round(r["restore_ms"], 3),
+                   layerwise={"notify": args.notify, "dummy_compute": args.dummy,
+                              "compute_units_per_layer": r["compute_reps_per_layer"],
+                              "restore_ms": round(r["restore_ms"], 3),
                               "first_layer_ms": round(r["first_layer_ms"], 3),
-                              "compute_only_ms": round(r["compute_ms"], 3),
+                              "compute_alone_ms": round(r["compute_ms"], 3),
+                              "compute_while_restoring_ms": round(r["compute_overlapped_ms"], 3),
+                              "compute_slowdown": round(
+                                  r["compute_overlapped_ms"] / r["compute_ms"], 3),
                               "restore_plus_compute_ms": round(r["total_ms"], 3),
-                              "exposed_ms": round(exposed, 3),
+                              "compute_stream_stall_ms": round(r["stall_ms"], 3),
+                              "stall_beyond_first_layer_ms": round(stall_beyond_first, 3),
                               "overlap_frac_beyond_first_layer": round(
-                                  1.0 - max(0.0, exposed - r["first_layer_ms"]) /
+                                  1.0 - stall_beyond_first /
                                   max(1e-9, r["restore_ms"] - r["first_layer_ms"]), 4)})
         if not args.no_verify:
             out["bit_exact"] = all(

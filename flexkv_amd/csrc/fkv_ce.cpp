@@ -387,6 +387,11 @@ int device_staging_copy(const fkv_transfer_desc &d, int it0, int nit, int p0, in
     int n = (v && *v) ? std::atoi(v) : 2048;
     return n > 0 ? n : 2048;
   }();
+  static const int kStagingThreads = [] {
+    const char *v = std::getenv("FKV_STAGING_THREADS");
+    int n = (v && *v) ? std::atoi(v) : 1024;
+    return n > 0 ? n : 1024;
+  }();
   int device = 0;
   FKV_HIP_TRY(hipGetDevice(&device));
   for (int b0 = 0; b0 < nit; b0 += kCopyMaxLK) {
@@ -427,7 +432,8 @@ int device_staging_copy(const fkv_transfer_desc &d, int it0, int nit, int p0, in
       a.num_blocks = np;
       a.lk = lk;
       a.vec = common_vector_width(&acc, 1);
-      rc = launch_copy_kernel(a, kStagingWorkgroups, stream);
+      a.nt_store = 1;
+      rc = launch_copy_kernel(a, kStagingWorkgroups, kStagingThreads, stream);
     }
     plan_release(slot, stream, false);
     if (rc != FKV_OK)

@@ -215,6 +215,35 @@ int default_num_cta(bool is_h2d) {
   return is_h2d ? h2d : d2h;
 }
 
+// Measured on MI355X with 4 requested CTAs: GB/s over the link (a plain pinned
+// hipMemcpy reaches 57.0 GPU->host / 57.3 host->GPU) and the slowdown of a kernel
+// running next to the copy (a 2048^3 bf16 GEMM / fused attention / a streaming
+// elementwise kernel):
+//   host->GPU  16 x  64 lanes : 57.2 GB/s,  1.9x /  1.10x /  1.05x   <- default
+//              24 x  64       : 57.4 GB/s,  2.9x /  1.16x /  1.10x
+//              12 x 1024      : 57.1 GB/s, 16x   /  2.1x  / 11x (stalled until the copy ends)
+//   GPU->host  48 x  64 lanes : 56.4 GB/s, streaming neighbour 2.7x   <- default
+//              24 x  64       : 54.7 GB/s, streaming neighbour 1.9x
+//              12 x 1024      : 56.6 GB/s, streaming neighbour 4.2x
+// So every requested CTA becomes four (host->GPU) or twelve (GPU->host)
+// single-wavefront workgroups.  FKV_{H2D,D2H}_WG_PER_CTA and
+// FKV_{H2D,D2H}_WG_THREADS override this (read once, or on every call when
+// FKV_TUNE_DYNAMIC=1).
+LinkLaunchShape link_launch_shape(bool is_h2d) {
+  static const bool dynamic = env_int("FKV_TUNE_DYNAMIC", 0) != 0;
+  auto read = [](bool h2d) {
+    LinkLaunchShape s;
+    s.workgroups_per_cta =
+        h2d ? env_int("FKV_H2D_WG_PER_CTA", 4) : env_int("FKV_D2H_WG_PER_CTA", 12);
+    s.threads = env_int(h2d ? "FKV_H2D_WG_THREADS" : "FKV_D2H_WG_THREADS", 64);
+    if (s.workgroups_per_cta < 1)
+      s.workgroups_per_cta = 1;
+    return s;
+  };
+  static const LinkLaunchShape fixed[2] = {read(false), read(true)};
+  return dynamic ? read(is_h2d) : fixed[is_h2d ? 1 : 0];
+}
+
 int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream) {
   set_last_path(FKV_PATH_KERNEL);
   // Device-visible alias of the host pool.  hipHostMalloc / torch pinned memory
@@ -230,12 +259,12 @@ int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream) {
   }
   const bool h2d = d.is_host_to_device != 0;
   static const bool mirror_plan = env_int("FKV_PLAN_MIRROR", 1) != 0;
-  // A CTA of the reference is 1024 threads = 32 warps (csrc/transfer.cu:176).  A
-  // workgroup here is 1024 lanes = 16 wavefronts, so each requested CTA becomes
-  // kWorkgroupsPerCta workgroups: the same number of independent instruction
-  // streams, which is what bounds the reads a CU keeps in flight over the link.
+  // A CTA of the reference is 1024 threads on one SM (csrc/transfer.cu:176) and
+  // its default of 4 CTAs is tuned for that hardware.  Here each requested CTA
+  // becomes `workgroups_per_cta` small workgroups (see link_launch_shape).
+  const LinkLaunchShape shape = link_launch_shape(h2d);
   const int num_cta = (d.transfer_num_cta > 0 ? d.transfer_num_cta : default_num_cta(h2d)) *
-                      kWorkgroupsPerCta;
+                      shape.workgroups_per_cta;
 
   // Layers go out in groups whose (layer, kv) base tables fit the kernel's LDS.
   const int layers_per_launch = kCopyMaxLK / d.kv_dim;
@@ -295,7 +324,8 @@ int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream) {
     a.num_blocks = d.num_blocks;
     a.lk = lk;
     a.vec = common_vector_width(align_bits, 4);
-    rc = launch_copy_kernel(a, num_cta, stream);
+    a.nt_store = h2d ? 1 : 0;
+    rc = launch_copy_kernel(a, num_cta, shape.threads, stream);
     plan_release(slot, stream, false);
     if (rc != FKV_OK)
       return rc;

@@ -111,14 +111,21 @@ struct CopyKernelArgs {
   int32_t num_blocks;
   int32_t lk;
   int32_t slices_per_chunk;
-  int32_t vec; // 16, 8, 4, 2 or 1: widest access all addresses allow
+  int32_t vec;      // 16, 8, 4, 2 or 1: widest access all addresses allow
+  int32_t nt_store; // 1: nontemporal stores (destination in HBM), 0: plain (pinned host)
 };
-constexpr int kCopyBlockThreads = 1024;  // 16 wavefronts, one CU
-constexpr int kWorkgroupsPerCta = 2;      // workgroups launched per requested CTA
+constexpr int kCopyBlockThreads = 1024;  // largest workgroup the kernel is built for
 constexpr int kCopyUnroll = 8;           // vector accesses in flight per lane
 constexpr int kCopyMaxLK = 1024;         // base-table entries staged in LDS
 constexpr int kCopyIdTile = 1024;        // block positions staged in LDS at a time
-int launch_copy_kernel(CopyKernelArgs args, int num_workgroups, hipStream_t stream);
+int launch_copy_kernel(CopyKernelArgs args, int num_workgroups, int threads_per_workgroup,
+                       hipStream_t stream);
+// Launch shape of the link-bound kernel for one direction.
+struct LinkLaunchShape {
+  int workgroups_per_cta; // workgroups launched per requested CTA
+  int threads;            // lanes per workgroup
+};
+LinkLaunchShape link_launch_shape(bool is_h2d);
 // Widest vector width (bytes) that divides every value in `vals`.
 int common_vector_width(const uint64_t *vals, int n);
 

@@ -15,15 +15,25 @@
 // address order inside a block-first host block.  Each workgroup owns one
 // contiguous run of slice numbers, hence a contiguous run of block positions
 // whose ids it stages in LDS (premultiplied by the block strides) together
-// with the two base tables; its 16 wavefronts take slices round-robin, so the
+// with the two base tables; its wavefronts take slices round-robin, so the
 // requests a workgroup has in flight target neighbouring addresses.  A
 // wavefront issues all kCopyUnroll loads of a slice before the first store, which
 // is what keeps enough reads outstanding to cover the host-link latency in
 // the host->GPU direction.
 //
-// Data moves as raw integer vectors with nontemporal loads and stores: KV
-// bytes are not reused by this kernel, and integer types cannot canonicalise
-// NaN payloads of fp8/bf16 data.
+// Launch shape.  The link is saturated by roughly 200 KB of requests in flight.
+// Requests to host memory sit in the memory-request queues of the XCD that
+// issued them until the link has served them, and every other kernel on that
+// XCD shares those queues: a few fat workgroups (16 wavefronts each) stall
+// memory-bound neighbours for the whole duration of the copy, while the same
+// number of bytes in flight spread as single-wavefront workgroups over all
+// XCDs costs them little.  The link-bound launches therefore use one
+// wavefront per workgroup; only the HBM-to-HBM staging pass uses big ones.
+//
+// Data moves as raw integer vectors (integer types cannot canonicalise NaN
+// payloads of fp8/bf16 data).  Loads are nontemporal: KV bytes are not reused
+// by this kernel.  Stores into HBM are nontemporal too; stores into pinned host
+// memory are plain, which measured about 1 GB/s faster over the link.
 #include "fkv_internal.h"
 
 namespace fkv {
@@ -38,7 +48,14 @@ template <> struct VecType<4>  { typedef unsigned int type; };
 template <> struct VecType<2>  { typedef unsigned short type; };
 template <> struct VecType<1>  { typedef unsigned char type; };
 
-template <int VEC>
+template <typename V, bool NT> __device__ __forceinline__ void put(V v, V *p) {
+  if (NT)
+    __builtin_nontemporal_store(v, p);
+  else
+    *p = v;
+}
+
+template <int VEC, bool NTS>
 __device__ __forceinline__ void copy_slice(const uint8_t *__restrict__ src,
                                            uint8_t *__restrict__ dst,
                                            int64_t bytes_in_slice, int lane) {
@@ -53,16 +70,15 @@ __device__ __forceinline__ void copy_slice(const uint8_t *__restrict__ src,
       r[u] = __builtin_nontemporal_load(s + u * kWave);
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u)
-      __builtin_nontemporal_store(r[u], d + u * kWave);
+      put<V, NTS>(r[u], d + u * kWave);
   } else {
     const int64_t nvec = bytes_in_slice / VEC;
     for (int64_t i = lane; i < nvec; i += kWave)
-      __builtin_nontemporal_store(__builtin_nontemporal_load(s + (i - lane)),
-                                  d + (i - lane));
+      put<V, NTS>(__builtin_nontemporal_load(s + (i - lane)), d + (i - lane));
   }
 }
 
-template <int VEC>
+template <int VEC, bool NTS>
 __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
     CopyKernelArgs a) {
   extern __shared__ uint64_t lds[];
@@ -116,15 +132,20 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
       const uint8_t *src =
           reinterpret_cast<const uint8_t *>(s_base_src[i] + (uint64_t)s_off_src[p]) + off;
       uint8_t *dst = reinterpret_cast<uint8_t *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + off;
-      copy_slice<VEC>(src, dst, left < kSliceBytes ? left : kSliceBytes, lane);
+      copy_slice<VEC, NTS>(src, dst, left < kSliceBytes ? left : kSliceBytes, lane);
     }
   }
 }
 
 template <int VEC>
-int launch_vec(const CopyKernelArgs &a, int grid, size_t lds_bytes, hipStream_t stream) {
-  hipLaunchKernelGGL(fkv_copy_chunks_kernel<VEC>, dim3(grid), dim3(kCopyBlockThreads),
-                     lds_bytes, stream, a);
+int launch_vec(const CopyKernelArgs &a, int grid, int threads, size_t lds_bytes,
+               hipStream_t stream) {
+  if (a.nt_store)
+    hipLaunchKernelGGL((fkv_copy_chunks_kernel<VEC, true>), dim3(grid), dim3(threads), lds_bytes,
+                       stream, a);
+  else
+    hipLaunchKernelGGL((fkv_copy_chunks_kernel<VEC, false>), dim3(grid), dim3(threads),
+                       lds_bytes, stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess)
     return fail(FKV_ERR_RUNTIME, "copy kernel launch failed: %s", hipGetErrorString(e));
@@ -143,7 +164,8 @@ int common_vector_width(const uint64_t *vals, int n) {
   return 1;
 }
 
-int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, hipStream_t stream) {
+int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_workgroup,
+                       hipStream_t stream) {
   if (a.num_blocks <= 0 || a.lk <= 0 || a.chunk_bytes <= 0)
     return FKV_OK;
   if (a.lk > kCopyMaxLK)
@@ -164,7 +186,13 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, hipStream_t stream)
                 (long long)a.chunk_bytes, a.lk);
   a.slices_per_chunk = (int32_t)slices;
   const int64_t total = spp * a.num_blocks;
-  const int waves_per_wg = kCopyBlockThreads / kWave;
+  int threads = threads_per_workgroup;
+  if (threads < kWave)
+    threads = kWave;
+  if (threads > kCopyBlockThreads)
+    threads = kCopyBlockThreads;
+  threads = threads / kWave * kWave;
+  const int waves_per_wg = threads / kWave;
   int64_t grid = num_workgroups > 0 ? num_workgroups : 1;
   const int64_t useful = (total + waves_per_wg - 1) / waves_per_wg;
   if (grid > useful)
@@ -174,11 +202,11 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, hipStream_t stream)
   const size_t lds_bytes = (size_t)(2 * a.lk + 2 * kCopyIdTile) * sizeof(uint64_t);
   stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);
   switch (a.vec) {
-  case 16: return launch_vec<16>(a, (int)grid, lds_bytes, stream);
-  case 8:  return launch_vec<8>(a, (int)grid, lds_bytes, stream);
-  case 4:  return launch_vec<4>(a, (int)grid, lds_bytes, stream);
-  case 2:  return launch_vec<2>(a, (int)grid, lds_bytes, stream);
-  default: return launch_vec<1>(a, (int)grid, lds_bytes, stream);
+  case 16: return launch_vec<16>(a, (int)grid, threads, lds_bytes, stream);
+  case 8:  return launch_vec<8>(a, (int)grid, threads, lds_bytes, stream);
+  case 4:  return launch_vec<4>(a, (int)grid, threads, lds_bytes, stream);
+  case 2:  return launch_vec<2>(a, (int)grid, threads, lds_bytes, stream);
+  default: return launch_vec<1>(a, (int)grid, threads, lds_bytes, stream);
   }
 }
 

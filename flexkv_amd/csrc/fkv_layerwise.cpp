@@ -324,7 +324,9 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
 
   if (notify_mode == FKV_NOTIFY_POLLING) {
     g->poller_stop.store(false, std::memory_order_release);
-    if (num_batches > 0)
+    // Nobody listens when no eventfd table was given: in-process consumers wait
+    // on the batch events directly, so there is nothing to poll for.
+    if (num_batches > 0 && !g->eventfds.empty())
       g->poller = std::thread([g] { g->poll_loop(); });
   } else {
     for (int i = 0; i < g->num_gpus; ++i) { // csrc/layerwise.cpp:1249-1256

@@ -104,8 +104,9 @@ typedef struct fkv_transfer_desc {
   /* how */
   int32_t is_host_to_device;
   int32_t use_ce_transfer;
-  int32_t transfer_num_cta; /* CTAs in the reference's unit (32 warps); each becomes two
-                               16-wavefront workgroups; <= 0 = library default (4) */
+  int32_t transfer_num_cta; /* CTAs as the reference counts them; each becomes 4 (host->GPU)
+                               or 12 (GPU->host) single-wavefront workgroups;
+                               <= 0 = library default (4) */
   int32_t sync;             /* 1: hipStreamSynchronize before returning */
   int32_t enable_trace;     /* 1: print an "[XFER]" line per call to stderr */
   int32_t reserved;
@@ -171,7 +172,8 @@ typedef struct fkv_tp_rank_plan {
 /* csrc/tp_transfer_thread_group.cpp:222-323 (offset / layer-range rules of
  * tp_group_transfer).  `mode` is the kv_shared_across_ranks_mode string;
  * `rotate_counter` is the value of the round-robin counter for rank_rotate.
- * Returns FKV_ERR_INVALID_ARG for the sharded/indivisible case (:237-247). */
+ * Returns FKV_ERR_RUNTIME for the sharded/indivisible case (:237-247 throws
+ * std::runtime_error). */
 int fkv_tp_rank_plan_compute(int32_t rank, int32_t num_gpus, int32_t num_kv_heads,
                              int32_t is_host_to_device, const char *mode,
                              int32_t designated_rank, int32_t rotate_counter,
