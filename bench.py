@@ -35,9 +35,9 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 METRIC = "KV block transfer GB/s (D2H, H2D) on 1 GPU; % of measured host-link peak"
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs of this script scaled by a plain copy kernel of known size;
-# see the summaries under profiles/.  None where no such run has been made.
-MEASURED_TRAFFIC_BYTES = {}
+# WRITE_SIZE runs of this script scaled by plain copy kernels of known size
+# (profiles/fkv_copy_chunks_kernel_c1_pmc.md).  None where no such run was made.
+MEASURED_TRAFFIC_BYTES = {("c1", "kernel"): 8591004672}
 
 
 def _median(xs):
@@ -503,7 +503,7 @@ def main():
         # dominant kernel: the gather/scatter kernel; one launch per direction moves B bytes
         avg_ms = (sum(d2h_ms) + sum(h2d_ms)) / (len(d2h_ms) + len(h2d_ms))
         achieved = B / (avg_ms * 1e-3) / 1e9
-        kernel = "fkv_copy_chunks_kernel<16>" if not args.use_ce else taken
+        kernel = "fkv_copy_chunks_kernel<16, false|true>" if not args.use_ce else taken
         out["roofline"] = {"bound": "hbm", "achieved": round(achieved, 3), "peak": HBM_PEAK_GBPS,
                            "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 5),
                            "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, path_name)),
@@ -548,7 +548,7 @@ def main():
         achieved = restore
         out["roofline"] = {"bound": "hbm", "achieved": round(achieved, 3), "peak": HBM_PEAK_GBPS,
                            "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 5),
-                           "traffic": None, "kernel": "fkv_copy_chunks_kernel<16>",
+                           "traffic": None, "kernel": "fkv_copy_chunks_kernel<16, true>",
                            "algorithmic_bytes_per_launch": r["layer_bytes"],
                            "limited_by": "host link (PCIe), not HBM",
                            "link_peak_GBps": round(link["h2d"], 3),
@@ -564,7 +564,7 @@ def main():
                                "frac_of_bidir_link": round(agg / (link["d2h"] + link["h2d"]), 4)})
         out["roofline"] = {"bound": "hbm", "achieved": round(agg, 3), "peak": HBM_PEAK_GBPS,
                            "unit": "GB/s", "frac": round(agg / HBM_PEAK_GBPS, 5), "traffic": None,
-                           "kernel": "fkv_copy_chunks_kernel<16>",
+                           "kernel": "fkv_copy_chunks_kernel<16, false|true>",
                            "limited_by": "host link (PCIe), both directions at once"}
     out["link_peak"] = {"d2h_GBps": round(link["d2h"], 3), "h2d_GBps": round(link["h2d"], 3),
                         "method": "1 GiB pinned hipMemcpyAsync x10, best, same run"}
