@@ -324,6 +324,14 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy):
     reps = max(1, int(round(target_ms / per_unit)))
     compute_ms = _median([compute_only(reps) for _ in range(3)])
 
+    alone = []
+    for _ in range(max(2, warmup + 1)):   # restore with nobody computing next to it
+        torch.cuda.synchronize()
+        restore()
+        grp.synchronize()
+        alone.append(grp.batch_times_ms()[-1])
+    restore_alone_ms = min(alone[1:]) if len(alone) > 1 else alone[0]
+
     totals, restores, firsts, stalls, busy = [], [], [], [], []
     for it in range(warmup + steps):
         torch.cuda.synchronize()
@@ -356,7 +364,8 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy):
     return dict(total_ms=_median(totals), restore_ms=_median(restores),
                 first_layer_ms=_median(firsts), compute_ms=compute_ms,
                 compute_overlapped_ms=_median(busy), stall_ms=_median(stalls),
-                compute_reps_per_layer=reps, layer_bytes=layer_bytes)
+                compute_reps_per_layer=reps, layer_bytes=layer_bytes,
+                restore_alone_ms=restore_alone_ms)
 
 
 def run_concurrent(w, torch, steps, warmup, num_cta):
@@ -530,6 +539,9 @@ def main():
                    h2d_GBps=round(restore, 3), h2d_frac_of_link=round(restore / link["h2d"], 4),
                    layerwise={"notify": args.notify, "dummy_compute": args.dummy,
                               "compute_units_per_layer": r["compute_reps_per_layer"],
+                              "restore_alone_ms": round(r["restore_alone_ms"], 3),
+                              "restore_alone_GBps": round(
+                                  B / (r["restore_alone_ms"] * 1e-3) / 1e9, 3),
                               "restore_ms": round(r["restore_ms"], 3),
                               "first_layer_ms": round(r["first_layer_ms"], 3),
                               "compute_alone_ms": round(r["compute_ms"], 3),

@@ -244,8 +244,7 @@ LinkLaunchShape link_launch_shape(bool is_h2d) {
   return dynamic ? read(is_h2d) : fixed[is_h2d ? 1 : 0];
 }
 
-int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream) {
-  set_last_path(FKV_PATH_KERNEL);
+int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan *out) {
   // Device-visible alias of the host pool.  hipHostMalloc / torch pinned memory
   // map to the same address; hipHostRegister-ed memory may not.
   void *cpu_dev = nullptr;
@@ -257,80 +256,109 @@ int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream) {
                 "before a kernel transfer): %s",
                 d.cpu_ptr, hipGetErrorString(e));
   }
-  const bool h2d = d.is_host_to_device != 0;
   static const bool mirror_plan = env_int("FKV_PLAN_MIRROR", 1) != 0;
+  int device = 0;
+  FKV_HIP_TRY(hipGetDevice(&device));
+  const int lk = d.num_layers * d.kv_dim;
+  const size_t tab_bytes = (size_t)lk * 8;
+  const size_t ids_bytes = (size_t)d.num_blocks * 8;
+  const size_t plan_bytes = 2 * tab_bytes + 2 * ids_bytes;
+  PlanSlot *slot = plan_acquire(device, plan_bytes);
+  if (!slot)
+    return FKV_ERR_RUNTIME;
+  uint8_t *h = plan_host(slot);
+  uint64_t *gbase = reinterpret_cast<uint64_t *>(h);
+  uint64_t *cbase = reinterpret_cast<uint64_t *>(h + tab_bytes);
+  uint64_t acc = (uint64_t)d.chunk_size | (uint64_t)d.gpu_block_stride |
+                 (uint64_t)d.cpu_block_stride;
+  for (int li = 0; li < d.num_layers; ++li) {
+    const int64_t layer = (int64_t)d.start_layer_id + li;
+    for (int kv = 0; kv < d.kv_dim; ++kv) {
+      const uint64_t g = gpu_chunk_addr(d, layer, kv, 0);
+      const uint64_t c =
+          (uint64_t)(uintptr_t)cpu_dev + (uint64_t)(layer * d.cpu_layer_stride +
+                                                    kv * d.cpu_kv_stride +
+                                                    d.cpu_startoff_inside_chunks);
+      gbase[li * d.kv_dim + kv] = g;
+      cbase[li * d.kv_dim + kv] = c;
+      acc |= g | c;
+    }
+  }
+  std::memcpy(h + 2 * tab_bytes, d.gpu_block_ids, ids_bytes);
+  std::memcpy(h + 2 * tab_bytes + ids_bytes, d.cpu_block_ids, ids_bytes);
+  uint8_t *dv = nullptr;
+  int rc = plan_publish(slot, plan_bytes, mirror_plan, stream, &dv);
+  if (rc != FKV_OK) {
+    plan_release(slot, stream, false);
+    return rc;
+  }
+  out->slot = slot;
+  out->gpu_base = reinterpret_cast<const uint64_t *>(dv);
+  out->cpu_base = reinterpret_cast<const uint64_t *>(dv + tab_bytes);
+  out->gpu_ids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes);
+  out->cpu_ids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes + ids_bytes);
+  out->vec = common_vector_width(&acc, 1);
+  out->h2d = d.is_host_to_device != 0;
+  out->kv_dim = d.kv_dim;
+  out->num_layers = d.num_layers;
+  out->num_blocks = d.num_blocks;
+  out->chunk_size = d.chunk_size;
+  out->gpu_block_stride = d.gpu_block_stride;
+  out->cpu_block_stride = d.cpu_block_stride;
   // A CTA of the reference is 1024 threads on one SM (csrc/transfer.cu:176) and
   // its default of 4 CTAs is tuned for that hardware.  Here each requested CTA
   // becomes `workgroups_per_cta` small workgroups (see link_launch_shape).
-  const LinkLaunchShape shape = link_launch_shape(h2d);
-  const int num_cta = (d.transfer_num_cta > 0 ? d.transfer_num_cta : default_num_cta(h2d)) *
-                      shape.workgroups_per_cta;
+  const LinkLaunchShape shape = link_launch_shape(out->h2d);
+  out->workgroups =
+      (d.transfer_num_cta > 0 ? d.transfer_num_cta : default_num_cta(out->h2d)) *
+      shape.workgroups_per_cta;
+  out->threads = shape.threads;
+  return FKV_OK;
+}
 
+int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
+                       hipStream_t stream) {
+  if (layer_offset < 0 || num_layers < 0 || layer_offset + num_layers > p.num_layers)
+    return fail(FKV_ERR_RUNTIME, "kernel plan: layers [%d, %d) outside the plan's %d", layer_offset,
+                layer_offset + num_layers, p.num_layers);
   // Layers go out in groups whose (layer, kv) base tables fit the kernel's LDS.
-  const int layers_per_launch = kCopyMaxLK / d.kv_dim;
+  const int layers_per_launch = kCopyMaxLK / p.kv_dim;
   if (layers_per_launch < 1)
-    return fail(FKV_ERR_INVALID_ARG, "kv_dim %d too large", d.kv_dim);
-  for (int l0 = 0; l0 < d.num_layers; l0 += layers_per_launch) {
-    const int nl = std::min(layers_per_launch, d.num_layers - l0);
-    const int lk = nl * d.kv_dim;
-    const size_t tab_bytes = (size_t)lk * 8;
-    const size_t ids_bytes = (size_t)d.num_blocks * 8;
-    const size_t plan_bytes = 2 * tab_bytes + 2 * ids_bytes;
-    PlanSlot *slot = plan_acquire(DeviceGuard(-1).device(), plan_bytes);
-    if (!slot)
-      return FKV_ERR_RUNTIME;
-    uint8_t *h = plan_host(slot);
-    uint64_t *gbase = reinterpret_cast<uint64_t *>(h);
-    uint64_t *cbase = reinterpret_cast<uint64_t *>(h + tab_bytes);
-    int64_t *gids = reinterpret_cast<int64_t *>(h + 2 * tab_bytes);
-    int64_t *cids = reinterpret_cast<int64_t *>(h + 2 * tab_bytes + ids_bytes);
-    uint64_t align_bits[8] = {(uint64_t)d.chunk_size, (uint64_t)d.gpu_block_stride,
-                              (uint64_t)d.cpu_block_stride, 0, 0, 0, 0, 0};
-    uint64_t acc = 0;
-    for (int li = 0; li < nl; ++li) {
-      const int64_t layer = (int64_t)d.start_layer_id + l0 + li;
-      for (int kv = 0; kv < d.kv_dim; ++kv) {
-        const uint64_t g = gpu_chunk_addr(d, layer, kv, 0);
-        const uint64_t c = (uint64_t)(uintptr_t)cpu_dev +
-                           (uint64_t)(layer * d.cpu_layer_stride + kv * d.cpu_kv_stride +
-                                      d.cpu_startoff_inside_chunks);
-        gbase[li * d.kv_dim + kv] = g;
-        cbase[li * d.kv_dim + kv] = c;
-        acc |= g | c;
-      }
-    }
-    align_bits[3] = acc;
-    std::memcpy(gids, d.gpu_block_ids, ids_bytes);
-    std::memcpy(cids, d.cpu_block_ids, ids_bytes);
-
-    uint8_t *dv = nullptr;
-    int rc = plan_publish(slot, plan_bytes, mirror_plan, stream, &dv);
-    if (rc != FKV_OK) {
-      plan_release(slot, stream, false);
-      return rc;
-    }
+    return fail(FKV_ERR_INVALID_ARG, "kv_dim %d too large", p.kv_dim);
+  for (int l0 = layer_offset; l0 < layer_offset + num_layers; l0 += layers_per_launch) {
+    const int nl = std::min(layers_per_launch, layer_offset + num_layers - l0);
+    const uint64_t *gb = p.gpu_base + (size_t)l0 * p.kv_dim;
+    const uint64_t *cb = p.cpu_base + (size_t)l0 * p.kv_dim;
     CopyKernelArgs a{};
-    const uint64_t *dv_gbase = reinterpret_cast<const uint64_t *>(dv);
-    const uint64_t *dv_cbase = reinterpret_cast<const uint64_t *>(dv + tab_bytes);
-    const int64_t *dv_gids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes);
-    const int64_t *dv_cids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes + ids_bytes);
-    a.base_src = h2d ? dv_cbase : dv_gbase;
-    a.base_dst = h2d ? dv_gbase : dv_cbase;
-    a.ids_src = h2d ? dv_cids : dv_gids;
-    a.ids_dst = h2d ? dv_gids : dv_cids;
-    a.stride_src = h2d ? d.cpu_block_stride : d.gpu_block_stride;
-    a.stride_dst = h2d ? d.gpu_block_stride : d.cpu_block_stride;
-    a.chunk_bytes = d.chunk_size;
-    a.num_blocks = d.num_blocks;
-    a.lk = lk;
-    a.vec = common_vector_width(align_bits, 4);
-    a.nt_store = h2d ? 1 : 0;
-    rc = launch_copy_kernel(a, num_cta, shape.threads, stream);
-    plan_release(slot, stream, false);
-    if (rc != FKV_OK)
-      return rc;
+    a.base_src = p.h2d ? cb : gb;
+    a.base_dst = p.h2d ? gb : cb;
+    a.ids_src = p.h2d ? p.cpu_ids : p.gpu_ids;
+    a.ids_dst = p.h2d ? p.gpu_ids : p.cpu_ids;
+    a.stride_src = p.h2d ? p.cpu_block_stride : p.gpu_block_stride;
+    a.stride_dst = p.h2d ? p.gpu_block_stride : p.cpu_block_stride;
+    a.chunk_bytes = p.chunk_size;
+    a.num_blocks = p.num_blocks;
+    a.lk = nl * p.kv_dim;
+    a.vec = p.vec;
+    a.nt_store = p.h2d ? 1 : 0;
+    FKV_TRY(launch_copy_kernel(a, p.workgroups, p.threads, stream));
   }
   return FKV_OK;
+}
+
+void kernel_plan_release(KernelPlan *p, hipStream_t stream) {
+  if (p->slot)
+    plan_release(p->slot, stream, false);
+  p->slot = nullptr;
+}
+
+int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream) {
+  set_last_path(FKV_PATH_KERNEL);
+  KernelPlan plan;
+  FKV_TRY(kernel_plan_build(d, stream, &plan));
+  int rc = kernel_plan_launch(plan, 0, d.num_layers, stream);
+  kernel_plan_release(&plan, stream);
+  return rc;
 }
 
 namespace {

@@ -146,6 +146,27 @@ int plan_publish(PlanSlot *s, size_t bytes, bool mirror, hipStream_t stream,
 void plan_release(PlanSlot *s, hipStream_t stream, bool drained);
 
 // ---- paths ----------------------------------------------------------------
+// The kernel path in two steps, so that a caller that launches layer by layer
+// (the layerwise restore) uploads the id lists and base tables once.
+struct KernelPlan {
+  PlanSlot *slot = nullptr;
+  const uint64_t *gpu_base = nullptr; // device-visible, [num_layers * kv_dim]
+  const uint64_t *cpu_base = nullptr;
+  const int64_t *gpu_ids = nullptr;   // device-visible, [num_blocks]
+  const int64_t *cpu_ids = nullptr;
+  int vec = 1;
+  bool h2d = false;
+  int kv_dim = 1, num_layers = 0, num_blocks = 0;
+  int64_t chunk_size = 0, gpu_block_stride = 0, cpu_block_stride = 0;
+  int workgroups = 1, threads = 64;
+};
+// Builds and uploads (on `stream`) the plan for all layers of `d`.
+int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan *out);
+// Enqueues the copy of layers [layer_offset, layer_offset + num_layers) of the plan.
+int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
+                       hipStream_t stream);
+// The plan memory is recycled once everything enqueued on `stream` so far has run.
+void kernel_plan_release(KernelPlan *p, hipStream_t stream);
 int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream);
 int run_ce_path(const fkv_transfer_desc &d, hipStream_t stream);
 // Device-side compaction between the engine's KV tensors and a packed device

@@ -261,42 +261,75 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
   FKV_HIP_TRY(hipEventCreate(&g->started));
   FKV_HIP_TRY(hipEventRecord(g->started, g->streams[0]));
 
+  // descriptor of rank i for layers [start, start + layers)
+  auto describe = [&](int i, int start, int layers) {
+    // host offset of rank i, csrc/layerwise.cpp:1143-1166
+    int64_t cpu_off = (int64_t)i * cpu_tp_stride;
+    if (num_kv_heads == 1)
+      cpu_off = is(mode, "all_write") ? (int64_t)i * num_blocks * cpu_block_stride : 0;
+    fkv_transfer_desc d{};
+    d.backend = g->backend;
+    d.num_layers_total = g->num_layers;
+    d.gpu_tensor_ptrs = g->gpu_ptrs.data() + (size_t)i * g->num_tensors_per_gpu;
+    d.num_gpu_tensor_ptrs = g->num_tensors_per_gpu;
+    d.device = g->device_ids[i];
+    d.gpu_kv_stride = g->kv_strides[i];
+    d.gpu_block_stride = g->block_strides[i];
+    d.gpu_layer_stride = g->layer_strides[i];
+    d.gpu_startoff_inside_chunks = 0;
+    d.cpu_ptr = g->cpu_blocks;
+    d.cpu_kv_stride = h2d_cpu_kv_stride;
+    d.cpu_layer_stride = h2d_cpu_layer_stride;
+    d.cpu_block_stride = cpu_block_stride;
+    d.cpu_startoff_inside_chunks = cpu_off;
+    d.chunk_size = g->chunk_sizes[i];
+    d.start_layer_id = start;
+    d.num_layers = layers;
+    d.kv_dim = kv_dim;
+    d.num_blocks = num_blocks;
+    d.gpu_block_ids = gpu_block_ids;
+    d.cpu_block_ids = cpu_block_ids;
+    d.is_host_to_device = 1;
+    d.use_ce_transfer = use_ce_transfer;
+    d.transfer_num_cta = transfer_cta_num;
+    d.sync = 0;
+    d.ce = g->ce;
+    return d;
+  };
+
   int rc = FKV_OK;
+  // Kernel path: the id lists and the base tables of all layers go to the device
+  // once per GPU; every batch is then a single kernel launch.
+  const bool direct = !use_ce_transfer && num_blocks > 0 && num_layers > 0;
+  std::vector<KernelPlan> plans(direct ? g->num_gpus : 0);
+  if (direct) {
+    for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
+      fkv_transfer_desc d = describe(i, 0, num_layers);
+      if (!d.gpu_tensor_ptrs || !d.cpu_ptr || !gpu_block_ids || !cpu_block_ids ||
+          d.chunk_size <= 0 || kv_dim < 1) {
+        rc = fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_transfer: bad pointers or sizes");
+        break;
+      }
+      (void)hipSetDevice(g->device_ids[i]);
+      rc = kernel_plan_build(d, g->streams[i], &plans[i]);
+    }
+  }
   for (int b = 0; b < num_batches && rc == FKV_OK; ++b) {
     fkv_layerwise::Batch &batch = *g->batches[b];
     for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
-      // host offset of rank i, csrc/layerwise.cpp:1143-1166
-      int64_t cpu_off = (int64_t)i * cpu_tp_stride;
-      if (num_kv_heads == 1)
-        cpu_off = is(mode, "all_write") ? (int64_t)i * num_blocks * cpu_block_stride : 0;
-      fkv_transfer_desc d{};
-      d.backend = g->backend;
-      d.num_layers_total = g->num_layers;
-      d.gpu_tensor_ptrs = g->gpu_ptrs.data() + (size_t)i * g->num_tensors_per_gpu;
-      d.num_gpu_tensor_ptrs = g->num_tensors_per_gpu;
-      d.device = g->device_ids[i];
-      d.gpu_kv_stride = g->kv_strides[i];
-      d.gpu_block_stride = g->block_strides[i];
-      d.gpu_layer_stride = g->layer_strides[i];
-      d.gpu_startoff_inside_chunks = 0;
-      d.cpu_ptr = g->cpu_blocks;
-      d.cpu_kv_stride = h2d_cpu_kv_stride;
-      d.cpu_layer_stride = h2d_cpu_layer_stride;
-      d.cpu_block_stride = cpu_block_stride;
-      d.cpu_startoff_inside_chunks = cpu_off;
-      d.chunk_size = g->chunk_sizes[i];
-      d.start_layer_id = batch.start_layer;
-      d.num_layers = batch.layers;
-      d.kv_dim = kv_dim;
-      d.num_blocks = num_blocks;
-      d.gpu_block_ids = gpu_block_ids;
-      d.cpu_block_ids = cpu_block_ids;
-      d.is_host_to_device = 1;
-      d.use_ce_transfer = use_ce_transfer;
-      d.transfer_num_cta = transfer_cta_num;
-      d.sync = 0;
-      d.ce = g->ce;
-      rc = fkv_transfer_kv_blocks(&d, g->streams[i]);
+      (void)hipSetDevice(g->device_ids[i]);
+      if (direct) {
+        rc = kernel_plan_launch(plans[i], batch.start_layer, batch.layers, g->streams[i]);
+        if (rc == FKV_OK) {
+          stats().calls.fetch_add(1, std::memory_order_relaxed);
+          stats().bytes_h2d.fetch_add((uint64_t)num_blocks * batch.layers * kv_dim *
+                                          (uint64_t)g->chunk_sizes[i],
+                                      std::memory_order_relaxed);
+        }
+      } else {
+        fkv_transfer_desc d = describe(i, batch.start_layer, batch.layers);
+        rc = fkv_transfer_kv_blocks(&d, g->streams[i]);
+      }
       if (rc != FKV_OK)
         break;
       (void)hipSetDevice(g->device_ids[i]);
@@ -311,6 +344,10 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
     }
   }
   std::string saved_error = fkv_last_error();
+  for (int i = 0; i < (int)plans.size(); ++i) {
+    (void)hipSetDevice(g->device_ids[i]);
+    kernel_plan_release(&plans[i], g->streams[i]);
+  }
   if (rc != FKV_OK) {
     // Drain what was enqueued so no callback outlives this call's batches.
     for (int i = 0; i < g->num_gpus; ++i) {
