@@ -94,7 +94,17 @@ struct StageSet {
   DeviceStage dev[2];
   HostStage host;
   hipEvent_t pingpong[2] = {nullptr, nullptr};
+  // second DMA stream + the events that fork it off / join it back into the
+  // caller's stream
+  hipStream_t aux = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
   ~StageSet() {
+    if (aux)
+      (void)hipStreamDestroy(aux);
+    if (fork)
+      (void)hipEventDestroy(fork);
+    if (join)
+      (void)hipEventDestroy(join);
     // Best effort: the thread is ending; errors (including a runtime that is
     // already shutting down) are ignored.
     for (auto &d : dev) {
@@ -193,6 +203,14 @@ size_t staging_cap_bytes() {
   return cap;
 }
 
+bool fan_enabled() {
+  static const bool on = [] {
+    const char *v = std::getenv("FKV_CE_TWO_STREAMS");
+    return !(v && *v == '0');
+  }();
+  return on;
+}
+
 // ---- one transfer's state ------------------------------------------------
 struct Job {
   const fkv_transfer_desc &d;
@@ -201,6 +219,43 @@ struct Job {
   bool h2d;
   hipMemcpyKind kind;
   Analysis an;
+  // While fanned out, independent DMAs alternate between the caller's stream and
+  // a second stream: the fixed cost of one copy (about 10 us) then overlaps the
+  // transfer time of the other.  Two streams measured best; more are slower.
+  mutable hipStream_t aux = nullptr;
+  mutable unsigned turn = 0;
+
+  // Call when at least `copies` independent DMAs follow.  Work already on
+  // `stream` is ordered before everything issued on the second stream.
+  int fan_out(size_t copies) const {
+    if (aux || copies < 8 || !fan_enabled())
+      return FKV_OK;
+    StageSet &s = stage_set(device);
+    if (!s.aux) {
+      if (hipStreamCreateWithFlags(&s.aux, hipStreamNonBlocking) != hipSuccess ||
+          hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) != hipSuccess ||
+          hipEventCreateWithFlags(&s.join, hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError();
+        return FKV_OK; // stay on one stream
+      }
+    }
+    FKV_HIP_TRY(hipEventRecord(s.fork, stream));
+    FKV_HIP_TRY(hipStreamWaitEvent(s.aux, s.fork, 0));
+    aux = s.aux;
+    turn = 0;
+    return FKV_OK;
+  }
+  // Everything issued since fan_out() is ordered before later work on `stream`.
+  int fan_in() const {
+    if (!aux)
+      return FKV_OK;
+    StageSet &s = stage_set(device);
+    aux = nullptr;
+    FKV_HIP_TRY(hipEventRecord(s.join, s.aux));
+    FKV_HIP_TRY(hipStreamWaitEvent(stream, s.join, 0));
+    return FKV_OK;
+  }
+  hipStream_t next_stream() const { return (aux && (turn++ & 1u)) ? aux : stream; }
 
   uint8_t *gpu(int layer_local, int kv, int64_t block) const {
     return reinterpret_cast<uint8_t *>(
@@ -211,7 +266,7 @@ struct Job {
   }
   int dma(void *dst, const void *src, size_t bytes, hipMemcpyKind k) const {
     stats().dma_copies.fetch_add(1, std::memory_order_relaxed);
-    FKV_HIP_TRY(hipMemcpyAsync(dst, src, bytes, k, stream));
+    FKV_HIP_TRY(hipMemcpyAsync(dst, src, bytes, k, next_stream()));
     return FKV_OK;
   }
   // gpu <-> cpu copy in the direction of the transfer
@@ -221,7 +276,7 @@ struct Job {
   int dma2d(void *dst, size_t dpitch, const void *src, size_t spitch, size_t width,
             size_t height, hipMemcpyKind k) const {
     stats().dma_copies.fetch_add(1, std::memory_order_relaxed);
-    FKV_HIP_TRY(hipMemcpy2DAsync(dst, dpitch, src, spitch, width, height, k, stream));
+    FKV_HIP_TRY(hipMemcpy2DAsync(dst, dpitch, src, spitch, width, height, k, next_stream()));
     return FKV_OK;
   }
 };
@@ -229,35 +284,45 @@ struct Job {
 // csrc/ce_transfer.cu:196-229
 int per_block(const Job &j) {
   const auto &d = j.d;
-  for (int i = 0; i < d.num_layers; ++i)
-    for (int kv = 0; kv < d.kv_dim; ++kv)
-      for (int b = 0; b < d.num_blocks; ++b)
-        FKV_TRY(j.dma_dir(j.gpu(i, kv, d.gpu_block_ids[b]), j.cpu(i, kv, d.cpu_block_ids[b]),
-                          (size_t)d.chunk_size));
-  return FKV_OK;
+  FKV_TRY(j.fan_out((size_t)d.num_layers * d.kv_dim * d.num_blocks));
+  int rc = FKV_OK;
+  for (int i = 0; i < d.num_layers && rc == FKV_OK; ++i)
+    for (int kv = 0; kv < d.kv_dim && rc == FKV_OK; ++kv)
+      for (int b = 0; b < d.num_blocks && rc == FKV_OK; ++b)
+        rc = j.dma_dir(j.gpu(i, kv, d.gpu_block_ids[b]), j.cpu(i, kv, d.cpu_block_ids[b]),
+                       (size_t)d.chunk_size);
+  int rc2 = j.fan_in();
+  return rc != FKV_OK ? rc : rc2;
 }
 
 // csrc/ce_transfer.cu:235-267
 int contig_direct(const Job &j) {
   const auto &d = j.d;
   const size_t run = (size_t)d.chunk_size * (size_t)d.num_blocks;
-  for (int i = 0; i < d.num_layers; ++i)
-    for (int kv = 0; kv < d.kv_dim; ++kv)
-      FKV_TRY(j.dma_dir(j.gpu(i, kv, d.gpu_block_ids[0]), j.cpu(i, kv, d.cpu_block_ids[0]),
-                        run));
-  return FKV_OK;
+  FKV_TRY(j.fan_out((size_t)d.num_layers * d.kv_dim));
+  int rc = FKV_OK;
+  for (int i = 0; i < d.num_layers && rc == FKV_OK; ++i)
+    for (int kv = 0; kv < d.kv_dim && rc == FKV_OK; ++kv)
+      rc = j.dma_dir(j.gpu(i, kv, d.gpu_block_ids[0]), j.cpu(i, kv, d.cpu_block_ids[0]), run);
+  int rc2 = j.fan_in();
+  return rc != FKV_OK ? rc : rc2;
 }
 
 // csrc/ce_transfer.cu:271-309
 int segment_direct(const Job &j) {
   const auto &d = j.d;
-  for (int i = 0; i < d.num_layers; ++i)
-    for (int kv = 0; kv < d.kv_dim; ++kv)
-      for (const auto &s : j.an.segs)
-        FKV_TRY(j.dma_dir(j.gpu(i, kv, d.gpu_block_ids[s.start_k]),
-                          j.cpu(i, kv, d.cpu_block_ids[s.start_k]),
-                          (size_t)s.nr_blocks * (size_t)d.chunk_size));
-  return FKV_OK;
+  FKV_TRY(j.fan_out((size_t)d.num_layers * d.kv_dim * j.an.segs.size()));
+  int rc = FKV_OK;
+  for (int i = 0; i < d.num_layers && rc == FKV_OK; ++i)
+    for (int kv = 0; kv < d.kv_dim && rc == FKV_OK; ++kv)
+      for (size_t si = 0; si < j.an.segs.size() && rc == FKV_OK; ++si) {
+        const auto &s = j.an.segs[si];
+        rc = j.dma_dir(j.gpu(i, kv, d.gpu_block_ids[s.start_k]),
+                       j.cpu(i, kv, d.cpu_block_ids[s.start_k]),
+                       (size_t)s.nr_blocks * (size_t)d.chunk_size);
+      }
+  int rc2 = j.fan_in();
+  return rc != FKV_OK ? rc : rc2;
 }
 
 bool use_memcpy2d(const Job &j) {
@@ -335,19 +400,21 @@ int segment_scatter(const Job &j) {
   const auto &d = j.d;
   if (use_memcpy2d(j)) {
     // one strided 2-D copy per (layer, kv, segment): rows = blocks of the segment
-    for (int i = 0; i < d.num_layers; ++i)
-      for (int kv = 0; kv < d.kv_dim; ++kv)
-        for (const auto &s : j.an.segs) {
+    FKV_TRY(j.fan_out((size_t)d.num_layers * d.kv_dim * j.an.segs.size()));
+    int rc = FKV_OK;
+    for (int i = 0; i < d.num_layers && rc == FKV_OK; ++i)
+      for (int kv = 0; kv < d.kv_dim && rc == FKV_OK; ++kv)
+        for (size_t si = 0; si < j.an.segs.size() && rc == FKV_OK; ++si) {
+          const auto &s = j.an.segs[si];
           uint8_t *g = j.gpu(i, kv, d.gpu_block_ids[s.start_k]);
           uint8_t *c = j.cpu(i, kv, d.cpu_block_ids[s.start_k]);
-          if (j.h2d)
-            FKV_TRY(j.dma2d(g, (size_t)d.gpu_block_stride, c, (size_t)d.cpu_block_stride,
-                            (size_t)d.chunk_size, (size_t)s.nr_blocks, j.kind));
-          else
-            FKV_TRY(j.dma2d(c, (size_t)d.cpu_block_stride, g, (size_t)d.gpu_block_stride,
-                            (size_t)d.chunk_size, (size_t)s.nr_blocks, j.kind));
+          rc = j.h2d ? j.dma2d(g, (size_t)d.gpu_block_stride, c, (size_t)d.cpu_block_stride,
+                               (size_t)d.chunk_size, (size_t)s.nr_blocks, j.kind)
+                     : j.dma2d(c, (size_t)d.cpu_block_stride, g, (size_t)d.gpu_block_stride,
+                               (size_t)d.chunk_size, (size_t)s.nr_blocks, j.kind);
         }
-    return FKV_OK;
+    int rc2 = j.fan_in();
+    return rc != FKV_OK ? rc : rc2;
   }
   if (!j.h2d) {
     return d2h_pingpong(j, [&](int it, uint8_t *buf) {
@@ -445,9 +512,55 @@ int device_staging_copy(const fkv_transfer_desc &d, int it0, int nit, int p0, in
 
 namespace {
 
+// Whole-block shortcut.  When the (layer, kv) chunks of a block are adjacent and
+// in the same order on the GPU (single-tensor, block-major engine layout) as in
+// the host block, the bytes of a block form one run on both sides: no staging
+// and no per-(layer, kv) pass is needed, one DMA moves a block, or a run of
+// adjacent blocks.  The reference stages such transfers through GATHER_SCATTER.
+bool blocks_are_runs_on_both_sides(const Job &j) {
+  const auto &d = j.d;
+  if (d.backend != FKV_BACKEND_TRTLLM)
+    return false;
+  const bool gpu_dense = (d.kv_dim == 1 || d.gpu_kv_stride == d.chunk_size) &&
+                         (d.num_layers == 1 || d.gpu_layer_stride == (int64_t)d.kv_dim * d.chunk_size);
+  const bool cpu_dense = (d.kv_dim == 1 || d.cpu_kv_stride == d.chunk_size) &&
+                         (d.num_layers == 1 || d.cpu_layer_stride == (int64_t)d.kv_dim * d.chunk_size);
+  return gpu_dense && cpu_dense;
+}
+
+int block_runs_direct(const Job &j) {
+  const auto &d = j.d;
+  const size_t width = (size_t)d.num_layers * d.kv_dim * (size_t)d.chunk_size;
+  const bool linear = (int64_t)width == d.gpu_block_stride && (int64_t)width == d.cpu_block_stride;
+  FKV_TRY(j.fan_out(linear || d.ce.enable_memcpy2d ? j.an.segs.size() : (size_t)d.num_blocks));
+  int rc = FKV_OK;
+  for (size_t si = 0; si < j.an.segs.size() && rc == FKV_OK; ++si) {
+    const auto &s = j.an.segs[si];
+    uint8_t *g = j.gpu(0, 0, d.gpu_block_ids[s.start_k]);
+    uint8_t *c = j.cpu(0, 0, d.cpu_block_ids[s.start_k]);
+    const size_t rows = (size_t)s.nr_blocks;
+    if (linear) {
+      rc = j.dma_dir(g, c, rows * width);
+    } else if (d.ce.enable_memcpy2d) {
+      rc = j.h2d ? j.dma2d(g, (size_t)d.gpu_block_stride, c, (size_t)d.cpu_block_stride, width,
+                           rows, j.kind)
+                 : j.dma2d(c, (size_t)d.cpu_block_stride, g, (size_t)d.gpu_block_stride, width,
+                           rows, j.kind);
+    } else {
+      for (size_t r = 0; r < rows && rc == FKV_OK; ++r)
+        rc = j.dma_dir(g + r * (size_t)d.gpu_block_stride, c + r * (size_t)d.cpu_block_stride,
+                       width);
+    }
+  }
+  int rc2 = j.fan_in();
+  return rc != FKV_OK ? rc : rc2;
+}
+
 // csrc/ce_transfer.cu:816-1179
 int gather_scatter(const Job &j) {
   const auto &d = j.d;
+  if (blocks_are_runs_on_both_sides(j))
+    return block_runs_direct(j);
   const bool gpu_run = j.an.a.gpu_log_contig && j.an.a.gpu_phys_contig; // one linear GPU run
   const bool cpu_run = j.an.a.cpu_log_contig && j.an.a.cpu_phys_contig; // one linear host run
   const size_t layer_bytes = (size_t)d.num_blocks * (size_t)d.chunk_size;
@@ -556,6 +669,8 @@ int gather_direct(const Job &j) {
     if (!j.h2d)
       rc = device_staging_copy(d, 0, lk, p0, np, stage, true, true, j.stream);
     // segments (cpu- and gpu-adjacent runs) clipped to this group
+    if (rc == FKV_OK)
+      rc = j.fan_out(full_block || d.ce.enable_memcpy2d ? j.an.segs.size() - seg_i : (size_t)np);
     while (seg_i < j.an.segs.size() && rc == FKV_OK) {
       const auto &s = j.an.segs[seg_i];
       const int b = std::max(s.start_k, p0);
@@ -579,6 +694,11 @@ int gather_direct(const Job &j) {
       if (s.start_k + s.nr_blocks > p0 + np)
         break; // the rest of this segment belongs to the next group
       ++seg_i;
+    }
+    {
+      int rc2 = j.fan_in();
+      if (rc == FKV_OK)
+        rc = rc2;
     }
     if (rc == FKV_OK && j.h2d)
       rc = device_staging_copy(d, 0, lk, p0, np, stage, true, false, j.stream);
