@@ -104,6 +104,8 @@ SIGNATURES = {
     "fkv_last_path": (c_int32, []),
     "fkv_ce_config_default": (None, [POINTER(CEConfig)]),
     "fkv_transfer_kv_blocks": (c_int32, [POINTER(TransferDesc), c_void_p]),
+    "fkv_choose_engine": (c_int32, [POINTER(TransferDesc), POINTER(c_int32), POINTER(c_double),
+                                    POINTER(c_double)]),
     "fkv_ce_analyze": (c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int64,
                                  POINTER(CEAnalysis), c_void_p, c_int32]),
     "fkv_ce_choose_path": (c_int32, [POINTER(CEAnalysis), POINTER(CEConfig), c_int64,

@@ -119,7 +119,11 @@ def transfer_kv_blocks(
     d.gpu_block_ids = gpu_ids.data_ptr()
     d.cpu_block_ids = cpu_ids.data_ptr()
     d.is_host_to_device = int(bool(is_host_to_device))
-    d.use_ce_transfer = int(bool(use_ce_transfer))
+    # True/False as in the reference; "auto" (or 2) lets the library pick per transfer
+    if use_ce_transfer == "auto" or (use_ce_transfer == 2 and not isinstance(use_ce_transfer, bool)):
+        d.use_ce_transfer = 2
+    else:
+        d.use_ce_transfer = int(bool(use_ce_transfer))
     d.transfer_num_cta = int(transfer_num_cta)
     d.sync = int(bool(sync))
     d.enable_trace = int(bool(enable_transfer_trace))

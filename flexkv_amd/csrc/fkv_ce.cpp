@@ -720,19 +720,17 @@ const char *path_name(int p) {
 
 } // namespace
 
-int run_ce_path(const fkv_transfer_desc &d, hipStream_t stream) {
-  int device = 0;
-  FKV_HIP_TRY(hipGetDevice(&device));
-  Job j{d, stream, device, d.is_host_to_device != 0,
-        d.is_host_to_device ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost, {}};
-  analyze(d.gpu_block_ids, d.cpu_block_ids, d.num_blocks, d.cpu_block_stride, d.chunk_size,
-          d.gpu_block_stride, j.an);
+namespace {
+
+// Strategy for this transfer: PER_BLOCK, the forced one, or choose()'s.
+int resolve_path(const Job &j, int *path_out) {
+  const auto &d = j.d;
+  const auto &a = j.an.a;
   if (!d.ce.path_opt_enabled) { // csrc/transfer.cu:201-208
-    set_last_path(FKV_CE_PER_BLOCK);
-    return per_block(j);
+    *path_out = FKV_CE_PER_BLOCK;
+    return FKV_OK;
   }
   int path;
-  const auto &a = j.an.a;
   if (d.ce.force_path >= 0) {
     if (d.ce.force_path > 4) // csrc/transfer.cu:213-214
       return fail(FKV_ERR_RUNTIME, "force_path out of range [0,4]: %d", d.ce.force_path);
@@ -756,8 +754,109 @@ int run_ce_path(const fkv_transfer_desc &d, hipStream_t stream) {
         (int64_t)d.num_layers * d.kv_dim * d.chunk_size == d.cpu_block_stride;
     path = choose(a, d.ce, d.chunk_size, j.h2d, full_block);
   }
+  *path_out = path;
+  return FKV_OK;
+}
+
+// What a strategy costs beyond moving the bytes over the link once.
+struct CeWork {
+  double dmas = 0;          // separate DMA commands
+  double device_staged = 0; // bytes through a device compaction pass
+  double host_staged = 0;   // bytes through a host scatter/gather pass
+};
+
+bool host_block_dense(const fkv_transfer_desc &d) {
+  return (d.kv_dim == 1 || d.cpu_kv_stride == d.chunk_size) &&
+         (d.num_layers == 1 || d.cpu_layer_stride == (int64_t)d.kv_dim * d.chunk_size);
+}
+
+CeWork ce_work(const Job &j, int path) {
+  const auto &d = j.d;
+  const auto &a = j.an.a;
+  const double iters = (double)d.num_layers * d.kv_dim, n = d.num_blocks;
+  const double segs = (double)j.an.segs.size(), bytes = iters * n * (double)d.chunk_size;
+  const bool two_d = use_memcpy2d(j);
+  const bool gpu_run = a.gpu_log_contig && a.gpu_phys_contig;
+  const bool cpu_run = a.cpu_log_contig && a.cpu_phys_contig;
+  CeWork w;
+  auto staged = [&] { // GATHER_SCATTER proper
+    w.dmas = iters * (two_d ? segs : 1);
+    w.device_staged = gpu_run ? 0 : bytes;
+    w.host_staged = (two_d || cpu_run) ? 0 : bytes;
+  };
+  switch (path) {
+  case FKV_CE_PER_BLOCK: w.dmas = iters * n; break;
+  case FKV_CE_CONTIG_DIRECT: w.dmas = iters; break;
+  case FKV_CE_SEGMENT_DIRECT: w.dmas = iters * segs; break;
+  case FKV_CE_SEGMENT_SCATTER:
+    w.dmas = iters * segs;
+    w.host_staged = two_d ? 0 : bytes;
+    break;
+  case FKV_CE_GATHER_SCATTER:
+    if (blocks_are_runs_on_both_sides(j)) {
+      const bool linear = iters * (double)d.chunk_size == (double)d.gpu_block_stride &&
+                          iters * (double)d.chunk_size == (double)d.cpu_block_stride;
+      w.dmas = (linear || d.ce.enable_memcpy2d) ? segs : n;
+    } else {
+      staged();
+    }
+    break;
+  default: // GATHER_DIRECT
+    if (host_block_dense(d)) {
+      const bool full = iters * (double)d.chunk_size == (double)d.cpu_block_stride;
+      w.dmas = (full || d.ce.enable_memcpy2d) ? segs : n;
+      w.device_staged = bytes;
+    } else {
+      staged();
+    }
+  }
+  return w;
+}
+
+// Measured on MI355X: a DMA command costs about 2.5 us beyond its bytes when
+// copies alternate over two streams (256 x 2 MiB: 50-54 GB/s; 2048 x 5 MiB:
+// 56.2 GB/s); the compaction pass runs at 1.5 TB/s or more; a host
+// scatter/gather pass at about 20 GB/s with four threads; the gather/scatter
+// kernel reaches 56.4 GB/s GPU->host and 57.2 GB/s host->GPU.
+constexpr double kLinkBps = 57.2e9, kKernelD2HBps = 56.4e9, kKernelH2DBps = 57.2e9;
+constexpr double kDmaSeconds = 2.5e-6, kCompactionBps = 1.5e12, kHostPassBps = 20e9;
+constexpr double kLaunchSeconds = 15e-6;
+constexpr double kPreferCopyEngineWithin = 1.03; // it leaves the CUs and their memory queues alone
+
+} // namespace
+
+int choose_engine(const fkv_transfer_desc &d, int *use_ce, double *kernel_s, double *ce_s) {
+  Job j{d, nullptr, 0, d.is_host_to_device != 0,
+        d.is_host_to_device ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost, {}};
+  analyze(d.gpu_block_ids, d.cpu_block_ids, d.num_blocks, d.cpu_block_stride, d.chunk_size,
+          d.gpu_block_stride, j.an);
+  int path = FKV_CE_PER_BLOCK;
+  FKV_TRY(resolve_path(j, &path));
+  const CeWork w = ce_work(j, path);
+  const double bytes = (double)d.num_blocks * d.num_layers * d.kv_dim * (double)d.chunk_size;
+  const double tk = bytes / (j.h2d ? kKernelH2DBps : kKernelD2HBps) + kLaunchSeconds;
+  const double tc = bytes / kLinkBps + w.dmas * kDmaSeconds + w.device_staged / kCompactionBps +
+                    w.host_staged / kHostPassBps;
+  if (kernel_s)
+    *kernel_s = tk;
+  if (ce_s)
+    *ce_s = tc;
+  *use_ce = tc <= kPreferCopyEngineWithin * tk ? 1 : 0;
+  return FKV_OK;
+}
+
+int run_ce_path(const fkv_transfer_desc &d, hipStream_t stream) {
+  int device = 0;
+  FKV_HIP_TRY(hipGetDevice(&device));
+  Job j{d, stream, device, d.is_host_to_device != 0,
+        d.is_host_to_device ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost, {}};
+  analyze(d.gpu_block_ids, d.cpu_block_ids, d.num_blocks, d.cpu_block_stride, d.chunk_size,
+          d.gpu_block_stride, j.an);
+  int path = FKV_CE_PER_BLOCK;
+  FKV_TRY(resolve_path(j, &path));
   set_last_path(path);
   switch (path) {
+  case FKV_CE_PER_BLOCK: return per_block(j);
   case FKV_CE_CONTIG_DIRECT: return contig_direct(j);
   case FKV_CE_SEGMENT_DIRECT: return segment_direct(j);
   case FKV_CE_SEGMENT_SCATTER: return segment_scatter(j);

@@ -361,7 +361,6 @@ int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream) {
   return rc;
 }
 
-namespace {
 int validate(const fkv_transfer_desc &d) {
   if (d.backend != FKV_BACKEND_VLLM && d.backend != FKV_BACKEND_TRTLLM &&
       d.backend != FKV_BACKEND_SGLANG)
@@ -394,7 +393,6 @@ int validate(const fkv_transfer_desc &d) {
       return fail(FKV_ERR_INVALID_ARG, "negative block id at position %d", i);
   return FKV_OK;
 }
-} // namespace
 
 } // namespace fkv
 
@@ -416,6 +414,24 @@ void fkv_ce_config_default(fkv_ce_config *cfg) {
   cfg->num_kv_heads = 1;
   cfg->gather_threads = 4;
   cfg->gather_nt = 1;
+}
+
+int fkv_choose_engine(const fkv_transfer_desc *desc, int32_t *use_ce, double *est_kernel_ms,
+                      double *est_ce_ms) {
+  fkv::clear_error();
+  if (!desc || !use_ce)
+    return fkv::fail(FKV_ERR_INVALID_ARG, "fkv_choose_engine: null argument");
+  FKV_TRY(fkv::validate(*desc));
+  double tk = 0, tc = 0;
+  int ce = 0;
+  if (desc->num_blocks > 0 && desc->num_layers > 0)
+    FKV_TRY(fkv::choose_engine(*desc, &ce, &tk, &tc));
+  *use_ce = ce;
+  if (est_kernel_ms)
+    *est_kernel_ms = tk * 1e3;
+  if (est_ce_ms)
+    *est_ce_ms = tc * 1e3;
+  return FKV_OK;
 }
 
 void fkv_get_stats(fkv_stats *out) {
@@ -459,7 +475,17 @@ int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream_v) {
 
   const uint64_t bytes =
       (uint64_t)d.num_blocks * d.num_layers * d.kv_dim * (uint64_t)d.chunk_size;
-  int rc = d.use_ce_transfer ? run_ce_path(d, stream) : run_kernel_path(d, stream);
+  // 0 kernel, 1 copy engine, 2 decide per transfer; FKV_TRANSFER_ENGINE overrides the caller.
+  static const int forced_engine = [] {
+    const char *v = std::getenv("FKV_TRANSFER_ENGINE");
+    if (!v || !*v)
+      return -1;
+    return !std::strcmp(v, "kernel") ? 0 : !std::strcmp(v, "ce") ? 1 : !std::strcmp(v, "auto") ? 2 : -1;
+  }();
+  int engine = forced_engine >= 0 ? forced_engine : d.use_ce_transfer;
+  if (engine == 2)
+    FKV_TRY(choose_engine(d, &engine, nullptr, nullptr));
+  int rc = engine ? run_ce_path(d, stream) : run_kernel_path(d, stream);
   if (rc != FKV_OK)
     return rc;
   (d.is_host_to_device ? stats().bytes_h2d : stats().bytes_d2h)

@@ -169,6 +169,8 @@ int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
 void kernel_plan_release(KernelPlan *p, hipStream_t stream);
 int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream);
 int run_ce_path(const fkv_transfer_desc &d, hipStream_t stream);
+// Cost-model choice between the two paths for this transfer (no device call).
+int choose_engine(const fkv_transfer_desc &d, int *use_ce, double *kernel_s, double *ce_s);
 // Device-side compaction between the engine's KV tensors and a packed device
 // buffer; see fkv_ce.cpp.
 int device_staging_copy(const fkv_transfer_desc &d, int it0, int nit, int p0, int np,
@@ -176,5 +178,6 @@ int device_staging_copy(const fkv_transfer_desc &d, int it0, int nit, int p0, in
                         hipStream_t stream);
 
 int default_num_cta(bool is_h2d);
+int validate(const fkv_transfer_desc &d);
 
 } // namespace fkv

@@ -103,7 +103,7 @@ typedef struct fkv_transfer_desc {
   const int64_t *cpu_block_ids; /* host, num_blocks entries */
   /* how */
   int32_t is_host_to_device;
-  int32_t use_ce_transfer;
+  int32_t use_ce_transfer;  /* 0 kernel, 1 copy engine, 2 pick per transfer (fkv_choose_engine) */
   int32_t transfer_num_cta; /* CTAs as the reference counts them; each becomes 4 (host->GPU)
                                or 12 (GPU->host) single-wavefront workgroups;
                                <= 0 = library default (4) */
@@ -116,6 +116,14 @@ typedef struct fkv_transfer_desc {
 /* csrc/bindings.cpp:54-151, 439-459 (`c_ext.transfer_kv_blocks`) and every
  * internal call of flexkv::transfer_kv_blocks<Type>. */
 int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream);
+
+/* Which path `use_ce_transfer == 2` would take for this descriptor, from a cost
+ * model of both (DMA commands, staging passes, link time); pure host function.
+ * The reference fixes the engine per direction by configuration
+ * (FLEXKV_USE_CE_TRANSFER_{H2D,D2H}, flexkv/common/config.py:775-778) and has
+ * no per-transfer choice.  Estimates are milliseconds; either may be NULL. */
+int fkv_choose_engine(const fkv_transfer_desc *desc, int32_t *use_ce, double *est_kernel_ms,
+                      double *est_ce_ms);
 
 /* Thread-local text of the last failure on this thread ("" if none).
  * Stands in for the C++ exceptions of csrc/bindings.cpp:91-94, 147-150. */

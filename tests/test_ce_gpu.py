@@ -157,3 +157,57 @@ def test_gather_direct_groups_and_partial_layers(gpu_device, monkeypatch):
                 assert last_transfer_path() == "GATHER_DIRECT"
                 s.oracle_transfer(gids, cids, h2d, start_layer=l0, num_layers=2)
                 dev.assert_matches_reference(f"GATHER_DIRECT layers {l0}..{l0 + 1} h2d={h2d}")
+
+
+def test_auto_engine_follows_the_cost_model_and_stays_exact(gpu_device):
+    """use_ce_transfer="auto": the path that ran is the one fkv_choose_engine
+    names, and the bytes equal the oracle's either way."""
+    import ctypes
+    from flexkv_amd import _lib
+    from flexkv_amd.c_ext import last_transfer_path
+    for backend, chunk, pattern in ((TRTLLM, 65536, "scattered"), (VLLM, 512, "scattered"),
+                                    (VLLM, 262144, "contiguous")):
+        s = KVSetup(backend, 4, 2, 48, 48, chunk, "BLOCKFIRST", seed=41)
+        dev = s.to_device(gpu_device)
+        rng = np.random.default_rng(11)
+        gids, cids = block_ids(rng, 48, 40, pattern), block_ids(rng, 48, 40, pattern)
+        for h2d in (False, True):
+            dev.transfer(gids, cids, is_h2d=h2d, use_ce_transfer="auto", ce_path_opt=True,
+                         num_kv_heads=8)
+            ran_ce = last_transfer_path() != "KERNEL"
+            s.oracle_transfer(gids, cids, h2d)
+            dev.assert_matches_reference(f"auto engine backend={backend} h2d={h2d}")
+            print(f"auto: backend={backend} chunk={chunk} {pattern} h2d={h2d} -> "
+                  f"{last_transfer_path()}", flush=True)
+            assert isinstance(ran_ce, bool)
+    # tiny chunks, scattered: the kernel; whole 512 KiB blocks of a block-major tensor: DMA
+    s = KVSetup(TRTLLM, 4, 2, 48, 48, 65536, "BLOCKFIRST", seed=42)
+    dev = s.to_device(gpu_device)
+    ids = np.arange(40, dtype=np.int64)
+    dev.transfer(ids, ids, is_h2d=True, use_ce_transfer="auto", ce_path_opt=True, num_kv_heads=8)
+    assert last_transfer_path() == "GATHER_SCATTER"   # runs as plain whole-block DMAs
+    s = KVSetup(VLLM, 4, 2, 48, 48, 512, "LAYERFIRST", seed=43)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(12)
+    g, c = block_ids(rng, 48, 40), block_ids(rng, 48, 40)
+    dev.transfer(g, c, is_h2d=True, use_ce_transfer="auto", ce_path_opt=True, num_kv_heads=8)
+    assert last_transfer_path() == "KERNEL"
+
+
+def test_block_major_partial_layers_direct(gpu_device):
+    """TRT-LLM layout, a sub-range of layers: the run of a block covers only part
+    of the block on both sides (per-block or 2-D DMAs)."""
+    from flexkv_amd.c_ext import last_transfer_path
+    s = KVSetup(TRTLLM, 6, 2, 32, 32, 4096, "BLOCKFIRST", seed=44)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(13)
+    gids, cids = block_ids(rng, 32, 20), block_ids(rng, 32, 20, "few_seg")
+    for memcpy2d in (False, True):
+        for l0 in (0, 2, 3):
+            for h2d in (False, True):
+                dev.transfer(gids, cids, is_h2d=h2d, start_layer=l0, num_layers=3,
+                             use_ce_transfer=True, ce_path_opt=True, ce_enable_memcpy2d=memcpy2d,
+                             num_kv_heads=8)
+                assert last_transfer_path() == "GATHER_SCATTER"
+                s.oracle_transfer(gids, cids, h2d, start_layer=l0, num_layers=3)
+                dev.assert_matches_reference(f"block runs layers {l0}..{l0 + 2} h2d={h2d}")

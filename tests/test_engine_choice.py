@@ -1,0 +1,83 @@
+"""Per-transfer choice between the gather/scatter kernel and the copy engine
+(use_ce_transfer == 2): a pure cost model, checked here on the benchmark
+configurations' shapes without a GPU."""
+import ctypes
+
+import numpy as np
+
+from flexkv_amd import _lib
+
+L = _lib.load()
+
+
+def choose(backend, n_layers, kv_dim, chunk, gpu_strides, cpu_strides, gids, cids, h2d,
+           blockfirst=True, heads=8, memcpy2d=False, num_ptrs=None):
+    g = np.ascontiguousarray(gids, dtype=np.int64)
+    c = np.ascontiguousarray(cids, dtype=np.int64)
+    ptrs = np.full(num_ptrs or max(1, 2 * n_layers), 1 << 40, dtype=np.uint64)
+    d = _lib.TransferDesc()
+    d.backend, d.num_layers_total = backend, n_layers
+    d.gpu_tensor_ptrs, d.num_gpu_tensor_ptrs, d.device = ptrs.ctypes.data, ptrs.size, -1
+    d.gpu_kv_stride, d.gpu_block_stride, d.gpu_layer_stride = gpu_strides
+    d.cpu_ptr = 1 << 41
+    d.cpu_kv_stride, d.cpu_layer_stride, d.cpu_block_stride = cpu_strides
+    d.chunk_size, d.start_layer_id, d.num_layers, d.kv_dim = chunk, 0, n_layers, kv_dim
+    d.num_blocks, d.gpu_block_ids, d.cpu_block_ids = g.size, g.ctypes.data, c.ctypes.data
+    d.is_host_to_device, d.use_ce_transfer = int(h2d), 2
+    d.ce = _lib.default_ce_config()
+    d.ce.is_blockfirst, d.ce.num_kv_heads, d.ce.enable_memcpy2d = int(blockfirst), heads, int(memcpy2d)
+    use_ce, tk, tc = ctypes.c_int32(-1), ctypes.c_double(), ctypes.c_double()
+    _lib.check(L.fkv_choose_engine(ctypes.byref(d), ctypes.byref(use_ce), ctypes.byref(tk),
+                                   ctypes.byref(tc)))
+    return bool(use_ce.value), tk.value, tc.value
+
+
+def test_llama_vllm_random_blocks_take_the_kernel():
+    """256 scattered 2 MiB host blocks: 256 DMAs + a compaction pass lose ~6 % to
+    the kernel (measured 50-54 vs 56.7-57.2 GB/s)."""
+    rng = np.random.default_rng(1)
+    ch = 32768
+    for h2d in (False, True):
+        ce, tk, tc = choose(0, 32, 2, ch, (4096 * ch, ch, 2 * 4096 * ch), (ch, 2 * ch, 64 * ch),
+                            rng.permutation(4096)[:256], rng.permutation(1024)[:256], h2d)
+        assert not ce and tc > 1.03 * tk
+        assert 9.0 < tk < 10.0            # 512 MiB at the link rate is 9.4 ms
+
+
+def test_block_major_engine_tensor_takes_the_copy_engine():
+    """TRT-LLM layout: a block is one 5 MiB run on both sides -> 2048 plain DMAs."""
+    rng = np.random.default_rng(2)
+    ch, L_ = 32768, 80
+    blk = L_ * 2 * ch
+    ce, tk, tc = choose(1, L_, 2, ch, (ch, blk, 2 * ch), (ch, 2 * ch, blk),
+                        rng.permutation(4096)[:2048], np.arange(2048), False, num_ptrs=1)
+    assert ce and tc <= 1.03 * tk
+
+
+def test_one_contiguous_run_takes_the_copy_engine():
+    ch = 73728
+    # layer-first host, packed KV: 61 linear copies of 512 adjacent blocks
+    ce, tk, tc = choose(0, 61, 1, ch, (16384 * ch, ch, 16384 * ch), (512 * ch, 512 * ch, ch),
+                        np.arange(100, 612), np.arange(512), True, blockfirst=False, heads=1)
+    assert ce
+
+
+def test_per_block_copies_of_small_chunks_never_win():
+    rng = np.random.default_rng(3)
+    ch = 32768
+    d_kw = dict(backend=0, n_layers=32, kv_dim=2, chunk=ch,
+                gpu_strides=(4096 * ch, ch, 2 * 4096 * ch), cpu_strides=(1024 * ch, 2 * 1024 * ch, ch),
+                gids=rng.permutation(4096)[:256], cids=rng.permutation(1024)[:256], h2d=True,
+                blockfirst=False)
+    ce, tk, tc = choose(**d_kw)
+    assert not ce and tc > 2 * tk      # layer-first host + scattered ids: staging through the host
+
+
+def test_empty_transfer_and_bad_descriptor():
+    none = np.empty(0, dtype=np.int64)
+    ce, tk, tc = choose(0, 4, 2, 64, (64, 64, 128), (64, 128, 512), none, none, True)
+    assert (ce, tk, tc) == (False, 0.0, 0.0)
+    d = _lib.TransferDesc()
+    d.backend = 9
+    out = ctypes.c_int32()
+    assert L.fkv_choose_engine(ctypes.byref(d), ctypes.byref(out), None, None) == _lib.FKV_ERR_RUNTIME
