@@ -406,6 +406,49 @@ def run_concurrent(w, torch, steps, warmup, num_cta):
                 blocks=[int(g.numel()) for g, _ in reqs])
 
 
+def run_notify_scales(torch, device, num_cta, iters=20, warmup=3):
+    """Layerwise host->GPU restore end to end (call + device synchronize) at the
+    three scales of the reference's notify-mode microbenchmark
+    (benchmarks/microbenchmark_notify_mode.py:28-33, 87-147): MLA fp16, 16 tokens
+    x 512 dims per block, layer_granularity 1, one GPU, no eventfd consumer."""
+    from flexkv_amd.c_ext import LayerwiseTransferGroup
+    scales = {"small": (8, 16), "medium": (32, 64), "large": (80, 256)}
+    out = {}
+    for name, (L, N) in scales.items():
+        chunk = 16 * 512 * 2
+        full = torch.zeros((L, 1, N, 16, 1, 512), dtype=torch.float16, device=device)
+        gpu = [full[i] for i in range(L)]
+        cpu = torch.zeros((N, L, 1, 16, 1, 512), dtype=torch.float16, pin_memory=True)
+        i64 = lambda v: torch.tensor([v], dtype=torch.int64)
+        ids = torch.arange(N, dtype=torch.int64)
+        empty = torch.empty(0, dtype=torch.int64)
+        row = {"bytes": L * N * chunk}
+        for use_ce in (False, True):
+            grp = LayerwiseTransferGroup(
+                num_gpus=1, gpu_blocks=[gpu], cpu_blocks=cpu, ssd_files={}, num_layers=L,
+                gpu_kv_strides_tensor=i64(N * chunk), gpu_block_strides_tensor=i64(chunk),
+                gpu_layer_strides_tensor=i64(N * chunk), gpu_chunk_sizes_tensor=i64(chunk),
+                iouring_entries=0, iouring_flags=0,
+                layer_eventfds_tensor=torch.empty(0, dtype=torch.int32), tp_size=1,
+                is_blockfirst=True)
+            for notify in ("hostfunc", "polling"):
+                ts = []
+                for it in range(warmup + iters):
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    grp.layerwise_transfer(empty, empty, 0, 0, 0, 0, 0, ids, ids, chunk, chunk,
+                                           L * chunk, chunk, chunk, chunk, L * chunk, num_cta,
+                                           use_ce, L, 1, 1, 1, notify_mode=notify)
+                    torch.cuda.synchronize()
+                    if it >= warmup:
+                        ts.append((time.perf_counter() - t0) * 1e3)
+                key = ("ce_" if use_ce else "kernel_") + notify + "_p50_ms"
+                row[key] = round(_median(ts), 4)
+            grp.close()
+        out[name] = row
+    return out
+
+
 # ---------------------------------------------------------------------------
 # CPU baseline: the reference's CPU path (torch index-gather into the host
 # cache layout), timed on this machine's host cores on a bounded sample.
@@ -453,7 +496,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal"])
+    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify"])
     ap.add_argument("--num-cta", type=int, default=4,
                     help="transfer_num_cta (reference default FLEXKV_TRANSFER_NUM_CTA_*=4)")
     ap.add_argument("--use-ce", action="store_true", help="copy-engine path instead of the kernel")
@@ -486,6 +529,20 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"config": {"workload": "copycal"}, "copy_bytes": n,
                           "copies_of_each_kind": max(1, args.steps)}))
+        return
+    if args.config == "notify":
+        res = run_notify_scales(torch, device, args.num_cta)
+        print(json.dumps({
+            "metric": "layerwise H2D end-to-end ms (p50) by notify mode and scale",
+            "unit": "ms", "n_gpus": 1, "higher_is_better": False, "data": "synthetic",
+            "config": {"workload": "notify: MLA fp16, 16 tok x 512 dim blocks; small 8 layers x 16 "
+                                   "blocks, medium 32 x 64, large 80 x 256; layer_granularity 1"},
+            "results": res,
+            "reference_published_ms": {  # docs/flexkv_config_reference/README_en.md:119
+                "hardware": "NVIDIA 8x GPU, kernel engine, 8 GPUs transferring at once",
+                "small": {"hostfunc": 0.60, "polling": 0.40},
+                "medium": {"hostfunc": 4.39, "polling": 1.87},
+                "large": {"hostfunc": 16.79, "polling": 16.62}}}))
         return
     link = measure_link()
     w = Workload(args.config, torch, device)

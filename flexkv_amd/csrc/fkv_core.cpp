@@ -238,6 +238,12 @@ LinkLaunchShape link_launch_shape(bool is_h2d) {
     s.threads = env_int(h2d ? "FKV_H2D_WG_THREADS" : "FKV_D2H_WG_THREADS", 64);
     if (s.workgroups_per_cta < 1)
       s.workgroups_per_cta = 1;
+    // FKV_{H2D,D2H}_XCD_MASK (e.g. 0xf0 / 0x0f) keeps the two directions on disjoint
+    // XCDs when puts and gets run at the same time; default: all XCDs.
+    const char *m = std::getenv(h2d ? "FKV_H2D_XCD_MASK" : "FKV_D2H_XCD_MASK");
+    s.xcd_mask = (m && *m) ? (unsigned)std::strtoul(m, nullptr, 0) & 0xffu : 0xffu;
+    if (s.xcd_mask == 0)
+      s.xcd_mask = 0xffu;
     return s;
   };
   static const LinkLaunchShape fixed[2] = {read(false), read(true)};
@@ -313,6 +319,7 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
       (d.transfer_num_cta > 0 ? d.transfer_num_cta : default_num_cta(out->h2d)) *
       shape.workgroups_per_cta;
   out->threads = shape.threads;
+  out->xcd_mask = shape.xcd_mask;
   return FKV_OK;
 }
 
@@ -341,6 +348,7 @@ int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
     a.lk = nl * p.kv_dim;
     a.vec = p.vec;
     a.nt_store = p.h2d ? 1 : 0;
+    a.xcd_mask = p.xcd_mask;
     FKV_TRY(launch_copy_kernel(a, p.workgroups, p.threads, stream));
   }
   return FKV_OK;

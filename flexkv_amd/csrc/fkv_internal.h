@@ -113,6 +113,7 @@ struct CopyKernelArgs {
   int32_t slices_per_chunk;
   int32_t vec;      // 16, 8, 4, 2 or 1: widest access all addresses allow
   int32_t nt_store; // 1: nontemporal stores (destination in HBM), 0: plain (pinned host)
+  uint32_t xcd_mask; // bit k: workgroups with blockIdx % 8 == k take part; 0 or 0xff = all
 };
 constexpr int kCopyBlockThreads = 1024;  // largest workgroup the kernel is built for
 constexpr int kCopyUnroll = 8;           // vector accesses in flight per lane
@@ -124,6 +125,7 @@ int launch_copy_kernel(CopyKernelArgs args, int num_workgroups, int threads_per_
 struct LinkLaunchShape {
   int workgroups_per_cta; // workgroups launched per requested CTA
   int threads;            // lanes per workgroup
+  unsigned xcd_mask;      // XCD slots the launch is confined to (0xff = all)
 };
 LinkLaunchShape link_launch_shape(bool is_h2d);
 // Widest vector width (bytes) that divides every value in `vals`.
@@ -159,6 +161,7 @@ struct KernelPlan {
   int kv_dim = 1, num_layers = 0, num_blocks = 0;
   int64_t chunk_size = 0, gpu_block_stride = 0, cpu_block_stride = 0;
   int workgroups = 1, threads = 64;
+  unsigned xcd_mask = 0xff;
 };
 // Builds and uploads (on `stream`) the plan for all layers of `d`.
 int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan *out);

@@ -29,6 +29,10 @@
 // number of bytes in flight spread as single-wavefront workgroups over all
 // XCDs costs them little.  The link-bound launches therefore use one
 // wavefront per workgroup; only the HBM-to-HBM staging pass uses big ones.
+// For the same reason a GPU->host and a host->GPU copy that run at the same
+// time slow each other down when they share XCDs (62 GB/s in sum against
+// 87-90 GB/s on disjoint halves of the chip); `xcd_mask` confines a launch to
+// a subset of the XCDs.
 //
 // Data moves as raw integer vectors (integer types cannot canonicalise NaN
 // payloads of fp8/bf16 data).  Loads are nontemporal: KV bytes are not reused
@@ -91,8 +95,20 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
   const uint32_t slices = (uint32_t)a.slices_per_chunk;
   const uint32_t spp = (uint32_t)a.lk * slices; // slices per block position
   const uint64_t total = (uint64_t)a.num_blocks * spp;
-  const uint64_t s0 = total * blockIdx.x / gridDim.x;
-  const uint64_t s1 = total * (blockIdx.x + 1) / gridDim.x;
+  // Workgroups are handed to the 8 XCDs round-robin by blockIdx.x.  With a
+  // partial mask only the workgroups that land on the selected XCDs take part;
+  // they are renumbered densely, the others leave at once.
+  uint32_t wg = blockIdx.x, nwg = gridDim.x;
+  if ((a.xcd_mask & 0xffu) != 0xffu) {
+    const uint32_t slot = blockIdx.x & 7u;
+    if (!((a.xcd_mask >> slot) & 1u))
+      return;
+    const uint32_t per_round = __popc(a.xcd_mask & 0xffu);
+    wg = (blockIdx.x >> 3) * per_round + __popc(a.xcd_mask & ((1u << slot) - 1u));
+    nwg = (gridDim.x >> 3) * per_round;
+  }
+  const uint64_t s0 = total * wg / nwg;
+  const uint64_t s1 = total * (wg + 1) / nwg;
   if (s0 >= s1)
     return; // whole workgroup leaves together
 
@@ -199,6 +215,14 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_wor
     grid = useful;
   if (grid < 1)
     grid = 1;
+  a.xcd_mask &= 0xffu;
+  if (a.xcd_mask == 0)
+    a.xcd_mask = 0xffu;
+  if (a.xcd_mask != 0xffu) {
+    // `grid` working workgroups need grid / popcount(mask) rounds of 8
+    const int per_round = __builtin_popcount(a.xcd_mask);
+    grid = (grid + per_round - 1) / per_round * 8;
+  }
   const size_t lds_bytes = (size_t)(2 * a.lk + 2 * kCopyIdTile) * sizeof(uint64_t);
   stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);
   switch (a.vec) {

@@ -7,9 +7,14 @@
 // non-blocking stream per GPU.  Behind every batch a hip event is recorded on
 // each GPU's stream.  Completion of a batch is announced
 //   * to consumers in other processes through semaphore eventfds, one
-//     write(1) per (layer, tp_rank), issued either from a stream-ordered host
-//     function (HOSTFUNC) or from a thread that polls the batch events in
-//     order (POLLING) — csrc/layerwise.cpp:15-137, 907-942;
+//     write(1) per (layer, tp_rank) — csrc/layerwise.cpp:15-137, 907-942.
+//     HOSTFUNC mode returns after all copies have landed: the calling thread
+//     waits on the batch events in order and writes the eventfds as each batch
+//     completes.  (The reference enqueues a host function behind every batch;
+//     on this runtime a host function holds its stream for about 50 us, which
+//     would serialise an 80-layer restore by 4 ms, and nothing observable
+//     depends on which thread does the write.)  POLLING mode returns right
+//     after the launches and a thread polls the batch events in order;
 //   * to consumers in this process through fkv_layerwise_wait_layer(), which
 //     makes their stream wait on the batch event (no host round trip).
 //
@@ -45,7 +50,6 @@ struct fkv_layerwise {
     int start_layer = 0;
     int layers = 0;
     std::vector<hipEvent_t> done; // one per GPU
-    std::atomic<int> gpus_left{0};
     fkv_layerwise *owner = nullptr;
   };
   std::vector<std::unique_ptr<Batch>> batches;
@@ -124,14 +128,6 @@ struct fkv_layerwise {
 namespace {
 
 bool is(const char *a, const char *b) { return std::strcmp(a, b) == 0; }
-
-// Runs on a runtime-owned thread, stream-ordered after the batch's copies on
-// one GPU.  Must not call into HIP.
-void batch_done_on_gpu(void *user) {
-  auto *b = static_cast<fkv_layerwise::Batch *>(user);
-  if (b->gpus_left.fetch_sub(1, std::memory_order_acq_rel) == 1)
-    b->owner->notify(*b);
-}
 
 } // namespace
 
@@ -249,7 +245,6 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
     batch->start_layer = b * layer_granularity;
     batch->layers = std::min(layer_granularity, num_layers - batch->start_layer);
     batch->owner = g;
-    batch->gpus_left.store(g->num_gpus);
     batch->done.assign(g->num_gpus, nullptr);
     for (int i = 0; i < g->num_gpus; ++i) {
       FKV_HIP_TRY(hipSetDevice(g->device_ids[i]));
@@ -334,8 +329,6 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
         break;
       (void)hipSetDevice(g->device_ids[i]);
       hipError_t e = hipEventRecord(batch.done[i], g->streams[i]);
-      if (e == hipSuccess && notify_mode == FKV_NOTIFY_HOSTFUNC)
-        e = hipLaunchHostFunc(g->streams[i], batch_done_on_gpu, &batch);
       if (e != hipSuccess) {
         (void)hipGetLastError();
         rc = fail(FKV_ERR_RUNTIME, "layerwise_transfer failed on GPU %d: %s", i,
@@ -366,6 +359,20 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
     if (num_batches > 0 && !g->eventfds.empty())
       g->poller = std::thread([g] { g->poll_loop(); });
   } else {
+    // announce every batch as soon as all GPUs have finished it, in order
+    for (int b = 0; b < num_batches; ++b) {
+      for (int i = 0; i < g->num_gpus; ++i) {
+        (void)hipSetDevice(g->device_ids[i]);
+        hipError_t e = hipEventSynchronize(g->batches[b]->done[i]);
+        if (e != hipSuccess) {
+          (void)hipGetLastError();
+          (void)hipSetDevice(restore.device());
+          return fail(FKV_ERR_RUNTIME, "layerwise_transfer failed on GPU %d: %s", i,
+                      hipGetErrorString(e));
+        }
+      }
+      g->notify(*g->batches[b]);
+    }
     for (int i = 0; i < g->num_gpus; ++i) { // csrc/layerwise.cpp:1249-1256
       (void)hipSetDevice(g->device_ids[i]);
       hipError_t e = hipStreamSynchronize(g->streams[i]);

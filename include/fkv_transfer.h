@@ -260,7 +260,9 @@ int fkv_layerwise_create(const fkv_layerwise_params *params, fkv_layerwise **out
 
 /* csrc/layerwise.cpp:944-1311, host->GPU restore in batches of
  * `layer_granularity` layers.  HOSTFUNC returns after every stream has
- * drained (:1249-1256); POLLING returns right after the launches (:1240-1247).
+ * drained (:1249-1256), the eventfds of a batch having been written as soon as
+ * the batch landed; POLLING returns right after the launches (:1240-1247) and a
+ * library thread writes the eventfds.
  * `mode` is kv_shared_across_ranks_mode (:1112-1166). */
 int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
                            const int64_t *cpu_block_ids, int32_t num_blocks,
