@@ -90,6 +90,44 @@ class LayerwiseParams(Structure):
                 ("num_layer_eventfds", c_int32), ("reserved", c_int32), ("ce", CEConfig)]
 
 
+class LayerGroup(Structure):
+    _fields_ = [("num_layers", c_int32), ("num_tensors_per_gpu", c_int32),
+                ("gpu_block_ptrs_flat", c_void_p), ("cpu_offset_bytes", c_int64),
+                ("h2d_cpu_kv_stride", c_int64), ("h2d_cpu_layer_stride", c_int64),
+                ("cpu_block_stride", c_int64), ("cpu_tp_stride", c_int64),
+                ("gpu_kv_strides", c_void_p), ("gpu_block_strides", c_void_p),
+                ("gpu_layer_strides", c_void_p), ("gpu_chunk_sizes", c_void_p)]
+
+
+class LayerMember(Structure):
+    _fields_ = [("group", c_int32), ("local_layer", c_int32)]
+
+
+class LayerwiseMGParams(Structure):
+    _fields_ = [("num_gpus", c_int32), ("num_original_layers", c_int32),
+                ("tp_size", c_int32), ("num_groups", c_int32),
+                ("groups", POINTER(LayerGroup)), ("member_offsets", c_void_p),
+                ("members", POINTER(LayerMember)), ("cpu_blocks_ptr", c_void_p),
+                ("gpu_device_ids", c_void_p), ("layer_eventfds", c_void_p),
+                ("num_layer_eventfds", c_int32), ("reserved", c_int32), ("ce", CEConfig)]
+
+
+class LayerwiseCall(Structure):
+    _fields_ = [("gpu_block_ids", c_void_p), ("cpu_block_ids", c_void_p),
+                ("num_blocks", c_int32), ("multi_group", c_int32),
+                ("cpu_block_stride", c_int64), ("h2d_cpu_kv_stride", c_int64),
+                ("h2d_cpu_layer_stride", c_int64), ("cpu_tp_stride", c_int64),
+                ("num_layers", c_int32), ("layer_granularity", c_int32),
+                ("transfer_cta_num", c_int32), ("use_ce_transfer", c_int32),
+                ("kv_dim", c_int32), ("num_kv_heads", c_int32),
+                ("counter_id", c_int32), ("notify_mode", c_int32),
+                ("enable_trace", c_int32), ("swa_num_blocks", c_int32),
+                ("kv_shared_across_ranks_mode", c_char_p),
+                ("swa_gpu_block_ids", c_void_p), ("swa_cpu_block_ids", c_void_p),
+                ("swa_h2d_cpu_kv_stride", c_int64), ("swa_h2d_cpu_layer_stride", c_int64),
+                ("swa_cpu_block_stride", c_int64)]
+
+
 class Stats(Structure):
     _fields_ = [("calls", c_uint64), ("bytes_h2d", c_uint64), ("bytes_d2h", c_uint64),
                 ("kernel_launches", c_uint64), ("dma_copies", c_uint64),
@@ -121,6 +159,13 @@ SIGNATURES = {
                                         c_int32, c_int32, c_char_p, c_int32]),
     "fkv_tp_group_destroy": (None, [c_void_p]),
     "fkv_layerwise_create": (c_int32, [POINTER(LayerwiseParams), POINTER(c_void_p)]),
+    "fkv_layerwise_create_multi_group": (c_int32, [POINTER(LayerwiseMGParams),
+                                                   POINTER(c_void_p)]),
+    "fkv_layerwise_init_swa": (c_int32, [c_void_p, POINTER(LayerGroup), c_void_p]),
+    "fkv_layerwise_init_swa_multi_group": (c_int32, [c_void_p, POINTER(LayerGroup), c_int32,
+                                                     c_void_p, POINTER(LayerMember),
+                                                     c_void_p]),
+    "fkv_layerwise_transfer_call": (c_int32, [c_void_p, POINTER(LayerwiseCall)]),
     "fkv_layerwise_transfer": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32,
                                          c_int64, c_int64, c_int64, c_int64,
                                          c_int32, c_int32, c_int32, c_int32, c_int32,

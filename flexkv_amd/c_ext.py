@@ -22,7 +22,8 @@ import numpy as np
 import torch
 
 from . import _lib
-from ._lib import (CEConfig, LayerwiseParams, TPGroupParams, TransferDesc, check,
+from ._lib import (CEConfig, LayerGroup, LayerMember, LayerwiseCall, LayerwiseMGParams,
+                   LayerwiseParams, TPGroupParams, TransferDesc, check,
                    NOTIFY_HOSTFUNC, NOTIFY_POLLING)
 
 _L = _lib.load()
@@ -47,6 +48,14 @@ def _current_stream_handle() -> int:
     if not torch.cuda.is_available():
         return 0
     return int(torch.cuda.current_stream().cuda_stream)
+
+
+def _engine_code(use_ce_transfer) -> int:
+    """False -> copy kernel, True -> copy engine, "auto" (or the integer 2) -> the
+    library's per-transfer choice."""
+    if use_ce_transfer == "auto" or (use_ce_transfer == 2 and not isinstance(use_ce_transfer, bool)):
+        return 2
+    return int(bool(use_ce_transfer))
 
 
 def _ce_config(segment_threshold, path_opt, force_path, enable_memcpy2d, is_blockfirst,
@@ -120,10 +129,7 @@ def transfer_kv_blocks(
     d.cpu_block_ids = cpu_ids.data_ptr()
     d.is_host_to_device = int(bool(is_host_to_device))
     # True/False as in the reference; "auto" (or 2) lets the library pick per transfer
-    if use_ce_transfer == "auto" or (use_ce_transfer == 2 and not isinstance(use_ce_transfer, bool)):
-        d.use_ce_transfer = 2
-    else:
-        d.use_ce_transfer = int(bool(use_ce_transfer))
+    d.use_ce_transfer = _engine_code(use_ce_transfer)
     d.transfer_num_cta = int(transfer_num_cta)
     d.sync = int(bool(sync))
     d.enable_trace = int(bool(enable_transfer_trace))
@@ -242,44 +248,173 @@ def _numel(t) -> int:
     return int(t.numel()) if isinstance(t, torch.Tensor) else len(t)
 
 
+class _GroupArrays:
+    """C descriptions of layer groups plus the numpy buffers they point into."""
+
+    def __init__(self, num_gpus: int, gpu_blocks_per_group, num_layers: Sequence[int],
+                 cpu_offset_bytes, h2d_cpu_kv_strides, h2d_cpu_layer_strides,
+                 cpu_block_strides, cpu_tp_strides, gpu_kv_strides, gpu_block_strides,
+                 gpu_layer_strides, gpu_chunk_sizes, ctx: str) -> None:
+        n = len(num_layers)
+        if len(gpu_blocks_per_group) != n:  # csrc/layerwise.cpp:721-727, 398-404
+            raise RuntimeError(f"{ctx} gpu_blocks_per_group size {len(gpu_blocks_per_group)} "
+                               f"does not match num_groups {n}")
+        self.count = n
+        self.array = (LayerGroup * n)()
+        self.devices: List[int] = []
+        self._keep = []
+        for gi in range(n):
+            per_gpu = gpu_blocks_per_group[gi]
+            if len(per_gpu) != num_gpus:  # :753-757
+                raise RuntimeError(f"{ctx} gpu_blocks_per_group[{gi}].size() != num_gpus")
+            tensors = len(per_gpu[0])
+            ptrs = []
+            for d in range(num_gpus):
+                if len(per_gpu[d]) != tensors:  # :766-772
+                    raise RuntimeError(f"{ctx} gpu_blocks_per_group[{gi}][{d}] tensor count "
+                                       "mismatch")
+                for t in per_gpu[d]:
+                    if t.device.type != "cuda":
+                        raise ValueError("gpu_blocks_per_group must hold device tensors")
+                    ptrs.append(t.data_ptr())
+            if gi == 0:
+                self.devices = [per_gpu[d][0].device.index for d in range(num_gpus)]
+            ptr_arr = np.ascontiguousarray(np.asarray(ptrs, dtype=np.uint64))
+            per_dev = [np.ascontiguousarray(
+                np.asarray(list(a)[gi * num_gpus:(gi + 1) * num_gpus], dtype=np.int64))
+                for a in (gpu_kv_strides, gpu_block_strides, gpu_layer_strides, gpu_chunk_sizes)]
+            for a in per_dev:
+                if a.size != num_gpus:
+                    raise ValueError(f"{ctx} per-GPU stride arrays must hold num_groups*num_gpus "
+                                     "entries")
+            g = self.array[gi]
+            g.num_layers = int(num_layers[gi])
+            g.num_tensors_per_gpu = tensors
+            g.gpu_block_ptrs_flat = ptr_arr.ctypes.data
+            g.cpu_offset_bytes = int(cpu_offset_bytes[gi])
+            g.h2d_cpu_kv_stride = int(h2d_cpu_kv_strides[gi])
+            g.h2d_cpu_layer_stride = int(h2d_cpu_layer_strides[gi])
+            g.cpu_block_stride = int(cpu_block_strides[gi])
+            g.cpu_tp_stride = int(cpu_tp_strides[gi])
+            g.gpu_kv_strides = per_dev[0].ctypes.data
+            g.gpu_block_strides = per_dev[1].ctypes.data
+            g.gpu_layer_strides = per_dev[2].ctypes.data
+            g.gpu_chunk_sizes = per_dev[3].ctypes.data
+            self._keep.append((ptr_arr, per_dev))
+
+
+def _member_csr(layer_members, num_original_layers: int, what: str):
+    if len(layer_members) != num_original_layers:
+        raise RuntimeError(f"{what} length {len(layer_members)} != num_original_layers "
+                           f"{num_original_layers}")
+    offsets = np.zeros(num_original_layers + 1, dtype=np.int32)
+    flat = []
+    for i, ms in enumerate(layer_members):
+        for gi, local in ms:
+            flat.append((int(gi), int(local)))
+        offsets[i + 1] = len(flat)
+    arr = (LayerMember * max(1, len(flat)))()
+    for k, (gi, local) in enumerate(flat):
+        arr[k].group, arr[k].local_layer = gi, local
+    return offsets, arr
+
+
+def _eventfd_array(layer_eventfds_tensor):
+    if layer_eventfds_tensor is None or layer_eventfds_tensor.numel() == 0:
+        return None
+    if layer_eventfds_tensor.dtype != torch.int32:
+        raise TypeError("layer_eventfds_tensor must be int32")
+    return np.ascontiguousarray(layer_eventfds_tensor.cpu().numpy().reshape(-1))
+
+
 class LayerwiseTransferGroup:
     """Per-layer host->GPU restore with completion signalling
-    (``csrc/bindings.cpp:471-545, 657-691``, ``csrc/layerwise.cpp``).
+    (``csrc/bindings.cpp:471-757``, ``csrc/layerwise.cpp``).
 
-    Only the single-group, main-KV form is provided.  SSD pre-load, SWA
-    sidecars and the multi-group constructor raise ``RuntimeError``.
+    Both constructors of the reference are provided and are told apart the way
+    pybind does, by their argument names: the single-group form
+    (``gpu_blocks``, ``num_layers``, ``gpu_*_strides_tensor``) and the
+    multi-group form (``gpu_blocks_per_group``, ``num_original_layers``,
+    ``layer_members``, ``group_*``).  SSD pre-load is not part of this library:
+    non-empty ``ssd_files`` / ``swa_ssd_files`` raise ``RuntimeError``.
     """
 
-    def __init__(self, num_gpus: int = None, gpu_blocks: List[List[torch.Tensor]] = None,
-                 cpu_blocks: torch.Tensor = None, ssd_files: dict = None,
-                 num_layers: int = None, gpu_kv_strides_tensor: torch.Tensor = None,
-                 gpu_block_strides_tensor: torch.Tensor = None,
-                 gpu_layer_strides_tensor: torch.Tensor = None,
-                 gpu_chunk_sizes_tensor: torch.Tensor = None, iouring_entries: int = 0,
-                 iouring_flags: int = 0, layer_eventfds_tensor: torch.Tensor = None,
-                 tp_size: int = 1, has_swa: bool = False, swa_gpu_blocks=(),
-                 swa_cpu_blocks=None, swa_ssd_files=None,
-                 swa_gpu_kv_strides_tensor=None, swa_gpu_block_strides_tensor=None,
-                 swa_gpu_layer_strides_tensor=None, swa_gpu_chunk_sizes_tensor=None,
-                 ce_segment_threshold: int = 8, ce_path_opt: bool = True,
-                 ce_force_path: int = -1, ce_enable_memcpy2d: bool = False,
-                 is_blockfirst: bool = False, num_kv_heads: int = 1,
-                 ce_gather_threads: int = 4, ce_gather_nt: bool = True,
-                 ssd_io_opt: bool = True, **multi_group_kwargs) -> None:
+    _MULTI_NAMES = ("num_gpus", "gpu_blocks_per_group", "cpu_blocks", "ssd_files",
+                    "num_original_layers", "layer_members", "group_num_layers",
+                    "group_cpu_offset_bytes", "group_ssd_offset_bytes",
+                    "group_cpu_layer_strides", "group_cpu_kv_strides",
+                    "group_ssd_layer_strides", "group_ssd_kv_strides", "group_chunk_sizes",
+                    "group_h2d_cpu_kv_strides", "group_h2d_cpu_layer_strides",
+                    "group_cpu_block_strides", "group_cpu_tp_strides", "group_gpu_kv_strides",
+                    "group_gpu_block_strides", "group_gpu_layer_strides",
+                    "group_gpu_chunk_sizes", "iouring_entries", "iouring_flags",
+                    "layer_eventfds_tensor", "tp_size")
+    _SINGLE_NAMES = ("num_gpus", "gpu_blocks", "cpu_blocks", "ssd_files", "num_layers",
+                     "gpu_kv_strides_tensor", "gpu_block_strides_tensor",
+                     "gpu_layer_strides_tensor", "gpu_chunk_sizes_tensor", "iouring_entries",
+                     "iouring_flags", "layer_eventfds_tensor", "tp_size")
+    _COMMON_DEFAULTS = dict(has_swa=False, swa_gpu_blocks=(), swa_cpu_blocks=None,
+                            swa_ssd_files=None, swa_gpu_kv_strides_tensor=None,
+                            swa_gpu_block_strides_tensor=None,
+                            swa_gpu_layer_strides_tensor=None, swa_gpu_chunk_sizes_tensor=None,
+                            ce_segment_threshold=8, ce_path_opt=True, ce_force_path=-1,
+                            ce_enable_memcpy2d=False, is_blockfirst=False, num_kv_heads=1,
+                            ce_gather_threads=4, ce_gather_nt=True, ssd_io_opt=True)
+
+    def __init__(self, *args, **kwargs) -> None:
         self._h = ctypes.c_void_p()
-        if multi_group_kwargs:
-            raise RuntimeError(
-                "the multi-group LayerwiseTransferGroup constructor "
-                f"({sorted(multi_group_kwargs)[0]}, ...) is not part of this library")
-        if ssd_files:
-            raise RuntimeError("SSD->CPU pre-load is not part of this library (ssd_files must be empty)")
-        if has_swa or len(swa_gpu_blocks or ()) > 0:
-            raise RuntimeError("SWA sidecar transfer is not part of this library")
+        multi = ("gpu_blocks_per_group" in kwargs or "layer_members" in kwargs or
+                 (len(args) >= 6 and isinstance(args[5], (list, tuple))))
+        required = self._MULTI_NAMES if multi else self._SINGLE_NAMES
+        names = required + tuple(self._COMMON_DEFAULTS)
+        if len(args) > len(names):
+            raise TypeError(f"LayerwiseTransferGroup takes at most {len(names)} arguments")
+        a = dict(self._COMMON_DEFAULTS)
+        given = dict(zip(names, args))
+        for k, v in kwargs.items():
+            if k not in names:
+                raise TypeError(f"LayerwiseTransferGroup got an unexpected argument {k!r}")
+            if k in given:
+                raise TypeError(f"LayerwiseTransferGroup got {k!r} twice")
+            given[k] = v
+        a.update(given)
+        # tp_size is the one required name the reference's single-group form defaults
+        if not multi:
+            a.setdefault("tp_size", 1)
+            a.setdefault("iouring_entries", 0)
+            a.setdefault("iouring_flags", 0)
+            a.setdefault("layer_eventfds_tensor", None)
+            a.setdefault("ssd_files", None)
+        missing = [k for k in required if k not in a]
+        if missing:
+            raise TypeError(f"LayerwiseTransferGroup missing arguments: {missing}")
+        if a["ssd_files"]:
+            raise RuntimeError("SSD->CPU pre-load is not part of this library "
+                               "(ssd_files must be empty)")
+        if a["swa_ssd_files"]:
+            raise RuntimeError("SSD->CPU pre-load is not part of this library "
+                               "(swa_ssd_files must be empty)")
+        ce = _ce_config(a["ce_segment_threshold"], a["ce_path_opt"], a["ce_force_path"],
+                        a["ce_enable_memcpy2d"], a["is_blockfirst"], a["num_kv_heads"],
+                        a["ce_gather_threads"], a["ce_gather_nt"])
+        num_gpus = int(a["num_gpus"])
+        fds = _eventfd_array(a["layer_eventfds_tensor"])
+        self._num_gpus = num_gpus
+        self._multi_group = multi
+        self._keepalive = [a["cpu_blocks"]]
+        if multi:
+            self._init_multi(a, num_gpus, fds, ce)
+        else:
+            self._init_single(a, num_gpus, fds, ce)
+        self._init_uniform_swa(a, num_gpus)
+
+    def _init_single(self, a, num_gpus, fds, ce) -> None:
+        gpu_blocks = a["gpu_blocks"]
         if gpu_blocks is None or len(gpu_blocks) != num_gpus:
             raise ValueError("gpu_blocks must hold one tensor list per GPU")
         per_gpu = len(gpu_blocks[0])
         ptrs, devs = [], []
-        for g, tensors in enumerate(gpu_blocks):
+        for tensors in gpu_blocks:
             if len(tensors) != per_gpu:
                 raise ValueError("every GPU must bring the same number of KV tensors")
             for t in tensors:
@@ -288,23 +423,20 @@ class LayerwiseTransferGroup:
                 ptrs.append(t.data_ptr())
             devs.append(tensors[0].device.index)
         ptr_arr = np.ascontiguousarray(np.asarray(ptrs, dtype=np.uint64))
-        kvs = _i64_array(gpu_kv_strides_tensor.tolist(), "gpu_kv_strides_tensor", num_gpus)
-        bs = _i64_array(gpu_block_strides_tensor.tolist(), "gpu_block_strides_tensor", num_gpus)
-        ls = _i64_array(gpu_layer_strides_tensor.tolist(), "gpu_layer_strides_tensor", num_gpus)
-        cs = _i64_array(gpu_chunk_sizes_tensor.tolist(), "gpu_chunk_sizes_tensor", num_gpus)
+        kvs = _i64_array(a["gpu_kv_strides_tensor"].tolist(), "gpu_kv_strides_tensor", num_gpus)
+        bs = _i64_array(a["gpu_block_strides_tensor"].tolist(), "gpu_block_strides_tensor",
+                        num_gpus)
+        ls = _i64_array(a["gpu_layer_strides_tensor"].tolist(), "gpu_layer_strides_tensor",
+                        num_gpus)
+        cs = _i64_array(a["gpu_chunk_sizes_tensor"].tolist(), "gpu_chunk_sizes_tensor", num_gpus)
         dev = _i64_array(devs, "gpu_device_ids", num_gpus)
-        fds = None
-        if layer_eventfds_tensor is not None and layer_eventfds_tensor.numel() > 0:
-            if layer_eventfds_tensor.dtype != torch.int32:
-                raise TypeError("layer_eventfds_tensor must be int32")
-            fds = np.ascontiguousarray(layer_eventfds_tensor.cpu().numpy().reshape(-1))
         p = LayerwiseParams()
-        p.num_gpus = int(num_gpus)
+        p.num_gpus = num_gpus
         p.num_tensors_per_gpu = per_gpu
         p.gpu_block_ptrs_flat = ptr_arr.ctypes.data
-        p.cpu_blocks_ptr = cpu_blocks.data_ptr()
-        p.num_layers = int(num_layers)
-        p.tp_size = int(tp_size)
+        p.cpu_blocks_ptr = a["cpu_blocks"].data_ptr()
+        p.num_layers = int(a["num_layers"])
+        p.tp_size = int(a["tp_size"])
         p.gpu_kv_strides = kvs.ctypes.data
         p.gpu_block_strides = bs.ctypes.data
         p.gpu_layer_strides = ls.ctypes.data
@@ -312,21 +444,150 @@ class LayerwiseTransferGroup:
         p.gpu_device_ids = dev.ctypes.data
         p.layer_eventfds = fds.ctypes.data if fds is not None else None
         p.num_layer_eventfds = int(fds.size) if fds is not None else 0
-        p.ce = _ce_config(ce_segment_threshold, ce_path_opt, ce_force_path, ce_enable_memcpy2d,
-                          is_blockfirst, num_kv_heads, ce_gather_threads, ce_gather_nt)
+        p.ce = ce
         # the library keeps raw addresses only: hold the tensors for its lifetime
-        self._keepalive = (gpu_blocks, cpu_blocks)
-        self._num_layers = int(num_layers)
+        self._keepalive.append(gpu_blocks)
+        self._num_layers = int(a["num_layers"])
         check(_L.fkv_layerwise_create(ctypes.byref(p), ctypes.byref(self._h)))
 
-    def init_swa_multi_group(self, *args, **kwargs) -> None:
-        raise RuntimeError("SWA sidecar transfer is not part of this library")
+    def _init_multi(self, a, num_gpus, fds, ce) -> None:
+        n_orig = int(a["num_original_layers"])
+        ctx = "[LayerwiseTransferGroup multi-group]"
+        if len(a["layer_members"]) != n_orig:  # csrc/layerwise.cpp:711-718
+            raise RuntimeError(f"{ctx} layer_members must have length num_original_layers, got "
+                               f"{len(a['layer_members'])} vs expected {n_orig}")
+        groups = _GroupArrays(
+            num_gpus, a["gpu_blocks_per_group"], a["group_num_layers"],
+            a["group_cpu_offset_bytes"], a["group_h2d_cpu_kv_strides"],
+            a["group_h2d_cpu_layer_strides"], a["group_cpu_block_strides"],
+            a["group_cpu_tp_strides"], a["group_gpu_kv_strides"], a["group_gpu_block_strides"],
+            a["group_gpu_layer_strides"], a["group_gpu_chunk_sizes"], ctx)
+        offsets, members = _member_csr(a["layer_members"], n_orig, "layer_members")
+        dev = _i64_array(groups.devices, "gpu_device_ids", num_gpus)
+        p = LayerwiseMGParams()
+        p.num_gpus = num_gpus
+        p.num_original_layers = n_orig
+        p.tp_size = int(a["tp_size"])
+        p.num_groups = groups.count
+        p.groups = groups.array
+        p.member_offsets = offsets.ctypes.data
+        p.members = members
+        p.cpu_blocks_ptr = a["cpu_blocks"].data_ptr()
+        p.gpu_device_ids = dev.ctypes.data
+        p.layer_eventfds = fds.ctypes.data if fds is not None else None
+        p.num_layer_eventfds = int(fds.size) if fds is not None else 0
+        p.ce = ce
+        self._keepalive.append(a["gpu_blocks_per_group"])
+        self._num_layers = n_orig
+        check(_L.fkv_layerwise_create_multi_group(ctypes.byref(p), ctypes.byref(self._h)))
 
-    def layerwise_transfer_multi_group(self, *args, **kwargs) -> None:
-        # csrc/layerwise.cpp:1335-1339
-        raise RuntimeError(
-            "[LayerwiseTransferGroup] layerwise_transfer_multi_group() invoked on a "
-            "single-group instance; use layerwise_transfer() instead.")
+    def _init_uniform_swa(self, a, num_gpus) -> None:
+        # init_swa_sidecar_, csrc/layerwise.cpp:149-153: silently off unless all three hold
+        swa_gpu_blocks = a["swa_gpu_blocks"] or ()
+        swa_cpu = a["swa_cpu_blocks"]
+        if not (a["has_swa"] and len(swa_gpu_blocks) > 0 and swa_cpu is not None
+                and swa_cpu.numel() > 0):
+            return
+        zeros = [0]
+        groups = _GroupArrays(
+            num_gpus, [swa_gpu_blocks], [self._num_layers], zeros, zeros, zeros, zeros, zeros,
+            a["swa_gpu_kv_strides_tensor"].tolist(), a["swa_gpu_block_strides_tensor"].tolist(),
+            a["swa_gpu_layer_strides_tensor"].tolist(),
+            a["swa_gpu_chunk_sizes_tensor"].tolist(), "[LayerwiseTransferGroup SWA]")
+        self._keepalive.append((swa_gpu_blocks, swa_cpu))
+        check(_L.fkv_layerwise_init_swa(self._h, groups.array, swa_cpu.data_ptr()))
+
+    def init_swa_multi_group(
+            self, swa_gpu_blocks_per_group, swa_cpu_blocks, swa_ssd_files, swa_layer_members,
+            swa_group_num_layers, swa_group_cpu_offset_bytes, swa_group_ssd_offset_bytes,
+            swa_group_cpu_layer_strides, swa_group_cpu_kv_strides, swa_group_ssd_layer_strides,
+            swa_group_ssd_kv_strides, swa_group_chunk_sizes, swa_group_h2d_cpu_kv_strides,
+            swa_group_h2d_cpu_layer_strides, swa_group_cpu_block_strides,
+            swa_group_cpu_tp_strides, swa_group_gpu_kv_strides, swa_group_gpu_block_strides,
+            swa_group_gpu_layer_strides, swa_group_gpu_chunk_sizes, iouring_entries: int = 512,
+            iouring_flags: int = 0) -> None:
+        """Attach a sidecar made of its own layer groups
+        (``csrc/layerwise.cpp:355-429``, ``csrc/bindings.cpp:632-656``)."""
+        if swa_ssd_files:
+            raise RuntimeError("SSD->CPU pre-load is not part of this library "
+                               "(swa_ssd_files must be empty)")
+        if swa_cpu_blocks is None or swa_cpu_blocks.numel() == 0:
+            raise RuntimeError("[LayerwiseTransferGroup] init_swa_multi_group() requires "
+                               "non-empty swa_cpu_blocks")
+        if len(swa_layer_members) != self._num_layers:  # :388-393
+            raise RuntimeError(f"[LayerwiseTransferGroup] swa_layer_members length "
+                               f"{len(swa_layer_members)} != num_original_layers "
+                               f"{self._num_layers}")
+        groups = _GroupArrays(
+            self._num_gpus, swa_gpu_blocks_per_group, swa_group_num_layers,
+            swa_group_cpu_offset_bytes, swa_group_h2d_cpu_kv_strides,
+            swa_group_h2d_cpu_layer_strides, swa_group_cpu_block_strides,
+            swa_group_cpu_tp_strides, swa_group_gpu_kv_strides, swa_group_gpu_block_strides,
+            swa_group_gpu_layer_strides, swa_group_gpu_chunk_sizes,
+            "[LayerwiseTransferGroup SWA multi-group]")
+        offsets, members = _member_csr(swa_layer_members, self._num_layers, "swa_layer_members")
+        check(_L.fkv_layerwise_init_swa_multi_group(
+            self._h, groups.array, groups.count, offsets.ctypes.data, members,
+            swa_cpu_blocks.data_ptr()))
+        self._keepalive.append((swa_gpu_blocks_per_group, swa_cpu_blocks))
+
+    def _run(self, call: LayerwiseCall, gpu_block_id_tensor, cpu_block_id_tensor, swa_h2d_src,
+             swa_h2d_dst, ssd_block_ids, swa_disk2h_src, notify_mode: str) -> None:
+        if ssd_block_ids is not None and _numel(ssd_block_ids) > 0:
+            raise RuntimeError("SSD->CPU pre-load is not part of this library")
+        if swa_disk2h_src is not None and _numel(swa_disk2h_src) > 0:
+            raise RuntimeError("SSD->CPU pre-load is not part of this library (swa_disk2h_src)")
+        gpu_ids = _ids(gpu_block_id_tensor, "gpu_block_id_tensor")
+        cpu_ids = _ids(cpu_block_id_tensor, "cpu_block_id_tensor")
+        if gpu_ids.numel() != cpu_ids.numel():
+            raise ValueError("gpu_block_id_tensor and cpu_block_id_tensor differ in length")
+        call.gpu_block_ids = gpu_ids.data_ptr()
+        call.cpu_block_ids = cpu_ids.data_ptr()
+        call.num_blocks = gpu_ids.numel()
+        keep = None
+        if swa_h2d_src is not None and _numel(swa_h2d_src) > 0:
+            src = _ids(swa_h2d_src, "swa_h2d_src")
+            dst = _ids(swa_h2d_dst, "swa_h2d_dst")
+            if src.numel() != dst.numel():
+                raise ValueError("swa_h2d_src and swa_h2d_dst differ in length")
+            call.swa_cpu_block_ids = src.data_ptr()
+            call.swa_gpu_block_ids = dst.data_ptr()
+            call.swa_num_blocks = dst.numel()
+            keep = (src, dst)
+        # any string but "polling" selects the host-function mode, csrc/layerwise.cpp:987-988
+        call.notify_mode = NOTIFY_POLLING if notify_mode == "polling" else NOTIFY_HOSTFUNC
+        check(_L.fkv_layerwise_transfer_call(self._h, ctypes.byref(call)))
+        del keep
+
+    def layerwise_transfer_multi_group(
+            self, ssd_block_ids, cpu_block_ids_d2h, num_blocks_per_file: int, round_robin: int,
+            num_threads_per_device: int, gpu_block_id_tensor: torch.Tensor,
+            cpu_block_id_tensor: torch.Tensor, transfer_cta_num: int, use_ce_transfer: bool,
+            kv_dim: int, num_kv_heads: int, counter_id: int = 0,
+            swa_h2d_src=None, swa_h2d_dst=None, swa_disk2h_src=None, swa_disk2h_dst=None,
+            swa_cpu_kv_stride_in_bytes: int = 0, swa_cpu_layer_stride_in_bytes: int = 0,
+            swa_cpu_block_stride_in_bytes: int = 0, swa_cpu_chunk_size_in_bytes: int = 0,
+            swa_h2d_cpu_kv_stride_in_bytes: int = 0,
+            swa_h2d_cpu_layer_stride_in_bytes: int = 0, swa_cpu_tp_stride_in_bytes: int = 0,
+            swa_ssd_layer_stride_in_bytes: int = 0, swa_ssd_kv_stride_in_bytes: int = 0,
+            swa_num_blocks_per_file: int = 0, kv_shared_across_ranks_mode: str = "sharded",
+            notify_mode: str = "hostfunc", enable_trace: bool = False) -> None:
+        """Restore every group member (and sidecar) of each original layer, one
+        notification per original layer (``csrc/layerwise.cpp:1313-1682``)."""
+        c = LayerwiseCall()
+        c.multi_group = 1
+        c.transfer_cta_num = int(transfer_cta_num)
+        c.use_ce_transfer = _engine_code(use_ce_transfer)
+        c.kv_dim = int(kv_dim)
+        c.num_kv_heads = int(num_kv_heads)
+        c.counter_id = int(counter_id)
+        c.enable_trace = int(bool(enable_trace))
+        c.kv_shared_across_ranks_mode = str(kv_shared_across_ranks_mode).encode()
+        c.swa_h2d_cpu_kv_stride = int(swa_h2d_cpu_kv_stride_in_bytes)
+        c.swa_h2d_cpu_layer_stride = int(swa_h2d_cpu_layer_stride_in_bytes)
+        c.swa_cpu_block_stride = int(swa_cpu_block_stride_in_bytes)
+        self._run(c, gpu_block_id_tensor, cpu_block_id_tensor, swa_h2d_src, swa_h2d_dst,
+                  ssd_block_ids, swa_disk2h_src, notify_mode)
 
     def layerwise_transfer(
             self, ssd_block_ids, cpu_block_ids_d2h, ssd_layer_stride_in_bytes: int,
@@ -346,25 +607,28 @@ class LayerwiseTransferGroup:
             swa_ssd_layer_stride_in_bytes: int = 0, swa_ssd_kv_stride_in_bytes: int = 0,
             swa_num_blocks_per_file: int = 0, kv_shared_across_ranks_mode: str = "sharded",
             notify_mode: str = "hostfunc", enable_trace: bool = False) -> None:
-        if ssd_block_ids is not None and _numel(ssd_block_ids) > 0:
-            raise RuntimeError("SSD->CPU pre-load is not part of this library")
-        for name, t in (("swa_h2d_src", swa_h2d_src), ("swa_h2d_dst", swa_h2d_dst),
-                        ("swa_disk2h_src", swa_disk2h_src), ("swa_disk2h_dst", swa_disk2h_dst)):
-            if t is not None and _numel(t) > 0:
-                raise RuntimeError(f"SWA sidecar transfer is not part of this library ({name})")
-        gpu_ids = _ids(gpu_block_id_tensor, "gpu_block_id_tensor")
-        cpu_ids = _ids(cpu_block_id_tensor, "cpu_block_id_tensor")
-        if gpu_ids.numel() != cpu_ids.numel():
-            raise ValueError("gpu_block_id_tensor and cpu_block_id_tensor differ in length")
-        # any string but "polling" selects the host-function mode, csrc/layerwise.cpp:987-988
-        mode = NOTIFY_POLLING if notify_mode == "polling" else NOTIFY_HOSTFUNC
-        check(_L.fkv_layerwise_transfer(
-            self._h, gpu_ids.data_ptr(), cpu_ids.data_ptr(), gpu_ids.numel(),
-            int(cpu_block_stride_in_bytes), int(h2d_cpu_kv_stride_in_bytes),
-            int(h2d_cpu_layer_stride_in_bytes), int(cpu_tp_stride_in_bytes),
-            int(transfer_cta_num), int(bool(use_ce_transfer)), int(num_layers),
-            int(layer_granularity), int(kv_dim), int(num_kv_heads), int(counter_id),
-            str(kv_shared_across_ranks_mode).encode(), mode, int(bool(enable_trace))))
+        """Restore ``num_layers`` layers in batches of ``layer_granularity``
+        (``csrc/layerwise.cpp:944-1311``)."""
+        c = LayerwiseCall()
+        c.multi_group = 0
+        c.cpu_block_stride = int(cpu_block_stride_in_bytes)
+        c.h2d_cpu_kv_stride = int(h2d_cpu_kv_stride_in_bytes)
+        c.h2d_cpu_layer_stride = int(h2d_cpu_layer_stride_in_bytes)
+        c.cpu_tp_stride = int(cpu_tp_stride_in_bytes)
+        c.num_layers = int(num_layers)
+        c.layer_granularity = int(layer_granularity)
+        c.transfer_cta_num = int(transfer_cta_num)
+        c.use_ce_transfer = _engine_code(use_ce_transfer)
+        c.kv_dim = int(kv_dim)
+        c.num_kv_heads = int(num_kv_heads)
+        c.counter_id = int(counter_id)
+        c.enable_trace = int(bool(enable_trace))
+        c.kv_shared_across_ranks_mode = str(kv_shared_across_ranks_mode).encode()
+        c.swa_h2d_cpu_kv_stride = int(swa_h2d_cpu_kv_stride_in_bytes)
+        c.swa_h2d_cpu_layer_stride = int(swa_h2d_cpu_layer_stride_in_bytes)
+        c.swa_cpu_block_stride = int(swa_cpu_block_stride_in_bytes)
+        self._run(c, gpu_block_id_tensor, cpu_block_id_tensor, swa_h2d_src, swa_h2d_dst,
+                  ssd_block_ids, swa_disk2h_src, notify_mode)
 
     # ---- additions for consumers in the same process -------------------------
     def wait_layer(self, layer: int, stream: Optional["torch.cuda.Stream"] = None,

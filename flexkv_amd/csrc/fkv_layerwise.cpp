@@ -1,11 +1,15 @@
 // Layer-by-layer host->GPU restore with per-layer completion signalling, so
 // that attention on layer L can start while layer L+1 is still on the link.
-// Replaces the single-group, main-KV part of LayerwiseTransferGroup in the
-// reference (csrc/layerwise.{h,cpp}).
+// Replaces LayerwiseTransferGroup of the reference (csrc/layerwise.{h,cpp})
+// without its SSD pre-load: the single-group form, the multi-group form (layer
+// groups of different KV shape that share the original layers of the model) and
+// the sliding-window sidecars of both.
 //
-// Per call, layers go out in batches of `layer_granularity` on one
-// non-blocking stream per GPU.  Behind every batch a hip event is recorded on
-// each GPU's stream.  Completion of a batch is announced
+// A restore is a sequence of batches on one non-blocking stream per GPU.  A
+// batch is `layer_granularity` consecutive layers (single group) or everything
+// attached to one original layer (multi-group: the members of every group, then
+// the sidecar).  Behind every batch a hip event is recorded on each GPU's
+// stream.  Completion of a batch is announced
 //   * to consumers in other processes through semaphore eventfds, one
 //     write(1) per (layer, tp_rank) — csrc/layerwise.cpp:15-137, 907-942.
 //     HOSTFUNC mode returns after all copies have landed: the calling thread
@@ -18,6 +22,10 @@
 //   * to consumers in this process through fkv_layerwise_wait_layer(), which
 //     makes their stream wait on the batch event (no host round trip).
 //
+// On the kernel path the id lists and the base tables of every layer of a group
+// go to the device once per call and GPU; each (batch, group) is then a single
+// kernel launch.
+//
 // The transfer streams keep the default priority.
 #include "fkv_internal.h"
 
@@ -29,15 +37,116 @@
 #include <memory>
 #include <thread>
 
+namespace {
+
+bool is(const char *a, const char *b) { return std::strcmp(a, b) == 0; }
+
+// csrc/layerwise.cpp:586-595, 792-806
+int backend_of(int tensors_per_gpu, int num_layers) {
+  if (tensors_per_gpu == 1)
+    return FKV_BACKEND_TRTLLM;
+  if (tensors_per_gpu == num_layers)
+    return FKV_BACKEND_VLLM;
+  if (tensors_per_gpu == 2 * num_layers)
+    return FKV_BACKEND_SGLANG;
+  return -1;
+}
+
+// Device tensors of one layer group and where the group lives inside a host
+// block (GroupParams of the reference).
+struct Source {
+  int num_layers = 0;
+  int num_tensors_per_gpu = 0;
+  int backend = 0;
+  std::vector<uint64_t> gpu_ptrs; // [num_gpus][num_tensors_per_gpu]
+  std::vector<int64_t> kv_strides, block_strides, layer_strides, chunk_sizes; // per GPU
+  int64_t cpu_offset_bytes = 0;
+  int64_t h2d_cpu_kv_stride = 0, h2d_cpu_layer_stride = 0;
+  int64_t cpu_block_stride = 0, cpu_tp_stride = 0;
+};
+
+bool fill_source(Source &s, const fkv_layer_group &in, int num_gpus) {
+  if (in.num_layers < 1 || in.num_tensors_per_gpu < 1 || !in.gpu_block_ptrs_flat ||
+      !in.gpu_kv_strides || !in.gpu_block_strides || !in.gpu_layer_strides ||
+      !in.gpu_chunk_sizes)
+    return false;
+  s.num_layers = in.num_layers;
+  s.num_tensors_per_gpu = in.num_tensors_per_gpu;
+  s.backend = backend_of(in.num_tensors_per_gpu, in.num_layers);
+  const size_t nptr = (size_t)num_gpus * in.num_tensors_per_gpu;
+  s.gpu_ptrs.assign(in.gpu_block_ptrs_flat, in.gpu_block_ptrs_flat + nptr);
+  s.kv_strides.assign(in.gpu_kv_strides, in.gpu_kv_strides + num_gpus);
+  s.block_strides.assign(in.gpu_block_strides, in.gpu_block_strides + num_gpus);
+  s.layer_strides.assign(in.gpu_layer_strides, in.gpu_layer_strides + num_gpus);
+  s.chunk_sizes.assign(in.gpu_chunk_sizes, in.gpu_chunk_sizes + num_gpus);
+  s.cpu_offset_bytes = in.cpu_offset_bytes;
+  s.h2d_cpu_kv_stride = in.h2d_cpu_kv_stride;
+  s.h2d_cpu_layer_stride = in.h2d_cpu_layer_stride;
+  s.cpu_block_stride = in.cpu_block_stride;
+  s.cpu_tp_stride = in.cpu_tp_stride;
+  return true;
+}
+
+using MemberTable = std::vector<std::vector<fkv_layer_member>>;
+
+// Unpacks the CSR member lists and checks every entry against the groups.
+int fill_members(MemberTable &out, int num_original_layers, const int32_t *offsets,
+                 const fkv_layer_member *members, const std::vector<Source> &groups,
+                 const char *what) {
+  using namespace fkv;
+  if (!offsets)
+    return fail(FKV_ERR_INVALID_ARG, "%s: member_offsets is null", what);
+  out.assign(num_original_layers, {});
+  for (int l = 0; l < num_original_layers; ++l) {
+    if (offsets[l + 1] < offsets[l] || offsets[l] < 0)
+      return fail(FKV_ERR_INVALID_ARG, "%s: member_offsets must be non-decreasing", what);
+    for (int k = offsets[l]; k < offsets[l + 1]; ++k) {
+      const fkv_layer_member m = members[k];
+      if (m.group < 0 || m.group >= (int)groups.size() || m.local_layer < 0 ||
+          m.local_layer >= groups[m.group].num_layers)
+        return fail(FKV_ERR_INVALID_ARG,
+                    "%s: member (group %d, layer %d) of original layer %d is out of range", what,
+                    m.group, m.local_layer, l);
+      out[l].push_back(m);
+    }
+  }
+  return FKV_OK;
+}
+
+// A Source as one call uses it: block ids, host strides and per-GPU host
+// offsets resolved, plus the uploaded kernel plans.
+struct Lane {
+  const Source *src = nullptr;
+  void *cpu_ptr = nullptr;
+  int64_t cpu_kv_stride = 0, cpu_layer_stride = 0, cpu_block_stride = 0;
+  std::vector<int64_t> cpu_off; // per GPU
+  const int64_t *gpu_ids = nullptr, *cpu_ids = nullptr;
+  int num_blocks = 0;
+  int kv_dim = 1;
+  bool used = false;
+  std::vector<fkv::KernelPlan> plans; // per GPU, kernel path only
+};
+
+struct Item {
+  int lane = 0;
+  int start_layer = 0;
+  int layers = 0;
+};
+
+} // namespace
+
 struct fkv_layerwise {
   int num_gpus = 0;
-  int num_tensors_per_gpu = 0;
-  int num_layers = 0;
+  int num_layers = 0; // original layers: the extent of the eventfd table
   int tp_size = 1;
-  int backend = 0;
+  bool multi_group = false;
   void *cpu_blocks = nullptr;
-  std::vector<uint64_t> gpu_ptrs;
-  std::vector<int64_t> kv_strides, block_strides, layer_strides, chunk_sizes;
+  std::vector<Source> groups; // exactly one for a single-group instance
+  MemberTable members;        // multi-group only
+  bool has_swa = false, swa_multi_group = false;
+  void *swa_cpu_blocks = nullptr;
+  std::vector<Source> swa_groups; // exactly one for the uniform sidecar
+  MemberTable swa_members;
   std::vector<int> device_ids;
   std::vector<hipStream_t> streams;
   fkv_ce_config ce{};
@@ -49,23 +158,24 @@ struct fkv_layerwise {
   struct Batch {
     int start_layer = 0;
     int layers = 0;
+    std::vector<Item> items;
     std::vector<hipEvent_t> done; // one per GPU
-    fkv_layerwise *owner = nullptr;
+    int num_members = 0;          // multi-group: main members of the original layer
+    double trace_bytes = 0;
   };
   std::vector<std::unique_ptr<Batch>> batches;
+  std::vector<int> layer_batch; // layer -> index into batches, -1: nothing in flight
   hipEvent_t started = nullptr; // on streams[0], before the first batch
-  int granularity = 1;
   int counter_id = 0;
-  int notify_mode = FKV_NOTIFY_HOSTFUNC;
   std::thread poller;
   std::atomic<bool> poller_stop{false};
 
   // csrc/layerwise.cpp:15-34
-  void notify(const Batch &b) const {
+  void notify_layers(int start_layer, int layers) const {
     if (eventfds.empty())
       return;
     const int32_t *base = eventfds.data() + (size_t)counter_id * tp_size * num_layers;
-    for (int layer = b.start_layer; layer < b.start_layer + b.layers; ++layer)
+    for (int layer = start_layer; layer < start_layer + layers; ++layer)
       for (int r = 0; r < tp_size; ++r) {
         const int fd = base[(size_t)r * num_layers + layer];
         if (fd >= 0) {
@@ -75,6 +185,7 @@ struct fkv_layerwise {
         }
       }
   }
+  void notify(const Batch &b) const { notify_layers(b.start_layer, b.layers); }
 
   void poll_loop() {
     size_t next = 0;
@@ -115,6 +226,7 @@ struct fkv_layerwise {
           (void)hipEventDestroy(b->done[g]);
       }
     batches.clear();
+    layer_batch.clear();
     if (started) {
       (void)hipSetDevice(device_ids[0]);
       (void)hipEventDestroy(started);
@@ -127,58 +239,24 @@ struct fkv_layerwise {
 
 namespace {
 
-bool is(const char *a, const char *b) { return std::strcmp(a, b) == 0; }
-
-} // namespace
-
-extern "C" {
-
-int fkv_layerwise_create(const fkv_layerwise_params *p, fkv_layerwise **out) {
+// Devices, eventfd table and streams: what both constructors share.
+int finish_create(std::unique_ptr<fkv_layerwise> &g, const int64_t *gpu_device_ids,
+                  const int32_t *layer_eventfds, int num_layer_eventfds) {
   using namespace fkv;
-  clear_error();
-  if (!p || !out || p->num_gpus < 1 || p->num_tensors_per_gpu < 1 || p->num_layers < 1 ||
-      p->tp_size < 1 || !p->gpu_block_ptrs_flat || !p->gpu_kv_strides ||
-      !p->gpu_block_strides || !p->gpu_layer_strides || !p->gpu_chunk_sizes ||
-      !p->gpu_device_ids)
-    return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_create: bad arguments");
-  int backend;
-  if (p->num_tensors_per_gpu == 1)
-    backend = FKV_BACKEND_TRTLLM;
-  else if (p->num_tensors_per_gpu == p->num_layers)
-    backend = FKV_BACKEND_VLLM;
-  else if (p->num_tensors_per_gpu == 2 * p->num_layers)
-    backend = FKV_BACKEND_SGLANG;
-  else // csrc/layerwise.cpp:586-595
-    return fail(FKV_ERR_RUNTIME, "Unsupported GPU block type: %d", p->num_tensors_per_gpu);
-  if (p->num_layer_eventfds > 0) {
-    if (!p->layer_eventfds || p->num_layer_eventfds % (p->tp_size * p->num_layers) != 0)
+  if (num_layer_eventfds > 0) {
+    const int per_counter = g->tp_size * g->num_layers;
+    if (!layer_eventfds || num_layer_eventfds % per_counter != 0)
       return fail(FKV_ERR_INVALID_ARG,
                   "layer_eventfds must hold a multiple of tp_size*num_layers = %d entries, got %d",
-                  p->tp_size * p->num_layers, p->num_layer_eventfds);
+                  per_counter, num_layer_eventfds);
+    g->eventfds.assign(layer_eventfds, layer_eventfds + num_layer_eventfds);
+    g->num_counters = num_layer_eventfds / per_counter;
   }
-  auto g = std::make_unique<fkv_layerwise>();
-  g->num_gpus = p->num_gpus;
-  g->num_tensors_per_gpu = p->num_tensors_per_gpu;
-  g->num_layers = p->num_layers;
-  g->tp_size = p->tp_size;
-  g->backend = backend;
-  g->cpu_blocks = p->cpu_blocks_ptr;
-  g->ce = p->ce;
-  const size_t nptr = (size_t)p->num_gpus * p->num_tensors_per_gpu;
-  g->gpu_ptrs.assign(p->gpu_block_ptrs_flat, p->gpu_block_ptrs_flat + nptr);
-  g->kv_strides.assign(p->gpu_kv_strides, p->gpu_kv_strides + p->num_gpus);
-  g->block_strides.assign(p->gpu_block_strides, p->gpu_block_strides + p->num_gpus);
-  g->layer_strides.assign(p->gpu_layer_strides, p->gpu_layer_strides + p->num_gpus);
-  g->chunk_sizes.assign(p->gpu_chunk_sizes, p->gpu_chunk_sizes + p->num_gpus);
-  for (int i = 0; i < p->num_gpus; ++i)
-    g->device_ids.push_back((int)p->gpu_device_ids[i]);
-  if (p->num_layer_eventfds > 0) {
-    g->eventfds.assign(p->layer_eventfds, p->layer_eventfds + p->num_layer_eventfds);
-    g->num_counters = p->num_layer_eventfds / (p->tp_size * p->num_layers);
-  }
+  for (int i = 0; i < g->num_gpus; ++i)
+    g->device_ids.push_back((int)gpu_device_ids[i]);
   DeviceGuard restore(-1);
-  g->streams.assign(p->num_gpus, nullptr);
-  for (int i = 0; i < p->num_gpus; ++i) {
+  g->streams.assign(g->num_gpus, nullptr);
+  for (int i = 0; i < g->num_gpus; ++i) {
     hipError_t e = hipSetDevice(g->device_ids[i]);
     if (e == hipSuccess)
       e = hipStreamCreateWithFlags(&g->streams[i], hipStreamNonBlocking);
@@ -194,42 +272,213 @@ int fkv_layerwise_create(const fkv_layerwise_params *p, fkv_layerwise **out) {
     }
   }
   (void)hipSetDevice(restore.device());
+  return FKV_OK;
+}
+
+fkv_transfer_desc describe(const fkv_layerwise *g, const Lane &lane, int gpu, int start,
+                           int layers, const fkv_layerwise_call &c) {
+  const Source &s = *lane.src;
+  fkv_transfer_desc d{};
+  d.backend = s.backend;
+  d.num_layers_total = s.num_layers;
+  d.gpu_tensor_ptrs = s.gpu_ptrs.data() + (size_t)gpu * s.num_tensors_per_gpu;
+  d.num_gpu_tensor_ptrs = s.num_tensors_per_gpu;
+  d.device = g->device_ids[gpu];
+  d.gpu_kv_stride = s.kv_strides[gpu];
+  d.gpu_block_stride = s.block_strides[gpu];
+  d.gpu_layer_stride = s.layer_strides[gpu];
+  d.gpu_startoff_inside_chunks = 0;
+  d.cpu_ptr = lane.cpu_ptr;
+  d.cpu_kv_stride = lane.cpu_kv_stride;
+  d.cpu_layer_stride = lane.cpu_layer_stride;
+  d.cpu_block_stride = lane.cpu_block_stride;
+  d.cpu_startoff_inside_chunks = lane.cpu_off[gpu];
+  d.chunk_size = s.chunk_sizes[gpu];
+  d.start_layer_id = start;
+  d.num_layers = layers;
+  d.kv_dim = lane.kv_dim;
+  d.num_blocks = lane.num_blocks;
+  d.gpu_block_ids = lane.gpu_ids;
+  d.cpu_block_ids = lane.cpu_ids;
+  d.is_host_to_device = 1;
+  d.use_ce_transfer = c.use_ce_transfer;
+  d.transfer_num_cta = c.transfer_cta_num;
+  d.sync = 0;
+  d.ce = g->ce;
+  return d;
+}
+
+} // namespace
+
+extern "C" {
+
+int fkv_layerwise_create(const fkv_layerwise_params *p, fkv_layerwise **out) {
+  using namespace fkv;
+  clear_error();
+  if (!p || !out || p->num_gpus < 1 || p->num_tensors_per_gpu < 1 || p->num_layers < 1 ||
+      p->tp_size < 1 || !p->gpu_block_ptrs_flat || !p->gpu_kv_strides ||
+      !p->gpu_block_strides || !p->gpu_layer_strides || !p->gpu_chunk_sizes ||
+      !p->gpu_device_ids)
+    return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_create: bad arguments");
+  if (backend_of(p->num_tensors_per_gpu, p->num_layers) < 0) // csrc/layerwise.cpp:586-595
+    return fail(FKV_ERR_RUNTIME, "Unsupported GPU block type: %d", p->num_tensors_per_gpu);
+  auto g = std::make_unique<fkv_layerwise>();
+  g->num_gpus = p->num_gpus;
+  g->num_layers = p->num_layers;
+  g->tp_size = p->tp_size;
+  g->cpu_blocks = p->cpu_blocks_ptr;
+  g->ce = p->ce;
+  fkv_layer_group in{};
+  in.num_layers = p->num_layers;
+  in.num_tensors_per_gpu = p->num_tensors_per_gpu;
+  in.gpu_block_ptrs_flat = p->gpu_block_ptrs_flat;
+  in.gpu_kv_strides = p->gpu_kv_strides;
+  in.gpu_block_strides = p->gpu_block_strides;
+  in.gpu_layer_strides = p->gpu_layer_strides;
+  in.gpu_chunk_sizes = p->gpu_chunk_sizes;
+  g->groups.resize(1);
+  fill_source(g->groups[0], in, p->num_gpus);
+  FKV_TRY(finish_create(g, p->gpu_device_ids, p->layer_eventfds, p->num_layer_eventfds));
   *out = g.release();
   return FKV_OK;
 }
 
-int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
-                           const int64_t *cpu_block_ids, int32_t num_blocks,
-                           int64_t cpu_block_stride, int64_t h2d_cpu_kv_stride,
-                           int64_t h2d_cpu_layer_stride, int64_t cpu_tp_stride,
-                           int32_t transfer_cta_num, int32_t use_ce_transfer,
-                           int32_t num_layers, int32_t layer_granularity, int32_t kv_dim,
-                           int32_t num_kv_heads, int32_t counter_id, const char *mode_in,
-                           int32_t notify_mode, int32_t enable_trace) {
+int fkv_layerwise_create_multi_group(const fkv_layerwise_mg_params *p, fkv_layerwise **out) {
   using namespace fkv;
   clear_error();
-  if (!g)
-    return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_transfer: null group");
-  if (num_layers < 0 || num_layers > g->num_layers || layer_granularity < 1 || num_blocks < 0)
+  if (!p || !out || p->num_gpus < 1 || p->num_original_layers < 1 || p->tp_size < 1 ||
+      p->num_groups < 1 || !p->groups || !p->gpu_device_ids)
+    return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_create_multi_group: bad arguments");
+  auto g = std::make_unique<fkv_layerwise>();
+  g->num_gpus = p->num_gpus;
+  g->num_layers = p->num_original_layers;
+  g->tp_size = p->tp_size;
+  g->multi_group = true;
+  g->cpu_blocks = p->cpu_blocks_ptr;
+  g->ce = p->ce;
+  g->groups.resize(p->num_groups);
+  for (int gi = 0; gi < p->num_groups; ++gi) {
+    if (!fill_source(g->groups[gi], p->groups[gi], p->num_gpus))
+      return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_create_multi_group: group %d is incomplete",
+                  gi);
+    if (g->groups[gi].backend < 0) // csrc/layerwise.cpp:792-806
+      return fail(FKV_ERR_RUNTIME,
+                  "[LayerwiseTransferGroup multi-group] group %d has unsupported "
+                  "tensors_per_gpu=%d for num_layers=%d",
+                  gi, g->groups[gi].num_tensors_per_gpu, g->groups[gi].num_layers);
+  }
+  FKV_TRY(fill_members(g->members, p->num_original_layers, p->member_offsets, p->members,
+                       g->groups, "fkv_layerwise_create_multi_group"));
+  FKV_TRY(finish_create(g, p->gpu_device_ids, p->layer_eventfds, p->num_layer_eventfds));
+  *out = g.release();
+  return FKV_OK;
+}
+
+int fkv_layerwise_init_swa(fkv_layerwise *g, const fkv_layer_group *swa,
+                           void *swa_cpu_blocks_ptr) {
+  using namespace fkv;
+  clear_error();
+  if (!g || !swa || !swa_cpu_blocks_ptr)
+    return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_init_swa: null argument");
+  if (g->has_swa)
+    return fail(FKV_ERR_RUNTIME, "[LayerwiseTransferGroup] SWA was already initialized");
+  // The sidecar holds one ring per layer of the model (csrc/layerwise.cpp:180-190).
+  fkv_layer_group in = *swa;
+  in.num_layers = g->num_layers;
+  Source s;
+  if (!fill_source(s, in, g->num_gpus))
+    return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_init_swa: incomplete group description");
+  if (s.backend < 0)
+    return fail(FKV_ERR_RUNTIME, "Unsupported SWA GPU block type: %d", s.num_tensors_per_gpu);
+  g->retire_previous();
+  g->swa_groups.assign(1, s);
+  g->swa_members.clear();
+  g->swa_cpu_blocks = swa_cpu_blocks_ptr;
+  g->has_swa = true;
+  g->swa_multi_group = false;
+  return FKV_OK;
+}
+
+int fkv_layerwise_init_swa_multi_group(fkv_layerwise *g, const fkv_layer_group *groups,
+                                       int32_t num_groups, const int32_t *member_offsets,
+                                       const fkv_layer_member *members,
+                                       void *swa_cpu_blocks_ptr) {
+  using namespace fkv;
+  clear_error();
+  if (!g || !groups || num_groups < 1)
+    return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_init_swa_multi_group: null argument");
+  if (g->has_swa) // csrc/layerwise.cpp:378-382
+    return fail(FKV_ERR_RUNTIME,
+                "[LayerwiseTransferGroup] init_swa_multi_group() called but SWA was "
+                "already initialized (uniform or multi-group)");
+  if (!swa_cpu_blocks_ptr) // :383-387
+    return fail(FKV_ERR_RUNTIME,
+                "[LayerwiseTransferGroup] init_swa_multi_group() requires non-empty "
+                "swa_cpu_blocks");
+  std::vector<Source> srcs(num_groups);
+  for (int gi = 0; gi < num_groups; ++gi) {
+    if (!fill_source(srcs[gi], groups[gi], g->num_gpus))
+      return fail(FKV_ERR_INVALID_ARG,
+                  "fkv_layerwise_init_swa_multi_group: group %d is incomplete", gi);
+    if (srcs[gi].backend < 0) // :335-346
+      return fail(FKV_ERR_RUNTIME,
+                  "[LayerwiseTransferGroup SWA multi-group] group %d has unsupported "
+                  "tensors_per_gpu=%d for num_layers=%d",
+                  gi, srcs[gi].num_tensors_per_gpu, srcs[gi].num_layers);
+  }
+  MemberTable table;
+  FKV_TRY(fill_members(table, g->num_layers, member_offsets, members, srcs,
+                       "fkv_layerwise_init_swa_multi_group"));
+  g->retire_previous();
+  g->swa_groups = std::move(srcs);
+  g->swa_members = std::move(table);
+  g->swa_cpu_blocks = swa_cpu_blocks_ptr;
+  g->has_swa = true;
+  g->swa_multi_group = true;
+  return FKV_OK;
+}
+
+int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call) {
+  using namespace fkv;
+  clear_error();
+  if (!g || !call)
+    return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_transfer_call: null argument");
+  const fkv_layerwise_call &c = *call;
+  if (c.multi_group && !g->multi_group) // csrc/layerwise.cpp:1335-1339
+    return fail(FKV_ERR_RUNTIME,
+                "[LayerwiseTransferGroup] layerwise_transfer_multi_group() invoked on "
+                "a single-group instance; use layerwise_transfer() instead.");
+  if (!c.multi_group && g->multi_group) // :975-979
+    return fail(FKV_ERR_RUNTIME,
+                "[LayerwiseTransferGroup] layerwise_transfer() invoked on a "
+                "multi-group instance; use layerwise_transfer_multi_group() instead.");
+  if (c.num_blocks < 0 || c.swa_num_blocks < 0 || c.kv_dim < 1)
+    return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_transfer: num_blocks=%d swa_num_blocks=%d "
+                "kv_dim=%d", c.num_blocks, c.swa_num_blocks, c.kv_dim);
+  if (!g->multi_group &&
+      (c.num_layers < 0 || c.num_layers > g->num_layers || c.layer_granularity < 1))
     return fail(FKV_ERR_INVALID_ARG,
-                "fkv_layerwise_transfer: num_layers=%d (group has %d) layer_granularity=%d "
-                "num_blocks=%d",
-                num_layers, g->num_layers, layer_granularity, num_blocks);
-  if (!g->eventfds.empty() && (counter_id < 0 || counter_id >= g->num_counters))
-    return fail(FKV_ERR_INVALID_ARG, "counter_id %d outside [0, %d)", counter_id,
+                "fkv_layerwise_transfer: num_layers=%d (group has %d) layer_granularity=%d",
+                c.num_layers, g->num_layers, c.layer_granularity);
+  if (c.num_blocks > 0 && (!c.gpu_block_ids || !c.cpu_block_ids))
+    return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_transfer: null block id list");
+  if (!g->eventfds.empty() && (c.counter_id < 0 || c.counter_id >= g->num_counters))
+    return fail(FKV_ERR_INVALID_ARG, "counter_id %d outside [0, %d)", c.counter_id,
                 g->num_counters);
-  if (notify_mode != FKV_NOTIFY_HOSTFUNC && notify_mode != FKV_NOTIFY_POLLING)
-    return fail(FKV_ERR_INVALID_ARG, "unknown notify mode %d", notify_mode);
+  if (c.notify_mode != FKV_NOTIFY_HOSTFUNC && c.notify_mode != FKV_NOTIFY_POLLING)
+    return fail(FKV_ERR_INVALID_ARG, "unknown notify mode %d", c.notify_mode);
+  // csrc/layerwise.cpp:1091, 1362: the sidecar moves only when ids came along
+  const bool swa_active = g->has_swa && c.swa_num_blocks > 0;
+  if (swa_active && (!c.swa_gpu_block_ids || !c.swa_cpu_block_ids))
+    return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_transfer: null SWA block id list");
 
   g->retire_previous();
-  g->counter_id = counter_id;
-  g->granularity = layer_granularity;
-  g->notify_mode = notify_mode;
+  g->counter_id = c.counter_id;
 
-  // csrc/layerwise.cpp:1112-1121: only these three names are meaningful for a
-  // restore; anything else is treated as "sharded".
-  const char *mode = mode_in ? mode_in : "sharded";
-  if (num_kv_heads == 1 && !is(mode, "sharded") && !is(mode, "all_write") &&
+  // csrc/layerwise.cpp:1112-1121, 1349-1360: only these three names are
+  // meaningful for a restore; anything else is treated as "sharded".
+  const char *mode = c.kv_shared_across_ranks_mode ? c.kv_shared_across_ranks_mode : "sharded";
+  if (c.num_kv_heads == 1 && !is(mode, "sharded") && !is(mode, "all_write") &&
       !is(mode, "rank0_only")) {
     fprintf(stderr,
             "[fkv] warning: kv_shared_across_ranks_mode \"%s\" is not valid for layerwise "
@@ -238,96 +487,173 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
     mode = "sharded";
   }
 
+  // ---- lanes: [0, groups) main KV, [groups, groups + swa_groups) sidecar ----
+  const int num_main = (int)g->groups.size();
+  std::vector<Lane> lanes(num_main + (swa_active ? g->swa_groups.size() : 0));
+  // host offset of a rank, csrc/layerwise.cpp:1143-1166, 1519-1526, 448-453
+  auto rank_offsets = [&](int num_kv_heads, int64_t tp_stride, int64_t block_stride,
+                          int num_blocks) {
+    std::vector<int64_t> off(g->num_gpus);
+    for (int i = 0; i < g->num_gpus; ++i) {
+      off[i] = (int64_t)i * tp_stride;
+      if (num_kv_heads == 1)
+        off[i] = is(mode, "all_write") ? (int64_t)i * num_blocks * block_stride : 0;
+    }
+    return off;
+  };
+  for (int gi = 0; gi < num_main; ++gi) {
+    const Source &s = g->groups[gi];
+    Lane &l = lanes[gi];
+    l.src = &s;
+    l.gpu_ids = c.gpu_block_ids;
+    l.cpu_ids = c.cpu_block_ids;
+    l.num_blocks = c.num_blocks;
+    l.kv_dim = c.kv_dim;
+    if (g->multi_group) {
+      l.cpu_ptr = static_cast<char *>(g->cpu_blocks) + s.cpu_offset_bytes;
+      l.cpu_kv_stride = s.h2d_cpu_kv_stride;
+      l.cpu_layer_stride = s.h2d_cpu_layer_stride;
+      l.cpu_block_stride = s.cpu_block_stride;
+      l.cpu_off = rank_offsets(c.num_kv_heads, s.cpu_tp_stride, s.cpu_block_stride, c.num_blocks);
+    } else {
+      l.cpu_ptr = g->cpu_blocks;
+      l.cpu_kv_stride = c.h2d_cpu_kv_stride;
+      l.cpu_layer_stride = c.h2d_cpu_layer_stride;
+      l.cpu_block_stride = c.cpu_block_stride;
+      l.cpu_off = rank_offsets(c.num_kv_heads, c.cpu_tp_stride, c.cpu_block_stride, c.num_blocks);
+    }
+  }
+  if (swa_active)
+    for (int si = 0; si < (int)g->swa_groups.size(); ++si) {
+      const Source &s = g->swa_groups[si];
+      Lane &l = lanes[num_main + si];
+      l.src = &s;
+      l.gpu_ids = c.swa_gpu_block_ids;
+      l.cpu_ids = c.swa_cpu_block_ids;
+      l.num_blocks = c.swa_num_blocks;
+      l.kv_dim = 1; // csrc/layerwise.cpp:231, 1599
+      if (g->swa_multi_group) {
+        l.cpu_ptr = static_cast<char *>(g->swa_cpu_blocks) + s.cpu_offset_bytes;
+        l.cpu_kv_stride = s.h2d_cpu_kv_stride;
+        l.cpu_layer_stride = s.h2d_cpu_layer_stride;
+        l.cpu_block_stride = s.cpu_block_stride;
+        l.cpu_off = rank_offsets(1, s.cpu_tp_stride, s.cpu_block_stride, c.swa_num_blocks);
+      } else {
+        l.cpu_ptr = g->swa_cpu_blocks;
+        l.cpu_kv_stride = c.swa_h2d_cpu_kv_stride;
+        l.cpu_layer_stride = c.swa_h2d_cpu_layer_stride;
+        l.cpu_block_stride = c.swa_cpu_block_stride;
+        l.cpu_off.assign(g->num_gpus, 0); // :229
+      }
+    }
+
+  // ---- batches ----
   DeviceGuard restore(-1);
-  const int num_batches = (num_layers + layer_granularity - 1) / layer_granularity;
-  for (int b = 0; b < num_batches; ++b) {
+  g->layer_batch.assign(g->num_layers, -1);
+  auto new_batch = [&](int start_layer, int layers) -> fkv_layerwise::Batch & {
     auto batch = std::make_unique<fkv_layerwise::Batch>();
-    batch->start_layer = b * layer_granularity;
-    batch->layers = std::min(layer_granularity, num_layers - batch->start_layer);
-    batch->owner = g;
+    batch->start_layer = start_layer;
+    batch->layers = layers;
     batch->done.assign(g->num_gpus, nullptr);
+    for (int l = start_layer; l < start_layer + layers; ++l)
+      g->layer_batch[l] = (int)g->batches.size();
+    g->batches.push_back(std::move(batch));
+    return *g->batches.back();
+  };
+  auto add_item = [&](fkv_layerwise::Batch &b, int lane, int start, int layers) {
+    if (lanes[lane].num_blocks == 0 || layers == 0)
+      return;
+    lanes[lane].used = true;
+    b.items.push_back(Item{lane, start, layers});
+  };
+  if (!g->multi_group) {
+    for (int start = 0; start < c.num_layers; start += c.layer_granularity) {
+      const int n = std::min(c.layer_granularity, c.num_layers - start);
+      fkv_layerwise::Batch &b = new_batch(start, n);
+      add_item(b, 0, start, n);
+      // csrc/layerwise.cpp:1202-1209; the uniform form only (:219-221)
+      if (swa_active && !g->swa_multi_group)
+        add_item(b, num_main, start, n);
+      for (int i = 0; i < g->num_gpus; ++i)
+        b.trace_bytes += (double)g->groups[0].chunk_sizes[i] * c.kv_dim * n * c.num_blocks;
+    }
+  } else {
+    for (int orig = 0; orig < g->num_layers; ++orig) {
+      const int swa_slots = // swa_slots_for_orig_, csrc/layerwise.cpp:431-440
+          !swa_active ? 0 : g->swa_multi_group ? (int)g->swa_members[orig].size() : 1;
+      if (g->members[orig].empty() && swa_slots == 0) {
+        g->notify_layers(orig, 1); // nothing will ever land: announce now (:1437-1457)
+        continue;
+      }
+      fkv_layerwise::Batch &b = new_batch(orig, 1);
+      b.num_members = (int)g->members[orig].size();
+      for (const fkv_layer_member &m : g->members[orig]) {
+        add_item(b, m.group, m.local_layer, 1);
+        for (int i = 0; i < g->num_gpus; ++i)
+          b.trace_bytes += (double)g->groups[m.group].chunk_sizes[i] * c.kv_dim * c.num_blocks;
+      }
+      if (swa_active) {
+        if (g->swa_multi_group)
+          for (const fkv_layer_member &m : g->swa_members[orig])
+            add_item(b, num_main + m.group, m.local_layer, 1);
+        else
+          add_item(b, num_main, orig, 1);
+      }
+    }
+  }
+  const int num_batches = (int)g->batches.size();
+  for (auto &b : g->batches)
     for (int i = 0; i < g->num_gpus; ++i) {
       FKV_HIP_TRY(hipSetDevice(g->device_ids[i]));
-      FKV_HIP_TRY(hipEventCreate(&batch->done[i]));
+      FKV_HIP_TRY(hipEventCreate(&b->done[i]));
     }
-    g->batches.push_back(std::move(batch));
-  }
   FKV_HIP_TRY(hipSetDevice(g->device_ids[0]));
   FKV_HIP_TRY(hipEventCreate(&g->started));
   FKV_HIP_TRY(hipEventRecord(g->started, g->streams[0]));
 
-  // descriptor of rank i for layers [start, start + layers)
-  auto describe = [&](int i, int start, int layers) {
-    // host offset of rank i, csrc/layerwise.cpp:1143-1166
-    int64_t cpu_off = (int64_t)i * cpu_tp_stride;
-    if (num_kv_heads == 1)
-      cpu_off = is(mode, "all_write") ? (int64_t)i * num_blocks * cpu_block_stride : 0;
-    fkv_transfer_desc d{};
-    d.backend = g->backend;
-    d.num_layers_total = g->num_layers;
-    d.gpu_tensor_ptrs = g->gpu_ptrs.data() + (size_t)i * g->num_tensors_per_gpu;
-    d.num_gpu_tensor_ptrs = g->num_tensors_per_gpu;
-    d.device = g->device_ids[i];
-    d.gpu_kv_stride = g->kv_strides[i];
-    d.gpu_block_stride = g->block_strides[i];
-    d.gpu_layer_stride = g->layer_strides[i];
-    d.gpu_startoff_inside_chunks = 0;
-    d.cpu_ptr = g->cpu_blocks;
-    d.cpu_kv_stride = h2d_cpu_kv_stride;
-    d.cpu_layer_stride = h2d_cpu_layer_stride;
-    d.cpu_block_stride = cpu_block_stride;
-    d.cpu_startoff_inside_chunks = cpu_off;
-    d.chunk_size = g->chunk_sizes[i];
-    d.start_layer_id = start;
-    d.num_layers = layers;
-    d.kv_dim = kv_dim;
-    d.num_blocks = num_blocks;
-    d.gpu_block_ids = gpu_block_ids;
-    d.cpu_block_ids = cpu_block_ids;
-    d.is_host_to_device = 1;
-    d.use_ce_transfer = use_ce_transfer;
-    d.transfer_num_cta = transfer_cta_num;
-    d.sync = 0;
-    d.ce = g->ce;
-    return d;
-  };
-
   int rc = FKV_OK;
-  // Kernel path: the id lists and the base tables of all layers go to the device
-  // once per GPU; every batch is then a single kernel launch.
-  const bool direct = !use_ce_transfer && num_blocks > 0 && num_layers > 0;
-  std::vector<KernelPlan> plans(direct ? g->num_gpus : 0);
-  if (direct) {
-    for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
-      fkv_transfer_desc d = describe(i, 0, num_layers);
-      if (!d.gpu_tensor_ptrs || !d.cpu_ptr || !gpu_block_ids || !cpu_block_ids ||
-          d.chunk_size <= 0 || kv_dim < 1) {
-        rc = fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_transfer: bad pointers or sizes");
-        break;
+  // Kernel path: one plan per used lane and GPU, covering all layers of its group.
+  const bool direct = !c.use_ce_transfer;
+  if (direct)
+    for (Lane &lane : lanes) {
+      if (!lane.used || rc != FKV_OK)
+        continue;
+      lane.plans.resize(g->num_gpus);
+      const int layers = g->multi_group || lane.src != &g->groups[0] ? lane.src->num_layers
+                                                                     : c.num_layers;
+      for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
+        fkv_transfer_desc d = describe(g, lane, i, 0, layers, c);
+        rc = validate(d);
+        if (rc != FKV_OK)
+          break;
+        (void)hipSetDevice(g->device_ids[i]);
+        rc = kernel_plan_build(d, g->streams[i], &lane.plans[i]);
       }
-      (void)hipSetDevice(g->device_ids[i]);
-      rc = kernel_plan_build(d, g->streams[i], &plans[i]);
     }
-  }
   for (int b = 0; b < num_batches && rc == FKV_OK; ++b) {
     fkv_layerwise::Batch &batch = *g->batches[b];
     for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
       (void)hipSetDevice(g->device_ids[i]);
-      if (direct) {
-        rc = kernel_plan_launch(plans[i], batch.start_layer, batch.layers, g->streams[i]);
-        if (rc == FKV_OK) {
-          stats().calls.fetch_add(1, std::memory_order_relaxed);
-          stats().bytes_h2d.fetch_add((uint64_t)num_blocks * batch.layers * kv_dim *
-                                          (uint64_t)g->chunk_sizes[i],
-                                      std::memory_order_relaxed);
+      for (const Item &it : batch.items) {
+        const Lane &lane = lanes[it.lane];
+        if (direct) {
+          rc = kernel_plan_launch(lane.plans[i], it.start_layer, it.layers, g->streams[i]);
+          if (rc == FKV_OK) {
+            stats().calls.fetch_add(1, std::memory_order_relaxed);
+            stats().bytes_h2d.fetch_add((uint64_t)lane.num_blocks * it.layers * lane.kv_dim *
+                                            (uint64_t)lane.src->chunk_sizes[i],
+                                        std::memory_order_relaxed);
+          }
+        } else {
+          fkv_transfer_desc d = describe(g, lane, i, it.start_layer, it.layers, c);
+          rc = fkv_transfer_kv_blocks(&d, g->streams[i]);
+          (void)hipSetDevice(g->device_ids[i]);
         }
-      } else {
-        fkv_transfer_desc d = describe(i, batch.start_layer, batch.layers);
-        rc = fkv_transfer_kv_blocks(&d, g->streams[i]);
+        if (rc != FKV_OK)
+          break;
       }
       if (rc != FKV_OK)
         break;
-      (void)hipSetDevice(g->device_ids[i]);
       hipError_t e = hipEventRecord(batch.done[i], g->streams[i]);
       if (e != hipSuccess) {
         (void)hipGetLastError();
@@ -337,22 +663,24 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
     }
   }
   std::string saved_error = fkv_last_error();
-  for (int i = 0; i < (int)plans.size(); ++i) {
-    (void)hipSetDevice(g->device_ids[i]);
-    kernel_plan_release(&plans[i], g->streams[i]);
-  }
+  for (Lane &lane : lanes)
+    for (int i = 0; i < (int)lane.plans.size(); ++i) {
+      (void)hipSetDevice(g->device_ids[i]);
+      kernel_plan_release(&lane.plans[i], g->streams[i]);
+    }
   if (rc != FKV_OK) {
-    // Drain what was enqueued so no callback outlives this call's batches.
+    // Drain what was enqueued; nothing of this call is announced.
     for (int i = 0; i < g->num_gpus; ++i) {
       (void)hipSetDevice(g->device_ids[i]);
       (void)hipStreamSynchronize(g->streams[i]);
     }
+    g->layer_batch.assign(g->num_layers, -1);
     (void)hipSetDevice(restore.device());
     (void)hipGetLastError();
     return fail(rc, "%s", saved_error.c_str());
   }
 
-  if (notify_mode == FKV_NOTIFY_POLLING) {
+  if (c.notify_mode == FKV_NOTIFY_POLLING) {
     g->poller_stop.store(false, std::memory_order_release);
     // Nobody listens when no eventfd table was given: in-process consumers wait
     // on the batch events directly, so there is nothing to poll for.
@@ -373,18 +701,19 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
       }
       g->notify(*g->batches[b]);
     }
-    for (int i = 0; i < g->num_gpus; ++i) { // csrc/layerwise.cpp:1249-1256
+    for (int i = 0; i < g->num_gpus; ++i) { // csrc/layerwise.cpp:1249-1256, 1634-1642
       (void)hipSetDevice(g->device_ids[i]);
       hipError_t e = hipStreamSynchronize(g->streams[i]);
       if (e != hipSuccess) {
         (void)hipGetLastError();
         (void)hipSetDevice(restore.device());
-        return fail(FKV_ERR_RUNTIME, "layerwise_transfer failed on GPU %d: %s", i,
+        return fail(FKV_ERR_RUNTIME, "%s failed on GPU %d: %s",
+                    g->multi_group ? "layerwise_transfer_multi_group" : "layerwise_transfer", i,
                     hipGetErrorString(e));
       }
     }
-    if (enable_trace && num_batches > 0) {
-      // per-batch line with the fields of csrc/layerwise.cpp:1281-1285
+    if (c.enable_trace && num_batches > 0) {
+      // per-batch line with the fields of csrc/layerwise.cpp:1281-1285, 1655-1661
       (void)hipSetDevice(g->device_ids[0]);
       float prev = 0;
       for (int b = 0; b < num_batches; ++b) {
@@ -394,16 +723,19 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
           continue;
         }
         const fkv_layerwise::Batch &bt = *g->batches[b];
-        double bytes = 0;
-        for (int i = 0; i < g->num_gpus; ++i)
-          bytes += (double)g->chunk_sizes[i] * kv_dim * bt.layers * num_blocks;
-        const double mb = bytes / (1024.0 * 1024.0);
+        const double mb = bt.trace_bytes / (1024.0 * 1024.0);
         const double dt = ms - prev;
-        fprintf(stderr,
-                "[XFER] type=layerwise_h2d layer_range=[%d,%d) blocks=%d data=%.2fMB "
-                "sync_ms=%.3f bw=%.0fMB/s\n",
-                bt.start_layer, bt.start_layer + bt.layers, num_blocks, mb, dt,
-                dt > 0 ? mb / (dt / 1000.0) : 0.0);
+        const double bw = dt > 0 ? mb / (dt / 1000.0) : 0.0;
+        if (g->multi_group)
+          fprintf(stderr,
+                  "[XFER] type=layerwise_mg_h2d orig=%d members=%d gpus=%d sync_ms=%.3f "
+                  "data=%.2fMB bw=%.0fMB/s\n",
+                  bt.start_layer, bt.num_members, g->num_gpus, dt, mb, bw);
+        else
+          fprintf(stderr,
+                  "[XFER] type=layerwise_h2d layer_range=[%d,%d) blocks=%d data=%.2fMB "
+                  "sync_ms=%.3f bw=%.0fMB/s\n",
+                  bt.start_layer, bt.start_layer + bt.layers, c.num_blocks, mb, dt, bw);
         prev = ms;
       }
     }
@@ -412,15 +744,51 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
   return FKV_OK;
 }
 
+int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
+                           const int64_t *cpu_block_ids, int32_t num_blocks,
+                           int64_t cpu_block_stride, int64_t h2d_cpu_kv_stride,
+                           int64_t h2d_cpu_layer_stride, int64_t cpu_tp_stride,
+                           int32_t transfer_cta_num, int32_t use_ce_transfer,
+                           int32_t num_layers, int32_t layer_granularity, int32_t kv_dim,
+                           int32_t num_kv_heads, int32_t counter_id, const char *mode,
+                           int32_t notify_mode, int32_t enable_trace) {
+  fkv_layerwise_call c{};
+  c.gpu_block_ids = gpu_block_ids;
+  c.cpu_block_ids = cpu_block_ids;
+  c.num_blocks = num_blocks;
+  c.multi_group = 0;
+  c.cpu_block_stride = cpu_block_stride;
+  c.h2d_cpu_kv_stride = h2d_cpu_kv_stride;
+  c.h2d_cpu_layer_stride = h2d_cpu_layer_stride;
+  c.cpu_tp_stride = cpu_tp_stride;
+  c.num_layers = num_layers;
+  c.layer_granularity = layer_granularity;
+  c.transfer_cta_num = transfer_cta_num;
+  c.use_ce_transfer = use_ce_transfer;
+  c.kv_dim = kv_dim;
+  c.num_kv_heads = num_kv_heads;
+  c.counter_id = counter_id;
+  c.notify_mode = notify_mode;
+  c.enable_trace = enable_trace;
+  c.kv_shared_across_ranks_mode = mode;
+  return fkv_layerwise_transfer_call(g, &c);
+}
+
 int fkv_layerwise_wait_layer(fkv_layerwise *g, int32_t gpu_index, int32_t layer,
                              void *consumer_stream) {
   using namespace fkv;
   clear_error();
   if (!g || gpu_index < 0 || gpu_index >= g->num_gpus)
     return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_wait_layer: bad group or GPU index");
-  const int b = layer / g->granularity;
-  if (layer < 0 || b >= (int)g->batches.size())
+  if (layer < 0 || layer >= (int)g->layer_batch.size())
     return fail(FKV_ERR_INVALID_ARG, "layer %d was not part of the last transfer", layer);
+  const int b = g->layer_batch[layer];
+  if (b < 0) {
+    // An original layer without members or sidecar work: nothing is in flight.
+    if (g->multi_group)
+      return FKV_OK;
+    return fail(FKV_ERR_INVALID_ARG, "layer %d was not part of the last transfer", layer);
+  }
   FKV_HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(consumer_stream),
                                  g->batches[b]->done[gpu_index], 0));
   return FKV_OK;

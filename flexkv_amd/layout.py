@@ -9,12 +9,20 @@ GPU addressing mode from the number of engine tensors (``worker.py:804-814``,
 
 All getters return ELEMENT counts like the reference; multiply by
 ``dtype.itemsize`` for bytes (``TransferStrides`` does that).
+
+Models whose layers do not share one KV shape (a latent cache plus an indexer
+cache on the same layer, groups compressed along the token axis) are described
+by ``LayerGroupSpec`` / ``LayerMemberMap`` (``flexkv/common/config.py:33-119``)
+and stored in byte-flat host blocks, ``MultiGroupBlockLayout``
+(storage.py:87-127, 249-286); ``multi_group_tables`` produces the per-group
+arrays the layerwise restore is constructed with
+(``flexkv/transfer/layerwise.py:431-537``).
 """
 from __future__ import annotations
 
 import enum
 from dataclasses import dataclass, replace
-from typing import Optional, Sequence, Tuple
+from typing import Dict, List, Optional, Sequence, Tuple
 
 
 class KVCacheLayoutType(enum.Enum):
@@ -171,3 +179,145 @@ def gpu_block_type_from_tensor_count(num_tensors: int, num_layers: int) -> int:
     if num_tensors == 2 * num_layers:
         return GPU_BLOCK_TYPE_SGLANG
     raise ValueError(f"Invalid GPU block type: {num_tensors} tensors for {num_layers} layers")
+
+
+# ---- heterogeneous layer groups -------------------------------------------------
+
+@dataclass(frozen=True)
+class LayerGroupSpec:
+    """Layers that share one KV shape (config.py:33-65).
+
+    ``layer_indices[k]`` is the original layer the group's k-th layer belongs to;
+    several groups may name the same original layer.  ``itemsize`` is the byte
+    width of the group's storage dtype; ``compress_ratio`` divides
+    ``tokens_per_block`` for this group.
+    """
+    num_layers: int
+    num_kv_heads: int
+    head_size: int
+    layer_indices: Tuple[int, ...]
+    itemsize: int = 2
+    compress_ratio: int = 1
+
+    def __post_init__(self) -> None:
+        object.__setattr__(self, "layer_indices", tuple(self.layer_indices))
+        if self.num_layers != len(self.layer_indices):
+            raise ValueError("num_layers must equal len(layer_indices)")
+        if len(set(self.layer_indices)) != len(self.layer_indices):
+            raise ValueError("layer_indices must not repeat inside one group")
+
+
+@dataclass(frozen=True)
+class LayerMemberMap:
+    """``members[i]``: the (group, layer-inside-group) pairs of original layer i,
+    by ascending group (config.py:68-99)."""
+    members: Tuple[Tuple[Tuple[int, int], ...], ...]
+
+    @property
+    def num_original_layers(self) -> int:
+        return len(self.members)
+
+    def members_of(self, original_layer_id: int) -> Tuple[Tuple[int, int], ...]:
+        return self.members[original_layer_id]
+
+
+def build_layer_member_map(layer_groups: Sequence[LayerGroupSpec],
+                           num_original_layers: int) -> LayerMemberMap:
+    """config.py:102-119."""
+    buckets: List[List[Tuple[int, int]]] = [[] for _ in range(num_original_layers)]
+    for gi, g in enumerate(layer_groups):
+        for local_id, orig in enumerate(g.layer_indices):
+            if not 0 <= orig < num_original_layers:
+                raise ValueError(f"layer_groups[{gi}] names original layer {orig} outside "
+                                 f"[0, {num_original_layers})")
+            buckets[orig].append((gi, local_id))
+    return LayerMemberMap(tuple(tuple(sorted(b, key=lambda m: m[0])) for b in buckets))
+
+
+@dataclass(frozen=True)
+class MultiGroupBlockLayout:
+    """Byte-flat BLOCKFIRST host pool of a multi-group model: block b holds, group
+    after group, ``[layer-in-group, kv, token, head, dim]`` of every group, once
+    per tensor-parallel rank (storage.py:87-127)."""
+    num_block: int
+    tokens_per_block: int
+    layer_groups: Tuple[LayerGroupSpec, ...]
+    kv_dim: int = 1
+    tp_size: int = 1
+
+    def __post_init__(self) -> None:
+        object.__setattr__(self, "layer_groups", tuple(self.layer_groups))
+        for gi, g in enumerate(self.layer_groups):
+            if self.tokens_per_block % g.compress_ratio:
+                raise ValueError(
+                    f"layer_groups[{gi}].compress_ratio={g.compress_ratio} does not divide "
+                    f"tokens_per_block={self.tokens_per_block}")
+
+    def group_chunk_bytes(self, gi: int) -> int:
+        g = self.layer_groups[gi]
+        return (self.tokens_per_block // g.compress_ratio) * g.num_kv_heads * g.head_size \
+            * g.itemsize
+
+    def get_block_stride(self) -> int:
+        """Bytes per block (storage.py:120-127, 222-226)."""
+        return self.tp_size * sum(g.num_layers * self.kv_dim * self.group_chunk_bytes(gi)
+                                  for gi, g in enumerate(self.layer_groups))
+
+    @property
+    def kv_shape(self) -> Tuple[int, int]:
+        return (self.num_block, self.get_block_stride())
+
+    def get_group_strides(self) -> List[Dict[str, int]]:
+        """Per group, in bytes: offset inside a block, layer / kv strides and chunk
+        size (storage.py:249-286, there in elements of the group's dtype)."""
+        out, offset = [], 0
+        for gi, g in enumerate(self.layer_groups):
+            chunk = self.group_chunk_bytes(gi)
+            layer_stride = self.kv_dim * chunk
+            out.append({"num_layers": g.num_layers, "offset_bytes": offset,
+                        "layer_stride": layer_stride, "kv_stride": chunk, "chunk_size": chunk})
+            offset += g.num_layers * layer_stride
+        return out
+
+
+def multi_group_tables(cpu_layout: MultiGroupBlockLayout, num_original_layers: int,
+                       gpu_layouts_per_group: Sequence[Sequence[KVCacheLayout]],
+                       tp_group_size: int = 1) -> Dict[str, object]:
+    """The per-group arrays of the multi-group ``LayerwiseTransferGroup``
+    constructor and of ``init_swa_multi_group`` (layerwise.py:431-537).
+    ``gpu_layouts_per_group[gi][d]`` is the device layout of group gi on GPU d;
+    the per-GPU arrays are flattened group-major."""
+    member_map = build_layer_member_map(cpu_layout.layer_groups, num_original_layers)
+    block_stride = cpu_layout.get_block_stride()
+    tp_stride = block_stride // tp_group_size
+    t: Dict[str, list] = {k: [] for k in (
+        "group_num_layers", "group_cpu_offset_bytes", "group_ssd_offset_bytes",
+        "group_cpu_layer_strides", "group_cpu_kv_strides", "group_ssd_layer_strides",
+        "group_ssd_kv_strides", "group_chunk_sizes", "group_h2d_cpu_kv_strides",
+        "group_h2d_cpu_layer_strides", "group_cpu_block_strides", "group_cpu_tp_strides",
+        "group_gpu_kv_strides", "group_gpu_block_strides", "group_gpu_layer_strides",
+        "group_gpu_chunk_sizes")}
+    for gi, (g, st) in enumerate(zip(cpu_layout.layer_groups, cpu_layout.get_group_strides())):
+        t["group_num_layers"].append(g.num_layers)
+        t["group_cpu_offset_bytes"].append(st["offset_bytes"])
+        t["group_ssd_offset_bytes"].append(st["offset_bytes"])
+        for k in ("group_cpu_layer_strides", "group_ssd_layer_strides",
+                  "group_h2d_cpu_layer_strides"):
+            t[k].append(st["layer_stride"])
+        for k in ("group_cpu_kv_strides", "group_ssd_kv_strides", "group_h2d_cpu_kv_strides"):
+            t[k].append(st["kv_stride"])
+        t["group_chunk_sizes"].append(st["chunk_size"])
+        t["group_cpu_block_strides"].append(block_stride)
+        t["group_cpu_tp_strides"].append(tp_stride)
+        for layout in gpu_layouts_per_group[gi]:
+            s = TransferStrides.from_layout(layout, g.itemsize)
+            t["group_gpu_kv_strides"].append(s.kv)
+            t["group_gpu_block_strides"].append(s.block)
+            t["group_gpu_layer_strides"].append(s.layer)
+            t["group_gpu_chunk_sizes"].append(s.chunk)
+    out: Dict[str, object] = dict(t)
+    out["layer_members"] = [list(m) for m in member_map.members]
+    out["layer_member_map"] = member_map
+    out["cpu_block_stride"] = block_stride
+    out["cpu_tp_stride"] = tp_stride
+    return out

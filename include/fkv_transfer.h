@@ -228,8 +228,8 @@ int fkv_tp_group_transfer(fkv_tp_group *g, const int64_t *gpu_block_ids,
 /* dtor, csrc/tp_transfer_thread_group.cpp:164-185 */
 void fkv_tp_group_destroy(fkv_tp_group *g);
 
-/* ---- LayerwiseTransferGroup (single group, main KV):
- *      csrc/layerwise.h:59-362, csrc/bindings.cpp:471-545, 657-691 ---- */
+/* ---- LayerwiseTransferGroup: csrc/layerwise.h:59-362,
+ *      csrc/bindings.cpp:471-757 ---- */
 
 typedef struct fkv_layerwise fkv_layerwise;
 
@@ -254,16 +254,114 @@ typedef struct fkv_layerwise_params {
 #define FKV_NOTIFY_HOSTFUNC 0
 #define FKV_NOTIFY_POLLING 1
 
-/* ctor, csrc/layerwise.cpp:507-646 (SSD and SWA arguments are outside this
- * library; the Python shim rejects non-empty ones). */
+/* Single-group ctor, csrc/layerwise.cpp:507-646.  The SSD arguments are
+ * outside this library (the Python shim rejects non-empty ones); a uniform SWA
+ * sidecar is attached afterwards with fkv_layerwise_init_swa. */
 int fkv_layerwise_create(const fkv_layerwise_params *params, fkv_layerwise **out);
 
-/* csrc/layerwise.cpp:944-1311, host->GPU restore in batches of
- * `layer_granularity` layers.  HOSTFUNC returns after every stream has
- * drained (:1249-1256), the eventfds of a batch having been written as soon as
- * the batch landed; POLLING returns right after the launches (:1240-1247) and a
- * library thread writes the eventfds.
- * `mode` is kv_shared_across_ranks_mode (:1112-1166). */
+/* One layer group: layers that share a KV shape, with their own device
+ * tensors and their own byte range inside every host block -- GroupParams,
+ * csrc/layerwise.h (filled by fill_group_params_from_arrays,
+ * csrc/layerwise.cpp:264-353).  The backend follows from
+ * num_tensors_per_gpu vs num_layers (1 -> TRT-LLM, L -> vLLM, 2L -> SGLang). */
+typedef struct fkv_layer_group {
+  int32_t num_layers;
+  int32_t num_tensors_per_gpu;
+  const uint64_t *gpu_block_ptrs_flat; /* num_gpus * num_tensors_per_gpu */
+  int64_t cpu_offset_bytes;            /* of the group inside a host block */
+  int64_t h2d_cpu_kv_stride;
+  int64_t h2d_cpu_layer_stride;
+  int64_t cpu_block_stride;
+  int64_t cpu_tp_stride;
+  const int64_t *gpu_kv_strides; /* num_gpus entries each */
+  const int64_t *gpu_block_strides;
+  const int64_t *gpu_layer_strides;
+  const int64_t *gpu_chunk_sizes;
+} fkv_layer_group;
+
+/* (group, layer inside the group) attached to one original layer --
+ * LayerMemberMap, flexkv/common/config.py:68-119. */
+typedef struct fkv_layer_member {
+  int32_t group;
+  int32_t local_layer;
+} fkv_layer_member;
+
+typedef struct fkv_layerwise_mg_params {
+  int32_t num_gpus;
+  int32_t num_original_layers;
+  int32_t tp_size;
+  int32_t num_groups;
+  const fkv_layer_group *groups;
+  /* members of original layer i: members[member_offsets[i] .. member_offsets[i+1]) */
+  const int32_t *member_offsets; /* num_original_layers + 1 entries */
+  const fkv_layer_member *members;
+  void *cpu_blocks_ptr;
+  const int64_t *gpu_device_ids;
+  const int32_t *layer_eventfds; /* [num_counters, tp_size, num_original_layers] */
+  int32_t num_layer_eventfds;
+  int32_t reserved;
+  fkv_ce_config ce;
+} fkv_layerwise_mg_params;
+
+/* Multi-group ctor, csrc/layerwise.cpp:647-838. */
+int fkv_layerwise_create_multi_group(const fkv_layerwise_mg_params *params,
+                                     fkv_layerwise **out);
+
+/* Uniform SWA sidecar (one ring of sliding-window blocks per layer with its own
+ * host pool) -- init_swa_sidecar_, csrc/layerwise.cpp:139-207.  Of `swa` the
+ * device fields and num_layers are read; the host strides come with each call.
+ * Errors: "Unsupported SWA GPU block type: N". */
+int fkv_layerwise_init_swa(fkv_layerwise *g, const fkv_layer_group *swa,
+                           void *swa_cpu_blocks_ptr);
+/* SWA / state sidecar made of its own layer groups --
+ * init_swa_multi_group, csrc/layerwise.cpp:355-429. */
+int fkv_layerwise_init_swa_multi_group(fkv_layerwise *g, const fkv_layer_group *groups,
+                                       int32_t num_groups, const int32_t *member_offsets,
+                                       const fkv_layer_member *members,
+                                       void *swa_cpu_blocks_ptr);
+
+/* Arguments of one restore: layerwise_transfer (csrc/layerwise.cpp:944-1311)
+ * when multi_group == 0, layerwise_transfer_multi_group (:1313-1682) otherwise. */
+typedef struct fkv_layerwise_call {
+  const int64_t *gpu_block_ids; /* host arrays, num_blocks entries */
+  const int64_t *cpu_block_ids;
+  int32_t num_blocks;
+  int32_t multi_group;
+  /* single group only; a multi-group instance takes these from its groups */
+  int64_t cpu_block_stride;
+  int64_t h2d_cpu_kv_stride;
+  int64_t h2d_cpu_layer_stride;
+  int64_t cpu_tp_stride;
+  int32_t num_layers;
+  int32_t layer_granularity;
+  int32_t transfer_cta_num;
+  int32_t use_ce_transfer;
+  int32_t kv_dim;
+  int32_t num_kv_heads;
+  int32_t counter_id;
+  int32_t notify_mode;
+  int32_t enable_trace;
+  int32_t swa_num_blocks; /* 0 = no sidecar work in this call */
+  const char *kv_shared_across_ranks_mode;
+  /* sidecar: swa_h2d_dst (device block ids) / swa_h2d_src (host block ids) */
+  const int64_t *swa_gpu_block_ids;
+  const int64_t *swa_cpu_block_ids;
+  /* uniform sidecar only */
+  int64_t swa_h2d_cpu_kv_stride;
+  int64_t swa_h2d_cpu_layer_stride;
+  int64_t swa_cpu_block_stride;
+} fkv_layerwise_call;
+
+/* Host->GPU restore, one completion per layer batch (single group: batches of
+ * `layer_granularity` layers; multi-group: one batch per original layer that
+ * has members or sidecar work, original layers with neither get their eventfd
+ * written on entry, csrc/layerwise.cpp:1437-1457).  HOSTFUNC returns after
+ * every stream has drained (:1249-1256, 1634-1642), the eventfds of a batch
+ * having been written as soon as the batch landed; POLLING returns right after
+ * the launches and a library thread writes the eventfds. */
+int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call);
+
+/* layerwise_transfer without sidecar work, positional form of the above. */
 int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
                            const int64_t *cpu_block_ids, int32_t num_blocks,
                            int64_t cpu_block_stride, int64_t h2d_cpu_kv_stride,
@@ -275,10 +373,10 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
                            int32_t enable_trace);
 
 /* Make `consumer_stream` (a hipStream_t on GPU `gpu_index` of the group) wait
- * until `layer` of the most recent fkv_layerwise_transfer has landed.  This is
- * the in-process counterpart of the eventfd a consumer in another process
- * blocks on (flexkv/integration/sglang/comm.py:705-744); the reference has no
- * such call. */
+ * until `layer` (an original layer id for a multi-group instance) of the most
+ * recent transfer has landed.  This is the in-process counterpart of the
+ * eventfd a consumer in another process blocks on
+ * (flexkv/integration/sglang/comm.py:705-744); the reference has no such call. */
 int fkv_layerwise_wait_layer(fkv_layerwise *g, int32_t gpu_index, int32_t layer,
                              void *consumer_stream);
 /* Block the host until the most recent transfer has finished on all GPUs and

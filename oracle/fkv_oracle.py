@@ -242,3 +242,102 @@ def torch_index_scatter(layers, host_cache, gpu_ids, cpu_ids) -> None:
     for l, layer in enumerate(layers):
         picked = torch.index_select(host_cache[:, l], 0, cpu_ids)  # [n, kv, T, H, D]
         layer.index_copy_(1, gpu_ids, picked.transpose(0, 1))
+
+
+# ---- layerwise restore of heterogeneous layer groups ---------------------------
+
+class GroupRef:
+    """Host-memory stand-in of one layer group: ``tensors[d]`` are the numpy byte
+    buffers that play the group's device tensors on GPU d (GroupParams,
+    csrc/layerwise.h)."""
+
+    def __init__(self, num_layers: int, tensors: List[List[np.ndarray]], gpu_kv_strides,
+                 gpu_block_strides, gpu_layer_strides, gpu_chunk_sizes, cpu_offset_bytes=0,
+                 h2d_cpu_kv_stride=0, h2d_cpu_layer_stride=0, cpu_block_stride=0,
+                 cpu_tp_stride=0) -> None:
+        self.num_layers = num_layers
+        self.tensors = tensors
+        n = len(tensors[0])
+        # csrc/layerwise.cpp:792-806
+        self.backend = (BACKEND_TRTLLM if n == 1 else BACKEND_VLLM if n == num_layers
+                        else BACKEND_SGLANG if n == 2 * num_layers else None)
+        if self.backend is None:
+            raise RuntimeError(f"unsupported tensors_per_gpu={n} for num_layers={num_layers}")
+        self.gpu_kv_strides = list(gpu_kv_strides)
+        self.gpu_block_strides = list(gpu_block_strides)
+        self.gpu_layer_strides = list(gpu_layer_strides)
+        self.gpu_chunk_sizes = list(gpu_chunk_sizes)
+        self.cpu_offset_bytes = cpu_offset_bytes
+        self.h2d_cpu_kv_stride = h2d_cpu_kv_stride
+        self.h2d_cpu_layer_stride = h2d_cpu_layer_stride
+        self.cpu_block_stride = cpu_block_stride
+        self.cpu_tp_stride = cpu_tp_stride
+
+
+def _group_layer_h2d(g: GroupRef, d: int, host: np.ndarray, local_layer: int, num_layers: int,
+                     gpu_ids, cpu_ids, kv_dim: int, cpu_kv_stride: int, cpu_layer_stride: int,
+                     cpu_block_stride: int, cpu_off: int) -> None:
+    transfer_c(g.backend, [t.ctypes.data for t in g.tensors[d]], g.num_layers,
+               g.gpu_kv_strides[d], g.gpu_block_strides[d], g.gpu_layer_strides[d], 0,
+               host.ctypes.data + g.cpu_offset_bytes, cpu_kv_stride, cpu_layer_stride,
+               cpu_block_stride, cpu_off, g.gpu_chunk_sizes[d], local_layer, num_layers, kv_dim,
+               gpu_ids, cpu_ids, True)
+
+
+def _rank_off(d: int, num_kv_heads: int, mode: str, num_blocks: int, tp_stride: int,
+              block_stride: int) -> int:
+    # csrc/layerwise.cpp:1519-1526 (same rule at :448-453 and :1143-1166)
+    if num_kv_heads == 1:
+        return d * num_blocks * block_stride if mode == "all_write" else 0
+    return d * tp_stride
+
+
+def layerwise_multi_group(num_gpus: int, groups: List[GroupRef], layer_members, host: np.ndarray,
+                          gpu_ids, cpu_ids, kv_dim: int, num_kv_heads: int,
+                          mode: str = "sharded", swa: Optional[dict] = None):
+    """layerwise_transfer_multi_group, csrc/layerwise.cpp:1313-1682, on host
+    memory.  ``swa`` is None, ``{"kind": "uniform", "group", "host", "gpu_ids",
+    "cpu_ids", "kv_stride", "layer_stride", "block_stride"}`` (launch_swa_h2d_layer_,
+    :209-258) or ``{"kind": "multi", "groups", "members", "host", "gpu_ids",
+    "cpu_ids"}`` (launch_swa_mg_h2d_layer_, :442-503).
+
+    Returns ``(immediate, work)``: the original layers announced on entry because
+    nothing is attached to them, and those announced once after their copies, in
+    order."""
+    if num_kv_heads == 1 and mode not in ("sharded", "all_write", "rank0_only"):
+        mode = "sharded"  # :1349-1360
+    swa_active = swa is not None and len(swa["cpu_ids"]) > 0
+    immediate, work = [], []
+    for orig, members in enumerate(layer_members):
+        slots = 0
+        if swa_active:
+            slots = len(swa["members"][orig]) if swa["kind"] == "multi" else 1
+        if not members and slots == 0:
+            immediate.append(orig)  # :1437-1457
+            continue
+        work.append(orig)
+        for gi, local in members:
+            g = groups[gi]
+            for d in range(num_gpus):
+                off = _rank_off(d, num_kv_heads, mode, len(gpu_ids), g.cpu_tp_stride,
+                                g.cpu_block_stride)
+                _group_layer_h2d(g, d, host, local, 1, gpu_ids, cpu_ids, kv_dim,
+                                 g.h2d_cpu_kv_stride, g.h2d_cpu_layer_stride,
+                                 g.cpu_block_stride, off)
+        if not swa_active:
+            continue
+        if swa["kind"] == "multi":
+            for gi, local in swa["members"][orig]:
+                g = swa["groups"][gi]
+                for d in range(num_gpus):
+                    off = _rank_off(d, 1, mode, len(swa["gpu_ids"]), g.cpu_tp_stride,
+                                    g.cpu_block_stride)
+                    _group_layer_h2d(g, d, swa["host"], local, 1, swa["gpu_ids"],
+                                     swa["cpu_ids"], 1, g.h2d_cpu_kv_stride,
+                                     g.h2d_cpu_layer_stride, g.cpu_block_stride, off)
+        else:
+            g = swa["group"]
+            for d in range(num_gpus):
+                _group_layer_h2d(g, d, swa["host"], orig, 1, swa["gpu_ids"], swa["cpu_ids"], 1,
+                                 swa["kv_stride"], swa["layer_stride"], swa["block_stride"], 0)
+    return immediate, work

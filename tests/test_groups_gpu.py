@@ -429,7 +429,7 @@ def test_layerwise_rejects_what_it_does_not_provide(gpu_device):
     gl, cl = make_layouts(L, N, T, H, D, "BLOCKFIRST", 1, 1)
     gpu = make_gpu_tensors(L, N, T, H, D, 1, gpu_device)
     cpu = torch.zeros(cl.kv_shape, dtype=DTYPE, pin_memory=True)
-    with pytest.raises(RuntimeError, match="multi-group"):
+    with pytest.raises(TypeError, match="missing arguments"):
         LayerwiseTransferGroup(num_gpus=1, gpu_blocks_per_group=[[gpu]], cpu_blocks=cpu)
     st = torch.tensor([8], dtype=torch.int64)
     with pytest.raises(RuntimeError, match="SSD"):
@@ -439,6 +439,10 @@ def test_layerwise_rejects_what_it_does_not_provide(gpu_device):
         LayerwiseTransferGroup(1, [gpu + [gpu[0]]], cpu, {}, L, st, st, st, st, 0, 0,
                                torch.empty(0, dtype=torch.int32), 1)
     lw = layerwise_group(cpu, [gpu], gl, L)
+    ids = torch.tensor([1], dtype=torch.int64)
+    none = torch.empty(0, dtype=torch.int64)
     with pytest.raises(RuntimeError, match="single-group instance"):
-        lw.layerwise_transfer_multi_group()
+        lw.layerwise_transfer_multi_group(none, none, 0, 1, 4, ids, ids, 4, False, 1, 1)
+    with pytest.raises(RuntimeError, match="SSD"):
+        lw.layerwise_transfer_multi_group(ids, none, 0, 1, 4, ids, ids, 4, False, 1, 1)
     lw.close()
