@@ -16,6 +16,10 @@ Configurations (BASELINE.json "configs"):
   c2  TRT-LLM layout, fp8 e4m3: [4096,80,2,8,32,128]; 2048 random blocks
   c3  DeepSeek-V3 MLA, bf16: 61 x [16384,64,576]; layerwise restore of 512 blocks
   c4  64 concurrent requests on the c0 shape with a 32768-block pool
+Beyond BASELINE.json (the rows next to the path):
+  mg      layerwise restore of heterogeneous layer groups + sliding-window sidecar
+          (DeepSeek-V4-like: 61 layers, two compressed latent groups, an indexer group)
+  worker  c0-shaped put/get ops through a transfer worker process (pipe + shared op pool)
 """
 from __future__ import annotations
 
@@ -453,6 +457,163 @@ def run_notify_scales(torch, device, num_cta, iters=20, warmup=3):
 # CPU baseline: the reference's CPU path (torch index-gather into the host
 # cache layout), timed on this machine's host cores on a bounded sample.
 # ---------------------------------------------------------------------------
+def run_multi_group(torch, device, steps, warmup, num_cta, notify, use_ce, verify=True):
+    """Layer groups of different shape restored layer by layer, one notification per
+    original layer: members of every group attached to the layer, then its sidecar."""
+    from flexkv_amd.c_ext import LayerwiseTransferGroup
+    from flexkv_amd.layout import (KVCacheLayout, KVCacheLayoutType, LayerGroupSpec,
+                                   MultiGroupBlockLayout, TransferStrides, multi_group_tables)
+    t = torch
+    L, page, n_gpu, n_cpu, nblk = 61, 256, 2048, 512, 512
+    swa_tok, swa_width, swa_gpu, swa_cpu, nswa = 128, 1152, 256, 64, 64
+    c4_layers = tuple(l for l in range(L) if l % 2 == 1)            # 30 layers, ratio 4
+    c128_layers = tuple(l for l in range(L) if l % 2 == 0)          # 31 layers, ratio 128
+    groups = [LayerGroupSpec(len(c4_layers), 1, 576, c4_layers, 2, 4),
+              LayerGroupSpec(len(c128_layers), 1, 576, c128_layers, 2, 128),
+              LayerGroupSpec(len(c4_layers), 1, 128, c4_layers, 1, 4)]  # indexer, one byte/elem
+    cl = MultiGroupBlockLayout(n_cpu, page, tuple(groups), kv_dim=1)
+    gls = [KVCacheLayout(KVCacheLayoutType.LAYERFIRST, g.num_layers, n_gpu,
+                         page // g.compress_ratio, 1, g.head_size, kv_dim=1) for g in groups]
+    tables = multi_group_tables(cl, L, [[x] for x in gls])
+    gen = t.Generator(device=device).manual_seed(6)
+    gpu = [[t.randint(0, 256, (n_gpu, page // g.compress_ratio, 1, g.head_size * g.itemsize),
+                      device=device, dtype=t.uint8, generator=gen) for _ in range(g.num_layers)]
+           for g in groups]
+    host = t.randint(0, 256, (n_cpu, cl.get_block_stride()), dtype=t.uint8).pin_memory()
+    scl = KVCacheLayout(KVCacheLayoutType.LAYERFIRST, L, swa_cpu, swa_tok, 1, swa_width, kv_dim=1)
+    sgl = KVCacheLayout(KVCacheLayoutType.LAYERFIRST, L, swa_gpu, swa_tok, 1, swa_width, kv_dim=1)
+    sc, sg = TransferStrides.from_layout(scl, 1), TransferStrides.from_layout(sgl, 1)
+    swa_host = t.randint(0, 256, scl.kv_shape, dtype=t.uint8).pin_memory()
+    swa_dev = [t.zeros((swa_gpu, swa_tok, 1, swa_width), device=device, dtype=t.uint8)
+               for _ in range(L)]
+    i64 = lambda v: t.tensor([v], dtype=t.int64)
+    grp = LayerwiseTransferGroup(
+        num_gpus=1, gpu_blocks_per_group=[[x] for x in gpu], cpu_blocks=host, ssd_files={},
+        num_original_layers=L, layer_members=tables["layer_members"], iouring_entries=0,
+        iouring_flags=0, layer_eventfds_tensor=t.empty(0, dtype=t.int32), tp_size=1,
+        is_blockfirst=True, has_swa=True, swa_gpu_blocks=[swa_dev], swa_cpu_blocks=swa_host,
+        swa_gpu_kv_strides_tensor=i64(sg.kv), swa_gpu_block_strides_tensor=i64(sg.block),
+        swa_gpu_layer_strides_tensor=i64(sg.layer), swa_gpu_chunk_sizes_tensor=i64(sg.chunk),
+        **{k: v for k, v in tables.items() if k.startswith("group_")})
+    gg = t.Generator().manual_seed(6)
+    gpu_ids = t.randperm(n_gpu, generator=gg)[:nblk].to(t.int64)
+    cpu_ids = t.randperm(n_cpu, generator=gg)[:nblk].to(t.int64)
+    swa_g = t.randperm(swa_gpu, generator=gg)[:nswa].to(t.int64)
+    swa_c = t.randperm(swa_cpu, generator=gg)[:nswa].to(t.int64)
+    empty = t.empty(0, dtype=t.int64)
+
+    def restore():
+        grp.layerwise_transfer_multi_group(
+            empty, empty, 0, 1, 4, gpu_ids, cpu_ids, num_cta, use_ce, 1, 1, swa_h2d_src=swa_c,
+            swa_h2d_dst=swa_g, swa_h2d_cpu_kv_stride_in_bytes=sc.kv,
+            swa_h2d_cpu_layer_stride_in_bytes=sc.layer, swa_cpu_block_stride_in_bytes=sc.block,
+            notify_mode=notify)
+        grp.synchronize()
+
+    for _ in range(warmup):
+        restore()
+    walls, last_layer = [], []
+    for _ in range(steps):
+        t.cuda.synchronize()
+        t0 = time.perf_counter()
+        restore()
+        walls.append(time.perf_counter() - t0)
+        last_layer.append(grp.batch_times_ms()[-1])
+    main_bytes = sum(tables["group_chunk_sizes"][gi] * g.num_layers for gi, g in enumerate(groups)) \
+        * nblk
+    swa_bytes = L * nswa * sc.chunk
+    ok = None
+    if verify:
+        ok = True
+        st = cl.get_group_strides()
+        gi_dev = gpu_ids.to(device)
+        for gi, g in enumerate(groups):
+            for l in range(g.num_layers):
+                o = st[gi]["offset_bytes"] + l * st[gi]["layer_stride"]
+                want = host[:, o:o + st[gi]["chunk_size"]].index_select(0, cpu_ids).to(device)
+                got = gpu[gi][l].reshape(n_gpu, -1).index_select(0, gi_dev)
+                ok = ok and bool(t.equal(want, got))
+        for l in range(L):
+            want = swa_host[l, 0].reshape(swa_cpu, -1).index_select(0, swa_c).to(device)
+            ok = ok and bool(t.equal(want, swa_dev[l].reshape(swa_gpu, -1)
+                                     .index_select(0, swa_g.to(device))))
+    launches = sum(len(m) for m in tables["layer_members"]) + L
+    grp.close()
+    return {"wall_s": _median(walls), "device_ms": _median(last_layer), "bytes": main_bytes + swa_bytes,
+            "main_bytes": main_bytes, "swa_bytes": swa_bytes, "bit_exact": ok,
+            "copies_per_restore": launches, "layers": L,
+            "desc": ("61 layers; groups: 30 x [2048,64,576] bf16 (ratio 4), 31 x [2048,2,576] bf16 "
+                     "(ratio 128), 30 x [2048,64,128] u8 indexer; sidecar 61 x [256,128,1152] u8; "
+                     "512 blocks + 64 sidecar slots, page 256")}
+
+
+def run_worker_process(torch, device, steps, warmup, num_cta, use_ce):
+    """c0-shaped put and get ops through a GPUCPUTransferWorker in its own process:
+    what the pipe, the shared op pool and the completion queue add to a transfer."""
+    import numpy as np
+    import torch.multiprocessing as mp
+    from flexkv_amd.layout import KVCacheLayout, KVCacheLayoutType
+    from flexkv_amd.transfer import trace
+    from flexkv_amd.transfer.memory_handle import TensorSharedHandle
+    from flexkv_amd.transfer.op_pool import SharedOpPool
+    from flexkv_amd.transfer.ops import TransferOp, TransferType
+    from flexkv_amd.transfer.worker import GPUCPUTransferWorker, PinnedPoolHandle
+    os.environ["FLEXKV_TRANSFER_TRACE"] = "1"   # the worker reports its own timings
+    trace.configure(True)
+    t = torch
+    # 1024 engine blocks: every shared allocation stays far below 2 GiB
+    L, N, T, H, D, NH, n = 32, 1024, 16, 8, 128, 1024, 256
+    gen = t.Generator(device=device).manual_seed(0)
+    tensors = [t.randn(2, N, T, H, D, device=device, dtype=t.bfloat16, generator=gen)
+               for _ in range(L)]
+    gl = KVCacheLayout(KVCacheLayoutType.LAYERFIRST, L, N, T, H, D, kv_dim=2, num_kv_heads=H)
+    cl = KVCacheLayout(KVCacheLayoutType.BLOCKFIRST, L, NH, T, H, D, kv_dim=2, num_kv_heads=H)
+    ctx = mp.get_context("spawn")
+    q = ctx.Queue()
+    pool = SharedOpPool(64, 1024)
+    h = GPUCPUTransferWorker.create_worker(
+        ctx, q, pool.get_buffer(), [TensorSharedHandle(x) for x in tensors],
+        PinnedPoolHandle(cl.kv_shape, t.bfloat16), gl, cl, t.bfloat16, 0,
+        use_ce_transfer_h2d=use_ce, use_ce_transfer_d2h=use_ce, transfer_num_cta_h2d=num_cta,
+        transfer_num_cta_d2h=num_cta)
+    h.wait_ready(300)
+    gg = t.Generator().manual_seed(1)
+    gpu_ids = t.randperm(N, generator=gg)[:n].numpy().astype(np.int64)
+    cpu_ids = t.randperm(NH, generator=gg)[:n].numpy().astype(np.int64)
+    nbytes = n * L * 2 * T * H * D * 2
+    rec = {"D2H": [], "H2D": []}
+    t_all = None
+    for it in range(warmup + steps):
+        if it == warmup:
+            t_all = time.perf_counter()
+        for kind, src, dst in ((TransferType.D2H, gpu_ids, cpu_ids),
+                               (TransferType.H2D, cpu_ids, gpu_ids)):
+            op = TransferOp(it, kind, src, dst)
+            op.src_slot_id = pool.allocate_slot(src, 1 if kind == TransferType.D2H else 2)
+            op.dst_slot_id = pool.allocate_slot(dst, 2 if kind == TransferType.D2H else 1)
+            t0 = time.perf_counter()
+            h.submit_transfer(op)
+            op_id, ok, m = q.get(timeout=300)
+            e2e = (time.perf_counter() - t0) * 1e3
+            assert ok and op_id == op.op_id
+            pool.free_slot(op.src_slot_id)
+            pool.free_slot(op.dst_slot_id)
+            if it >= warmup:
+                rec[kind.value].append((e2e, m["xfer_ms"], m["ipc_ms"], m["wait_ms"]))
+    wall = time.perf_counter() - t_all
+    h.shutdown()
+    med = lambda xs: _median(list(xs))
+    res = {"bytes_per_op": nbytes, "wall_s": wall, "exit_code": h.process.exitcode}
+    for k, rows in rec.items():
+        res[k] = {"e2e_ms": round(med(r[0] for r in rows), 3),
+                  "worker_xfer_ms": round(med(r[1] for r in rows), 3),
+                  "pipe_ms": round(med(r[2] for r in rows), 3),
+                  "queue_wait_ms": round(med(r[3] for r in rows), 3),
+                  "GBps_e2e": round(nbytes / (med(r[0] for r in rows) * 1e-3) / 1e9, 3),
+                  "GBps_in_worker": round(nbytes / (med(r[1] for r in rows) * 1e-3) / 1e9, 3)}
+    return res
+
+
 def cpu_baseline(cfg, budget_s=20.0):
     import torch
     from oracle import fkv_oracle as O
@@ -496,7 +657,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify"])
+    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker"])
     ap.add_argument("--num-cta", type=int, default=4,
                     help="transfer_num_cta (reference default FLEXKV_TRANSFER_NUM_CTA_*=4)")
     ap.add_argument("--use-ce", action="store_true", help="copy-engine path instead of the kernel")
@@ -543,6 +704,44 @@ def main():
                 "small": {"hostfunc": 0.60, "polling": 0.40},
                 "medium": {"hostfunc": 4.39, "polling": 1.87},
                 "large": {"hostfunc": 16.79, "polling": 16.62}}}))
+        return
+    if args.config == "mg":
+        link = measure_link()
+        r = run_multi_group(torch, device, args.steps, args.warmup, args.num_cta, args.notify,
+                            args.use_ce, verify=not args.no_verify)
+        rate = r["bytes"] / (r["device_ms"] * 1e-3) / 1e9
+        print(json.dumps({
+            "metric": "multi-group layerwise restore GB/s (H2D) on 1 GPU", "unit": "GB/s",
+            "value": round(rate, 3), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(r["wall_s"] * 1e3, 3), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": "mg: " + r["desc"], "notify": args.notify,
+                       "path": "copy-engine" if args.use_ce else "kernel",
+                       "transfer_num_cta": args.num_cta},
+            "restore_device_ms": round(r["device_ms"], 3),
+            "bytes": r["bytes"], "main_bytes": r["main_bytes"], "sidecar_bytes": r["swa_bytes"],
+            "copies_per_restore": r["copies_per_restore"],
+            "ms_per_original_layer": round(r["device_ms"] / r["layers"], 4),
+            "h2d_frac_of_link": round(rate / link["h2d"], 4), "bit_exact": r["bit_exact"],
+            "link_peak": {"h2d_GBps": round(link["h2d"], 3)}}))
+        return
+    if args.config == "worker":
+        link = measure_link()
+        r = run_worker_process(torch, device, args.steps, args.warmup, args.num_cta, args.use_ce)
+        print(json.dumps({
+            "metric": "put/get through a transfer worker process: GB/s seen by the submitter",
+            "unit": "GB/s", "value": round(2 * r["bytes_per_op"] * args.steps / r["wall_s"] / 1e9, 3),
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(r["wall_s"] / args.steps * 1e3, 3), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": "worker: c0 chunk shape (32 layers x [2,1024,16,8,128] bf16), "
+                                   "256 random blocks per op, ids through the shared op pool, "
+                                   "worker-owned pinned host pool",
+                       "path": "copy-engine" if args.use_ce else "kernel",
+                       "transfer_num_cta": args.num_cta},
+            "put": r["D2H"], "get": r["H2D"], "bytes_per_op": r["bytes_per_op"],
+            "worker_exit_code": r["exit_code"],
+            "link_peak": {"d2h_GBps": round(link["d2h"], 3), "h2d_GBps": round(link["h2d"], 3)}}))
         return
     link = measure_link()
     w = Workload(args.config, torch, device)

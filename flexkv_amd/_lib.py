@@ -181,6 +181,9 @@ SIGNATURES = {
     "fkv_host_unregister": (c_int32, [c_void_p, c_size_t, c_size_t]),
     "fkv_host_register_plan": (c_int64, [c_size_t, c_size_t, c_void_p, c_void_p, c_int64]),
     "fkv_host_chunk_bytes_from_gb": (c_size_t, [c_double]),
+    "fkv_ipc_export": (c_int32, [c_void_p, c_void_p, POINTER(c_int64), POINTER(c_int64)]),
+    "fkv_ipc_open": (c_int32, [c_void_p, c_int32, POINTER(c_void_p)]),
+    "fkv_ipc_close": (c_int32, [c_void_p]),
     "fkv_get_stats": (None, [POINTER(Stats)]),
     "fkv_reset_stats": (None, []),
     "fkv_measure_link_peak": (c_int32, [c_int32, c_size_t, c_int32, c_int32,

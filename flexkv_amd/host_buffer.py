@@ -47,12 +47,13 @@ hipHostUnregister = cudaHostUnregister
 
 def alloc_mapped_host_tensor(num_elements: int, dtype: torch.dtype) -> torch.Tensor:
     """Pinned, device-mapped host tensor (hipHostMalloc Portable|Mapped); freed
-    when the tensor is garbage collected."""
+    when the last tensor that views the allocation is garbage collected."""
     nbytes = int(num_elements) * dtype.itemsize
     ptr = ctypes.c_void_p()
     check(_L.fkv_host_alloc(nbytes, ctypes.byref(ptr)))
     raw = (ctypes.c_uint8 * nbytes).from_address(ptr.value)
     arr = np.frombuffer(raw, dtype=np.uint8, count=nbytes)
-    tensor = torch.from_numpy(arr).view(dtype)[:num_elements]
-    weakref.finalize(tensor, _L.fkv_host_free, ctypes.c_void_p(ptr.value))
-    return tensor
+    # The storage of every view keeps `arr`, and through it `raw`, alive: the
+    # allocation goes when `raw` does, not when the first tensor object does.
+    weakref.finalize(raw, _L.fkv_host_free, ctypes.c_void_p(ptr.value))
+    return torch.from_numpy(arr).view(dtype)[:num_elements]

@@ -408,6 +408,25 @@ int64_t fkv_host_register_plan(size_t bytes, size_t chunk_bytes, size_t *offsets
 /* FLEXKV_CUDAHOST_CHUNK_SIZE_GB -> chunk bytes, host_buffer.py:57-63. */
 size_t fkv_host_chunk_bytes_from_gb(double chunk_gb);
 
+/* ---- engine tensors shared with a worker process:
+ *      flexkv/common/memory_handle.py:1144-1250 (direct IPC branch of
+ *      TensorSharedHandle) ---- */
+
+#define FKV_IPC_HANDLE_BYTES 64
+
+/* Owner side: handle of the device allocation `device_ptr` lives in
+ * (hipIpcGetMemHandle of its base address), the offset of `device_ptr` inside
+ * it and, optionally, the size of the allocation.  Allocations of 2 GiB or
+ * more should not be shared this way. */
+int fkv_ipc_export(const void *device_ptr, uint8_t *handle_out /* 64 bytes */,
+                   int64_t *offset_out, int64_t *allocation_bytes_out);
+/* Worker side: map the allocation on `device` (-1 = current) and return its
+ * base address.  Repeated opens of one handle in a process return the same
+ * mapping and are counted. */
+int fkv_ipc_open(const uint8_t *handle /* 64 bytes */, int32_t device, void **base_out);
+/* Drop one reference; the mapping goes with the last one. */
+int fkv_ipc_close(void *base);
+
 /* ---- counters (the reference's FLEXKV_GPU_CPU_TRANSFER metric hook is a
  *      no-op unless monitoring is compiled in, csrc/ce_transfer.cu:29-31) ---- */
 typedef struct fkv_stats {

@@ -1,0 +1,283 @@
+"""Transfer workers in their own processes, on the GPU: engine tensors shared
+through both handle forms, ops submitted through the pipe and the shared op
+pool, completions read from the queue, bytes checked against the oracle or by a
+put -> erase -> get round trip."""
+import os
+import queue as pyqueue
+import struct
+import time
+
+import numpy as np
+import pytest
+import torch
+import torch.multiprocessing as mp
+
+from flexkv_amd.layout import (KVCacheLayout, KVCacheLayoutType, LayerGroupSpec,
+                               MultiGroupBlockLayout, TransferStrides)
+from flexkv_amd.transfer.eventfd_channel import make_eventfd, send_layer_eventfds
+from flexkv_amd.transfer.memory_handle import TensorSharedHandle
+from flexkv_amd.transfer.op_pool import SharedOpPool
+from flexkv_amd.transfer.ops import LayerwiseTransferOp, TransferOp, TransferType
+from flexkv_amd.transfer.worker import (GPUCPUTransferWorker, LayerwiseTransferWorker,
+                                        PinnedPoolHandle, tpGPUCPUTransferWorker)
+
+pytestmark = pytest.mark.gpu
+
+I64 = np.int64
+L, N_GPU, N_CPU, T, H, D = 4, 24, 32, 8, 2, 64
+DT = torch.int16  # two-byte elements, like bf16 KV
+
+
+def _gpu_layout(kv_dim=2, heads=H, layers=L):
+    return KVCacheLayout(KVCacheLayoutType.LAYERFIRST, layers, N_GPU, T, heads, D, kv_dim=kv_dim,
+                         num_kv_heads=heads)
+
+
+def _cpu_layout(kind, kv_dim=2, heads=H, layers=L):
+    return KVCacheLayout(kind, layers, N_CPU, T, heads, D, kv_dim=kv_dim, num_kv_heads=heads)
+
+
+def _engine_tensors(device, seed, kv_dim=2, heads=H, layers=L):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(-30000, 30000, (kv_dim, N_GPU, T, heads, D), dtype=DT, generator=g)
+            .to(device) for _ in range(layers)]
+
+
+def _collect(q, n, timeout=120):
+    got = []
+    end = time.time() + timeout
+    while len(got) < n:
+        try:
+            got.append(q.get(timeout=max(0.1, end - time.time())))
+        except pyqueue.Empty:
+            break
+    return got
+
+
+@pytest.fixture
+def engine():
+    ctx = mp.get_context("spawn")
+    q = ctx.Queue()
+    pool = SharedOpPool(16, 64)
+    handles = []
+
+    def start(cls, *args, **kw):
+        h = cls.create_worker(ctx, q, pool.get_buffer(), *args, **kw)
+        handles.append(h)
+        h.wait_ready(180)
+        return h
+    yield start, q, pool
+    for h in handles:
+        if h.process.is_alive():
+            h.shutdown()
+
+
+def _op(kind, src, dst, pool=None, graph=0):
+    op = TransferOp(graph, kind, np.asarray(src, dtype=I64), np.asarray(dst, dtype=I64))
+    if pool is not None:
+        op.src_slot_id = pool.allocate_slot(op.src_block_ids, 1)
+        op.dst_slot_id = pool.allocate_slot(op.dst_block_ids, 2)
+        assert op.src_slot_id >= 0 and op.dst_slot_id >= 0
+    return op
+
+
+@pytest.mark.parametrize("direct_ipc", [False, True])
+@pytest.mark.parametrize("engine_kind", [False, True])
+def test_worker_owned_pinned_pool_round_trip(gpu_device, engine, direct_ipc, engine_kind):
+    """Put through the worker, erase, get into other blocks: the worker's pool is
+    its own pinned allocation, so the copy kernel's path runs inside the worker."""
+    start, q, pool = engine
+    tensors = _engine_tensors(gpu_device, 1)
+    want = [t.clone() for t in tensors]
+    handles = [TensorSharedHandle(t, force_direct_ipc=direct_ipc) for t in tensors]
+    assert handles[0].handle_type == ("hip_ipc" if direct_ipc else "torch_reduce")
+    cl = _cpu_layout(KVCacheLayoutType.BLOCKFIRST)
+    h = start(GPUCPUTransferWorker, handles, PinnedPoolHandle(cl.kv_shape, DT), _gpu_layout(), cl,
+              DT, 0, use_ce_transfer_h2d=engine_kind, use_ce_transfer_d2h=engine_kind)
+    assert h.control("ping")["pageable_host"] is False
+    rng = np.random.default_rng(3)
+    src_blocks = rng.permutation(N_GPU)[:10]
+    host_blocks = rng.permutation(N_CPU)[:10]
+    back_blocks = np.setdiff1d(np.arange(N_GPU), src_blocks)[:10]
+    put = _op(TransferType.D2H, src_blocks, host_blocks, pool)
+    h.submit_transfer(put)
+    assert _collect(q, 1) == [(put.op_id, True, None)]
+    get = _op(TransferType.H2D, host_blocks, back_blocks)  # ids travel with the op
+    h.submit_transfer(get)
+    assert _collect(q, 1) == [(get.op_id, True, None)]
+    torch.cuda.synchronize()
+    for l in range(L):
+        assert torch.equal(tensors[l][:, back_blocks], want[l][:, src_blocks]), l
+        untouched = np.setdiff1d(np.arange(N_GPU), back_blocks)
+        assert torch.equal(tensors[l][:, untouched], want[l][:, untouched]), l
+    # an op this worker cannot run is reported as failed, and the worker keeps serving
+    e = np.array([], dtype=I64)
+    wrong = LayerwiseTransferOp(0, TransferType.LAYERWISE, e, e)
+    h.submit_transfer(wrong)
+    assert _collect(q, 1) == [(wrong.op_id, False, None)]
+    again = _op(TransferType.D2H, src_blocks[:2], host_blocks[:2])
+    h.submit_transfer(again)
+    assert _collect(q, 1) == [(again.op_id, True, None)]
+    h.shutdown()
+    assert h.process.exitcode == 0
+
+
+@pytest.mark.parametrize("kind", [KVCacheLayoutType.BLOCKFIRST, KVCacheLayoutType.LAYERFIRST])
+def test_shared_memory_pool_matches_the_oracle(gpu_device, engine, kind):
+    """The reference's arrangement: the pool is a shared-memory tensor the engine
+    can read.  The worker registers it; where the runtime refuses that, it keeps it
+    pageable and moves everything with the copy engine."""
+    from oracle import fkv_oracle as O
+    start, q, pool = engine
+    tensors = _engine_tensors(gpu_device, 2)
+    cl, gl = _cpu_layout(kind), _gpu_layout()
+    host = torch.zeros(cl.kv_shape, dtype=DT).share_memory_()
+    h = start(GPUCPUTransferWorker, [TensorSharedHandle(t) for t in tensors], host, gl, cl, DT, 0,
+              allow_pageable_host=True)
+    print("pageable host pool:", h.control("ping")["pageable_host"], flush=True)
+    rng = np.random.default_rng(5)
+    gpu_ids = rng.permutation(N_GPU)[:12]
+    cpu_ids = rng.permutation(N_CPU)[:12]
+    put = _op(TransferType.D2H, gpu_ids, cpu_ids, pool)
+    h.submit_transfer(put)
+    assert _collect(q, 1) == [(put.op_id, True, None)]
+    ref_gpu = [t.cpu().numpy().view(np.uint8).reshape(-1) for t in tensors]
+    ref_host = np.zeros(host.numel() * 2, dtype=np.uint8)
+    gs, cs = TransferStrides.from_layout(gl, 2), TransferStrides.from_layout(cl, 2)
+    O.transfer_c(O.BACKEND_VLLM, [a.ctypes.data for a in ref_gpu], L, gs.kv, gs.block, gs.layer, 0,
+                 ref_host.ctypes.data, cs.kv, cs.layer, cs.block, 0, gs.chunk, 0, L, 2,
+                 gpu_ids, cpu_ids, False)
+    assert np.array_equal(host.numpy().view(np.uint8).reshape(-1), ref_host)
+    h.shutdown()
+    assert h.process.exitcode == 0
+
+
+def test_multi_group_worker_round_trip(gpu_device, engine):
+    """Layer groups of different width and compression behind one worker
+    (worker.py:850-1030 of the reference): one call per group into its byte range of
+    the host block."""
+    start, q, pool = engine
+    tpb = 32
+    groups = [LayerGroupSpec(3, 1, 48, (0, 1, 2), 2, 1), LayerGroupSpec(2, 1, 24, (1, 2), 2, 4),
+              LayerGroupSpec(2, 1, 40, (0, 2), 1, 2)]
+    gpu_layouts = [KVCacheLayout(KVCacheLayoutType.LAYERFIRST, g.num_layers, N_GPU,
+                                 tpb // g.compress_ratio, 1, g.head_size, kv_dim=1)
+                   for g in groups]
+    cl = MultiGroupBlockLayout(N_CPU, tpb, tuple(groups), kv_dim=1)
+    gen = torch.Generator().manual_seed(9)
+    per_group = [[torch.randint(0, 256, (N_GPU, tpb // g.compress_ratio, 1,
+                                         g.head_size * g.itemsize), dtype=torch.uint8,
+                                generator=gen).to(gpu_device) for _ in range(g.num_layers)]
+                 for g in groups]
+    want = [[t.clone() for t in grp] for grp in per_group]
+    handles = [[TensorSharedHandle(t) for t in grp] for grp in per_group]
+    h = start(GPUCPUTransferWorker, handles[0], PinnedPoolHandle(cl.kv_shape, torch.uint8),
+              gpu_layouts[0], cl, torch.uint8, 0, layer_groups=groups,
+              gpu_blocks_per_group=handles, gpu_layouts_per_group=gpu_layouts)
+    src, mid, back = [1, 7, 3, 20], [9, 0, 31, 4], [11, 12, 13, 2]
+    put, get = _op(TransferType.D2H, src, mid), _op(TransferType.H2D, mid, back, pool)
+    h.submit_transfer(put)
+    h.submit_transfer(get)
+    assert _collect(q, 2) == [(put.op_id, True, None), (get.op_id, True, None)]
+    torch.cuda.synchronize()
+    for gi, grp in enumerate(per_group):
+        for l, t in enumerate(grp):
+            assert torch.equal(t[back], want[gi][l][src]), (gi, l)
+    h.shutdown()
+
+
+@pytest.mark.parametrize("heads,kv_dim,mode", [(4, 2, "sharded"), (1, 1, "sharded"),
+                                               (1, 1, "rank0_only")])
+def test_tp_worker_two_ranks_round_trip(gpu_device, engine, heads, kv_dim, mode, monkeypatch):
+    """Two ranks of a tensor-parallel group (both placed on this GPU) behind one
+    worker.  With separate heads each rank owns half the heads of every host
+    chunk; with shared KV both ranks hold the same bytes."""
+    import flexkv_amd.transfer.env as env
+    monkeypatch.setenv("FLEXKV_KV_SHARED_ACROSS_RANKS_MODE", mode)
+    monkeypatch.setattr(env, "_ENV", None)
+    start, q, pool = engine
+    tp = 2
+    rank_heads = heads // tp if heads > 1 else 1
+    ranks = [_engine_tensors(gpu_device, 20 + r if heads > 1 else 20, kv_dim, rank_heads)
+             for r in range(tp)]
+    want = [[t.clone() for t in ts] for ts in ranks]
+    gl = [KVCacheLayout(KVCacheLayoutType.LAYERFIRST, L, N_GPU, T, rank_heads, D, kv_dim=kv_dim,
+                        num_kv_heads=heads) for _ in range(tp)]
+    cl = KVCacheLayout(KVCacheLayoutType.BLOCKFIRST, L, N_CPU, T, heads, D, kv_dim=kv_dim,
+                       num_kv_heads=heads)
+    h = start(tpGPUCPUTransferWorker, [[TensorSharedHandle(t) for t in ts] for ts in ranks],
+              PinnedPoolHandle(cl.kv_shape, DT), gl, cl, DT, tp)
+    src, mid, back = [2, 9, 5], [30, 1, 17], [20, 21, 22]
+    put, get = _op(TransferType.D2H, src, mid, pool), _op(TransferType.H2D, mid, back, pool)
+    h.submit_transfer(put)
+    h.submit_transfer(get)
+    assert _collect(q, 2) == [(put.op_id, True, None), (get.op_id, True, None)]
+    torch.cuda.synchronize()
+    for r in range(tp):
+        for l in range(L):
+            assert torch.equal(ranks[r][l][:, back], want[r][l][:, src]), (r, l)
+    h.shutdown()
+    monkeypatch.setattr(env, "_ENV", None)
+
+
+def _wait_units(fd, timeout=60.0):
+    """Blocks like an engine does: one read per unit of the semaphore eventfd."""
+    os.set_blocking(fd, True)
+    import select
+    r, _, _ = select.select([fd], [], [], timeout)
+    assert r, "no notification"
+    return struct.unpack("Q", os.read(fd, 8))[0]
+
+
+@pytest.mark.parametrize("notify", ["hostfunc", "polling"])
+def test_layerwise_worker_with_engine_eventfds(gpu_device, engine, tmp_path, notify,
+                                               monkeypatch):
+    """The engine hands its per-layer eventfds to the worker over the unix socket,
+    submits a layerwise op and wakes up once per layer."""
+    import threading
+    import flexkv_amd.transfer.env as env
+    monkeypatch.setenv("FLEXKV_LAYERWISE_NOTIFY_MODE", notify)
+    monkeypatch.setattr(env, "_ENV", None)
+    start, q, pool = engine
+    kv_dim, heads, counters = 1, 1, 3
+    tensors = _engine_tensors(gpu_device, 40, kv_dim, heads)
+    want = [t.clone() for t in tensors]
+    gl = _gpu_layout(kv_dim, heads)
+    cl = _cpu_layout(KVCacheLayoutType.BLOCKFIRST, kv_dim, heads)
+    sock = str(tmp_path / "lw.sock")
+    fds = [[make_eventfd() for _ in range(L)] for _ in range(counters)]
+    sender = threading.Thread(target=send_layer_eventfds, args=(sock, 0, 1, fds),
+                              kwargs=dict(retry_interval_s=0.2))
+    sender.start()
+    # the host pool is shared memory, so the engine side of the test can fill it
+    host = torch.zeros(cl.kv_shape, dtype=DT).share_memory_()
+    src = [3, 8, 1, 15]
+    mid = [4, 5, 20, 9]
+    back = [10, 11, 12, 13]
+    for l in range(L):  # the engine-side image of blocks `src` at host blocks `mid`
+        host[mid, l, 0] = tensors[l][0, src].cpu()
+    h = start(LayerwiseTransferWorker, [[TensorSharedHandle(t) for t in tensors]], host, [gl], cl,
+              DT, 1, layerwise_eventfd_socket=sock, use_ce_transfer_h2d=False,
+              allow_pageable_host=True)
+    sender.join(60)
+    assert not sender.is_alive()
+    e = np.array([], dtype=I64)
+    op = LayerwiseTransferOp(0, TransferType.LAYERWISE, e, e,
+                             src_block_ids_h2d=np.asarray(mid, dtype=I64),
+                             dst_block_ids_h2d=np.asarray(back, dtype=I64), counter_id=1)
+    h.submit_transfer(op)
+    for l in range(L):
+        assert _wait_units(fds[1][l]) == 1   # layer l has landed
+        assert torch.equal(tensors[l][:, back], want[l][:, src]), l
+    assert _collect(q, 1) == [(op.op_id, True, None)]
+    for c in (0, 2):  # the other counter sets stayed silent
+        for fd in fds[c]:
+            os.set_blocking(fd, False)
+            with pytest.raises(BlockingIOError):
+                os.read(fd, 8)
+    h.shutdown()
+    assert h.process.exitcode == 0
+    for cs in fds:
+        for fd in cs:
+            os.close(fd)
+    monkeypatch.setattr(env, "_ENV", None)
