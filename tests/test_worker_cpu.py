@@ -328,7 +328,9 @@ def test_worker_metrics_when_trace_is_on(harness, monkeypatch):
         assert m["type"] == "H2D" and m["nb"] == 4 and m["bytes"] == 4 * 4096 and m["is_h2d"]
         assert m["xfer_ms"] >= 20.0 and m["ipc_ms"] >= 0.0 and m["worker_id"] == h.worker_id
         trace.record_xfer(op_id, m)
-        assert len(lines) == 1 and XFER_RE.match(lines[0]) and " backlog=0" in lines[0]
+        assert XFER_RE.match(lines[0]) and " backlog=0" in lines[0]
+        # the process-wide window may have been open for more than its ten seconds
+        assert all(SUMMARY_RE.match(x) for x in lines[1:]) and len(lines) <= 2
     finally:
         trace.configure(False)
         monkeypatch.setattr(env, "_ENV", None)
