@@ -348,6 +348,11 @@ int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
     a.lk = nl * p.kv_dim;
     a.vec = p.vec;
     a.nt_store = p.h2d ? 1 : 0;
+    // Packed short chunks cost a wavefront more address arithmetic per request, so
+    // the host->GPU direction, which lives on requests in flight, gets half as many
+    // workgroups again: 16 x 64 lanes reach 45 GB/s on 2304-byte chunks, 24 x 64
+    // reach 55.8, 32 x 64 reach 56.2.
+    a.packed_grid_pct = p.h2d ? 150 : 100;
     a.xcd_mask = p.xcd_mask;
     FKV_TRY(launch_copy_kernel(a, p.workgroups, p.threads, stream));
   }

@@ -113,6 +113,8 @@ struct CopyKernelArgs {
   int32_t slices_per_chunk;
   int32_t vec;      // 16, 8, 4, 2 or 1: widest access all addresses allow
   int32_t nt_store; // 1: nontemporal stores (destination in HBM), 0: plain (pinned host)
+  int32_t packed;   // set by launch_copy_kernel: chunks shorter than a slice, see the kernel
+  int32_t packed_grid_pct; // workgroups to launch in packed mode, percent of the request (0 = 100)
   uint32_t xcd_mask; // bit k: workgroups with blockIdx % 8 == k take part; 0 or 0xff = all
 };
 constexpr int kCopyBlockThreads = 1024;  // largest workgroup the kernel is built for

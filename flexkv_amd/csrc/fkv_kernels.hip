@@ -19,7 +19,12 @@
 // requests a workgroup has in flight target neighbouring addresses.  A
 // wavefront issues all kCopyUnroll loads of a slice before the first store, which
 // is what keeps enough reads outstanding to cover the host-link latency in
-// the host->GPU direction.
+// the host->GPU direction.  Chunks shorter than a slice (compressed layer
+// groups, small pages) are packed: the 16-byte vectors of all chunks form one
+// flat sequence that is cut into full slices regardless of chunk boundaries,
+// every lane resolving the chunk of each of its vectors from the LDS tables, so
+// that a wavefront keeps a full slice of requests in flight however short the
+// chunks are.
 //
 // Launch shape.  The link is saturated by roughly 200 KB of requests in flight.
 // Requests to host memory sit in the memory-request queues of the XCD that
@@ -39,6 +44,8 @@
 // by this kernel.  Stores into HBM are nontemporal too; stores into pinned host
 // memory are plain, which measured about 1 GB/s faster over the link.
 #include "fkv_internal.h"
+
+#include <cstdlib>
 
 namespace fkv {
 namespace {
@@ -76,9 +83,17 @@ __device__ __forceinline__ void copy_slice(const uint8_t *__restrict__ src,
     for (int u = 0; u < kCopyUnroll; ++u)
       put<V, NTS>(r[u], d + u * kWave);
   } else {
-    const int64_t nvec = bytes_in_slice / VEC;
-    for (int64_t i = lane; i < nvec; i += kWave)
-      put<V, NTS>(__builtin_nontemporal_load(s + (i - lane)), d + (i - lane));
+    // the short last slice of a chunk: same shape, lanes beyond the end sit out
+    // (they re-read the last vector rather than branch around the load)
+    const int nvec = (int)(bytes_in_slice / VEC);
+    V r[kCopyUnroll];
+#pragma unroll
+    for (int u = 0; u < kCopyUnroll; ++u)
+      r[u] = __builtin_nontemporal_load(s - lane + min(lane + u * kWave, nvec - 1));
+#pragma unroll
+    for (int u = 0; u < kCopyUnroll; ++u)
+      if (lane + u * kWave < nvec)
+        put<V, NTS>(r[u], d + u * kWave);
   }
 }
 
@@ -92,9 +107,15 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
   int64_t *s_off_dst = s_off_src + kCopyIdTile;
 
   constexpr int64_t kSliceBytes = (int64_t)kWave * kCopyUnroll * VEC;
+  constexpr uint32_t kPiece = kWave * kCopyUnroll; // vectors a wavefront moves per step
   const uint32_t slices = (uint32_t)a.slices_per_chunk;
-  const uint32_t spp = (uint32_t)a.lk * slices; // slices per block position
-  const uint64_t total = (uint64_t)a.num_blocks * spp;
+  // Work units.  Normal mode: slices of a chunk, `spp` per block position.  Packed
+  // mode (chunks shorter than a slice): the vectors of all chunks form one flat
+  // sequence, cut into pieces of kPiece vectors regardless of chunk boundaries.
+  const uint32_t vpc = (uint32_t)(a.chunk_bytes / VEC);  // vectors per chunk
+  const uint32_t spp = a.packed ? (uint32_t)a.lk * vpc : (uint32_t)a.lk * slices;
+  const uint64_t total_units = (uint64_t)a.num_blocks * spp;
+  const uint64_t total = a.packed ? (total_units + kPiece - 1) / kPiece : total_units;
   // Workgroups are handed to the 8 XCDs round-robin by blockIdx.x.  With a
   // partial mask only the workgroups that land on the selected XCDs take part;
   // they are renumbered densely, the others leave at once.
@@ -107,10 +128,14 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
     wg = (blockIdx.x >> 3) * per_round + __popc(a.xcd_mask & ((1u << slot) - 1u));
     nwg = (gridDim.x >> 3) * per_round;
   }
-  const uint64_t s0 = total * wg / nwg;
-  const uint64_t s1 = total * (wg + 1) / nwg;
+  uint64_t s0 = total * wg / nwg;
+  uint64_t s1 = total * (wg + 1) / nwg;
   if (s0 >= s1)
     return; // whole workgroup leaves together
+  if (a.packed) { // from pieces to vectors
+    s0 *= kPiece;
+    s1 = s1 * kPiece < total_units ? s1 * kPiece : total_units;
+  }
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -137,6 +162,57 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
     const uint64_t t0 = s0 > tile_s0 ? s0 : tile_s0;
     const uint64_t tile_s1 = tile_s0 + (uint64_t)n * spp;
     const uint64_t t1 = s1 < tile_s1 ? s1 : tile_s1;
+    if (a.packed) {
+      using V = typename VecType<VEC>::type;
+      const uint32_t lim = (uint32_t)(t1 - tile_s0); // < kCopyIdTile * spp, checked on host
+      const uint32_t ulk = (uint32_t)a.lk;
+      const uint32_t q64 = kWave / vpc, r64 = kWave % vpc; // kWave vectors = q64 chunks + r64
+      const uint32_t qlk = q64 / ulk, rlk = q64 % ulk;     // q64 chunks = qlk positions + rlk
+      for (uint32_t v0 = (uint32_t)(t0 - tile_s0) + wave * kPiece; v0 < lim;
+           v0 += nwaves * kPiece) {
+        V r[kCopyUnroll];
+        V *d[kCopyUnroll];
+        // A lane's vectors are kWave apart.  The first one is located by division;
+        // each further one by adding the precomputed quotients and remainders of
+        // kWave, which costs a few compares instead of two divisions.  Lanes beyond
+        // the end stay on their last valid vector and re-read it rather than branch
+        // around the load: all loads of a piece are issued back to back, only the
+        // stores are predicated.
+        uint32_t v = v0 + lane;
+        const uint32_t vc = min(v, lim - 1);
+        const uint32_t c = vc / vpc; // chunk inside the tile: position * lk + i
+        uint32_t w = vc - c * vpc;
+        uint32_t p = c / ulk;
+        uint32_t i = c - p * ulk;
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u) {
+          if (u > 0) {
+            v += kWave;
+            uint32_t w2 = w + r64, i2 = i + rlk, p2 = p + qlk;
+            if (w2 >= vpc) {
+              w2 -= vpc;
+              i2 += 1;
+            }
+            if (i2 >= ulk) {
+              i2 -= ulk;
+              p2 += 1;
+            }
+            const bool ok = v < lim;
+            w = ok ? w2 : w;
+            i = ok ? i2 : i;
+            p = ok ? p2 : p;
+          }
+          const V *src = reinterpret_cast<const V *>(s_base_src[i] + (uint64_t)s_off_src[p]) + w;
+          d[u] = reinterpret_cast<V *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + w;
+          r[u] = __builtin_nontemporal_load(src);
+        }
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u)
+          if (v0 + u * kWave + lane < lim)
+            put<V, NTS>(r[u], d[u]);
+      }
+      continue;
+    }
     for (uint64_t s = t0 + wave; s < t1; s += nwaves) {
       const uint32_t rel = (uint32_t)(s - tile_s0); // < kCopyIdTile * spp, checked on host
       const uint32_t p = rel / spp;
@@ -201,7 +277,22 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_wor
                 "copy kernel: chunk of %lld B x %d (layer,kv) pairs is too large for one launch",
                 (long long)a.chunk_bytes, a.lk);
   a.slices_per_chunk = (int32_t)slices;
-  const int64_t total = spp * a.num_blocks;
+  int64_t total = spp * a.num_blocks;
+  // Chunks shorter than one slice would leave most lanes of a wavefront idle and
+  // most of its requests unissued: pack them (the kernel indexes vectors inside an
+  // id tile with 32 bits).
+  const int64_t vpp = a.chunk_bytes / a.vec * a.lk;
+  a.packed = (a.chunk_bytes < slice_bytes && vpp * kCopyIdTile <= (int64_t)UINT32_MAX) ? 1 : 0;
+  static const bool no_pack = [] {
+    const char *v = std::getenv("FKV_COPY_NO_PACK");
+    return v && *v == '1';
+  }();
+  if (no_pack)
+    a.packed = 0;
+  if (a.packed) {
+    const int64_t piece = (int64_t)kWave * kCopyUnroll;
+    total = (vpp * a.num_blocks + piece - 1) / piece;
+  }
   int threads = threads_per_workgroup;
   if (threads < kWave)
     threads = kWave;
@@ -210,6 +301,8 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_wor
   threads = threads / kWave * kWave;
   const int waves_per_wg = threads / kWave;
   int64_t grid = num_workgroups > 0 ? num_workgroups : 1;
+  if (a.packed && a.packed_grid_pct > 0)
+    grid = (grid * a.packed_grid_pct + 99) / 100;
   const int64_t useful = (total + waves_per_wg - 1) / waves_per_wg;
   if (grid > useful)
     grid = useful;

@@ -120,6 +120,32 @@ def test_many_blocks_cross_id_tiles(gpu_device):
     dev.assert_matches_reference("4500 blocks H2D")
 
 
+@pytest.mark.parametrize("backend,L,K,chunk,n", [
+    (VLLM, 31, 1, 2 * 576 * 2, 512),      # a 128x-compressed latent group: 2304-byte chunks
+    (VLLM, 3, 2, 144, 700),                # 9 vectors per chunk, more positions than an id tile holds
+    (SGLANG, 5, 2, 8176, 40),              # one vector short of a full slice
+    (TRTLLM, 7, 2, 520, 300),              # 8-byte vectors (520 = 8 * 65)
+    (VLLM, 2, 2, 1028, 90),                # 4-byte vectors
+])
+def test_short_chunks_are_packed(gpu_device, backend, L, K, chunk, n):
+    """Chunks shorter than a slice travel as one flat sequence of vectors: pieces,
+    workgroup ranges and id tiles all cut through chunks at arbitrary places."""
+    N = n + n // 2
+    s = KVSetup(backend, L, K, N, N, chunk, "BLOCKFIRST", seed=31)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(6)
+    for cta in (1, 4, 37):
+        gids, cids = block_ids(rng, N, n), block_ids(rng, N, n)
+        print(f"case backend={backend} chunk={chunk} n={n} cta={cta}", flush=True)
+        assert dev.transfer_raw(gids, cids, False, num_cta=cta) == 0
+        s.oracle_transfer(gids, cids, False)
+        dev.assert_matches_reference(f"D2H cta={cta}")
+        gids2 = block_ids(rng, N, n)
+        assert dev.transfer_raw(gids2, cids, True, num_cta=cta) == 0
+        s.oracle_transfer(gids2, cids, True)
+        dev.assert_matches_reference(f"H2D cta={cta}")
+
+
 def test_more_layer_kv_pairs_than_one_launch_holds(gpu_device):
     """700 layers x 2 = 1400 (layer, kv) pairs: split over two launches."""
     s = KVSetup(VLLM, 700, 2, 6, 6, 32, "BLOCKFIRST", seed=9)
