@@ -164,7 +164,11 @@ struct KernelPlan {
   int64_t chunk_size = 0, gpu_block_stride = 0, cpu_block_stride = 0;
   int workgroups = 1, threads = 64;
   unsigned xcd_mask = 0xff;
+  int device = 0;
 };
+// Link-bound launches of the last while, per device and direction (see fkv_core.cpp).
+bool link_direction_busy(int device, bool h2d);
+void link_direction_mark(int device, bool h2d, hipStream_t stream);
 // Builds and uploads (on `stream`) the plan for all layers of `d`.
 int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan *out);
 // Enqueues the copy of layers [layer_offset, layer_offset + num_layers) of the plan.

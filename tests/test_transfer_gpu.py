@@ -146,6 +146,41 @@ def test_short_chunks_are_packed(gpu_device, backend, L, K, chunk, n):
         dev.assert_matches_reference(f"H2D cta={cta}")
 
 
+def test_puts_and_gets_at_the_same_time(gpu_device):
+    """A GPU->host and a host->GPU transfer in flight together on two streams: a
+    launch that finds the other direction busy confines itself to half of the
+    XCDs.  Which workgroups take part must not change a byte."""
+    import threading
+    import torch
+    s = KVSetup(VLLM, 8, 2, 600, 600, 16 * 8 * 128 * 2, "BLOCKFIRST", seed=41)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(8)
+    perm_g, perm_c = rng.permutation(600), rng.permutation(600)
+    # disjoint blocks on both sides, so the two directions never touch the same bytes
+    put_g, put_c = perm_g[:250], perm_c[:250]
+    get_g, get_c = perm_g[250:500], perm_c[250:500]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    errors = []
+
+    def run(i):
+        try:
+            for _ in range(6):
+                rc = dev.transfer_raw(put_g if i == 0 else get_g, put_c if i == 0 else get_c,
+                                      i == 1, sync=False, stream=streams[i].cuda_stream)
+                assert rc == 0
+            streams[i].synchronize()
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(2)]
+    [t.start() for t in threads]
+    [t.join() for t in threads]
+    assert not errors, errors
+    torch.cuda.synchronize()
+    s.oracle_transfer(put_g, put_c, False)
+    s.oracle_transfer(get_g, get_c, True)
+    dev.assert_matches_reference("concurrent put and get")
+
+
 def test_more_layer_kv_pairs_than_one_launch_holds(gpu_device):
     """700 layers x 2 = 1400 (layer, kv) pairs: split over two launches."""
     s = KVSetup(VLLM, 700, 2, 6, 6, 32, "BLOCKFIRST", seed=9)
