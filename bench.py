@@ -614,6 +614,87 @@ def run_worker_process(torch, device, steps, warmup, num_cta, use_ce):
     return res
 
 
+def run_ssd(torch, steps, warmup, ssd_dir, blocks, pinned):
+    """Host pool <-> SSD files in the shape of the reference's SSD microbenchmark
+    (benchmarks/microbenchmark_ssd_simulation.py): "small" MHA preset, both pool
+    layouts, contiguous and scattered block ids, both directions, chunk-at-a-time
+    requests (ssd_io_opt off) against coalesced ones, threads against io_uring."""
+    import ctypes
+    import mmap
+    import shutil
+    import tempfile
+    import numpy as np
+    from flexkv_amd import _lib
+    from flexkv_amd.c_ext import SSDIOCTX, transfer_kv_blocks_ssd
+    from flexkv_amd.layout import KVCacheLayout, KVCacheLayoutType, TransferStrides
+    L_, H, D, T, KV, ES = 32, 8, 128, 16, 2, 2
+    n_cpu, n_ssd, nfiles = blocks + blocks // 4, 2 * blocks, 4
+    lib = _lib.load()
+    work = tempfile.mkdtemp(prefix="fkv_ssd_bench_", dir=ssd_dir)
+    rng = np.random.default_rng(1)
+    out = {"cases": [], "dir": work}
+    try:
+        for kind in ("BLOCKFIRST", "LAYERFIRST"):
+            cl = KVCacheLayout(KVCacheLayoutType[kind], L_, n_cpu, T, H, D, kv_dim=KV, num_kv_heads=H)
+            fl = KVCacheLayout(KVCacheLayoutType[kind], L_, n_ssd, T, H, D, kv_dim=KV,
+                               num_kv_heads=H).div_block(nfiles, padding=True)
+            c, f = TransferStrides.from_layout(cl, ES), TransferStrides.from_layout(fl, ES)
+            pool_bytes = cl.get_total_elements() * ES
+            if pinned:
+                pool_t = torch.empty(pool_bytes, dtype=torch.uint8, pin_memory=True)
+                pool = pool_t.numpy()
+            else:
+                keep = mmap.mmap(-1, pool_bytes)
+                pool = np.frombuffer(keep, dtype=np.uint8)
+            pool[:] = rng.integers(0, 256, pool_bytes, dtype=np.uint8)
+            paths = {0: [os.path.join(work, f"{kind}_{i}.bin") for i in range(nfiles)]}
+            for p in paths[0]:
+                with open(p, "wb") as fh:
+                    fh.truncate(fl.get_total_elements() * ES)
+            nbytes = blocks * L_ * KV * c.chunk
+            for order in ("contiguous", "scattered"):
+                if order == "contiguous":
+                    ssd_ids, cpu_ids = np.arange(blocks), np.arange(blocks)
+                else:
+                    ssd_ids, cpu_ids = rng.permutation(n_ssd)[:blocks], rng.permutation(n_cpu)[:blocks]
+                s_t, c_t = torch.from_numpy(ssd_ids.astype(np.int64)), torch.from_numpy(cpu_ids.astype(np.int64))
+                for opt in (False, True):
+                    rows = lib.fkv_ssd_plan(1, nfiles, 0, L_, s_t.data_ptr(), c_t.data_ptr(), blocks,
+                                            c.layer, c.kv, f.layer, f.kv, c.chunk, c.block, 1, KV,
+                                            int(opt), None, 0)
+                    buf = np.zeros((rows, 5), dtype=np.int64)
+                    lib.fkv_ssd_plan(1, nfiles, 0, L_, s_t.data_ptr(), c_t.data_ptr(), blocks,
+                                     c.layer, c.kv, f.layer, f.kv, c.chunk, c.block, 1, KV,
+                                     int(opt), buf.ctypes.data_as(ctypes.POINTER(ctypes.c_int64)), rows)
+                    requests = int(buf[:, 0].max()) + 1
+                    for entries in (0, 512):
+                        ctx = SSDIOCTX(paths, 1, entries, 0)
+                        rec = {"layout": kind, "order": order, "ssd_io_opt": opt,
+                               "engine": "io_uring" if ctx.uses_iouring else "threads",
+                               "requests": requests, "iovecs": int(rows)}
+                        for name, is_read in (("write", False), ("read", True)):
+                            times = []
+                            for it in range(warmup + steps):
+                                t0 = time.perf_counter()
+                                transfer_kv_blocks_ssd(
+                                    ctx, torch.arange(0, L_, dtype=torch.int32), pool.ctypes.data,
+                                    s_t, c_t, c.layer, c.kv, f.layer, f.kv, c.chunk, c.block,
+                                    is_read, n_ssd // nfiles, 1, 16, KV, opt)
+                                if it >= warmup:
+                                    times.append(time.perf_counter() - t0)
+                            rec[name + "_GBps"] = round(nbytes / _median(times) / 1e9, 3)
+                        rec["o_direct"] = ctx.last_transfer_was_direct
+                        ctx.close()
+                        out["cases"].append(rec)
+            for p in paths[0]:
+                os.unlink(p)
+            del pool
+        out["bytes_per_direction"] = nbytes
+    finally:
+        shutil.rmtree(work, ignore_errors=True)
+    return out
+
+
 def cpu_baseline(cfg, budget_s=20.0):
     import torch
     from oracle import fkv_oracle as O
@@ -657,7 +738,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker"])
+    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker", "ssd"])
+    ap.add_argument("--ssd-dir", default=None,
+                    help="ssd: directory for the cache files (default: the system temp dir)")
+    ap.add_argument("--ssd-blocks", type=int, default=256,
+                    help="ssd: 2 MiB blocks per transfer")
+    ap.add_argument("--pageable-pool", action="store_true",
+                    help="ssd: page-aligned ordinary memory for the host pool instead of pinned")
     ap.add_argument("--num-cta", type=int, default=4,
                     help="transfer_num_cta (reference default FLEXKV_TRANSFER_NUM_CTA_*=4)")
     ap.add_argument("--use-ce", action="store_true", help="copy-engine path instead of the kernel")
@@ -674,6 +761,21 @@ def main():
 
     import torch
     import flexkv_amd.c_ext as c_ext  # fails loudly if libfkv_hip.so is missing
+    if args.config == "ssd":  # host pool <-> files: no GPU work in this one
+        pinned = torch.cuda.is_available() and not args.pageable_pool
+        r = run_ssd(torch, args.steps, args.warmup, args.ssd_dir, args.ssd_blocks, pinned)
+        best = max(r["cases"], key=lambda x: x["read_GBps"])
+        print(json.dumps({
+            "metric": "host pool <-> SSD files GB/s (best read case)", "unit": "GB/s",
+            "value": best["read_GBps"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
+            "data": "synthetic",
+            "config": {"workload": f"ssd: 32 layers x K+V x 32 KiB chunks (16 tok x 8 heads x 128 "
+                                   f"bf16), {args.ssd_blocks} blocks of 2 MiB per transfer, 1 "
+                                   f"device x 4 files, 16 threads or a 512-entry ring",
+                       "host_pool": "pinned" if pinned else "pageable, page-aligned"},
+            "bytes_per_direction": r["bytes_per_direction"], "cases": r["cases"]}))
+        return
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     device = "cuda:0"
     torch.cuda.set_device(0)

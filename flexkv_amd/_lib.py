@@ -181,6 +181,19 @@ SIGNATURES = {
     "fkv_host_unregister": (c_int32, [c_void_p, c_size_t, c_size_t]),
     "fkv_host_register_plan": (c_int64, [c_size_t, c_size_t, c_void_p, c_void_p, c_int64]),
     "fkv_host_chunk_bytes_from_gb": (c_size_t, [c_double]),
+    "fkv_ssd_open": (c_int32, [POINTER(c_char_p), c_int32, c_int32, c_int32, c_int32,
+                               POINTER(c_void_p)]),
+    "fkv_ssd_close": (None, [c_void_p]),
+    "fkv_ssd_uses_iouring": (c_int32, [c_void_p]),
+    "fkv_ssd_last_direct": (c_int32, [c_void_p]),
+    "fkv_ssd_transfer": (c_int32, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
+                                   c_int32, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                   c_int32, c_int32, c_int32, c_int32, c_int32]),
+    "fkv_ssd_locate": (c_int32, [c_int64, c_int32, c_int32, c_int32, POINTER(c_int32),
+                                 POINTER(c_int32), POINTER(c_int64)]),
+    "fkv_ssd_plan": (c_int64, [c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_int32,
+                               c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int32,
+                               c_int32, c_int32, c_void_p, c_int64]),
     "fkv_ipc_export": (c_int32, [c_void_p, c_void_p, POINTER(c_int64), POINTER(c_int64)]),
     "fkv_ipc_open": (c_int32, [c_void_p, c_int32, POINTER(c_void_p)]),
     "fkv_ipc_close": (c_int32, [c_void_p]),

@@ -28,7 +28,8 @@ from ._lib import (CEConfig, LayerGroup, LayerMember, LayerwiseCall, LayerwiseMG
 
 _L = _lib.load()
 
-__all__ = ["transfer_kv_blocks", "TPTransferThreadGroup", "LayerwiseTransferGroup",
+__all__ = ["transfer_kv_blocks", "transfer_kv_blocks_ssd", "SSDIOCTX", "TPTransferThreadGroup",
+           "LayerwiseTransferGroup",
            "last_transfer_path", "get_stats", "reset_stats"]
 
 
@@ -152,6 +153,88 @@ def get_stats() -> Dict[str, int]:
 
 def reset_stats() -> None:
     _L.fkv_reset_stats()
+
+
+class SSDIOCTX:
+    """Open SSD cache files plus the I/O engine that serves them
+    (``csrc/transfer_ssd.h:244-309``, ``csrc/bindings.cpp:785-787``).
+
+    ``ssd_files`` maps device index -> list of file paths (every device the same
+    number of files).  ``iouring_entries > 0`` asks for io_uring; when the kernel
+    refuses it the context falls back to threads (``uses_iouring`` tells which).
+    """
+
+    def __init__(self, ssd_files: Dict[int, List[str]], num_devices: int, iouring_entries: int,
+                 iouring_flags: int) -> None:
+        self._h = ctypes.c_void_p()
+        if num_devices < 1 or any(d not in ssd_files for d in range(num_devices)):
+            raise RuntimeError("ssd_files must hold a path list for devices 0..num_devices-1")
+        per_device = len(ssd_files[0])
+        if per_device < 1 or any(len(ssd_files[d]) != per_device for d in range(num_devices)):
+            raise RuntimeError("every SSD device must bring the same, non-zero number of files")
+        flat = [str(p).encode() for d in range(num_devices) for p in ssd_files[d]]
+        arr = (ctypes.c_char_p * len(flat))(*flat)
+        self.num_devices, self.num_files_per_device = int(num_devices), per_device
+        check(_L.fkv_ssd_open(arr, int(num_devices), per_device, int(iouring_entries),
+                              int(iouring_flags), ctypes.byref(self._h)))
+
+    @property
+    def uses_iouring(self) -> bool:
+        return bool(_L.fkv_ssd_uses_iouring(self._h))
+
+    @property
+    def last_transfer_was_direct(self) -> bool:
+        """Whether the last transfer bypassed the page cache (O_DIRECT)."""
+        return bool(_L.fkv_ssd_last_direct(self._h))
+
+    def get_num_devices(self) -> int:
+        return self.num_devices
+
+    def get_num_files_per_device(self) -> int:
+        return self.num_files_per_device
+
+    def close(self) -> None:
+        if getattr(self, "_h", None) is not None and self._h.value:
+            _L.fkv_ssd_close(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self) -> None:
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def transfer_kv_blocks_ssd(
+        ioctx: SSDIOCTX, cpu_layer_id_list: torch.Tensor, cpu_tensor_ptr: int,
+        ssd_block_ids: torch.Tensor, cpu_block_ids: torch.Tensor,
+        cpu_layer_stride_in_bytes: int, cpu_kv_stride_in_bytes: int,
+        ssd_layer_stride_in_bytes: int, ssd_kv_stride_in_bytes: int, chunk_size_in_bytes: int,
+        block_stride_in_bytes: int, is_read: bool, num_blocks_per_file: int,
+        round_robin: int = 1, num_threads_per_device: int = 16, kv_dim: int = 2,
+        ssd_io_opt: bool = True) -> None:
+    """Move KV blocks between the host pool and SSD files
+    (``csrc/bindings.cpp:460-470``, ``csrc/transfer_ssd.cpp:327-512``).
+
+    ``cpu_layer_id_list`` is an int32 tensor of consecutive layer ids; like the
+    reference, the call covers ``[list[0], list[0] + len(list))``.  Blocks until
+    the bytes have moved.  ``num_blocks_per_file`` is accepted for signature
+    compatibility (the reference does not read it either).
+    """
+    ssd_ids = _ids(ssd_block_ids, "ssd_block_ids")
+    cpu_ids = _ids(cpu_block_ids, "cpu_block_ids")
+    if ssd_ids.numel() != cpu_ids.numel():
+        raise ValueError("ssd_block_ids and cpu_block_ids differ in length")
+    if cpu_layer_id_list.dtype != torch.int32:
+        raise TypeError("cpu_layer_id_list must be int32")
+    n_layers = int(cpu_layer_id_list.numel())
+    start = int(cpu_layer_id_list[0]) if n_layers else 0
+    check(_L.fkv_ssd_transfer(
+        ioctx._h, start, n_layers, int(cpu_tensor_ptr), ssd_ids.data_ptr(), cpu_ids.data_ptr(),
+        ssd_ids.numel(), int(cpu_layer_stride_in_bytes), int(cpu_kv_stride_in_bytes),
+        int(ssd_layer_stride_in_bytes), int(ssd_kv_stride_in_bytes), int(chunk_size_in_bytes),
+        int(block_stride_in_bytes), int(bool(is_read)), int(round_robin),
+        int(num_threads_per_device), int(kv_dim), int(bool(ssd_io_opt))))
 
 
 def _i64_array(values: Sequence[int], name: str, expect: Optional[int] = None) -> np.ndarray:
@@ -335,8 +418,11 @@ class LayerwiseTransferGroup:
     pybind does, by their argument names: the single-group form
     (``gpu_blocks``, ``num_layers``, ``gpu_*_strides_tensor``) and the
     multi-group form (``gpu_blocks_per_group``, ``num_original_layers``,
-    ``layer_members``, ``group_*``).  SSD pre-load is not part of this library:
-    non-empty ``ssd_files`` / ``swa_ssd_files`` raise ``RuntimeError``.
+    ``layer_members``, ``group_*``).  With ``ssd_files`` / ``swa_ssd_files`` the
+    group also performs the reference's step 0: blocks named by ``ssd_block_ids`` /
+    ``swa_disk2h_src`` are read from the SSD files into the host pool, all layers
+    at once, before the first layer goes to the GPU (``csrc/layerwise.cpp:1060-1110,
+    1371-1432``).
     """
 
     _MULTI_NAMES = ("num_gpus", "gpu_blocks_per_group", "cpu_blocks", "ssd_files",
@@ -388,12 +474,20 @@ class LayerwiseTransferGroup:
         missing = [k for k in required if k not in a]
         if missing:
             raise TypeError(f"LayerwiseTransferGroup missing arguments: {missing}")
+        self._ssd_io_opt = bool(a["ssd_io_opt"])
+        self._ioctx = self._swa_ioctx = None
         if a["ssd_files"]:
-            raise RuntimeError("SSD->CPU pre-load is not part of this library "
-                               "(ssd_files must be empty)")
+            self._ioctx = SSDIOCTX(a["ssd_files"], len(a["ssd_files"]), a["iouring_entries"],
+                                   a["iouring_flags"])
         if a["swa_ssd_files"]:
-            raise RuntimeError("SSD->CPU pre-load is not part of this library "
-                               "(swa_ssd_files must be empty)")
+            self._swa_ioctx = SSDIOCTX(a["swa_ssd_files"], len(a["swa_ssd_files"]),
+                                       a["iouring_entries"], a["iouring_flags"])
+        self._cpu_ptr = a["cpu_blocks"].data_ptr()
+        self._swa_cpu_ptr = (a["swa_cpu_blocks"].data_ptr()
+                             if a["swa_cpu_blocks"] is not None and a["swa_cpu_blocks"].numel()
+                             else 0)
+        self._opaque_block_stride = (int(a["group_cpu_block_strides"][0]) if multi else 0)
+        self._swa_opaque_block_stride = 0
         ce = _ce_config(a["ce_segment_threshold"], a["ce_path_opt"], a["ce_force_path"],
                         a["ce_enable_memcpy2d"], a["is_blockfirst"], a["num_kv_heads"],
                         a["ce_gather_threads"], a["ce_gather_nt"])
@@ -508,9 +602,6 @@ class LayerwiseTransferGroup:
             iouring_flags: int = 0) -> None:
         """Attach a sidecar made of its own layer groups
         (``csrc/layerwise.cpp:355-429``, ``csrc/bindings.cpp:632-656``)."""
-        if swa_ssd_files:
-            raise RuntimeError("SSD->CPU pre-load is not part of this library "
-                               "(swa_ssd_files must be empty)")
         if swa_cpu_blocks is None or swa_cpu_blocks.numel() == 0:
             raise RuntimeError("[LayerwiseTransferGroup] init_swa_multi_group() requires "
                                "non-empty swa_cpu_blocks")
@@ -530,13 +621,23 @@ class LayerwiseTransferGroup:
             self._h, groups.array, groups.count, offsets.ctypes.data, members,
             swa_cpu_blocks.data_ptr()))
         self._keepalive.append((swa_gpu_blocks_per_group, swa_cpu_blocks))
+        self._swa_cpu_ptr = swa_cpu_blocks.data_ptr()
+        self._swa_opaque_block_stride = int(swa_group_cpu_block_strides[0])
+        if swa_ssd_files:
+            self._swa_ioctx = SSDIOCTX(swa_ssd_files, len(swa_ssd_files), iouring_entries,
+                                       iouring_flags)
+
+    @staticmethod
+    def _opaque_blocks_from_ssd(ioctx, cpu_ptr, ssd_ids, cpu_ids, block_stride, num_blocks_per_file,
+                                round_robin, threads, kv_dim, opt) -> None:
+        """Multi-group pools hold byte-flat blocks of identical layout in the host pool
+        and on disk: a block moves as one piece (csrc/layerwise.cpp:1373-1397)."""
+        transfer_kv_blocks_ssd(ioctx, torch.zeros(1, dtype=torch.int32), cpu_ptr, ssd_ids, cpu_ids,
+                               block_stride, 0, block_stride, 0, block_stride, block_stride, True,
+                               num_blocks_per_file, round_robin, threads, kv_dim, opt)
 
     def _run(self, call: LayerwiseCall, gpu_block_id_tensor, cpu_block_id_tensor, swa_h2d_src,
-             swa_h2d_dst, ssd_block_ids, swa_disk2h_src, notify_mode: str) -> None:
-        if ssd_block_ids is not None and _numel(ssd_block_ids) > 0:
-            raise RuntimeError("SSD->CPU pre-load is not part of this library")
-        if swa_disk2h_src is not None and _numel(swa_disk2h_src) > 0:
-            raise RuntimeError("SSD->CPU pre-load is not part of this library (swa_disk2h_src)")
+             swa_h2d_dst, notify_mode: str) -> None:
         gpu_ids = _ids(gpu_block_id_tensor, "gpu_block_id_tensor")
         cpu_ids = _ids(cpu_block_id_tensor, "cpu_block_id_tensor")
         if gpu_ids.numel() != cpu_ids.numel():
@@ -586,8 +687,39 @@ class LayerwiseTransferGroup:
         c.swa_h2d_cpu_kv_stride = int(swa_h2d_cpu_kv_stride_in_bytes)
         c.swa_h2d_cpu_layer_stride = int(swa_h2d_cpu_layer_stride_in_bytes)
         c.swa_cpu_block_stride = int(swa_cpu_block_stride_in_bytes)
+        # step 0a / 0b: SSD -> host pool, csrc/layerwise.cpp:1371-1432
+        if self._ioctx is not None and ssd_block_ids is not None and _numel(ssd_block_ids) > 0:
+            self._opaque_blocks_from_ssd(self._ioctx, self._cpu_ptr, ssd_block_ids,
+                                         cpu_block_ids_d2h, self._opaque_block_stride,
+                                         num_blocks_per_file, round_robin, num_threads_per_device,
+                                         int(kv_dim), self._ssd_io_opt)
+        if self._swa_ioctx is not None and swa_disk2h_src is not None \
+                and _numel(swa_disk2h_src) > 0:
+            if self._swa_opaque_block_stride:
+                self._opaque_blocks_from_ssd(self._swa_ioctx, self._swa_cpu_ptr, swa_disk2h_src,
+                                             swa_disk2h_dst, self._swa_opaque_block_stride,
+                                             swa_num_blocks_per_file, round_robin,
+                                             num_threads_per_device, 1, self._ssd_io_opt)
+            else:
+                self._uniform_swa_from_ssd(
+                    swa_disk2h_src, swa_disk2h_dst, swa_cpu_layer_stride_in_bytes,
+                    swa_cpu_kv_stride_in_bytes, swa_ssd_layer_stride_in_bytes,
+                    swa_ssd_kv_stride_in_bytes, swa_cpu_chunk_size_in_bytes,
+                    swa_cpu_block_stride_in_bytes, swa_num_blocks_per_file, round_robin,
+                    num_threads_per_device)
         self._run(c, gpu_block_id_tensor, cpu_block_id_tensor, swa_h2d_src, swa_h2d_dst,
-                  ssd_block_ids, swa_disk2h_src, notify_mode)
+                  notify_mode)
+
+    def _uniform_swa_from_ssd(self, src, dst, cpu_layer_stride, cpu_kv_stride, ssd_layer_stride,
+                              ssd_kv_stride, chunk, block_stride, num_blocks_per_file, round_robin,
+                              threads) -> None:
+        """All layers of the uniform sidecar in one call (csrc/layerwise.cpp:1098-1110,
+        1412-1430)."""
+        transfer_kv_blocks_ssd(
+            self._swa_ioctx, torch.arange(0, self._num_layers, dtype=torch.int32),
+            self._swa_cpu_ptr, src, dst, cpu_layer_stride, cpu_kv_stride, ssd_layer_stride,
+            ssd_kv_stride, chunk, block_stride, True, num_blocks_per_file, round_robin, threads, 1,
+            self._ssd_io_opt)
 
     def layerwise_transfer(
             self, ssd_block_ids, cpu_block_ids_d2h, ssd_layer_stride_in_bytes: int,
@@ -627,8 +759,24 @@ class LayerwiseTransferGroup:
         c.swa_h2d_cpu_kv_stride = int(swa_h2d_cpu_kv_stride_in_bytes)
         c.swa_h2d_cpu_layer_stride = int(swa_h2d_cpu_layer_stride_in_bytes)
         c.swa_cpu_block_stride = int(swa_cpu_block_stride_in_bytes)
+        # step 0: SSD -> host pool for all layers at once, csrc/layerwise.cpp:1060-1110
+        if self._ioctx is not None and ssd_block_ids is not None and _numel(ssd_block_ids) > 0:
+            transfer_kv_blocks_ssd(
+                self._ioctx, torch.arange(0, int(num_layers), dtype=torch.int32), self._cpu_ptr,
+                ssd_block_ids, cpu_block_ids_d2h, cpu_layer_stride_in_bytes,
+                cpu_kv_stride_in_bytes, ssd_layer_stride_in_bytes, ssd_kv_stride_in_bytes,
+                cpu_chunk_size_in_bytes, cpu_block_stride_in_bytes, True, num_blocks_per_file,
+                round_robin, num_threads_per_device, int(kv_dim), self._ssd_io_opt)
+        if self._swa_ioctx is not None and swa_disk2h_src is not None \
+                and _numel(swa_disk2h_src) > 0:
+            self._uniform_swa_from_ssd(
+                swa_disk2h_src, swa_disk2h_dst, swa_cpu_layer_stride_in_bytes,
+                swa_cpu_kv_stride_in_bytes, swa_ssd_layer_stride_in_bytes,
+                swa_ssd_kv_stride_in_bytes, swa_cpu_chunk_size_in_bytes,
+                swa_cpu_block_stride_in_bytes, swa_num_blocks_per_file, round_robin,
+                num_threads_per_device)
         self._run(c, gpu_block_id_tensor, cpu_block_id_tensor, swa_h2d_src, swa_h2d_dst,
-                  ssd_block_ids, swa_disk2h_src, notify_mode)
+                  notify_mode)
 
     # ---- additions for consumers in the same process -------------------------
     def wait_layer(self, layer: int, stream: Optional["torch.cuda.Stream"] = None,

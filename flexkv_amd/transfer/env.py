@@ -21,6 +21,9 @@ class TransferEnv:
     kv_shared_across_ranks_mode: str
     layerwise_notify_mode: str
     worker_shutdown_timeout_s: float
+    ssd_io_opt: bool
+    iouring_entries: int
+    iouring_flags: int
 
     @classmethod
     def from_env(cls) -> "TransferEnv":
@@ -39,6 +42,9 @@ class TransferEnv:
             kv_shared_across_ranks_mode=g("FLEXKV_KV_SHARED_ACROSS_RANKS_MODE", "sharded"),
             layerwise_notify_mode=g("FLEXKV_LAYERWISE_NOTIFY_MODE", "hostfunc"),
             worker_shutdown_timeout_s=float(g("FLEXKV_WORKER_SHUTDOWN_TIMEOUT_S", 600)),
+            ssd_io_opt=bool(int(g("FLEXKV_SSD_IO_OPT", 1))),
+            iouring_entries=int(g("FLEXKV_IOURING_ENTRIES", 512)),
+            iouring_flags=int(g("FLEXKV_IOURING_FLAGS", 0)),
         )
 
 

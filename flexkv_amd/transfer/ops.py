@@ -18,6 +18,8 @@ import numpy as np
 class TransferType(Enum):
     H2D = "H2D"
     D2H = "D2H"
+    DISK2H = "DISK2H"
+    H2DISK = "H2DISK"
     VIRTUAL = "Virtual"
     LAYERWISE = "LAYERWISE"
 

@@ -11,8 +11,8 @@ Contract and names follow ``flexkv/transfer/worker.py`` of the reference
 (``TransferWorkerBase`` :120-633, ``WorkerHandle`` :635-707,
 ``GPUCPUTransferWorker`` :709-1097, ``tpGPUCPUTransferWorker`` :1098-1520) and
 ``flexkv/transfer/layerwise.py`` (``LayerwiseTransferWorker`` :69-1059).  What a
-worker of this library does *not* do: compression, SSD / remote tiers, GPU
-memory re-mapping controls.
+worker of this library does *not* do: compression, remote tiers, GPU memory
+re-mapping controls.
 
 Host pools.  A worker either receives the pool as a shared-memory tensor and
 registers it with the runtime (the reference's way), or receives a
@@ -646,6 +646,93 @@ class tpGPUCPUTransferWorker(TransferWorkerBase):  # noqa: N801 - the reference'
         return True
 
 
+class CPUSSDDiskTransferWorker(TransferWorkerBase):
+    """Host pool <-> SSD files (worker.py:1522-1722): H2DISK and DISK2H ops, no GPU
+    involved.  The files of ``ssd_files`` (device -> paths) together hold
+    ``ssd_kv_layout.num_block`` blocks, striped over devices and files."""
+
+    def __init__(self, worker_id: int, transfer_conn: Connection, finished_ops_queue,
+                 op_buffer_tensor: torch.Tensor, cpu_blocks: torch.Tensor,
+                 ssd_files: Dict[int, List[str]],
+                 cpu_kv_layout: Union[KVCacheLayout, MultiGroupBlockLayout],
+                 ssd_kv_layout: Union[KVCacheLayout, MultiGroupBlockLayout], dtype: torch.dtype,
+                 num_blocks_per_file: int, layer_groups: Optional[List[LayerGroupSpec]] = None,
+                 num_threads_per_device: int = 32) -> None:
+        from ..c_ext import SSDIOCTX
+        super().__init__(worker_id, transfer_conn, finished_ops_queue, op_buffer_tensor)
+        self.cpu_blocks = materialize_worker_tensor(cpu_blocks)
+        self.ssd_files = ssd_files
+        self.num_blocks_per_file = num_blocks_per_file
+        self.num_files = sum(len(v) for v in ssd_files.values())
+        self.round_robin = 1
+        self.num_threads_per_device = num_threads_per_device
+        self.dtype = dtype
+        self.has_multi_group = layer_groups is not None
+        if self.has_multi_group:
+            # identical byte-flat blocks on both sides: a block moves as one piece
+            self.block_stride_in_bytes = cpu_kv_layout.get_block_stride()
+            self.kv_dim, self.num_layers = 1, 1
+            self._bytes_per_block = self.block_stride_in_bytes
+        else:
+            if cpu_kv_layout.type != ssd_kv_layout.type:
+                raise ValueError("no support for different CPU and SSD KV cache layout type")
+            self.kv_dim = cpu_kv_layout.kv_dim
+            self.num_layers = cpu_kv_layout.num_layer
+            per_file = ssd_kv_layout.div_block(self.num_files, padding=True)
+            c = TransferStrides.from_layout(cpu_kv_layout, dtype.itemsize)
+            f = TransferStrides.from_layout(per_file, dtype.itemsize)
+            self.chunk_size_in_bytes = c.chunk
+            self.block_stride_in_bytes = c.block
+            self.cpu_kv_stride_in_bytes, self.cpu_layer_stride_in_bytes = c.kv, c.layer
+            self.ssd_kv_stride_in_bytes, self.ssd_layer_stride_in_bytes = f.kv, f.layer
+            self._bytes_per_block = c.chunk * self.num_layers * self.kv_dim
+        env = global_env()
+        try:
+            self.ioctx = SSDIOCTX(ssd_files, len(ssd_files), env.iouring_entries, env.iouring_flags)
+        except Exception as e:
+            logger.error("Error setting ssd ioctx: %s", e)
+            raise RuntimeError("SSD Worker init failed") from e
+
+    def _transfer_impl(self, src_block_ids: torch.Tensor, dst_block_ids: torch.Tensor,
+                       transfer_type: TransferType) -> None:
+        from ..c_ext import transfer_kv_blocks_ssd
+        if transfer_type == TransferType.H2DISK:
+            ssd_ids, cpu_ids, is_read = dst_block_ids, src_block_ids, False
+        elif transfer_type == TransferType.DISK2H:
+            ssd_ids, cpu_ids, is_read = src_block_ids, dst_block_ids, True
+        else:
+            raise ValueError(f"Invalid transfer type: {transfer_type} for "
+                             "CPUSSDDiskTransferWorker")
+        opt = global_env().ssd_io_opt
+        base = self.cpu_blocks.data_ptr()
+        if self.has_multi_group:
+            b = self.block_stride_in_bytes
+            transfer_kv_blocks_ssd(self.ioctx, torch.zeros(1, dtype=torch.int32), base, ssd_ids,
+                                   cpu_ids, b, 0, b, 0, b, b, is_read, self.num_blocks_per_file,
+                                   self.round_robin, self.num_threads_per_device, 1, opt)
+            return
+        transfer_kv_blocks_ssd(
+            self.ioctx, torch.arange(0, self.num_layers, dtype=torch.int32), base, ssd_ids,
+            cpu_ids, self.cpu_layer_stride_in_bytes, self.cpu_kv_stride_in_bytes,
+            self.ssd_layer_stride_in_bytes, self.ssd_kv_stride_in_bytes, self.chunk_size_in_bytes,
+            self.block_stride_in_bytes, is_read, self.num_blocks_per_file, self.round_robin,
+            self.num_threads_per_device, self.kv_dim, opt)
+
+    def launch_transfer(self, transfer_op: WorkerTransferOp) -> bool:
+        src, dst = self.get_transfer_block_ids(transfer_op)
+        t0 = time.time()
+        self._transfer_impl(src.contiguous(), dst.contiguous(), transfer_op.transfer_type)
+        self._log_transfer_performance(
+            transfer_op, self._bytes_per_block * transfer_op.valid_block_num, t0, time.time())
+        return True
+
+    def shutdown(self) -> None:
+        ctx = getattr(self, "ioctx", None)
+        if ctx is not None:
+            ctx.close()
+        super().shutdown()
+
+
 class LayerwiseTransferWorker(TransferWorkerBase):
     """Layer-by-layer restore for an engine that starts attention on layer L while
     layer L+1 is still on the link (layerwise.py:69-1059).  The engine's per-layer
@@ -669,7 +756,13 @@ class LayerwiseTransferWorker(TransferWorkerBase):
                  swa_cpu_kv_layout: Optional[KVCacheLayout] = None,
                  swa_dtype: Optional[torch.dtype] = None,
                  eventfd_deadline_s: float = 180.0,
-                 allow_pageable_host: Optional[bool] = None) -> None:
+                 allow_pageable_host: Optional[bool] = None,
+                 ssd_files: Optional[Dict[int, List[str]]] = None,
+                 ssd_kv_layout: Optional[Union[KVCacheLayout, MultiGroupBlockLayout]] = None,
+                 num_blocks_per_file: int = 0,
+                 swa_ssd_files: Optional[Dict[int, List[str]]] = None,
+                 swa_ssd_kv_layout: Optional[KVCacheLayout] = None,
+                 swa_num_blocks_per_file: int = 0) -> None:
         from .eventfd_channel import receive_layer_eventfds
         super().__init__(worker_id, transfer_conn, finished_ops_queue, op_buffer_tensor)
         assert len(gpu_blocks) == tp_group_size, \
@@ -703,6 +796,14 @@ class LayerwiseTransferWorker(TransferWorkerBase):
         self.h2d_cta_num = h2d_cta_num
         self.kv_shared_across_ranks_mode = env.kv_shared_across_ranks_mode
         self.layerwise_notify_mode = env.layerwise_notify_mode
+        self.ssd_files = ssd_files or {}
+        self.enable_ssd = len(self.ssd_files) > 0
+        self.num_blocks_per_file = num_blocks_per_file if self.enable_ssd else 0
+        self.round_robin = 1
+        self.swa_ssd_files = swa_ssd_files or {}
+        self._swa_num_blocks_per_file = swa_num_blocks_per_file
+        self.ssd_layer_stride_in_bytes = self.ssd_kv_stride_in_bytes = 0
+        self.swa_ssd = None
         swa_kwargs: Dict[str, Any] = {"has_swa": False}
         if self.has_swa:
             self.swa_gpu_blocks = [import_tensor_handles(h) for h in swa_gpu_blocks]
@@ -715,14 +816,19 @@ class LayerwiseTransferWorker(TransferWorkerBase):
             per_gpu = [TransferStrides.from_layout(l, isz) for l in swa_gpu_kv_layouts]
             self.swa_cpu = TransferStrides.from_layout(swa_cpu_kv_layout, isz)
             i64 = lambda xs: torch.tensor(list(xs), dtype=torch.int64)  # noqa: E731
+            if self.swa_ssd_files:
+                files = sum(len(v) for v in self.swa_ssd_files.values())
+                self.swa_ssd = TransferStrides.from_layout(
+                    swa_ssd_kv_layout.div_block(files, padding=True), isz)
             swa_kwargs = dict(
                 has_swa=True, swa_gpu_blocks=self.swa_gpu_blocks,
-                swa_cpu_blocks=self.swa_cpu_blocks, swa_ssd_files={},
+                swa_cpu_blocks=self.swa_cpu_blocks, swa_ssd_files=self.swa_ssd_files,
                 swa_gpu_kv_strides_tensor=i64(s.kv for s in per_gpu),
                 swa_gpu_block_strides_tensor=i64(s.block for s in per_gpu),
                 swa_gpu_layer_strides_tensor=i64(s.layer for s in per_gpu),
                 swa_gpu_chunk_sizes_tensor=i64(s.chunk for s in per_gpu))
-        common = dict(iouring_entries=0, iouring_flags=0, layer_eventfds_tensor=fds,
+        common = dict(iouring_entries=env.iouring_entries, iouring_flags=env.iouring_flags,
+                      ssd_io_opt=env.ssd_io_opt, layer_eventfds_tensor=fds,
                       tp_size=tp_group_size, ce_segment_threshold=env.ce_segment_threshold,
                       ce_path_opt=env.ce_path_opt, ce_enable_memcpy2d=env.enable_ce_memcpy2d,
                       num_kv_heads=self.num_kv_heads, ce_gather_threads=env.ce_gather_threads,
@@ -736,7 +842,8 @@ class LayerwiseTransferWorker(TransferWorkerBase):
             self.group_cpu_block_stride = tables["cpu_block_stride"]
             self.layerwise_transfer_group = LayerwiseTransferGroup(
                 num_gpus=self.num_gpus, gpu_blocks_per_group=self._group_tensors,
-                cpu_blocks=self.cpu_blocks, ssd_files={}, num_original_layers=self.num_layers,
+                cpu_blocks=self.cpu_blocks, ssd_files=self.ssd_files,
+                num_original_layers=self.num_layers,
                 layer_members=tables["layer_members"], is_blockfirst=True,
                 **{k: v for k, v in tables.items() if k.startswith("group_")}, **common)
             self._bytes_per_block = self.group_cpu_block_stride
@@ -754,10 +861,14 @@ class LayerwiseTransferWorker(TransferWorkerBase):
         self.cpu_tp_stride_in_bytes = c.block // tp_group_size
         self.h2d_cpu_kv_stride_in_bytes = rank_layout.get_kv_stride() * sz
         self.h2d_cpu_layer_stride_in_bytes = rank_layout.get_layer_stride() * sz
+        if self.enable_ssd:  # the files split the block axis, layerwise.py:630-638
+            files = sum(len(v) for v in self.ssd_files.values())
+            f = TransferStrides.from_layout(ssd_kv_layout.div_block(files, padding=True), sz)
+            self.ssd_layer_stride_in_bytes, self.ssd_kv_stride_in_bytes = f.layer, f.kv
         i64 = lambda xs: torch.tensor(list(xs), dtype=torch.int64)  # noqa: E731
         self.layerwise_transfer_group = LayerwiseTransferGroup(
             num_gpus=self.num_gpus, gpu_blocks=self.gpu_blocks, cpu_blocks=self.cpu_blocks,
-            ssd_files={}, num_layers=self.num_layers,
+            ssd_files=self.ssd_files, num_layers=self.num_layers,
             gpu_kv_strides_tensor=i64(s.kv for s in per_gpu),
             gpu_block_strides_tensor=i64(s.block for s in per_gpu),
             gpu_layer_strides_tensor=i64(s.layer for s in per_gpu),
@@ -765,47 +876,67 @@ class LayerwiseTransferWorker(TransferWorkerBase):
             **common)
         self._bytes_per_block = c.chunk * self.num_layers * self.kv_dim
 
-    def _swa_call_kwargs(self, src: Optional[torch.Tensor], dst: Optional[torch.Tensor]) -> dict:
-        if not self.has_swa or src is None or src.numel() == 0:
+    def _swa_call_kwargs(self, src: Optional[torch.Tensor], dst: Optional[torch.Tensor],
+                         disk_src: Optional[torch.Tensor] = None,
+                         disk_dst: Optional[torch.Tensor] = None) -> dict:
+        if not self.has_swa or ((src is None or src.numel() == 0) and disk_src is None):
             return {}
         c = self.swa_cpu
-        return dict(swa_h2d_src=src, swa_h2d_dst=dst, swa_cpu_kv_stride_in_bytes=c.kv,
+        empty = torch.empty(0, dtype=torch.int64)
+        src = empty if src is None else src
+        dst = empty if dst is None else dst
+        extra = {}
+        if disk_src is not None and self.swa_ssd is not None:
+            extra = dict(swa_disk2h_src=disk_src, swa_disk2h_dst=disk_dst,
+                         swa_ssd_layer_stride_in_bytes=self.swa_ssd.layer,
+                         swa_ssd_kv_stride_in_bytes=self.swa_ssd.kv,
+                         swa_num_blocks_per_file=self._swa_num_blocks_per_file)
+        return dict(**extra, swa_h2d_src=src, swa_h2d_dst=dst, swa_cpu_kv_stride_in_bytes=c.kv,
                     swa_cpu_layer_stride_in_bytes=c.layer, swa_cpu_block_stride_in_bytes=c.block,
                     swa_cpu_chunk_size_in_bytes=c.chunk, swa_h2d_cpu_kv_stride_in_bytes=c.kv,
                     swa_h2d_cpu_layer_stride_in_bytes=c.layer,
                     swa_cpu_tp_stride_in_bytes=c.block // self.tp_group_size)
 
     def _transfer_impl(self, src_h2d: torch.Tensor, dst_h2d: torch.Tensor, counter_id: int,
-                       swa_src: Optional[torch.Tensor], swa_dst: Optional[torch.Tensor]) -> None:
+                       swa_src: Optional[torch.Tensor], swa_dst: Optional[torch.Tensor],
+                       disk_src: Optional[torch.Tensor] = None,
+                       disk_dst: Optional[torch.Tensor] = None,
+                       swa_disk_src: Optional[torch.Tensor] = None,
+                       swa_disk_dst: Optional[torch.Tensor] = None) -> None:
         if swa_src is not None and swa_src.numel() > 0:
             assert self.has_swa, "SWA block ids given but the worker has no SWA pool"
             assert len(swa_src) == len(swa_dst)
         empty = torch.empty(0, dtype=torch.int64)
+        if disk_src is not None and not self.enable_ssd:
+            raise RuntimeError("disk2h block ids given but the worker has no SSD files")
+        ssd_ids = disk_src if disk_src is not None else empty
+        ssd_dst = disk_dst if disk_dst is not None else empty
         use_ce = self._engine(self.use_ce_transfer_h2d)
         tail = dict(counter_id=counter_id,
                     kv_shared_across_ranks_mode=self.kv_shared_across_ranks_mode,
                     notify_mode=self.layerwise_notify_mode,
                     enable_trace=global_env().enable_transfer_trace,
-                    **self._swa_call_kwargs(swa_src, swa_dst))
+                    **self._swa_call_kwargs(swa_src, swa_dst, swa_disk_src, swa_disk_dst))
         if self.has_multi_group:
             self.layerwise_transfer_group.layerwise_transfer_multi_group(
-                ssd_block_ids=empty, cpu_block_ids_d2h=empty, num_blocks_per_file=0,
-                round_robin=1, num_threads_per_device=32, gpu_block_id_tensor=dst_h2d,
+                ssd_block_ids=ssd_ids, cpu_block_ids_d2h=ssd_dst,
+                num_blocks_per_file=self.num_blocks_per_file,
+                round_robin=self.round_robin, num_threads_per_device=32,
+                gpu_block_id_tensor=dst_h2d,
                 cpu_block_id_tensor=src_h2d, transfer_cta_num=self.h2d_cta_num,
                 use_ce_transfer=use_ce, kv_dim=self.kv_dim, num_kv_heads=self.num_kv_heads, **tail)
             return
         # one layer per batch: the protocol posts one eventfd per layer
         self.layerwise_transfer_group.layerwise_transfer(
-            empty, empty, 0, 0, 0, 1, 32, dst_h2d, src_h2d, self.cpu_kv_stride_in_bytes,
+            ssd_ids, ssd_dst, self.ssd_layer_stride_in_bytes, self.ssd_kv_stride_in_bytes,
+            self.num_blocks_per_file, self.round_robin, 32, dst_h2d, src_h2d,
+            self.cpu_kv_stride_in_bytes,
             self.cpu_layer_stride_in_bytes, self.cpu_block_stride_in_bytes,
             self.cpu_chunk_size_in_bytes, self.h2d_cpu_kv_stride_in_bytes,
             self.h2d_cpu_layer_stride_in_bytes, self.cpu_tp_stride_in_bytes, self.h2d_cta_num,
             use_ce, self.num_layers, 1, self.kv_dim, self.num_kv_heads, **tail)
 
     def launch_transfer(self, transfer_op: WorkerLayerwiseTransferOp) -> bool:
-        if transfer_op.src_block_ids_disk2h.size or transfer_op.swa_src_block_ids_disk2h.size:
-            raise RuntimeError("SSD->CPU pre-load is not part of this worker")
-
         def ids(a: np.ndarray) -> Optional[torch.Tensor]:
             return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int64)) if a.size else None
 
@@ -814,7 +945,11 @@ class LayerwiseTransferWorker(TransferWorkerBase):
         t0 = time.time()
         self._transfer_impl(src, dst, transfer_op.counter_id,
                             ids(transfer_op.swa_src_block_ids_h2d),
-                            ids(transfer_op.swa_dst_block_ids_h2d))
+                            ids(transfer_op.swa_dst_block_ids_h2d),
+                            ids(transfer_op.src_block_ids_disk2h),
+                            ids(transfer_op.dst_block_ids_disk2h),
+                            ids(transfer_op.swa_src_block_ids_disk2h),
+                            ids(transfer_op.swa_dst_block_ids_disk2h))
         t1 = time.time()
         if self.has_multi_group:
             size = self.group_cpu_block_stride * len(src)

@@ -408,6 +408,52 @@ int64_t fkv_host_register_plan(size_t bytes, size_t chunk_bytes, size_t *offsets
 /* FLEXKV_CUDAHOST_CHUNK_SIZE_GB -> chunk bytes, host_buffer.py:57-63. */
 size_t fkv_host_chunk_bytes_from_gb(double chunk_gb);
 
+/* ---- host pool <-> SSD files: csrc/transfer_ssd.h:215-333,
+ *      csrc/transfer_ssd.cpp:327-512 ---- */
+
+typedef struct fkv_ssd_ctx fkv_ssd_ctx;
+
+/* SSDIOCTX (csrc/transfer_ssd.h:244-309): opens every file buffered and, where
+ * the file system allows, with O_DIRECT.  `paths` is device-major,
+ * num_devices * files_per_device entries.  iouring_entries > 0 asks for the
+ * io_uring engine (falls back to threads when the kernel refuses it). */
+int fkv_ssd_open(const char *const *paths, int32_t num_devices, int32_t files_per_device,
+                 int32_t iouring_entries, int32_t iouring_flags, fkv_ssd_ctx **out);
+void fkv_ssd_close(fkv_ssd_ctx *ctx);
+/* 1 when the context drives an io_uring, 0 when it uses threads. */
+int fkv_ssd_uses_iouring(const fkv_ssd_ctx *ctx);
+/* 1 when the context's last transfer went through O_DIRECT descriptors (aligned
+ * call, file system with O_DIRECT, host memory the kernel can pin), 0 when it
+ * went through the page cache.  A request refused with EFAULT/EINVAL on the
+ * O_DIRECT descriptor is repeated buffered, and later calls on that host pool
+ * start buffered.  No counterpart in the reference, which fails such a call. */
+int fkv_ssd_last_direct(const fkv_ssd_ctx *ctx);
+/* transfer_kv_blocks_ssd (csrc/transfer_ssd.cpp:327-512) for layers
+ * [start_layer, start_layer + num_layers).  Blocks until all bytes have moved.
+ * `block_stride` applies to the host pool and to the files alike. */
+int fkv_ssd_transfer(fkv_ssd_ctx *ctx, int32_t start_layer, int32_t num_layers, void *cpu_ptr,
+                     const int64_t *ssd_block_ids, const int64_t *cpu_block_ids,
+                     int32_t num_blocks, int64_t cpu_layer_stride, int64_t cpu_kv_stride,
+                     int64_t ssd_layer_stride, int64_t ssd_kv_stride, int64_t chunk_size,
+                     int64_t block_stride, int32_t is_read, int32_t round_robin,
+                     int32_t num_threads_per_device, int32_t kv_dim, int32_t ssd_io_opt);
+/* (device, file, block inside the file) of an SSD block id --
+ * partition_and_remap_blocks_by_device, csrc/transfer_ssd.cpp:22-44, and the
+ * file split at :65-67. */
+int fkv_ssd_locate(int64_t ssd_block_id, int32_t round_robin, int32_t num_devices,
+                   int32_t files_per_device, int32_t *device, int32_t *file,
+                   int64_t *block_in_file);
+/* The requests fkv_ssd_transfer would issue, without touching any file: one row
+ * of five int64 per iovec -- request number, device * files_per_device + file,
+ * file offset of the request, host offset of the iovec, iovec length.  Returns
+ * the number of rows (also when it exceeds `capacity`), -1 on bad arguments. */
+int64_t fkv_ssd_plan(int32_t num_devices, int32_t files_per_device, int32_t start_layer,
+                     int32_t num_layers, const int64_t *ssd_block_ids,
+                     const int64_t *cpu_block_ids, int32_t num_blocks, int64_t cpu_layer_stride,
+                     int64_t cpu_kv_stride, int64_t ssd_layer_stride, int64_t ssd_kv_stride,
+                     int64_t chunk_size, int64_t block_stride, int32_t round_robin,
+                     int32_t kv_dim, int32_t ssd_io_opt, int64_t *out, int64_t capacity);
+
 /* ---- engine tensors shared with a worker process:
  *      flexkv/common/memory_handle.py:1144-1250 (direct IPC branch of
  *      TensorSharedHandle) ---- */

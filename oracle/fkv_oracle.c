@@ -31,6 +31,15 @@
  *   fkv_oracle_tp_rank_plan   closed forms + partition properties (shards
  *                             tile the chunk, layer slices tile the range)
  *   fkv_oracle_host_scatter   equality with numpy fancy indexing
+ *   fkv_oracle_ssd_locate     the reference's second statement of the same
+ *                             mapping (flexkv/transfer/nixlutil.py:351-385) as
+ *                             closed forms, bijection onto a dense
+ *                             (device, file, block) grid by brute force
+ *   fkv_oracle_ssd_transfer   the reference tests' fixture (host pool filled
+ *                             with arange % 9973, identity ids, one file of the
+ *                             pool's own layout): the file image equals the
+ *                             pool image; round trip; several files / devices
+ *                             against numpy indexing of per-file arrays
  */
 #include <stdint.h>
 #include <stdlib.h>
@@ -327,4 +336,55 @@ uint64_t fkv_oracle_host_chunk_bytes(double chunk_gb) {
     return 0;
   int64_t c = (int64_t)(chunk_gb * (double)(1024LL * 1024 * 1024)) - 4096;
   return (uint64_t)(c & ~0xFFFLL);
+}
+
+
+/* ---- host pool <-> SSD files ------------------------------------------- */
+
+/* partition_and_remap_blocks_by_device, csrc/transfer_ssd.cpp:22-44, and the
+ * split of a device's blocks over its files, :65-67. */
+void fkv_oracle_ssd_locate(int64_t ssd_block_id, int round_robin, int num_devices,
+                           int files_per_device, int *device, int *file,
+                           int64_t *block_in_file) {
+  int64_t in_device;
+  *device = (int)((ssd_block_id / round_robin) % num_devices);
+  in_device = ((ssd_block_id / round_robin) / num_devices) * round_robin +
+              (ssd_block_id % round_robin);
+  *file = (int)(in_device % files_per_device);
+  *block_in_file = in_device / files_per_device;
+}
+
+/* transfer_kv_blocks_ssd in its baseline form, csrc/transfer_ssd.cpp:187-255:
+ * one chunk per (block, layer, kv).  `files[device * files_per_device + file]`
+ * are byte arrays standing in for the files.  Returns -1 when a chunk would
+ * fall outside its file (`file_bytes`). */
+int fkv_oracle_ssd_transfer(uint8_t *const *files, int64_t file_bytes, int num_devices,
+                            int files_per_device, int start_layer, int num_layers,
+                            uint8_t *cpu_ptr, const int64_t *ssd_block_ids,
+                            const int64_t *cpu_block_ids, int num_blocks,
+                            int64_t cpu_layer_stride, int64_t cpu_kv_stride,
+                            int64_t ssd_layer_stride, int64_t ssd_kv_stride,
+                            int64_t chunk, int64_t block_stride, int is_read,
+                            int round_robin, int kv_dim) {
+  int b, l, kv;
+  for (b = 0; b < num_blocks; ++b) {
+    int device, file;
+    int64_t in_file;
+    fkv_oracle_ssd_locate(ssd_block_ids[b], round_robin, num_devices, files_per_device,
+                          &device, &file, &in_file);
+    for (l = start_layer; l < start_layer + num_layers; ++l)
+      for (kv = 0; kv < kv_dim; ++kv) {
+        const int64_t fo = in_file * block_stride + l * ssd_layer_stride + kv * ssd_kv_stride;
+        uint8_t *h = cpu_ptr + cpu_block_ids[b] * block_stride + l * cpu_layer_stride +
+                     kv * cpu_kv_stride;
+        uint8_t *f = files[device * files_per_device + file] + fo;
+        if (fo < 0 || fo + chunk > file_bytes)
+          return -1;
+        if (is_read)
+          memcpy(h, f, (size_t)chunk);
+        else
+          memcpy(f, h, (size_t)chunk);
+      }
+  }
+  return 0;
 }

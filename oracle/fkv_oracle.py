@@ -98,6 +98,12 @@ def lib() -> ctypes.CDLL:
         L.fkv_oracle_host_scatter.argtypes = [vp, vp, vp, i32, i64, i64, i64, i32,
                                               i32, i64, i64, i32]
         L.fkv_oracle_host_scatter.restype = None
+        L.fkv_oracle_ssd_locate.argtypes = [i64, i32, i32, i32, ctypes.POINTER(i32),
+                                            ctypes.POINTER(i32), ctypes.POINTER(i64)]
+        L.fkv_oracle_ssd_locate.restype = None
+        L.fkv_oracle_ssd_transfer.argtypes = [vp, i64, i32, i32, i32, i32, vp, vp, vp, i32,
+                                              i64, i64, i64, i64, i64, i64, i32, i32, i32]
+        L.fkv_oracle_ssd_transfer.restype = i32
         L.fkv_oracle_eventfd_index.argtypes = [i32] * 5
         L.fkv_oracle_eventfd_index.restype = i64
         L.fkv_oracle_host_chunk_bytes.argtypes = [ctypes.c_double]
@@ -341,3 +347,29 @@ def layerwise_multi_group(num_gpus: int, groups: List[GroupRef], layer_members, 
                 _group_layer_h2d(g, d, swa["host"], orig, 1, swa["gpu_ids"], swa["cpu_ids"], 1,
                                  swa["kv_stride"], swa["layer_stride"], swa["block_stride"], 0)
     return immediate, work
+
+
+# ---- host pool <-> SSD files -----------------------------------------------------
+
+def ssd_locate(ssd_block_id: int, round_robin: int, num_devices: int, files_per_device: int):
+    d, f, b = ctypes.c_int32(), ctypes.c_int32(), ctypes.c_int64()
+    lib().fkv_oracle_ssd_locate(ssd_block_id, round_robin, num_devices, files_per_device,
+                                ctypes.byref(d), ctypes.byref(f), ctypes.byref(b))
+    return d.value, f.value, b.value
+
+
+def ssd_transfer(files: List[np.ndarray], num_devices: int, files_per_device: int,
+                 start_layer: int, num_layers: int, host: np.ndarray, ssd_ids, cpu_ids,
+                 cpu_layer_stride: int, cpu_kv_stride: int, ssd_layer_stride: int,
+                 ssd_kv_stride: int, chunk: int, block_stride: int, is_read: bool,
+                 round_robin: int = 1, kv_dim: int = 2) -> None:
+    """``files[device * files_per_device + file]``: equally long uint8 arrays."""
+    s, c = _i64(ssd_ids), _i64(cpu_ids)
+    ptrs = (ctypes.c_void_p * len(files))(*[f.ctypes.data for f in files])
+    rc = lib().fkv_oracle_ssd_transfer(
+        ptrs, int(files[0].size), num_devices, files_per_device, start_layer, num_layers,
+        host.ctypes.data, _ptr(s), _ptr(c), int(s.size), cpu_layer_stride, cpu_kv_stride,
+        ssd_layer_stride, ssd_kv_stride, chunk, block_stride, int(bool(is_read)), round_robin,
+        kv_dim)
+    if rc != 0:
+        raise ValueError("oracle ssd transfer: a chunk lies outside its file")

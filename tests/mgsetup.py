@@ -141,7 +141,8 @@ class MGCase:
 
     # ---- device view ---------------------------------------------------------------
     def to_device(self, device: str = "cuda:0", eventfds=None, tp_size: int = 1,
-                  has_swa: bool = True):
+                  has_swa: bool = True, ssd_files=None, swa_ssd_files=None,
+                  iouring_entries: int = 512):
         """Builds the library's group over device copies of the (zeroed or seeded)
         buffers.  Returns a DeviceMG."""
         import torch
@@ -158,15 +159,17 @@ class MGCase:
         swa_kw = {}
         if has_swa:
             swa_kw = dict(
-                has_swa=True, swa_gpu_blocks=[swa_gpu], swa_cpu_blocks=swa_host, swa_ssd_files={},
+                has_swa=True, swa_gpu_blocks=[swa_gpu], swa_cpu_blocks=swa_host,
+                swa_ssd_files=swa_ssd_files or {},
                 swa_gpu_kv_strides_tensor=torch.tensor([s.kv], dtype=torch.int64),
                 swa_gpu_block_strides_tensor=torch.tensor([s.block], dtype=torch.int64),
                 swa_gpu_layer_strides_tensor=torch.tensor([s.layer], dtype=torch.int64),
                 swa_gpu_chunk_sizes_tensor=torch.tensor([s.chunk], dtype=torch.int64))
         group = LayerwiseTransferGroup(
-            num_gpus=1, gpu_blocks_per_group=[[g] for g in gpu], cpu_blocks=host, ssd_files={},
+            num_gpus=1, gpu_blocks_per_group=[[g] for g in gpu], cpu_blocks=host,
+            ssd_files=ssd_files or {},
             num_original_layers=self.num_original_layers, layer_members=t["layer_members"],
-            iouring_entries=512, iouring_flags=0,
+            iouring_entries=iouring_entries, iouring_flags=0,
             layer_eventfds_tensor=(eventfds if eventfds is not None
                                    else torch.empty(0, dtype=torch.int32)),
             tp_size=tp_size, is_blockfirst=True, **ctor, **swa_kw)

@@ -432,8 +432,8 @@ def test_layerwise_rejects_what_it_does_not_provide(gpu_device):
     with pytest.raises(TypeError, match="missing arguments"):
         LayerwiseTransferGroup(num_gpus=1, gpu_blocks_per_group=[[gpu]], cpu_blocks=cpu)
     st = torch.tensor([8], dtype=torch.int64)
-    with pytest.raises(RuntimeError, match="SSD"):
-        LayerwiseTransferGroup(1, [gpu], cpu, {0: ["/tmp/x"]}, L, st, st, st, st, 0, 0,
+    with pytest.raises(RuntimeError, match="Failed to open file"):
+        LayerwiseTransferGroup(1, [gpu], cpu, {0: ["/nonexistent/x"]}, L, st, st, st, st, 0, 0,
                                torch.empty(0, dtype=torch.int32), 1)
     with pytest.raises(RuntimeError, match="Unsupported GPU block type: 3"):
         LayerwiseTransferGroup(1, [gpu + [gpu[0]]], cpu, {}, L, st, st, st, st, 0, 0,
@@ -443,6 +443,62 @@ def test_layerwise_rejects_what_it_does_not_provide(gpu_device):
     none = torch.empty(0, dtype=torch.int64)
     with pytest.raises(RuntimeError, match="single-group instance"):
         lw.layerwise_transfer_multi_group(none, none, 0, 1, 4, ids, ids, 4, False, 1, 1)
-    with pytest.raises(RuntimeError, match="SSD"):
-        lw.layerwise_transfer_multi_group(ids, none, 0, 1, 4, ids, ids, 4, False, 1, 1)
+    lw.close()
+
+
+@pytest.mark.parametrize("kv_dim", [1, 2], ids=["mla", "kv_sep_1h"])
+@pytest.mark.parametrize("entries", [0, 64], ids=["threads", "iouring"])
+@pytest.mark.parametrize("use_ce", [False, True], ids=["kernel", "ce"])
+def test_layerwise_restore_reads_ssd_blocks_first(gpu_device, tmp_path, kv_dim, entries, use_ce):
+    """Some blocks of the request live only in the SSD files: the call first reads
+    them into the host blocks named by ``cpu_block_ids_d2h`` (all layers), then
+    restores host -> GPU layer by layer.  Host pool and GPU bytes vs the oracle."""
+    from flexkv_amd.layout import TransferStrides
+    L, N, T, H, D, heads, NSSD, ndev, nfiles = 3, 8, 16, 1, 128, 1, 12, 2, 2
+    gl, cl = make_layouts(L, N, T, H, D, "BLOCKFIRST", kv_dim, heads)
+    sl = KVCacheLayout(KVCacheLayoutType.BLOCKFIRST, L, NSSD, T, H, D, kv_dim=kv_dim,
+                       num_kv_heads=heads).div_block(ndev * nfiles, padding=True)
+    c, s = TransferStrides.from_layout(cl, ES), TransferStrides.from_layout(sl, ES)
+    rng = np.random.default_rng(17)
+    file_bytes = sl.get_total_elements() * ES
+    ref_files = [rng.integers(0, 256, file_bytes, dtype=np.uint8) for _ in range(ndev * nfiles)]
+    paths = {}
+    for d in range(ndev):
+        os.makedirs(tmp_path / f"d{d}")
+        paths[d] = [str(tmp_path / f"d{d}" / f"f{f}.bin") for f in range(nfiles)]
+        for f in range(nfiles):
+            ref_files[d * nfiles + f].tofile(paths[d][f])
+    cpu = torch.zeros(cl.kv_shape, dtype=DTYPE, pin_memory=True)
+    cpu.view(torch.uint8).view(-1).copy_(torch.from_numpy(
+        rng.integers(0, 256, cpu.numel() * ES, dtype=np.uint8)))
+    ref_host = cpu.view(torch.uint8).view(-1).numpy().copy()
+    gpu = make_gpu_tensors(L, N, T, H, D, kv_dim, gpu_device)
+    ssd_ids, staged = [7, 2, 11, 4], [6, 1, 3, 0]      # SSD block -> host block
+    cids = torch.tensor([5, 6, 1, 3, 0, 2], dtype=torch.int64)  # resident and just-staged
+    gids = torch.tensor([0, 7, 3, 4, 1, 6], dtype=torch.int64)
+    O.ssd_transfer(ref_files, ndev, nfiles, 0, L, ref_host, ssd_ids, staged, c.layer, c.kv,
+                   s.layer, s.kv, c.chunk, c.block, True, 1, kv_dim)
+    from flexkv_amd.c_ext import LayerwiseTransferGroup
+    st = lambda v: torch.tensor([v * ES], dtype=torch.int64)
+    lw = LayerwiseTransferGroup(
+        num_gpus=1, gpu_blocks=[gpu], cpu_blocks=cpu, ssd_files=paths, num_layers=L,
+        gpu_kv_strides_tensor=st(gl.get_kv_stride()),
+        gpu_block_strides_tensor=st(gl.get_block_stride()),
+        gpu_layer_strides_tensor=st(gl.get_layer_stride()),
+        gpu_chunk_sizes_tensor=st(gl.get_chunk_size()), iouring_entries=entries, iouring_flags=0,
+        layer_eventfds_tensor=torch.empty(0, dtype=torch.int32), tp_size=1, is_blockfirst=True,
+        num_kv_heads=heads)
+    e = torch.empty(0, dtype=torch.int64)
+    lw.layerwise_transfer(
+        torch.tensor(ssd_ids, dtype=torch.int64), torch.tensor(staged, dtype=torch.int64),
+        s.layer, s.kv, NSSD // (ndev * nfiles), 1, 4, gids, cids, c.kv, c.layer, c.block, c.chunk,
+        c.kv, c.layer, c.block, 4, use_ce, L, 1, kv_dim, heads, swa_h2d_src=e, swa_h2d_dst=e,
+        swa_disk2h_src=e, swa_disk2h_dst=e)
+    lw.synchronize()
+    assert np.array_equal(cpu.view(torch.uint8).view(-1).numpy(), ref_host)
+    host = torch.from_numpy(ref_host).view(DTYPE).view(cl.kv_shape)  # [block, layer, kv, ...]
+    for l in range(L):
+        for g, cb in zip(gids.tolist(), cids.tolist()):
+            assert torch.equal(gpu[l][:, g].cpu().view(torch.int16),
+                               host[cb, l].view(torch.int16)), (l, g, cb)
     lw.close()

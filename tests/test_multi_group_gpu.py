@@ -390,6 +390,64 @@ def test_single_group_with_uniform_sidecar(gpu_device, engine, granularity):
     grp.close()
 
 
+@pytest.mark.parametrize("engine", [False, True])
+@pytest.mark.parametrize("entries", [0, 64], ids=["threads", "iouring"])
+def test_blocks_and_sidecar_staged_from_ssd_files(gpu_device, tmp_path, engine, entries):
+    """Step 0 of the multi-group restore: byte-flat blocks come out of the SSD
+    files whole, the uniform sidecar layer by layer, into the host blocks the call
+    names; then the restore proper runs on the refreshed pools
+    (csrc/layerwise.cpp:1371-1432)."""
+    from oracle import fkv_oracle as O
+    rng = np.random.default_rng(31)
+    case = MGCase(_t6_groups(), 4, num_gpu_blocks=16, num_cpu_blocks=12, swa_width=48)
+    _randomize(case, rng)
+    B, n_ssd, nfiles = case.block_stride, 18, 3
+    main_files = [rng.integers(0, 256, (n_ssd // nfiles) * B, dtype=np.uint8)
+                  for _ in range(nfiles)]
+    swa_file_layout = swa_layout_of(4, n_ssd, case.tpb, 48).div_block(2, padding=True)
+    fs = TransferStrides.from_layout(swa_file_layout, 1)
+    swa_files = [rng.integers(0, 256, swa_file_layout.get_total_elements(), dtype=np.uint8)
+                 for _ in range(2)]
+
+    def write(arrays, tag):
+        paths = []
+        for i, a in enumerate(arrays):
+            paths.append(str(tmp_path / f"{tag}_{i}.bin"))
+            a.tofile(paths[-1])
+        return {0: paths}
+    dev = case.to_device(gpu_device, ssd_files=write(main_files, "main"),
+                         swa_ssd_files=write(swa_files, "swa"), iouring_entries=entries)
+    ssd_ids, staged = [17, 3, 10, 5], [11, 0, 6, 2]
+    swa_ssd_ids, swa_staged = [9, 14, 0], [4, 10, 1]
+    gpu_ids, cpu_ids = [3, 9, 4, 15, 0], [11, 7, 0, 2, 6]
+    swa_g, swa_c = [11, 2, 6], [4, 9, 1]
+    # expected host pools: whole blocks by the striping rule, sidecar through the oracle
+    for sb, cb in zip(ssd_ids, staged):
+        f, inf = sb % nfiles, sb // nfiles
+        case.host[cb * B:(cb + 1) * B] = main_files[f][inf * B:(inf + 1) * B]
+    c = case.swa_cpu_strides
+    O.ssd_transfer(swa_files, 1, 2, 0, 4, case.swa_host.reshape(-1), swa_ssd_ids, swa_staged,
+                   c.layer, c.kv, fs.layer, fs.kv, c.chunk, c.block, True, 1, 1)
+    O.layerwise_multi_group(1, case.oracle_groups(), case.members, case.host, gpu_ids, cpu_ids,
+                            1, 1, "sharded", case.oracle_swa(swa_c, swa_g))
+    kw = dev.swa_call_kwargs(swa_c, swa_g)
+    kw.update(swa_disk2h_src=torch.tensor(swa_ssd_ids), swa_disk2h_dst=torch.tensor(swa_staged),
+              swa_ssd_layer_stride_in_bytes=fs.layer, swa_ssd_kv_stride_in_bytes=fs.kv,
+              swa_num_blocks_per_file=n_ssd // 2)
+    dev.group.layerwise_transfer_multi_group(
+        torch.tensor(ssd_ids), torch.tensor(staged), n_ssd // nfiles, 1, 4,
+        torch.tensor(gpu_ids), torch.tensor(cpu_ids), 4, engine, 1, 1, **kw)
+    torch.cuda.synchronize()
+    assert np.array_equal(dev.host.numpy(), case.host)
+    assert np.array_equal(dev.swa_host.numpy(), case.swa_host)
+    for gi, grp in enumerate(case.gpu):
+        for local, ref in enumerate(grp):
+            assert np.array_equal(dev.gpu[gi][local].cpu().numpy(), ref), (gi, local)
+    for orig, ref in enumerate(case.swa_gpu):
+        assert np.array_equal(dev.swa_gpu[orig].cpu().numpy(), ref), orig
+    dev.group.close()
+
+
 # ---- error behaviour ------------------------------------------------------------------------------
 
 def test_wrong_entry_point_for_the_instance(gpu_device):
@@ -435,8 +493,8 @@ def test_constructor_rejects_inconsistent_groups(gpu_device):
     with pytest.raises(RuntimeError, match="unsupported tensors_per_gpu=2 for num_layers=4"):
         LayerwiseTransferGroup(gpu_blocks_per_group=[[dev.gpu[0][:2]], [dev.gpu[1]]],
                                layer_members=t["layer_members"], **ctor, **common)
-    with pytest.raises(RuntimeError, match="SSD"):
+    with pytest.raises(RuntimeError, match="Failed to open file"):
         LayerwiseTransferGroup(gpu_blocks_per_group=[[g] for g in dev.gpu],
                                layer_members=t["layer_members"], **ctor,
-                               **{**common, "ssd_files": {0: ["/tmp/x"]}})
+                               **{**common, "ssd_files": {0: ["/nonexistent/x"]}})
     dev.group.close()

@@ -281,3 +281,49 @@ def test_layerwise_worker_with_engine_eventfds(gpu_device, engine, tmp_path, not
         for fd in cs:
             os.close(fd)
     monkeypatch.setattr(env, "_ENV", None)
+
+
+def test_layerwise_worker_stages_ssd_blocks_first(gpu_device, engine, tmp_path):
+    """A layerwise op whose disk2h ids name blocks that live only in the SSD files:
+    the worker reads them into the host pool, then restores everything."""
+    from oracle import fkv_oracle as O
+    start, q, pool = engine
+    kv_dim, heads, n_ssd, nfiles = 1, 1, 20, 2
+    tensors = _engine_tensors(gpu_device, 41, kv_dim, heads)
+    gl = _gpu_layout(kv_dim, heads)
+    cl = _cpu_layout(KVCacheLayoutType.BLOCKFIRST, kv_dim, heads)
+    sl = KVCacheLayout(KVCacheLayoutType.BLOCKFIRST, L, n_ssd, T, heads, D, kv_dim=kv_dim,
+                       num_kv_heads=heads)
+    fl = sl.div_block(nfiles, padding=True)
+    c, s = TransferStrides.from_layout(cl, 2), TransferStrides.from_layout(fl, 2)
+    rng = np.random.default_rng(8)
+    files = [rng.integers(0, 256, fl.get_total_elements() * 2, dtype=np.uint8)
+             for _ in range(nfiles)]
+    paths = {0: [str(tmp_path / f"ssd_{i}.bin") for i in range(nfiles)]}
+    for a, p in zip(files, paths[0]):
+        a.tofile(p)
+    host = torch.zeros(cl.kv_shape, dtype=DT).share_memory_()
+    host.view(torch.uint8).view(-1).copy_(torch.from_numpy(
+        rng.integers(0, 256, host.numel() * 2, dtype=np.uint8)))
+    ref_host = host.view(torch.uint8).view(-1).numpy().copy()
+    ssd_ids, staged = [19, 4, 11], [30, 2, 7]
+    src, dst = [30, 5, 2, 7, 16], [0, 23, 9, 1, 14]
+    O.ssd_transfer(files, 1, nfiles, 0, L, ref_host, ssd_ids, staged, c.layer, c.kv, s.layer,
+                   s.kv, c.chunk, c.block, True, 1, kv_dim)
+    h = start(LayerwiseTransferWorker, [[TensorSharedHandle(t) for t in tensors]], host, [gl], cl,
+              DT, 1, enable_eventfd=False, use_ce_transfer_h2d=False, allow_pageable_host=True,
+              ssd_files=paths, ssd_kv_layout=sl, num_blocks_per_file=n_ssd // nfiles)
+    e = np.array([], dtype=I64)
+    op = LayerwiseTransferOp(0, TransferType.LAYERWISE, e, e,
+                             src_block_ids_h2d=np.asarray(src, dtype=I64),
+                             dst_block_ids_h2d=np.asarray(dst, dtype=I64),
+                             src_block_ids_disk2h=np.asarray(ssd_ids, dtype=I64),
+                             dst_block_ids_disk2h=np.asarray(staged, dtype=I64))
+    h.submit_transfer(op)
+    assert _collect(q, 1) == [(op.op_id, True, None)]
+    assert np.array_equal(host.view(torch.uint8).view(-1).numpy(), ref_host)
+    want = torch.from_numpy(ref_host).view(DT).view(cl.kv_shape)  # [block, layer, kv, ...]
+    for l in range(L):
+        assert torch.equal(tensors[l][:, dst].cpu(), want[src, l].transpose(0, 1)), l
+    h.shutdown()
+    assert h.process.exitcode == 0
