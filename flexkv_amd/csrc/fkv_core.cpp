@@ -259,13 +259,16 @@ LinkLaunchShape link_launch_shape(bool is_h2d) {
 // and direction, the events recorded behind its most recent link-bound launches;
 // a launch that finds the other direction still busy confines itself to its half
 // (GPU->host: XCD slots 0-3, host->GPU: 4-7) and asks for enough workgroups to
-// saturate the link from four XCDs.  FKV_LINK_ARBITER=0 switches this off; an
+// saturate the link from four XCDs.  Work recorded on the launching stream itself
+// does not count: it has finished before the new launch starts.
+// FKV_LINK_ARBITER=0 switches this off; an
 // explicit FKV_{H2D,D2H}_XCD_MASK takes precedence.
 namespace {
 constexpr int kActivityRing = 16;
 struct DirectionActivity {
   hipEvent_t ev[kActivityRing] = {};
   bool pending[kActivityRing] = {};
+  hipStream_t stream[kActivityRing] = {};
   int next = 0;
 };
 struct DeviceActivity {
@@ -287,7 +290,7 @@ bool arbiter_enabled() {
 }
 } // namespace
 
-bool link_direction_busy(int device, bool h2d) {
+bool link_direction_busy(int device, bool h2d, hipStream_t launching_stream) {
   DeviceActivity &a = activity_of(device);
   std::lock_guard<std::mutex> lk(a.mu);
   DirectionActivity &d = a.dir[h2d ? 1 : 0];
@@ -299,7 +302,7 @@ bool link_direction_busy(int device, bool h2d) {
       d.pending[i] = false;
     } else {
       (void)hipGetLastError();
-      busy = true;
+      busy = busy || d.stream[i] != launching_stream;
     }
   }
   return busy;
@@ -322,6 +325,7 @@ void link_direction_mark(int device, bool h2d, hipStream_t stream) {
     return;
   }
   d.pending[i] = true;
+  d.stream[i] = stream;
   d.next = (i + 1) % kActivityRing;
 }
 
@@ -396,7 +400,7 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
   out->threads = shape.threads;
   out->xcd_mask = shape.xcd_mask;
   out->device = device;
-  if (arbiter_enabled() && shape.xcd_mask == 0xffu && link_direction_busy(device, !out->h2d)) {
+  if (arbiter_enabled() && shape.xcd_mask == 0xffu && link_direction_busy(device, !out->h2d, stream)) {
     // four XCDs: 24 single-wavefront workgroups host->GPU, 48 GPU->host per 4 requested CTAs
     out->xcd_mask = out->h2d ? 0xf0u : 0x0fu;
     if (out->h2d)

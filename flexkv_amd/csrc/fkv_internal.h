@@ -167,7 +167,7 @@ struct KernelPlan {
   int device = 0;
 };
 // Link-bound launches of the last while, per device and direction (see fkv_core.cpp).
-bool link_direction_busy(int device, bool h2d);
+bool link_direction_busy(int device, bool h2d, hipStream_t launching_stream);
 void link_direction_mark(int device, bool h2d, hipStream_t stream);
 // Builds and uploads (on `stream`) the plan for all layers of `d`.
 int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan *out);
