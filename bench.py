@@ -614,6 +614,67 @@ def run_worker_process(torch, device, steps, warmup, num_cta, use_ce):
     return res
 
 
+def run_layout_transform(torch, device, steps, warmup, shape, verify=True):
+    """Engine blocks <-> dense device buffer, both in HBM: the re-layout step of a
+    direct-storage read or write (csrc/gds/layout_transform.cu), all blocks of a
+    request in one call.  Times both directions with events on the current stream
+    and a plain device copy of the same bytes as the yardstick."""
+    import numpy as np
+    from flexkv_amd.c_ext import layout_transform
+    shapes = {  # name: (layers, kv_dim, pool blocks, blocks moved, chunk bytes, description)
+        "c0": (32, 2, 4096, 2048, 32768, "32 x [2,4096,16,8,128] bf16, 2048 random blocks"),
+        "c3": (61, 1, 2048, 1024, 73728, "61 x [1,2048,64,576] bf16 (MLA), 1024 random blocks"),
+    }
+    L_, K, N, nb, C, desc = shapes[shape]
+    g = torch.Generator(device="cpu").manual_seed(5)
+    tensors = [torch.randint(0, 256, (K, N, C), dtype=torch.uint8, device=device) for _ in range(L_)]
+    ptrs = torch.tensor([t.data_ptr() for t in tensors], dtype=torch.int64)
+    ids = torch.randperm(N, generator=g)[:nb]
+    block = L_ * K * C
+    buf = torch.zeros(nb * block, dtype=torch.uint8, device=device)
+    B = nb * block
+    args = (buf, K * C, C, block, C, ptrs, N * C, C, K * N * C, ids, L_, K)
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    res = {}
+    for name, to_target in (("to_buffer", False), ("to_engine", True)):
+        times = []
+        for it in range(warmup + steps):
+            a, b = ev(), ev()
+            a.record()
+            layout_transform(*args, to_target)
+            b.record()
+            b.synchronize()
+            if it >= warmup:
+                times.append(a.elapsed_time(b))
+        res[name + "_ms"] = _median(times)
+    other = torch.empty_like(buf)
+    times = []
+    for it in range(warmup + steps):
+        a, b = ev(), ev()
+        a.record()
+        other.copy_(buf)
+        b.record()
+        b.synchronize()
+        if it >= warmup:
+            times.append(a.elapsed_time(b))
+    res["plain_copy_ms"] = _median(times)
+    ok = None
+    if verify:
+        layout_transform(*args, False)
+        view = buf.view(nb, L_, K, C)
+        di = ids.to(device)
+        ok = all(torch.equal(view[:, l], tensors[l].index_select(1, di).transpose(0, 1))
+                 for l in range(L_))
+        back = torch.randperm(N, generator=g)[:nb]
+        for t in tensors:
+            t.index_fill_(1, back.to(device), 0)
+        layout_transform(buf, K * C, C, block, C, ptrs, N * C, C, K * N * C, back, L_, K, True)
+        ok = ok and all(torch.equal(tensors[l].index_select(1, back.to(device)).transpose(0, 1),
+                                    view[:, l]) for l in range(L_))
+    res.update(bytes=B, desc=desc, bit_exact=ok)
+    return res
+
+
 def run_ssd(torch, steps, warmup, ssd_dir, blocks, pinned):
     """Host pool <-> SSD files in the shape of the reference's SSD microbenchmark
     (benchmarks/microbenchmark_ssd_simulation.py): "small" MHA preset, both pool
@@ -738,7 +799,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker", "ssd"])
+    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker", "ssd", "transform"])
+    ap.add_argument("--shape", default="c0", choices=["c0", "c3"],
+                    help="transform: which engine shape to re-lay out")
     ap.add_argument("--ssd-dir", default=None,
                     help="ssd: directory for the cache files (default: the system temp dir)")
     ap.add_argument("--ssd-blocks", type=int, default=256,
@@ -806,6 +869,31 @@ def main():
                 "small": {"hostfunc": 0.60, "polling": 0.40},
                 "medium": {"hostfunc": 4.39, "polling": 1.87},
                 "large": {"hostfunc": 16.79, "polling": 16.62}}}))
+        return
+    if args.config == "transform":
+        r = run_layout_transform(torch, device, args.steps, args.warmup, args.shape,
+                                 verify=not args.no_verify)
+        avg_ms = (r["to_buffer_ms"] + r["to_engine_ms"]) / 2
+        achieved = 2 * r["bytes"] / (avg_ms * 1e-3) / 1e9    # bytes read + bytes written
+        plain = 2 * r["bytes"] / (r["plain_copy_ms"] * 1e-3) / 1e9
+        print(json.dumps({
+            "metric": "engine blocks <-> dense device buffer, GB/s of HBM traffic (read + write)",
+            "unit": "GB/s", "value": round(achieved, 1), "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(avg_ms, 4), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": f"transform-{args.shape}: " + r["desc"]},
+            "to_buffer_ms": round(r["to_buffer_ms"], 4), "to_engine_ms": round(r["to_engine_ms"], 4),
+            "to_buffer_GBps": round(2 * r["bytes"] / (r["to_buffer_ms"] * 1e-3) / 1e9, 1),
+            "to_engine_GBps": round(2 * r["bytes"] / (r["to_engine_ms"] * 1e-3) / 1e9, 1),
+            "plain_device_copy_ms": round(r["plain_copy_ms"], 4),
+            "plain_device_copy_GBps": round(plain, 1),
+            "frac_of_plain_device_copy": round(achieved / plain, 4),
+            "bytes_moved": r["bytes"], "bit_exact": r["bit_exact"],
+            "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                         "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                         "traffic": None, "kernel": "fkv_copy_chunks_kernel<16, true>",
+                         "algorithmic_bytes_per_launch": 2 * r["bytes"],
+                         "avg_launch_ms": round(avg_ms, 4)}}))
         return
     if args.config == "mg":
         link = measure_link()

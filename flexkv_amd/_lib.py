@@ -55,6 +55,21 @@ class TransferDesc(Structure):
                 ("ce", CEConfig)]
 
 
+class LayoutTransformDesc(Structure):
+    _fields_ = [("backend", c_int32), ("num_layers_total", c_int32),
+                ("gpu_tensor_ptrs", c_void_p), ("num_gpu_tensor_ptrs", c_int32),
+                ("device", c_int32),
+                ("gpu_kv_stride", c_int64), ("gpu_block_stride", c_int64),
+                ("gpu_layer_stride", c_int64),
+                ("buffer_ptr", c_void_p),
+                ("buffer_layer_stride", c_int64), ("buffer_kv_stride", c_int64),
+                ("buffer_block_stride", c_int64), ("chunk_size", c_int64),
+                ("start_layer_id", c_int32), ("num_layers", c_int32),
+                ("kv_dim", c_int32), ("num_blocks", c_int32),
+                ("gpu_block_ids", c_void_p),
+                ("buffer_to_target", c_int32), ("sync", c_int32)]
+
+
 class CEAnalysis(Structure):
     _fields_ = [("gpu_log_contig", c_int32), ("cpu_log_contig", c_int32),
                 ("cpu_phys_contig", c_int32), ("gpu_phys_contig", c_int32),
@@ -184,6 +199,7 @@ SIGNATURES = {
     "fkv_ssd_open": (c_int32, [POINTER(c_char_p), c_int32, c_int32, c_int32, c_int32,
                                POINTER(c_void_p)]),
     "fkv_ssd_close": (None, [c_void_p]),
+    "fkv_layout_transform": (c_int32, [POINTER(LayoutTransformDesc), c_void_p]),
     "fkv_ssd_uses_iouring": (c_int32, [c_void_p]),
     "fkv_ssd_last_direct": (c_int32, [c_void_p]),
     "fkv_ssd_transfer": (c_int32, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p,

@@ -139,6 +139,54 @@ def transfer_kv_blocks(
     check(_L.fkv_transfer_kv_blocks(ctypes.byref(d), _current_stream_handle()))
 
 
+def layout_transform(
+        buffer: torch.Tensor, buffer_layer_stride_in_bytes: int, buffer_kv_stride_in_bytes: int,
+        buffer_block_stride_in_bytes: int, chunk_size_in_bytes: int,
+        gpu_tensor_ptrs_tensor: torch.Tensor, gpu_kv_stride_in_bytes: int,
+        gpu_block_stride_in_bytes: int, gpu_layer_stride_in_bytes: int,
+        gpu_block_id_tensor: torch.Tensor, num_layers: int, kv_dim: int, buffer_to_target: bool,
+        gpu_block_type: int = 0, start_layer_id: int = 0, sync: bool = False) -> None:
+    """Engine KV blocks <-> a dense device buffer on the current stream
+    (``launch_layout_transform_kernel``, ``csrc/gds/layout_transform.cu:26-108``;
+    strides in bytes where the reference counts 8-byte words).
+
+    Chunk (l, kv) of the i-th block id sits at ``buffer + i*block_stride +
+    l*layer_stride + kv*kv_stride``.  ``buffer_to_target`` True writes the engine's
+    tensors, False fills the buffer.  The block ids are a host tensor.
+    """
+    ids = _ids(gpu_block_id_tensor, "gpu_block_id_tensor")
+    ptrs = _ids(gpu_tensor_ptrs_tensor, "gpu_tensor_ptrs_tensor")
+    if buffer.device.type != "cuda":
+        raise ValueError("buffer must live in device memory")
+    d = _lib.LayoutTransformDesc()
+    d.backend = int(gpu_block_type)
+    d.num_layers_total = ptrs.numel() // 2 if int(gpu_block_type) == 2 else int(num_layers)
+    d.gpu_tensor_ptrs = ptrs.data_ptr()
+    d.num_gpu_tensor_ptrs = ptrs.numel()
+    d.device = buffer.device.index if buffer.device.index is not None else -1
+    d.gpu_kv_stride = int(gpu_kv_stride_in_bytes)
+    d.gpu_block_stride = int(gpu_block_stride_in_bytes)
+    d.gpu_layer_stride = int(gpu_layer_stride_in_bytes)
+    d.buffer_ptr = buffer.data_ptr()
+    d.buffer_layer_stride = int(buffer_layer_stride_in_bytes)
+    d.buffer_kv_stride = int(buffer_kv_stride_in_bytes)
+    d.buffer_block_stride = int(buffer_block_stride_in_bytes)
+    d.chunk_size = int(chunk_size_in_bytes)
+    d.start_layer_id = int(start_layer_id)
+    d.num_layers = int(num_layers)
+    d.kv_dim = int(kv_dim)
+    d.num_blocks = ids.numel()
+    d.gpu_block_ids = ids.data_ptr()
+    d.buffer_to_target = int(bool(buffer_to_target))
+    d.sync = int(bool(sync))
+    need = ((d.num_blocks - 1) * d.buffer_block_stride + (d.num_layers - 1) * d.buffer_layer_stride
+            + (d.kv_dim - 1) * d.buffer_kv_stride + d.chunk_size) if d.num_blocks and d.num_layers else 0
+    if need > buffer.numel() * buffer.element_size():
+        raise ValueError(f"buffer of {buffer.numel() * buffer.element_size()} bytes is shorter than "
+                         f"the {need} bytes the strides address")
+    check(_L.fkv_layout_transform(ctypes.byref(d), _current_stream_handle()))
+
+
 def last_transfer_path() -> str:
     """Name of the path the last transfer issued by this thread took: KERNEL or
     one of the copy-engine strategies."""

@@ -454,6 +454,40 @@ int64_t fkv_ssd_plan(int32_t num_devices, int32_t files_per_device, int32_t star
                      int64_t chunk_size, int64_t block_stride, int32_t round_robin,
                      int32_t kv_dim, int32_t ssd_io_opt, int64_t *out, int64_t capacity);
 
+/* ---- engine KV blocks <-> a dense device buffer: csrc/gds/layout_transform.{cu,cuh}
+ *      (the re-layout step between the engine's tensors and the device staging
+ *      buffer a direct-storage read or write works on) ---- */
+
+typedef struct fkv_layout_transform_desc {
+  /* engine side, as in fkv_transfer_desc */
+  int32_t backend;
+  int32_t num_layers_total;
+  const uint64_t *gpu_tensor_ptrs; /* host array of device addresses */
+  int32_t num_gpu_tensor_ptrs;
+  int32_t device;                  /* -1 = current */
+  int64_t gpu_kv_stride;
+  int64_t gpu_block_stride;
+  int64_t gpu_layer_stride;
+  /* buffer side: chunk (l, kv) of the i-th block of the call lives at
+   * buffer_ptr + i*buffer_block_stride + l*buffer_layer_stride + kv*buffer_kv_stride */
+  void *buffer_ptr;                /* device memory */
+  int64_t buffer_layer_stride;
+  int64_t buffer_kv_stride;
+  int64_t buffer_block_stride;
+  int64_t chunk_size;              /* bytes */
+  int32_t start_layer_id;          /* engine layer of buffer layer 0; the reference always uses 0 */
+  int32_t num_layers;
+  int32_t kv_dim;
+  int32_t num_blocks;
+  const int64_t *gpu_block_ids;    /* host, num_blocks entries (device memory in the reference) */
+  int32_t buffer_to_target;        /* 1: buffer -> engine tensors, 0: engine tensors -> buffer */
+  int32_t sync;
+} fkv_layout_transform_desc;
+
+/* launch_layout_transform_kernel<Type> (csrc/gds/layout_transform.cu:26-108), any
+ * number of blocks per call. */
+int fkv_layout_transform(const fkv_layout_transform_desc *desc, void *stream);
+
 /* ---- engine tensors shared with a worker process:
  *      flexkv/common/memory_handle.py:1144-1250 (direct IPC branch of
  *      TensorSharedHandle) ---- */

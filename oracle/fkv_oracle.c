@@ -40,6 +40,10 @@
  *                             pool's own layout): the file image equals the
  *                             pool image; round trip; several files / devices
  *                             against numpy indexing of per-file arrays
+ *   fkv_oracle_layout_transform  torch fancy indexing of shaped engine tensors
+ *                             into a shaped [block, layer, kv, chunk] buffer,
+ *                             for the three engine layouts; padded buffer
+ *                             strides leave the padding untouched; round trip
  */
 #include <stdint.h>
 #include <stdlib.h>
@@ -385,6 +389,39 @@ int fkv_oracle_ssd_transfer(uint8_t *const *files, int64_t file_bytes, int num_d
         else
           memcpy(f, h, (size_t)chunk);
       }
+  }
+  return 0;
+}
+
+/* csrc/gds/layout_transform.cu:41-70: chunk index c in [0, L*K*N) names
+ *   block position  c % N,  layer  c / (N*K),  kv  (c % (N*K)) / N;
+ *   buffer = base + pos*bBs + layer*bLs + kv*bKs
+ *   engine = ptr_at(start_layer + layer, kv, gpu_ids[pos])
+ * (the reference passes layer itself, i.e. start_layer = 0).  Bytes here,
+ * 8-byte words there.  Returns 0, or -1 for an unknown backend. */
+int fkv_oracle_layout_transform(uint8_t *buffer, int64_t buffer_layer_stride,
+                                int64_t buffer_kv_stride, int64_t buffer_block_stride,
+                                int64_t chunk, int backend, const uint64_t *tensor_ptrs,
+                                int64_t num_layers_total, int64_t gpu_kv_stride,
+                                int64_t gpu_block_stride, int64_t gpu_layer_stride,
+                                const int64_t *gpu_ids, int num_blocks, int start_layer,
+                                int num_layers, int kv_dim, int buffer_to_target) {
+  if (backend < 0 || backend > 2)
+    return -1;
+  const int64_t num_chunks = (int64_t)num_layers * kv_dim * num_blocks;
+  for (int64_t c = 0; c < num_chunks; ++c) {
+    const int64_t pos = c % num_blocks;
+    const int64_t layer = c / ((int64_t)num_blocks * kv_dim);
+    const int64_t kv = (c % ((int64_t)num_blocks * kv_dim)) / num_blocks;
+    uint8_t *buf = buffer + pos * buffer_block_stride + layer * buffer_layer_stride +
+                   kv * buffer_kv_stride;
+    uint8_t *gpu = (uint8_t *)(uintptr_t)fkv_oracle_chunk_addr(
+        backend, tensor_ptrs, num_layers_total, gpu_kv_stride, gpu_block_stride,
+        gpu_layer_stride, start_layer + layer, kv, gpu_ids[pos]);
+    if (buffer_to_target)
+      memcpy(gpu, buf, (size_t)chunk);
+    else
+      memcpy(buf, gpu, (size_t)chunk);
   }
   return 0;
 }

@@ -104,6 +104,9 @@ def lib() -> ctypes.CDLL:
         L.fkv_oracle_ssd_transfer.argtypes = [vp, i64, i32, i32, i32, i32, vp, vp, vp, i32,
                                               i64, i64, i64, i64, i64, i64, i32, i32, i32]
         L.fkv_oracle_ssd_transfer.restype = i32
+        L.fkv_oracle_layout_transform.argtypes = [vp, i64, i64, i64, i64, i32, vp, i64, i64, i64,
+                                                  i64, vp, i32, i32, i32, i32, i32]
+        L.fkv_oracle_layout_transform.restype = i32
         L.fkv_oracle_eventfd_index.argtypes = [i32] * 5
         L.fkv_oracle_eventfd_index.restype = i64
         L.fkv_oracle_host_chunk_bytes.argtypes = [ctypes.c_double]
@@ -138,6 +141,22 @@ def transfer_c(backend: int, tensor_ptrs: Sequence[int], num_layers_total: int,
         int(g.size), _ptr(g), _ptr(c), int(bool(is_host_to_device)))
     if rc != 0:
         raise ValueError(f"oracle transfer rejected backend {backend}")
+
+
+def layout_transform(buffer_ptr: int, buffer_layer_stride: int, buffer_kv_stride: int,
+                     buffer_block_stride: int, chunk: int, backend: int,
+                     tensor_ptrs: Sequence[int], num_layers_total: int, gpu_kv_stride: int,
+                     gpu_block_stride: int, gpu_layer_stride: int, gpu_ids, num_layers: int,
+                     kv_dim: int, buffer_to_target: bool, start_layer: int = 0) -> None:
+    """Engine blocks <-> dense buffer; all pointers are HOST addresses (ints)."""
+    ptrs = np.ascontiguousarray(np.asarray(tensor_ptrs, dtype=np.uint64))
+    g = _i64(gpu_ids)
+    rc = lib().fkv_oracle_layout_transform(
+        buffer_ptr, buffer_layer_stride, buffer_kv_stride, buffer_block_stride, chunk, backend,
+        _ptr(ptrs), num_layers_total, gpu_kv_stride, gpu_block_stride, gpu_layer_stride,
+        _ptr(g), int(g.size), start_layer, num_layers, kv_dim, int(bool(buffer_to_target)))
+    if rc != 0:
+        raise ValueError(f"oracle layout transform rejected backend {backend}")
 
 
 def chunk_addr(backend, tensor_ptrs, num_layers_total, kvs, bs, ls, layer, kv, block) -> int:
