@@ -41,7 +41,7 @@ METRIC = "KV block transfer GB/s (D2H, H2D) on 1 GPU; % of measured host-link pe
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs of this script scaled by plain copy kernels of known size
 # (profiles/fkv_copy_chunks_kernel_c1_pmc.md).  None where no such run was made.
-MEASURED_TRAFFIC_BYTES = {("c1", "kernel"): 8591004672}
+MEASURED_TRAFFIC_BYTES = {("c1", "kernel"): 8591004672, ("transform-c0", "kernel"): 8590449664}
 
 
 def _median(xs):
@@ -891,7 +891,8 @@ def main():
             "bytes_moved": r["bytes"], "bit_exact": r["bit_exact"],
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                          "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                         "traffic": None, "kernel": "fkv_copy_chunks_kernel<16, true>",
+                         "traffic": MEASURED_TRAFFIC_BYTES.get(("transform-" + args.shape, "kernel")),
+                         "kernel": "fkv_copy_chunks_kernel<16, true>",
                          "algorithmic_bytes_per_launch": 2 * r["bytes"],
                          "avg_launch_ms": round(avg_ms, 4)}}))
         return
