@@ -372,11 +372,15 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy):
                 restore_alone_ms=restore_alone_ms)
 
 
-def run_concurrent(w, torch, steps, warmup, num_cta):
-    """c4: 32 D2H puts and 32 H2D gets issued at once from 64 threads, one
-    stream each."""
+def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32):
+    """c4: 32 D2H puts and 32 H2D gets issued at once from 64 threads.  Each
+    direction has its own set of streams (one per request by default); the
+    process has 4 hardware queues, so with more than 2 streams per direction
+    puts and gets also share queues and partly serialize."""
     reqs = w.requests
-    streams = [torch.cuda.Stream() for _ in reqs]
+    per_dir = max(1, min(streams_per_direction, len(reqs) // 2))
+    pool = [[torch.cuda.Stream() for _ in range(per_dir)] for _ in range(2)]
+    streams = [pool[i % 2][(i // 2) % per_dir] for i in range(len(reqs))]
     lat = [[] for _ in reqs]
     walls = []
     w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=num_cta, sync=True)  # fill the host cache
@@ -802,6 +806,8 @@ def main():
     ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker", "ssd", "transform"])
     ap.add_argument("--shape", default="c0", choices=["c0", "c3"],
                     help="transform: which engine shape to re-lay out")
+    ap.add_argument("--streams-per-direction", type=int, default=32,
+                    help="c4: streams the 32 puts (and the 32 gets) are spread over")
     ap.add_argument("--ssd-dir", default=None,
                     help="ssd: directory for the cache files (default: the system temp dir)")
     ap.add_argument("--ssd-blocks", type=int, default=256,
@@ -1013,10 +1019,12 @@ def main():
                            "link_peak_GBps": round(link["h2d"], 3),
                            "frac_of_link_peak": round(achieved / link["h2d"], 4)}
     else:  # c4
-        r = run_concurrent(w, torch, args.steps, args.warmup, args.num_cta)
+        r = run_concurrent(w, torch, args.steps, args.warmup, args.num_cta,
+                           args.streams_per_direction)
         agg = r["total_bytes"] / _median(r["walls"]) / 1e9
         out.update(value=round(agg, 3), ms_per_step=round(_median(r["walls"]) * 1e3, 3),
-                   concurrent={"requests": 64, "total_blocks": sum(r["blocks"]),
+                   concurrent={"requests": 64, "streams_per_direction": args.streams_per_direction,
+                               "total_blocks": sum(r["blocks"]),
                                "aggregate_bytes": r["total_bytes"],
                                "p50_latency_ms": round(r["p50_ms"], 3),
                                "p99_latency_ms": round(r["p99_ms"], 3),

@@ -259,8 +259,12 @@ LinkLaunchShape link_launch_shape(bool is_h2d) {
 // and direction, the events recorded behind its most recent link-bound launches;
 // a launch that finds the other direction still busy confines itself to its half
 // (GPU->host: XCD slots 0-3, host->GPU: 4-7) and asks for enough workgroups to
-// saturate the link from four XCDs.  Work recorded on the launching stream itself
-// does not count: it has finished before the new launch starts.
+// saturate the link from four XCDs.  A direction also counts as busy for a short
+// while after its last launch (FKV_LINK_ARBITER_WINDOW_MS, default 20): with many
+// small requests in flight the other direction is often between two kernels at
+// the moment of a launch, and a full-chip launch would then collide with its next
+// one.  Work recorded on the launching stream itself does not count: it has
+// finished before the new launch starts.
 // FKV_LINK_ARBITER=0 switches this off; an
 // explicit FKV_{H2D,D2H}_XCD_MASK takes precedence.
 namespace {
@@ -269,6 +273,7 @@ struct DirectionActivity {
   hipEvent_t ev[kActivityRing] = {};
   bool pending[kActivityRing] = {};
   hipStream_t stream[kActivityRing] = {};
+  int64_t launched_ns[kActivityRing] = {}; // steady clock at launch
   int next = 0;
 };
 struct DeviceActivity {
@@ -284,6 +289,11 @@ DeviceActivity &activity_of(int device) {
     p = new DeviceActivity();
   return *p;
 }
+int64_t steady_ns() {
+  return std::chrono::duration_cast<std::chrono::nanoseconds>(
+             std::chrono::steady_clock::now().time_since_epoch())
+      .count();
+}
 bool arbiter_enabled() {
   static const bool on = env_int("FKV_LINK_ARBITER", 1) != 0;
   return on;
@@ -294,8 +304,12 @@ bool link_direction_busy(int device, bool h2d, hipStream_t launching_stream) {
   DeviceActivity &a = activity_of(device);
   std::lock_guard<std::mutex> lk(a.mu);
   DirectionActivity &d = a.dir[h2d ? 1 : 0];
+  static const int64_t window_ns = (int64_t)env_int("FKV_LINK_ARBITER_WINDOW_MS", 20) * 1000000;
+  const int64_t now = steady_ns();
   bool busy = false;
   for (int i = 0; i < kActivityRing; ++i) {
+    if (d.stream[i] != launching_stream && d.launched_ns[i] && now - d.launched_ns[i] < window_ns)
+      busy = true;
     if (!d.pending[i])
       continue;
     if (hipEventQuery(d.ev[i]) == hipSuccess) {
@@ -326,6 +340,7 @@ void link_direction_mark(int device, bool h2d, hipStream_t stream) {
   }
   d.pending[i] = true;
   d.stream[i] = stream;
+  d.launched_ns[i] = steady_ns();
   d.next = (i + 1) % kActivityRing;
 }
 
@@ -403,8 +418,9 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
   if (arbiter_enabled() && shape.xcd_mask == 0xffu && link_direction_busy(device, !out->h2d, stream)) {
     // four XCDs: 24 single-wavefront workgroups host->GPU, 48 GPU->host per 4 requested CTAs
     out->xcd_mask = out->h2d ? 0xf0u : 0x0fu;
-    if (out->h2d)
-      out->workgroups = out->workgroups * 3 / 2;
+    static const int h2d_pct = std::max(50, env_int("FKV_ARBITER_H2D_PCT", 150));
+    static const int d2h_pct = std::max(25, env_int("FKV_ARBITER_D2H_PCT", 100));
+    out->workgroups = std::max(1, out->workgroups * (out->h2d ? h2d_pct : d2h_pct) / 100);
   }
   return FKV_OK;
 }
