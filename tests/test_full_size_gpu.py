@@ -1,0 +1,88 @@
+"""The benchmark configurations at their full sizes, checked through properties
+that do not need a CPU pass over gigabytes: the host image equals torch's own
+index_select of the engine tensors (compared on the GPU), gather -> erase ->
+scatter restores every byte, and a checksum over whole tensors shows that no
+other block was touched."""
+import gc
+import os
+import sys
+
+import pytest
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+import bench  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+def checksums(w):
+    """One 64-bit wrap-around sum per engine tensor."""
+    return [int(t.contiguous().view(torch.uint8).view(torch.int64).sum()) for t in w.tensors]
+
+
+@pytest.fixture
+def workload(request, gpu_device):
+    w = bench.Workload(request.param, torch, gpu_device)
+    yield w
+    del w
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("workload,use_ce", [("c0", False), ("c0", True), ("c1", False),
+                                             ("c1", True), ("c2", False)],
+                         indirect=["workload"], ids=["c0-kernel", "c0-ce", "c1-kernel", "c1-ce",
+                                                     "c2-kernel"])
+def test_gather_erase_scatter_at_full_size(workload, use_ce):
+    w = workload
+    kw = dict(transfer_num_cta=4, use_ce_transfer=use_ce, ce_path_opt=True, sync=True)
+    before = checksums(w)
+    w.host.zero_()
+    w.transfer(w.gpu_ids, w.cpu_ids, False, **kw)
+    assert w.verify_host_image(w.gpu_ids, w.cpu_ids)
+    assert checksums(w) == before                         # a put does not write the engine's tensors
+    gi = w.gpu_ids.to(w.device)
+    back = getattr(w, "gpu_ids_reload", w.gpu_ids)        # c2 reloads into another permutation
+    bi = back.to(w.device)
+    saved = [[w.gpu_rows(l, kv).index_select(0, gi) for kv in range(w.kv_dim)]
+             for l in range(w.L)]
+    for l in range(w.L):
+        for kv in range(w.kv_dim):
+            w.gpu_rows(l, kv).index_fill_(0, bi, 0)
+    w.transfer(back, w.cpu_ids, True, **kw)
+    for l in range(w.L):
+        for kv in range(w.kv_dim):
+            assert torch.equal(w.gpu_rows(l, kv).index_select(0, bi), saved[l][kv]), (l, kv)
+    if back is w.gpu_ids:
+        assert checksums(w) == before                     # every other block is as it was
+
+
+@pytest.mark.parametrize("workload", ["c3"], indirect=True)
+@pytest.mark.parametrize("notify", ["polling", "hostfunc"])
+def test_layerwise_restore_at_full_size(workload, notify):
+    from flexkv_amd.c_ext import LayerwiseTransferGroup
+    w = workload
+    before = checksums(w)
+    w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=4, sync=True)
+    assert w.verify_host_image(w.gpu_ids, w.cpu_ids)
+    gi = w.gpu_ids.to(w.device)
+    for l in range(w.L):
+        w.gpu_rows(l, 0).index_fill_(0, gi, 0)
+    assert checksums(w) != before
+    i64 = lambda v: torch.tensor([v], dtype=torch.int64)  # noqa: E731
+    grp = LayerwiseTransferGroup(
+        num_gpus=1, gpu_blocks=[w.tensors], cpu_blocks=w.host, ssd_files={}, num_layers=w.L,
+        gpu_kv_strides_tensor=i64(w.gks), gpu_block_strides_tensor=i64(w.gbs),
+        gpu_layer_strides_tensor=i64(w.gls), gpu_chunk_sizes_tensor=i64(w.chunk),
+        iouring_entries=0, iouring_flags=0,
+        layer_eventfds_tensor=torch.empty(0, dtype=torch.int32), tp_size=1, is_blockfirst=True)
+    e = torch.empty(0, dtype=torch.int64)
+    grp.layerwise_transfer(e, e, 0, 0, 0, 0, 0, w.gpu_ids, w.cpu_ids, w.cks, w.cls, w.cbs,
+                           w.chunk, w.cks, w.cls, w.cbs, 4, False, w.L, 1, w.kv_dim, 1,
+                           counter_id=0, kv_shared_across_ranks_mode="sharded",
+                           notify_mode=notify)
+    grp.synchronize()
+    torch.cuda.synchronize()
+    assert checksums(w) == before
+    grp.close()

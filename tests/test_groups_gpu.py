@@ -449,14 +449,16 @@ def test_layerwise_rejects_what_it_does_not_provide(gpu_device):
 @pytest.mark.parametrize("kv_dim", [1, 2], ids=["mla", "kv_sep_1h"])
 @pytest.mark.parametrize("entries", [0, 64], ids=["threads", "iouring"])
 @pytest.mark.parametrize("use_ce", [False, True], ids=["kernel", "ce"])
-def test_layerwise_restore_reads_ssd_blocks_first(gpu_device, tmp_path, kv_dim, entries, use_ce):
+@pytest.mark.parametrize("cpu_name", ["BLOCKFIRST", "LAYERFIRST"])
+def test_layerwise_restore_reads_ssd_blocks_first(gpu_device, tmp_path, kv_dim, entries, use_ce,
+                                                  cpu_name):
     """Some blocks of the request live only in the SSD files: the call first reads
     them into the host blocks named by ``cpu_block_ids_d2h`` (all layers), then
     restores host -> GPU layer by layer.  Host pool and GPU bytes vs the oracle."""
     from flexkv_amd.layout import TransferStrides
     L, N, T, H, D, heads, NSSD, ndev, nfiles = 3, 8, 16, 1, 128, 1, 12, 2, 2
-    gl, cl = make_layouts(L, N, T, H, D, "BLOCKFIRST", kv_dim, heads)
-    sl = KVCacheLayout(KVCacheLayoutType.BLOCKFIRST, L, NSSD, T, H, D, kv_dim=kv_dim,
+    gl, cl = make_layouts(L, N, T, H, D, cpu_name, kv_dim, heads)
+    sl = KVCacheLayout(KVCacheLayoutType[cpu_name], L, NSSD, T, H, D, kv_dim=kv_dim,
                        num_kv_heads=heads).div_block(ndev * nfiles, padding=True)
     c, s = TransferStrides.from_layout(cl, ES), TransferStrides.from_layout(sl, ES)
     rng = np.random.default_rng(17)
@@ -486,8 +488,8 @@ def test_layerwise_restore_reads_ssd_blocks_first(gpu_device, tmp_path, kv_dim, 
         gpu_block_strides_tensor=st(gl.get_block_stride()),
         gpu_layer_strides_tensor=st(gl.get_layer_stride()),
         gpu_chunk_sizes_tensor=st(gl.get_chunk_size()), iouring_entries=entries, iouring_flags=0,
-        layer_eventfds_tensor=torch.empty(0, dtype=torch.int32), tp_size=1, is_blockfirst=True,
-        num_kv_heads=heads)
+        layer_eventfds_tensor=torch.empty(0, dtype=torch.int32), tp_size=1,
+        is_blockfirst=cpu_name == "BLOCKFIRST", num_kv_heads=heads)
     e = torch.empty(0, dtype=torch.int64)
     lw.layerwise_transfer(
         torch.tensor(ssd_ids, dtype=torch.int64), torch.tensor(staged, dtype=torch.int64),
@@ -496,9 +498,11 @@ def test_layerwise_restore_reads_ssd_blocks_first(gpu_device, tmp_path, kv_dim, 
         swa_disk2h_src=e, swa_disk2h_dst=e)
     lw.synchronize()
     assert np.array_equal(cpu.view(torch.uint8).view(-1).numpy(), ref_host)
-    host = torch.from_numpy(ref_host).view(DTYPE).view(cl.kv_shape)  # [block, layer, kv, ...]
+    host = torch.from_numpy(ref_host).view(DTYPE).view(cl.kv_shape)
     for l in range(L):
         for g, cb in zip(gids.tolist(), cids.tolist()):
-            assert torch.equal(gpu[l][:, g].cpu().view(torch.int16),
-                               host[cb, l].view(torch.int16)), (l, g, cb)
+            # [block, layer, kv, ...] or [layer, kv, block, ...]
+            want = host[cb, l] if cpu_name == "BLOCKFIRST" else host[l, :, cb]
+            assert torch.equal(gpu[l][:, g].cpu().view(torch.int16), want.view(torch.int16)), \
+                (l, g, cb)
     lw.close()

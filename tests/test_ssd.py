@@ -162,6 +162,37 @@ def test_round_trip_like_the_reference(tmp_path, size, kv_dim, kind, entries, op
 
 @pytest.mark.parametrize("kind", ["LAYERFIRST", "BLOCKFIRST"])
 @pytest.mark.parametrize("kv_dim", [1, 2])
+@pytest.mark.parametrize("entries", ENGINES)
+@pytest.mark.parametrize("opt", [False, True], ids=["baseline", "optimized"])
+def test_partial_blocks_like_the_reference(tmp_path, kind, kv_dim, entries, opt):
+    """tests/test_kv_transfer_correctness.py:2139-2262: write blocks [0,2,4,6], zero
+    them in the pool, read them back into [1,3,5,7]; the odd blocks then hold what
+    the even ones held, everything else is as the zeroing left it."""
+    layers, blocks, tpb, heads, dim = 4, 8, 16, 8, 128
+    case = SsdCase(tmp_path, kind, layers, blocks, tpb, heads, dim, kv_dim)
+    shape = tuple(case.layout.kv_shape)
+    orig = case.host.view(np.float16).reshape(shape).copy()
+    pool = case.host.view(np.float16).reshape(shape)
+    ctx = SSDIOCTX(case.paths, 1, entries, 0)
+    even, odd = [0, 2, 4, 6], [1, 3, 5, 7]
+    case.run(ctx, even, even, False, opt=opt)
+    if kind == "LAYERFIRST":
+        pool[:, :, even] = 0
+    else:
+        pool[even] = 0
+    case.run(ctx, even, odd, True, opt=opt)
+    for src, dst in zip(even, odd):
+        if kind == "LAYERFIRST":
+            assert np.array_equal(pool[:, :, dst], orig[:, :, src])
+            assert not pool[:, :, src].any()
+        else:
+            assert np.array_equal(pool[dst], orig[src])
+            assert not pool[src].any()
+    ctx.close()
+
+
+@pytest.mark.parametrize("kind", ["LAYERFIRST", "BLOCKFIRST"])
+@pytest.mark.parametrize("kv_dim", [1, 2])
 @pytest.mark.parametrize("ndev,nfiles,rr", [(1, 1, 1), (2, 2, 1), (3, 2, 4), (1, 3, 2)])
 @pytest.mark.parametrize("entries", ENGINES)
 def test_striped_files_match_the_oracle(tmp_path, kind, kv_dim, ndev, nfiles, rr, entries):
