@@ -173,6 +173,7 @@ bool transfer_iov_full(int fd, const iovec *iov, int iovcnt, int64_t offset, int
     }
   };
   advance(already);
+  errno = 0; // so that a transfer cut short by the end of the file reports no stale code
   while (done < total) {
     const int cnt = (int)std::min<size_t>(rest.size() - head, kMaxIov);
     const ssize_t n = is_read ? preadv(fd, rest.data() + head, cnt, offset + done)
@@ -544,9 +545,11 @@ int fkv_ssd_open(const char *const *paths, int32_t num_devices, int32_t files_pe
     }
   }
   // reads ahead of writes where the scheduler lets us (csrc/transfer_ssd.h:49-58)
+  // (probe whether this thread may use the real-time class, then put back what it had)
+  const long had = syscall(SYS_ioprio_get, 1, 0);
   const bool rt = syscall(SYS_ioprio_set, 1, 0, ioprio_value(kIoprioRT, 0)) == 0;
   if (rt)
-    (void)syscall(SYS_ioprio_set, 1, 0, ioprio_value(kIoprioBE, 4));
+    (void)syscall(SYS_ioprio_set, 1, 0, had >= 0 ? (int)had : 0);
   ctx->read_ioprio = rt ? ioprio_value(kIoprioRT, 0) : ioprio_value(kIoprioBE, 0);
   ctx->write_ioprio = ioprio_value(kIoprioBE, 4);
   *out = ctx.release();
