@@ -362,7 +362,9 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
   const int lk = d.num_layers * d.kv_dim;
   const size_t tab_bytes = (size_t)lk * 8;
   const size_t ids_bytes = (size_t)d.num_blocks * 8;
-  const size_t plan_bytes = 2 * tab_bytes + 2 * ids_bytes;
+  // base tables, the two id lists, one claim counter per layer (see CopyKernelArgs::claim)
+  const size_t claims_bytes = ((size_t)d.num_layers * 4 + 7) & ~(size_t)7;
+  const size_t plan_bytes = 2 * tab_bytes + 2 * ids_bytes + claims_bytes;
   PlanSlot *slot = plan_acquire(device, plan_bytes);
   if (!slot)
     return FKV_ERR_RUNTIME;
@@ -386,6 +388,7 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
   }
   std::memcpy(h + 2 * tab_bytes, d.gpu_block_ids, ids_bytes);
   std::memcpy(h + 2 * tab_bytes + ids_bytes, d.cpu_block_ids, ids_bytes);
+  std::memset(h + 2 * tab_bytes + 2 * ids_bytes, 0, claims_bytes);
   uint8_t *dv = nullptr;
   int rc = plan_publish(slot, plan_bytes, mirror_plan, stream, &dv);
   if (rc != FKV_OK) {
@@ -397,6 +400,9 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
   out->cpu_base = reinterpret_cast<const uint64_t *>(dv + tab_bytes);
   out->gpu_ids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes);
   out->cpu_ids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes + ids_bytes);
+  // counters are updated by the device: only a device copy of the plan can hold them
+  out->claims = mirror_plan ? reinterpret_cast<uint32_t *>(dv + 2 * tab_bytes + 2 * ids_bytes)
+                            : nullptr;
   out->vec = common_vector_width(&acc, 1);
   out->h2d = d.is_host_to_device != 0;
   out->kv_dim = d.kv_dim;
@@ -419,7 +425,7 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
     // four XCDs: 24 single-wavefront workgroups host->GPU, 48 GPU->host per 4 requested CTAs
     out->xcd_mask = out->h2d ? 0xf0u : 0x0fu;
     static const int h2d_pct = std::max(50, env_int("FKV_ARBITER_H2D_PCT", 150));
-    static const int d2h_pct = std::max(25, env_int("FKV_ARBITER_D2H_PCT", 100));
+    static const int d2h_pct = std::max(5, env_int("FKV_ARBITER_D2H_PCT", 100));
     out->workgroups = std::max(1, out->workgroups * (out->h2d ? h2d_pct : d2h_pct) / 100);
   }
   return FKV_OK;
@@ -456,6 +462,7 @@ int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
     // reach 55.8, 32 x 64 reach 56.2.
     a.packed_grid_pct = p.h2d ? 150 : 100;
     a.xcd_mask = p.xcd_mask;
+    a.claim = p.claims ? p.claims + l0 : nullptr; // a launch per first layer at most
     FKV_TRY(launch_copy_kernel(a, p.workgroups, p.threads, stream));
   }
   link_direction_mark(p.device, p.h2d, stream);
@@ -561,7 +568,7 @@ void fkv_get_stats(fkv_stats *out) {
   out->dma_copies = s.dma_copies.load();
   out->staging_bytes_device = s.staging_bytes_device.load();
   out->staging_bytes_host = s.staging_bytes_host.load();
-  out->reserved = 0;
+  out->confined_launches = s.confined_launches.load();
 }
 void fkv_reset_stats(void) {
   fkv::Stats &s = fkv::stats();
@@ -572,6 +579,7 @@ void fkv_reset_stats(void) {
   s.dma_copies = 0;
   s.staging_bytes_device = 0;
   s.staging_bytes_host = 0;
+  s.confined_launches = 0;
 }
 
 int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream_v) {

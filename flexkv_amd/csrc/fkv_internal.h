@@ -39,7 +39,7 @@ void clear_error();
 // ---- counters -----------------------------------------------------------
 struct Stats {
   std::atomic<uint64_t> calls{0}, bytes_h2d{0}, bytes_d2h{0}, kernel_launches{0},
-      dma_copies{0}, staging_bytes_device{0}, staging_bytes_host{0};
+      dma_copies{0}, staging_bytes_device{0}, staging_bytes_host{0}, confined_launches{0};
 };
 Stats &stats();
 
@@ -115,7 +115,12 @@ struct CopyKernelArgs {
   int32_t nt_store; // 1: nontemporal stores (destination in HBM), 0: plain (pinned host)
   int32_t packed;   // set by launch_copy_kernel: chunks shorter than a slice, see the kernel
   int32_t packed_grid_pct; // workgroups to launch in packed mode, percent of the request (0 = 100)
-  uint32_t xcd_mask; // bit k: workgroups with blockIdx % 8 == k take part; 0 or 0xff = all
+  uint32_t xcd_mask; // bit k: workgroups that run on XCD k take part; 0 or 0xff = all
+  // Confined launches only: a zeroed counter in device memory from which the
+  // workgroups that take part claim `num_claims` ranges of the work (set by
+  // launch_copy_kernel).  Without a counter the mask is ignored.
+  uint32_t *claim;
+  uint32_t num_claims;
 };
 constexpr int kCopyBlockThreads = 1024;  // largest workgroup the kernel is built for
 constexpr int kCopyUnroll = 8;           // vector accesses in flight per lane
@@ -165,6 +170,7 @@ struct KernelPlan {
   int workgroups = 1, threads = 64;
   unsigned xcd_mask = 0xff;
   int device = 0;
+  uint32_t *claims = nullptr; // one zeroed counter per layer of the plan, device memory
 };
 // Link-bound launches of the last while, per device and direction (see fkv_core.cpp).
 bool link_direction_busy(int device, bool h2d, hipStream_t launching_stream);

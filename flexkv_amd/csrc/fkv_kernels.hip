@@ -37,7 +37,11 @@
 // For the same reason a GPU->host and a host->GPU copy that run at the same
 // time slow each other down when they share XCDs (62 GB/s in sum against
 // 87-90 GB/s on disjoint halves of the chip); `xcd_mask` confines a launch to
-// a subset of the XCDs.
+// a subset of the XCDs.  Workgroups of a launch go to the XCDs round-robin, but
+// the XCD of workgroup 0 differs from launch to launch (it depends on what was
+// dispatched before), so a workgroup reads the id of the XCD it actually runs on
+// and leaves if that XCD is not selected; the ones that stay share the work by
+// claiming ranges from a counter in device memory.
 //
 // Data moves as raw integer vectors (integer types cannot canonicalise NaN
 // payloads of fp8/bf16 data).  Loads are nontemporal: KV bytes are not reused
@@ -45,6 +49,7 @@
 // memory are plain, which measured about 1 GB/s faster over the link.
 #include "fkv_internal.h"
 
+#include <algorithm>
 #include <cstdlib>
 
 namespace fkv {
@@ -58,6 +63,13 @@ template <> struct VecType<8>  { typedef unsigned int type __attribute__((ext_ve
 template <> struct VecType<4>  { typedef unsigned int type; };
 template <> struct VecType<2>  { typedef unsigned short type; };
 template <> struct VecType<1>  { typedef unsigned char type; };
+
+// Id of the XCD this wavefront runs on (0-7).
+__device__ __forceinline__ uint32_t xcd_of_this_wave() {
+  uint32_t v;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(v));
+  return v & 7u;
+}
 
 template <typename V, bool NT> __device__ __forceinline__ void put(V v, V *p) {
   if (NT)
@@ -116,28 +128,13 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
   const uint32_t spp = a.packed ? (uint32_t)a.lk * vpc : (uint32_t)a.lk * slices;
   const uint64_t total_units = (uint64_t)a.num_blocks * spp;
   const uint64_t total = a.packed ? (total_units + kPiece - 1) / kPiece : total_units;
-  // Workgroups are handed to the 8 XCDs round-robin by blockIdx.x.  With a
-  // partial mask only the workgroups that land on the selected XCDs take part;
-  // they are renumbered densely, the others leave at once.
-  uint32_t wg = blockIdx.x, nwg = gridDim.x;
-  if ((a.xcd_mask & 0xffu) != 0xffu) {
-    const uint32_t slot = blockIdx.x & 7u;
-    if (!((a.xcd_mask >> slot) & 1u))
-      return;
-    const uint32_t per_round = __popc(a.xcd_mask & 0xffu);
-    wg = (blockIdx.x >> 3) * per_round + __popc(a.xcd_mask & ((1u << slot) - 1u));
-    nwg = (gridDim.x >> 3) * per_round;
-  }
-  uint64_t s0 = total * wg / nwg;
-  uint64_t s1 = total * (wg + 1) / nwg;
-  if (s0 >= s1)
-    return; // whole workgroup leaves together
-  if (a.packed) { // from pieces to vectors
-    s0 *= kPiece;
-    s1 = s1 * kPiece < total_units ? s1 * kPiece : total_units;
-  }
-
   const int tid = threadIdx.x;
+  // A launch confined to some XCDs: workgroups elsewhere leave (workgroup 0 always
+  // stays, so the work gets done wherever the launch lands); the others claim ranges.
+  const bool confined = (a.xcd_mask & 0xffu) != 0xffu;
+  if (confined && blockIdx.x != 0 && !((a.xcd_mask >> xcd_of_this_wave()) & 1u))
+    return;
+  __shared__ uint32_t s_claim;
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
   const int nwaves = blockDim.x / kWave;
@@ -147,86 +144,115 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
     s_base_dst[i] = a.base_dst[i];
   }
 
-  const uint32_t pos_lo = (uint32_t)(s0 / spp);
-  const uint32_t pos_hi = (uint32_t)((s1 - 1) / spp);
-  for (uint32_t tile = pos_lo; tile <= pos_hi; tile += kCopyIdTile) {
-    const uint32_t n = min((uint32_t)kCopyIdTile, pos_hi - tile + 1);
-    __syncthreads(); // previous tile fully consumed; base tables visible
-    for (uint32_t i = tid; i < n; i += blockDim.x) {
-      const int64_t p = (int64_t)tile + i;
-      s_off_src[i] = (a.ids_src ? a.ids_src[p] : p) * a.stride_src;
-      s_off_dst[i] = (a.ids_dst ? a.ids_dst[p] : p) * a.stride_dst;
+  for (;;) {
+    // This workgroup's range of work units: its own share of the launch, or the next
+    // unclaimed one.
+    uint32_t part = blockIdx.x, parts = gridDim.x;
+    if (confined) {
+      if (tid == 0)
+        s_claim = atomicAdd(a.claim, 1u);
+      __syncthreads();
+      part = s_claim;
+      parts = a.num_claims;
+      __syncthreads(); // everyone has read the claim before it is overwritten
+      if (part >= parts)
+        return; // whole workgroup leaves together
     }
-    __syncthreads();
-    const uint64_t tile_s0 = (uint64_t)tile * spp;
-    const uint64_t t0 = s0 > tile_s0 ? s0 : tile_s0;
-    const uint64_t tile_s1 = tile_s0 + (uint64_t)n * spp;
-    const uint64_t t1 = s1 < tile_s1 ? s1 : tile_s1;
-    if (a.packed) {
-      using V = typename VecType<VEC>::type;
-      const uint32_t lim = (uint32_t)(t1 - tile_s0); // < kCopyIdTile * spp, checked on host
-      const uint32_t ulk = (uint32_t)a.lk;
-      const uint32_t q64 = kWave / vpc, r64 = kWave % vpc; // kWave vectors = q64 chunks + r64
-      const uint32_t qlk = q64 / ulk, rlk = q64 % ulk;     // q64 chunks = qlk positions + rlk
-      for (uint32_t v0 = (uint32_t)(t0 - tile_s0) + wave * kPiece; v0 < lim;
-           v0 += nwaves * kPiece) {
-        V r[kCopyUnroll];
-        V *d[kCopyUnroll];
-        // A lane's vectors are kWave apart.  The first one is located by division;
-        // each further one by adding the precomputed quotients and remainders of
-        // kWave, which costs a few compares instead of two divisions.  Lanes beyond
-        // the end stay on their last valid vector and re-read it rather than branch
-        // around the load: all loads of a piece are issued back to back, only the
-        // stores are predicated.
-        uint32_t v = v0 + lane;
-        const uint32_t vc = min(v, lim - 1);
-        const uint32_t c = vc / vpc; // chunk inside the tile: position * lk + i
-        uint32_t w = vc - c * vpc;
-        uint32_t p = c / ulk;
-        uint32_t i = c - p * ulk;
-#pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u) {
-          if (u > 0) {
-            v += kWave;
-            uint32_t w2 = w + r64, i2 = i + rlk, p2 = p + qlk;
-            if (w2 >= vpc) {
-              w2 -= vpc;
-              i2 += 1;
-            }
-            if (i2 >= ulk) {
-              i2 -= ulk;
-              p2 += 1;
-            }
-            const bool ok = v < lim;
-            w = ok ? w2 : w;
-            i = ok ? i2 : i;
-            p = ok ? p2 : p;
-          }
-          const V *src = reinterpret_cast<const V *>(s_base_src[i] + (uint64_t)s_off_src[p]) + w;
-          d[u] = reinterpret_cast<V *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + w;
-          r[u] = __builtin_nontemporal_load(src);
-        }
-#pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u)
-          if (v0 + u * kWave + lane < lim)
-            put<V, NTS>(r[u], d[u]);
+    uint64_t s0 = total * part / parts;
+    uint64_t s1 = total * (part + 1) / parts;
+    if (s0 >= s1) {
+      if (confined)
+        continue;
+      return;
+    }
+    if (a.packed) { // from pieces to vectors
+      s0 *= kPiece;
+      s1 = s1 * kPiece < total_units ? s1 * kPiece : total_units;
+    }
+
+    const uint32_t pos_lo = (uint32_t)(s0 / spp);
+    const uint32_t pos_hi = (uint32_t)((s1 - 1) / spp);
+    for (uint32_t tile = pos_lo; tile <= pos_hi; tile += kCopyIdTile) {
+      const uint32_t n = min((uint32_t)kCopyIdTile, pos_hi - tile + 1);
+      __syncthreads(); // previous tile fully consumed; base tables visible
+      for (uint32_t i = tid; i < n; i += blockDim.x) {
+        const int64_t p = (int64_t)tile + i;
+        s_off_src[i] = (a.ids_src ? a.ids_src[p] : p) * a.stride_src;
+        s_off_dst[i] = (a.ids_dst ? a.ids_dst[p] : p) * a.stride_dst;
       }
-      continue;
+      __syncthreads();
+      const uint64_t tile_s0 = (uint64_t)tile * spp;
+      const uint64_t t0 = s0 > tile_s0 ? s0 : tile_s0;
+      const uint64_t tile_s1 = tile_s0 + (uint64_t)n * spp;
+      const uint64_t t1 = s1 < tile_s1 ? s1 : tile_s1;
+      if (a.packed) {
+        using V = typename VecType<VEC>::type;
+        const uint32_t lim = (uint32_t)(t1 - tile_s0); // < kCopyIdTile * spp, checked on host
+        const uint32_t ulk = (uint32_t)a.lk;
+        const uint32_t q64 = kWave / vpc, r64 = kWave % vpc; // kWave vectors = q64 chunks + r64
+        const uint32_t qlk = q64 / ulk, rlk = q64 % ulk;     // q64 chunks = qlk positions + rlk
+        for (uint32_t v0 = (uint32_t)(t0 - tile_s0) + wave * kPiece; v0 < lim;
+             v0 += nwaves * kPiece) {
+          V r[kCopyUnroll];
+          V *d[kCopyUnroll];
+          // A lane's vectors are kWave apart.  The first one is located by division;
+          // each further one by adding the precomputed quotients and remainders of
+          // kWave, which costs a few compares instead of two divisions.  Lanes beyond
+          // the end stay on their last valid vector and re-read it rather than branch
+          // around the load: all loads of a piece are issued back to back, only the
+          // stores are predicated.
+          uint32_t v = v0 + lane;
+          const uint32_t vc = min(v, lim - 1);
+          const uint32_t c = vc / vpc; // chunk inside the tile: position * lk + i
+          uint32_t w = vc - c * vpc;
+          uint32_t p = c / ulk;
+          uint32_t i = c - p * ulk;
+  #pragma unroll
+          for (int u = 0; u < kCopyUnroll; ++u) {
+            if (u > 0) {
+              v += kWave;
+              uint32_t w2 = w + r64, i2 = i + rlk, p2 = p + qlk;
+              if (w2 >= vpc) {
+                w2 -= vpc;
+                i2 += 1;
+              }
+              if (i2 >= ulk) {
+                i2 -= ulk;
+                p2 += 1;
+              }
+              const bool ok = v < lim;
+              w = ok ? w2 : w;
+              i = ok ? i2 : i;
+              p = ok ? p2 : p;
+            }
+            const V *src = reinterpret_cast<const V *>(s_base_src[i] + (uint64_t)s_off_src[p]) + w;
+            d[u] = reinterpret_cast<V *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + w;
+            r[u] = __builtin_nontemporal_load(src);
+          }
+  #pragma unroll
+          for (int u = 0; u < kCopyUnroll; ++u)
+            if (v0 + u * kWave + lane < lim)
+              put<V, NTS>(r[u], d[u]);
+        }
+        continue;
+      }
+      for (uint64_t s = t0 + wave; s < t1; s += nwaves) {
+        const uint32_t rel = (uint32_t)(s - tile_s0); // < kCopyIdTile * spp, checked on host
+        const uint32_t p = rel / spp;
+        const uint32_t r = rel - p * spp;
+        const uint32_t i = r / slices;
+        const uint32_t sl = r - i * slices;
+        const int64_t off = (int64_t)sl * kSliceBytes;
+        const int64_t left = a.chunk_bytes - off;
+        const uint8_t *src =
+            reinterpret_cast<const uint8_t *>(s_base_src[i] + (uint64_t)s_off_src[p]) + off;
+        uint8_t *dst = reinterpret_cast<uint8_t *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + off;
+        copy_slice<VEC, NTS>(src, dst, left < kSliceBytes ? left : kSliceBytes, lane);
+      }
     }
-    for (uint64_t s = t0 + wave; s < t1; s += nwaves) {
-      const uint32_t rel = (uint32_t)(s - tile_s0); // < kCopyIdTile * spp, checked on host
-      const uint32_t p = rel / spp;
-      const uint32_t r = rel - p * spp;
-      const uint32_t i = r / slices;
-      const uint32_t sl = r - i * slices;
-      const int64_t off = (int64_t)sl * kSliceBytes;
-      const int64_t left = a.chunk_bytes - off;
-      const uint8_t *src =
-          reinterpret_cast<const uint8_t *>(s_base_src[i] + (uint64_t)s_off_src[p]) + off;
-      uint8_t *dst = reinterpret_cast<uint8_t *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + off;
-      copy_slice<VEC, NTS>(src, dst, left < kSliceBytes ? left : kSliceBytes, lane);
-    }
-  }
+    if (!confined)
+      return;
+  } // next claim
 }
 
 template <int VEC>
@@ -309,15 +335,20 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_wor
   if (grid < 1)
     grid = 1;
   a.xcd_mask &= 0xffu;
-  if (a.xcd_mask == 0)
+  if (a.xcd_mask == 0 || !a.claim)
     a.xcd_mask = 0xffu;
   if (a.xcd_mask != 0xffu) {
-    // `grid` working workgroups need grid / popcount(mask) rounds of 8
+    // One range per working workgroup (finer ranges shift the balance between two
+    // concurrent directions towards GPU->host and lower their sum); `grid` working
+    // workgroups need grid / popcount(mask) rounds of 8.
+    a.num_claims = (uint32_t)std::min<int64_t>(grid, total);
     const int per_round = __builtin_popcount(a.xcd_mask);
     grid = (grid + per_round - 1) / per_round * 8;
   }
   const size_t lds_bytes = (size_t)(2 * a.lk + 2 * kCopyIdTile) * sizeof(uint64_t);
   stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);
+  if (a.xcd_mask != 0xffu)
+    stats().confined_launches.fetch_add(1, std::memory_order_relaxed);
   switch (a.vec) {
   case 16: return launch_vec<16>(a, (int)grid, threads, lds_bytes, stream);
   case 8:  return launch_vec<8>(a, (int)grid, threads, lds_bytes, stream);

@@ -517,7 +517,7 @@ typedef struct fkv_stats {
   uint64_t dma_copies;
   uint64_t staging_bytes_device;
   uint64_t staging_bytes_host;
-  uint64_t reserved;
+  uint64_t confined_launches; /* kernel launches restricted to a subset of the XCDs */
 } fkv_stats;
 void fkv_get_stats(fkv_stats *out);
 void fkv_reset_stats(void);

@@ -161,6 +161,8 @@ def test_puts_and_gets_at_the_same_time(gpu_device):
     get_g, get_c = perm_g[250:500], perm_c[250:500]
     streams = [torch.cuda.Stream(), torch.cuda.Stream()]
     errors = []
+    from flexkv_amd.c_ext import get_stats, reset_stats
+    reset_stats()
 
     def run(i):
         try:
@@ -176,6 +178,8 @@ def test_puts_and_gets_at_the_same_time(gpu_device):
     [t.join() for t in threads]
     assert not errors, errors
     torch.cuda.synchronize()
+    st = get_stats()
+    assert st["kernel_launches"] == 12 and st["confined_launches"] >= 6, st
     s.oracle_transfer(put_g, put_c, False)
     s.oracle_transfer(get_g, get_c, True)
     dev.assert_matches_reference("concurrent put and get")
