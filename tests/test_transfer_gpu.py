@@ -146,13 +146,15 @@ def test_short_chunks_are_packed(gpu_device, backend, L, K, chunk, n):
         dev.assert_matches_reference(f"H2D cta={cta}")
 
 
-def test_puts_and_gets_at_the_same_time(gpu_device):
+@pytest.mark.parametrize("chunk", [16 * 8 * 128 * 2, 1152, 24], ids=["32k", "packed", "narrow"])
+def test_puts_and_gets_at_the_same_time(gpu_device, chunk):
     """A GPU->host and a host->GPU transfer in flight together on two streams: a
     launch that finds the other direction busy confines itself to half of the
-    XCDs.  Which workgroups take part must not change a byte."""
+    XCDs.  Which workgroups take part must not change a byte (also for chunks
+    shorter than a slice, which are packed, and for 8-byte vectors)."""
     import threading
     import torch
-    s = KVSetup(VLLM, 8, 2, 600, 600, 16 * 8 * 128 * 2, "BLOCKFIRST", seed=41)
+    s = KVSetup(VLLM, 8, 2, 600, 600, chunk, "BLOCKFIRST", seed=41)
     dev = s.to_device(gpu_device)
     rng = np.random.default_rng(8)
     perm_g, perm_c = rng.permutation(600), rng.permutation(600)
