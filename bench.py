@@ -220,6 +220,27 @@ def measure_link(device_index=0, nbytes=1 << 30, reps=10):
     return out
 
 
+def measure_link_bidirectional(torch, device, nbytes=1 << 30, reps=6):
+    """Plain pinned copies in both directions at once (two streams), best of `reps`:
+    the yardstick for puts running next to gets."""
+    hd = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+    hu = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+    dd = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    du = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    s_up, s_down = torch.cuda.Stream(), torch.cuda.Stream()
+    best = float("inf")
+    for _ in range(reps + 1):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        with torch.cuda.stream(s_up):
+            hu.copy_(du, non_blocking=True)
+        with torch.cuda.stream(s_down):
+            dd.copy_(hd, non_blocking=True)
+        torch.cuda.synchronize()
+        best = min(best, time.perf_counter() - t0)
+    return 2 * nbytes / best / 1e9
+
+
 def run_gather_scatter(w, torch, steps, warmup, num_cta, use_ce):
     """c0 / c1 / c2: D2H gather then H2D scatter per step."""
     st = torch.cuda.Stream()
@@ -789,8 +810,18 @@ def cpu_baseline(cfg, budget_s=20.0):
         if time.perf_counter() - t_start > budget_s or reps >= 200:
             break
     elapsed = time.perf_counter() - t_start
+    threads = torch.get_num_threads()
+    torch.set_num_threads(1)
+    t1, reps1 = time.perf_counter(), 0
+    while time.perf_counter() - t1 < budget_s / 4 or reps1 < 1:
+        O.torch_index_gather(layers, host, gi, ci)
+        O.torch_index_scatter(layers, host, gi, ci)
+        reps1 += 1
+    one_thread = nbytes * reps1 / (time.perf_counter() - t1) / 1e9
+    torch.set_num_threads(threads)
     return {"value": round(nbytes * reps / elapsed / 1e9, 3), "best": round(nbytes / best / 1e9, 3),
-            "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "one_thread": round(one_thread, 3),
+            "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": (f"{L} of 32 layers, {n} blocks of {T}x{H}x{D} bf16 K+V out of a {N}-block "
                        f"pool, torch index_select/index_copy_ gather into the block-first host "
                        f"cache then scatter back, {reps} repetitions ({elapsed:.1f} s), "
@@ -960,6 +991,7 @@ def main():
         out.update(value=round(2 * B * args.steps / wall / 1e9, 3),
                    ms_per_step=round(wall / args.steps * 1e3, 3),
                    d2h_GBps=round(d2h, 3), h2d_GBps=round(h2d, 3),
+                   d2h_GiBps=round(d2h * 1e9 / 2**30, 3), h2d_GiBps=round(h2d * 1e9 / 2**30, 3),
                    d2h_frac_of_link=round(d2h / link["d2h"], 4),
                    h2d_frac_of_link=round(h2d / link["h2d"], 4))
         # dominant kernel: the gather/scatter kernel; one launch per direction moves B bytes
@@ -1021,6 +1053,7 @@ def main():
     else:  # c4
         r = run_concurrent(w, torch, args.steps, args.warmup, args.num_cta,
                            args.streams_per_direction)
+        bidir = measure_link_bidirectional(torch, device)
         agg = r["total_bytes"] / _median(r["walls"]) / 1e9
         out.update(value=round(agg, 3), ms_per_step=round(_median(r["walls"]) * 1e3, 3),
                    concurrent={"requests": 64, "streams_per_direction": args.streams_per_direction,
@@ -1028,7 +1061,10 @@ def main():
                                "aggregate_bytes": r["total_bytes"],
                                "p50_latency_ms": round(r["p50_ms"], 3),
                                "p99_latency_ms": round(r["p99_ms"], 3),
-                               "frac_of_bidir_link": round(agg / (link["d2h"] + link["h2d"]), 4)})
+                               "bidir_link_peak_GBps": round(bidir, 3),
+                               "frac_of_bidir_link": round(agg / bidir, 4),
+                               "frac_of_sum_of_one_way_peaks": round(
+                                   agg / (link["d2h"] + link["h2d"]), 4)})
         out["roofline"] = {"bound": "hbm", "achieved": round(agg, 3), "peak": HBM_PEAK_GBPS,
                            "unit": "GB/s", "frac": round(agg / HBM_PEAK_GBPS, 5), "traffic": None,
                            "kernel": "fkv_copy_chunks_kernel<16, false|true>",
