@@ -1,4 +1,5 @@
-"""Host code of the library under AddressSanitizer + UndefinedBehaviorSanitizer.
+"""Host code of the library under AddressSanitizer + UndefinedBehaviorSanitizer and
+under ThreadSanitizer.
 
 Two small native drivers (tests/native/) include a host-only translation unit
 of the library each, run it on seeded random inputs against a plain model, and
@@ -15,26 +16,32 @@ CLANG = shutil.which("clang++", path="/opt/rocm/llvm/bin") or shutil.which("clan
 pytestmark = pytest.mark.skipif(CLANG is None, reason="no clang++ for a sanitizer build")
 
 
-def build_and_run(tmp_path, driver, extra=()):
+SANITIZERS = [pytest.param(("-fsanitize=address,undefined", "-fno-sanitize-recover=undefined"),
+                           id="asan-ubsan"),
+              pytest.param(("-fsanitize=thread",), id="tsan")]
+
+
+def build_and_run(tmp_path, driver, sanitizer, extra=()):
     exe = str(tmp_path / "driver")
-    cmd = [CLANG, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined",
-           "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
+    cmd = [CLANG, "-std=c++17", "-O1", "-g", *sanitizer, "-fno-omit-frame-pointer",
            "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", "-I" + os.path.join(ROOT, "include"),
            "-I" + os.path.join(ROOT, "flexkv_amd", "csrc"), *extra,
            os.path.join(ROOT, "tests", "native", driver), "-o", exe, "-pthread"]
     subprocess.run(cmd, check=True, capture_output=True, text=True)
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:verify_asan_link_order=0",
-               TMPDIR=str(tmp_path))
+               TSAN_OPTIONS="halt_on_error=1", TMPDIR=str(tmp_path))
     r = subprocess.run([exe], capture_output=True, text=True, env=env, timeout=600)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-4000:]
     return r.stdout
 
 
-def test_ssd_engine_under_sanitizers(tmp_path):
-    out = build_and_run(tmp_path, "ssd_sanitizer_driver.cpp")
+@pytest.mark.parametrize("sanitizer", SANITIZERS)
+def test_ssd_engine_under_sanitizers(tmp_path, sanitizer):
+    out = build_and_run(tmp_path, "ssd_sanitizer_driver.cpp", sanitizer)
     assert "240 transfers round-tripped" in out
 
 
-def test_host_row_copies_under_sanitizers(tmp_path):
-    out = build_and_run(tmp_path, "host_copy_sanitizer_driver.cpp", extra=("-mavx2",))
+@pytest.mark.parametrize("sanitizer", SANITIZERS)
+def test_host_row_copies_under_sanitizers(tmp_path, sanitizer):
+    out = build_and_run(tmp_path, "host_copy_sanitizer_driver.cpp", sanitizer, extra=("-mavx2",))
     assert "400 scatter/gather pairs" in out
