@@ -298,6 +298,22 @@ bool arbiter_enabled() {
   static const bool on = env_int("FKV_LINK_ARBITER", 1) != 0;
   return on;
 }
+// The halves of the split are XCDs 0-3 and 4-7: only a device that exposes all
+// eight (an unpartitioned MI355X, 256 CUs) can be split that way.
+bool device_has_eight_xcds(int device) {
+  static std::mutex mu;
+  static std::map<int, bool> known;
+  std::lock_guard<std::mutex> lk(mu);
+  auto it = known.find(device);
+  if (it != known.end())
+    return it->second;
+  int cus = 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) {
+    (void)hipGetLastError();
+    cus = 0;
+  }
+  return known[device] = cus >= 8 * 28; // 32 CUs per XCD, some may be fused off
+}
 } // namespace
 
 bool link_direction_busy(int device, bool h2d, hipStream_t launching_stream) {
@@ -421,7 +437,8 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
   out->threads = shape.threads;
   out->xcd_mask = shape.xcd_mask;
   out->device = device;
-  if (arbiter_enabled() && shape.xcd_mask == 0xffu && link_direction_busy(device, !out->h2d, stream)) {
+  if (arbiter_enabled() && shape.xcd_mask == 0xffu && device_has_eight_xcds(device) &&
+      link_direction_busy(device, !out->h2d, stream)) {
     // four XCDs: 24 single-wavefront workgroups host->GPU, 48 GPU->host per 4 requested CTAs
     out->xcd_mask = out->h2d ? 0xf0u : 0x0fu;
     static const int h2d_pct = std::max(50, env_int("FKV_ARBITER_H2D_PCT", 150));

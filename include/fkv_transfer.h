@@ -254,8 +254,9 @@ typedef struct fkv_layerwise_params {
 #define FKV_NOTIFY_HOSTFUNC 0
 #define FKV_NOTIFY_POLLING 1
 
-/* Single-group ctor, csrc/layerwise.cpp:507-646.  The SSD arguments are
- * outside this library (the Python shim rejects non-empty ones); a uniform SWA
+/* Single-group ctor, csrc/layerwise.cpp:507-646.  The SSD files of the
+ * reference's ctor are served by fkv_ssd_open / fkv_ssd_transfer, which the
+ * caller runs before the restore (the Python operator does); a uniform SWA
  * sidecar is attached afterwards with fkv_layerwise_init_swa. */
 int fkv_layerwise_create(const fkv_layerwise_params *params, fkv_layerwise **out);
 

@@ -1,0 +1,294 @@
+// A consumer of libfkv_hip.so that knows nothing but include/fkv_transfer.h and
+// the HIP runtime: no Python, no torch.  Moves blocks of a vLLM-shaped cache
+// through every engine of the library and checks each byte against a plain
+// host model.  Also the program that is run with the library's host code built
+// under AddressSanitizer.
+#include <hip/hip_runtime.h>
+#include <sys/eventfd.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <numeric>
+#include <random>
+#include <vector>
+
+#include "fkv_transfer.h"
+
+#define HIP_OK(x)                                                                          \
+  do {                                                                                     \
+    hipError_t e_ = (x);                                                                   \
+    if (e_ != hipSuccess) {                                                                \
+      fprintf(stderr, "%s:%d %s: %s\n", __FILE__, __LINE__, #x, hipGetErrorString(e_));    \
+      return 1;                                                                            \
+    }                                                                                      \
+  } while (0)
+#define FKV_OK_OR_DIE(x)                                                                   \
+  do {                                                                                     \
+    int rc_ = (x);                                                                         \
+    if (rc_ != FKV_OK) {                                                                   \
+      fprintf(stderr, "%s:%d %s -> %d: %s\n", __FILE__, __LINE__, #x, rc_, fkv_last_error()); \
+      return 1;                                                                            \
+    }                                                                                      \
+  } while (0)
+
+namespace {
+constexpr int L = 6, KV = 2, N = 96, NH = 80;
+constexpr int64_t CHUNK = 4096 + 512; // not a power of two
+constexpr int64_t GKS = N * CHUNK, GBS = CHUNK, GLS = KV * N * CHUNK;           // per layer [kv, N, chunk]
+constexpr int64_t CKS = CHUNK, CLS = KV * CHUNK, CBS = (int64_t)L * KV * CHUNK; // [NH, L, kv, chunk]
+
+struct Model {
+  std::vector<std::vector<uint8_t>> gpu; // L tensors
+  std::vector<uint8_t> host;
+  void put(const std::vector<int64_t> &g, const std::vector<int64_t> &c, bool h2d) {
+    for (size_t i = 0; i < g.size(); ++i)
+      for (int l = 0; l < L; ++l)
+        for (int kv = 0; kv < KV; ++kv) {
+          uint8_t *gp = gpu[l].data() + kv * GKS + g[i] * GBS;
+          uint8_t *cp = host.data() + c[i] * CBS + l * CLS + kv * CKS;
+          if (h2d)
+            memcpy(gp, cp, CHUNK);
+          else
+            memcpy(cp, gp, CHUNK);
+        }
+  }
+};
+
+std::vector<int64_t> pick(std::mt19937_64 &rng, int pool, int n) {
+  std::vector<int64_t> v(pool);
+  std::iota(v.begin(), v.end(), 0);
+  std::shuffle(v.begin(), v.end(), rng);
+  v.resize(n);
+  return v;
+}
+} // namespace
+
+int main() {
+  int ndev = 0;
+  HIP_OK(hipGetDeviceCount(&ndev));
+  if (ndev < 1) {
+    fprintf(stderr, "no GPU\n");
+    return 2;
+  }
+  HIP_OK(hipSetDevice(0));
+  std::mt19937_64 rng(11);
+  Model m;
+  m.gpu.assign(L, std::vector<uint8_t>(GLS));
+  m.host.assign((size_t)NH * CBS, 0);
+  std::vector<void *> dev(L);
+  std::vector<uint64_t> ptrs(L);
+  for (int l = 0; l < L; ++l) {
+    for (auto &b : m.gpu[l])
+      b = (uint8_t)rng();
+    HIP_OK(hipMalloc(&dev[l], GLS));
+    HIP_OK(hipMemcpy(dev[l], m.gpu[l].data(), GLS, hipMemcpyHostToDevice));
+    ptrs[l] = (uint64_t)(uintptr_t)dev[l];
+  }
+  void *host = nullptr;
+  FKV_OK_OR_DIE(fkv_host_alloc((size_t)NH * CBS, &host));
+  memset(host, 0, (size_t)NH * CBS);
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+
+  auto check = [&](const char *what) -> int {
+    HIP_OK(hipDeviceSynchronize());
+    if (memcmp(host, m.host.data(), m.host.size())) {
+      fprintf(stderr, "%s: host pool differs\n", what);
+      return 1;
+    }
+    std::vector<uint8_t> back(GLS);
+    for (int l = 0; l < L; ++l) {
+      HIP_OK(hipMemcpy(back.data(), dev[l], GLS, hipMemcpyDeviceToHost));
+      if (back != m.gpu[l]) {
+        fprintf(stderr, "%s: device layer %d differs\n", what, l);
+        return 1;
+      }
+    }
+    return 0;
+  };
+
+  int cases = 0, refused = 0;
+  // ---- fkv_transfer_kv_blocks: kernel, copy engine (chosen and each forced strategy) ----
+  struct Mode { int use_ce, force; const char *name; };
+  const Mode modes[] = {{0, -1, "kernel"}, {1, -1, "ce"}, {2, -1, "auto"}, {1, 0, "ce0"},
+                        {1, 1, "ce1"}, {1, 2, "ce2"}, {1, 3, "ce3"}, {1, 4, "ce4"}};
+  for (const Mode &mode : modes)
+    for (int pattern = 0; pattern < 3; ++pattern) {
+      const int n = pattern == 0 ? 40 : pattern == 1 ? 1 : 17;
+      std::vector<int64_t> g = pick(rng, N, n), c = pick(rng, NH, n);
+      if (pattern == 0) { // runs of consecutive ids on both sides
+        std::iota(g.begin(), g.end(), 8);
+        std::iota(c.begin(), c.end(), 3);
+      }
+      fkv_transfer_desc d;
+      memset(&d, 0, sizeof(d));
+      d.backend = FKV_BACKEND_VLLM;
+      d.num_layers_total = L;
+      d.gpu_tensor_ptrs = ptrs.data();
+      d.num_gpu_tensor_ptrs = L;
+      d.device = -1;
+      d.gpu_kv_stride = GKS, d.gpu_block_stride = GBS, d.gpu_layer_stride = GLS;
+      d.cpu_ptr = host;
+      d.cpu_kv_stride = CKS, d.cpu_layer_stride = CLS, d.cpu_block_stride = CBS;
+      d.chunk_size = CHUNK;
+      d.start_layer_id = 0, d.num_layers = L, d.kv_dim = KV, d.num_blocks = n;
+      d.gpu_block_ids = g.data(), d.cpu_block_ids = c.data();
+      d.use_ce_transfer = mode.use_ce;
+      d.transfer_num_cta = 4;
+      d.sync = 1;
+      fkv_ce_config_default(&d.ce);
+      d.ce.is_blockfirst = 1;
+      d.ce.force_path = mode.force;
+      d.ce.path_opt_enabled = 1;
+      d.is_host_to_device = 0;
+      if (mode.force >= 0) { // a forced strategy that does not fit the ids is refused, not run
+        const int rc = fkv_transfer_kv_blocks(&d, stream);
+        if (rc == FKV_ERR_INVALID_ARG && strstr(fkv_last_error(), "does not fit")) {
+          ++refused;
+          continue;
+        }
+        FKV_OK_OR_DIE(rc);
+      } else {
+        FKV_OK_OR_DIE(fkv_transfer_kv_blocks(&d, stream));
+      }
+      m.put(g, c, false);
+      if (check(mode.name))
+        return 1;
+      std::vector<int64_t> g2 = pick(rng, N, n);
+      d.gpu_block_ids = g2.data();
+      d.is_host_to_device = 1;
+      FKV_OK_OR_DIE(fkv_transfer_kv_blocks(&d, stream));
+      m.put(g2, c, true);
+      if (check(mode.name))
+        return 1;
+      ++cases;
+    }
+
+  // ---- TP group with one rank ----
+  {
+    const int64_t ks = GKS, bs = GBS, ls = GLS, cs = CHUNK, did = 0;
+    fkv_tp_group_params p;
+    memset(&p, 0, sizeof(p));
+    p.num_gpus = 1, p.num_tensors_per_gpu = L;
+    p.gpu_block_ptrs_flat = ptrs.data();
+    p.cpu_blocks_ptr = host;
+    p.num_layers = L;
+    p.gpu_kv_strides = &ks, p.gpu_block_strides = &bs, p.gpu_layer_strides = &ls;
+    p.gpu_chunk_sizes = &cs, p.gpu_device_ids = &did;
+    fkv_ce_config_default(&p.ce);
+    p.ce.is_blockfirst = 1;
+    fkv_tp_group *grp = nullptr;
+    FKV_OK_OR_DIE(fkv_tp_group_create(&p, &grp));
+    for (int use_ce = 0; use_ce < 2; ++use_ce) {
+      std::vector<int64_t> g = pick(rng, N, 23), c = pick(rng, NH, 23);
+      FKV_OK_OR_DIE(fkv_tp_group_transfer(grp, g.data(), c.data(), 23, CKS, CLS, CBS, CBS, 4, 0,
+                                          use_ce, 0, L, KV, 8, "sharded", 0));
+      m.put(g, c, false);
+      if (check("tp d2h"))
+        return 1;
+      std::vector<int64_t> g2 = pick(rng, N, 23);
+      FKV_OK_OR_DIE(fkv_tp_group_transfer(grp, g2.data(), c.data(), 23, CKS, CLS, CBS, CBS, 4, 1,
+                                          use_ce, 0, L, KV, 8, "sharded", 0));
+      m.put(g2, c, true);
+      if (check("tp h2d"))
+        return 1;
+      ++cases;
+    }
+    if (fkv_tp_group_transfer(grp, nullptr, nullptr, 3, CKS, CLS, CBS, CBS, 4, 1, 0, 0, L, KV, 8,
+                              "sharded", 0) == FKV_OK) {
+      fprintf(stderr, "null id arrays were accepted\n");
+      return 1;
+    }
+    fkv_tp_group_destroy(grp);
+  }
+
+  // ---- layerwise restore, both notification modes, eventfds read back ----
+  {
+    const int64_t ks = GKS, bs = GBS, ls = GLS, cs = CHUNK, did = 0;
+    std::vector<int32_t> fds(2 * L);
+    for (auto &fd : fds)
+      fd = eventfd(0, EFD_SEMAPHORE | EFD_NONBLOCK);
+    fkv_layerwise_params p;
+    memset(&p, 0, sizeof(p));
+    p.num_gpus = 1, p.num_tensors_per_gpu = L;
+    p.gpu_block_ptrs_flat = ptrs.data();
+    p.cpu_blocks_ptr = host;
+    p.num_layers = L, p.tp_size = 1;
+    p.gpu_kv_strides = &ks, p.gpu_block_strides = &bs, p.gpu_layer_strides = &ls;
+    p.gpu_chunk_sizes = &cs, p.gpu_device_ids = &did;
+    p.layer_eventfds = fds.data(), p.num_layer_eventfds = (int32_t)fds.size();
+    fkv_ce_config_default(&p.ce);
+    p.ce.is_blockfirst = 1;
+    fkv_layerwise *lw = nullptr;
+    FKV_OK_OR_DIE(fkv_layerwise_create(&p, &lw));
+    for (int notify = 0; notify < 2; ++notify)
+      for (int use_ce = 0; use_ce < 2; ++use_ce) {
+        std::vector<int64_t> g = pick(rng, N, 31), c = pick(rng, NH, 31);
+        const int gran = 1 + (notify + use_ce) % 3;
+        FKV_OK_OR_DIE(fkv_layerwise_transfer(lw, g.data(), c.data(), 31, CBS, CKS, CLS, CBS, 4,
+                                             use_ce, L, gran, KV, 8, notify, "sharded", notify, 0));
+        FKV_OK_OR_DIE(fkv_layerwise_synchronize(lw));
+        m.put(g, c, true);
+        if (check("layerwise"))
+          return 1;
+        for (int l = 0; l < L; ++l) { // one unit per layer on the chosen counter set
+          uint64_t v = 0;
+          if (read(fds[notify * L + l], &v, 8) != 8 || v != 1) {
+            fprintf(stderr, "layer %d was not announced\n", l);
+            return 1;
+          }
+        }
+        ++cases;
+      }
+    fkv_layerwise_destroy(lw);
+    for (int fd : fds)
+      close(fd);
+  }
+
+  // ---- engine blocks <-> dense device buffer ----
+  {
+    const int n = 29;
+    void *buf = nullptr;
+    HIP_OK(hipMalloc(&buf, (size_t)n * CBS));
+    std::vector<int64_t> g = pick(rng, N, n);
+    fkv_layout_transform_desc t;
+    memset(&t, 0, sizeof(t));
+    t.backend = FKV_BACKEND_VLLM, t.num_layers_total = L;
+    t.gpu_tensor_ptrs = ptrs.data(), t.num_gpu_tensor_ptrs = L, t.device = -1;
+    t.gpu_kv_stride = GKS, t.gpu_block_stride = GBS, t.gpu_layer_stride = GLS;
+    t.buffer_ptr = buf;
+    t.buffer_layer_stride = CLS, t.buffer_kv_stride = CKS, t.buffer_block_stride = CBS;
+    t.chunk_size = CHUNK, t.num_layers = L, t.kv_dim = KV, t.num_blocks = n;
+    t.gpu_block_ids = g.data();
+    t.sync = 1;
+    FKV_OK_OR_DIE(fkv_layout_transform(&t, stream));
+    std::vector<uint8_t> got((size_t)n * CBS), want((size_t)n * CBS);
+    HIP_OK(hipMemcpy(got.data(), buf, got.size(), hipMemcpyDeviceToHost));
+    for (int i = 0; i < n; ++i)
+      for (int l = 0; l < L; ++l)
+        for (int kv = 0; kv < KV; ++kv)
+          memcpy(want.data() + i * CBS + l * CLS + kv * CKS, m.gpu[l].data() + kv * GKS + g[i] * GBS,
+                 CHUNK);
+    if (got != want) {
+      fprintf(stderr, "layout transform differs\n");
+      return 1;
+    }
+    HIP_OK(hipFree(buf));
+    ++cases;
+  }
+
+  fkv_stats st;
+  fkv_get_stats(&st);
+  HIP_OK(hipStreamDestroy(stream));
+  FKV_OK_OR_DIE(fkv_host_free(host));
+  for (void *p : dev)
+    HIP_OK(hipFree(p));
+  printf("ok: %d cases through the C ABI (%d forced strategies refused), %llu calls, "
+         "%llu kernel launches, %llu DMA copies\n",
+         cases, refused, (unsigned long long)st.calls, (unsigned long long)st.kernel_launches,
+         (unsigned long long)st.dma_copies);
+  return 0;
+}

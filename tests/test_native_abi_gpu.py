@@ -1,0 +1,32 @@
+"""A consumer of the library that is neither Python nor torch: the native program
+of tests/native/abi_roundtrip_driver.cpp drives every engine through the C ABI
+and checks each byte against its own host model.  It runs twice: against the
+shipped library, and against a build of the library whose host code is under
+AddressSanitizer (the device code is the same).  Both are built beforehand by
+``make -C tests/native`` (``__graft_entry__.build()`` does it)."""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+BUILD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "native", "build")
+
+
+def run(exe, **env):
+    assert os.path.exists(exe), f"{exe} is missing: run make -C tests/native"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=300,
+                       env=dict(os.environ, **env))
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
+    assert "ok: 25 cases through the C ABI" in r.stdout, r.stdout
+    return r
+
+
+def test_native_consumer_of_the_c_abi(gpu_device):
+    run(os.path.join(BUILD, "abi_roundtrip_driver"))
+
+
+def test_host_code_under_address_sanitizer(gpu_device):
+    r = run(os.path.join(BUILD, "asan", "abi_roundtrip_driver"),
+            ASAN_OPTIONS="protect_shadow_gap=0:detect_leaks=0:verify_asan_link_order=0")
+    assert "AddressSanitizer" not in r.stderr
