@@ -248,6 +248,143 @@ int main() {
       close(fd);
   }
 
+  // ---- multi-group restore with a uniform sliding-window sidecar ----
+  {
+    constexpr int OL = 4, NB = 24, NHB = 20, NS = 10, NHS = 12; // original layers, pool sizes
+    constexpr int64_t C0 = 512, C1 = 256, CS = 1024;           // chunk of main, indexer, sidecar
+    constexpr int64_t BLK = 4 * C0 + 3 * C1, OFF1 = 4 * C0;    // byte-flat host block
+    const int group_layers[2] = {4, 3};
+    const int64_t group_chunk[2] = {C0, C1};
+    std::vector<std::vector<uint8_t>> gmodel[2];
+    std::vector<void *> gdev[2];
+    std::vector<uint64_t> gptrs[2];
+    for (int g = 0; g < 2; ++g)
+      for (int l = 0; l < group_layers[g]; ++l) {
+        gmodel[g].emplace_back((size_t)NB * group_chunk[g], 0);
+        void *p = nullptr;
+        HIP_OK(hipMalloc(&p, NB * group_chunk[g]));
+        HIP_OK(hipMemset(p, 0, NB * group_chunk[g]));
+        gdev[g].push_back(p);
+        gptrs[g].push_back((uint64_t)(uintptr_t)p);
+      }
+    std::vector<std::vector<uint8_t>> smodel(OL, std::vector<uint8_t>((size_t)NS * CS, 0));
+    std::vector<void *> sdev(OL);
+    std::vector<uint64_t> sptrs(OL);
+    for (int l = 0; l < OL; ++l) {
+      HIP_OK(hipMalloc(&sdev[l], NS * CS));
+      HIP_OK(hipMemset(sdev[l], 0, NS * CS));
+      sptrs[l] = (uint64_t)(uintptr_t)sdev[l];
+    }
+    void *mhost = nullptr, *shost = nullptr;
+    FKV_OK_OR_DIE(fkv_host_alloc((size_t)NHB * BLK, &mhost));
+    FKV_OK_OR_DIE(fkv_host_alloc((size_t)OL * NHS * CS, &shost)); // [layer, 1, block, chunk]
+    uint8_t *mh = static_cast<uint8_t *>(mhost), *sh = static_cast<uint8_t *>(shost);
+    for (size_t i = 0; i < (size_t)NHB * BLK; ++i)
+      mh[i] = (uint8_t)rng();
+    for (size_t i = 0; i < (size_t)OL * NHS * CS; ++i)
+      sh[i] = (uint8_t)rng();
+
+    fkv_layer_group groups[2], swa;
+    int64_t kvs[2], bls[2], lys[2], chs[2];
+    for (int g = 0; g < 2; ++g) {
+      memset(&groups[g], 0, sizeof(groups[g]));
+      kvs[g] = NB * group_chunk[g], bls[g] = group_chunk[g], lys[g] = NB * group_chunk[g];
+      chs[g] = group_chunk[g];
+      groups[g].num_layers = group_layers[g];
+      groups[g].num_tensors_per_gpu = group_layers[g];
+      groups[g].gpu_block_ptrs_flat = gptrs[g].data();
+      groups[g].cpu_offset_bytes = g ? OFF1 : 0;
+      groups[g].h2d_cpu_kv_stride = group_chunk[g];
+      groups[g].h2d_cpu_layer_stride = group_chunk[g];
+      groups[g].cpu_block_stride = BLK;
+      groups[g].cpu_tp_stride = BLK;
+      groups[g].gpu_kv_strides = &kvs[g], groups[g].gpu_block_strides = &bls[g];
+      groups[g].gpu_layer_strides = &lys[g], groups[g].gpu_chunk_sizes = &chs[g];
+    }
+    const int32_t member_offsets[OL + 1] = {0, 1, 3, 5, 7};
+    const fkv_layer_member members[7] = {{0, 0}, {0, 1}, {1, 0}, {0, 2}, {1, 1}, {0, 3}, {1, 2}};
+    const int64_t did = 0;
+    std::vector<int32_t> fds(OL);
+    for (auto &fd : fds)
+      fd = eventfd(0, EFD_SEMAPHORE | EFD_NONBLOCK);
+    fkv_layerwise_mg_params p;
+    memset(&p, 0, sizeof(p));
+    p.num_gpus = 1, p.num_original_layers = OL, p.tp_size = 1, p.num_groups = 2;
+    p.groups = groups, p.member_offsets = member_offsets, p.members = members;
+    p.cpu_blocks_ptr = mhost, p.gpu_device_ids = &did;
+    p.layer_eventfds = fds.data(), p.num_layer_eventfds = OL;
+    fkv_ce_config_default(&p.ce);
+    p.ce.is_blockfirst = 1;
+    fkv_layerwise *lw = nullptr;
+    FKV_OK_OR_DIE(fkv_layerwise_create_multi_group(&p, &lw));
+    const int64_t sks = NS * CS, sbs = CS, sls = NS * CS, scs = CS;
+    memset(&swa, 0, sizeof(swa));
+    swa.num_layers = OL, swa.num_tensors_per_gpu = OL, swa.gpu_block_ptrs_flat = sptrs.data();
+    swa.gpu_kv_strides = &sks, swa.gpu_block_strides = &sbs, swa.gpu_layer_strides = &sls;
+    swa.gpu_chunk_sizes = &scs;
+    FKV_OK_OR_DIE(fkv_layerwise_init_swa(lw, &swa, shost));
+    for (int round = 0; round < 4; ++round) {
+      const int n = 9, ns = 4;
+      std::vector<int64_t> g = pick(rng, NB, n), c = pick(rng, NHB, n);
+      std::vector<int64_t> sg = pick(rng, NS, ns), sc = pick(rng, NHS, ns);
+      fkv_layerwise_call call;
+      memset(&call, 0, sizeof(call));
+      call.gpu_block_ids = g.data(), call.cpu_block_ids = c.data(), call.num_blocks = n;
+      call.multi_group = 1;
+      call.transfer_cta_num = 4, call.use_ce_transfer = round & 1, call.kv_dim = 1;
+      call.num_kv_heads = 1, call.counter_id = 0, call.notify_mode = round >> 1;
+      call.kv_shared_across_ranks_mode = "sharded";
+      call.swa_num_blocks = ns, call.swa_gpu_block_ids = sg.data(), call.swa_cpu_block_ids = sc.data();
+      call.swa_h2d_cpu_kv_stride = NHS * CS, call.swa_h2d_cpu_layer_stride = NHS * CS;
+      call.swa_cpu_block_stride = CS;
+      FKV_OK_OR_DIE(fkv_layerwise_transfer_call(lw, &call));
+      FKV_OK_OR_DIE(fkv_layerwise_synchronize(lw));
+      for (int i = 0; i < n; ++i)
+        for (int gi = 0; gi < 2; ++gi)
+          for (int l = 0; l < group_layers[gi]; ++l)
+            memcpy(gmodel[gi][l].data() + g[i] * group_chunk[gi],
+                   mh + c[i] * BLK + (gi ? OFF1 : 0) + l * group_chunk[gi], group_chunk[gi]);
+      for (int i = 0; i < ns; ++i)
+        for (int l = 0; l < OL; ++l)
+          memcpy(smodel[l].data() + sg[i] * CS, sh + (size_t)l * NHS * CS + sc[i] * CS, CS);
+      HIP_OK(hipDeviceSynchronize());
+      std::vector<uint8_t> back;
+      for (int gi = 0; gi < 2; ++gi)
+        for (int l = 0; l < group_layers[gi]; ++l) {
+          back.resize(gmodel[gi][l].size());
+          HIP_OK(hipMemcpy(back.data(), gdev[gi][l], back.size(), hipMemcpyDeviceToHost));
+          if (back != gmodel[gi][l]) {
+            fprintf(stderr, "multi-group: group %d layer %d differs\n", gi, l);
+            return 1;
+          }
+        }
+      for (int l = 0; l < OL; ++l) {
+        back.resize(smodel[l].size());
+        HIP_OK(hipMemcpy(back.data(), sdev[l], back.size(), hipMemcpyDeviceToHost));
+        if (back != smodel[l]) {
+          fprintf(stderr, "multi-group: sidecar layer %d differs\n", l);
+          return 1;
+        }
+        uint64_t v = 0;
+        if (read(fds[l], &v, 8) != 8 || v != 1) {
+          fprintf(stderr, "multi-group: original layer %d was not announced once\n", l);
+          return 1;
+        }
+      }
+      ++cases;
+    }
+    fkv_layerwise_destroy(lw);
+    for (int fd : fds)
+      close(fd);
+    for (int g = 0; g < 2; ++g)
+      for (void *q : gdev[g])
+        HIP_OK(hipFree(q));
+    for (void *q : sdev)
+      HIP_OK(hipFree(q));
+    FKV_OK_OR_DIE(fkv_host_free(mhost));
+    FKV_OK_OR_DIE(fkv_host_free(shost));
+  }
+
   // ---- engine blocks <-> dense device buffer ----
   {
     const int n = 29;
