@@ -401,6 +401,13 @@ def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32):
     reqs = w.requests
     per_dir = max(1, min(streams_per_direction, len(reqs) // 2))
     pool = [[torch.cuda.Stream() for _ in range(per_dir)] for _ in range(2)]
+    if per_dir == 1:
+        # one put stream and one get stream: take a pair that does not share a hardware queue
+        from flexkv_amd.c_ext import streams_run_concurrently
+        spare = []
+        while not streams_run_concurrently(pool[0][0], pool[1][0]) and len(spare) < 8:
+            spare.append(pool[1][0])       # keep it alive so the next one is a different stream
+            pool[1][0] = torch.cuda.Stream()
     streams = [pool[i % 2][(i // 2) % per_dir] for i in range(len(reqs))]
     lat = [[] for _ in reqs]
     walls = []

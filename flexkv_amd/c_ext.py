@@ -187,6 +187,16 @@ def layout_transform(
     check(_L.fkv_layout_transform(ctypes.byref(d), _current_stream_handle()))
 
 
+def streams_run_concurrently(stream_a, stream_b, device: int = -1) -> bool:
+    """Whether kernels on the two torch streams can overlap, i.e. whether the
+    streams sit on different hardware queues of this process.  Synchronises both."""
+    out = ctypes.c_int32(0)
+    check(_L.fkv_streams_run_concurrently(int(device), ctypes.c_void_p(stream_a.cuda_stream),
+                                          ctypes.c_void_p(stream_b.cuda_stream),
+                                          ctypes.byref(out)))
+    return bool(out.value)
+
+
 def last_transfer_path() -> str:
     """Name of the path the last transfer issued by this thread took: KERNEL or
     one of the copy-engine strategies."""

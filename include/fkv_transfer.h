@@ -530,6 +530,16 @@ void fkv_reset_stats(void);
 int fkv_measure_link_peak(int32_t device, size_t bytes, int32_t reps,
                           int32_t direction, double *best_gbps, double *median_gbps);
 
+/* Whether kernels on two streams of `device` can run at the same time.  A
+ * process has few hardware queues (GPU_MAX_HW_QUEUES, 4 by default) and streams
+ * that share one run their kernels one after the other: a stream of puts and a
+ * stream of gets on the same queue move the one-way rate in sum.  The call times
+ * a short wait kernel on `stream_a` alone and then on both streams at once (it
+ * synchronises both streams) and sets *concurrent to 1 when the pair took less
+ * than 1.5x the single one.  No counterpart in the reference. */
+int fkv_streams_run_concurrently(int32_t device, void *stream_a, void *stream_b,
+                                 int32_t *concurrent);
+
 #ifdef __cplusplus
 }
 #endif

@@ -244,3 +244,15 @@ def test_pageable_host_tensor_is_refused_by_the_kernel_path(gpu_device):
     s.host_ref[:] = 0
     s.oracle_transfer(ids.numpy(), ids.numpy(), False)
     np.testing.assert_array_equal(pageable.numpy(), s.host_ref)
+
+
+def test_streams_run_concurrently_tells_hardware_queue_sharing(gpu_device):
+    """The same stream never overlaps with itself; among six streams of a process
+    with four hardware queues some pair does."""
+    import torch
+    from flexkv_amd.c_ext import streams_run_concurrently
+    streams = [torch.cuda.Stream() for _ in range(6)]
+    assert streams_run_concurrently(streams[0], streams[0]) is False
+    table = [[streams_run_concurrently(a, b) for b in streams] for a in streams]
+    assert any(table[i][j] for i in range(6) for j in range(6) if i != j), table
+    assert all(not table[i][i] for i in range(6))
