@@ -474,10 +474,10 @@ int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
     a.vec = p.vec;
     a.nt_store = p.h2d ? 1 : 0;
     // Packed short chunks cost a wavefront more address arithmetic per request, so
-    // the host->GPU direction, which lives on requests in flight, gets half as many
-    // workgroups again: 16 x 64 lanes reach 45 GB/s on 2304-byte chunks, 24 x 64
-    // reach 55.8, 32 x 64 reach 56.2.
-    a.packed_grid_pct = p.h2d ? 150 : 100;
+    // such launches get half as many workgroups again.  Host->GPU, 2304-byte chunks:
+    // 16 x 64 lanes reach 45 GB/s, 24 x 64 reach 55.8, 32 x 64 reach 56.2; GPU->host:
+    // 48 x 64 lanes 50.7 GB/s, 72 x 64 52.5, 96 x 64 53.0.
+    a.packed_grid_pct = 150;
     a.xcd_mask = p.xcd_mask;
     a.claim = p.claims ? p.claims + l0 : nullptr; // a launch per first layer at most
     FKV_TRY(launch_copy_kernel(a, p.workgroups, p.threads, stream));
