@@ -608,18 +608,26 @@ namespace {
 // device, reused.
 int wait_for_work_queued_so_far(hipStream_t stream) {
   constexpr int kMaxDevices = 64;
-  thread_local hipEvent_t events[kMaxDevices] = {};
+  struct PerThread { // events go when their thread ends
+    hipEvent_t ev[kMaxDevices] = {};
+    ~PerThread() {
+      for (hipEvent_t e : ev)
+        if (e && hipEventDestroy(e) != hipSuccess)
+          (void)hipGetLastError();
+    }
+  };
+  thread_local PerThread mine;
   int device = 0;
   FKV_HIP_TRY(hipGetDevice(&device));
   if (device < 0 || device >= kMaxDevices) {
     FKV_HIP_TRY(hipStreamSynchronize(stream));
     return FKV_OK;
   }
-  if (!events[device])
-    FKV_HIP_TRY(hipEventCreateWithFlags(&events[device],
+  if (!mine.ev[device])
+    FKV_HIP_TRY(hipEventCreateWithFlags(&mine.ev[device],
                                         hipEventBlockingSync | hipEventDisableTiming));
-  FKV_HIP_TRY(hipEventRecord(events[device], stream));
-  FKV_HIP_TRY(hipEventSynchronize(events[device]));
+  FKV_HIP_TRY(hipEventRecord(mine.ev[device], stream));
+  FKV_HIP_TRY(hipEventSynchronize(mine.ev[device]));
   return FKV_OK;
 }
 } // namespace
