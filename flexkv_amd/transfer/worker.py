@@ -455,7 +455,10 @@ class GPUCPUTransferWorker(TransferWorkerBase):
                  layer_groups: Optional[List[LayerGroupSpec]] = None,
                  gpu_blocks_per_group: Optional[List[List[Any]]] = None,
                  gpu_layouts_per_group: Optional[List[KVCacheLayout]] = None,
-                 allow_pageable_host: Optional[bool] = None) -> None:
+                 allow_pageable_host: Optional[bool] = None,
+                 ssd_files: Optional[Dict[int, List[str]]] = None,
+                 ssd_kv_layout: Optional[Union[KVCacheLayout, MultiGroupBlockLayout]] = None,
+                 num_blocks_per_file: int = 0) -> None:
         super().__init__(worker_id, transfer_conn, finished_ops_queue, op_buffer_tensor)
         # the device first: everything below creates state on the current device
         torch.cuda.set_device(gpu_device_id)
@@ -499,6 +502,14 @@ class GPUCPUTransferWorker(TransferWorkerBase):
         self.ce_path_opt = env.ce_path_opt
         self.ce_segment_threshold = env.ce_segment_threshold
         self.ce_enable_memcpy2d = env.enable_ce_memcpy2d
+        # A pinned pool lives in the process that allocated it (existing memory cannot
+        # be registered on every platform), so the worker that owns the pool can also
+        # serve its H2DISK / DISK2H ops: given SSD files it is both workers in one.
+        self.ssd: Optional[SSDPoolMover] = None
+        if ssd_files:
+            self.ssd = SSDPoolMover(self.cpu_tensor, ssd_files, cpu_kv_layout, ssd_kv_layout, dtype,
+                                    num_blocks_per_file,
+                                    multi_group=self.group_transfer_params is not None)
 
     def _init_multi_group(self, gpu_blocks_per_group, gpu_layouts_per_group,
                           cpu_kv_layout: MultiGroupBlockLayout, layer_groups) -> None:
@@ -559,6 +570,17 @@ class GPUCPUTransferWorker(TransferWorkerBase):
 
     def launch_transfer(self, transfer_op: WorkerTransferOp) -> bool:
         src, dst = self.get_transfer_block_ids(transfer_op)
+        if transfer_op.transfer_type in (TransferType.H2DISK, TransferType.DISK2H):
+            if self.ssd is None:
+                raise ValueError(f"Invalid transfer type: {transfer_op.transfer_type} for "
+                                 "GPUCPUTransferWorker without SSD files")
+            t0 = time.time()
+            self.ssd.move(src.contiguous(), dst.contiguous(), transfer_op.transfer_type,
+                          "GPUCPUTransferWorker")
+            self._log_transfer_performance(
+                transfer_op, self.ssd.bytes_per_block * transfer_op.valid_block_num, t0,
+                time.time())
+            return True
         with torch.cuda.stream(self.transfer_stream):
             t0 = time.time()
             self._transfer_impl(src, dst, transfer_op.transfer_type)
@@ -566,6 +588,11 @@ class GPUCPUTransferWorker(TransferWorkerBase):
         self._log_transfer_performance(
             transfer_op, self._bytes_per_block * transfer_op.valid_block_num, t0, t1)
         return True
+
+    def shutdown(self) -> None:
+        if getattr(self, "ssd", None) is not None:
+            self.ssd.close()
+        super().shutdown()
 
 
 class tpGPUCPUTransferWorker(TransferWorkerBase):  # noqa: N801 - the reference's name
@@ -646,33 +673,28 @@ class tpGPUCPUTransferWorker(TransferWorkerBase):  # noqa: N801 - the reference'
         return True
 
 
-class CPUSSDDiskTransferWorker(TransferWorkerBase):
-    """Host pool <-> SSD files (worker.py:1522-1722): H2DISK and DISK2H ops, no GPU
-    involved.  The files of ``ssd_files`` (device -> paths) together hold
-    ``ssd_kv_layout.num_block`` blocks, striped over devices and files."""
+class SSDPoolMover:
+    """Host pool <-> SSD files for one pool (the arithmetic and the calls of
+    worker.py:1522-1722).  The files of ``ssd_files`` (device -> paths) together
+    hold ``ssd_kv_layout.num_block`` blocks, striped over devices and files."""
 
-    def __init__(self, worker_id: int, transfer_conn: Connection, finished_ops_queue,
-                 op_buffer_tensor: torch.Tensor, cpu_blocks: torch.Tensor,
-                 ssd_files: Dict[int, List[str]],
+    def __init__(self, cpu_blocks: torch.Tensor, ssd_files: Dict[int, List[str]],
                  cpu_kv_layout: Union[KVCacheLayout, MultiGroupBlockLayout],
                  ssd_kv_layout: Union[KVCacheLayout, MultiGroupBlockLayout], dtype: torch.dtype,
-                 num_blocks_per_file: int, layer_groups: Optional[List[LayerGroupSpec]] = None,
+                 num_blocks_per_file: int, multi_group: bool = False,
                  num_threads_per_device: int = 32) -> None:
         from ..c_ext import SSDIOCTX
-        super().__init__(worker_id, transfer_conn, finished_ops_queue, op_buffer_tensor)
-        self.cpu_blocks = materialize_worker_tensor(cpu_blocks)
-        self.ssd_files = ssd_files
+        self.cpu_blocks = cpu_blocks
         self.num_blocks_per_file = num_blocks_per_file
         self.num_files = sum(len(v) for v in ssd_files.values())
         self.round_robin = 1
         self.num_threads_per_device = num_threads_per_device
-        self.dtype = dtype
-        self.has_multi_group = layer_groups is not None
-        if self.has_multi_group:
+        self.multi_group = multi_group
+        if multi_group:
             # identical byte-flat blocks on both sides: a block moves as one piece
             self.block_stride_in_bytes = cpu_kv_layout.get_block_stride()
             self.kv_dim, self.num_layers = 1, 1
-            self._bytes_per_block = self.block_stride_in_bytes
+            self.bytes_per_block = self.block_stride_in_bytes
         else:
             if cpu_kv_layout.type != ssd_kv_layout.type:
                 raise ValueError("no support for different CPU and SSD KV cache layout type")
@@ -685,7 +707,7 @@ class CPUSSDDiskTransferWorker(TransferWorkerBase):
             self.block_stride_in_bytes = c.block
             self.cpu_kv_stride_in_bytes, self.cpu_layer_stride_in_bytes = c.kv, c.layer
             self.ssd_kv_stride_in_bytes, self.ssd_layer_stride_in_bytes = f.kv, f.layer
-            self._bytes_per_block = c.chunk * self.num_layers * self.kv_dim
+            self.bytes_per_block = c.chunk * self.num_layers * self.kv_dim
         env = global_env()
         try:
             self.ioctx = SSDIOCTX(ssd_files, len(ssd_files), env.iouring_entries, env.iouring_flags)
@@ -693,19 +715,18 @@ class CPUSSDDiskTransferWorker(TransferWorkerBase):
             logger.error("Error setting ssd ioctx: %s", e)
             raise RuntimeError("SSD Worker init failed") from e
 
-    def _transfer_impl(self, src_block_ids: torch.Tensor, dst_block_ids: torch.Tensor,
-                       transfer_type: TransferType) -> None:
+    def move(self, src_block_ids: torch.Tensor, dst_block_ids: torch.Tensor,
+             transfer_type: TransferType, who: str) -> None:
         from ..c_ext import transfer_kv_blocks_ssd
         if transfer_type == TransferType.H2DISK:
             ssd_ids, cpu_ids, is_read = dst_block_ids, src_block_ids, False
         elif transfer_type == TransferType.DISK2H:
             ssd_ids, cpu_ids, is_read = src_block_ids, dst_block_ids, True
         else:
-            raise ValueError(f"Invalid transfer type: {transfer_type} for "
-                             "CPUSSDDiskTransferWorker")
+            raise ValueError(f"Invalid transfer type: {transfer_type} for {who}")
         opt = global_env().ssd_io_opt
         base = self.cpu_blocks.data_ptr()
-        if self.has_multi_group:
+        if self.multi_group:
             b = self.block_stride_in_bytes
             transfer_kv_blocks_ssd(self.ioctx, torch.zeros(1, dtype=torch.int32), base, ssd_ids,
                                    cpu_ids, b, 0, b, 0, b, b, is_read, self.num_blocks_per_file,
@@ -718,18 +739,42 @@ class CPUSSDDiskTransferWorker(TransferWorkerBase):
             self.block_stride_in_bytes, is_read, self.num_blocks_per_file, self.round_robin,
             self.num_threads_per_device, self.kv_dim, opt)
 
-    def launch_transfer(self, transfer_op: WorkerTransferOp) -> bool:
-        src, dst = self.get_transfer_block_ids(transfer_op)
-        t0 = time.time()
-        self._transfer_impl(src.contiguous(), dst.contiguous(), transfer_op.transfer_type)
-        self._log_transfer_performance(
-            transfer_op, self._bytes_per_block * transfer_op.valid_block_num, t0, time.time())
-        return True
-
-    def shutdown(self) -> None:
+    def close(self) -> None:
         ctx = getattr(self, "ioctx", None)
         if ctx is not None:
             ctx.close()
+
+
+class CPUSSDDiskTransferWorker(TransferWorkerBase):
+    """Host pool <-> SSD files (worker.py:1522-1722): H2DISK and DISK2H ops, no GPU
+    involved."""
+
+    def __init__(self, worker_id: int, transfer_conn: Connection, finished_ops_queue,
+                 op_buffer_tensor: torch.Tensor, cpu_blocks: torch.Tensor,
+                 ssd_files: Dict[int, List[str]],
+                 cpu_kv_layout: Union[KVCacheLayout, MultiGroupBlockLayout],
+                 ssd_kv_layout: Union[KVCacheLayout, MultiGroupBlockLayout], dtype: torch.dtype,
+                 num_blocks_per_file: int, layer_groups: Optional[List[LayerGroupSpec]] = None,
+                 num_threads_per_device: int = 32) -> None:
+        super().__init__(worker_id, transfer_conn, finished_ops_queue, op_buffer_tensor)
+        self.cpu_blocks = materialize_worker_tensor(cpu_blocks)
+        self.ssd = SSDPoolMover(self.cpu_blocks, ssd_files, cpu_kv_layout, ssd_kv_layout, dtype,
+                                num_blocks_per_file, multi_group=layer_groups is not None,
+                                num_threads_per_device=num_threads_per_device)
+
+    def launch_transfer(self, transfer_op: WorkerTransferOp) -> bool:
+        src, dst = self.get_transfer_block_ids(transfer_op)
+        t0 = time.time()
+        self.ssd.move(src.contiguous(), dst.contiguous(), transfer_op.transfer_type,
+                      "CPUSSDDiskTransferWorker")
+        self._log_transfer_performance(
+            transfer_op, self.ssd.bytes_per_block * transfer_op.valid_block_num, t0, time.time())
+        return True
+
+    def shutdown(self) -> None:
+        ssd = getattr(self, "ssd", None)
+        if ssd is not None:
+            ssd.close()
         super().shutdown()
 
 

@@ -327,3 +327,49 @@ def test_layerwise_worker_stages_ssd_blocks_first(gpu_device, engine, tmp_path):
         assert torch.equal(tensors[l][:, dst].cpu(), want[src, l].transpose(0, 1)), l
     h.shutdown()
     assert h.process.exitcode == 0
+
+
+@pytest.mark.parametrize("entries", [0, 64], ids=["threads", "iouring"])
+def test_gpu_worker_that_also_serves_the_ssd_tier(gpu_device, engine, tmp_path, monkeypatch,
+                                                  entries):
+    """Three tiers behind one worker: the process that owns the pinned pool runs the
+    kernel path GPU<->host and the host<->SSD ops on the same pool.  put -> spill ->
+    wipe the host blocks -> stage back into other host blocks -> get."""
+    monkeypatch.setenv("FLEXKV_IOURING_ENTRIES", str(entries))
+    start, q, pool = engine
+    n_ssd, nfiles = 40, 2
+    tensors = _engine_tensors(gpu_device, 50)
+    want = [t.clone() for t in tensors]
+    cl = _cpu_layout(KVCacheLayoutType.BLOCKFIRST)
+    sl = KVCacheLayout(KVCacheLayoutType.BLOCKFIRST, L, n_ssd, T, H, D, kv_dim=2, num_kv_heads=H)
+    fl = sl.div_block(nfiles, padding=True)
+    paths = {0: [str(tmp_path / f"tier_{i}.bin") for i in range(nfiles)]}
+    for p in paths[0]:
+        with open(p, "wb") as fh:
+            fh.truncate(fl.get_total_elements() * 2)
+    h = start(GPUCPUTransferWorker, [TensorSharedHandle(t) for t in tensors],
+              PinnedPoolHandle(cl.kv_shape, DT), _gpu_layout(), cl, DT, 0,
+              ssd_files=paths, ssd_kv_layout=sl, num_blocks_per_file=n_ssd // nfiles)
+    rng = np.random.default_rng(12)
+    gpu_src = rng.permutation(N_GPU)[:9]
+    host_a = rng.permutation(N_CPU)[:9]
+    ssd_ids = rng.permutation(n_ssd)[:9]
+    host_b = np.setdiff1d(np.arange(N_CPU), host_a)[:9]
+    gpu_dst = np.setdiff1d(np.arange(N_GPU), gpu_src)[:9]
+    zero_src = np.setdiff1d(np.arange(N_GPU), np.concatenate([gpu_src, gpu_dst]))[:1]
+    for t in tensors:
+        t[:, zero_src] = 0                                      # a block of zeros to wipe with
+    torch.cuda.synchronize()
+    ops = [_op(TransferType.D2H, gpu_src, host_a, pool),        # put
+           _op(TransferType.H2DISK, host_a, ssd_ids),           # spill
+           _op(TransferType.D2H, np.repeat(zero_src, 9), host_a),   # wipe the host copies
+           _op(TransferType.DISK2H, ssd_ids, host_b),           # stage back elsewhere
+           _op(TransferType.H2D, host_b, gpu_dst)]              # get
+    for op in ops:
+        h.submit_transfer(op)
+        assert _collect(q, 1) == [(op.op_id, True, None)]
+    torch.cuda.synchronize()
+    for l in range(L):
+        assert torch.equal(tensors[l][:, gpu_dst], want[l][:, gpu_src]), l
+    h.shutdown()
+    assert h.process.exitcode == 0
