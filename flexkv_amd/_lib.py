@@ -201,6 +201,8 @@ SIGNATURES = {
     "fkv_ssd_close": (None, [c_void_p]),
     "fkv_layout_transform": (c_int32, [POINTER(LayoutTransformDesc), c_void_p]),
     "fkv_streams_run_concurrently": (c_int32, [c_int32, c_void_p, c_void_p, POINTER(c_int32)]),
+    "fkv_range_push": (c_int32, [c_char_p]),
+    "fkv_range_pop": (c_int32, []),
     "fkv_ssd_uses_iouring": (c_int32, [c_void_p]),
     "fkv_ssd_last_direct": (c_int32, [c_void_p]),
     "fkv_ssd_transfer": (c_int32, [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p,

@@ -649,6 +649,8 @@ int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream_v) {
 
   const uint64_t bytes =
       (uint64_t)d.num_blocks * d.num_layers * d.kv_dim * (uint64_t)d.chunk_size;
+  Range range("fkv %s %d blocks x %d layers (%.2f MB)", d.is_host_to_device ? "H2D" : "D2H",
+              d.num_blocks, d.num_layers, bytes / (1024.0 * 1024.0));
   // 0 kernel, 1 copy engine, 2 decide per transfer; FKV_TRANSFER_ENGINE overrides the caller.
   static const int forced_engine = [] {
     const char *v = std::getenv("FKV_TRANSFER_ENGINE");

@@ -36,6 +36,19 @@ void clear_error();
       return fkv_rc_;                                                          \
   } while (0)
 
+// ---- profiler ranges ------------------------------------------------------
+// Pushes a named range for its lifetime when FKV_ROCTX=1 (see fkv_range_push).
+class Range {
+public:
+  explicit Range(const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+  ~Range();
+  Range(const Range &) = delete;
+  Range &operator=(const Range &) = delete;
+
+private:
+  bool pushed_ = false;
+};
+
 // ---- counters -----------------------------------------------------------
 struct Stats {
   std::atomic<uint64_t> calls{0}, bytes_h2d{0}, bytes_d2h{0}, kernel_launches{0},

@@ -474,6 +474,8 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
 
   g->retire_previous();
   g->counter_id = c.counter_id;
+  Range range("fkv layerwise%s H2D %d blocks, %d sidecar blocks", g->multi_group ? " multi-group" : "",
+              c.num_blocks, c.swa_num_blocks);
 
   // csrc/layerwise.cpp:1112-1121, 1349-1360: only these three names are
   // meaningful for a restore; anything else is treated as "sharded".

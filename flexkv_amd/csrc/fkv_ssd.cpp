@@ -577,6 +577,9 @@ int fkv_ssd_transfer(fkv_ssd_ctx *ctx, int32_t start_layer, int32_t num_layers, 
   FKV_TRY(check_call(c));
   if (num_blocks == 0 || num_layers == 0)
     return FKV_OK;
+  // the label of the reference's range, csrc/layerwise.cpp:1068-1073
+  fkv::Range range("%s Blocks (%d blocks, %.2fMB each)", is_read ? "SSD->CPU" : "CPU->SSD",
+                   num_blocks, (double)num_layers * kv_dim * chunk_size / (1024.0 * 1024.0));
   bool direct = direct_io_possible(c) &&
                 ctx->no_direct_pool.load(std::memory_order_relaxed) != (uintptr_t)cpu_ptr;
   for (int fd : ctx->fd_direct)

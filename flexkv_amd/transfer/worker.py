@@ -40,6 +40,7 @@ from typing import Any, Dict, List, Optional, Sequence, Tuple, Union
 import numpy as np
 import torch
 
+from .. import _lib
 from ..layout import (KVCacheLayout, KVCacheLayoutType, LayerGroupSpec, MultiGroupBlockLayout,
                       TransferStrides, gpu_block_type_from_tensor_count, gpu_strides_from_tensor,
                       multi_group_tables)
@@ -285,10 +286,15 @@ class TransferWorkerBase(ABC):
     def _run_one(self, op) -> None:
         ok: Union[bool, WorkerTransferResult] = False
         t_launch = time.perf_counter_ns()
+        layerwise = op.transfer_type == TransferType.LAYERWISE
+        # a range on the profiler's timeline per op, as the reference annotates (worker.py:556-587)
+        pushed = _lib.load().fkv_range_push(
+            (f"launch {op.transfer_type.name} op_id: {op.transfer_op_id}, graph_id: "
+             f"{op.transfer_graph_id}, num_blocks: "
+             f"{len(op.src_block_ids_h2d) if layerwise else op.valid_block_num}").encode())
         try:
             ok = self.launch_transfer(op)
         except Exception as e:  # noqa: BLE001 - a failed op is reported, not fatal
-            layerwise = op.transfer_type == TransferType.LAYERWISE
             logger.error(
                 "[FlexKV-IO] operation=transfer act=complete status=failed direction=%s "
                 "blocks=%d op_id=%d graph_id=%d mode=%s transfer_time=%.4fs error=%r",
@@ -297,6 +303,9 @@ class TransferWorkerBase(ABC):
                 op.transfer_op_id, op.transfer_graph_id,
                 "layerwise" if layerwise else "no-layerwise",
                 (time.perf_counter_ns() - t_launch) / 1e9, str(e), exc_info=True)
+        finally:
+            if pushed:
+                _lib.load().fkv_range_pop()
         t_done = time.perf_counter_ns()
         metrics = trace.build_worker_metrics(
             op, getattr(op, "prof_submitted_ns", 0), getattr(op, "_received_ns", t_done), t_launch,

@@ -530,6 +530,16 @@ void fkv_reset_stats(void);
 int fkv_measure_link_peak(int32_t device, size_t bytes, int32_t reps,
                           int32_t direction, double *best_gbps, double *median_gbps);
 
+/* Named ranges for a profiler's timeline (rocprofv3 --marker-trace), where the
+ * reference annotates with NVTX (csrc/layerwise.cpp:1073, 1380;
+ * flexkv/transfer/worker.py:556-587, 1062-1095).  With FKV_ROCTX=1 in the
+ * environment the two calls forward to roctxRangePushA / roctxRangePop of the
+ * ROCm marker library, loaded on first use; otherwise, or when the library is
+ * not installed, they do nothing.  The library brackets its own transfers the
+ * same way.  Return 1 when the range was forwarded, 0 when not. */
+int fkv_range_push(const char *label);
+int fkv_range_pop(void);
+
 /* Whether kernels on two streams of `device` can run at the same time.  A
  * process has few hardware queues (GPU_MAX_HW_QUEUES, 4 by default) and streams
  * that share one run their kernels one after the other: a stream of puts and a

@@ -1,6 +1,7 @@
 // Host-only sanitizer run of the SSD engine: random layouts and id lists, both
 // engines, both request modes; files vs a straightforward per-chunk model.
 #include "fkv_ssd.cpp"
+#include "fkv_ranges.cpp"
 #include <random>
 #include <cassert>
 namespace fkv {

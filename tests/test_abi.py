@@ -134,3 +134,20 @@ def test_host_registration_chunking():
         assert all(int(o + s) == int(o2) for o, s, o2 in zip(off, sz, off[1:]))
         if chunk and total > chunk:
             assert (sz[:-1] == chunk).all() and sz[-1] <= chunk
+
+
+def test_profiler_ranges_are_off_unless_asked_for():
+    """fkv_range_push / fkv_range_pop forward to the ROCm marker library only with
+    FKV_ROCTX=1 (read once per process, so each case runs in its own process)."""
+    import subprocess
+    import sys
+    code = ("from flexkv_amd import _lib; L = _lib.load(); "
+            "print(L.fkv_range_push(b'x'), L.fkv_range_pop())")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = {k: v for k, v in os.environ.items() if k != "FKV_ROCTX"}
+    off = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True,
+                         text=True, check=True).stdout.split()
+    assert off == ["0", "0"]
+    on = subprocess.run([sys.executable, "-c", code], cwd=root, env=dict(env, FKV_ROCTX="1"),
+                        capture_output=True, text=True, check=True).stdout.split()
+    assert on in (["1", "1"], ["0", "0"])       # 0 0 only where no marker library is installed

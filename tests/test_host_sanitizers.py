@@ -26,7 +26,7 @@ def build_and_run(tmp_path, driver, sanitizer, extra=()):
     cmd = [CLANG, "-std=c++17", "-O1", "-g", *sanitizer, "-fno-omit-frame-pointer",
            "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", "-I" + os.path.join(ROOT, "include"),
            "-I" + os.path.join(ROOT, "flexkv_amd", "csrc"), *extra,
-           os.path.join(ROOT, "tests", "native", driver), "-o", exe, "-pthread"]
+           os.path.join(ROOT, "tests", "native", driver), "-o", exe, "-pthread", "-ldl"]
     subprocess.run(cmd, check=True, capture_output=True, text=True)
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:verify_asan_link_order=0",
                TSAN_OPTIONS="halt_on_error=1", TMPDIR=str(tmp_path))
