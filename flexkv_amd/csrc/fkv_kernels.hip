@@ -130,12 +130,28 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
   const uint64_t total_units = (uint64_t)a.num_blocks * spp;
   const uint64_t total = a.packed ? (total_units + kPiece - 1) / kPiece : total_units;
   const int tid = threadIdx.x;
-  // A launch confined to some XCDs: workgroups elsewhere leave (workgroup 0 always
-  // stays, so the work gets done wherever the launch lands); the others claim ranges.
+  // A launch confined to some XCDs: workgroups elsewhere leave, the others claim
+  // ranges.  A workgroup that runs on the other direction's XCDs next to that
+  // direction's traffic moves its range at a third of the rate and holds up the
+  // whole launch, so none may stay there.  Workgroup 0 is the safety net for a
+  // launch of which no workgroup landed on a selected XCD: it looks at the claim
+  // counter after a while and takes over only if nobody has claimed anything.
   const bool confined = (a.xcd_mask & 0xffu) != 0xffu;
-  if (confined && blockIdx.x != 0 && !((a.xcd_mask >> xcd_of_this_wave()) & 1u))
-    return;
   __shared__ uint32_t s_claim;
+  if (confined && !((a.xcd_mask >> xcd_of_this_wave()) & 1u)) {
+    if (blockIdx.x != 0)
+      return;
+    if (tid == 0) {
+      const long long t0 = wall_clock64();
+      while (wall_clock64() - t0 < 5000) // 50 us of the constant 100 MHz clock
+        __builtin_amdgcn_s_sleep(32);
+      s_claim = __hip_atomic_load(a.claim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (s_claim != 0)
+      return; // the selected XCDs are at work
+    __syncthreads();
+  }
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
   const int nwaves = blockDim.x / kWave;
