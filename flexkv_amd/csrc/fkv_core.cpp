@@ -68,6 +68,9 @@ struct PlanSlot {
   uint8_t *dev = nullptr;
   size_t cap = 0;
   hipEvent_t done = nullptr;
+  // kPlanCounterPairs pairs of zeroed counters in device memory for confined
+  // launches (CopyKernelArgs::claim); each launch leaves its pair zeroed.
+  uint32_t *counters = nullptr;
   bool busy = false;          // handed out, not yet released
   bool event_pending = false; // released behind an event that may not have fired
   int device = 0;
@@ -85,6 +88,7 @@ PlanPool &pool() {
   return *p;
 }
 constexpr size_t kPlanMinBytes = 64 * 1024;
+constexpr int kPlanCounterPairs = 1024;
 
 bool slot_grow(PlanSlot *s, size_t bytes) {
   if (s->cap >= bytes)
@@ -146,12 +150,24 @@ PlanSlot *plan_acquire(int device, size_t bytes) {
     if (!pick) {
       pick = new PlanSlot();
       pick->device = device;
-      if (hipEventCreateWithFlags(&pick->done, hipEventDisableTiming) != hipSuccess) {
+      if (hipEventCreateWithFlags(&pick->done, kBookkeepingEvent) != hipSuccess) {
         (void)hipGetLastError();
         delete pick;
         fail(FKV_ERR_RUNTIME, "plan memory: hipEventCreate failed");
         return nullptr;
       }
+      void *c = nullptr;
+      const size_t cbytes = (size_t)kPlanCounterPairs * 2 * sizeof(uint32_t);
+      if (hipMalloc(&c, cbytes) != hipSuccess || hipMemset(c, 0, cbytes) != hipSuccess) {
+        (void)hipGetLastError();
+        if (c)
+          (void)hipFree(c);
+        (void)hipEventDestroy(pick->done);
+        delete pick;
+        fail(FKV_ERR_RUNTIME, "plan memory: cannot allocate the claim counters");
+        return nullptr;
+      }
+      pick->counters = static_cast<uint32_t *>(c);
       p.slots.push_back(pick);
     }
     pick->busy = true;
@@ -171,6 +187,9 @@ PlanSlot *plan_acquire(int device, size_t bytes) {
 }
 
 uint8_t *plan_host(PlanSlot *s) { return s->host; }
+uint32_t *plan_counters(PlanSlot *s, int pairs) {
+  return pairs <= kPlanCounterPairs ? s->counters : nullptr;
+}
 
 int plan_publish(PlanSlot *s, size_t bytes, bool mirror, hipStream_t stream,
                  uint8_t **device_visible) {
@@ -178,7 +197,19 @@ int plan_publish(PlanSlot *s, size_t bytes, bool mirror, hipStream_t stream,
     *device_visible = s->host; // hipHostMalloc memory: same address on the device
     return FKV_OK;
   }
-  FKV_HIP_TRY(hipMemcpyAsync(s->dev, s->host, bytes, hipMemcpyHostToDevice, stream));
+  // A kernel, not hipMemcpyAsync: copies of different streams share the copy
+  // engines' queues, where the small upload of one stream waits behind the upload
+  // of another stream that is itself waiting for that stream's previous transfer.
+  // With a put stream next to a get stream that tied the start of every get to the
+  // end of a put (0.8 ms idle per 3.8 ms transfer).
+  static const bool by_memcpy = [] {
+    const char *v = std::getenv("FKV_PLAN_UPLOAD");
+    return v && !std::strcmp(v, "memcpy");
+  }();
+  if (by_memcpy)
+    FKV_HIP_TRY(hipMemcpyAsync(s->dev, s->host, bytes, hipMemcpyHostToDevice, stream));
+  else
+    FKV_TRY(launch_plan_upload(s->dev, s->host, bytes, stream));
   *device_visible = s->dev;
   return FKV_OK;
 }
@@ -206,7 +237,7 @@ int env_int(const char *name, int fallback) {
   const char *v = std::getenv(name);
   if (!v || !*v)
     return fallback;
-  return std::atoi(v);
+  return (int)std::strtol(v, nullptr, 0); // decimal, 0x.. or 0.. as written
 }
 } // namespace
 
@@ -257,9 +288,15 @@ LinkLaunchShape link_launch_shape(bool is_h2d) {
 // memory-request queues: 62 GB/s in sum, against 87-90 GB/s when each direction
 // keeps to its own half of the chip.  The library therefore remembers, per device
 // and direction, the events recorded behind its most recent link-bound launches;
-// a launch that finds the other direction still busy confines itself to its half
-// (GPU->host: XCD slots 0-3, host->GPU: 4-7) and asks for enough workgroups to
-// saturate the link from four XCDs.  A direction also counts as busy for a short
+// a launch that finds the other direction still busy confines itself to its own
+// XCDs (GPU->host: XCDs 1-2, host->GPU: 4-7) and asks for enough workgroups to
+// saturate the link from there.  GPU->host keeps to two XCDs because the time a
+// stream stands idle between two commands grows with the number of XCDs that
+// post writes to the host at that moment: measured next to a writer on 1/2/3/4
+// XCDs, a host->GPU stream with one small kernel between its copies idles
+// 65/100/150/780 us per copy, while 48 workgroups write 43/48.5/49/50 GB/s; a
+// writer that includes XCD 0 loses another 4 GB/s.  With the writer on two XCDs
+// the reader also moves 55 instead of 49 GB/s.  A direction also counts as busy for a short
 // while after its last launch (FKV_LINK_ARBITER_WINDOW_MS, default 20): with many
 // small requests in flight the other direction is often between two kernels at
 // the moment of a launch, and a full-chip launch would then collide with its next
@@ -345,7 +382,7 @@ void link_direction_mark(int device, bool h2d, hipStream_t stream) {
   std::lock_guard<std::mutex> lk(a.mu);
   DirectionActivity &d = a.dir[h2d ? 1 : 0];
   const int i = d.next;
-  if (!d.ev[i] && hipEventCreateWithFlags(&d.ev[i], hipEventDisableTiming) != hipSuccess) {
+  if (!d.ev[i] && hipEventCreateWithFlags(&d.ev[i], kBookkeepingEvent) != hipSuccess) {
     (void)hipGetLastError();
     d.ev[i] = nullptr;
     return;
@@ -372,15 +409,12 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
                 "before a kernel transfer): %s",
                 d.cpu_ptr, hipGetErrorString(e));
   }
-  static const bool mirror_plan = env_int("FKV_PLAN_MIRROR", 1) != 0;
   int device = 0;
   FKV_HIP_TRY(hipGetDevice(&device));
   const int lk = d.num_layers * d.kv_dim;
   const size_t tab_bytes = (size_t)lk * 8;
   const size_t ids_bytes = (size_t)d.num_blocks * 8;
-  // base tables, the two id lists, one claim counter per layer (see CopyKernelArgs::claim)
-  const size_t claims_bytes = ((size_t)d.num_layers * 4 + 7) & ~(size_t)7;
-  const size_t plan_bytes = 2 * tab_bytes + 2 * ids_bytes + claims_bytes;
+  const size_t plan_bytes = 2 * tab_bytes + 2 * ids_bytes; // base tables, the two id lists
   PlanSlot *slot = plan_acquire(device, plan_bytes);
   if (!slot)
     return FKV_ERR_RUNTIME;
@@ -404,7 +438,30 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
   }
   std::memcpy(h + 2 * tab_bytes, d.gpu_block_ids, ids_bytes);
   std::memcpy(h + 2 * tab_bytes + ids_bytes, d.cpu_block_ids, ids_bytes);
-  std::memset(h + 2 * tab_bytes + 2 * ids_bytes, 0, claims_bytes);
+  // A CTA of the reference is 1024 threads on one SM (csrc/transfer.cu:176) and
+  // its default of 4 CTAs is tuned for that hardware.  Here each requested CTA
+  // becomes `workgroups_per_cta` small workgroups (see link_launch_shape).
+  out->h2d = d.is_host_to_device != 0;
+  const LinkLaunchShape shape = link_launch_shape(out->h2d);
+  out->workgroups =
+      (d.transfer_num_cta > 0 ? d.transfer_num_cta : default_num_cta(out->h2d)) *
+      shape.workgroups_per_cta;
+  out->threads = shape.threads;
+  out->xcd_mask = shape.xcd_mask;
+  out->device = device;
+  if (arbiter_enabled() && shape.xcd_mask == 0xffu && device_has_eight_xcds(device) &&
+      link_direction_busy(device, !out->h2d, stream)) {
+    // GPU->host on two XCDs, host->GPU on four others; see the note above
+    static const unsigned h2d_mask = (unsigned)env_int("FKV_ARBITER_H2D_MASK", 0xf0) & 0xffu;
+    static const unsigned d2h_mask = (unsigned)env_int("FKV_ARBITER_D2H_MASK", 0x06) & 0xffu;
+    out->xcd_mask = out->h2d ? (h2d_mask ? h2d_mask : 0xf0u) : (d2h_mask ? d2h_mask : 0x06u);
+    static const int h2d_pct = std::max(50, env_int("FKV_ARBITER_H2D_PCT", 150));
+    static const int d2h_pct = std::max(5, env_int("FKV_ARBITER_D2H_PCT", 100));
+    out->workgroups = std::max(1, out->workgroups * (out->h2d ? h2d_pct : d2h_pct) / 100);
+  }
+  // FKV_PLAN_MIRROR=0: kernels read the plan in the pinned slot instead of a device
+  // copy (one command less per transfer; measured no faster, so not the default).
+  static const bool mirror_plan = env_int("FKV_PLAN_MIRROR", 1) != 0;
   uint8_t *dv = nullptr;
   int rc = plan_publish(slot, plan_bytes, mirror_plan, stream, &dv);
   if (rc != FKV_OK) {
@@ -416,35 +473,14 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
   out->cpu_base = reinterpret_cast<const uint64_t *>(dv + tab_bytes);
   out->gpu_ids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes);
   out->cpu_ids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes + ids_bytes);
-  // counters are updated by the device: only a device copy of the plan can hold them
-  out->claims = mirror_plan ? reinterpret_cast<uint32_t *>(dv + 2 * tab_bytes + 2 * ids_bytes)
-                            : nullptr;
+  out->claims = plan_counters(slot, d.num_layers); // nullptr: launches are not confined
   out->vec = common_vector_width(&acc, 1);
-  out->h2d = d.is_host_to_device != 0;
   out->kv_dim = d.kv_dim;
   out->num_layers = d.num_layers;
   out->num_blocks = d.num_blocks;
   out->chunk_size = d.chunk_size;
   out->gpu_block_stride = d.gpu_block_stride;
   out->cpu_block_stride = d.cpu_block_stride;
-  // A CTA of the reference is 1024 threads on one SM (csrc/transfer.cu:176) and
-  // its default of 4 CTAs is tuned for that hardware.  Here each requested CTA
-  // becomes `workgroups_per_cta` small workgroups (see link_launch_shape).
-  const LinkLaunchShape shape = link_launch_shape(out->h2d);
-  out->workgroups =
-      (d.transfer_num_cta > 0 ? d.transfer_num_cta : default_num_cta(out->h2d)) *
-      shape.workgroups_per_cta;
-  out->threads = shape.threads;
-  out->xcd_mask = shape.xcd_mask;
-  out->device = device;
-  if (arbiter_enabled() && shape.xcd_mask == 0xffu && device_has_eight_xcds(device) &&
-      link_direction_busy(device, !out->h2d, stream)) {
-    // four XCDs: 24 single-wavefront workgroups host->GPU, 48 GPU->host per 4 requested CTAs
-    out->xcd_mask = out->h2d ? 0xf0u : 0x0fu;
-    static const int h2d_pct = std::max(50, env_int("FKV_ARBITER_H2D_PCT", 150));
-    static const int d2h_pct = std::max(5, env_int("FKV_ARBITER_D2H_PCT", 100));
-    out->workgroups = std::max(1, out->workgroups * (out->h2d ? h2d_pct : d2h_pct) / 100);
-  }
   return FKV_OK;
 }
 
@@ -479,7 +515,7 @@ int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
     // 48 x 64 lanes 50.7 GB/s, 72 x 64 52.5, 96 x 64 53.0.
     a.packed_grid_pct = 150;
     a.xcd_mask = p.xcd_mask;
-    a.claim = p.claims ? p.claims + l0 : nullptr; // a launch per first layer at most
+    a.claim = p.claims ? p.claims + 2 * l0 : nullptr; // a launch per first layer at most
     FKV_TRY(launch_copy_kernel(a, p.workgroups, p.threads, stream));
   }
   link_direction_mark(p.device, p.h2d, stream);
@@ -606,14 +642,19 @@ namespace {
 // requests in flight over two streams the median request took 25 ms instead of
 // 82 ms, the slowest percentile 55 ms instead of 113 ms.  One event per thread and
 // device, reused.
-int wait_for_work_queued_so_far(hipStream_t stream) {
+// `host_reads_result`: the transfer wrote host memory that the caller will read
+// (GPU->host): the event then keeps its system-scope fence.  A host->GPU transfer
+// leaves nothing for the host to read, and its event goes without (see
+// kBookkeepingEvent).
+int wait_for_work_queued_so_far(hipStream_t stream, bool host_reads_result) {
   constexpr int kMaxDevices = 64;
   struct PerThread { // events go when their thread ends
-    hipEvent_t ev[kMaxDevices] = {};
+    hipEvent_t ev[kMaxDevices][2] = {};
     ~PerThread() {
-      for (hipEvent_t e : ev)
-        if (e && hipEventDestroy(e) != hipSuccess)
-          (void)hipGetLastError();
+      for (auto &pair : ev)
+        for (hipEvent_t e : pair)
+          if (e && hipEventDestroy(e) != hipSuccess)
+            (void)hipGetLastError();
     }
   };
   thread_local PerThread mine;
@@ -623,11 +664,12 @@ int wait_for_work_queued_so_far(hipStream_t stream) {
     FKV_HIP_TRY(hipStreamSynchronize(stream));
     return FKV_OK;
   }
-  if (!mine.ev[device])
-    FKV_HIP_TRY(hipEventCreateWithFlags(&mine.ev[device],
-                                        hipEventBlockingSync | hipEventDisableTiming));
-  FKV_HIP_TRY(hipEventRecord(mine.ev[device], stream));
-  FKV_HIP_TRY(hipEventSynchronize(mine.ev[device]));
+  hipEvent_t &ev = mine.ev[device][host_reads_result ? 1 : 0];
+  if (!ev)
+    FKV_HIP_TRY(hipEventCreateWithFlags(
+        &ev, hipEventBlockingSync | (host_reads_result ? (unsigned)hipEventDisableTiming : fkv::kBookkeepingEvent)));
+  FKV_HIP_TRY(hipEventRecord(ev, stream));
+  FKV_HIP_TRY(hipEventSynchronize(ev));
   return FKV_OK;
 }
 } // namespace
@@ -669,7 +711,7 @@ int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream_v) {
 
   if (d.sync) {
     auto t0 = std::chrono::steady_clock::now();
-    FKV_TRY(wait_for_work_queued_so_far(stream));
+    FKV_TRY(wait_for_work_queued_so_far(stream, /*host_reads_result=*/!d.is_host_to_device));
     if (d.enable_trace) {
       double ms = std::chrono::duration<double, std::milli>(
                       std::chrono::steady_clock::now() - t0)

@@ -49,6 +49,17 @@ private:
   bool pushed_ = false;
 };
 
+// ---- events ---------------------------------------------------------------
+// Flags for events that only order or time work and never publish bytes the GPU
+// wrote to *host* memory.  An event recorded with the default flags carries a
+// system-scope fence; behind a host->GPU kernel that fence does not retire while
+// another stream keeps posted writes to host memory in flight, and the stream
+// stands idle for ~0.77 ms after every such kernel (measured: 12 back-to-back
+// 2 ms host->GPU kernels next to a GPU->host kernel, 770 us between them with a
+// default event after each, 20 us with these flags or with no event).
+constexpr unsigned kBookkeepingEvent = hipEventDisableTiming | hipEventDisableSystemFence;
+constexpr unsigned kTimingEventNoFence = hipEventDisableSystemFence;
+
 // ---- counters -----------------------------------------------------------
 struct Stats {
   std::atomic<uint64_t> calls{0}, bytes_h2d{0}, bytes_d2h{0}, kernel_launches{0},
@@ -129,9 +140,10 @@ struct CopyKernelArgs {
   int32_t packed;   // set by launch_copy_kernel: chunks shorter than a slice, see the kernel
   int32_t packed_grid_pct; // workgroups to launch in packed mode, percent of the request (0 = 100)
   uint32_t xcd_mask; // bit k: workgroups that run on XCD k take part; 0 or 0xff = all
-  // Confined launches only: a zeroed counter in device memory from which the
-  // workgroups that take part claim `num_claims` ranges of the work (set by
-  // launch_copy_kernel).  Without a counter the mask is ignored.
+  // Confined launches only: two zeroed counters in device memory.  From claim[0]
+  // the workgroups that take part claim `num_claims` ranges of the work (set by
+  // launch_copy_kernel); claim[1] counts the workgroups that have left, and the
+  // last one zeroes both again.  Without counters the mask is ignored.
   uint32_t *claim;
   uint32_t num_claims;
 };
@@ -141,6 +153,9 @@ constexpr int kCopyMaxLK = 1024;         // base-table entries staged in LDS
 constexpr int kCopyIdTile = 1024;        // block positions staged in LDS at a time
 int launch_copy_kernel(CopyKernelArgs args, int num_workgroups, int threads_per_workgroup,
                        hipStream_t stream);
+// Copies `bytes` (rounded up to 16) from a pinned, device-mapped host buffer to
+// device memory with a small kernel on `stream`.
+int launch_plan_upload(void *device_dst, const void *pinned_src, size_t bytes, hipStream_t stream);
 // Launch shape of the link-bound kernel for one direction.
 struct LinkLaunchShape {
   int workgroups_per_cta; // workgroups launched per requested CTA
@@ -159,6 +174,9 @@ struct PlanSlot;
 // Returns nullptr (and sets the error) on allocation failure.
 PlanSlot *plan_acquire(int device, size_t bytes);
 uint8_t *plan_host(PlanSlot *s);
+// `pairs` pairs of zeroed counters in device memory that belong to the slot
+// (CopyKernelArgs::claim), or nullptr when a slot holds fewer.
+uint32_t *plan_counters(PlanSlot *s, int pairs);
 // Publishes the first `bytes` of the slot to the device on `stream` and returns
 // the address kernels must use (the device mirror, or the pinned buffer itself
 // when `mirror` is false).
@@ -183,7 +201,7 @@ struct KernelPlan {
   int workgroups = 1, threads = 64;
   unsigned xcd_mask = 0xff;
   int device = 0;
-  uint32_t *claims = nullptr; // one zeroed counter per layer of the plan, device memory
+  uint32_t *claims = nullptr; // a zeroed pair of counters per layer of the plan, device memory
 };
 // Link-bound launches of the last while, per device and direction (see fkv_core.cpp).
 bool link_direction_busy(int device, bool h2d, hipStream_t launching_stream);

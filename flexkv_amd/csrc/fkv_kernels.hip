@@ -138,9 +138,21 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
   // counter after a while and takes over only if nobody has claimed anything.
   const bool confined = (a.xcd_mask & 0xffu) != 0xffu;
   __shared__ uint32_t s_claim;
+  // Every workgroup of a confined launch counts itself out; the last one leaves the
+  // two counters zeroed for the next launch that is given them.
+  auto leave = [&]() {
+    if (tid == 0 &&
+        __hip_atomic_fetch_add(a.claim + 1, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) ==
+            gridDim.x - 1) {
+      __hip_atomic_store(a.claim, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(a.claim + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
   if (confined && !((a.xcd_mask >> xcd_of_this_wave()) & 1u)) {
-    if (blockIdx.x != 0)
+    if (blockIdx.x != 0) {
+      leave();
       return;
+    }
     if (tid == 0) {
       const long long t0 = wall_clock64();
       while (wall_clock64() - t0 < 5000) // 50 us of the constant 100 MHz clock
@@ -148,8 +160,10 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
       s_claim = __hip_atomic_load(a.claim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
-    if (s_claim != 0)
-      return; // the selected XCDs are at work
+    if (s_claim != 0) { // the selected XCDs are at work
+      leave();
+      return;
+    }
     __syncthreads();
   }
   const int lane = tid & (kWave - 1);
@@ -172,8 +186,10 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
       part = s_claim;
       parts = a.num_claims;
       __syncthreads(); // everyone has read the claim before it is overwritten
-      if (part >= parts)
-        return; // whole workgroup leaves together
+      if (part >= parts) { // whole workgroup leaves together
+        leave();
+        return;
+      }
     }
     uint64_t s0 = total * part / parts;
     uint64_t s1 = total * (part + 1) / parts;
@@ -290,6 +306,14 @@ int launch_vec(const CopyKernelArgs &a, int grid, int threads, size_t lds_bytes,
 } // namespace
 
 namespace {
+// Copies a plan from its pinned host slot to the device mirror.
+__global__ void fkv_plan_upload_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src,
+                                       uint32_t vectors) {
+  for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < vectors;
+       i += gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
 // Keeps one wavefront busy for `ticks` of the constant 100 MHz clock.
 __global__ void fkv_wait_kernel(long long ticks, int *sink) {
   const long long t0 = wall_clock64();
@@ -299,6 +323,22 @@ __global__ void fkv_wait_kernel(long long ticks, int *sink) {
     *sink = 1;
 }
 } // namespace
+
+int launch_plan_upload(void *device_dst, const void *pinned_src, size_t bytes,
+                       hipStream_t stream) {
+  const uint32_t vectors = (uint32_t)((bytes + 15) / 16);
+  if (vectors == 0)
+    return FKV_OK;
+  const int threads = 256;
+  const int grid = (int)std::min<uint32_t>((vectors + threads - 1) / threads, 64);
+  hipLaunchKernelGGL(fkv_plan_upload_kernel, dim3(grid), dim3(threads), 0, stream,
+                     static_cast<uint4 *>(device_dst), static_cast<const uint4 *>(pinned_src),
+                     vectors);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return fail(FKV_ERR_RUNTIME, "plan upload launch failed: %s", hipGetErrorString(e));
+  return FKV_OK;
+}
 
 int common_vector_width(const uint64_t *vals, int n) {
   uint64_t acc = 0;

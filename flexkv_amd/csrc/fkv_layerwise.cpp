@@ -607,10 +607,11 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
   for (auto &b : g->batches)
     for (int i = 0; i < g->num_gpus; ++i) {
       FKV_HIP_TRY(hipSetDevice(g->device_ids[i]));
-      FKV_HIP_TRY(hipEventCreate(&b->done[i]));
+      // a restore writes device memory only: no system-scope fence (see kBookkeepingEvent)
+      FKV_HIP_TRY(hipEventCreateWithFlags(&b->done[i], kTimingEventNoFence));
     }
   FKV_HIP_TRY(hipSetDevice(g->device_ids[0]));
-  FKV_HIP_TRY(hipEventCreate(&g->started));
+  FKV_HIP_TRY(hipEventCreateWithFlags(&g->started, kTimingEventNoFence));
   FKV_HIP_TRY(hipEventRecord(g->started, g->streams[0]));
 
   int rc = FKV_OK;

@@ -187,6 +187,29 @@ def test_puts_and_gets_at_the_same_time(gpu_device, chunk):
     dev.assert_matches_reference("concurrent put and get")
 
 
+def test_confined_launches_one_after_another_each_do_their_work(gpu_device):
+    """Confined launches share counters that each launch must leave zeroed: 24
+    transfers of different blocks, alternating directions with a wait after each,
+    reuse the same plan memory, and every one of them has to move its blocks."""
+    from flexkv_amd.c_ext import get_stats, reset_stats
+    s = KVSetup(VLLM, 4, 2, 520, 520, 4096, "BLOCKFIRST", seed=43)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(12)
+    perm_g, perm_c = rng.permutation(520), rng.permutation(520)
+    import torch
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]  # work of the launching stream never counts as busy
+    reset_stats()
+    for k in range(24):
+        h2d = k % 2 == 1
+        g, c = perm_g[k * 20:(k + 1) * 20 + (k % 3)], perm_c[k * 20:(k + 1) * 20 + (k % 3)]
+        with torch.cuda.stream(streams[k % 2]):
+            dev.transfer(g, c, is_h2d=h2d)
+        s.oracle_transfer(g, c, h2d)
+    st = get_stats()
+    assert st["confined_launches"] >= 20, st
+    dev.assert_matches_reference("24 confined launches in a row")
+
+
 def test_more_layer_kv_pairs_than_one_launch_holds(gpu_device):
     """700 layers x 2 = 1400 (layer, kv) pairs: split over two launches."""
     s = KVSetup(VLLM, 700, 2, 6, 6, 32, "BLOCKFIRST", seed=9)
