@@ -291,9 +291,12 @@ def verify_round_trip(w, torch, num_cta):
     return bool(ok)
 
 
-def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy):
+def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=False):
     """c3: per-layer restore with a dummy per-layer compute kernel on a second
-    stream gated on each layer's event."""
+    stream gated on each layer's event.  `layer_spans` brackets every layer's
+    compute with two timing events; torch creates them with default flags, and
+    next to a transfer over the host link each such event idles the compute
+    stream for 0.1 ms or more, so the spans are off unless asked for."""
     from flexkv_amd.c_ext import LayerwiseTransferGroup
     i64 = lambda v: torch.tensor([v], dtype=torch.int64)
     grp = LayerwiseTransferGroup(
@@ -320,8 +323,11 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy):
     if dummy == "sdpa":
         q = torch.randn(1, 32, 2048, 128, device=w.device, dtype=torch.bfloat16)
         unit = lambda: torch.nn.functional.scaled_dot_product_attention(q, q, q)
-    elif dummy == "gemm":
-        n = 2048
+    elif dummy in ("gemm", "gemm4k"):
+        # 2048^3: one round of workgroups on 256 CUs, so a single CU held by a copy
+        # wavefront costs a second round; 4096^3: several rounds, the loss is the
+        # share of CUs the copy holds
+        n = 2048 if dummy == "gemm" else 4096
         a = torch.randn(n, n, device=w.device, dtype=torch.bfloat16)
         b = torch.randn(n, n, device=w.device, dtype=torch.bfloat16)
         c = torch.empty(n, n, device=w.device, dtype=torch.bfloat16)
@@ -368,18 +374,22 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy):
         with torch.cuda.stream(comp):
             for l in range(w.L):
                 grp.wait_layer(l, comp)
-                a0, a1 = ev(), ev()
-                a0.record(comp)        # stamped once layer l has landed
+                if layer_spans:
+                    a0, a1 = ev(), ev()
+                    a0.record(comp)        # stamped once layer l has landed
                 layer_compute(reps)
-                a1.record(comp)
-                spans.append((a0, a1))
+                if layer_spans:
+                    a1.record(comp)
+                    spans.append((a0, a1))
             e.record(comp)
         e.synchronize()
         grp.synchronize()
         if it >= warmup:
             bt = grp.batch_times_ms()
             total = s.elapsed_time(e)
-            computing = sum(x.elapsed_time(y) for x, y in spans)
+            # without spans: what the compute stream needs alone, i.e. every ms beyond
+            # that counts as stalled (waiting for a layer, or slowed down by the copies)
+            computing = sum(x.elapsed_time(y) for x, y in spans) if layer_spans else compute_ms
             totals.append(total)
             restores.append(bt[-1])
             firsts.append(bt[0])
@@ -856,8 +866,11 @@ def main():
                     help="transfer_num_cta (reference default FLEXKV_TRANSFER_NUM_CTA_*=4)")
     ap.add_argument("--use-ce", action="store_true", help="copy-engine path instead of the kernel")
     ap.add_argument("--notify", default="polling", choices=["polling", "hostfunc"])
-    ap.add_argument("--dummy", default="sdpa", choices=["sdpa", "gemm", "elementwise"],
+    ap.add_argument("--dummy", default="sdpa", choices=["sdpa", "gemm", "gemm4k", "elementwise"],
                     help="c3: the per-layer compute kernel the restore is overlapped with")
+    ap.add_argument("--layer-spans", action="store_true",
+                    help="c3: time every layer's compute with its own pair of events "
+                         "(the events themselves slow the compute stream down)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     args = ap.parse_args()
@@ -1024,7 +1037,8 @@ def main():
         saved = [w.gpu_rows(l, 0).index_select(0, gi) for l in range(w.L)]
         for l in range(w.L):
             w.gpu_rows(l, 0).index_fill_(0, gi, 0)
-        r = run_layerwise(w, torch, args.steps, args.warmup, args.num_cta, args.notify, args.dummy)
+        r = run_layerwise(w, torch, args.steps, args.warmup, args.num_cta, args.notify, args.dummy,
+                          layer_spans=args.layer_spans)
         restore = B / (r["restore_ms"] * 1e-3) / 1e9
         stall_beyond_first = max(0.0, r["stall_ms"] - r["first_layer_ms"])
         out.update(value=round(restore, 3), ms_per_step=round(r["total_ms"], 3),
@@ -1037,15 +1051,22 @@ def main():
                               "restore_ms": round(r["restore_ms"], 3),
                               "first_layer_ms": round(r["first_layer_ms"], 3),
                               "compute_alone_ms": round(r["compute_ms"], 3),
-                              "compute_while_restoring_ms": round(r["compute_overlapped_ms"], 3),
-                              "compute_slowdown": round(
-                                  r["compute_overlapped_ms"] / r["compute_ms"], 3),
                               "restore_plus_compute_ms": round(r["total_ms"], 3),
+                              # the compute stream cannot finish before the last layer
+                              # has landed and been computed on
+                              "compute_tail_after_restore_ms": round(
+                                  r["total_ms"] - r["restore_ms"], 3),
+                              "compute_per_layer_ms": round(r["compute_ms"] / w.L, 3),
+                              "layer_spans": bool(args.layer_spans),
                               "compute_stream_stall_ms": round(r["stall_ms"], 3),
                               "stall_beyond_first_layer_ms": round(stall_beyond_first, 3),
                               "overlap_frac_beyond_first_layer": round(
                                   1.0 - stall_beyond_first /
                                   max(1e-9, r["restore_ms"] - r["first_layer_ms"]), 4)})
+        if args.layer_spans:
+            out["layerwise"].update(
+                compute_while_restoring_ms=round(r["compute_overlapped_ms"], 3),
+                compute_slowdown=round(r["compute_overlapped_ms"] / r["compute_ms"], 3))
         if not args.no_verify:
             out["bit_exact"] = all(
                 torch.equal(w.gpu_rows(l, 0).index_select(0, gi), saved[l]) for l in range(w.L))

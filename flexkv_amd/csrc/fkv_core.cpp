@@ -296,7 +296,12 @@ LinkLaunchShape link_launch_shape(bool is_h2d) {
 // XCDs, a host->GPU stream with one small kernel between its copies idles
 // 65/100/150/780 us per copy, while 48 workgroups write 43/48.5/49/50 GB/s; a
 // writer that includes XCD 0 loses another 4 GB/s.  With the writer on two XCDs
-// the reader also moves 55 instead of 49 GB/s.  A direction also counts as busy for a short
+// the reader also moves 55 instead of 49 GB/s.  A lone GPU->host transfer loses 2 %
+// on two XCDs and nothing on three (1-3), a lone host->GPU transfer nothing on 4-7,
+// so launches of 8 MiB and more (FKV_HOME_MIN_KB, -1: never) keep to these home
+// XCDs even when the link is idle: a put launched alone and a get that arrives
+// 1 ms later reach 90 GB/s instead of 78, in the other order instead of 66.
+// A direction also counts as busy for a short
 // while after its last launch (FKV_LINK_ARBITER_WINDOW_MS, default 20): with many
 // small requests in flight the other direction is often between two kernels at
 // the moment of a launch, and a full-chip launch would then collide with its next
@@ -448,16 +453,26 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
       shape.workgroups_per_cta;
   out->threads = shape.threads;
   out->xcd_mask = shape.xcd_mask;
+  out->home_mask = 0xffu;
+  out->home_workgroups = out->workgroups;
   out->device = device;
-  if (arbiter_enabled() && shape.xcd_mask == 0xffu && device_has_eight_xcds(device) &&
-      link_direction_busy(device, !out->h2d, stream)) {
-    // GPU->host on two XCDs, host->GPU on four others; see the note above
+  if (arbiter_enabled() && shape.xcd_mask == 0xffu && device_has_eight_xcds(device)) {
     static const unsigned h2d_mask = (unsigned)env_int("FKV_ARBITER_H2D_MASK", 0xf0) & 0xffu;
     static const unsigned d2h_mask = (unsigned)env_int("FKV_ARBITER_D2H_MASK", 0x06) & 0xffu;
-    out->xcd_mask = out->h2d ? (h2d_mask ? h2d_mask : 0xf0u) : (d2h_mask ? d2h_mask : 0x06u);
+    static const unsigned d2h_home = (unsigned)env_int("FKV_HOME_D2H_MASK", 0x0e) & 0xffu;
     static const int h2d_pct = std::max(50, env_int("FKV_ARBITER_H2D_PCT", 150));
     static const int d2h_pct = std::max(5, env_int("FKV_ARBITER_D2H_PCT", 100));
-    out->workgroups = std::max(1, out->workgroups * (out->h2d ? h2d_pct : d2h_pct) / 100);
+    const int scaled = std::max(1, out->workgroups * (out->h2d ? h2d_pct : d2h_pct) / 100);
+    // Large launches keep to their direction's home XCDs even when the link is
+    // idle, so that a transfer of the other direction that starts while they run
+    // finds its own XCDs free; see the note above.
+    out->home_mask = out->h2d ? (h2d_mask ? h2d_mask : 0xf0u) : (d2h_home ? d2h_home : 0x0eu);
+    out->home_workgroups = scaled;
+    if (link_direction_busy(device, !out->h2d, stream)) {
+      // GPU->host on two XCDs, host->GPU on four others
+      out->xcd_mask = out->h2d ? (h2d_mask ? h2d_mask : 0xf0u) : (d2h_mask ? d2h_mask : 0x06u);
+      out->workgroups = scaled;
+    }
   }
   // FKV_PLAN_MIRROR=0: kernels read the plan in the pinned slot instead of a device
   // copy (one command less per transfer; measured no faster, so not the default).
@@ -515,8 +530,15 @@ int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
     // 48 x 64 lanes 50.7 GB/s, 72 x 64 52.5, 96 x 64 53.0.
     a.packed_grid_pct = 150;
     a.xcd_mask = p.xcd_mask;
+    int workgroups = p.workgroups;
+    static const int64_t home_min_bytes = (int64_t)env_int("FKV_HOME_MIN_KB", 8192) * 1024;
+    if (p.xcd_mask == 0xffu && p.home_mask != 0xffu && home_min_bytes >= 0 &&
+        (int64_t)p.num_blocks * a.lk * p.chunk_size >= home_min_bytes) {
+      a.xcd_mask = p.home_mask;
+      workgroups = p.home_workgroups;
+    }
     a.claim = p.claims ? p.claims + 2 * l0 : nullptr; // a launch per first layer at most
-    FKV_TRY(launch_copy_kernel(a, p.workgroups, p.threads, stream));
+    FKV_TRY(launch_copy_kernel(a, workgroups, p.threads, stream));
   }
   link_direction_mark(p.device, p.h2d, stream);
   return FKV_OK;

@@ -200,6 +200,9 @@ struct KernelPlan {
   int64_t chunk_size = 0, gpu_block_stride = 0, cpu_block_stride = 0;
   int workgroups = 1, threads = 64;
   unsigned xcd_mask = 0xff;
+  // XCDs (and workgroups) of launches that move a lot while the link is idle
+  unsigned home_mask = 0xff;
+  int home_workgroups = 1;
   int device = 0;
   uint32_t *claims = nullptr; // a zeroed pair of counters per layer of the plan, device memory
 };
