@@ -589,9 +589,11 @@ def run_multi_group(torch, device, steps, warmup, num_cta, notify, use_ce, verif
                      "512 blocks + 64 sidecar slots, page 256")}
 
 
-def run_worker_process(torch, device, steps, warmup, num_cta, use_ce):
+def run_worker_process(torch, device, steps, warmup, num_cta, use_ce, overlap=False):
     """c0-shaped put and get ops through a GPUCPUTransferWorker in its own process:
-    what the pipe, the shared op pool and the completion queue add to a transfer."""
+    what the pipe, the shared op pool and the completion queue add to a transfer.
+    Then 8 puts and 8 gets of 64 blocks each, submitted together: one after the
+    other, or gets next to puts when the worker overlaps the directions."""
     import numpy as np
     import torch.multiprocessing as mp
     from flexkv_amd.layout import KVCacheLayout, KVCacheLayoutType
@@ -617,7 +619,7 @@ def run_worker_process(torch, device, steps, warmup, num_cta, use_ce):
         ctx, q, pool.get_buffer(), [TensorSharedHandle(x) for x in tensors],
         PinnedPoolHandle(cl.kv_shape, t.bfloat16), gl, cl, t.bfloat16, 0,
         use_ce_transfer_h2d=use_ce, use_ce_transfer_d2h=use_ce, transfer_num_cta_h2d=num_cta,
-        transfer_num_cta_d2h=num_cta)
+        transfer_num_cta_d2h=num_cta, overlap_directions=overlap)
     h.wait_ready(300)
     gg = t.Generator().manual_seed(1)
     gpu_ids = t.randperm(N, generator=gg)[:n].numpy().astype(np.int64)
@@ -643,9 +645,38 @@ def run_worker_process(torch, device, steps, warmup, num_cta, use_ce):
             if it >= warmup:
                 rec[kind.value].append((e2e, m["xfer_ms"], m["ipc_ms"], m["wait_ms"]))
     wall = time.perf_counter() - t_all
+    # mixed traffic: puts from engine blocks [0, 512) to host [0, 512), gets from host
+    # [512, 1024) to engine blocks [512, 1024), 64 blocks per op, all submitted at once
+    m_ops, m_blocks = 8, 64
+    mixed_bytes = 2 * m_ops * m_blocks * L * 2 * T * H * D * 2
+    mixed = []
+    for it in range(warmup + steps):
+        ops = []
+        for k in range(m_ops):
+            a = np.arange(k * m_blocks, (k + 1) * m_blocks, dtype=np.int64)
+            for kind, src, dst in ((TransferType.D2H, a, a), (TransferType.H2D, a + 512, a + 512)):
+                op = TransferOp(1000 + it, kind, src, dst)
+                op.src_slot_id = pool.allocate_slot(src, 1 if kind == TransferType.D2H else 2)
+                op.dst_slot_id = pool.allocate_slot(dst, 2 if kind == TransferType.D2H else 1)
+                ops.append(op)
+        t0 = time.perf_counter()
+        for op in ops:
+            h.submit_transfer(op)
+        done = [q.get(timeout=300) for _ in ops]
+        dt = time.perf_counter() - t0
+        assert all(d[1] for d in done) and sorted(d[0] for d in done) == sorted(o.op_id for o in ops)
+        for op in ops:
+            pool.free_slot(op.src_slot_id)
+            pool.free_slot(op.dst_slot_id)
+        if it >= warmup:
+            mixed.append(dt)
     h.shutdown()
     med = lambda xs: _median(list(xs))
-    res = {"bytes_per_op": nbytes, "wall_s": wall, "exit_code": h.process.exitcode}
+    res = {"bytes_per_op": nbytes, "wall_s": wall, "exit_code": h.process.exitcode,
+           "mixed": {"ops": 2 * m_ops, "blocks_per_op": m_blocks, "bytes": mixed_bytes,
+                     "overlap_directions": bool(overlap),
+                     "ms": round(med(mixed) * 1e3, 3),
+                     "GBps": round(mixed_bytes / med(mixed) / 1e9, 3)}}
     for k, rows in rec.items():
         res[k] = {"e2e_ms": round(med(r[0] for r in rows), 3),
                   "worker_xfer_ms": round(med(r[1] for r in rows), 3),
@@ -868,6 +899,8 @@ def main():
     ap.add_argument("--notify", default="polling", choices=["polling", "hostfunc"])
     ap.add_argument("--dummy", default="sdpa", choices=["sdpa", "gemm", "gemm4k", "elementwise"],
                     help="c3: the per-layer compute kernel the restore is overlapped with")
+    ap.add_argument("--overlap-directions", action="store_true",
+                    help="worker: the worker runs gets next to puts (second thread and stream)")
     ap.add_argument("--layer-spans", action="store_true",
                     help="c3: time every layer's compute with its own pair of events "
                          "(the events themselves slow the compute stream down)")
@@ -975,7 +1008,8 @@ def main():
         return
     if args.config == "worker":
         link = measure_link()
-        r = run_worker_process(torch, device, args.steps, args.warmup, args.num_cta, args.use_ce)
+        r = run_worker_process(torch, device, args.steps, args.warmup, args.num_cta, args.use_ce,
+                               overlap=args.overlap_directions)
         print(json.dumps({
             "metric": "put/get through a transfer worker process: GB/s seen by the submitter",
             "unit": "GB/s", "value": round(2 * r["bytes_per_op"] * args.steps / r["wall_s"] / 1e9, 3),
@@ -988,6 +1022,7 @@ def main():
                        "path": "copy-engine" if args.use_ce else "kernel",
                        "transfer_num_cta": args.num_cta},
             "put": r["D2H"], "get": r["H2D"], "bytes_per_op": r["bytes_per_op"],
+            "puts_and_gets_submitted_together": r["mixed"],
             "worker_exit_code": r["exit_code"],
             "link_peak": {"d2h_GBps": round(link["d2h"], 3), "h2d_GBps": round(link["h2d"], 3)}}))
         return

@@ -2,7 +2,8 @@
 
 One worker process owns one kind of transfer.  The engine submits ops through a
 pipe (``WorkerHandle.submit_transfer``), the worker runs them one at a time in
-arrival order and reports every op on a shared queue:
+arrival order (a GPU worker with ``overlap_directions`` runs gets next to puts)
+and reports every op on a shared queue:
 
     (op_id, True,  metrics-or-None)      the op ran
     (op_id, False, None)                 the op raised; logged, never dropped
@@ -80,6 +81,70 @@ def _allow_pageable(flag: Optional[bool]) -> bool:
     return bool(int(os.getenv("FKV_WORKER_ALLOW_PAGEABLE_HOST", "0")))
 
 
+class _SideLane:
+    """A second thread of a worker that runs the ops handed to it in order, next to
+    the ops the worker runs itself.  It remembers the block ids of its unfinished ops
+    so that the worker can hold back an op of its own that touches the same blocks."""
+
+    def __init__(self, name: str, run_op, device: Optional[int]) -> None:
+        import queue
+        self.name = name
+        self._run_op = run_op
+        self._device = device
+        self._q: "queue.Queue[Any]" = queue.Queue()
+        self._cond = threading.Condition()
+        self._inflight: Dict[int, Tuple[np.ndarray, np.ndarray]] = {}
+        self._seq = 0
+        self._thread = threading.Thread(target=self._loop, name=f"fkv-lane-{name}", daemon=True)
+        self._thread.start()
+
+    def submit(self, op: Any, cpu_ids: np.ndarray, gpu_ids: np.ndarray) -> None:
+        with self._cond:
+            self._seq += 1
+            key = self._seq
+            self._inflight[key] = (np.array(cpu_ids, copy=True), np.array(gpu_ids, copy=True))
+        self._q.put((key, op))
+
+    def wait_until_clear_of(self, cpu_ids: Optional[np.ndarray],
+                            gpu_ids: Optional[np.ndarray]) -> None:
+        """Returns once no unfinished op of the lane shares a host block with
+        `cpu_ids` or an engine block with `gpu_ids` (None: that side is not touched)."""
+        def clash() -> bool:
+            for c, g in self._inflight.values():
+                if cpu_ids is not None and len(cpu_ids) and np.isin(cpu_ids, c).any():
+                    return True
+                if gpu_ids is not None and len(gpu_ids) and np.isin(gpu_ids, g).any():
+                    return True
+            return False
+        with self._cond:
+            while clash():
+                self._cond.wait(0.5)
+
+    def drain(self) -> None:
+        with self._cond:
+            while self._inflight:
+                self._cond.wait(0.5)
+
+    def close(self) -> None:
+        self._q.put(None)
+        self._thread.join(timeout=60)
+
+    def _loop(self) -> None:
+        if self._device is not None:
+            torch.cuda.set_device(self._device)
+        while True:
+            item = self._q.get()
+            if item is None:
+                return
+            key, op = item
+            try:
+                self._run_op(op)   # reports the op itself, never raises
+            finally:
+                with self._cond:
+                    self._inflight.pop(key, None)
+                    self._cond.notify_all()
+
+
 class TransferWorkerBase(ABC):
     _worker_id_counter = 0
     _worker_id_lock = threading.Lock()
@@ -91,6 +156,7 @@ class TransferWorkerBase(ABC):
         obj._host_registered = []
         obj._shutdown_done = False
         obj._pageable_host = False
+        obj._lanes = {}
         return obj
 
     def __init__(self, worker_id: int, transfer_conn: Connection, finished_ops_queue,
@@ -102,6 +168,7 @@ class TransferWorkerBase(ABC):
         self._host_registered: List[Tuple[torch.Tensor, str]] = []
         self._shutdown_done = False
         self._pageable_host = False
+        self._lanes: Dict[str, _SideLane] = {}
         trace.configure(global_env().enable_transfer_trace)
 
     # ---- host memory --------------------------------------------------------------
@@ -137,6 +204,8 @@ class TransferWorkerBase(ABC):
         if getattr(self, "_shutdown_done", False):
             return
         self._shutdown_done = True
+        for lane in (getattr(self, "_lanes", None) or {}).values():
+            lane.close()
         registered = getattr(self, "_host_registered", None) or []
         wid = getattr(self, "worker_id", -1)
         logger.info("[worker %s] shutdown: unregistering %d host region(s)", wid, len(registered))
@@ -320,6 +389,10 @@ class TransferWorkerBase(ABC):
             # dropping it would leave the op's graph unfinished for ever
             self.finished_ops_queue.put((op.transfer_op_id, False, None))
 
+    def _dispatch(self, op) -> None:
+        """Runs the op on this thread.  A worker with side lanes overrides this."""
+        self._run_one(op)
+
     def run(self) -> None:
         """Receive, drain what else is already queued, run the batch in order.  Ends
         on the ``None`` sentinel or when the pipe closes; cleaning up is the process
@@ -345,8 +418,10 @@ class TransferWorkerBase(ABC):
                         if msg.get("type") == "control":
                             self._reply_control(msg)
                         continue
-                    self._run_one(msg)
+                    self._dispatch(msg)
                 if stop:
+                    for lane in self._lanes.values():
+                        lane.drain()
                     return
             except EOFError:
                 logger.warning("[worker %s] transfer pipe EOF; exiting run loop", self.worker_id)
@@ -467,7 +542,7 @@ class GPUCPUTransferWorker(TransferWorkerBase):
                  allow_pageable_host: Optional[bool] = None,
                  ssd_files: Optional[Dict[int, List[str]]] = None,
                  ssd_kv_layout: Optional[Union[KVCacheLayout, MultiGroupBlockLayout]] = None,
-                 num_blocks_per_file: int = 0) -> None:
+                 num_blocks_per_file: int = 0, overlap_directions: Optional[bool] = None) -> None:
         super().__init__(worker_id, transfer_conn, finished_ops_queue, op_buffer_tensor)
         # the device first: everything below creates state on the current device
         torch.cuda.set_device(gpu_device_id)
@@ -503,6 +578,20 @@ class GPUCPUTransferWorker(TransferWorkerBase):
             ref_tensors, ref_layers = len(self.gpu_blocks), self.num_layers
         self.gpu_block_type_ = gpu_block_type_from_tensor_count(ref_tensors, ref_layers)
         self.transfer_stream = torch.cuda.Stream()
+        # Gets next to puts.  The link carries both directions at once (93 GB/s in
+        # sum against 57 one after the other), so with `overlap_directions` H2D ops
+        # run on a second thread and stream while this thread runs everything else.
+        # Ops of one direction still run in arrival order; an op that shares a block
+        # with an unfinished op of the other direction waits for it.  Completions
+        # of different directions may therefore overtake each other, which the
+        # reference's one-at-a-time worker never does: opt-in
+        # (FKV_WORKER_OVERLAP_DIRECTIONS=1 sets the default).
+        if overlap_directions is None:
+            overlap_directions = os.environ.get("FKV_WORKER_OVERLAP_DIRECTIONS", "0") == "1"
+        self.h2d_stream: Optional[torch.cuda.Stream] = None
+        if overlap_directions:
+            self.h2d_stream = self._stream_on_another_queue(self.transfer_stream)
+            self._lanes["h2d"] = _SideLane("h2d", self._run_one, gpu_device_id)
         self.transfer_num_cta_h2d = transfer_num_cta_h2d
         self.transfer_num_cta_d2h = transfer_num_cta_d2h
         self.use_ce_transfer_h2d = use_ce_transfer_h2d
@@ -519,6 +608,36 @@ class GPUCPUTransferWorker(TransferWorkerBase):
             self.ssd = SSDPoolMover(self.cpu_tensor, ssd_files, cpu_kv_layout, ssd_kv_layout, dtype,
                                     num_blocks_per_file,
                                     multi_group=self.group_transfer_params is not None)
+
+    @staticmethod
+    def _stream_on_another_queue(first: "torch.cuda.Stream") -> "torch.cuda.Stream":
+        """A stream whose kernels can run next to those of `first`: streams that the
+        runtime maps to one hardware queue take turns."""
+        from ..c_ext import streams_run_concurrently
+        spare: List[torch.cuda.Stream] = []   # kept alive so that the next one differs
+        s = torch.cuda.Stream()
+        while not streams_run_concurrently(first, s) and len(spare) < 8:
+            spare.append(s)
+            s = torch.cuda.Stream()
+        return s
+
+    def _dispatch(self, op) -> None:
+        lane = self._lanes.get("h2d")
+        if lane is None:
+            return self._run_one(op)
+        src, dst = self.get_transfer_block_ids(op)
+        src_ids, dst_ids = src.numpy(), dst.numpy()
+        kind = op.transfer_type
+        if kind == TransferType.H2D:
+            # ops of this thread are finished when it gets here: nothing to wait for
+            lane.submit(op, src_ids, dst_ids)
+            return
+        if kind == TransferType.D2H:      # writes host blocks, reads engine blocks
+            lane.wait_until_clear_of(dst_ids, src_ids)
+        elif kind == TransferType.DISK2H:  # writes host blocks
+            lane.wait_until_clear_of(dst_ids, None)
+        # H2DISK only reads host blocks, as the gets do
+        self._run_one(op)
 
     def _init_multi_group(self, gpu_blocks_per_group, gpu_layouts_per_group,
                           cpu_kv_layout: MultiGroupBlockLayout, layer_groups) -> None:
@@ -590,7 +709,10 @@ class GPUCPUTransferWorker(TransferWorkerBase):
                 transfer_op, self.ssd.bytes_per_block * transfer_op.valid_block_num, t0,
                 time.time())
             return True
-        with torch.cuda.stream(self.transfer_stream):
+        stream = self.transfer_stream
+        if self.h2d_stream is not None and transfer_op.transfer_type == TransferType.H2D:
+            stream = self.h2d_stream
+        with torch.cuda.stream(stream):
             t0 = time.time()
             self._transfer_impl(src, dst, transfer_op.transfer_type)
             t1 = time.time()

@@ -334,3 +334,37 @@ def test_worker_metrics_when_trace_is_on(harness, monkeypatch):
     finally:
         trace.configure(False)
         monkeypatch.setattr(env, "_ENV", None)
+
+
+def test_side_lane_runs_in_order_and_holds_back_ops_that_share_blocks():
+    """The second thread of a GPU worker that overlaps gets with puts: ops handed
+    to it run in order, and the worker's own thread can wait until no unfinished
+    op of the lane touches given host or engine blocks."""
+    import threading
+    from flexkv_amd.transfer.worker import _SideLane
+    gate, ran = threading.Event(), []
+
+    def run_op(op):
+        if op == "slow":
+            gate.wait(10)
+        ran.append(op)
+    lane = _SideLane("t", run_op, None)
+    lane.submit("slow", np.array([1, 2, 3]), np.array([10, 11]))
+    lane.submit("next", np.array([7]), np.array([12]))
+    t0 = time.time()
+    lane.wait_until_clear_of(np.array([4, 5]), np.array([13]))       # shares nothing
+    lane.wait_until_clear_of(np.array([], dtype=np.int64), None)     # touches nothing
+    assert time.time() - t0 < 0.3
+    cleared = []
+    for ids in ((np.array([3]), None), (None, np.array([12, 99]))):  # a host block; an engine block
+        done = threading.Event()
+        threading.Thread(target=lambda i=ids, d=done: (lane.wait_until_clear_of(*i), d.set()),
+                         daemon=True).start()
+        cleared.append(done)
+    time.sleep(0.3)
+    assert not cleared[0].is_set() and not cleared[1].is_set()
+    gate.set()
+    assert cleared[0].wait(5) and cleared[1].wait(5)
+    lane.drain()
+    assert ran == ["slow", "next"]
+    lane.close()

@@ -373,3 +373,43 @@ def test_gpu_worker_that_also_serves_the_ssd_tier(gpu_device, engine, tmp_path, 
         assert torch.equal(tensors[l][:, gpu_dst], want[l][:, gpu_src]), l
     h.shutdown()
     assert h.process.exitcode == 0
+
+
+def test_gpu_worker_runs_gets_next_to_puts(gpu_device, engine):
+    """overlap_directions: H2D ops run on a second thread and stream of the worker.
+    Four ops are submitted back to back; the put that overwrites host blocks an
+    unfinished get still reads has to wait for that get, the others may overlap.
+    Every op is reported once, in whatever order."""
+    start, q, pool = engine
+    tensors = _engine_tensors(gpu_device, 77)
+    want = [t.clone() for t in tensors]
+    cl = _cpu_layout(KVCacheLayoutType.BLOCKFIRST)
+    h = start(GPUCPUTransferWorker, [TensorSharedHandle(t) for t in tensors],
+              PinnedPoolHandle(cl.kv_shape, DT), _gpu_layout(), cl, DT, 0,
+              overlap_directions=True)
+    rng = np.random.default_rng(21)
+    perm = rng.permutation(N_GPU)
+    P, G1, G2, G3 = perm[:8], perm[8:12], perm[12:16], perm[16:20]
+    hperm = rng.permutation(N_CPU)
+    HA, HB = hperm[:8], hperm[8:12]
+    first = _op(TransferType.D2H, P, HA, pool)
+    h.submit_transfer(first)
+    assert _collect(q, 1) == [(first.op_id, True, None)]
+    ops = [_op(TransferType.H2D, HA[:4], G1),        # reads host HA[:4]
+           _op(TransferType.D2H, P[4:8], HA[:4]),    # overwrites them: after that get
+           _op(TransferType.H2D, HA[4:], G2),
+           _op(TransferType.D2H, P[:4], HB)]
+    for op in ops:
+        h.submit_transfer(op)
+    done = _collect(q, 4)
+    assert sorted(d[0] for d in done) == sorted(op.op_id for op in ops) and all(d[1] for d in done)
+    last = _op(TransferType.H2D, HA[:4], G3)
+    h.submit_transfer(last)
+    assert _collect(q, 1) == [(last.op_id, True, None)]
+    torch.cuda.synchronize()
+    for l in range(L):
+        assert torch.equal(tensors[l][:, G1], want[l][:, P[:4]]), l   # what was there before the put
+        assert torch.equal(tensors[l][:, G2], want[l][:, P[4:8]]), l
+        assert torch.equal(tensors[l][:, G3], want[l][:, P[4:8]]), l  # what the put wrote
+    h.shutdown()
+    assert h.process.exitcode == 0
