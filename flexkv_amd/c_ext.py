@@ -197,6 +197,22 @@ def streams_run_concurrently(stream_a, stream_b, device: int = -1) -> bool:
     return bool(out.value)
 
 
+def link_activity_post(is_host_to_device: bool, expected_us: int, device: int = -1) -> None:
+    """Tell the other processes that use this GPU that this one keeps the host link
+    busy in one direction for about `expected_us` more.  The library posts its own
+    transfers; this is for bytes moved by other means."""
+    check(_L.fkv_link_activity_post(int(device), int(bool(is_host_to_device)), int(expected_us)))
+
+
+def link_activity_elsewhere(is_host_to_device: bool, window_ms: int = 20, device: int = -1) -> bool:
+    """Whether another process has posted link activity of that direction on this
+    GPU that has not ended more than `window_ms` ago."""
+    out = ctypes.c_int32(0)
+    check(_L.fkv_link_activity_elsewhere(int(device), int(bool(is_host_to_device)),
+                                         int(window_ms), ctypes.byref(out)))
+    return bool(out.value)
+
+
 def last_transfer_path() -> str:
     """Name of the path the last transfer issued by this thread took: KERNEL or
     one of the copy-engine strategies."""

@@ -306,7 +306,8 @@ LinkLaunchShape link_launch_shape(bool is_h2d) {
 // small requests in flight the other direction is often between two kernels at
 // the moment of a launch, and a full-chip launch would then collide with its next
 // one.  Work recorded on the launching stream itself does not count: it has
-// finished before the new launch starts.
+// finished before the new launch starts.  Launches of other processes on the same
+// GPU count through the board of fkv_linkboard.cpp.
 // FKV_LINK_ARBITER=0 switches this off; an
 // explicit FKV_{H2D,D2H}_XCD_MASK takes precedence.
 namespace {
@@ -364,7 +365,8 @@ bool link_direction_busy(int device, bool h2d, hipStream_t launching_stream) {
   DirectionActivity &d = a.dir[h2d ? 1 : 0];
   static const int64_t window_ns = (int64_t)env_int("FKV_LINK_ARBITER_WINDOW_MS", 20) * 1000000;
   const int64_t now = steady_ns();
-  bool busy = false;
+  // launches of other processes on this GPU, as far as they post them
+  bool busy = link_board_busy_elsewhere(device, h2d, window_ns);
   for (int i = 0; i < kActivityRing; ++i) {
     if (d.stream[i] != launching_stream && d.launched_ns[i] && now - d.launched_ns[i] < window_ns)
       busy = true;
@@ -380,9 +382,12 @@ bool link_direction_busy(int device, bool h2d, hipStream_t launching_stream) {
   return busy;
 }
 
-void link_direction_mark(int device, bool h2d, hipStream_t stream) {
+void link_direction_mark(int device, bool h2d, hipStream_t stream, int64_t bytes) {
   if (!arbiter_enabled())
     return;
+  // what other processes get to see: the link is taken for about this long
+  // (45 GB/s: rather a little too long than too short)
+  link_board_post(device, h2d, bytes > 0 ? bytes / 45 : 0);
   DeviceActivity &a = activity_of(device);
   std::lock_guard<std::mutex> lk(a.mu);
   DirectionActivity &d = a.dir[h2d ? 1 : 0];
@@ -540,7 +545,8 @@ int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
     a.claim = p.claims ? p.claims + 2 * l0 : nullptr; // a launch per first layer at most
     FKV_TRY(launch_copy_kernel(a, workgroups, p.threads, stream));
   }
-  link_direction_mark(p.device, p.h2d, stream);
+  link_direction_mark(p.device, p.h2d, stream,
+                      (int64_t)p.num_blocks * num_layers * p.kv_dim * p.chunk_size);
   return FKV_OK;
 }
 

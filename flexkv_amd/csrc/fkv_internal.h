@@ -208,7 +208,12 @@ struct KernelPlan {
 };
 // Link-bound launches of the last while, per device and direction (see fkv_core.cpp).
 bool link_direction_busy(int device, bool h2d, hipStream_t launching_stream);
-void link_direction_mark(int device, bool h2d, hipStream_t stream);
+void link_direction_mark(int device, bool h2d, hipStream_t stream, int64_t bytes);
+// The same across processes (fkv_linkboard.cpp): post that this process keeps the
+// link busy in one direction for about `expected_ns` more, and ask whether another
+// process has posted activity that ends less than `window_ns` ago or later.
+void link_board_post(int device, bool h2d, int64_t expected_ns);
+bool link_board_busy_elsewhere(int device, bool h2d, int64_t window_ns);
 // Builds and uploads (on `stream`) the plan for all layers of `d`.
 int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan *out);
 // Enqueues the copy of layers [layer_offset, layer_offset + num_layers) of the plan.

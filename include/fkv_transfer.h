@@ -550,6 +550,21 @@ int fkv_range_pop(void);
 int fkv_streams_run_concurrently(int32_t device, void *stream_a, void *stream_b,
                                  int32_t *concurrent);
 
+/* Link activity across processes.  A put and a get that run at the same time are
+ * kept on different XCDs; so that this also works when they come from different
+ * processes (a worker for puts, another for layerwise restores), every process
+ * posts its link-bound launches on a small board in /dev/shm (one per user and
+ * GPU, keyed by the PCI address; FKV_LINK_BOARD=0 disables it,
+ * FKV_LINK_BOARD_KEY replaces the PCI address).  The library posts its own
+ * launches; a process that moves bytes over the link by other means can post
+ * them with fkv_link_activity_post (`expected_us`: for how long from now, or from
+ * the end of what it has already posted).  fkv_link_activity_elsewhere sets *busy
+ * to 1 when another process has posted activity in that direction that has not
+ * ended more than `window_ms` ago.  No counterpart in the reference. */
+int fkv_link_activity_post(int32_t device, int32_t is_host_to_device, int64_t expected_us);
+int fkv_link_activity_elsewhere(int32_t device, int32_t is_host_to_device, int32_t window_ms,
+                                int32_t *busy);
+
 #ifdef __cplusplus
 }
 #endif

@@ -151,3 +151,52 @@ def test_profiler_ranges_are_off_unless_asked_for():
     on = subprocess.run([sys.executable, "-c", code], cwd=root, env=dict(env, FKV_ROCTX="1"),
                         capture_output=True, text=True, check=True).stdout.split()
     assert on in (["1", "1"], ["0", "0"])       # 0 0 only where no marker library is installed
+
+
+def test_link_activity_board_is_shared_between_processes():
+    """The board on which processes post their link-bound launches: what one
+    process posts, another one sees for that direction and GPU only, until it has
+    ended `window_ms` ago; a process never sees its own postings, and the posting
+    of a process that is gone is dropped."""
+    import subprocess
+    import sys
+    key = f"abitest{os.getpid()}"
+    env = dict(os.environ, FKV_LINK_BOARD_KEY=key)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    head = ("import ctypes, sys, time; sys.path.insert(0, sys.argv[1])\n"
+            "from flexkv_amd import _lib\n"
+            "L = _lib.load()\n"
+            "b = ctypes.c_int32(7)\n"
+            "def busy(dev, h2d, win):\n"
+            "    assert L.fkv_link_activity_elsewhere(dev, h2d, win, ctypes.byref(b)) == 0\n"
+            "    return b.value\n")
+    poster = subprocess.Popen(
+        [sys.executable, "-c", head +
+         "assert L.fkv_link_activity_post(0, 1, 400000) == 0\n"      # host->GPU, 0.4 s
+         "assert busy(0, 1, 20) == 0\n"                               # not its own
+         "print('posted', flush=True); sys.stdin.readline()\n", root],
+        env=env, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    try:
+        assert poster.stdout.readline().strip() == "posted"
+        probe = subprocess.run(
+            [sys.executable, "-c", head +
+             "print(busy(0, 1, 20), busy(0, 0, 20), busy(1, 1, 20))\n"
+             "time.sleep(0.6)\n"
+             "print(busy(0, 1, 20), busy(0, 1, 5000))\n"
+             "print(L.fkv_link_activity_post(0, 0, -1) != 0)\n", root],
+            env=env, capture_output=True, text=True, timeout=120)
+        assert probe.returncode == 0, probe.stderr
+        # busy host->GPU on device 0 only; over 20 ms after its 0.4 s, still within 5 s of
+        # its end; a negative duration is refused
+        assert probe.stdout.split("\n")[:3] == ["1 0 0", "0 1", "True"], probe.stdout
+    finally:
+        poster.stdin.write("\n")
+        poster.stdin.close()
+        assert poster.wait(30) == 0
+    gone = subprocess.run([sys.executable, "-c", head + "print(busy(0, 1, 5000))\n", root],
+                          env=env, capture_output=True, text=True, timeout=120)
+    assert gone.stdout.strip() == "0", gone.stdout + gone.stderr   # its slot was taken over
+    for dev in (0, 1):
+        path = f"/dev/shm/fkv_link_{os.getuid()}_{key}_{dev}"
+        if os.path.exists(path):
+            os.unlink(path)

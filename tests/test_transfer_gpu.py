@@ -1,4 +1,7 @@
 """HIP gather/scatter kernel vs the CPU oracle, through the C ABI, bit-exact."""
+import os
+import time
+
 import numpy as np
 import pytest
 
@@ -279,3 +282,56 @@ def test_streams_run_concurrently_tells_hardware_queue_sharing(gpu_device):
     table = [[streams_run_concurrently(a, b) for b in streams] for a in streams]
     assert any(table[i][j] for i in range(6) for j in range(6) if i != j), table
     assert all(not table[i][i] for i in range(6))
+
+
+def test_a_put_in_another_process_confines_the_gets_of_this_one(gpu_device):
+    """Two processes on one GPU: a child keeps posting puts, and the gets of this
+    process (too small to keep to home XCDs by themselves) confine themselves
+    because the board the processes share says that the other direction is busy.
+    Once the child has gone they run on all XCDs again."""
+    import subprocess
+    import sys
+    from flexkv_amd.c_ext import get_stats, link_activity_elsewhere, reset_stats
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    if os.environ.get("FKV_LINK_BOARD_KEY"):
+        pytest.skip("the board key of this process is fixed from outside")
+    script = (
+        "import sys, time; sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[1] + '/tests')\n"
+        "import numpy as np, torch\n"
+        "from kvsetup import KVSetup\n"
+        "dev = KVSetup(0, 4, 2, 64, 64, 65536, 'BLOCKFIRST', seed=3).to_device('cuda:0')\n"
+        "ids = np.arange(64)\n"
+        "dev.transfer(ids, ids, is_h2d=False)\n"
+        "print('putting', flush=True)\n"
+        "end = time.time() + 60\n"
+        "import select\n"
+        "while time.time() < end and not select.select([sys.stdin], [], [], 0)[0]:\n"
+        "    dev.transfer(ids, ids, is_h2d=False)\n")
+    # both processes address the GPU by its PCI address: no key in the environment
+    child = subprocess.Popen([sys.executable, "-c", script, root], stdin=subprocess.PIPE,
+                             stdout=subprocess.PIPE, text=True)
+    try:
+        assert child.stdout.readline().strip() == "putting"
+        s = KVSetup(VLLM, 4, 2, 64, 64, 4096, "BLOCKFIRST", seed=44)
+        dev = s.to_device(gpu_device)
+        rng = np.random.default_rng(3)
+        assert link_activity_elsewhere(False) and not link_activity_elsewhere(True)
+        reset_stats()
+        for _ in range(5):
+            g, c = rng.permutation(64)[:40], rng.permutation(64)[:40]
+            dev.transfer(g, c, is_h2d=True)
+            s.oracle_transfer(g, c, True)
+        st = get_stats()
+        assert st["confined_launches"] == 5, st
+        dev.assert_matches_reference("gets next to another process's puts")
+    finally:
+        child.stdin.write("\n")
+        child.stdin.close()
+        assert child.wait(60) == 0
+    time.sleep(0.1)
+    reset_stats()
+    g = np.arange(40)
+    dev.transfer(g, g, is_h2d=True)
+    s.oracle_transfer(g, g, True)
+    assert get_stats()["confined_launches"] == 0
+    dev.assert_matches_reference("get after the other process has gone")
