@@ -458,8 +458,8 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
       shape.workgroups_per_cta;
   out->threads = shape.threads;
   out->xcd_mask = shape.xcd_mask;
-  out->home_mask = 0xffu;
-  out->home_workgroups = out->workgroups;
+  out->home_mask = out->busy_mask = 0xffu;
+  out->confined_workgroups = out->workgroups;
   out->device = device;
   if (arbiter_enabled() && shape.xcd_mask == 0xffu && device_has_eight_xcds(device)) {
     static const unsigned h2d_mask = (unsigned)env_int("FKV_ARBITER_H2D_MASK", 0xf0) & 0xffu;
@@ -467,17 +467,16 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
     static const unsigned d2h_home = (unsigned)env_int("FKV_HOME_D2H_MASK", 0x0e) & 0xffu;
     static const int h2d_pct = std::max(50, env_int("FKV_ARBITER_H2D_PCT", 150));
     static const int d2h_pct = std::max(5, env_int("FKV_ARBITER_D2H_PCT", 100));
-    const int scaled = std::max(1, out->workgroups * (out->h2d ? h2d_pct : d2h_pct) / 100);
-    // Large launches keep to their direction's home XCDs even when the link is
-    // idle, so that a transfer of the other direction that starts while they run
-    // finds its own XCDs free; see the note above.
-    out->home_mask = out->h2d ? (h2d_mask ? h2d_mask : 0xf0u) : (d2h_home ? d2h_home : 0x0eu);
-    out->home_workgroups = scaled;
-    if (link_direction_busy(device, !out->h2d, stream)) {
-      // GPU->host on two XCDs, host->GPU on four others
-      out->xcd_mask = out->h2d ? (h2d_mask ? h2d_mask : 0xf0u) : (d2h_mask ? d2h_mask : 0x06u);
-      out->workgroups = scaled;
-    }
+    out->confined_workgroups =
+        std::max(1, out->workgroups * (out->h2d ? h2d_pct : d2h_pct) / 100);
+    // Which XCDs a launch of this plan keeps to is decided when it is launched (a
+    // layerwise restore launches for tens of milliseconds after its plan was
+    // built): while the other direction is busy GPU->host keeps to two XCDs and
+    // host->GPU to four others; on an idle link large launches keep to their
+    // direction's home XCDs, so that a transfer of the other direction that starts
+    // while they run finds its own XCDs free.  See the note above.
+    out->busy_mask = out->h2d ? (h2d_mask ? h2d_mask : 0xf0u) : (d2h_mask ? d2h_mask : 0x06u);
+    out->home_mask = out->h2d ? out->busy_mask : (d2h_home ? d2h_home : 0x0eu);
   }
   // FKV_PLAN_MIRROR=0: kernels read the plan in the pinned slot instead of a device
   // copy (one command less per transfer; measured no faster, so not the default).
@@ -537,10 +536,13 @@ int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
     a.xcd_mask = p.xcd_mask;
     int workgroups = p.workgroups;
     static const int64_t home_min_bytes = (int64_t)env_int("FKV_HOME_MIN_KB", 8192) * 1024;
-    if (p.xcd_mask == 0xffu && p.home_mask != 0xffu && home_min_bytes >= 0 &&
-        (int64_t)p.num_blocks * a.lk * p.chunk_size >= home_min_bytes) {
+    if (p.busy_mask != 0xffu && link_direction_busy(p.device, !p.h2d, stream)) {
+      a.xcd_mask = p.busy_mask;
+      workgroups = p.confined_workgroups;
+    } else if (p.home_mask != 0xffu && home_min_bytes >= 0 &&
+               (int64_t)p.num_blocks * a.lk * p.chunk_size >= home_min_bytes) {
       a.xcd_mask = p.home_mask;
-      workgroups = p.home_workgroups;
+      workgroups = p.confined_workgroups;
     }
     a.claim = p.claims ? p.claims + 2 * l0 : nullptr; // a launch per first layer at most
     FKV_TRY(launch_copy_kernel(a, workgroups, p.threads, stream));

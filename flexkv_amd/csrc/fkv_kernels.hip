@@ -130,15 +130,19 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
   const uint64_t total_units = (uint64_t)a.num_blocks * spp;
   const uint64_t total = a.packed ? (total_units + kPiece - 1) / kPiece : total_units;
   const int tid = threadIdx.x;
-  // A launch confined to some XCDs: workgroups elsewhere leave, the others claim
-  // ranges.  A workgroup that runs on the other direction's XCDs next to that
-  // direction's traffic moves its range at a third of the rate and holds up the
-  // whole launch, so none may stay there.  Workgroup 0 is the safety net for a
-  // launch of which no workgroup landed on a selected XCD: it looks at the claim
-  // counter after a while and takes over only if nobody has claimed anything.
+  // Launches with claim counters hand their work out in `num_claims` ranges that
+  // the workgroups claim one after the other, so that a workgroup which is slowed
+  // down (it shares its XCD with a transfer in the other direction) takes fewer.
+  // A launch confined to some XCDs: workgroups elsewhere leave.  A workgroup of one
+  // direction that runs on the other direction's XCDs next to that direction's
+  // traffic moves its range at a third of the rate and holds up the whole launch, so
+  // none may stay there.  Workgroup 0 is the safety net for a launch of which no
+  // workgroup landed on a selected XCD: it looks at the claim counter after a while
+  // and takes over only if nobody has claimed anything.
   const bool confined = (a.xcd_mask & 0xffu) != 0xffu;
+  const bool dynamic = a.num_claims != 0; // set for every confined launch
   __shared__ uint32_t s_claim;
-  // Every workgroup of a confined launch counts itself out; the last one leaves the
+  // Every workgroup of such a launch counts itself out; the last one leaves the
   // two counters zeroed for the next launch that is given them.
   auto leave = [&]() {
     if (tid == 0 &&
@@ -166,6 +170,11 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
     }
     __syncthreads();
   }
+  // lane 0 keeps the next claim in a register: it is asked for before the current
+  // range is copied and has long arrived when the range is done
+  uint32_t next_claim = 0;
+  if (dynamic && tid == 0)
+    next_claim = atomicAdd(a.claim, 1u);
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
   const int nwaves = blockDim.x / kWave;
@@ -179,9 +188,9 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
     // This workgroup's range of work units: its own share of the launch, or the next
     // unclaimed one.
     uint32_t part = blockIdx.x, parts = gridDim.x;
-    if (confined) {
+    if (dynamic) {
       if (tid == 0)
-        s_claim = atomicAdd(a.claim, 1u);
+        s_claim = next_claim;
       __syncthreads();
       part = s_claim;
       parts = a.num_claims;
@@ -190,11 +199,13 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
         leave();
         return;
       }
+      if (tid == 0)
+        next_claim = atomicAdd(a.claim, 1u);
     }
     uint64_t s0 = total * part / parts;
     uint64_t s1 = total * (part + 1) / parts;
     if (s0 >= s1) {
-      if (confined)
+      if (dynamic)
         continue;
       return;
     }
@@ -283,7 +294,7 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
         copy_slice<VEC, NTS>(src, dst, left < kSliceBytes ? left : kSliceBytes, lane);
       }
     }
-    if (!confined)
+    if (!dynamic)
       return;
   } // next claim
 }
@@ -405,6 +416,7 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_wor
   a.xcd_mask &= 0xffu;
   if (a.xcd_mask == 0 || !a.claim)
     a.xcd_mask = 0xffu;
+  a.num_claims = 0;
   if (a.xcd_mask != 0xffu) {
     // One range per working workgroup (finer ranges shift the balance between two
     // concurrent directions towards GPU->host and lower their sum); `grid` working
@@ -412,6 +424,23 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_wor
     a.num_claims = (uint32_t)std::min<int64_t>(grid, total);
     const int per_round = __builtin_popcount(a.xcd_mask);
     grid = (grid + per_round - 1) / per_round * 8;
+  } else if (a.claim) {
+    // All XCDs, some of which may be busy with the other direction (a transfer of
+    // another stream or process that started later).  With several ranges per
+    // workgroup (FKV_CLAIMS_PER_WORKGROUP=8) the workgroups there take fewer of them:
+    // a restore that stays on all XCDs next to a put loop moves 23-24 instead of
+    // 16-17 GB/s.  Off by default: alone, the same restore loses 2 % to the claims.
+    static const int per_wg = [] {
+      const char *v = std::getenv("FKV_CLAIMS_PER_WORKGROUP");
+      const int n = v && *v ? std::atoi(v) : 0;
+      return n < 0 ? 0 : n;
+    }();
+    // ranges of 128 KiB at least: a claim costs a round trip to device memory
+    const int64_t bytes = (int64_t)a.num_blocks * a.lk * a.chunk_bytes;
+    a.num_claims = (uint32_t)std::min<int64_t>(std::min<int64_t>(grid * per_wg, total),
+                                                bytes / (128 * 1024));
+    if (a.num_claims <= (uint32_t)grid) // nothing to hand out: fixed shares
+      a.num_claims = 0;
   }
   const size_t lds_bytes = (size_t)(2 * a.lk + 2 * kCopyIdTile) * sizeof(uint64_t);
   stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);

@@ -417,6 +417,19 @@ int main() {
     ++cases;
   }
 
+  // ---- the board processes share: one's own postings never count as "elsewhere" ----
+  {
+    int32_t busy = 7;
+    FKV_OK_OR_DIE(fkv_link_activity_post(-1, 1, 50000));
+    FKV_OK_OR_DIE(fkv_link_activity_elsewhere(-1, 1, 20, &busy));
+    if (busy != 0 || fkv_link_activity_post(-1, 1, -5) == FKV_OK ||
+        fkv_link_activity_elsewhere(-1, 1, 20, nullptr) == FKV_OK) {
+      fprintf(stderr, "link activity board: busy=%d\n", busy);
+      return 1;
+    }
+    ++cases;
+  }
+
   fkv_stats st;
   fkv_get_stats(&st);
   HIP_OK(hipStreamDestroy(stream));

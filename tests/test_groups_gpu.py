@@ -4,6 +4,7 @@ placement with several "ranks" sharing device 0, notification contract."""
 import ctypes
 import os
 import struct
+import time
 
 import numpy as np
 import pytest
@@ -505,4 +506,68 @@ def test_layerwise_restore_reads_ssd_blocks_first(gpu_device, tmp_path, kv_dim, 
             want = host[cb, l] if cpu_name == "BLOCKFIRST" else host[l, :, cb]
             assert torch.equal(gpu[l][:, g].cpu().view(torch.int16), want.view(torch.int16)), \
                 (l, g, cb)
+    lw.close()
+
+
+def test_layerwise_restore_while_another_stream_puts(gpu_device):
+    """Restores are launched layer by layer and decide per launch whether the other
+    direction is busy.  A thread keeps putting other blocks of the same pool while
+    restores run: some restore launches must have confined themselves, and every
+    byte is where it belongs afterwards."""
+    import threading
+    from flexkv_amd.c_ext import get_stats, reset_stats, transfer_kv_blocks
+    L, N, T, H, D, heads, kv_dim = 24, 64, 16, 1, 512, 1, 1
+    gl, cl = make_layouts(L, N, T, H, D, "BLOCKFIRST", kv_dim, heads)
+    gpu = make_gpu_tensors(L, N, T, H, D, kv_dim, gpu_device)
+    fill_gpu(gpu, 0, L, N, T, H, D, kv_dim)
+    orig = [t.clone() for t in gpu]
+    cpu = torch.zeros(cl.kv_shape, dtype=DTYPE, pin_memory=True)
+    rng = np.random.default_rng(17)
+    perm = rng.permutation(N)
+    get_ids = torch.from_numpy(perm[:24].astype(np.int64))      # restored: engine block i <- host block i
+    put_ids = torch.from_numpy(perm[24:56].astype(np.int64))    # put next to it, other blocks
+    ptrs = torch.tensor([t.data_ptr() for t in gpu], dtype=torch.int64)
+    strides = (cl.get_kv_stride() * ES, cl.get_layer_stride() * ES, cl.get_block_stride() * ES)
+
+    def put(ids, stream):
+        with torch.cuda.stream(stream):
+            transfer_kv_blocks(ids, ptrs, gl.get_kv_stride() * ES, gl.get_block_stride() * ES,
+                               gl.get_layer_stride() * ES, ids, cpu, *strides,
+                               gl.get_chunk_size() * ES, 0, L, is_host_to_device=False,
+                               kv_dim=kv_dim, num_kv_heads=heads, gpu_block_type=0, sync=True,
+                               is_blockfirst=True)
+    put(get_ids, torch.cuda.current_stream())
+    for t in gpu:
+        t[:, get_ids.to(gpu_device)] = 0
+    torch.cuda.synchronize()
+    lw = layerwise_group(cpu, [gpu], gl, L, is_blockfirst=True, num_kv_heads=heads)
+    stop, errors = threading.Event(), []
+
+    def putter():
+        s = torch.cuda.Stream()
+        try:
+            while not stop.is_set():
+                put(put_ids, s)
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+    th = threading.Thread(target=putter)
+    reset_stats()
+    th.start()
+    try:
+        time.sleep(0.02)
+        for _ in range(4):
+            run_layerwise(lw, get_ids, get_ids, cl, gl.get_chunk_size() * ES, L, kv_dim, heads,
+                          False, 1, "polling")
+            lw.synchronize()
+    finally:
+        stop.set()
+        th.join()
+    assert not errors, errors
+    torch.cuda.synchronize()
+    assert get_stats()["confined_launches"] > 0
+    for l in range(L):
+        assert torch.equal(gpu[l].view(torch.int16), orig[l].view(torch.int16)), l
+        want = orig[l][:, torch.cat([get_ids, put_ids]).to(gpu_device)].cpu().view(torch.int16)
+        got = cpu[torch.cat([get_ids, put_ids]), l].view(torch.int16).reshape(want.shape)
+        assert torch.equal(got, want), l
     lw.close()

@@ -335,3 +335,31 @@ def test_a_put_in_another_process_confines_the_gets_of_this_one(gpu_device):
     s.oracle_transfer(g, g, True)
     assert get_stats()["confined_launches"] == 0
     dev.assert_matches_reference("get after the other process has gone")
+
+
+def test_ranges_claimed_by_workgroups_on_all_xcds(gpu_device):
+    """FKV_CLAIMS_PER_WORKGROUP hands the work of a launch that uses all XCDs out
+    in ranges (read once per process, hence a child process): normal and packed
+    chunks, several transfers in a row through the same counters."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = (
+        "import sys; sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[1] + '/tests')\n"
+        "import numpy as np\n"
+        "from kvsetup import KVSetup\n"
+        "from flexkv_amd.c_ext import get_stats\n"
+        "for chunk, n in ((32768, 300), (1152, 2500), (73728, 200)):\n"
+        "    s = KVSetup(0, 6, 2, n + 50, n + 50, chunk, 'BLOCKFIRST', seed=chunk)\n"
+        "    dev = s.to_device('cuda:0')\n"
+        "    rng = np.random.default_rng(chunk)\n"
+        "    for h2d in (False, True, False, True):\n"
+        "        g, c = rng.permutation(n + 50)[:n], rng.permutation(n + 50)[:n]\n"
+        "        dev.transfer(g, c, is_h2d=h2d)\n"
+        "        s.oracle_transfer(g, c, h2d)\n"
+        "    dev.assert_matches_reference(f'chunk {chunk}')\n"
+        "print('ok', get_stats()['confined_launches'])\n")
+    env = dict(os.environ, FKV_CLAIMS_PER_WORKGROUP="8", FKV_LINK_ARBITER="0")
+    r = subprocess.run([sys.executable, "-c", script, root], env=env, capture_output=True,
+                       text=True, timeout=170)
+    assert r.returncode == 0 and r.stdout.split()[-2:] == ["ok", "0"], r.stdout + r.stderr
