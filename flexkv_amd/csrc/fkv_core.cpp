@@ -7,6 +7,7 @@
 
 #include <map>
 
+#include <algorithm>
 #include <chrono>
 #include <cstdlib>
 #include <cstring>
@@ -666,40 +667,146 @@ void fkv_reset_stats(void) {
 }
 
 namespace {
-// Blocks until everything queued on `stream` up to now has finished.  Unlike
-// hipStreamSynchronize it does not wait for work that other threads queue behind
-// it in the meantime, and the waiting thread sleeps instead of spinning: with 64
-// requests in flight over two streams the median request took 25 ms instead of
-// 82 ms, the slowest percentile 55 ms instead of 113 ms.  One event per thread and
-// device, reused.
+constexpr int kMaxDevices = 64;
+struct PerThreadEvents { // events go when their thread ends
+  hipEvent_t done[kMaxDevices][2] = {}; // blocking; [1] with the system-scope fence
+  hipEvent_t order[kMaxDevices][2] = {}; // hand-over between a caller's stream and a lane
+  ~PerThreadEvents() {
+    for (auto *set : {done, order})
+      for (int d = 0; d < kMaxDevices; ++d)
+        for (hipEvent_t e : set[d])
+          if (e && hipEventDestroy(e) != hipSuccess)
+            (void)hipGetLastError();
+  }
+};
+PerThreadEvents &my_events() {
+  thread_local PerThreadEvents mine;
+  return mine;
+}
+
+// Records, behind what is queued on `stream` so far, the event a synchronous call
+// waits on (nullptr: devices beyond the table, synchronise the stream instead).
+// Unlike hipStreamSynchronize, waiting on it does not wait for work that other
+// threads queue behind it in the meantime, and the waiting thread sleeps instead of
+// spinning: with 64 requests in flight over two streams the median request took
+// 25 ms instead of 82 ms, the slowest percentile 55 ms instead of 113 ms.  One
+// event per thread and device, reused.
 // `host_reads_result`: the transfer wrote host memory that the caller will read
 // (GPU->host): the event then keeps its system-scope fence.  A host->GPU transfer
 // leaves nothing for the host to read, and its event goes without (see
 // kBookkeepingEvent).
-int wait_for_work_queued_so_far(hipStream_t stream, bool host_reads_result) {
-  constexpr int kMaxDevices = 64;
-  struct PerThread { // events go when their thread ends
-    hipEvent_t ev[kMaxDevices][2] = {};
-    ~PerThread() {
-      for (auto &pair : ev)
-        for (hipEvent_t e : pair)
-          if (e && hipEventDestroy(e) != hipSuccess)
-            (void)hipGetLastError();
-    }
-  };
-  thread_local PerThread mine;
+int record_completion(hipStream_t stream, bool host_reads_result, hipEvent_t *out) {
+  *out = nullptr;
   int device = 0;
   FKV_HIP_TRY(hipGetDevice(&device));
-  if (device < 0 || device >= kMaxDevices) {
-    FKV_HIP_TRY(hipStreamSynchronize(stream));
+  if (device < 0 || device >= kMaxDevices)
     return FKV_OK;
-  }
-  hipEvent_t &ev = mine.ev[device][host_reads_result ? 1 : 0];
+  hipEvent_t &ev = my_events().done[device][host_reads_result ? 1 : 0];
   if (!ev)
     FKV_HIP_TRY(hipEventCreateWithFlags(
-        &ev, hipEventBlockingSync | (host_reads_result ? (unsigned)hipEventDisableTiming : fkv::kBookkeepingEvent)));
+        &ev, hipEventBlockingSync | (host_reads_result ? (unsigned)hipEventDisableTiming
+                                                        : fkv::kBookkeepingEvent)));
   FKV_HIP_TRY(hipEventRecord(ev, stream));
-  FKV_HIP_TRY(hipEventSynchronize(ev));
+  *out = ev;
+  return FKV_OK;
+}
+
+// ---- lane streams ---------------------------------------------------------
+// A process has few hardware queues (4 by default), and streams that share one
+// run their kernels in turn.  A caller that issues puts and gets from many
+// streams therefore ends up with both directions on every queue: 64 requests on
+// 64 streams move 72 GB/s, the same requests on one put stream and one get stream
+// 92-94 GB/s.  For such callers kernel transfers run on two streams of the
+// library per device, one per direction and on different hardware queues,
+// whatever stream the caller names; the caller's stream and the lane are ordered
+// by events (the lane waits for what the caller's stream holds so far; an
+// asynchronous call makes the caller's stream wait for the transfer).
+struct Lane {
+  std::mutex mu; // keeps the commands of one transfer together
+  hipStream_t stream = nullptr;
+};
+struct DeviceLanes {
+  std::mutex init;
+  bool tried = false, ok = false;
+  Lane dir[2]; // [0] GPU->host, [1] host->GPU
+};
+// FKV_LANE_STREAMS: 1 always, 0 never; unset: synchronous calls, once kernel
+// transfers of a device have been issued on more than two different streams (a
+// stream per request is then likely, and with it both directions on every
+// hardware queue).  Asynchronous calls stay on the caller's stream unless asked:
+// the hand-over to the lane and back is two more commands per transfer on each
+// stream, and a caller that pipelines many small asynchronous transfers on one
+// stream pays for them (125 transfers of 25 MB per direction: 76 instead of
+// 89 GB/s).
+bool lanes_wanted(int device, hipStream_t caller_stream, bool synchronous) {
+  static const int mode = [] {
+    const char *v = std::getenv("FKV_LANE_STREAMS");
+    return (v && *v) ? (std::strcmp(v, "0") != 0 ? 1 : 0) : -1;
+  }();
+  if (mode >= 0)
+    return mode == 1;
+  if (!synchronous)
+    return false;
+  static std::mutex mu;
+  static std::map<int, std::vector<hipStream_t>> seen;
+  std::lock_guard<std::mutex> lk(mu);
+  std::vector<hipStream_t> &v = seen[device];
+  if (v.size() > 2)
+    return true;
+  if (std::find(v.begin(), v.end(), caller_stream) == v.end())
+    v.push_back(caller_stream);
+  return v.size() > 2;
+}
+Lane *lane_of(int device, bool h2d) {
+  static std::mutex mu;
+  static std::map<int, DeviceLanes *> all; // live until the process ends
+  DeviceLanes *dl;
+  {
+    std::lock_guard<std::mutex> lk(mu);
+    DeviceLanes *&p = all[device];
+    if (!p)
+      p = new DeviceLanes();
+    dl = p;
+  }
+  std::lock_guard<std::mutex> lk(dl->init);
+  if (!dl->tried) {
+    dl->tried = true;
+    hipStream_t a = nullptr, b = nullptr;
+    if (hipStreamCreateWithFlags(&a, hipStreamNonBlocking) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    // a partner on another hardware queue; streams that are not kept stay alive, so
+    // that the next one lands on a different queue
+    for (int attempt = 0; attempt < 8; ++attempt) {
+      if (hipStreamCreateWithFlags(&b, hipStreamNonBlocking) != hipSuccess) {
+        (void)hipGetLastError();
+        b = nullptr;
+        break;
+      }
+      int32_t concurrent = 0;
+      if (fkv_streams_run_concurrently(device, a, b, &concurrent) == FKV_OK && concurrent)
+        break;
+    }
+    if (b) {
+      dl->dir[0].stream = a;
+      dl->dir[1].stream = b;
+      dl->ok = true;
+    }
+  }
+  return dl->ok ? &dl->dir[h2d ? 1 : 0] : nullptr;
+}
+// A hand-over event of this thread, recorded on `from`, that `to` waits for.
+int order_after(hipStream_t from, hipStream_t to, int device, int which) {
+  if (device < 0 || device >= kMaxDevices) {
+    FKV_HIP_TRY(hipStreamSynchronize(from));
+    return FKV_OK;
+  }
+  hipEvent_t &ev = my_events().order[device][which];
+  if (!ev)
+    FKV_HIP_TRY(hipEventCreateWithFlags(&ev, fkv::kBookkeepingEvent));
+  FKV_HIP_TRY(hipEventRecord(ev, from));
+  FKV_HIP_TRY(hipStreamWaitEvent(to, ev, 0));
   return FKV_OK;
 }
 } // namespace
@@ -733,15 +840,43 @@ int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream_v) {
   int engine = forced_engine >= 0 ? forced_engine : d.use_ce_transfer;
   if (engine == 2)
     FKV_TRY(choose_engine(d, &engine, nullptr, nullptr));
-  int rc = engine ? run_ce_path(d, stream) : run_kernel_path(d, stream);
-  if (rc != FKV_OK)
-    return rc;
+  int device = 0;
+  FKV_HIP_TRY(hipGetDevice(&device));
+  Lane *lane = (!engine && lanes_wanted(device, stream, d.sync != 0)) ? lane_of(device, d.is_host_to_device != 0)
+                                                         : nullptr;
+  hipEvent_t done = nullptr;
+  int rc;
+  if (lane) {
+    std::lock_guard<std::mutex> lk(lane->mu);
+    // the lane starts after what the caller's stream holds; an idle stream holds nothing
+    if (hipStreamQuery(stream) != hipSuccess) {
+      (void)hipGetLastError();
+      FKV_TRY(order_after(stream, lane->stream, device, 0));
+    }
+    rc = run_kernel_path(d, lane->stream);
+    if (rc != FKV_OK)
+      return rc;
+    if (d.sync)
+      FKV_TRY(record_completion(lane->stream, !d.is_host_to_device, &done));
+    else
+      FKV_TRY(order_after(lane->stream, stream, device, 1));
+    stream = lane->stream;
+  } else {
+    rc = engine ? run_ce_path(d, stream) : run_kernel_path(d, stream);
+    if (rc != FKV_OK)
+      return rc;
+    if (d.sync)
+      FKV_TRY(record_completion(stream, /*host_reads_result=*/!d.is_host_to_device, &done));
+  }
   (d.is_host_to_device ? stats().bytes_h2d : stats().bytes_d2h)
       .fetch_add(bytes, std::memory_order_relaxed);
 
   if (d.sync) {
     auto t0 = std::chrono::steady_clock::now();
-    FKV_TRY(wait_for_work_queued_so_far(stream, /*host_reads_result=*/!d.is_host_to_device));
+    if (done)
+      FKV_HIP_TRY(hipEventSynchronize(done));
+    else
+      FKV_HIP_TRY(hipStreamSynchronize(stream));
     if (d.enable_trace) {
       double ms = std::chrono::duration<double, std::milli>(
                       std::chrono::steady_clock::now() - t0)

@@ -363,3 +363,66 @@ def test_ranges_claimed_by_workgroups_on_all_xcds(gpu_device):
     r = subprocess.run([sys.executable, "-c", script, root], env=env, capture_output=True,
                        text=True, timeout=170)
     assert r.returncode == 0 and r.stdout.split()[-2:] == ["ok", "0"], r.stdout + r.stderr
+
+
+def test_lane_streams_keep_the_order_of_the_callers_stream(gpu_device):
+    """FKV_LANE_STREAMS=1 (read once per process, hence a child process): transfers
+    run on the library's own two streams.  What the caller's stream held before a
+    call is finished before the transfer starts, and work queued on the caller's
+    stream behind an asynchronous call sees the transferred bytes; puts and gets
+    from several threads and streams at once still land where they belong."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = (
+        "import sys, threading; sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[1] + '/tests')\n"
+        "import numpy as np, torch\n"
+        "from kvsetup import KVSetup\n"
+        "s = KVSetup(0, 4, 2, 96, 96, 65536, 'BLOCKFIRST', seed=5)\n"
+        "dev = s.to_device('cuda:0')\n"
+        "st = torch.cuda.Stream()\n"
+        "big = torch.empty(1 << 28, dtype=torch.uint8, device='cuda')\n"
+        "ids = np.arange(8)\n"
+        "with torch.cuda.stream(st):\n"
+        "    for rep in range(5):\n"
+        "        # (1) the stream is busy, then overwrites the blocks; the put must see that\n"
+        "        for _ in range(4): big.add_(1)\n"
+        "        for l, t in enumerate(dev.gpu):\n"
+        "            t.view(torch.uint8).view(2, 96, -1)[:, :8] = rep * 16 + l\n"
+        "            s.gpu_ref[l].view(np.uint8).reshape(2, 96, -1)[:, :8] = rep * 16 + l\n"
+        "        dev.transfer(ids, ids + 40, is_h2d=False)          # synchronous\n"
+        "        s.oracle_transfer(ids, ids + 40, False)\n"
+        "        # (2) asynchronous get; a copy queued behind it on the stream must see it\n"
+        "        dev.transfer(ids + 20, ids + 40, is_h2d=True, sync=False)\n"
+        "        s.oracle_transfer(ids + 20, ids + 40, True)\n"
+        "        seen = [t.view(torch.uint8).view(2, 96, -1)[:, 20:28].clone() for t in dev.gpu]\n"
+        "        st.synchronize()\n"
+        "        for l, x in enumerate(seen):\n"
+        "            assert int(x.min()) == int(x.max()) == rep * 16 + l, (rep, l, int(x.min()), int(x.max()))\n"
+        "dev.assert_matches_reference('ordering')\n"
+        "# (3) eight threads, eight streams, puts and gets of disjoint blocks\n"
+        "rng = np.random.default_rng(2)\n"
+        "pg, pc = rng.permutation(96), rng.permutation(96)\n"
+        "errs = []\n"
+        "def work(i):\n"
+        "    try:\n"
+        "        with torch.cuda.stream(torch.cuda.Stream()):\n"
+        "            for k in range(3):\n"
+        "                lo = (i * 3 + k) * 4\n"
+        "                dev.transfer(pg[lo:lo + 4], pc[lo:lo + 4], is_h2d=(i % 2 == 1))\n"
+        "    except Exception as e:\n"
+        "        errs.append(e)\n"
+        "ths = [threading.Thread(target=work, args=(i,)) for i in range(8)]\n"
+        "[t.start() for t in ths]; [t.join() for t in ths]\n"
+        "assert not errs, errs\n"
+        "for i in range(8):\n"
+        "    for k in range(3):\n"
+        "        lo = (i * 3 + k) * 4\n"
+        "        s.oracle_transfer(pg[lo:lo + 4], pc[lo:lo + 4], i % 2 == 1)\n"
+        "torch.cuda.synchronize()\n"
+        "dev.assert_matches_reference('threads')\n"
+        "print('ok')\n")
+    env = dict(os.environ, FKV_LANE_STREAMS="1")
+    r = subprocess.run([sys.executable, "-c", script, root], env=env, capture_output=True,
+                       text=True, timeout=170)
+    assert r.returncode == 0 and r.stdout.split()[-1:] == ["ok"], r.stdout + r.stderr
