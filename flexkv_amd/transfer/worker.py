@@ -579,12 +579,12 @@ class GPUCPUTransferWorker(TransferWorkerBase):
         self.gpu_block_type_ = gpu_block_type_from_tensor_count(ref_tensors, ref_layers)
         self.transfer_stream = torch.cuda.Stream()
         # Gets next to puts.  The link carries both directions at once (93 GB/s in
-        # sum against 57 one after the other), so with `overlap_directions` H2D ops
-        # run on a second thread and stream while this thread runs everything else.
-        # Ops of one direction still run in arrival order; an op that shares a block
-        # with an unfinished op of the other direction waits for it.  Completions
-        # of different directions may therefore overtake each other, which the
-        # reference's one-at-a-time worker never does: opt-in
+        # sum against 57 one after the other), so with `overlap_directions` D2H and
+        # H2D ops each run on a thread and stream of their own while this thread only
+        # hands them out.  Ops of one direction still run in arrival order; an op
+        # that shares a block with an unfinished op of the other direction waits for
+        # it.  Completions of different directions may therefore overtake each
+        # other, which the reference's one-at-a-time worker never does: opt-in
         # (FKV_WORKER_OVERLAP_DIRECTIONS=1 sets the default).
         if overlap_directions is None:
             overlap_directions = os.environ.get("FKV_WORKER_OVERLAP_DIRECTIONS", "0") == "1"
@@ -592,6 +592,7 @@ class GPUCPUTransferWorker(TransferWorkerBase):
         if overlap_directions:
             self.h2d_stream = self._stream_on_another_queue(self.transfer_stream)
             self._lanes["h2d"] = _SideLane("h2d", self._run_one, gpu_device_id)
+            self._lanes["d2h"] = _SideLane("d2h", self._run_one, gpu_device_id)
         self.transfer_num_cta_h2d = transfer_num_cta_h2d
         self.transfer_num_cta_d2h = transfer_num_cta_d2h
         self.use_ce_transfer_h2d = use_ce_transfer_h2d
@@ -622,22 +623,24 @@ class GPUCPUTransferWorker(TransferWorkerBase):
         return s
 
     def _dispatch(self, op) -> None:
-        lane = self._lanes.get("h2d")
-        if lane is None:
+        if not self._lanes:
+            return self._run_one(op)
+        kind = op.transfer_type
+        if kind not in (TransferType.H2D, TransferType.D2H):
+            # host<->SSD ops run on this thread once both lanes are empty
+            for lane in self._lanes.values():
+                lane.drain()
             return self._run_one(op)
         src, dst = self.get_transfer_block_ids(op)
         src_ids, dst_ids = src.numpy(), dst.numpy()
-        kind = op.transfer_type
-        if kind == TransferType.H2D:
-            # ops of this thread are finished when it gets here: nothing to wait for
-            lane.submit(op, src_ids, dst_ids)
-            return
-        if kind == TransferType.D2H:      # writes host blocks, reads engine blocks
-            lane.wait_until_clear_of(dst_ids, src_ids)
-        elif kind == TransferType.DISK2H:  # writes host blocks
-            lane.wait_until_clear_of(dst_ids, None)
-        # H2DISK only reads host blocks, as the gets do
-        self._run_one(op)
+        if kind == TransferType.H2D:   # reads host blocks `src`, writes engine blocks `dst`
+            cpu_ids, gpu_ids, mine, other = src_ids, dst_ids, "h2d", "d2h"
+        else:                          # reads engine blocks `src`, writes host blocks `dst`
+            cpu_ids, gpu_ids, mine, other = dst_ids, src_ids, "d2h", "h2d"
+        # ops of one lane run in order; an unfinished op of the other lane that touches
+        # the same host or engine blocks goes first (nothing else is handed out meanwhile)
+        self._lanes[other].wait_until_clear_of(cpu_ids, gpu_ids)
+        self._lanes[mine].submit(op, cpu_ids, gpu_ids)
 
     def _init_multi_group(self, gpu_blocks_per_group, gpu_layouts_per_group,
                           cpu_kv_layout: MultiGroupBlockLayout, layer_groups) -> None:

@@ -376,10 +376,11 @@ def test_gpu_worker_that_also_serves_the_ssd_tier(gpu_device, engine, tmp_path, 
 
 
 def test_gpu_worker_runs_gets_next_to_puts(gpu_device, engine):
-    """overlap_directions: H2D ops run on a second thread and stream of the worker.
-    Four ops are submitted back to back; the put that overwrites host blocks an
-    unfinished get still reads has to wait for that get, the others may overlap.
-    Every op is reported once, in whatever order."""
+    """overlap_directions: D2H and H2D ops each run on a thread and stream of their
+    own.  Five ops are submitted back to back; the put that overwrites host blocks
+    an unfinished get still reads has to wait for that get, the get that reads what
+    an unfinished put writes for that put, the others may overlap.  Every op is
+    reported once, in whatever order."""
     start, q, pool = engine
     tensors = _engine_tensors(gpu_device, 77)
     want = [t.clone() for t in tensors]
@@ -389,7 +390,7 @@ def test_gpu_worker_runs_gets_next_to_puts(gpu_device, engine):
               overlap_directions=True)
     rng = np.random.default_rng(21)
     perm = rng.permutation(N_GPU)
-    P, G1, G2, G3 = perm[:8], perm[8:12], perm[12:16], perm[16:20]
+    P, G1, G2, G3, G4 = perm[:8], perm[8:12], perm[12:16], perm[16:20], perm[20:24]
     hperm = rng.permutation(N_CPU)
     HA, HB = hperm[:8], hperm[8:12]
     first = _op(TransferType.D2H, P, HA, pool)
@@ -398,10 +399,11 @@ def test_gpu_worker_runs_gets_next_to_puts(gpu_device, engine):
     ops = [_op(TransferType.H2D, HA[:4], G1),        # reads host HA[:4]
            _op(TransferType.D2H, P[4:8], HA[:4]),    # overwrites them: after that get
            _op(TransferType.H2D, HA[4:], G2),
-           _op(TransferType.D2H, P[:4], HB)]
+           _op(TransferType.D2H, P[:4], HB),
+           _op(TransferType.H2D, HB, G4)]            # reads what the put before it writes
     for op in ops:
         h.submit_transfer(op)
-    done = _collect(q, 4)
+    done = _collect(q, 5)
     assert sorted(d[0] for d in done) == sorted(op.op_id for op in ops) and all(d[1] for d in done)
     last = _op(TransferType.H2D, HA[:4], G3)
     h.submit_transfer(last)
@@ -411,5 +413,6 @@ def test_gpu_worker_runs_gets_next_to_puts(gpu_device, engine):
         assert torch.equal(tensors[l][:, G1], want[l][:, P[:4]]), l   # what was there before the put
         assert torch.equal(tensors[l][:, G2], want[l][:, P[4:8]]), l
         assert torch.equal(tensors[l][:, G3], want[l][:, P[4:8]]), l  # what the put wrote
+        assert torch.equal(tensors[l][:, G4], want[l][:, P[:4]]), l   # the get waited for its put
     h.shutdown()
     assert h.process.exitcode == 0
