@@ -403,7 +403,7 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=F
                 restore_alone_ms=restore_alone_ms)
 
 
-def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32):
+def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, verify=True):
     """c4: 32 D2H puts and 32 H2D gets issued at once from 64 threads.  Each
     direction has its own set of streams (one per request by default); the
     process has 4 hardware queues, so with more than 2 streams per direction
@@ -422,6 +422,19 @@ def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32):
     lat = [[] for _ in reqs]
     walls = []
     w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=num_cta, sync=True)  # fill the host cache
+    if verify:
+        # make every request visible: engine blocks of the puts change sign (the host still
+        # holds the old values), engine blocks of the gets are wiped (the host holds them)
+        for i, (gi, _) in enumerate(reqs):
+            idx = gi.to(w.device)
+            for l in range(w.L):
+                for kv in range(w.kv_dim):
+                    rows = w.gpu_rows(l, kv)
+                    if i % 2 == 0:
+                        rows.index_copy_(0, idx, rows.index_select(0, idx) ^ 0x80)
+                    else:
+                        rows.index_fill_(0, idx, 0)
+        torch.cuda.synchronize()
 
     def worker(i, barrier, record):
         gi, ci = reqs[i]
@@ -448,8 +461,15 @@ def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32):
     all_lat = sorted(x for l in lat for x in l)
     p99 = all_lat[min(len(all_lat) - 1, int(0.99 * len(all_lat)))]
     total_bytes = sum(int(g.numel()) for g, _ in reqs) * w.L * w.kv_dim * w.chunk
+    # after the requests the host image of every block equals its engine block, and no
+    # block of a get is still wiped
+    ok = None
+    if verify:
+        ok = w.verify_host_image(w.gpu_ids, w.cpu_ids) and all(
+            bool(w.gpu_rows(l, 0).index_select(0, reqs[1][0].to(w.device)).any())
+            for l in (0, w.L - 1))
     return dict(walls=walls, p99_ms=p99, p50_ms=_median(all_lat), total_bytes=total_bytes,
-                blocks=[int(g.numel()) for g, _ in reqs])
+                blocks=[int(g.numel()) for g, _ in reqs], bit_exact=ok)
 
 
 def run_notify_scales(torch, device, num_cta, iters=20, warmup=3):
@@ -1115,7 +1135,9 @@ def main():
                            "frac_of_link_peak": round(achieved / link["h2d"], 4)}
     else:  # c4
         r = run_concurrent(w, torch, args.steps, args.warmup, args.num_cta,
-                           args.streams_per_direction)
+                           args.streams_per_direction, verify=not args.no_verify)
+        if r["bit_exact"] is not None:
+            out["bit_exact"] = r["bit_exact"]
         bidir = measure_link_bidirectional(torch, device)
         agg = r["total_bytes"] / _median(r["walls"]) / 1e9
         out.update(value=round(agg, 3), ms_per_step=round(_median(r["walls"]) * 1e3, 3),
