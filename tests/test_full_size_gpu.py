@@ -86,3 +86,24 @@ def test_layerwise_restore_at_full_size(workload, notify):
     torch.cuda.synchronize()
     assert checksums(w) == before
     grp.close()
+
+
+@pytest.mark.parametrize("workload", ["c4"], indirect=True)
+@pytest.mark.parametrize("streams_per_direction", [32, 1])
+def test_concurrent_requests_at_full_size(workload, streams_per_direction):
+    """c4: 32 puts and 32 gets from 64 threads at once on a 32768-block pool, a
+    stream per request or one per direction.  The engine blocks of the puts are
+    changed and those of the gets wiped beforehand; afterwards the host image of
+    every block equals its engine block, and blocks of no request are untouched."""
+    w = workload
+    used = torch.zeros(w.num_gpu_blocks, dtype=torch.bool)
+    used[w.gpu_ids] = True
+    idle = (~used).nonzero().flatten()[:4096].to(w.device)
+    before = [int(w.gpu_rows(l, kv).index_select(0, idle).view(torch.int64).sum())
+              for l in (0, w.L // 2, w.L - 1) for kv in range(w.kv_dim)]
+    r = bench.run_concurrent(w, torch, steps=2, warmup=1, num_cta=4,
+                             streams_per_direction=streams_per_direction, verify=True)
+    assert r["bit_exact"] is True
+    after = [int(w.gpu_rows(l, kv).index_select(0, idle).view(torch.int64).sum())
+             for l in (0, w.L // 2, w.L - 1) for kv in range(w.kv_dim)]
+    assert before == after
