@@ -301,7 +301,7 @@ LinkLaunchShape link_launch_shape(bool is_h2d) {
 // on two XCDs and nothing on three (1-3), a lone host->GPU transfer nothing on 4-7,
 // so launches of 8 MiB and more (FKV_HOME_MIN_KB, -1: never) keep to these home
 // XCDs even when the link is idle: a put launched alone and a get that arrives
-// 1 ms later reach 90 GB/s instead of 78, in the other order instead of 66.
+// 1 ms later reach 93 GB/s instead of 78, in the other order 80 instead of 66.
 // A direction also counts as busy for a short
 // while after its last launch (FKV_LINK_ARBITER_WINDOW_MS, default 20): with many
 // small requests in flight the other direction is often between two kernels at
@@ -460,7 +460,7 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
   out->threads = shape.threads;
   out->xcd_mask = shape.xcd_mask;
   out->home_mask = out->busy_mask = 0xffu;
-  out->confined_workgroups = out->workgroups;
+  out->confined_workgroups = out->home_workgroups = out->workgroups;
   out->device = device;
   if (arbiter_enabled() && shape.xcd_mask == 0xffu && device_has_eight_xcds(device)) {
     static const unsigned h2d_mask = (unsigned)env_int("FKV_ARBITER_H2D_MASK", 0xf0) & 0xffu;
@@ -478,6 +478,11 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
     // while they run finds its own XCDs free.  See the note above.
     out->busy_mask = out->h2d ? (h2d_mask ? h2d_mask : 0xf0u) : (d2h_mask ? d2h_mask : 0x06u);
     out->home_mask = out->h2d ? out->busy_mask : (d2h_home ? d2h_home : 0x0eu);
+    // on an idle link the home XCDs get no more workgroups than a launch on all XCDs
+    // would: what a copy costs the kernels next to it grows with their number (a
+    // 2048^3 GEMM takes 47 us next to 16 host->GPU workgroups, confined or not, and
+    // 67 us next to 24), and 16 on four XCDs already reach the link rate
+    out->home_workgroups = out->workgroups;
   }
   // Kernels read the plan from a device copy, which a small kernel uploads first,
   // or where it is, in the pinned slot.  Next to a transfer in the other direction
@@ -551,7 +556,7 @@ int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
     } else if (p.home_mask != 0xffu && home_min_bytes >= 0 &&
                (int64_t)p.num_blocks * a.lk * p.chunk_size >= home_min_bytes) {
       a.xcd_mask = p.home_mask;
-      workgroups = p.confined_workgroups;
+      workgroups = p.home_workgroups;
     }
     a.claim = p.claims ? p.claims + 2 * l0 : nullptr; // a launch per first layer at most
     FKV_TRY(launch_copy_kernel(a, workgroups, p.threads, stream));

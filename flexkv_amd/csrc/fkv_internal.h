@@ -200,12 +200,12 @@ struct KernelPlan {
   int64_t chunk_size = 0, gpu_block_stride = 0, cpu_block_stride = 0;
   int workgroups = 1, threads = 64;
   unsigned xcd_mask = 0xff;  // XCDs every launch is restricted to by configuration
-  // XCDs of a launch that finds the other direction busy, XCDs of a launch that
-  // moves a lot while the link is idle, and the workgroups of either (0xff: all
-  // XCDs with `workgroups`)
+  // XCDs and workgroups of a launch that finds the other direction busy, and of a
+  // launch that moves a lot while the link is idle (0xff: all XCDs with `workgroups`)
   unsigned busy_mask = 0xff;
-  unsigned home_mask = 0xff;
   int confined_workgroups = 1;
+  unsigned home_mask = 0xff;
+  int home_workgroups = 1;
   int device = 0;
   uint32_t *claims = nullptr; // a zeroed pair of counters per layer of the plan, device memory
 };

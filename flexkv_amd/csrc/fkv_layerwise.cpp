@@ -631,10 +631,6 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
           break;
         (void)hipSetDevice(g->device_ids[i]);
         rc = kernel_plan_build(d, g->streams[i], &lane.plans[i]);
-        // A restore runs next to the engine's compute kernels, which suffer less from
-        // copy wavefronts spread over all XCDs than from the same on four (compute
-        // 1.46x against 1.72x slower, the restore 53.7 against 50.1 GB/s): no home XCDs.
-        lane.plans[i].home_mask = 0xffu;
       }
     }
   for (int b = 0; b < num_batches && rc == FKV_OK; ++b) {
