@@ -550,13 +550,23 @@ int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
     a.xcd_mask = p.xcd_mask;
     int workgroups = p.workgroups;
     static const int64_t home_min_bytes = (int64_t)env_int("FKV_HOME_MIN_KB", 8192) * 1024;
+    // Ranges per workgroup.  Next to a transfer in the other direction one each is
+    // best (finer ranges shift the balance towards GPU->host and lower the sum: two
+    // threads with 25 MB requests 88.9 against 87.5 GB/s).  On an idle link the
+    // neighbours are the engine's compute kernels, which slow down single
+    // workgroups of a copy, and with one range each the slowest one holds up the
+    // launch: a restore next to fused-attention calls moves 37 GB/s with one range
+    // per workgroup and 54 GB/s with two.
+    static const int home_claims = std::max(1, env_int("FKV_HOME_CLAIMS_PER_WORKGROUP", 2));
     if (p.busy_mask != 0xffu && link_direction_busy(p.device, !p.h2d, stream)) {
       a.xcd_mask = p.busy_mask;
       workgroups = p.confined_workgroups;
+      a.claims_per_wg = 1;
     } else if (p.home_mask != 0xffu && home_min_bytes >= 0 &&
                (int64_t)p.num_blocks * a.lk * p.chunk_size >= home_min_bytes) {
       a.xcd_mask = p.home_mask;
       workgroups = p.home_workgroups;
+      a.claims_per_wg = home_claims;
     }
     a.claim = p.claims ? p.claims + 2 * l0 : nullptr; // a launch per first layer at most
     FKV_TRY(launch_copy_kernel(a, workgroups, p.threads, stream));

@@ -146,6 +146,7 @@ struct CopyKernelArgs {
   // last one zeroes both again.  Without counters the mask is ignored.
   uint32_t *claim;
   uint32_t num_claims;
+  int32_t claims_per_wg; // confined launches: ranges per working workgroup (0 = 1)
 };
 constexpr int kCopyBlockThreads = 1024;  // largest workgroup the kernel is built for
 constexpr int kCopyUnroll = 8;           // vector accesses in flight per lane

@@ -418,10 +418,10 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_wor
     a.xcd_mask = 0xffu;
   a.num_claims = 0;
   if (a.xcd_mask != 0xffu) {
-    // One range per working workgroup (finer ranges shift the balance between two
-    // concurrent directions towards GPU->host and lower their sum); `grid` working
-    // workgroups need grid / popcount(mask) rounds of 8.
-    a.num_claims = (uint32_t)std::min<int64_t>(grid, total);
+    // `claims_per_wg` ranges per working workgroup (the caller's choice, 1 if it
+    // makes none); `grid` working workgroups need grid / popcount(mask) rounds of 8.
+    const int per_wg = a.claims_per_wg > 0 ? a.claims_per_wg : 1;
+    a.num_claims = (uint32_t)std::min<int64_t>(grid * per_wg, total);
     const int per_round = __builtin_popcount(a.xcd_mask);
     grid = (grid + per_round - 1) / per_round * 8;
   } else if (a.claim) {
