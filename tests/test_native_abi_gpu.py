@@ -32,14 +32,21 @@ def test_host_code_under_address_sanitizer(gpu_device):
     assert "AddressSanitizer" not in r.stderr
 
 
-def test_two_threads_of_a_native_program_put_and_get_at_once(gpu_device):
+@pytest.mark.parametrize("asan", [False, True], ids=["plain", "asan"])
+def test_two_threads_of_a_native_program_put_and_get_at_once(gpu_device, asan):
     """tests/native/two_way_driver.cpp: concurrent calls from plain C++ threads,
     every block compared afterwards; both directions together move more than
-    either alone."""
-    exe = os.path.join(BUILD, "two_way_driver")
+    either alone.  Also against the library whose host code is under
+    AddressSanitizer, with the lane streams forced on."""
+    exe = os.path.join(BUILD, "asan" if asan else "", "two_way_driver")
     assert os.path.exists(exe), f"{exe} is missing: run make -C tests/native"
-    r = subprocess.run([exe, "0.4", "64"], capture_output=True, text=True, timeout=120)
+    env = dict(os.environ)
+    if asan:
+        env.update(ASAN_OPTIONS="protect_shadow_gap=0:detect_leaks=0:verify_asan_link_order=0",
+                   FKV_LANE_STREAMS="1")
+    r = subprocess.run([exe, "0.4", "64"], capture_output=True, text=True, timeout=120, env=env)
     assert r.returncode == 0 and r.stdout.startswith("ok:"), r.stdout + r.stderr
+    assert "AddressSanitizer" not in r.stderr
     import re
     nums = [float(x) for x in re.findall(r"([0-9.]+) GB/s", r.stdout)]
     assert len(nums) == 3 and nums[2] > 1.2 * max(nums[0], nums[1]), r.stdout
