@@ -686,12 +686,16 @@ class GPUCPUTransferWorker(TransferWorkerBase):
                     enable_transfer_trace=global_env().enable_transfer_trace)
         if self.group_transfer_params is not None:
             flat = self.cpu_tensor.view(torch.uint8).view(-1)
-            for gp in self.group_transfer_params:  # one call per group, its slice of the block
+            # one call per group, its slice of the block; the calls share a stream, so only
+            # the last one waits (the library copies the ids of an asynchronous call)
+            last = len(self.group_transfer_params) - 1
+            for i, gp in enumerate(self.group_transfer_params):
                 transfer_kv_blocks(gpu_ids, gp["gpu_ptrs"], gp["gpu_kv_stride"],
                                    gp["gpu_block_stride"], gp["gpu_layer_stride"], cpu_ids,
                                    flat[gp["cpu_offset_bytes"]:], gp["cpu_kv_stride"],
                                    gp["cpu_layer_stride"], gp["cpu_block_stride"],
-                                   gp["chunk_size"], 0, gp["num_layers"], **tail)
+                                   gp["chunk_size"], 0, gp["num_layers"],
+                                   **dict(tail, sync=(i == last)))
             return
         transfer_kv_blocks(gpu_ids, self.gpu_blocks_ptrs, self.gpu_kv_stride_in_bytes,
                            self.gpu_block_stride_in_bytes, self.gpu_layer_stride_in_bytes,
