@@ -426,3 +426,21 @@ def test_lane_streams_keep_the_order_of_the_callers_stream(gpu_device):
     r = subprocess.run([sys.executable, "-c", script, root], env=env, capture_output=True,
                        text=True, timeout=170)
     assert r.returncode == 0 and r.stdout.split()[-1:] == ["ok"], r.stdout + r.stderr
+
+
+@pytest.mark.parametrize("chunk,n", [(64, 200000), (16384, 12000)], ids=["200k-x-64B", "12k-x-16KiB"])
+def test_very_many_blocks_in_one_call(gpu_device, chunk, n):
+    """Hundreds of thousands of block positions in one call: plan memory of several
+    MiB, hundreds of id tiles per workgroup, work-unit counts beyond 2^21 (packed
+    mode for the short chunks)."""
+    s = KVSetup(VLLM, 2, 2, n + 1000, n + 1000, chunk, "BLOCKFIRST", seed=n)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(n)
+    gids, cids = rng.permutation(n + 1000)[:n], rng.permutation(n + 1000)[:n]
+    dev.transfer(gids, cids, is_h2d=False)
+    s.oracle_transfer(gids, cids, False)
+    dev.assert_matches_reference(f"{n} blocks D2H")
+    back = rng.permutation(n + 1000)[:n]
+    dev.transfer(back, cids, is_h2d=True)
+    s.oracle_transfer(back, cids, True)
+    dev.assert_matches_reference(f"{n} blocks H2D")
