@@ -159,7 +159,16 @@ PlanSlot *plan_acquire(int device, size_t bytes) {
       }
       void *c = nullptr;
       const size_t cbytes = (size_t)kPlanCounterPairs * 2 * sizeof(uint32_t);
-      if (hipMalloc(&c, cbytes) != hipSuccess || hipMemset(c, 0, cbytes) != hipSuccess) {
+      // Zeroed by a copy that has finished when it returns.  hipMemset runs on the
+      // null stream and need not be over when the first kernel on a non-blocking
+      // stream uses the counters: cleared under a running launch, its workgroups never
+      // count to the end, the counters stay dirty, and the next launch that is given
+      // them finds no work to claim and is left to the lone safety-net workgroup
+      // (8 GiB at 7.7 GB/s, once in a few dozen processes).
+      static const std::vector<uint32_t> zeros((size_t)kPlanCounterPairs * 2, 0u);
+      if (hipMalloc(&c, cbytes) != hipSuccess ||
+          hipMemcpy(c, zeros.data(), cbytes, hipMemcpyHostToDevice) != hipSuccess ||
+          hipStreamSynchronize(nullptr) != hipSuccess) {
         (void)hipGetLastError();
         if (c)
           (void)hipFree(c);
@@ -517,6 +526,59 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
   return FKV_OK;
 }
 
+namespace {
+// The kernel's view of layers [l0, l0 + nl) of a plan.
+CopyKernelArgs plan_job(const KernelPlan &p, int l0, int nl) {
+  const uint64_t *gb = p.gpu_base + (size_t)l0 * p.kv_dim;
+  const uint64_t *cb = p.cpu_base + (size_t)l0 * p.kv_dim;
+  CopyKernelArgs a{};
+  a.base_src = p.h2d ? cb : gb;
+  a.base_dst = p.h2d ? gb : cb;
+  a.ids_src = p.h2d ? p.cpu_ids : p.gpu_ids;
+  a.ids_dst = p.h2d ? p.gpu_ids : p.cpu_ids;
+  a.stride_src = p.h2d ? p.cpu_block_stride : p.gpu_block_stride;
+  a.stride_dst = p.h2d ? p.gpu_block_stride : p.cpu_block_stride;
+  a.chunk_bytes = p.chunk_size;
+  a.num_blocks = p.num_blocks;
+  a.lk = nl * p.kv_dim;
+  a.vec = p.vec;
+  a.nt_store = p.h2d ? 1 : 0;
+  // Packed short chunks cost a wavefront more address arithmetic per request, so
+  // such launches get half as many workgroups again.  Host->GPU, 2304-byte chunks:
+  // 16 x 64 lanes reach 45 GB/s, 24 x 64 reach 55.8, 32 x 64 reach 56.2; GPU->host:
+  // 48 x 64 lanes 50.7 GB/s, 72 x 64 52.5, 96 x 64 53.0.
+  a.packed_grid_pct = 150;
+  a.xcd_mask = p.xcd_mask;
+  a.claim = p.claims ? p.claims + 2 * l0 : nullptr; // a launch per first layer at most
+  return a;
+}
+
+// Which XCDs, how many workgroups and how many ranges per workgroup a launch of
+// `bytes` gets now; `a` is the (first) job of the launch.
+int shape_for_now(const KernelPlan &p, int64_t bytes, hipStream_t stream, CopyKernelArgs *a) {
+  int workgroups = p.workgroups;
+  static const int64_t home_min_bytes = (int64_t)env_int("FKV_HOME_MIN_KB", 8192) * 1024;
+  // Ranges per workgroup.  Next to a transfer in the other direction one each is
+  // best (finer ranges shift the balance towards GPU->host and lower the sum: two
+  // threads with 25 MB requests 88.9 against 87.5 GB/s).  On an idle link the
+  // neighbours are the engine's compute kernels, which slow down single
+  // workgroups of a copy, and with one range each the slowest one holds up the
+  // launch: a restore next to fused-attention calls moves 37 GB/s with one range
+  // per workgroup and 54 GB/s with two.
+  static const int home_claims = std::max(1, env_int("FKV_HOME_CLAIMS_PER_WORKGROUP", 2));
+  if (p.busy_mask != 0xffu && link_direction_busy(p.device, !p.h2d, stream)) {
+    a->xcd_mask = p.busy_mask;
+    workgroups = p.confined_workgroups;
+    a->claims_per_wg = 1;
+  } else if (p.home_mask != 0xffu && home_min_bytes >= 0 && bytes >= home_min_bytes) {
+    a->xcd_mask = p.home_mask;
+    workgroups = p.home_workgroups;
+    a->claims_per_wg = home_claims;
+  }
+  return workgroups;
+}
+} // namespace
+
 int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
                        hipStream_t stream) {
   if (layer_offset < 0 || num_layers < 0 || layer_offset + num_layers > p.num_layers)
@@ -528,51 +590,45 @@ int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
     return fail(FKV_ERR_INVALID_ARG, "kv_dim %d too large", p.kv_dim);
   for (int l0 = layer_offset; l0 < layer_offset + num_layers; l0 += layers_per_launch) {
     const int nl = std::min(layers_per_launch, layer_offset + num_layers - l0);
-    const uint64_t *gb = p.gpu_base + (size_t)l0 * p.kv_dim;
-    const uint64_t *cb = p.cpu_base + (size_t)l0 * p.kv_dim;
-    CopyKernelArgs a{};
-    a.base_src = p.h2d ? cb : gb;
-    a.base_dst = p.h2d ? gb : cb;
-    a.ids_src = p.h2d ? p.cpu_ids : p.gpu_ids;
-    a.ids_dst = p.h2d ? p.gpu_ids : p.cpu_ids;
-    a.stride_src = p.h2d ? p.cpu_block_stride : p.gpu_block_stride;
-    a.stride_dst = p.h2d ? p.gpu_block_stride : p.cpu_block_stride;
-    a.chunk_bytes = p.chunk_size;
-    a.num_blocks = p.num_blocks;
-    a.lk = nl * p.kv_dim;
-    a.vec = p.vec;
-    a.nt_store = p.h2d ? 1 : 0;
-    // Packed short chunks cost a wavefront more address arithmetic per request, so
-    // such launches get half as many workgroups again.  Host->GPU, 2304-byte chunks:
-    // 16 x 64 lanes reach 45 GB/s, 24 x 64 reach 55.8, 32 x 64 reach 56.2; GPU->host:
-    // 48 x 64 lanes 50.7 GB/s, 72 x 64 52.5, 96 x 64 53.0.
-    a.packed_grid_pct = 150;
-    a.xcd_mask = p.xcd_mask;
-    int workgroups = p.workgroups;
-    static const int64_t home_min_bytes = (int64_t)env_int("FKV_HOME_MIN_KB", 8192) * 1024;
-    // Ranges per workgroup.  Next to a transfer in the other direction one each is
-    // best (finer ranges shift the balance towards GPU->host and lower the sum: two
-    // threads with 25 MB requests 88.9 against 87.5 GB/s).  On an idle link the
-    // neighbours are the engine's compute kernels, which slow down single
-    // workgroups of a copy, and with one range each the slowest one holds up the
-    // launch: a restore next to fused-attention calls moves 37 GB/s with one range
-    // per workgroup and 54 GB/s with two.
-    static const int home_claims = std::max(1, env_int("FKV_HOME_CLAIMS_PER_WORKGROUP", 2));
-    if (p.busy_mask != 0xffu && link_direction_busy(p.device, !p.h2d, stream)) {
-      a.xcd_mask = p.busy_mask;
-      workgroups = p.confined_workgroups;
-      a.claims_per_wg = 1;
-    } else if (p.home_mask != 0xffu && home_min_bytes >= 0 &&
-               (int64_t)p.num_blocks * a.lk * p.chunk_size >= home_min_bytes) {
-      a.xcd_mask = p.home_mask;
-      workgroups = p.home_workgroups;
-      a.claims_per_wg = home_claims;
-    }
-    a.claim = p.claims ? p.claims + 2 * l0 : nullptr; // a launch per first layer at most
+    CopyKernelArgs a = plan_job(p, l0, nl);
+    const int workgroups =
+        shape_for_now(p, (int64_t)p.num_blocks * a.lk * p.chunk_size, stream, &a);
     FKV_TRY(launch_copy_kernel(a, workgroups, p.threads, stream));
   }
   link_direction_mark(p.device, p.h2d, stream,
                       (int64_t)p.num_blocks * num_layers * p.kv_dim * p.chunk_size);
+  return FKV_OK;
+}
+
+int kernel_plans_launch(const KernelPlan *const *plans, const int *layer_offsets,
+                        const int *num_layers, int count, hipStream_t stream) {
+  // One launch for all of them when they can share one: same direction, device,
+  // vector width and launch shape, each range within one LDS table.
+  static const bool fuse = env_int("FKV_FUSE_LAUNCHES", 1) != 0;
+  bool together = fuse && count >= 2 && count <= kCopyMaxJobs;
+  for (int i = 0; i < count && together; ++i) {
+    const KernelPlan &p = *plans[i], &q = *plans[0];
+    together = p.h2d == q.h2d && p.device == q.device && p.vec == q.vec &&
+               p.threads == q.threads && p.workgroups == q.workgroups &&
+               p.xcd_mask == q.xcd_mask && p.busy_mask == q.busy_mask &&
+               p.home_mask == q.home_mask && layer_offsets[i] >= 0 && num_layers[i] > 0 &&
+               layer_offsets[i] + num_layers[i] <= p.num_layers &&
+               num_layers[i] * p.kv_dim <= kCopyMaxLK;
+  }
+  if (!together) {
+    for (int i = 0; i < count; ++i)
+      FKV_TRY(kernel_plan_launch(*plans[i], layer_offsets[i], num_layers[i], stream));
+    return FKV_OK;
+  }
+  CopyKernelArgs jobs[kCopyMaxJobs];
+  int64_t bytes = 0;
+  for (int i = 0; i < count; ++i) {
+    jobs[i] = plan_job(*plans[i], layer_offsets[i], num_layers[i]);
+    bytes += (int64_t)plans[i]->num_blocks * jobs[i].lk * plans[i]->chunk_size;
+  }
+  const int workgroups = shape_for_now(*plans[0], bytes, stream, &jobs[0]);
+  FKV_TRY(launch_copy_jobs(jobs, count, workgroups, plans[0]->threads, stream));
+  link_direction_mark(plans[0]->device, plans[0]->h2d, stream, bytes);
   return FKV_OK;
 }
 

@@ -154,6 +154,17 @@ constexpr int kCopyMaxLK = 1024;         // base-table entries staged in LDS
 constexpr int kCopyIdTile = 1024;        // block positions staged in LDS at a time
 int launch_copy_kernel(CopyKernelArgs args, int num_workgroups, int threads_per_workgroup,
                        hipStream_t stream);
+// Up to kCopyMaxJobs jobs of one direction and vector width in one launch: the work
+// of all of them is shared out among the workgroups by bytes.  Mask, counters and
+// ranges per workgroup are taken from jobs[0].
+constexpr int kCopyMaxJobs = 4;
+struct CopyJobs {
+  int32_t njobs;
+  uint32_t weight[kCopyMaxJobs]; // length of each job on the line the shares are cut from
+  CopyKernelArgs job[kCopyMaxJobs];
+};
+int launch_copy_jobs(const CopyKernelArgs *jobs, int njobs, int num_workgroups,
+                     int threads_per_workgroup, hipStream_t stream);
 // Copies `bytes` (rounded up to 16) from a pinned, device-mapped host buffer to
 // device memory with a small kernel on `stream`.
 int launch_plan_upload(void *device_dst, const void *pinned_src, size_t bytes, hipStream_t stream);
@@ -223,6 +234,11 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
 // Enqueues the copy of layers [layer_offset, layer_offset + num_layers) of the plan.
 int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
                        hipStream_t stream);
+// The same for layer ranges of several plans of one direction in one launch (the
+// members of one original layer of a multi-group restore); falls back to one launch
+// per plan where the plans cannot share one.
+int kernel_plans_launch(const KernelPlan *const *plans, const int *layer_offsets,
+                        const int *num_layers, int count, hipStream_t stream);
 // The plan memory is recycled once everything enqueued on `stream` so far has run.
 void kernel_plan_release(KernelPlan *p, hipStream_t stream);
 int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream);

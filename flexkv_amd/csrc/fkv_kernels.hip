@@ -110,10 +110,96 @@ __device__ __forceinline__ void copy_slice(const uint8_t *__restrict__ src,
   }
 }
 
+// How the workgroups of a launch come by their work.  Launches with claim counters
+// hand it out in `num_claims` ranges that the workgroups claim one after the other,
+// so that a workgroup which is slowed down (it shares its XCD with a transfer in the
+// other direction, or its CU with a compute kernel) takes fewer; the others give
+// workgroup i the i-th of gridDim.x shares.
+// A launch confined to some XCDs: workgroups elsewhere leave.  A workgroup of one
+// direction that runs on the other direction's XCDs next to that direction's
+// traffic moves its range at a third of the rate and holds up the whole launch, so
+// none may stay there.  Workgroup 0 is the safety net for a launch of which no
+// workgroup landed on a selected XCD: it looks at the claim counter after a while
+// and takes over only if nobody has claimed anything.
+struct Shares {
+  uint32_t *claim;
+  uint32_t num_claims, xcd_mask;
+  uint32_t next_claim; // lane 0: asked for before the current range is copied
+  bool confined, dynamic, first;
+
+  __device__ __forceinline__ Shares(const CopyKernelArgs &a)
+      : claim(a.claim), num_claims(a.num_claims), xcd_mask(a.xcd_mask & 0xffu), next_claim(0),
+        confined((a.xcd_mask & 0xffu) != 0xffu), dynamic(a.num_claims != 0), first(true) {}
+
+  // Every workgroup of a launch with counters counts itself out; the last one leaves
+  // the two counters zeroed for the next launch that is given them.
+  __device__ __forceinline__ void leave() const {
+    if (threadIdx.x == 0 &&
+        __hip_atomic_fetch_add(claim + 1, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) ==
+            gridDim.x - 1) {
+      __hip_atomic_store(claim, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(claim + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+
+  // False: this workgroup takes no part (and has counted itself out).
+  __device__ __forceinline__ bool enter(uint32_t *s_claim) {
+    if (confined && !((xcd_mask >> xcd_of_this_wave()) & 1u)) {
+      if (blockIdx.x != 0) {
+        leave();
+        return false;
+      }
+      if (threadIdx.x == 0) {
+        const long long t0 = wall_clock64();
+        while (wall_clock64() - t0 < 5000) // 50 us of the constant 100 MHz clock
+          __builtin_amdgcn_s_sleep(32);
+        *s_claim = __hip_atomic_load(claim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __syncthreads();
+      if (*s_claim != 0) { // the selected XCDs are at work
+        leave();
+        return false;
+      }
+      __syncthreads();
+    }
+    // lane 0 keeps the next claim in a register: it is asked for before the current
+    // range is copied and has long arrived when the range is done
+    if (dynamic && threadIdx.x == 0)
+      next_claim = atomicAdd(claim, 1u);
+    return true;
+  }
+
+  // The next share [part/parts, (part+1)/parts) of this workgroup; false: none left
+  // (the whole workgroup leaves together, counted out).
+  __device__ __forceinline__ bool next(uint32_t *s_claim, uint32_t *part, uint32_t *parts) {
+    if (!dynamic) {
+      *part = blockIdx.x;
+      *parts = gridDim.x;
+      const bool mine = first;
+      first = false;
+      return mine;
+    }
+    if (threadIdx.x == 0)
+      *s_claim = next_claim;
+    __syncthreads();
+    *part = *s_claim;
+    *parts = num_claims;
+    __syncthreads(); // everyone has read the claim before it is overwritten
+    if (*part >= *parts) {
+      leave();
+      return false;
+    }
+    if (threadIdx.x == 0)
+      next_claim = atomicAdd(claim, 1u);
+    return true;
+  }
+};
+
+// Copies the work units of `a` that fall into [num0/den, num1/den) of the job.
+// `load_tables`: the base tables of `a` are not in LDS yet.
 template <int VEC, bool NTS>
-__global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
-    CopyKernelArgs a) {
-  extern __shared__ uint64_t lds[];
+__device__ __forceinline__ void copy_share(const CopyKernelArgs &a, uint64_t num0, uint64_t num1,
+                                           uint64_t den, uint64_t *lds, bool load_tables) {
   uint64_t *s_base_src = lds;
   uint64_t *s_base_dst = lds + a.lk;
   int64_t *s_off_src = reinterpret_cast<int64_t *>(lds + 2 * a.lk);
@@ -130,173 +216,151 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
   const uint64_t total_units = (uint64_t)a.num_blocks * spp;
   const uint64_t total = a.packed ? (total_units + kPiece - 1) / kPiece : total_units;
   const int tid = threadIdx.x;
-  // Launches with claim counters hand their work out in `num_claims` ranges that
-  // the workgroups claim one after the other, so that a workgroup which is slowed
-  // down (it shares its XCD with a transfer in the other direction) takes fewer.
-  // A launch confined to some XCDs: workgroups elsewhere leave.  A workgroup of one
-  // direction that runs on the other direction's XCDs next to that direction's
-  // traffic moves its range at a third of the rate and holds up the whole launch, so
-  // none may stay there.  Workgroup 0 is the safety net for a launch of which no
-  // workgroup landed on a selected XCD: it looks at the claim counter after a while
-  // and takes over only if nobody has claimed anything.
-  const bool confined = (a.xcd_mask & 0xffu) != 0xffu;
-  const bool dynamic = a.num_claims != 0; // set for every confined launch
-  __shared__ uint32_t s_claim;
-  // Every workgroup of such a launch counts itself out; the last one leaves the
-  // two counters zeroed for the next launch that is given them.
-  auto leave = [&]() {
-    if (tid == 0 &&
-        __hip_atomic_fetch_add(a.claim + 1, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) ==
-            gridDim.x - 1) {
-      __hip_atomic_store(a.claim, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(a.claim + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  };
-  if (confined && !((a.xcd_mask >> xcd_of_this_wave()) & 1u)) {
-    if (blockIdx.x != 0) {
-      leave();
-      return;
-    }
-    if (tid == 0) {
-      const long long t0 = wall_clock64();
-      while (wall_clock64() - t0 < 5000) // 50 us of the constant 100 MHz clock
-        __builtin_amdgcn_s_sleep(32);
-      s_claim = __hip_atomic_load(a.claim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (s_claim != 0) { // the selected XCDs are at work
-      leave();
-      return;
-    }
-    __syncthreads();
-  }
-  // lane 0 keeps the next claim in a register: it is asked for before the current
-  // range is copied and has long arrived when the range is done
-  uint32_t next_claim = 0;
-  if (dynamic && tid == 0)
-    next_claim = atomicAdd(a.claim, 1u);
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
   const int nwaves = blockDim.x / kWave;
 
-  for (int i = tid; i < a.lk; i += blockDim.x) {
-    s_base_src[i] = a.base_src[i];
-    s_base_dst[i] = a.base_dst[i];
+  if (load_tables) {
+    __syncthreads(); // nobody still reads the tables of the job before
+    for (int i = tid; i < a.lk; i += blockDim.x) {
+      s_base_src[i] = a.base_src[i];
+      s_base_dst[i] = a.base_dst[i];
+    }
+  }
+  uint64_t s0 = total * num0 / den;
+  uint64_t s1 = total * num1 / den;
+  if (s0 >= s1)
+    return;
+  if (a.packed) { // from pieces to vectors
+    s0 *= kPiece;
+    s1 = s1 * kPiece < total_units ? s1 * kPiece : total_units;
   }
 
-  for (;;) {
-    // This workgroup's range of work units: its own share of the launch, or the next
-    // unclaimed one.
-    uint32_t part = blockIdx.x, parts = gridDim.x;
-    if (dynamic) {
-      if (tid == 0)
-        s_claim = next_claim;
-      __syncthreads();
-      part = s_claim;
-      parts = a.num_claims;
-      __syncthreads(); // everyone has read the claim before it is overwritten
-      if (part >= parts) { // whole workgroup leaves together
-        leave();
-        return;
-      }
-      if (tid == 0)
-        next_claim = atomicAdd(a.claim, 1u);
+  const uint32_t pos_lo = (uint32_t)(s0 / spp);
+  const uint32_t pos_hi = (uint32_t)((s1 - 1) / spp);
+  for (uint32_t tile = pos_lo; tile <= pos_hi; tile += kCopyIdTile) {
+    const uint32_t n = min((uint32_t)kCopyIdTile, pos_hi - tile + 1);
+    __syncthreads(); // previous tile fully consumed; base tables visible
+    for (uint32_t i = tid; i < n; i += blockDim.x) {
+      const int64_t p = (int64_t)tile + i;
+      s_off_src[i] = (a.ids_src ? a.ids_src[p] : p) * a.stride_src;
+      s_off_dst[i] = (a.ids_dst ? a.ids_dst[p] : p) * a.stride_dst;
     }
-    uint64_t s0 = total * part / parts;
-    uint64_t s1 = total * (part + 1) / parts;
-    if (s0 >= s1) {
-      if (dynamic)
-        continue;
-      return;
-    }
-    if (a.packed) { // from pieces to vectors
-      s0 *= kPiece;
-      s1 = s1 * kPiece < total_units ? s1 * kPiece : total_units;
-    }
-
-    const uint32_t pos_lo = (uint32_t)(s0 / spp);
-    const uint32_t pos_hi = (uint32_t)((s1 - 1) / spp);
-    for (uint32_t tile = pos_lo; tile <= pos_hi; tile += kCopyIdTile) {
-      const uint32_t n = min((uint32_t)kCopyIdTile, pos_hi - tile + 1);
-      __syncthreads(); // previous tile fully consumed; base tables visible
-      for (uint32_t i = tid; i < n; i += blockDim.x) {
-        const int64_t p = (int64_t)tile + i;
-        s_off_src[i] = (a.ids_src ? a.ids_src[p] : p) * a.stride_src;
-        s_off_dst[i] = (a.ids_dst ? a.ids_dst[p] : p) * a.stride_dst;
-      }
-      __syncthreads();
-      const uint64_t tile_s0 = (uint64_t)tile * spp;
-      const uint64_t t0 = s0 > tile_s0 ? s0 : tile_s0;
-      const uint64_t tile_s1 = tile_s0 + (uint64_t)n * spp;
-      const uint64_t t1 = s1 < tile_s1 ? s1 : tile_s1;
-      if (a.packed) {
-        using V = typename VecType<VEC>::type;
-        const uint32_t lim = (uint32_t)(t1 - tile_s0); // < kCopyIdTile * spp, checked on host
-        const uint32_t ulk = (uint32_t)a.lk;
-        const uint32_t q64 = kWave / vpc, r64 = kWave % vpc; // kWave vectors = q64 chunks + r64
-        const uint32_t qlk = q64 / ulk, rlk = q64 % ulk;     // q64 chunks = qlk positions + rlk
-        for (uint32_t v0 = (uint32_t)(t0 - tile_s0) + wave * kPiece; v0 < lim;
-             v0 += nwaves * kPiece) {
-          V r[kCopyUnroll];
-          V *d[kCopyUnroll];
-          // A lane's vectors are kWave apart.  The first one is located by division;
-          // each further one by adding the precomputed quotients and remainders of
-          // kWave, which costs a few compares instead of two divisions.  Lanes beyond
-          // the end stay on their last valid vector and re-read it rather than branch
-          // around the load: all loads of a piece are issued back to back, only the
-          // stores are predicated.
-          uint32_t v = v0 + lane;
-          const uint32_t vc = min(v, lim - 1);
-          const uint32_t c = vc / vpc; // chunk inside the tile: position * lk + i
-          uint32_t w = vc - c * vpc;
-          uint32_t p = c / ulk;
-          uint32_t i = c - p * ulk;
-  #pragma unroll
-          for (int u = 0; u < kCopyUnroll; ++u) {
-            if (u > 0) {
-              v += kWave;
-              uint32_t w2 = w + r64, i2 = i + rlk, p2 = p + qlk;
-              if (w2 >= vpc) {
-                w2 -= vpc;
-                i2 += 1;
-              }
-              if (i2 >= ulk) {
-                i2 -= ulk;
-                p2 += 1;
-              }
-              const bool ok = v < lim;
-              w = ok ? w2 : w;
-              i = ok ? i2 : i;
-              p = ok ? p2 : p;
+    __syncthreads();
+    const uint64_t tile_s0 = (uint64_t)tile * spp;
+    const uint64_t t0 = s0 > tile_s0 ? s0 : tile_s0;
+    const uint64_t tile_s1 = tile_s0 + (uint64_t)n * spp;
+    const uint64_t t1 = s1 < tile_s1 ? s1 : tile_s1;
+    if (a.packed) {
+      using V = typename VecType<VEC>::type;
+      const uint32_t lim = (uint32_t)(t1 - tile_s0); // < kCopyIdTile * spp, checked on host
+      const uint32_t ulk = (uint32_t)a.lk;
+      const uint32_t q64 = kWave / vpc, r64 = kWave % vpc; // kWave vectors = q64 chunks + r64
+      const uint32_t qlk = q64 / ulk, rlk = q64 % ulk;     // q64 chunks = qlk positions + rlk
+      for (uint32_t v0 = (uint32_t)(t0 - tile_s0) + wave * kPiece; v0 < lim;
+           v0 += nwaves * kPiece) {
+        V r[kCopyUnroll];
+        V *d[kCopyUnroll];
+        // A lane's vectors are kWave apart.  The first one is located by division;
+        // each further one by adding the precomputed quotients and remainders of
+        // kWave, which costs a few compares instead of two divisions.  Lanes beyond
+        // the end stay on their last valid vector and re-read it rather than branch
+        // around the load: all loads of a piece are issued back to back, only the
+        // stores are predicated.
+        uint32_t v = v0 + lane;
+        const uint32_t vc = min(v, lim - 1);
+        const uint32_t c = vc / vpc; // chunk inside the tile: position * lk + i
+        uint32_t w = vc - c * vpc;
+        uint32_t p = c / ulk;
+        uint32_t i = c - p * ulk;
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u) {
+          if (u > 0) {
+            v += kWave;
+            uint32_t w2 = w + r64, i2 = i + rlk, p2 = p + qlk;
+            if (w2 >= vpc) {
+              w2 -= vpc;
+              i2 += 1;
             }
-            const V *src = reinterpret_cast<const V *>(s_base_src[i] + (uint64_t)s_off_src[p]) + w;
-            d[u] = reinterpret_cast<V *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + w;
-            r[u] = __builtin_nontemporal_load(src);
+            if (i2 >= ulk) {
+              i2 -= ulk;
+              p2 += 1;
+            }
+            const bool ok = v < lim;
+            w = ok ? w2 : w;
+            i = ok ? i2 : i;
+            p = ok ? p2 : p;
           }
-  #pragma unroll
-          for (int u = 0; u < kCopyUnroll; ++u)
-            if (v0 + u * kWave + lane < lim)
-              put<V, NTS>(r[u], d[u]);
+          const V *src = reinterpret_cast<const V *>(s_base_src[i] + (uint64_t)s_off_src[p]) + w;
+          d[u] = reinterpret_cast<V *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + w;
+          r[u] = __builtin_nontemporal_load(src);
         }
-        continue;
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u)
+          if (v0 + u * kWave + lane < lim)
+            put<V, NTS>(r[u], d[u]);
       }
-      for (uint64_t s = t0 + wave; s < t1; s += nwaves) {
-        const uint32_t rel = (uint32_t)(s - tile_s0); // < kCopyIdTile * spp, checked on host
-        const uint32_t p = rel / spp;
-        const uint32_t r = rel - p * spp;
-        const uint32_t i = r / slices;
-        const uint32_t sl = r - i * slices;
-        const int64_t off = (int64_t)sl * kSliceBytes;
-        const int64_t left = a.chunk_bytes - off;
-        const uint8_t *src =
-            reinterpret_cast<const uint8_t *>(s_base_src[i] + (uint64_t)s_off_src[p]) + off;
-        uint8_t *dst = reinterpret_cast<uint8_t *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + off;
-        copy_slice<VEC, NTS>(src, dst, left < kSliceBytes ? left : kSliceBytes, lane);
-      }
+      continue;
     }
-    if (!dynamic)
-      return;
-  } // next claim
+    for (uint64_t s = t0 + wave; s < t1; s += nwaves) {
+      const uint32_t rel = (uint32_t)(s - tile_s0); // < kCopyIdTile * spp, checked on host
+      const uint32_t p = rel / spp;
+      const uint32_t r = rel - p * spp;
+      const uint32_t i = r / slices;
+      const uint32_t sl = r - i * slices;
+      const int64_t off = (int64_t)sl * kSliceBytes;
+      const int64_t left = a.chunk_bytes - off;
+      const uint8_t *src =
+          reinterpret_cast<const uint8_t *>(s_base_src[i] + (uint64_t)s_off_src[p]) + off;
+      uint8_t *dst = reinterpret_cast<uint8_t *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + off;
+      copy_slice<VEC, NTS>(src, dst, left < kSliceBytes ? left : kSliceBytes, lane);
+    }
+  }
+}
+
+template <int VEC, bool NTS>
+__global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
+    CopyKernelArgs a) {
+  extern __shared__ uint64_t lds[];
+  __shared__ uint32_t s_claim;
+  Shares shares(a);
+  if (!shares.enter(&s_claim))
+    return;
+  bool load_tables = true;
+  uint32_t part, parts;
+  while (shares.next(&s_claim, &part, &parts)) {
+    copy_share<VEC, NTS>(a, part, part + 1, parts, lds, load_tables);
+    load_tables = false;
+  }
+}
+
+// Several jobs in one launch (the members of one original layer of a multi-group
+// restore, which differ in chunk size and strides): the jobs lie one behind the
+// other on a line, each as long as its weight (its bytes), and a share of the launch
+// is a stretch of that line.  Counters, mask and grid are those of job 0.
+template <int VEC, bool NTS>
+__global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_jobs_kernel(CopyJobs t) {
+  extern __shared__ uint64_t lds[];
+  __shared__ uint32_t s_claim;
+  Shares shares(t.job[0]);
+  if (!shares.enter(&s_claim))
+    return;
+  uint64_t line = 0;
+  for (int j = 0; j < t.njobs; ++j)
+    line += t.weight[j];
+  uint32_t part, parts;
+  while (shares.next(&s_claim, &part, &parts)) {
+    const uint64_t b0 = line * part / parts, b1 = line * (part + 1) / parts;
+    uint64_t off = 0;
+    for (int j = 0; j < t.njobs; ++j) {
+      const uint64_t w = t.weight[j];
+      const uint64_t lo = b0 > off ? (b0 - off < w ? b0 - off : w) : 0;
+      const uint64_t hi = b1 > off ? (b1 - off < w ? b1 - off : w) : 0;
+      if (lo < hi)
+        copy_share<VEC, NTS>(t.job[j], lo, hi, w, lds, true);
+      off += w;
+    }
+  }
 }
 
 template <int VEC>
@@ -361,8 +425,11 @@ int common_vector_width(const uint64_t *vals, int n) {
   return 1;
 }
 
-int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_workgroup,
-                       hipStream_t stream) {
+namespace {
+// Checks one job and fills in what the kernel derives from its shape; `total` = its
+// work units (slices, or pieces in packed mode).  FKV_OK with *total == 0: nothing to do.
+int prepare_job(CopyKernelArgs &a, int64_t *total) {
+  *total = 0;
   if (a.num_blocks <= 0 || a.lk <= 0 || a.chunk_bytes <= 0)
     return FKV_OK;
   if (a.lk > kCopyMaxLK)
@@ -382,7 +449,7 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_wor
                 "copy kernel: chunk of %lld B x %d (layer,kv) pairs is too large for one launch",
                 (long long)a.chunk_bytes, a.lk);
   a.slices_per_chunk = (int32_t)slices;
-  int64_t total = spp * a.num_blocks;
+  *total = spp * a.num_blocks;
   // Chunks shorter than one slice would leave most lanes of a wavefront idle and
   // most of its requests unissued: pack them (the kernel indexes vectors inside an
   // id tile with 32 bits).
@@ -396,8 +463,16 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_wor
     a.packed = 0;
   if (a.packed) {
     const int64_t piece = (int64_t)kWave * kCopyUnroll;
-    total = (vpp * a.num_blocks + piece - 1) / piece;
+    *total = (vpp * a.num_blocks + piece - 1) / piece;
   }
+  return FKV_OK;
+}
+
+// Grid, workgroup size, mask and claims of a launch with `total` work units and
+// `bytes` to move; `a` is the (first) job, whose mask, counters and choices count.
+void shape_launch(CopyKernelArgs &a, int64_t total, int64_t bytes, bool any_packed,
+                  int num_workgroups, int threads_per_workgroup, int64_t *grid_out,
+                  int *threads_out) {
   int threads = threads_per_workgroup;
   if (threads < kWave)
     threads = kWave;
@@ -406,7 +481,7 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_wor
   threads = threads / kWave * kWave;
   const int waves_per_wg = threads / kWave;
   int64_t grid = num_workgroups > 0 ? num_workgroups : 1;
-  if (a.packed && a.packed_grid_pct > 0)
+  if (any_packed && a.packed_grid_pct > 0)
     grid = (grid * a.packed_grid_pct + 99) / 100;
   const int64_t useful = (total + waves_per_wg - 1) / waves_per_wg;
   if (grid > useful)
@@ -436,22 +511,97 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_wor
       return n < 0 ? 0 : n;
     }();
     // ranges of 128 KiB at least: a claim costs a round trip to device memory
-    const int64_t bytes = (int64_t)a.num_blocks * a.lk * a.chunk_bytes;
     a.num_claims = (uint32_t)std::min<int64_t>(std::min<int64_t>(grid * per_wg, total),
                                                 bytes / (128 * 1024));
     if (a.num_claims <= (uint32_t)grid) // nothing to hand out: fixed shares
       a.num_claims = 0;
   }
-  const size_t lds_bytes = (size_t)(2 * a.lk + 2 * kCopyIdTile) * sizeof(uint64_t);
   stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);
   if (a.xcd_mask != 0xffu)
     stats().confined_launches.fetch_add(1, std::memory_order_relaxed);
+  *grid_out = grid;
+  *threads_out = threads;
+}
+
+template <int VEC>
+int launch_jobs_vec(const CopyJobs &t, int grid, int threads, size_t lds_bytes,
+                    hipStream_t stream) {
+  if (t.job[0].nt_store)
+    hipLaunchKernelGGL((fkv_copy_jobs_kernel<VEC, true>), dim3(grid), dim3(threads), lds_bytes,
+                       stream, t);
+  else
+    hipLaunchKernelGGL((fkv_copy_jobs_kernel<VEC, false>), dim3(grid), dim3(threads), lds_bytes,
+                       stream, t);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return fail(FKV_ERR_RUNTIME, "copy kernel launch failed: %s", hipGetErrorString(e));
+  return FKV_OK;
+}
+} // namespace
+
+int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_workgroup,
+                       hipStream_t stream) {
+  int64_t total = 0;
+  FKV_TRY(prepare_job(a, &total));
+  if (total == 0)
+    return FKV_OK;
+  int64_t grid = 1;
+  int threads = kWave;
+  shape_launch(a, total, (int64_t)a.num_blocks * a.lk * a.chunk_bytes, a.packed != 0,
+               num_workgroups, threads_per_workgroup, &grid, &threads);
+  const size_t lds_bytes = (size_t)(2 * a.lk + 2 * kCopyIdTile) * sizeof(uint64_t);
   switch (a.vec) {
   case 16: return launch_vec<16>(a, (int)grid, threads, lds_bytes, stream);
   case 8:  return launch_vec<8>(a, (int)grid, threads, lds_bytes, stream);
   case 4:  return launch_vec<4>(a, (int)grid, threads, lds_bytes, stream);
   case 2:  return launch_vec<2>(a, (int)grid, threads, lds_bytes, stream);
   default: return launch_vec<1>(a, (int)grid, threads, lds_bytes, stream);
+  }
+}
+
+int launch_copy_jobs(const CopyKernelArgs *jobs, int njobs, int num_workgroups,
+                     int threads_per_workgroup, hipStream_t stream) {
+  if (njobs < 1 || njobs > kCopyMaxJobs)
+    return fail(FKV_ERR_RUNTIME, "copy kernel: %d jobs in one launch (1..%d)", njobs, kCopyMaxJobs);
+  CopyJobs t{};
+  int64_t total = 0, bytes = 0;
+  int max_lk = 0;
+  bool any_packed = false;
+  for (int j = 0; j < njobs; ++j) {
+    CopyKernelArgs a = jobs[j];
+    if (a.vec != jobs[0].vec || a.nt_store != jobs[0].nt_store)
+      return fail(FKV_ERR_RUNTIME, "copy kernel: jobs of one launch differ in vector width or store kind");
+    int64_t job_total = 0;
+    FKV_TRY(prepare_job(a, &job_total));
+    if (job_total == 0)
+      continue;
+    const int64_t job_bytes = (int64_t)a.num_blocks * a.lk * a.chunk_bytes;
+    // the line is measured in 4 KiB, so that units x weight stays far from 64 bits
+    t.weight[t.njobs] = (uint32_t)std::max<int64_t>(1, std::min<int64_t>(job_bytes >> 12, UINT32_MAX));
+    t.job[t.njobs++] = a;
+    total += job_total;
+    bytes += job_bytes;
+    max_lk = std::max(max_lk, (int)a.lk);
+    any_packed = any_packed || a.packed;
+  }
+  if (t.njobs == 0)
+    return FKV_OK;
+  // mask, counters and ranges per workgroup are those of the first job given
+  t.job[0].xcd_mask = jobs[0].xcd_mask;
+  t.job[0].claim = jobs[0].claim;
+  t.job[0].claims_per_wg = jobs[0].claims_per_wg;
+  t.job[0].packed_grid_pct = jobs[0].packed_grid_pct;
+  int64_t grid = 1;
+  int threads = kWave;
+  shape_launch(t.job[0], total, bytes, any_packed, num_workgroups, threads_per_workgroup, &grid,
+               &threads);
+  const size_t lds_bytes = (size_t)(2 * max_lk + 2 * kCopyIdTile) * sizeof(uint64_t);
+  switch (t.job[0].vec) {
+  case 16: return launch_jobs_vec<16>(t, (int)grid, threads, lds_bytes, stream);
+  case 8:  return launch_jobs_vec<8>(t, (int)grid, threads, lds_bytes, stream);
+  case 4:  return launch_jobs_vec<4>(t, (int)grid, threads, lds_bytes, stream);
+  case 2:  return launch_jobs_vec<2>(t, (int)grid, threads, lds_bytes, stream);
+  default: return launch_jobs_vec<1>(t, (int)grid, threads, lds_bytes, stream);
   }
 }
 

@@ -637,23 +637,36 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
     fkv_layerwise::Batch &batch = *g->batches[b];
     for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
       (void)hipSetDevice(g->device_ids[i]);
-      for (const Item &it : batch.items) {
-        const Lane &lane = lanes[it.lane];
-        if (direct) {
-          rc = kernel_plan_launch(lane.plans[i], it.start_layer, it.layers, g->streams[i]);
-          if (rc == FKV_OK) {
+      if (direct) {
+        // the members of one batch go out together: up to kCopyMaxJobs per launch
+        const KernelPlan *plans[kCopyMaxJobs];
+        int first[kCopyMaxJobs], count[kCopyMaxJobs];
+        for (size_t k = 0; k < batch.items.size() && rc == FKV_OK; k += kCopyMaxJobs) {
+          const int n = (int)std::min<size_t>(kCopyMaxJobs, batch.items.size() - k);
+          for (int j = 0; j < n; ++j) {
+            const Item &it = batch.items[k + j];
+            plans[j] = &lanes[it.lane].plans[i];
+            first[j] = it.start_layer;
+            count[j] = it.layers;
+          }
+          rc = kernel_plans_launch(plans, first, count, n, g->streams[i]);
+          if (rc != FKV_OK)
+            break;
+          for (int j = 0; j < n; ++j) {
+            const Item &it = batch.items[k + j];
+            const Lane &lane = lanes[it.lane];
             stats().calls.fetch_add(1, std::memory_order_relaxed);
             stats().bytes_h2d.fetch_add((uint64_t)lane.num_blocks * it.layers * lane.kv_dim *
                                             (uint64_t)lane.src->chunk_sizes[i],
                                         std::memory_order_relaxed);
           }
-        } else {
-          fkv_transfer_desc d = describe(g, lane, i, it.start_layer, it.layers, c);
-          rc = fkv_transfer_kv_blocks(&d, g->streams[i]);
-          (void)hipSetDevice(g->device_ids[i]);
         }
-        if (rc != FKV_OK)
-          break;
+      }
+      for (size_t k = 0; !direct && k < batch.items.size() && rc == FKV_OK; ++k) {
+        const Item &it = batch.items[k];
+        fkv_transfer_desc d = describe(g, lanes[it.lane], i, it.start_layer, it.layers, c);
+        rc = fkv_transfer_kv_blocks(&d, g->streams[i]);
+        (void)hipSetDevice(g->device_ids[i]);
       }
       if (rc != FKV_OK)
         break;
