@@ -196,6 +196,23 @@ PlanSlot *plan_acquire(int device, size_t bytes) {
   return pick;
 }
 
+int plan_counters_dirty(int *dirty) {
+  *dirty = 0;
+  std::vector<uint32_t> host((size_t)kPlanCounterPairs * 2);
+  PlanPool &p = pool();
+  std::lock_guard<std::mutex> lk(p.mu);
+  for (PlanSlot *s : p.slots) {
+    if (!s->counters)
+      continue;
+    DeviceGuard guard(s->device);
+    FKV_HIP_TRY(hipMemcpy(host.data(), s->counters, host.size() * sizeof(uint32_t),
+                          hipMemcpyDeviceToHost));
+    for (uint32_t v : host)
+      *dirty += v != 0;
+  }
+  return FKV_OK;
+}
+
 uint8_t *plan_host(PlanSlot *s) { return s->host; }
 uint32_t *plan_counters(PlanSlot *s, int pairs) {
   return pairs <= kPlanCounterPairs ? s->counters : nullptr;
@@ -889,6 +906,17 @@ int order_after(hipStream_t from, hipStream_t to, int device, int which) {
   return FKV_OK;
 }
 } // namespace
+
+int fkv_plan_counters_dirty(int32_t *dirty) {
+  using namespace fkv;
+  clear_error();
+  if (!dirty)
+    return fail(FKV_ERR_INVALID_ARG, "fkv_plan_counters_dirty: null result pointer");
+  int n = 0;
+  FKV_TRY(plan_counters_dirty(&n));
+  *dirty = n;
+  return FKV_OK;
+}
 
 int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream_v) {
   using namespace fkv;

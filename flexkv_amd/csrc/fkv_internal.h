@@ -189,6 +189,9 @@ uint8_t *plan_host(PlanSlot *s);
 // `pairs` pairs of zeroed counters in device memory that belong to the slot
 // (CopyKernelArgs::claim), or nullptr when a slot holds fewer.
 uint32_t *plan_counters(PlanSlot *s, int pairs);
+// Number of counters of all slots that are not zero (they all are whenever no
+// launch is under way); copies them from the device.
+int plan_counters_dirty(int *dirty);
 // Publishes the first `bytes` of the slot to the device on `stream` and returns
 // the address kernels must use (the device mirror, or the pinned buffer itself
 // when `mirror` is false).
