@@ -197,14 +197,6 @@ def streams_run_concurrently(stream_a, stream_b, device: int = -1) -> bool:
     return bool(out.value)
 
 
-def plan_counters_dirty() -> int:
-    """Self-check of the library's launch bookkeeping: how many of its work-claim
-    counters are not zero.  0 whenever no transfer is under way."""
-    out = ctypes.c_int32(-1)
-    check(_L.fkv_plan_counters_dirty(ctypes.byref(out)))
-    return int(out.value)
-
-
 def link_activity_post(is_host_to_device: bool, expected_us: int, device: int = -1) -> None:
     """Tell the other processes that use this GPU that this one keeps the host link
     busy in one direction for about `expected_us` more.  The library posts its own

@@ -64,14 +64,21 @@ DeviceGuard::~DeviceGuard() {
 }
 
 // ---- plan memory ---------------------------------------------------------
+namespace {
+bool env_flag(const char *name) {
+  const char *v = std::getenv(name);
+  return v && *v && std::strcmp(v, "0") != 0;
+}
+} // namespace
+
 struct PlanSlot {
   uint8_t *host = nullptr;
   uint8_t *dev = nullptr;
   size_t cap = 0;
   hipEvent_t done = nullptr;
-  // kPlanCounterPairs pairs of zeroed counters in device memory for confined
-  // launches (CopyKernelArgs::claim); each launch leaves its pair zeroed.
-  uint32_t *counters = nullptr;
+  // kPlanCounters claim counters in device memory for launches whose workgroups
+  // claim their work (CopyKernelArgs::claim)
+  uint64_t *counters = nullptr;
   bool busy = false;          // handed out, not yet released
   bool event_pending = false; // released behind an event that may not have fired
   int device = 0;
@@ -89,7 +96,7 @@ PlanPool &pool() {
   return *p;
 }
 constexpr size_t kPlanMinBytes = 64 * 1024;
-constexpr int kPlanCounterPairs = 1024;
+constexpr int kPlanCounters = 1024;
 
 bool slot_grow(PlanSlot *s, size_t bytes) {
   if (s->cap >= bytes)
@@ -157,18 +164,17 @@ PlanSlot *plan_acquire(int device, size_t bytes) {
         fail(FKV_ERR_RUNTIME, "plan memory: hipEventCreate failed");
         return nullptr;
       }
+      // Zeroed for tidiness only, by a copy that has finished when it returns (a
+      // hipMemset on the null stream can still be under way when the first kernel on
+      // a non-blocking stream claims from the counters): a launch takes a counter
+      // over whatever it holds, see Shares::adopt.
       void *c = nullptr;
-      const size_t cbytes = (size_t)kPlanCounterPairs * 2 * sizeof(uint32_t);
-      // Zeroed by a copy that has finished when it returns.  hipMemset runs on the
-      // null stream and need not be over when the first kernel on a non-blocking
-      // stream uses the counters: cleared under a running launch, its workgroups never
-      // count to the end, the counters stay dirty, and the next launch that is given
-      // them finds no work to claim and is left to the lone safety-net workgroup
-      // (8 GiB at 7.7 GB/s, once in a few dozen processes).
-      static const std::vector<uint32_t> zeros((size_t)kPlanCounterPairs * 2, 0u);
+      const size_t cbytes = (size_t)kPlanCounters * sizeof(uint64_t);
+      // FKV_TEST_DIRTY_COUNTERS=1 (tests): start them with garbage instead
+      static const std::vector<uint64_t> zeros(
+          (size_t)kPlanCounters, env_flag("FKV_TEST_DIRTY_COUNTERS") ? 0xdeadbeef00000007ull : 0u);
       if (hipMalloc(&c, cbytes) != hipSuccess ||
-          hipMemcpy(c, zeros.data(), cbytes, hipMemcpyHostToDevice) != hipSuccess ||
-          hipStreamSynchronize(nullptr) != hipSuccess) {
+          hipMemcpy(c, zeros.data(), cbytes, hipMemcpyHostToDevice) != hipSuccess) {
         (void)hipGetLastError();
         if (c)
           (void)hipFree(c);
@@ -177,7 +183,7 @@ PlanSlot *plan_acquire(int device, size_t bytes) {
         fail(FKV_ERR_RUNTIME, "plan memory: cannot allocate the claim counters");
         return nullptr;
       }
-      pick->counters = static_cast<uint32_t *>(c);
+      pick->counters = static_cast<uint64_t *>(c);
       p.slots.push_back(pick);
     }
     pick->busy = true;
@@ -196,26 +202,9 @@ PlanSlot *plan_acquire(int device, size_t bytes) {
   return pick;
 }
 
-int plan_counters_dirty(int *dirty) {
-  *dirty = 0;
-  std::vector<uint32_t> host((size_t)kPlanCounterPairs * 2);
-  PlanPool &p = pool();
-  std::lock_guard<std::mutex> lk(p.mu);
-  for (PlanSlot *s : p.slots) {
-    if (!s->counters)
-      continue;
-    DeviceGuard guard(s->device);
-    FKV_HIP_TRY(hipMemcpy(host.data(), s->counters, host.size() * sizeof(uint32_t),
-                          hipMemcpyDeviceToHost));
-    for (uint32_t v : host)
-      *dirty += v != 0;
-  }
-  return FKV_OK;
-}
-
 uint8_t *plan_host(PlanSlot *s) { return s->host; }
-uint32_t *plan_counters(PlanSlot *s, int pairs) {
-  return pairs <= kPlanCounterPairs ? s->counters : nullptr;
+uint64_t *plan_counters(PlanSlot *s, int count) {
+  return count <= kPlanCounters ? s->counters : nullptr;
 }
 
 int plan_publish(PlanSlot *s, size_t bytes, bool mirror, hipStream_t stream,
@@ -566,7 +555,7 @@ CopyKernelArgs plan_job(const KernelPlan &p, int l0, int nl) {
   // 48 x 64 lanes 50.7 GB/s, 72 x 64 52.5, 96 x 64 53.0.
   a.packed_grid_pct = 150;
   a.xcd_mask = p.xcd_mask;
-  a.claim = p.claims ? p.claims + 2 * l0 : nullptr; // a launch per first layer at most
+  a.claim = p.claims ? p.claims + l0 : nullptr; // a launch per first layer at most
   return a;
 }
 
@@ -906,17 +895,6 @@ int order_after(hipStream_t from, hipStream_t to, int device, int which) {
   return FKV_OK;
 }
 } // namespace
-
-int fkv_plan_counters_dirty(int32_t *dirty) {
-  using namespace fkv;
-  clear_error();
-  if (!dirty)
-    return fail(FKV_ERR_INVALID_ARG, "fkv_plan_counters_dirty: null result pointer");
-  int n = 0;
-  FKV_TRY(plan_counters_dirty(&n));
-  *dirty = n;
-  return FKV_OK;
-}
 
 int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream_v) {
   using namespace fkv;

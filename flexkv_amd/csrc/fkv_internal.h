@@ -140,12 +140,14 @@ struct CopyKernelArgs {
   int32_t packed;   // set by launch_copy_kernel: chunks shorter than a slice, see the kernel
   int32_t packed_grid_pct; // workgroups to launch in packed mode, percent of the request (0 = 100)
   uint32_t xcd_mask; // bit k: workgroups that run on XCD k take part; 0 or 0xff = all
-  // Confined launches only: two zeroed counters in device memory.  From claim[0]
-  // the workgroups that take part claim `num_claims` ranges of the work (set by
-  // launch_copy_kernel); claim[1] counts the workgroups that have left, and the
-  // last one zeroes both again.  Without counters the mask is ignored.
-  uint32_t *claim;
+  // Launches whose workgroups claim their work: a 64-bit counter in device memory
+  // (high half: `epoch` of the launch that owns the count, low half: ranges handed
+  // out of `num_claims`, set by launch_copy_kernel).  The counter need not be clean:
+  // the first workgroup that finds another epoch in it starts it at zero.  Without
+  // a counter the mask is ignored.
+  uint64_t *claim;
   uint32_t num_claims;
+  uint32_t epoch; // set by launch_copy_kernel: a number no other launch in flight has
   int32_t claims_per_wg; // confined launches: ranges per working workgroup (0 = 1)
 };
 constexpr int kCopyBlockThreads = 1024;  // largest workgroup the kernel is built for
@@ -186,12 +188,9 @@ struct PlanSlot;
 // Returns nullptr (and sets the error) on allocation failure.
 PlanSlot *plan_acquire(int device, size_t bytes);
 uint8_t *plan_host(PlanSlot *s);
-// `pairs` pairs of zeroed counters in device memory that belong to the slot
+// `count` claim counters in device memory that belong to the slot
 // (CopyKernelArgs::claim), or nullptr when a slot holds fewer.
-uint32_t *plan_counters(PlanSlot *s, int pairs);
-// Number of counters of all slots that are not zero (they all are whenever no
-// launch is under way); copies them from the device.
-int plan_counters_dirty(int *dirty);
+uint64_t *plan_counters(PlanSlot *s, int count);
 // Publishes the first `bytes` of the slot to the device on `stream` and returns
 // the address kernels must use (the device mirror, or the pinned buffer itself
 // when `mirror` is false).
@@ -222,7 +221,7 @@ struct KernelPlan {
   unsigned home_mask = 0xff;
   int home_workgroups = 1;
   int device = 0;
-  uint32_t *claims = nullptr; // a zeroed pair of counters per layer of the plan, device memory
+  uint64_t *claims = nullptr; // a claim counter per layer of the plan, device memory
 };
 // Link-bound launches of the last while, per device and direction (see fkv_core.cpp).
 bool link_direction_busy(int device, bool h2d, hipStream_t launching_stream);

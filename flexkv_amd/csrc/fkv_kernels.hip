@@ -122,55 +122,68 @@ __device__ __forceinline__ void copy_slice(const uint8_t *__restrict__ src,
 // workgroup landed on a selected XCD: it looks at the claim counter after a while
 // and takes over only if nobody has claimed anything.
 struct Shares {
-  uint32_t *claim;
-  uint32_t num_claims, xcd_mask;
+  unsigned long long *claim; // high half: the launch that owns the count, low half: ranges handed out
+  uint32_t num_claims, xcd_mask, epoch;
   uint32_t next_claim; // lane 0: asked for before the current range is copied
-  bool confined, dynamic, first;
+  uint32_t taken;      // lane 0 of the safety net: ranges it has claimed itself
+  bool confined, dynamic, first, safety_net;
 
   __device__ __forceinline__ Shares(const CopyKernelArgs &a)
-      : claim(a.claim), num_claims(a.num_claims), xcd_mask(a.xcd_mask & 0xffu), next_claim(0),
-        confined((a.xcd_mask & 0xffu) != 0xffu), dynamic(a.num_claims != 0), first(true) {}
+      : claim(reinterpret_cast<unsigned long long *>(a.claim)), num_claims(a.num_claims),
+        xcd_mask(a.xcd_mask & 0xffu), epoch(a.epoch), next_claim(0), taken(0),
+        confined((a.xcd_mask & 0xffu) != 0xffu), dynamic(a.num_claims != 0), first(true),
+        safety_net(false) {}
 
-  // Every workgroup of a launch with counters counts itself out; the last one leaves
-  // the two counters zeroed for the next launch that is given them.
-  __device__ __forceinline__ void leave() const {
-    if (threadIdx.x == 0 &&
-        __hip_atomic_fetch_add(claim + 1, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) ==
-            gridDim.x - 1) {
-      __hip_atomic_store(claim, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(claim + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // The counter of a launch need not be clean: it counts for this launch from the
+  // moment its high half holds the launch's number, and whoever finds another
+  // number there starts it at zero.  Returns the counter as found or made.
+  __device__ __forceinline__ unsigned long long adopt() const {
+    unsigned long long cur = __hip_atomic_load(claim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((uint32_t)(cur >> 32) != epoch) {
+      const unsigned long long fresh = (unsigned long long)epoch << 32;
+      // lost to another workgroup of this launch: then it is this launch's already
+      if (atomicCAS(claim, cur, fresh) == cur)
+        cur = fresh;
+      else
+        cur = __hip_atomic_load(claim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    return cur;
+  }
+  __device__ __forceinline__ uint32_t claim_one() const {
+    return (uint32_t)atomicAdd(claim, 1ull);
   }
 
-  // False: this workgroup takes no part (and has counted itself out).
+  // False: this workgroup takes no part.
   __device__ __forceinline__ bool enter(uint32_t *s_claim) {
     if (confined && !((xcd_mask >> xcd_of_this_wave()) & 1u)) {
-      if (blockIdx.x != 0) {
-        leave();
+      if (blockIdx.x != 0)
         return false;
-      }
       if (threadIdx.x == 0) {
         const long long t0 = wall_clock64();
         while (wall_clock64() - t0 < 5000) // 50 us of the constant 100 MHz clock
           __builtin_amdgcn_s_sleep(32);
-        *s_claim = __hip_atomic_load(claim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *s_claim = (uint32_t)adopt();
       }
       __syncthreads();
-      if (*s_claim != 0) { // the selected XCDs are at work
-        leave();
+      if (*s_claim != 0) // the selected XCDs are at work
         return false;
-      }
       __syncthreads();
+      // It works from the wrong XCD, so only for as long as nobody else claims anything:
+      // no claim ahead of time, and a look at the counter before every claim.
+      safety_net = true;
+      return true;
     }
     // lane 0 keeps the next claim in a register: it is asked for before the current
     // range is copied and has long arrived when the range is done
-    if (dynamic && threadIdx.x == 0)
-      next_claim = atomicAdd(claim, 1u);
+    if (dynamic && threadIdx.x == 0) {
+      (void)adopt();
+      next_claim = claim_one();
+    }
     return true;
   }
 
   // The next share [part/parts, (part+1)/parts) of this workgroup; false: none left
-  // (the whole workgroup leaves together, counted out).
+  // (the whole workgroup leaves together).
   __device__ __forceinline__ bool next(uint32_t *s_claim, uint32_t *part, uint32_t *parts) {
     if (!dynamic) {
       *part = blockIdx.x;
@@ -179,18 +192,23 @@ struct Shares {
       first = false;
       return mine;
     }
-    if (threadIdx.x == 0)
-      *s_claim = next_claim;
+    if (threadIdx.x == 0) {
+      if (!safety_net)
+        *s_claim = next_claim;
+      else if ((uint32_t)__hip_atomic_load(claim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) !=
+               taken)
+        *s_claim = 0xffffffffu; // the selected XCDs have turned up
+      else
+        *s_claim = claim_one(), ++taken;
+    }
     __syncthreads();
     *part = *s_claim;
     *parts = num_claims;
     __syncthreads(); // everyone has read the claim before it is overwritten
-    if (*part >= *parts) {
-      leave();
+    if (*part >= *parts)
       return false;
-    }
-    if (threadIdx.x == 0)
-      next_claim = atomicAdd(claim, 1u);
+    if (threadIdx.x == 0 && !safety_net)
+      next_claim = claim_one();
     return true;
   }
 };
@@ -492,6 +510,12 @@ void shape_launch(CopyKernelArgs &a, int64_t total, int64_t bytes, bool any_pack
   if (a.xcd_mask == 0 || !a.claim)
     a.xcd_mask = 0xffu;
   a.num_claims = 0;
+  // a number for this launch that no counter can hold by accident for long: counters
+  // are zero at first, and 2^32 - 1 launches pass before a number comes back
+  static std::atomic<uint32_t> launches{0};
+  do {
+    a.epoch = launches.fetch_add(1, std::memory_order_relaxed) + 1;
+  } while (a.epoch == 0);
   if (a.xcd_mask != 0xffu) {
     // `claims_per_wg` ranges per working workgroup (the caller's choice, 1 if it
     // makes none); `grid` working workgroups need grid / popcount(mask) rounds of 8.

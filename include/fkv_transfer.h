@@ -550,13 +550,6 @@ int fkv_range_pop(void);
 int fkv_streams_run_concurrently(int32_t device, void *stream_a, void *stream_b,
                                  int32_t *concurrent);
 
-/* Self-check: the counters from which the workgroups of a launch claim their work
- * are left zeroed by every launch.  Sets *dirty to the number of counters that are
- * not zero; call it when no transfer is under way (it copies them from the
- * device).  Anything but 0 means a launch was disturbed and a later one may have
- * run on a single workgroup.  No counterpart in the reference. */
-int fkv_plan_counters_dirty(int32_t *dirty);
-
 /* Link activity across processes.  A put and a get that run at the same time are
  * kept on different XCDs; so that this also works when they come from different
  * processes (a worker for puts, another for layerwise restores), every process
