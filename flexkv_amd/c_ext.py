@@ -43,11 +43,21 @@ def _ids(t: torch.Tensor, name: str) -> torch.Tensor:
     return t if t.is_contiguous() else t.contiguous()
 
 
+_gpu_seen = False
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _current_stream_handle() -> int:
     # Without a GPU the null stream is passed on: descriptor validation still runs
     # in the library, and the first device call there fails with a RuntimeError.
-    if not torch.cuda.is_available():
-        return 0
+    # (torch.cuda.is_available() costs 7 us a call; once a GPU has been seen it stays.)
+    global _gpu_seen
+    if not _gpu_seen:
+        if not torch.cuda.is_available():
+            return 0
+        _gpu_seen = True
+    if _raw_stream is not None:
+        return int(_raw_stream(torch.cuda.current_device()))
     return int(torch.cuda.current_stream().cuda_stream)
 
 
