@@ -107,14 +107,19 @@ typedef struct fkv_transfer_desc {
   int32_t transfer_num_cta; /* CTAs as the reference counts them; each becomes 4 (host->GPU)
                                or 12 (GPU->host) single-wavefront workgroups;
                                <= 0 = library default (4) */
-  int32_t sync;             /* 1: hipStreamSynchronize before returning */
+  int32_t sync;             /* 1: return when the transfer (and what `stream` held before it)
+                               has finished; where the reference calls cudaStreamSynchronize */
   int32_t enable_trace;     /* 1: print an "[XFER]" line per call to stderr */
   int32_t reserved;
   fkv_ce_config ce;
 } fkv_transfer_desc;
 
 /* csrc/bindings.cpp:54-151, 439-459 (`c_ext.transfer_kv_blocks`) and every
- * internal call of flexkv::transfer_kv_blocks<Type>. */
+ * internal call of flexkv::transfer_kv_blocks<Type>.  The transfer is ordered
+ * after the work `stream` holds at the call; with sync == 0, work queued on
+ * `stream` afterwards is ordered after the transfer.  The kernels themselves may
+ * run on a stream of the library (see FKV_LANE_STREAMS in the integration notes);
+ * the block-id arrays may be reused as soon as the call returns. */
 int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream);
 
 /* Which path `use_ce_transfer == 2` would take for this descriptor, from a cost
