@@ -118,8 +118,9 @@ typedef struct fkv_transfer_desc {
  * internal call of flexkv::transfer_kv_blocks<Type>.  The transfer is ordered
  * after the work `stream` holds at the call; with sync == 0, work queued on
  * `stream` afterwards is ordered after the transfer.  The kernels themselves may
- * run on a stream of the library (see FKV_LANE_STREAMS in the integration notes);
- * the block-id arrays may be reused as soon as the call returns. */
+ * run on a stream of the library when synchronous calls come in on more than two
+ * streams (FKV_LANE_STREAMS=0: never, =1: always); the block-id arrays may be
+ * reused as soon as the call returns. */
 int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream);
 
 /* Which path `use_ce_transfer == 2` would take for this descriptor, from a cost
