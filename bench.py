@@ -248,6 +248,7 @@ def run_gather_scatter(w, torch, steps, warmup, num_cta, use_ce):
     reload_ids = getattr(w, "gpu_ids_reload", w.gpu_ids)
     ev = lambda: torch.cuda.Event(enable_timing=True)
     d2h_ms, h2d_ms = [], []
+    torch.cuda.synchronize()   # the tensors were filled on another stream
     with torch.cuda.stream(st):
         for _ in range(warmup):
             w.transfer(w.gpu_ids, w.cpu_ids, False, **kw)
