@@ -147,7 +147,7 @@ class Stats(Structure):
     _fields_ = [("calls", c_uint64), ("bytes_h2d", c_uint64), ("bytes_d2h", c_uint64),
                 ("kernel_launches", c_uint64), ("dma_copies", c_uint64),
                 ("staging_bytes_device", c_uint64), ("staging_bytes_host", c_uint64),
-                ("confined_launches", c_uint64)]
+                ("confined_launches", c_uint64), ("safety_net_ranges", c_uint64)]
 
 
 # name -> (restype, argtypes); the complete export list of include/fkv_transfer.h

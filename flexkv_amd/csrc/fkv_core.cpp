@@ -738,6 +738,9 @@ void fkv_get_stats(fkv_stats *out) {
   out->staging_bytes_device = s.staging_bytes_device.load();
   out->staging_bytes_host = s.staging_bytes_host.load();
   out->confined_launches = s.confined_launches.load();
+  // a device counter: only worth a device call once a confined launch has been made
+  out->safety_net_ranges =
+      out->confined_launches ? fkv::safety_net_ranges_of_current_device() : 0;
 }
 void fkv_reset_stats(void) {
   fkv::Stats &s = fkv::stats();

@@ -167,6 +167,9 @@ struct CopyJobs {
 };
 int launch_copy_jobs(const CopyKernelArgs *jobs, int njobs, int num_workgroups,
                      int threads_per_workgroup, hipStream_t stream);
+// Ranges of work that safety-net workgroups (see the kernel) have copied on the
+// current device since the process started; reads a device counter.
+uint64_t safety_net_ranges_of_current_device();
 // Copies `bytes` (rounded up to 16) from a pinned, device-mapped host buffer to
 // device memory with a small kernel on `stream`.
 int launch_plan_upload(void *device_dst, const void *pinned_src, size_t bytes, hipStream_t stream);

@@ -121,6 +121,10 @@ __device__ __forceinline__ void copy_slice(const uint8_t *__restrict__ src,
 // none may stay there.  Workgroup 0 is the safety net for a launch of which no
 // workgroup landed on a selected XCD: it looks at the claim counter after a while
 // and takes over only if nobody has claimed anything.
+// Ranges that safety-net workgroups have copied on this device since the process
+// started: zero unless launches found none of their workgroups on the selected XCDs.
+__device__ unsigned long long g_safety_net_ranges;
+
 struct Shares {
   unsigned long long *claim; // high half: the launch that owns the count, low half: ranges handed out
   uint32_t num_claims, xcd_mask, epoch;
@@ -198,8 +202,11 @@ struct Shares {
       else if ((uint32_t)__hip_atomic_load(claim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) !=
                taken)
         *s_claim = 0xffffffffu; // the selected XCDs have turned up
-      else
+      else {
         *s_claim = claim_one(), ++taken;
+        if (*s_claim < num_claims)
+          atomicAdd(&g_safety_net_ranges, 1ull);
+      }
     }
     __syncthreads();
     *part = *s_claim;
@@ -416,6 +423,15 @@ __global__ void fkv_wait_kernel(long long ticks, int *sink) {
     *sink = 1;
 }
 } // namespace
+
+uint64_t safety_net_ranges_of_current_device() {
+  unsigned long long v = 0;
+  if (hipMemcpyFromSymbol(&v, HIP_SYMBOL(g_safety_net_ranges), sizeof(v)) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return v;
+}
 
 int launch_plan_upload(void *device_dst, const void *pinned_src, size_t bytes,
                        hipStream_t stream) {

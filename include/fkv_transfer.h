@@ -525,6 +525,10 @@ typedef struct fkv_stats {
   uint64_t staging_bytes_device;
   uint64_t staging_bytes_host;
   uint64_t confined_launches; /* kernel launches restricted to a subset of the XCDs */
+  uint64_t safety_net_ranges; /* current device, since the process started (not reset): pieces of
+                                 confined launches copied by the fallback workgroup because no
+                                 workgroup on the chosen XCDs had claimed anything in time;
+                                 expected to stay 0 */
 } fkv_stats;
 void fkv_get_stats(fkv_stats *out);
 void fkv_reset_stats(void);

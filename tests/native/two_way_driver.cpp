@@ -163,8 +163,8 @@ int main(int argc, char **argv) {
   fkv_stats st;
   fkv_get_stats(&st);
   printf("ok: puts alone %.1f GB/s, gets alone %.1f GB/s, together puts %.1f + gets %.1f = %.1f GB/s "
-         "(%ld + %ld calls of %d blocks, %llu confined launches)\n",
+         "(%ld + %ld calls of %d blocks, %llu confined launches, %llu ranges left to the safety net)\n",
          put_alone, get_alone, put.rate, get.rate, put.rate + get.rate, put.calls, get.calls, per,
-         (unsigned long long)st.confined_launches);
+         (unsigned long long)st.confined_launches, (unsigned long long)st.safety_net_ranges);
   return 0;
 }
