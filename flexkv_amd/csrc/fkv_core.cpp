@@ -754,6 +754,8 @@ void fkv_reset_stats(void) {
   s.confined_launches = 0;
 }
 
+} // extern "C"
+
 namespace {
 constexpr int kMaxDevices = 64;
 struct PerThreadEvents { // events go when their thread ends
@@ -898,6 +900,8 @@ int order_after(hipStream_t from, hipStream_t to, int device, int which) {
   return FKV_OK;
 }
 } // namespace
+
+extern "C" {
 
 int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream_v) {
   using namespace fkv;
