@@ -473,6 +473,207 @@ def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, v
                 blocks=[int(g.numel()) for g, _ in reqs], bit_exact=ok)
 
 
+def _concurrent_pair(torch):
+    """A put stream and a get stream that do not share a hardware queue."""
+    from flexkv_amd.c_ext import streams_run_concurrently
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    spare = []
+    while not streams_run_concurrently(a, b) and len(spare) < 8:
+        spare.append(b)
+        b = torch.cuda.Stream()
+    return a, b, spare
+
+
+def run_two_way(torch, device, num_cta):
+    """Puts next to gets, the situations the link arbiter is there for (one
+    process unless said otherwise; Llama-3-8B vLLM blocks of 2 MiB):
+    request streams of several sizes, a large transfer that starts 1 ms after one
+    of the other direction, a layerwise restore next to a put loop and one that
+    puts interrupt, and a get loop next to the put loop of another process."""
+    import subprocess
+    import threading
+    from flexkv_amd.c_ext import LayerwiseTransferGroup
+    res = {}
+    # every transfer stays on the stream it is issued on (read at the first transfer)
+    os.environ.setdefault("FKV_LANE_STREAMS", "0")
+    w = Workload("c4", torch, device)
+    w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=num_cta, sync=True)
+    sp, sg, _keep = _concurrent_pair(torch)
+    block = w.L * w.kv_dim * w.chunk
+
+    def streams_of(sizes_put, sizes_get):
+        reqs, off = [], 0
+        for a, b in zip(sizes_put, sizes_get):
+            reqs.append((w.gpu_ids[off:off + a].contiguous(), w.cpu_ids[off:off + a].contiguous(), False))
+            off += a
+            reqs.append((w.gpu_ids[off:off + b].contiguous(), w.cpu_ids[off:off + b].contiguous(), True))
+            off += b
+        best = 1e9
+        for _ in range(4):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for g, c, h2d in reqs:
+                with torch.cuda.stream(sg if h2d else sp):
+                    w.transfer(g, c, h2d=h2d, transfer_num_cta=num_cta, sync=False)
+            torch.cuda.synchronize()
+            best = min(best, time.perf_counter() - t0)
+        return round(off * block / best / 1e9, 2)
+
+    res["request_streams_GBps"] = {
+        "1 x 1500 blocks per direction": streams_of([1500], [1500]),
+        "4 x 375": streams_of([375] * 4, [375] * 4),
+        "16 x 94": streams_of([94] * 16, [94] * 16),
+        "125 x 12": streams_of([12] * 125, [12] * 125)}
+
+    def second_starts_later(n, first_h2d):
+        a = (w.gpu_ids[:n].contiguous(), w.cpu_ids[:n].contiguous())
+        b = (w.gpu_ids[n:2 * n].contiguous(), w.cpu_ids[n:2 * n].contiguous())
+        best = 1e9
+        for _ in range(4):
+            time.sleep(0.05)   # the first launch finds the link idle
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            with torch.cuda.stream(sg if first_h2d else sp):
+                w.transfer(*a, h2d=first_h2d, transfer_num_cta=num_cta, sync=False)
+            time.sleep(0.001)
+            with torch.cuda.stream(sp if first_h2d else sg):
+                w.transfer(*b, h2d=not first_h2d, transfer_num_cta=num_cta, sync=False)
+            torch.cuda.synchronize()
+            best = min(best, time.perf_counter() - t0)
+        return round(2 * n * block / best / 1e9, 2)
+
+    res["second_direction_starts_1ms_later_GBps"] = {
+        "put first, 400 blocks each": second_starts_later(400, False),
+        "get first, 400 blocks each": second_starts_later(400, True),
+        "put first, 1500 blocks each": second_starts_later(1500, False),
+        "get first, 1500 blocks each": second_starts_later(1500, True)}
+
+    # a get loop next to the put loop of another process (94 blocks = 197 MB per request)
+    n = 94
+    g, c = w.gpu_ids[:n].contiguous(), w.cpu_ids[:n].contiguous()
+
+    def loop(h2d, seconds):
+        k, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            w.transfer(g, c, h2d=h2d, transfer_num_cta=num_cta, sync=True)
+            k += 1
+        return k * n * block / (time.perf_counter() - t0) / 1e9
+    alone = loop(True, 1.0)
+    child = subprocess.Popen([sys.executable, os.path.abspath(__file__), "--config", "twoway",
+                              "--role", "putter"], stdin=subprocess.PIPE, stdout=subprocess.PIPE,
+                             text=True)
+    try:
+        assert child.stdout.readline().strip() == "ready"
+        child.stdin.write("\n")
+        child.stdin.flush()
+        time.sleep(0.3)
+        gets = loop(True, 2.0)
+        puts = float(child.stdout.readline())
+    finally:
+        child.wait(120)
+    res["two_processes_GBps"] = {"gets_alone": round(alone, 2), "gets": round(gets, 2),
+                                 "puts_of_the_other_process": round(puts, 2),
+                                 "sum": round(gets + puts, 2)}
+    del w
+    torch.cuda.empty_cache()
+
+    # a layerwise restore (MLA, 61 layers x 18 MiB for 256 blocks) next to puts
+    w = Workload("c3", torch, device)
+    w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=num_cta, sync=True)
+    i64 = lambda v: torch.tensor([v], dtype=torch.int64)
+    grp = LayerwiseTransferGroup(
+        num_gpus=1, gpu_blocks=[w.tensors], cpu_blocks=w.host, ssd_files={}, num_layers=w.L,
+        gpu_kv_strides_tensor=i64(w.gks), gpu_block_strides_tensor=i64(w.gbs),
+        gpu_layer_strides_tensor=i64(w.gls), gpu_chunk_sizes_tensor=i64(w.chunk),
+        iouring_entries=0, iouring_flags=0,
+        layer_eventfds_tensor=torch.empty(0, dtype=torch.int32), tp_size=1, is_blockfirst=True)
+    empty = torch.empty(0, dtype=torch.int64)
+    half = w.num_blocks // 2
+    gi, ci = w.gpu_ids[:half].contiguous(), w.cpu_ids[:half].contiguous()
+    pg, pc = w.gpu_ids[half:half + 128].contiguous(), w.cpu_ids[half:half + 128].contiguous()
+    rbytes = half * w.L * w.kv_dim * w.chunk
+
+    def enqueue_restore():
+        grp.layerwise_transfer(empty, empty, 0, 0, 0, 0, 0, gi, ci, w.cks, w.cls, w.cbs, w.chunk,
+                               w.cks, w.cls, w.cbs, num_cta, False, w.L, 1, w.kv_dim, 1,
+                               counter_id=0, kv_shared_across_ranks_mode="sharded",
+                               notify_mode="polling")
+
+    def restore():
+        enqueue_restore()
+        grp.synchronize()
+    for _ in range(2):
+        restore()
+    t0 = time.perf_counter()
+    restore()
+    restore_alone = rbytes / (time.perf_counter() - t0) / 1e9
+    go, stop, moved = threading.Event(), threading.Event(), [0, 0.0]
+
+    def putter():
+        with torch.cuda.stream(torch.cuda.Stream()):
+            go.wait()
+            t0 = time.perf_counter()
+            while not stop.is_set():
+                w.transfer(pg, pc, h2d=False, transfer_num_cta=num_cta, sync=True)
+                moved[0] += 128 * w.L * w.kv_dim * w.chunk
+            moved[1] = time.perf_counter() - t0
+    th = threading.Thread(target=putter)
+    th.start()
+    go.set()
+    time.sleep(0.05)
+    t0 = time.perf_counter()
+    for _ in range(5):
+        restore()
+    dt = time.perf_counter() - t0
+    stop.set()
+    th.join()
+    res["restore_next_to_a_put_loop_GBps"] = {"restore_alone": round(restore_alone, 2),
+                                              "restore": round(5 * rbytes / dt / 1e9, 2),
+                                              "puts": round(moved[0] / moved[1] / 1e9, 2)}
+    # The whole restore is enqueued on an idle link; the puts start 5 ms later.  Streams
+    # that share a hardware queue with the restore's stream wait for it instead of
+    # running next to it, so four put streams are tried: the longest restore is the one
+    # that was interrupted.
+    tries = []
+    for _ in range(4):
+        go.clear()
+        stop.clear()
+        th = threading.Thread(target=putter)
+        th.start()
+        time.sleep(0.1)
+        t0 = time.perf_counter()
+        enqueue_restore()
+        time.sleep(0.005)
+        go.set()
+        grp.synchronize()
+        tries.append(time.perf_counter() - t0)
+        stop.set()
+        th.join()
+    dt = max(tries)
+    res["puts_start_5ms_into_a_restore"] = {"restore_GBps": round(rbytes / dt / 1e9, 2),
+                                            "restore_ms": round(dt * 1e3, 2),
+                                            "restore_alone_ms": round(rbytes / restore_alone / 1e6, 2),
+                                            "all_tries_ms": [round(t * 1e3, 2) for t in tries]}
+    grp.close()
+    return res
+
+
+def run_two_way_putter(torch, device, num_cta):
+    """The other process of run_two_way: waits for a line on stdin, puts 94-block
+    requests for 3 s and prints its rate."""
+    w = Workload("c0", torch, device)
+    n = 94
+    g, c = w.gpu_ids[:n].contiguous(), w.cpu_ids[:n].contiguous()
+    w.transfer(g, c, False, transfer_num_cta=num_cta, sync=True)
+    print("ready", flush=True)
+    sys.stdin.readline()
+    k, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < 3.0:
+        w.transfer(g, c, h2d=False, transfer_num_cta=num_cta, sync=True)
+        k += 1
+    print(f"{k * n * w.L * w.kv_dim * w.chunk / (time.perf_counter() - t0) / 1e9:.2f}", flush=True)
+
+
 def run_notify_scales(torch, device, num_cta, iters=20, warmup=3):
     """Layerwise host->GPU restore end to end (call + device synchronize) at the
     three scales of the reference's notify-mode microbenchmark
@@ -903,7 +1104,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker", "ssd", "transform"])
+    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker", "ssd", "transform", "twoway"])
+    ap.add_argument("--role", default="", help=argparse.SUPPRESS)
     ap.add_argument("--shape", default="c0", choices=["c0", "c3"],
                     help="transform: which engine shape to re-lay out")
     ap.add_argument("--streams-per-direction", type=int, default=32,
@@ -966,6 +1168,22 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"config": {"workload": "copycal"}, "copy_bytes": n,
                           "copies_of_each_kind": max(1, args.steps)}))
+        return
+    if args.config == "twoway":
+        if args.role == "putter":
+            run_two_way_putter(torch, device, args.num_cta)
+            return
+        bidir = measure_link_bidirectional(torch, device)
+        res = run_two_way(torch, device, args.num_cta)
+        print(json.dumps({
+            "metric": "puts next to gets: GB/s in sum over the host link",
+            "unit": "GB/s", "value": res["request_streams_GBps"]["16 x 94"], "n_gpus": 1,
+            "higher_is_better": True, "dtype": "u8", "data": "synthetic", "vs_baseline": None,
+            "config": {"workload": "twoway: Llama-3-8B vLLM blocks of 2 MiB (request streams, "
+                                   "late second direction, two processes); MLA restore of 256 "
+                                   "blocks x 61 layers next to puts",
+                       "transfer_num_cta": args.num_cta},
+            "bidir_link_peak_GBps": round(bidir, 3), "results": res}))
         return
     if args.config == "notify":
         res = run_notify_scales(torch, device, args.num_cta)

@@ -316,7 +316,7 @@ LinkLaunchShape link_launch_shape(bool is_h2d) {
 // on two XCDs and nothing on three (1-3), a lone host->GPU transfer nothing on 4-7,
 // so launches of 8 MiB and more (FKV_HOME_MIN_KB, -1: never) keep to these home
 // XCDs even when the link is idle: a put launched alone and a get that arrives
-// 1 ms later reach 93 GB/s instead of 78, in the other order 80 instead of 66.
+// 1 ms later reach 93 GB/s instead of 61, in the other order 80 instead of 72.
 // A direction also counts as busy for a short
 // while after its last launch (FKV_LINK_ARBITER_WINDOW_MS, default 20): with many
 // small requests in flight the other direction is often between two kernels at
