@@ -658,6 +658,54 @@ def run_two_way(torch, device, num_cta):
     return res
 
 
+def run_neighbour(torch, device, num_cta, n=2048, count=150):
+    """What a transfer costs a compute kernel that runs next to it: the time of
+    one n^3 bf16 GEMM (150 in a row on a stream of their own) alone, next to a
+    one-thread spin kernel, next to kernel transfers of either direction, and next
+    to pinned copies of the copy engines."""
+    w = Workload("c0", torch, device)
+    w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=num_cta, sync=True)
+    comp, other, _keep = _concurrent_pair(torch)
+    a = torch.randn(n, n, device=device, dtype=torch.bfloat16)
+    b = torch.randn(n, n, device=device, dtype=torch.bfloat16)
+    c = torch.empty(n, n, device=device, dtype=torch.bfloat16)
+    big_h = torch.empty(1 << 30, dtype=torch.uint8, pin_memory=True)
+    big_d = torch.empty(1 << 30, dtype=torch.uint8, device=device)
+
+    def case(background):
+        torch.cuda.synchronize()
+        if background:
+            with torch.cuda.stream(other):
+                background()
+        time.sleep(0.002)
+        with torch.cuda.stream(comp):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record(comp)
+            for _ in range(count):
+                torch.matmul(a, b, out=c)
+            e.record(comp)
+        e.synchronize()
+        still_running = not other.query()
+        torch.cuda.synchronize()
+        return {"us_per_gemm": round(s.elapsed_time(e) / count * 1e3, 1),
+                "background_outlasted_the_gemms": still_running}
+    xfer = lambda h2d, cta, reps: (lambda: [w.transfer(w.gpu_ids, w.cpu_ids, h2d,
+                                                       transfer_num_cta=cta, sync=False)
+                                            for _ in range(reps)])
+    for _ in range(2):
+        case(None)
+    return {
+        "alone": case(None),
+        "next to a one-thread spin kernel": case(lambda: torch.cuda._sleep(int(2.4e9 * 0.05))),
+        "next to a host->GPU kernel transfer": case(xfer(True, num_cta, 3)),
+        "next to a GPU->host kernel transfer": case(xfer(False, num_cta, 3)),
+        "next to a host->GPU kernel transfer, transfer_num_cta=1": case(xfer(True, 1, 1)),
+        "next to pinned hipMemcpyAsync host->GPU": case(
+            lambda: [big_d.copy_(big_h, non_blocking=True) for _ in range(3)]),
+        "next to pinned hipMemcpyAsync GPU->host": case(
+            lambda: [big_h.copy_(big_d, non_blocking=True) for _ in range(3)])}
+
+
 def run_two_way_putter(torch, device, num_cta):
     """The other process of run_two_way: waits for a line on stdin, puts 94-block
     requests for 3 s and prints its rate."""
@@ -1104,7 +1152,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker", "ssd", "transform", "twoway"])
+    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker", "ssd", "transform", "twoway", "neighbour"])
+    ap.add_argument("--gemm-n", type=int, default=2048, help="neighbour: size of the GEMM")
     ap.add_argument("--role", default="", help=argparse.SUPPRESS)
     ap.add_argument("--shape", default="c0", choices=["c0", "c3"],
                     help="transform: which engine shape to re-lay out")
@@ -1168,6 +1217,16 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"config": {"workload": "copycal"}, "copy_bytes": n,
                           "copies_of_each_kind": max(1, args.steps)}))
+        return
+    if args.config == "neighbour":
+        res = run_neighbour(torch, device, args.num_cta, n=args.gemm_n)
+        print(json.dumps({
+            "metric": "time of a bf16 GEMM next to a transfer", "unit": "us",
+            "value": res["next to a host->GPU kernel transfer"]["us_per_gemm"], "n_gpus": 1,
+            "higher_is_better": False, "data": "synthetic", "vs_baseline": None,
+            "config": {"workload": f"neighbour: {args.gemm_n}^3 bf16 GEMM x150 next to c0-shaped "
+                                   "transfers of 512 MiB", "transfer_num_cta": args.num_cta},
+            "results": res}))
         return
     if args.config == "twoway":
         if args.role == "putter":
