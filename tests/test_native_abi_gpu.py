@@ -50,3 +50,13 @@ def test_two_threads_of_a_native_program_put_and_get_at_once(gpu_device, asan):
     import re
     nums = [float(x) for x in re.findall(r"([0-9.]+) GB/s", r.stdout)]
     assert len(nums) == 3 and nums[2] > 1.2 * max(nums[0], nums[1]), r.stdout
+
+
+def test_link_gap_probe_runs(gpu_device):
+    """tests/native/link_gap_probe.hip, the stand-alone measurement behind the XCD
+    split and the event flags: it has to build and run; its figures are for reading."""
+    exe = os.path.join(BUILD, "link_gap_probe")
+    assert os.path.exists(exe), f"{exe} is missing: run make -C tests/native"
+    r = subprocess.run([exe, "--between", "event-nofence"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 0 and "mean gap" in r.stdout, r.stdout + r.stderr
