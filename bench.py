@@ -41,7 +41,7 @@ METRIC = "KV block transfer GB/s (D2H, H2D) on 1 GPU; % of measured host-link pe
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs of this script scaled by plain copy kernels of known size
 # (profiles/fkv_copy_chunks_kernel_c1_pmc.md).  None where no such run was made.
-MEASURED_TRAFFIC_BYTES = {("c1", "kernel"): 8591004672, ("transform-c0", "kernel"): 8590453760}
+MEASURED_TRAFFIC_BYTES = {("c1", "kernel"): 8590414848, ("transform-c0", "kernel"): 8590474240}
 
 
 def _median(xs):
