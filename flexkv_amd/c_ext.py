@@ -16,7 +16,7 @@ when the library is missing.
 from __future__ import annotations
 
 import ctypes
-from typing import Dict, List, Optional, Sequence
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -28,7 +28,7 @@ from ._lib import (CEConfig, LayerGroup, LayerMember, LayerwiseCall, LayerwiseMG
 
 _L = _lib.load()
 
-__all__ = ["transfer_kv_blocks", "transfer_kv_blocks_ssd", "SSDIOCTX", "TPTransferThreadGroup",
+__all__ = ["transfer_kv_blocks", "transfer_kv_blocks_multi", "transfer_kv_blocks_ssd", "SSDIOCTX", "TPTransferThreadGroup",
            "LayerwiseTransferGroup",
            "last_transfer_path", "get_stats", "reset_stats"]
 
@@ -83,7 +83,7 @@ def _ce_config(segment_threshold, path_opt, force_path, enable_memcpy2d, is_bloc
     return cfg
 
 
-def transfer_kv_blocks(
+def _transfer_desc(
         gpu_block_id_tensor: torch.Tensor, gpu_tensor_ptrs_tensor: torch.Tensor,
         gpu_kv_stride_in_bytes: int, gpu_block_stride_in_bytes: int,
         gpu_layer_stride_in_bytes: int, cpu_block_id_tensor: torch.Tensor,
@@ -96,14 +96,9 @@ def transfer_kv_blocks(
         ce_segment_threshold: int = 8, ce_force_path: int = -1,
         ce_enable_memcpy2d: bool = False, is_blockfirst: bool = False,
         ce_gather_threads: int = 4, ce_gather_nt: bool = True,
-        enable_transfer_trace: bool = False) -> None:
-    """Transfer multi-layer KV-cache between CPU and GPU on the current stream
-    (``csrc/bindings.cpp:54-151``).
-
-    ``gpu_tensor_ptrs_tensor`` is an int64 host tensor of device addresses: L
-    entries for vLLM (``gpu_block_type`` 0), one for TRT-LLM (1), K₀..K_{L-1},
-    V₀..V_{L-1} for SGLang (2).
-    """
+        enable_transfer_trace: bool = False) -> Tuple[TransferDesc, tuple]:
+    """The descriptor of one transfer and the tensors it points into (to be kept
+    alive until the call has been made)."""
     gpu_ids = _ids(gpu_block_id_tensor, "gpu_block_id_tensor")
     cpu_ids = _ids(cpu_block_id_tensor, "cpu_block_id_tensor")
     if gpu_ids.numel() != cpu_ids.numel():
@@ -139,14 +134,63 @@ def transfer_kv_blocks(
     d.gpu_block_ids = gpu_ids.data_ptr()
     d.cpu_block_ids = cpu_ids.data_ptr()
     d.is_host_to_device = int(bool(is_host_to_device))
-    # True/False as in the reference; "auto" (or 2) lets the library pick per transfer
     d.use_ce_transfer = _engine_code(use_ce_transfer)
     d.transfer_num_cta = int(transfer_num_cta)
     d.sync = int(bool(sync))
     d.enable_trace = int(bool(enable_transfer_trace))
     d.ce = _ce_config(ce_segment_threshold, ce_path_opt, ce_force_path, ce_enable_memcpy2d,
                       is_blockfirst, num_kv_heads, ce_gather_threads, ce_gather_nt)
+    return d, (gpu_ids, cpu_ids, ptrs, cpu_tensor)
+
+
+def transfer_kv_blocks(
+        gpu_block_id_tensor: torch.Tensor, gpu_tensor_ptrs_tensor: torch.Tensor,
+        gpu_kv_stride_in_bytes: int, gpu_block_stride_in_bytes: int,
+        gpu_layer_stride_in_bytes: int, cpu_block_id_tensor: torch.Tensor,
+        cpu_tensor: torch.Tensor, cpu_kv_stride_in_bytes: int,
+        cpu_layer_stride_in_bytes: int, cpu_block_stride_in_bytes: int,
+        chunk_size_in_bytes: int, start_layer_id: int, num_layers: int,
+        transfer_num_cta: int = 4, is_host_to_device: bool = True,
+        use_ce_transfer: bool = False, kv_dim: int = 2, num_kv_heads: int = 1,
+        gpu_block_type: int = 0, sync: bool = True, ce_path_opt: bool = False,
+        ce_segment_threshold: int = 8, ce_force_path: int = -1,
+        ce_enable_memcpy2d: bool = False, is_blockfirst: bool = False,
+        ce_gather_threads: int = 4, ce_gather_nt: bool = True,
+        enable_transfer_trace: bool = False) -> None:
+    """Transfer multi-layer KV-cache between CPU and GPU on the current stream
+    (``csrc/bindings.cpp:54-151``).
+
+    ``gpu_tensor_ptrs_tensor`` is an int64 host tensor of device addresses: L
+    entries for vLLM (``gpu_block_type`` 0), one for TRT-LLM (1), K₀..K_{L-1},
+    V₀..V_{L-1} for SGLang (2).
+    """
+    d, _alive = _transfer_desc(
+        gpu_block_id_tensor, gpu_tensor_ptrs_tensor, gpu_kv_stride_in_bytes,
+        gpu_block_stride_in_bytes, gpu_layer_stride_in_bytes, cpu_block_id_tensor, cpu_tensor,
+        cpu_kv_stride_in_bytes, cpu_layer_stride_in_bytes, cpu_block_stride_in_bytes,
+        chunk_size_in_bytes, start_layer_id, num_layers, transfer_num_cta, is_host_to_device,
+        use_ce_transfer, kv_dim, num_kv_heads, gpu_block_type, sync, ce_path_opt,
+        ce_segment_threshold, ce_force_path, ce_enable_memcpy2d, is_blockfirst,
+        ce_gather_threads, ce_gather_nt, enable_transfer_trace)
     check(_L.fkv_transfer_kv_blocks(ctypes.byref(d), _current_stream_handle()))
+
+
+def transfer_kv_blocks_multi(calls) -> None:
+    """Several transfers of one direction in one call: ``calls`` is a sequence of
+    ``(args, kwargs)`` as ``transfer_kv_blocks`` takes them, e.g. one per layer group
+    of a multi-group model (``flexkv/transfer/worker.py:998-1015`` issues them one
+    after the other).  Equivalent to making the calls in order; ``sync`` of the last
+    one applies to all.  On the kernel path up to four of them share one launch."""
+    calls = list(calls)
+    if not calls:
+        return
+    descs = (TransferDesc * len(calls))()
+    alive = []
+    for i, (args, kwargs) in enumerate(calls):
+        d, keep = _transfer_desc(*args, **kwargs)
+        descs[i] = d
+        alive.append(keep)
+    check(_L.fkv_transfer_kv_blocks_multi(descs, len(calls), _current_stream_handle()))
 
 
 def layout_transform(

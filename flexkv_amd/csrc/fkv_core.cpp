@@ -899,6 +899,122 @@ int order_after(hipStream_t from, hipStream_t to, int device, int which) {
   FKV_HIP_TRY(hipStreamWaitEvent(to, ev, 0));
   return FKV_OK;
 }
+
+// Several descriptors of one direction on the kernel path: a plan each, one launch
+// for all of them where they can share one.
+int run_kernel_path_multi(const fkv_transfer_desc *descs, int count, hipStream_t stream) {
+  fkv::set_last_path(FKV_PATH_KERNEL);
+  std::vector<fkv::KernelPlan> plans(count);
+  int rc = FKV_OK, built = 0;
+  for (; built < count && rc == FKV_OK; ++built)
+    rc = fkv::kernel_plan_build(descs[built], stream, &plans[built]);
+  if (rc != FKV_OK)
+    --built; // the one that failed holds nothing
+  for (int k = 0; k < built && rc == FKV_OK; k += fkv::kCopyMaxJobs) {
+    const int n = std::min(fkv::kCopyMaxJobs, built - k);
+    const fkv::KernelPlan *group[fkv::kCopyMaxJobs];
+    int first[fkv::kCopyMaxJobs], layers[fkv::kCopyMaxJobs];
+    for (int j = 0; j < n; ++j) {
+      group[j] = &plans[k + j];
+      first[j] = 0;
+      layers[j] = descs[k + j].num_layers;
+    }
+    rc = fkv::kernel_plans_launch(group, first, layers, n, stream);
+  }
+  for (int i = 0; i < built; ++i)
+    fkv::kernel_plan_release(&plans[i], stream);
+  return rc;
+}
+
+// The body of fkv_transfer_kv_blocks{,_multi}: `count` validated, non-empty
+// descriptors of one direction and device; the last one says whether to wait.
+int transfer_descs(const fkv_transfer_desc *descs, int count, hipStream_t stream) {
+  using namespace fkv;
+  const fkv_transfer_desc &d = descs[0];
+  const bool sync = descs[count - 1].sync != 0, trace = descs[count - 1].enable_trace != 0;
+  DeviceGuard guard(d.device);
+  if (!guard.ok())
+    return fail(FKV_ERR_RUNTIME, "cannot select HIP device %d", d.device);
+  uint64_t bytes = 0;
+  int64_t blocks = 0;
+  for (int i = 0; i < count; ++i) {
+    bytes += (uint64_t)descs[i].num_blocks * descs[i].num_layers * descs[i].kv_dim *
+             (uint64_t)descs[i].chunk_size;
+    blocks += descs[i].num_blocks;
+  }
+  Range range("fkv %s %d blocks x %d layers (%.2f MB)%s", d.is_host_to_device ? "H2D" : "D2H",
+              d.num_blocks, d.num_layers, bytes / (1024.0 * 1024.0),
+              count > 1 ? " and more groups" : "");
+  // 0 kernel, 1 copy engine, 2 decide per transfer; FKV_TRANSFER_ENGINE overrides the caller.
+  static const int forced_engine = [] {
+    const char *v = std::getenv("FKV_TRANSFER_ENGINE");
+    if (!v || !*v)
+      return -1;
+    return !std::strcmp(v, "kernel") ? 0 : !std::strcmp(v, "ce") ? 1 : !std::strcmp(v, "auto") ? 2 : -1;
+  }();
+  // the engine of every descriptor; the kernel path takes them together
+  std::vector<int> engines(count);
+  bool all_kernel = true;
+  for (int i = 0; i < count; ++i) {
+    engines[i] = forced_engine >= 0 ? forced_engine : descs[i].use_ce_transfer;
+    if (engines[i] == 2)
+      FKV_TRY(choose_engine(descs[i], &engines[i], nullptr, nullptr));
+    all_kernel = all_kernel && engines[i] == 0;
+  }
+  auto run_all = [&](hipStream_t on) -> int {
+    if (all_kernel)
+      return count == 1 ? run_kernel_path(d, on) : run_kernel_path_multi(descs, count, on);
+    for (int i = 0; i < count; ++i)
+      FKV_TRY(engines[i] ? run_ce_path(descs[i], on) : run_kernel_path(descs[i], on));
+    return FKV_OK;
+  };
+  int device = 0;
+  FKV_HIP_TRY(hipGetDevice(&device));
+  Lane *lane = (all_kernel && lanes_wanted(device, stream, sync))
+                   ? lane_of(device, d.is_host_to_device != 0)
+                   : nullptr;
+  hipEvent_t done = nullptr;
+  if (lane) {
+    std::lock_guard<std::mutex> lk(lane->mu);
+    // the lane starts after what the caller's stream holds; an idle stream holds nothing
+    if (hipStreamQuery(stream) != hipSuccess) {
+      (void)hipGetLastError();
+      FKV_TRY(order_after(stream, lane->stream, device, 0));
+    }
+    FKV_TRY(run_all(lane->stream));
+    if (sync)
+      FKV_TRY(record_completion(lane->stream, !d.is_host_to_device, &done));
+    else
+      FKV_TRY(order_after(lane->stream, stream, device, 1));
+    stream = lane->stream;
+  } else {
+    FKV_TRY(run_all(stream));
+    if (sync)
+      FKV_TRY(record_completion(stream, /*host_reads_result=*/!d.is_host_to_device, &done));
+  }
+  (d.is_host_to_device ? stats().bytes_h2d : stats().bytes_d2h)
+      .fetch_add(bytes, std::memory_order_relaxed);
+
+  if (sync) {
+    auto t0 = std::chrono::steady_clock::now();
+    if (done)
+      FKV_HIP_TRY(hipEventSynchronize(done));
+    else
+      FKV_HIP_TRY(hipStreamSynchronize(stream));
+    if (trace) {
+      double ms = std::chrono::duration<double, std::milli>(
+                      std::chrono::steady_clock::now() - t0)
+                      .count();
+      // same fields as the reference's trace line, csrc/transfer.cu:304-311
+      fprintf(stderr, "[XFER] type=%s blocks=%lld sync_ms=%.3f\n",
+              d.is_host_to_device ? "H2D" : "D2H", (long long)blocks, ms);
+    }
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return fail(FKV_ERR_RUNTIME, "%s", hipGetErrorString(e));
+  return FKV_OK;
+}
 } // namespace
 
 extern "C" {
@@ -908,80 +1024,35 @@ int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream_v) {
   clear_error();
   if (!desc)
     return fail(FKV_ERR_INVALID_ARG, "null descriptor");
-  const fkv_transfer_desc &d = *desc;
-  FKV_TRY(validate(d));
-  hipStream_t stream = static_cast<hipStream_t>(stream_v);
+  FKV_TRY(validate(*desc));
   stats().calls.fetch_add(1, std::memory_order_relaxed);
-  if (d.num_blocks == 0 || d.num_layers == 0)
+  if (desc->num_blocks == 0 || desc->num_layers == 0)
     return FKV_OK;
-  DeviceGuard guard(d.device);
-  if (!guard.ok())
-    return fail(FKV_ERR_RUNTIME, "cannot select HIP device %d", d.device);
+  return transfer_descs(desc, 1, static_cast<hipStream_t>(stream_v));
+}
 
-  const uint64_t bytes =
-      (uint64_t)d.num_blocks * d.num_layers * d.kv_dim * (uint64_t)d.chunk_size;
-  Range range("fkv %s %d blocks x %d layers (%.2f MB)", d.is_host_to_device ? "H2D" : "D2H",
-              d.num_blocks, d.num_layers, bytes / (1024.0 * 1024.0));
-  // 0 kernel, 1 copy engine, 2 decide per transfer; FKV_TRANSFER_ENGINE overrides the caller.
-  static const int forced_engine = [] {
-    const char *v = std::getenv("FKV_TRANSFER_ENGINE");
-    if (!v || !*v)
-      return -1;
-    return !std::strcmp(v, "kernel") ? 0 : !std::strcmp(v, "ce") ? 1 : !std::strcmp(v, "auto") ? 2 : -1;
-  }();
-  int engine = forced_engine >= 0 ? forced_engine : d.use_ce_transfer;
-  if (engine == 2)
-    FKV_TRY(choose_engine(d, &engine, nullptr, nullptr));
-  int device = 0;
-  FKV_HIP_TRY(hipGetDevice(&device));
-  Lane *lane = (!engine && lanes_wanted(device, stream, d.sync != 0)) ? lane_of(device, d.is_host_to_device != 0)
-                                                         : nullptr;
-  hipEvent_t done = nullptr;
-  int rc;
-  if (lane) {
-    std::lock_guard<std::mutex> lk(lane->mu);
-    // the lane starts after what the caller's stream holds; an idle stream holds nothing
-    if (hipStreamQuery(stream) != hipSuccess) {
-      (void)hipGetLastError();
-      FKV_TRY(order_after(stream, lane->stream, device, 0));
-    }
-    rc = run_kernel_path(d, lane->stream);
-    if (rc != FKV_OK)
-      return rc;
-    if (d.sync)
-      FKV_TRY(record_completion(lane->stream, !d.is_host_to_device, &done));
-    else
-      FKV_TRY(order_after(lane->stream, stream, device, 1));
-    stream = lane->stream;
-  } else {
-    rc = engine ? run_ce_path(d, stream) : run_kernel_path(d, stream);
-    if (rc != FKV_OK)
-      return rc;
-    if (d.sync)
-      FKV_TRY(record_completion(stream, /*host_reads_result=*/!d.is_host_to_device, &done));
+int fkv_transfer_kv_blocks_multi(const fkv_transfer_desc *descs, int32_t count, void *stream_v) {
+  using namespace fkv;
+  clear_error();
+  if (count < 0 || (count > 0 && !descs))
+    return fail(FKV_ERR_INVALID_ARG, "fkv_transfer_kv_blocks_multi: bad descriptor array");
+  std::vector<fkv_transfer_desc> work;
+  for (int i = 0; i < count; ++i) {
+    FKV_TRY(validate(descs[i]));
+    stats().calls.fetch_add(1, std::memory_order_relaxed);
+    if (descs[i].num_blocks == 0 || descs[i].num_layers == 0)
+      continue;
+    if (!work.empty() && ((descs[i].is_host_to_device != 0) != (work[0].is_host_to_device != 0) ||
+                          descs[i].device != work[0].device))
+      return fail(FKV_ERR_INVALID_ARG,
+                  "fkv_transfer_kv_blocks_multi: descriptors differ in direction or device");
+    work.push_back(descs[i]);
   }
-  (d.is_host_to_device ? stats().bytes_h2d : stats().bytes_d2h)
-      .fetch_add(bytes, std::memory_order_relaxed);
-
-  if (d.sync) {
-    auto t0 = std::chrono::steady_clock::now();
-    if (done)
-      FKV_HIP_TRY(hipEventSynchronize(done));
-    else
-      FKV_HIP_TRY(hipStreamSynchronize(stream));
-    if (d.enable_trace) {
-      double ms = std::chrono::duration<double, std::milli>(
-                      std::chrono::steady_clock::now() - t0)
-                      .count();
-      // same fields as the reference's trace line, csrc/transfer.cu:304-311
-      fprintf(stderr, "[XFER] type=%s blocks=%d sync_ms=%.3f\n",
-              d.is_host_to_device ? "H2D" : "D2H", d.num_blocks, ms);
-    }
-  }
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess)
-    return fail(FKV_ERR_RUNTIME, "%s", hipGetErrorString(e));
-  return FKV_OK;
+  if (work.empty())
+    return FKV_OK;
+  work.back().sync = descs[count - 1].sync;
+  work.back().enable_trace = descs[count - 1].enable_trace;
+  return transfer_descs(work.data(), (int)work.size(), static_cast<hipStream_t>(stream_v));
 }
 
 } // extern "C"

@@ -668,7 +668,7 @@ class GPUCPUTransferWorker(TransferWorkerBase):
 
     def _transfer_impl(self, src_block_ids: torch.Tensor, dst_block_ids: torch.Tensor,
                        transfer_type: TransferType) -> None:
-        from ..c_ext import transfer_kv_blocks
+        from ..c_ext import transfer_kv_blocks, transfer_kv_blocks_multi
         assert src_block_ids.dtype == torch.int64 and dst_block_ids.dtype == torch.int64
         assert len(src_block_ids) == len(dst_block_ids)
         gpu_ids, cpu_ids, h2d = _direction(transfer_type, src_block_ids, dst_block_ids,
@@ -686,16 +686,14 @@ class GPUCPUTransferWorker(TransferWorkerBase):
                     enable_transfer_trace=global_env().enable_transfer_trace)
         if self.group_transfer_params is not None:
             flat = self.cpu_tensor.view(torch.uint8).view(-1)
-            # one call per group, its slice of the block; the calls share a stream, so only
-            # the last one waits (the library copies the ids of an asynchronous call)
-            last = len(self.group_transfer_params) - 1
-            for i, gp in enumerate(self.group_transfer_params):
-                transfer_kv_blocks(gpu_ids, gp["gpu_ptrs"], gp["gpu_kv_stride"],
-                                   gp["gpu_block_stride"], gp["gpu_layer_stride"], cpu_ids,
-                                   flat[gp["cpu_offset_bytes"]:], gp["cpu_kv_stride"],
-                                   gp["cpu_layer_stride"], gp["cpu_block_stride"],
-                                   gp["chunk_size"], 0, gp["num_layers"],
-                                   **dict(tail, sync=(i == last)))
+            # one descriptor per group, its slice of the block, in one call: the library
+            # puts groups of like shape into one launch and waits once, after the last
+            transfer_kv_blocks_multi(
+                ((gpu_ids, gp["gpu_ptrs"], gp["gpu_kv_stride"], gp["gpu_block_stride"],
+                  gp["gpu_layer_stride"], cpu_ids, flat[gp["cpu_offset_bytes"]:],
+                  gp["cpu_kv_stride"], gp["cpu_layer_stride"], gp["cpu_block_stride"],
+                  gp["chunk_size"], 0, gp["num_layers"]), tail)
+                for gp in self.group_transfer_params)
             return
         transfer_kv_blocks(gpu_ids, self.gpu_blocks_ptrs, self.gpu_kv_stride_in_bytes,
                            self.gpu_block_stride_in_bytes, self.gpu_layer_stride_in_bytes,

@@ -123,6 +123,14 @@ typedef struct fkv_transfer_desc {
  * reused as soon as the call returns. */
 int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream);
 
+/* The same for `count` descriptors of one direction and device at once, as the
+ * reference's worker issues them one after the other for the layer groups of a
+ * multi-group model (flexkv/transfer/worker.py:998-1015): one call per group with
+ * the group's tensors, strides and chunk size.  Equivalent to `count` calls in
+ * order; `sync` and `enable_trace` of the last descriptor apply to the whole.  On
+ * the kernel path up to four of them share one launch. */
+int fkv_transfer_kv_blocks_multi(const fkv_transfer_desc *descs, int32_t count, void *stream);
+
 /* Which path `use_ce_transfer == 2` would take for this descriptor, from a cost
  * model of both (DMA commands, staging passes, link time); pure host function.
  * The reference fixes the engine per direction by configuration

@@ -167,6 +167,44 @@ int main() {
       ++cases;
     }
 
+  // ---- fkv_transfer_kv_blocks_multi: the layers in three descriptors, one call ----
+  for (int h2d = 0; h2d < 2; ++h2d) {
+    std::vector<int64_t> g = pick(rng, N, 29), c = pick(rng, NH, 29);
+    const int first[3] = {0, 2, 5}, count[3] = {2, 3, 1};
+    fkv_transfer_desc ds[3];
+    memset(ds, 0, sizeof(ds));
+    for (int k = 0; k < 3; ++k) {
+      fkv_transfer_desc &d = ds[k];
+      d.backend = FKV_BACKEND_VLLM;
+      d.num_layers_total = L;
+      d.gpu_tensor_ptrs = ptrs.data();
+      d.num_gpu_tensor_ptrs = L;
+      d.device = -1;
+      d.gpu_kv_stride = GKS, d.gpu_block_stride = GBS, d.gpu_layer_stride = GLS;
+      d.cpu_ptr = host;
+      d.cpu_kv_stride = CKS, d.cpu_layer_stride = CLS, d.cpu_block_stride = CBS;
+      d.chunk_size = CHUNK;
+      d.start_layer_id = first[k], d.num_layers = count[k], d.kv_dim = KV, d.num_blocks = 29;
+      d.gpu_block_ids = g.data(), d.cpu_block_ids = c.data();
+      d.transfer_num_cta = 4;
+      d.sync = k == 2;
+      d.is_host_to_device = h2d;
+      fkv_ce_config_default(&d.ce);
+      d.ce.is_blockfirst = 1;
+    }
+    FKV_OK_OR_DIE(fkv_transfer_kv_blocks_multi(ds, 3, stream));
+    m.put(g, c, h2d != 0);
+    if (check("multi"))
+      return 1;
+    ds[1].is_host_to_device = !h2d; // one call has one direction
+    if (fkv_transfer_kv_blocks_multi(ds, 3, stream) != FKV_ERR_INVALID_ARG ||
+        !strstr(fkv_last_error(), "direction")) {
+      fprintf(stderr, "mixed directions were not refused\n");
+      return 1;
+    }
+    ++cases;
+  }
+
   // ---- TP group with one rank ----
   {
     const int64_t ks = GKS, bs = GBS, ls = GLS, cs = CHUNK, did = 0;

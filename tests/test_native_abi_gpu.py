@@ -18,7 +18,7 @@ def run(exe, **env):
     r = subprocess.run([exe], capture_output=True, text=True, timeout=300,
                        env=dict(os.environ, **env))
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
-    assert "ok: 30 cases through the C ABI" in r.stdout, r.stdout
+    assert "ok: 32 cases through the C ABI" in r.stdout, r.stdout
     return r
 
 

@@ -444,3 +444,107 @@ def test_very_many_blocks_in_one_call(gpu_device, chunk, n):
     dev.transfer(back, cids, is_h2d=True)
     s.oracle_transfer(back, cids, True)
     dev.assert_matches_reference(f"{n} blocks H2D")
+
+
+# ---- several transfers in one call (fkv_transfer_kv_blocks_multi) ----------------------
+
+def _multi_call(devs, gids, cids, h2d, engines=None, sync=True, **kw):
+    """One descriptor per device-side setup, all with the same block ids."""
+    import torch
+    from flexkv_amd.c_ext import transfer_kv_blocks_multi
+    g = torch.as_tensor(np.asarray(gids, dtype=np.int64))
+    c = torch.as_tensor(np.asarray(cids, dtype=np.int64))
+    calls = []
+    for i, dev in enumerate(devs):
+        s = dev.s
+        calls.append(((g, dev.ptrs, s.gpu_kv_stride, s.gpu_block_stride, s.gpu_layer_stride, c,
+                       dev.host, s.cpu_kv_stride, s.cpu_layer_stride, s.cpu_block_stride,
+                       s.chunk, 0, s.num_layers),
+                      dict(kw, is_host_to_device=h2d, kv_dim=s.kv_dim, gpu_block_type=s.backend,
+                           is_blockfirst=s.cpu_layout == "BLOCKFIRST", sync=sync,
+                           use_ce_transfer=engines[i] if engines else False)))
+    transfer_kv_blocks_multi(calls)
+
+
+@pytest.mark.parametrize("case", ["alike", "mixed_widths", "six_groups", "with_copy_engine"])
+def test_several_transfers_in_one_call_match_oracle(gpu_device, case):
+    from flexkv_amd.c_ext import get_stats, reset_stats
+    setups = {
+        # same vector width and launch shape: one launch
+        "alike": [KVSetup(VLLM, 5, 2, 40, 40, 4096, "BLOCKFIRST", seed=21),
+                  KVSetup(VLLM, 3, 1, 40, 40, 1024, "LAYERFIRST", seed=22),
+                  KVSetup(SGLANG, 2, 2, 40, 40, 2048, "BLOCKFIRST", seed=23)],
+        # a 200-byte chunk needs 8-byte vectors: launches of its own
+        "mixed_widths": [KVSetup(VLLM, 4, 2, 40, 40, 4096, "BLOCKFIRST", seed=24),
+                         KVSetup(VLLM, 4, 1, 40, 40, 200, "BLOCKFIRST", seed=25),
+                         KVSetup(TRTLLM, 2, 2, 40, 40, 512, "BLOCKFIRST", seed=26)],
+        # more than one launch holds
+        "six_groups": [KVSetup(VLLM, 2 + i, 1 + i % 2, 40, 40, 256 << i, "BLOCKFIRST", seed=30 + i)
+                       for i in range(6)],
+        "with_copy_engine": [KVSetup(VLLM, 3, 2, 40, 40, 4096, "BLOCKFIRST", seed=27),
+                             KVSetup(VLLM, 3, 2, 40, 40, 8192, "LAYERFIRST", seed=28)],
+    }[case]
+    engines = [False, True] if case == "with_copy_engine" else None
+    devs = [s.to_device(gpu_device) for s in setups]
+    rng = np.random.default_rng(9)
+    gids, cids = block_ids(rng, 40, 17), block_ids(rng, 40, 17)
+    for h2d in (False, True):
+        reset_stats()
+        _multi_call(devs, gids, cids, h2d, engines)
+        for s in setups:
+            s.oracle_transfer(gids, cids, h2d)
+        for i, dev in enumerate(devs):
+            dev.assert_matches_reference(f"{case} member {i} h2d={h2d}")
+        st = get_stats()
+        assert st["calls"] == len(setups)
+        want = sum(17 * s.num_layers * s.kv_dim * s.chunk for s in setups)
+        assert st["bytes_h2d" if h2d else "bytes_d2h"] == want
+        if case == "alike":
+            assert st["kernel_launches"] == 1
+        elif case == "six_groups":
+            assert st["kernel_launches"] == 2
+        gids, cids = block_ids(rng, 40, 17), block_ids(rng, 40, 17)
+
+
+def test_several_transfers_in_one_call_edge_cases(gpu_device):
+    import torch
+    from flexkv_amd.c_ext import transfer_kv_blocks_multi
+    a = KVSetup(VLLM, 2, 2, 16, 16, 1024, "BLOCKFIRST", seed=41)
+    b = KVSetup(VLLM, 3, 2, 16, 16, 2048, "BLOCKFIRST", seed=42)
+    da, db = a.to_device(gpu_device), b.to_device(gpu_device)
+    transfer_kv_blocks_multi([])
+    none = np.empty(0, dtype=np.int64)
+    _multi_call([da, db], none, none, False)
+    da.assert_matches_reference("no blocks")
+    db.assert_matches_reference("no blocks")
+
+    # the last descriptor's sync flag governs: without it the caller waits on the stream
+    ids, host_ids = np.array([3, 1, 8], dtype=np.int64), np.array([0, 5, 2], dtype=np.int64)
+    _multi_call([da, db], ids, host_ids, False, sync=False)
+    torch.cuda.synchronize()
+    for s in (a, b):
+        s.oracle_transfer(ids, host_ids, False)
+    da.assert_matches_reference("asynchronous")
+    db.assert_matches_reference("asynchronous")
+
+    # an empty member between two others is skipped
+    g = torch.as_tensor(ids)
+    c = torch.as_tensor(host_ids)
+    e = torch.as_tensor(none)
+
+    def call(dev, gi, ci, h2d):
+        s = dev.s
+        return ((gi, dev.ptrs, s.gpu_kv_stride, s.gpu_block_stride, s.gpu_layer_stride, ci,
+                 dev.host, s.cpu_kv_stride, s.cpu_layer_stride, s.cpu_block_stride, s.chunk, 0,
+                 s.num_layers), dict(is_host_to_device=h2d, kv_dim=s.kv_dim, sync=True))
+    transfer_kv_blocks_multi([call(da, c, g, True), call(db, e, e, True), call(db, c, g, True)])
+    for s in (a, b):
+        s.oracle_transfer(host_ids, ids, True)
+    da.assert_matches_reference("empty member in the middle")
+    db.assert_matches_reference("empty member in the middle")
+
+    # both directions in one call are refused before anything moves
+    with pytest.raises(ValueError, match="direction"):
+        transfer_kv_blocks_multi([call(da, g, c, False), call(db, c, g, True)])
+    da.assert_matches_reference("refused call")
+    db.assert_matches_reference("refused call")
