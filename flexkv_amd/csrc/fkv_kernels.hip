@@ -462,8 +462,9 @@ int common_vector_width(const uint64_t *vals, int n) {
 namespace {
 // Checks one job and fills in what the kernel derives from its shape; `total` = its
 // work units (slices, or pieces in packed mode).  FKV_OK with *total == 0: nothing to do.
-int prepare_job(CopyKernelArgs &a, int64_t *total) {
+int prepare_job(CopyKernelArgs &a, int64_t *total, int *grid_pct) {
   *total = 0;
+  *grid_pct = 100;
   if (a.num_blocks <= 0 || a.lk <= 0 || a.chunk_bytes <= 0)
     return FKV_OK;
   if (a.lk > kCopyMaxLK)
@@ -498,13 +499,21 @@ int prepare_job(CopyKernelArgs &a, int64_t *total) {
   if (a.packed) {
     const int64_t piece = (int64_t)kWave * kCopyUnroll;
     *total = (vpp * a.num_blocks + piece - 1) / piece;
+    if (a.packed_grid_pct > 0)
+      *grid_pct = a.packed_grid_pct;
+  } else {
+    // A wavefront has one slice in flight, and the last slice of a chunk is short
+    // when the chunk is no multiple of a slice (18 KiB = 8 + 8 + 2): the bytes in
+    // flight, which set the rate of a launch with few workgroups, shrink to
+    // chunk / (slices x slice).  As many workgroups more make up for it.
+    *grid_pct = (int)((slices * slice_bytes * 100 + a.chunk_bytes - 1) / a.chunk_bytes);
   }
   return FKV_OK;
 }
 
 // Grid, workgroup size, mask and claims of a launch with `total` work units and
 // `bytes` to move; `a` is the (first) job, whose mask, counters and choices count.
-void shape_launch(CopyKernelArgs &a, int64_t total, int64_t bytes, bool any_packed,
+void shape_launch(CopyKernelArgs &a, int64_t total, int64_t bytes, int grid_pct,
                   int num_workgroups, int threads_per_workgroup, int64_t *grid_out,
                   int *threads_out) {
   int threads = threads_per_workgroup;
@@ -515,8 +524,8 @@ void shape_launch(CopyKernelArgs &a, int64_t total, int64_t bytes, bool any_pack
   threads = threads / kWave * kWave;
   const int waves_per_wg = threads / kWave;
   int64_t grid = num_workgroups > 0 ? num_workgroups : 1;
-  if (any_packed && a.packed_grid_pct > 0)
-    grid = (grid * a.packed_grid_pct + 99) / 100;
+  if (grid_pct > 100)
+    grid = (grid * grid_pct + 99) / 100;
   const int64_t useful = (total + waves_per_wg - 1) / waves_per_wg;
   if (grid > useful)
     grid = useful;
@@ -582,12 +591,13 @@ int launch_jobs_vec(const CopyJobs &t, int grid, int threads, size_t lds_bytes,
 int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_workgroup,
                        hipStream_t stream) {
   int64_t total = 0;
-  FKV_TRY(prepare_job(a, &total));
+  int grid_pct = 100;
+  FKV_TRY(prepare_job(a, &total, &grid_pct));
   if (total == 0)
     return FKV_OK;
   int64_t grid = 1;
   int threads = kWave;
-  shape_launch(a, total, (int64_t)a.num_blocks * a.lk * a.chunk_bytes, a.packed != 0,
+  shape_launch(a, total, (int64_t)a.num_blocks * a.lk * a.chunk_bytes, grid_pct,
                num_workgroups, threads_per_workgroup, &grid, &threads);
   const size_t lds_bytes = (size_t)(2 * a.lk + 2 * kCopyIdTile) * sizeof(uint64_t);
   switch (a.vec) {
@@ -606,13 +616,14 @@ int launch_copy_jobs(const CopyKernelArgs *jobs, int njobs, int num_workgroups,
   CopyJobs t{};
   int64_t total = 0, bytes = 0;
   int max_lk = 0;
-  bool any_packed = false;
+  int grid_pct = 100; // the largest any job asks for
   for (int j = 0; j < njobs; ++j) {
     CopyKernelArgs a = jobs[j];
     if (a.vec != jobs[0].vec || a.nt_store != jobs[0].nt_store)
       return fail(FKV_ERR_RUNTIME, "copy kernel: jobs of one launch differ in vector width or store kind");
     int64_t job_total = 0;
-    FKV_TRY(prepare_job(a, &job_total));
+    int job_pct = 100;
+    FKV_TRY(prepare_job(a, &job_total, &job_pct));
     if (job_total == 0)
       continue;
     const int64_t job_bytes = (int64_t)a.num_blocks * a.lk * a.chunk_bytes;
@@ -622,7 +633,7 @@ int launch_copy_jobs(const CopyKernelArgs *jobs, int njobs, int num_workgroups,
     total += job_total;
     bytes += job_bytes;
     max_lk = std::max(max_lk, (int)a.lk);
-    any_packed = any_packed || a.packed;
+    grid_pct = std::max(grid_pct, job_pct);
   }
   if (t.njobs == 0)
     return FKV_OK;
@@ -633,7 +644,7 @@ int launch_copy_jobs(const CopyKernelArgs *jobs, int njobs, int num_workgroups,
   t.job[0].packed_grid_pct = jobs[0].packed_grid_pct;
   int64_t grid = 1;
   int threads = kWave;
-  shape_launch(t.job[0], total, bytes, any_packed, num_workgroups, threads_per_workgroup, &grid,
+  shape_launch(t.job[0], total, bytes, grid_pct, num_workgroups, threads_per_workgroup, &grid,
                &threads);
   const size_t lds_bytes = (size_t)(2 * max_lk + 2 * kCopyIdTile) * sizeof(uint64_t);
   switch (t.job[0].vec) {
