@@ -20,6 +20,8 @@ Beyond BASELINE.json (the rows next to the path):
   mg      layerwise restore of heterogeneous layer groups + sliding-window sidecar
           (DeepSeek-V4-like: 61 layers, two compressed latent groups, an indexer group)
   worker  c0-shaped put/get ops through a transfer worker process (pipe + shared op pool)
+  groups  whole-block ops of a model with three layer groups: one call per group against
+          one call for all; chunk sizes that are no whole number of slices
 """
 from __future__ import annotations
 
@@ -706,6 +708,88 @@ def run_neighbour(torch, device, num_cta, n=2048, count=150):
             lambda: [big_h.copy_(big_d, non_blocking=True) for _ in range(3)])}
 
 
+def run_groups(torch, device, num_cta, reps=30):
+    """Whole-block ops of a model with layer groups of different chunk size (a latent
+    group of 18 KiB chunks, a sliding-window group of 2.25 KiB, an indexer group of
+    2 KiB): one transfer_kv_blocks call per group, as the reference's worker issues
+    them, against one transfer_kv_blocks_multi call; then single groups of chunk
+    sizes around 16 KiB, of which only some are a whole number of 8 KiB slices."""
+    from flexkv_amd.c_ext import get_stats, reset_stats, transfer_kv_blocks, transfer_kv_blocks_multi
+    pool = 1024
+
+    class Group:
+        def __init__(self, layers, chunk):
+            self.layers, self.chunk = layers, chunk
+            self.gpu = [torch.randint(0, 256, (pool, chunk), dtype=torch.uint8, device=device)
+                        for _ in range(layers)]
+            self.host = torch.zeros((pool, layers, chunk), dtype=torch.uint8).pin_memory()
+            self.ptrs = torch.tensor([t.data_ptr() for t in self.gpu], dtype=torch.int64)
+
+        def call(self, gids, cids, h2d, sync):
+            c = self.chunk
+            return ((gids, self.ptrs, pool * c, c, pool * c, cids, self.host, c, c, self.layers * c,
+                     c, 0, self.layers),
+                    dict(transfer_num_cta=num_cta, is_host_to_device=h2d, kv_dim=1, sync=sync))
+
+        def check(self, gids, cids):
+            for l in (0, self.layers - 1):
+                if not torch.equal(self.host[cids, l], self.gpu[l][gids.to(device)].cpu()):
+                    return False
+            return True
+
+    def timed(fn):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        reset_stats()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        dt = (time.perf_counter() - t0) / reps
+        return dt, get_stats()["kernel_launches"] / reps
+
+    res = {"one_op_of_three_groups": {}, "one_group_alone": {}}
+    exact = True
+    groups = [Group(30, 18432), Group(31, 2304), Group(30, 2048)]
+    g = torch.Generator().manual_seed(3)
+    for nblk in (64, 512):
+        gids = torch.randperm(pool, generator=g)[:nblk].contiguous()
+        cids = torch.randperm(pool, generator=g)[:nblk].contiguous()
+        nbytes = sum(nblk * x.layers * x.chunk for x in groups)
+        for h2d in (False, True):
+            def per_group():
+                for i, x in enumerate(groups):
+                    a, k = x.call(gids, cids, h2d, i == len(groups) - 1)
+                    transfer_kv_blocks(*a, **k)
+
+            def together():
+                transfer_kv_blocks_multi([x.call(gids, cids, h2d, True) for x in groups])
+            for name, fn in (("one call per group", per_group), ("one call", together)):
+                dt, launches = timed(fn)
+                if not h2d:
+                    exact = exact and all(x.check(gids, cids) for x in groups)
+                res["one_op_of_three_groups"][
+                    f"{nblk} blocks {'host->GPU' if h2d else 'GPU->host'}, {name}"] = {
+                        "GBps": round(nbytes / dt / 1e9, 2), "us": round(dt * 1e6, 1),
+                        "launches": launches}
+    del groups
+    gids = torch.randperm(pool, generator=g)[:512].contiguous()
+    cids = torch.randperm(pool, generator=g)[:512].contiguous()
+    for chunk in (16384, 18432, 20480, 9216, 12288):
+        x = Group(30, chunk)
+        for h2d in (False, True):
+            a, k = x.call(gids, cids, h2d, True)
+            dt, _ = timed(lambda: transfer_kv_blocks(*a, **k))
+            if not h2d:
+                exact = exact and x.check(gids, cids)
+            res["one_group_alone"][f"30 layers x 512 blocks x {chunk} B "
+                                   f"{'host->GPU' if h2d else 'GPU->host'}"] = \
+                round(512 * 30 * chunk / dt / 1e9, 2)
+        del x
+    res["bit_exact"] = exact
+    return res
+
+
 def run_two_way_putter(torch, device, num_cta):
     """The other process of run_two_way: waits for a line on stdin, puts 94-block
     requests for 3 s and prints its rate."""
@@ -1152,7 +1236,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker", "ssd", "transform", "twoway", "neighbour"])
+    ap.add_argument("--config", default="c1", choices=["c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker", "ssd", "transform", "twoway", "neighbour", "groups"])
     ap.add_argument("--gemm-n", type=int, default=2048, help="neighbour: size of the GEMM")
     ap.add_argument("--role", default="", help=argparse.SUPPRESS)
     ap.add_argument("--shape", default="c0", choices=["c0", "c3"],
@@ -1226,6 +1310,18 @@ def main():
             "higher_is_better": False, "data": "synthetic", "vs_baseline": None,
             "config": {"workload": f"neighbour: {args.gemm_n}^3 bf16 GEMM x150 next to c0-shaped "
                                    "transfers of 512 MiB", "transfer_num_cta": args.num_cta},
+            "results": res}))
+        return
+    if args.config == "groups":
+        res = run_groups(torch, device, args.num_cta)
+        print(json.dumps({
+            "metric": "whole-block op of a multi-group model: GB/s host->GPU", "unit": "GB/s",
+            "value": res["one_op_of_three_groups"]["512 blocks host->GPU, one call"]["GBps"],
+            "n_gpus": 1, "higher_is_better": True, "dtype": "u8", "data": "synthetic",
+            "vs_baseline": None, "bit_exact": res["bit_exact"],
+            "config": {"workload": "groups: 30 layers x 18432 B + 31 x 2304 B + 30 x 2048 B per "
+                                   "block, 64 and 512 blocks; single groups of 9-20 KiB chunks",
+                       "transfer_num_cta": args.num_cta},
             "results": res}))
         return
     if args.config == "twoway":
