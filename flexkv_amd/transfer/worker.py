@@ -738,10 +738,14 @@ class tpGPUCPUTransferWorker(TransferWorkerBase):  # noqa: N801 - the reference'
     def __init__(self, worker_id: int, transfer_conn: Connection, finished_ops_queue,
                  op_buffer_tensor: torch.Tensor, gpu_blocks: List[List[Any]],
                  cpu_blocks: Union[torch.Tensor, PinnedPoolHandle],
-                 gpu_kv_layouts: List[KVCacheLayout], cpu_kv_layout: KVCacheLayout,
+                 gpu_kv_layouts: List[KVCacheLayout],
+                 cpu_kv_layout: Union[KVCacheLayout, MultiGroupBlockLayout],
                  dtype: torch.dtype, tp_group_size: int, use_ce_transfer_h2d: Any = False,
                  use_ce_transfer_d2h: Any = False, transfer_num_cta_h2d: int = 4,
                  transfer_num_cta_d2h: int = 4,
+                 layer_groups: Optional[List[LayerGroupSpec]] = None,
+                 gpu_blocks_per_group: Optional[List[List[List[Any]]]] = None,
+                 gpu_layouts_per_group: Optional[List[List[KVCacheLayout]]] = None,
                  allow_pageable_host: Optional[bool] = None) -> None:
         from ..c_ext import TPTransferThreadGroup
         super().__init__(worker_id, transfer_conn, finished_ops_queue, op_buffer_tensor)
@@ -761,10 +765,23 @@ class tpGPUCPUTransferWorker(TransferWorkerBase):  # noqa: N801 - the reference'
         self.use_ce_transfer_d2h = use_ce_transfer_d2h
         env = global_env()
         self.kv_shared_across_ranks_mode = env.kv_shared_across_ranks_mode
+        self.layer_groups = layer_groups
+        # the byte-flat pool of a multi-group model is block-first by construction
+        self.cpu_is_blockfirst = isinstance(cpu_kv_layout, MultiGroupBlockLayout) \
+            or cpu_kv_layout.type == KVCacheLayoutType.BLOCKFIRST
+        self._ce = dict(ce_segment_threshold=env.ce_segment_threshold, ce_path_opt=env.ce_path_opt,
+                        ce_enable_memcpy2d=env.enable_ce_memcpy2d,
+                        is_blockfirst=self.cpu_is_blockfirst, num_kv_heads=self.num_kv_heads,
+                        ce_gather_threads=env.ce_gather_threads, ce_gather_nt=env.ce_gather_nt)
+        self.tp_group_transfer_groups: Optional[List[dict]] = None
+        if layer_groups is not None and gpu_blocks_per_group is not None \
+                and gpu_layouts_per_group is not None:
+            self._init_tp_multi_group(gpu_blocks_per_group, gpu_layouts_per_group, cpu_kv_layout,
+                                      layer_groups)
+            return
         sz = dtype.itemsize
         per_gpu = [_measured_gpu_strides(self.gpu_blocks[i], lay, lay.tokens_per_block, sz,
                                          self.kv_dim) for i, lay in enumerate(gpu_kv_layouts)]
-        self.cpu_is_blockfirst = cpu_kv_layout.type == KVCacheLayoutType.BLOCKFIRST
         self.cpu_block_stride_in_bytes = cpu_kv_layout.get_block_stride() * sz
         self.chunk_size_in_bytes = cpu_kv_layout.get_chunk_size() * sz
         self._bytes_per_block = self.chunk_size_in_bytes * self.num_layers * self.kv_dim
@@ -782,16 +799,63 @@ class tpGPUCPUTransferWorker(TransferWorkerBase):  # noqa: N801 - the reference'
             len(self.gpu_blocks[0]), self.cpu_tensor.data_ptr(), self.num_layers,
             [s.kv for s in per_gpu], [s.block for s in per_gpu], [s.layer for s in per_gpu],
             [s.chunk for s in per_gpu], [ts[0].device.index for ts in self.gpu_blocks],
-            ce_segment_threshold=env.ce_segment_threshold, ce_path_opt=env.ce_path_opt,
-            ce_enable_memcpy2d=env.enable_ce_memcpy2d, is_blockfirst=self.cpu_is_blockfirst,
-            num_kv_heads=self.num_kv_heads, ce_gather_threads=env.ce_gather_threads,
-            ce_gather_nt=env.ce_gather_nt)
+            **self._ce)
+
+    def _init_tp_multi_group(self, gpu_blocks_per_group, gpu_layouts_per_group,
+                             cpu_kv_layout: MultiGroupBlockLayout, layer_groups) -> None:
+        """One thread group per layer group, each on its byte range of the host
+        block (worker.py:1240-1383): the block holds the groups back to back, once
+        per rank, so every group shares the block stride and the stride between
+        the ranks' regions."""
+        from ..c_ext import TPTransferThreadGroup
+        if not isinstance(cpu_kv_layout, MultiGroupBlockLayout):
+            raise ValueError("layer groups need a MultiGroupBlockLayout host pool")
+        # the imported tensors stay referenced: the thread groups hold addresses only
+        self._group_tensors = [[import_tensor_handles(h) for h in per_gpu]
+                               for per_gpu in gpu_blocks_per_group]
+        block_bytes = cpu_kv_layout.get_block_stride()
+        flat = self.cpu_tensor.view(torch.uint8).view(-1)
+        self.tp_group_transfer_groups = []
+        total = 0
+        for gi, (g, st) in enumerate(zip(layer_groups, cpu_kv_layout.get_group_strides())):
+            per_rank = self._group_tensors[gi]
+            if len(per_rank) != self.num_gpus:
+                raise ValueError(f"layer group {gi}: tensors of {len(per_rank)} GPUs, "
+                                 f"{self.num_gpus} expected")
+            tpb_g = cpu_kv_layout.tokens_per_block // g.compress_ratio
+            strides = [_measured_gpu_strides(per_rank[i], gpu_layouts_per_group[gi][i], tpb_g,
+                                             g.itemsize, self.kv_dim)
+                       for i in range(self.num_gpus)]
+            group = TPTransferThreadGroup(
+                self.num_gpus, [t.data_ptr() for ts in per_rank for t in ts], len(per_rank[0]),
+                flat[st["offset_bytes"]:].data_ptr(), g.num_layers,
+                [s.kv for s in strides], [s.block for s in strides], [s.layer for s in strides],
+                [s.chunk for s in strides], [ts[0].device.index for ts in per_rank], **self._ce)
+            self.tp_group_transfer_groups.append({
+                "tp_thread_group": group, "cpu_kv_stride": st["kv_stride"],
+                "cpu_layer_stride": st["layer_stride"], "cpu_block_stride": block_bytes,
+                "cpu_tp_stride": block_bytes // self.tp_group_size,
+                "cpu_offset_bytes": st["offset_bytes"], "num_layers": g.num_layers,
+                "chunk_size": st["chunk_size"]})
+            total += st["chunk_size"] * g.num_layers * self.kv_dim
+        self._bytes_per_block = total
 
     def _transfer_impl(self, src_block_ids: torch.Tensor, dst_block_ids: torch.Tensor,
                        transfer_type: TransferType) -> None:
         gpu_ids, cpu_ids, h2d = _direction(transfer_type, src_block_ids, dst_block_ids,
                                            "tpGPUCPUTransferWorker")
         if len(gpu_ids) == 0:
+            return
+        num_cta = self.transfer_num_cta_h2d if h2d else self.transfer_num_cta_d2h
+        use_ce = self._engine(self.use_ce_transfer_h2d if h2d else self.use_ce_transfer_d2h)
+        if self.tp_group_transfer_groups is not None:
+            # one call per layer group, all layers of the group (worker.py:1461-1482)
+            for gp in self.tp_group_transfer_groups:
+                gp["tp_thread_group"].tp_group_transfer(
+                    gpu_ids, cpu_ids, gp["cpu_kv_stride"], gp["cpu_layer_stride"],
+                    gp["cpu_block_stride"], gp["cpu_tp_stride"], num_cta, h2d, use_ce, 0,
+                    gp["num_layers"], self.kv_dim, self.num_kv_heads,
+                    self.kv_shared_across_ranks_mode)
             return
         self.tp_transfer_thread_group.tp_group_transfer(
             gpu_ids, cpu_ids, self.cpu_kv_stride_in_bytes, self.cpu_layer_stride_in_bytes,

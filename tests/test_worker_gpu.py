@@ -220,6 +220,59 @@ def test_tp_worker_two_ranks_round_trip(gpu_device, engine, heads, kv_dim, mode,
     monkeypatch.setattr(env, "_ENV", None)
 
 
+@pytest.mark.parametrize("rank_heads,mode", [(1, "sharded"), (1, "rank0_only"), (2, "sharded")])
+def test_tp_worker_layer_groups_round_trip(gpu_device, engine, rank_heads, mode, monkeypatch):
+    """Layer groups behind the tensor-parallel worker (worker.py:1240-1383, 1461-1482
+    of the reference): one thread group per layer group on its byte range of the host
+    block.  One head: both ranks hold the same bytes and share one region of the
+    block; two heads per rank: every rank has its own region, groups back to back
+    inside it."""
+    import flexkv_amd.transfer.env as env
+    monkeypatch.setenv("FLEXKV_KV_SHARED_ACROSS_RANKS_MODE", mode)
+    monkeypatch.setattr(env, "_ENV", None)
+    start, q, pool = engine
+    tp, tpb = 2, 32
+    shared = rank_heads == 1
+    total_heads = 1 if shared else rank_heads * tp
+    groups = [LayerGroupSpec(3, rank_heads, 48, (0, 1, 2), 2, 1),
+              LayerGroupSpec(2, rank_heads, 24, (1, 2), 2, 4),
+              LayerGroupSpec(2, rank_heads, 40, (0, 2), 1, 2)]
+    layouts = [[KVCacheLayout(KVCacheLayoutType.LAYERFIRST, g.num_layers, N_GPU,
+                              tpb // g.compress_ratio, rank_heads, g.head_size, kv_dim=1,
+                              num_kv_heads=total_heads) for _ in range(tp)] for g in groups]
+    cl = MultiGroupBlockLayout(N_CPU, tpb, tuple(groups), kv_dim=1, tp_size=1 if shared else tp)
+    # per group, per rank, per layer
+    tensors = []
+    for gi, g in enumerate(groups):
+        per_rank = []
+        for r in range(tp):
+            gen = torch.Generator().manual_seed(100 + gi if shared else 100 + 10 * r + gi)
+            per_rank.append([torch.randint(0, 256, (N_GPU, tpb // g.compress_ratio, rank_heads,
+                                                    g.head_size * g.itemsize), dtype=torch.uint8,
+                                           generator=gen).to(gpu_device)
+                             for _ in range(g.num_layers)])
+        tensors.append(per_rank)
+    want = [[[t.clone() for t in ts] for ts in per_rank] for per_rank in tensors]
+    handles = [[[TensorSharedHandle(t) for t in ts] for ts in per_rank] for per_rank in tensors]
+    h = start(tpGPUCPUTransferWorker, handles[0], PinnedPoolHandle(cl.kv_shape, torch.uint8),
+              layouts[0], cl, torch.uint8, tp, layer_groups=groups, gpu_blocks_per_group=handles,
+              gpu_layouts_per_group=layouts)
+    src, mid, back = [1, 7, 3, 20], [9, 0, 31, 4], [11, 12, 13, 2]
+    put, get = _op(TransferType.D2H, src, mid, pool), _op(TransferType.H2D, mid, back, pool)
+    h.submit_transfer(put)
+    h.submit_transfer(get)
+    assert _collect(q, 2) == [(put.op_id, True, None), (get.op_id, True, None)]
+    torch.cuda.synchronize()
+    for gi, per_rank in enumerate(tensors):
+        for r, ts in enumerate(per_rank):
+            for l, t in enumerate(ts):
+                assert torch.equal(t[back], want[gi][r][l][src]), (gi, r, l)
+                rest = [b for b in range(N_GPU) if b not in back]
+                assert torch.equal(t[rest], want[gi][r][l][rest]), (gi, r, l, "other blocks")
+    h.shutdown()
+    monkeypatch.setattr(env, "_ENV", None)
+
+
 def _wait_units(fd, timeout=60.0):
     """Blocks like an engine does: one read per unit of the semaphore eventfd."""
     os.set_blocking(fd, True)
