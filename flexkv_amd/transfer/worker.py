@@ -12,8 +12,7 @@ Contract and names follow ``flexkv/transfer/worker.py`` of the reference
 (``TransferWorkerBase`` :120-633, ``WorkerHandle`` :635-707,
 ``GPUCPUTransferWorker`` :709-1097, ``tpGPUCPUTransferWorker`` :1098-1520) and
 ``flexkv/transfer/layerwise.py`` (``LayerwiseTransferWorker`` :69-1059).  What a
-worker of this library does *not* do: compression, remote tiers, GPU memory
-re-mapping controls.
+worker of this library does *not* do: compression, remote tiers.
 
 Host pools.  A worker either receives the pool as a shared-memory tensor and
 registers it with the runtime (the reference's way), or receives a
@@ -47,7 +46,7 @@ from ..layout import (KVCacheLayout, KVCacheLayoutType, LayerGroupSpec, MultiGro
                       multi_group_tables)
 from . import trace
 from .env import global_env
-from .memory_handle import import_tensor_handles
+from .memory_handle import TensorSharedHandle, import_tensor_handles
 from .ops import (LayerwiseTransferOp, TransferOp, TransferType, WorkerLayerwiseTransferOp,
                   WorkerTransferOp, WorkerTransferResult)
 
@@ -517,6 +516,17 @@ def _measured_gpu_strides(tensors: Sequence[torch.Tensor], layout: KVCacheLayout
     return TransferStrides(kv=probed[0], block=probed[1], layer=probed[2], chunk=s.chunk)
 
 
+def _release_imported(handles, tensors) -> int:
+    """Gives back what importing ``handles`` mapped into this process: the tensors
+    are dropped by the caller, mappings opened through the runtime's IPC calls are
+    closed here.  Returns how many tensors were let go."""
+    n = len(tensors)
+    for h in handles:
+        if isinstance(h, TensorSharedHandle):
+            h.release()
+    return n
+
+
 def _direction(transfer_type: TransferType, src: torch.Tensor, dst: torch.Tensor, who: str):
     """(gpu ids, host ids, is_h2d) of a D2H / H2D op."""
     if transfer_type == TransferType.H2D:
@@ -548,6 +558,8 @@ class GPUCPUTransferWorker(TransferWorkerBase):
         torch.cuda.set_device(gpu_device_id)
         self.gpu_device_id = gpu_device_id
         self.cpu_tensor = self._adopt_host_pool(cpu_blocks, "cpu_kv_pool", allow_pageable_host)
+        self._gpu_handles = list(gpu_blocks)
+        self._gpu_block_count = len(gpu_blocks)
         self.gpu_blocks = import_tensor_handles(gpu_blocks)
         self.gpu_blocks_ptrs = _layer_ptrs(self.gpu_blocks)
         self.dtype = dtype
@@ -666,6 +678,36 @@ class GPUCPUTransferWorker(TransferWorkerBase):
             total += s.chunk * g.num_layers * self.kv_dim
         self._bytes_per_block = total
 
+    def _control_suspend_gpu(self, payload: Any) -> int:
+        """The engine is about to free its KV tensors (worker.py:928-946): finish what
+        runs, let go of the tensors and their mappings.  Ops that need them fail
+        until ``resume_gpu`` brings new ones."""
+        if self.group_transfer_params is not None:
+            raise NotImplementedError("GPU hot remap does not support multi-group KV layouts")
+        if not self.gpu_blocks:
+            return 0
+        for lane in self._lanes.values():
+            lane.drain()
+        with torch.cuda.device(self.gpu_device_id):
+            torch.cuda.synchronize()
+        old, self.gpu_blocks = self.gpu_blocks, []
+        self.gpu_blocks_ptrs = torch.zeros_like(self.gpu_blocks_ptrs)
+        handles, self._gpu_handles = self._gpu_handles, []
+        released = _release_imported(handles, old)
+        del old
+        return released
+
+    def _control_resume_gpu(self, gpu_blocks: List[Any]) -> int:
+        """New KV tensors of the same count and shape (worker.py:948-962)."""
+        if self.gpu_blocks:
+            raise RuntimeError("GPU blocks are already registered")
+        if len(gpu_blocks) != self._gpu_block_count:
+            raise ValueError(f"Expected {self._gpu_block_count} GPU blocks, got {len(gpu_blocks)}")
+        self._gpu_handles = list(gpu_blocks)
+        self.gpu_blocks = import_tensor_handles(gpu_blocks)
+        self.gpu_blocks_ptrs = _layer_ptrs(self.gpu_blocks)
+        return len(self.gpu_blocks)
+
     def _transfer_impl(self, src_block_ids: torch.Tensor, dst_block_ids: torch.Tensor,
                        transfer_type: TransferType) -> None:
         from ..c_ext import transfer_kv_blocks, transfer_kv_blocks_multi
@@ -675,6 +717,8 @@ class GPUCPUTransferWorker(TransferWorkerBase):
                                            "GPUCPUTransferWorker")
         if len(gpu_ids) == 0:
             return
+        if not self.gpu_blocks:
+            raise RuntimeError("GPU blocks are suspended: no transfer until resume_gpu")
         use_ce = self._engine(self.use_ce_transfer_h2d if h2d else self.use_ce_transfer_d2h)
         num_cta = self.transfer_num_cta_h2d if h2d else self.transfer_num_cta_d2h
         tail = dict(transfer_num_cta=num_cta, is_host_to_device=h2d, use_ce_transfer=use_ce,
@@ -750,6 +794,8 @@ class tpGPUCPUTransferWorker(TransferWorkerBase):  # noqa: N801 - the reference'
         from ..c_ext import TPTransferThreadGroup
         super().__init__(worker_id, transfer_conn, finished_ops_queue, op_buffer_tensor)
         assert len(gpu_blocks) == tp_group_size
+        self._gpu_handles = [list(h) for h in gpu_blocks]
+        self._gpu_block_counts = [len(h) for h in gpu_blocks]
         self.gpu_blocks = [import_tensor_handles(h) for h in gpu_blocks]
         torch.cuda.set_device(self.gpu_blocks[0][0].device)
         self.cpu_tensor = self._adopt_host_pool(cpu_blocks, "tp_cpu_kv_pool", allow_pageable_host)
@@ -840,12 +886,42 @@ class tpGPUCPUTransferWorker(TransferWorkerBase):  # noqa: N801 - the reference'
             total += st["chunk_size"] * g.num_layers * self.kv_dim
         self._bytes_per_block = total
 
+    def _control_suspend_gpu(self, payload: Any) -> int:
+        """As for the one-GPU worker (worker.py:1385-1406): the thread group is left
+        with null addresses and refuses transfers until ``resume_gpu``."""
+        if self.tp_group_transfer_groups is not None:
+            raise NotImplementedError("GPU hot remap does not support multi-group KV layouts")
+        if not self.gpu_blocks:
+            return 0
+        self.tp_transfer_thread_group.update_gpu_block_ptrs([0] * sum(self._gpu_block_counts))
+        old, self.gpu_blocks = self.gpu_blocks, []
+        handles, self._gpu_handles = self._gpu_handles, []
+        released = sum(_release_imported(h, ts) for h, ts in zip(handles, old))
+        del old
+        return released
+
+    def _control_resume_gpu(self, gpu_blocks: List[List[Any]]) -> int:
+        """New KV tensors for every rank, as many as before (worker.py:1408-1430)."""
+        if self.gpu_blocks:
+            raise RuntimeError("GPU blocks are already registered")
+        counts = [len(h) for h in gpu_blocks]
+        if counts != self._gpu_block_counts:
+            raise ValueError(f"Expected GPU block counts {self._gpu_block_counts}, got {counts}")
+        self._gpu_handles = [list(h) for h in gpu_blocks]
+        imported = [import_tensor_handles(h) for h in gpu_blocks]
+        flat = [t.data_ptr() for ts in imported for t in ts]
+        self.tp_transfer_thread_group.update_gpu_block_ptrs(flat)
+        self.gpu_blocks = imported
+        return len(flat)
+
     def _transfer_impl(self, src_block_ids: torch.Tensor, dst_block_ids: torch.Tensor,
                        transfer_type: TransferType) -> None:
         gpu_ids, cpu_ids, h2d = _direction(transfer_type, src_block_ids, dst_block_ids,
                                            "tpGPUCPUTransferWorker")
         if len(gpu_ids) == 0:
             return
+        if not self.gpu_blocks:
+            raise RuntimeError("GPU blocks are suspended: no transfer until resume_gpu")
         num_cta = self.transfer_num_cta_h2d if h2d else self.transfer_num_cta_d2h
         use_ce = self._engine(self.use_ce_transfer_h2d if h2d else self.use_ce_transfer_d2h)
         if self.tp_group_transfer_groups is not None:

@@ -273,6 +273,81 @@ def test_tp_worker_layer_groups_round_trip(gpu_device, engine, rank_heads, mode,
     monkeypatch.setattr(env, "_ENV", None)
 
 
+@pytest.mark.parametrize("direct_ipc", [False, True])
+def test_suspend_and_resume_gpu_blocks(gpu_device, engine, direct_ipc):
+    """The engine frees its KV tensors and comes back with new ones
+    (worker.py:928-962 of the reference): what was put before is restored into the
+    new tensors; between the two controls an op fails instead of touching memory
+    that is gone."""
+    start, q, pool = engine
+    first = _engine_tensors(gpu_device, 31)
+    want = [t.clone() for t in first]
+    cl = _cpu_layout(KVCacheLayoutType.BLOCKFIRST)
+    h = start(GPUCPUTransferWorker,
+              [TensorSharedHandle(t, force_direct_ipc=direct_ipc) for t in first],
+              PinnedPoolHandle(cl.kv_shape, DT), _gpu_layout(), cl, DT, 0)
+    src, mid, back = [4, 8, 15], [16, 23, 2], [1, 2, 3]
+    put = _op(TransferType.D2H, src, mid, pool)
+    h.submit_transfer(put)
+    assert _collect(q, 1) == [(put.op_id, True, None)]
+    assert h.control("suspend_gpu") == L
+    assert h.control("suspend_gpu") == 0  # nothing left to let go
+    lost = _op(TransferType.H2D, mid, back, pool)
+    h.submit_transfer(lost)
+    assert _collect(q, 1) == [(lost.op_id, False, None)]
+    del first
+    second = [torch.zeros_like(t) for t in want]
+    fresh = [TensorSharedHandle(t, force_direct_ipc=direct_ipc) for t in second]
+    with pytest.raises(RuntimeError, match="Expected 4 GPU blocks"):
+        h.control("resume_gpu", fresh[:2])
+    assert h.control("resume_gpu", fresh) == L
+    with pytest.raises(RuntimeError, match="already registered"):
+        h.control("resume_gpu", fresh)
+    get = _op(TransferType.H2D, mid, back, pool)
+    h.submit_transfer(get)
+    assert _collect(q, 1) == [(get.op_id, True, None)]
+    torch.cuda.synchronize()
+    for l in range(L):
+        assert torch.equal(second[l][:, back], want[l][:, src]), l
+        assert not second[l][:, [b for b in range(N_GPU) if b not in back]].any()
+    h.shutdown()
+
+
+def test_tp_worker_suspend_and_resume_gpu_blocks(gpu_device, engine):
+    """The same for a tensor-parallel group of two ranks (worker.py:1385-1430)."""
+    start, q, pool = engine
+    tp, heads = 2, 4
+    ranks = [_engine_tensors(gpu_device, 40 + r, 2, heads // tp) for r in range(tp)]
+    want = [[t.clone() for t in ts] for ts in ranks]
+    gl = [KVCacheLayout(KVCacheLayoutType.LAYERFIRST, L, N_GPU, T, heads // tp, D, kv_dim=2,
+                        num_kv_heads=heads) for _ in range(tp)]
+    cl = KVCacheLayout(KVCacheLayoutType.BLOCKFIRST, L, N_CPU, T, heads, D, kv_dim=2,
+                       num_kv_heads=heads)
+    h = start(tpGPUCPUTransferWorker, [[TensorSharedHandle(t) for t in ts] for ts in ranks],
+              PinnedPoolHandle(cl.kv_shape, DT), gl, cl, DT, tp)
+    src, mid, back = [2, 9, 5], [30, 1, 17], [20, 21, 22]
+    put = _op(TransferType.D2H, src, mid, pool)
+    h.submit_transfer(put)
+    assert _collect(q, 1) == [(put.op_id, True, None)]
+    assert h.control("suspend_gpu") == tp * L
+    lost = _op(TransferType.H2D, mid, back, pool)
+    h.submit_transfer(lost)
+    assert _collect(q, 1) == [(lost.op_id, False, None)]
+    del ranks
+    second = [[torch.zeros_like(t) for t in ts] for ts in want]
+    with pytest.raises(RuntimeError, match="Expected GPU block counts"):
+        h.control("resume_gpu", [[TensorSharedHandle(t) for t in second[0]]])
+    assert h.control("resume_gpu", [[TensorSharedHandle(t) for t in ts] for ts in second]) == tp * L
+    get = _op(TransferType.H2D, mid, back, pool)
+    h.submit_transfer(get)
+    assert _collect(q, 1) == [(get.op_id, True, None)]
+    torch.cuda.synchronize()
+    for r in range(tp):
+        for l in range(L):
+            assert torch.equal(second[r][l][:, back], want[r][l][:, src]), (r, l)
+    h.shutdown()
+
+
 def _wait_units(fd, timeout=60.0):
     """Blocks like an engine does: one read per unit of the semaphore eventfd."""
     os.set_blocking(fd, True)
