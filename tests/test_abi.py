@@ -101,6 +101,44 @@ def test_empty_transfer_is_a_no_op_without_a_gpu():
     _call(num_layers=0)
 
 
+def _multi(*overs):
+    """transfer_kv_blocks_multi with one descriptor per dict of overrides."""
+    from flexkv_amd.c_ext import transfer_kv_blocks_multi
+    ids = torch.arange(2, dtype=torch.int64)
+    calls = []
+    for over in overs:
+        kw = dict(gpu_block_id_tensor=ids, gpu_tensor_ptrs_tensor=torch.zeros(4, dtype=torch.int64),
+                  gpu_kv_stride_in_bytes=64, gpu_block_stride_in_bytes=16,
+                  gpu_layer_stride_in_bytes=128, cpu_block_id_tensor=ids,
+                  cpu_tensor=torch.zeros(1024, dtype=torch.uint8), cpu_kv_stride_in_bytes=16,
+                  cpu_layer_stride_in_bytes=32, cpu_block_stride_in_bytes=128,
+                  chunk_size_in_bytes=16, start_layer_id=0, num_layers=4)
+        kw.update(over)
+        calls.append(((), kw))
+    transfer_kv_blocks_multi(calls)
+
+
+def test_multi_descriptor_call_checks_every_descriptor_on_the_host():
+    empty = torch.empty(0, dtype=torch.int64)
+    none = dict(gpu_block_id_tensor=empty, cpu_block_id_tensor=empty)
+    _multi()                       # no descriptors, or only empty ones: no device call
+    _multi(none, none, none)
+    # a bad descriptor behind good ones is found before anything runs
+    with pytest.raises(ValueError, match="chunk_size_in_bytes"):
+        _multi(none, dict(none, chunk_size_in_bytes=0))
+    with pytest.raises(RuntimeError, match="Unsupported gpu_block_type: 9"):
+        _multi(none, none, dict(none, gpu_block_type=9))
+    with pytest.raises(ValueError, match="differ in length"):
+        _multi(none, dict(cpu_block_id_tensor=torch.arange(3, dtype=torch.int64)))
+    with pytest.raises(ValueError, match="negative block id"):
+        _multi(none, dict(gpu_block_id_tensor=torch.tensor([0, -1], dtype=torch.int64)))
+    # the C entry point itself refuses a bad array
+    lib = _lib.load()
+    assert lib.fkv_transfer_kv_blocks_multi(None, 2, None) == _lib.FKV_ERR_INVALID_ARG
+    assert b"descriptor array" in lib.fkv_last_error()
+    assert lib.fkv_transfer_kv_blocks_multi(None, 0, None) == _lib.FKV_OK
+
+
 def test_status_codes_map_to_exception_classes():
     lib = _lib.load()
     out = _lib.TPRankPlan()
