@@ -169,6 +169,9 @@ struct fkv_layerwise {
   int counter_id = 0;
   std::thread poller;
   std::atomic<bool> poller_stop{false};
+  // hipError_t of the first device error the poller or a retire saw (0 = none); the
+  // layers behind it were not announced.  Reported, and cleared, by the next call.
+  std::atomic<int> restore_error{0};
 
   // csrc/layerwise.cpp:15-34
   void notify_layers(int start_layer, int layers) const {
@@ -198,6 +201,13 @@ struct fkv_layerwise {
         if (e != hipSuccess) {
           (void)hipGetLastError();
           all = false;
+          if (e != hipErrorNotReady) {
+            // A real device error: the batches behind it will never land.  Stop
+            // without announcing them; the next call on the group reports it.
+            int none = 0;
+            restore_error.compare_exchange_strong(none, (int)e);
+            return;
+          }
         }
       }
       if (all) {
@@ -209,15 +219,50 @@ struct fkv_layerwise {
     }
   }
 
-  // Ends the notification machinery of the previous transfer and frees its
-  // events.  All work of that transfer has completed when this returns.
-  void retire_previous() {
-    if (poller.joinable())
-      poller.join(); // runs until every batch has been announced
+  // Waits for the poller: it ends by itself once every batch has been announced or
+  // a device error has been seen.  Should the streams drain and the poller still
+  // run (a failed stream leaves its events unready for good), it is told to stop.
+  void join_poller() {
+    if (!poller.joinable())
+      return;
     fkv::DeviceGuard restore(-1);
     for (int g = 0; g < num_gpus; ++g) {
       (void)hipSetDevice(device_ids[g]);
-      (void)hipStreamSynchronize(streams[g]);
+      hipError_t e = hipStreamSynchronize(streams[g]);
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        int none = 0;
+        restore_error.compare_exchange_strong(none, (int)e);
+        poller_stop.store(true, std::memory_order_release);
+      }
+    }
+    (void)hipSetDevice(restore.device());
+    // Streams drained without error: every batch event is ready, so the poller
+    // announces what is left and returns.
+    poller.join();
+  }
+
+  // The error of the previous restore, if any, as a status of the current call.
+  int take_restore_error(const char *where) {
+    const int e = restore_error.exchange(0);
+    if (e == 0)
+      return FKV_OK;
+    return fkv::fail(FKV_ERR_RUNTIME, "%s: the previous layerwise restore failed on the device: %s",
+                     where, hipGetErrorString((hipError_t)e));
+  }
+
+  // Ends the notification machinery of the previous transfer and frees its
+  // events.  All work of that transfer has completed when this returns.
+  void retire_previous() {
+    join_poller();
+    fkv::DeviceGuard restore(-1);
+    for (int g = 0; g < num_gpus; ++g) {
+      (void)hipSetDevice(device_ids[g]);
+      hipError_t e = hipStreamSynchronize(streams[g]);
+      if (e != hipSuccess) {
+        int none = 0;
+        restore_error.compare_exchange_strong(none, (int)e);
+      }
     }
     for (auto &b : batches)
       for (int g = 0; g < num_gpus; ++g) {
@@ -473,6 +518,7 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
     return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_transfer: null SWA block id list");
 
   g->retire_previous();
+  FKV_TRY(g->take_restore_error("fkv_layerwise_transfer"));
   g->counter_id = c.counter_id;
   Range range("fkv layerwise%s H2D %d blocks, %d sidecar blocks", g->multi_group ? " multi-group" : "",
               c.num_blocks, c.swa_num_blocks);
@@ -815,15 +861,14 @@ int fkv_layerwise_synchronize(fkv_layerwise *g) {
   clear_error();
   if (!g)
     return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_synchronize: null group");
-  if (g->poller.joinable())
-    g->poller.join();
+  g->join_poller();
   DeviceGuard restore(-1);
   for (int i = 0; i < g->num_gpus; ++i) {
     FKV_HIP_TRY(hipSetDevice(g->device_ids[i]));
     FKV_HIP_TRY(hipStreamSynchronize(g->streams[i]));
   }
   (void)hipSetDevice(restore.device());
-  return FKV_OK;
+  return g->take_restore_error("fkv_layerwise_synchronize");
 }
 
 int fkv_layerwise_batch_times_ms(fkv_layerwise *g, float *out_ms, int32_t capacity,

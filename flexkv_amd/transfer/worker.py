@@ -80,6 +80,15 @@ def _allow_pageable(flag: Optional[bool]) -> bool:
     return bool(int(os.getenv("FKV_WORKER_ALLOW_PAGEABLE_HOST", "0")))
 
 
+def _register_foreign_pools() -> bool:
+    """Whether a host pool that is not pinned is handed to hipHostRegister.  Opt-in
+    (``FKV_HOST_REGISTER=1``): some platforms refuse registration of memory that
+    already exists, and the error such a refusal leaves behind can surface at a
+    later device call.  A pool the worker allocates itself (``PinnedPoolHandle``)
+    or a tensor that is already pinned needs none."""
+    return bool(int(os.getenv("FKV_HOST_REGISTER", "0")))
+
+
 class _SideLane:
     """A second thread of a worker that runs the ops handed to it in order, next to
     the ops the worker runs itself.  It remembers the block ids of its unfinished ops
@@ -178,6 +187,16 @@ class TransferWorkerBase(ABC):
         if isinstance(pool, PinnedPoolHandle):
             return materialize_worker_tensor(pool)
         if pool.is_pinned():
+            return pool
+        if not _register_foreign_pools():
+            if not _allow_pageable(allow_pageable):
+                raise RuntimeError(
+                    f"{label} is neither pinned nor worker-owned: pass a PinnedPoolHandle or a "
+                    "pinned tensor, set FKV_HOST_REGISTER=1 to have the worker register it, or "
+                    "allow_pageable_host=True to move it with the copy engine")
+            logger.info("[worker %s] %s stays pageable: every transfer of this worker goes "
+                        "through the copy engine", self.worker_id, label)
+            self._pageable_host = True
             return pool
         from ..host_buffer import cudaHostRegister
         size_gb = pool.numel() * pool.element_size() / (1024 ** 3)

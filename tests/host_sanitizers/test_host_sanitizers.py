@@ -1,17 +1,19 @@
 """Host code of the library under AddressSanitizer + UndefinedBehaviorSanitizer and
 under ThreadSanitizer.
 
-Two small native drivers (tests/native/) include a host-only translation unit
+Two small native drivers (beside this file) include a host-only translation unit
 of the library each, run it on seeded random inputs against a plain model, and
 are built here with clang's sanitizers (statically linked runtime).  GPU code is
-not involved."""
+not involved, and this folder is kept off the GPU box (it is listed in
+.gpurunignore): sanitizer builds belong on the CPU."""
 import os
 import shutil
 import subprocess
 
 import pytest
 
-ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
 CLANG = shutil.which("clang++", path="/opt/rocm/llvm/bin") or shutil.which("clang++")
 pytestmark = pytest.mark.skipif(CLANG is None, reason="no clang++ for a sanitizer build")
 
@@ -26,7 +28,7 @@ def build_and_run(tmp_path, driver, sanitizer, extra=()):
     cmd = [CLANG, "-std=c++17", "-O1", "-g", *sanitizer, "-fno-omit-frame-pointer",
            "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", "-I" + os.path.join(ROOT, "include"),
            "-I" + os.path.join(ROOT, "flexkv_amd", "csrc"), *extra,
-           os.path.join(ROOT, "tests", "native", driver), "-o", exe, "-pthread", "-ldl"]
+           os.path.join(HERE, driver), "-o", exe, "-pthread", "-ldl"]
     subprocess.run(cmd, check=True, capture_output=True, text=True)
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:verify_asan_link_order=0",
                TSAN_OPTIONS="halt_on_error=1", TMPDIR=str(tmp_path))

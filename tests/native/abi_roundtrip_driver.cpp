@@ -1,8 +1,7 @@
 // A consumer of libfkv_hip.so that knows nothing but include/fkv_transfer.h and
 // the HIP runtime: no Python, no torch.  Moves blocks of a vLLM-shaped cache
 // through every engine of the library and checks each byte against a plain
-// host model.  Also the program that is run with the library's host code built
-// under AddressSanitizer.
+// host model.
 #include <hip/hip_runtime.h>
 #include <sys/eventfd.h>
 #include <unistd.h>

@@ -368,3 +368,58 @@ def test_side_lane_runs_in_order_and_holds_back_ops_that_share_blocks():
     lane.drain()
     assert ran == ["slow", "next"]
     lane.close()
+
+
+class _PoolAdopter:
+    """TransferWorkerBase's host-pool logic without a process, a pipe or a device."""
+
+    def __new__(cls):
+        from worker_fakes import RecordingWorker
+        w = RecordingWorker.__new__(RecordingWorker)
+        w.worker_id = 0
+        return w
+
+
+def test_host_pool_adoption_register_is_opt_in(monkeypatch):
+    """A pageable pool is registered only with FKV_HOST_REGISTER=1; without it the
+    pool stays pageable when that is allowed and is refused otherwise.  The
+    registration itself is replaced by a recorder: no device is involved."""
+    from flexkv_amd import host_buffer
+    calls = []
+    monkeypatch.setattr(host_buffer, "cudaHostRegister", lambda t: calls.append(("reg", t.data_ptr())))
+    monkeypatch.setattr(host_buffer, "cudaHostUnregister",
+                        lambda t: calls.append(("unreg", t.data_ptr())))
+    pool = torch.zeros(1024, dtype=torch.uint8)
+
+    monkeypatch.delenv("FKV_HOST_REGISTER", raising=False)
+    w = _PoolAdopter()
+    with pytest.raises(RuntimeError, match="neither pinned nor worker-owned"):
+        w._adopt_host_pool(pool, "pool", allow_pageable=False)
+    assert w._adopt_host_pool(pool, "pool", allow_pageable=True) is pool
+    assert w._pageable_host and w._engine(False) is True and calls == []
+
+    monkeypatch.setenv("FKV_HOST_REGISTER", "1")
+    w = _PoolAdopter()
+    assert w._adopt_host_pool(pool, "pool", allow_pageable=False) is pool
+    assert not w._pageable_host and w._engine(False) is False
+    assert calls == [("reg", pool.data_ptr())]
+    w.shutdown()
+    assert calls == [("reg", pool.data_ptr()), ("unreg", pool.data_ptr())]
+    w.shutdown()  # idempotent
+    assert len(calls) == 2
+
+
+def test_host_pool_adoption_falls_back_when_registration_is_refused(monkeypatch):
+    from flexkv_amd import host_buffer
+
+    def refuse(t):
+        raise RuntimeError("registration refused")
+    monkeypatch.setattr(host_buffer, "cudaHostRegister", refuse)
+    monkeypatch.setenv("FKV_HOST_REGISTER", "1")
+    pool = torch.zeros(1024, dtype=torch.uint8)
+    w = _PoolAdopter()
+    with pytest.raises(RuntimeError, match="registration refused"):
+        w._adopt_host_pool(pool, "pool", allow_pageable=False)
+    assert w._host_registered == []
+    assert w._adopt_host_pool(pool, "pool", allow_pageable=True) is pool
+    assert w._pageable_host and w._host_registered == []

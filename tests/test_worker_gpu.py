@@ -125,8 +125,9 @@ def test_worker_owned_pinned_pool_round_trip(gpu_device, engine, direct_ipc, eng
 @pytest.mark.parametrize("kind", [KVCacheLayoutType.BLOCKFIRST, KVCacheLayoutType.LAYERFIRST])
 def test_shared_memory_pool_matches_the_oracle(gpu_device, engine, kind):
     """The reference's arrangement: the pool is a shared-memory tensor the engine
-    can read.  The worker registers it; where the runtime refuses that, it keeps it
-    pageable and moves everything with the copy engine."""
+    can read.  The worker does not register foreign memory unless asked to
+    (FKV_HOST_REGISTER=1, not set here): the pool stays pageable and everything moves
+    with the copy engine."""
     from oracle import fkv_oracle as O
     start, q, pool = engine
     tensors = _engine_tensors(gpu_device, 2)
@@ -134,7 +135,7 @@ def test_shared_memory_pool_matches_the_oracle(gpu_device, engine, kind):
     host = torch.zeros(cl.kv_shape, dtype=DT).share_memory_()
     h = start(GPUCPUTransferWorker, [TensorSharedHandle(t) for t in tensors], host, gl, cl, DT, 0,
               allow_pageable_host=True)
-    print("pageable host pool:", h.control("ping")["pageable_host"], flush=True)
+    assert h.control("ping")["pageable_host"] is True
     rng = np.random.default_rng(5)
     gpu_ids = rng.permutation(N_GPU)[:12]
     cpu_ids = rng.permutation(N_CPU)[:12]
