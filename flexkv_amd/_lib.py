@@ -10,7 +10,7 @@ from __future__ import annotations
 import ctypes
 import os
 from ctypes import (POINTER, Structure, c_char_p, c_double, c_float, c_int32, c_int64,
-                    c_size_t, c_uint64, c_void_p)
+                    c_size_t, c_uint32, c_uint64, c_void_p)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libfkv_hip.so")
@@ -147,7 +147,31 @@ class Stats(Structure):
     _fields_ = [("calls", c_uint64), ("bytes_h2d", c_uint64), ("bytes_d2h", c_uint64),
                 ("kernel_launches", c_uint64), ("dma_copies", c_uint64),
                 ("staging_bytes_device", c_uint64), ("staging_bytes_host", c_uint64),
-                ("confined_launches", c_uint64), ("safety_net_ranges", c_uint64)]
+                ("confined_launches", c_uint64), ("safety_net_ranges", c_uint64),
+                ("staged_batches", c_uint64)]
+
+
+class LaunchPolicy(Structure):
+    """fkv_launch_policy: every tunable of the kernel path, per device."""
+    _fields_ = [("xcd_count", c_int32), ("xcd_present_mask", c_uint32),
+                ("arbiter", c_int32),
+                ("d2h_busy_mask", c_uint32), ("h2d_busy_mask", c_uint32),
+                ("d2h_home_mask", c_uint32), ("h2d_home_mask", c_uint32),
+                ("busy_window_ms", c_int32), ("home_min_kb", c_int32),
+                ("d2h_busy_pct", c_int32), ("h2d_busy_pct", c_int32),
+                ("busy_claims_per_wg", c_int32), ("home_claims_per_wg", c_int32),
+                ("all_claims_per_wg", c_int32), ("safety_net_wait_us", c_int32),
+                ("link_gbps_estimate", c_int32),
+                ("d2h_wg_per_cta", c_int32), ("h2d_wg_per_cta", c_int32),
+                ("d2h_wg_threads", c_int32), ("h2d_wg_threads", c_int32),
+                ("packed_grid_pct", c_int32), ("plan_mirror", c_int32),
+                ("fuse_launches", c_int32), ("lane_streams", c_int32),
+                ("staged_restore", c_int32), ("staged_ring", c_int32),
+                ("staged_copy_overhead_us", c_int32), ("staged_overhead_pct", c_int32),
+                ("staged_bridge_kb", c_int32), ("staged_max_mb", c_int32),
+                ("hbm_workgroups", c_int32), ("hbm_wg_threads", c_int32),
+                ("ce_staging_mb", c_int32), ("ce_two_streams", c_int32),
+                ("reserved", c_int32 * 8)]
 
 
 # name -> (restype, argtypes); the complete export list of include/fkv_transfer.h
@@ -221,6 +245,9 @@ SIGNATURES = {
     "fkv_ipc_close": (c_int32, [c_void_p]),
     "fkv_get_stats": (None, [POINTER(Stats)]),
     "fkv_reset_stats": (None, []),
+    "fkv_launch_policy_get": (c_int32, [c_int32, POINTER(LaunchPolicy)]),
+    "fkv_launch_policy_set": (c_int32, [c_int32, POINTER(LaunchPolicy)]),
+    "fkv_launch_policy_reset": (c_int32, [c_int32]),
     "fkv_measure_link_peak": (c_int32, [c_int32, c_size_t, c_int32, c_int32,
                                         POINTER(c_double), POINTER(c_double)]),
 }

@@ -283,6 +283,47 @@ def reset_stats() -> None:
     _L.fkv_reset_stats()
 
 
+def get_launch_policy(device: int = -1) -> Dict[str, int]:
+    """The launch policy of ``device`` (-1: the current one) as a dict: XCD masks of
+    the two directions, workgroup counts, windows, the staged restore's thresholds."""
+    p = _lib.LaunchPolicy()
+    check(_L.fkv_launch_policy_get(int(device), ctypes.byref(p)))
+    return {name: int(getattr(p, name)) for name, _ in p._fields_ if name != "reserved"}
+
+
+def set_launch_policy(device: int = -1, **fields: int) -> Dict[str, int]:
+    """Change fields of the launch policy of ``device``; returns the table as it is
+    afterwards (values are clamped, masks cut to the XCDs the device has)."""
+    p = _lib.LaunchPolicy()
+    check(_L.fkv_launch_policy_get(int(device), ctypes.byref(p)))
+    known = {name for name, _ in p._fields_}
+    for name, value in fields.items():
+        if name not in known or name == "reserved":
+            raise ValueError(f"unknown launch policy field {name!r}")
+        setattr(p, name, int(value))
+    check(_L.fkv_launch_policy_set(int(device), ctypes.byref(p)))
+    return get_launch_policy(device)
+
+
+def reset_launch_policy(device: int = -1) -> None:
+    check(_L.fkv_launch_policy_reset(int(device)))
+
+
+class launch_policy:
+    """``with launch_policy(arbiter=2): ...`` -- fields changed for the block only."""
+
+    def __init__(self, device: int = -1, **fields: int) -> None:
+        self.device, self.fields = device, fields
+
+    def __enter__(self) -> Dict[str, int]:
+        self.saved = get_launch_policy(self.device)
+        return set_launch_policy(self.device, **self.fields)
+
+    def __exit__(self, *exc) -> None:
+        saved = {k: v for k, v in self.saved.items() if k not in ("xcd_count", "xcd_present_mask")}
+        set_launch_policy(self.device, **saved)
+
+
 class SSDIOCTX:
     """Open SSD cache files plus the I/O engine that serves them
     (``csrc/transfer_ssd.h:244-309``, ``csrc/bindings.cpp:785-787``).

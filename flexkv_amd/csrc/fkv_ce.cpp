@@ -192,24 +192,16 @@ hipEvent_t *pingpong_events(int device) {
   return s.pingpong;
 }
 
-size_t staging_cap_bytes() {
-  static const size_t cap = [] {
-    const char *v = std::getenv("FKV_CE_STAGING_MB");
-    long mb = (v && *v) ? std::atol(v) : 1024;
-    if (mb < 1)
-      mb = 1;
-    return (size_t)mb << 20;
-  }();
-  return cap;
+int current_device() {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return device;
 }
-
-bool fan_enabled() {
-  static const bool on = [] {
-    const char *v = std::getenv("FKV_CE_TWO_STREAMS");
-    return !(v && *v == '0');
-  }();
-  return on;
-}
+size_t staging_cap_bytes() { return (size_t)policy_of(current_device()).ce_staging_mb << 20; }
+bool fan_enabled() { return policy_of(current_device()).ce_two_streams != 0; }
 
 // ---- one transfer's state ------------------------------------------------
 struct Job {
@@ -449,18 +441,10 @@ int segment_scatter(const Job &j) {
 int device_staging_copy(const fkv_transfer_desc &d, int it0, int nit, int p0, int np,
                         uint8_t *staging, bool blockfirst, bool to_staging,
                         hipStream_t stream) {
-  static const int kStagingWorkgroups = [] {
-    const char *v = std::getenv("FKV_STAGING_WORKGROUPS");
-    int n = (v && *v) ? std::atoi(v) : 2048;
-    return n > 0 ? n : 2048;
-  }();
-  static const int kStagingThreads = [] {
-    const char *v = std::getenv("FKV_STAGING_THREADS");
-    int n = (v && *v) ? std::atoi(v) : 1024;
-    return n > 0 ? n : 1024;
-  }();
   int device = 0;
   FKV_HIP_TRY(hipGetDevice(&device));
+  const fkv_launch_policy pol = policy_of(device);
+  const int kStagingWorkgroups = pol.hbm_workgroups, kStagingThreads = pol.hbm_wg_threads;
   for (int b0 = 0; b0 < nit; b0 += kCopyMaxLK) {
     const int lk = std::min(kCopyMaxLK, nit - b0);
     const size_t tab = (size_t)lk * 8, ids = (size_t)np * 8;

@@ -218,14 +218,7 @@ int plan_publish(PlanSlot *s, size_t bytes, bool mirror, hipStream_t stream,
   // of another stream that is itself waiting for that stream's previous transfer.
   // With a put stream next to a get stream that tied the start of every get to the
   // end of a put (0.8 ms idle per 3.8 ms transfer).
-  static const bool by_memcpy = [] {
-    const char *v = std::getenv("FKV_PLAN_UPLOAD");
-    return v && !std::strcmp(v, "memcpy");
-  }();
-  if (by_memcpy)
-    FKV_HIP_TRY(hipMemcpyAsync(s->dev, s->host, bytes, hipMemcpyHostToDevice, stream));
-  else
-    FKV_TRY(launch_plan_upload(s->dev, s->host, bytes, stream));
+  FKV_TRY(launch_plan_upload(s->dev, s->host, bytes, stream));
   *device_visible = s->dev;
   return FKV_OK;
 }
@@ -264,10 +257,10 @@ int default_num_cta(bool is_h2d) {
   return is_h2d ? h2d : d2h;
 }
 
-// Measured on MI355X with 4 requested CTAs: GB/s over the link (a plain pinned
-// hipMemcpy reaches 57.0 GPU->host / 57.3 host->GPU) and the slowdown of a kernel
-// running next to the copy (a 2048^3 bf16 GEMM / fused attention / a streaming
-// elementwise kernel):
+// Launch shape of the link-bound kernel.  Measured on MI355X with 4 requested CTAs:
+// GB/s over the link (a plain pinned hipMemcpy reaches 57.0 GPU->host / 57.3
+// host->GPU) and the slowdown of a kernel running next to the copy (a 2048^3 bf16
+// GEMM / fused attention / a streaming elementwise kernel):
 //   host->GPU  16 x  64 lanes : 57.2 GB/s,  1.9x /  1.10x /  1.05x   <- default
 //              24 x  64       : 57.4 GB/s,  2.9x /  1.16x /  1.10x
 //              12 x 1024      : 57.1 GB/s, 16x   /  2.1x  / 11x (stalled until the copy ends)
@@ -275,29 +268,8 @@ int default_num_cta(bool is_h2d) {
 //              24 x  64       : 54.7 GB/s, streaming neighbour 1.9x
 //              12 x 1024      : 56.6 GB/s, streaming neighbour 4.2x
 // So every requested CTA becomes four (host->GPU) or twelve (GPU->host)
-// single-wavefront workgroups.  FKV_{H2D,D2H}_WG_PER_CTA and
-// FKV_{H2D,D2H}_WG_THREADS override this (read once, or on every call when
-// FKV_TUNE_DYNAMIC=1).
-LinkLaunchShape link_launch_shape(bool is_h2d) {
-  static const bool dynamic = env_int("FKV_TUNE_DYNAMIC", 0) != 0;
-  auto read = [](bool h2d) {
-    LinkLaunchShape s;
-    s.workgroups_per_cta =
-        h2d ? env_int("FKV_H2D_WG_PER_CTA", 4) : env_int("FKV_D2H_WG_PER_CTA", 12);
-    s.threads = env_int(h2d ? "FKV_H2D_WG_THREADS" : "FKV_D2H_WG_THREADS", 64);
-    if (s.workgroups_per_cta < 1)
-      s.workgroups_per_cta = 1;
-    // FKV_{H2D,D2H}_XCD_MASK (e.g. 0xf0 / 0x0f) keeps the two directions on disjoint
-    // XCDs when puts and gets run at the same time; default: all XCDs.
-    const char *m = std::getenv(h2d ? "FKV_H2D_XCD_MASK" : "FKV_D2H_XCD_MASK");
-    s.xcd_mask = (m && *m) ? (unsigned)std::strtoul(m, nullptr, 0) & 0xffu : 0xffu;
-    if (s.xcd_mask == 0)
-      s.xcd_mask = 0xffu;
-    return s;
-  };
-  static const LinkLaunchShape fixed[2] = {read(false), read(true)};
-  return dynamic ? read(is_h2d) : fixed[is_h2d ? 1 : 0];
-}
+// single-wavefront workgroups: {h2d,d2h}_wg_per_cta and {h2d,d2h}_wg_threads of the
+// launch policy.
 
 // ---- both directions at once ---------------------------------------------
 // A GPU->host and a host->GPU copy that share XCDs compete for the same
@@ -314,18 +286,18 @@ LinkLaunchShape link_launch_shape(bool is_h2d) {
 // writer that includes XCD 0 loses another 4 GB/s.  With the writer on two XCDs
 // the reader also moves 55 instead of 49 GB/s.  A lone GPU->host transfer loses 2 %
 // on two XCDs and nothing on three (1-3), a lone host->GPU transfer nothing on 4-7,
-// so launches of 8 MiB and more (FKV_HOME_MIN_KB, -1: never) keep to these home
+// so launches of 8 MiB and more (home_min_kb of the launch policy, -1: never) keep to these home
 // XCDs even when the link is idle: a put launched alone and a get that arrives
 // 1 ms later reach 93 GB/s instead of 61, in the other order 80 instead of 72.
 // A direction also counts as busy for a short
-// while after its last launch (FKV_LINK_ARBITER_WINDOW_MS, default 20): with many
+// while after its last launch (busy_window_ms of the launch policy, default 20): with many
 // small requests in flight the other direction is often between two kernels at
 // the moment of a launch, and a full-chip launch would then collide with its next
 // one.  Work recorded on the launching stream itself does not count: it has
 // finished before the new launch starts.  Launches of other processes on the same
 // GPU count through the board of fkv_linkboard.cpp.
-// FKV_LINK_ARBITER=0 switches this off; an
-// explicit FKV_{H2D,D2H}_XCD_MASK takes precedence.
+// arbiter = 0 in the launch policy (FKV_LINK_ARBITER=0) switches this off.  Which
+// XCDs these are on a given device is derived in fkv_policy.cpp.
 namespace {
 constexpr int kActivityRing = 16;
 struct DirectionActivity {
@@ -353,33 +325,13 @@ int64_t steady_ns() {
              std::chrono::steady_clock::now().time_since_epoch())
       .count();
 }
-bool arbiter_enabled() {
-  static const bool on = env_int("FKV_LINK_ARBITER", 1) != 0;
-  return on;
-}
-// The halves of the split are XCDs 0-3 and 4-7: only a device that exposes all
-// eight (an unpartitioned MI355X, 256 CUs) can be split that way.
-bool device_has_eight_xcds(int device) {
-  static std::mutex mu;
-  static std::map<int, bool> known;
-  std::lock_guard<std::mutex> lk(mu);
-  auto it = known.find(device);
-  if (it != known.end())
-    return it->second;
-  int cus = 0;
-  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) {
-    (void)hipGetLastError();
-    cus = 0;
-  }
-  return known[device] = cus >= 8 * 28; // 32 CUs per XCD, some may be fused off
-}
 } // namespace
 
 bool link_direction_busy(int device, bool h2d, hipStream_t launching_stream) {
   DeviceActivity &a = activity_of(device);
   std::lock_guard<std::mutex> lk(a.mu);
   DirectionActivity &d = a.dir[h2d ? 1 : 0];
-  static const int64_t window_ns = (int64_t)env_int("FKV_LINK_ARBITER_WINDOW_MS", 20) * 1000000;
+  const int64_t window_ns = (int64_t)policy_of(device).busy_window_ms * 1000000;
   const int64_t now = steady_ns();
   // launches of other processes on this GPU, as far as they post them
   bool busy = link_board_busy_elsewhere(device, h2d, window_ns);
@@ -399,11 +351,12 @@ bool link_direction_busy(int device, bool h2d, hipStream_t launching_stream) {
 }
 
 void link_direction_mark(int device, bool h2d, hipStream_t stream, int64_t bytes) {
-  if (!arbiter_enabled())
+  const fkv_launch_policy pol = policy_of(device);
+  if (pol.arbiter == 0)
     return;
-  // what other processes get to see: the link is taken for about this long
-  // (45 GB/s: rather a little too long than too short)
-  link_board_post(device, h2d, bytes > 0 ? bytes / 45 : 0);
+  // what other processes get to see: the link is taken for about this long (the
+  // estimate is low on purpose: rather a little too long than too short)
+  link_board_post(device, h2d, bytes > 0 ? bytes / pol.link_gbps_estimate : 0);
   DeviceActivity &a = activity_of(device);
   std::lock_guard<std::mutex> lk(a.mu);
   DirectionActivity &d = a.dir[h2d ? 1 : 0];
@@ -468,48 +421,23 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
   // its default of 4 CTAs is tuned for that hardware.  Here each requested CTA
   // becomes `workgroups_per_cta` small workgroups (see link_launch_shape).
   out->h2d = d.is_host_to_device != 0;
-  const LinkLaunchShape shape = link_launch_shape(out->h2d);
+  const fkv_launch_policy pol = policy_of(device);
   out->workgroups =
       (d.transfer_num_cta > 0 ? d.transfer_num_cta : default_num_cta(out->h2d)) *
-      shape.workgroups_per_cta;
-  out->threads = shape.threads;
-  out->xcd_mask = shape.xcd_mask;
-  out->home_mask = out->busy_mask = 0xffu;
-  out->confined_workgroups = out->home_workgroups = out->workgroups;
+      (out->h2d ? pol.h2d_wg_per_cta : pol.d2h_wg_per_cta);
+  out->threads = out->h2d ? pol.h2d_wg_threads : pol.d2h_wg_threads;
   out->device = device;
-  if (arbiter_enabled() && shape.xcd_mask == 0xffu && device_has_eight_xcds(device)) {
-    static const unsigned h2d_mask = (unsigned)env_int("FKV_ARBITER_H2D_MASK", 0xf0) & 0xffu;
-    static const unsigned d2h_mask = (unsigned)env_int("FKV_ARBITER_D2H_MASK", 0x06) & 0xffu;
-    static const unsigned d2h_home = (unsigned)env_int("FKV_HOME_D2H_MASK", 0x0e) & 0xffu;
-    static const int h2d_pct = std::max(50, env_int("FKV_ARBITER_H2D_PCT", 150));
-    static const int d2h_pct = std::max(5, env_int("FKV_ARBITER_D2H_PCT", 100));
-    out->confined_workgroups =
-        std::max(1, out->workgroups * (out->h2d ? h2d_pct : d2h_pct) / 100);
-    // Which XCDs a launch of this plan keeps to is decided when it is launched (a
-    // layerwise restore launches for tens of milliseconds after its plan was
-    // built): while the other direction is busy GPU->host keeps to two XCDs and
-    // host->GPU to four others; on an idle link large launches keep to their
-    // direction's home XCDs, so that a transfer of the other direction that starts
-    // while they run finds its own XCDs free.  See the note above.
-    out->busy_mask = out->h2d ? (h2d_mask ? h2d_mask : 0xf0u) : (d2h_mask ? d2h_mask : 0x06u);
-    out->home_mask = out->h2d ? out->busy_mask : (d2h_home ? d2h_home : 0x0eu);
-    // on an idle link the home XCDs get no more workgroups than a launch on all XCDs
-    // would: what a copy costs the kernels next to it grows with their number (a
-    // 2048^3 GEMM takes 47 us next to 16 host->GPU workgroups, confined or not, and
-    // 67 us next to 24), and 16 on four XCDs already reach the link rate
-    out->home_workgroups = out->workgroups;
-  }
   // Kernels read the plan from a device copy, which a small kernel uploads first,
   // or where it is, in the pinned slot.  Next to a transfer in the other direction
   // every command on a stream costs idle time, and the upload is one: two threads
   // that put and get 25 MB (100 MB) requests move 88.8 (95.4) instead of 87.0 (94.1)
   // GB/s without it.  A lone transfer is no faster for it and a multi-group restore
   // 1.5 % slower, so the plan is read in place only while the other direction is
-  // busy.  FKV_PLAN_MIRROR=1 / 0: always / never upload.
-  static const int mirror_mode = env_int("FKV_PLAN_MIRROR", -1);
+  // busy.  plan_mirror of the launch policy = 1 / 0: always / never upload.
   const bool mirror_plan =
-      mirror_mode >= 0 ? mirror_mode != 0
-                       : !(out->busy_mask != 0xffu && link_direction_busy(device, !out->h2d, stream));
+      pol.plan_mirror >= 0
+          ? pol.plan_mirror != 0
+          : !(pol.arbiter == 1 && link_direction_busy(device, !out->h2d, stream));
   uint8_t *dv = nullptr;
   int rc = plan_publish(slot, plan_bytes, mirror_plan, stream, &dv);
   if (rc != FKV_OK) {
@@ -553,33 +481,58 @@ CopyKernelArgs plan_job(const KernelPlan &p, int l0, int nl) {
   // such launches get half as many workgroups again.  Host->GPU, 2304-byte chunks:
   // 16 x 64 lanes reach 45 GB/s, 24 x 64 reach 55.8, 32 x 64 reach 56.2; GPU->host:
   // 48 x 64 lanes 50.7 GB/s, 72 x 64 52.5, 96 x 64 53.0.
-  a.packed_grid_pct = 150;
-  a.xcd_mask = p.xcd_mask;
+  a.packed_grid_pct = 150; // replaced by the policy's when the launch is shaped
+  a.xcd_mask = 0;
   a.claim = p.claims ? p.claims + l0 : nullptr; // a launch per first layer at most
   return a;
 }
 
 // Which XCDs, how many workgroups and how many ranges per workgroup a launch of
-// `bytes` gets now; `a` is the (first) job of the launch.
+// `bytes` gets now; `a` is the (first) job of the launch.  Decided when a launch is
+// made, not when its plan is built (a layerwise restore launches for tens of
+// milliseconds after its plan was built): while the other direction is busy
+// GPU->host keeps to its busy XCDs and host->GPU to its own; on an idle link large
+// launches keep to their direction's home XCDs, so that a transfer of the other
+// direction that starts while they run finds its own XCDs free.  On the home XCDs
+// a launch gets no more workgroups than on all XCDs: what a copy costs the kernels
+// next to it grows with their number (a 2048^3 GEMM takes 47 us next to 16 host->GPU
+// workgroups, confined or not, and 67 us next to 24), and 16 on four XCDs already
+// reach the link rate.
+// Ranges per workgroup: next to a transfer in the other direction one each is best
+// (finer ranges shift the balance towards GPU->host and lower the sum: two threads
+// with 25 MB requests 88.9 against 87.5 GB/s).  On an idle link the neighbours are
+// the engine's compute kernels, which slow down single workgroups of a copy, and
+// with one range each the slowest one holds up the launch: a restore next to
+// fused-attention calls moves 37 GB/s with one range per workgroup and 54 GB/s with
+// two.
 int shape_for_now(const KernelPlan &p, int64_t bytes, hipStream_t stream, CopyKernelArgs *a) {
+  const fkv_launch_policy pol = policy_of(p.device);
   int workgroups = p.workgroups;
-  static const int64_t home_min_bytes = (int64_t)env_int("FKV_HOME_MIN_KB", 8192) * 1024;
-  // Ranges per workgroup.  Next to a transfer in the other direction one each is
-  // best (finer ranges shift the balance towards GPU->host and lower the sum: two
-  // threads with 25 MB requests 88.9 against 87.5 GB/s).  On an idle link the
-  // neighbours are the engine's compute kernels, which slow down single
-  // workgroups of a copy, and with one range each the slowest one holds up the
-  // launch: a restore next to fused-attention calls moves 37 GB/s with one range
-  // per workgroup and 54 GB/s with two.
-  static const int home_claims = std::max(1, env_int("FKV_HOME_CLAIMS_PER_WORKGROUP", 2));
-  if (p.busy_mask != 0xffu && link_direction_busy(p.device, !p.h2d, stream)) {
-    a->xcd_mask = p.busy_mask;
-    workgroups = p.confined_workgroups;
+  const uint32_t all = pol.xcd_present_mask;
+  const uint32_t busy_mask = p.h2d ? pol.h2d_busy_mask : pol.d2h_busy_mask;
+  const uint32_t home_mask = p.h2d ? pol.h2d_home_mask : pol.d2h_home_mask;
+  const int busy_workgroups =
+      std::max(1, p.workgroups * (p.h2d ? pol.h2d_busy_pct : pol.d2h_busy_pct) / 100);
+  a->xcd_present = all;
+  a->safety_net_wait_us = pol.safety_net_wait_us;
+  a->packed_grid_pct = pol.packed_grid_pct;
+  a->xcd_mask = 0;
+  a->claims_per_wg = pol.all_claims_per_wg;
+  if (pol.arbiter == 3) {
+    // tests: a mask that names no XCD of the device, every workgroup but the
+    // safety net leaves
+    a->xcd_mask = (all + 1u) & ~all ? ((all + 1u) & ~all) : 0x8000u;
     a->claims_per_wg = 1;
-  } else if (p.home_mask != 0xffu && home_min_bytes >= 0 && bytes >= home_min_bytes) {
-    a->xcd_mask = p.home_mask;
-    workgroups = p.home_workgroups;
-    a->claims_per_wg = home_claims;
+  } else if (pol.arbiter == 2 ||
+             (pol.arbiter == 1 && busy_mask != all &&
+              link_direction_busy(p.device, !p.h2d, stream))) {
+    a->xcd_mask = busy_mask;
+    workgroups = busy_workgroups;
+    a->claims_per_wg = pol.busy_claims_per_wg;
+  } else if (pol.arbiter == 1 && home_mask != all && pol.home_min_kb >= 0 &&
+             bytes >= (int64_t)pol.home_min_kb * 1024) {
+    a->xcd_mask = home_mask;
+    a->claims_per_wg = pol.home_claims_per_wg;
   }
   return workgroups;
 }
@@ -610,14 +563,13 @@ int kernel_plans_launch(const KernelPlan *const *plans, const int *layer_offsets
                         const int *num_layers, int count, hipStream_t stream) {
   // One launch for all of them when they can share one: same direction, device,
   // vector width and launch shape, each range within one LDS table.
-  static const bool fuse = env_int("FKV_FUSE_LAUNCHES", 1) != 0;
+  const bool fuse = policy_of(plans[0]->device).fuse_launches != 0;
   bool together = fuse && count >= 2 && count <= kCopyMaxJobs;
   for (int i = 0; i < count && together; ++i) {
     const KernelPlan &p = *plans[i], &q = *plans[0];
     together = p.h2d == q.h2d && p.device == q.device && p.vec == q.vec &&
                p.threads == q.threads && p.workgroups == q.workgroups &&
-               p.xcd_mask == q.xcd_mask && p.busy_mask == q.busy_mask &&
-               p.home_mask == q.home_mask && layer_offsets[i] >= 0 && num_layers[i] > 0 &&
+               layer_offsets[i] >= 0 && num_layers[i] > 0 &&
                layer_offsets[i] + num_layers[i] <= p.num_layers &&
                num_layers[i] * p.kv_dim <= kCopyMaxLK;
   }
@@ -741,6 +693,7 @@ void fkv_get_stats(fkv_stats *out) {
   // a device counter: only worth a device call once a confined launch has been made
   out->safety_net_ranges =
       out->confined_launches ? fkv::safety_net_ranges_of_current_device() : 0;
+  out->staged_batches = s.staged_batches.load();
 }
 void fkv_reset_stats(void) {
   fkv::Stats &s = fkv::stats();
@@ -752,6 +705,7 @@ void fkv_reset_stats(void) {
   s.staging_bytes_device = 0;
   s.staging_bytes_host = 0;
   s.confined_launches = 0;
+  s.staged_batches = 0;
 }
 
 } // extern "C"
@@ -820,7 +774,7 @@ struct DeviceLanes {
   bool tried = false, ok = false;
   Lane dir[2]; // [0] GPU->host, [1] host->GPU
 };
-// FKV_LANE_STREAMS: 1 always, 0 never; unset: synchronous calls, once kernel
+// lane_streams of the launch policy (FKV_LANE_STREAMS): 1 always, 0 never; -1: synchronous calls, once kernel
 // transfers of a device have been issued on more than two different streams (a
 // stream per request is then likely, and with it both directions on every
 // hardware queue).  Asynchronous calls stay on the caller's stream unless asked:
@@ -829,10 +783,7 @@ struct DeviceLanes {
 // stream pays for them (125 transfers of 25 MB per direction: 76 instead of
 // 89 GB/s).
 bool lanes_wanted(int device, hipStream_t caller_stream, bool synchronous) {
-  static const int mode = [] {
-    const char *v = std::getenv("FKV_LANE_STREAMS");
-    return (v && *v) ? (std::strcmp(v, "0") != 0 ? 1 : 0) : -1;
-  }();
+  const int mode = fkv::policy_of(device).lane_streams;
   if (mode >= 0)
     return mode == 1;
   if (!synchronous)

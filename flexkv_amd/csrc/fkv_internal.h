@@ -63,7 +63,8 @@ constexpr unsigned kTimingEventNoFence = hipEventDisableSystemFence;
 // ---- counters -----------------------------------------------------------
 struct Stats {
   std::atomic<uint64_t> calls{0}, bytes_h2d{0}, bytes_d2h{0}, kernel_launches{0},
-      dma_copies{0}, staging_bytes_device{0}, staging_bytes_host{0}, confined_launches{0};
+      dma_copies{0}, staging_bytes_device{0}, staging_bytes_host{0}, confined_launches{0},
+      staged_batches{0};
 };
 Stats &stats();
 
@@ -139,7 +140,9 @@ struct CopyKernelArgs {
   int32_t nt_store; // 1: nontemporal stores (destination in HBM), 0: plain (pinned host)
   int32_t packed;   // set by launch_copy_kernel: chunks shorter than a slice, see the kernel
   int32_t packed_grid_pct; // workgroups to launch in packed mode, percent of the request (0 = 100)
-  uint32_t xcd_mask; // bit k: workgroups that run on XCD k take part; 0 or 0xff = all
+  uint32_t xcd_mask; // bit k: workgroups that run on XCD k take part; 0 = all
+  uint32_t xcd_present;        // host side: the XCDs of the device (0 = eight, ids 0-7)
+  int32_t safety_net_wait_us;  // confined launches, see the kernel (0 = 50)
   // Launches whose workgroups claim their work: a 64-bit counter in device memory
   // (high half: `epoch` of the launch that owns the count, low half: ranges handed
   // out of `num_claims`, set by launch_copy_kernel).  The counter need not be clean:
@@ -148,7 +151,8 @@ struct CopyKernelArgs {
   uint64_t *claim;
   uint32_t num_claims;
   uint32_t epoch; // set by launch_copy_kernel: a number no other launch in flight has
-  int32_t claims_per_wg; // confined launches: ranges per working workgroup (0 = 1)
+  int32_t claims_per_wg; // ranges per working workgroup: confined launches (0 = 1), and
+                         // launches on all XCDs that have counters (0 = fixed shares)
 };
 constexpr int kCopyBlockThreads = 1024;  // largest workgroup the kernel is built for
 constexpr int kCopyUnroll = 8;           // vector accesses in flight per lane
@@ -173,13 +177,10 @@ uint64_t safety_net_ranges_of_current_device();
 // Copies `bytes` (rounded up to 16) from a pinned, device-mapped host buffer to
 // device memory with a small kernel on `stream`.
 int launch_plan_upload(void *device_dst, const void *pinned_src, size_t bytes, hipStream_t stream);
-// Launch shape of the link-bound kernel for one direction.
-struct LinkLaunchShape {
-  int workgroups_per_cta; // workgroups launched per requested CTA
-  int threads;            // lanes per workgroup
-  unsigned xcd_mask;      // XCD slots the launch is confined to (0xff = all)
-};
-LinkLaunchShape link_launch_shape(bool is_h2d);
+// The XCDs of the current device, by a probe kernel on the null stream (blocking).
+int probe_xcds(uint32_t *present_mask);
+// The launch policy of `device` (a copy; built on first use, see fkv_policy.cpp).
+fkv_launch_policy policy_of(int device);
 // Widest vector width (bytes) that divides every value in `vals`.
 int common_vector_width(const uint64_t *vals, int n);
 
@@ -216,13 +217,6 @@ struct KernelPlan {
   int kv_dim = 1, num_layers = 0, num_blocks = 0;
   int64_t chunk_size = 0, gpu_block_stride = 0, cpu_block_stride = 0;
   int workgroups = 1, threads = 64;
-  unsigned xcd_mask = 0xff;  // XCDs every launch is restricted to by configuration
-  // XCDs and workgroups of a launch that finds the other direction busy, and of a
-  // launch that moves a lot while the link is idle (0xff: all XCDs with `workgroups`)
-  unsigned busy_mask = 0xff;
-  int confined_workgroups = 1;
-  unsigned home_mask = 0xff;
-  int home_workgroups = 1;
   int device = 0;
   uint64_t *claims = nullptr; // a claim counter per layer of the plan, device memory
 };
@@ -255,6 +249,45 @@ int choose_engine(const fkv_transfer_desc &d, int *use_ce, double *kernel_s, dou
 int device_staging_copy(const fkv_transfer_desc &d, int it0, int nit, int p0, int np,
                         uint8_t *staging, bool blockfirst, bool to_staging,
                         hipStream_t stream);
+
+// ---- restore through the copy engines (fkv_staged_restore.cpp) ---------------
+// Staging buffers of one (layer group, GPU); they outlive the calls.
+struct StagedRing {
+  std::vector<uint8_t *> buf;
+  size_t cap = 0;
+  std::vector<hipEvent_t> copied, freed; // per buffer: copies landed / scatter done
+  std::vector<bool> used;
+  int next = 0;
+  void release(); // frees everything; the device must have finished with the buffers
+};
+// What one call derives for one (layer group, GPU).
+struct StagedPlan {
+  struct Seg {
+    int64_t first_id; // first host block of the run
+    int32_t rows;     // host blocks it spans (holes read along included)
+    int32_t row0;     // staging row of the first
+  };
+  bool usable = false;
+  std::vector<Seg> segs;
+  int32_t total_rows = 0;
+  int kind = 0; // chunks of a host block that are adjacent: 0 all of a batch, 1 K and V of a layer, 2 none
+  int max_lk = 0, batch_layers = 0, kv_dim = 1, num_blocks = 0;
+  int64_t chunk = 0, cpu_kv_stride = 0, cpu_layer_stride = 0, cpu_block_stride = 0;
+  const uint8_t *host0 = nullptr;
+  PlanSlot *slot = nullptr;
+  const uint64_t *base_tables = nullptr; // device-visible, [ring buffers][max_lk]
+  const int64_t *stage_rows = nullptr;   // device-visible, [num_blocks]
+};
+// Decides whether the restore described by `d` (all its layers, in batches of
+// `batch_layers`) goes through the copy engines on the current device and, if so,
+// sizes the ring and uploads the tables on `scatter_stream`.  FKV_OK with
+// out->usable == false: use the kernel path.
+int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &ring,
+                      hipStream_t scatter_stream, StagedPlan *out);
+// Layers [l0, l0 + nl) of the plan: copies on `dma_stream`, scatter on `scatter_stream`.
+int staged_launch(const StagedPlan &sp, StagedRing &ring, const KernelPlan &kp, int l0, int nl,
+                  hipStream_t dma_stream, hipStream_t scatter_stream);
+void staged_plan_release(StagedPlan *sp, hipStream_t scatter_stream);
 
 int default_num_cta(bool is_h2d);
 int validate(const fkv_transfer_desc &d);

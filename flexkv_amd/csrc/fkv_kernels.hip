@@ -65,11 +65,11 @@ template <> struct VecType<4>  { typedef unsigned int type; };
 template <> struct VecType<2>  { typedef unsigned short type; };
 template <> struct VecType<1>  { typedef unsigned char type; };
 
-// Id of the XCD this wavefront runs on (0-7).
+// Id of the XCD this wavefront runs on (the low four bits of the register).
 __device__ __forceinline__ uint32_t xcd_of_this_wave() {
   uint32_t v;
   asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(v));
-  return v & 7u;
+  return v & 15u;
 }
 
 template <typename V, bool NT> __device__ __forceinline__ void put(V v, V *p) {
@@ -132,11 +132,13 @@ struct Shares {
   uint32_t taken;      // lane 0 of the safety net: ranges it has claimed itself
   bool confined, dynamic, first, safety_net;
 
+  long long wait_ticks; // of the 100 MHz clock, before the safety net looks at the counter
+
   __device__ __forceinline__ Shares(const CopyKernelArgs &a)
       : claim(reinterpret_cast<unsigned long long *>(a.claim)), num_claims(a.num_claims),
-        xcd_mask(a.xcd_mask & 0xffu), epoch(a.epoch), next_claim(0), taken(0),
-        confined((a.xcd_mask & 0xffu) != 0xffu), dynamic(a.num_claims != 0), first(true),
-        safety_net(false) {}
+        xcd_mask(a.xcd_mask), epoch(a.epoch), next_claim(0), taken(0),
+        confined(a.xcd_mask != 0), dynamic(a.num_claims != 0), first(true),
+        safety_net(false), wait_ticks((long long)a.safety_net_wait_us * 100) {}
 
   // The counter of a launch need not be clean: it counts for this launch from the
   // moment its high half holds the launch's number, and whoever finds another
@@ -164,7 +166,7 @@ struct Shares {
         return false;
       if (threadIdx.x == 0) {
         const long long t0 = wall_clock64();
-        while (wall_clock64() - t0 < 5000) // 50 us of the constant 100 MHz clock
+        while (wall_clock64() - t0 < wait_ticks) // bounded: the constant 100 MHz clock
           __builtin_amdgcn_s_sleep(32);
         *s_claim = (uint32_t)adopt();
       }
@@ -424,6 +426,31 @@ __global__ void fkv_wait_kernel(long long ticks, int *sink) {
 }
 } // namespace
 
+namespace {
+__global__ void fkv_xcd_probe_kernel(uint32_t *present) {
+  if (threadIdx.x == 0)
+    atomicOr(present, 1u << xcd_of_this_wave());
+}
+} // namespace
+
+int probe_xcds(uint32_t *present_mask) {
+  uint32_t *d = nullptr;
+  *present_mask = 0;
+  FKV_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&d), sizeof(uint32_t)));
+  hipError_t e = hipMemset(d, 0, sizeof(uint32_t));
+  if (e == hipSuccess) {
+    // far more workgroups than XCDs: the dispatcher deals them out round-robin
+    hipLaunchKernelGGL(fkv_xcd_probe_kernel, dim3(1024), dim3(64), 0, nullptr, d);
+    e = hipGetLastError();
+  }
+  if (e == hipSuccess)
+    e = hipMemcpy(present_mask, d, sizeof(uint32_t), hipMemcpyDeviceToHost);
+  (void)hipFree(d);
+  if (e != hipSuccess)
+    return fail(FKV_ERR_RUNTIME, "XCD probe failed: %s", hipGetErrorString(e));
+  return FKV_OK;
+}
+
 uint64_t safety_net_ranges_of_current_device() {
   unsigned long long v = 0;
   if (hipMemcpyFromSymbol(&v, HIP_SYMBOL(g_safety_net_ranges), sizeof(v)) != hipSuccess) {
@@ -490,12 +517,6 @@ int prepare_job(CopyKernelArgs &a, int64_t *total, int *grid_pct) {
   // id tile with 32 bits).
   const int64_t vpp = a.chunk_bytes / a.vec * a.lk;
   a.packed = (a.chunk_bytes < slice_bytes && vpp * kCopyIdTile <= (int64_t)UINT32_MAX) ? 1 : 0;
-  static const bool no_pack = [] {
-    const char *v = std::getenv("FKV_COPY_NO_PACK");
-    return v && *v == '1';
-  }();
-  if (no_pack)
-    a.packed = 0;
   if (a.packed) {
     const int64_t piece = (int64_t)kWave * kCopyUnroll;
     *total = (vpp * a.num_blocks + piece - 1) / piece;
@@ -531,9 +552,12 @@ void shape_launch(CopyKernelArgs &a, int64_t total, int64_t bytes, int grid_pct,
     grid = useful;
   if (grid < 1)
     grid = 1;
-  a.xcd_mask &= 0xffu;
-  if (a.xcd_mask == 0 || !a.claim)
-    a.xcd_mask = 0xffu;
+  // 0 = every XCD; a mask needs claim counters and must leave some XCD of the device out
+  const uint32_t present = a.xcd_present ? a.xcd_present : 0xffu;
+  if (!a.claim || (a.xcd_mask & present) == present)
+    a.xcd_mask = 0;
+  if (a.safety_net_wait_us <= 0)
+    a.safety_net_wait_us = 50;
   a.num_claims = 0;
   // a number for this launch that no counter can hold by accident for long: counters
   // are zero at first, and 2^32 - 1 launches pass before a number comes back
@@ -541,24 +565,22 @@ void shape_launch(CopyKernelArgs &a, int64_t total, int64_t bytes, int grid_pct,
   do {
     a.epoch = launches.fetch_add(1, std::memory_order_relaxed) + 1;
   } while (a.epoch == 0);
-  if (a.xcd_mask != 0xffu) {
+  if (a.xcd_mask != 0) {
     // `claims_per_wg` ranges per working workgroup (the caller's choice, 1 if it
-    // makes none); `grid` working workgroups need grid / popcount(mask) rounds of 8.
+    // makes none); `grid` working workgroups need grid / (selected XCDs) rounds over
+    // all XCDs of the device.
     const int per_wg = a.claims_per_wg > 0 ? a.claims_per_wg : 1;
     a.num_claims = (uint32_t)std::min<int64_t>(grid * per_wg, total);
-    const int per_round = __builtin_popcount(a.xcd_mask);
-    grid = (grid + per_round - 1) / per_round * 8;
-  } else if (a.claim) {
+    const int per_round = std::max(1, __builtin_popcount(a.xcd_mask & present));
+    grid = (grid + per_round - 1) / per_round * __builtin_popcount(present);
+  } else if (a.claim && a.claims_per_wg > 0) {
     // All XCDs, some of which may be busy with the other direction (a transfer of
     // another stream or process that started later).  With several ranges per
-    // workgroup (FKV_CLAIMS_PER_WORKGROUP=8) the workgroups there take fewer of them:
+    // workgroup (all_claims_per_wg of the launch policy, e.g. 8) the workgroups there
+    // take fewer of them:
     // a restore that stays on all XCDs next to a put loop moves 23-24 instead of
     // 16-17 GB/s.  Off by default: alone, the same restore loses 2 % to the claims.
-    static const int per_wg = [] {
-      const char *v = std::getenv("FKV_CLAIMS_PER_WORKGROUP");
-      const int n = v && *v ? std::atoi(v) : 0;
-      return n < 0 ? 0 : n;
-    }();
+    const int per_wg = a.claims_per_wg;
     // ranges of 128 KiB at least: a claim costs a round trip to device memory
     a.num_claims = (uint32_t)std::min<int64_t>(std::min<int64_t>(grid * per_wg, total),
                                                 bytes / (128 * 1024));
@@ -566,7 +588,7 @@ void shape_launch(CopyKernelArgs &a, int64_t total, int64_t bytes, int grid_pct,
       a.num_claims = 0;
   }
   stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);
-  if (a.xcd_mask != 0xffu)
+  if (a.xcd_mask != 0)
     stats().confined_launches.fetch_add(1, std::memory_order_relaxed);
   *grid_out = grid;
   *threads_out = threads;
@@ -641,6 +663,8 @@ int launch_copy_jobs(const CopyKernelArgs *jobs, int njobs, int num_workgroups,
   t.job[0].xcd_mask = jobs[0].xcd_mask;
   t.job[0].claim = jobs[0].claim;
   t.job[0].claims_per_wg = jobs[0].claims_per_wg;
+  t.job[0].xcd_present = jobs[0].xcd_present;
+  t.job[0].safety_net_wait_us = jobs[0].safety_net_wait_us;
   t.job[0].packed_grid_pct = jobs[0].packed_grid_pct;
   int64_t grid = 1;
   int threads = kWave;

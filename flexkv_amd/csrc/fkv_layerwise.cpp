@@ -34,6 +34,7 @@
 
 #include <atomic>
 #include <cstring>
+#include <map>
 #include <memory>
 #include <thread>
 
@@ -125,6 +126,7 @@ struct Lane {
   int kv_dim = 1;
   bool used = false;
   std::vector<fkv::KernelPlan> plans; // per GPU, kernel path only
+  std::vector<fkv::StagedPlan> staged; // per GPU: usable where this call goes through the copy engines
 };
 
 struct Item {
@@ -149,6 +151,11 @@ struct fkv_layerwise {
   MemberTable swa_members;
   std::vector<int> device_ids;
   std::vector<hipStream_t> streams;
+  // Restores through the copy engines (fkv_staged_restore.cpp): a second stream per
+  // GPU for the copies, created on first use, and the staging buffers by
+  // (lane, GPU), kept from call to call.
+  std::vector<hipStream_t> dma_streams;
+  std::map<std::pair<int, int>, fkv::StagedRing> rings;
   fkv_ce_config ce{};
 
   std::vector<int32_t> eventfds; // [num_counters][tp_size][num_layers]
@@ -264,6 +271,11 @@ struct fkv_layerwise {
         restore_error.compare_exchange_strong(none, (int)e);
       }
     }
+    for (int g = 0; g < (int)dma_streams.size(); ++g)
+      if (dma_streams[g]) {
+        (void)hipSetDevice(device_ids[g]);
+        (void)hipStreamSynchronize(dma_streams[g]);
+      }
     for (auto &b : batches)
       for (int g = 0; g < num_gpus; ++g) {
         (void)hipSetDevice(device_ids[g]);
@@ -677,6 +689,24 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
           break;
         (void)hipSetDevice(g->device_ids[i]);
         rc = kernel_plan_build(d, g->streams[i], &lane.plans[i]);
+        // Few runs of host blocks: the lane's batches go through the copy engines
+        // and a staging buffer instead (the plan still gives the device side).
+        if (rc == FKV_OK) {
+          if ((int)g->dma_streams.size() < g->num_gpus)
+            g->dma_streams.resize(g->num_gpus, nullptr);
+          lane.staged.resize(g->num_gpus);
+          const int lane_index = (int)(&lane - lanes.data());
+          rc = staged_plan_build(d, g->multi_group ? 1 : c.layer_granularity,
+                                 g->rings[{lane_index, i}], g->streams[i], &lane.staged[i]);
+          if (rc == FKV_OK && lane.staged[i].usable && !g->dma_streams[i]) {
+            hipError_t e = hipStreamCreateWithFlags(&g->dma_streams[i], hipStreamNonBlocking);
+            if (e != hipSuccess) {
+              (void)hipGetLastError();
+              g->dma_streams[i] = nullptr;
+              staged_plan_release(&lane.staged[i], g->streams[i]); // kernel path then
+            }
+          }
+        }
       }
     }
   for (int b = 0; b < num_batches && rc == FKV_OK; ++b) {
@@ -687,25 +717,33 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
         // the members of one batch go out together: up to kCopyMaxJobs per launch
         const KernelPlan *plans[kCopyMaxJobs];
         int first[kCopyMaxJobs], count[kCopyMaxJobs];
-        for (size_t k = 0; k < batch.items.size() && rc == FKV_OK; k += kCopyMaxJobs) {
-          const int n = (int)std::min<size_t>(kCopyMaxJobs, batch.items.size() - k);
+        // items of lanes that go through the copy engines first, the rest by kernel
+        std::vector<const Item *> by_kernel;
+        for (const Item &it : batch.items) {
+          Lane &lane = lanes[it.lane];
+          if (rc == FKV_OK && !lane.staged.empty() && lane.staged[i].usable)
+            rc = staged_launch(lane.staged[i], g->rings[{it.lane, i}], lane.plans[i],
+                               it.start_layer, it.layers, g->dma_streams[i], g->streams[i]);
+          else
+            by_kernel.push_back(&it);
+        }
+        for (size_t k = 0; k < by_kernel.size() && rc == FKV_OK; k += kCopyMaxJobs) {
+          const int n = (int)std::min<size_t>(kCopyMaxJobs, by_kernel.size() - k);
           for (int j = 0; j < n; ++j) {
-            const Item &it = batch.items[k + j];
+            const Item &it = *by_kernel[k + j];
             plans[j] = &lanes[it.lane].plans[i];
             first[j] = it.start_layer;
             count[j] = it.layers;
           }
           rc = kernel_plans_launch(plans, first, count, n, g->streams[i]);
-          if (rc != FKV_OK)
-            break;
-          for (int j = 0; j < n; ++j) {
-            const Item &it = batch.items[k + j];
-            const Lane &lane = lanes[it.lane];
-            stats().calls.fetch_add(1, std::memory_order_relaxed);
-            stats().bytes_h2d.fetch_add((uint64_t)lane.num_blocks * it.layers * lane.kv_dim *
-                                            (uint64_t)lane.src->chunk_sizes[i],
-                                        std::memory_order_relaxed);
-          }
+        }
+        for (size_t k = 0; k < batch.items.size() && rc == FKV_OK; ++k) {
+          const Item &it = batch.items[k];
+          const Lane &lane = lanes[it.lane];
+          stats().calls.fetch_add(1, std::memory_order_relaxed);
+          stats().bytes_h2d.fetch_add((uint64_t)lane.num_blocks * it.layers * lane.kv_dim *
+                                          (uint64_t)lane.src->chunk_sizes[i],
+                                      std::memory_order_relaxed);
         }
       }
       for (size_t k = 0; !direct && k < batch.items.size() && rc == FKV_OK; ++k) {
@@ -729,11 +767,15 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
     for (int i = 0; i < (int)lane.plans.size(); ++i) {
       (void)hipSetDevice(g->device_ids[i]);
       kernel_plan_release(&lane.plans[i], g->streams[i]);
+      if (i < (int)lane.staged.size())
+        staged_plan_release(&lane.staged[i], g->streams[i]);
     }
   if (rc != FKV_OK) {
     // Drain what was enqueued; nothing of this call is announced.
     for (int i = 0; i < g->num_gpus; ++i) {
       (void)hipSetDevice(g->device_ids[i]);
+      if (i < (int)g->dma_streams.size() && g->dma_streams[i])
+        (void)hipStreamSynchronize(g->dma_streams[i]);
       (void)hipStreamSynchronize(g->streams[i]);
     }
     g->layer_batch.assign(g->num_layers, -1);
@@ -889,8 +931,14 @@ void fkv_layerwise_destroy(fkv_layerwise *g) {
     return;
   g->retire_previous();
   fkv::DeviceGuard restore(-1);
+  for (auto &ring : g->rings) {
+    (void)hipSetDevice(g->device_ids[ring.first.second]);
+    ring.second.release();
+  }
   for (int i = 0; i < g->num_gpus; ++i) {
     (void)hipSetDevice(g->device_ids[i]);
+    if (i < (int)g->dma_streams.size() && g->dma_streams[i])
+      (void)hipStreamDestroy(g->dma_streams[i]);
     (void)hipStreamDestroy(g->streams[i]);
   }
   (void)hipSetDevice(restore.device());

@@ -1,0 +1,284 @@
+// Layer-by-layer restore through the copy engines.
+//
+// The kernel path reads host memory from the compute units.  That reaches the
+// link rate, but the requests it keeps in flight sit in the same memory queues
+// as those of the engine's own kernels, which run measurably slower next to it
+// (a fused-attention chain sized to the restore: 38 ms alone, 56 ms next to a
+// 41 ms restore).  A copy-engine transfer costs the neighbours nothing (the same
+// chain next to 2-D copies of the same bytes: 40.8 ms for both together), but the
+// engines move contiguous runs or regular 2-D shapes only, one command each at
+// about 10 us of overhead.  So where the host blocks of a restore form few runs
+// of consecutive block ids, each batch of layers goes
+//     host rows --(one 2-D copy per run: width = the batch's bytes of a block,
+//                  pitch = host block stride)--> dense staging buffer in HBM
+//     staging   --(one launch of the gather/scatter kernel, HBM-bound, ~20 us for
+//                  36 MiB)--> the engine's blocks
+// on two streams: the copies of batch b+1 run while batch b is scattered.  The
+// staging buffers form a small ring per (layer group, GPU); a buffer is reused
+// once the scatter that read it has finished (event).  Small holes between runs
+// are read along (their bytes cost less link time than one more command).
+//
+// Replaces, for restores with few runs, the per-layer kernel launches of
+// csrc/layerwise.cpp:1129-1257; related to SEGMENT_SCATTER of
+// csrc/ce_transfer.cu:645-812, which stages in host memory instead.
+#include "fkv_internal.h"
+
+#include <algorithm>
+#include <cstring>
+
+namespace fkv {
+
+void StagedRing::release() {
+  for (uint8_t *b : buf)
+    if (b && hipFree(b) != hipSuccess)
+      (void)hipGetLastError();
+  for (auto *set : {&copied, &freed})
+    for (hipEvent_t e : *set)
+      if (e && hipEventDestroy(e) != hipSuccess)
+        (void)hipGetLastError();
+  buf.clear();
+  copied.clear();
+  freed.clear();
+  used.clear();
+  cap = 0;
+  next = 0;
+}
+
+namespace {
+
+int ring_prepare(StagedRing &ring, int slots, size_t bytes) {
+  if ((int)ring.buf.size() == slots && ring.cap >= bytes)
+    return FKV_OK;
+  // Only called while nothing of an earlier restore is in flight.
+  ring.release();
+  ring.buf.assign(slots, nullptr);
+  ring.copied.assign(slots, nullptr);
+  ring.freed.assign(slots, nullptr);
+  ring.used.assign(slots, false);
+  size_t cap = (bytes + (2u << 20) - 1) & ~(size_t)((2u << 20) - 1);
+  for (int k = 0; k < slots; ++k) {
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&ring.buf[k]), cap);
+    // `copied` publishes bytes the copy engine wrote for a kernel on another
+    // stream: default fence.  `freed` only orders work.
+    if (e == hipSuccess)
+      e = hipEventCreateWithFlags(&ring.copied[k], hipEventDisableTiming);
+    if (e == hipSuccess)
+      e = hipEventCreateWithFlags(&ring.freed[k], kBookkeepingEvent);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      ring.release();
+      return fail(FKV_ERR_RUNTIME, "staged restore: cannot allocate %d staging buffers of %zu MiB: %s",
+                  slots, cap >> 20, hipGetErrorString(e));
+    }
+  }
+  ring.cap = cap;
+  stats().staging_bytes_device.fetch_add((uint64_t)cap * slots, std::memory_order_relaxed);
+  return FKV_OK;
+}
+
+} // namespace
+
+int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &ring,
+                      hipStream_t scatter_stream, StagedPlan *out) {
+  *out = StagedPlan{};
+  int device = 0;
+  FKV_HIP_TRY(hipGetDevice(&device));
+  const fkv_launch_policy pol = policy_of(device);
+  if (pol.staged_restore == 0 || d.num_blocks <= 0 || d.num_layers <= 0 || batch_layers < 1)
+    return FKV_OK;
+  const int nl = std::min(batch_layers, d.num_layers);
+  const int lk = nl * d.kv_dim;
+  if (lk > kCopyMaxLK)
+    return FKV_OK;
+  // which chunks of one host block are adjacent
+  const bool kv_adjacent = d.kv_dim == 1 || d.cpu_kv_stride == d.chunk_size;
+  const bool layers_adjacent = kv_adjacent && d.cpu_layer_stride == d.kv_dim * d.chunk_size;
+  out->kind = layers_adjacent ? 0 : kv_adjacent ? 1 : 2;
+  const int64_t batch_row_bytes = (int64_t)lk * d.chunk_size; // of one block, all pieces
+  const int pieces = out->kind == 0 ? 1 : out->kind == 1 ? nl : lk;
+
+  // runs of consecutive host block ids
+  std::vector<int64_t> ids(d.cpu_block_ids, d.cpu_block_ids + d.num_blocks);
+  std::sort(ids.begin(), ids.end());
+  ids.erase(std::unique(ids.begin(), ids.end()), ids.end());
+  struct Hole {
+    int64_t rows;
+    size_t after; // index into ids of the last block before the hole
+  };
+  std::vector<Hole> holes;
+  for (size_t k = 0; k + 1 < ids.size(); ++k)
+    if (ids[k + 1] != ids[k] + 1)
+      holes.push_back(Hole{ids[k + 1] - ids[k] - 1, k});
+  // Holes are read along, smallest first, while each stays below the bridge size
+  // and all together below the allowed share of the useful bytes.
+  const double useful = (double)ids.size() * batch_row_bytes;
+  const double max_waste = useful * pol.staged_overhead_pct / 100.0;
+  std::vector<size_t> order(holes.size());
+  for (size_t k = 0; k < order.size(); ++k)
+    order[k] = k;
+  std::sort(order.begin(), order.end(),
+            [&](size_t a, size_t b) { return holes[a].rows < holes[b].rows; });
+  std::vector<bool> bridged(holes.size(), false);
+  double waste = 0;
+  int64_t extra_rows = 0;
+  for (size_t k : order) {
+    const double bytes = (double)holes[k].rows * batch_row_bytes;
+    if (bytes > (double)pol.staged_bridge_kb * 1024 || waste + bytes > max_waste)
+      break;
+    bridged[k] = true;
+    waste += bytes;
+    extra_rows += holes[k].rows;
+  }
+  int64_t nsegs = 1;
+  for (size_t k = 0; k < holes.size(); ++k)
+    nsegs += bridged[k] ? 0 : 1;
+  const int64_t total_rows = (int64_t)ids.size() + extra_rows;
+  const int64_t slot_bytes = total_rows * batch_row_bytes;
+  if (slot_bytes > (int64_t)pol.staged_max_mb << 20)
+    return FKV_OK;
+  if (pol.staged_restore == 1) {
+    // the copy commands of a batch against the batch's time on the link
+    const double batch_us = useful / (pol.link_gbps_estimate * 1e3);
+    if ((double)(nsegs * pieces) * pol.staged_copy_overhead_us >
+        batch_us * pol.staged_overhead_pct / 100.0)
+      return FKV_OK;
+  }
+  if (nsegs * pieces > 4096) // a batch of thousands of commands is never the better way
+    return FKV_OK;
+
+  out->segs.reserve((size_t)nsegs);
+  {
+    StagedPlan::Seg cur{ids[0], 1, 0};
+    size_t h = 0;
+    for (size_t k = 0; k + 1 < ids.size(); ++k) {
+      if (ids[k + 1] == ids[k] + 1) {
+        cur.rows += 1;
+        continue;
+      }
+      if (bridged[h]) {
+        cur.rows += (int32_t)(ids[k + 1] - ids[k]);
+      } else {
+        out->segs.push_back(cur);
+        cur = StagedPlan::Seg{ids[k + 1], 1, cur.row0 + cur.rows};
+      }
+      ++h;
+    }
+    out->segs.push_back(cur);
+  }
+  out->total_rows = (int32_t)total_rows;
+  out->max_lk = lk;
+  out->batch_layers = nl;
+  out->kv_dim = d.kv_dim;
+  out->chunk = d.chunk_size;
+  out->cpu_kv_stride = d.cpu_kv_stride;
+  out->cpu_layer_stride = d.cpu_layer_stride;
+  out->cpu_block_stride = d.cpu_block_stride;
+  out->host0 = static_cast<const uint8_t *>(d.cpu_ptr) + d.cpu_startoff_inside_chunks;
+  out->num_blocks = d.num_blocks;
+
+  FKV_TRY(ring_prepare(ring, pol.staged_ring, (size_t)slot_bytes));
+  const int slots = (int)ring.buf.size();
+  const size_t tab = (size_t)slots * lk * 8, rows_bytes = (size_t)d.num_blocks * 8;
+  PlanSlot *slot = plan_acquire(device, tab + rows_bytes);
+  if (!slot)
+    return FKV_ERR_RUNTIME;
+  uint8_t *h = plan_host(slot);
+  uint64_t *bases = reinterpret_cast<uint64_t *>(h);
+  // staging layout of a batch: [piece][row][chunks of the piece]
+  const int m = out->kind == 0 ? lk : out->kind == 1 ? d.kv_dim : 1; // chunks per piece (full batch)
+  for (int k = 0; k < slots; ++k)
+    for (int i = 0; i < lk; ++i) {
+      // kind 0 has one piece whatever the batch length: chunk i of a row sits at i * chunk
+      const uint64_t piece_off =
+          out->kind == 0 ? 0 : (uint64_t)(i / m) * (uint64_t)total_rows * (uint64_t)(m * d.chunk_size);
+      bases[(size_t)k * lk + i] = (uint64_t)(uintptr_t)ring.buf[k] + piece_off +
+                                  (uint64_t)(i % m) * (uint64_t)d.chunk_size;
+    }
+  int64_t *rows = reinterpret_cast<int64_t *>(h + tab);
+  for (int pos = 0; pos < d.num_blocks; ++pos) {
+    const int64_t id = d.cpu_block_ids[pos];
+    // the last segment whose first id is <= id
+    size_t lo = 0, hi = out->segs.size();
+    while (hi - lo > 1) {
+      const size_t mid = (lo + hi) / 2;
+      if (out->segs[mid].first_id <= id)
+        lo = mid;
+      else
+        hi = mid;
+    }
+    rows[pos] = out->segs[lo].row0 + (id - out->segs[lo].first_id);
+  }
+  uint8_t *dv = nullptr;
+  int rc = plan_publish(slot, tab + rows_bytes, /*mirror=*/true, scatter_stream, &dv);
+  if (rc != FKV_OK) {
+    plan_release(slot, scatter_stream, false);
+    return rc;
+  }
+  out->slot = slot;
+  out->base_tables = reinterpret_cast<const uint64_t *>(dv);
+  out->stage_rows = reinterpret_cast<const int64_t *>(dv + tab);
+  out->usable = true;
+  return FKV_OK;
+}
+
+int staged_launch(const StagedPlan &sp, StagedRing &ring, const KernelPlan &kp, int l0, int nl,
+                  hipStream_t dma_stream, hipStream_t scatter_stream) {
+  if (!sp.usable || nl < 1 || nl > sp.batch_layers || nl * sp.kv_dim > sp.max_lk)
+    return fail(FKV_ERR_RUNTIME, "staged restore: batch of %d layers does not fit its plan", nl);
+  const int k = ring.next;
+  ring.next = (ring.next + 1) % (int)ring.buf.size();
+  if (ring.used[k]) // the scatter that read this buffer last
+    FKV_HIP_TRY(hipStreamWaitEvent(dma_stream, ring.freed[k], 0));
+  const int lk = nl * sp.kv_dim;
+  const int m = sp.kind == 0 ? lk : sp.kind == 1 ? sp.kv_dim : 1;
+  const int pieces = lk / m;
+  const int64_t w = (int64_t)m * sp.chunk;
+  uint64_t copies = 0;
+  for (int p = 0; p < pieces; ++p) {
+    const int i0 = p * m;
+    const int64_t layer = l0 + i0 / sp.kv_dim, kv = i0 % sp.kv_dim;
+    const uint8_t *src0 = sp.host0 + layer * sp.cpu_layer_stride + kv * sp.cpu_kv_stride;
+    uint8_t *dst0 = ring.buf[k] + (sp.kind == 0 ? 0 : (int64_t)p * sp.total_rows * w);
+    for (const StagedPlan::Seg &s : sp.segs) {
+      const uint8_t *src = src0 + s.first_id * sp.cpu_block_stride;
+      uint8_t *dst = dst0 + (int64_t)s.row0 * w;
+      if (s.rows == 1 || sp.cpu_block_stride == w)
+        FKV_HIP_TRY(hipMemcpyAsync(dst, src, (size_t)s.rows * w, hipMemcpyHostToDevice, dma_stream));
+      else
+        FKV_HIP_TRY(hipMemcpy2DAsync(dst, (size_t)w, src, (size_t)sp.cpu_block_stride, (size_t)w,
+                                     (size_t)s.rows, hipMemcpyHostToDevice, dma_stream));
+      ++copies;
+    }
+  }
+  FKV_HIP_TRY(hipEventRecord(ring.copied[k], dma_stream));
+  FKV_HIP_TRY(hipStreamWaitEvent(scatter_stream, ring.copied[k], 0));
+  CopyKernelArgs a{};
+  a.base_src = sp.base_tables + (size_t)k * sp.max_lk;
+  a.base_dst = kp.gpu_base + (size_t)l0 * kp.kv_dim;
+  a.ids_src = sp.stage_rows;
+  a.ids_dst = kp.gpu_ids;
+  a.stride_src = w;
+  a.stride_dst = kp.gpu_block_stride;
+  a.chunk_bytes = sp.chunk;
+  a.num_blocks = sp.num_blocks;
+  a.lk = lk;
+  a.vec = kp.vec; // staging addresses are multiples of the chunk size off a 2 MiB-aligned buffer
+  a.nt_store = 1;
+  a.xcd_mask = 0;
+  const fkv_launch_policy pol = policy_of(kp.device);
+  FKV_TRY(launch_copy_kernel(a, pol.hbm_workgroups, pol.hbm_wg_threads, scatter_stream));
+  FKV_HIP_TRY(hipEventRecord(ring.freed[k], scatter_stream));
+  ring.used[k] = true;
+  stats().dma_copies.fetch_add(copies, std::memory_order_relaxed);
+  stats().staged_batches.fetch_add(1, std::memory_order_relaxed);
+  return FKV_OK;
+}
+
+void staged_plan_release(StagedPlan *sp, hipStream_t scatter_stream) {
+  if (sp->slot)
+    plan_release(sp->slot, scatter_stream, false);
+  sp->slot = nullptr;
+  sp->usable = false;
+}
+
+} // namespace fkv

@@ -16,14 +16,6 @@
 
 using namespace fkv;
 
-namespace {
-int env_or(const char *name, int fallback) {
-  const char *v = std::getenv(name);
-  const int n = (v && *v) ? std::atoi(v) : fallback;
-  return n > 0 ? n : fallback;
-}
-} // namespace
-
 extern "C" int fkv_layout_transform(const fkv_layout_transform_desc *dp, void *stream_v) {
   clear_error();
   if (!dp)
@@ -58,8 +50,8 @@ extern "C" int fkv_layout_transform(const fkv_layout_transform_desc *dp, void *s
   int device = 0;
   FKV_HIP_TRY(hipGetDevice(&device));
   hipStream_t stream = static_cast<hipStream_t>(stream_v);
-  static const int workgroups = env_or("FKV_TRANSFORM_WORKGROUPS", 2048);
-  static const int threads = env_or("FKV_TRANSFORM_THREADS", 1024);
+  const fkv_launch_policy pol = policy_of(device);
+  const int workgroups = pol.hbm_workgroups, threads = pol.hbm_wg_threads;
   const bool to_buffer = d.buffer_to_target == 0;
   const int pairs = d.num_layers * d.kv_dim;
   for (int p0 = 0; p0 < pairs; p0 += kCopyMaxLK) {
@@ -101,7 +93,7 @@ extern "C" int fkv_layout_transform(const fkv_layout_transform_desc *dp, void *s
       a.lk = lk;
       a.vec = common_vector_width(&acc, 1);
       a.nt_store = 1;
-      a.xcd_mask = 0xffu;
+      a.xcd_mask = 0;
       rc = launch_copy_kernel(a, workgroups, threads, stream);
     }
     plan_release(slot, stream, false);

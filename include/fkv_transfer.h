@@ -537,9 +537,78 @@ typedef struct fkv_stats {
                                  confined launches copied by the fallback workgroup because no
                                  workgroup on the chosen XCDs had claimed anything in time;
                                  expected to stay 0 */
+  uint64_t staged_batches;    /* layer batches of a layerwise restore that went through the copy
+                                 engines and a device staging buffer */
 } fkv_stats;
 void fkv_get_stats(fkv_stats *out);
 void fkv_reset_stats(void);
+
+/* ---- launch policy: every tunable of the kernel path, per device, in one table ----
+ *
+ * No counterpart in the reference, whose only launch parameter is transfer_num_cta.
+ * The defaults are derived from the device (the XCDs it exposes are found by a probe
+ * kernel on first use); a field can be preset through the environment variable named
+ * beside it, read once when the device's table is first built, and changed at run
+ * time with fkv_launch_policy_set.  XCD masks name physical XCD ids (bit k = XCD k);
+ * a mask that covers every XCD of the device means "not confined". */
+typedef struct fkv_launch_policy {
+  /* read-only (ignored by _set) */
+  int32_t xcd_count;          /* XCDs the device exposes */
+  uint32_t xcd_present_mask;  /* their ids */
+  /* both directions at once */
+  int32_t arbiter;            /* FKV_LINK_ARBITER: 0 never confine; 1 confine a launch while the
+                                 other direction is busy and keep large launches to home XCDs
+                                 (default on devices with 4 XCDs or more); 2 confine every
+                                 link-bound launch to its busy mask; 3 (tests) confine every
+                                 link-bound launch to an XCD the device does not have, so that
+                                 the safety-net workgroup alone does the work */
+  uint32_t d2h_busy_mask;     /* XCDs of a GPU->host launch while gets are running */
+  uint32_t h2d_busy_mask;     /* XCDs of a host->GPU launch while puts are running */
+  uint32_t d2h_home_mask;     /* XCDs of a large GPU->host launch on an idle link */
+  uint32_t h2d_home_mask;     /* the same, host->GPU */
+  int32_t busy_window_ms;     /* a direction counts as busy this long after its last launch */
+  int32_t home_min_kb;        /* launches of at least this size keep to home XCDs (-1: never) */
+  int32_t d2h_busy_pct;       /* workgroups of a confined launch, percent of the unconfined count */
+  int32_t h2d_busy_pct;
+  int32_t busy_claims_per_wg; /* ranges a working workgroup claims, confined by a busy link */
+  int32_t home_claims_per_wg; /* the same on home XCDs */
+  int32_t all_claims_per_wg;  /* launches on all XCDs: 0 = fixed shares */
+  int32_t safety_net_wait_us; /* how long workgroup 0 of a confined launch waits before it takes
+                                 over a launch of which nothing landed on a selected XCD */
+  int32_t link_gbps_estimate; /* what other processes are told a launch will take: bytes / this */
+  /* launch shape of the link-bound kernel */
+  int32_t d2h_wg_per_cta;     /* workgroups per requested CTA (transfer_num_cta) */
+  int32_t h2d_wg_per_cta;
+  int32_t d2h_wg_threads;     /* lanes per workgroup */
+  int32_t h2d_wg_threads;
+  int32_t packed_grid_pct;    /* packed short chunks: workgroups, percent of the normal count */
+  int32_t plan_mirror;        /* -1 upload the plan unless the other direction is busy, 0 never, 1 always */
+  int32_t fuse_launches;      /* members of one layer in one launch */
+  int32_t lane_streams;       /* FKV_LANE_STREAMS: -1 auto, 0 never, 1 always */
+  /* layerwise restore through the copy engines (see fkv_layerwise_transfer) */
+  int32_t staged_restore;     /* FKV_STAGED_RESTORE: 0 never, 1 when the host blocks form few
+                                 runs (default), 2 whenever the layout allows it */
+  int32_t staged_ring;        /* staging buffers per layer group and GPU */
+  int32_t staged_copy_overhead_us; /* cost of one more copy command, for the choice */
+  int32_t staged_overhead_pct;     /* staged when copies x overhead stays below this share of
+                                      the batch's time on the link */
+  int32_t staged_bridge_kb;   /* holes between runs of host blocks up to this size are read along */
+  int32_t staged_max_mb;      /* largest staging buffer (one of the ring) */
+  /* HBM-bound launches: device compaction of the copy-engine strategies, layout transform,
+   * the scatter of a staged restore */
+  int32_t hbm_workgroups;
+  int32_t hbm_wg_threads;
+  int32_t ce_staging_mb;      /* FKV_CE_STAGING_MB: device staging of the copy-engine strategies */
+  int32_t ce_two_streams;     /* direct copy-engine strategies fan out over a second stream */
+  int32_t reserved[8];
+} fkv_launch_policy;
+/* The table of `device` (-1 = current).  The first call for a device runs the probe kernel. */
+int fkv_launch_policy_get(int32_t device, fkv_launch_policy *out);
+/* Replaces the table of `device`; read-only fields are ignored, masks are cut to the
+ * XCDs the device has (except with arbiter == 3), counts are clamped to sane ranges. */
+int fkv_launch_policy_set(int32_t device, const fkv_launch_policy *in);
+/* Back to the defaults derived from the device and the environment. */
+int fkv_launch_policy_reset(int32_t device);
 
 /* Host-link reference rate: `reps` plain hipMemcpyAsync copies of `bytes`
  * between a pinned host buffer and a device buffer (both owned by the call),

@@ -1,0 +1,122 @@
+"""Layerwise restore through the copy engines (host rows -> staging buffer ->
+scatter kernel) against the oracle, next to the same restore on the kernel path.
+
+The choice between the two is a matter of the launch policy; the tests force it
+either way, so which path a case runs does not depend on the box."""
+import numpy as np
+import pytest
+import torch
+
+from kvsetup import KVSetup, SGLANG, TRTLLM, VLLM
+
+pytestmark = pytest.mark.gpu
+
+
+def group_of(s, dev):
+    from flexkv_amd.c_ext import LayerwiseTransferGroup
+    i64 = lambda v: torch.tensor([v], dtype=torch.int64)
+    return LayerwiseTransferGroup(
+        num_gpus=1, gpu_blocks=[dev.gpu], cpu_blocks=dev.host, ssd_files={}, num_layers=s.num_layers,
+        gpu_kv_strides_tensor=i64(s.gpu_kv_stride), gpu_block_strides_tensor=i64(s.gpu_block_stride),
+        gpu_layer_strides_tensor=i64(s.gpu_layer_stride), gpu_chunk_sizes_tensor=i64(s.chunk),
+        iouring_entries=0, iouring_flags=0,
+        layer_eventfds_tensor=torch.empty(0, dtype=torch.int32), tp_size=1,
+        is_blockfirst=s.cpu_layout == "BLOCKFIRST")
+
+
+def restore(grp, s, gids, cids, gran, notify="polling", num_layers=None):
+    e = torch.empty(0, dtype=torch.int64)
+    grp.layerwise_transfer(
+        e, e, 0, 0, 0, 0, 0, torch.as_tensor(gids), torch.as_tensor(cids), s.cpu_kv_stride,
+        s.cpu_layer_stride, s.cpu_block_stride, s.chunk, s.cpu_kv_stride, s.cpu_layer_stride,
+        s.cpu_block_stride, 4, False, s.num_layers if num_layers is None else num_layers, gran,
+        s.kv_dim, 1, counter_id=0, kv_shared_across_ranks_mode="sharded", notify_mode=notify)
+    grp.synchronize()
+
+
+def host_ids(rng, pool, n, pattern):
+    if pattern == "one_run":
+        a = int(rng.integers(0, pool - n + 1))
+        ids = np.arange(a, a + n)
+    elif pattern == "runs_and_holes":  # runs of 1-6 blocks, holes of 1-3 blocks between them
+        ids, at = [], 0
+        while len(ids) < n and at < pool:
+            run = int(rng.integers(1, 7))
+            ids.extend(range(at, min(pool, at + run)))
+            at += run + int(rng.integers(1, 4))
+        ids = np.array(ids[:n])
+    else:  # scattered
+        ids = rng.permutation(pool)[:n]
+    return rng.permutation(ids).astype(np.int64)  # positions in any order
+
+
+@pytest.mark.parametrize("staged", [2, 0], ids=["copy_engines", "kernel"])
+@pytest.mark.parametrize("pattern", ["one_run", "runs_and_holes", "scattered"])
+@pytest.mark.parametrize("backend,kv_dim,cpu_layout,gran", [
+    (VLLM, 1, "BLOCKFIRST", 1), (VLLM, 2, "BLOCKFIRST", 3), (VLLM, 2, "LAYERFIRST", 2),
+    (TRTLLM, 2, "BLOCKFIRST", 2), (SGLANG, 2, "BLOCKFIRST", 1), (SGLANG, 2, "LAYERFIRST", 4)])
+def test_restore_matches_the_oracle(gpu_device, staged, pattern, backend, kv_dim, cpu_layout, gran):
+    """Seven layers (more batches than staging buffers), three restores in a row
+    through the same group with fresh host bytes each time: a stale staging buffer
+    or a buffer reused too early would show up as old bytes."""
+    from flexkv_amd.c_ext import get_stats, launch_policy, reset_stats
+    L, NG, NC, n, chunk = 7, 96, 80, 41, 4608
+    s = KVSetup(backend, L, kv_dim, NG, NC, chunk, cpu_layout, seed=17 + gran)
+    dev = s.to_device(gpu_device)
+    grp = group_of(s, dev)
+    rng = np.random.default_rng(5 * gran + kv_dim)
+    with launch_policy(staged_restore=staged, staged_ring=3):
+        reset_stats()
+        for rep in range(3):
+            fresh = rng.integers(0, 256, s.host_bytes, dtype=np.uint8)
+            s.host_ref[:] = fresh
+            dev.host.copy_(torch.from_numpy(fresh))
+            gids = rng.permutation(NG)[:n].astype(np.int64)
+            cids = host_ids(rng, NC, n, pattern)
+            restore(grp, s, gids, cids, gran, notify="hostfunc" if rep == 1 else "polling")
+            s.oracle_transfer(gids, cids, True)
+            dev.assert_matches_reference(f"restore {rep} ({pattern})")
+        st = get_stats()
+    batches = 3 * ((L + gran - 1) // gran)
+    assert st["staged_batches"] == (batches if staged else 0), st
+    grp.close()
+
+
+def test_restore_of_a_layer_prefix_and_duplicate_host_blocks(gpu_device):
+    """num_layers below the group's, a short last batch, and two GPU blocks that
+    take the same host block."""
+    from flexkv_amd.c_ext import get_stats, launch_policy, reset_stats
+    s = KVSetup(VLLM, 9, 2, 64, 64, 2048, "BLOCKFIRST", seed=3)
+    dev = s.to_device(gpu_device)
+    grp = group_of(s, dev)
+    gids = np.array([5, 9, 60, 2, 33, 34], dtype=np.int64)
+    cids = np.array([10, 11, 10, 12, 40, 13], dtype=np.int64)
+    with launch_policy(staged_restore=2):
+        reset_stats()
+        restore(grp, s, gids, cids, gran=4, num_layers=7)   # batches of 4 + 3 layers
+        assert get_stats()["staged_batches"] == 2
+    s.oracle_transfer(gids, cids, True, num_layers=7)
+    dev.assert_matches_reference("prefix of 7 layers")
+    grp.close()
+
+
+def test_the_choice_follows_the_runs_of_host_blocks(gpu_device):
+    """With the default policy a restore whose host blocks form one run goes
+    through the copy engines, one whose host blocks are scattered does not; both
+    give the oracle's bytes.  (The choice is arithmetic on the id list: no timing.)"""
+    from flexkv_amd.c_ext import get_stats, launch_policy, reset_stats
+    L, n, chunk = 4, 256, 73728
+    s = KVSetup(VLLM, L, 1, 300, 300, chunk, "BLOCKFIRST", seed=9)
+    dev = s.to_device(gpu_device)
+    grp = group_of(s, dev)
+    rng = np.random.default_rng(2)
+    with launch_policy(staged_restore=1):
+        for pattern, want in (("one_run", L), ("scattered", 0)):
+            gids = rng.permutation(300)[:n].astype(np.int64)
+            cids = host_ids(rng, 300, n, pattern)
+            reset_stats()
+            restore(grp, s, gids, cids, gran=1)
+            assert get_stats()["staged_batches"] == want, (pattern, get_stats())
+            s.oracle_transfer(gids, cids, True)
+            dev.assert_matches_reference(pattern)
+    grp.close()

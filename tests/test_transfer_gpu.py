@@ -338,32 +338,65 @@ def test_a_put_in_another_process_confines_the_gets_of_this_one(gpu_device):
     dev.assert_matches_reference("get after the other process has gone")
 
 
-def test_ranges_claimed_by_workgroups_on_all_xcds(gpu_device):
-    """FKV_CLAIMS_PER_WORKGROUP hands the work of a launch that uses all XCDs out
-    in ranges (read once per process, hence a child process): normal and packed
-    chunks, several transfers in a row through the same counters."""
-    import subprocess
-    import sys
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    script = (
-        "import sys; sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[1] + '/tests')\n"
-        "import numpy as np\n"
-        "from kvsetup import KVSetup\n"
-        "from flexkv_amd.c_ext import get_stats\n"
-        "for chunk, n in ((32768, 300), (1152, 2500), (73728, 200)):\n"
-        "    s = KVSetup(0, 6, 2, n + 50, n + 50, chunk, 'BLOCKFIRST', seed=chunk)\n"
-        "    dev = s.to_device('cuda:0')\n"
-        "    rng = np.random.default_rng(chunk)\n"
-        "    for h2d in (False, True, False, True):\n"
-        "        g, c = rng.permutation(n + 50)[:n], rng.permutation(n + 50)[:n]\n"
-        "        dev.transfer(g, c, is_h2d=h2d)\n"
-        "        s.oracle_transfer(g, c, h2d)\n"
-        "    dev.assert_matches_reference(f'chunk {chunk}')\n"
-        "print('ok', get_stats()['confined_launches'])\n")
-    env = dict(os.environ, FKV_CLAIMS_PER_WORKGROUP="8", FKV_LINK_ARBITER="0")
-    r = subprocess.run([sys.executable, "-c", script, root], env=env, capture_output=True,
-                       text=True, timeout=170)
-    assert r.returncode == 0 and r.stdout.split()[-2:] == ["ok", "0"], r.stdout + r.stderr
+@pytest.mark.parametrize("mode", ["arbiter_off", "confined", "home", "safety_net", "claims_on_all_xcds"])
+def test_every_way_a_launch_can_share_out_its_work(gpu_device, mode):
+    """The launch policy forces each way the workgroups of a launch come by their
+    work, whatever the link is doing: fixed shares on all XCDs (arbiter off),
+    confined to the XCDs of a busy link, confined to the home XCDs, no workgroup on
+    a selected XCD so that the safety-net workgroup copies everything, and ranges
+    claimed on all XCDs.  Normal, packed and long chunks, both directions, several
+    transfers through the same counters: the oracle's bytes every time."""
+    from flexkv_amd.c_ext import get_launch_policy, get_stats, launch_policy, reset_stats
+    fields = {"arbiter_off": dict(arbiter=0), "confined": dict(arbiter=2),
+              "home": dict(arbiter=1, home_min_kb=0, busy_window_ms=0),
+              "safety_net": dict(arbiter=3, safety_net_wait_us=5),
+              "claims_on_all_xcds": dict(arbiter=0, all_claims_per_wg=8)}[mode]
+    xcds = get_launch_policy()["xcd_count"]
+    launches = 0
+    with launch_policy(**fields):
+        reset_stats()
+        before = get_stats()["safety_net_ranges"]
+        for chunk, n in ((32768, 120), (1152, 700), (73728, 60)):
+            s = KVSetup(VLLM, 6, 2, n + 50, n + 50, chunk, "BLOCKFIRST", seed=chunk)
+            dev = s.to_device(gpu_device)
+            rng = np.random.default_rng(chunk)
+            for h2d in (False, True, False, True):
+                g, c = rng.permutation(n + 50)[:n], rng.permutation(n + 50)[:n]
+                dev.transfer(g, c, is_h2d=h2d)
+                s.oracle_transfer(g, c, h2d)
+                launches += 1
+            dev.assert_matches_reference(f"{mode}, chunk {chunk}")
+        st = get_stats()
+    assert st["kernel_launches"] == launches
+    if mode in ("arbiter_off", "claims_on_all_xcds") or xcds < 4:
+        assert st["confined_launches"] == 0 or mode == "safety_net", st
+    if mode in ("confined", "home") and xcds >= 4:
+        assert st["confined_launches"] == launches, st
+    if mode == "safety_net":
+        assert st["confined_launches"] == launches, st
+        assert st["safety_net_ranges"] - before > 0, st   # the fallback workgroup did the work
+
+
+def test_the_launch_policy_follows_the_device(gpu_device):
+    """Masks are derived from the XCDs the device exposes: disjoint halves for the
+    two directions, the home XCDs of a direction include its busy XCDs, and a set
+    never names an XCD the device lacks."""
+    from flexkv_amd.c_ext import get_launch_policy, reset_launch_policy, set_launch_policy
+    p = get_launch_policy()
+    present = p["xcd_present_mask"]
+    assert p["xcd_count"] == bin(present).count("1") >= 1
+    for name in ("d2h_busy_mask", "h2d_busy_mask", "d2h_home_mask", "h2d_home_mask"):
+        assert p[name] and p[name] & ~present == 0, (name, p)
+    if p["xcd_count"] >= 4:
+        assert p["d2h_busy_mask"] & p["h2d_busy_mask"] == 0
+        assert p["d2h_home_mask"] & p["h2d_home_mask"] == 0
+        assert p["d2h_busy_mask"] & ~p["d2h_home_mask"] == 0
+    q = set_launch_policy(d2h_busy_mask=0xffff0000 | present, busy_window_ms=-5, staged_ring=99)
+    assert q["d2h_busy_mask"] == present and q["busy_window_ms"] == 0 and q["staged_ring"] == 8
+    with pytest.raises(ValueError):
+        set_launch_policy(no_such_field=1)
+    reset_launch_policy()
+    assert get_launch_policy() == p
 
 
 def test_lane_streams_keep_the_order_of_the_callers_stream(gpu_device):
