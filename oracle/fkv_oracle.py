@@ -269,6 +269,25 @@ def torch_index_scatter(layers, host_cache, gpu_ids, cpu_ids) -> None:
         layer.index_copy_(1, gpu_ids, picked.transpose(0, 1))
 
 
+def torch_index_gather_planes(planes, host_cache, gpu_ids, cpu_ids) -> None:
+    """The same for engines that keep one tensor per (layer, K-or-V) with the block
+    axis first (SGLang pages, MLA latent blocks): ``planes[l][kv]`` is
+    ``[N, ...]``, ``host_cache`` is ``[NH, L, kv, ...]``;
+    host_cache[cpu_ids, l, kv] = planes[l][kv][gpu_ids]."""
+    import torch
+    for l, kvs in enumerate(planes):
+        for kv, plane in enumerate(kvs):
+            host_cache[:, l, kv].index_copy_(0, cpu_ids, torch.index_select(plane, 0, gpu_ids))
+
+
+def torch_index_scatter_planes(planes, host_cache, gpu_ids, cpu_ids) -> None:
+    """Inverse of torch_index_gather_planes."""
+    import torch
+    for l, kvs in enumerate(planes):
+        for kv, plane in enumerate(kvs):
+            plane.index_copy_(0, gpu_ids, torch.index_select(host_cache[:, l, kv], 0, cpu_ids))
+
+
 # ---- layerwise restore of heterogeneous layer groups ---------------------------
 
 class GroupRef:

@@ -160,6 +160,35 @@ def test_reference_cpu_path_gather_equals_oracle():
         assert not r[:, mask].view(torch.int16).any()
 
 
+@pytest.mark.parametrize("kv_dim", [1, 2])
+def test_reference_cpu_path_on_planes_equals_oracle(kv_dim):
+    """The per-(layer, K-or-V) form of the CPU baseline (SGLang pages, MLA blocks):
+    same host cache as the byte-address oracle with SGLang addressing, and the
+    scatter puts the selected blocks back."""
+    L, N, NH, T, H, D = 3, 12, 9, 4, 2, 8
+    g = torch.Generator().manual_seed(4)
+    planes = [[torch.randn(N, T, H, D, generator=g).to(torch.bfloat16) for _ in range(kv_dim)]
+              for _ in range(L)]
+    host_a = torch.zeros(NH, L, kv_dim, T, H, D, dtype=torch.bfloat16)
+    host_b = torch.zeros_like(host_a)
+    gids = torch.randperm(N, generator=g)[:6]
+    cids = torch.randperm(NH, generator=g)[:6]
+    O.torch_index_gather_planes(planes, host_a, gids, cids)
+    chunk = T * H * D * 2
+    ptrs = [planes[l][kv].data_ptr() for kv in range(kv_dim) for l in range(L)]  # K_0.., V_0..
+    O.transfer_c(O.BACKEND_SGLANG, ptrs, L, 0, chunk, N * chunk, 0, host_b.data_ptr(), chunk,
+                 kv_dim * chunk, L * kv_dim * chunk, 0, chunk, 0, L, kv_dim, gids.numpy(),
+                 cids.numpy(), False)
+    assert torch.equal(host_a.view(torch.int16), host_b.view(torch.int16))
+    restored = [[torch.zeros_like(x) for x in kvs] for kvs in planes]
+    O.torch_index_scatter_planes(restored, host_a, gids, cids)
+    for l in range(L):
+        for kv in range(kv_dim):
+            want = torch.zeros_like(planes[l][kv])
+            want[gids] = planes[l][kv][gids]
+            assert torch.equal(restored[l][kv].view(torch.int16), want.view(torch.int16))
+
+
 # ---- the reference tests' deterministic fill as a known answer --------------
 
 def _reference_fill(gpu_id, L, N, T, H, D, kv_dim):
