@@ -181,6 +181,7 @@ SIGNATURES = {
     "fkv_last_path": (c_int32, []),
     "fkv_ce_config_default": (None, [POINTER(CEConfig)]),
     "fkv_transfer_kv_blocks": (c_int32, [POINTER(TransferDesc), c_void_p]),
+    "fkv_transfer_kv_blocks_noalloc": (c_int32, [POINTER(TransferDesc), c_void_p]),
     "fkv_transfer_kv_blocks_multi": (c_int32, [POINTER(TransferDesc), c_int32, c_void_p]),
     "fkv_choose_engine": (c_int32, [POINTER(TransferDesc), POINTER(c_int32), POINTER(c_double),
                                     POINTER(c_double)]),

@@ -376,7 +376,12 @@ void link_direction_mark(int device, bool h2d, hipStream_t stream, int64_t bytes
   d.next = (i + 1) % kActivityRing;
 }
 
-int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan *out) {
+size_t kernel_plan_bytes(const fkv_transfer_desc &d) {
+  return 2 * (size_t)d.num_layers * d.kv_dim * 8 + 2 * (size_t)d.num_blocks * 8;
+}
+
+int kernel_plan_fill(const fkv_transfer_desc &d, uint8_t *h, bool may_probe_device,
+                     KernelPlan *out) {
   // Device-visible alias of the host pool.  hipHostMalloc / torch pinned memory
   // map to the same address; hipHostRegister-ed memory may not.
   void *cpu_dev = nullptr;
@@ -393,11 +398,6 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
   const int lk = d.num_layers * d.kv_dim;
   const size_t tab_bytes = (size_t)lk * 8;
   const size_t ids_bytes = (size_t)d.num_blocks * 8;
-  const size_t plan_bytes = 2 * tab_bytes + 2 * ids_bytes; // base tables, the two id lists
-  PlanSlot *slot = plan_acquire(device, plan_bytes);
-  if (!slot)
-    return FKV_ERR_RUNTIME;
-  uint8_t *h = plan_host(slot);
   uint64_t *gbase = reinterpret_cast<uint64_t *>(h);
   uint64_t *cbase = reinterpret_cast<uint64_t *>(h + tab_bytes);
   uint64_t acc = (uint64_t)d.chunk_size | (uint64_t)d.gpu_block_stride |
@@ -419,14 +419,48 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
   std::memcpy(h + 2 * tab_bytes + ids_bytes, d.cpu_block_ids, ids_bytes);
   // A CTA of the reference is 1024 threads on one SM (csrc/transfer.cu:176) and
   // its default of 4 CTAs is tuned for that hardware.  Here each requested CTA
-  // becomes `workgroups_per_cta` small workgroups (see link_launch_shape).
+  // becomes several small workgroups (see the note on the launch shape above).
   out->h2d = d.is_host_to_device != 0;
-  const fkv_launch_policy pol = policy_of(device);
+  const fkv_launch_policy pol = may_probe_device ? policy_of(device) : policy_peek(device);
+  out->no_alloc = !may_probe_device;
   out->workgroups =
       (d.transfer_num_cta > 0 ? d.transfer_num_cta : default_num_cta(out->h2d)) *
       (out->h2d ? pol.h2d_wg_per_cta : pol.d2h_wg_per_cta);
   out->threads = out->h2d ? pol.h2d_wg_threads : pol.d2h_wg_threads;
   out->device = device;
+  out->vec = common_vector_width(&acc, 1);
+  out->kv_dim = d.kv_dim;
+  out->num_layers = d.num_layers;
+  out->num_blocks = d.num_blocks;
+  out->chunk_size = d.chunk_size;
+  out->gpu_block_stride = d.gpu_block_stride;
+  out->cpu_block_stride = d.cpu_block_stride;
+  return FKV_OK;
+}
+
+void kernel_plan_point(KernelPlan *out, const uint8_t *dv, uint64_t *claims) {
+  const size_t tab_bytes = (size_t)out->num_layers * out->kv_dim * 8;
+  const size_t ids_bytes = (size_t)out->num_blocks * 8;
+  out->gpu_base = reinterpret_cast<const uint64_t *>(dv);
+  out->cpu_base = reinterpret_cast<const uint64_t *>(dv + tab_bytes);
+  out->gpu_ids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes);
+  out->cpu_ids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes + ids_bytes);
+  out->claims = claims;
+}
+
+int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan *out) {
+  int device = 0;
+  FKV_HIP_TRY(hipGetDevice(&device));
+  const size_t plan_bytes = kernel_plan_bytes(d);
+  PlanSlot *slot = plan_acquire(device, plan_bytes);
+  if (!slot)
+    return FKV_ERR_RUNTIME;
+  int rc = kernel_plan_fill(d, plan_host(slot), /*may_probe_device=*/true, out);
+  if (rc != FKV_OK) {
+    plan_release(slot, stream, true);
+    return rc;
+  }
+  const fkv_launch_policy pol = policy_of(device);
   // Kernels read the plan from a device copy, which a small kernel uploads first,
   // or where it is, in the pinned slot.  Next to a transfer in the other direction
   // every command on a stream costs idle time, and the upload is one: two threads
@@ -439,24 +473,13 @@ int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan
           ? pol.plan_mirror != 0
           : !(pol.arbiter == 1 && link_direction_busy(device, !out->h2d, stream));
   uint8_t *dv = nullptr;
-  int rc = plan_publish(slot, plan_bytes, mirror_plan, stream, &dv);
+  rc = plan_publish(slot, plan_bytes, mirror_plan, stream, &dv);
   if (rc != FKV_OK) {
     plan_release(slot, stream, false);
     return rc;
   }
   out->slot = slot;
-  out->gpu_base = reinterpret_cast<const uint64_t *>(dv);
-  out->cpu_base = reinterpret_cast<const uint64_t *>(dv + tab_bytes);
-  out->gpu_ids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes);
-  out->cpu_ids = reinterpret_cast<const int64_t *>(dv + 2 * tab_bytes + ids_bytes);
-  out->claims = plan_counters(slot, d.num_layers); // nullptr: launches are not confined
-  out->vec = common_vector_width(&acc, 1);
-  out->kv_dim = d.kv_dim;
-  out->num_layers = d.num_layers;
-  out->num_blocks = d.num_blocks;
-  out->chunk_size = d.chunk_size;
-  out->gpu_block_stride = d.gpu_block_stride;
-  out->cpu_block_stride = d.cpu_block_stride;
+  kernel_plan_point(out, dv, plan_counters(slot, d.num_layers)); // nullptr: launches are not confined
   return FKV_OK;
 }
 
@@ -506,7 +529,7 @@ CopyKernelArgs plan_job(const KernelPlan &p, int l0, int nl) {
 // fused-attention calls moves 37 GB/s with one range per workgroup and 54 GB/s with
 // two.
 int shape_for_now(const KernelPlan &p, int64_t bytes, hipStream_t stream, CopyKernelArgs *a) {
-  const fkv_launch_policy pol = policy_of(p.device);
+  const fkv_launch_policy pol = p.no_alloc ? policy_peek(p.device) : policy_of(p.device);
   int workgroups = p.workgroups;
   const uint32_t all = pol.xcd_present_mask;
   const uint32_t busy_mask = p.h2d ? pol.h2d_busy_mask : pol.d2h_busy_mask;
@@ -554,8 +577,9 @@ int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
         shape_for_now(p, (int64_t)p.num_blocks * a.lk * p.chunk_size, stream, &a);
     FKV_TRY(launch_copy_kernel(a, workgroups, p.threads, stream));
   }
-  link_direction_mark(p.device, p.h2d, stream,
-                      (int64_t)p.num_blocks * num_layers * p.kv_dim * p.chunk_size);
+  if (!p.no_alloc) // the bookkeeping creates events on first use
+    link_direction_mark(p.device, p.h2d, stream,
+                        (int64_t)p.num_blocks * num_layers * p.kv_dim * p.chunk_size);
   return FKV_OK;
 }
 

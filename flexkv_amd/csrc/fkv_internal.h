@@ -181,6 +181,9 @@ int launch_plan_upload(void *device_dst, const void *pinned_src, size_t bytes, h
 int probe_xcds(uint32_t *present_mask);
 // The launch policy of `device` (a copy; built on first use, see fkv_policy.cpp).
 fkv_launch_policy policy_of(int device);
+// The same without the probe: the table of a device that has none yet is the one
+// of a device of unknown shape (nothing is confined).
+fkv_launch_policy policy_peek(int device);
 // Widest vector width (bytes) that divides every value in `vals`.
 int common_vector_width(const uint64_t *vals, int n);
 
@@ -218,6 +221,8 @@ struct KernelPlan {
   int64_t chunk_size = 0, gpu_block_stride = 0, cpu_block_stride = 0;
   int workgroups = 1, threads = 64;
   int device = 0;
+  bool no_alloc = false; // built by the entry point that allocates nothing: launches of this
+                         // plan create no events and do not probe the device
   uint64_t *claims = nullptr; // a claim counter per layer of the plan, device memory
 };
 // Link-bound launches of the last while, per device and direction (see fkv_core.cpp).
@@ -228,6 +233,14 @@ void link_direction_mark(int device, bool h2d, hipStream_t stream, int64_t bytes
 // process has posted activity that ends less than `window_ns` ago or later.
 void link_board_post(int device, bool h2d, int64_t expected_ns);
 bool link_board_busy_elsewhere(int device, bool h2d, int64_t window_ns);
+// The two halves of kernel_plan_build, for a caller that brings its own plan
+// memory: bytes a plan of `d` takes; fill them into host memory `h` (and every
+// field of `out` but the addresses); point `out` at the device-visible copy `dv`
+// and at `claims` (num_layers counters, or nullptr).
+size_t kernel_plan_bytes(const fkv_transfer_desc &d);
+int kernel_plan_fill(const fkv_transfer_desc &d, uint8_t *h, bool may_probe_device,
+                     KernelPlan *out);
+void kernel_plan_point(KernelPlan *out, const uint8_t *dv, uint64_t *claims);
 // Builds and uploads (on `stream`) the plan for all layers of `d`.
 int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan *out);
 // Enqueues the copy of layers [layer_offset, layer_offset + num_layers) of the plan.

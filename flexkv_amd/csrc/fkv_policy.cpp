@@ -111,16 +111,9 @@ void sanitize(fkv_launch_policy &p, const fkv_launch_policy &derived) {
   p.ce_two_streams = p.ce_two_streams != 0;
 }
 
-void build(int device, DevicePolicy &t) {
+// The table of a device with the XCDs `present`, environment applied.
+fkv_launch_policy defaults_for(uint32_t present) {
   fkv_launch_policy p{};
-  uint32_t present = 0;
-  {
-    DeviceGuard guard(device);
-    if (!guard.ok() || probe_xcds(&present) != FKV_OK || present == 0) {
-      (void)hipGetLastError();
-      present = 1; // one XCD as far as anybody can tell: nothing is split
-    }
-  }
   p.xcd_present_mask = present;
   p.xcd_count = __builtin_popcount(present);
   derive_masks(p);
@@ -159,7 +152,19 @@ void build(int device, DevicePolicy &t) {
   }
   fkv_launch_policy derived = p;
   sanitize(p, derived);
-  t.derived = t.current = p;
+  return p;
+}
+
+void build(int device, DevicePolicy &t) {
+  uint32_t present = 0;
+  {
+    DeviceGuard guard(device);
+    if (!guard.ok() || probe_xcds(&present) != FKV_OK || present == 0) {
+      (void)hipGetLastError();
+      present = 1; // one XCD as far as anybody can tell: nothing is split
+    }
+  }
+  t.derived = t.current = defaults_for(present);
   t.built = true;
 }
 
@@ -178,6 +183,14 @@ fkv_launch_policy policy_of(int device) {
   if (!t.built)
     build(device, t);
   return t.current;
+}
+
+fkv_launch_policy policy_peek(int device) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  auto it = tables().find(device);
+  if (it != tables().end() && it->second.built)
+    return it->second.current;
+  return defaults_for(1u);
 }
 
 } // namespace fkv

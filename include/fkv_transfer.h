@@ -131,6 +131,26 @@ int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream);
  * the kernel path up to four of them share one launch. */
 int fkv_transfer_kv_blocks_multi(const fkv_transfer_desc *descs, int32_t count, void *stream);
 
+/* The kernel path of fkv_transfer_kv_blocks without any allocation.  No counterpart
+ * in the reference; it is for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The plan
+ * of the launch (base tables, block-id lists) and the claim counters live in a fixed
+ * array in device memory that belongs to the library's code object (one copy per GPU,
+ * held until the process ends) instead of memory allocated on demand; the call makes
+ * no hipMalloc / hipHostMalloc / hipFree and creates no streams or events.
+ *   - same descriptor, same bytes moved as fkv_transfer_kv_blocks on the kernel path;
+ *     use_ce_transfer must be 0 (FKV_ERR_UNSUPPORTED otherwise);
+ *   - limit: 16 * num_blocks + 16 * num_layers * kv_dim <= FKV_NOALLOC_MAX_PLAN_BYTES and
+ *     num_layers <= 1024 (FKV_ERR_INVALID_ARG beyond; split the call);
+ *   - all calls on one GPU share the array: calls on one stream are ordered by the
+ *     stream; a call first waits on the host for the stream of the previous call on
+ *     that GPU; calls that are in flight at the same time on different streams of one
+ *     GPU race and must be ordered by the caller;
+ *   - desc->sync waits with hipStreamSynchronize; the launches are not confined by the
+ *     link arbiter of fkv_transfer_kv_blocks until that call has set up the device. */
+#define FKV_NOALLOC_MAX_PLAN_BYTES (1u << 20)
+int fkv_transfer_kv_blocks_noalloc(const fkv_transfer_desc *desc, void *stream);
+
 /* Which path `use_ce_transfer == 2` would take for this descriptor, from a cost
  * model of both (DMA commands, staging passes, link time); pure host function.
  * The reference fixes the engine per direction by configuration

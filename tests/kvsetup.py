@@ -126,7 +126,8 @@ class DeviceSide:
     def transfer_raw(self, gpu_ids, cpu_ids, is_h2d: bool, start_layer: int = 0,
                      num_layers: Optional[int] = None, gpu_off: int = 0, cpu_off: int = 0,
                      chunk: Optional[int] = None, use_ce: bool = False, num_cta: int = 4,
-                     sync: bool = True, stream: int = 0, ce: Optional[dict] = None) -> int:
+                     sync: bool = True, stream: int = 0, ce: Optional[dict] = None,
+                     entry: str = "fkv_transfer_kv_blocks") -> int:
         """Straight through the C ABI (fkv_transfer_kv_blocks), including the
         in-chunk offsets the Python operator does not expose.  Returns the status."""
         import ctypes
@@ -155,7 +156,7 @@ class DeviceSide:
         d.ce.is_blockfirst = int(s.cpu_layout == "BLOCKFIRST")
         for k, v in (ce or {}).items():
             setattr(d.ce, k, v)
-        return int(L.fkv_transfer_kv_blocks(ctypes.byref(d), stream))
+        return int(getattr(L, entry)(ctypes.byref(d), stream))
 
     def gpu_bytes(self) -> List[np.ndarray]:
         return [t.cpu().numpy() for t in self.gpu]
