@@ -47,7 +47,7 @@ METRIC = "KV block transfer GB/s (D2H, H2D) on 1 GPU; % of measured host-link pe
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs of this script scaled by plain copy kernels of known size
 # (profiles/fkv_copy_chunks_kernel_c1_pmc.md).  None where no such run was made.
-MEASURED_TRAFFIC_BYTES = {("c1", "kernel"): 8590414848, ("transform-c0", "kernel"): 8590474240}
+MEASURED_TRAFFIC_BYTES = {("c1", "kernel"): 8590414848, ("transform-c0", "kernel"): 8593325056}
 
 
 def _median(xs):
@@ -223,6 +223,23 @@ def measure_link(device_index=0, nbytes=1 << 30, reps=10):
         _lib.check(L.fkv_measure_link_peak(device_index, nbytes, reps, direction,
                                            ctypes.byref(best), ctypes.byref(med)))
         out[name] = best.value
+    return out
+
+
+def measure_hbm(device_index=0, nbytes=4 << 30, reps=10):
+    """What HBM delivers to a streaming kernel on contiguous memory: read only, write
+    only, copy (read + written bytes), GB/s, best of `reps`."""
+    from flexkv_amd import _lib
+    L = _lib.load()
+    out = {}
+    for name, mode in (("read_only", 0), ("write_only", 1), ("copy", 2)):
+        best, med = ctypes.c_double(), ctypes.c_double()
+        _lib.check(L.fkv_measure_hbm_rate(device_index, nbytes, reps, mode, ctypes.byref(best),
+                                          ctypes.byref(med)))
+        out[name + "_GBps"] = round(best.value, 1)
+    r, w = out["read_only_GBps"], out["write_only_GBps"]
+    # a copy moves half its bytes at the read rate and half at the write rate at best
+    out["copy_bound_from_read_and_write_GBps"] = round(2.0 / (1.0 / r + 1.0 / w), 1)
     return out
 
 
@@ -1373,7 +1390,10 @@ def transform_record(torch, device, args, steps, warmup):
     avg_ms = (r["to_buffer_ms"] + r["to_engine_ms"]) / 2
     achieved = 2 * r["bytes"] / (avg_ms * 1e-3) / 1e9    # bytes read + bytes written
     plain = 2 * r["bytes"] / (r["plain_copy_ms"] * 1e-3) / 1e9
+    hbm = measure_hbm()
     return {
+        "hbm_yardsticks": hbm,
+        "frac_of_contiguous_copy_yardstick": round(achieved / hbm["copy_GBps"], 4),
         "metric": "engine blocks <-> dense device buffer, GB/s of HBM traffic (read + write)",
         "unit": "GB/s", "value": round(achieved, 1), "n_gpus": 1, "steps": steps,
         "warmup": warmup, "ms_per_step": round(avg_ms, 4), "higher_is_better": True,
@@ -1392,7 +1412,9 @@ def transform_record(torch, device, args, steps, warmup):
                      "kernel": "fkv_copy_chunks_kernel<16, true>",
                      "workload": f"transform-{args.shape}: " + r["desc"],
                      "algorithmic_bytes_per_launch": 2 * r["bytes"],
-                     "avg_launch_ms": round(avg_ms, 4), "bit_exact": r["bit_exact"]}}
+                     "avg_launch_ms": round(avg_ms, 4), "bit_exact": r["bit_exact"],
+                     "hbm_yardsticks": hbm,
+                     "frac_of_contiguous_copy_yardstick": round(achieved / hbm["copy_GBps"], 4)}}
 
 
 if __name__ == "__main__":

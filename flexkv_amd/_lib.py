@@ -169,9 +169,9 @@ class LaunchPolicy(Structure):
                 ("staged_restore", c_int32), ("staged_ring", c_int32),
                 ("staged_copy_overhead_us", c_int32), ("staged_overhead_pct", c_int32),
                 ("staged_bridge_kb", c_int32), ("staged_max_mb", c_int32),
-                ("hbm_workgroups", c_int32), ("hbm_wg_threads", c_int32),
+                ("hbm_workgroups", c_int32), ("hbm_wg_threads", c_int32), ("hbm_unroll", c_int32),
                 ("ce_staging_mb", c_int32), ("ce_two_streams", c_int32),
-                ("reserved", c_int32 * 8)]
+                ("reserved", c_int32 * 7)]
 
 
 # name -> (restype, argtypes); the complete export list of include/fkv_transfer.h
@@ -246,6 +246,8 @@ SIGNATURES = {
     "fkv_ipc_close": (c_int32, [c_void_p]),
     "fkv_get_stats": (None, [POINTER(Stats)]),
     "fkv_reset_stats": (None, []),
+    "fkv_measure_hbm_rate": (c_int32, [c_int32, c_size_t, c_int32, c_int32,
+                                       POINTER(c_double), POINTER(c_double)]),
     "fkv_launch_policy_get": (c_int32, [c_int32, POINTER(LaunchPolicy)]),
     "fkv_launch_policy_set": (c_int32, [c_int32, POINTER(LaunchPolicy)]),
     "fkv_launch_policy_reset": (c_int32, [c_int32]),

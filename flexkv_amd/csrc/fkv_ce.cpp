@@ -484,6 +484,7 @@ int device_staging_copy(const fkv_transfer_desc &d, int it0, int nit, int p0, in
       a.lk = lk;
       a.vec = common_vector_width(&acc, 1);
       a.nt_store = 1;
+      a.unroll = pol.hbm_unroll;
       rc = launch_copy_kernel(a, kStagingWorkgroups, kStagingThreads, stream);
     }
     plan_release(slot, stream, false);

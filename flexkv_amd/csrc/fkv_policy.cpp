@@ -107,6 +107,7 @@ void sanitize(fkv_launch_policy &p, const fkv_launch_policy &derived) {
   p.staged_max_mb = clampi(p.staged_max_mb, 1, 1 << 16);
   p.hbm_workgroups = clampi(p.hbm_workgroups, 1, 1 << 16);
   p.hbm_wg_threads = clampi(p.hbm_wg_threads, 64, kCopyBlockThreads);
+  p.hbm_unroll = p.hbm_unroll >= kCopyUnrollDeep ? kCopyUnrollDeep : kCopyUnroll;
   p.ce_staging_mb = clampi(p.ce_staging_mb, 1, 1 << 18);
   p.ce_two_streams = p.ce_two_streams != 0;
 }
@@ -140,8 +141,9 @@ fkv_launch_policy defaults_for(uint32_t present) {
   p.staged_overhead_pct = 10;
   p.staged_bridge_kb = 512;
   p.staged_max_mb = 512;
-  p.hbm_workgroups = 2048;
+  p.hbm_workgroups = 8192;
   p.hbm_wg_threads = 1024;
+  p.hbm_unroll = kCopyUnrollDeep;
   p.ce_staging_mb = 1024;
   p.ce_two_streams = 1;
   for (const EnvField &f : kEnv) {

@@ -266,6 +266,7 @@ int staged_launch(const StagedPlan &sp, StagedRing &ring, const KernelPlan &kp, 
   a.nt_store = 1;
   a.xcd_mask = 0;
   const fkv_launch_policy pol = policy_of(kp.device);
+  a.unroll = pol.hbm_unroll;
   FKV_TRY(launch_copy_kernel(a, pol.hbm_workgroups, pol.hbm_wg_threads, scatter_stream));
   FKV_HIP_TRY(hipEventRecord(ring.freed[k], scatter_stream));
   ring.used[k] = true;

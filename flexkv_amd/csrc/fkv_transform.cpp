@@ -93,6 +93,7 @@ extern "C" int fkv_layout_transform(const fkv_layout_transform_desc *dp, void *s
       a.lk = lk;
       a.vec = common_vector_width(&acc, 1);
       a.nt_store = 1;
+      a.unroll = pol.hbm_unroll;
       a.xcd_mask = 0;
       rc = launch_copy_kernel(a, workgroups, threads, stream);
     }

@@ -563,6 +563,14 @@ typedef struct fkv_stats {
 void fkv_get_stats(fkv_stats *out);
 void fkv_reset_stats(void);
 
+/* HBM reference rates for the launches whose both ends are device memory (device
+ * staging, layout transform): `reps` launches of a streaming kernel over `bytes` of
+ * contiguous device memory owned by the call, timed with hip events.  mode: 0 = read
+ * only, 1 = write only, 2 = copy (result counts bytes read + bytes written).  GB/s
+ * (1e9 B/s) of the best repetition.  No counterpart in the reference. */
+int fkv_measure_hbm_rate(int32_t device, size_t bytes, int32_t reps, int32_t mode,
+                         double *best_gbps, double *median_gbps);
+
 /* ---- launch policy: every tunable of the kernel path, per device, in one table ----
  *
  * No counterpart in the reference, whose only launch parameter is transfer_num_cta.
@@ -618,9 +626,10 @@ typedef struct fkv_launch_policy {
    * the scatter of a staged restore */
   int32_t hbm_workgroups;
   int32_t hbm_wg_threads;
+  int32_t hbm_unroll;         /* 16-byte vectors in flight per lane in these launches: 8 or 16 */
   int32_t ce_staging_mb;      /* FKV_CE_STAGING_MB: device staging of the copy-engine strategies */
   int32_t ce_two_streams;     /* direct copy-engine strategies fan out over a second stream */
-  int32_t reserved[8];
+  int32_t reserved[7];
 } fkv_launch_policy;
 /* The table of `device` (-1 = current).  The first call for a device runs the probe kernel. */
 int fkv_launch_policy_get(int32_t device, fkv_launch_policy *out);
