@@ -886,6 +886,52 @@ def run_layout_transform(torch, device, steps, warmup, shape, verify=True):
     return res
 
 
+def run_staging(torch, device, steps, warmup, num_cta):
+    """Variable-size payloads between a dense device staging buffer and the host cache
+    with a host-side size table (the device half of a compressed transfer around the
+    codec): c0-shaped slots (32 layers x K+V x 32 KiB, 256 blocks = 16384 chunks), payload
+    sizes uniform in 50-90 % of a slot.  GB/s of payload bytes, both directions."""
+    import numpy as np
+    from flexkv_amd.c_ext import staging_transfer
+    L, K, NB, N, cap = 32, 2, 256, 1024, 32768
+    total = L * K * NB
+    g = torch.Generator().manual_seed(11)
+    sizes_h = torch.randint(cap // 2, cap * 9 // 10, (total,), generator=g, dtype=torch.int64)
+    sizes = sizes_h.to(device)
+    staging = torch.randint(0, 256, (total * cap,), dtype=torch.uint8, device=device)
+    host = torch.zeros(N * L * K * cap, dtype=torch.uint8, pin_memory=True)
+    table = torch.zeros(N * L * K, dtype=torch.int32, pin_memory=True)
+    ids = torch.randperm(N, generator=g)[:NB].to(torch.int64)
+    overflow = torch.zeros(1, dtype=torch.int32, device=device)
+    payload = int(sizes_h.sum())
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+
+    def timed(write, sz):
+        ms = []
+        for it in range(warmup + steps):
+            a, b = ev(), ev()
+            a.record()
+            staging_transfer(staging, cap, sz, host, cap, overflow, cap, K * cap, L * K * cap, ids,
+                             table, L * K, K, 0, K, 0, total, write, transfer_num_cta=num_cta)
+            b.record()
+            b.synchronize()
+            if it >= warmup:
+                ms.append(a.elapsed_time(b))
+        return _median(ms)
+    write_ms = timed(True, sizes)
+    want = staging.clone()
+    staging.zero_()
+    got_sizes = torch.zeros_like(sizes)
+    read_ms = timed(False, got_sizes)
+    # every payload came back, sizes restored from the table, nothing beyond a payload written
+    idx = torch.arange(cap, device=device).unsqueeze(0) < sizes.unsqueeze(1)
+    ok = bool(torch.equal(got_sizes, sizes)) and int(overflow.item()) == 0 and bool(
+        torch.equal(staging.view(total, cap)[idx], want.view(total, cap)[idx])) and not bool(
+        staging.view(total, cap)[~idx].any())
+    return dict(write_ms=write_ms, read_ms=read_ms, payload_bytes=payload, chunks=total,
+                bit_exact=ok)
+
+
 def run_ssd(torch, steps, warmup, ssd_dir, blocks, pinned):
     """Host pool <-> SSD files in the shape of the reference's SSD microbenchmark
     (benchmarks/microbenchmark_ssd_simulation.py): "small" MHA preset, both pool
@@ -1192,7 +1238,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--config", default="all",
                     choices=["all", "c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker",
-                             "ssd", "transform", "groups"])
+                             "ssd", "transform", "groups", "staging"])
     ap.add_argument("--shape", default="c0", choices=["c0", "c3"],
                     help="transform: which engine shape to re-lay out")
     ap.add_argument("--streams-per-direction", type=int, default=32,
@@ -1291,6 +1337,26 @@ def main():
         return
     if args.config == "transform":
         print(json.dumps(transform_record(torch, device, args, args.steps, args.warmup)))
+        return
+    if args.config == "staging":
+        link = measure_link()
+        r = run_staging(torch, device, args.steps, args.warmup, args.num_cta)
+        wr = r["payload_bytes"] / (r["write_ms"] * 1e-3) / 1e9
+        rd = r["payload_bytes"] / (r["read_ms"] * 1e-3) / 1e9
+        print(json.dumps({
+            "metric": "compressed-staging payloads <-> host cache, GB/s of payload (to host, from host)",
+            "unit": "GB/s", "value": round((wr + rd) / 2, 3), "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(r["write_ms"] + r["read_ms"], 3),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
+            "data": "synthetic",
+            "config": {"workload": "staging: 16384 slots of 32 KiB (32 layers x K+V x 256 blocks), "
+                                   "payloads uniform in 16-29 KiB, block-first host cache, uint32 "
+                                   "size table", "transfer_num_cta": args.num_cta},
+            "to_host_GBps": round(wr, 3), "from_host_GBps": round(rd, 3),
+            "to_host_frac_of_link": round(wr / link["d2h"], 4),
+            "from_host_frac_of_link": round(rd / link["h2d"], 4),
+            "payload_bytes": r["payload_bytes"], "chunks": r["chunks"], "bit_exact": r["bit_exact"],
+            "link_peak": {"d2h_GBps": round(link["d2h"], 3), "h2d_GBps": round(link["h2d"], 3)}}))
         return
     if args.config == "mg":
         link = measure_link()

@@ -143,6 +143,28 @@ class LayerwiseCall(Structure):
                 ("swa_cpu_block_stride", c_int64)]
 
 
+class StagingTransferDesc(Structure):
+    _fields_ = [("staging", c_void_p), ("staging_stride", c_int64), ("comp_sizes", c_void_p),
+                ("cpu_ptr", c_void_p), ("chunk_capacity", c_int64), ("overflow", c_void_p),
+                ("cpu_kv_stride", c_int64), ("cpu_layer_stride", c_int64),
+                ("cpu_block_stride", c_int64), ("cpu_block_ids", c_void_p),
+                ("size_table", c_void_p), ("size_table_block_stride", c_int64),
+                ("size_table_layer_stride", c_int64),
+                ("start_layer_id", c_int32), ("kv_dim", c_int32), ("num_blocks", c_int32),
+                ("batch_start", c_int32), ("bsz", c_int32), ("is_write_cpu", c_int32),
+                ("transfer_num_cta", c_int32), ("device", c_int32), ("sync", c_int32)]
+
+
+class ChunkPtrsDesc(Structure):
+    _fields_ = [("out_ptrs", c_void_p), ("backend", c_int32), ("num_layers_total", c_int32),
+                ("gpu_tensor_ptrs", c_void_p), ("num_gpu_tensor_ptrs", c_int32),
+                ("device", c_int32),
+                ("gpu_kv_stride", c_int64), ("gpu_block_stride", c_int64),
+                ("gpu_layer_stride", c_int64), ("gpu_block_ids", c_void_p),
+                ("start_layer_id", c_int32), ("kv_dim", c_int32), ("num_blocks", c_int32),
+                ("batch_start", c_int32), ("bsz", c_int32), ("sync", c_int32)]
+
+
 class Stats(Structure):
     _fields_ = [("calls", c_uint64), ("bytes_h2d", c_uint64), ("bytes_d2h", c_uint64),
                 ("kernel_launches", c_uint64), ("dma_copies", c_uint64),
@@ -246,6 +268,8 @@ SIGNATURES = {
     "fkv_ipc_close": (c_int32, [c_void_p]),
     "fkv_get_stats": (None, [POINTER(Stats)]),
     "fkv_reset_stats": (None, []),
+    "fkv_staging_transfer": (c_int32, [POINTER(StagingTransferDesc), c_void_p]),
+    "fkv_build_gpu_chunk_ptrs": (c_int32, [POINTER(ChunkPtrsDesc), c_void_p]),
     "fkv_measure_hbm_rate": (c_int32, [c_int32, c_size_t, c_int32, c_int32,
                                        POINTER(c_double), POINTER(c_double)]),
     "fkv_launch_policy_get": (c_int32, [c_int32, POINTER(LaunchPolicy)]),

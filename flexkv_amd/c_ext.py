@@ -241,6 +241,89 @@ def layout_transform(
     check(_L.fkv_layout_transform(ctypes.byref(d), _current_stream_handle()))
 
 
+def staging_transfer(
+        comp_staging: torch.Tensor, staging_stride_in_bytes: int, comp_sizes: torch.Tensor,
+        cpu_tensor: torch.Tensor, chunk_capacity_in_bytes: int, overflow: Optional[torch.Tensor],
+        cpu_kv_stride_in_bytes: int, cpu_layer_stride_in_bytes: int, cpu_block_stride_in_bytes: int,
+        cpu_block_id_tensor: torch.Tensor, cpu_size_table: torch.Tensor,
+        cpu_size_table_block_stride: int, cpu_size_table_layer_stride: int, start_layer_id: int,
+        kv_dim: int, batch_start: int, bsz: int, is_write_cpu: bool, transfer_num_cta: int = 0,
+        sync: bool = False) -> None:
+    """Payloads of different sizes between a dense device staging buffer and the host
+    cache on the current stream, sizes kept in a host-side uint32 table
+    (``staging_transfer_kernel<is_write_cpu>``,
+    ``csrc/compression/common/staging_transfer.cuh:16-101``; same argument order).
+
+    ``comp_staging`` (device, uint8) holds ``bsz`` slots of ``staging_stride`` bytes,
+    ``comp_sizes`` (device, uint64-as-int64) their sizes, ``overflow`` a device int32
+    counter of payloads that did not fit (may be None when reading).  ``cpu_tensor``
+    and ``cpu_size_table`` are pinned host tensors, the block ids a host tensor."""
+    ids = _ids(cpu_block_id_tensor, "cpu_block_id_tensor")
+    if comp_staging.device.type != "cuda" or comp_sizes.device.type != "cuda":
+        raise ValueError("comp_staging and comp_sizes must live in device memory")
+    if comp_sizes.dtype not in (torch.int64, torch.uint64) or comp_sizes.numel() < bsz:
+        raise ValueError("comp_sizes must hold bsz 64-bit sizes")
+    if cpu_size_table.dtype not in (torch.int32, torch.uint32):
+        raise ValueError("cpu_size_table must hold 32-bit entries")
+    if comp_staging.numel() * comp_staging.element_size() < int(bsz) * int(staging_stride_in_bytes):
+        raise ValueError("comp_staging is shorter than bsz slots of staging_stride bytes")
+    if overflow is not None and (overflow.device.type != "cuda" or overflow.dtype != torch.int32):
+        raise ValueError("overflow must be a device int32 tensor")
+    d = _lib.StagingTransferDesc()
+    d.staging = comp_staging.data_ptr()
+    d.staging_stride = int(staging_stride_in_bytes)
+    d.comp_sizes = comp_sizes.data_ptr()
+    d.cpu_ptr = cpu_tensor.data_ptr()
+    d.chunk_capacity = int(chunk_capacity_in_bytes)
+    d.overflow = overflow.data_ptr() if overflow is not None else None
+    d.cpu_kv_stride = int(cpu_kv_stride_in_bytes)
+    d.cpu_layer_stride = int(cpu_layer_stride_in_bytes)
+    d.cpu_block_stride = int(cpu_block_stride_in_bytes)
+    d.cpu_block_ids = ids.data_ptr()
+    d.size_table = cpu_size_table.data_ptr()
+    d.size_table_block_stride = int(cpu_size_table_block_stride)
+    d.size_table_layer_stride = int(cpu_size_table_layer_stride)
+    d.start_layer_id, d.kv_dim, d.num_blocks = int(start_layer_id), int(kv_dim), ids.numel()
+    d.batch_start, d.bsz = int(batch_start), int(bsz)
+    d.is_write_cpu = int(bool(is_write_cpu))
+    d.transfer_num_cta = int(transfer_num_cta)
+    d.device = comp_staging.device.index if comp_staging.device.index is not None else -1
+    d.sync = int(bool(sync))
+    check(_L.fkv_staging_transfer(ctypes.byref(d), _current_stream_handle()))
+
+
+def build_gpu_chunk_ptrs(
+        out_ptrs: torch.Tensor, gpu_tensor_ptrs_tensor: torch.Tensor, gpu_kv_stride_in_bytes: int,
+        gpu_block_stride_in_bytes: int, gpu_layer_stride_in_bytes: int,
+        gpu_block_id_tensor: torch.Tensor, start_layer_id: int, kv_dim: int, batch_start: int,
+        bsz: int, num_layers: int, gpu_block_type: int = 0, sync: bool = False) -> None:
+    """``out_ptrs[i]`` (device, int64) = address of chunk ``batch_start + i`` of the call in
+    the engine's tensors, chunks numbered layer-major, then K/V, then block position
+    (``build_gpu_chunk_ptrs_kernel<Type>``,
+    ``csrc/compression/common/staging_transfer.cuh:103-122``)."""
+    ids = _ids(gpu_block_id_tensor, "gpu_block_id_tensor")
+    ptrs = _ids(gpu_tensor_ptrs_tensor, "gpu_tensor_ptrs_tensor")
+    if out_ptrs.device.type != "cuda" or out_ptrs.dtype not in (torch.int64, torch.uint64):
+        raise ValueError("out_ptrs must be a 64-bit device tensor")
+    if out_ptrs.numel() < bsz:
+        raise ValueError("out_ptrs is shorter than bsz")
+    d = _lib.ChunkPtrsDesc()
+    d.out_ptrs = out_ptrs.data_ptr()
+    d.backend = int(gpu_block_type)
+    d.num_layers_total = ptrs.numel() // 2 if int(gpu_block_type) == 2 else int(num_layers)
+    d.gpu_tensor_ptrs = ptrs.data_ptr()
+    d.num_gpu_tensor_ptrs = ptrs.numel()
+    d.device = out_ptrs.device.index if out_ptrs.device.index is not None else -1
+    d.gpu_kv_stride = int(gpu_kv_stride_in_bytes)
+    d.gpu_block_stride = int(gpu_block_stride_in_bytes)
+    d.gpu_layer_stride = int(gpu_layer_stride_in_bytes)
+    d.gpu_block_ids = ids.data_ptr()
+    d.start_layer_id, d.kv_dim, d.num_blocks = int(start_layer_id), int(kv_dim), ids.numel()
+    d.batch_start, d.bsz = int(batch_start), int(bsz)
+    d.sync = int(bool(sync))
+    check(_L.fkv_build_gpu_chunk_ptrs(ctypes.byref(d), _current_stream_handle()))
+
+
 def streams_run_concurrently(stream_a, stream_b, device: int = -1) -> bool:
     """Whether kernels on the two torch streams can overlap, i.e. whether the
     streams sit on different hardware queues of this process.  Synchronises both."""

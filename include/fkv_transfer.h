@@ -563,6 +563,64 @@ typedef struct fkv_stats {
 void fkv_get_stats(fkv_stats *out);
 void fkv_reset_stats(void);
 
+/* ---- compressed staging: the codec-independent device half -------------------
+ *
+ * A batched codec (nvcomp ANS in the reference, csrc/compression/ans/nvcomp_ans.cu:355-500)
+ * works on a table of chunk addresses and leaves payloads of different sizes in a dense
+ * staging buffer.  These two calls are what surrounds it: the address table, and the
+ * movement of the payloads between staging and the host cache with their sizes recorded
+ * in a host-side table.  Chunk i of a batch is chunk g = batch_start + i of the call:
+ *   layer = g / (kv_dim * num_blocks), kv = (g % (kv_dim * num_blocks)) / num_blocks,
+ *   b = g % num_blocks.
+ * Block ids are host arrays here (the reference hands its kernels device-readable ones). */
+
+/* Replaces staging_transfer_kernel<is_write_cpu>
+ * (csrc/compression/common/staging_transfer.cuh:16-101).
+ *   is_write_cpu != 0: payload i (comp_sizes[i] bytes at staging + i * staging_stride) goes
+ *     to the host slot of its chunk and its size into the size table; a payload larger than
+ *     chunk_capacity is not copied, its table entry becomes 0 and *overflow is incremented.
+ *   is_write_cpu == 0: the table entry of chunk i says how many bytes to read from its host
+ *     slot into staging slot i; the size is also stored into comp_sizes[i].  An entry larger
+ *     than staging_stride (the reference would overrun the slot) is not copied:
+ *     comp_sizes[i] = 0 and *overflow is incremented when a counter was given. */
+typedef struct fkv_staging_transfer_desc {
+  void *staging;            /* device memory, bsz slots of staging_stride bytes */
+  int64_t staging_stride;
+  uint64_t *comp_sizes;     /* device memory, [bsz] */
+  void *cpu_ptr;            /* host cache, pinned / device-visible */
+  int64_t chunk_capacity;   /* bytes of one host slot */
+  int32_t *overflow;        /* device memory counter (the caller clears and reads it); may be
+                               NULL when reading */
+  int64_t cpu_kv_stride, cpu_layer_stride, cpu_block_stride; /* bytes */
+  const int64_t *cpu_block_ids; /* host array, [num_blocks] */
+  uint32_t *size_table;     /* host memory, pinned / device-visible */
+  int64_t size_table_block_stride, size_table_layer_stride; /* in entries; K and V adjacent */
+  int32_t start_layer_id, kv_dim, num_blocks, batch_start, bsz;
+  int32_t is_write_cpu;
+  int32_t transfer_num_cta; /* 0 = default */
+  int32_t device;           /* -1 = current */
+  int32_t sync;             /* wait for the stream before returning */
+} fkv_staging_transfer_desc;
+int fkv_staging_transfer(const fkv_staging_transfer_desc *desc, void *stream);
+
+/* Replaces build_gpu_chunk_ptrs_kernel<Type>
+ * (csrc/compression/common/staging_transfer.cuh:103-122): out_ptrs[i] = address of chunk
+ * (start_layer_id + layer, kv, gpu_block_ids[b]) in the engine's tensors, ptr_at<> of
+ * csrc/gtensor_handler.cuh:43-67. */
+typedef struct fkv_chunk_ptrs_desc {
+  void **out_ptrs;          /* device memory, [bsz] */
+  int32_t backend;          /* FKV_BACKEND_* */
+  int32_t num_layers_total;
+  const uint64_t *gpu_tensor_ptrs; /* host array */
+  int32_t num_gpu_tensor_ptrs;
+  int32_t device;           /* -1 = current */
+  int64_t gpu_kv_stride, gpu_block_stride, gpu_layer_stride; /* bytes */
+  const int64_t *gpu_block_ids; /* host array, [num_blocks] */
+  int32_t start_layer_id, kv_dim, num_blocks, batch_start, bsz;
+  int32_t sync;
+} fkv_chunk_ptrs_desc;
+int fkv_build_gpu_chunk_ptrs(const fkv_chunk_ptrs_desc *desc, void *stream);
+
 /* HBM reference rates for the launches whose both ends are device memory (device
  * staging, layout transform): `reps` launches of a streaming kernel over `bytes` of
  * contiguous device memory owned by the call, timed with hip events.  mode: 0 = read

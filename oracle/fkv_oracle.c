@@ -44,6 +44,13 @@
  *                             into a shaped [block, layer, kv, chunk] buffer,
  *                             for the three engine layouts; padded buffer
  *                             strides leave the padding untouched; round trip
+ *   fkv_oracle_staging_transfer  a second, shaped statement in numpy (host cache
+ *                             [N, L, kv, capacity] and size table [N, L, kv] indexed
+ *                             by (layer, kv, id) in Python loops), oversize payloads,
+ *                             batches that start and end inside a layer, write ->
+ *                             read round trip (tests/test_staging.py)
+ *   fkv_oracle_chunk_ptrs     equality with fkv_oracle_chunk_addr per (layer, kv,
+ *                             block) enumerated in Python, all three engines
  */
 #include <stdint.h>
 #include <stdlib.h>
@@ -422,6 +429,79 @@ int fkv_oracle_layout_transform(uint8_t *buffer, int64_t buffer_layer_stride,
       memcpy(gpu, buf, (size_t)chunk);
     else
       memcpy(buf, gpu, (size_t)chunk);
+  }
+  return 0;
+}
+
+/* csrc/compression/common/staging_transfer.cuh:16-101 (staging_transfer_kernel):
+ * chunk i of the batch is chunk g = batch_start + i of the call,
+ *   layer = g / (kv_dim*num_blocks), kv = (g % (kv_dim*num_blocks)) / num_blocks,
+ *   b = g % num_blocks;
+ * host slot = cpu + (layer+start_layer)*cLs + kv*cKs + cpu_ids[b]*cBs,
+ * table entry = table + cpu_ids[b]*tBs + (start_layer+layer)*tLs + kv.
+ * Write: size > capacity -> ++overflow, entry = 0, no copy; else entry = size and
+ * `size` bytes go staging -> host.  Read: size = entry, comp_sizes[i] = size, `size`
+ * bytes go host -> staging.  The reference does not guard a read entry larger than
+ * the staging slot (it would overrun it); here such an entry is counted in
+ * *overflow, comp_sizes[i] = 0 and nothing is copied.  `overflow` may be NULL. */
+void fkv_oracle_staging_transfer(uint8_t *staging, int64_t staging_stride, uint64_t *comp_sizes,
+                                 uint8_t *cpu, int64_t chunk_capacity, int32_t *overflow,
+                                 int64_t cpu_kv_stride, int64_t cpu_layer_stride,
+                                 int64_t cpu_block_stride, const int64_t *cpu_ids,
+                                 uint32_t *size_table, int64_t table_block_stride,
+                                 int64_t table_layer_stride, int start_layer, int kv_dim,
+                                 int num_blocks, int batch_start, int bsz, int is_write_cpu) {
+  for (int64_t i = 0; i < bsz; ++i) {
+    const int64_t g = (int64_t)batch_start + i;
+    const int64_t layer = g / ((int64_t)kv_dim * num_blocks);
+    const int64_t kv = (g % ((int64_t)kv_dim * num_blocks)) / num_blocks;
+    const int64_t b = g % num_blocks;
+    uint8_t *slot = cpu + (layer + start_layer) * cpu_layer_stride + kv * cpu_kv_stride +
+                    cpu_ids[b] * cpu_block_stride;
+    uint32_t *entry = size_table + cpu_ids[b] * table_block_stride +
+                      (start_layer + layer) * table_layer_stride + kv;
+    uint8_t *payload = staging + i * staging_stride;
+    if (is_write_cpu) {
+      const uint64_t sz = comp_sizes[i];
+      if (sz > (uint64_t)chunk_capacity) {
+        if (overflow)
+          ++*overflow;
+        *entry = 0;
+        continue;
+      }
+      *entry = (uint32_t)sz;
+      memcpy(slot, payload, (size_t)sz);
+    } else {
+      const uint64_t sz = *entry;
+      if (sz > (uint64_t)staging_stride) {
+        if (overflow)
+          ++*overflow;
+        comp_sizes[i] = 0;
+        continue;
+      }
+      comp_sizes[i] = sz;
+      memcpy(payload, slot, (size_t)sz);
+    }
+  }
+}
+
+/* csrc/compression/common/staging_transfer.cuh:103-122 (build_gpu_chunk_ptrs_kernel):
+ * out[i] = ptr_at(start_layer + layer, kv, gpu_ids[b]) with the same numbering. */
+int fkv_oracle_chunk_ptrs(uint64_t *out, int backend, const uint64_t *tensor_ptrs,
+                          int64_t num_layers_total, int64_t gpu_kv_stride,
+                          int64_t gpu_block_stride, int64_t gpu_layer_stride,
+                          const int64_t *gpu_ids, int start_layer, int kv_dim, int num_blocks,
+                          int batch_start, int bsz) {
+  if (backend < 0 || backend > 2)
+    return -1;
+  for (int64_t i = 0; i < bsz; ++i) {
+    const int64_t g = (int64_t)batch_start + i;
+    const int64_t layer = g / ((int64_t)kv_dim * num_blocks);
+    const int64_t kv = (g % ((int64_t)kv_dim * num_blocks)) / num_blocks;
+    const int64_t b = g % num_blocks;
+    out[i] = fkv_oracle_chunk_addr(backend, tensor_ptrs, num_layers_total, gpu_kv_stride,
+                                   gpu_block_stride, gpu_layer_stride, start_layer + layer, kv,
+                                   gpu_ids[b]);
   }
   return 0;
 }

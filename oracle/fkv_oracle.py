@@ -107,6 +107,12 @@ def lib() -> ctypes.CDLL:
         L.fkv_oracle_layout_transform.argtypes = [vp, i64, i64, i64, i64, i32, vp, i64, i64, i64,
                                                   i64, vp, i32, i32, i32, i32, i32]
         L.fkv_oracle_layout_transform.restype = i32
+        L.fkv_oracle_staging_transfer.argtypes = [vp, i64, vp, vp, i64, vp, i64, i64, i64, vp, vp,
+                                                  i64, i64, i32, i32, i32, i32, i32, i32]
+        L.fkv_oracle_staging_transfer.restype = None
+        L.fkv_oracle_chunk_ptrs.argtypes = [vp, i32, vp, i64, i64, i64, i64, vp, i32, i32, i32,
+                                            i32, i32]
+        L.fkv_oracle_chunk_ptrs.restype = i32
         L.fkv_oracle_eventfd_index.argtypes = [i32] * 5
         L.fkv_oracle_eventfd_index.restype = i64
         L.fkv_oracle_host_chunk_bytes.argtypes = [ctypes.c_double]
@@ -157,6 +163,42 @@ def layout_transform(buffer_ptr: int, buffer_layer_stride: int, buffer_kv_stride
         _ptr(g), int(g.size), start_layer, num_layers, kv_dim, int(bool(buffer_to_target)))
     if rc != 0:
         raise ValueError(f"oracle layout transform rejected backend {backend}")
+
+
+def staging_transfer(staging: np.ndarray, staging_stride: int, comp_sizes: np.ndarray,
+                     cpu: np.ndarray, chunk_capacity: int, cpu_kv_stride: int,
+                     cpu_layer_stride: int, cpu_block_stride: int, cpu_ids, size_table: np.ndarray,
+                     table_block_stride: int, table_layer_stride: int, start_layer: int,
+                     kv_dim: int, num_blocks: int, batch_start: int, bsz: int,
+                     is_write_cpu: bool) -> int:
+    """Payloads of different sizes between a dense staging buffer (uint8) and the
+    host cache (uint8) with their sizes in ``size_table`` (uint32); ``comp_sizes`` is
+    uint64.  All arrays are host memory, modified in place.  Returns the number of
+    chunks that did not fit."""
+    assert staging.dtype == np.uint8 and cpu.dtype == np.uint8
+    assert comp_sizes.dtype == np.uint64 and size_table.dtype == np.uint32
+    ids = _i64(cpu_ids)
+    overflow = np.zeros(1, dtype=np.int32)
+    lib().fkv_oracle_staging_transfer(
+        _ptr(staging), staging_stride, _ptr(comp_sizes), _ptr(cpu), chunk_capacity, _ptr(overflow),
+        cpu_kv_stride, cpu_layer_stride, cpu_block_stride, _ptr(ids), _ptr(size_table),
+        table_block_stride, table_layer_stride, start_layer, kv_dim, num_blocks, batch_start, bsz,
+        int(bool(is_write_cpu)))
+    return int(overflow[0])
+
+
+def chunk_ptrs(backend, tensor_ptrs, num_layers_total, kvs, bs, ls, gpu_ids, start_layer, kv_dim,
+               batch_start, bsz) -> np.ndarray:
+    """Addresses of the chunks of a batch, numbered layer-major, then K/V, then block."""
+    ptrs = np.ascontiguousarray(np.asarray(tensor_ptrs, dtype=np.uint64))
+    ids = _i64(gpu_ids)
+    out = np.zeros(bsz, dtype=np.uint64)
+    rc = lib().fkv_oracle_chunk_ptrs(_ptr(out), backend, _ptr(ptrs), num_layers_total, kvs, bs, ls,
+                                     _ptr(ids), start_layer, kv_dim, int(ids.size), batch_start,
+                                     bsz)
+    if rc != 0:
+        raise ValueError(f"oracle chunk_ptrs rejected backend {backend}")
+    return out
 
 
 def chunk_addr(backend, tensor_ptrs, num_layers_total, kvs, bs, ls, layer, kv, block) -> int:
