@@ -84,10 +84,19 @@ BoardHandle open_board(const std::string &key) {
   std::string name = "/dev/shm/fkv_link_" + std::to_string((unsigned)getuid()) + "_";
   for (char c : key)
     name += (std::isalnum((unsigned char)c) ? c : '_');
-  int fd = open(name.c_str(), O_RDWR | O_CREAT | O_CLOEXEC, 0600);
+  // The path is predictable: never follow a link planted there, and use the file
+  // only if it is a regular file of this user that is empty (new) or a board already.
+  int fd = open(name.c_str(), O_RDWR | O_CREAT | O_CLOEXEC | O_NOFOLLOW, 0600);
   if (fd < 0)
     return h;
-  if (ftruncate(fd, sizeof(Board)) != 0) {
+  struct stat st;
+  if (fstat(fd, &st) != 0 || !S_ISREG(st.st_mode) || st.st_uid != getuid() ||
+      (st.st_size != 0 && st.st_size != (off_t)sizeof(Board))) {
+    close(fd);
+    return h;
+  }
+  const bool fresh = st.st_size == 0;
+  if (fresh && ftruncate(fd, sizeof(Board)) != 0) {
     close(fd);
     return h;
   }
@@ -95,8 +104,16 @@ BoardHandle open_board(const std::string &key) {
   close(fd);
   if (p == MAP_FAILED)
     return h;
-  h.board = static_cast<Board *>(p); // a fresh file is all zeroes: no slot taken
-  h.board->magic.store(kBoardMagic, std::memory_order_relaxed);
+  Board *b = static_cast<Board *>(p); // a fresh file is all zeroes: no slot taken
+  // Whoever finds the magic absent writes it (a process that created the file at the
+  // same moment does the same); any other content is not a board and is left alone.
+  uint32_t expect = 0;
+  if (!b->magic.compare_exchange_strong(expect, kBoardMagic, std::memory_order_acq_rel) &&
+      expect != kBoardMagic) {
+    munmap(p, sizeof(Board));
+    return h;
+  }
+  h.board = b;
   claim_slot(h);
   return h;
 }
