@@ -58,10 +58,11 @@ int ring_prepare(StagedRing &ring, int slots, size_t bytes) {
   size_t cap = (bytes + (2u << 20) - 1) & ~(size_t)((2u << 20) - 1);
   for (int k = 0; k < slots; ++k) {
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&ring.buf[k]), cap);
-    // `copied` publishes bytes the copy engine wrote for a kernel on another
-    // stream: default fence.  `freed` only orders work.
+    // Both events only order work.  `copied` stands behind copy-engine writes, which
+    // pass no cache that a fence at the event would have to flush; the scatter
+    // kernel that waits on it invalidates its caches when it starts, like any kernel.
     if (e == hipSuccess)
-      e = hipEventCreateWithFlags(&ring.copied[k], hipEventDisableTiming);
+      e = hipEventCreateWithFlags(&ring.copied[k], kBookkeepingEvent);
     if (e == hipSuccess)
       e = hipEventCreateWithFlags(&ring.freed[k], kBookkeepingEvent);
     if (e != hipSuccess) {
