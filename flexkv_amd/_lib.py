@@ -296,8 +296,8 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.fkv_abi_version() != 1:
-        raise ImportError(f"{LIB_PATH}: ABI version {lib.fkv_abi_version()} != 1")
+    if lib.fkv_abi_version() != 2:
+        raise ImportError(f"{LIB_PATH}: ABI version {lib.fkv_abi_version()} != 2")
     _lib = lib
     return lib
 

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define FKV_ABI_VERSION 1
+#define FKV_ABI_VERSION 2 /* 2: fkv_stats grew by staged_batches; launch policy, no-alloc transfer, staging and HBM-rate entry points added */
 
 /* status codes */
 #define FKV_OK 0
