@@ -1167,8 +1167,11 @@ def measure_config(name, args, torch, device, link, steps, warmup):
         out.update(value=round(2 * B * steps / wall / 1e9, 3),
                    ms_per_step=round(wall / steps * 1e3, 3),
                    d2h_GBps=round(d2h, 3), h2d_GBps=round(h2d, 3),
+                   d2h_GiBps=round(d2h * 1e9 / 2**30, 3), h2d_GiBps=round(h2d * 1e9 / 2**30, 3),
                    d2h_frac_of_link=round(d2h / link["d2h"], 4),
                    h2d_frac_of_link=round(h2d / link["h2d"], 4),
+                   d2h_ms_median=round(_median(d2h_ms), 4), d2h_ms_min=round(min(d2h_ms), 4),
+                   h2d_ms_median=round(_median(h2d_ms), 4), h2d_ms_min=round(min(h2d_ms), 4),
                    avg_launch_ms=round(avg_ms, 4), path_taken=taken)
         if not args.no_verify:
             out["bit_exact"] = verify_round_trip(w, torch, args.num_cta)
@@ -1432,8 +1435,17 @@ def main():
     # c0, c2, c3 and c4 follow with `--other-steps` timed steps each.
     head = "c1"
     records = {head: measure_config(head, args, torch, device, link, args.steps, args.warmup)}
+    if not args.use_ce:
+        # c1 is also the configuration that is asked for on both engines: the same pages
+        # through the copy-engine strategies (the library's choice among them)
+        ce_args = argparse.Namespace(**{**vars(args), "use_ce": True, "no_verify": True})
+        ce = measure_config(head, ce_args, torch, device, link, min(3, args.steps), 2)  # staging buffers are allocated in the first calls
+        records[head]["copy_engine"] = {k: ce[k] for k in (
+            "d2h_GBps", "h2d_GBps", "d2h_frac_of_link", "h2d_frac_of_link", "path_taken", "steps")}
     for name in ("c0", "c2", "c3", "c4"):
-        records[name] = measure_config(name, args, torch, device, link, args.other_steps, 1)
+        # c4's latency percentiles want repetitions: 20 bursts of its 64 requests
+        records[name] = measure_config(name, args, torch, device, link,
+                                       20 if name == "c4" else args.other_steps, 1)
     rec = records[head]
     out.update(value=rec["value"], ms_per_step=rec["ms_per_step"],
                d2h_GBps=rec["d2h_GBps"], h2d_GBps=rec["h2d_GBps"],
