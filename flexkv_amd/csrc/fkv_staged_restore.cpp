@@ -177,7 +177,10 @@ int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &
   out->host0 = static_cast<const uint8_t *>(d.cpu_ptr) + d.cpu_startoff_inside_chunks;
   out->num_blocks = d.num_blocks;
 
-  FKV_TRY(ring_prepare(ring, pol.staged_ring, (size_t)slot_bytes));
+  if (ring_prepare(ring, pol.staged_ring, (size_t)slot_bytes) != FKV_OK) {
+    clear_error(); // no room for the staging buffers: the kernel path needs none
+    return FKV_OK;
+  }
   const int slots = (int)ring.buf.size();
   const size_t tab = (size_t)slots * lk * 8, rows_bytes = (size_t)d.num_blocks * 8;
   PlanSlot *slot = plan_acquire(device, tab + rows_bytes);

@@ -400,9 +400,17 @@ def test_layerwise_wait_layer_orders_a_consumer_stream(gpu_device):
     lw.close()
 
 
-def test_layerwise_all_write_offsets_two_ranks(gpu_device):
+@pytest.mark.parametrize("staged", [0, 2], ids=["kernel", "copy_engines"])
+def test_layerwise_all_write_offsets_two_ranks(gpu_device, staged):
     """all_write restore: rank r reads its own region of the host pool
-    (csrc/layerwise.cpp:1155-1162)."""
+    (csrc/layerwise.cpp:1155-1162); on the kernel path and through the copy engines
+    (a staging ring and a copy stream per rank)."""
+    from flexkv_amd.c_ext import launch_policy
+    with launch_policy(staged_restore=staged):
+        _all_write_two_ranks(gpu_device)
+
+
+def _all_write_two_ranks(gpu_device):
     n, L, N, T, H, D = 2, 3, 6, 4, 1, 64
     gl, cl = make_layouts(L, N, T, H, D, "BLOCKFIRST", 1, 1, cpu_blocks=N * n)
     all_gpu = [make_gpu_tensors(L, N, T, H, D, 1, gpu_device) for _ in range(n)]

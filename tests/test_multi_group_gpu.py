@@ -20,6 +20,16 @@ pytestmark = pytest.mark.gpu
 ENGINES = [False, True, "auto"]
 
 
+@pytest.fixture(autouse=True, params=[1, 2], ids=["restore_as_chosen", "restore_by_copy_engines"])
+def _staged_restore(request):
+    """Every case twice: with the library's own choice between the kernel path and
+    the copy engines (the small pools here stay on the kernel path), and with the
+    kernel-path restores forced through the copy engines and a staging ring."""
+    from flexkv_amd.c_ext import launch_policy
+    with launch_policy(staged_restore=request.param):
+        yield
+
+
 def _t6_groups(num_layers=4):
     main = LayerGroupSpec(num_layers, 1, MAIN_HEAD_SIZE, tuple(range(num_layers)), itemsize=1)
     indexer = LayerGroupSpec(3, 1, INDEXER_HEAD_SIZE, (1, 2, 3), itemsize=1)
