@@ -13,14 +13,14 @@ K timed steps) are c1's, and `configs` holds a record of each of c0..c4 with its
 GB/s, fraction of the link rate measured in the same run, bit-exactness and CPU
 baseline on its own shape.
 
-Configurations (BASELINE.json "configs"):
+The five benchmark configurations:
   c0  Llama-3-8B, vLLM layout, bf16: 32 x [2,4096,16,8,128]; 256 random blocks
   c1  SGLang token-major, bf16, page 64: 64 x [262144,8,128]; 1024 pages
       (64 runs of 8 + 512 isolated)                      <- the headline of the default run
   c2  TRT-LLM layout, fp8 e4m3: [4096,80,2,8,32,128]; 2048 random blocks
   c3  DeepSeek-V3 MLA, bf16: 61 x [16384,64,576]; layerwise restore of 512 blocks
   c4  64 concurrent requests on the c0 shape with a 32768-block pool
-Beyond BASELINE.json (the rows next to the path):
+Beyond those (the callers and formats either side of the path):
   mg      layerwise restore of heterogeneous layer groups + sliding-window sidecar
           (DeepSeek-V4-like: 61 layers, two compressed latent groups, an indexer group)
   worker  c0-shaped put/get ops through a transfer worker process (pipe + shared op pool)

@@ -4,8 +4,7 @@ under ThreadSanitizer.
 Two small native drivers (beside this file) include a host-only translation unit
 of the library each, run it on seeded random inputs against a plain model, and
 are built here with clang's sanitizers (statically linked runtime).  GPU code is
-not involved, and this folder is kept off the GPU box (it is listed in
-.gpurunignore): sanitizer builds belong on the CPU."""
+not involved and nothing here is marked gpu: sanitizer builds belong on the CPU."""
 import os
 import shutil
 import subprocess
