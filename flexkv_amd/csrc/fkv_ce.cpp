@@ -633,35 +633,67 @@ int gather_scatter(const Job &j) {
 // csrc/ce_transfer.cu:1183-1400.  Device staging holds whole host blocks
 // ([block][layer*kv][chunk] == the block-first host layout), so every DMA moves
 // at least one complete block and cpu-adjacent blocks merge into one DMA.
+// Positions of a transfer in ascending order of their host block ids, and the ids in
+// that order.  The device side of GATHER_DIRECT goes through the compaction kernel,
+// which takes the GPU blocks in any order; staging them in host order makes every
+// run of consecutive host blocks one copy command, however the GPU blocks lie
+// (1024 pages into host blocks 0..1023: 8 commands of 1 GiB instead of 578).
+struct HostOrder {
+  std::vector<int64_t> gpu_ids, cpu_ids;
+  std::vector<int> run_start; // first sorted position of every run, then the count as sentinel
+};
+HostOrder host_order(const fkv_transfer_desc &d) {
+  HostOrder o;
+  std::vector<int> pos(d.num_blocks);
+  for (int i = 0; i < d.num_blocks; ++i)
+    pos[i] = i;
+  std::stable_sort(pos.begin(), pos.end(),
+                   [&](int a, int b) { return d.cpu_block_ids[a] < d.cpu_block_ids[b]; });
+  o.gpu_ids.resize(d.num_blocks);
+  o.cpu_ids.resize(d.num_blocks);
+  for (int i = 0; i < d.num_blocks; ++i) {
+    o.gpu_ids[i] = d.gpu_block_ids[pos[i]];
+    o.cpu_ids[i] = d.cpu_block_ids[pos[i]];
+    if (i == 0 || o.cpu_ids[i] != o.cpu_ids[i - 1] + 1)
+      o.run_start.push_back(i);
+  }
+  o.run_start.push_back(d.num_blocks);
+  return o;
+}
+
 int gather_direct(const Job &j) {
-  const auto &d = j.d;
-  const int lk = d.num_layers * d.kv_dim;
-  const bool dense = (d.kv_dim == 1 || d.cpu_kv_stride == d.chunk_size) &&
-                     (d.num_layers == 1 || d.cpu_layer_stride == (int64_t)d.kv_dim * d.chunk_size);
+  const auto &d0 = j.d;
+  const int lk = d0.num_layers * d0.kv_dim;
+  const bool dense = (d0.kv_dim == 1 || d0.cpu_kv_stride == d0.chunk_size) &&
+                     (d0.num_layers == 1 || d0.cpu_layer_stride == (int64_t)d0.kv_dim * d0.chunk_size);
   if (!dense)
     return gather_scatter(j); // host chunks of a block are not adjacent: stage per (layer, kv)
+  const HostOrder order = host_order(d0);
+  fkv_transfer_desc d = d0; // the same transfer, positions in host order
+  d.gpu_block_ids = order.gpu_ids.data();
+  d.cpu_block_ids = order.cpu_ids.data();
   const size_t block_bytes = (size_t)lk * (size_t)d.chunk_size;
   const bool full_block = (int64_t)block_bytes == d.cpu_block_stride;
+  const bool merged = full_block || d.ce.enable_memcpy2d; // a run of host blocks is one command
   const int group =
       (int)std::min<size_t>((size_t)d.num_blocks, std::max<size_t>(1, staging_cap_bytes() / block_bytes));
   uint8_t *stage = device_stage(j.device, 0, (size_t)group * block_bytes, j.stream);
   if (!stage)
     return per_block(j);
   int rc = FKV_OK;
-  size_t seg_i = 0;
+  size_t run_i = 0;
   for (int p0 = 0; p0 < d.num_blocks && rc == FKV_OK; p0 += group) {
     const int np = std::min(group, d.num_blocks - p0);
     if (!j.h2d)
       rc = device_staging_copy(d, 0, lk, p0, np, stage, true, true, j.stream);
-    // segments (cpu- and gpu-adjacent runs) clipped to this group
+    // runs of consecutive host blocks, clipped to this group
     if (rc == FKV_OK)
-      rc = j.fan_out(full_block || d.ce.enable_memcpy2d ? j.an.segs.size() - seg_i : (size_t)np);
-    while (seg_i < j.an.segs.size() && rc == FKV_OK) {
-      const auto &s = j.an.segs[seg_i];
-      const int b = std::max(s.start_k, p0);
-      const int e = std::min(s.start_k + s.nr_blocks, p0 + np);
+      rc = j.fan_out(merged ? order.run_start.size() - 1 - run_i : (size_t)np);
+    while (run_i + 1 < order.run_start.size() && rc == FKV_OK) {
+      const int b = std::max(order.run_start[run_i], p0);
+      const int e = std::min(order.run_start[run_i + 1], p0 + np);
       if (b < e) {
-        uint8_t *c = j.cpu(0, 0, d.cpu_block_ids[b]);
+        uint8_t *c = cpu_chunk_ptr(d, (int64_t)d.start_layer_id, 0, d.cpu_block_ids[b]);
         uint8_t *g = stage + (size_t)(b - p0) * block_bytes;
         const size_t rows = (size_t)(e - b);
         if (full_block) {
@@ -676,9 +708,9 @@ int gather_direct(const Job &j) {
             rc = j.dma_dir(g + r * block_bytes, c + r * (size_t)d.cpu_block_stride, block_bytes);
         }
       }
-      if (s.start_k + s.nr_blocks > p0 + np)
-        break; // the rest of this segment belongs to the next group
-      ++seg_i;
+      if (order.run_start[run_i + 1] > p0 + np)
+        break; // the rest of this run belongs to the next group
+      ++run_i;
     }
     {
       int rc2 = j.fan_in();
@@ -789,7 +821,8 @@ CeWork ce_work(const Job &j, int path) {
   default: // GATHER_DIRECT
     if (host_block_dense(d)) {
       const bool full = iters * (double)d.chunk_size == (double)d.cpu_block_stride;
-      w.dmas = (full || d.ce.enable_memcpy2d) ? segs : n;
+      // one command per run of consecutive host blocks, whatever the GPU side looks like
+      w.dmas = (full || d.ce.enable_memcpy2d) ? (double)(host_order(d).run_start.size() - 1) : n;
       w.device_staged = bytes;
     } else {
       staged();
@@ -797,16 +830,6 @@ CeWork ce_work(const Job &j, int path) {
   }
   return w;
 }
-
-// Measured on MI355X: a DMA command costs about 2.5 us beyond its bytes when
-// copies alternate over two streams (256 x 2 MiB: 50-54 GB/s; 2048 x 5 MiB:
-// 56.2 GB/s); the compaction pass runs at 1.5 TB/s or more; a host
-// scatter/gather pass at about 20 GB/s with four threads; the gather/scatter
-// kernel reaches 56.4 GB/s GPU->host and 57.2 GB/s host->GPU.
-constexpr double kLinkBps = 57.2e9, kKernelD2HBps = 56.4e9, kKernelH2DBps = 57.2e9;
-constexpr double kDmaSeconds = 2.5e-6, kCompactionBps = 1.5e12, kHostPassBps = 20e9;
-constexpr double kLaunchSeconds = 15e-6;
-constexpr double kPreferCopyEngineWithin = 1.03; // it leaves the CUs and their memory queues alone
 
 } // namespace
 
@@ -819,14 +842,24 @@ int choose_engine(const fkv_transfer_desc &d, int *use_ce, double *kernel_s, dou
   FKV_TRY(resolve_path(j, &path));
   const CeWork w = ce_work(j, path);
   const double bytes = (double)d.num_blocks * d.num_layers * d.kv_dim * (double)d.chunk_size;
-  const double tk = bytes / (j.h2d ? kKernelH2DBps : kKernelD2HBps) + kLaunchSeconds;
-  const double tc = bytes / kLinkBps + w.dmas * kDmaSeconds + w.device_staged / kCompactionBps +
-                    w.host_staged / kHostPassBps;
+  // the rates and costs of the model are fields of the launch policy (no device call:
+  // a device whose table has not been built yet gets the defaults)
+  int device = d.device;
+  if (device < 0 && hipGetDevice(&device) != hipSuccess) {
+    (void)hipGetLastError();
+    device = 0;
+  }
+  const fkv_launch_policy pol = policy_peek(device);
+  const double tk = bytes / ((j.h2d ? pol.model_kernel_h2d_mbps : pol.model_kernel_d2h_mbps) * 1e6) +
+                    pol.model_launch_ns * 1e-9;
+  const double tc = bytes / (pol.model_link_mbps * 1e6) + w.dmas * pol.model_dma_ns * 1e-9 +
+                    w.device_staged / (pol.model_compaction_gbps * 1e9) +
+                    w.host_staged / (pol.model_host_pass_mbps * 1e6);
   if (kernel_s)
     *kernel_s = tk;
   if (ce_s)
     *ce_s = tc;
-  *use_ce = tc <= kPreferCopyEngineWithin * tk ? 1 : 0;
+  *use_ce = tc * 100.0 <= pol.model_prefer_ce_pct * tk ? 1 : 0;
   return FKV_OK;
 }
 

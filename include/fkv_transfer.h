@@ -687,6 +687,16 @@ typedef struct fkv_launch_policy {
   int32_t hbm_unroll;         /* 16-byte vectors in flight per lane in these launches: 8 or 16 */
   int32_t ce_staging_mb;      /* FKV_CE_STAGING_MB: device staging of the copy-engine strategies */
   int32_t ce_two_streams;     /* direct copy-engine strategies fan out over a second stream */
+  /* cost model of fkv_choose_engine (use_ce_transfer = 2): what each engine is expected to take */
+  int32_t model_link_mbps;          /* the link under plain copy-engine copies, MB/s */
+  int32_t model_kernel_d2h_mbps;    /* the gather/scatter kernel GPU->host */
+  int32_t model_kernel_h2d_mbps;    /* ... host->GPU */
+  int32_t model_dma_ns;             /* cost of one more copy command over two streams */
+  int32_t model_compaction_gbps;    /* device compaction pass, GB/s of bytes staged */
+  int32_t model_host_pass_mbps;     /* host scatter/gather pass */
+  int32_t model_launch_ns;          /* plan + launch of the kernel path */
+  int32_t model_prefer_ce_pct;      /* the copy engine wins up to this percentage of the kernel's
+                                       time: it leaves the CUs and their memory queues alone */
   int32_t reserved[7];
 } fkv_launch_policy;
 /* The table of `device` (-1 = current).  The first call for a device runs the probe kernel. */
