@@ -193,11 +193,12 @@ class LaunchPolicy(Structure):
                 ("staged_bridge_kb", c_int32), ("staged_max_mb", c_int32),
                 ("hbm_workgroups", c_int32), ("hbm_wg_threads", c_int32), ("hbm_unroll", c_int32),
                 ("ce_staging_mb", c_int32), ("ce_two_streams", c_int32),
+                ("ce_rect_min_kb", c_int32),
                 ("model_link_mbps", c_int32), ("model_kernel_d2h_mbps", c_int32),
                 ("model_kernel_h2d_mbps", c_int32), ("model_dma_ns", c_int32),
                 ("model_compaction_gbps", c_int32), ("model_host_pass_mbps", c_int32),
                 ("model_launch_ns", c_int32), ("model_prefer_ce_pct", c_int32),
-                ("reserved", c_int32 * 7)]
+                ("reserved", c_int32 * 6)]
 
 
 # name -> (restype, argtypes); the complete export list of include/fkv_transfer.h

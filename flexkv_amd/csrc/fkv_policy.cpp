@@ -110,6 +110,7 @@ void sanitize(fkv_launch_policy &p, const fkv_launch_policy &derived) {
   p.hbm_unroll = p.hbm_unroll >= kCopyUnrollDeep ? kCopyUnrollDeep : kCopyUnroll;
   p.ce_staging_mb = clampi(p.ce_staging_mb, 1, 1 << 18);
   p.ce_two_streams = p.ce_two_streams != 0;
+  p.ce_rect_min_kb = clampi(p.ce_rect_min_kb, -1, 1 << 24);
   p.model_link_mbps = clampi(p.model_link_mbps, 100, 10000000);
   p.model_kernel_d2h_mbps = clampi(p.model_kernel_d2h_mbps, 100, 10000000);
   p.model_kernel_h2d_mbps = clampi(p.model_kernel_h2d_mbps, 100, 10000000);
@@ -154,6 +155,8 @@ fkv_launch_policy defaults_for(uint32_t present) {
   p.hbm_unroll = kCopyUnrollDeep;
   p.ce_staging_mb = 1024;
   p.ce_two_streams = 1;
+  p.ce_rect_min_kb = -1; // 8 GiB in 1 GiB copies: the same rate either way; 5 MiB copies: 51 against
+                         // 56 GB/s; copies a host thread waits for one by one: far slower
   // Measured on MI355X: a DMA command costs about 2.5 us beyond its bytes when copies
   // alternate over two streams (256 x 2 MiB: 50-54 GB/s; 2048 x 5 MiB: 56.2 GB/s); the
   // compaction pass runs at 1.5 TB/s or more; a host scatter/gather pass at about

@@ -246,11 +246,14 @@ int staged_launch(const StagedPlan &sp, StagedRing &ring, const KernelPlan &kp, 
     for (const StagedPlan::Seg &s : sp.segs) {
       const uint8_t *src = src0 + s.first_id * sp.cpu_block_stride;
       uint8_t *dst = dst0 + (int64_t)s.row0 * w;
-      if (s.rows == 1 || sp.cpu_block_stride == w)
-        FKV_HIP_TRY(hipMemcpyAsync(dst, src, (size_t)s.rows * w, hipMemcpyHostToDevice, dma_stream));
-      else
-        FKV_HIP_TRY(hipMemcpy2DAsync(dst, (size_t)w, src, (size_t)sp.cpu_block_stride, (size_t)w,
-                                     (size_t)s.rows, hipMemcpyHostToDevice, dma_stream));
+      // Always the 2-D call, also for one row or adjacent rows: the runtime hands 2-D
+      // copies to the copy engines, while it runs hipMemcpyAsync between pinned host and
+      // device memory as a kernel on the compute units (seen in kernel traces: one
+      // __amd_rocclr_copyBuffer launch per 1-D copy of any size, none for 2-D copies),
+      // which is what this path exists to avoid.
+      const size_t pitch = s.rows == 1 ? (size_t)w : (size_t)sp.cpu_block_stride;
+      FKV_HIP_TRY(hipMemcpy2DAsync(dst, (size_t)w, src, pitch, (size_t)w, (size_t)s.rows,
+                                   hipMemcpyHostToDevice, dma_stream));
       ++copies;
     }
   }

@@ -687,6 +687,10 @@ typedef struct fkv_launch_policy {
   int32_t hbm_unroll;         /* 16-byte vectors in flight per lane in these launches: 8 or 16 */
   int32_t ce_staging_mb;      /* FKV_CE_STAGING_MB: device staging of the copy-engine strategies */
   int32_t ce_two_streams;     /* direct copy-engine strategies fan out over a second stream */
+  int32_t ce_rect_min_kb;     /* copies of at least this size are issued as 2-D copies of one row,
+                                 which the runtime hands to the copy engines (it runs 1-D
+                                 hipMemcpyAsync between pinned host and device memory as a kernel
+                                 on the compute units); 0 = all copies, -1 = none (default) */
   /* cost model of fkv_choose_engine (use_ce_transfer = 2): what each engine is expected to take */
   int32_t model_link_mbps;          /* the link under plain copy-engine copies, MB/s */
   int32_t model_kernel_d2h_mbps;    /* the gather/scatter kernel GPU->host */
@@ -697,7 +701,7 @@ typedef struct fkv_launch_policy {
   int32_t model_launch_ns;          /* plan + launch of the kernel path */
   int32_t model_prefer_ce_pct;      /* the copy engine wins up to this percentage of the kernel's
                                        time: it leaves the CUs and their memory queues alone */
-  int32_t reserved[7];
+  int32_t reserved[6];
 } fkv_launch_policy;
 /* The table of `device` (-1 = current).  The first call for a device runs the probe kernel. */
 int fkv_launch_policy_get(int32_t device, fkv_launch_policy *out);

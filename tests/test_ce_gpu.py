@@ -107,6 +107,34 @@ def test_forced_general_strategies(gpu_device, force, backend, L, K, N, NH, chun
             dev.assert_matches_reference(f"forced {force} {pattern} h2d={h2d}")
 
 
+@pytest.mark.parametrize("force", ["PER_BLOCK", "SEGMENT_SCATTER", "GATHER_SCATTER", "GATHER_DIRECT"])
+def test_every_copy_as_a_2d_copy_of_one_row(gpu_device, force):
+    """ce_rect_min_kb = 0 hands every copy of the copy-engine path to the runtime as a
+    2-D copy of one row (the form the runtime gives to the copy engines): same bytes,
+    and the GPU blocks of GATHER_DIRECT in host order with duplicates on the host side."""
+    from flexkv_amd.c_ext import last_transfer_path, launch_policy
+    s = KVSetup(VLLM, 5, 2, 64, 64, 4096, "BLOCKFIRST", seed=12)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(3)
+    with launch_policy(ce_rect_min_kb=0):
+        for pattern in ("scattered", "few_seg", "contiguous"):
+            cids = block_ids(rng, 64, 20, pattern)
+            gids = block_ids(rng, 64, 20, "scattered")
+            for h2d in (False, True):
+                dev.transfer(gids, cids, is_h2d=h2d, use_ce_transfer=True,
+                             ce_path_opt=force != "PER_BLOCK", ce_force_path=PATHS.get(force, -1),
+                             ce_enable_memcpy2d=True)
+                assert last_transfer_path() == force
+                s.oracle_transfer(gids, cids, h2d)
+                dev.assert_matches_reference(f"{force} {pattern} h2d={h2d} as 2-D copies")
+        # the same host block restored into two GPU blocks (host order puts them side by side)
+        gids, cids = np.array([7, 3, 50, 9], dtype=np.int64), np.array([11, 12, 11, 10], dtype=np.int64)
+        dev.transfer(gids, cids, is_h2d=True, use_ce_transfer=True, ce_path_opt=True,
+                     ce_force_path=PATHS["GATHER_DIRECT"])
+        s.oracle_transfer(gids, cids, True)
+        dev.assert_matches_reference("duplicate host block")
+
+
 def test_forced_direct_strategies_on_fitting_input(gpu_device):
     from flexkv_amd.c_ext import last_transfer_path
     s = KVSetup(VLLM, 3, 1, 40, 40, 4096, "LAYERFIRST", seed=34)   # adjacent blocks on both sides
