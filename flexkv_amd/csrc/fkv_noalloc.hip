@@ -104,7 +104,11 @@ extern "C" int fkv_transfer_kv_blocks_noalloc(const fkv_transfer_desc *desc, voi
   // The host buffer and the device array still belong to the previous call on
   // this GPU until its stream has run the copy and the kernels behind it.
   if (pd.in_flight) {
-    FKV_HIP_TRY(hipStreamSynchronize(pd.last_stream));
+    if (hipStreamSynchronize(pd.last_stream) != hipSuccess) {
+      // the caller has destroyed that stream in the meantime; what it held may still run
+      (void)hipGetLastError();
+      FKV_HIP_TRY(hipDeviceSynchronize());
+    }
     pd.in_flight = false;
   }
   unsigned char *host_plan = g_host_plan[device];

@@ -40,9 +40,11 @@ def test_header_compiles_as_c_and_struct_sizes_match():
     src = r'''
 #include "fkv_transfer.h"
 #include <stdio.h>
-int main(void){ printf("%zu %zu %zu %zu %zu %zu %zu\n", sizeof(fkv_ce_config),
+int main(void){ printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(fkv_ce_config),
   sizeof(fkv_transfer_desc), sizeof(fkv_ce_analysis), sizeof(fkv_tp_rank_plan),
-  sizeof(fkv_tp_group_params), sizeof(fkv_layerwise_params), sizeof(fkv_stats)); return 0; }
+  sizeof(fkv_tp_group_params), sizeof(fkv_layerwise_params), sizeof(fkv_stats),
+  sizeof(fkv_launch_policy), sizeof(fkv_staging_transfer_desc), sizeof(fkv_chunk_ptrs_desc));
+  return 0; }
 '''
     import tempfile
     with tempfile.TemporaryDirectory() as d:
@@ -54,7 +56,8 @@ int main(void){ printf("%zu %zu %zu %zu %zu %zu %zu\n", sizeof(fkv_ce_config),
         sizes = list(map(int, subprocess.check_output([exe]).split()))
     want = [ctypes.sizeof(x) for x in (_lib.CEConfig, _lib.TransferDesc, _lib.CEAnalysis,
                                        _lib.TPRankPlan, _lib.TPGroupParams, _lib.LayerwiseParams,
-                                       _lib.Stats)]
+                                       _lib.Stats, _lib.LaunchPolicy, _lib.StagingTransferDesc,
+                                       _lib.ChunkPtrsDesc)]
     assert sizes == want
 
 
