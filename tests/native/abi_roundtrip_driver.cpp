@@ -454,6 +454,163 @@ int main() {
     ++cases;
   }
 
+  // ---- launch policy: every way a launch shares out its work, and the entry point that
+  //      allocates nothing, on the same descriptor ----
+  {
+    fkv_launch_policy saved, p;
+    FKV_OK_OR_DIE(fkv_launch_policy_get(-1, &saved));
+    if (saved.xcd_count < 1 || (saved.d2h_busy_mask & ~saved.xcd_present_mask) ||
+        (saved.h2d_busy_mask & ~saved.xcd_present_mask)) {
+      fprintf(stderr, "launch policy: masks beyond the device's XCDs\n");
+      return 1;
+    }
+    const int arbiters[] = {0, 2, 3};
+    for (int pass = 0; pass < 4; ++pass) {
+      p = saved;
+      if (pass < 3)
+        p.arbiter = arbiters[pass], p.safety_net_wait_us = 5;
+      FKV_OK_OR_DIE(fkv_launch_policy_set(-1, &p));
+      const int n = 33;
+      std::vector<int64_t> g = pick(rng, N, n), c = pick(rng, NH, n);
+      fkv_transfer_desc d;
+      memset(&d, 0, sizeof(d));
+      d.backend = FKV_BACKEND_VLLM;
+      d.num_layers_total = L;
+      d.gpu_tensor_ptrs = ptrs.data();
+      d.num_gpu_tensor_ptrs = L;
+      d.device = -1;
+      d.gpu_kv_stride = GKS, d.gpu_block_stride = GBS, d.gpu_layer_stride = GLS;
+      d.cpu_ptr = host;
+      d.cpu_kv_stride = CKS, d.cpu_layer_stride = CLS, d.cpu_block_stride = CBS;
+      d.chunk_size = CHUNK;
+      d.start_layer_id = 0, d.num_layers = L, d.kv_dim = KV, d.num_blocks = n;
+      d.gpu_block_ids = g.data(), d.cpu_block_ids = c.data();
+      d.transfer_num_cta = 4;
+      d.sync = 1;
+      fkv_ce_config_default(&d.ce);
+      for (int h2d = 0; h2d < 2; ++h2d) {
+        d.is_host_to_device = h2d;
+        // the last pass goes through the entry point that allocates nothing
+        FKV_OK_OR_DIE(pass == 3 ? fkv_transfer_kv_blocks_noalloc(&d, stream)
+                                : fkv_transfer_kv_blocks(&d, stream));
+        m.put(g, c, h2d != 0);
+        if (check(pass == 3 ? "no-alloc entry point" : "forced launch policy"))
+          return 1;
+      }
+      if (pass == 3) {
+        d.use_ce_transfer = 1;
+        if (fkv_transfer_kv_blocks_noalloc(&d, stream) != FKV_ERR_UNSUPPORTED) {
+          fprintf(stderr, "no-alloc entry point accepted the copy-engine path\n");
+          return 1;
+        }
+      }
+    }
+    FKV_OK_OR_DIE(fkv_launch_policy_reset(-1));
+    ++cases;
+  }
+
+  // ---- compressed staging: address table, payloads of different sizes out and back ----
+  {
+    const int n = 9, total = L * KV * n, first = 5, bsz = total - first;
+    const int64_t stride = CHUNK + 64;
+    std::vector<int64_t> g = pick(rng, N, n), c = pick(rng, NH, n);
+    void **d_ptrs = nullptr;
+    HIP_OK(hipMalloc(reinterpret_cast<void **>(&d_ptrs), sizeof(void *) * bsz));
+    fkv_chunk_ptrs_desc cp;
+    memset(&cp, 0, sizeof(cp));
+    cp.out_ptrs = d_ptrs;
+    cp.backend = FKV_BACKEND_VLLM;
+    cp.num_layers_total = L;
+    cp.gpu_tensor_ptrs = ptrs.data();
+    cp.num_gpu_tensor_ptrs = L;
+    cp.device = -1;
+    cp.gpu_kv_stride = GKS, cp.gpu_block_stride = GBS, cp.gpu_layer_stride = GLS;
+    cp.gpu_block_ids = g.data();
+    cp.start_layer_id = 0, cp.kv_dim = KV, cp.num_blocks = n, cp.batch_start = first, cp.bsz = bsz;
+    cp.sync = 1;
+    FKV_OK_OR_DIE(fkv_build_gpu_chunk_ptrs(&cp, stream));
+    std::vector<void *> got_ptrs(bsz);
+    HIP_OK(hipMemcpy(got_ptrs.data(), d_ptrs, sizeof(void *) * bsz, hipMemcpyDeviceToHost));
+    for (int i = 0; i < bsz; ++i) {
+      const int gi = first + i, l = gi / (KV * n), kv = (gi % (KV * n)) / n, b = gi % n;
+      if (got_ptrs[i] != static_cast<uint8_t *>(dev[l]) + kv * GKS + g[b] * GBS) {
+        fprintf(stderr, "chunk pointer %d differs\n", i);
+        return 1;
+      }
+    }
+    // payloads: the first `sz` bytes of every chunk the table names, written to the host
+    // cache with their sizes, then read back into scrubbed staging
+    uint8_t *d_stage = nullptr;
+    uint64_t *d_sizes = nullptr;
+    int32_t *d_over = nullptr;
+    void *table_v = nullptr;
+    HIP_OK(hipMalloc(reinterpret_cast<void **>(&d_stage), (size_t)bsz * stride));
+    HIP_OK(hipMalloc(reinterpret_cast<void **>(&d_sizes), sizeof(uint64_t) * bsz));
+    HIP_OK(hipMalloc(reinterpret_cast<void **>(&d_over), sizeof(int32_t)));
+    HIP_OK(hipMemset(d_over, 0, sizeof(int32_t)));
+    FKV_OK_OR_DIE(fkv_host_alloc(sizeof(uint32_t) * NH * L * KV, &table_v));
+    uint32_t *table = static_cast<uint32_t *>(table_v);
+    memset(table, 0xff, sizeof(uint32_t) * NH * L * KV);
+    std::vector<uint8_t> stage((size_t)bsz * stride);
+    std::vector<uint64_t> sizes(bsz);
+    for (int i = 0; i < bsz; ++i) {
+      const int gi = first + i, l = gi / (KV * n), kv = (gi % (KV * n)) / n, b = gi % n;
+      sizes[i] = i == 3 ? (uint64_t)CHUNK + 1 : (uint64_t)(rng() % (CHUNK + 1)); // one does not fit
+      memcpy(stage.data() + (size_t)i * stride, m.gpu[l].data() + kv * GKS + g[b] * GBS,
+             (size_t)std::min<uint64_t>(sizes[i], CHUNK));
+    }
+    HIP_OK(hipMemcpy(d_stage, stage.data(), stage.size(), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d_sizes, sizes.data(), sizeof(uint64_t) * bsz, hipMemcpyHostToDevice));
+    fkv_staging_transfer_desc sd;
+    memset(&sd, 0, sizeof(sd));
+    sd.staging = d_stage, sd.staging_stride = stride, sd.comp_sizes = d_sizes;
+    sd.cpu_ptr = host, sd.chunk_capacity = CHUNK, sd.overflow = d_over;
+    sd.cpu_kv_stride = CKS, sd.cpu_layer_stride = CLS, sd.cpu_block_stride = CBS;
+    sd.cpu_block_ids = c.data();
+    sd.size_table = table, sd.size_table_block_stride = L * KV, sd.size_table_layer_stride = KV;
+    sd.start_layer_id = 0, sd.kv_dim = KV, sd.num_blocks = n, sd.batch_start = first, sd.bsz = bsz;
+    sd.is_write_cpu = 1, sd.device = -1, sd.sync = 1;
+    FKV_OK_OR_DIE(fkv_staging_transfer(&sd, stream));
+    int32_t over = 0;
+    HIP_OK(hipMemcpy(&over, d_over, sizeof(over), hipMemcpyDeviceToHost));
+    for (int i = 0; i < bsz; ++i) {
+      const int gi = first + i, l = gi / (KV * n), kv = (gi % (KV * n)) / n, b = gi % n;
+      const uint32_t want_sz = sizes[i] > (uint64_t)CHUNK ? 0 : (uint32_t)sizes[i];
+      if (table[c[b] * L * KV + l * KV + kv] != want_sz) {
+        fprintf(stderr, "size table entry of chunk %d differs\n", i);
+        return 1;
+      }
+      if (sizes[i] <= (uint64_t)CHUNK)
+        memcpy(m.host.data() + c[b] * CBS + l * CLS + kv * CKS, stage.data() + (size_t)i * stride,
+               (size_t)sizes[i]);
+    }
+    if (over != 1 || check("staging transfer to the host"))
+      return 1;
+    HIP_OK(hipMemset(d_stage, 0xEE, stage.size()));
+    HIP_OK(hipMemset(d_sizes, 0, sizeof(uint64_t) * bsz));
+    sd.is_write_cpu = 0;
+    FKV_OK_OR_DIE(fkv_staging_transfer(&sd, stream));
+    std::vector<uint8_t> back(stage.size());
+    std::vector<uint64_t> back_sizes(bsz);
+    HIP_OK(hipMemcpy(back.data(), d_stage, back.size(), hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(back_sizes.data(), d_sizes, sizeof(uint64_t) * bsz, hipMemcpyDeviceToHost));
+    for (int i = 0; i < bsz; ++i) {
+      const uint64_t want_sz = sizes[i] > (uint64_t)CHUNK ? 0 : sizes[i];
+      if (back_sizes[i] != want_sz ||
+          memcmp(back.data() + (size_t)i * stride, stage.data() + (size_t)i * stride, (size_t)want_sz) ||
+          (want_sz < (uint64_t)stride && back[(size_t)i * stride + want_sz] != 0xEE)) {
+        fprintf(stderr, "staging transfer from the host: payload %d differs\n", i);
+        return 1;
+      }
+    }
+    HIP_OK(hipFree(d_ptrs));
+    HIP_OK(hipFree(d_stage));
+    HIP_OK(hipFree(d_sizes));
+    HIP_OK(hipFree(d_over));
+    FKV_OK_OR_DIE(fkv_host_free(table_v));
+    ++cases;
+  }
+
   // ---- the board processes share: one's own postings never count as "elsewhere" ----
   {
     int32_t busy = 7;
