@@ -165,6 +165,10 @@ class ChunkPtrsDesc(Structure):
                 ("batch_start", c_int32), ("bsz", c_int32), ("sync", c_int32)]
 
 
+class StagedRun(Structure):
+    _fields_ = [("first_id", c_int64), ("rows", c_int32), ("row0", c_int32)]
+
+
 class Stats(Structure):
     _fields_ = [("calls", c_uint64), ("bytes_h2d", c_uint64), ("bytes_d2h", c_uint64),
                 ("kernel_launches", c_uint64), ("dma_copies", c_uint64),
@@ -275,6 +279,10 @@ SIGNATURES = {
     "fkv_reset_stats": (None, []),
     "fkv_staging_transfer": (c_int32, [POINTER(StagingTransferDesc), c_void_p]),
     "fkv_build_gpu_chunk_ptrs": (c_int32, [POINTER(ChunkPtrsDesc), c_void_p]),
+    "fkv_staged_restore_plan": (c_int32, [c_void_p, c_int32, c_int64, c_int32,
+                                          POINTER(LaunchPolicy), POINTER(c_int32),
+                                          POINTER(c_int32), POINTER(c_int64), c_void_p, c_int32,
+                                          c_void_p]),
     "fkv_measure_hbm_rate": (c_int32, [c_int32, c_size_t, c_int32, c_int32,
                                        POINTER(c_double), POINTER(c_double)]),
     "fkv_launch_policy_get": (c_int32, [c_int32, POINTER(LaunchPolicy)]),

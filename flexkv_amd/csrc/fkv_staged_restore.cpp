@@ -79,6 +79,97 @@ int ring_prepare(StagedRing &ring, int slots, size_t bytes) {
 
 } // namespace
 
+// The arithmetic of the choice, without a device: runs of consecutive host block ids,
+// which holes between them are read along, and whether the copy engines are worth it.
+// `row_bytes` = bytes of one host block that a batch moves, `pieces` = copy commands
+// per run and batch.  Returns false when the restore stays on the kernel path.
+bool staged_layout(const int64_t *cpu_ids, int num_blocks, int64_t row_bytes, int pieces,
+                   const fkv_launch_policy &pol, std::vector<StagedPlan::Seg> *segs,
+                   int64_t *total_rows_out) {
+  segs->clear();
+  *total_rows_out = 0;
+  if (pol.staged_restore == 0 || num_blocks <= 0 || row_bytes <= 0 || pieces < 1)
+    return false;
+  std::vector<int64_t> ids(cpu_ids, cpu_ids + num_blocks);
+  std::sort(ids.begin(), ids.end());
+  ids.erase(std::unique(ids.begin(), ids.end()), ids.end());
+  struct Hole {
+    int64_t rows;
+    size_t after; // index into ids of the last block before the hole
+  };
+  std::vector<Hole> holes;
+  for (size_t k = 0; k + 1 < ids.size(); ++k)
+    if (ids[k + 1] != ids[k] + 1)
+      holes.push_back(Hole{ids[k + 1] - ids[k] - 1, k});
+  // Holes are read along, smallest first, while each stays below the bridge size
+  // and all together below the allowed share of the useful bytes.
+  const double useful = (double)ids.size() * (double)row_bytes;
+  const double max_waste = useful * pol.staged_overhead_pct / 100.0;
+  std::vector<size_t> order(holes.size());
+  for (size_t k = 0; k < order.size(); ++k)
+    order[k] = k;
+  std::stable_sort(order.begin(), order.end(),
+                   [&](size_t x, size_t y) { return holes[x].rows < holes[y].rows; });
+  std::vector<bool> bridged(holes.size(), false);
+  double waste = 0;
+  int64_t extra_rows = 0;
+  for (size_t k : order) {
+    const double bytes = (double)holes[k].rows * (double)row_bytes;
+    if (bytes > (double)pol.staged_bridge_kb * 1024 || waste + bytes > max_waste)
+      break;
+    bridged[k] = true;
+    waste += bytes;
+    extra_rows += holes[k].rows;
+  }
+  int64_t nsegs = 1;
+  for (size_t k = 0; k < holes.size(); ++k)
+    nsegs += bridged[k] ? 0 : 1;
+  const int64_t total_rows = (int64_t)ids.size() + extra_rows;
+  if (total_rows * row_bytes > (int64_t)pol.staged_max_mb << 20)
+    return false;
+  if (pol.staged_restore == 1) {
+    // the copy commands of a batch against the batch's time on the link
+    const double batch_us = useful / (pol.link_gbps_estimate * 1e3);
+    if ((double)(nsegs * pieces) * pol.staged_copy_overhead_us >
+        batch_us * pol.staged_overhead_pct / 100.0)
+      return false;
+  }
+  if (nsegs * pieces > 4096) // a batch of thousands of commands is never the better way
+    return false;
+  segs->reserve((size_t)nsegs);
+  StagedPlan::Seg cur{ids[0], 1, 0};
+  size_t h = 0;
+  for (size_t k = 0; k + 1 < ids.size(); ++k) {
+    if (ids[k + 1] == ids[k] + 1) {
+      cur.rows += 1;
+      continue;
+    }
+    if (bridged[h]) {
+      cur.rows += (int32_t)(ids[k + 1] - ids[k]);
+    } else {
+      segs->push_back(cur);
+      cur = StagedPlan::Seg{ids[k + 1], 1, cur.row0 + cur.rows};
+    }
+    ++h;
+  }
+  segs->push_back(cur);
+  *total_rows_out = total_rows;
+  return true;
+}
+
+// Staging row of host block `id`: the last run whose first id is <= id.
+int64_t staged_row_of(const std::vector<StagedPlan::Seg> &segs, int64_t id) {
+  size_t lo = 0, hi = segs.size();
+  while (hi - lo > 1) {
+    const size_t mid = (lo + hi) / 2;
+    if (segs[mid].first_id <= id)
+      lo = mid;
+    else
+      hi = mid;
+  }
+  return segs[lo].row0 + (id - segs[lo].first_id);
+}
+
 int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &ring,
                       hipStream_t scatter_stream, StagedPlan *out) {
   *out = StagedPlan{};
@@ -97,75 +188,11 @@ int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &
   out->kind = layers_adjacent ? 0 : kv_adjacent ? 1 : 2;
   const int64_t batch_row_bytes = (int64_t)lk * d.chunk_size; // of one block, all pieces
   const int pieces = out->kind == 0 ? 1 : out->kind == 1 ? nl : lk;
-
-  // runs of consecutive host block ids
-  std::vector<int64_t> ids(d.cpu_block_ids, d.cpu_block_ids + d.num_blocks);
-  std::sort(ids.begin(), ids.end());
-  ids.erase(std::unique(ids.begin(), ids.end()), ids.end());
-  struct Hole {
-    int64_t rows;
-    size_t after; // index into ids of the last block before the hole
-  };
-  std::vector<Hole> holes;
-  for (size_t k = 0; k + 1 < ids.size(); ++k)
-    if (ids[k + 1] != ids[k] + 1)
-      holes.push_back(Hole{ids[k + 1] - ids[k] - 1, k});
-  // Holes are read along, smallest first, while each stays below the bridge size
-  // and all together below the allowed share of the useful bytes.
-  const double useful = (double)ids.size() * batch_row_bytes;
-  const double max_waste = useful * pol.staged_overhead_pct / 100.0;
-  std::vector<size_t> order(holes.size());
-  for (size_t k = 0; k < order.size(); ++k)
-    order[k] = k;
-  std::sort(order.begin(), order.end(),
-            [&](size_t a, size_t b) { return holes[a].rows < holes[b].rows; });
-  std::vector<bool> bridged(holes.size(), false);
-  double waste = 0;
-  int64_t extra_rows = 0;
-  for (size_t k : order) {
-    const double bytes = (double)holes[k].rows * batch_row_bytes;
-    if (bytes > (double)pol.staged_bridge_kb * 1024 || waste + bytes > max_waste)
-      break;
-    bridged[k] = true;
-    waste += bytes;
-    extra_rows += holes[k].rows;
-  }
-  int64_t nsegs = 1;
-  for (size_t k = 0; k < holes.size(); ++k)
-    nsegs += bridged[k] ? 0 : 1;
-  const int64_t total_rows = (int64_t)ids.size() + extra_rows;
+  int64_t total_rows = 0;
+  if (!staged_layout(d.cpu_block_ids, d.num_blocks, batch_row_bytes, pieces, pol, &out->segs,
+                     &total_rows))
+    return FKV_OK;
   const int64_t slot_bytes = total_rows * batch_row_bytes;
-  if (slot_bytes > (int64_t)pol.staged_max_mb << 20)
-    return FKV_OK;
-  if (pol.staged_restore == 1) {
-    // the copy commands of a batch against the batch's time on the link
-    const double batch_us = useful / (pol.link_gbps_estimate * 1e3);
-    if ((double)(nsegs * pieces) * pol.staged_copy_overhead_us >
-        batch_us * pol.staged_overhead_pct / 100.0)
-      return FKV_OK;
-  }
-  if (nsegs * pieces > 4096) // a batch of thousands of commands is never the better way
-    return FKV_OK;
-
-  out->segs.reserve((size_t)nsegs);
-  {
-    StagedPlan::Seg cur{ids[0], 1, 0};
-    size_t h = 0;
-    for (size_t k = 0; k + 1 < ids.size(); ++k) {
-      if (ids[k + 1] == ids[k] + 1) {
-        cur.rows += 1;
-        continue;
-      }
-      if (bridged[h]) {
-        cur.rows += (int32_t)(ids[k + 1] - ids[k]);
-      } else {
-        out->segs.push_back(cur);
-        cur = StagedPlan::Seg{ids[k + 1], 1, cur.row0 + cur.rows};
-      }
-      ++h;
-    }
-    out->segs.push_back(cur);
-  }
   out->total_rows = (int32_t)total_rows;
   out->max_lk = lk;
   out->batch_layers = nl;
@@ -199,19 +226,8 @@ int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &
                                   (uint64_t)(i % m) * (uint64_t)d.chunk_size;
     }
   int64_t *rows = reinterpret_cast<int64_t *>(h + tab);
-  for (int pos = 0; pos < d.num_blocks; ++pos) {
-    const int64_t id = d.cpu_block_ids[pos];
-    // the last segment whose first id is <= id
-    size_t lo = 0, hi = out->segs.size();
-    while (hi - lo > 1) {
-      const size_t mid = (lo + hi) / 2;
-      if (out->segs[mid].first_id <= id)
-        lo = mid;
-      else
-        hi = mid;
-    }
-    rows[pos] = out->segs[lo].row0 + (id - out->segs[lo].first_id);
-  }
+  for (int pos = 0; pos < d.num_blocks; ++pos)
+    rows[pos] = staged_row_of(out->segs, d.cpu_block_ids[pos]);
   uint8_t *dv = nullptr;
   int rc = plan_publish(slot, tab + rows_bytes, /*mirror=*/true, scatter_stream, &dv);
   if (rc != FKV_OK) {
@@ -281,6 +297,36 @@ int staged_launch(const StagedPlan &sp, StagedRing &ring, const KernelPlan &kp, 
   stats().staged_batches.fetch_add(1, std::memory_order_relaxed);
   return FKV_OK;
 }
+
+} // namespace fkv
+
+extern "C" int fkv_staged_restore_plan(const int64_t *cpu_block_ids, int32_t num_blocks,
+                                       int64_t row_bytes, int32_t pieces,
+                                       const fkv_launch_policy *policy, int32_t *staged,
+                                       int32_t *num_runs, int64_t *total_rows,
+                                       fkv_staged_run *runs, int32_t run_capacity,
+                                       int64_t *row_of_position) {
+  using namespace fkv;
+  clear_error();
+  if (!policy || !staged || num_blocks < 0 || (num_blocks > 0 && !cpu_block_ids))
+    return fail(FKV_ERR_INVALID_ARG, "fkv_staged_restore_plan: bad arguments");
+  std::vector<StagedPlan::Seg> segs;
+  int64_t rows = 0;
+  *staged = staged_layout(cpu_block_ids, num_blocks, row_bytes, pieces, *policy, &segs, &rows) ? 1 : 0;
+  if (num_runs)
+    *num_runs = (int32_t)segs.size();
+  if (total_rows)
+    *total_rows = rows;
+  if (runs)
+    for (int i = 0; i < (int)segs.size() && i < run_capacity; ++i)
+      runs[i] = fkv_staged_run{segs[i].first_id, segs[i].rows, segs[i].row0};
+  if (row_of_position && *staged)
+    for (int pos = 0; pos < num_blocks; ++pos)
+      row_of_position[pos] = staged_row_of(segs, cpu_block_ids[pos]);
+  return FKV_OK;
+}
+
+namespace fkv {
 
 void staged_plan_release(StagedPlan *sp, hipStream_t scatter_stream) {
   if (sp->slot)

@@ -711,6 +711,22 @@ int fkv_launch_policy_set(int32_t device, const fkv_launch_policy *in);
 /* Back to the defaults derived from the device and the environment. */
 int fkv_launch_policy_reset(int32_t device);
 
+/* The arithmetic behind the staged layerwise restore, without a device (tests,
+ * inspection): the runs of consecutive host block ids of a call, with the holes that are
+ * read along, and whether a restore of these blocks goes through the copy engines under
+ * `policy`.  `row_bytes` = bytes of one host block that one batch of layers moves,
+ * `pieces` = copy commands per run and batch (1 when a batch's chunks of a block are
+ * adjacent on the host).  No counterpart in the reference. */
+typedef struct fkv_staged_run {
+  int64_t first_id; /* first host block of the run */
+  int32_t rows;     /* host blocks it spans, holes read along included */
+  int32_t row0;     /* staging row of the first */
+} fkv_staged_run;
+int fkv_staged_restore_plan(const int64_t *cpu_block_ids, int32_t num_blocks, int64_t row_bytes,
+                            int32_t pieces, const fkv_launch_policy *policy, int32_t *staged,
+                            int32_t *num_runs, int64_t *total_rows, fkv_staged_run *runs,
+                            int32_t run_capacity, int64_t *row_of_position);
+
 /* Host-link reference rate: `reps` plain hipMemcpyAsync copies of `bytes`
  * between a pinned host buffer and a device buffer (both owned by the call),
  * timed with hip events.  direction: 0 = D2H, 1 = H2D.  Result in GB/s
