@@ -28,6 +28,7 @@
 //
 // The transfer streams keep the default priority.
 #include "fkv_internal.h"
+#include "fkv_poll.h"
 
 #include <sys/eventfd.h>
 #include <unistd.h>
@@ -198,31 +199,21 @@ struct fkv_layerwise {
   void notify(const Batch &b) const { notify_layers(b.start_layer, b.layers); }
 
   void poll_loop() {
-    size_t next = 0;
-    while (next < batches.size() && !poller_stop.load(std::memory_order_acquire)) {
-      Batch &b = *batches[next];
-      bool all = true;
-      for (int g = 0; g < num_gpus && all; ++g) {
-        (void)hipSetDevice(device_ids[g]);
-        hipError_t e = hipEventQuery(b.done[g]);
-        if (e != hipSuccess) {
-          (void)hipGetLastError();
-          all = false;
-          if (e != hipErrorNotReady) {
-            // A real device error: the batches behind it will never land.  Stop
-            // without announcing them; the next call on the group reports it.
-            int none = 0;
-            restore_error.compare_exchange_strong(none, (int)e);
-            return;
-          }
-        }
-      }
-      if (all) {
-        notify(b);
-        ++next;
-      } else {
-        std::this_thread::yield();
-      }
+    const int status = fkv::poll_batches_in_order(
+        batches.size(), num_gpus, (int)hipSuccess, (int)hipErrorNotReady,
+        [this](size_t b, int g) {
+          (void)hipSetDevice(device_ids[g]);
+          const hipError_t e = hipEventQuery(batches[b]->done[g]);
+          if (e != hipSuccess)
+            (void)hipGetLastError();
+          return (int)e;
+        },
+        [this](size_t b) { notify(*batches[b]); }, poller_stop);
+    if (status != (int)hipSuccess) {
+      // A real device error: the layers behind it were not announced; the next call
+      // on the group reports it.
+      int none = 0;
+      restore_error.compare_exchange_strong(none, status);
     }
   }
 

@@ -46,3 +46,12 @@ def test_ssd_engine_under_sanitizers(tmp_path, sanitizer):
 def test_host_row_copies_under_sanitizers(tmp_path, sanitizer):
     out = build_and_run(tmp_path, "host_copy_sanitizer_driver.cpp", sanitizer, extra=("-mavx2",))
     assert "400 scatter/gather pairs" in out
+
+
+@pytest.mark.parametrize("sanitizer", SANITIZERS)
+def test_layerwise_poll_loop_under_sanitizers(tmp_path, sanitizer):
+    """The polling loop of the layerwise restore (fkv_poll.h) on scripted event
+    statuses: in-order announcements, a device error ends it without announcing what
+    is left, a stop request ends it."""
+    out = build_and_run(tmp_path, "poll_loop_driver.cpp", sanitizer)
+    assert "ok: 301 scripted polls" in out
