@@ -69,7 +69,7 @@ class Workload:
             L, N, T, H, D = 32, (4096 if name == "c0" else 32768), 16, 8, 128
             self.desc = ("Llama-3-8B vLLM layout bf16: 32 x [2,%d,16,8,128], host [NH,32,2,16,8,128]"
                          % N)
-            self.backend, self.kv_dim, self.L = 0, 2, L
+            self.backend, self.kv_dim, self.L, self.num_kv_heads = 0, 2, L, H
             self.chunk = T * H * D * 2
             gen = t.Generator(device=device).manual_seed(0)
             self.tensors = [t.randn(2, N, T, H, D, device=device, dtype=t.bfloat16, generator=gen)
@@ -98,7 +98,7 @@ class Workload:
             L, tokens, H, D, page = 32, 262144, 8, 128, 64
             self.desc = ("SGLang token-major bf16 page 64: 64 x [262144,8,128] (K then V, 32 layers), "
                          "1024 pages = 64 runs of 8 + 512 isolated, host [1024,32,2,64,8,128]")
-            self.backend, self.kv_dim, self.L = 2, 2, L
+            self.backend, self.kv_dim, self.L, self.num_kv_heads = 2, 2, L, H
             self.chunk = page * H * D * 2
             gen = t.Generator(device=device).manual_seed(2)
             self.tensors = [t.randn(tokens, H, D, device=device, dtype=t.bfloat16, generator=gen)
@@ -113,7 +113,7 @@ class Workload:
             N, L, H, T, D = 4096, 80, 8, 32, 128
             self.desc = ("TRT-LLM layout fp8 e4m3: one [4096,80,2,8,32,128] tensor, 2048 random "
                          "blocks, host [2048,80,2,8,32,128]")
-            self.backend, self.kv_dim, self.L = 1, 2, L
+            self.backend, self.kv_dim, self.L, self.num_kv_heads = 1, 2, L, H
             self.chunk = H * T * D
             gen = t.Generator(device=device).manual_seed(3)
             codes = t.randint(0, 254, (N, L, 2, H, T, D), device=device, dtype=t.uint8,
@@ -131,7 +131,7 @@ class Workload:
             L, N, T, D = 61, 16384, 64, 576
             self.desc = ("DeepSeek-V3 MLA latent KV bf16: 61 x [16384,64,576], layerwise restore of "
                          "512 blocks, host [512,61,1,64,1,576]")
-            self.backend, self.kv_dim, self.L = 0, 1, L
+            self.backend, self.kv_dim, self.L, self.num_kv_heads = 0, 1, L, 1
             self.chunk = T * D * 2
             gen = t.Generator(device=device).manual_seed(4)
             self.tensors = [(t.randn(N, T, D, device=device, dtype=t.bfloat16, generator=gen) * 0.5)
@@ -156,6 +156,9 @@ class Workload:
     def transfer(self, gpu_ids, cpu_ids, h2d, **kw):
         from flexkv_amd.c_ext import transfer_kv_blocks
         kw.setdefault("sync", False)
+        # the reference's workers pass the layout's head count (flexkv/transfer/worker.py:1020,
+        # 1050); the copy-engine strategy tree reads it (csrc/ce_transfer.cu:71-104)
+        kw.setdefault("num_kv_heads", self.num_kv_heads)
         transfer_kv_blocks(gpu_ids, self.ptrs, self.gks, self.gbs, self.gls, cpu_ids, self.host,
                            self.cks, self.cls, self.cbs, self.chunk, 0, self.L,
                            is_host_to_device=h2d, kv_dim=self.kv_dim, gpu_block_type=self.backend,
