@@ -257,9 +257,9 @@ struct Job {
   uint8_t *cpu(int layer_local, int kv, int64_t block) const {
     return cpu_chunk_ptr(d, (int64_t)d.start_layer_id + layer_local, kv, block);
   }
-  // The runtime runs a 1-D hipMemcpyAsync between pinned host and device memory as a
-  // kernel on the compute units (one __amd_rocclr_copyBuffer launch per copy in a
-  // kernel trace, whatever the size) and hands 2-D copies to the copy engines.  A
+  // The runtime is free to run a 1-D hipMemcpyAsync between pinned host and device
+  // memory as a kernel on the compute units (one __amd_rocclr_copyBuffer launch per copy
+  // in a kernel trace, whatever the size); 2-D copies it hands to the copy engines.  A
   // 2-D copy costs about 9 us of fixed time against about 3 us and its completion
   // reaches a waiting host thread late, so this is opt-in: with `ce_rect_min_kb` >= 0
   // copies of that size and more go as 2-D copies of one row (8 GiB in 1 GiB copies:

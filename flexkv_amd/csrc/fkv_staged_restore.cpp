@@ -263,8 +263,8 @@ int staged_launch(const StagedPlan &sp, StagedRing &ring, const KernelPlan &kp, 
       const uint8_t *src = src0 + s.first_id * sp.cpu_block_stride;
       uint8_t *dst = dst0 + (int64_t)s.row0 * w;
       // Always the 2-D call, also for one row or adjacent rows: the runtime hands 2-D
-      // copies to the copy engines, while it runs hipMemcpyAsync between pinned host and
-      // device memory as a kernel on the compute units (seen in kernel traces: one
+      // copies to the copy engines, while it is free to run hipMemcpyAsync between pinned
+      // host and device memory as a kernel on the compute units (kernel traces show one
       // __amd_rocclr_copyBuffer launch per 1-D copy of any size, none for 2-D copies),
       // which is what this path exists to avoid.
       const size_t pitch = s.rows == 1 ? (size_t)w : (size_t)sp.cpu_block_stride;
