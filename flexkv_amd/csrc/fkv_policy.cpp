@@ -109,7 +109,7 @@ void sanitize(fkv_launch_policy &p, const fkv_launch_policy &derived) {
   p.hbm_wg_threads = clampi(p.hbm_wg_threads, 64, kCopyBlockThreads);
   p.hbm_unroll = p.hbm_unroll >= kCopyUnrollDeep ? kCopyUnrollDeep : kCopyUnroll;
   p.ce_staging_mb = clampi(p.ce_staging_mb, 1, 1 << 18);
-  p.ce_two_streams = p.ce_two_streams != 0;
+  p.ce_two_streams = clampi(p.ce_two_streams, 0, 2);
   p.ce_rect_min_kb = clampi(p.ce_rect_min_kb, -1, 1 << 24);
   p.model_link_mbps = clampi(p.model_link_mbps, 100, 10000000);
   p.model_kernel_d2h_mbps = clampi(p.model_kernel_d2h_mbps, 100, 10000000);

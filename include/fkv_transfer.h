@@ -686,7 +686,12 @@ typedef struct fkv_launch_policy {
   int32_t hbm_wg_threads;
   int32_t hbm_unroll;         /* 16-byte vectors in flight per lane in these launches: 8 or 16 */
   int32_t ce_staging_mb;      /* FKV_CE_STAGING_MB: device staging of the copy-engine strategies */
-  int32_t ce_two_streams;     /* direct copy-engine strategies fan out over a second stream */
+  int32_t ce_two_streams;     /* 0: every copy of a copy-engine strategy on the caller's stream;
+                                 2: runs of eight and more independent copies alternate between it
+                                 and a second stream; 1 (default): that, and a GATHER_DIRECT that
+                                 needs several staging groups of few, large copies alternates
+                                 between two staging buffers, compaction launches on the caller's
+                                 stream next to the copies on the second */
   int32_t ce_rect_min_kb;     /* copies of at least this size are issued as 2-D copies of one row,
                                  which the runtime hands to the copy engines (it runs 1-D
                                  hipMemcpyAsync between pinned host and device memory as a kernel

@@ -187,6 +187,34 @@ def test_gather_direct_groups_and_partial_layers(gpu_device, monkeypatch):
                 dev.assert_matches_reference(f"GATHER_DIRECT layers {l0}..{l0 + 1} h2d={h2d}")
 
 
+@pytest.mark.parametrize("memcpy2d", [False, True], ids=["no2d", "2d"])
+def test_gather_direct_in_many_staging_groups(gpu_device, memcpy2d):
+    """A staging buffer of 1 MiB holds two blocks of 384 KiB: 37 blocks go in 19 groups
+    (or, where the host blocks form few runs, in 37 groups of one block that alternate
+    between two buffers while their copies run on a second stream); runs of consecutive
+    host blocks are cut at group boundaries, and the last group is short.  Whole blocks
+    and layer batches, both directions, and the same with the second stream off."""
+    from flexkv_amd.c_ext import last_transfer_path, launch_policy
+    s = KVSetup(VLLM, 6, 2, 64, 64, 32768, "BLOCKFIRST", seed=37)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(11)
+    for two_streams, pattern in [(m, p) for m in (1, 2, 0) for p in ("contiguous", "few_seg", "scattered")]:
+        with launch_policy(ce_staging_mb=1, ce_two_streams=two_streams):
+            cids = block_ids(rng, 64, 37, pattern)
+            gids = block_ids(rng, 64, 37, "scattered")
+            for l0, nl in ((0, 6), (1, 3)):
+                for h2d in (False, True):
+                    print(f"case {pattern} layers {l0}+{nl} h2d={h2d} 2d={memcpy2d} "
+                          f"two_streams={two_streams}", flush=True)
+                    dev.transfer(gids, cids, is_h2d=h2d, start_layer=l0, num_layers=nl,
+                                 use_ce_transfer=True, ce_path_opt=True, ce_force_path=4,
+                                 ce_enable_memcpy2d=memcpy2d, num_kv_heads=8)
+                    assert last_transfer_path() == "GATHER_DIRECT"
+                    s.oracle_transfer(gids, cids, h2d, start_layer=l0, num_layers=nl)
+                    dev.assert_matches_reference(
+                        f"GATHER_DIRECT in groups, {pattern}, layers {l0}+{nl}, h2d={h2d}")
+
+
 def test_auto_engine_follows_the_cost_model_and_stays_exact(gpu_device):
     """use_ce_transfer="auto": the path that ran is the one fkv_choose_engine
     names, and the bytes equal the oracle's either way."""
