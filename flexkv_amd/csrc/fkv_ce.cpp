@@ -256,6 +256,8 @@ struct Job {
   // which carries the compaction launches.
   mutable hipStream_t lane = nullptr;
   int64_t rect_min_bytes = -1; // from ce_rect_min_kb of the launch policy (run_ce_path)
+  // set by the strategies whose host thread waits for each copy (staging ping-pong)
+  mutable bool host_waits = false;
 
   // Call when at least `copies` independent DMAs follow.  Work already on
   // `stream` is ordered before everything issued on the second stream.
@@ -296,15 +298,17 @@ struct Job {
   }
   // The runtime is free to run a 1-D hipMemcpyAsync between pinned host and device
   // memory as a kernel on the compute units (one __amd_rocclr_copyBuffer launch per copy
-  // in a kernel trace, whatever the size); 2-D copies it hands to the copy engines.  A
-  // 2-D copy costs about 9 us of fixed time against about 3 us and its completion
-  // reaches a waiting host thread late, so this is opt-in: with `ce_rect_min_kb` >= 0
-  // copies of that size and more go as 2-D copies of one row (8 GiB in 1 GiB copies:
-  // the same rate either way; 5 MiB copies: 51 against 56 GB/s; 2 MiB copies: 45
-  // against 55 GB/s), everything else as the runtime likes.
+  // in a kernel trace, whatever the size); 2-D copies it hands to the copy engines,
+  // which leaves the compute units to the engine's own kernels.  A 2-D copy costs about
+  // 9 us of fixed time against about 3 us (5 MiB copies: 51 against 56 GB/s; 2 MiB: 45
+  // against 55 GB/s; 32 MiB and more: the same rate either way), and its completion
+  // reaches a waiting host thread late (8 MiB copies with a host scatter behind each:
+  // 10 against 44 GB/s).  So copies of `ce_rect_min_kb` and more go as 2-D copies of one
+  // row unless a host thread waits for each of them; everything else as the runtime
+  // likes.
   int dma(void *dst, const void *src, size_t bytes, hipMemcpyKind k) const {
     stats().dma_copies.fetch_add(1, std::memory_order_relaxed);
-    if (rect_min_bytes >= 0 && (int64_t)bytes >= rect_min_bytes)
+    if (rect_min_bytes >= 0 && (int64_t)bytes >= rect_min_bytes && !host_waits)
       FKV_HIP_TRY(hipMemcpy2DAsync(dst, bytes, src, bytes, bytes, 1, k, next_stream()));
     else
       FKV_HIP_TRY(hipMemcpyAsync(dst, src, bytes, k, next_stream()));
@@ -395,6 +399,7 @@ int d2h_pingpong(const Job &j, Produce produce) {
   stats().staging_bytes_host.fetch_add((uint64_t)layer_bytes * d.num_layers * d.kv_dim);
   uint8_t *bufs[2] = {base, base + layer_bytes};
   const int iters = d.num_layers * d.kv_dim;
+  j.host_waits = true;
   for (int it = 0; it <= iters; ++it) {
     if (it < iters) {
       FKV_TRY(produce(it, bufs[it & 1]));
@@ -424,6 +429,7 @@ int h2d_pingpong(const Job &j, Consume consume) {
   stats().staging_bytes_host.fetch_add((uint64_t)layer_bytes * d.num_layers * d.kv_dim);
   uint8_t *bufs[2] = {base, base + layer_bytes};
   const int iters = d.num_layers * d.kv_dim;
+  j.host_waits = true;
   for (int it = 0; it < iters; ++it) {
     if (it >= 2)
       FKV_HIP_TRY(hipEventSynchronize(ev[it & 1]));

@@ -155,8 +155,9 @@ fkv_launch_policy defaults_for(uint32_t present) {
   p.hbm_unroll = kCopyUnrollDeep;
   p.ce_staging_mb = 1024;
   p.ce_two_streams = 1;
-  p.ce_rect_min_kb = -1; // 8 GiB in 1 GiB copies: the same rate either way; 5 MiB copies: 51 against
-                         // 56 GB/s; copies a host thread waits for one by one: far slower
+  p.ce_rect_min_kb = 32768; // 32 MiB and more: the same rate either way (3 GiB in copies of 32 MiB:
+                            // 54.7 against 54.8 GB/s; of 128 MiB and of 1.5 GiB: equal), and the
+                            // compute units stay free; 5 MiB copies: 51 against 56 GB/s
   // Measured on MI355X: a DMA command costs about 2.5 us beyond its bytes when copies
   // alternate over two streams (256 x 2 MiB: 50-54 GB/s; 2048 x 5 MiB: 56.2 GB/s); the
   // compaction pass runs at 1.5 TB/s or more; a host scatter/gather pass at about

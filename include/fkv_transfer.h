@@ -693,9 +693,11 @@ typedef struct fkv_launch_policy {
                                  between two staging buffers, compaction launches on the caller's
                                  stream next to the copies on the second */
   int32_t ce_rect_min_kb;     /* copies of at least this size are issued as 2-D copies of one row,
-                                 which the runtime hands to the copy engines (it runs 1-D
-                                 hipMemcpyAsync between pinned host and device memory as a kernel
-                                 on the compute units); 0 = all copies, -1 = none (default) */
+                                 which the runtime hands to the copy engines (it is free to run a
+                                 1-D hipMemcpyAsync between pinned host and device memory as a
+                                 kernel on the compute units), except where a host thread waits
+                                 for each copy (the staging ping-pong of SEGMENT_SCATTER and
+                                 GATHER_SCATTER); 0 = all copies, -1 = none; default 32768 */
   /* cost model of fkv_choose_engine (use_ce_transfer = 2): what each engine is expected to take */
   int32_t model_link_mbps;          /* the link under plain copy-engine copies, MB/s */
   int32_t model_kernel_d2h_mbps;    /* the gather/scatter kernel GPU->host */

@@ -109,8 +109,9 @@ def test_forced_general_strategies(gpu_device, force, backend, L, K, N, NH, chun
 
 @pytest.mark.parametrize("force", ["PER_BLOCK", "SEGMENT_SCATTER", "GATHER_SCATTER", "GATHER_DIRECT"])
 def test_every_copy_as_a_2d_copy_of_one_row(gpu_device, force):
-    """ce_rect_min_kb = 0 hands every copy of the copy-engine path to the runtime as a
-    2-D copy of one row (the form the runtime gives to the copy engines): same bytes,
+    """ce_rect_min_kb = 0 hands every copy of the copy-engine path that no host thread
+    waits for to the runtime as a 2-D copy of one row (the form the runtime gives to the
+    copy engines; the staging ping-pong of the two *_SCATTER strategies keeps 1-D copies): same bytes,
     and the GPU blocks of GATHER_DIRECT in host order with duplicates on the host side."""
     from flexkv_amd.c_ext import last_transfer_path, launch_policy
     s = KVSetup(VLLM, 5, 2, 64, 64, 4096, "BLOCKFIRST", seed=12)
