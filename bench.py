@@ -326,7 +326,7 @@ def verify_round_trip(w, torch, num_cta):
     return bool(ok)
 
 
-def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=False):
+def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=False, use_ce=False):
     """c3: per-layer restore with a dummy per-layer compute kernel on a second
     stream gated on each layer's event.  `layer_spans` brackets every layer's
     compute with two timing events; torch creates them with default flags, and
@@ -345,7 +345,7 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=F
     def restore():
         grp.layerwise_transfer(
             empty, empty, 0, 0, 0, 0, 0, w.gpu_ids, w.cpu_ids, w.cks, w.cls, w.cbs, w.chunk,
-            w.cks, w.cls, w.cbs, num_cta, False, w.L, 1, w.kv_dim, 1, counter_id=0,
+            w.cks, w.cls, w.cbs, num_cta, use_ce, w.L, 1, w.kv_dim, 1, counter_id=0,
             kv_shared_across_ranks_mode="sharded", notify_mode=notify)
 
     layer_bytes = w.num_blocks * w.kv_dim * w.chunk
@@ -1187,7 +1187,7 @@ def measure_config(name, args, torch, device, link, steps, warmup):
             w.gpu_rows(l, 0).index_fill_(0, gi, 0)
         c_ext.reset_stats()
         r = run_layerwise(w, torch, steps, warmup, args.num_cta, args.notify, args.dummy,
-                          layer_spans=args.layer_spans)
+                          layer_spans=args.layer_spans, use_ce=args.use_ce)
         r["layers"] = w.L
         restore = B / (r["restore_ms"] * 1e-3) / 1e9
         out.update(value=round(restore, 3), ms_per_step=round(r["total_ms"], 3),
