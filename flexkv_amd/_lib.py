@@ -202,7 +202,7 @@ class LaunchPolicy(Structure):
                 ("model_kernel_h2d_mbps", c_int32), ("model_dma_ns", c_int32),
                 ("model_compaction_gbps", c_int32), ("model_host_pass_mbps", c_int32),
                 ("model_launch_ns", c_int32), ("model_prefer_ce_pct", c_int32),
-                ("reserved", c_int32 * 6)]
+                ("d2h_lane_runs", c_int32), ("reserved", c_int32 * 5)]
 
 
 # name -> (restype, argtypes); the complete export list of include/fkv_transfer.h

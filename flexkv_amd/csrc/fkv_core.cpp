@@ -541,6 +541,7 @@ int shape_for_now(const KernelPlan &p, int64_t bytes, hipStream_t stream, CopyKe
   a->packed_grid_pct = pol.packed_grid_pct;
   a->xcd_mask = 0;
   a->claims_per_wg = pol.all_claims_per_wg;
+  a->lane_runs = !p.h2d && pol.d2h_lane_runs != 0;
   if (pol.arbiter == 3) {
     // tests: a mask that names no XCD of the device, every workgroup but the
     // safety net leaves
@@ -552,6 +553,7 @@ int shape_for_now(const KernelPlan &p, int64_t bytes, hipStream_t stream, CopyKe
     a->xcd_mask = busy_mask;
     workgroups = busy_workgroups;
     a->claims_per_wg = pol.busy_claims_per_wg;
+    a->lane_runs = !p.h2d && pol.d2h_lane_runs == 2; // next to traffic the other way: see copy_slice
   } else if (pol.arbiter == 1 && home_mask != all && pol.home_min_kb >= 0 &&
              bytes >= (int64_t)pol.home_min_kb * 1024) {
     a->xcd_mask = home_mask;

@@ -141,6 +141,7 @@ struct CopyKernelArgs {
   int32_t unroll;   // vector accesses in flight per lane: kCopyUnroll (also for 0), or
                     // kCopyUnrollDeep where launch_copy_kernel finds the launch fit for it
   int32_t packed;   // set by launch_copy_kernel: chunks shorter than a slice, see the kernel
+  int32_t lane_runs; // stores into pinned host memory: a lane moves adjacent vectors (see copy_slice)
   int32_t packed_grid_pct; // workgroups to launch in packed mode, percent of the request (0 = 100)
   uint32_t xcd_mask; // bit k: workgroups that run on XCD k take part; 0 = all
   uint32_t xcd_present;        // host side: the XCDs of the device (0 = eight, ids 0-7)

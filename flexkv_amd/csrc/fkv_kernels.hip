@@ -80,23 +80,34 @@ template <typename V, bool NT> __device__ __forceinline__ void put(V v, V *p) {
     *p = v;
 }
 
-template <int VEC, bool NTS, int UNR>
+// Which vector of the slice access u of a lane moves.  Ordinarily an access of the
+// wavefront covers 64 adjacent vectors (1 KiB).  With LANE_RUNS a lane moves UNR
+// adjacent vectors instead, 128 bytes with 16-byte vectors: the stores of a wavefront
+// then complete whole 128-byte lines lane by lane, which the link towards pinned host
+// memory takes about 1 % faster when nothing comes the other way (8 GiB GPU->host:
+// 57.0 against 56.4 GB/s; a pinned hipMemcpy: 57.0), and 2 % slower in sum when the
+// other direction is busy (64 requests both ways: 91.2 against 93.0 GB/s).  The launch
+// chooses (CopyKernelArgs::lane_runs); the form is a template parameter because a
+// kernel that carries both runs the ordinary one slower (55.8 against 56.2 GB/s).
+template <int VEC, bool NTS, int UNR, bool LANE_RUNS>
 __device__ __forceinline__ void copy_slice(const uint8_t *__restrict__ src,
-                                           uint8_t *__restrict__ dst,
-                                           int64_t bytes_in_slice, int lane) {
+                                              uint8_t *__restrict__ dst,
+                                              int64_t bytes_in_slice, int lane) {
   using V = typename VecType<VEC>::type;
   constexpr int64_t kSliceBytes = (int64_t)kWave * UNR * VEC;
-  const V *__restrict__ s = reinterpret_cast<const V *>(src) + lane;
-  V *__restrict__ d = reinterpret_cast<V *>(dst) + lane;
+  constexpr int kLaneStep = LANE_RUNS ? UNR : 1, kAccessStep = LANE_RUNS ? 1 : kWave;
+  const int first = lane * kLaneStep;
+  const V *__restrict__ s = reinterpret_cast<const V *>(src);
+  V *__restrict__ d = reinterpret_cast<V *>(dst);
   // launches with deep unroll have whole slices only (checked where they are shaped)
   if (UNR != kCopyUnroll || bytes_in_slice == kSliceBytes) {
     V r[UNR];
 #pragma unroll
     for (int u = 0; u < UNR; ++u)
-      r[u] = __builtin_nontemporal_load(s + u * kWave);
+      r[u] = __builtin_nontemporal_load(s + first + u * kAccessStep);
 #pragma unroll
     for (int u = 0; u < UNR; ++u)
-      put<V, NTS>(r[u], d + u * kWave);
+      put<V, NTS>(r[u], d + first + u * kAccessStep);
   } else {
     // the short last slice of a chunk: same shape, lanes beyond the end sit out
     // (they re-read the last vector rather than branch around the load)
@@ -104,11 +115,11 @@ __device__ __forceinline__ void copy_slice(const uint8_t *__restrict__ src,
     V r[UNR];
 #pragma unroll
     for (int u = 0; u < UNR; ++u)
-      r[u] = __builtin_nontemporal_load(s - lane + min(lane + u * kWave, nvec - 1));
+      r[u] = __builtin_nontemporal_load(s + min(first + u * kAccessStep, nvec - 1));
 #pragma unroll
     for (int u = 0; u < UNR; ++u)
-      if (lane + u * kWave < nvec)
-        put<V, NTS>(r[u], d + u * kWave);
+      if (first + u * kAccessStep < nvec)
+        put<V, NTS>(r[u], d + first + u * kAccessStep);
   }
 }
 
@@ -226,7 +237,7 @@ struct Shares {
 
 // Copies the work units of `a` that fall into [num0/den, num1/den) of the job.
 // `load_tables`: the base tables of `a` are not in LDS yet.
-template <int VEC, bool NTS, int UNR>
+template <int VEC, bool NTS, int UNR, bool LR>
 __device__ __forceinline__ void copy_share(const CopyKernelArgs &a, uint64_t num0, uint64_t num1,
                                            uint64_t den, uint64_t *lds, bool load_tables) {
   uint64_t *s_base_src = lds;
@@ -342,12 +353,12 @@ __device__ __forceinline__ void copy_share(const CopyKernelArgs &a, uint64_t num
       const uint8_t *src =
           reinterpret_cast<const uint8_t *>(s_base_src[i] + (uint64_t)s_off_src[p]) + off;
       uint8_t *dst = reinterpret_cast<uint8_t *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + off;
-      copy_slice<VEC, NTS, UNR>(src, dst, left < kSliceBytes ? left : kSliceBytes, lane);
+      copy_slice<VEC, NTS, UNR, LR>(src, dst, left < kSliceBytes ? left : kSliceBytes, lane);
     }
   }
 }
 
-template <int VEC, bool NTS, int U>
+template <int VEC, bool NTS, int U, bool LR = false>
 __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
     CopyKernelArgs a) {
   extern __shared__ uint64_t lds[];
@@ -358,7 +369,7 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
   bool load_tables = true;
   uint32_t part, parts;
   while (shares.next(&s_claim, &part, &parts)) {
-    copy_share<VEC, NTS, U>(a, part, part + 1, parts, lds, load_tables);
+    copy_share<VEC, NTS, U, LR>(a, part, part + 1, parts, lds, load_tables);
     load_tables = false;
   }
 }
@@ -367,7 +378,7 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_chunks_kernel(
 // restore, which differ in chunk size and strides): the jobs lie one behind the
 // other on a line, each as long as its weight (its bytes), and a share of the launch
 // is a stretch of that line.  Counters, mask and grid are those of job 0.
-template <int VEC, bool NTS, int U>
+template <int VEC, bool NTS, int U, bool LR = false>
 __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_jobs_kernel(CopyJobs t) {
   extern __shared__ uint64_t lds[];
   __shared__ uint32_t s_claim;
@@ -386,7 +397,7 @@ __global__ __launch_bounds__(kCopyBlockThreads) void fkv_copy_jobs_kernel(CopyJo
       const uint64_t lo = b0 > off ? (b0 - off < w ? b0 - off : w) : 0;
       const uint64_t hi = b1 > off ? (b1 - off < w ? b1 - off : w) : 0;
       if (lo < hi)
-        copy_share<VEC, NTS, U>(t.job[j], lo, hi, w, lds, true);
+        copy_share<VEC, NTS, U, LR>(t.job[j], lo, hi, w, lds, true);
       off += w;
     }
   }
@@ -401,6 +412,9 @@ int launch_vec(const CopyKernelArgs &a, int grid, int threads, size_t lds_bytes,
   else if (a.nt_store)
     hipLaunchKernelGGL((fkv_copy_chunks_kernel<VEC, true, kCopyUnroll>), dim3(grid), dim3(threads),
                        lds_bytes, stream, a);
+  else if (VEC == 16 && a.lane_runs)
+    hipLaunchKernelGGL((fkv_copy_chunks_kernel<16, false, kCopyUnroll, true>), dim3(grid),
+                       dim3(threads), lds_bytes, stream, a);
   else
     hipLaunchKernelGGL((fkv_copy_chunks_kernel<VEC, false, kCopyUnroll>), dim3(grid),
                        dim3(threads), lds_bytes, stream, a);
@@ -611,6 +625,9 @@ int launch_jobs_vec(const CopyJobs &t, int grid, int threads, size_t lds_bytes,
   if (t.job[0].nt_store)
     hipLaunchKernelGGL((fkv_copy_jobs_kernel<VEC, true, kCopyUnroll>), dim3(grid), dim3(threads),
                        lds_bytes, stream, t);
+  else if (VEC == 16 && t.job[0].lane_runs)
+    hipLaunchKernelGGL((fkv_copy_jobs_kernel<16, false, kCopyUnroll, true>), dim3(grid),
+                       dim3(threads), lds_bytes, stream, t);
   else
     hipLaunchKernelGGL((fkv_copy_jobs_kernel<VEC, false, kCopyUnroll>), dim3(grid), dim3(threads),
                        lds_bytes, stream, t);
@@ -653,6 +670,7 @@ int launch_copy_jobs(const CopyKernelArgs *jobs, int njobs, int num_workgroups,
   for (int j = 0; j < njobs; ++j) {
     CopyKernelArgs a = jobs[j];
     a.unroll = kCopyUnroll;
+    a.lane_runs = jobs[0].lane_runs; // the launch's choice, made for the first job
     if (a.vec != jobs[0].vec || a.nt_store != jobs[0].nt_store)
       return fail(FKV_ERR_RUNTIME, "copy kernel: jobs of one launch differ in vector width or store kind");
     int64_t job_total = 0;

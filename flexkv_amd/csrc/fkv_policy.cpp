@@ -35,6 +35,7 @@ const EnvField kEnv[] = {
     FKV_FIELD("FKV_STAGED_RESTORE", staged_restore),
     FKV_FIELD("FKV_CE_STAGING_MB", ce_staging_mb),
     FKV_FIELD("FKV_CE_TWO_STREAMS", ce_two_streams),
+    FKV_FIELD("FKV_D2H_LANE_RUNS", d2h_lane_runs),
 };
 #undef FKV_FIELD
 
@@ -119,6 +120,7 @@ void sanitize(fkv_launch_policy &p, const fkv_launch_policy &derived) {
   p.model_host_pass_mbps = clampi(p.model_host_pass_mbps, 100, 10000000);
   p.model_launch_ns = clampi(p.model_launch_ns, 0, 10000000);
   p.model_prefer_ce_pct = clampi(p.model_prefer_ce_pct, 1, 1000);
+  p.d2h_lane_runs = clampi(p.d2h_lane_runs, 0, 2);
 }
 
 // The table of a device with the XCDs `present`, environment applied.
@@ -171,6 +173,7 @@ fkv_launch_policy defaults_for(uint32_t present) {
   p.model_host_pass_mbps = 20000;
   p.model_launch_ns = 15000;
   p.model_prefer_ce_pct = 103;
+  p.d2h_lane_runs = 1;
   for (const EnvField &f : kEnv) {
     const char *v = std::getenv(f.name);
     if (v && *v) // decimal, 0x.. or 0.. as written

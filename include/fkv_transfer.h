@@ -708,7 +708,11 @@ typedef struct fkv_launch_policy {
   int32_t model_launch_ns;          /* plan + launch of the kernel path */
   int32_t model_prefer_ce_pct;      /* the copy engine wins up to this percentage of the kernel's
                                        time: it leaves the CUs and their memory queues alone */
-  int32_t reserved[6];
+  int32_t d2h_lane_runs;      /* GPU->host launches with 16-byte vectors let every lane store 128
+                                 adjacent bytes instead of every wavefront access 1 KiB: 0 never,
+                                 1 (default) unless the other direction is busy, 2 always (about
+                                 +1 % alone on the link, -2 % in sum next to traffic the other way) */
+  int32_t reserved[5];
 } fkv_launch_policy;
 /* The table of `device` (-1 = current).  The first call for a device runs the probe kernel. */
 int fkv_launch_policy_get(int32_t device, fkv_launch_policy *out);

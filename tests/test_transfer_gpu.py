@@ -378,6 +378,29 @@ def test_every_way_a_launch_can_share_out_its_work(gpu_device, mode):
         assert st["safety_net_ranges"] - before > 0, st   # the fallback workgroup did the work
 
 
+@pytest.mark.parametrize("lane_runs", [0, 1, 2])
+def test_both_store_orders_towards_host_memory(gpu_device, lane_runs):
+    """GPU->host launches with 16-byte vectors store either 1 KiB per wavefront access
+    or 128 adjacent bytes per lane (d2h_lane_runs: never / unless the link is busy the
+    other way / always, here also with launches forced into the busy shape).  Whole
+    slices, chunks that end in a short slice, chunks shorter than a slice, 8-byte
+    vectors and the fused launch of several groups: the oracle's bytes every time."""
+    from flexkv_amd.c_ext import launch_policy
+    for arbiter in (1, 2):
+        with launch_policy(d2h_lane_runs=lane_runs, arbiter=arbiter):
+            for chunk, n in ((32768, 90), (18432, 70), (8192 + 16, 64), (2304, 300), (4104, 80)):
+                s = KVSetup(VLLM, 5, 2, n + 20, n + 20, chunk, "BLOCKFIRST", seed=chunk + lane_runs)
+                dev = s.to_device(gpu_device)
+                rng = np.random.default_rng(chunk)
+                for h2d in (False, True, False):
+                    g, c = rng.permutation(n + 20)[:n], rng.permutation(n + 20)[:n]
+                    print(f"case lane_runs={lane_runs} arbiter={arbiter} chunk={chunk} h2d={h2d}",
+                          flush=True)
+                    dev.transfer(g, c, is_h2d=h2d)
+                    s.oracle_transfer(g, c, h2d)
+                dev.assert_matches_reference(f"lane_runs={lane_runs}, chunk {chunk}")
+
+
 def test_the_launch_policy_follows_the_device(gpu_device):
     """Masks are derived from the XCDs the device exposes: disjoint halves for the
     two directions, the home XCDs of a direction include its busy XCDs, and a set
