@@ -47,7 +47,7 @@ METRIC = "KV block transfer GB/s (D2H, H2D) on 1 GPU; % of measured host-link pe
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs of this script scaled by plain copy kernels of known size
 # (profiles/fkv_copy_chunks_kernel_c1_pmc.md).  None where no such run was made.
-MEASURED_TRAFFIC_BYTES = {("c1", "kernel"): 8590414848, ("transform-c0", "kernel"): 8593325056}
+MEASURED_TRAFFIC_BYTES = {("c1", "kernel"): 8590410496, ("transform-c0", "kernel"): 8593325056}
 
 
 def _median(xs):
@@ -1229,7 +1229,7 @@ def link_roofline(rec, link, traffic=None):
     peak_link = (link["d2h"] + link["h2d"]) / 2
     return {"bound": "hbm", "achieved": round(achieved, 3), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 5), "traffic": traffic,
-            "kernel": "fkv_copy_chunks_kernel<16, false|true>",
+            "kernel": "fkv_copy_chunks_kernel<16, false, 8, true> (GPU->host), <16, true, 8, false> (host->GPU)",
             "algorithmic_bytes_per_launch": B, "avg_launch_ms": rec["avg_launch_ms"],
             "limited_by": "host link (PCIe), not HBM: one side of every copy is host memory",
             "link_peak_GBps": round(peak_link, 3),
