@@ -1495,7 +1495,7 @@ def transform_record(torch, device, args, steps, warmup):
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(("transform-" + args.shape, "kernel")),
-                     "kernel": "fkv_copy_chunks_kernel<16, true>",
+                     "kernel": "fkv_copy_chunks_kernel<16, true, 16, false>",
                      "workload": f"transform-{args.shape}: " + r["desc"],
                      "algorithmic_bytes_per_launch": 2 * r["bytes"],
                      "avg_launch_ms": round(avg_ms, 4), "bit_exact": r["bit_exact"],
