@@ -716,6 +716,48 @@ HostOrder host_order(const fkv_transfer_desc &d) {
   return o;
 }
 
+// How GATHER_DIRECT cuts a transfer into staging groups (also what the engine choice
+// prices): copy commands per run of consecutive host blocks, blocks per group, and
+// whether two half-size buffers alternate.
+struct GatherDirectShape {
+  size_t block_bytes = 0;
+  bool full_block = false;
+  size_t cap_blocks = 1, total_cmds = 0, group = 1;
+  bool pipelined = false;
+  bool enable_memcpy2d = false;
+  // Copy commands of `rows` consecutive host blocks: one where the bytes are one run
+  // (whole blocks) or a 2-D copy takes the rows (asked for by the caller, or three rows
+  // and more: a layer-by-layer restore of 512 adjacent host blocks, 72 KiB of each per
+  // layer, runs at 53.5 GB/s with one 2-D copy per layer, and a multi-group restore went
+  // from 9.9 to 40.8 GB/s); else one per row.
+  bool two_d(size_t rows) const { return enable_memcpy2d || rows >= 3; }
+  size_t cmds_of(size_t rows) const { return full_block || two_d(rows) ? (size_t)1 : rows; }
+};
+GatherDirectShape gather_direct_shape(const fkv_transfer_desc &d, const HostOrder &order,
+                                      size_t staging_cap, bool may_pipeline) {
+  GatherDirectShape g;
+  g.block_bytes = (size_t)d.num_layers * d.kv_dim * (size_t)d.chunk_size;
+  g.full_block = (int64_t)g.block_bytes == d.cpu_block_stride;
+  g.enable_memcpy2d = d.ce.enable_memcpy2d != 0;
+  g.cap_blocks = std::max<size_t>(1, staging_cap / std::max<size_t>(1, g.block_bytes));
+  for (size_t r = 0; r + 1 < order.run_start.size(); ++r)
+    g.total_cmds += g.cmds_of((size_t)(order.run_start[r + 1] - order.run_start[r]));
+  // A transfer that needs several groups and moves in few, large copies alternates
+  // between two buffers of half the size: the compaction launch of a group runs next
+  // to the copies of its neighbour instead of between them (8 GiB in 1 GiB groups:
+  // 8 x 0.36 ms of launches off the critical path of 8 x 18.7 ms of copies; 55.9 ->
+  // 56.6 GB/s).  Transfers of many small copies stay on the one-buffer path, whose
+  // copies alternate between two streams: that hides the fixed cost per copy, which is
+  // worth more there, and GPU->host transfers of 2 MiB copies on two copy streams next
+  // to the compaction launches ran at half rate every few calls.
+  const size_t half = std::max<size_t>(1, g.cap_blocks / 2);
+  const size_t groups_if_pipelined = ((size_t)d.num_blocks + half - 1) / half;
+  g.pipelined = may_pipeline && (size_t)d.num_blocks > g.cap_blocks && g.cap_blocks >= 2 &&
+                g.total_cmds <= 2 * groups_if_pipelined;
+  g.group = std::min<size_t>((size_t)std::max(d.num_blocks, 1), g.pipelined ? half : g.cap_blocks);
+  return g;
+}
+
 int gather_direct(const Job &j) {
   const auto &d0 = j.d;
   const int lk = d0.num_layers * d0.kv_dim;
@@ -727,35 +769,16 @@ int gather_direct(const Job &j) {
   fkv_transfer_desc d = d0; // the same transfer, positions in host order
   d.gpu_block_ids = order.gpu_ids.data();
   d.cpu_block_ids = order.cpu_ids.data();
-  const size_t block_bytes = (size_t)lk * (size_t)d.chunk_size;
-  const bool full_block = (int64_t)block_bytes == d.cpu_block_stride;
-  // Copy commands of `rows` consecutive host blocks: one where the bytes are one run
-  // (whole blocks) or a 2-D copy takes the rows (asked for by the caller, or three rows
-  // and more: a layer-by-layer restore of 512 adjacent host blocks, 72 KiB of each per
-  // layer, runs at 53.5 GB/s with one 2-D copy per layer, and a multi-group restore went
-  // from 9.9 to 40.8 GB/s); else one per row.
-  auto two_d = [&](size_t rows) { return d.ce.enable_memcpy2d || rows >= 3; };
-  auto cmds_of = [&](size_t rows) { return full_block || two_d(rows) ? (size_t)1 : rows; };
-  const size_t cap_blocks = std::max<size_t>(1, staging_cap_bytes() / block_bytes);
-  // A transfer that needs several groups and moves in few, large copies alternates
-  // between two buffers of half the size: the compaction launch of a group runs next
-  // to the copies of its neighbour instead of between them (8 GiB in 1 GiB groups:
-  // 8 x 0.36 ms of launches off the critical path of 8 x 18.7 ms of copies; 55.9 ->
-  // 56.6 GB/s).  Transfers of many small copies stay on the one-buffer path, whose
-  // copies alternate between two streams: that hides the fixed cost per copy, which is
-  // worth more there, and GPU->host transfers of 2 MiB copies on two copy streams next
-  // to the compaction launches ran at half rate every few calls.
   StageSet &ss = stage_set(j.device);
-  const size_t half = std::max<size_t>(1, cap_blocks / 2);
-  const size_t groups_if_pipelined = ((size_t)d.num_blocks + half - 1) / half;
-  size_t total_cmds = 0;
-  for (size_t r = 0; r + 1 < order.run_start.size(); ++r)
-    total_cmds += cmds_of((size_t)(order.run_start[r + 1] - order.run_start[r]));
-  const bool pipelined = (size_t)d.num_blocks > cap_blocks && cap_blocks >= 2 &&
-                         total_cmds <= 2 * groups_if_pipelined && pipeline_enabled() &&
-                         ss.ensure_pipeline();
+  GatherDirectShape shape = gather_direct_shape(d, order, staging_cap_bytes(), pipeline_enabled());
+  if (shape.pipelined && !ss.ensure_pipeline())
+    shape = gather_direct_shape(d, order, staging_cap_bytes(), false);
+  const size_t block_bytes = shape.block_bytes;
+  const bool full_block = shape.full_block, pipelined = shape.pipelined;
+  auto two_d = [&](size_t rows) { return shape.two_d(rows); };
+  auto cmds_of = [&](size_t rows) { return shape.cmds_of(rows); };
   const int nbuf = pipelined ? 2 : 1;
-  const int group = (int)std::min<size_t>((size_t)d.num_blocks, pipelined ? half : cap_blocks);
+  const int group = (int)shape.group;
   uint8_t *stages[2] = {nullptr, nullptr};
   for (int k = 0; k < nbuf; ++k) {
     stages[k] = device_stage(j.device, k, (size_t)group * block_bytes, j.stream);
@@ -955,10 +978,13 @@ CeWork ce_work(const Job &j, int path) {
     break;
   default: // GATHER_DIRECT
     if (host_block_dense(d)) {
-      const bool full = iters * (double)d.chunk_size == (double)d.cpu_block_stride;
-      // one command per run of consecutive host blocks, whatever the GPU side looks like
-      w.dmas = (full || d.ce.enable_memcpy2d) ? (double)(host_order(d).run_start.size() - 1) : n;
-      w.device_staged = bytes;
+      // one command per run of consecutive host blocks, whatever the GPU side looks like;
+      // with two staging buffers only the first group's compaction is on the critical path
+      const fkv_launch_policy pol = policy_peek(d.device < 0 ? current_device() : d.device);
+      const GatherDirectShape g = gather_direct_shape(d, host_order(d), (size_t)pol.ce_staging_mb << 20,
+                                                      pol.ce_two_streams == 1);
+      w.dmas = (double)g.total_cmds;
+      w.device_staged = g.pipelined ? (double)g.group * (double)g.block_bytes : bytes;
     } else {
       staged();
     }

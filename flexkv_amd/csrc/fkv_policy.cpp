@@ -162,14 +162,14 @@ fkv_launch_policy defaults_for(uint32_t present) {
                             // compute units stay free; 5 MiB copies: 51 against 56 GB/s
   // Measured on MI355X: a DMA command costs about 2.5 us beyond its bytes when copies
   // alternate over two streams (256 x 2 MiB: 50-54 GB/s; 2048 x 5 MiB: 56.2 GB/s); the
-  // compaction pass runs at 1.5 TB/s or more; a host scatter/gather pass at about
-  // 20 GB/s with four threads; the gather/scatter kernel reaches 56.4 GB/s GPU->host
-  // and 57.2 GB/s host->GPU.
+  // compaction pass stages 2.8 TB/s (512 MiB in 0.19 ms); a host scatter/gather pass
+  // runs at about 20 GB/s with four threads; the gather/scatter kernel reaches
+  // 57.0 GB/s GPU->host and 57.2 GB/s and more host->GPU.
   p.model_link_mbps = 57200;
-  p.model_kernel_d2h_mbps = 56400;
+  p.model_kernel_d2h_mbps = 57000;
   p.model_kernel_h2d_mbps = 57200;
   p.model_dma_ns = 2500;
-  p.model_compaction_gbps = 1500;
+  p.model_compaction_gbps = 2800;
   p.model_host_pass_mbps = 20000;
   p.model_launch_ns = 15000;
   p.model_prefer_ce_pct = 103;
