@@ -1031,6 +1031,15 @@ int run_ce_path(const fkv_transfer_desc &d, hipStream_t stream) {
         d.is_host_to_device ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost, {}};
   const int rect_min_kb = policy_of(device).ce_rect_min_kb;
   j.rect_min_bytes = rect_min_kb < 0 ? -1 : (int64_t)rect_min_kb * 1024;
+  if (j.rect_min_bytes >= 0) {
+    // 2-D copies for pinned host memory only: the runtime stages pageable memory
+    // through buffers of its own whatever the call
+    hipPointerAttribute_t at{};
+    if (hipPointerGetAttributes(&at, d.cpu_ptr) != hipSuccess || at.type != hipMemoryTypeHost) {
+      (void)hipGetLastError();
+      j.rect_min_bytes = -1;
+    }
+  }
   analyze(d.gpu_block_ids, d.cpu_block_ids, d.num_blocks, d.cpu_block_stride, d.chunk_size,
           d.gpu_block_stride, j.an);
   int path = FKV_CE_PER_BLOCK;

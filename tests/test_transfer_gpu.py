@@ -263,13 +263,18 @@ def test_pageable_host_tensor_is_refused_by_the_kernel_path(gpu_device):
                            ids, pageable, s.cpu_kv_stride, s.cpu_layer_stride, s.cpu_block_stride,
                            s.chunk, 0, 2, is_host_to_device=False)
     # the copy-engine path reads ids and data through the runtime and accepts pageable memory
-    transfer_kv_blocks(ids, dev.ptrs, s.gpu_kv_stride, s.gpu_block_stride, s.gpu_layer_stride,
-                       ids, pageable, s.cpu_kv_stride, s.cpu_layer_stride, s.cpu_block_stride,
-                       s.chunk, 0, 2, is_host_to_device=False, use_ce_transfer=True)
-    torch.cuda.synchronize()
-    s.host_ref[:] = 0
-    s.oracle_transfer(ids.numpy(), ids.numpy(), False)
-    np.testing.assert_array_equal(pageable.numpy(), s.host_ref)
+    # (also when every copy of pinned memory would go out as a 2-D copy)
+    from flexkv_amd.c_ext import launch_policy
+    for rect_min_kb in (-1, 0):
+        pageable.zero_()
+        with launch_policy(ce_rect_min_kb=rect_min_kb):
+            transfer_kv_blocks(ids, dev.ptrs, s.gpu_kv_stride, s.gpu_block_stride, s.gpu_layer_stride,
+                               ids, pageable, s.cpu_kv_stride, s.cpu_layer_stride, s.cpu_block_stride,
+                               s.chunk, 0, 2, is_host_to_device=False, use_ce_transfer=True)
+            torch.cuda.synchronize()
+        s.host_ref[:] = 0
+        s.oracle_transfer(ids.numpy(), ids.numpy(), False)
+        np.testing.assert_array_equal(pageable.numpy(), s.host_ref)
 
 
 def test_streams_run_concurrently_tells_hardware_queue_sharing(gpu_device):
