@@ -304,19 +304,22 @@ __device__ __forceinline__ void copy_share(const CopyKernelArgs &a, uint64_t num
       using V = typename VecType<VEC>::type;
       const uint32_t lim = (uint32_t)(t1 - tile_s0); // < kCopyIdTile * spp, checked on host
       const uint32_t ulk = (uint32_t)a.lk;
-      const uint32_t q64 = kWave / vpc, r64 = kWave % vpc; // kWave vectors = q64 chunks + r64
+      // distance between two accesses of a lane and between the first accesses of two
+      // lanes, in vectors (see copy_slice for the two orders)
+      constexpr uint32_t kStep = LR ? 1 : kWave, kLaneStep = LR ? UNR : 1;
+      const uint32_t q64 = kStep / vpc, r64 = kStep % vpc; // kStep vectors = q64 chunks + r64
       const uint32_t qlk = q64 / ulk, rlk = q64 % ulk;     // q64 chunks = qlk positions + rlk
       for (uint32_t v0 = (uint32_t)(t0 - tile_s0) + wave * kPiece; v0 < lim;
            v0 += nwaves * kPiece) {
         V r[UNR];
         V *d[UNR];
-        // A lane's vectors are kWave apart.  The first one is located by division;
+        // A lane's vectors are kStep apart.  The first one is located by division;
         // each further one by adding the precomputed quotients and remainders of
-        // kWave, which costs a few compares instead of two divisions.  Lanes beyond
+        // kStep, which costs a few compares instead of two divisions.  Lanes beyond
         // the end stay on their last valid vector and re-read it rather than branch
         // around the load: all loads of a piece are issued back to back, only the
         // stores are predicated.
-        uint32_t v = v0 + lane;
+        uint32_t v = v0 + lane * kLaneStep;
         const uint32_t vc = min(v, lim - 1);
         const uint32_t c = vc / vpc; // chunk inside the tile: position * lk + i
         uint32_t w = vc - c * vpc;
@@ -325,7 +328,7 @@ __device__ __forceinline__ void copy_share(const CopyKernelArgs &a, uint64_t num
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
           if (u > 0) {
-            v += kWave;
+            v += kStep;
             uint32_t w2 = w + r64, i2 = i + rlk, p2 = p + qlk;
             if (w2 >= vpc) {
               w2 -= vpc;
@@ -342,11 +345,11 @@ __device__ __forceinline__ void copy_share(const CopyKernelArgs &a, uint64_t num
           }
           const V *src = reinterpret_cast<const V *>(s_base_src[i] + (uint64_t)s_off_src[p]) + w;
           d[u] = reinterpret_cast<V *>(s_base_dst[i] + (uint64_t)s_off_dst[p]) + w;
-          r[u] = __builtin_nontemporal_load(src);
+          r[u] = get<V, !LR>(src);
         }
 #pragma unroll
         for (int u = 0; u < UNR; ++u)
-          if (v0 + u * kWave + lane < lim)
+          if (v0 + u * kStep + lane * kLaneStep < lim)
             put<V, NTS>(r[u], d[u]);
       }
       continue;
