@@ -308,7 +308,9 @@ struct Job {
   // likes.
   int dma(void *dst, const void *src, size_t bytes, hipMemcpyKind k) const {
     stats().dma_copies.fetch_add(1, std::memory_order_relaxed);
-    if (rect_min_bytes >= 0 && (int64_t)bytes >= rect_min_bytes && !host_waits)
+    // (a row of a 2-D copy, and its pitch, stay below 2 GiB)
+    if (rect_min_bytes >= 0 && (int64_t)bytes >= rect_min_bytes && !host_waits &&
+        bytes < ((size_t)1 << 31))
       FKV_HIP_TRY(hipMemcpy2DAsync(dst, bytes, src, bytes, bytes, 1, k, next_stream()));
     else
       FKV_HIP_TRY(hipMemcpyAsync(dst, src, bytes, k, next_stream()));
