@@ -127,10 +127,13 @@ class Workload:
             self.gpu_ids = t.randperm(N, generator=gg)[:2048].to(t.int64)
             self.gpu_ids_reload = t.randperm(N, generator=gg)[:2048].to(t.int64)
             self.cpu_ids = t.arange(2048, dtype=t.int64)
-        elif name == "c3":
+        elif name in ("c3", "c3f"):
             L, N, T, D = 61, 16384, 64, 576
+            self.NH = 512 if name == "c3" else 4096
             self.desc = ("DeepSeek-V3 MLA latent KV bf16: 61 x [16384,64,576], layerwise restore of "
-                         "512 blocks, host [512,61,1,64,1,576]")
+                         "512 blocks, host [%d,61,1,64,1,576]%s" % (
+                             self.NH, "" if name == "c3" else
+                             ", host block ids scattered over the pool (512 runs of one block)"))
             self.backend, self.kv_dim, self.L, self.num_kv_heads = 0, 1, L, 1
             self.chunk = T * D * 2
             gen = t.Generator(device=device).manual_seed(4)
@@ -138,7 +141,6 @@ class Workload:
                             for _ in range(L)]
             self.num_gpu_blocks = N
             self.gks, self.gbs, self.gls = N * self.chunk, self.chunk, N * self.chunk
-            self.NH = 512
             gg = g(4)
             self.gpu_ids = t.randperm(N, generator=gg)[:512].to(t.int64)
             self.cpu_ids = t.randperm(self.NH, generator=gg)[:512].to(t.int64)
@@ -152,6 +154,18 @@ class Workload:
         self.ptrs = t.tensor([x.data_ptr() for x in self.tensors], dtype=t.int64).pin_memory()
         self.num_blocks = int(self.gpu_ids.numel())
         self.bytes_per_direction = self.num_blocks * self.L * self.kv_dim * self.chunk
+
+    def fragment_host_pool(self, pool_blocks=4096, seed=44):
+        """c3 -> c3f in place: the same engine tensors and GPU blocks, a host pool of
+        `pool_blocks` blocks and host block ids scattered over it."""
+        t = self.torch
+        self.name, self.NH = "c3f", pool_blocks
+        self.desc = self.desc.replace("host [512,", "host [%d," % pool_blocks) + \
+            ", host block ids scattered over the pool (512 runs of one block)"
+        self.host = None
+        self.host = t.empty(self.NH * self.cbs, dtype=t.uint8, pin_memory=True)
+        gg = t.Generator().manual_seed(seed)
+        self.cpu_ids = t.randperm(self.NH, generator=gg)[:self.num_blocks].to(t.int64)
 
     def transfer(self, gpu_ids, cpu_ids, h2d, **kw):
         from flexkv_amd.c_ext import transfer_kv_blocks
@@ -399,7 +413,7 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=F
     restore_alone_ms = min(alone[1:]) if len(alone) > 1 else alone[0]
 
     from flexkv_amd.c_ext import get_stats
-    staged_before = get_stats()["staged_batches"]
+    st0 = get_stats()
     totals, restores, firsts, stalls, busy = [], [], [], [], []
     for it in range(warmup + steps):
         torch.cuda.synchronize()
@@ -433,8 +447,16 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=F
             busy.append(computing)
             stalls.append(total - computing)  # compute stream idle, waiting for a layer
     grp.close()
-    staged = (get_stats()["staged_batches"] - staged_before) // (warmup + steps)
-    return dict(staged_batches_per_restore=staged,
+    st1 = get_stats()
+    per = lambda k: (st1[k] - st0[k]) / (warmup + steps)
+    staged, gathered = int(per("staged_batches")), int(per("gathered_batches"))
+    route = ("copy engine (use_ce_transfer)" if use_ce else
+             "kernel" if staged == 0 else
+             "host threads gather each layer into a pinned buffer, one copy-engine command per "
+             "layer, scatter launch%s" % (" (first layer by kernel)" if staged < w.L else "")
+             if gathered else "copy engines, one command per run of host blocks, scatter launch")
+    return dict(staged_batches_per_restore=staged, gathered_batches_per_restore=gathered,
+                gather_busy_ms_per_restore=round(per("gather_busy_us") / 1e3, 3), route=route,
                 total_ms=_median(totals), restore_ms=_median(restores),
                 first_layer_ms=_median(firsts), compute_ms=compute_ms,
                 compute_overlapped_ms=_median(busy), stall_ms=_median(stalls),
@@ -1090,18 +1112,19 @@ def cpu_baseline(cfg, budget_s=5.0):
         sample = (f"{n} of 2048 blocks of [80,2,8,32,128] fp8 bytes out of a {N}-block pool, "
                   f"whole-block index_select into the host cache and index_copy_ back into another "
                   f"permutation")
-    elif cfg == "c3":
+    elif cfg in ("c3", "c3f"):
         L, N, T, D, n = 8, 2048, 64, 576, 512
+        pool = n if cfg == "c3" else 4 * n   # c3f: host blocks scattered over a larger pool
         planes = [[filled(N, T, D)] for _ in range(L)]
-        host = filled(n, L, 1, T, D)
+        host = filled(pool, L, 1, T, D)
         gi = torch.randperm(N, generator=g)[:n]
-        ci = torch.randperm(n, generator=g)
+        ci = torch.randperm(pool, generator=g)[:n]
         nbytes = n * L * T * D * 2
 
         def step():
             O.torch_index_scatter_planes(planes, host, gi, ci)     # the restore direction only
         sample = (f"{L} of 61 layers, 512 blocks of 64x576 bf16 (kv_dim 1) into a {N}-block pool "
-                  f"per layer, index_select from the host cache [512,L,1,64,576] + index_copy_")
+                  f"per layer, index_select from the host cache [{pool},L,1,64,576] + index_copy_")
     else:
         raise ValueError(cfg)
     step()
@@ -1150,7 +1173,10 @@ def overlap_record(r, B, link):
             "overlap_frac_beyond_first_layer": round(1.0 - beyond_first / max(1e-9, shorter), 4),
             "fully_overlapped_beyond_first_layer": bool(
                 r["total_ms"] <= 1.1 * longer + r["first_layer_ms"]),
-            "staged_batches_per_restore": r.get("staged_batches_per_restore")}
+            "staged_batches_per_restore": r.get("staged_batches_per_restore"),
+            "gathered_batches_per_restore": r.get("gathered_batches_per_restore"),
+            "host_gather_thread_ms_per_restore": r.get("gather_busy_ms_per_restore"),
+            "route": r.get("route")}
 
 
 def measure_config(name, args, torch, device, link, steps, warmup):
@@ -1178,29 +1204,16 @@ def measure_config(name, args, torch, device, link, steps, warmup):
                    avg_launch_ms=round(avg_ms, 4), path_taken=taken)
         if not args.no_verify:
             out["bit_exact"] = verify_round_trip(w, torch, args.num_cta)
-    elif name == "c3":
-        # fill the host cache with the blocks to restore, then erase them on the GPU
-        w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=args.num_cta, sync=True)
-        gi = w.gpu_ids.to(device)
-        saved = [w.gpu_rows(l, 0).index_select(0, gi) for l in range(w.L)]
-        for l in range(w.L):
-            w.gpu_rows(l, 0).index_fill_(0, gi, 0)
-        c_ext.reset_stats()
-        r = run_layerwise(w, torch, steps, warmup, args.num_cta, args.notify, args.dummy,
-                          layer_spans=args.layer_spans, use_ce=args.use_ce)
-        r["layers"] = w.L
-        restore = B / (r["restore_ms"] * 1e-3) / 1e9
-        out.update(value=round(restore, 3), ms_per_step=round(r["total_ms"], 3),
-                   h2d_GBps=round(restore, 3), h2d_frac_of_link=round(restore / link["h2d"], 4),
-                   notify=args.notify, dummy_compute=args.dummy, layer_bytes=r["layer_bytes"],
-                   layerwise=overlap_record(r, B, link))
-        if args.layer_spans:
-            out["layerwise"].update(
-                compute_while_restoring_ms=round(r["compute_overlapped_ms"], 3),
-                compute_slowdown=round(r["compute_overlapped_ms"] / r["compute_ms"], 3))
-        if not args.no_verify:
-            out["bit_exact"] = all(
-                torch.equal(w.gpu_rows(l, 0).index_select(0, gi), saved[l]) for l in range(w.L))
+    elif name in ("c3", "c3f"):
+        out.update(measure_layerwise(w, args, torch, device, link, steps, warmup))
+        if name == "c3" and getattr(args, "with_fragmented", False):
+            # the same restore out of a host pool after churn: 4096 host blocks, ids scattered
+            w.fragment_host_pool()
+            frag = {"workload": f"c3f: {w.desc}", "transfer_num_cta": args.num_cta,
+                    "blocks": w.num_blocks, "bytes_per_direction": B, "steps": steps,
+                    "warmup": warmup}
+            frag.update(measure_layerwise(w, args, torch, device, link, steps, warmup))
+            out["fragmented_record"] = frag
     else:  # c4
         r = run_concurrent(w, torch, steps, warmup, args.num_cta, args.streams_per_direction,
                            verify=not args.no_verify)
@@ -1217,6 +1230,38 @@ def measure_config(name, args, torch, device, link, steps, warmup):
                    frac_of_sum_of_one_way_peaks=round(agg / (link["d2h"] + link["h2d"]), 4))
     del w
     torch.cuda.empty_cache()
+    return out
+
+
+def measure_layerwise(w, args, torch, device, link, steps, warmup):
+    """c3 / c3f: the fields of a layerwise-restore record."""
+    import flexkv_amd.c_ext as c_ext
+    B = w.bytes_per_direction
+    # fill the host cache with the blocks to restore, then erase them on the GPU
+    w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=args.num_cta, sync=True)
+    gi = w.gpu_ids.to(device)
+    saved = [w.gpu_rows(l, 0).index_select(0, gi) for l in range(w.L)]
+    for l in range(w.L):
+        w.gpu_rows(l, 0).index_fill_(0, gi, 0)
+    c_ext.reset_stats()
+    r = run_layerwise(w, torch, steps, warmup, args.num_cta, args.notify, args.dummy,
+                      layer_spans=args.layer_spans, use_ce=args.use_ce)
+    r["layers"] = w.L
+    restore = B / (r["restore_ms"] * 1e-3) / 1e9
+    pol = c_ext.get_launch_policy()
+    out = dict(value=round(restore, 3), ms_per_step=round(r["total_ms"], 3),
+               h2d_GBps=round(restore, 3), h2d_frac_of_link=round(restore / link["h2d"], 4),
+               notify=args.notify, dummy_compute=args.dummy, layer_bytes=r["layer_bytes"],
+               path=r["route"], layerwise=overlap_record(r, B, link))
+    if r["gathered_batches_per_restore"]:
+        out["layerwise"]["host_gather_threads"] = pol["gather_threads"]
+    if args.layer_spans:
+        out["layerwise"].update(
+            compute_while_restoring_ms=round(r["compute_overlapped_ms"], 3),
+            compute_slowdown=round(r["compute_overlapped_ms"] / r["compute_ms"], 3))
+    if not args.no_verify:
+        out["bit_exact"] = all(
+            torch.equal(w.gpu_rows(l, 0).index_select(0, gi), saved[l]) for l in range(w.L))
     return out
 
 
@@ -1243,7 +1288,7 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--config", default="all",
-                    choices=["all", "c0", "c1", "c2", "c3", "c4", "copycal", "notify", "mg", "worker",
+                    choices=["all", "c0", "c1", "c2", "c3", "c3f", "c4", "copycal", "notify", "mg", "worker",
                              "ssd", "transform", "groups", "staging"])
     ap.add_argument("--shape", default="c0", choices=["c0", "c3"],
                     help="transform: which engine shape to re-lay out")
@@ -1264,6 +1309,12 @@ def main():
     ap.add_argument("--staged-restore", type=int, default=None, choices=[0, 1, 2],
                     help="c3: 0 keeps the restore on the kernel path, 1 lets the library choose "
                          "(default), 2 sends it through the copy engines whenever the layout allows")
+    ap.add_argument("--staged-gather", type=int, default=None, choices=[0, 1, 2],
+                    help="c3 / c3f: 0 never lets host threads gather the rows of a layer, 1 lets "
+                         "the library choose (default), 2 whenever the run-by-run route is not taken")
+    ap.add_argument("--gather-threads", type=int, default=None,
+                    help="c3 / c3f: host threads that gather (default 6)")
+    ap.add_argument("--gather-first-by-kernel", type=int, default=None, choices=[0, 1])
     ap.add_argument("--overlap-directions", action="store_true",
                     help="worker: the worker runs gets next to puts (second thread and stream)")
     ap.add_argument("--layer-spans", action="store_true",
@@ -1301,6 +1352,12 @@ def main():
     torch.cuda.set_device(0)
     if args.staged_restore is not None:
         c_ext.set_launch_policy(staged_restore=args.staged_restore)
+    if args.staged_gather is not None:
+        c_ext.set_launch_policy(staged_gather=args.staged_gather)
+    if args.gather_threads is not None:
+        c_ext.set_launch_policy(gather_threads=args.gather_threads)
+    if args.gather_first_by_kernel is not None:
+        c_ext.set_launch_policy(gather_first_by_kernel=args.gather_first_by_kernel)
 
     if args.config == "copycal":
         # Plain device-to-device copies of a known size: the yardstick the
@@ -1445,10 +1502,12 @@ def main():
         ce = measure_config(head, ce_args, torch, device, link, min(3, args.steps), 2)  # staging buffers are allocated in the first calls
         records[head]["copy_engine"] = {k: ce[k] for k in (
             "d2h_GBps", "h2d_GBps", "d2h_frac_of_link", "h2d_frac_of_link", "path_taken", "steps")}
+    args.with_fragmented = True
     for name in ("c0", "c2", "c3", "c4"):
         # c4's latency percentiles want repetitions: 20 bursts of its 64 requests
         records[name] = measure_config(name, args, torch, device, link,
                                        20 if name == "c4" else args.other_steps, 1)
+    records["c3_fragmented"] = records["c3"].pop("fragmented_record")
     rec = records[head]
     out.update(value=rec["value"], ms_per_step=rec["ms_per_step"],
                d2h_GBps=rec["d2h_GBps"], h2d_GBps=rec["h2d_GBps"],
@@ -1465,7 +1524,7 @@ def main():
     if not args.no_cpu_baseline:
         torch.cuda.empty_cache()
         for name, r in records.items():
-            r["cpu_baseline"] = cpu_baseline(name, budget_s=5.0)
+            r["cpu_baseline"] = cpu_baseline("c3f" if name == "c3_fragmented" else name, budget_s=5.0)
         out["cpu_baseline"] = records[head]["cpu_baseline"]
     out["configs"] = records
     print(json.dumps(out))

@@ -174,7 +174,8 @@ class Stats(Structure):
                 ("kernel_launches", c_uint64), ("dma_copies", c_uint64),
                 ("staging_bytes_device", c_uint64), ("staging_bytes_host", c_uint64),
                 ("confined_launches", c_uint64), ("safety_net_ranges", c_uint64),
-                ("staged_batches", c_uint64)]
+                ("staged_batches", c_uint64), ("gathered_batches", c_uint64),
+                ("gather_busy_us", c_uint64)]
 
 
 class LaunchPolicy(Structure):
@@ -202,7 +203,11 @@ class LaunchPolicy(Structure):
                 ("model_kernel_h2d_mbps", c_int32), ("model_dma_ns", c_int32),
                 ("model_compaction_gbps", c_int32), ("model_host_pass_mbps", c_int32),
                 ("model_launch_ns", c_int32), ("model_prefer_ce_pct", c_int32),
-                ("d2h_lane_runs", c_int32), ("reserved", c_int32 * 5)]
+                ("d2h_lane_runs", c_int32),
+                ("staged_gather", c_int32), ("gather_threads", c_int32), ("gather_ring", c_int32),
+                ("gather_first_by_kernel", c_int32), ("model_gather_thread_mbps", c_int32),
+                ("model_seed", c_int32), ("model_seeded", c_int32),
+                ("reserved", c_int32 * 5)]
 
 
 # name -> (restype, argtypes); the complete export list of include/fkv_transfer.h
@@ -309,8 +314,8 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.fkv_abi_version() != 2:
-        raise ImportError(f"{LIB_PATH}: ABI version {lib.fkv_abi_version()} != 2")
+    if lib.fkv_abi_version() != 3:
+        raise ImportError(f"{LIB_PATH}: ABI version {lib.fkv_abi_version()} != 3")
     _lib = lib
     return lib
 

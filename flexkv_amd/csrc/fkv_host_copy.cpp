@@ -1,6 +1,8 @@
 #include "fkv_host_copy.h"
 
 #include <algorithm>
+#include <atomic>
+#include <chrono>
 #include <condition_variable>
 #include <cstring>
 #include <functional>
@@ -70,90 +72,94 @@ __attribute__((target("avx2"))) void copy_avx2(uint8_t *dst, const uint8_t *src,
 }
 #endif
 
-// Helper threads that belong to one calling thread.  A call to run() hands
-// every helper a [begin, end) share, the caller works on its own share, then
-// waits for the helpers.  Shares are published under the mutex with a
-// generation counter, so a helper never sees a half-written job.
-class RowCopyCrew {
-public:
-  explicit RowCopyCrew(int helpers) {
+} // namespace
+
+// A call to run() hands every helper a [begin, end) share, the caller works on its
+// own share, then waits for the helpers.  Shares are published under the mutex with
+// a generation counter, so a helper never sees a half-written job.
+struct HostCrew::Impl {
+  explicit Impl(int helpers) {
+    ranges.resize(helpers);
     for (int i = 0; i < helpers; ++i)
-      threads_.emplace_back([this, i] { loop(i); });
-    ranges_.resize(helpers);
+      threads.emplace_back([this, i] { loop(i); });
   }
-  ~RowCopyCrew() {
+  ~Impl() {
     {
-      std::lock_guard<std::mutex> lk(mu_);
-      quit_ = true;
+      std::lock_guard<std::mutex> lk(mu);
+      quit = true;
     }
-    wake_.notify_all();
-    for (auto &t : threads_)
+    wake.notify_all();
+    for (auto &t : threads)
       if (t.joinable())
         t.join();
   }
-  int helpers() const { return (int)threads_.size(); }
-
-  void run(int total, const std::function<void(int, int)> &body) {
-    const int parts = helpers() + 1;
-    const int share = (total + parts - 1) / parts;
-    {
-      std::lock_guard<std::mutex> lk(mu_);
-      body_ = &body;
-      pending_ = 0;
-      for (int h = 0; h < helpers(); ++h) {
-        int b = std::min(total, (h + 1) * share);
-        int e = std::min(total, b + share);
-        ranges_[h] = {b, e};
-        if (b < e)
-          ++pending_;
-      }
-      ++generation_;
-    }
-    wake_.notify_all();
-    body(0, std::min(share, total));
-    std::unique_lock<std::mutex> lk(mu_);
-    done_.wait(lk, [this] { return pending_ == 0; });
-    body_ = nullptr;
-  }
-
-private:
   void loop(int idx) {
     uint64_t seen = 0;
     for (;;) {
       const std::function<void(int, int)> *fn = nullptr;
       std::pair<int, int> r;
       {
-        std::unique_lock<std::mutex> lk(mu_);
-        wake_.wait(lk, [&] { return quit_ || generation_ != seen; });
-        if (quit_)
+        std::unique_lock<std::mutex> lk(mu);
+        wake.wait(lk, [&] { return quit || generation != seen; });
+        if (quit)
           return;
-        seen = generation_;
-        fn = body_;
-        r = ranges_[idx];
+        seen = generation;
+        fn = body;
+        r = ranges[idx];
       }
       if (r.first < r.second) {
         (*fn)(r.first, r.second);
-        std::lock_guard<std::mutex> lk(mu_);
-        if (--pending_ == 0)
-          done_.notify_one();
+        std::lock_guard<std::mutex> lk(mu);
+        if (--pending == 0)
+          done.notify_one();
       }
     }
   }
 
-  std::vector<std::thread> threads_;
-  std::vector<std::pair<int, int>> ranges_;
-  std::mutex mu_;
-  std::condition_variable wake_, done_;
-  const std::function<void(int, int)> *body_ = nullptr;
-  uint64_t generation_ = 0;
-  int pending_ = 0;
-  bool quit_ = false;
+  std::vector<std::thread> threads;
+  std::vector<std::pair<int, int>> ranges;
+  std::mutex mu;
+  std::condition_variable wake, done;
+  const std::function<void(int, int)> *body = nullptr;
+  uint64_t generation = 0;
+  int pending = 0;
+  bool quit = false;
 };
 
-RowCopyCrew &crew_for_thread(int threads) {
+HostCrew::HostCrew(int helpers) : impl_(new Impl(std::max(0, helpers))) {}
+HostCrew::~HostCrew() { delete impl_; }
+int HostCrew::helpers() const { return (int)impl_->threads.size(); }
+
+void HostCrew::run(int total, const std::function<void(int, int)> &body) {
+  Impl &m = *impl_;
+  const int parts = helpers() + 1;
+  const int share = (total + parts - 1) / parts;
+  {
+    std::lock_guard<std::mutex> lk(m.mu);
+    m.body = &body;
+    m.pending = 0;
+    for (int h = 0; h < helpers(); ++h) {
+      int b = std::min(total, (h + 1) * share);
+      int e = std::min(total, b + share);
+      m.ranges[h] = {b, e};
+      if (b < e)
+        ++m.pending;
+    }
+    ++m.generation;
+  }
+  m.wake.notify_all();
+  body(0, std::min(share, total));
+  std::unique_lock<std::mutex> lk(m.mu);
+  m.done.wait(lk, [&m] { return m.pending == 0; });
+  m.body = nullptr;
+}
+
+namespace {
+
+HostCrew &crew_for_thread(int threads) {
   // Sized on first use by this thread, like the reference's thread_local pool
   // (csrc/ce_transfer.cu:412-418).
-  thread_local RowCopyCrew crew(std::max(0, threads - 1));
+  thread_local HostCrew crew(std::max(0, threads - 1));
   return crew;
 }
 
@@ -230,11 +236,38 @@ void host_rows_copy(uint8_t *staging, uint8_t *row_base, const int64_t *cpu_ids,
     body(0, num_blocks);
     return;
   }
-  RowCopyCrew &crew = crew_for_thread(threads);
+  HostCrew &crew = crew_for_thread(threads);
   if (crew.helpers() == 0)
     body(0, num_blocks);
   else
     crew.run(num_blocks, body);
+}
+
+uint64_t host_gather_rows(HostCrew &crew, uint8_t *dense, const uint8_t *row0, const int64_t *ids,
+                          int num_rows, int64_t row_stride, int outer, int64_t outer_stride,
+                          int inner, int64_t inner_stride, int64_t piece_bytes) {
+  std::atomic<uint64_t> busy_ns{0};
+  const std::function<void(int, int)> body = [&](int begin, int end) {
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int pos = begin; pos < end; ++pos) {
+      const uint8_t *src = row0 + ids[pos] * row_stride;
+      uint8_t *dst = dense + (int64_t)pos * outer * inner * piece_bytes;
+      for (int o = 0; o < outer; ++o)
+        for (int i = 0; i < inner; ++i, dst += piece_bytes)
+          host_copy_bytes(dst, src + (int64_t)o * outer_stride + (int64_t)i * inner_stride,
+                          (size_t)piece_bytes, true);
+    }
+    host_copy_fence(true);
+    busy_ns.fetch_add((uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(
+                          std::chrono::steady_clock::now() - t0)
+                          .count(),
+                      std::memory_order_relaxed);
+  };
+  if (crew.helpers() == 0 || num_rows < 2 * (crew.helpers() + 1))
+    body(0, num_rows);
+  else
+    crew.run(num_rows, body);
+  return busy_ns.load(std::memory_order_relaxed);
 }
 
 } // namespace fkv

@@ -64,7 +64,7 @@ constexpr unsigned kTimingEventNoFence = hipEventDisableSystemFence;
 struct Stats {
   std::atomic<uint64_t> calls{0}, bytes_h2d{0}, bytes_d2h{0}, kernel_launches{0},
       dma_copies{0}, staging_bytes_device{0}, staging_bytes_host{0}, confined_launches{0},
-      staged_batches{0};
+      staged_batches{0}, gathered_batches{0}, gather_busy_ns{0};
 };
 Stats &stats();
 
@@ -188,6 +188,9 @@ fkv_launch_policy policy_of(int device);
 // The same without the probe: the table of a device that has none yet is the one
 // of a device of unknown shape (nothing is confined).
 fkv_launch_policy policy_peek(int device);
+// `p` with every field brought into its allowed range (what fkv_launch_policy_set
+// would store), for callers that bring a table of their own.
+fkv_launch_policy policy_sanitized(const fkv_launch_policy &p);
 // Widest vector width (bytes) that divides every value in `vals`.
 int common_vector_width(const uint64_t *vals, int n);
 
@@ -275,8 +278,25 @@ struct StagedRing {
   std::vector<hipEvent_t> copied, freed; // per buffer: copies landed / scatter done
   std::vector<bool> used;
   int next = 0;
+  int idle_calls = 0;   // restores of the group in a row that did not use the buffers
+  bool touched = false; // used by the restore that is being set up
   void release(); // frees everything; the device must have finished with the buffers
 };
+// Pinned host buffers of one (layer group, GPU) for restores whose rows host threads
+// gather first; they outlive the calls like the staging buffers.
+struct GatherRing {
+  std::vector<uint8_t *> buf;
+  size_t cap = 0;
+  std::vector<hipEvent_t> read; // per buffer: the copy engine has read it
+  std::vector<bool> used;
+  int next = 0;
+  int idle_calls = 0;
+  bool touched = false;
+  void release(); // the device must have finished with the buffers
+};
+class HostCrew;
+// Routes of a layerwise batch other than the kernel path.
+enum : int { kRouteKernel = 0, kRouteRuns = 1, kRouteGathered = 2 };
 // What one call derives for one (layer group, GPU).
 struct StagedPlan {
   struct Seg {
@@ -285,6 +305,11 @@ struct StagedPlan {
     int32_t row0;     // staging row of the first
   };
   bool usable = false;
+  int route = kRouteKernel; // kRouteRuns: a copy command per run of host blocks; kRouteGathered:
+                            // host threads gather the rows, one copy command per batch
+  bool first_by_kernel = false;  // kRouteGathered: the first batch of the restore goes the kernel way
+  std::vector<int64_t> host_ids; // kRouteGathered: the call's host block ids (the launching
+                                 // thread may outlive the caller's list)
   std::vector<Seg> segs;
   int32_t total_rows = 0;
   int kind = 0; // chunks of a host block that are adjacent: 0 all of a batch, 1 K and V of a layer, 2 none
@@ -300,7 +325,20 @@ struct StagedPlan {
 // sizes the ring and uploads the tables on `scatter_stream`.  FKV_OK with
 // out->usable == false: use the kernel path.
 int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &ring,
-                      hipStream_t scatter_stream, StagedPlan *out);
+                      GatherRing &pinned, hipStream_t scatter_stream, StagedPlan *out);
+// The choice alone (no device): kRouteKernel, kRouteRuns (fills `segs` and `total_rows`)
+// or kRouteGathered.
+int staged_route(const int64_t *cpu_ids, int num_blocks, int64_t row_bytes, int pieces,
+                 const fkv_launch_policy &pol, std::vector<StagedPlan::Seg> *segs,
+                 int64_t *total_rows);
+// Host threads a gathered restore uses under `pol` on this machine (>= 1).
+int gather_threads_of(const fkv_launch_policy &pol);
+// Layers [l0, l0 + nl) of a kRouteGathered plan: gathers the rows on the calling thread
+// and `crew` (blocks for that long, and before that until a pinned buffer is free),
+// then enqueues one copy and the scatter.
+int gathered_launch(const StagedPlan &sp, StagedRing &ring, GatherRing &pinned, HostCrew &crew,
+                    const KernelPlan &kp, int l0, int nl, hipStream_t dma_stream,
+                    hipStream_t scatter_stream);
 // Layers [l0, l0 + nl) of the plan: copies on `dma_stream`, scatter on `scatter_stream`.
 int staged_launch(const StagedPlan &sp, StagedRing &ring, const KernelPlan &kp, int l0, int nl,
                   hipStream_t dma_stream, hipStream_t scatter_stream);

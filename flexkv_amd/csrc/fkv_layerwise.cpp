@@ -26,7 +26,14 @@
 // go to the device once per call and GPU; each (batch, group) is then a single
 // kernel launch.
 //
+// A restore whose host rows are gathered by host threads first (see
+// fkv_staged_restore.cpp) cannot enqueue everything at once: the copy of a batch is
+// enqueued when its rows have been gathered.  Such a restore is launched batch by
+// batch from a thread of its own, and everything that looks at a batch event first
+// waits until that event has been recorded.
+//
 // The transfer streams keep the default priority.
+#include "fkv_host_copy.h"
 #include "fkv_internal.h"
 #include "fkv_poll.h"
 
@@ -34,9 +41,11 @@
 #include <unistd.h>
 
 #include <atomic>
+#include <condition_variable>
 #include <cstring>
 #include <map>
 #include <memory>
+#include <mutex>
 #include <thread>
 
 namespace {
@@ -157,6 +166,18 @@ struct fkv_layerwise {
   // (lane, GPU), kept from call to call.
   std::vector<hipStream_t> dma_streams;
   std::map<std::pair<int, int>, fkv::StagedRing> rings;
+  // Restores whose rows host threads gather first: pinned buffers by (lane, GPU), the
+  // helper threads, and the thread that launches such a restore batch by batch.
+  std::map<std::pair<int, int>, fkv::GatherRing> pinned_rings;
+  std::unique_ptr<fkv::HostCrew> crew;
+  std::thread feeder;
+  std::vector<Lane> feed_lanes; // what the feeder works on
+  std::mutex feed_mu;
+  std::condition_variable feed_cv;
+  std::atomic<int> recorded{0};  // batches whose events have been recorded (written under feed_mu)
+  bool feed_failed = false;      // the launching thread gave up; the batches from `recorded` on never land
+  int feed_rc = 0;
+  std::string feed_error;
   fkv_ce_config ce{};
 
   std::vector<int32_t> eventfds; // [num_counters][tp_size][num_layers]
@@ -202,6 +223,12 @@ struct fkv_layerwise {
     const int status = fkv::poll_batches_in_order(
         batches.size(), num_gpus, (int)hipSuccess, (int)hipErrorNotReady,
         [this](size_t b, int g) {
+          // an event that has not been recorded yet reads as complete
+          if ((int)b >= recorded.load(std::memory_order_acquire)) {
+            std::lock_guard<std::mutex> lk(feed_mu);
+            if ((int)b >= recorded.load(std::memory_order_relaxed))
+              return (int)(feed_failed ? hipErrorLaunchFailure : hipErrorNotReady);
+          }
           (void)hipSetDevice(device_ids[g]);
           const hipError_t e = hipEventQuery(batches[b]->done[g]);
           if (e != hipSuccess)
@@ -217,10 +244,33 @@ struct fkv_layerwise {
     }
   }
 
+  void publish_recorded(int n) {
+    {
+      std::lock_guard<std::mutex> lk(feed_mu);
+      recorded.store(n, std::memory_order_release);
+    }
+    feed_cv.notify_all();
+  }
+  // Blocks until the event of batch `b` has been recorded; false when it never will be.
+  bool wait_recorded(int b) {
+    if (b < recorded.load(std::memory_order_acquire))
+      return true;
+    std::unique_lock<std::mutex> lk(feed_mu);
+    feed_cv.wait(lk, [&] { return feed_failed || b < recorded.load(std::memory_order_relaxed); });
+    return b < recorded.load(std::memory_order_relaxed);
+  }
+  // The launching thread ends by itself: it waits for nothing but copies that are
+  // already enqueued.
+  void join_feeder() {
+    if (feeder.joinable())
+      feeder.join();
+  }
+
   // Waits for the poller: it ends by itself once every batch has been announced or
   // a device error has been seen.  Should the streams drain and the poller still
   // run (a failed stream leaves its events unready for good), it is told to stop.
   void join_poller() {
+    join_feeder();
     if (!poller.joinable())
       return;
     fkv::DeviceGuard restore(-1);
@@ -243,6 +293,12 @@ struct fkv_layerwise {
   // The error of the previous restore, if any, as a status of the current call.
   int take_restore_error(const char *where) {
     const int e = restore_error.exchange(0);
+    if (feed_failed) { // only read after the launching thread has been joined
+      feed_failed = false;
+      return fkv::fail(feed_rc ? feed_rc : FKV_ERR_RUNTIME,
+                       "%s: the previous layerwise restore failed while it was launched: %s", where,
+                       feed_error.c_str());
+    }
     if (e == 0)
       return FKV_OK;
     return fkv::fail(FKV_ERR_RUNTIME, "%s: the previous layerwise restore failed on the device: %s",
@@ -252,6 +308,7 @@ struct fkv_layerwise {
   // Ends the notification machinery of the previous transfer and frees its
   // events.  All work of that transfer has completed when this returns.
   void retire_previous() {
+    join_feeder();
     join_poller();
     fkv::DeviceGuard restore(-1);
     for (int g = 0; g < num_gpus; ++g) {
@@ -354,6 +411,102 @@ fkv_transfer_desc describe(const fkv_layerwise *g, const Lane &lane, int gpu, in
   d.sync = 0;
   d.ce = g->ce;
   return d;
+}
+
+// Enqueues every batch of the restore that is being set up, in order, records the batch
+// events and hands the plan memory back; `rc` is the status of the set-up so far (a
+// failed set-up enqueues nothing).  Runs on the calling thread, or on the group's
+// launching thread where host threads gather rows (`on_feeder`; `c` is not used there).
+int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, bool direct,
+                   const fkv_layerwise_call *c, bool on_feeder, int rc) {
+  using namespace fkv;
+  DeviceGuard restore(-1);
+  const int num_batches = (int)g->batches.size();
+  for (int b = 0; b < num_batches && rc == FKV_OK; ++b) {
+    fkv_layerwise::Batch &batch = *g->batches[b];
+    for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
+      (void)hipSetDevice(g->device_ids[i]);
+      if (direct) {
+        // the members of one batch go out together: up to kCopyMaxJobs per launch
+        const KernelPlan *plans[kCopyMaxJobs];
+        int first[kCopyMaxJobs], count[kCopyMaxJobs];
+        // items of lanes that go through the copy engines first, the rest by kernel
+        std::vector<const Item *> by_kernel;
+        for (const Item &it : batch.items) {
+          Lane &lane = lanes[it.lane];
+          const StagedPlan *sp =
+              !lane.staged.empty() && lane.staged[i].usable ? &lane.staged[i] : nullptr;
+          if (rc != FKV_OK || !sp || (b == 0 && sp->first_by_kernel))
+            by_kernel.push_back(&it);
+          else if (sp->route == kRouteGathered)
+            rc = gathered_launch(*sp, g->rings[{it.lane, i}], g->pinned_rings[{it.lane, i}],
+                                 *g->crew, lane.plans[i], it.start_layer, it.layers,
+                                 g->dma_streams[i], g->streams[i]);
+          else
+            rc = staged_launch(*sp, g->rings[{it.lane, i}], lane.plans[i], it.start_layer,
+                               it.layers, g->dma_streams[i], g->streams[i]);
+        }
+        for (size_t k = 0; k < by_kernel.size() && rc == FKV_OK; k += kCopyMaxJobs) {
+          const int n = (int)std::min<size_t>(kCopyMaxJobs, by_kernel.size() - k);
+          for (int j = 0; j < n; ++j) {
+            const Item &it = *by_kernel[k + j];
+            plans[j] = &lanes[it.lane].plans[i];
+            first[j] = it.start_layer;
+            count[j] = it.layers;
+          }
+          rc = kernel_plans_launch(plans, first, count, n, g->streams[i]);
+        }
+        for (size_t k = 0; k < batch.items.size() && rc == FKV_OK; ++k) {
+          const Item &it = batch.items[k];
+          const Lane &lane = lanes[it.lane];
+          stats().calls.fetch_add(1, std::memory_order_relaxed);
+          stats().bytes_h2d.fetch_add((uint64_t)lane.num_blocks * it.layers * lane.kv_dim *
+                                          (uint64_t)lane.src->chunk_sizes[i],
+                                      std::memory_order_relaxed);
+        }
+      }
+      for (size_t k = 0; !direct && k < batch.items.size() && rc == FKV_OK; ++k) {
+        const Item &it = batch.items[k];
+        fkv_transfer_desc d = describe(g, lanes[it.lane], i, it.start_layer, it.layers, *c);
+        rc = fkv_transfer_kv_blocks(&d, g->streams[i]);
+        (void)hipSetDevice(g->device_ids[i]);
+      }
+      if (rc != FKV_OK)
+        break;
+      hipError_t e = hipEventRecord(batch.done[i], g->streams[i]);
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        rc = fail(FKV_ERR_RUNTIME, "layerwise_transfer failed on GPU %d: %s", i,
+                  hipGetErrorString(e));
+      }
+    }
+    if (rc == FKV_OK)
+      g->publish_recorded(b + 1);
+  }
+  std::string saved_error = fkv_last_error();
+  for (Lane &lane : lanes)
+    for (int i = 0; i < (int)lane.plans.size(); ++i) {
+      (void)hipSetDevice(g->device_ids[i]);
+      kernel_plan_release(&lane.plans[i], g->streams[i]);
+      if (i < (int)lane.staged.size())
+        staged_plan_release(&lane.staged[i], g->streams[i]);
+    }
+  if (rc != FKV_OK) {
+    // Drain what was enqueued; nothing more of this call is announced.
+    for (int i = 0; i < g->num_gpus; ++i) {
+      (void)hipSetDevice(g->device_ids[i]);
+      if (i < (int)g->dma_streams.size() && g->dma_streams[i])
+        (void)hipStreamSynchronize(g->dma_streams[i]);
+      (void)hipStreamSynchronize(g->streams[i]);
+    }
+    if (!on_feeder) // on the launching thread consumers may be reading the table
+      g->layer_batch.assign(g->num_layers, -1);
+    (void)hipSetDevice(restore.device());
+    (void)hipGetLastError();
+    return fail(rc, "%s", saved_error.c_str());
+  }
+  (void)hipSetDevice(restore.device());
+  return FKV_OK;
 }
 
 } // namespace
@@ -522,6 +675,8 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
 
   g->retire_previous();
   FKV_TRY(g->take_restore_error("fkv_layerwise_transfer"));
+  g->recorded.store(0, std::memory_order_relaxed);
+  g->feed_lanes.clear();
   g->counter_id = c.counter_id;
   Range range("fkv layerwise%s H2D %d blocks, %d sidecar blocks", g->multi_group ? " multi-group" : "",
               c.num_blocks, c.swa_num_blocks);
@@ -688,7 +843,8 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
           lane.staged.resize(g->num_gpus);
           const int lane_index = (int)(&lane - lanes.data());
           rc = staged_plan_build(d, g->multi_group ? 1 : c.layer_granularity,
-                                 g->rings[{lane_index, i}], g->streams[i], &lane.staged[i]);
+                                 g->rings[{lane_index, i}], g->pinned_rings[{lane_index, i}],
+                                 g->streams[i], &lane.staged[i]);
           if (rc == FKV_OK && lane.staged[i].usable && !g->dma_streams[i]) {
             hipError_t e = hipStreamCreateWithFlags(&g->dma_streams[i], hipStreamNonBlocking);
             if (e != hipSuccess) {
@@ -700,80 +856,59 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
         }
       }
     }
-  for (int b = 0; b < num_batches && rc == FKV_OK; ++b) {
-    fkv_layerwise::Batch &batch = *g->batches[b];
-    for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
-      (void)hipSetDevice(g->device_ids[i]);
-      if (direct) {
-        // the members of one batch go out together: up to kCopyMaxJobs per launch
-        const KernelPlan *plans[kCopyMaxJobs];
-        int first[kCopyMaxJobs], count[kCopyMaxJobs];
-        // items of lanes that go through the copy engines first, the rest by kernel
-        std::vector<const Item *> by_kernel;
-        for (const Item &it : batch.items) {
-          Lane &lane = lanes[it.lane];
-          if (rc == FKV_OK && !lane.staged.empty() && lane.staged[i].usable)
-            rc = staged_launch(lane.staged[i], g->rings[{it.lane, i}], lane.plans[i],
-                               it.start_layer, it.layers, g->dma_streams[i], g->streams[i]);
-          else
-            by_kernel.push_back(&it);
-        }
-        for (size_t k = 0; k < by_kernel.size() && rc == FKV_OK; k += kCopyMaxJobs) {
-          const int n = (int)std::min<size_t>(kCopyMaxJobs, by_kernel.size() - k);
-          for (int j = 0; j < n; ++j) {
-            const Item &it = *by_kernel[k + j];
-            plans[j] = &lanes[it.lane].plans[i];
-            first[j] = it.start_layer;
-            count[j] = it.layers;
-          }
-          rc = kernel_plans_launch(plans, first, count, n, g->streams[i]);
-        }
-        for (size_t k = 0; k < batch.items.size() && rc == FKV_OK; ++k) {
-          const Item &it = batch.items[k];
-          const Lane &lane = lanes[it.lane];
-          stats().calls.fetch_add(1, std::memory_order_relaxed);
-          stats().bytes_h2d.fetch_add((uint64_t)lane.num_blocks * it.layers * lane.kv_dim *
-                                          (uint64_t)lane.src->chunk_sizes[i],
-                                      std::memory_order_relaxed);
+  // Staging memory that several restores in a row had no use for goes back (a group
+  // with many lanes would otherwise hold buffers for every route it ever took).
+  constexpr int kRingIdleCalls = 8;
+  for (auto &r : g->rings) {
+    if (!r.second.touched && !r.second.buf.empty() && ++r.second.idle_calls >= kRingIdleCalls) {
+      (void)hipSetDevice(g->device_ids[r.first.second]);
+      r.second.release();
+    }
+    r.second.touched = false;
+  }
+  for (auto &r : g->pinned_rings) {
+    if (!r.second.touched && !r.second.buf.empty() && ++r.second.idle_calls >= kRingIdleCalls) {
+      (void)hipSetDevice(g->device_ids[r.first.second]);
+      r.second.release();
+    }
+    r.second.touched = false;
+  }
+  // Rows gathered by host threads: the restore is launched from a thread of its own.
+  bool gathered = false;
+  for (const Lane &lane : lanes)
+    for (const StagedPlan &sp : lane.staged)
+      gathered = gathered || (sp.usable && sp.route == kRouteGathered);
+  if (rc == FKV_OK && gathered) {
+    const int helpers = gather_threads_of(policy_of(g->device_ids[0])) - 1;
+    if (!g->crew || g->crew->helpers() != helpers)
+      g->crew = std::make_unique<HostCrew>(helpers);
+    g->feed_lanes = std::move(lanes);
+    g->feeder = std::thread([g] {
+      const int frc = launch_batches(g, g->feed_lanes, true, nullptr, true, FKV_OK);
+      {
+        std::lock_guard<std::mutex> lk(g->feed_mu);
+        if (frc != FKV_OK) {
+          g->feed_failed = true;
+          g->feed_rc = frc;
+          g->feed_error = fkv_last_error();
         }
       }
-      for (size_t k = 0; !direct && k < batch.items.size() && rc == FKV_OK; ++k) {
-        const Item &it = batch.items[k];
-        fkv_transfer_desc d = describe(g, lanes[it.lane], i, it.start_layer, it.layers, c);
-        rc = fkv_transfer_kv_blocks(&d, g->streams[i]);
-        (void)hipSetDevice(g->device_ids[i]);
-      }
-      if (rc != FKV_OK)
-        break;
-      hipError_t e = hipEventRecord(batch.done[i], g->streams[i]);
-      if (e != hipSuccess) {
-        (void)hipGetLastError();
-        rc = fail(FKV_ERR_RUNTIME, "layerwise_transfer failed on GPU %d: %s", i,
-                  hipGetErrorString(e));
-      }
+      g->feed_cv.notify_all();
+    });
+  } else {
+    const int lrc = launch_batches(g, lanes, direct, &c, false, rc);
+    if (lrc != FKV_OK) {
+      (void)hipSetDevice(restore.device());
+      return lrc;
     }
   }
-  std::string saved_error = fkv_last_error();
-  for (Lane &lane : lanes)
-    for (int i = 0; i < (int)lane.plans.size(); ++i) {
-      (void)hipSetDevice(g->device_ids[i]);
-      kernel_plan_release(&lane.plans[i], g->streams[i]);
-      if (i < (int)lane.staged.size())
-        staged_plan_release(&lane.staged[i], g->streams[i]);
-    }
-  if (rc != FKV_OK) {
-    // Drain what was enqueued; nothing of this call is announced.
-    for (int i = 0; i < g->num_gpus; ++i) {
-      (void)hipSetDevice(g->device_ids[i]);
-      if (i < (int)g->dma_streams.size() && g->dma_streams[i])
-        (void)hipStreamSynchronize(g->dma_streams[i]);
-      (void)hipStreamSynchronize(g->streams[i]);
-    }
-    g->layer_batch.assign(g->num_layers, -1);
+  // The launching thread gave up: nothing of the call is announced from here on.
+  auto launch_failure = [&]() {
+    g->join_feeder();
+    g->feed_failed = false;
     (void)hipSetDevice(restore.device());
-    (void)hipGetLastError();
-    return fail(rc, "%s", saved_error.c_str());
-  }
+    return fail(g->feed_rc ? g->feed_rc : FKV_ERR_RUNTIME, "%s", g->feed_error.c_str());
+  };
 
   if (c.notify_mode == FKV_NOTIFY_POLLING) {
     g->poller_stop.store(false, std::memory_order_release);
@@ -784,6 +919,8 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
   } else {
     // announce every batch as soon as all GPUs have finished it, in order
     for (int b = 0; b < num_batches; ++b) {
+      if (!g->wait_recorded(b))
+        return launch_failure();
       for (int i = 0; i < g->num_gpus; ++i) {
         (void)hipSetDevice(g->device_ids[i]);
         hipError_t e = hipEventSynchronize(g->batches[b]->done[i]);
@@ -796,6 +933,7 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
       }
       g->notify(*g->batches[b]);
     }
+    g->join_feeder();
     for (int i = 0; i < g->num_gpus; ++i) { // csrc/layerwise.cpp:1249-1256, 1634-1642
       (void)hipSetDevice(g->device_ids[i]);
       hipError_t e = hipStreamSynchronize(g->streams[i]);
@@ -884,6 +1022,11 @@ int fkv_layerwise_wait_layer(fkv_layerwise *g, int32_t gpu_index, int32_t layer,
       return FKV_OK;
     return fail(FKV_ERR_INVALID_ARG, "layer %d was not part of the last transfer", layer);
   }
+  // A batch whose rows are still being gathered has no event on its stream yet, and a
+  // wait on an event that was never recorded returns at once: wait for the record first.
+  if (!g->wait_recorded(b))
+    return fail(FKV_ERR_RUNTIME, "layer %d will not land: the restore failed while it was launched",
+                layer);
   FKV_HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(consumer_stream),
                                  g->batches[b]->done[gpu_index], 0));
   return FKV_OK;
@@ -911,6 +1054,9 @@ int fkv_layerwise_batch_times_ms(fkv_layerwise *g, float *out_ms, int32_t capaci
   if (!g || !num_batches)
     return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_batch_times_ms: null argument");
   *num_batches = (int32_t)g->batches.size();
+  g->join_feeder();
+  if (g->recorded.load(std::memory_order_acquire) < (int)g->batches.size())
+    return fail(FKV_ERR_RUNTIME, "fkv_layerwise_batch_times_ms: the restore was not launched completely");
   DeviceGuard restore(g->device_ids[0]);
   for (int b = 0; b < (int)g->batches.size() && b < capacity; ++b)
     FKV_HIP_TRY(hipEventElapsedTime(&out_ms[b], g->started, g->batches[b]->done[0]));
@@ -926,6 +1072,11 @@ void fkv_layerwise_destroy(fkv_layerwise *g) {
     (void)hipSetDevice(g->device_ids[ring.first.second]);
     ring.second.release();
   }
+  for (auto &ring : g->pinned_rings) {
+    (void)hipSetDevice(g->device_ids[ring.first.second]);
+    ring.second.release();
+  }
+  g->crew.reset();
   for (int i = 0; i < g->num_gpus; ++i) {
     (void)hipSetDevice(g->device_ids[i]);
     if (i < (int)g->dma_streams.size() && g->dma_streams[i])

@@ -36,6 +36,9 @@ const EnvField kEnv[] = {
     FKV_FIELD("FKV_CE_STAGING_MB", ce_staging_mb),
     FKV_FIELD("FKV_CE_TWO_STREAMS", ce_two_streams),
     FKV_FIELD("FKV_D2H_LANE_RUNS", d2h_lane_runs),
+    FKV_FIELD("FKV_STAGED_GATHER", staged_gather),
+    FKV_FIELD("FKV_GATHER_THREADS", gather_threads),
+    FKV_FIELD("FKV_MODEL_SEED", model_seed),
 };
 #undef FKV_FIELD
 
@@ -121,6 +124,13 @@ void sanitize(fkv_launch_policy &p, const fkv_launch_policy &derived) {
   p.model_launch_ns = clampi(p.model_launch_ns, 0, 10000000);
   p.model_prefer_ce_pct = clampi(p.model_prefer_ce_pct, 1, 1000);
   p.d2h_lane_runs = clampi(p.d2h_lane_runs, 0, 2);
+  p.staged_gather = clampi(p.staged_gather, 0, 2);
+  p.gather_threads = clampi(p.gather_threads, 1, 64);
+  p.gather_ring = clampi(p.gather_ring, 2, 8);
+  p.gather_first_by_kernel = p.gather_first_by_kernel != 0;
+  p.model_gather_thread_mbps = clampi(p.model_gather_thread_mbps, 100, 10000000);
+  p.model_seed = p.model_seed != 0;
+  p.model_seeded = derived.model_seeded;
 }
 
 // The table of a device with the XCDs `present`, environment applied.
@@ -174,6 +184,19 @@ fkv_launch_policy defaults_for(uint32_t present) {
   p.model_launch_ns = 15000;
   p.model_prefer_ce_pct = 103;
   p.d2h_lane_runs = 1;
+  // Host gather of scattered rows (72 KiB each, 16-core host of an MI355X box): one thread
+  // 25-34 GB/s, four threads 79-96 GB/s, eight 120-125 GB/s; next to the copy engine reading
+  // the previous buffer four threads still gather 36 MiB in 0.31-0.41 ms (0.67 ms on the
+  // link), though once, in the first process on a fresh box, in 0.79 ms: six threads by
+  // default, for the same thread time in sum.  20 GB/s a thread is the figure the choice
+  // assumes.
+  p.staged_gather = 1;
+  p.gather_threads = 6;
+  p.gather_ring = 4;
+  p.gather_first_by_kernel = 1;
+  p.model_gather_thread_mbps = 20000;
+  p.model_seed = 1;
+  p.model_seeded = 0;
   for (const EnvField &f : kEnv) {
     const char *v = std::getenv(f.name);
     if (v && *v) // decimal, 0x.. or 0.. as written
@@ -213,6 +236,17 @@ fkv_launch_policy policy_of(int device) {
   if (!t.built)
     build(device, t);
   return t.current;
+}
+
+fkv_launch_policy policy_sanitized(const fkv_launch_policy &in) {
+  fkv_launch_policy p = in;
+  fkv_launch_policy shape = in; // keeps the caller's XCD fields: no device is asked
+  if (shape.xcd_present_mask == 0) {
+    shape.xcd_present_mask = 1u;
+    shape.xcd_count = 1;
+  }
+  sanitize(p, shape);
+  return p;
 }
 
 fkv_launch_policy policy_peek(int device) {

@@ -18,13 +18,28 @@
 // once the scatter that read it has finished (event).  Small holes between runs
 // are read along (their bytes cost less link time than one more command).
 //
+//
+// Where the host blocks are scattered (a host pool after some churn hands out ids
+// in no order), a command per run is too many.  Then host threads gather the rows
+// of a batch into a pinned buffer first and ONE copy command moves the batch:
+//     host rows --(host threads, streaming stores)--> pinned buffer
+//               --(one 2-D copy of one row)--> staging buffer in HBM --(scatter)--> blocks
+// The thread that launches the restore gathers batch b+1 (with its helpers) while
+// the engine copies batch b; four threads gather 36 MiB of 72 KiB rows in 0.3 ms
+// against 0.67 ms on the link.  This is the host->GPU half of SEGMENT_SCATTER
+// (gather_from_cpu + one DMA, csrc/ce_transfer.cu:585-641, 645-812) under the
+// per-layer loop of csrc/layerwise.cpp:1129-1257, pipelined instead of
+// synchronised per (layer, kv).
+//
 // Replaces, for restores with few runs, the per-layer kernel launches of
 // csrc/layerwise.cpp:1129-1257; related to SEGMENT_SCATTER of
 // csrc/ce_transfer.cu:645-812, which stages in host memory instead.
+#include "fkv_host_copy.h"
 #include "fkv_internal.h"
 
 #include <algorithm>
 #include <cstring>
+#include <thread>
 
 namespace fkv {
 
@@ -44,7 +59,46 @@ void StagedRing::release() {
   next = 0;
 }
 
+void GatherRing::release() {
+  for (uint8_t *b : buf)
+    if (b && hipHostFree(b) != hipSuccess)
+      (void)hipGetLastError();
+  for (hipEvent_t e : read)
+    if (e && hipEventDestroy(e) != hipSuccess)
+      (void)hipGetLastError();
+  buf.clear();
+  read.clear();
+  used.clear();
+  cap = 0;
+  next = 0;
+}
+
 namespace {
+
+int pinned_prepare(GatherRing &ring, int slots, size_t bytes) {
+  if ((int)ring.buf.size() == slots && ring.cap >= bytes)
+    return FKV_OK;
+  // Only called while nothing of an earlier restore is in flight.
+  ring.release();
+  ring.buf.assign(slots, nullptr);
+  ring.read.assign(slots, nullptr);
+  ring.used.assign(slots, false);
+  size_t cap = (bytes + (2u << 20) - 1) & ~(size_t)((2u << 20) - 1);
+  for (int k = 0; k < slots; ++k) {
+    hipError_t e = hipHostMalloc(reinterpret_cast<void **>(&ring.buf[k]), cap, hipHostMallocDefault);
+    if (e == hipSuccess)
+      e = hipEventCreateWithFlags(&ring.read[k], kBookkeepingEvent);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      ring.release();
+      return fail(FKV_ERR_RUNTIME, "gathered restore: cannot allocate %d pinned buffers of %zu MiB: %s",
+                  slots, cap >> 20, hipGetErrorString(e));
+    }
+  }
+  ring.cap = cap;
+  stats().staging_bytes_host.fetch_add((uint64_t)cap * slots, std::memory_order_relaxed);
+  return FKV_OK;
+}
 
 int ring_prepare(StagedRing &ring, int slots, size_t bytes) {
   if ((int)ring.buf.size() == slots && ring.cap >= bytes)
@@ -129,7 +183,7 @@ bool staged_layout(const int64_t *cpu_ids, int num_blocks, int64_t row_bytes, in
     return false;
   if (pol.staged_restore == 1) {
     // the copy commands of a batch against the batch's time on the link
-    const double batch_us = useful / (pol.link_gbps_estimate * 1e3);
+    const double batch_us = useful / (std::max(1, pol.link_gbps_estimate) * 1e3);
     if ((double)(nsegs * pieces) * pol.staged_copy_overhead_us >
         batch_us * pol.staged_overhead_pct / 100.0)
       return false;
@@ -157,6 +211,45 @@ bool staged_layout(const int64_t *cpu_ids, int num_blocks, int64_t row_bytes, in
   return true;
 }
 
+int gather_threads_of(const fkv_launch_policy &pol) {
+  const int cores = (int)std::thread::hardware_concurrency();
+  const int most = cores > 1 ? cores - 1 : 1;
+  return std::max(1, std::min(pol.gather_threads, most));
+}
+
+// Per piece a gathering thread pays a call, an alignment head and a fence on top of
+// the bytes; only matters for rows cut into many small pieces.
+constexpr double kGatherPieceNs = 50.0;
+
+int staged_route(const int64_t *cpu_ids, int num_blocks, int64_t row_bytes, int pieces,
+                 const fkv_launch_policy &pol, std::vector<StagedPlan::Seg> *segs,
+                 int64_t *total_rows) {
+  if (staged_layout(cpu_ids, num_blocks, row_bytes, pieces, pol, segs, total_rows))
+    return kRouteRuns;
+  segs->clear();
+  *total_rows = 0;
+  if (pol.staged_gather == 0 || num_blocks <= 0 || row_bytes <= 0 || pieces < 1)
+    return kRouteKernel;
+  const double bytes = (double)num_blocks * (double)row_bytes;
+  if (bytes > (double)((int64_t)pol.staged_max_mb << 20))
+    return kRouteKernel;
+  if (pol.staged_gather == 1) {
+    const double link_us = bytes / (double)std::max(1, pol.model_link_mbps); // B / (MB/s) = us
+    // the one copy command of a batch against the batch's time on the link
+    if ((double)pol.staged_copy_overhead_us > link_us * pol.staged_overhead_pct / 100.0)
+      return kRouteKernel;
+    // the gather of batch b+1 has to fit, with room, into the copy of batch b
+    const int threads = gather_threads_of(pol);
+    const double gather_us =
+        bytes / ((double)threads * (double)std::max(1, pol.model_gather_thread_mbps)) +
+        (double)num_blocks * pieces * kGatherPieceNs / 1e3 / threads;
+    if (gather_us > 0.8 * link_us)
+      return kRouteKernel;
+  }
+  *total_rows = num_blocks;
+  return kRouteGathered;
+}
+
 // Staging row of host block `id`: the last run whose first id is <= id.
 int64_t staged_row_of(const std::vector<StagedPlan::Seg> &segs, int64_t id) {
   size_t lo = 0, hi = segs.size();
@@ -171,12 +264,13 @@ int64_t staged_row_of(const std::vector<StagedPlan::Seg> &segs, int64_t id) {
 }
 
 int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &ring,
-                      hipStream_t scatter_stream, StagedPlan *out) {
+                      GatherRing &pinned, hipStream_t scatter_stream, StagedPlan *out) {
   *out = StagedPlan{};
   int device = 0;
   FKV_HIP_TRY(hipGetDevice(&device));
   const fkv_launch_policy pol = policy_of(device);
-  if (pol.staged_restore == 0 || d.num_blocks <= 0 || d.num_layers <= 0 || batch_layers < 1)
+  if ((pol.staged_restore == 0 && pol.staged_gather == 0) || d.num_blocks <= 0 ||
+      d.num_layers <= 0 || batch_layers < 1)
     return FKV_OK;
   const int nl = std::min(batch_layers, d.num_layers);
   const int lk = nl * d.kv_dim;
@@ -189,9 +283,11 @@ int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &
   const int64_t batch_row_bytes = (int64_t)lk * d.chunk_size; // of one block, all pieces
   const int pieces = out->kind == 0 ? 1 : out->kind == 1 ? nl : lk;
   int64_t total_rows = 0;
-  if (!staged_layout(d.cpu_block_ids, d.num_blocks, batch_row_bytes, pieces, pol, &out->segs,
-                     &total_rows))
+  out->route = staged_route(d.cpu_block_ids, d.num_blocks, batch_row_bytes, pieces, pol, &out->segs,
+                            &total_rows);
+  if (out->route == kRouteKernel)
     return FKV_OK;
+  const bool gathered = out->route == kRouteGathered;
   const int64_t slot_bytes = total_rows * batch_row_bytes;
   out->total_rows = (int32_t)total_rows;
   out->max_lk = lk;
@@ -204,46 +300,97 @@ int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &
   out->host0 = static_cast<const uint8_t *>(d.cpu_ptr) + d.cpu_startoff_inside_chunks;
   out->num_blocks = d.num_blocks;
 
-  if (ring_prepare(ring, pol.staged_ring, (size_t)slot_bytes) != FKV_OK) {
-    clear_error(); // no room for the staging buffers: the kernel path needs none
+  // Whatever the set-up lacks from here on (device or pinned memory, plan memory), the
+  // kernel path needs none of it: the restore goes that way and the call succeeds.
+  auto kernel_path_instead = [&]() {
+    clear_error();
+    out->route = kRouteKernel;
     return FKV_OK;
-  }
+  };
+  if (ring_prepare(ring, pol.staged_ring, (size_t)slot_bytes) != FKV_OK)
+    return kernel_path_instead();
+  if (gathered && pinned_prepare(pinned, pol.gather_ring, (size_t)slot_bytes) != FKV_OK)
+    return kernel_path_instead();
   const int slots = (int)ring.buf.size();
-  const size_t tab = (size_t)slots * lk * 8, rows_bytes = (size_t)d.num_blocks * 8;
+  const size_t tab = (size_t)slots * lk * 8, rows_bytes = gathered ? 0 : (size_t)d.num_blocks * 8;
   PlanSlot *slot = plan_acquire(device, tab + rows_bytes);
   if (!slot)
-    return FKV_ERR_RUNTIME;
+    return kernel_path_instead();
   uint8_t *h = plan_host(slot);
   uint64_t *bases = reinterpret_cast<uint64_t *>(h);
-  // staging layout of a batch: [piece][row][chunks of the piece]
+  // staging layout of a batch: runs [piece][row][chunks of the piece]; gathered
+  // [position][chunks of the batch]
   const int m = out->kind == 0 ? lk : out->kind == 1 ? d.kv_dim : 1; // chunks per piece (full batch)
   for (int k = 0; k < slots; ++k)
     for (int i = 0; i < lk; ++i) {
       // kind 0 has one piece whatever the batch length: chunk i of a row sits at i * chunk
       const uint64_t piece_off =
-          out->kind == 0 ? 0 : (uint64_t)(i / m) * (uint64_t)total_rows * (uint64_t)(m * d.chunk_size);
+          gathered || out->kind == 0
+              ? 0
+              : (uint64_t)(i / m) * (uint64_t)total_rows * (uint64_t)(m * d.chunk_size);
       bases[(size_t)k * lk + i] = (uint64_t)(uintptr_t)ring.buf[k] + piece_off +
-                                  (uint64_t)(i % m) * (uint64_t)d.chunk_size;
+                                  (uint64_t)(gathered ? i : i % m) * (uint64_t)d.chunk_size;
     }
-  int64_t *rows = reinterpret_cast<int64_t *>(h + tab);
-  for (int pos = 0; pos < d.num_blocks; ++pos)
-    rows[pos] = staged_row_of(out->segs, d.cpu_block_ids[pos]);
+  if (gathered) {
+    out->host_ids.assign(d.cpu_block_ids, d.cpu_block_ids + d.num_blocks);
+    out->first_by_kernel = pol.gather_first_by_kernel != 0;
+  } else {
+    int64_t *rows = reinterpret_cast<int64_t *>(h + tab);
+    for (int pos = 0; pos < d.num_blocks; ++pos)
+      rows[pos] = staged_row_of(out->segs, d.cpu_block_ids[pos]);
+  }
   uint8_t *dv = nullptr;
-  int rc = plan_publish(slot, tab + rows_bytes, /*mirror=*/true, scatter_stream, &dv);
-  if (rc != FKV_OK) {
+  if (plan_publish(slot, tab + rows_bytes, /*mirror=*/true, scatter_stream, &dv) != FKV_OK) {
     plan_release(slot, scatter_stream, false);
-    return rc;
+    return kernel_path_instead();
   }
   out->slot = slot;
   out->base_tables = reinterpret_cast<const uint64_t *>(dv);
-  out->stage_rows = reinterpret_cast<const int64_t *>(dv + tab);
+  out->stage_rows = gathered ? nullptr : reinterpret_cast<const int64_t *>(dv + tab);
   out->usable = true;
+  ring.idle_calls = 0;
+  ring.touched = true;
+  if (gathered) {
+    pinned.idle_calls = 0;
+    pinned.touched = true;
+  }
   return FKV_OK;
 }
 
+namespace {
+
+// Staging buffer k -> the engine's blocks, layers [l0, l0 + lk / kv_dim) of the plan.
+int staged_scatter(const StagedPlan &sp, StagedRing &ring, const KernelPlan &kp, int k, int l0,
+                   int lk, int64_t stride_src, hipStream_t scatter_stream) {
+  FKV_HIP_TRY(hipStreamWaitEvent(scatter_stream, ring.copied[k], 0));
+  CopyKernelArgs a{};
+  a.base_src = sp.base_tables + (size_t)k * sp.max_lk;
+  a.base_dst = kp.gpu_base + (size_t)l0 * kp.kv_dim;
+  a.ids_src = sp.stage_rows; // nullptr: row of position p is p
+  a.ids_dst = kp.gpu_ids;
+  a.stride_src = stride_src;
+  a.stride_dst = kp.gpu_block_stride;
+  a.chunk_bytes = sp.chunk;
+  a.num_blocks = sp.num_blocks;
+  a.lk = lk;
+  a.vec = kp.vec; // staging addresses are multiples of the chunk size off a 2 MiB-aligned buffer
+  a.nt_store = 1;
+  a.xcd_mask = 0;
+  const fkv_launch_policy pol = policy_of(kp.device);
+  a.unroll = pol.hbm_unroll;
+  FKV_TRY(launch_copy_kernel(a, pol.hbm_workgroups, pol.hbm_wg_threads, scatter_stream));
+  FKV_HIP_TRY(hipEventRecord(ring.freed[k], scatter_stream));
+  ring.used[k] = true;
+  stats().staged_batches.fetch_add(1, std::memory_order_relaxed);
+  return FKV_OK;
+}
+
+} // namespace
+
 int staged_launch(const StagedPlan &sp, StagedRing &ring, const KernelPlan &kp, int l0, int nl,
                   hipStream_t dma_stream, hipStream_t scatter_stream) {
-  if (!sp.usable || nl < 1 || nl > sp.batch_layers || nl * sp.kv_dim > sp.max_lk)
+  if (!sp.usable || sp.route != kRouteRuns || nl < 1 || nl > sp.batch_layers ||
+      nl * sp.kv_dim > sp.max_lk)
     return fail(FKV_ERR_RUNTIME, "staged restore: batch of %d layers does not fit its plan", nl);
   const int k = ring.next;
   ring.next = (ring.next + 1) % (int)ring.buf.size();
@@ -274,28 +421,49 @@ int staged_launch(const StagedPlan &sp, StagedRing &ring, const KernelPlan &kp, 
     }
   }
   FKV_HIP_TRY(hipEventRecord(ring.copied[k], dma_stream));
-  FKV_HIP_TRY(hipStreamWaitEvent(scatter_stream, ring.copied[k], 0));
-  CopyKernelArgs a{};
-  a.base_src = sp.base_tables + (size_t)k * sp.max_lk;
-  a.base_dst = kp.gpu_base + (size_t)l0 * kp.kv_dim;
-  a.ids_src = sp.stage_rows;
-  a.ids_dst = kp.gpu_ids;
-  a.stride_src = w;
-  a.stride_dst = kp.gpu_block_stride;
-  a.chunk_bytes = sp.chunk;
-  a.num_blocks = sp.num_blocks;
-  a.lk = lk;
-  a.vec = kp.vec; // staging addresses are multiples of the chunk size off a 2 MiB-aligned buffer
-  a.nt_store = 1;
-  a.xcd_mask = 0;
-  const fkv_launch_policy pol = policy_of(kp.device);
-  a.unroll = pol.hbm_unroll;
-  FKV_TRY(launch_copy_kernel(a, pol.hbm_workgroups, pol.hbm_wg_threads, scatter_stream));
-  FKV_HIP_TRY(hipEventRecord(ring.freed[k], scatter_stream));
-  ring.used[k] = true;
   stats().dma_copies.fetch_add(copies, std::memory_order_relaxed);
-  stats().staged_batches.fetch_add(1, std::memory_order_relaxed);
-  return FKV_OK;
+  return staged_scatter(sp, ring, kp, k, l0, lk, w, scatter_stream);
+}
+
+int gathered_launch(const StagedPlan &sp, StagedRing &ring, GatherRing &pinned, HostCrew &crew,
+                    const KernelPlan &kp, int l0, int nl, hipStream_t dma_stream,
+                    hipStream_t scatter_stream) {
+  if (!sp.usable || sp.route != kRouteGathered || nl < 1 || nl > sp.batch_layers ||
+      nl * sp.kv_dim > sp.max_lk)
+    return fail(FKV_ERR_RUNTIME, "gathered restore: batch of %d layers does not fit its plan", nl);
+  const int p = pinned.next;
+  pinned.next = (pinned.next + 1) % (int)pinned.buf.size();
+  if (pinned.used[p]) // the copy that read this buffer last
+    FKV_HIP_TRY(hipEventSynchronize(pinned.read[p]));
+  const int lk = nl * sp.kv_dim;
+  const uint8_t *row0 = sp.host0 + (int64_t)l0 * sp.cpu_layer_stride;
+  uint64_t busy_ns;
+  if (sp.kind == 0)
+    busy_ns = host_gather_rows(crew, pinned.buf[p], row0, sp.host_ids.data(), sp.num_blocks,
+                               sp.cpu_block_stride, 1, 0, 1, 0, (int64_t)lk * sp.chunk);
+  else if (sp.kind == 1)
+    busy_ns = host_gather_rows(crew, pinned.buf[p], row0, sp.host_ids.data(), sp.num_blocks,
+                               sp.cpu_block_stride, nl, sp.cpu_layer_stride, 1, 0,
+                               (int64_t)sp.kv_dim * sp.chunk);
+  else
+    busy_ns = host_gather_rows(crew, pinned.buf[p], row0, sp.host_ids.data(), sp.num_blocks,
+                               sp.cpu_block_stride, nl, sp.cpu_layer_stride, sp.kv_dim,
+                               sp.cpu_kv_stride, sp.chunk);
+  const int k = ring.next;
+  ring.next = (ring.next + 1) % (int)ring.buf.size();
+  if (ring.used[k]) // the scatter that read this buffer last
+    FKV_HIP_TRY(hipStreamWaitEvent(dma_stream, ring.freed[k], 0));
+  const size_t bytes = (size_t)sp.num_blocks * (size_t)lk * (size_t)sp.chunk;
+  // a 2-D copy of one row: the runtime hands those to the copy engines (see staged_launch)
+  FKV_HIP_TRY(hipMemcpy2DAsync(ring.buf[k], bytes, pinned.buf[p], bytes, bytes, 1,
+                               hipMemcpyHostToDevice, dma_stream));
+  FKV_HIP_TRY(hipEventRecord(pinned.read[p], dma_stream));
+  pinned.used[p] = true;
+  FKV_HIP_TRY(hipEventRecord(ring.copied[k], dma_stream));
+  stats().dma_copies.fetch_add(1, std::memory_order_relaxed);
+  stats().gathered_batches.fetch_add(1, std::memory_order_relaxed);
+  stats().gather_busy_ns.fetch_add(busy_ns, std::memory_order_relaxed);
+  return staged_scatter(sp, ring, kp, k, l0, lk, (int64_t)lk * sp.chunk, scatter_stream);
 }
 
 } // namespace fkv
@@ -312,7 +480,8 @@ extern "C" int fkv_staged_restore_plan(const int64_t *cpu_block_ids, int32_t num
     return fail(FKV_ERR_INVALID_ARG, "fkv_staged_restore_plan: bad arguments");
   std::vector<StagedPlan::Seg> segs;
   int64_t rows = 0;
-  *staged = staged_layout(cpu_block_ids, num_blocks, row_bytes, pieces, *policy, &segs, &rows) ? 1 : 0;
+  const fkv_launch_policy pol = policy_sanitized(*policy);
+  *staged = staged_route(cpu_block_ids, num_blocks, row_bytes, pieces, pol, &segs, &rows);
   if (num_runs)
     *num_runs = (int32_t)segs.size();
   if (total_rows)
@@ -320,9 +489,12 @@ extern "C" int fkv_staged_restore_plan(const int64_t *cpu_block_ids, int32_t num
   if (runs)
     for (int i = 0; i < (int)segs.size() && i < run_capacity; ++i)
       runs[i] = fkv_staged_run{segs[i].first_id, segs[i].rows, segs[i].row0};
-  if (row_of_position && *staged)
+  if (row_of_position && *staged == kRouteRuns)
     for (int pos = 0; pos < num_blocks; ++pos)
       row_of_position[pos] = staged_row_of(segs, cpu_block_ids[pos]);
+  if (row_of_position && *staged == kRouteGathered)
+    for (int pos = 0; pos < num_blocks; ++pos)
+      row_of_position[pos] = pos;
   return FKV_OK;
 }
 

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define FKV_ABI_VERSION 2 /* 2: fkv_stats grew by staged_batches; launch policy, no-alloc transfer, staging and HBM-rate entry points added */
+#define FKV_ABI_VERSION 3 /* 3: fkv_stats grew by gathered_batches and gather_busy_us, fkv_launch_policy by the host-gather and link-seeding fields; 2: fkv_stats grew by staged_batches; launch policy, no-alloc transfer, staging and HBM-rate entry points added */
 
 /* status codes */
 #define FKV_OK 0
@@ -559,6 +559,9 @@ typedef struct fkv_stats {
                                  expected to stay 0 */
   uint64_t staged_batches;    /* layer batches of a layerwise restore that went through the copy
                                  engines and a device staging buffer */
+  uint64_t gathered_batches;  /* of those, the batches whose host rows were first gathered into a
+                                 pinned buffer by host threads (one copy command per batch) */
+  uint64_t gather_busy_us;    /* time host threads spent gathering such rows, summed over threads */
 } fkv_stats;
 void fkv_get_stats(fkv_stats *out);
 void fkv_reset_stats(void);
@@ -712,6 +715,26 @@ typedef struct fkv_launch_policy {
                                  adjacent bytes instead of every wavefront access 1 KiB: 0 never,
                                  1 (default) unless the other direction is busy, 2 always (about
                                  +1 % alone on the link, -2 % in sum next to traffic the other way) */
+  /* layerwise restore of scattered host blocks: host threads gather a batch's rows into a
+   * pinned buffer, one copy command moves it (see fkv_layerwise_transfer) */
+  int32_t staged_gather;      /* FKV_STAGED_GATHER: 0 never; 1 (default) where the host blocks form
+                                 too many runs for one copy command each and the gather threads
+                                 keep up with the link; 2 whenever the copies-per-run route is
+                                 not taken */
+  int32_t gather_threads;     /* FKV_GATHER_THREADS: host threads that gather (the launching thread
+                                 of the restore is one of them); default 6, at most the cores of
+                                 the machine less one */
+  int32_t gather_ring;        /* pinned buffers per layer group and GPU */
+  int32_t gather_first_by_kernel; /* 1 (default): the first batch of such a restore goes the kernel
+                                 way, so that it lands one gather pass earlier while the rows of
+                                 the second batch are being gathered */
+  int32_t model_gather_thread_mbps; /* what one host thread gathers, MB/s, for the choice */
+  /* where the rates of the cost model come from */
+  int32_t model_seed;         /* FKV_MODEL_SEED: 1 (default) the first call that needs the model on a
+                                 device measures the link once (two short pinned copies per direction)
+                                 and scales the link-bound rates above by measured / compiled-in;
+                                 0 keeps the compiled-in figures */
+  int32_t model_seeded;       /* read-only: 1 once the rates of this table come from a measurement */
   int32_t reserved[5];
 } fkv_launch_policy;
 /* The table of `device` (-1 = current).  The first call for a device runs the probe kernel. */
@@ -724,9 +747,13 @@ int fkv_launch_policy_reset(int32_t device);
 
 /* The arithmetic behind the staged layerwise restore, without a device (tests,
  * inspection): the runs of consecutive host block ids of a call, with the holes that are
- * read along, and whether a restore of these blocks goes through the copy engines under
- * `policy`.  `row_bytes` = bytes of one host block that one batch of layers moves,
- * `pieces` = copy commands per run and batch (1 when a batch's chunks of a block are
+ * read along, and which way a restore of these blocks goes under `policy` (brought into
+ * its allowed ranges first): *staged = 0 the kernel path, 1 through the copy engines with
+ * one copy command per run (runs, rows and row_of_position describe the staging buffer),
+ * 2 through the copy engines after host threads have gathered the rows (no runs; the
+ * staging row of position p is p).  `row_bytes` = bytes of one host block that one batch
+ * of layers moves, `pieces` = copy commands per run and batch, which is also the number
+ * of pieces a gathering thread copies per block (1 when a batch's chunks of a block are
  * adjacent on the host).  No counterpart in the reference. */
 typedef struct fkv_staged_run {
   int64_t first_id; /* first host block of the run */

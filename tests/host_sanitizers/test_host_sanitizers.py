@@ -45,7 +45,7 @@ def test_ssd_engine_under_sanitizers(tmp_path, sanitizer):
 @pytest.mark.parametrize("sanitizer", SANITIZERS)
 def test_host_row_copies_under_sanitizers(tmp_path, sanitizer):
     out = build_and_run(tmp_path, "host_copy_sanitizer_driver.cpp", sanitizer, extra=("-mavx2",))
-    assert "400 scatter/gather pairs" in out
+    assert "400 scatter/gather pairs and 300 crew gathers" in out
 
 
 @pytest.mark.parametrize("sanitizer", SANITIZERS)

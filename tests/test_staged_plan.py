@@ -1,7 +1,9 @@
-"""The arithmetic that decides whether a layerwise restore goes through the copy
-engines (fkv_staged_restore_plan, no device involved): runs of consecutive host
-block ids, holes that are read along, the staging row of every position.  Checked by
-invariants and by a brute-force statement of the same rules on small id sets."""
+"""The arithmetic that decides which way a layerwise restore goes
+(fkv_staged_restore_plan, no device involved): runs of consecutive host block ids,
+holes that are read along, the staging row of every position, and the choice among
+the kernel path, one copy command per run, and rows gathered by host threads with
+one copy command per batch.  Checked by invariants and by a brute-force statement of
+the same rules on small id sets."""
 import ctypes
 
 import numpy as np
@@ -31,8 +33,11 @@ def plan(ids, row_bytes, pieces, pol):
                                          ctypes.byref(pol), ctypes.byref(staged),
                                          ctypes.byref(nruns), ctypes.byref(rows), runs, ids.size,
                                          row_of.ctypes.data))
-    return bool(staged.value), [(r.first_id, r.rows, r.row0) for r in runs[:nruns.value]], \
+    return staged.value, [(r.first_id, r.rows, r.row0) for r in runs[:nruns.value]], \
         rows.value, row_of
+
+
+KERNEL, RUNS, GATHERED = 0, 1, 2
 
 
 def brute_force(ids, row_bytes, pieces, pol):
@@ -61,6 +66,7 @@ def brute_force(ids, row_bytes, pieces, pol):
         batch_us = useful / (pol.link_gbps_estimate * 1e3)
         chosen = chosen and len(runs) * pieces * pol.staged_copy_overhead_us <= \
             batch_us * pol.staged_overhead_pct / 100
+    chosen = chosen and len(runs) * pieces <= 4096   # never thousands of commands per batch
     return chosen and pol.staged_restore != 0, runs, total
 
 
@@ -79,7 +85,7 @@ def test_runs_and_rows_against_brute_force(seed):
     pol = policy(staged_restore=2)          # the layout itself, whatever the cost rule says
     staged, runs, total, row_of = plan(ids, row_bytes, pieces, pol)
     want_staged, want_runs, want_total = brute_force(ids, row_bytes, pieces, pol)
-    assert staged == want_staged
+    assert staged == (RUNS if want_staged else KERNEL)
     if not staged:
         return
     assert [(f, r) for f, r, _ in runs] == want_runs and total == want_total
@@ -109,6 +115,77 @@ def test_the_choice():
     # K and V apart on the host: twice the commands per run
     few = np.concatenate([np.arange(0, 200), np.arange(300, 500), np.arange(700, 900)])
     assert plan(few, 73728, 1, pol)[0] and not plan(few, 73728, 4, pol)[0]
+
+
+def gather_policy(**kw):
+    kw.setdefault("staged_gather", 1)
+    kw.setdefault("gather_threads", 4)
+    kw.setdefault("model_gather_thread_mbps", 20000)
+    kw.setdefault("model_link_mbps", 57200)
+    return policy(**kw)
+
+
+def route_by_the_rules(ids, row_bytes, pieces, pol, cores):
+    """The three-way choice restated: runs first; else the gather when the one copy
+    command of a batch is cheap against the batch's link time and the threads finish
+    a batch in 80 % of that time."""
+    if brute_force(ids, row_bytes, pieces, pol)[0]:
+        return RUNS
+    n = len(ids)
+    nbytes = n * row_bytes
+    if pol.staged_gather == 0 or nbytes > pol.staged_max_mb << 20:
+        return KERNEL
+    if pol.staged_gather == 2:
+        return GATHERED
+    link_us = nbytes / pol.model_link_mbps
+    if pol.staged_copy_overhead_us > link_us * pol.staged_overhead_pct / 100:
+        return KERNEL
+    threads = max(1, min(pol.gather_threads, max(1, cores - 1)))
+    gather_us = nbytes / (threads * pol.model_gather_thread_mbps) + n * pieces * 0.05 / threads
+    return GATHERED if gather_us <= 0.8 * link_us else KERNEL
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_the_three_way_choice_against_its_rules(seed):
+    import os
+    rng = np.random.default_rng(100 + seed)
+    pool = int(rng.integers(64, 5000))
+    n = int(rng.integers(1, min(pool, 600) + 1))
+    ids = rng.permutation(pool)[:n] if seed % 4 else np.arange(7, 7 + n)
+    row_bytes = int(rng.choice([2048, 73728, 262144, 1 << 20]))
+    pieces = int(rng.choice([1, 2, 16, 64]))
+    pol = gather_policy(staged_restore=int(rng.choice([0, 1, 1, 2])),
+                        staged_gather=int(rng.choice([0, 1, 1, 2])),
+                        gather_threads=int(rng.choice([1, 2, 4, 6])),
+                        model_link_mbps=int(rng.choice([14000, 28600, 57200])))
+    got, runs, total, row_of = plan(ids, row_bytes, pieces, pol)
+    assert got == route_by_the_rules(ids, row_bytes, pieces, pol, os.cpu_count() or 1), \
+        (n, row_bytes, pieces, pol.staged_restore, pol.staged_gather, pol.gather_threads)
+    if got == GATHERED:   # no runs; position p is staged on row p
+        assert runs == [] and total == n and (row_of == np.arange(n)).all()
+
+
+def test_scattered_host_blocks_are_gathered_when_the_threads_keep_up():
+    scattered = np.random.default_rng(1).permutation(4096)[:512]
+    one_run = np.arange(100, 612)
+    c3 = (scattered, 73728, 1)                                    # 36 MiB per batch, 512 runs
+    assert plan(*c3, gather_policy())[0] == GATHERED
+    assert plan(one_run, 73728, 1, gather_policy())[0] == RUNS    # a run needs no host pass
+    assert plan(*c3, gather_policy(staged_gather=0))[0] == KERNEL
+    # two threads at 20 GB/s each do not finish 36 MiB inside 80 % of its link time ...
+    assert plan(*c3, gather_policy(gather_threads=2))[0] == KERNEL
+    # ... unless the link is half as fast: the choice follows the link figure
+    assert plan(*c3, gather_policy(gather_threads=2, model_link_mbps=28600))[0] == GATHERED
+    # a batch of 16 KiB: one copy command costs more than the batch's time on the link
+    assert plan(scattered[:4], 4096, 1, gather_policy())[0] == KERNEL
+    assert plan(scattered[:4], 4096, 1, gather_policy(staged_gather=2))[0] == GATHERED
+    # rows cut into 64 small pieces each: the per-piece cost eats the margin
+    assert plan(scattered, 73728, 64, gather_policy())[0] == KERNEL
+    # forced routes for tests: runs wins where both are forced
+    assert plan(*c3, gather_policy(staged_restore=2, staged_gather=2))[0] == RUNS
+    assert plan(*c3, gather_policy(staged_restore=0, staged_gather=2))[0] == GATHERED
+    # a batch beyond the largest staging buffer stays on the kernel path
+    assert plan(scattered, 2 << 20, 1, gather_policy(staged_gather=2))[0] == KERNEL
 
 
 def test_holes_are_bridged_smallest_first_within_the_allowance():

@@ -1,8 +1,10 @@
-"""Layerwise restore through the copy engines (host rows -> staging buffer ->
-scatter kernel) against the oracle, next to the same restore on the kernel path.
+"""Layerwise restore through the copy engines against the oracle, next to the same
+restore on the kernel path: host rows -> staging buffer -> scatter kernel with one
+copy command per run of host blocks, and host rows -> pinned buffer (gathered by host
+threads) -> staging buffer -> scatter kernel with one copy command per batch.
 
-The choice between the two is a matter of the launch policy; the tests force it
-either way, so which path a case runs does not depend on the box."""
+The choice among the three is a matter of the launch policy; the tests force it,
+so which route a case runs does not depend on the box."""
 import numpy as np
 import pytest
 import torch
@@ -50,22 +52,28 @@ def host_ids(rng, pool, n, pattern):
     return rng.permutation(ids).astype(np.int64)  # positions in any order
 
 
-@pytest.mark.parametrize("staged", [2, 0], ids=["copy_engines", "kernel"])
+ROUTES = {"copy_engines": dict(staged_restore=2, staged_gather=0),
+          "gathered": dict(staged_restore=0, staged_gather=2, gather_first_by_kernel=0),
+          "gathered_first_by_kernel": dict(staged_restore=0, staged_gather=2, gather_first_by_kernel=1),
+          "kernel": dict(staged_restore=0, staged_gather=0)}
+
+
+@pytest.mark.parametrize("route", list(ROUTES))
 @pytest.mark.parametrize("pattern", ["one_run", "runs_and_holes", "scattered"])
 @pytest.mark.parametrize("backend,kv_dim,cpu_layout,gran", [
     (VLLM, 1, "BLOCKFIRST", 1), (VLLM, 2, "BLOCKFIRST", 3), (VLLM, 2, "LAYERFIRST", 2),
     (TRTLLM, 2, "BLOCKFIRST", 2), (SGLANG, 2, "BLOCKFIRST", 1), (SGLANG, 2, "LAYERFIRST", 4)])
-def test_restore_matches_the_oracle(gpu_device, staged, pattern, backend, kv_dim, cpu_layout, gran):
-    """Seven layers (more batches than staging buffers), three restores in a row
-    through the same group with fresh host bytes each time: a stale staging buffer
-    or a buffer reused too early would show up as old bytes."""
+def test_restore_matches_the_oracle(gpu_device, route, pattern, backend, kv_dim, cpu_layout, gran):
+    """Seven layers (more batches than staging or pinned buffers), three restores in a
+    row through the same group with fresh host bytes each time: a stale buffer or a
+    buffer reused too early would show up as old bytes."""
     from flexkv_amd.c_ext import get_stats, launch_policy, reset_stats
     L, NG, NC, n, chunk = 7, 96, 80, 41, 4608
     s = KVSetup(backend, L, kv_dim, NG, NC, chunk, cpu_layout, seed=17 + gran)
     dev = s.to_device(gpu_device)
     grp = group_of(s, dev)
     rng = np.random.default_rng(5 * gran + kv_dim)
-    with launch_policy(staged_restore=staged, staged_ring=3):
+    with launch_policy(staged_ring=3, gather_ring=2, gather_threads=3, **ROUTES[route]):
         reset_stats()
         for rep in range(3):
             fresh = rng.integers(0, 256, s.host_bytes, dtype=np.uint8)
@@ -77,8 +85,11 @@ def test_restore_matches_the_oracle(gpu_device, staged, pattern, backend, kv_dim
             s.oracle_transfer(gids, cids, True)
             dev.assert_matches_reference(f"restore {rep} ({pattern})")
         st = get_stats()
-    batches = 3 * ((L + gran - 1) // gran)
-    assert st["staged_batches"] == (batches if staged else 0), st
+    batches = (L + gran - 1) // gran
+    want_staged = {"copy_engines": 3 * batches, "gathered": 3 * batches,
+                   "gathered_first_by_kernel": 3 * (batches - 1), "kernel": 0}[route]
+    assert st["staged_batches"] == want_staged, st
+    assert st["gathered_batches"] == (want_staged if route.startswith("gathered") else 0), st
     grp.close()
 
 
@@ -100,23 +111,88 @@ def test_restore_of_a_layer_prefix_and_duplicate_host_blocks(gpu_device):
     grp.close()
 
 
+def test_gathered_restore_announces_layers_in_order_and_serves_waiting_streams(gpu_device):
+    """The gathered route launches batch by batch from a thread of its own.  A consumer
+    stream that asks for a layer before its batch has been enqueued must still see the
+    layer's bytes (fkv_layerwise_wait_layer waits for the record first), the eventfds
+    count one unit per layer, and the caller's id lists may be dropped right after the
+    call returns."""
+    import os
+    import select
+    from flexkv_amd.c_ext import LayerwiseTransferGroup, get_stats, launch_policy, reset_stats
+    L, NG, NC, n, chunk = 9, 128, 160, 77, 18432
+    s = KVSetup(VLLM, L, 1, NG, NC, chunk, "BLOCKFIRST", seed=41)
+    dev = s.to_device(gpu_device)
+    fds = [os.eventfd(0, os.EFD_SEMAPHORE | os.EFD_NONBLOCK) for _ in range(L)]
+    i64 = lambda v: torch.tensor([v], dtype=torch.int64)
+    grp = LayerwiseTransferGroup(
+        num_gpus=1, gpu_blocks=[dev.gpu], cpu_blocks=dev.host, ssd_files={}, num_layers=L,
+        gpu_kv_strides_tensor=i64(s.gpu_kv_stride), gpu_block_strides_tensor=i64(s.gpu_block_stride),
+        gpu_layer_strides_tensor=i64(s.gpu_layer_stride), gpu_chunk_sizes_tensor=i64(s.chunk),
+        iouring_entries=0, iouring_flags=0,
+        layer_eventfds_tensor=torch.tensor(fds, dtype=torch.int32), tp_size=1, is_blockfirst=True)
+    rng = np.random.default_rng(8)
+    e = torch.empty(0, dtype=torch.int64)
+    comp = torch.cuda.Stream()
+    with launch_policy(staged_restore=0, staged_gather=2, gather_ring=2, gather_threads=2):
+        for notify in ("polling", "hostfunc", "polling"):
+            gids = rng.permutation(NG)[:n].astype(np.int64)
+            cids = rng.permutation(NC)[:n].astype(np.int64)
+            reset_stats()
+            g_t, c_t = torch.from_numpy(gids.copy()), torch.from_numpy(cids.copy())
+            grp.layerwise_transfer(
+                e, e, 0, 0, 0, 0, 0, g_t, c_t, s.cpu_kv_stride, s.cpu_layer_stride,
+                s.cpu_block_stride, s.chunk, s.cpu_kv_stride, s.cpu_layer_stride,
+                s.cpu_block_stride, 4, False, L, 1, 1, 1, counter_id=0,
+                kv_shared_across_ranks_mode="sharded", notify_mode=notify)
+            g_t.zero_()   # the library keeps what it needs of the id lists
+            c_t.zero_()
+            del g_t, c_t
+            # every layer, read on a consumer stream right behind its event
+            seen = []
+            gi = torch.from_numpy(gids).to(gpu_device)
+            with torch.cuda.stream(comp):
+                for l in range(L):
+                    grp.wait_layer(l, comp)
+                    seen.append(dev.gpu[l].view(torch.uint8).view(NG, -1).index_select(0, gi).clone())
+            comp.synchronize()
+            grp.synchronize()
+            s.oracle_transfer(gids, cids, True)
+            dev.assert_matches_reference(f"gathered restore, {notify}")
+            for l in range(L):
+                want = s.host_ref.reshape(NC, L, chunk)[cids, l]
+                assert np.array_equal(seen[l].cpu().numpy(), want), (notify, l)
+            assert get_stats()["gathered_batches"] == L - 1   # the first batch by kernel
+            for l, fd in enumerate(fds):
+                assert select.select([fd], [], [], 5.0)[0], (notify, l)
+                assert os.eventfd_read(fd) == 1
+                assert not select.select([fd], [], [], 0)[0], (notify, l)
+    grp.close()
+    for fd in fds:
+        os.close(fd)
+
+
 def test_the_choice_follows_the_runs_of_host_blocks(gpu_device):
-    """With the default policy a restore whose host blocks form one run goes
-    through the copy engines, one whose host blocks are scattered does not; both
-    give the oracle's bytes.  (The choice is arithmetic on the id list: no timing.)"""
+    """With the default policy a restore whose host blocks form one run goes through
+    the copy engines with one copy command, one whose host blocks are scattered has its
+    rows gathered by host threads first (or stays on the kernel path where that route
+    is switched off); all give the oracle's bytes.  (The choice is arithmetic on the id
+    list: no timing.)"""
     from flexkv_amd.c_ext import get_stats, launch_policy, reset_stats
     L, n, chunk = 4, 256, 73728
     s = KVSetup(VLLM, L, 1, 300, 300, chunk, "BLOCKFIRST", seed=9)
     dev = s.to_device(gpu_device)
     grp = group_of(s, dev)
     rng = np.random.default_rng(2)
-    with launch_policy(staged_restore=1):
-        for pattern, want in (("one_run", L), ("scattered", 0)):
+    for gather, pattern, want, want_gathered in ((1, "one_run", L, 0), (1, "scattered", L - 1, L - 1),
+                                                 (0, "scattered", 0, 0)):
+        with launch_policy(staged_restore=1, staged_gather=gather):
             gids = rng.permutation(300)[:n].astype(np.int64)
             cids = host_ids(rng, 300, n, pattern)
             reset_stats()
             restore(grp, s, gids, cids, gran=1)
-            assert get_stats()["staged_batches"] == want, (pattern, get_stats())
+            st = get_stats()
+            assert (st["staged_batches"], st["gathered_batches"]) == (want, want_gathered), (pattern, st)
             s.oracle_transfer(gids, cids, True)
             dev.assert_matches_reference(pattern)
     grp.close()
