@@ -514,8 +514,10 @@ class TPTransferThreadGroup:
                  num_kv_heads: int = 1, ce_gather_threads: int = 4,
                  ce_gather_nt: bool = True) -> None:
         self._h = ctypes.c_void_p()
-        if enable_nvcomp:
-            raise RuntimeError("nvcomp compressed transfer is not part of this library")
+        # enable_nvcomp, nvcomp_batch_size and nvcomp_data_type are accepted and ignored, as
+        # in a build of the reference without the codec (csrc/tp_transfer_thread_group.cpp:
+        # 132-136).  The reference's own worker passes its copy-engine settings in these
+        # positions (flexkv/transfer/worker.py:1218-1236), so a truthy value is no request.
         ptrs = np.ascontiguousarray(np.asarray(list(gpu_block_ptrs_flat), dtype=np.uint64))
         if ptrs.size != num_gpus * num_tensors_per_gpu:
             raise ValueError("gpu_block_ptrs_flat must hold num_gpus * num_tensors_per_gpu pointers")

@@ -30,7 +30,18 @@
  *                             names (tests/test_ce_analysis.py)
  *   fkv_oracle_tp_rank_plan   closed forms + partition properties (shards
  *                             tile the chunk, layer slices tile the range)
- *   fkv_oracle_host_scatter   equality with numpy fancy indexing
+ *   fkv_oracle_host_scatter   numpy fancy indexing of shaped [N,L,kv,chunk] and
+ *                             [L,kv,N,chunk] pools, both directions, untouched bytes,
+ *                             in-chunk offsets (tests/test_oracle.py)
+ *   fkv_oracle_is_full_block  the shapes the reference names: rank0_only / all_write
+ *                             calls are full blocks, layer_parallel and sharded puts
+ *                             are not (per-rank shapes from the rank plan, host block
+ *                             from the layout's closed form; tests/test_oracle.py)
+ *   fkv_oracle_eventfd_index  enumeration of a [3, tp, layers] table in Python loops
+ *                             (tests/test_oracle.py); the GPU tests of the
+ *                             notification contract index their eventfds with it
+ *   fkv_oracle_layerwise_cpu_startoff  closed forms per mode (tests/test_tp_plan.py)
+ *   fkv_oracle_host_chunk_bytes  the reference's constants (tests/test_abi.py)
  *   fkv_oracle_ssd_locate     the reference's second statement of the same
  *                             mapping (flexkv/transfer/nixlutil.py:351-385) as
  *                             closed forms, bijection onto a dense

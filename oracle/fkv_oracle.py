@@ -227,6 +227,28 @@ def ce_choose_path(analysis: Analysis, is_blockfirst: bool, num_kv_heads: int,
         chunk, int(is_host_to_device), int(is_full_block)))
 
 
+def is_full_block(num_layers: int, kv_dim: int, chunk: int, cpu_block_stride: int) -> bool:
+    return bool(lib().fkv_oracle_is_full_block(num_layers, kv_dim, chunk, cpu_block_stride))
+
+
+def eventfd_index(counter: int, tp_rank: int, layer: int, tp_size: int, num_layers: int) -> int:
+    return int(lib().fkv_oracle_eventfd_index(counter, tp_rank, layer, tp_size, num_layers))
+
+
+def host_scatter(staging: np.ndarray, cpu: np.ndarray, cpu_ids, cpu_block_stride: int,
+                 cpu_off: int, chunk: int, layer: int, kv: int, cpu_kv_stride: int,
+                 cpu_layer_stride: int, to_cpu: bool) -> None:
+    """Rows of one (layer, kv) between a dense staging array and the host cache,
+    in place on the two uint8 arrays."""
+    ids = _i64(cpu_ids)
+    assert staging.dtype == np.uint8 and cpu.dtype == np.uint8
+    assert staging.flags.c_contiguous and cpu.flags.c_contiguous
+    assert staging.size >= ids.size * chunk
+    lib().fkv_oracle_host_scatter(_ptr(staging), _ptr(cpu), _ptr(ids), ids.size, cpu_block_stride,
+                                  cpu_off, chunk, layer, kv, cpu_kv_stride, cpu_layer_stride,
+                                  int(to_cpu))
+
+
 def tp_rank_plan(rank, num_gpus, num_kv_heads, is_h2d, mode, designated_rank,
                  rotate_counter, layer_id, layer_granularity, num_blocks,
                  gpu_chunk_size, cpu_block_stride, cpu_tp_stride):

@@ -156,7 +156,7 @@ def test_strategy_matrix(pattern, cpu_layout, kv_dim, num_kv_heads, thr):
                     layers_in_call = Lyr // tp        # a rank moves 1/tp of the layers
             cbs = cpu.get_block_stride() * es
             an, _ = lib_analyze(ids, ids, cbs, chunk, gbs)
-            full = layers_in_call * kv_dim * chunk == cbs
+            full = O.is_full_block(layers_in_call, kv_dim, chunk, cbs)
             got = NAMES[lib_choose(an, cpu_layout == "BLOCKFIRST", num_kv_heads, thr, chunk, h2d,
                                    full)]
             want = predicted(pattern, cpu_layout, kv_dim, num_kv_heads, mode, h2d, n, thr)

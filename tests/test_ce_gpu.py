@@ -14,7 +14,7 @@ PATHS = {"CONTIG_DIRECT": 0, "SEGMENT_DIRECT": 1, "SEGMENT_SCATTER": 2, "GATHER_
 
 def expected_path(s, gids, cids, heads, thr, h2d, num_layers):
     an, _ = O.ce_analyze(gids, cids, s.cpu_block_stride, s.chunk, s.gpu_block_stride)
-    full = num_layers * s.kv_dim * s.chunk == s.cpu_block_stride
+    full = O.is_full_block(num_layers, s.kv_dim, s.chunk, s.cpu_block_stride)
     return O.CE_NAMES[O.ce_choose_path(an, s.cpu_layout == "BLOCKFIRST", heads, thr, s.chunk,
                                        h2d, full)]
 

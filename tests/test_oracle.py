@@ -345,3 +345,86 @@ def test_units_precondition():
     assert L.fkv_oracle_units_ok(32768, 0, 0, 64, 32768, 128, 32768, 65536, 2097152) == 16
     assert L.fkv_oracle_units_ok(37440, 4680, 4680, 0, 37440, 0, 37440, 37440, 37440) == 8
     assert L.fkv_oracle_units_ok(100, 0, 0, 0, 100, 0, 100, 100, 100) == 0
+
+
+# ---- host staging rows, full-block test, eventfd table ----------------------
+
+@pytest.mark.parametrize("cpu_layout", ["BLOCKFIRST", "LAYERFIRST"])
+@pytest.mark.parametrize("kv_dim", [1, 2])
+def test_host_scatter_equals_numpy_indexing_of_a_shaped_pool(cpu_layout, kv_dim):
+    """scatter_to_cpu / gather_from_cpu (csrc/ce_transfer.cu:523-641) move the rows of
+    one (layer, kv) between a dense staging array [n, chunk] and the host cache.  On a
+    shaped pool that is pool[ids, l, kv] = staging (block-first) or pool[l, kv, ids] =
+    staging (layer-first), and the reverse; nothing else may change."""
+    L, N, n, chunk = 3, 11, 6, 40
+    rng = np.random.default_rng(kv_dim + (7 if cpu_layout == "BLOCKFIRST" else 0))
+    shape = (N, L, kv_dim, chunk) if cpu_layout == "BLOCKFIRST" else (L, kv_dim, N, chunk)
+    pool = rng.integers(0, 256, shape, dtype=np.uint8)
+    s = pool.strides
+    cbs, cls, cks = (s[0], s[1], s[2]) if cpu_layout == "BLOCKFIRST" else (s[2], s[0], s[1])
+    ids = rng.permutation(N)[:n]
+    for l in range(L):
+        for kv in range(kv_dim):
+            staging = rng.integers(0, 256, (n, chunk), dtype=np.uint8)
+            want = pool.copy()
+            if cpu_layout == "BLOCKFIRST":
+                want[ids, l, kv] = staging
+            else:
+                want[l, kv, ids] = staging
+            O.host_scatter(staging, pool.reshape(-1), ids, cbs, 0, chunk, l, kv, cks, cls, True)
+            assert np.array_equal(pool, want), (l, kv)
+            back = np.zeros_like(staging)
+            O.host_scatter(back, pool.reshape(-1), ids, cbs, 0, chunk, l, kv, cks, cls, False)
+            assert np.array_equal(back, staging), (l, kv)
+    # an in-chunk offset with a shorter row moves that byte range of every chunk only
+    staging = rng.integers(0, 256, (n, 8), dtype=np.uint8)
+    want = pool.copy()
+    if cpu_layout == "BLOCKFIRST":
+        want[ids, 1, 0, 16:24] = staging
+    else:
+        want[1, 0, ids, 16:24] = staging
+    O.host_scatter(staging, pool.reshape(-1), ids, cbs, 16, 8, 1, 0, cks, cls, True)
+    assert np.array_equal(pool, want)
+
+
+def test_is_full_block_on_the_shapes_the_reference_names():
+    """csrc/transfer.cu:219-220: a call is a full block when the layers, K/V planes and
+    chunk bytes it moves fill one block-first host block.  The reference's comment and
+    its test predictor (tests/test_kv_transfer_correctness.py:1292-1300) name the
+    shapes: rank0_only / all_write move all layers of the whole chunk -> full;
+    layer_parallel moves a slice of the layers and a sharded put a slice of every
+    chunk -> not full.  The per-rank shapes come from the rank plan (pinned by its own
+    partition properties), the host block from the layout's closed form."""
+    L, N, T, H, D, es = 6, 16, 8, 1, 64, 2
+    for kv_dim in (1, 2):
+        lay = KVCacheLayout(KVCacheLayoutType.BLOCKFIRST, L, N, T, H, D, kv_dim=kv_dim)
+        chunk, cbs = lay.get_chunk_size() * es, lay.get_block_stride() * es
+        assert cbs == torch.empty(lay.kv_shape, dtype=torch.int16).stride()[0] * es
+        for n in (1, 2, 4):
+            for mode, want_full in (("rank0_only", True), ("all_write", True),
+                                    ("layer_parallel", n == 1), ("sharded", n == 1)):
+                for rank in range(n):
+                    p = O.tp_rank_plan(rank, n, 1, False, mode, 0, 0, 0, L, 4, chunk, cbs, cbs // n)
+                    if not p.active:
+                        continue
+                    got = O.is_full_block(p.num_layers, kv_dim, p.chunk_size, cbs)
+                    assert got == want_full, (kv_dim, n, mode, rank)
+        # a host block with padding behind the layers is never full
+        assert not O.is_full_block(L, kv_dim, chunk, cbs + 64)
+        assert not O.is_full_block(L - 1, kv_dim, chunk, cbs)
+
+
+def test_eventfd_index_enumerates_the_table():
+    """csrc/layerwise.cpp:15-34, 537-544: the eventfd of (counter, tp_rank, layer) in the
+    flat table the engine hands over as [num_counters, tp_size, num_layers]
+    (flexkv/integration/sglang/comm.py:771 builds it with three counters)."""
+    for tp, L in ((1, 5), (2, 6), (8, 61)):
+        table = np.arange(3 * tp * L).reshape(3, tp, L)
+        seen = set()
+        for c in range(3):
+            for r in range(tp):
+                for l in range(L):
+                    i = O.eventfd_index(c, r, l, tp, L)
+                    assert table[c, r, l] == i
+                    seen.add(i)
+        assert seen == set(range(3 * tp * L))
