@@ -548,7 +548,7 @@ int shape_for_now(const KernelPlan &p, int64_t bytes, hipStream_t stream, CopyKe
     a->xcd_mask = (all + 1u) & ~all ? ((all + 1u) & ~all) : 0x8000u;
     a->claims_per_wg = 1;
   } else if (pol.arbiter == 2 ||
-             (pol.arbiter == 1 && busy_mask != all &&
+             (pol.arbiter == 1 && busy_mask != all && !p.recorded &&
               link_direction_busy(p.device, !p.h2d, stream))) {
     a->xcd_mask = busy_mask;
     workgroups = busy_workgroups;

@@ -230,6 +230,8 @@ struct KernelPlan {
   int device = 0;
   bool no_alloc = false; // built by the entry point that allocates nothing: launches of this
                          // plan create no events and do not probe the device
+  bool recorded = false; // the launches are being recorded into a graph: shaped once for every
+                         // replay, without a look at what the link is doing right now
   uint64_t *claims = nullptr; // a claim counter per layer of the plan, device memory
 };
 // Link-bound launches of the last while, per device and direction (see fkv_core.cpp).

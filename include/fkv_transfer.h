@@ -137,17 +137,25 @@ int fkv_transfer_kv_blocks_multi(const fkv_transfer_desc *descs, int32_t count, 
  * of the launch (base tables, block-id lists) and the claim counters live in a fixed
  * array in device memory that belongs to the library's code object (one copy per GPU,
  * held until the process ends) instead of memory allocated on demand; the call makes
- * no hipMalloc / hipHostMalloc / hipFree and creates no streams or events.
+ * no hipMalloc / hipHostMalloc / hipFree, creates no streams or events, copies nothing
+ * with hipMemcpy and keeps no stream handle.  All it enqueues on `stream` is kernel
+ * launches (the plan travels in the arguments of small fill kernels), so a stream
+ * capture can record it; a replay moves the bytes that the tensors hold at that time.
  *   - same descriptor, same bytes moved as fkv_transfer_kv_blocks on the kernel path;
  *     use_ce_transfer must be 0 (FKV_ERR_UNSUPPORTED otherwise);
  *   - limit: 16 * num_blocks + 16 * num_layers * kv_dim <= FKV_NOALLOC_MAX_PLAN_BYTES and
  *     num_layers <= 1024 (FKV_ERR_INVALID_ARG beyond; split the call);
+ *   - block-id arrays in pinned, registered or device memory are read in place by the
+ *     kernel, as the reference's kernel reads its id tensors (csrc/transfer.cu:121-122):
+ *     keep them unchanged until the transfer has run (a recorded graph reads them anew
+ *     at every replay); id arrays in pageable memory are copied into the launches and
+ *     may be reused as soon as the call returns;
  *   - all calls on one GPU share the array: calls on one stream are ordered by the
- *     stream; a call first waits on the host for the stream of the previous call on
- *     that GPU; calls that are in flight at the same time on different streams of one
- *     GPU race and must be ordered by the caller;
- *   - desc->sync waits with hipStreamSynchronize; the launches are not confined by the
- *     link arbiter of fkv_transfer_kv_blocks until that call has set up the device. */
+ *     stream; calls that are in flight at the same time on different streams of one GPU
+ *     race for it and must be ordered by the caller; the call itself waits for nothing;
+ *   - desc->sync waits with hipStreamSynchronize (leave it 0 under capture); the launches
+ *     are not confined by the link arbiter of fkv_transfer_kv_blocks until that call has
+ *     set up the device, and a recorded launch keeps the shape it was recorded with. */
 #define FKV_NOALLOC_MAX_PLAN_BYTES (1u << 20)
 int fkv_transfer_kv_blocks_noalloc(const fkv_transfer_desc *desc, void *stream);
 
