@@ -235,6 +235,9 @@ SIGNATURES = {
                                         c_int32, c_int32, c_int32, c_int32, c_int32,
                                         c_int32, c_int32, c_char_p, c_int32]),
     "fkv_tp_group_destroy": (None, [c_void_p]),
+    "fkv_launch_policy_seed": (c_int32, [c_int32]),
+    "fkv_launch_policy_seeded": (c_int32, [POINTER(LaunchPolicy), c_double, c_double, c_double,
+                                           POINTER(LaunchPolicy)]),
     "fkv_layerwise_create": (c_int32, [POINTER(LayerwiseParams), POINTER(c_void_p)]),
     "fkv_layerwise_create_multi_group": (c_int32, [POINTER(LayerwiseMGParams),
                                                    POINTER(c_void_p)]),

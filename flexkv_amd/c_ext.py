@@ -388,6 +388,14 @@ def set_launch_policy(device: int = -1, **fields: int) -> Dict[str, int]:
     return get_launch_policy(device)
 
 
+def seed_launch_policy(device: int = -1) -> Dict[str, int]:
+    """Re-base the link-dependent figures of the cost model on a measurement of ``device``
+    (once per device; the library does it by itself before the first layerwise restore and
+    the first transfer with ``use_ce_transfer=2``).  Returns the table."""
+    check(_L.fkv_launch_policy_seed(int(device)))
+    return get_launch_policy(device)
+
+
 def reset_launch_policy(device: int = -1) -> None:
     check(_L.fkv_launch_policy_reset(int(device)))
 

@@ -256,6 +256,8 @@ struct Job {
   // which carries the compaction launches.
   mutable hipStream_t lane = nullptr;
   int64_t rect_min_bytes = -1; // from ce_rect_min_kb of the launch policy (run_ce_path)
+  bool host_pinned = true;     // the host pool is pinned or registered memory (run_ce_path);
+                               // the runtime stages 2-D copies of pageable memory synchronously
   // set by the strategies whose host thread waits for each copy (staging ping-pong)
   mutable bool host_waits = false;
 
@@ -727,17 +729,20 @@ struct GatherDirectShape {
   size_t cap_blocks = 1, total_cmds = 0, group = 1;
   bool pipelined = false;
   bool enable_memcpy2d = false;
+  bool rows_as_2d = true; // pinned host pool: runs of three rows and more go as one 2-D copy
   // Copy commands of `rows` consecutive host blocks: one where the bytes are one run
   // (whole blocks) or a 2-D copy takes the rows (asked for by the caller, or three rows
-  // and more: a layer-by-layer restore of 512 adjacent host blocks, 72 KiB of each per
-  // layer, runs at 53.5 GB/s with one 2-D copy per layer, and a multi-group restore went
-  // from 9.9 to 40.8 GB/s); else one per row.
-  bool two_d(size_t rows) const { return enable_memcpy2d || rows >= 3; }
+  // and more of a pinned pool: a layer-by-layer restore of 512 adjacent host blocks,
+  // 72 KiB of each per layer, runs at 53.5 GB/s with one 2-D copy per layer, and a
+  // multi-group restore went from 9.9 to 40.8 GB/s); else one per row.  A pageable pool
+  // gets 2-D copies only where the caller asks for them, as in the reference.
+  bool two_d(size_t rows) const { return enable_memcpy2d || (rows_as_2d && rows >= 3); }
   size_t cmds_of(size_t rows) const { return full_block || two_d(rows) ? (size_t)1 : rows; }
 };
 GatherDirectShape gather_direct_shape(const fkv_transfer_desc &d, const HostOrder &order,
-                                      size_t staging_cap, bool may_pipeline) {
+                                      size_t staging_cap, bool may_pipeline, bool host_pinned) {
   GatherDirectShape g;
+  g.rows_as_2d = host_pinned;
   g.block_bytes = (size_t)d.num_layers * d.kv_dim * (size_t)d.chunk_size;
   g.full_block = (int64_t)g.block_bytes == d.cpu_block_stride;
   g.enable_memcpy2d = d.ce.enable_memcpy2d != 0;
@@ -772,9 +777,10 @@ int gather_direct(const Job &j) {
   d.gpu_block_ids = order.gpu_ids.data();
   d.cpu_block_ids = order.cpu_ids.data();
   StageSet &ss = stage_set(j.device);
-  GatherDirectShape shape = gather_direct_shape(d, order, staging_cap_bytes(), pipeline_enabled());
+  GatherDirectShape shape =
+      gather_direct_shape(d, order, staging_cap_bytes(), pipeline_enabled(), j.host_pinned);
   if (shape.pipelined && !ss.ensure_pipeline())
-    shape = gather_direct_shape(d, order, staging_cap_bytes(), false);
+    shape = gather_direct_shape(d, order, staging_cap_bytes(), false, j.host_pinned);
   const size_t block_bytes = shape.block_bytes;
   const bool full_block = shape.full_block, pipelined = shape.pipelined;
   auto two_d = [&](size_t rows) { return shape.two_d(rows); };
@@ -983,8 +989,9 @@ CeWork ce_work(const Job &j, int path) {
       // one command per run of consecutive host blocks, whatever the GPU side looks like;
       // with two staging buffers only the first group's compaction is on the critical path
       const fkv_launch_policy pol = policy_peek(d.device < 0 ? current_device() : d.device);
+      // priced for a pinned pool (no device call here to ask the runtime about the pointer)
       const GatherDirectShape g = gather_direct_shape(d, host_order(d), (size_t)pol.ce_staging_mb << 20,
-                                                      pol.ce_two_streams == 1);
+                                                      pol.ce_two_streams == 1, true);
       w.dmas = (double)g.total_cmds;
       w.device_staged = g.pipelined ? (double)g.group * (double)g.block_bytes : bytes;
     } else {
@@ -1033,13 +1040,14 @@ int run_ce_path(const fkv_transfer_desc &d, hipStream_t stream) {
         d.is_host_to_device ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost, {}};
   const int rect_min_kb = policy_of(device).ce_rect_min_kb;
   j.rect_min_bytes = rect_min_kb < 0 ? -1 : (int64_t)rect_min_kb * 1024;
-  if (j.rect_min_bytes >= 0) {
-    // 2-D copies for pinned host memory only: the runtime stages pageable memory
-    // through buffers of its own whatever the call
+  {
+    // 2-D copies the caller did not ask for are for pinned host memory only: the runtime
+    // stages pageable memory through buffers of its own whatever the call
     hipPointerAttribute_t at{};
     if (hipPointerGetAttributes(&at, d.cpu_ptr) != hipSuccess || at.type != hipMemoryTypeHost) {
       (void)hipGetLastError();
       j.rect_min_bytes = -1;
+      j.host_pinned = false;
     }
   }
   analyze(d.gpu_block_ids, d.cpu_block_ids, d.num_blocks, d.cpu_block_stride, d.chunk_size,

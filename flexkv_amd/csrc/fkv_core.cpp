@@ -938,8 +938,15 @@ int transfer_descs(const fkv_transfer_desc *descs, int count, hipStream_t stream
   bool all_kernel = true;
   for (int i = 0; i < count; ++i) {
     engines[i] = forced_engine >= 0 ? forced_engine : descs[i].use_ce_transfer;
-    if (engines[i] == 2)
+    if (engines[i] == 2) {
+      // the model's link figures come from this device, measured once
+      int dev = 0;
+      if (hipGetDevice(&dev) == hipSuccess)
+        (void)policy_of_seeded(dev);
+      else
+        (void)hipGetLastError();
       FKV_TRY(choose_engine(descs[i], &engines[i], nullptr, nullptr));
+    }
     all_kernel = all_kernel && engines[i] == 0;
   }
   auto run_all = [&](hipStream_t on) -> int {

@@ -185,6 +185,9 @@ int launch_plan_upload(void *device_dst, const void *pinned_src, size_t bytes, h
 int probe_xcds(uint32_t *present_mask);
 // The launch policy of `device` (a copy; built on first use, see fkv_policy.cpp).
 fkv_launch_policy policy_of(int device);
+// The same with the link-dependent figures of the cost model re-based on a measurement
+// of the device (once per device, a few tens of milliseconds; see fkv_policy.cpp).
+fkv_launch_policy policy_of_seeded(int device);
 // The same without the probe: the table of a device that has none yet is the one
 // of a device of unknown shape (nothing is confined).
 fkv_launch_policy policy_peek(int device);

@@ -11,6 +11,7 @@
 // changed at run time through fkv_launch_policy_set.
 #include "fkv_internal.h"
 
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -54,6 +55,40 @@ std::map<int, DevicePolicy> &tables() {
 }
 
 int clampi(int v, int lo, int hi) { return v < lo ? lo : v > hi ? hi : v; }
+
+// The figures of the cost model that depend on the host link of the box, as compiled in
+// (an MI355X on PCIe Gen5 x16).  A table is re-based on a measurement of the device it
+// belongs to the first time the model is needed (seed_from_measurement below); a field
+// that no longer holds the compiled-in figure was set by the caller or the environment
+// and is left alone.
+struct LinkFigures {
+  int link_mbps = 57200, kernel_d2h_mbps = 57000, kernel_h2d_mbps = 57200;
+  int link_gbps_estimate = 45; // what other processes are told: 79 % of the link
+  int copy_overhead_us = 10;
+};
+constexpr LinkFigures kCompiled{};
+
+void seed_from_measurement(fkv_launch_policy &p, double d2h_gbps, double h2d_gbps,
+                           double copy_overhead_us) {
+  const bool rates_ok = d2h_gbps > 1.0 && d2h_gbps < 2000.0 && h2d_gbps > 1.0 && h2d_gbps < 2000.0;
+  if (rates_ok) {
+    const double mean = (d2h_gbps + h2d_gbps) / 2;
+    if (p.model_link_mbps == kCompiled.link_mbps)
+      p.model_link_mbps = (int)(mean * 1000 + 0.5);
+    if (p.model_kernel_d2h_mbps == kCompiled.kernel_d2h_mbps)
+      p.model_kernel_d2h_mbps = (int)(d2h_gbps * 1000 + 0.5);
+    if (p.model_kernel_h2d_mbps == kCompiled.kernel_h2d_mbps)
+      p.model_kernel_h2d_mbps = (int)(h2d_gbps * 1000 + 0.5);
+    if (p.link_gbps_estimate == kCompiled.link_gbps_estimate)
+      p.link_gbps_estimate = std::max(
+          1, (int)(mean * kCompiled.link_gbps_estimate * 1000.0 / kCompiled.link_mbps + 0.5));
+  }
+  if (copy_overhead_us > 0.05 && copy_overhead_us < 1000.0 &&
+      p.staged_copy_overhead_us == kCompiled.copy_overhead_us)
+    p.staged_copy_overhead_us = std::max(1, (int)(copy_overhead_us + 0.5));
+  if (rates_ok)
+    p.model_seeded = 1;
+}
 
 // Masks from the sorted XCD ids of the device.
 void derive_masks(fkv_launch_policy &p) {
@@ -148,7 +183,7 @@ fkv_launch_policy defaults_for(uint32_t present) {
   p.home_claims_per_wg = 2;
   p.all_claims_per_wg = 0;
   p.safety_net_wait_us = 50;
-  p.link_gbps_estimate = 45;
+  p.link_gbps_estimate = kCompiled.link_gbps_estimate;
   p.d2h_wg_per_cta = 12;
   p.h2d_wg_per_cta = 4;
   p.d2h_wg_threads = p.h2d_wg_threads = 64;
@@ -158,7 +193,7 @@ fkv_launch_policy defaults_for(uint32_t present) {
   p.lane_streams = -1;
   p.staged_restore = 1;
   p.staged_ring = 3;
-  p.staged_copy_overhead_us = 10;
+  p.staged_copy_overhead_us = kCompiled.copy_overhead_us;
   p.staged_overhead_pct = 10;
   p.staged_bridge_kb = 512;
   p.staged_max_mb = 512;
@@ -175,9 +210,9 @@ fkv_launch_policy defaults_for(uint32_t present) {
   // compaction pass stages 2.8 TB/s (512 MiB in 0.19 ms); a host scatter/gather pass
   // runs at about 20 GB/s with four threads; the gather/scatter kernel reaches
   // 57.0 GB/s GPU->host and 57.2 GB/s and more host->GPU.
-  p.model_link_mbps = 57200;
-  p.model_kernel_d2h_mbps = 57000;
-  p.model_kernel_h2d_mbps = 57200;
+  p.model_link_mbps = kCompiled.link_mbps;
+  p.model_kernel_d2h_mbps = kCompiled.kernel_d2h_mbps;
+  p.model_kernel_h2d_mbps = kCompiled.kernel_h2d_mbps;
   p.model_dma_ns = 2500;
   p.model_compaction_gbps = 2800;
   p.model_host_pass_mbps = 20000;
@@ -238,6 +273,80 @@ fkv_launch_policy policy_of(int device) {
   return t.current;
 }
 
+namespace {
+
+// Cost of one more small copy command on the copy engines: a burst of 32 one-row 2-D
+// copies of 2 KiB, host -> device, per copy, best of two bursts after a warm-up.
+double measure_copy_overhead_us() {
+  constexpr int kCopies = 32;
+  constexpr size_t kBytes = 2048;
+  void *h = nullptr, *d = nullptr;
+  hipStream_t st = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  double best = 0;
+  bool ok = hipHostMalloc(&h, kCopies * kBytes, hipHostMallocDefault) == hipSuccess &&
+            hipMalloc(&d, kCopies * kBytes) == hipSuccess &&
+            hipStreamCreateWithFlags(&st, hipStreamNonBlocking) == hipSuccess &&
+            hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess;
+  if (ok)
+    std::memset(h, 0x3c, kCopies * kBytes);
+  for (int burst = 0; ok && burst < 3; ++burst) {
+    ok = hipEventRecord(e0, st) == hipSuccess;
+    for (int i = 0; ok && i < kCopies; ++i)
+      ok = hipMemcpy2DAsync(static_cast<char *>(d) + i * kBytes, kBytes,
+                            static_cast<char *>(h) + i * kBytes, kBytes, kBytes, 1,
+                            hipMemcpyHostToDevice, st) == hipSuccess;
+    float ms = 0;
+    ok = ok && hipEventRecord(e1, st) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+         hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+    if (ok && burst > 0 && ms > 0) {
+      const double us = ms * 1e3 / kCopies;
+      best = best == 0 ? us : std::min(best, us);
+    }
+  }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  if (st) (void)hipStreamDestroy(st);
+  if (d) (void)hipFree(d);
+  if (h) (void)hipHostFree(h);
+  (void)hipGetLastError();
+  return ok ? best : 0;
+}
+
+std::mutex g_seed_mu; // one measurement at a time
+
+} // namespace
+
+fkv_launch_policy policy_of_seeded(int device) {
+  fkv_launch_policy p = policy_of(device);
+  if (!p.model_seed || p.model_seeded)
+    return p;
+  std::lock_guard<std::mutex> seeding(g_seed_mu);
+  p = policy_of(device);
+  if (!p.model_seed || p.model_seeded) // another thread was faster
+    return p;
+  double d2h = 0, h2d = 0, overhead_us = 0;
+  {
+    DeviceGuard guard(device);
+    const std::string keep = fkv_last_error(); // a failed measurement is no error of the caller
+    if (guard.ok() && fkv_measure_link_peak(device, (size_t)64 << 20, 3, 0, &d2h, nullptr) == FKV_OK &&
+        fkv_measure_link_peak(device, (size_t)64 << 20, 3, 1, &h2d, nullptr) == FKV_OK)
+      overhead_us = measure_copy_overhead_us();
+    else
+      d2h = h2d = 0;
+    clear_error();
+    if (!keep.empty())
+      (void)fail(FKV_ERR_RUNTIME, "%s", keep.c_str());
+  }
+  std::lock_guard<std::mutex> lk(g_mu);
+  DevicePolicy &t = tables()[device];
+  seed_from_measurement(t.derived, d2h, h2d, overhead_us);
+  seed_from_measurement(t.current, d2h, h2d, overhead_us);
+  if (!t.current.model_seeded) // nothing usable came out: do not try again on every call
+    t.derived.model_seed = t.current.model_seed = 0;
+  return t.current;
+}
+
 fkv_launch_policy policy_sanitized(const fkv_launch_policy &in) {
   fkv_launch_policy p = in;
   fkv_launch_policy shape = in; // keeps the caller's XCD fields: no device is asked
@@ -285,6 +394,28 @@ int fkv_launch_policy_set(int32_t device, const fkv_launch_policy *in) {
   fkv_launch_policy p = *in;
   sanitize(p, t.derived);
   t.current = p;
+  return FKV_OK;
+}
+
+int fkv_launch_policy_seed(int32_t device) {
+  using namespace fkv;
+  clear_error();
+  int dev = 0;
+  FKV_TRY(resolve(device, &dev));
+  (void)policy_of_seeded(dev);
+  return FKV_OK;
+}
+
+int fkv_launch_policy_seeded(const fkv_launch_policy *in, double d2h_gbps, double h2d_gbps,
+                             double copy_overhead_us, fkv_launch_policy *out) {
+  using namespace fkv;
+  clear_error();
+  if (!in || !out)
+    return fail(FKV_ERR_INVALID_ARG, "fkv_launch_policy_seeded: null argument");
+  fkv_launch_policy p = *in;
+  p.model_seeded = 0;
+  seed_from_measurement(p, d2h_gbps, h2d_gbps, copy_overhead_us);
+  *out = p;
   return FKV_OK;
 }
 

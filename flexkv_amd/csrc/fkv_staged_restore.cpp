@@ -268,7 +268,8 @@ int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &
   *out = StagedPlan{};
   int device = 0;
   FKV_HIP_TRY(hipGetDevice(&device));
-  const fkv_launch_policy pol = policy_of(device);
+  // the choice prices copy commands and gather passes against this device's link
+  const fkv_launch_policy pol = policy_of_seeded(device);
   if ((pol.staged_restore == 0 && pol.staged_gather == 0) || d.num_blocks <= 0 ||
       d.num_layers <= 0 || batch_layers < 1)
     return FKV_OK;

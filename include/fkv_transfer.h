@@ -752,6 +752,19 @@ int fkv_launch_policy_get(int32_t device, fkv_launch_policy *out);
 int fkv_launch_policy_set(int32_t device, const fkv_launch_policy *in);
 /* Back to the defaults derived from the device and the environment. */
 int fkv_launch_policy_reset(int32_t device);
+/* Re-bases the figures of the table that depend on the host link of the box
+ * (model_link_mbps, model_kernel_{d2h,h2d}_mbps, link_gbps_estimate, staged_copy_overhead_us)
+ * on a measurement of `device`: three pinned copies of 64 MiB per direction and a burst of
+ * small 2-D copies, once per device and process.  The library does this by itself before the
+ * first layerwise restore and the first transfer with use_ce_transfer == 2 on a device
+ * (model_seed = 0 / FKV_MODEL_SEED=0: never); fields that the caller or the environment has
+ * changed from the compiled-in figure are left alone.  The reference fixes the engine per
+ * direction by configuration (flexkv/common/config.py:770-786) and has no such model. */
+int fkv_launch_policy_seed(int32_t device);
+/* The arithmetic of the above without a device: `in` re-based on the given rates (GB/s) and
+ * cost of a copy command (us; 0 = unknown). */
+int fkv_launch_policy_seeded(const fkv_launch_policy *in, double d2h_gbps, double h2d_gbps,
+                             double copy_overhead_us, fkv_launch_policy *out);
 
 /* The arithmetic behind the staged layerwise restore, without a device (tests,
  * inspection): the runs of consecutive host block ids of a call, with the holes that are

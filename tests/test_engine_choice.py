@@ -100,3 +100,65 @@ def test_empty_transfer_and_bad_descriptor():
     d.backend = 9
     out = ctypes.c_int32()
     assert L.fkv_choose_engine(ctypes.byref(d), ctypes.byref(out), None, None) == _lib.FKV_ERR_RUNTIME
+
+
+# ---- the model's link figures follow the device --------------------------------
+
+def table_of_device_0():
+    p = _lib.LaunchPolicy()
+    _lib.check(L.fkv_launch_policy_get(0, ctypes.byref(p)))   # no GPU: the table of a device of unknown shape
+    return p
+
+
+def seeded(p, d2h, h2d, overhead_us):
+    out = _lib.LaunchPolicy()
+    _lib.check(L.fkv_launch_policy_seeded(ctypes.byref(p), d2h, h2d, overhead_us, ctypes.byref(out)))
+    return out
+
+
+def test_link_figures_are_rebased_on_a_measurement():
+    p = table_of_device_0()
+    assert (p.model_link_mbps, p.model_kernel_d2h_mbps, p.model_kernel_h2d_mbps) == (57200, 57000, 57200)
+    assert (p.link_gbps_estimate, p.staged_copy_overhead_us, p.model_seed, p.model_seeded) == (45, 10, 1, 0)
+    q = seeded(p, 28.0, 29.0, 14.2)             # a Gen4 slot, slower copy commands
+    assert (q.model_link_mbps, q.model_kernel_d2h_mbps, q.model_kernel_h2d_mbps) == (28500, 28000, 29000)
+    assert q.link_gbps_estimate == 22           # the same 79 % of the link other processes are told
+    assert (q.staged_copy_overhead_us, q.model_seeded) == (14, 1)
+    # everything that does not depend on the link is untouched
+    for f in ("model_dma_ns", "model_compaction_gbps", "model_host_pass_mbps", "model_launch_ns",
+              "model_gather_thread_mbps", "staged_overhead_pct", "gather_threads", "h2d_wg_per_cta"):
+        assert getattr(q, f) == getattr(p, f), f
+    # a figure the caller (or the environment) has set stays
+    p.model_link_mbps, p.staged_copy_overhead_us = 50000, 3
+    q = seeded(p, 28.0, 29.0, 14.2)
+    assert (q.model_link_mbps, q.staged_copy_overhead_us, q.model_kernel_h2d_mbps) == (50000, 3, 29000)
+    # a measurement that cannot be right changes nothing
+    p = table_of_device_0()
+    q = seeded(p, 0.0, 29.0, 14.2)
+    assert (q.model_link_mbps, q.model_kernel_h2d_mbps, q.model_seeded) == (57200, 57200, 0)
+    q = seeded(p, 28.0, 29.0, 0.0)              # rates without a copy-command figure
+    assert (q.model_link_mbps, q.staged_copy_overhead_us, q.model_seeded) == (28500, 10, 1)
+
+
+def test_the_engine_choice_moves_with_the_link_figure():
+    """Fixed costs (copy commands, the compaction pass) weigh half as much on a link half
+    as fast: a transfer the kernel wins by 5 % at 57 GB/s goes to the copy engine at
+    28.5 GB/s, and what the copy engine costs beyond the bytes stays the same."""
+    rng = np.random.default_rng(11)
+    ch = 65536                                   # 4 MiB host blocks: 256 copy commands of 4 MiB
+    args = (0, 32, 2, ch, (4096 * ch, ch, 2 * 4096 * ch), (ch, 2 * ch, 64 * ch),
+            rng.permutation(4096)[:256], rng.permutation(1024)[:256], True)
+    nbytes = 256 * 64 * ch
+    p = table_of_device_0()
+    try:
+        ce, tk, tc = choose(*args)
+        assert not ce and 1.03 * tk < tc < 1.08 * tk
+        extra = tc - nbytes / 57.2e6
+        half = seeded(p, 28.5, 28.6, 10.0)
+        _lib.check(L.fkv_launch_policy_set(0, ctypes.byref(half)))
+        ce2, tk2, tc2 = choose(*args)
+        assert ce2 and tc2 <= 1.03 * tk2
+        assert abs(tk2 - 2 * tk) < 0.02 * tk2
+        assert abs((tc2 - nbytes / 28.55e6) - extra) < 0.05 * extra
+    finally:
+        _lib.check(L.fkv_launch_policy_reset(0))

@@ -297,7 +297,8 @@ def test_a_put_in_another_process_confines_the_gets_of_this_one(gpu_device):
     Once the child has gone they run on all XCDs again."""
     import subprocess
     import sys
-    from flexkv_amd.c_ext import get_stats, link_activity_elsewhere, reset_stats
+    from flexkv_amd.c_ext import (get_launch_policy, get_stats, launch_policy,
+                                  link_activity_elsewhere, reset_stats)
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     if os.environ.get("FKV_LINK_BOARD_KEY"):
         pytest.skip("the board key of this process is fixed from outside")
@@ -321,27 +322,73 @@ def test_a_put_in_another_process_confines_the_gets_of_this_one(gpu_device):
         s = KVSetup(VLLM, 4, 2, 64, 64, 4096, "BLOCKFIRST", seed=44)
         dev = s.to_device(gpu_device)
         rng = np.random.default_rng(3)
-        print("link activity elsewhere (d2h, h2d):", link_activity_elsewhere(False),
-              link_activity_elsewhere(True))
-        reset_stats()
-        for _ in range(5):
-            g, c = rng.permutation(64)[:40], rng.permutation(64)[:40]
-            dev.transfer(g, c, is_h2d=True)
-            s.oracle_transfer(g, c, True)
-        st = get_stats()
-        print("launch counters next to the other process (reported, not asserted):", st)
+        # the child posts a put every millisecond or so: within a window of a second its
+        # activity is always in sight (the default window of 20 ms is a matter of timing)
+        assert link_activity_elsewhere(False, window_ms=1000)
+        split = get_launch_policy()["xcd_count"] >= 4
+        with launch_policy(arbiter=1, busy_window_ms=1000, lane_streams=0):
+            reset_stats()
+            for _ in range(5):
+                g, c = rng.permutation(64)[:40], rng.permutation(64)[:40]
+                dev.transfer(g, c, is_h2d=True)
+                s.oracle_transfer(g, c, True)
+            st = get_stats()
+        assert st["kernel_launches"] == 5 and st["confined_launches"] == (5 if split else 0), st
         dev.assert_matches_reference("gets next to another process's puts")
     finally:
         child.stdin.write("\n")
         child.stdin.close()
         assert child.wait(60) == 0
     time.sleep(0.1)
-    reset_stats()
     g = np.arange(40)
-    dev.transfer(g, g, is_h2d=True)
+    with launch_policy(arbiter=1, busy_window_ms=0, lane_streams=0):
+        reset_stats()
+        dev.transfer(g, g, is_h2d=True)
+        st = get_stats()
+    # what the child posted has ended, and nothing of this process runs the other way
+    assert st["kernel_launches"] == 1 and st["confined_launches"] == 0, st
     s.oracle_transfer(g, g, True)
-    print("launch counters afterwards (reported, not asserted):", get_stats())
     dev.assert_matches_reference("get after the other process has gone")
+
+
+def test_the_arbiter_confines_a_launch_while_the_other_direction_counts_as_busy(gpu_device):
+    """arbiter = 1, the setting production runs with: a get launched within the busy window
+    of a put on another stream confines itself to the host->GPU XCDs; with no window and
+    the put long finished it runs on all XCDs.  A long window makes the first case
+    independent of timing."""
+    import torch
+    from flexkv_amd.c_ext import get_launch_policy, get_stats, launch_policy, reset_stats
+    if get_launch_policy()["xcd_count"] < 4:
+        pytest.skip("a device with fewer than four XCDs is not split")
+    s = KVSetup(VLLM, 4, 2, 96, 96, 4096, "BLOCKFIRST", seed=47)   # 1.3 MB a transfer: below
+    dev = s.to_device(gpu_device)                                    # the home threshold
+    rng = np.random.default_rng(6)
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+
+    def move(stream, h2d):
+        g, c = rng.permutation(96)[:40], rng.permutation(96)[:40]
+        with torch.cuda.stream(stream):
+            dev.transfer(g, c, is_h2d=h2d)       # synchronous
+        s.oracle_transfer(g, c, h2d)
+
+    with launch_policy(arbiter=1, busy_window_ms=10000, lane_streams=0):
+        move(a, False)                            # a put: GPU->host counts as busy from now on
+        reset_stats()
+        for _ in range(3):
+            move(b, True)
+        st = get_stats()
+        assert st["kernel_launches"] == 3 and st["confined_launches"] == 3, st
+        reset_stats()
+        move(a, False)                            # and the gets make host->GPU busy for the puts
+        st = get_stats()
+        assert st["kernel_launches"] == 1 and st["confined_launches"] == 1, st
+    torch.cuda.synchronize()
+    with launch_policy(arbiter=1, busy_window_ms=0, lane_streams=0):
+        reset_stats()
+        move(b, True)
+        st = get_stats()
+        assert st["kernel_launches"] == 1 and st["confined_launches"] == 0, st
+    dev.assert_matches_reference("confined and unconfined launches")
 
 
 @pytest.mark.parametrize("mode", ["arbiter_off", "confined", "home", "safety_net", "claims_on_all_xcds"])
@@ -426,6 +473,26 @@ def test_the_launch_policy_follows_the_device(gpu_device):
         set_launch_policy(no_such_field=1)
     reset_launch_policy()
     assert get_launch_policy() == p
+
+
+def test_the_cost_model_is_rebased_on_this_device(gpu_device):
+    """The figures of the cost model that depend on the host link come from a
+    measurement of the device, taken once: plausible for any PCIe slot, stable across
+    calls, kept by a reset, and a figure the caller has set beforehand stays."""
+    from flexkv_amd.c_ext import (get_launch_policy, reset_launch_policy, seed_launch_policy,
+                                  set_launch_policy)
+    p = seed_launch_policy()
+    assert p["model_seeded"] == 1
+    assert 5000 < p["model_link_mbps"] < 130000, p
+    for k in ("model_kernel_d2h_mbps", "model_kernel_h2d_mbps"):
+        assert 0.8 * p["model_link_mbps"] < p[k] < 1.25 * p["model_link_mbps"], (k, p)
+    assert abs(p["link_gbps_estimate"] - p["model_link_mbps"] * 45 / 57200e0) <= 1.0
+    assert 1 <= p["staged_copy_overhead_us"] <= 200, p
+    assert seed_launch_policy() == p                  # measured once
+    set_launch_policy(model_link_mbps=12345)
+    assert seed_launch_policy()["model_link_mbps"] == 12345
+    reset_launch_policy()
+    assert get_launch_policy() == p                   # the reset keeps the measurement
 
 
 def test_lane_streams_keep_the_order_of_the_callers_stream(gpu_device):
