@@ -31,9 +31,9 @@ def workload(request, gpu_device):
 
 
 @pytest.mark.parametrize("workload,use_ce", [("c0", False), ("c0", True), ("c1", False),
-                                             ("c1", True), ("c2", False)],
+                                             ("c1", True), ("c2", False), ("c2", True)],
                          indirect=["workload"], ids=["c0-kernel", "c0-ce", "c1-kernel", "c1-ce",
-                                                     "c2-kernel"])
+                                                     "c2-kernel", "c2-ce"])
 def test_gather_erase_scatter_at_full_size(workload, use_ce):
     w = workload
     kw = dict(transfer_num_cta=4, use_ce_transfer=use_ce, ce_path_opt=True, sync=True)
@@ -58,11 +58,41 @@ def test_gather_erase_scatter_at_full_size(workload, use_ce):
         assert checksums(w) == before                     # every other block is as it was
 
 
-@pytest.mark.parametrize("workload", ["c3"], indirect=True)
-@pytest.mark.parametrize("notify", ["polling", "hostfunc"])
-def test_layerwise_restore_at_full_size(workload, notify):
-    from flexkv_amd.c_ext import LayerwiseTransferGroup
-    w = workload
+@pytest.fixture(scope="module")
+def c3(gpu_device):
+    """One c3 workload (68 GiB of engine tensors) for all its cases; the cases with
+    scattered host blocks re-make its host pool in place when they are reached."""
+    w = bench.Workload("c3", torch, gpu_device)
+    yield w
+    del w
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+# every route the library can take for a layerwise restore, forced through the launch policy
+ROUTES = {"default": {},
+          "kernel": dict(staged_restore=0, staged_gather=0),
+          "copy_per_run": dict(staged_restore=2, staged_gather=0),
+          "gathered": dict(staged_restore=0, staged_gather=2)}
+
+
+@pytest.mark.parametrize("host_ids,route,notify", [
+    ("one_run", "default", "polling"), ("one_run", "default", "hostfunc"),
+    ("one_run", "kernel", "polling"), ("one_run", "copy_per_run", "hostfunc"),
+    ("one_run", "gathered", "polling"),
+    ("scattered", "default", "polling"), ("scattered", "default", "hostfunc"),
+    ("scattered", "kernel", "polling"), ("scattered", "copy_per_run", "polling"),
+    ("scattered", "gathered", "hostfunc")])
+def test_layerwise_restore_at_full_size(c3, host_ids, route, notify):
+    """c3 (61 layers x 512 blocks of 72 KiB) out of a host pool whose 512 blocks are one
+    run, and out of a 4096-block pool with the 512 blocks scattered over it, on every
+    route: after put -> erase -> restore the checksum of every engine tensor is what it
+    was, and the counters say which route ran."""
+    from flexkv_amd.c_ext import LayerwiseTransferGroup, get_stats, launch_policy, reset_stats
+    w = c3
+    if host_ids == "scattered" and w.name == "c3":
+        w.fragment_host_pool()
+    assert (w.name == "c3f") == (host_ids == "scattered")   # the cases run in the order given
     before = checksums(w)
     w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=4, sync=True)
     assert w.verify_host_image(w.gpu_ids, w.cpu_ids)
@@ -78,13 +108,20 @@ def test_layerwise_restore_at_full_size(workload, notify):
         iouring_entries=0, iouring_flags=0,
         layer_eventfds_tensor=torch.empty(0, dtype=torch.int32), tp_size=1, is_blockfirst=True)
     e = torch.empty(0, dtype=torch.int64)
-    grp.layerwise_transfer(e, e, 0, 0, 0, 0, 0, w.gpu_ids, w.cpu_ids, w.cks, w.cls, w.cbs,
-                           w.chunk, w.cks, w.cls, w.cbs, 4, False, w.L, 1, w.kv_dim, 1,
-                           counter_id=0, kv_shared_across_ranks_mode="sharded",
-                           notify_mode=notify)
-    grp.synchronize()
+    with launch_policy(**ROUTES[route]):
+        reset_stats()
+        grp.layerwise_transfer(e, e, 0, 0, 0, 0, 0, w.gpu_ids, w.cpu_ids, w.cks, w.cls, w.cbs,
+                               w.chunk, w.cks, w.cls, w.cbs, 4, False, w.L, 1, w.kv_dim, 1,
+                               counter_id=0, kv_shared_across_ranks_mode="sharded",
+                               notify_mode=notify)
+        grp.synchronize()
+        st = get_stats()
     torch.cuda.synchronize()
     assert checksums(w) == before
+    taken = (st["staged_batches"], st["gathered_batches"])
+    want = {("one_run", "default"): (w.L, 0), ("scattered", "default"): (w.L - 1, w.L - 1),
+            "kernel": (0, 0), "copy_per_run": (w.L, 0), "gathered": (w.L - 1, w.L - 1)}
+    assert taken == want.get((host_ids, route), want.get(route)), (host_ids, route, st)
     grp.close()
 
 
