@@ -48,6 +48,8 @@ METRIC = "KV block transfer GB/s (D2H, H2D) on 1 GPU; % of measured host-link pe
 # WRITE_SIZE runs of this script scaled by plain copy kernels of known size
 # (profiles/fkv_copy_chunks_kernel_c1_pmc.md).  None where no such run was made.
 MEASURED_TRAFFIC_BYTES = {("c1", "kernel"): 8590410496, ("transform-c0", "kernel"): 8593325056}
+TRAFFIC_SOURCE = {("c1", "kernel"): "profiles/fkv_copy_chunks_kernel_c1_pmc.md",
+                  ("transform-c0", "kernel"): "profiles/fkv_copy_chunks_kernel_transform_c0.md"}
 
 
 def _median(xs):
@@ -163,6 +165,7 @@ class Workload:
         self.desc = self.desc.replace("host [512,", "host [%d," % pool_blocks) + \
             ", host block ids scattered over the pool (512 runs of one block)"
         self.host = None
+        release_cached_memory(t)
         self.host = t.empty(self.NH * self.cbs, dtype=t.uint8, pin_memory=True)
         gg = t.Generator().manual_seed(seed)
         self.cpu_ids = t.randperm(self.NH, generator=gg)[:self.num_blocks].to(t.int64)
@@ -204,6 +207,18 @@ class Workload:
                 if not t.equal(want, got):
                     return False
         return True
+
+
+def release_cached_memory(torch):
+    """Device memory and pinned host memory that torch keeps cached after a workload has
+    gone: the next configuration (and a worker process that pins a pool of its own)
+    needs the room."""
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
+    empty_host = getattr(torch._C, "_host_emptyCache", None)
+    if empty_host is not None:
+        empty_host()
 
 
 def sglang_page_ids(t, num_pages, seed, runs=64, run_len=8, isolated=512):
@@ -314,7 +329,16 @@ def run_gather_scatter(w, torch, steps, warmup, num_cta, use_ce):
     for a, b, c in marks:
         d2h_ms.append(a.elapsed_time(b))
         h2d_ms.append(b.elapsed_time(c))
-    return wall, d2h_ms, h2d_ms
+    # what a worker sees: host wall clock around one call with sync=True, per direction
+    # (the reference's own method, benchmarks/benchmark_workers.py:524-556)
+    sync_ms = {"d2h": [], "h2d": []}
+    with torch.cuda.stream(st):
+        for _ in range(min(steps, 5)):
+            for name, ids, h2d in (("d2h", w.gpu_ids, False), ("h2d", reload_ids, True)):
+                t1 = time.perf_counter()
+                w.transfer(ids, w.cpu_ids, h2d, **dict(kw, sync=True))
+                sync_ms[name].append((time.perf_counter() - t1) * 1e3)
+    return wall, d2h_ms, h2d_ms, sync_ms
 
 
 def verify_round_trip(w, torch, num_cta):
@@ -1188,7 +1212,8 @@ def measure_config(name, args, torch, device, link, steps, warmup):
     out = {"workload": f"{name}: {w.desc}", "path": path_name, "transfer_num_cta": args.num_cta,
            "blocks": w.num_blocks, "bytes_per_direction": B, "steps": steps, "warmup": warmup}
     if name in ("c0", "c1", "c2"):
-        wall, d2h_ms, h2d_ms = run_gather_scatter(w, torch, steps, warmup, args.num_cta, args.use_ce)
+        wall, d2h_ms, h2d_ms, sync_ms = run_gather_scatter(w, torch, steps, warmup, args.num_cta,
+                                                           args.use_ce)
         taken = c_ext.last_transfer_path()
         d2h = B / (sum(d2h_ms) / len(d2h_ms) * 1e-3) / 1e9
         h2d = B / (sum(h2d_ms) / len(h2d_ms) * 1e-3) / 1e9
@@ -1201,7 +1226,16 @@ def measure_config(name, args, torch, device, link, steps, warmup):
                    h2d_frac_of_link=round(h2d / link["h2d"], 4),
                    d2h_ms_median=round(_median(d2h_ms), 4), d2h_ms_min=round(min(d2h_ms), 4),
                    h2d_ms_median=round(_median(h2d_ms), 4), h2d_ms_min=round(min(h2d_ms), 4),
-                   avg_launch_ms=round(avg_ms, 4), path_taken=taken)
+                   avg_launch_ms=round(avg_ms, 4), path_taken=taken,
+                   sync_call_wall={
+                       "what": "host wall clock around one call with sync=True, %d calls per "
+                               "direction" % len(sync_ms["d2h"]),
+                       "d2h_ms_median": round(_median(sync_ms["d2h"]), 4),
+                       "d2h_ms_min": round(min(sync_ms["d2h"]), 4),
+                       "h2d_ms_median": round(_median(sync_ms["h2d"]), 4),
+                       "h2d_ms_min": round(min(sync_ms["h2d"]), 4),
+                       "d2h_GBps": round(B / (_median(sync_ms["d2h"]) * 1e-3) / 1e9, 3),
+                       "h2d_GBps": round(B / (_median(sync_ms["h2d"]) * 1e-3) / 1e9, 3)})
         if not args.no_verify:
             out["bit_exact"] = verify_round_trip(w, torch, args.num_cta)
     elif name in ("c3", "c3f"):
@@ -1229,7 +1263,7 @@ def measure_config(name, args, torch, device, link, steps, warmup):
                    bidir_link_peak_GBps=round(bidir, 3), frac_of_bidir_link=round(agg / bidir, 4),
                    frac_of_sum_of_one_way_peaks=round(agg / (link["d2h"] + link["h2d"]), 4))
     del w
-    torch.cuda.empty_cache()
+    release_cached_memory(torch)
     return out
 
 
@@ -1265,7 +1299,7 @@ def measure_layerwise(w, args, torch, device, link, steps, warmup):
     return out
 
 
-def link_roofline(rec, link, traffic=None):
+def link_roofline(rec, link, traffic=None, traffic_source=None):
     """The contract's roofline object for the dominant kernel of a c0/c1/c2 record: the
     gather/scatter kernel against the published HBM peak, and against the roof that
     actually bounds it, the host link measured in the same run."""
@@ -1274,6 +1308,8 @@ def link_roofline(rec, link, traffic=None):
     peak_link = (link["d2h"] + link["h2d"]) / 2
     return {"bound": "hbm", "achieved": round(achieved, 3), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 5), "traffic": traffic,
+            "traffic_source": (traffic_source + " (rocprofv3 --pmc runs of this script, not a "
+                               "quantity of this run)") if traffic_source else None,
             "kernel": "fkv_copy_chunks_kernel<16, false, 8, true> (GPU->host), <16, true, 8, false> (host->GPU)",
             "algorithmic_bytes_per_launch": B, "avg_launch_ms": rec["avg_launch_ms"],
             "limited_by": "host link (PCIe), not HBM: one side of every copy is host memory",
@@ -1320,8 +1356,9 @@ def main():
     ap.add_argument("--layer-spans", action="store_true",
                     help="c3: time every layer's compute with its own pair of events "
                          "(the events themselves slow the compute stream down)")
-    ap.add_argument("--other-steps", type=int, default=3,
-                    help="all: timed steps of the configurations next to the headline one")
+    ap.add_argument("--other-steps", type=int, default=10,
+                    help="all: timed steps of the configurations next to the headline one "
+                         "(3 warm-up steps each)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     args = ap.parse_args()
@@ -1479,7 +1516,9 @@ def main():
         out.update({k: v for k, v in rec.items() if k not in ("workload", "path", "transfer_num_cta",
                                                               "blocks", "bytes_per_direction")})
         if "avg_launch_ms" in rec:
-            out["roofline"] = link_roofline(rec, link, MEASURED_TRAFFIC_BYTES.get((args.config, rec["path"])))
+            key = (args.config, rec["path"])
+            out["roofline"] = link_roofline(rec, link, MEASURED_TRAFFIC_BYTES.get(key),
+                                            TRAFFIC_SOURCE.get(key))
         out["link_peak"] = link_rec
         out["config"] = {k: rec[k] for k in ("workload", "path", "transfer_num_cta", "blocks",
                                              "bytes_per_direction")}
@@ -1495,30 +1534,55 @@ def main():
     # c0, c2, c3 and c4 follow with `--other-steps` timed steps each.
     head = "c1"
     records = {head: measure_config(head, args, torch, device, link, args.steps, args.warmup)}
-    if not args.use_ce:
-        # c1 is also the configuration that is asked for on both engines: the same pages
-        # through the copy-engine strategies (the library's choice among them)
+
+    def copy_engine_record(name, steps):
+        # the same blocks through the copy-engine strategies (the library's choice among them)
         ce_args = argparse.Namespace(**{**vars(args), "use_ce": True, "no_verify": True})
-        ce = measure_config(head, ce_args, torch, device, link, min(3, args.steps), 2)  # staging buffers are allocated in the first calls
-        records[head]["copy_engine"] = {k: ce[k] for k in (
-            "d2h_GBps", "h2d_GBps", "d2h_frac_of_link", "h2d_frac_of_link", "path_taken", "steps")}
+        ce = measure_config(name, ce_args, torch, device, link, steps, 2)  # staging buffers are allocated in the first calls
+        return {k: ce[k] for k in ("d2h_GBps", "h2d_GBps", "d2h_frac_of_link", "h2d_frac_of_link",
+                                   "d2h_ms_median", "d2h_ms_min", "h2d_ms_median", "h2d_ms_min",
+                                   "path_taken", "steps")}
+    if not args.use_ce:
+        records[head]["copy_engine"] = copy_engine_record(head, min(3, args.steps))
     args.with_fragmented = True
     for name in ("c0", "c2", "c3", "c4"):
         # c4's latency percentiles want repetitions: 20 bursts of its 64 requests
         records[name] = measure_config(name, args, torch, device, link,
-                                       20 if name == "c4" else args.other_steps, 1)
+                                       20 if name == "c4" else args.other_steps,
+                                       1 if name == "c4" else 3)
+        if name in ("c0", "c2") and not args.use_ce:
+            records[name]["copy_engine"] = copy_engine_record(name, min(5, args.other_steps))
     records["c3_fragmented"] = records["c3"].pop("fragmented_record")
+    # one c0-shaped op at a time through a spawned transfer worker: submit -> completion on
+    # the submitter's wall clock, 1 warm-up + 10 rounds (benchmarks/benchmark_workers.py:524-556)
+    wk = run_worker_process(torch, device, 10, 1, args.num_cta, args.use_ce)
+    records["c0"]["through_worker"] = {
+        "what": "256-block put and get ops (536870912 B each) submitted one at a time to a "
+                "GPUCPUTransferWorker process with a 1024-block engine pool; wall clock from "
+                "submit to completion, median of 10",
+        "put": wk["D2H"], "get": wk["H2D"], "worker_exit_code": wk["exit_code"]}
     rec = records[head]
     out.update(value=rec["value"], ms_per_step=rec["ms_per_step"],
                d2h_GBps=rec["d2h_GBps"], h2d_GBps=rec["h2d_GBps"],
                d2h_frac_of_link=rec["d2h_frac_of_link"], h2d_frac_of_link=rec["h2d_frac_of_link"],
                bit_exact=all(r.get("bit_exact", True) for r in records.values()))
-    out["roofline"] = link_roofline(rec, link, MEASURED_TRAFFIC_BYTES.get((head, rec["path"])))
+    out["roofline"] = link_roofline(rec, link, MEASURED_TRAFFIC_BYTES.get((head, rec["path"])),
+                                    TRAFFIC_SOURCE.get((head, rec["path"])))
     out["config"] = {"workload": rec["workload"], "path": rec["path"],
                      "transfer_num_cta": args.num_cta, "blocks": rec["blocks"],
                      "bytes_per_direction": rec["bytes_per_direction"],
-                     "headline": "c1; c0, c2, c3, c4 under `configs`"}
+                     "headline": "c1 = configs[1] of BASELINE.json, the first configuration beyond "
+                                 "the reference's own CPU-runnable case (c0) and the one that is "
+                                 "asked for on both engines; BASELINE.json's metric names no "
+                                 "configuration.  c0, c2 (the most bytes: 10 GiB a direction), c3, "
+                                 "c3_fragmented and c4 are under `configs`, each with its own "
+                                 "steps / warmup"}
     out["link_peak"] = link_rec
+    pol = c_ext.get_launch_policy()
+    out["launch_policy"] = {k: pol[k] for k in (
+        "model_seeded", "model_link_mbps", "model_kernel_d2h_mbps", "model_kernel_h2d_mbps",
+        "link_gbps_estimate", "staged_copy_overhead_us", "staged_restore", "staged_gather",
+        "gather_threads", "xcd_count")}
     # the one launch on this path that HBM bounds: engine blocks <-> dense device buffer
     out["device_staging"] = transform_record(torch, device, args, 5, 2)["roofline"]
     if not args.no_cpu_baseline:
@@ -1554,6 +1618,7 @@ def transform_record(torch, device, args, steps, warmup):
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(("transform-" + args.shape, "kernel")),
+                     "traffic_source": TRAFFIC_SOURCE.get(("transform-" + args.shape, "kernel")),
                      "kernel": "fkv_copy_chunks_kernel<16, true, 16, false>",
                      "workload": f"transform-{args.shape}: " + r["desc"],
                      "algorithmic_bytes_per_launch": 2 * r["bytes"],

@@ -26,8 +26,7 @@ def workload(request, gpu_device):
     w = bench.Workload(request.param, torch, gpu_device)
     yield w
     del w
-    gc.collect()
-    torch.cuda.empty_cache()
+    bench.release_cached_memory(torch)   # device and pinned host memory torch keeps cached
 
 
 @pytest.mark.parametrize("workload,use_ce", [("c0", False), ("c0", True), ("c1", False),
@@ -65,8 +64,7 @@ def c3(gpu_device):
     w = bench.Workload("c3", torch, gpu_device)
     yield w
     del w
-    gc.collect()
-    torch.cuda.empty_cache()
+    bench.release_cached_memory(torch)   # device and pinned host memory torch keeps cached
 
 
 # every route the library can take for a layerwise restore, forced through the launch policy
