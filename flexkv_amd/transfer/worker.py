@@ -236,6 +236,24 @@ class TransferWorkerBase(ABC):
             except Exception as e:  # noqa: BLE001 - best effort, the process is ending
                 logger.warning("[worker %s] unregister of %s failed: %s", wid, label, e)
         self._host_registered = registered
+        self._release_engine_tensors()
+
+    def _release_engine_tensors(self) -> None:
+        """Drop the engine's tensors this process imported, and tell torch's IPC layer at
+        once: the owner of a tensor shared through torch keeps its memory (and warns when it
+        exits) until every importer has let go, which an importer that simply ends never
+        does.  The transfer groups hold addresses only and are gone or idle by now."""
+        for name in ("gpu_blocks", "gpu_blocks_ptrs", "swa_gpu_blocks", "_group_tensors"):
+            if hasattr(self, name):
+                setattr(self, name, None)
+        try:
+            import gc
+            gc.collect()
+            if torch.cuda.is_initialized():
+                torch.cuda.ipc_collect()
+        except Exception as e:  # noqa: BLE001 - best effort, the process is ending
+            logger.warning("[worker %s] releasing imported tensors failed: %s",
+                           getattr(self, "worker_id", -1), e)
 
     @staticmethod
     def _drain_device_bounded(worker_id: Any, timeout_s: float) -> bool:
@@ -506,6 +524,13 @@ class WorkerHandle:
                 self.process.join()
         try:
             self.transfer_conn.close()
+        except Exception:  # noqa: BLE001
+            pass
+        # tensors this process shared with the worker through torch: the worker has let go
+        # of them, reclaim what torch kept on their behalf
+        try:
+            if torch.cuda.is_initialized():
+                torch.cuda.ipc_collect()
         except Exception:  # noqa: BLE001
             pass
 
