@@ -21,6 +21,7 @@ from __future__ import annotations
 
 import ctypes
 import logging
+import weakref
 from typing import Any, Callable, Optional, Tuple, Union
 
 import torch
@@ -178,6 +179,45 @@ class TensorSharedHandle:
         return state
 
 
+def discard_tensor_handles(handles) -> None:
+    """Let go of handles this process received and will not use (a rejected request).  The
+    owner of a tensor shared through torch keeps its memory until every handle it sent has
+    been opened and dropped by a receiver; a handle that is just forgotten holds that
+    memory until the owner exits.  Accepts nested lists."""
+    for h in handles or ():
+        if isinstance(h, (list, tuple)):
+            discard_tensor_handles(h)
+        elif isinstance(h, TensorSharedHandle) and not h.use_direct_ipc:
+            try:
+                t = h.get_tensor()
+                del t
+            except Exception as e:  # noqa: BLE001 - nothing more can be done for it
+                logger.warning("could not open a shared tensor to release it: %s", e)
+    try:
+        if torch.cuda.is_initialized():
+            torch.cuda.ipc_collect()
+    except Exception:  # noqa: BLE001
+        pass
+
+
+# handle object -> weak reference to the tensor this process made of it
+_OPENED: "weakref.WeakKeyDictionary[TensorSharedHandle, weakref.ref]" = weakref.WeakKeyDictionary()
+
+
+def _tensor_of(h: "TensorSharedHandle") -> torch.Tensor:
+    """One tensor per handle object and process while that tensor is alive.  A worker for a
+    model with layer groups is handed the first group's handles twice (as ``gpu_blocks`` and
+    inside ``gpu_blocks_per_group``, ``flexkv/transfer/worker.py:850-870``); a handle made by
+    torch's own sharing counts one receiver, and opening it twice leaves the owner's
+    count off by one for good."""
+    ref = _OPENED.get(h)
+    t = ref() if ref is not None else None
+    if t is None:
+        t = h.get_tensor()
+        _OPENED[h] = weakref.ref(t)
+    return t
+
+
 def import_tensor_handles(handles) -> list:
     """Tensors of a list of handles, after switching to their device
     (``flexkv/transfer/worker.py:70-76``)."""
@@ -185,4 +225,4 @@ def import_tensor_handles(handles) -> list:
         dev = handles[0].device
         if isinstance(dev, torch.device) and dev.type == "cuda":
             torch.cuda.set_device(0 if dev.index is None else dev.index)
-    return [h.get_tensor() if isinstance(h, TensorSharedHandle) else h for h in handles]
+    return [_tensor_of(h) if isinstance(h, TensorSharedHandle) else h for h in handles]

@@ -46,7 +46,7 @@ from ..layout import (KVCacheLayout, KVCacheLayoutType, LayerGroupSpec, MultiGro
                       multi_group_tables)
 from . import trace
 from .env import global_env
-from .memory_handle import TensorSharedHandle, import_tensor_handles
+from .memory_handle import TensorSharedHandle, discard_tensor_handles, import_tensor_handles
 from .ops import (LayerwiseTransferOp, TransferOp, TransferType, WorkerLayerwiseTransferOp,
                   WorkerTransferOp, WorkerTransferResult)
 
@@ -744,8 +744,10 @@ class GPUCPUTransferWorker(TransferWorkerBase):
     def _control_resume_gpu(self, gpu_blocks: List[Any]) -> int:
         """New KV tensors of the same count and shape (worker.py:948-962)."""
         if self.gpu_blocks:
+            discard_tensor_handles(gpu_blocks)
             raise RuntimeError("GPU blocks are already registered")
         if len(gpu_blocks) != self._gpu_block_count:
+            discard_tensor_handles(gpu_blocks)
             raise ValueError(f"Expected {self._gpu_block_count} GPU blocks, got {len(gpu_blocks)}")
         self._gpu_handles = list(gpu_blocks)
         self.gpu_blocks = import_tensor_handles(gpu_blocks)
@@ -947,9 +949,11 @@ class tpGPUCPUTransferWorker(TransferWorkerBase):  # noqa: N801 - the reference'
     def _control_resume_gpu(self, gpu_blocks: List[List[Any]]) -> int:
         """New KV tensors for every rank, as many as before (worker.py:1408-1430)."""
         if self.gpu_blocks:
+            discard_tensor_handles(gpu_blocks)
             raise RuntimeError("GPU blocks are already registered")
         counts = [len(h) for h in gpu_blocks]
         if counts != self._gpu_block_counts:
+            discard_tensor_handles(gpu_blocks)
             raise ValueError(f"Expected GPU block counts {self._gpu_block_counts}, got {counts}")
         self._gpu_handles = [list(h) for h in gpu_blocks]
         imported = [import_tensor_handles(h) for h in gpu_blocks]

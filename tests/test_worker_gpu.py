@@ -298,12 +298,14 @@ def test_suspend_and_resume_gpu_blocks(gpu_device, engine, direct_ipc):
     assert _collect(q, 1) == [(lost.op_id, False, None)]
     del first
     second = [torch.zeros_like(t) for t in want]
-    fresh = [TensorSharedHandle(t, force_direct_ipc=direct_ipc) for t in second]
+    # a handle made by torch's own sharing is good for one receiver: new ones for every send
+    # (the worker opens and drops the ones it rejects, so that this process gets them back)
+    fresh = lambda ts: [TensorSharedHandle(t, force_direct_ipc=direct_ipc) for t in ts]  # noqa: E731
     with pytest.raises(RuntimeError, match="Expected 4 GPU blocks"):
-        h.control("resume_gpu", fresh[:2])
-    assert h.control("resume_gpu", fresh) == L
+        h.control("resume_gpu", fresh(second[:2]))
+    assert h.control("resume_gpu", fresh(second)) == L
     with pytest.raises(RuntimeError, match="already registered"):
-        h.control("resume_gpu", fresh)
+        h.control("resume_gpu", fresh(second))
     get = _op(TransferType.H2D, mid, back, pool)
     h.submit_transfer(get)
     assert _collect(q, 1) == [(get.op_id, True, None)]
