@@ -686,7 +686,8 @@ def run_notify_scales(torch, device, num_cta, iters=20, warmup=3):
 # CPU baseline: the reference's CPU path (torch index-gather into the host
 # cache layout), timed on this machine's host cores on a bounded sample.
 # ---------------------------------------------------------------------------
-def run_multi_group(torch, device, steps, warmup, num_cta, notify, use_ce, verify=True):
+def run_multi_group(torch, device, steps, warmup, num_cta, notify, use_ce, verify=True,
+                    fragmented=False):
     """Layer groups of different shape restored layer by layer, one notification per
     original layer: members of every group attached to the layer, then its sidecar."""
     from flexkv_amd.c_ext import LayerwiseTransferGroup
@@ -695,6 +696,8 @@ def run_multi_group(torch, device, steps, warmup, num_cta, notify, use_ce, verif
     t = torch
     L, page, n_gpu, n_cpu, nblk = 61, 256, 2048, 512, 512
     swa_tok, swa_width, swa_gpu, swa_cpu, nswa = 128, 1152, 256, 64, 64
+    if fragmented:   # host pools after churn: the blocks to restore are scattered over them
+        n_cpu, swa_cpu = 4096, 512
     c4_layers = tuple(l for l in range(L) if l % 2 == 1)            # 30 layers, ratio 4
     c128_layers = tuple(l for l in range(L) if l % 2 == 0)          # 31 layers, ratio 128
     groups = [LayerGroupSpec(len(c4_layers), 1, 576, c4_layers, 2, 4),
@@ -1351,6 +1354,9 @@ def main():
     ap.add_argument("--gather-threads", type=int, default=None,
                     help="c3 / c3f: host threads that gather (default 6)")
     ap.add_argument("--gather-first-by-kernel", type=int, default=None, choices=[0, 1])
+    ap.add_argument("--fragmented", action="store_true",
+                    help="mg: host pools of 4096 / 512 blocks with the blocks to restore scattered "
+                         "over them (default: pools of 512 / 64 blocks, all of them restored)")
     ap.add_argument("--overlap-directions", action="store_true",
                     help="worker: the worker runs gets next to puts (second thread and stream)")
     ap.add_argument("--layer-spans", action="store_true",
@@ -1460,8 +1466,10 @@ def main():
         return
     if args.config == "mg":
         link = measure_link()
+        c_ext.reset_stats()
         r = run_multi_group(torch, device, args.steps, args.warmup, args.num_cta, args.notify,
-                            args.use_ce, verify=not args.no_verify)
+                            args.use_ce, verify=not args.no_verify, fragmented=args.fragmented)
+        st = c_ext.get_stats()
         rate = r["bytes"] / (r["device_ms"] * 1e-3) / 1e9
         print(json.dumps({
             "metric": "multi-group layerwise restore GB/s (H2D) on 1 GPU", "unit": "GB/s",
@@ -1474,6 +1482,11 @@ def main():
             "restore_device_ms": round(r["device_ms"], 3),
             "bytes": r["bytes"], "main_bytes": r["main_bytes"], "sidecar_bytes": r["swa_bytes"],
             "copies_per_restore": r["copies_per_restore"],
+            "host_blocks": "scattered over pools of 4096 / 512 blocks" if args.fragmented
+                           else "all blocks of pools of 512 / 64 blocks (one run each)",
+            "batches_through_copy_engines": st["staged_batches"],
+            "batches_gathered_by_host_threads": st["gathered_batches"],
+            "host_gather_thread_ms": round(st["gather_busy_us"] / 1e3, 3),
             "ms_per_original_layer": round(r["device_ms"] / r["layers"], 4),
             "h2d_frac_of_link": round(rate / link["h2d"], 4), "bit_exact": r["bit_exact"],
             "link_peak": {"h2d_GBps": round(link["h2d"], 3)}}))

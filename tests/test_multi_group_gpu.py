@@ -20,13 +20,20 @@ pytestmark = pytest.mark.gpu
 ENGINES = [False, True, "auto"]
 
 
-@pytest.fixture(autouse=True, params=[1, 2], ids=["restore_as_chosen", "restore_by_copy_engines"])
+@pytest.fixture(autouse=True, params=[
+    dict(staged_restore=1, staged_gather=1), dict(staged_restore=2, staged_gather=0),
+    dict(staged_restore=0, staged_gather=2, gather_first_by_kernel=0, gather_threads=3, gather_ring=2),
+    dict(staged_restore=0, staged_gather=2, gather_first_by_kernel=1, gather_threads=2)],
+    ids=["restore_as_chosen", "restore_by_copy_engines", "restore_gathered",
+         "restore_gathered_first_by_kernel"])
 def _staged_restore(request):
-    """Every case twice: with the library's own choice between the kernel path and
-    the copy engines (the small pools here stay on the kernel path), and with the
-    kernel-path restores forced through the copy engines and a staging ring."""
+    """Every case four times: with the library's own choice of route (the small pools here
+    stay on the kernel path), with the kernel-path restores forced through the copy engines
+    and a staging ring one copy per run of host blocks, and with the rows of every group
+    member and sidecar gathered by host threads first (batches launched one by one from the
+    library's own thread; with and without the first batch by kernel)."""
     from flexkv_amd.c_ext import launch_policy
-    with launch_policy(staged_restore=request.param):
+    with launch_policy(**request.param):
         yield
 
 
@@ -286,8 +293,19 @@ def test_random_pools_match_the_oracle(gpu_device, engine, seed, nblk, nswa):
     immediate, work = O.layerwise_multi_group(1, case.oracle_groups(), case.members, case.host,
                                               gpu_ids, cpu_ids, 1, 1, "sharded", swa)
     assert immediate == ([6] if not nswa else [])
+    from flexkv_amd.c_ext import get_launch_policy, get_stats, reset_stats
+    reset_stats()
     dev.run_h2d(cpu_ids=cpu_ids, gpu_ids=gpu_ids, swa=(swa_c, swa_g) if nswa else None,
                 use_ce_transfer=engine)
+    pol, st = get_launch_policy(), get_stats()
+    if engine is False and pol["staged_gather"] == 2 and pol["staged_restore"] == 0:
+        # every group member and sidecar of every layer with work had its rows gathered
+        # (less the first batch where that one goes by kernel)
+        members = sum(len(m) for m in case.members) * (nblk > 0) + 7 * (nswa > 0)
+        first = 0
+        if pol["gather_first_by_kernel"]:
+            first = len(case.members[0]) * (nblk > 0) + (nswa > 0)
+        assert st["gathered_batches"] == members - first, (st, members, first)
     for gi, grp in enumerate(case.gpu):
         for local, ref in enumerate(grp):
             assert np.array_equal(dev.gpu[gi][local].cpu().numpy(), ref), (gi, local)
