@@ -422,7 +422,12 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, bool direct,
   using namespace fkv;
   DeviceGuard restore(-1);
   const int num_batches = (int)g->batches.size();
+  const int give_up_at = policy_of(g->device_ids[0]).test_fail_restore_batch; // tests only
   for (int b = 0; b < num_batches && rc == FKV_OK; ++b) {
+    if (give_up_at > 0 && b == give_up_at - 1) {
+      rc = fail(FKV_ERR_RUNTIME, "layerwise restore made to give up before batch %d (test_fail_restore_batch)", b);
+      break;
+    }
     fkv_layerwise::Batch &batch = *g->batches[b];
     for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
       (void)hipSetDevice(g->device_ids[i]);

@@ -166,6 +166,7 @@ void sanitize(fkv_launch_policy &p, const fkv_launch_policy &derived) {
   p.model_gather_thread_mbps = clampi(p.model_gather_thread_mbps, 100, 10000000);
   p.model_seed = p.model_seed != 0;
   p.model_seeded = derived.model_seeded;
+  p.test_fail_restore_batch = clampi(p.test_fail_restore_batch, 0, 1 << 20);
 }
 
 // The table of a device with the XCDs `present`, environment applied.

@@ -172,6 +172,80 @@ def test_gathered_restore_announces_layers_in_order_and_serves_waiting_streams(g
         os.close(fd)
 
 
+@pytest.mark.parametrize("notify", ["polling", "hostfunc"])
+@pytest.mark.parametrize("route", ["gathered", "kernel"])
+def test_a_restore_that_gives_up_part_way_is_reported_and_the_group_stays_usable(gpu_device, route,
+                                                                                notify):
+    """The launch of a restore can fail part-way (here the launch policy makes it give up
+    before its fourth batch; nothing faults).  The layers enqueued before that land and are
+    announced, the others are not; whoever waits for one of them is told instead of waiting
+    for good; the failure is reported by the call (when it happens inside the call) or by
+    synchronize and the waiters (when the library's own thread launches the restore); and
+    the next restore through the same group gives the oracle's bytes."""
+    import os
+    import select
+    from flexkv_amd.c_ext import LayerwiseTransferGroup, launch_policy
+    L, NG, NC, n, chunk = 7, 96, 120, 50, 9216
+    s = KVSetup(VLLM, L, 1, NG, NC, chunk, "BLOCKFIRST", seed=52)
+    dev = s.to_device(gpu_device)
+    fds = [os.eventfd(0, os.EFD_SEMAPHORE | os.EFD_NONBLOCK) for _ in range(L)]
+    i64 = lambda v: torch.tensor([v], dtype=torch.int64)
+    grp = LayerwiseTransferGroup(
+        num_gpus=1, gpu_blocks=[dev.gpu], cpu_blocks=dev.host, ssd_files={}, num_layers=L,
+        gpu_kv_strides_tensor=i64(s.gpu_kv_stride), gpu_block_strides_tensor=i64(s.gpu_block_stride),
+        gpu_layer_strides_tensor=i64(s.gpu_layer_stride), gpu_chunk_sizes_tensor=i64(s.chunk),
+        iouring_entries=0, iouring_flags=0,
+        layer_eventfds_tensor=torch.tensor(fds, dtype=torch.int32), tp_size=1, is_blockfirst=True)
+    rng = np.random.default_rng(13)
+    gids = rng.permutation(NG)[:n].astype(np.int64)
+    cids = rng.permutation(NC)[:n].astype(np.int64)
+    e = torch.empty(0, dtype=torch.int64)
+
+    def call():
+        grp.layerwise_transfer(
+            e, e, 0, 0, 0, 0, 0, torch.from_numpy(gids), torch.from_numpy(cids), s.cpu_kv_stride,
+            s.cpu_layer_stride, s.cpu_block_stride, s.chunk, s.cpu_kv_stride, s.cpu_layer_stride,
+            s.cpu_block_stride, 4, False, L, 1, 1, 1, counter_id=0,
+            kv_shared_across_ranks_mode="sharded", notify_mode=notify)
+
+    forced = dict(ROUTES[route], gather_first_by_kernel=0) if route == "gathered" else ROUTES[route]
+    in_the_call = route == "kernel" or notify == "hostfunc"
+    with launch_policy(test_fail_restore_batch=4, **forced):
+        if in_the_call:
+            with pytest.raises(RuntimeError, match="give up before batch 3"):
+                call()
+        else:
+            call()                                  # returns while the restore is being launched
+            comp = torch.cuda.Stream()
+            for l in range(3):
+                grp.wait_layer(l, comp)             # these land
+            with pytest.raises(RuntimeError, match="will not land"):
+                grp.wait_layer(3, comp)
+            with pytest.raises(RuntimeError, match="give up before batch 3"):
+                grp.synchronize()
+        torch.cuda.synchronize()
+    announced = [bool(select.select([fd], [], [], 0.5 if l < 3 else 0)[0]) for l, fd in enumerate(fds)]
+    if route == "gathered":                         # announced as they landed, in order
+        assert announced == [True] * 3 + [False] * 4, announced
+    else:                                           # a call that fails on its own thread announces nothing
+        assert announced == [False] * L, announced
+    for l, fd in enumerate(fds):
+        if announced[l]:
+            assert os.eventfd_read(fd) == 1
+    # the layers before the failure are where the oracle puts them; then a whole restore
+    s.oracle_transfer(gids, cids, True, num_layers=3)
+    dev.assert_matches_reference("layers enqueued before the restore gave up")
+    with launch_policy(**forced):
+        call()
+        grp.synchronize()
+    s.oracle_transfer(gids, cids, True)
+    dev.assert_matches_reference("the next restore through the same group")
+    for fd in fds:
+        assert os.eventfd_read(fd) == 1
+        os.close(fd)
+    grp.close()
+
+
 def test_the_choice_follows_the_runs_of_host_blocks(gpu_device):
     """With the default policy a restore whose host blocks form one run goes through
     the copy engines with one copy command, one whose host blocks are scattered has its
