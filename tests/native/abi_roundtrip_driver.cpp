@@ -280,6 +280,58 @@ int main() {
         }
         ++cases;
       }
+    // the same restore on every route the library has, forced through the launch policy:
+    // kernel, one copy-engine command per run of host blocks, rows gathered by host threads
+    // (batches launched one by one from the library's own thread), the latter also with
+    // the cost model re-based on this device first
+    fkv_launch_policy saved, pol;
+    FKV_OK_OR_DIE(fkv_launch_policy_seed(-1));
+    FKV_OK_OR_DIE(fkv_launch_policy_get(-1, &saved));
+    if (!saved.model_seeded || saved.model_link_mbps < 1000 || saved.staged_copy_overhead_us < 1) {
+      fprintf(stderr, "launch policy: the cost model was not re-based on the device\n");
+      return 1;
+    }
+    const int routes[3][2] = {{0, 0}, {2, 0}, {0, 2}}; // staged_restore, staged_gather
+    for (int route = 0; route < 3; ++route)
+      for (int notify = 0; notify < 2; ++notify) {
+        pol = saved;
+        pol.staged_restore = routes[route][0], pol.staged_gather = routes[route][1];
+        pol.gather_threads = 3, pol.gather_ring = 2, pol.gather_first_by_kernel = notify;
+        FKV_OK_OR_DIE(fkv_launch_policy_set(-1, &pol));
+        fkv_stats before, after;
+        fkv_get_stats(&before);
+        std::vector<int64_t> g = pick(rng, N, 29), c = pick(rng, NH, 29);
+        std::vector<int64_t> g_arg = g, c_arg = c;
+        FKV_OK_OR_DIE(fkv_layerwise_transfer(lw, g_arg.data(), c_arg.data(), 29, CBS, CKS, CLS, CBS, 4,
+                                             0, L, 1, KV, 8, notify, "sharded", notify, 0));
+        // the lists belong to the caller again as soon as the call returns
+        std::fill(g_arg.begin(), g_arg.end(), 0);
+        std::fill(c_arg.begin(), c_arg.end(), 0);
+        FKV_OK_OR_DIE(fkv_layerwise_synchronize(lw));
+        fkv_get_stats(&after);
+        m.put(g, c, true);
+        if (check("layerwise restore, forced route"))
+          return 1;
+        const uint64_t staged = after.staged_batches - before.staged_batches;
+        const uint64_t gathered = after.gathered_batches - before.gathered_batches;
+        const uint64_t want_staged = route == 0 ? 0 : route == 2 && notify ? L - 1 : L;
+        const uint64_t want_gathered = route == 2 ? want_staged : 0;
+        if (staged != want_staged || gathered != want_gathered) {
+          fprintf(stderr, "route %d: %llu staged and %llu gathered batches, expected %llu and %llu\n",
+                  route, (unsigned long long)staged, (unsigned long long)gathered,
+                  (unsigned long long)want_staged, (unsigned long long)want_gathered);
+          return 1;
+        }
+        for (int l = 0; l < L; ++l) {
+          uint64_t v = 0;
+          if (read(fds[notify * L + l], &v, 8) != 8 || v != 1) {
+            fprintf(stderr, "route %d: layer %d was not announced\n", route, l);
+            return 1;
+          }
+        }
+      }
+    FKV_OK_OR_DIE(fkv_launch_policy_reset(-1));
+    ++cases;
     fkv_layerwise_destroy(lw);
     for (int fd : fds)
       close(fd);
