@@ -1354,6 +1354,9 @@ def main():
     ap.add_argument("--gather-threads", type=int, default=None,
                     help="c3 / c3f: host threads that gather (default 6)")
     ap.add_argument("--gather-first-by-kernel", type=int, default=None, choices=[0, 1])
+    ap.add_argument("--policy", action="append", default=[], metavar="FIELD=VALUE",
+                    help="set a field of the launch policy (fkv_launch_policy) before the run; "
+                         "may be given several times")
     ap.add_argument("--fragmented", action="store_true",
                     help="mg: host pools of 4096 / 512 blocks with the blocks to restore scattered "
                          "over them (default: pools of 512 / 64 blocks, all of them restored)")
@@ -1393,6 +1396,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     device = "cuda:0"
     torch.cuda.set_device(0)
+    for item in args.policy:
+        field, _, value = item.partition("=")
+        c_ext.set_launch_policy(**{field.strip(): int(value, 0)})
     if args.staged_restore is not None:
         c_ext.set_launch_policy(staged_restore=args.staged_restore)
     if args.staged_gather is not None:

@@ -207,7 +207,8 @@ class LaunchPolicy(Structure):
                 ("staged_gather", c_int32), ("gather_threads", c_int32), ("gather_ring", c_int32),
                 ("gather_first_by_kernel", c_int32), ("model_gather_thread_mbps", c_int32),
                 ("model_seed", c_int32), ("model_seeded", c_int32),
-                ("test_fail_restore_batch", c_int32), ("reserved", c_int32 * 4)]
+                ("staged_scatter_threads", c_int32), ("test_fail_restore_batch", c_int32),
+                ("reserved", c_int32 * 3)]
 
 
 # name -> (restype, argtypes); the complete export list of include/fkv_transfer.h

@@ -166,6 +166,7 @@ void sanitize(fkv_launch_policy &p, const fkv_launch_policy &derived) {
   p.model_gather_thread_mbps = clampi(p.model_gather_thread_mbps, 100, 10000000);
   p.model_seed = p.model_seed != 0;
   p.model_seeded = derived.model_seeded;
+  p.staged_scatter_threads = clampi(p.staged_scatter_threads, 64, kCopyBlockThreads);
   p.test_fail_restore_batch = clampi(p.test_fail_restore_batch, 0, 1 << 20);
 }
 
@@ -233,6 +234,7 @@ fkv_launch_policy defaults_for(uint32_t present) {
   p.model_gather_thread_mbps = 20000;
   p.model_seed = 1;
   p.model_seeded = 0;
+  p.staged_scatter_threads = 256;
   for (const EnvField &f : kEnv) {
     const char *v = std::getenv(f.name);
     if (v && *v) // decimal, 0x.. or 0.. as written

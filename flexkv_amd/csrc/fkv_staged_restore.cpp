@@ -379,7 +379,10 @@ int staged_scatter(const StagedPlan &sp, StagedRing &ring, const KernelPlan &kp,
   a.xcd_mask = 0;
   const fkv_launch_policy pol = policy_of(kp.device);
   a.unroll = pol.hbm_unroll;
-  FKV_TRY(launch_copy_kernel(a, pol.hbm_workgroups, pol.hbm_wg_threads, scatter_stream));
+  // Small workgroups: the launch is short (one 8 KiB slice per wavefront for a 36 MiB batch)
+  // and runs next to the engine's kernels, where a workgroup of 1024 lanes waits for a CU
+  // with room for all of it.
+  FKV_TRY(launch_copy_kernel(a, pol.hbm_workgroups, pol.staged_scatter_threads, scatter_stream));
   FKV_HIP_TRY(hipEventRecord(ring.freed[k], scatter_stream));
   ring.used[k] = true;
   stats().staged_batches.fetch_add(1, std::memory_order_relaxed);

@@ -743,10 +743,15 @@ typedef struct fkv_launch_policy {
                                  and scales the link-bound rates above by measured / compiled-in;
                                  0 keeps the compiled-in figures */
   int32_t model_seeded;       /* read-only: 1 once the rates of this table come from a measurement */
+  int32_t staged_scatter_threads; /* lanes per workgroup of the launch that places a staged batch
+                                 (staging buffer -> engine blocks); default 256: next to the
+                                 engine's own kernels a workgroup of 256 lanes finds room on a
+                                 CU where one of 1024 waits (36 MiB: 26 us against 146 us at the
+                                 median next to fused attention, 17 us against 21 us alone) */
   int32_t test_fail_restore_batch; /* tests: n > 0 makes a layerwise restore give up before it
                                  enqueues its n-th batch, as a failed launch would (nothing faults:
                                  the batches before it run and are announced, the rest never lands) */
-  int32_t reserved[4];
+  int32_t reserved[3];
 } fkv_launch_policy;
 /* The table of `device` (-1 = current).  The first call for a device runs the probe kernel. */
 int fkv_launch_policy_get(int32_t device, fkv_launch_policy *out);
