@@ -5,6 +5,7 @@
 #include <chrono>
 #include <condition_variable>
 #include <cstring>
+#include <exception>
 #include <functional>
 #include <memory>
 #include <mutex>
@@ -80,8 +81,15 @@ __attribute__((target("avx2"))) void copy_avx2(uint8_t *dst, const uint8_t *src,
 struct HostCrew::Impl {
   explicit Impl(int helpers) {
     ranges.resize(helpers);
-    for (int i = 0; i < helpers; ++i)
-      threads.emplace_back([this, i] { loop(i); });
+    threads.reserve(helpers);
+    for (int i = 0; i < helpers; ++i) {
+      try {
+        threads.emplace_back([this, i] { loop(i); });
+      } catch (const std::exception &) { // the system has no more threads: work with those there are
+        break;
+      }
+    }
+    ranges.resize(threads.size());
   }
   ~Impl() {
     {

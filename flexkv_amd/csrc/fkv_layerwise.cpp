@@ -33,6 +33,7 @@
 // waits until that event has been recorded.
 //
 // The transfer streams keep the default priority.
+#include "fkv_gate.h"
 #include "fkv_host_copy.h"
 #include "fkv_internal.h"
 #include "fkv_poll.h"
@@ -172,11 +173,8 @@ struct fkv_layerwise {
   std::unique_ptr<fkv::HostCrew> crew;
   std::thread feeder;
   std::vector<Lane> feed_lanes; // what the feeder works on
-  std::mutex feed_mu;
-  std::condition_variable feed_cv;
-  std::atomic<int> recorded{0};  // batches whose events have been recorded (written under feed_mu)
-  bool feed_failed = false;      // the launching thread gave up; the batches from `recorded` on never land
-  int feed_rc = 0;
+  fkv::BatchGate gate;          // which batches have had their events recorded, or never will
+  int feed_rc = 0;              // why the launching thread gave up (read once it has been joined)
   std::string feed_error;
   fkv_ce_config ce{};
 
@@ -224,11 +222,9 @@ struct fkv_layerwise {
         batches.size(), num_gpus, (int)hipSuccess, (int)hipErrorNotReady,
         [this](size_t b, int g) {
           // an event that has not been recorded yet reads as complete
-          if ((int)b >= recorded.load(std::memory_order_acquire)) {
-            std::lock_guard<std::mutex> lk(feed_mu);
-            if ((int)b >= recorded.load(std::memory_order_relaxed))
-              return (int)(feed_failed ? hipErrorLaunchFailure : hipErrorNotReady);
-          }
+          const int state = gate.peek((int)b);
+          if (state <= 0)
+            return (int)(state < 0 ? hipErrorLaunchFailure : hipErrorNotReady);
           (void)hipSetDevice(device_ids[g]);
           const hipError_t e = hipEventQuery(batches[b]->done[g]);
           if (e != hipSuccess)
@@ -244,21 +240,6 @@ struct fkv_layerwise {
     }
   }
 
-  void publish_recorded(int n) {
-    {
-      std::lock_guard<std::mutex> lk(feed_mu);
-      recorded.store(n, std::memory_order_release);
-    }
-    feed_cv.notify_all();
-  }
-  // Blocks until the event of batch `b` has been recorded; false when it never will be.
-  bool wait_recorded(int b) {
-    if (b < recorded.load(std::memory_order_acquire))
-      return true;
-    std::unique_lock<std::mutex> lk(feed_mu);
-    feed_cv.wait(lk, [&] { return feed_failed || b < recorded.load(std::memory_order_relaxed); });
-    return b < recorded.load(std::memory_order_relaxed);
-  }
   // The launching thread ends by itself: it waits for nothing but copies that are
   // already enqueued.
   void join_feeder() {
@@ -293,8 +274,8 @@ struct fkv_layerwise {
   // The error of the previous restore, if any, as a status of the current call.
   int take_restore_error(const char *where) {
     const int e = restore_error.exchange(0);
-    if (feed_failed) { // only read after the launching thread has been joined
-      feed_failed = false;
+    if (gate.failed()) { // the launching thread has been joined
+      gate.clear_failure();
       return fkv::fail(feed_rc ? feed_rc : FKV_ERR_RUNTIME,
                        "%s: the previous layerwise restore failed while it was launched: %s", where,
                        feed_error.c_str());
@@ -486,7 +467,7 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, bool direct,
       }
     }
     if (rc == FKV_OK)
-      g->publish_recorded(b + 1);
+      g->gate.publish(b + 1);
   }
   std::string saved_error = fkv_last_error();
   for (Lane &lane : lanes)
@@ -680,7 +661,7 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
 
   g->retire_previous();
   FKV_TRY(g->take_restore_error("fkv_layerwise_transfer"));
-  g->recorded.store(0, std::memory_order_relaxed);
+  g->gate.reset();
   g->feed_lanes.clear();
   g->counter_id = c.counter_id;
   Range range("fkv layerwise%s H2D %d blocks, %d sidecar blocks", g->multi_group ? " multi-group" : "",
@@ -885,21 +866,27 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
       gathered = gathered || (sp.usable && sp.route == kRouteGathered);
   if (rc == FKV_OK && gathered) {
     const int helpers = gather_threads_of(policy_of(g->device_ids[0])) - 1;
-    if (!g->crew || g->crew->helpers() != helpers)
-      g->crew = std::make_unique<HostCrew>(helpers);
-    g->feed_lanes = std::move(lanes);
-    g->feeder = std::thread([g] {
-      const int frc = launch_batches(g, g->feed_lanes, true, nullptr, true, FKV_OK);
-      {
-        std::lock_guard<std::mutex> lk(g->feed_mu);
-        if (frc != FKV_OK) {
-          g->feed_failed = true;
-          g->feed_rc = frc;
-          g->feed_error = fkv_last_error();
-        }
+    if (!g->crew || g->crew->helpers() != helpers) {
+      try {
+        g->crew = std::make_unique<HostCrew>(helpers);
+      } catch (const std::exception &) { // no threads to be had: the launching thread gathers alone
+        g->crew = std::make_unique<HostCrew>(0);
       }
-      g->feed_cv.notify_all();
-    });
+    }
+    g->feed_lanes = std::move(lanes);
+    auto feed = [g] {
+      const int frc = launch_batches(g, g->feed_lanes, true, nullptr, true, FKV_OK);
+      if (frc != FKV_OK) {
+        g->feed_rc = frc; // read by others only after they have joined this thread
+        g->feed_error = fkv_last_error();
+        g->gate.fail();
+      }
+    };
+    try {
+      g->feeder = std::thread(feed);
+    } catch (const std::exception &) {
+      feed(); // no thread to be had: the same work on the calling thread, which then blocks for it
+    }
   } else {
     const int lrc = launch_batches(g, lanes, direct, &c, false, rc);
     if (lrc != FKV_OK) {
@@ -910,7 +897,7 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
   // The launching thread gave up: nothing of the call is announced from here on.
   auto launch_failure = [&]() {
     g->join_feeder();
-    g->feed_failed = false;
+    g->gate.clear_failure();
     (void)hipSetDevice(restore.device());
     return fail(g->feed_rc ? g->feed_rc : FKV_ERR_RUNTIME, "%s", g->feed_error.c_str());
   };
@@ -924,7 +911,7 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
   } else {
     // announce every batch as soon as all GPUs have finished it, in order
     for (int b = 0; b < num_batches; ++b) {
-      if (!g->wait_recorded(b))
+      if (!g->gate.wait(b))
         return launch_failure();
       for (int i = 0; i < g->num_gpus; ++i) {
         (void)hipSetDevice(g->device_ids[i]);
@@ -1029,7 +1016,7 @@ int fkv_layerwise_wait_layer(fkv_layerwise *g, int32_t gpu_index, int32_t layer,
   }
   // A batch whose rows are still being gathered has no event on its stream yet, and a
   // wait on an event that was never recorded returns at once: wait for the record first.
-  if (!g->wait_recorded(b))
+  if (!g->gate.wait(b))
     return fail(FKV_ERR_RUNTIME, "layer %d will not land: the restore failed while it was launched",
                 layer);
   FKV_HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(consumer_stream),
@@ -1060,7 +1047,7 @@ int fkv_layerwise_batch_times_ms(fkv_layerwise *g, float *out_ms, int32_t capaci
     return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_batch_times_ms: null argument");
   *num_batches = (int32_t)g->batches.size();
   g->join_feeder();
-  if (g->recorded.load(std::memory_order_acquire) < (int)g->batches.size())
+  if (g->gate.recorded() < (int)g->batches.size())
     return fail(FKV_ERR_RUNTIME, "fkv_layerwise_batch_times_ms: the restore was not launched completely");
   DeviceGuard restore(g->device_ids[0]);
   for (int b = 0; b < (int)g->batches.size() && b < capacity; ++b)

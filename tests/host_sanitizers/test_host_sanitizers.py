@@ -55,3 +55,12 @@ def test_layerwise_poll_loop_under_sanitizers(tmp_path, sanitizer):
     is left, a stop request ends it."""
     out = build_and_run(tmp_path, "poll_loop_driver.cpp", sanitizer)
     assert "ok: 301 scripted polls" in out
+
+
+@pytest.mark.parametrize("sanitizer", SANITIZERS)
+def test_batch_gate_of_a_gathered_restore_under_sanitizers(tmp_path, sanitizer):
+    """The gate between the thread that launches a gathered layerwise restore batch by batch
+    and its consumers (fkv_gate.h): scripted launchers that sometimes give up part-way,
+    blocking waiters and the polling loop, 200 runs through one gate."""
+    out = build_and_run(tmp_path, "batch_gate_driver.cpp", sanitizer)
+    assert "ok: 200 scripted restores through the gate" in out
