@@ -480,11 +480,12 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=F
     st1 = get_stats()
     per = lambda k: (st1[k] - st0[k]) / (warmup + steps)
     staged, gathered = int(per("staged_batches")), int(per("gathered_batches"))
-    route = ("copy engine (use_ce_transfer)" if use_ce else
-             "kernel" if staged == 0 else
+    route = (("copy-engine strategies (use_ce_transfer)" if use_ce else "kernel") if staged == 0 else
              "host threads gather each layer into a pinned buffer, one copy-engine command per "
              "layer, scatter launch%s" % (" (first layer by kernel)" if staged < w.L else "")
              if gathered else "copy engines, one command per run of host blocks, scatter launch")
+    if use_ce and staged:
+        route += " (asked for with use_ce_transfer)"
     return dict(staged_batches_per_restore=staged, gathered_batches_per_restore=gathered,
                 gather_busy_ms_per_restore=round(per("gather_busy_us") / 1e3, 3), route=route,
                 total_ms=_median(totals), restore_ms=_median(restores),

@@ -381,17 +381,20 @@ size_t kernel_plan_bytes(const fkv_transfer_desc &d) {
 }
 
 int kernel_plan_fill(const fkv_transfer_desc &d, uint8_t *h, bool may_probe_device,
-                     KernelPlan *out) {
+                     KernelPlan *out, bool host_optional) {
   // Device-visible alias of the host pool.  hipHostMalloc / torch pinned memory
   // map to the same address; hipHostRegister-ed memory may not.
   void *cpu_dev = nullptr;
   hipError_t e = hipHostGetDevicePointer(&cpu_dev, d.cpu_ptr, 0);
-  if (e != hipSuccess || !cpu_dev) {
+  out->host_visible = e == hipSuccess && cpu_dev;
+  if (!out->host_visible) {
     (void)hipGetLastError();
-    return fail(FKV_ERR_INVALID_ARG,
-                "cpu_tensor at %p is not device-visible (allocate it pinned or register it "
-                "before a kernel transfer): %s",
-                d.cpu_ptr, hipGetErrorString(e));
+    cpu_dev = nullptr;
+    if (!host_optional)
+      return fail(FKV_ERR_INVALID_ARG,
+                  "cpu_tensor at %p is not device-visible (allocate it pinned or register it "
+                  "before a kernel transfer): %s",
+                  d.cpu_ptr, hipGetErrorString(e));
   }
   int device = 0;
   FKV_HIP_TRY(hipGetDevice(&device));
@@ -411,8 +414,8 @@ int kernel_plan_fill(const fkv_transfer_desc &d, uint8_t *h, bool may_probe_devi
                                                     kv * d.cpu_kv_stride +
                                                     d.cpu_startoff_inside_chunks);
       gbase[li * d.kv_dim + kv] = g;
-      cbase[li * d.kv_dim + kv] = c;
-      acc |= g | c;
+      cbase[li * d.kv_dim + kv] = out->host_visible ? c : 0;
+      acc |= out->host_visible ? (g | c) : g;
     }
   }
   std::memcpy(h + 2 * tab_bytes, d.gpu_block_ids, ids_bytes);
@@ -448,14 +451,15 @@ void kernel_plan_point(KernelPlan *out, const uint8_t *dv, uint64_t *claims) {
   out->claims = claims;
 }
 
-int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan *out) {
+int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan *out,
+                      bool host_optional) {
   int device = 0;
   FKV_HIP_TRY(hipGetDevice(&device));
   const size_t plan_bytes = kernel_plan_bytes(d);
   PlanSlot *slot = plan_acquire(device, plan_bytes);
   if (!slot)
     return FKV_ERR_RUNTIME;
-  int rc = kernel_plan_fill(d, plan_host(slot), /*may_probe_device=*/true, out);
+  int rc = kernel_plan_fill(d, plan_host(slot), /*may_probe_device=*/true, out, host_optional);
   if (rc != FKV_OK) {
     plan_release(slot, stream, true);
     return rc;
@@ -565,6 +569,9 @@ int shape_for_now(const KernelPlan &p, int64_t bytes, hipStream_t stream, CopyKe
 
 int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
                        hipStream_t stream) {
+  if (!p.host_visible)
+    return fail(FKV_ERR_INVALID_ARG, "kernel transfer: the host pool is not device-visible "
+                "(allocate it pinned or register it)");
   if (layer_offset < 0 || num_layers < 0 || layer_offset + num_layers > p.num_layers)
     return fail(FKV_ERR_RUNTIME, "kernel plan: layers [%d, %d) outside the plan's %d", layer_offset,
                 layer_offset + num_layers, p.num_layers);
@@ -591,6 +598,8 @@ int kernel_plans_launch(const KernelPlan *const *plans, const int *layer_offsets
   // vector width and launch shape, each range within one LDS table.
   const bool fuse = policy_of(plans[0]->device).fuse_launches != 0;
   bool together = fuse && count >= 2 && count <= kCopyMaxJobs;
+  for (int i = 0; i < count; ++i)
+    together = together && plans[i]->host_visible; // the single launches refuse the others
   for (int i = 0; i < count && together; ++i) {
     const KernelPlan &p = *plans[i], &q = *plans[0];
     together = p.h2d == q.h2d && p.device == q.device && p.vec == q.vec &&

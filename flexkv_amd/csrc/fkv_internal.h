@@ -233,6 +233,9 @@ struct KernelPlan {
   int device = 0;
   bool no_alloc = false; // built by the entry point that allocates nothing: launches of this
                          // plan create no events and do not probe the device
+  bool host_visible = true; // false: the host pool is ordinary pageable memory, the plan has no
+                            // host addresses and serves only as the device side of a restore
+                            // whose rows host threads gather (kernel_plan_launch refuses it)
   bool recorded = false; // the launches are being recorded into a graph: shaped once for every
                          // replay, without a look at what the link is doing right now
   uint64_t *claims = nullptr; // a claim counter per layer of the plan, device memory
@@ -251,10 +254,12 @@ bool link_board_busy_elsewhere(int device, bool h2d, int64_t window_ns);
 // and at `claims` (num_layers counters, or nullptr).
 size_t kernel_plan_bytes(const fkv_transfer_desc &d);
 int kernel_plan_fill(const fkv_transfer_desc &d, uint8_t *h, bool may_probe_device,
-                     KernelPlan *out);
+                     KernelPlan *out, bool host_optional = false);
 void kernel_plan_point(KernelPlan *out, const uint8_t *dv, uint64_t *claims);
-// Builds and uploads (on `stream`) the plan for all layers of `d`.
-int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan *out);
+// Builds and uploads (on `stream`) the plan for all layers of `d`.  With `host_optional` a
+// host pool the device cannot read is no error: the plan then has host_visible == false.
+int kernel_plan_build(const fkv_transfer_desc &d, hipStream_t stream, KernelPlan *out,
+                      bool host_optional = false);
 // Enqueues the copy of layers [layer_offset, layer_offset + num_layers) of the plan.
 int kernel_plan_launch(const KernelPlan &p, int layer_offset, int num_layers,
                        hipStream_t stream);
@@ -329,8 +334,11 @@ struct StagedPlan {
 // `batch_layers`) goes through the copy engines on the current device and, if so,
 // sizes the ring and uploads the tables on `scatter_stream`.  FKV_OK with
 // out->usable == false: use the kernel path.
+// `host_visible`: the device can read the host pool (else only the gathered route is open);
+// `kernel_allowed`: the caller lets batches go by kernel (the first batch of a gathered restore).
 int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &ring,
-                      GatherRing &pinned, hipStream_t scatter_stream, StagedPlan *out);
+                      GatherRing &pinned, hipStream_t scatter_stream, StagedPlan *out,
+                      bool host_visible = true, bool kernel_allowed = true);
 // The choice alone (no device): kRouteKernel, kRouteRuns (fills `segs` and `total_rows`)
 // or kRouteGathered.
 int staged_route(const int64_t *cpu_ids, int num_blocks, int64_t row_bytes, int pieces,

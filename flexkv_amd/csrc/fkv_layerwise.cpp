@@ -133,6 +133,7 @@ struct Lane {
   int64_t cpu_kv_stride = 0, cpu_layer_stride = 0, cpu_block_stride = 0;
   std::vector<int64_t> cpu_off; // per GPU
   const int64_t *gpu_ids = nullptr, *cpu_ids = nullptr;
+  std::vector<int64_t> own_gpu_ids, own_cpu_ids; // copies, where the launch outlives the call
   int num_blocks = 0;
   int kv_dim = 1;
   bool used = false;
@@ -173,6 +174,7 @@ struct fkv_layerwise {
   std::unique_ptr<fkv::HostCrew> crew;
   std::thread feeder;
   std::vector<Lane> feed_lanes; // what the feeder works on
+  int feed_use_ce = 0, feed_num_cta = 0;
   fkv::BatchGate gate;          // which batches have had their events recorded, or never will
   int feed_rc = 0;              // why the launching thread gave up (read once it has been joined)
   std::string feed_error;
@@ -361,8 +363,14 @@ int finish_create(std::unique_ptr<fkv_layerwise> &g, const int64_t *gpu_device_i
   return FKV_OK;
 }
 
+// What a call asks for that every transfer of it shares.
+struct EngineChoice {
+  int use_ce_transfer = 0;
+  int transfer_cta_num = 0;
+};
+
 fkv_transfer_desc describe(const fkv_layerwise *g, const Lane &lane, int gpu, int start,
-                           int layers, const fkv_layerwise_call &c) {
+                           int layers, const EngineChoice &c) {
   const Source &s = *lane.src;
   fkv_transfer_desc d{};
   d.backend = s.backend;
@@ -397,11 +405,15 @@ fkv_transfer_desc describe(const fkv_layerwise *g, const Lane &lane, int gpu, in
 // Enqueues every batch of the restore that is being set up, in order, records the batch
 // events and hands the plan memory back; `rc` is the status of the set-up so far (a
 // failed set-up enqueues nothing).  Runs on the calling thread, or on the group's
-// launching thread where host threads gather rows (`on_feeder`; `c` is not used there).
-int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, bool direct,
-                   const fkv_layerwise_call *c, bool on_feeder, int rc) {
+// launching thread where host threads gather rows.  Every item goes the way its lane
+// was set up for: through the copy engines and a staging buffer (one copy per run of
+// host blocks, or rows gathered first), else by kernel (`choice.use_ce_transfer == 0`)
+// or through the copy-engine strategies of fkv_transfer_kv_blocks.
+int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoice &choice,
+                   bool on_feeder, int rc) {
   using namespace fkv;
   DeviceGuard restore(-1);
+  const bool direct = choice.use_ce_transfer == 0;
   const int num_batches = (int)g->batches.size();
   const int give_up_at = policy_of(g->device_ids[0]).test_fail_restore_batch; // tests only
   for (int b = 0; b < num_batches && rc == FKV_OK; ++b) {
@@ -412,49 +424,53 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, bool direct,
     fkv_layerwise::Batch &batch = *g->batches[b];
     for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
       (void)hipSetDevice(g->device_ids[i]);
-      if (direct) {
-        // the members of one batch go out together: up to kCopyMaxJobs per launch
-        const KernelPlan *plans[kCopyMaxJobs];
-        int first[kCopyMaxJobs], count[kCopyMaxJobs];
-        // items of lanes that go through the copy engines first, the rest by kernel
-        std::vector<const Item *> by_kernel;
-        for (const Item &it : batch.items) {
-          Lane &lane = lanes[it.lane];
-          const StagedPlan *sp =
-              !lane.staged.empty() && lane.staged[i].usable ? &lane.staged[i] : nullptr;
-          if (rc != FKV_OK || !sp || (b == 0 && sp->first_by_kernel))
-            by_kernel.push_back(&it);
-          else if (sp->route == kRouteGathered)
-            rc = gathered_launch(*sp, g->rings[{it.lane, i}], g->pinned_rings[{it.lane, i}],
-                                 *g->crew, lane.plans[i], it.start_layer, it.layers,
-                                 g->dma_streams[i], g->streams[i]);
-          else
-            rc = staged_launch(*sp, g->rings[{it.lane, i}], lane.plans[i], it.start_layer,
-                               it.layers, g->dma_streams[i], g->streams[i]);
+      // the members of one batch that go by kernel go out together: up to kCopyMaxJobs per launch
+      const KernelPlan *plans[kCopyMaxJobs];
+      int first[kCopyMaxJobs], count[kCopyMaxJobs];
+      std::vector<const Item *> by_kernel, by_strategy;
+      auto account = [&](const Item &it) {
+        const Lane &lane = lanes[it.lane];
+        stats().calls.fetch_add(1, std::memory_order_relaxed);
+        stats().bytes_h2d.fetch_add((uint64_t)lane.num_blocks * it.layers * lane.kv_dim *
+                                        (uint64_t)lane.src->chunk_sizes[i],
+                                    std::memory_order_relaxed);
+      };
+      for (const Item &it : batch.items) {
+        if (rc != FKV_OK)
+          break;
+        Lane &lane = lanes[it.lane];
+        const StagedPlan *sp =
+            i < (int)lane.staged.size() && lane.staged[i].usable ? &lane.staged[i] : nullptr;
+        if (!sp || (b == 0 && sp->first_by_kernel)) {
+          (direct ? by_kernel : by_strategy).push_back(&it);
+          continue;
         }
-        for (size_t k = 0; k < by_kernel.size() && rc == FKV_OK; k += kCopyMaxJobs) {
-          const int n = (int)std::min<size_t>(kCopyMaxJobs, by_kernel.size() - k);
-          for (int j = 0; j < n; ++j) {
-            const Item &it = *by_kernel[k + j];
-            plans[j] = &lanes[it.lane].plans[i];
-            first[j] = it.start_layer;
-            count[j] = it.layers;
-          }
-          rc = kernel_plans_launch(plans, first, count, n, g->streams[i]);
-        }
-        for (size_t k = 0; k < batch.items.size() && rc == FKV_OK; ++k) {
-          const Item &it = batch.items[k];
-          const Lane &lane = lanes[it.lane];
-          stats().calls.fetch_add(1, std::memory_order_relaxed);
-          stats().bytes_h2d.fetch_add((uint64_t)lane.num_blocks * it.layers * lane.kv_dim *
-                                          (uint64_t)lane.src->chunk_sizes[i],
-                                      std::memory_order_relaxed);
-        }
+        if (sp->route == kRouteGathered)
+          rc = gathered_launch(*sp, g->rings[{it.lane, i}], g->pinned_rings[{it.lane, i}],
+                               *g->crew, lane.plans[i], it.start_layer, it.layers,
+                               g->dma_streams[i], g->streams[i]);
+        else
+          rc = staged_launch(*sp, g->rings[{it.lane, i}], lane.plans[i], it.start_layer, it.layers,
+                             g->dma_streams[i], g->streams[i]);
+        if (rc == FKV_OK)
+          account(it);
       }
-      for (size_t k = 0; !direct && k < batch.items.size() && rc == FKV_OK; ++k) {
-        const Item &it = batch.items[k];
-        fkv_transfer_desc d = describe(g, lanes[it.lane], i, it.start_layer, it.layers, *c);
-        rc = fkv_transfer_kv_blocks(&d, g->streams[i]);
+      for (size_t k = 0; k < by_kernel.size() && rc == FKV_OK; k += kCopyMaxJobs) {
+        const int n = (int)std::min<size_t>(kCopyMaxJobs, by_kernel.size() - k);
+        for (int j = 0; j < n; ++j) {
+          const Item &it = *by_kernel[k + j];
+          plans[j] = &lanes[it.lane].plans[i];
+          first[j] = it.start_layer;
+          count[j] = it.layers;
+        }
+        rc = kernel_plans_launch(plans, first, count, n, g->streams[i]);
+        for (int j = 0; j < n && rc == FKV_OK; ++j)
+          account(*by_kernel[k + j]);
+      }
+      for (size_t k = 0; k < by_strategy.size() && rc == FKV_OK; ++k) {
+        const Item &it = *by_strategy[k];
+        fkv_transfer_desc d = describe(g, lanes[it.lane], i, it.start_layer, it.layers, choice);
+        rc = fkv_transfer_kv_blocks(&d, g->streams[i]); // does its own accounting
         (void)hipSetDevice(g->device_ids[i]);
       }
       if (rc != FKV_OK)
@@ -805,43 +821,63 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
   FKV_HIP_TRY(hipEventRecord(g->started, g->streams[0]));
 
   int rc = FKV_OK;
-  // Kernel path: one plan per used lane and GPU, covering all layers of its group.
-  const bool direct = !c.use_ce_transfer;
-  if (direct)
-    for (Lane &lane : lanes) {
-      if (!lane.used || rc != FKV_OK)
-        continue;
-      lane.plans.resize(g->num_gpus);
-      const int layers = g->multi_group || lane.src != &g->groups[0] ? lane.src->num_layers
-                                                                     : c.num_layers;
-      for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
-        fkv_transfer_desc d = describe(g, lane, i, 0, layers, c);
-        rc = validate(d);
-        if (rc != FKV_OK)
+  // One plan per used lane and GPU, covering all layers of its group: the kernel path of
+  // a restore that was asked for on the kernel, and the device side of the batches that go
+  // through the copy engines and a staging buffer, whichever engine was asked for (a
+  // restore with use_ce_transfer whose host blocks are scattered would otherwise issue a
+  // copy command per block and layer: 8.7 GB/s on 512 blocks of 72 KiB).
+  const EngineChoice choice{c.use_ce_transfer, c.transfer_cta_num};
+  const bool direct = choice.use_ce_transfer == 0;
+  for (Lane &lane : lanes) {
+    if (!lane.used || rc != FKV_OK)
+      continue;
+    lane.plans.resize(g->num_gpus);
+    lane.staged.resize(g->num_gpus);
+    if ((int)g->dma_streams.size() < g->num_gpus)
+      g->dma_streams.resize(g->num_gpus, nullptr);
+    const int layers = g->multi_group || lane.src != &g->groups[0] ? lane.src->num_layers
+                                                                   : c.num_layers;
+    const int lane_index = (int)(&lane - lanes.data());
+    for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
+      fkv_transfer_desc d = describe(g, lane, i, 0, layers, choice);
+      rc = validate(d);
+      if (rc != FKV_OK)
+        break;
+      (void)hipSetDevice(g->device_ids[i]);
+      // A host pool the device cannot read (ordinary pageable memory) still serves a
+      // restore whose rows host threads gather; only the kernel path itself needs more.
+      rc = kernel_plan_build(d, g->streams[i], &lane.plans[i], /*host_optional=*/true);
+      if (rc != FKV_OK) {
+        if (direct)
           break;
-        (void)hipSetDevice(g->device_ids[i]);
-        rc = kernel_plan_build(d, g->streams[i], &lane.plans[i]);
-        // Few runs of host blocks: the lane's batches go through the copy engines
-        // and a staging buffer instead (the plan still gives the device side).
-        if (rc == FKV_OK) {
-          if ((int)g->dma_streams.size() < g->num_gpus)
-            g->dma_streams.resize(g->num_gpus, nullptr);
-          lane.staged.resize(g->num_gpus);
-          const int lane_index = (int)(&lane - lanes.data());
-          rc = staged_plan_build(d, g->multi_group ? 1 : c.layer_granularity,
-                                 g->rings[{lane_index, i}], g->pinned_rings[{lane_index, i}],
-                                 g->streams[i], &lane.staged[i]);
-          if (rc == FKV_OK && lane.staged[i].usable && !g->dma_streams[i]) {
-            hipError_t e = hipStreamCreateWithFlags(&g->dma_streams[i], hipStreamNonBlocking);
-            if (e != hipSuccess) {
-              (void)hipGetLastError();
-              g->dma_streams[i] = nullptr;
-              staged_plan_release(&lane.staged[i], g->streams[i]); // kernel path then
-            }
-          }
+        clear_error(); // the copy-engine strategies need no plan
+        rc = FKV_OK;
+        continue;
+      }
+      rc = staged_plan_build(d, g->multi_group ? 1 : c.layer_granularity,
+                             g->rings[{lane_index, i}], g->pinned_rings[{lane_index, i}],
+                             g->streams[i], &lane.staged[i], lane.plans[i].host_visible,
+                             /*kernel_allowed=*/direct);
+      if (rc == FKV_OK && lane.staged[i].usable && !g->dma_streams[i]) {
+        hipError_t e = hipStreamCreateWithFlags(&g->dma_streams[i], hipStreamNonBlocking);
+        if (e != hipSuccess) {
+          (void)hipGetLastError();
+          g->dma_streams[i] = nullptr;
+          staged_plan_release(&lane.staged[i], g->streams[i]); // kernel path then
         }
       }
+      if (rc == FKV_OK && !lane.staged[i].usable) {
+        if (!direct) // the strategies of the copy-engine path take it from here
+          kernel_plan_release(&lane.plans[i], g->streams[i]);
+        else if (!lane.plans[i].host_visible)
+          rc = fail(FKV_ERR_INVALID_ARG,
+                    "cpu_tensor at %p is not device-visible (allocate it pinned or register it "
+                    "before a kernel transfer), and the restore cannot go through gathered rows "
+                    "either (staged_gather of the launch policy, batch size)",
+                    d.cpu_ptr);
+      }
     }
+  }
   // Staging memory that several restores in a row had no use for goes back (a group
   // with many lanes would otherwise hold buffers for every route it ever took).
   constexpr int kRingIdleCalls = 8;
@@ -874,8 +910,20 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
       }
     }
     g->feed_lanes = std::move(lanes);
+    g->feed_use_ce = choice.use_ce_transfer;
+    g->feed_num_cta = choice.transfer_cta_num;
+    if (!direct) // the copy-engine strategies read the id lists when they are called
+      for (Lane &lane : g->feed_lanes) {
+        if (!lane.used)
+          continue;
+        lane.own_gpu_ids.assign(lane.gpu_ids, lane.gpu_ids + lane.num_blocks);
+        lane.own_cpu_ids.assign(lane.cpu_ids, lane.cpu_ids + lane.num_blocks);
+        lane.gpu_ids = lane.own_gpu_ids.data();
+        lane.cpu_ids = lane.own_cpu_ids.data();
+      }
     auto feed = [g] {
-      const int frc = launch_batches(g, g->feed_lanes, true, nullptr, true, FKV_OK);
+      const EngineChoice how{g->feed_use_ce, g->feed_num_cta};
+      const int frc = launch_batches(g, g->feed_lanes, how, true, FKV_OK);
       if (frc != FKV_OK) {
         g->feed_rc = frc; // read by others only after they have joined this thread
         g->feed_error = fkv_last_error();
@@ -888,7 +936,7 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
       feed(); // no thread to be had: the same work on the calling thread, which then blocks for it
     }
   } else {
-    const int lrc = launch_batches(g, lanes, direct, &c, false, rc);
+    const int lrc = launch_batches(g, lanes, choice, false, rc);
     if (lrc != FKV_OK) {
       (void)hipSetDevice(restore.device());
       return lrc;

@@ -264,12 +264,15 @@ int64_t staged_row_of(const std::vector<StagedPlan::Seg> &segs, int64_t id) {
 }
 
 int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &ring,
-                      GatherRing &pinned, hipStream_t scatter_stream, StagedPlan *out) {
+                      GatherRing &pinned, hipStream_t scatter_stream, StagedPlan *out,
+                      bool host_visible, bool kernel_allowed) {
   *out = StagedPlan{};
   int device = 0;
   FKV_HIP_TRY(hipGetDevice(&device));
   // the choice prices copy commands and gather passes against this device's link
-  const fkv_launch_policy pol = policy_of_seeded(device);
+  fkv_launch_policy pol = policy_of_seeded(device);
+  if (!host_visible) // a pageable pool: the copy engines cannot take its rows, host threads can
+    pol.staged_restore = 0;
   if ((pol.staged_restore == 0 && pol.staged_gather == 0) || d.num_blocks <= 0 ||
       d.num_layers <= 0 || batch_layers < 1)
     return FKV_OK;
@@ -334,7 +337,7 @@ int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &
     }
   if (gathered) {
     out->host_ids.assign(d.cpu_block_ids, d.cpu_block_ids + d.num_blocks);
-    out->first_by_kernel = pol.gather_first_by_kernel != 0;
+    out->first_by_kernel = pol.gather_first_by_kernel != 0 && host_visible && kernel_allowed;
   } else {
     int64_t *rows = reinterpret_cast<int64_t *>(h + tab);
     for (int pos = 0; pos < d.num_blocks; ++pos)

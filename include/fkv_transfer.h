@@ -783,7 +783,10 @@ int fkv_launch_policy_seeded(const fkv_launch_policy *in, double d2h_gbps, doubl
  * staging row of position p is p).  `row_bytes` = bytes of one host block that one batch
  * of layers moves, `pieces` = copy commands per run and batch, which is also the number
  * of pieces a gathering thread copies per block (1 when a batch's chunks of a block are
- * adjacent on the host).  No counterpart in the reference. */
+ * adjacent on the host).  A layerwise call applies it whichever engine it was asked for
+ * (use_ce_transfer only decides what the other batches fall back to), and with
+ * staged_restore = 0 for a host pool that the device cannot read.  No counterpart in the
+ * reference. */
 typedef struct fkv_staged_run {
   int64_t first_id; /* first host block of the run */
   int32_t rows;     /* host blocks it spans, holes read along included */

@@ -26,12 +26,12 @@ def group_of(s, dev):
         is_blockfirst=s.cpu_layout == "BLOCKFIRST")
 
 
-def restore(grp, s, gids, cids, gran, notify="polling", num_layers=None):
+def restore(grp, s, gids, cids, gran, notify="polling", num_layers=None, use_ce=False):
     e = torch.empty(0, dtype=torch.int64)
     grp.layerwise_transfer(
         e, e, 0, 0, 0, 0, 0, torch.as_tensor(gids), torch.as_tensor(cids), s.cpu_kv_stride,
         s.cpu_layer_stride, s.cpu_block_stride, s.chunk, s.cpu_kv_stride, s.cpu_layer_stride,
-        s.cpu_block_stride, 4, False, s.num_layers if num_layers is None else num_layers, gran,
+        s.cpu_block_stride, 4, use_ce, s.num_layers if num_layers is None else num_layers, gran,
         s.kv_dim, 1, counter_id=0, kv_shared_across_ranks_mode="sharded", notify_mode=notify)
     grp.synchronize()
 
@@ -108,6 +108,92 @@ def test_restore_of_a_layer_prefix_and_duplicate_host_blocks(gpu_device):
         assert get_stats()["staged_batches"] == 2
     s.oracle_transfer(gids, cids, True, num_layers=7)
     dev.assert_matches_reference("prefix of 7 layers")
+    grp.close()
+
+
+@pytest.mark.parametrize("route", ["copy_engines", "gathered_first_by_kernel", "kernel"])
+@pytest.mark.parametrize("notify", ["polling", "hostfunc"])
+def test_restore_asked_for_on_the_copy_engine_takes_the_staged_routes(gpu_device, route, notify):
+    """use_ce_transfer chooses what the batches that do not go through a staging buffer
+    fall back to; the staged routes themselves are open to it (with scattered host blocks
+    the copy-engine strategies issue a copy command per block and layer).  No batch of
+    such a restore goes by kernel, the first one included."""
+    from flexkv_amd.c_ext import get_stats, last_transfer_path, launch_policy, reset_stats
+    L, NG, NC, n, chunk, gran = 7, 96, 80, 41, 4608, 2
+    s = KVSetup(VLLM, L, 2, NG, NC, chunk, "BLOCKFIRST", seed=23)
+    dev = s.to_device(gpu_device)
+    grp = group_of(s, dev)
+    rng = np.random.default_rng(29)
+    batches = (L + gran - 1) // gran
+    with launch_policy(staged_ring=3, gather_ring=2, gather_threads=3, **ROUTES[route]):
+        reset_stats()
+        for rep, pattern in enumerate(("scattered", "one_run", "runs_and_holes")):
+            fresh = rng.integers(0, 256, s.host_bytes, dtype=np.uint8)
+            s.host_ref[:] = fresh
+            dev.host.copy_(torch.from_numpy(fresh))
+            gids = rng.permutation(NG)[:n].astype(np.int64)
+            cids = host_ids(rng, NC, n, pattern)
+            restore(grp, s, gids, cids, gran, notify=notify, use_ce=True)
+            s.oracle_transfer(gids, cids, True)
+            dev.assert_matches_reference(f"restore {rep} ({pattern}) on the copy engine")
+        st = get_stats()
+    staged = 0 if route == "kernel" else 3 * batches
+    assert st["staged_batches"] == staged, st
+    assert st["gathered_batches"] == (staged if route.startswith("gathered") else 0), st
+    if route == "kernel":
+        assert last_transfer_path() != "KERNEL"    # one of the copy-engine strategies
+    else:
+        assert st["kernel_launches"] == staged, st   # the scatter launches and nothing else
+    grp.close()
+
+
+@pytest.mark.parametrize("use_ce", [False, True])
+def test_restore_from_a_pageable_host_pool(gpu_device, use_ce):
+    """Ordinary host memory is not visible to the device: the kernel path and the copy
+    per run cannot take it, rows gathered by host threads into pinned buffers can.  A
+    restore that was asked for on the kernel and has no such route says what is wrong;
+    one on the copy engine falls back to the engine's own strategies."""
+    from flexkv_amd.c_ext import get_stats, launch_policy, reset_stats
+    L, NG, NC, n, chunk, gran = 6, 64, 72, 33, 9216, 1
+    s = KVSetup(SGLANG, L, 2, NG, NC, chunk, "BLOCKFIRST", seed=31)
+    dev = s.to_device(gpu_device)
+    dev.host = torch.empty(s.host_bytes, dtype=torch.uint8)   # pageable
+    assert not dev.host.is_pinned()
+    dev.host.copy_(torch.from_numpy(s.host_ref))
+    grp = group_of(s, dev)
+    rng = np.random.default_rng(37)
+    gids = rng.permutation(NG)[:n].astype(np.int64)
+    cids = host_ids(rng, NC, n, "scattered")
+    with launch_policy(staged_restore=2, staged_gather=2, gather_ring=2, gather_threads=3):
+        reset_stats()
+        restore(grp, s, gids, cids, gran, use_ce=use_ce)
+        st = get_stats()
+    assert (st["staged_batches"], st["gathered_batches"]) == (L, L), st   # no batch by kernel or per run
+    s.oracle_transfer(gids, cids, True)
+    dev.assert_matches_reference("gathered out of pageable memory")
+    # no staged route open
+    fresh = rng.integers(0, 256, s.host_bytes, dtype=np.uint8)
+    s.host_ref[:] = fresh
+    dev.host.copy_(torch.from_numpy(fresh))
+    with launch_policy(staged_restore=2, staged_gather=0):
+        reset_stats()
+        if use_ce:
+            restore(grp, s, gids, cids, gran, use_ce=True)
+            assert get_stats()["staged_batches"] == 0
+            s.oracle_transfer(gids, cids, True)
+            dev.assert_matches_reference("copy-engine strategies out of pageable memory")
+        else:
+            before = [t.clone() for t in dev.gpu]
+            with pytest.raises(ValueError, match="not device-visible"):
+                restore(grp, s, gids, cids, gran, use_ce=False)
+            torch.cuda.synchronize()
+            assert all(torch.equal(a, b) for a, b in zip(before, dev.gpu))   # nothing was enqueued
+    # and the group works afterwards
+    with launch_policy(staged_gather=2):
+        restore(grp, s, gids, cids, gran, use_ce=use_ce)
+    if not use_ce:
+        s.oracle_transfer(gids, cids, True)
+    dev.assert_matches_reference("after the refused restore")
     grp.close()
 
 
