@@ -1237,6 +1237,8 @@ def measure_config(name, args, torch, device, link, steps, warmup):
                    d2h_ms_median=round(_median(d2h_ms), 4), d2h_ms_min=round(min(d2h_ms), 4),
                    h2d_ms_median=round(_median(h2d_ms), 4), h2d_ms_min=round(min(h2d_ms), 4),
                    avg_launch_ms=round(avg_ms, 4), path_taken=taken,
+                   d2h_ms_steps=[round(x, 3) for x in d2h_ms],
+                   h2d_ms_steps=[round(x, 3) for x in h2d_ms],
                    sync_call_wall={
                        "what": "host wall clock around one call with sync=True, %d calls per "
                                "direction" % len(sync_ms["d2h"]),
@@ -1567,7 +1569,7 @@ def main():
         ce = measure_config(name, ce_args, torch, device, link, steps, 2)  # staging buffers are allocated in the first calls
         return {k: ce[k] for k in ("d2h_GBps", "h2d_GBps", "d2h_frac_of_link", "h2d_frac_of_link",
                                    "d2h_ms_median", "d2h_ms_min", "h2d_ms_median", "h2d_ms_min",
-                                   "path_taken", "steps")}
+                                   "d2h_ms_steps", "h2d_ms_steps", "path_taken", "steps")}
     if not args.use_ce:
         records[head]["copy_engine"] = copy_engine_record(head, min(3, args.steps))
     args.with_fragmented = True
