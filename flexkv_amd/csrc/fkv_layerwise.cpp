@@ -167,6 +167,19 @@ struct fkv_layerwise {
   // GPU for the copies, created on first use, and the staging buffers by
   // (lane, GPU), kept from call to call.
   std::vector<hipStream_t> dma_streams;
+  // A second one per GPU: the copies of consecutive batches alternate between the two, so
+  // that the event record and wait around one copy run next to the other stream's copy
+  // instead of between two copies (the engine takes the copies in the order of submission
+  // either way).  Created with the first; nullptr = all copies on the first.
+  std::vector<hipStream_t> dma_streams2;
+  std::vector<unsigned> dma_turn;
+  // Restores by kernel in small batches: every other batch is launched on a second stream
+  // per GPU, forked off `streams` after the plan uploads and joined back before the plans
+  // are released, so that a batch starts while its predecessor's last requests are in
+  // flight and its event is being recorded (8 us between two launches on one stream,
+  // next to 18 us of link time for 1 MiB).  Created on first use.
+  std::vector<hipStream_t> alt_streams;
+  std::vector<hipEvent_t> alt_fork, alt_join;
   std::map<std::pair<int, int>, fkv::StagedRing> rings;
   // Restores whose rows host threads gather first: pinned buffers by (lane, GPU), the
   // helper threads, and the thread that launches such a restore batch by batch.
@@ -303,10 +316,11 @@ struct fkv_layerwise {
       }
     }
     for (int g = 0; g < (int)dma_streams.size(); ++g)
-      if (dma_streams[g]) {
-        (void)hipSetDevice(device_ids[g]);
-        (void)hipStreamSynchronize(dma_streams[g]);
-      }
+      for (hipStream_t s : {dma_streams[g], dma_streams2[g]})
+        if (s) {
+          (void)hipSetDevice(device_ids[g]);
+          (void)hipStreamSynchronize(s);
+        }
     for (auto &b : batches)
       for (int g = 0; g < num_gpus; ++g) {
         (void)hipSetDevice(device_ids[g]);
@@ -416,6 +430,37 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
   const bool direct = choice.use_ce_transfer == 0;
   const int num_batches = (int)g->batches.size();
   const int give_up_at = policy_of(g->device_ids[0]).test_fail_restore_batch; // tests only
+  std::vector<char> two_dma_streams(g->num_gpus);
+  std::vector<int64_t> alt_max_bytes(g->num_gpus, 0); // batches by kernel up to this size alternate
+  for (int i = 0; i < g->num_gpus; ++i) {
+    const fkv_launch_policy pol = policy_of(g->device_ids[i]);
+    two_dma_streams[i] = pol.staged_dma_streams >= 2;
+    if (!direct || pol.kernel_alt_stream_kb <= 0 || num_batches < 2 || rc != FKV_OK)
+      continue;
+    if ((int)g->alt_streams.size() < g->num_gpus) {
+      g->alt_streams.resize(g->num_gpus, nullptr);
+      g->alt_fork.resize(g->num_gpus, nullptr);
+      g->alt_join.resize(g->num_gpus, nullptr);
+    }
+    (void)hipSetDevice(g->device_ids[i]);
+    if (!g->alt_streams[i] &&
+        (hipStreamCreateWithFlags(&g->alt_streams[i], hipStreamNonBlocking) != hipSuccess ||
+         hipEventCreateWithFlags(&g->alt_fork[i], hipEventDisableTiming) != hipSuccess ||
+         hipEventCreateWithFlags(&g->alt_join[i], hipEventDisableTiming) != hipSuccess)) {
+      (void)hipGetLastError(); // everything on the one stream then
+      continue;
+    }
+    if (!g->alt_fork[i] || !g->alt_join[i])
+      continue; // an earlier call could not create them
+    // behind the plan uploads of this call
+    if (hipEventRecord(g->alt_fork[i], g->streams[i]) != hipSuccess ||
+        hipStreamWaitEvent(g->alt_streams[i], g->alt_fork[i], 0) != hipSuccess) {
+      (void)hipGetLastError();
+      continue;
+    }
+    alt_max_bytes[i] = (int64_t)pol.kernel_alt_stream_kb * 1024;
+  }
+  std::vector<char> alt_used(g->num_gpus, 0);
   for (int b = 0; b < num_batches && rc == FKV_OK; ++b) {
     if (give_up_at > 0 && b == give_up_at - 1) {
       rc = fail(FKV_ERR_RUNTIME, "layerwise restore made to give up before batch %d (test_fail_restore_batch)", b);
@@ -445,15 +490,31 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
           (direct ? by_kernel : by_strategy).push_back(&it);
           continue;
         }
+        const bool second = two_dma_streams[i] && g->dma_streams2[i] && (g->dma_turn[i]++ & 1u);
+        const hipStream_t dma = second ? g->dma_streams2[i] : g->dma_streams[i];
         if (sp->route == kRouteGathered)
           rc = gathered_launch(*sp, g->rings[{it.lane, i}], g->pinned_rings[{it.lane, i}],
-                               *g->crew, lane.plans[i], it.start_layer, it.layers,
-                               g->dma_streams[i], g->streams[i]);
+                               *g->crew, lane.plans[i], it.start_layer, it.layers, dma,
+                               g->streams[i]);
         else
           rc = staged_launch(*sp, g->rings[{it.lane, i}], lane.plans[i], it.start_layer, it.layers,
-                             g->dma_streams[i], g->streams[i]);
+                             dma, g->streams[i]);
         if (rc == FKV_OK)
           account(it);
+      }
+      // a small batch that goes by kernel as a whole: every other one on the second stream
+      hipStream_t batch_stream = g->streams[i];
+      if (alt_max_bytes[i] > 0 && (b & 1) && !by_kernel.empty() &&
+          by_kernel.size() == batch.items.size()) {
+        int64_t bytes = 0;
+        for (const Item *it : by_kernel) {
+          const Lane &lane = lanes[it->lane];
+          bytes += (int64_t)lane.num_blocks * it->layers * lane.kv_dim * lane.src->chunk_sizes[i];
+        }
+        if (bytes <= alt_max_bytes[i]) {
+          batch_stream = g->alt_streams[i];
+          alt_used[i] = 1;
+        }
       }
       for (size_t k = 0; k < by_kernel.size() && rc == FKV_OK; k += kCopyMaxJobs) {
         const int n = (int)std::min<size_t>(kCopyMaxJobs, by_kernel.size() - k);
@@ -463,7 +524,7 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
           first[j] = it.start_layer;
           count[j] = it.layers;
         }
-        rc = kernel_plans_launch(plans, first, count, n, g->streams[i]);
+        rc = kernel_plans_launch(plans, first, count, n, batch_stream);
         for (int j = 0; j < n && rc == FKV_OK; ++j)
           account(*by_kernel[k + j]);
       }
@@ -475,7 +536,7 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
       }
       if (rc != FKV_OK)
         break;
-      hipError_t e = hipEventRecord(batch.done[i], g->streams[i]);
+      hipError_t e = hipEventRecord(batch.done[i], batch_stream);
       if (e != hipSuccess) {
         (void)hipGetLastError();
         rc = fail(FKV_ERR_RUNTIME, "layerwise_transfer failed on GPU %d: %s", i,
@@ -484,6 +545,20 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
     }
     if (rc == FKV_OK)
       g->gate.publish(b + 1);
+  }
+  // The second stream joins the first: what follows on `streams` (the release of the plan
+  // memory, a synchronize, the next call) is behind every batch.
+  for (int i = 0; i < g->num_gpus; ++i) {
+    if (!alt_used[i])
+      continue;
+    (void)hipSetDevice(g->device_ids[i]);
+    hipError_t e = hipEventRecord(g->alt_join[i], g->alt_streams[i]);
+    if (e == hipSuccess)
+      e = hipStreamWaitEvent(g->streams[i], g->alt_join[i], 0);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      (void)hipStreamSynchronize(g->alt_streams[i]); // the host waits instead
+    }
   }
   std::string saved_error = fkv_last_error();
   for (Lane &lane : lanes)
@@ -497,8 +572,12 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
     // Drain what was enqueued; nothing more of this call is announced.
     for (int i = 0; i < g->num_gpus; ++i) {
       (void)hipSetDevice(g->device_ids[i]);
-      if (i < (int)g->dma_streams.size() && g->dma_streams[i])
-        (void)hipStreamSynchronize(g->dma_streams[i]);
+      if (i < (int)g->dma_streams.size())
+        for (hipStream_t s : {g->dma_streams[i], g->dma_streams2[i]})
+          if (s)
+            (void)hipStreamSynchronize(s);
+      if (i < (int)g->alt_streams.size() && g->alt_streams[i])
+        (void)hipStreamSynchronize(g->alt_streams[i]);
       (void)hipStreamSynchronize(g->streams[i]);
     }
     if (!on_feeder) // on the launching thread consumers may be reading the table
@@ -833,8 +912,11 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
       continue;
     lane.plans.resize(g->num_gpus);
     lane.staged.resize(g->num_gpus);
-    if ((int)g->dma_streams.size() < g->num_gpus)
+    if ((int)g->dma_streams.size() < g->num_gpus) {
       g->dma_streams.resize(g->num_gpus, nullptr);
+      g->dma_streams2.resize(g->num_gpus, nullptr);
+      g->dma_turn.resize(g->num_gpus, 0u);
+    }
     const int layers = g->multi_group || lane.src != &g->groups[0] ? lane.src->num_layers
                                                                    : c.num_layers;
     const int lane_index = (int)(&lane - lanes.data());
@@ -864,6 +946,10 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
           (void)hipGetLastError();
           g->dma_streams[i] = nullptr;
           staged_plan_release(&lane.staged[i], g->streams[i]); // kernel path then
+        } else if (hipStreamCreateWithFlags(&g->dma_streams2[i], hipStreamNonBlocking) !=
+                   hipSuccess) {
+          (void)hipGetLastError();
+          g->dma_streams2[i] = nullptr; // all copies on the first then
         }
       }
       if (rc == FKV_OK && !lane.staged[i].usable) {
@@ -1119,8 +1205,17 @@ void fkv_layerwise_destroy(fkv_layerwise *g) {
   g->crew.reset();
   for (int i = 0; i < g->num_gpus; ++i) {
     (void)hipSetDevice(g->device_ids[i]);
-    if (i < (int)g->dma_streams.size() && g->dma_streams[i])
-      (void)hipStreamDestroy(g->dma_streams[i]);
+    if (i < (int)g->dma_streams.size())
+      for (hipStream_t s : {g->dma_streams[i], g->dma_streams2[i]})
+        if (s)
+          (void)hipStreamDestroy(s);
+    if (i < (int)g->alt_streams.size()) {
+      if (g->alt_streams[i])
+        (void)hipStreamDestroy(g->alt_streams[i]);
+      for (hipEvent_t e : {g->alt_fork[i], g->alt_join[i]})
+        if (e)
+          (void)hipEventDestroy(e);
+    }
     (void)hipStreamDestroy(g->streams[i]);
   }
   (void)hipSetDevice(restore.device());

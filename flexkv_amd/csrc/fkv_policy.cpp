@@ -168,6 +168,8 @@ void sanitize(fkv_launch_policy &p, const fkv_launch_policy &derived) {
   p.model_seeded = derived.model_seeded;
   p.staged_scatter_threads = clampi(p.staged_scatter_threads, 64, kCopyBlockThreads);
   p.test_fail_restore_batch = clampi(p.test_fail_restore_batch, 0, 1 << 20);
+  p.staged_dma_streams = clampi(p.staged_dma_streams, 1, 2);
+  p.kernel_alt_stream_kb = clampi(p.kernel_alt_stream_kb, 0, 1 << 20);
 }
 
 // The table of a device with the XCDs `present`, environment applied.
@@ -235,6 +237,8 @@ fkv_launch_policy defaults_for(uint32_t present) {
   p.model_seed = 1;
   p.model_seeded = 0;
   p.staged_scatter_threads = 256;
+  p.staged_dma_streams = 2;
+  p.kernel_alt_stream_kb = 4096;
   for (const EnvField &f : kEnv) {
     const char *v = std::getenv(f.name);
     if (v && *v) // decimal, 0x.. or 0.. as written

@@ -751,7 +751,19 @@ typedef struct fkv_launch_policy {
   int32_t test_fail_restore_batch; /* tests: n > 0 makes a layerwise restore give up before it
                                  enqueues its n-th batch, as a failed launch would (nothing faults:
                                  the batches before it run and are announced, the rest never lands) */
-  int32_t reserved[3];
+  int32_t staged_dma_streams; /* streams per GPU on which a layerwise restore issues its copy-engine
+                                 copies: 2 (default) consecutive batches alternate between two, so
+                                 that the event record and wait around a copy run next to the other
+                                 stream's copy (4 MiB a batch: 84 us against 93 us per batch; the
+                                 engine still takes the copies in the order of submission); 1 all
+                                 on one */
+  int32_t kernel_alt_stream_kb; /* a layerwise restore by kernel launches every other batch of at
+                                 most this many KiB on a second stream, so that it starts while
+                                 the last requests of its predecessor are in flight (two launches
+                                 on one stream lie 8 us apart, next to 18 us of link time for
+                                 1 MiB); events, notifications and wait_layer stay per batch and
+                                 in order.  Default 4096; 0 = one stream */
+  int32_t reserved[1];
 } fkv_launch_policy;
 /* The table of `device` (-1 = current).  The first call for a device runs the probe kernel. */
 int fkv_launch_policy_get(int32_t device, fkv_launch_policy *out);

@@ -55,7 +55,10 @@ def host_ids(rng, pool, n, pattern):
 ROUTES = {"copy_engines": dict(staged_restore=2, staged_gather=0),
           "gathered": dict(staged_restore=0, staged_gather=2, gather_first_by_kernel=0),
           "gathered_first_by_kernel": dict(staged_restore=0, staged_gather=2, gather_first_by_kernel=1),
-          "kernel": dict(staged_restore=0, staged_gather=0)}
+          "kernel": dict(staged_restore=0, staged_gather=0),
+          # every batch on the group's one stream (by default small batches alternate over two)
+          "kernel_one_stream": dict(staged_restore=0, staged_gather=0, kernel_alt_stream_kb=0),
+          "copy_engines_one_stream": dict(staged_restore=2, staged_gather=0, staged_dma_streams=1)}
 
 
 @pytest.mark.parametrize("route", list(ROUTES))
@@ -87,7 +90,8 @@ def test_restore_matches_the_oracle(gpu_device, route, pattern, backend, kv_dim,
         st = get_stats()
     batches = (L + gran - 1) // gran
     want_staged = {"copy_engines": 3 * batches, "gathered": 3 * batches,
-                   "gathered_first_by_kernel": 3 * (batches - 1), "kernel": 0}[route]
+                   "gathered_first_by_kernel": 3 * (batches - 1), "kernel": 0,
+                   "kernel_one_stream": 0, "copy_engines_one_stream": 3 * batches}[route]
     assert st["staged_batches"] == want_staged, st
     assert st["gathered_batches"] == (want_staged if route.startswith("gathered") else 0), st
     grp.close()
