@@ -651,6 +651,7 @@ def run_notify_scales(torch, device, num_cta, iters=20, warmup=3):
     three scales of the reference's notify-mode microbenchmark
     (benchmarks/microbenchmark_notify_mode.py:28-33, 87-147): MLA fp16, 16 tokens
     x 512 dims per block, layer_granularity 1, one GPU, no eventfd consumer."""
+    import flexkv_amd.c_ext as c_ext
     from flexkv_amd.c_ext import LayerwiseTransferGroup
     scales = {"small": (8, 16), "medium": (32, 64), "large": (80, 256)}
     out = {}
@@ -673,6 +674,7 @@ def run_notify_scales(torch, device, num_cta, iters=20, warmup=3):
                 is_blockfirst=True)
             for notify in ("hostfunc", "polling"):
                 ts = []
+                c_ext.reset_stats()
                 for it in range(warmup + iters):
                     torch.cuda.synchronize()
                     t0 = time.perf_counter()
@@ -684,6 +686,10 @@ def run_notify_scales(torch, device, num_cta, iters=20, warmup=3):
                         ts.append((time.perf_counter() - t0) * 1e3)
                 key = ("ce_" if use_ce else "kernel_") + notify + "_p50_ms"
                 row[key] = round(_median(ts), 4)
+                st = c_ext.get_stats()
+                if not use_ce and notify == "polling":   # which way the batches went
+                    row["batches_through_copy_engines"] = st["staged_batches"] // (warmup + iters)
+                    row["batches_on_second_stream"] = st["second_stream_batches"] // (warmup + iters)
             grp.close()
         out[name] = row
     return out

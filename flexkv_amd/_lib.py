@@ -175,7 +175,7 @@ class Stats(Structure):
                 ("staging_bytes_device", c_uint64), ("staging_bytes_host", c_uint64),
                 ("confined_launches", c_uint64), ("safety_net_ranges", c_uint64),
                 ("staged_batches", c_uint64), ("gathered_batches", c_uint64),
-                ("gather_busy_us", c_uint64)]
+                ("gather_busy_us", c_uint64), ("second_stream_batches", c_uint64)]
 
 
 class LaunchPolicy(Structure):
@@ -319,8 +319,8 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.fkv_abi_version() != 3:
-        raise ImportError(f"{LIB_PATH}: ABI version {lib.fkv_abi_version()} != 3")
+    if lib.fkv_abi_version() != 4:
+        raise ImportError(f"{LIB_PATH}: ABI version {lib.fkv_abi_version()} != 4")
     _lib = lib
     return lib
 

@@ -730,6 +730,7 @@ void fkv_get_stats(fkv_stats *out) {
       out->confined_launches ? fkv::safety_net_ranges_of_current_device() : 0;
   out->staged_batches = s.staged_batches.load();
   out->gathered_batches = s.gathered_batches.load();
+  out->second_stream_batches = s.second_stream_batches.load();
   out->gather_busy_us = s.gather_busy_ns.load() / 1000;
 }
 void fkv_reset_stats(void) {
@@ -744,6 +745,7 @@ void fkv_reset_stats(void) {
   s.confined_launches = 0;
   s.staged_batches = 0;
   s.gathered_batches = 0;
+  s.second_stream_batches = 0;
   s.gather_busy_ns = 0;
 }
 

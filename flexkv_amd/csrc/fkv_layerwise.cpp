@@ -174,12 +174,12 @@ struct fkv_layerwise {
   std::vector<hipStream_t> dma_streams2;
   std::vector<unsigned> dma_turn;
   // Restores by kernel in small batches: every other batch is launched on a second stream
-  // per GPU, forked off `streams` after the plan uploads and joined back before the plans
-  // are released, so that a batch starts while its predecessor's last requests are in
+  // per GPU, which starts behind the first batch of the call (and so behind its plan
+  // uploads) and is joined back into `streams` before the plans are released, so that a batch starts while its predecessor's last requests are in
   // flight and its event is being recorded (8 us between two launches on one stream,
   // next to 18 us of link time for 1 MiB).  Created on first use.
   std::vector<hipStream_t> alt_streams;
-  std::vector<hipEvent_t> alt_fork, alt_join;
+  std::vector<hipEvent_t> alt_join;
   std::map<std::pair<int, int>, fkv::StagedRing> rings;
   // Restores whose rows host threads gather first: pinned buffers by (lane, GPU), the
   // helper threads, and the thread that launches such a restore batch by batch.
@@ -430,34 +430,29 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
   const bool direct = choice.use_ce_transfer == 0;
   const int num_batches = (int)g->batches.size();
   const int give_up_at = policy_of(g->device_ids[0]).test_fail_restore_batch; // tests only
+  // Fewer batches than this and the call is bound by the host's launches, not by the gaps
+  // between them on the device (8 batches of 256 KiB: 0.15 ms either way).
+  constexpr int kAltMinBatches = 12;
   std::vector<char> two_dma_streams(g->num_gpus);
   std::vector<int64_t> alt_max_bytes(g->num_gpus, 0); // batches by kernel up to this size alternate
   for (int i = 0; i < g->num_gpus; ++i) {
     const fkv_launch_policy pol = policy_of(g->device_ids[i]);
     two_dma_streams[i] = pol.staged_dma_streams >= 2;
-    if (!direct || pol.kernel_alt_stream_kb <= 0 || num_batches < 2 || rc != FKV_OK)
+    if (!direct || pol.kernel_alt_stream_kb <= 0 || num_batches < kAltMinBatches || rc != FKV_OK)
       continue;
     if ((int)g->alt_streams.size() < g->num_gpus) {
       g->alt_streams.resize(g->num_gpus, nullptr);
-      g->alt_fork.resize(g->num_gpus, nullptr);
       g->alt_join.resize(g->num_gpus, nullptr);
     }
     (void)hipSetDevice(g->device_ids[i]);
     if (!g->alt_streams[i] &&
         (hipStreamCreateWithFlags(&g->alt_streams[i], hipStreamNonBlocking) != hipSuccess ||
-         hipEventCreateWithFlags(&g->alt_fork[i], hipEventDisableTiming) != hipSuccess ||
          hipEventCreateWithFlags(&g->alt_join[i], hipEventDisableTiming) != hipSuccess)) {
       (void)hipGetLastError(); // everything on the one stream then
       continue;
     }
-    if (!g->alt_fork[i] || !g->alt_join[i])
-      continue; // an earlier call could not create them
-    // behind the plan uploads of this call
-    if (hipEventRecord(g->alt_fork[i], g->streams[i]) != hipSuccess ||
-        hipStreamWaitEvent(g->alt_streams[i], g->alt_fork[i], 0) != hipSuccess) {
-      (void)hipGetLastError();
-      continue;
-    }
+    if (!g->alt_join[i])
+      continue; // an earlier call could not create it
     alt_max_bytes[i] = (int64_t)pol.kernel_alt_stream_kb * 1024;
   }
   std::vector<char> alt_used(g->num_gpus, 0);
@@ -502,18 +497,25 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
         if (rc == FKV_OK)
           account(it);
       }
-      // a small batch that goes by kernel as a whole: every other one on the second stream
+      // a small batch that goes by kernel as a whole: every other one on the second stream,
+      // from the third on (the first one has the link to itself and lands as early as it can)
       hipStream_t batch_stream = g->streams[i];
-      if (alt_max_bytes[i] > 0 && (b & 1) && !by_kernel.empty() &&
+      if (alt_max_bytes[i] > 0 && b >= 2 && !(b & 1) && !by_kernel.empty() &&
           by_kernel.size() == batch.items.size()) {
         int64_t bytes = 0;
         for (const Item *it : by_kernel) {
           const Lane &lane = lanes[it->lane];
           bytes += (int64_t)lane.num_blocks * it->layers * lane.kv_dim * lane.src->chunk_sizes[i];
         }
-        if (bytes <= alt_max_bytes[i]) {
+        // the second stream starts behind the first batch, which is behind the plan uploads
+        if (bytes <= alt_max_bytes[i] &&
+            (alt_used[i] ||
+             hipStreamWaitEvent(g->alt_streams[i], g->batches[0]->done[i], 0) == hipSuccess)) {
           batch_stream = g->alt_streams[i];
           alt_used[i] = 1;
+          stats().second_stream_batches.fetch_add(1, std::memory_order_relaxed);
+        } else {
+          (void)hipGetLastError();
         }
       }
       for (size_t k = 0; k < by_kernel.size() && rc == FKV_OK; k += kCopyMaxJobs) {
@@ -1212,9 +1214,8 @@ void fkv_layerwise_destroy(fkv_layerwise *g) {
     if (i < (int)g->alt_streams.size()) {
       if (g->alt_streams[i])
         (void)hipStreamDestroy(g->alt_streams[i]);
-      for (hipEvent_t e : {g->alt_fork[i], g->alt_join[i]})
-        if (e)
-          (void)hipEventDestroy(e);
+      if (g->alt_join[i])
+        (void)hipEventDestroy(g->alt_join[i]);
     }
     (void)hipStreamDestroy(g->streams[i]);
   }

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define FKV_ABI_VERSION 3 /* 3: fkv_stats grew by gathered_batches and gather_busy_us, fkv_launch_policy by the host-gather and link-seeding fields; 2: fkv_stats grew by staged_batches; launch policy, no-alloc transfer, staging and HBM-rate entry points added */
+#define FKV_ABI_VERSION 4 /* 4: fkv_stats grew by second_stream_batches; 3: fkv_stats grew by gathered_batches and gather_busy_us, fkv_launch_policy by the host-gather and link-seeding fields; 2: fkv_stats grew by staged_batches; launch policy, no-alloc transfer, staging and HBM-rate entry points added */
 
 /* status codes */
 #define FKV_OK 0
@@ -570,6 +570,8 @@ typedef struct fkv_stats {
   uint64_t gathered_batches;  /* of those, the batches whose host rows were first gathered into a
                                  pinned buffer by host threads (one copy command per batch) */
   uint64_t gather_busy_us;    /* time host threads spent gathering such rows, summed over threads */
+  uint64_t second_stream_batches; /* layer batches of a layerwise restore by kernel that were launched
+                                 on the group's second stream (kernel_alt_stream_kb of the policy) */
 } fkv_stats;
 void fkv_get_stats(fkv_stats *out);
 void fkv_reset_stats(void);
@@ -757,8 +759,9 @@ typedef struct fkv_launch_policy {
                                  stream's copy (4 MiB a batch: 84 us against 93 us per batch; the
                                  engine still takes the copies in the order of submission); 1 all
                                  on one */
-  int32_t kernel_alt_stream_kb; /* a layerwise restore by kernel launches every other batch of at
-                                 most this many KiB on a second stream, so that it starts while
+  int32_t kernel_alt_stream_kb; /* a layerwise restore by kernel of twelve and more batches launches
+                                 every other batch of at most this many KiB, from the third on, on a
+                                 second stream, so that it starts while
                                  the last requests of its predecessor are in flight (two launches
                                  on one stream lie 8 us apart, next to 18 us of link time for
                                  1 MiB); events, notifications and wait_layer stay per batch and

@@ -201,6 +201,69 @@ def test_restore_from_a_pageable_host_pool(gpu_device, use_ce):
     grp.close()
 
 
+@pytest.mark.parametrize("notify", ["polling", "hostfunc"])
+def test_small_batches_by_kernel_alternate_over_two_streams(gpu_device, notify):
+    """A restore by kernel in many small batches launches every other batch from the third
+    on on a second stream.  Bytes against the oracle, the eventfds of the layers in order
+    (the poller and the HOSTFUNC loop look at the batch events in order whichever stream
+    recorded them), a consumer stream gated per layer with wait_layer, three restores in a
+    row through one group, and the same with everything on one stream."""
+    import os
+    from flexkv_amd.c_ext import LayerwiseTransferGroup, get_stats, launch_policy, reset_stats
+    from flexkv_amd.transfer.eventfd_channel import make_eventfd
+    L, NG, NC, n, chunk = 17, 64, 64, 29, 8192
+    s = KVSetup(VLLM, L, 2, NG, NC, chunk, "BLOCKFIRST", seed=41)
+    dev = s.to_device(gpu_device)
+    fds = [make_eventfd() for _ in range(L)]
+    i64 = lambda v: torch.tensor([v], dtype=torch.int64)  # noqa: E731
+    grp = LayerwiseTransferGroup(
+        num_gpus=1, gpu_blocks=[dev.gpu], cpu_blocks=dev.host, ssd_files={}, num_layers=L,
+        gpu_kv_strides_tensor=i64(s.gpu_kv_stride), gpu_block_strides_tensor=i64(s.gpu_block_stride),
+        gpu_layer_strides_tensor=i64(s.gpu_layer_stride), gpu_chunk_sizes_tensor=i64(s.chunk),
+        iouring_entries=0, iouring_flags=0,
+        layer_eventfds_tensor=torch.tensor(fds, dtype=torch.int32), tp_size=1, is_blockfirst=True)
+    rng = np.random.default_rng(43)
+    comp = torch.cuda.Stream()
+    e = torch.empty(0, dtype=torch.int64)
+    for rep, alt_kb in enumerate((4096, 4096, 0, 4096)):
+        fresh = rng.integers(0, 256, s.host_bytes, dtype=np.uint8)
+        s.host_ref[:] = fresh
+        dev.host.copy_(torch.from_numpy(fresh))
+        gids = rng.permutation(NG)[:n].astype(np.int64)
+        cids = host_ids(rng, NC, n, "scattered")
+        gi = torch.as_tensor(gids).to(gpu_device)
+        seen = []
+        with launch_policy(staged_restore=0, staged_gather=0, kernel_alt_stream_kb=alt_kb):
+            reset_stats()
+            torch.cuda.synchronize()
+            grp.layerwise_transfer(
+                e, e, 0, 0, 0, 0, 0, torch.as_tensor(gids), torch.as_tensor(cids), s.cpu_kv_stride,
+                s.cpu_layer_stride, s.cpu_block_stride, s.chunk, s.cpu_kv_stride, s.cpu_layer_stride,
+                s.cpu_block_stride, 4, False, L, 1, s.kv_dim, 1, counter_id=0,
+                kv_shared_across_ranks_mode="sharded", notify_mode=notify)
+            with torch.cuda.stream(comp):
+                for l in range(L):      # what an engine does: gate layer l's kernels on layer l
+                    grp.wait_layer(l, comp)
+                    seen.append(dev.gpu[l].view(torch.uint8).reshape(2, NG, -1)
+                                .index_select(1, gi).clone())
+            grp.synchronize()
+            comp.synchronize()
+            st = get_stats()
+        # batches 2, 4, .. 16 of 17
+        assert st["second_stream_batches"] == (8 if alt_kb else 0), st
+        s.oracle_transfer(gids, cids, True)
+        dev.assert_matches_reference(f"restore {rep}, second stream {'on' if alt_kb else 'off'}")
+        for l in range(L):
+            want = torch.from_numpy(s.gpu_ref[l].view(np.uint8).reshape(2, NG, -1)[:, gids])
+            assert torch.equal(seen[l].cpu(), want), (rep, l)
+        for l, fd in enumerate(fds):       # one unit per layer and restore
+            os.set_blocking(fd, False)
+            assert int.from_bytes(os.read(fd, 8), "little") == 1, (rep, l)
+    grp.close()
+    for fd in fds:
+        os.close(fd)
+
+
 def test_gathered_restore_announces_layers_in_order_and_serves_waiting_streams(gpu_device):
     """The gathered route launches batch by batch from a thread of its own.  A consumer
     stream that asks for a layer before its batch has been enqueued must still see the
