@@ -268,3 +268,84 @@ def test_block_major_partial_layers_direct(gpu_device):
                 assert last_transfer_path() == "GATHER_SCATTER"
                 s.oracle_transfer(gids, cids, h2d, start_layer=l0, num_layers=3)
                 dev.assert_matches_reference(f"block runs layers {l0}..{l0 + 2} h2d={h2d}")
+
+
+# ---- host gather/scatter passes: thread counts and streaming stores -------------------
+# tests/test_kv_transfer_correctness.py:1730-1960 (test_gather_nt_roundtrip,
+# test_gather_nt_layerwise_h2d): ce_gather_threads 0 (single-thread fallback) / 1 / 4 / 8 and
+# ce_gather_nt on / off change how the host passes of the copy-engine path run, never a byte.
+GATHER_QUADRANTS = [   # (kv_dim, num_kv_heads, chunk): MLA, K/V apart with one head, packed MHA, MHA
+    pytest.param(1, 1, 16 * 512 * 2, id="mla"),
+    pytest.param(2, 1, 16 * 512 * 2, id="kv_sep_1h"),
+    pytest.param(1, 8, 16 * 8 * 128 * 2, id="packed_mha"),
+    pytest.param(2, 8, 16 * 8 * 128 * 2, id="plain_mha"),
+]
+
+
+@pytest.mark.parametrize("kv_dim,heads,chunk", GATHER_QUADRANTS)
+@pytest.mark.parametrize("cpu_layout", ["BLOCKFIRST", "LAYERFIRST"])
+@pytest.mark.parametrize("gather_threads", [0, 1, 4, 8], ids=["gt0", "gt1", "gt4", "gt8"])
+@pytest.mark.parametrize("gather_nt", [True, False], ids=["nt_on", "nt_off"])
+def test_gather_threads_and_streaming_stores_round_trip(gpu_device, kv_dim, heads, chunk, cpu_layout,
+                                                        gather_threads, gather_nt):
+    """Put, wipe the engine's blocks, get: the strategy the library picks for the shape, and
+    the two strategies with a host pass forced (rows gathered / scattered by host threads)."""
+    import torch
+    from flexkv_amd.c_ext import last_transfer_path
+    L, N, NH, n = 4, 48, 48, 21
+    s = KVSetup(VLLM, L, kv_dim, N, NH, chunk, cpu_layout, seed=51 + gather_threads)
+    dev = s.to_device(gpu_device)
+    rng = np.random.default_rng(53)
+    kw = dict(use_ce_transfer=True, ce_path_opt=True, num_kv_heads=heads,
+              ce_gather_threads=gather_threads, ce_gather_nt=gather_nt, ce_enable_memcpy2d=False)
+    for force in (None, "SEGMENT_SCATTER", "GATHER_SCATTER"):
+        gids, cids = block_ids(rng, N, n), block_ids(rng, NH, n)
+        extra = {} if force is None else dict(ce_force_path=PATHS[force])
+        dev.transfer(gids, cids, is_h2d=False, **kw, **extra)
+        if force is not None:
+            assert last_transfer_path() == force
+        s.oracle_transfer(gids, cids, False)
+        dev.assert_matches_reference(f"put {force} gt={gather_threads} nt={gather_nt}")
+        # other bytes in the engine's blocks, then back from the host
+        fresh = [np.random.default_rng(59).integers(0, 256, a.size, dtype=np.uint8) for a in s.gpu_ref]
+        for a, t, f in zip(s.gpu_ref, dev.gpu, fresh):
+            a[:] = f
+            t.copy_(torch.from_numpy(f).to(t.device).view(t.dtype).reshape(t.shape))
+        dev.transfer(gids, cids, is_h2d=True, **kw, **extra)
+        s.oracle_transfer(gids, cids, True)
+        dev.assert_matches_reference(f"get {force} gt={gather_threads} nt={gather_nt}")
+
+
+@pytest.mark.parametrize("kv_dim,heads,chunk", GATHER_QUADRANTS)
+@pytest.mark.parametrize("gather_threads", [0, 4], ids=["gt0", "gt4"])
+@pytest.mark.parametrize("gather_nt", [True, False], ids=["nt_on", "nt_off"])
+def test_gather_threads_and_streaming_stores_layerwise_restore(gpu_device, kv_dim, heads, chunk,
+                                                               gather_threads, gather_nt):
+    """The same settings through a layerwise restore on the copy engine, a layer at a time."""
+    import torch
+    from flexkv_amd.c_ext import LayerwiseTransferGroup, launch_policy
+    L, N, NH, n = 4, 48, 48, 21
+    s = KVSetup(VLLM, L, kv_dim, N, NH, chunk, "BLOCKFIRST", seed=61 + gather_threads)
+    dev = s.to_device(gpu_device)
+    i64 = lambda v: torch.tensor([v], dtype=torch.int64)  # noqa: E731
+    grp = LayerwiseTransferGroup(
+        num_gpus=1, gpu_blocks=[dev.gpu], cpu_blocks=dev.host, ssd_files={}, num_layers=L,
+        gpu_kv_strides_tensor=i64(s.gpu_kv_stride), gpu_block_strides_tensor=i64(s.gpu_block_stride),
+        gpu_layer_strides_tensor=i64(s.gpu_layer_stride), gpu_chunk_sizes_tensor=i64(s.chunk),
+        iouring_entries=0, iouring_flags=0,
+        layer_eventfds_tensor=torch.empty(0, dtype=torch.int32), tp_size=1, is_blockfirst=True,
+        num_kv_heads=heads, ce_gather_threads=gather_threads, ce_gather_nt=gather_nt)
+    rng = np.random.default_rng(67)
+    gids, cids = block_ids(rng, N, n), block_ids(rng, NH, n)
+    e = torch.empty(0, dtype=torch.int64)
+    with launch_policy(staged_restore=0, staged_gather=0):   # the copy-engine strategies themselves
+        for notify in ("hostfunc", "polling"):
+            grp.layerwise_transfer(
+                e, e, 0, 0, 0, 0, 0, torch.as_tensor(gids), torch.as_tensor(cids), s.cpu_kv_stride,
+                s.cpu_layer_stride, s.cpu_block_stride, s.chunk, s.cpu_kv_stride, s.cpu_layer_stride,
+                s.cpu_block_stride, 4, True, L, 1, s.kv_dim, heads, counter_id=0,
+                kv_shared_across_ranks_mode="sharded", notify_mode=notify)
+            grp.synchronize()
+            s.oracle_transfer(gids, cids, True)
+            dev.assert_matches_reference(f"layerwise on the copy engine, {notify}")
+    grp.close()
