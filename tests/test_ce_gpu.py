@@ -349,3 +349,61 @@ def test_gather_threads_and_streaming_stores_layerwise_restore(gpu_device, kv_di
             s.oracle_transfer(gids, cids, True)
             dev.assert_matches_reference(f"layerwise on the copy engine, {notify}")
     grp.close()
+
+
+# tests/test_kv_transfer_correctness.py:1327-1620 (test_ce_paths_roundtrip,
+# test_ce_paths_layerwise_h2d): every strategy the id pattern, the threshold and the shape
+# lead to, reached through a layerwise restore on the copy engine, a layer or all layers a batch.
+@pytest.mark.parametrize("kv_dim,heads,chunk", [GATHER_QUADRANTS[0], GATHER_QUADRANTS[1],
+                                                GATHER_QUADRANTS[3]])
+@pytest.mark.parametrize("cpu_layout", ["BLOCKFIRST", "LAYERFIRST"])
+@pytest.mark.parametrize("path_opt", [False, True], ids=["baseline", "optimized"])
+@pytest.mark.parametrize("memcpy2d", [False, True], ids=["no2d", "2d"])
+def test_layerwise_restore_on_the_copy_engine_by_id_pattern(gpu_device, kv_dim, heads, chunk,
+                                                            cpu_layout, path_opt, memcpy2d):
+    import torch
+    from flexkv_amd.c_ext import LayerwiseTransferGroup, last_transfer_path, launch_policy
+    L, N, NH, n = 4, 64, 64, 32
+    s = KVSetup(VLLM, L, kv_dim, N, NH, chunk, cpu_layout, seed=71)
+    dev = s.to_device(gpu_device)
+    i64 = lambda v: torch.tensor([v], dtype=torch.int64)  # noqa: E731
+    e = torch.empty(0, dtype=torch.int64)
+    rng = np.random.default_rng(73)
+    for thr in (8, 2):
+        grp = LayerwiseTransferGroup(
+            num_gpus=1, gpu_blocks=[dev.gpu], cpu_blocks=dev.host, ssd_files={}, num_layers=L,
+            gpu_kv_strides_tensor=i64(s.gpu_kv_stride),
+            gpu_block_strides_tensor=i64(s.gpu_block_stride),
+            gpu_layer_strides_tensor=i64(s.gpu_layer_stride), gpu_chunk_sizes_tensor=i64(s.chunk),
+            iouring_entries=0, iouring_flags=0,
+            layer_eventfds_tensor=torch.empty(0, dtype=torch.int32), tp_size=1,
+            is_blockfirst=cpu_layout == "BLOCKFIRST", num_kv_heads=heads,
+            ce_segment_threshold=thr, ce_path_opt=path_opt, ce_enable_memcpy2d=memcpy2d)
+        for pattern in ("contiguous", "few_seg", "scattered"):
+            if pattern == "scattered":
+                gids, cids = block_ids(rng, N, n), block_ids(rng, NH, n)
+            else:
+                cids = block_ids(rng, NH, n, pattern)
+                gids = cids - cids.min() + int(rng.integers(0, N - (cids.max() - cids.min())))
+            for gran in (1, L):
+                fresh = rng.integers(0, 256, s.host_bytes, dtype=np.uint8)
+                s.host_ref[:] = fresh
+                dev.host.copy_(torch.from_numpy(fresh))
+                # the strategies themselves (the library's staging routes are covered elsewhere)
+                with launch_policy(staged_restore=0, staged_gather=0):
+                    grp.layerwise_transfer(
+                        e, e, 0, 0, 0, 0, 0, torch.as_tensor(gids), torch.as_tensor(cids),
+                        s.cpu_kv_stride, s.cpu_layer_stride, s.cpu_block_stride, s.chunk,
+                        s.cpu_kv_stride, s.cpu_layer_stride, s.cpu_block_stride, 4, True, L, gran,
+                        s.kv_dim, heads, counter_id=0, kv_shared_across_ranks_mode="sharded",
+                        notify_mode="polling")
+                    grp.synchronize()
+                taken = last_transfer_path()
+                if not path_opt:
+                    assert taken == "PER_BLOCK"
+                else:   # the last batch: layers [L - gran, L) of the call
+                    assert taken == expected_path(s, gids, cids, heads, thr, True, gran), \
+                        (pattern, thr, gran)
+                s.oracle_transfer(gids, cids, True)
+                dev.assert_matches_reference(f"{pattern} thr={thr} gran={gran} -> {taken}")
+        grp.close()
