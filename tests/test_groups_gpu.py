@@ -439,6 +439,99 @@ def _all_write_two_ranks(gpu_device):
     lw.close()
 
 
+# ---- several ranks through the layerwise group -----------------------------------------
+# tests/test_kv_transfer_correctness.py:906-1060 (test_non_mla_roundtrip_layerwise,
+# test_mla_roundtrip_modes_layerwise): a host pool as N ranks left it, read back by the
+# N ranks of a LayerwiseTransferGroup.  Here the ranks share device 0 and the expectation
+# comes from the oracle's placement rule and byte loop, rank by rank.
+@pytest.mark.parametrize("mode", ["sharded", "all_write", "rank0_only", "rank_rotate"])
+@pytest.mark.parametrize("kv_dim", [1, 2], ids=["mla", "kv_sep_1h"])
+@pytest.mark.parametrize("cpu_name", ["LAYERFIRST", "BLOCKFIRST"])
+@pytest.mark.parametrize("use_ce", [False, True], ids=["kernel", "ce"])
+def test_layerwise_restore_of_shared_kv_with_four_ranks(gpu_device, mode, kv_dim, cpu_name, use_ce):
+    """KV shared across ranks: every rank ends up with the same blocks; all_write ranks
+    read their own region; a mode that is no restore mode is treated as sharded
+    (csrc/layerwise.cpp:1112-1121)."""
+    n, L, N, T, H, D, heads = 4, 5, 12, 16, 1, 64, 1
+    copies = n if mode == "all_write" else 1
+    gl, cl = make_layouts(L, N, T, H, D, cpu_name, kv_dim, heads, cpu_blocks=N * copies)
+    rng = np.random.default_rng(21)
+    layer_bytes = kv_dim * N * T * H * D * ES
+    all_ref = [[rng.integers(0, 256, size=layer_bytes, dtype=np.uint8) for _ in range(L)]
+               for _ in range(n)]
+    all_gpu = [[torch.from_numpy(a.copy()).to(gpu_device) for a in rank] for rank in all_ref]
+    host_ref = rng.integers(0, 256, size=cl.get_total_elements() * ES, dtype=np.uint8)
+    cpu = torch.empty(host_ref.size, dtype=torch.uint8, pin_memory=True)
+    cpu.copy_(torch.from_numpy(host_ref))
+    cl_strides = (cl.get_kv_stride() * ES, cl.get_layer_stride() * ES, cl.get_block_stride() * ES,
+                  cl.get_block_stride() * ES // n)
+    ids_g = rng.permutation(N)[:7].astype(np.int64)
+    ids_c = rng.permutation(7 if mode == "all_write" else N)[:7].astype(np.int64)
+    lw = layerwise_group(cpu, all_gpu, gl, L, is_blockfirst=(cpu_name == "BLOCKFIRST"),
+                         num_kv_heads=heads)
+    for gran, notify in ((1, "polling"), (2, "hostfunc")):
+        run_layerwise(lw, torch.from_numpy(ids_g), torch.from_numpy(ids_c), cl,
+                      gl.get_chunk_size() * ES, L, kv_dim, heads, use_ce, gran, notify, mode=mode,
+                      tp_stride=cl_strides[3])
+        lw.synchronize()
+        oracle_mode = mode if mode in ("sharded", "all_write", "rank0_only") else "sharded"
+        _oracle_tp(all_ref, host_ref, gl, cl_strides, ids_g, ids_c, n, heads, True, oracle_mode, 0,
+                   0, 0, L, kv_dim)
+        for r in range(n):
+            for l in range(L):
+                np.testing.assert_array_equal(all_gpu[r][l].cpu().numpy(), all_ref[r][l],
+                                              err_msg=f"rank {r} layer {l} gran {gran}")
+        ids_g = rng.permutation(N)[:7].astype(np.int64)     # other blocks the second time
+    np.testing.assert_array_equal(cpu.numpy(), host_ref)    # a restore never writes the pool
+    lw.close()
+
+
+@pytest.mark.parametrize("kv_dim", [1, 2], ids=["packed", "plain"])
+@pytest.mark.parametrize("cpu_name", ["LAYERFIRST", "BLOCKFIRST"])
+@pytest.mark.parametrize("use_ce", [False, True], ids=["kernel", "ce"])
+def test_layerwise_restore_of_head_slices_with_four_ranks(gpu_device, kv_dim, cpu_name, use_ce):
+    """Multi-head KV: rank r reads its quarter of the heads out of every host chunk
+    (host offset r * cpu_tp_stride, csrc/layerwise.cpp:1143-1166)."""
+    n, L, N, T, H, D = 4, 4, 8, 16, 8, 32
+    gl = KVCacheLayout(KVCacheLayoutType.LAYERFIRST, L, N, T, H // n, D, kv_dim=kv_dim,
+                       num_kv_heads=H)
+    cl = KVCacheLayout(KVCacheLayoutType[cpu_name], L, N, T, H, D, kv_dim=kv_dim, num_kv_heads=H)
+    cl_tp = cl.div_head(n)
+    rng = np.random.default_rng(23)
+    per_layer = kv_dim * N * T * (H // n) * D * ES
+    all_ref = [[rng.integers(0, 256, size=per_layer, dtype=np.uint8) for _ in range(L)]
+               for _ in range(n)]
+    all_gpu = [[torch.from_numpy(a.copy()).to(gpu_device) for a in rank] for rank in all_ref]
+    host_ref = rng.integers(0, 256, size=cl.get_total_elements() * ES, dtype=np.uint8)
+    cpu = torch.empty(host_ref.size, dtype=torch.uint8, pin_memory=True)
+    cpu.copy_(torch.from_numpy(host_ref))
+    # the reference's workers pass the per-rank host strides and the full block stride
+    # (flexkv/transfer/worker.py:1199-1204)
+    strides = (cl_tp.get_kv_stride() * ES, cl_tp.get_layer_stride() * ES,
+               cl.get_block_stride() * ES, cl.get_block_stride() * ES // n)
+    ids_g = rng.permutation(N)[:5].astype(np.int64)
+    ids_c = rng.permutation(N)[:5].astype(np.int64)
+    lw = layerwise_group(cpu, all_gpu, gl, L, is_blockfirst=(cpu_name == "BLOCKFIRST"),
+                         num_kv_heads=H)
+    e = torch.empty(0, dtype=torch.int64)
+    for gran, notify in ((1, "polling"), (L, "hostfunc")):
+        lw.layerwise_transfer(
+            e, e, 0, 0, 0, 0, 0, torch.from_numpy(ids_g), torch.from_numpy(ids_c), strides[0],
+            strides[1], strides[2], gl.get_chunk_size() * ES, strides[0], strides[1], strides[3], 4,
+            use_ce, L, gran, kv_dim, H, counter_id=0, swa_h2d_src=e, swa_h2d_dst=e,
+            swa_disk2h_src=e, swa_disk2h_dst=e, kv_shared_across_ranks_mode="sharded",
+            notify_mode=notify)
+        lw.synchronize()
+        _oracle_tp(all_ref, host_ref, gl, strides, ids_g, ids_c, n, H, True, "sharded", 0, 0, 0, L,
+                   kv_dim)
+        for r in range(n):
+            for l in range(L):
+                np.testing.assert_array_equal(all_gpu[r][l].cpu().numpy(), all_ref[r][l],
+                                              err_msg=f"rank {r} layer {l} gran {gran}")
+        ids_g = rng.permutation(N)[:5].astype(np.int64)
+    lw.close()
+
+
 def test_layerwise_rejects_what_it_does_not_provide(gpu_device):
     from flexkv_amd.c_ext import LayerwiseTransferGroup
     L, N, T, H, D = 2, 4, 4, 1, 32
