@@ -423,3 +423,52 @@ def test_host_pool_adoption_falls_back_when_registration_is_refused(monkeypatch)
     assert w._host_registered == []
     assert w._adopt_host_pool(pool, "pool", allow_pageable=True) is pool
     assert w._pageable_host and w._host_registered == []
+
+
+# tests/test_transfer_worker_device_selection.py: the device is made current before the host
+# pool is registered with the runtime (registration maps the pool for the current device).
+class _RegistrationReached(Exception):
+    pass
+
+
+def _stop_at_first_host_registration(monkeypatch, events):
+    from flexkv_amd import host_buffer
+    from flexkv_amd.transfer import worker
+    monkeypatch.setattr(worker.torch.cuda, "set_device",
+                        lambda device: events.append(("set_device", device)))
+
+    def register(_tensor):
+        events.append(("register", None))
+        raise _RegistrationReached
+    monkeypatch.setattr(host_buffer, "cudaHostRegister", register)
+    monkeypatch.setenv("FKV_HOST_REGISTER", "1")
+
+
+def test_gpu_cpu_worker_selects_device_before_host_registration(monkeypatch):
+    from flexkv_amd.transfer.worker import GPUCPUTransferWorker
+    events = []
+    _stop_at_first_host_registration(monkeypatch, events)
+    with pytest.raises(_RegistrationReached):
+        GPUCPUTransferWorker(
+            worker_id=0, transfer_conn=None, finished_ops_queue=None,
+            op_buffer_tensor=torch.empty(0), gpu_blocks=[], cpu_blocks=torch.zeros(64, dtype=torch.uint8),
+            gpu_kv_layout=None, cpu_kv_layout=None, dtype=torch.bfloat16, gpu_device_id=3)
+    assert events == [("set_device", 3), ("register", None)]
+
+
+def test_tp_worker_selects_device_of_its_tensors_before_host_registration(monkeypatch):
+    from flexkv_amd.transfer.worker import tpGPUCPUTransferWorker
+    events = []
+    _stop_at_first_host_registration(monkeypatch, events)
+    handle = type("Handle", (), {"device": torch.device("cuda:4")})()
+    with pytest.raises(_RegistrationReached):
+        tpGPUCPUTransferWorker(
+            worker_id=0, transfer_conn=None, finished_ops_queue=None,
+            op_buffer_tensor=torch.empty(0), gpu_blocks=[[handle], [handle]],
+            cpu_blocks=torch.zeros(64, dtype=torch.uint8), gpu_kv_layouts=[], cpu_kv_layout=None,
+            dtype=torch.bfloat16, tp_group_size=2)
+    assert events and events[-1] == ("register", None)
+    selected = [e[1] for e in events[:-1]]
+    assert selected and all(e[0] == "set_device" for e in events[:-1])
+    last = selected[-1]                      # the device that is current when the pool is registered
+    assert (last.index if isinstance(last, torch.device) else last) == 4
