@@ -792,7 +792,8 @@ def run_multi_group(torch, device, steps, warmup, num_cta, notify, use_ce, verif
                      "512 blocks + 64 sidecar slots, page 256")}
 
 
-def run_worker_process(torch, device, steps, warmup, num_cta, use_ce, overlap=False):
+def run_worker_process(torch, device, steps, warmup, num_cta, use_ce, overlap=False,
+                       sweep_blocks=None, shuffle_ids=True):
     """c0-shaped put and get ops through a GPUCPUTransferWorker in its own process:
     what the pipe, the shared op pool and the completion queue add to a transfer.
     Then 8 puts and 8 gets of 64 blocks each, submitted together: one after the
@@ -873,9 +874,41 @@ def run_worker_process(torch, device, steps, warmup, num_cta, use_ce, overlap=Fa
             pool.free_slot(op.dst_slot_id)
         if it >= warmup:
             mixed.append(dt)
+    # one op at a time for a list of block counts, with the worker and its pool kept
+    # (benchmarks/benchmark_workers.py --sweep-blocks / --shuffle-ids, :441-470)
+    sweep = []
+    for count in sweep_blocks or ():
+        count = max(1, min(int(count), N))
+        if shuffle_ids:
+            g_ids = t.randperm(N, generator=gg)[:count].numpy().astype(np.int64)
+            c_ids = t.randperm(NH, generator=gg)[:count].numpy().astype(np.int64)
+        else:
+            g_ids = c_ids = np.arange(count, dtype=np.int64)
+        row = {"blocks": count, "bytes": count * L * 2 * T * H * D * 2, "shuffled_ids": bool(shuffle_ids)}
+        for kind, src, dst, name in ((TransferType.D2H, g_ids, c_ids, "put"),
+                                     (TransferType.H2D, c_ids, g_ids, "get")):
+            e2e, inside = [], []
+            for it in range(warmup + steps):
+                op = TransferOp(2000 + it, kind, src, dst)
+                op.src_slot_id = pool.allocate_slot(src, 1 if kind == TransferType.D2H else 2)
+                op.dst_slot_id = pool.allocate_slot(dst, 2 if kind == TransferType.D2H else 1)
+                t0 = time.perf_counter()
+                h.submit_transfer(op)
+                op_id, ok, m = q.get(timeout=300)
+                dt = (time.perf_counter() - t0) * 1e3
+                assert ok and op_id == op.op_id
+                pool.free_slot(op.src_slot_id)
+                pool.free_slot(op.dst_slot_id)
+                if it >= warmup:
+                    e2e.append(dt)
+                    inside.append(m["xfer_ms"])
+            row[name + "_e2e_ms"] = round(_median(e2e), 4)
+            row[name + "_worker_xfer_ms"] = round(_median(inside), 4)
+            row[name + "_GBps_e2e"] = round(row["bytes"] / (_median(e2e) * 1e-3) / 1e9, 3)
+        sweep.append(row)
     h.shutdown()
     med = lambda xs: _median(list(xs))
-    res = {"bytes_per_op": nbytes, "wall_s": wall, "exit_code": h.process.exitcode,
+    res = {"bytes_per_op": nbytes, "wall_s": wall, "exit_code": h.process.exitcode, "sweep": sweep,
            "mixed": {"ops": 2 * m_ops, "blocks_per_op": m_blocks, "bytes": mixed_bytes,
                      "overlap_directions": bool(overlap),
                      "ms": round(med(mixed) * 1e3, 3),
@@ -1375,6 +1408,11 @@ def main():
     ap.add_argument("--fragmented", action="store_true",
                     help="mg: host pools of 4096 / 512 blocks with the blocks to restore scattered "
                          "over them (default: pools of 512 / 64 blocks, all of them restored)")
+    ap.add_argument("--sweep-blocks", default=None, metavar="N,N,...",
+                    help="--config worker: also one put and one get at a time for each of these "
+                         "block counts (at most 1024), worker and pool kept")
+    ap.add_argument("--sequential-ids", action="store_true",
+                    help="--sweep-blocks with block ids 0..n-1 on both sides instead of shuffled ones")
     ap.add_argument("--overlap-directions", action="store_true",
                     help="worker: the worker runs gets next to puts (second thread and stream)")
     ap.add_argument("--layer-spans", action="store_true",
@@ -1514,8 +1552,10 @@ def main():
         return
     if args.config == "worker":
         link = measure_link()
+        counts = [int(x) for x in args.sweep_blocks.split(",")] if args.sweep_blocks else None
         r = run_worker_process(torch, device, args.steps, args.warmup, args.num_cta, args.use_ce,
-                               overlap=args.overlap_directions)
+                               overlap=args.overlap_directions, sweep_blocks=counts,
+                               shuffle_ids=not args.sequential_ids)
         print(json.dumps({
             "metric": "put/get through a transfer worker process: GB/s seen by the submitter",
             "unit": "GB/s", "value": round(2 * r["bytes_per_op"] * args.steps / r["wall_s"] / 1e9, 3),
@@ -1529,6 +1569,7 @@ def main():
                        "transfer_num_cta": args.num_cta},
             "put": r["D2H"], "get": r["H2D"], "bytes_per_op": r["bytes_per_op"],
             "puts_and_gets_submitted_together": r["mixed"],
+            "sweep_blocks": r["sweep"],
             "worker_exit_code": r["exit_code"],
             "link_peak": {"d2h_GBps": round(link["d2h"], 3), "h2d_GBps": round(link["h2d"], 3)}}))
         return
