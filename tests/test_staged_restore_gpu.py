@@ -423,3 +423,46 @@ def test_the_choice_follows_the_runs_of_host_blocks(gpu_device):
             s.oracle_transfer(gids, cids, True)
             dev.assert_matches_reference(pattern)
     grp.close()
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_seeded_random_restores(gpu_device, seed):
+    """Shape, host layout, id pattern, granularity, layer prefix, route, engine asked for,
+    notify mode and ring sizes drawn from a seed; two restores through the same group with
+    fresh host bytes, every byte against the oracle."""
+    from flexkv_amd.c_ext import launch_policy
+    rng = np.random.default_rng(3000 + seed)
+    backend = int(rng.choice([VLLM, TRTLLM, SGLANG]))
+    L = int(rng.integers(1, 21))
+    kv_dim = 2 if backend == SGLANG else int(rng.choice([1, 2]))
+    NG, NC = int(rng.integers(8, 100)), int(rng.integers(8, 100))
+    gran16 = rng.random() < 0.8
+    chunk = 16 * int(rng.integers(1, 700)) if gran16 else 8 * int(rng.integers(1, 60)) + int(rng.choice([0, 4, 2]))
+    cpu_layout = str(rng.choice(["BLOCKFIRST", "LAYERFIRST"]))
+    n = int(rng.integers(1, min(NG, NC) + 1))
+    gran = int(rng.integers(1, L + 1))
+    layers = int(rng.integers(1, L + 1))
+    route = str(rng.choice(list(ROUTES) + ["default"]))
+    use_ce = bool(rng.random() < 0.3) and chunk % 8 == 0
+    policy = dict(ROUTES.get(route, {}), staged_ring=int(rng.integers(2, 5)),
+                  gather_ring=int(rng.integers(2, 5)), gather_threads=int(rng.integers(2, 6)))
+    s = KVSetup(backend, L, kv_dim, NG, NC, chunk, cpu_layout, seed=4000 + seed)
+    dev = s.to_device(gpu_device)
+    grp = group_of(s, dev)
+    print("case", dict(backend=backend, L=L, kv_dim=kv_dim, NG=NG, NC=NC, chunk=chunk,
+                       cpu_layout=cpu_layout, n=n, gran=gran, layers=layers, route=route,
+                       use_ce=use_ce, policy=policy), flush=True)
+    with launch_policy(**policy):
+        for rep in range(2):
+            fresh = rng.integers(0, 256, s.host_bytes, dtype=np.uint8)
+            s.host_ref[:] = fresh
+            dev.host.copy_(torch.from_numpy(fresh))
+            gids = rng.permutation(NG)[:n].astype(np.int64)
+            cids = host_ids(rng, NC, n, str(rng.choice(["one_run", "runs_and_holes", "scattered"])))
+            if cids.size < n:           # runs_and_holes may run out of pool
+                gids = gids[:cids.size]
+            restore(grp, s, gids, cids, gran, notify=str(rng.choice(["polling", "hostfunc"])),
+                    num_layers=layers, use_ce=use_ce)
+            s.oracle_transfer(gids, cids, True, num_layers=layers)
+            dev.assert_matches_reference(f"restore {rep}")
+    grp.close()

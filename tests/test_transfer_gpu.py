@@ -678,3 +678,72 @@ def test_several_transfers_in_one_call_edge_cases(gpu_device):
         transfer_kv_blocks_multi([call(da, g, c, False), call(db, c, g, True)])
     da.assert_matches_reference("refused call")
     db.assert_matches_reference("refused call")
+
+
+# ---- seeded random cases: every engine and entry point against the oracle ---------------
+def _random_case(seed):
+    rng = np.random.default_rng(1000 + seed)
+    backend = int(rng.choice([VLLM, TRTLLM, SGLANG]))
+    L, K = int(rng.integers(1, 7)), int(rng.choice([1, 2]))
+    if backend == SGLANG:
+        K = 2
+    N, NH = int(rng.integers(4, 90)), int(rng.integers(4, 90))
+    gran = int(rng.choice([16, 16, 16, 8, 4, 2, 1]))          # vector width the chunk allows
+    chunk = gran * int(rng.integers(1, 1 + 20000 // gran)) if rng.random() < 0.7 else \
+        gran * int(rng.integers(1, 40))
+    if gran < 16 and chunk % (2 * gran) == 0:
+        chunk += gran
+    cpu_layout = str(rng.choice(["BLOCKFIRST", "LAYERFIRST"]))
+    gpu_layout = str(rng.choice(["LAYERFIRST", "LAYERBLOCK"])) if backend == VLLM else "LAYERFIRST"
+    pad = int(rng.choice([0, 0, 16 * int(rng.integers(1, 9))])) if gran == 16 else 0
+    n = int(rng.integers(1, min(N, NH) + 1))
+    start = int(rng.integers(0, L))
+    nl = int(rng.integers(1, L - start + 1))
+    # an in-chunk window, as a rank that moves its share of every chunk would ask for
+    if rng.random() < 0.3 and chunk >= 4 * gran:
+        sub = gran * int(rng.integers(1, chunk // gran))
+        g_off = gran * int(rng.integers(0, (chunk - sub) // gran + 1))
+        c_off = gran * int(rng.integers(0, (chunk - sub) // gran + 1))
+    else:
+        sub, g_off, c_off = chunk, 0, 0
+    return dict(backend=backend, L=L, K=K, N=N, NH=NH, chunk=chunk, cpu_layout=cpu_layout,
+                gpu_layout=gpu_layout, pad=pad, n=n, start=start, nl=nl, sub=sub, g_off=g_off,
+                c_off=c_off, rng=rng)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_seeded_random_cases_on_every_engine(gpu_device, seed):
+    """Shapes, strides, id lists, layer ranges and in-chunk windows drawn from a seed: a put
+    and a get on the kernel path (two workgroup counts), through the copy-engine strategies
+    (the library's choice and per-block copies; whole chunks with 8-byte granularity, which
+    is their domain) and through the entry point that allocates nothing, each compared with
+    the oracle byte for byte on the whole host pool and every engine tensor."""
+    c = _random_case(seed)
+    rng = c["rng"]
+    s = KVSetup(c["backend"], c["L"], c["K"], c["N"], c["NH"], c["chunk"], c["cpu_layout"],
+                c["gpu_layout"], seed=2000 + seed, gpu_block_pad=c["pad"])
+    dev = s.to_device(gpu_device)
+    print("case", {k: v for k, v in c.items() if k != "rng"}, flush=True)
+    engines = [dict(num_cta=1), dict(num_cta=int(rng.integers(2, 40))),
+               dict(entry="fkv_transfer_kv_blocks_noalloc")]
+    if c["sub"] == c["chunk"] and c["chunk"] % 8 == 0:
+        engines += [dict(use_ce=True, ce=dict(path_opt_enabled=1)),
+                    dict(use_ce=True, ce=dict(path_opt_enabled=1, enable_memcpy2d=1,
+                                              segment_threshold=2)),
+                    dict(use_ce=True, ce=dict(path_opt_enabled=0))]
+    for kw in engines:
+        gids = rng.permutation(c["N"])[:c["n"]].astype(np.int64)
+        cids = rng.permutation(c["NH"])[:c["n"]].astype(np.int64)
+        for h2d in (False, True):
+            rc = dev.transfer_raw(gids, cids, h2d, start_layer=c["start"], num_layers=c["nl"],
+                                  gpu_off=c["g_off"], cpu_off=c["c_off"], chunk=c["sub"], **kw)
+            assert rc == 0, (kw, h2d, _last_error())
+            s.oracle_transfer(gids, cids, h2d, start_layer=c["start"], num_layers=c["nl"],
+                              gpu_off=c["g_off"], cpu_off=c["c_off"], chunk=c["sub"])
+            dev.assert_matches_reference(f"{kw} h2d={h2d}")
+            gids = rng.permutation(c["N"])[:c["n"]].astype(np.int64)   # the get lands elsewhere
+
+
+def _last_error():
+    from flexkv_amd import _lib
+    return _lib.last_error()
