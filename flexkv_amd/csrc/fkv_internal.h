@@ -338,7 +338,8 @@ struct StagedPlan {
 // `kernel_allowed`: the caller lets batches go by kernel (the first batch of a gathered restore).
 int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &ring,
                       GatherRing &pinned, hipStream_t scatter_stream, StagedPlan *out,
-                      bool host_visible = true, bool kernel_allowed = true);
+                      bool host_visible = true, bool kernel_allowed = true,
+                      bool several_gpus = false);
 // The choice alone (no device): kRouteKernel, kRouteRuns (fills `segs` and `total_rows`)
 // or kRouteGathered.
 int staged_route(const int64_t *cpu_ids, int num_blocks, int64_t row_bytes, int pieces,

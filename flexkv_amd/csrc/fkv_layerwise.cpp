@@ -941,7 +941,7 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
       rc = staged_plan_build(d, g->multi_group ? 1 : c.layer_granularity,
                              g->rings[{lane_index, i}], g->pinned_rings[{lane_index, i}],
                              g->streams[i], &lane.staged[i], lane.plans[i].host_visible,
-                             /*kernel_allowed=*/direct);
+                             /*kernel_allowed=*/direct, /*several_gpus=*/g->num_gpus > 1);
       if (rc == FKV_OK && lane.staged[i].usable && !g->dma_streams[i]) {
         hipError_t e = hipStreamCreateWithFlags(&g->dma_streams[i], hipStreamNonBlocking);
         if (e != hipSuccess) {

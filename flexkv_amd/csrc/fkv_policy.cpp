@@ -159,7 +159,7 @@ void sanitize(fkv_launch_policy &p, const fkv_launch_policy &derived) {
   p.model_launch_ns = clampi(p.model_launch_ns, 0, 10000000);
   p.model_prefer_ce_pct = clampi(p.model_prefer_ce_pct, 1, 1000);
   p.d2h_lane_runs = clampi(p.d2h_lane_runs, 0, 2);
-  p.staged_gather = clampi(p.staged_gather, 0, 2);
+  p.staged_gather = clampi(p.staged_gather, 0, 3);
   p.gather_threads = clampi(p.gather_threads, 1, 64);
   p.gather_ring = clampi(p.gather_ring, 2, 8);
   p.gather_first_by_kernel = p.gather_first_by_kernel != 0;

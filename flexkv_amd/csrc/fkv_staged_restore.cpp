@@ -265,7 +265,7 @@ int64_t staged_row_of(const std::vector<StagedPlan::Seg> &segs, int64_t id) {
 
 int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &ring,
                       GatherRing &pinned, hipStream_t scatter_stream, StagedPlan *out,
-                      bool host_visible, bool kernel_allowed) {
+                      bool host_visible, bool kernel_allowed, bool several_gpus) {
   *out = StagedPlan{};
   int device = 0;
   FKV_HIP_TRY(hipGetDevice(&device));
@@ -273,6 +273,13 @@ int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &
   fkv_launch_policy pol = policy_of_seeded(device);
   if (!host_visible) // a pageable pool: the copy engines cannot take its rows, host threads can
     pol.staged_restore = 0;
+  // Rows gathered by host threads are for groups of one GPU, unless the policy says 3: the
+  // launching thread would gather for one GPU after the other (the same rows again where
+  // the ranks share their KV), and the route has not run on several devices.
+  if (pol.staged_gather == 3)
+    pol.staged_gather = 2;
+  else if (several_gpus)
+    pol.staged_gather = 0;
   if ((pol.staged_restore == 0 && pol.staged_gather == 0) || d.num_blocks <= 0 ||
       d.num_layers <= 0 || batch_layers < 1)
     return FKV_OK;

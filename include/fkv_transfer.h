@@ -730,7 +730,11 @@ typedef struct fkv_launch_policy {
   int32_t staged_gather;      /* FKV_STAGED_GATHER: 0 never; 1 (default) where the host blocks form
                                  too many runs for one copy command each and the gather threads
                                  keep up with the link; 2 whenever the copies-per-run route is
-                                 not taken */
+                                 not taken.  Both in groups of one GPU only: with several, the
+                                 launching thread would gather for one GPU after the other (the
+                                 same rows again where the ranks share their KV), and the route
+                                 has run on one device only.  3 = like 2, groups of several GPUs
+                                 included (host-side tests) */
   int32_t gather_threads;     /* FKV_GATHER_THREADS: host threads that gather (the launching thread
                                  of the restore is one of them); default 6, at most the cores of
                                  the machine less one */

@@ -1,0 +1,499 @@
+// A HIP runtime made of host threads, for sanitizer builds of the library's host code.
+//
+// Test infrastructure only: it stands in for libamdhip64 and for the library's kernels so
+// that the host side of the library (plans, rings, launching thread, gates, pollers, the
+// copy-engine strategies) runs whole under AddressSanitizer / UndefinedBehaviorSanitizer /
+// ThreadSanitizer on a machine without a GPU.
+//
+//  * "Device memory" and pinned host memory are aligned host allocations kept in a table,
+//    so a kernel stand-in dereferences what the library hands it and the sanitizers see
+//    every access.  hipPointerGetAttributes / hipHostGetDevicePointer answer from the table;
+//    memory that is not in it is pageable.
+//  * A stream is a thread with a queue: commands run in order and asynchronously to the
+//    host, as on the device.  The null stream is one more such stream.
+//  * An event is a pair of counters (recorded, completed) under a mutex: a stream waits for
+//    the record that was current when the wait was enqueued, an event that was never
+//    recorded reads as complete, as in HIP.  Every hand-over goes through that mutex, so
+//    ThreadSanitizer sees exactly the ordering a HIP program may rely on: work that is not
+//    ordered by stream order, an event or a synchronize shows up as a race.
+//  * The copy kernel stand-ins do what the kernels do (rows of `chunk_bytes` between base
+//    tables and block ids) with memcpy, on the stream's thread.
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <atomic>
+#include <chrono>
+#include <condition_variable>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <deque>
+#include <functional>
+#include <map>
+#include <mutex>
+#include <thread>
+#include <vector>
+
+#include "fkv_internal.h"
+
+// ---- streams ----------------------------------------------------------------------
+struct ihipStream_t {
+  std::mutex mu;
+  std::condition_variable wake, idle;
+  std::deque<std::function<void()>> queue;
+  bool busy = false, quit = false;
+  std::thread worker;
+  ihipStream_t() : worker([this] { run(); }) {}
+  ~ihipStream_t() {
+    {
+      std::unique_lock<std::mutex> lk(mu);
+      idle.wait(lk, [this] { return queue.empty() && !busy; });
+      quit = true;
+    }
+    wake.notify_all();
+    worker.join();
+  }
+  void run() {
+    for (;;) {
+      std::function<void()> op;
+      {
+        std::unique_lock<std::mutex> lk(mu);
+        wake.wait(lk, [this] { return quit || !queue.empty(); });
+        if (queue.empty())
+          return;
+        op = std::move(queue.front());
+        queue.pop_front();
+        busy = true;
+      }
+      op();
+      {
+        std::lock_guard<std::mutex> lk(mu);
+        busy = false;
+        if (queue.empty())
+          idle.notify_all();
+      }
+    }
+  }
+  void push(std::function<void()> op) {
+    {
+      std::lock_guard<std::mutex> lk(mu);
+      queue.push_back(std::move(op));
+    }
+    wake.notify_one();
+  }
+  void drain() {
+    std::unique_lock<std::mutex> lk(mu);
+    idle.wait(lk, [this] { return queue.empty() && !busy; });
+  }
+  bool is_idle() {
+    std::lock_guard<std::mutex> lk(mu);
+    return queue.empty() && !busy;
+  }
+};
+
+struct ihipEvent_t {
+  std::mutex mu;
+  std::condition_variable cv;
+  uint64_t recorded = 0, completed = 0;
+  std::chrono::steady_clock::time_point when{};
+};
+
+namespace {
+
+thread_local int t_device = 0;
+thread_local hipError_t t_last = hipSuccess;
+constexpr int kDevices = 2;
+
+hipError_t remember(hipError_t e) {
+  if (e != hipSuccess)
+    t_last = e;
+  return e;
+}
+
+struct Runtime {
+  std::mutex mu;
+  std::vector<ihipStream_t *> streams; // every live stream, the null stream first
+  struct Block {
+    size_t size;
+    bool pinned;
+    bool registered; // pinned by hipHostRegister: memory of the caller
+  };
+  std::map<uintptr_t, Block> memory;
+  ihipStream_t *null_stream() {
+    std::lock_guard<std::mutex> lk(mu);
+    if (streams.empty())
+      streams.push_back(new ihipStream_t());
+    return streams[0];
+  }
+  const std::pair<const uintptr_t, Block> *find(const void *p) {
+    std::lock_guard<std::mutex> lk(mu);
+    auto it = memory.upper_bound((uintptr_t)p);
+    if (it == memory.begin())
+      return nullptr;
+    --it;
+    return (uintptr_t)p < it->first + it->second.size ? &*it : nullptr;
+  }
+  void drain_all() {
+    std::vector<ihipStream_t *> all;
+    {
+      std::lock_guard<std::mutex> lk(mu);
+      all = streams;
+    }
+    for (ihipStream_t *s : all)
+      s->drain();
+  }
+  ~Runtime() {
+    for (ihipStream_t *s : streams)
+      delete s;
+  }
+};
+Runtime &rt() {
+  static Runtime r;
+  return r;
+}
+ihipStream_t *of(hipStream_t s) { return s ? s : rt().null_stream(); }
+
+void *allocate(size_t size, bool pinned) {
+  // 2 MiB alignment, as the runtime gives large allocations
+  void *p = nullptr;
+  if (posix_memalign(&p, (size_t)2 << 20, std::max<size_t>(size, 64)) != 0)
+    return nullptr;
+  std::lock_guard<std::mutex> lk(rt().mu);
+  rt().memory[(uintptr_t)p] = Runtime::Block{std::max<size_t>(size, 64), pinned, false};
+  return p;
+}
+
+hipError_t release(void *p, bool pinned) {
+  if (!p)
+    return hipSuccess;
+  rt().drain_all(); // hipFree waits for the device
+  {
+    std::lock_guard<std::mutex> lk(rt().mu);
+    auto it = rt().memory.find((uintptr_t)p);
+    if (it == rt().memory.end() || it->second.pinned != pinned || it->second.registered)
+      return remember(hipErrorInvalidValue);
+    rt().memory.erase(it);
+  }
+  free(p);
+  return hipSuccess;
+}
+
+void copy_2d(void *dst, size_t dpitch, const void *src, size_t spitch, size_t width, size_t height) {
+  for (size_t r = 0; r < height; ++r)
+    std::memcpy(static_cast<char *>(dst) + r * dpitch, static_cast<const char *>(src) + r * spitch,
+                width);
+}
+
+} // namespace
+
+extern "C" {
+
+hipError_t hipGetLastError(void) {
+  hipError_t e = t_last;
+  t_last = hipSuccess;
+  return e;
+}
+const char *hipGetErrorString(hipError_t e) {
+  switch (e) {
+  case hipSuccess: return "no error";
+  case hipErrorNotReady: return "device not ready";
+  case hipErrorInvalidValue: return "invalid argument";
+  case hipErrorOutOfMemory: return "out of memory";
+  case hipErrorNotSupported: return "operation not supported";
+  default: return "emulated runtime error";
+  }
+}
+hipError_t hipGetDevice(int *d) {
+  *d = t_device;
+  return hipSuccess;
+}
+hipError_t hipSetDevice(int d) {
+  if (d < 0 || d >= kDevices)
+    return remember(hipErrorInvalidDevice);
+  t_device = d;
+  return hipSuccess;
+}
+hipError_t hipDeviceGetPCIBusId(char *id, int len, int device) {
+  snprintf(id, (size_t)len, "0000:%02x:00.0", device);
+  return hipSuccess;
+}
+
+hipError_t hipStreamCreateWithFlags(hipStream_t *s, unsigned int) {
+  *s = new ihipStream_t();
+  std::lock_guard<std::mutex> lk(rt().mu);
+  if (rt().streams.empty())
+    rt().streams.push_back(new ihipStream_t());
+  rt().streams.push_back(*s);
+  return hipSuccess;
+}
+hipError_t hipStreamCreate(hipStream_t *s) { return hipStreamCreateWithFlags(s, 0); }
+hipError_t hipStreamDestroy(hipStream_t s) {
+  if (!s)
+    return remember(hipErrorInvalidHandle);
+  {
+    std::lock_guard<std::mutex> lk(rt().mu);
+    auto &v = rt().streams;
+    v.erase(std::remove(v.begin(), v.end(), s), v.end());
+  }
+  delete s; // finishes what is queued, as the runtime does
+  return hipSuccess;
+}
+hipError_t hipStreamSynchronize(hipStream_t s) {
+  of(s)->drain();
+  return hipSuccess;
+}
+hipError_t hipStreamQuery(hipStream_t s) { return of(s)->is_idle() ? hipSuccess : hipErrorNotReady; }
+
+hipError_t hipEventCreateWithFlags(hipEvent_t *e, unsigned int) {
+  *e = new ihipEvent_t();
+  return hipSuccess;
+}
+hipError_t hipEventCreate(hipEvent_t *e) { return hipEventCreateWithFlags(e, 0); }
+hipError_t hipEventDestroy(hipEvent_t e) {
+  if (!e)
+    return remember(hipErrorInvalidHandle);
+  {
+    // whoever completes a record of this event does so under its mutex
+    std::unique_lock<std::mutex> lk(e->mu);
+    e->cv.wait(lk, [e] { return e->completed >= e->recorded; });
+  }
+  delete e;
+  return hipSuccess;
+}
+hipError_t hipEventRecord(hipEvent_t e, hipStream_t s) {
+  if (!e)
+    return remember(hipErrorInvalidHandle);
+  uint64_t gen;
+  {
+    std::lock_guard<std::mutex> lk(e->mu);
+    gen = ++e->recorded;
+  }
+  of(s)->push([e, gen] {
+    std::lock_guard<std::mutex> lk(e->mu);
+    e->completed = std::max(e->completed, gen);
+    e->when = std::chrono::steady_clock::now();
+    e->cv.notify_all();
+  });
+  return hipSuccess;
+}
+hipError_t hipEventQuery(hipEvent_t e) {
+  if (!e)
+    return remember(hipErrorInvalidHandle);
+  std::lock_guard<std::mutex> lk(e->mu);
+  return e->completed >= e->recorded ? hipSuccess : hipErrorNotReady;
+}
+hipError_t hipEventSynchronize(hipEvent_t e) {
+  if (!e)
+    return remember(hipErrorInvalidHandle);
+  std::unique_lock<std::mutex> lk(e->mu);
+  const uint64_t gen = e->recorded;
+  e->cv.wait(lk, [e, gen] { return e->completed >= gen; });
+  return hipSuccess;
+}
+hipError_t hipStreamWaitEvent(hipStream_t s, hipEvent_t e, unsigned int) {
+  if (!e)
+    return remember(hipErrorInvalidHandle);
+  uint64_t gen;
+  {
+    std::lock_guard<std::mutex> lk(e->mu);
+    gen = e->recorded;
+  }
+  of(s)->push([e, gen] {
+    std::unique_lock<std::mutex> lk(e->mu);
+    e->cv.wait(lk, [e, gen] { return e->completed >= gen; });
+  });
+  return hipSuccess;
+}
+hipError_t hipEventElapsedTime(float *ms, hipEvent_t a, hipEvent_t b) {
+  if (!a || !b)
+    return remember(hipErrorInvalidHandle);
+  std::chrono::steady_clock::time_point ta, tb;
+  {
+    std::lock_guard<std::mutex> lk(a->mu);
+    if (a->recorded == 0)
+      return remember(hipErrorInvalidHandle);
+    if (a->completed < a->recorded)
+      return remember(hipErrorNotReady);
+    ta = a->when;
+  }
+  {
+    std::lock_guard<std::mutex> lk(b->mu);
+    if (b->recorded == 0)
+      return remember(hipErrorInvalidHandle);
+    if (b->completed < b->recorded)
+      return remember(hipErrorNotReady);
+    tb = b->when;
+  }
+  *ms = std::chrono::duration<float, std::milli>(tb - ta).count();
+  return hipSuccess;
+}
+
+hipError_t hipMalloc(void **p, size_t size) {
+  *p = allocate(size, false);
+  return *p ? hipSuccess : remember(hipErrorOutOfMemory);
+}
+hipError_t hipFree(void *p) { return release(p, false); }
+hipError_t hipHostMalloc(void **p, size_t size, unsigned int) {
+  *p = allocate(size, true);
+  return *p ? hipSuccess : remember(hipErrorOutOfMemory);
+}
+hipError_t hipHostFree(void *p) { return release(p, true); }
+hipError_t hipHostRegister(void *p, size_t size, unsigned int) {
+  if (!p || size == 0)
+    return remember(hipErrorInvalidValue);
+  std::lock_guard<std::mutex> lk(rt().mu);
+  rt().memory[(uintptr_t)p] = Runtime::Block{size, true, true};
+  return hipSuccess;
+}
+hipError_t hipHostUnregister(void *p) {
+  rt().drain_all();
+  std::lock_guard<std::mutex> lk(rt().mu);
+  auto it = rt().memory.find((uintptr_t)p);
+  if (it == rt().memory.end() || !it->second.registered)
+    return remember(hipErrorHostMemoryNotRegistered);
+  rt().memory.erase(it);
+  return hipSuccess;
+}
+hipError_t hipHostGetDevicePointer(void **dev, void *host, unsigned int) {
+  const auto *b = rt().find(host);
+  if (!b || !b->second.pinned)
+    return remember(hipErrorInvalidValue);
+  *dev = host;
+  return hipSuccess;
+}
+hipError_t hipPointerGetAttributes(hipPointerAttribute_t *at, const void *p) {
+  const auto *b = rt().find(p);
+  if (!b)
+    return remember(hipErrorInvalidValue);
+  std::memset(at, 0, sizeof(*at));
+  at->type = b->second.pinned ? hipMemoryTypeHost : hipMemoryTypeDevice;
+  at->device = 0;
+  at->devicePointer = const_cast<void *>(p);
+  at->hostPointer = b->second.pinned ? const_cast<void *>(p) : nullptr;
+  return hipSuccess;
+}
+hipError_t hipMemGetAddressRange(hipDeviceptr_t *base, size_t *size, hipDeviceptr_t p) {
+  const auto *b = rt().find(p);
+  if (!b)
+    return remember(hipErrorInvalidValue);
+  if (base)
+    *base = (hipDeviceptr_t)b->first;
+  if (size)
+    *size = b->second.size;
+  return hipSuccess;
+}
+
+hipError_t hipMemcpyAsync(void *dst, const void *src, size_t n, hipMemcpyKind, hipStream_t s) {
+  of(s)->push([dst, src, n] { std::memcpy(dst, src, n); });
+  return hipSuccess;
+}
+hipError_t hipMemcpy(void *dst, const void *src, size_t n, hipMemcpyKind) {
+  rt().null_stream()->drain();
+  std::memcpy(dst, src, n);
+  return hipSuccess;
+}
+hipError_t hipMemcpy2DAsync(void *dst, size_t dpitch, const void *src, size_t spitch, size_t width,
+                            size_t height, hipMemcpyKind, hipStream_t s) {
+  if (width > dpitch || width > spitch)
+    return remember(hipErrorInvalidPitchValue);
+  of(s)->push([=] { copy_2d(dst, dpitch, src, spitch, width, height); });
+  return hipSuccess;
+}
+hipError_t hipMemsetAsync(void *dst, int value, size_t n, hipStream_t s) {
+  of(s)->push([dst, value, n] { std::memset(dst, value, n); });
+  return hipSuccess;
+}
+
+hipError_t hipIpcGetMemHandle(hipIpcMemHandle_t *, void *) { return remember(hipErrorNotSupported); }
+hipError_t hipIpcOpenMemHandle(void **, hipIpcMemHandle_t, unsigned int) {
+  return remember(hipErrorNotSupported);
+}
+hipError_t hipIpcCloseMemHandle(void *) { return remember(hipErrorNotSupported); }
+
+} // extern "C"
+
+// ---- the library's kernels, on the stream's thread ------------------------------------
+namespace fkv {
+
+namespace {
+// What fkv_copy_chunks_kernel does: row (i, p) of `chunk_bytes` from
+// base_src[i] + ids_src[p] * stride_src to base_dst[i] + ids_dst[p] * stride_dst; a null id
+// list stands for 0, 1, 2, ...
+void copy_rows(const CopyKernelArgs &a) {
+  for (int i = 0; i < a.lk; ++i)
+    for (int p = 0; p < a.num_blocks; ++p) {
+      const int64_t s = a.ids_src ? a.ids_src[p] : p, d = a.ids_dst ? a.ids_dst[p] : p;
+      std::memcpy(reinterpret_cast<void *>((uintptr_t)a.base_dst[i] + (uintptr_t)(d * a.stride_dst)),
+                  reinterpret_cast<const void *>((uintptr_t)a.base_src[i] + (uintptr_t)(s * a.stride_src)),
+                  (size_t)a.chunk_bytes);
+    }
+}
+std::atomic<uint64_t> g_launches{0};
+} // namespace
+
+int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_workgroup,
+                       hipStream_t stream) {
+  if (a.num_blocks < 0 || a.lk < 0 || a.lk > kCopyMaxLK || a.chunk_bytes < 0 || num_workgroups < 1 ||
+      threads_per_workgroup < 1)
+    return fail(FKV_ERR_RUNTIME, "emulated copy kernel: bad launch");
+  g_launches.fetch_add(1);
+  stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);
+  of(stream)->push([a] { copy_rows(a); });
+  return FKV_OK;
+}
+
+int launch_copy_jobs(const CopyKernelArgs *jobs, int njobs, int num_workgroups,
+                     int threads_per_workgroup, hipStream_t stream) {
+  if (njobs < 1 || njobs > kCopyMaxJobs)
+    return fail(FKV_ERR_RUNTIME, "copy kernel: %d jobs in one launch (1..%d)", njobs, kCopyMaxJobs);
+  std::vector<CopyKernelArgs> all(jobs, jobs + njobs);
+  stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);
+  of(stream)->push([all] {
+    for (const CopyKernelArgs &a : all)
+      copy_rows(a);
+  });
+  return FKV_OK;
+}
+
+uint64_t safety_net_ranges_of_current_device() { return 0; }
+
+int launch_plan_upload(void *device_dst, const void *pinned_src, size_t bytes, hipStream_t stream) {
+  of(stream)->push([=] { std::memcpy(device_dst, pinned_src, bytes); });
+  return FKV_OK;
+}
+
+int probe_xcds(uint32_t *present_mask) {
+  *present_mask = 0xffu;
+  return FKV_OK;
+}
+
+int common_vector_width(const uint64_t *vals, int n) {
+  uint64_t acc = 0;
+  for (int i = 0; i < n; ++i)
+    acc |= vals[i];
+  for (int w = 16; w > 1; w >>= 1)
+    if (acc % (uint64_t)w == 0)
+      return w;
+  return 1;
+}
+
+} // namespace fkv
+
+// Entry points of the library that live beside its kernels: not part of what runs here.
+extern "C" {
+int fkv_measure_hbm_rate(int32_t, size_t, int32_t, int32_t, double *, double *) {
+  return fkv::fail(FKV_ERR_UNSUPPORTED, "emulated runtime: no HBM to measure");
+}
+int fkv_streams_run_concurrently(int32_t, void *, void *, int32_t *) {
+  return fkv::fail(FKV_ERR_UNSUPPORTED, "emulated runtime: no hardware queues");
+}
+int fkv_transfer_kv_blocks_noalloc(const fkv_transfer_desc *, void *) {
+  return fkv::fail(FKV_ERR_UNSUPPORTED, "emulated runtime: the entry point lives beside the kernels");
+}
+int fkv_build_gpu_chunk_ptrs(const fkv_chunk_ptrs_desc *, void *) {
+  return fkv::fail(FKV_ERR_UNSUPPORTED, "emulated runtime: the entry point lives beside the kernels");
+}
+int fkv_staging_transfer(const fkv_staging_transfer_desc *, void *) {
+  return fkv::fail(FKV_ERR_UNSUPPORTED, "emulated runtime: the entry point lives beside the kernels");
+}
+}

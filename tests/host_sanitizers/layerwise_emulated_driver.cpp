@@ -1,0 +1,418 @@
+// The library's whole host side over the emulated HIP runtime (emulated_hip_runtime.cpp),
+// for sanitizer builds: layerwise restores with several ranks on every route (kernel, one
+// copy per run of host blocks, rows gathered by host threads), asked for on the kernel and
+// on the copy engine, from pinned and pageable host pools, in both notify modes with
+// eventfds, consumer streams gated per layer, restores made to give up part-way; and plain
+// puts and gets on the kernel path and through every copy-engine strategy.  Every result is
+// compared with a plain model of the addressing (vLLM-style tensors per layer).
+#include <hip/hip_runtime_api.h>
+#include <sys/eventfd.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <numeric>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "fkv_transfer.h"
+
+#define REQUIRE(cond, ...)                                                                          \
+  do {                                                                                              \
+    if (!(cond)) {                                                                                  \
+      fprintf(stderr, "FAILED %s:%d: %s\n  ", __FILE__, __LINE__, #cond);                           \
+      fprintf(stderr, __VA_ARGS__);                                                                 \
+      fprintf(stderr, "\n  last error: %s\n", fkv_last_error());                                    \
+      exit(1);                                                                                      \
+    }                                                                                               \
+  } while (0)
+
+namespace {
+
+struct Shape {
+  int ranks, L, kv, NG, NC;
+  int64_t chunk;
+  bool blockfirst;
+  // engine tensors: per rank and layer [kv, NG, chunk]
+  int64_t gpu_kv_stride() const { return (int64_t)NG * chunk; }
+  int64_t gpu_block_stride() const { return chunk; }
+  int64_t layer_bytes() const { return (int64_t)kv * NG * chunk; }
+  // host pool: block-first [NC, L, kv, chunk] or layer-first [L, kv, NC, chunk]
+  int64_t cpu_kv_stride() const { return blockfirst ? chunk : (int64_t)NC * chunk; }
+  int64_t cpu_layer_stride() const { return blockfirst ? kv * chunk : (int64_t)kv * NC * chunk; }
+  int64_t cpu_block_stride() const { return blockfirst ? (int64_t)L * kv * chunk : chunk; }
+  int64_t host_bytes() const { return (int64_t)NC * L * kv * chunk; }
+};
+
+struct Tensors {
+  std::vector<std::vector<uint8_t *>> dev; // [rank][layer], "device" memory
+  std::vector<std::vector<std::vector<uint8_t>>> model; // the same, as the model sees it
+  uint8_t *host = nullptr;
+  bool host_pinned = true;
+};
+
+void fill(std::mt19937_64 &rng, uint8_t *p, size_t n) {
+  for (size_t i = 0; i < n; i += 8) {
+    const uint64_t v = rng();
+    std::memcpy(p + i, &v, std::min<size_t>(8, n - i));
+  }
+}
+
+void set_policy(const std::vector<std::pair<std::string, int>> &fields) {
+  fkv_launch_policy p{};
+  REQUIRE(fkv_launch_policy_reset(0) == FKV_OK, "policy reset");
+  REQUIRE(fkv_launch_policy_get(0, &p) == FKV_OK, "policy get");
+  for (const auto &f : fields) {
+    if (f.first == "staged_restore") p.staged_restore = f.second;
+    else if (f.first == "staged_gather") p.staged_gather = f.second;
+    else if (f.first == "gather_threads") p.gather_threads = f.second;
+    else if (f.first == "gather_ring") p.gather_ring = f.second;
+    else if (f.first == "staged_ring") p.staged_ring = f.second;
+    else if (f.first == "gather_first_by_kernel") p.gather_first_by_kernel = f.second;
+    else if (f.first == "staged_dma_streams") p.staged_dma_streams = f.second;
+    else if (f.first == "kernel_alt_stream_kb") p.kernel_alt_stream_kb = f.second;
+    else if (f.first == "test_fail_restore_batch") p.test_fail_restore_batch = f.second;
+    else if (f.first == "model_seed") p.model_seed = f.second;
+    else REQUIRE(false, "unknown policy field %s", f.first.c_str());
+  }
+  REQUIRE(fkv_launch_policy_set(0, &p) == FKV_OK, "policy set");
+}
+
+int drain(int fd) {
+  uint64_t v = 0;
+  int units = 0;
+  while (read(fd, &v, 8) == 8)
+    units += (int)v;
+  return units;
+}
+
+// What a case is drawn from; a field >= 0 pins the choice.
+struct Pinned {
+  int ranks = -1, L = -1, kv = -1, NG = -1, NC = -1, chunk16 = -1, blockfirst = -1, mode = -1,
+      pageable = -1, route = -1, use_ce = -1, with_fds = -1;
+};
+
+// One group, a few restores, everything compared.
+void layerwise_case(uint64_t seed, const Pinned &fix = Pinned()) {
+  std::mt19937_64 rng(seed);
+  auto pick = [&](int lo, int hi) { return lo + (int)(rng() % (uint64_t)(hi - lo + 1)); };
+  auto pinned = [](int drawn, int fixed) { return fixed >= 0 ? fixed : drawn; };
+  Shape s{};
+  s.ranks = pinned(std::vector<int>{1, 2, 4}[pick(0, 2)], fix.ranks);
+  s.L = pinned(pick(1, 18), fix.L);
+  s.kv = pinned(pick(1, 2), fix.kv);
+  s.NG = pinned(pick(6, 40), fix.NG);
+  s.NC = pinned(pick(6, 48), fix.NC);
+  s.chunk = 16 * pinned(pick(1, 96), fix.chunk16);
+  s.blockfirst = pinned((int)(rng() & 1), fix.blockfirst);
+  const std::string mode =
+      std::vector<std::string>{"sharded", "all_write", "rank0_only"}[pinned(pick(0, 2), fix.mode)];
+  const int copies = mode == "all_write" ? s.ranks : 1;
+  const int pool_blocks = s.NC;
+  s.NC *= copies; // rank r of an all_write restore reads n blocks further on, see below
+  const bool pageable = pinned((rng() % 5) == 0, fix.pageable);
+  const int route = pinned(pick(0, 3), fix.route); // 0 the library's choice, 1 kernel, 2 copy per run, 3 gathered
+  const bool use_ce = pinned((rng() % 3) == 0, fix.use_ce);
+  const bool with_fds = pinned((int)(rng() & 1), fix.with_fds);
+  const int counters = 2;
+
+  Tensors t;
+  t.host_pinned = !pageable;
+  if (pageable)
+    t.host = static_cast<uint8_t *>(malloc((size_t)s.host_bytes()));
+  else
+    REQUIRE(hipHostMalloc((void **)&t.host, (size_t)s.host_bytes(), 0) == hipSuccess, "host pool");
+  t.dev.resize(s.ranks);
+  t.model.resize(s.ranks);
+  std::vector<uint64_t> ptrs;
+  for (int r = 0; r < s.ranks; ++r)
+    for (int l = 0; l < s.L; ++l) {
+      uint8_t *d = nullptr;
+      REQUIRE(hipMalloc((void **)&d, (size_t)s.layer_bytes()) == hipSuccess, "engine tensor");
+      std::vector<uint8_t> init((size_t)s.layer_bytes());
+      fill(rng, init.data(), init.size());
+      std::memcpy(d, init.data(), init.size());
+      t.dev[r].push_back(d);
+      t.model[r].push_back(std::move(init));
+      ptrs.push_back((uint64_t)(uintptr_t)d);
+    }
+  std::vector<int32_t> fds;
+  if (with_fds)
+    for (int i = 0; i < counters * s.ranks * s.L; ++i)
+      fds.push_back(eventfd(0, EFD_NONBLOCK));
+  std::vector<int64_t> kvs(s.ranks, s.gpu_kv_stride()), bs(s.ranks, s.gpu_block_stride()),
+      ls(s.ranks, s.layer_bytes()), cs(s.ranks, s.chunk), devs(s.ranks, 0);
+  fkv_layerwise_params p{};
+  p.num_gpus = s.ranks;
+  p.num_tensors_per_gpu = s.L;
+  p.gpu_block_ptrs_flat = ptrs.data();
+  p.cpu_blocks_ptr = t.host;
+  p.num_layers = s.L;
+  p.tp_size = s.ranks;
+  p.gpu_kv_strides = kvs.data();
+  p.gpu_block_strides = bs.data();
+  p.gpu_layer_strides = ls.data();
+  p.gpu_chunk_sizes = cs.data();
+  p.gpu_device_ids = devs.data();
+  p.layer_eventfds = fds.empty() ? nullptr : fds.data();
+  p.num_layer_eventfds = (int32_t)fds.size();
+  fkv_ce_config_default(&p.ce);
+  p.ce.is_blockfirst = s.blockfirst;
+  p.ce.num_kv_heads = 1;
+  p.ce.gather_threads = pick(0, 3);
+  p.ce.enable_memcpy2d = rng() & 1;
+  fkv_layerwise *g = nullptr;
+  REQUIRE(fkv_layerwise_create(&p, &g) == FKV_OK, "create");
+
+  std::vector<std::pair<std::string, int>> pol = {
+      {"model_seed", 0}, {"gather_threads", pick(2, 4)}, {"gather_ring", pick(2, 4)},
+      {"staged_ring", pick(2, 4)}, {"gather_first_by_kernel", pick(0, 1)},
+      {"staged_dma_streams", pick(1, 2)}, {"kernel_alt_stream_kb", (rng() & 1) ? 4096 : 0}};
+  if (route == 1) { pol.push_back({"staged_restore", 0}); pol.push_back({"staged_gather", 0}); }
+  if (route == 2) { pol.push_back({"staged_restore", 2}); pol.push_back({"staged_gather", 0}); }
+  // 3: also in groups of several GPUs, where the library does not take the route by itself
+  if (route == 3) { pol.push_back({"staged_restore", 0}); pol.push_back({"staged_gather", 3}); }
+  set_policy(pol);
+
+  hipStream_t consumer = nullptr;
+  REQUIRE(hipStreamCreateWithFlags(&consumer, hipStreamNonBlocking) == hipSuccess, "stream");
+  std::vector<uint8_t> seen((size_t)s.layer_bytes()); // what the consumer copies out of layer l
+  for (int rep = 0; rep < 3; ++rep) {
+    fill(rng, t.host, (size_t)s.host_bytes());
+    const int n = pick(0, std::min(s.NG, pool_blocks));
+    std::vector<int64_t> gids(s.NG), cids(pool_blocks);
+    std::iota(gids.begin(), gids.end(), 0);
+    std::iota(cids.begin(), cids.end(), 0);
+    std::shuffle(gids.begin(), gids.end(), rng);
+    if (rng() & 1)
+      std::shuffle(cids.begin(), cids.end(), rng);
+    else
+      std::rotate(cids.begin(), cids.begin() + pick(0, pool_blocks - 1), cids.end());
+    gids.resize(n);
+    cids.resize(n);
+    if (mode == "all_write") // rank r reads blocks [r*n, (r+1)*n) further on: ids stay below n
+      for (int i = 0; i < n; ++i)
+        cids[i] = i;
+    const int layers = pick(1, s.L), gran = pick(1, s.L);
+    const int notify = (rng() & 1) ? FKV_NOTIFY_POLLING : FKV_NOTIFY_HOSTFUNC;
+    const int counter = pick(0, counters - 1);
+    const int give_up = (rng() % 6) == 0 ? pick(1, (layers + gran - 1) / gran) : 0;
+    if (give_up) {
+      auto q = pol;
+      q.push_back({"test_fail_restore_batch", give_up});
+      set_policy(q);
+    }
+    const bool kernel_only = route == 1 || (pageable && route != 3 && route != 0);
+    const int rc = fkv_layerwise_transfer(
+        g, gids.data(), cids.data(), n, s.cpu_block_stride(), s.cpu_kv_stride(),
+        s.cpu_layer_stride(), s.cpu_block_stride(), 4, use_ce, layers, gran, s.kv, 1, counter,
+        mode.c_str(), notify, 0);
+    // a pageable pool has no kernel route: refused unless the copy engine was asked for or
+    // rows can be gathered
+    const bool refused_ok = pageable && !use_ce && n > 0;
+    if (rc != FKV_OK && !give_up) {
+      REQUIRE(refused_ok && (kernel_only || route == 0 || route == 2),
+              "seed %llu rep %d: restore refused", (unsigned long long)seed, rep);
+      REQUIRE(fkv_layerwise_synchronize(g) == FKV_OK, "synchronize after a refusal");
+      continue;
+    }
+    // a consumer gated on a layer sees that layer whole
+    const int watch = pick(0, layers - 1);
+    if (rc == FKV_OK) {
+      if (!give_up && n > 0) {
+        REQUIRE(fkv_layerwise_wait_layer(g, 0, watch, consumer) == FKV_OK, "wait_layer");
+        REQUIRE(hipMemcpyAsync(seen.data(), t.dev[0][watch], seen.size(), hipMemcpyDeviceToHost,
+                               consumer) == hipSuccess, "consumer copy");
+      }
+    }
+    const int src = fkv_layerwise_synchronize(g);
+    REQUIRE(hipStreamSynchronize(consumer) == hipSuccess, "consumer");
+    if (give_up) {
+      // the call or the synchronize reports it; what landed is a prefix of the batches
+      REQUIRE(rc != FKV_OK || src != FKV_OK || n == 0 || give_up > (layers + gran - 1) / gran,
+              "seed %llu: a restore that gave up went unreported", (unsigned long long)seed);
+      set_policy(pol);
+      // re-base the model on what is there: the next restore must be whole again
+      for (int r = 0; r < s.ranks; ++r)
+        for (int l = 0; l < s.L; ++l)
+          std::memcpy(t.model[r][l].data(), t.dev[r][l], (size_t)s.layer_bytes());
+      for (int fd : fds)
+        drain(fd);
+      continue;
+    }
+    REQUIRE(src == FKV_OK, "seed %llu rep %d: synchronize", (unsigned long long)seed, rep);
+    // the model: rank r, layer l < layers, kv, position p
+    for (int r = 0; r < s.ranks; ++r) {
+      const int64_t off = mode == "all_write" ? (int64_t)r * n * s.cpu_block_stride() : 0;
+      for (int l = 0; l < layers; ++l)
+        for (int k = 0; k < s.kv; ++k)
+          for (int q = 0; q < n; ++q)
+            std::memcpy(t.model[r][l].data() + k * s.gpu_kv_stride() + gids[q] * s.chunk,
+                        t.host + off + cids[q] * s.cpu_block_stride() + l * s.cpu_layer_stride() +
+                            k * s.cpu_kv_stride(),
+                        (size_t)s.chunk);
+    }
+    for (int r = 0; r < s.ranks; ++r)
+      for (int l = 0; l < s.L; ++l)
+        REQUIRE(std::memcmp(t.dev[r][l], t.model[r][l].data(), (size_t)s.layer_bytes()) == 0,
+                "seed %llu rep %d: rank %d layer %d differs (route %d use_ce %d pageable %d mode %s "
+                "gran %d layers %d n %d)", (unsigned long long)seed, rep, r, l, route, (int)use_ce,
+                (int)pageable, mode.c_str(), gran, layers, n);
+    if (n > 0)
+      REQUIRE(std::memcmp(seen.data(), t.model[0][watch].data(), seen.size()) == 0,
+              "seed %llu rep %d: the consumer gated on layer %d saw other bytes",
+              (unsigned long long)seed, rep, watch);
+    if (with_fds) {
+      for (int c = 0; c < counters; ++c)
+        for (int r = 0; r < s.ranks; ++r)
+          for (int l = 0; l < s.L; ++l) {
+            const int units = drain(fds[((size_t)c * s.ranks + r) * s.L + l]);
+            REQUIRE(units == (c == counter && l < layers ? 1 : 0),
+                    "seed %llu rep %d: eventfd counter %d rank %d layer %d has %d units",
+                    (unsigned long long)seed, rep, c, r, l, units);
+          }
+    }
+  }
+  REQUIRE(hipStreamDestroy(consumer) == hipSuccess, "stream destroy");
+  fkv_layerwise_destroy(g);
+  for (int fd : fds)
+    close(fd);
+  for (auto &rank : t.dev)
+    for (uint8_t *d : rank)
+      REQUIRE(hipFree(d) == hipSuccess, "free");
+  if (pageable)
+    free(t.host);
+  else
+    REQUIRE(hipHostFree(t.host) == hipSuccess, "host free");
+}
+
+// Plain puts and gets: kernel path and every copy-engine strategy the ids lead to.
+void transfer_case(uint64_t seed) {
+  std::mt19937_64 rng(seed);
+  auto pick = [&](int lo, int hi) { return lo + (int)(rng() % (uint64_t)(hi - lo + 1)); };
+  Shape s{};
+  s.ranks = 1;
+  s.L = pick(1, 6);
+  s.kv = pick(1, 2);
+  s.NG = pick(4, 40);
+  s.NC = pick(4, 40);
+  s.chunk = 8 * pick(1, 300);
+  s.blockfirst = rng() & 1;
+  std::vector<uint8_t *> dev;
+  std::vector<std::vector<uint8_t>> model;
+  std::vector<uint64_t> ptrs;
+  for (int l = 0; l < s.L; ++l) {
+    uint8_t *d = nullptr;
+    REQUIRE(hipMalloc((void **)&d, (size_t)s.layer_bytes()) == hipSuccess, "engine tensor");
+    std::vector<uint8_t> init((size_t)s.layer_bytes());
+    fill(rng, init.data(), init.size());
+    std::memcpy(d, init.data(), init.size());
+    dev.push_back(d);
+    model.push_back(std::move(init));
+    ptrs.push_back((uint64_t)(uintptr_t)d);
+  }
+  uint8_t *host = nullptr;
+  REQUIRE(hipHostMalloc((void **)&host, (size_t)s.host_bytes(), 0) == hipSuccess, "host pool");
+  std::vector<uint8_t> host_model((size_t)s.host_bytes());
+  fill(rng, host_model.data(), host_model.size());
+  std::memcpy(host, host_model.data(), host_model.size());
+  hipStream_t st = nullptr;
+  REQUIRE(hipStreamCreateWithFlags(&st, hipStreamNonBlocking) == hipSuccess, "stream");
+  set_policy({{"model_seed", 0}});
+  for (int rep = 0; rep < 8; ++rep) {
+    const int n = pick(0, std::min(s.NG, s.NC));
+    std::vector<int64_t> gids(s.NG), cids(s.NC);
+    std::iota(gids.begin(), gids.end(), 0);
+    std::iota(cids.begin(), cids.end(), 0);
+    const int pattern = pick(0, 2); // scattered, one run on both sides, runs on the host side
+    if (pattern == 0) {
+      std::shuffle(gids.begin(), gids.end(), rng);
+      std::shuffle(cids.begin(), cids.end(), rng);
+    } else if (pattern == 2) {
+      std::shuffle(gids.begin(), gids.end(), rng);
+    }
+    gids.resize(n);
+    cids.resize(n);
+    fkv_transfer_desc d{};
+    d.backend = FKV_BACKEND_VLLM;
+    d.num_layers_total = s.L;
+    d.gpu_tensor_ptrs = ptrs.data();
+    d.num_gpu_tensor_ptrs = s.L;
+    d.device = -1;
+    d.gpu_kv_stride = s.gpu_kv_stride();
+    d.gpu_block_stride = s.gpu_block_stride();
+    d.gpu_layer_stride = s.layer_bytes();
+    d.cpu_ptr = host;
+    d.cpu_kv_stride = s.cpu_kv_stride();
+    d.cpu_layer_stride = s.cpu_layer_stride();
+    d.cpu_block_stride = s.cpu_block_stride();
+    d.chunk_size = s.chunk;
+    d.start_layer_id = pick(0, s.L - 1);
+    d.num_layers = pick(1, s.L - d.start_layer_id);
+    d.kv_dim = s.kv;
+    d.num_blocks = n;
+    d.gpu_block_ids = gids.data();
+    d.cpu_block_ids = cids.data();
+    d.is_host_to_device = rng() & 1;
+    d.use_ce_transfer = pick(0, 2);
+    d.transfer_num_cta = pick(1, 8);
+    d.sync = rng() & 1;
+    fkv_ce_config_default(&d.ce);
+    d.ce.is_blockfirst = s.blockfirst;
+    d.ce.num_kv_heads = (rng() & 1) ? 1 : 8;
+    d.ce.segment_threshold = (rng() & 1) ? 8 : 2;
+    d.ce.path_opt_enabled = (rng() % 4) != 0;
+    d.ce.enable_memcpy2d = rng() & 1;
+    d.ce.gather_threads = pick(0, 4);
+    d.ce.gather_nt = rng() & 1;
+    REQUIRE(fkv_transfer_kv_blocks(&d, st) == FKV_OK, "seed %llu rep %d: transfer",
+            (unsigned long long)seed, rep);
+    REQUIRE(hipStreamSynchronize(st) == hipSuccess, "sync");
+    for (int l = d.start_layer_id; l < d.start_layer_id + d.num_layers; ++l)
+      for (int k = 0; k < s.kv; ++k)
+        for (int q = 0; q < n; ++q) {
+          uint8_t *gm = model[l].data() + k * s.gpu_kv_stride() + gids[q] * s.chunk;
+          uint8_t *hm = host_model.data() + cids[q] * s.cpu_block_stride() +
+                        l * s.cpu_layer_stride() + k * s.cpu_kv_stride();
+          if (d.is_host_to_device)
+            std::memcpy(gm, hm, (size_t)s.chunk);
+          else
+            std::memcpy(hm, gm, (size_t)s.chunk);
+        }
+    for (int l = 0; l < s.L; ++l)
+      REQUIRE(std::memcmp(dev[l], model[l].data(), (size_t)s.layer_bytes()) == 0,
+              "seed %llu rep %d: layer %d differs (path %d)", (unsigned long long)seed, rep, l,
+              fkv_last_path());
+    REQUIRE(std::memcmp(host, host_model.data(), host_model.size()) == 0,
+            "seed %llu rep %d: host pool differs (path %d)", (unsigned long long)seed, rep,
+            fkv_last_path());
+  }
+  REQUIRE(hipStreamDestroy(st) == hipSuccess, "stream destroy");
+  for (uint8_t *d : dev)
+    REQUIRE(hipFree(d) == hipSuccess, "free");
+  REQUIRE(hipHostFree(host) == hipSuccess, "host free");
+}
+
+} // namespace
+
+int main(int argc, char **argv) {
+  const int restores = argc > 1 ? atoi(argv[1]) : 120, transfers = argc > 2 ? atoi(argv[2]) : 60;
+  for (int i = 0; i < transfers; ++i)
+    transfer_case(7000 + i);
+  for (int i = 0; i < restores; ++i)
+    layerwise_case(9000 + i);
+  // four ranks that share their KV, rows gathered by host threads, asked for on the copy
+  // engine: the launching thread serves four staging rings and eight copy streams
+  Pinned four;
+  four.ranks = 4, four.L = 5, four.kv = 1, four.NG = 12, four.NC = 12, four.chunk16 = 128;
+  four.blockfirst = 1, four.mode = 0, four.pageable = 0, four.route = 3, four.use_ce = 1;
+  for (int i = 0; i < restores / 2; ++i)
+    layerwise_case(11000 + i, four);
+  printf("ok: %d groups of layerwise restores and %d sets of transfers over the emulated runtime\n",
+         restores, transfers);
+  return 0;
+}

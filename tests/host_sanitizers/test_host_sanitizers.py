@@ -64,3 +64,48 @@ def test_batch_gate_of_a_gathered_restore_under_sanitizers(tmp_path, sanitizer):
     blocking waiters and the polling loop, 200 runs through one gate."""
     out = build_and_run(tmp_path, "batch_gate_driver.cpp", sanitizer)
     assert "ok: 200 scripted restores through the gate" in out
+
+
+LIBRARY_HOST_SOURCES = ["fkv_core", "fkv_ce", "fkv_host", "fkv_host_copy", "fkv_tp_group",
+                        "fkv_layerwise", "fkv_ipc", "fkv_ssd", "fkv_transform", "fkv_ranges",
+                        "fkv_linkboard", "fkv_policy", "fkv_staged_restore"]
+
+
+def build_over_emulated_runtime(tmp_path, driver, sanitizer):
+    """Every host translation unit of the library, the emulated HIP runtime (streams as
+    threads, events as counters, the kernels as memcpy loops) and a driver, compiled with
+    the sanitizer and linked into one program."""
+    from concurrent.futures import ThreadPoolExecutor
+    csrc = os.path.join(ROOT, "flexkv_amd", "csrc")
+    flags = [CLANG, "-std=c++17", "-O1", "-g", *sanitizer, "-fno-omit-frame-pointer", "-mavx2",
+             "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", "-I" + os.path.join(ROOT, "include"),
+             "-I" + csrc]
+    units = [os.path.join(csrc, f + ".cpp") for f in LIBRARY_HOST_SOURCES]
+    units += [os.path.join(HERE, "emulated_hip_runtime.cpp"), os.path.join(HERE, driver)]
+    objects = [str(tmp_path / (os.path.basename(u)[:-4] + ".o")) for u in units]
+
+    def compile_one(pair):
+        subprocess.run(flags + ["-c", pair[0], "-o", pair[1]], check=True, capture_output=True,
+                       text=True)
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 2)) as pool:
+        list(pool.map(compile_one, zip(units, objects)))
+    exe = str(tmp_path / "driver")
+    subprocess.run([CLANG, *sanitizer, *objects, "-o", exe, "-pthread", "-ldl"], check=True,
+                   capture_output=True, text=True)
+    return exe
+
+
+@pytest.mark.parametrize("sanitizer", SANITIZERS)
+def test_whole_host_side_over_an_emulated_runtime_under_sanitizers(tmp_path, sanitizer):
+    """Layerwise restores with one, two and four ranks on every route and engine, pinned and
+    pageable pools, both notify modes with eventfds, consumers gated per layer, restores that
+    give up part-way, and plain puts and gets on the kernel path and through every
+    copy-engine strategy: the library's host code as it is shipped, over a HIP runtime made
+    of threads, every byte against a plain model.  The library keeps per-stream events and
+    staging memory until the process ends, so leak checking is off for this program."""
+    exe = build_over_emulated_runtime(tmp_path, "layerwise_emulated_driver.cpp", sanitizer)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:verify_asan_link_order=0",
+               TSAN_OPTIONS="halt_on_error=1", TMPDIR=str(tmp_path))
+    r = subprocess.run([exe, "80", "40"], capture_output=True, text=True, env=env, timeout=900)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
+    assert "ok: 80 groups of layerwise restores and 40 sets of transfers" in r.stdout
