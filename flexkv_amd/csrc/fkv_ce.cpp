@@ -434,6 +434,11 @@ int h2d_pingpong(const Job &j, Consume consume) {
   uint8_t *bufs[2] = {base, base + layer_bytes};
   const int iters = d.num_layers * d.kv_dim;
   j.host_waits = true;
+  // The calling thread reads the host pool itself, now: what the caller enqueued on the stream
+  // before this transfer (a put into the same host blocks, say) has to have landed, as it would
+  // have for a copy in stream order.  Workers wait for every op, so their streams are idle here.
+  if (iters > 0)
+    FKV_HIP_TRY(hipStreamSynchronize(j.stream));
   for (int it = 0; it < iters; ++it) {
     if (it >= 2)
       FKV_HIP_TRY(hipEventSynchronize(ev[it & 1]));

@@ -30,6 +30,7 @@
 #include <deque>
 #include <functional>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <thread>
 #include <vector>
@@ -112,7 +113,9 @@ hipError_t remember(hipError_t e) {
 
 struct Runtime {
   std::mutex mu;
-  std::vector<ihipStream_t *> streams; // every live stream, the null stream first
+  // every live stream, the null stream first; shared, so that a device-wide wait can outlive
+  // the destruction of a stream by another thread
+  std::vector<std::shared_ptr<ihipStream_t>> streams;
   struct Block {
     size_t size;
     bool pinned;
@@ -122,8 +125,8 @@ struct Runtime {
   ihipStream_t *null_stream() {
     std::lock_guard<std::mutex> lk(mu);
     if (streams.empty())
-      streams.push_back(new ihipStream_t());
-    return streams[0];
+      streams.push_back(std::make_shared<ihipStream_t>());
+    return streams[0].get();
   }
   const std::pair<const uintptr_t, Block> *find(const void *p) {
     std::lock_guard<std::mutex> lk(mu);
@@ -134,17 +137,13 @@ struct Runtime {
     return (uintptr_t)p < it->first + it->second.size ? &*it : nullptr;
   }
   void drain_all() {
-    std::vector<ihipStream_t *> all;
+    std::vector<std::shared_ptr<ihipStream_t>> all;
     {
       std::lock_guard<std::mutex> lk(mu);
       all = streams;
     }
-    for (ihipStream_t *s : all)
+    for (auto &s : all)
       s->drain();
-  }
-  ~Runtime() {
-    for (ihipStream_t *s : streams)
-      delete s;
   }
 };
 Runtime &rt() {
@@ -219,23 +218,32 @@ hipError_t hipDeviceGetPCIBusId(char *id, int len, int device) {
 }
 
 hipError_t hipStreamCreateWithFlags(hipStream_t *s, unsigned int) {
-  *s = new ihipStream_t();
+  auto made = std::make_shared<ihipStream_t>();
+  *s = made.get();
   std::lock_guard<std::mutex> lk(rt().mu);
   if (rt().streams.empty())
-    rt().streams.push_back(new ihipStream_t());
-  rt().streams.push_back(*s);
+    rt().streams.push_back(std::make_shared<ihipStream_t>());
+  rt().streams.push_back(std::move(made));
   return hipSuccess;
 }
 hipError_t hipStreamCreate(hipStream_t *s) { return hipStreamCreateWithFlags(s, 0); }
 hipError_t hipStreamDestroy(hipStream_t s) {
   if (!s)
     return remember(hipErrorInvalidHandle);
+  std::shared_ptr<ihipStream_t> mine;
   {
     std::lock_guard<std::mutex> lk(rt().mu);
     auto &v = rt().streams;
-    v.erase(std::remove(v.begin(), v.end(), s), v.end());
+    for (size_t i = 1; i < v.size(); ++i)
+      if (v[i].get() == s) {
+        mine = std::move(v[i]);
+        v.erase(v.begin() + (long)i);
+        break;
+      }
   }
-  delete s; // finishes what is queued, as the runtime does
+  if (!mine)
+    return remember(hipErrorInvalidHandle);
+  mine->drain(); // finishes what is queued, as the runtime does; the thread ends with the last owner
   return hipSuccess;
 }
 hipError_t hipStreamSynchronize(hipStream_t s) {

@@ -16,10 +16,36 @@
 #include <cstring>
 #include <numeric>
 #include <random>
+#include <atomic>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "fkv_transfer.h"
+
+// the CPU restatement of the reference's rank placement and byte loop (oracle/fkv_oracle.c)
+extern "C" {
+typedef struct {
+  int32_t active;
+  int32_t start_layer;
+  int32_t num_layers;
+  int32_t reserved;
+  int64_t cpu_startoff;
+  int64_t gpu_startoff;
+  int64_t chunk_size;
+} fkv_oracle_rank_plan;
+int fkv_oracle_tp_rank_plan(int rank, int num_gpus, int num_kv_heads, int is_host_to_device,
+                            const char *mode_in, int designated_rank, int rotate_counter,
+                            int layer_id, int layer_granularity, int num_blocks,
+                            int64_t gpu_chunk_size, int64_t cpu_block_stride, int64_t cpu_tp_stride,
+                            fkv_oracle_rank_plan *out);
+int fkv_oracle_transfer(int backend, const uint64_t *tensor_ptrs, int64_t num_layers_total,
+                        int64_t gpu_kv_stride, int64_t gpu_block_stride, int64_t gpu_layer_stride,
+                        int64_t gpu_off, uint8_t *cpu_ptr, int64_t cpu_kv_stride,
+                        int64_t cpu_layer_stride, int64_t cpu_block_stride, int64_t cpu_off,
+                        int64_t chunk, int start_layer, int num_layers, int kv_dim, int num_blocks,
+                        const int64_t *gpu_ids, const int64_t *cpu_ids, int is_host_to_device);
+}
 
 #define REQUIRE(cond, ...)                                                                          \
   do {                                                                                              \
@@ -397,12 +423,276 @@ void transfer_case(uint64_t seed) {
   REQUIRE(hipHostFree(host) == hipSuccess, "host free");
 }
 
+// The thread group of a tensor-parallel engine: a thread per rank inside the library, every
+// shared-KV mode and head slices of multi-head KV, against the oracle's rank plan and byte loop.
+void tp_case(uint64_t seed) {
+  std::mt19937_64 rng(seed);
+  auto pick = [&](int lo, int hi) { return lo + (int)(rng() % (uint64_t)(hi - lo + 1)); };
+  const int n = std::vector<int>{1, 2, 4}[pick(0, 2)];
+  const bool shared = rng() & 1;             // KV identical on all ranks (one KV head)
+  const int heads = shared ? 1 : n * pick(1, 2);
+  Shape s{};
+  s.ranks = n;
+  s.L = pick(1, 7);
+  s.kv = pick(1, 2);
+  s.NG = pick(4, 24);
+  s.chunk = 16 * n * pick(1, 24);            // what one rank holds of a block and layer
+  s.blockfirst = rng() & 1;
+  const std::string mode = std::vector<std::string>{"sharded", "all_write", "rank0_only",
+                                                    "layer_parallel", "rank_rotate", "bogus"}[pick(0, 5)];
+  const int copies = shared && mode == "all_write" ? n : 1;
+  const int pool_blocks = pick(4, 24);
+  const int64_t host_chunk = shared ? s.chunk : s.chunk * n; // multi-head: every rank's slice side by side
+  // host pool [NC, L, kv, host_chunk] or [L, kv, NC, host_chunk]
+  const int NC = pool_blocks * copies;
+  const int64_t cpu_block_stride = s.blockfirst ? (int64_t)s.L * s.kv * host_chunk : host_chunk;
+  const int64_t host_bytes = (int64_t)NC * s.L * s.kv * host_chunk;
+  // strides a rank uses inside its share: the per-rank layout of the reference's workers
+  // (flexkv/transfer/worker.py:1199-1204): block-first, a rank's chunks of a block lie together
+  int64_t cpu_kv_stride, cpu_layer_stride, cpu_tp_stride;
+  if (shared) {
+    cpu_kv_stride = s.blockfirst ? host_chunk : (int64_t)NC * host_chunk;
+    cpu_layer_stride = s.blockfirst ? s.kv * host_chunk : (int64_t)s.kv * NC * host_chunk;
+    cpu_tp_stride = cpu_block_stride;
+  } else {
+    cpu_kv_stride = s.blockfirst ? s.chunk : (int64_t)NC * host_chunk;
+    cpu_layer_stride = s.blockfirst ? s.kv * s.chunk : (int64_t)s.kv * NC * host_chunk;
+    cpu_tp_stride = cpu_block_stride / n;
+  }
+  uint8_t *host = nullptr;
+  REQUIRE(hipHostMalloc((void **)&host, (size_t)host_bytes, 0) == hipSuccess, "host pool");
+  std::vector<uint8_t> host_model((size_t)host_bytes);
+  fill(rng, host_model.data(), host_model.size());
+  std::memcpy(host, host_model.data(), host_model.size());
+  std::vector<std::vector<uint8_t *>> dev(n);
+  std::vector<std::vector<std::vector<uint8_t>>> model(n);
+  std::vector<uint64_t> ptrs;
+  for (int r = 0; r < n; ++r)
+    for (int l = 0; l < s.L; ++l) {
+      uint8_t *d = nullptr;
+      REQUIRE(hipMalloc((void **)&d, (size_t)s.layer_bytes()) == hipSuccess, "engine tensor");
+      std::vector<uint8_t> init((size_t)s.layer_bytes());
+      fill(rng, init.data(), init.size());
+      std::memcpy(d, init.data(), init.size());
+      dev[r].push_back(d);
+      model[r].push_back(std::move(init));
+      ptrs.push_back((uint64_t)(uintptr_t)d);
+    }
+  std::vector<int64_t> kvs(n, s.gpu_kv_stride()), bs(n, s.gpu_block_stride()), ls(n, s.layer_bytes()),
+      cs(n, s.chunk), devs(n, 0);
+  fkv_tp_group_params p{};
+  p.num_gpus = n;
+  p.num_tensors_per_gpu = s.L;
+  p.gpu_block_ptrs_flat = ptrs.data();
+  p.cpu_blocks_ptr = host;
+  p.num_layers = s.L;
+  p.gpu_kv_strides = kvs.data();
+  p.gpu_block_strides = bs.data();
+  p.gpu_layer_strides = ls.data();
+  p.gpu_chunk_sizes = cs.data();
+  p.gpu_device_ids = devs.data();
+  fkv_ce_config_default(&p.ce);
+  p.ce.is_blockfirst = s.blockfirst;
+  p.ce.num_kv_heads = heads;
+  p.ce.gather_threads = pick(0, 3);
+  fkv_tp_group *g = nullptr;
+  REQUIRE(fkv_tp_group_create(&p, &g) == FKV_OK, "tp group");
+  set_policy({{"model_seed", 0}});
+  int puts = 0; // rank_rotate moves on with every put
+  for (int rep = 0; rep < 6; ++rep) {
+    const int nb = pick(0, std::min(s.NG, pool_blocks));
+    std::vector<int64_t> gids(s.NG), cids(pool_blocks);
+    std::iota(gids.begin(), gids.end(), 0);
+    std::iota(cids.begin(), cids.end(), 0);
+    std::shuffle(gids.begin(), gids.end(), rng);
+    if (rng() & 1)
+      std::shuffle(cids.begin(), cids.end(), rng);
+    gids.resize(nb);
+    cids.resize(nb);
+    if (copies > 1) // rank r's region starts r * nb blocks further on
+      for (int i = 0; i < nb; ++i)
+        cids[i] = i;
+    const bool valid_get = !shared || mode == "sharded" || mode == "all_write" || mode == "rank0_only";
+    const int h2d = valid_get ? (int)(rng() & 1) : 0;
+    const int layer_id = pick(0, s.L - 1), gran = pick(1, s.L - layer_id);
+    const int use_ce = s.chunk % 8 == 0 ? pick(0, 1) : 0;
+    const int designated = pick(0, n - 1);
+    const int rc = fkv_tp_group_transfer(g, gids.data(), cids.data(), nb, cpu_kv_stride,
+                                         cpu_layer_stride, cpu_block_stride, cpu_tp_stride, 4, h2d,
+                                         use_ce, layer_id, gran, s.kv, heads, mode.c_str(), designated);
+    REQUIRE(rc == FKV_OK, "seed %llu rep %d: tp transfer (mode %s h2d %d ce %d)",
+            (unsigned long long)seed, rep, mode.c_str(), h2d, use_ce);
+    for (int r = 0; r < n; ++r) {
+      fkv_oracle_rank_plan plan{};
+      REQUIRE(fkv_oracle_tp_rank_plan(r, n, heads, h2d, mode.c_str(), designated, puts % n, layer_id,
+                                      gran, nb, s.chunk, cpu_block_stride, cpu_tp_stride, &plan) == 0,
+              "rank plan");
+      if (!plan.active)
+        continue;
+      std::vector<uint64_t> mp;
+      for (int l = 0; l < s.L; ++l)
+        mp.push_back((uint64_t)(uintptr_t)model[r][l].data());
+      REQUIRE(fkv_oracle_transfer(0, mp.data(), s.L, s.gpu_kv_stride(), s.gpu_block_stride(),
+                                  s.layer_bytes(), plan.gpu_startoff, host_model.data(), cpu_kv_stride,
+                                  cpu_layer_stride, cpu_block_stride, plan.cpu_startoff,
+                                  plan.chunk_size, plan.start_layer, plan.num_layers, s.kv, nb,
+                                  gids.data(), cids.data(), h2d) == 0, "oracle transfer");
+    }
+    if (!h2d)
+      ++puts;
+    for (int r = 0; r < n; ++r)
+      for (int l = 0; l < s.L; ++l)
+        REQUIRE(std::memcmp(dev[r][l], model[r][l].data(), (size_t)s.layer_bytes()) == 0,
+                "seed %llu rep %d: rank %d layer %d differs (mode %s h2d %d ce %d heads %d)",
+                (unsigned long long)seed, rep, r, l, mode.c_str(), h2d, use_ce, heads);
+    REQUIRE(std::memcmp(host, host_model.data(), host_model.size()) == 0,
+            "seed %llu rep %d: host pool differs (mode %s h2d %d ce %d heads %d ranks %d)",
+            (unsigned long long)seed, rep, mode.c_str(), h2d, use_ce, heads, n);
+  }
+  fkv_tp_group_destroy(g);
+  for (auto &rank : dev)
+    for (uint8_t *d : rank)
+      REQUIRE(hipFree(d) == hipSuccess, "free");
+  REQUIRE(hipHostFree(host) == hipSuccess, "host free");
+}
+
+// Puts and gets from several threads at once, a stream each, on blocks of their own: plan
+// memory, claim counters, the arbiter's view of the link and the library's lane streams under
+// concurrent calls.
+void concurrent_case(uint64_t seed) {
+  std::mt19937_64 rng(seed);
+  auto pick = [&](int lo, int hi) { return lo + (int)(rng() % (uint64_t)(hi - lo + 1)); };
+  const int threads = pick(2, 5), per = pick(3, 10);
+  Shape s{};
+  s.ranks = 1;
+  s.L = pick(1, 5);
+  s.kv = pick(1, 2);
+  s.NG = threads * per;
+  s.NC = threads * per;
+  s.chunk = 16 * pick(1, 64);
+  s.blockfirst = rng() & 1;
+  std::vector<uint8_t *> dev;
+  std::vector<std::vector<uint8_t>> model;
+  std::vector<uint64_t> ptrs;
+  for (int l = 0; l < s.L; ++l) {
+    uint8_t *d = nullptr;
+    REQUIRE(hipMalloc((void **)&d, (size_t)s.layer_bytes()) == hipSuccess, "engine tensor");
+    std::vector<uint8_t> init((size_t)s.layer_bytes());
+    fill(rng, init.data(), init.size());
+    std::memcpy(d, init.data(), init.size());
+    dev.push_back(d);
+    model.push_back(std::move(init));
+    ptrs.push_back((uint64_t)(uintptr_t)d);
+  }
+  uint8_t *host = nullptr;
+  REQUIRE(hipHostMalloc((void **)&host, (size_t)s.host_bytes(), 0) == hipSuccess, "host pool");
+  std::vector<uint8_t> host_model((size_t)s.host_bytes());
+  fill(rng, host_model.data(), host_model.size());
+  std::memcpy(host, host_model.data(), host_model.size());
+  set_policy({{"model_seed", 0}});
+  struct Op {
+    std::vector<int64_t> gids, cids;
+    int h2d, sync, use_ce;
+  };
+  std::vector<std::vector<Op>> script(threads);
+  for (int t = 0; t < threads; ++t)
+    for (int k = 0; k < 6; ++k) {
+      Op op;
+      const int n = pick(1, per);
+      std::vector<int64_t> mine(per);
+      std::iota(mine.begin(), mine.end(), (int64_t)t * per);
+      std::shuffle(mine.begin(), mine.end(), rng);
+      op.gids.assign(mine.begin(), mine.begin() + n);
+      std::shuffle(mine.begin(), mine.end(), rng);
+      op.cids.assign(mine.begin(), mine.begin() + n);
+      op.h2d = rng() & 1;
+      op.sync = rng() & 1;
+      op.use_ce = (rng() % 4) == 0;
+      script[t].push_back(std::move(op));
+    }
+  std::vector<std::thread> pool;
+  std::atomic<int> failures{0};
+  for (int t = 0; t < threads; ++t)
+    pool.emplace_back([&, t] {
+      hipStream_t st = nullptr;
+      if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess) {
+        failures.fetch_add(1);
+        return;
+      }
+      for (const Op &op : script[t]) {
+        fkv_transfer_desc d{};
+        d.backend = FKV_BACKEND_VLLM;
+        d.num_layers_total = s.L;
+        d.gpu_tensor_ptrs = ptrs.data();
+        d.num_gpu_tensor_ptrs = s.L;
+        d.device = -1;
+        d.gpu_kv_stride = s.gpu_kv_stride();
+        d.gpu_block_stride = s.gpu_block_stride();
+        d.gpu_layer_stride = s.layer_bytes();
+        d.cpu_ptr = host;
+        d.cpu_kv_stride = s.cpu_kv_stride();
+        d.cpu_layer_stride = s.cpu_layer_stride();
+        d.cpu_block_stride = s.cpu_block_stride();
+        d.chunk_size = s.chunk;
+        d.num_layers = s.L;
+        d.kv_dim = s.kv;
+        d.num_blocks = (int32_t)op.gids.size();
+        d.gpu_block_ids = op.gids.data();
+        d.cpu_block_ids = op.cids.data();
+        d.is_host_to_device = op.h2d;
+        d.use_ce_transfer = op.use_ce;
+        d.transfer_num_cta = 4;
+        d.sync = op.sync;
+        fkv_ce_config_default(&d.ce);
+        d.ce.is_blockfirst = s.blockfirst;
+        if (fkv_transfer_kv_blocks(&d, st) != FKV_OK) {
+          fprintf(stderr, "thread %d: %s\n", t, fkv_last_error());
+          failures.fetch_add(1);
+        }
+      }
+      if (hipStreamSynchronize(st) != hipSuccess || hipStreamDestroy(st) != hipSuccess)
+        failures.fetch_add(1);
+    });
+  for (auto &th : pool)
+    th.join();
+  REQUIRE(failures.load() == 0, "seed %llu: %d calls failed", (unsigned long long)seed, failures.load());
+  for (int t = 0; t < threads; ++t)
+    for (const Op &op : script[t])
+      for (int l = 0; l < s.L; ++l)
+        for (int k = 0; k < s.kv; ++k)
+          for (size_t q = 0; q < op.gids.size(); ++q) {
+            uint8_t *gm = model[l].data() + k * s.gpu_kv_stride() + op.gids[q] * s.chunk;
+            uint8_t *hm = host_model.data() + op.cids[q] * s.cpu_block_stride() +
+                          l * s.cpu_layer_stride() + k * s.cpu_kv_stride();
+            if (op.h2d)
+              std::memcpy(gm, hm, (size_t)s.chunk);
+            else
+              std::memcpy(hm, gm, (size_t)s.chunk);
+          }
+  { // a device-wide wait: the library's lane streams included
+    void *probe = nullptr;
+    REQUIRE(hipMalloc(&probe, 64) == hipSuccess && hipFree(probe) == hipSuccess, "drain");
+  }
+  for (int l = 0; l < s.L; ++l)
+    REQUIRE(std::memcmp(dev[l], model[l].data(), (size_t)s.layer_bytes()) == 0,
+            "seed %llu: layer %d differs after %d threads", (unsigned long long)seed, l, threads);
+  REQUIRE(std::memcmp(host, host_model.data(), host_model.size()) == 0,
+          "seed %llu: host pool differs after %d threads", (unsigned long long)seed, threads);
+  for (uint8_t *d : dev)
+    REQUIRE(hipFree(d) == hipSuccess, "free");
+  REQUIRE(hipHostFree(host) == hipSuccess, "host free");
+}
+
 } // namespace
 
 int main(int argc, char **argv) {
   const int restores = argc > 1 ? atoi(argv[1]) : 120, transfers = argc > 2 ? atoi(argv[2]) : 60;
   for (int i = 0; i < transfers; ++i)
     transfer_case(7000 + i);
+  for (int i = 0; i < transfers; ++i)
+    tp_case(8000 + i);
+  for (int i = 0; i < transfers; ++i)
+    concurrent_case(10000 + i);
   for (int i = 0; i < restores; ++i)
     layerwise_case(9000 + i);
   // four ranks that share their KV, rows gathered by host threads, asked for on the copy
@@ -412,7 +702,7 @@ int main(int argc, char **argv) {
   four.blockfirst = 1, four.mode = 0, four.pageable = 0, four.route = 3, four.use_ce = 1;
   for (int i = 0; i < restores / 2; ++i)
     layerwise_case(11000 + i, four);
-  printf("ok: %d groups of layerwise restores and %d sets of transfers over the emulated runtime\n",
-         restores, transfers);
+  printf("ok: %d groups of layerwise restores, %d sets of transfers, %d thread groups and %d bursts "
+         "of concurrent calls over the emulated runtime\n", restores, transfers, transfers, transfers);
   return 0;
 }

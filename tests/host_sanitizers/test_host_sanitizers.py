@@ -89,6 +89,14 @@ def build_over_emulated_runtime(tmp_path, driver, sanitizer):
                        text=True)
     with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 2)) as pool:
         list(pool.map(compile_one, zip(units, objects)))
+    # the CPU restatement of the reference's rank placement and byte loop: the driver's model
+    # for the thread-group cases
+    oracle = str(tmp_path / "fkv_oracle.o")
+    subprocess.run([shutil.which("clang", path=os.path.dirname(CLANG)) or "clang", "-O1", "-g",
+                    *sanitizer, "-fno-omit-frame-pointer", "-c",
+                    os.path.join(ROOT, "oracle", "fkv_oracle.c"), "-o", oracle],
+                   check=True, capture_output=True, text=True)
+    objects.append(oracle)
     exe = str(tmp_path / "driver")
     subprocess.run([CLANG, *sanitizer, *objects, "-o", exe, "-pthread", "-ldl"], check=True,
                    capture_output=True, text=True)
@@ -99,13 +107,16 @@ def build_over_emulated_runtime(tmp_path, driver, sanitizer):
 def test_whole_host_side_over_an_emulated_runtime_under_sanitizers(tmp_path, sanitizer):
     """Layerwise restores with one, two and four ranks on every route and engine, pinned and
     pageable pools, both notify modes with eventfds, consumers gated per layer, restores that
-    give up part-way, and plain puts and gets on the kernel path and through every
-    copy-engine strategy: the library's host code as it is shipped, over a HIP runtime made
-    of threads, every byte against a plain model.  The library keeps per-stream events and
-    staging memory until the process ends, so leak checking is off for this program."""
+    give up part-way; plain puts and gets on the kernel path and through every copy-engine
+    strategy; the thread group of a tensor-parallel engine in every shared-KV mode and with
+    head slices (against the oracle's rank plan); puts and gets from several threads at once:
+    the library's host code as it is shipped, over a HIP runtime made of threads, every byte
+    against a plain model.  The library keeps per-stream events and staging memory until the
+    process ends, so leak checking is off for this program."""
     exe = build_over_emulated_runtime(tmp_path, "layerwise_emulated_driver.cpp", sanitizer)
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:verify_asan_link_order=0",
                TSAN_OPTIONS="halt_on_error=1", TMPDIR=str(tmp_path))
     r = subprocess.run([exe, "80", "40"], capture_output=True, text=True, env=env, timeout=900)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
-    assert "ok: 80 groups of layerwise restores and 40 sets of transfers" in r.stdout
+    assert ("ok: 80 groups of layerwise restores, 40 sets of transfers, 40 thread groups and "
+            "40 bursts of concurrent calls") in r.stdout
