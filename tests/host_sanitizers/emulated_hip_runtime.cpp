@@ -212,6 +212,14 @@ hipError_t hipSetDevice(int d) {
   t_device = d;
   return hipSuccess;
 }
+hipError_t hipGetDeviceCount(int *n) {
+  *n = kDevices;
+  return hipSuccess;
+}
+hipError_t hipDeviceSynchronize(void) {
+  rt().drain_all();
+  return hipSuccess;
+}
 hipError_t hipDeviceGetPCIBusId(char *id, int len, int device) {
   snprintf(id, (size_t)len, "0000:%02x:00.0", device);
   return hipSuccess;
@@ -405,6 +413,11 @@ hipError_t hipMemcpy2DAsync(void *dst, size_t dpitch, const void *src, size_t sp
   if (width > dpitch || width > spitch)
     return remember(hipErrorInvalidPitchValue);
   of(s)->push([=] { copy_2d(dst, dpitch, src, spitch, width, height); });
+  return hipSuccess;
+}
+hipError_t hipMemset(void *dst, int value, size_t n) {
+  rt().null_stream()->drain();
+  std::memset(dst, value, n);
   return hipSuccess;
 }
 hipError_t hipMemsetAsync(void *dst, int value, size_t n, hipStream_t s) {

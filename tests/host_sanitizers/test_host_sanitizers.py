@@ -71,35 +71,43 @@ LIBRARY_HOST_SOURCES = ["fkv_core", "fkv_ce", "fkv_host", "fkv_host_copy", "fkv_
                         "fkv_linkboard", "fkv_policy", "fkv_staged_restore"]
 
 
-def build_over_emulated_runtime(tmp_path, driver, sanitizer):
+_LIBRARY_OBJECTS = {}   # sanitizer flags -> objects of the library over the emulated runtime
+
+
+def _compile(cmd):
+    subprocess.run(cmd, check=True, capture_output=True, text=True)
+
+
+def build_over_emulated_runtime(tmp_path, driver, sanitizer, defines=()):
     """Every host translation unit of the library, the emulated HIP runtime (streams as
-    threads, events as counters, the kernels as memcpy loops) and a driver, compiled with
-    the sanitizer and linked into one program."""
+    threads, events as counters, the kernels as memcpy loops), the oracle's C file (the model
+    of the thread-group cases) and a driver, compiled with the sanitizer and linked into one
+    program.  The library's objects are built once per sanitizer and test session."""
     from concurrent.futures import ThreadPoolExecutor
     csrc = os.path.join(ROOT, "flexkv_amd", "csrc")
     flags = [CLANG, "-std=c++17", "-O1", "-g", *sanitizer, "-fno-omit-frame-pointer", "-mavx2",
              "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", "-I" + os.path.join(ROOT, "include"),
              "-I" + csrc]
-    units = [os.path.join(csrc, f + ".cpp") for f in LIBRARY_HOST_SOURCES]
-    units += [os.path.join(HERE, "emulated_hip_runtime.cpp"), os.path.join(HERE, driver)]
-    objects = [str(tmp_path / (os.path.basename(u)[:-4] + ".o")) for u in units]
-
-    def compile_one(pair):
-        subprocess.run(flags + ["-c", pair[0], "-o", pair[1]], check=True, capture_output=True,
-                       text=True)
-    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 2)) as pool:
-        list(pool.map(compile_one, zip(units, objects)))
-    # the CPU restatement of the reference's rank placement and byte loop: the driver's model
-    # for the thread-group cases
-    oracle = str(tmp_path / "fkv_oracle.o")
-    subprocess.run([shutil.which("clang", path=os.path.dirname(CLANG)) or "clang", "-O1", "-g",
-                    *sanitizer, "-fno-omit-frame-pointer", "-c",
-                    os.path.join(ROOT, "oracle", "fkv_oracle.c"), "-o", oracle],
-                   check=True, capture_output=True, text=True)
-    objects.append(oracle)
+    key = tuple(sanitizer)
+    if key not in _LIBRARY_OBJECTS:
+        import tempfile
+        where = tempfile.mkdtemp(prefix="fkv_emulated_", dir=str(tmp_path.parent))
+        units = [os.path.join(csrc, f + ".cpp") for f in LIBRARY_HOST_SOURCES]
+        units.append(os.path.join(HERE, "emulated_hip_runtime.cpp"))
+        objects = [os.path.join(where, os.path.basename(u)[:-4] + ".o") for u in units]
+        jobs = [flags + ["-c", u, "-o", o] for u, o in zip(units, objects)]
+        oracle = os.path.join(where, "fkv_oracle.o")
+        jobs.append([shutil.which("clang", path=os.path.dirname(CLANG)) or "clang", "-O1", "-g",
+                     *sanitizer, "-fno-omit-frame-pointer", "-c",
+                     os.path.join(ROOT, "oracle", "fkv_oracle.c"), "-o", oracle])
+        with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 2)) as pool:
+            list(pool.map(_compile, jobs))
+        _LIBRARY_OBJECTS[key] = objects + [oracle]
+    source = driver if os.path.isabs(driver) else os.path.join(HERE, driver)
+    obj = str(tmp_path / "driver.o")
+    _compile(flags + [*defines, "-c", source, "-o", obj])
     exe = str(tmp_path / "driver")
-    subprocess.run([CLANG, *sanitizer, *objects, "-o", exe, "-pthread", "-ldl"], check=True,
-                   capture_output=True, text=True)
+    _compile([CLANG, *sanitizer, *_LIBRARY_OBJECTS[key], obj, "-o", exe, "-pthread", "-ldl"])
     return exe
 
 
@@ -120,3 +128,25 @@ def test_whole_host_side_over_an_emulated_runtime_under_sanitizers(tmp_path, san
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
     assert ("ok: 80 groups of layerwise restores, 40 sets of transfers, 40 thread groups and "
             "40 bursts of concurrent calls") in r.stdout
+
+
+@pytest.mark.parametrize("sanitizer", SANITIZERS)
+def test_native_consumers_over_an_emulated_runtime_under_sanitizers(tmp_path, sanitizer):
+    """The two native consumers of the C ABI (tests/native), which the GPU suite runs against
+    the shipped library, here linked with the library's host code over the emulated runtime:
+    every entry point that does not live beside the kernels (kernel path, each copy-engine
+    strategy, several transfers in one call, thread group, layerwise restore on each route
+    with eventfds, two-group restore with a sidecar, layout transform, the board processes
+    share), and a put thread next to a get thread."""
+    native = os.path.join(ROOT, "tests", "native")
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:verify_asan_link_order=0",
+               TSAN_OPTIONS="halt_on_error=1", TMPDIR=str(tmp_path))
+    for source, args, expect in (("abi_roundtrip_driver.cpp", [], "ok: 33 cases through the C ABI"),
+                                 ("two_way_driver.cpp", ["0.3", "8"], "ok: puts alone")):
+        sub = tmp_path / source[:-4]
+        sub.mkdir()
+        exe = build_over_emulated_runtime(sub, os.path.join(native, source), sanitizer,
+                                          defines=("-DFKV_EMULATED_RUNTIME",))
+        r = subprocess.run([exe, *args], capture_output=True, text=True, env=env, timeout=900)
+        assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
+        assert expect in r.stdout, r.stdout[-2000:]

@@ -287,10 +287,12 @@ int main() {
     fkv_launch_policy saved, pol;
     FKV_OK_OR_DIE(fkv_launch_policy_seed(-1));
     FKV_OK_OR_DIE(fkv_launch_policy_get(-1, &saved));
+#ifndef FKV_EMULATED_RUNTIME // an emulated link has no rate worth re-basing on
     if (!saved.model_seeded || saved.model_link_mbps < 1000 || saved.staged_copy_overhead_us < 1) {
       fprintf(stderr, "launch policy: the cost model was not re-based on the device\n");
       return 1;
     }
+#endif
     const int routes[3][2] = {{0, 0}, {2, 0}, {0, 2}}; // staged_restore, staged_gather
     for (int route = 0; route < 3; ++route)
       for (int notify = 0; notify < 2; ++notify) {
@@ -506,6 +508,7 @@ int main() {
     ++cases;
   }
 
+#ifndef FKV_EMULATED_RUNTIME // the next two sections are about the kernels themselves
   // ---- launch policy: every way a launch shares out its work, and the entry point that
   //      allocates nothing, on the same descriptor ----
   {
@@ -662,6 +665,7 @@ int main() {
     FKV_OK_OR_DIE(fkv_host_free(table_v));
     ++cases;
   }
+#endif
 
   // ---- the board processes share: one's own postings never count as "elsewhere" ----
   {
