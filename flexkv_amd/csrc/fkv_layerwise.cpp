@@ -485,7 +485,11 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
           (direct ? by_kernel : by_strategy).push_back(&it);
           continue;
         }
-        const bool second = two_dma_streams[i] && g->dma_streams2[i] && (g->dma_turn[i]++ & 1u);
+        // gathered batches are enqueued one by one as their rows become ready: nothing to hide
+        // there, and next to other work of the process the second stream cost 1 % (c3 with
+        // scattered host blocks behind c3 in one process: 42.3 ms against 41.9 ms)
+        const bool second = two_dma_streams[i] && g->dma_streams2[i] && sp->route == kRouteRuns &&
+                            (g->dma_turn[i]++ & 1u);
         const hipStream_t dma = second ? g->dma_streams2[i] : g->dma_streams[i];
         if (sp->route == kRouteGathered)
           rc = gathered_launch(*sp, g->rings[{it.lane, i}], g->pinned_rings[{it.lane, i}],

@@ -758,7 +758,8 @@ typedef struct fkv_launch_policy {
                                  enqueues its n-th batch, as a failed launch would (nothing faults:
                                  the batches before it run and are announced, the rest never lands) */
   int32_t staged_dma_streams; /* streams per GPU on which a layerwise restore issues its copy-engine
-                                 copies: 2 (default) consecutive batches alternate between two, so
+                                 copies, one per run of host blocks: 2 (default) consecutive batches
+                                 alternate between two (batches of gathered rows keep to one), so
                                  that the event record and wait around a copy run next to the other
                                  stream's copy (4 MiB a batch: 84 us against 93 us per batch; the
                                  engine still takes the copies in the order of submission); 1 all
