@@ -180,15 +180,24 @@ uint8_t *device_stage(int device, int slot, size_t bytes, hipStream_t stream) {
     }
     s.buf = static_cast<uint8_t *>(p);
     s.cap = bytes;
-  } else {
-    (void)hipStreamWaitEvent(stream, s.last_use, 0);
+  } else if (hipStreamWaitEvent(stream, s.last_use, 0) != hipSuccess) {
+    // the order behind the buffer's last user is not optional: the host waits instead
+    (void)hipGetLastError();
+    if (hipEventSynchronize(s.last_use) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
   }
   return s.buf;
 }
 void device_stage_mark(int device, int slot, hipStream_t stream) {
   DeviceStage &s = stage_set(device).dev[slot];
-  if (s.last_use)
-    (void)hipEventRecord(s.last_use, stream);
+  if (s.last_use && hipEventRecord(s.last_use, stream) != hipSuccess) {
+    // no mark for the next user to wait for: the buffer is idle before this returns
+    (void)hipGetLastError();
+    if (hipStreamSynchronize(stream) != hipSuccess)
+      (void)hipGetLastError();
+  }
 }
 
 uint8_t *host_stage(int device, size_t bytes) {
@@ -281,8 +290,13 @@ struct Job {
       return FKV_OK;
     StageSet &s = stage_set(device);
     aux = nullptr;
-    FKV_HIP_TRY(hipEventRecord(s.join, s.aux));
-    FKV_HIP_TRY(hipStreamWaitEvent(stream, s.join, 0));
+    // Also after an error part-way: nothing issued on the second stream may outlive the
+    // order of the caller's stream.  Where the runtime refuses the join, the host waits.
+    if (hipEventRecord(s.join, s.aux) != hipSuccess ||
+        hipStreamWaitEvent(stream, s.join, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      FKV_HIP_TRY(hipStreamSynchronize(s.aux));
+    }
     return FKV_OK;
   }
   hipStream_t next_stream() const {

@@ -924,6 +924,9 @@ int transfer_descs(const fkv_transfer_desc *descs, int count, hipStream_t stream
   using namespace fkv;
   const fkv_transfer_desc &d = descs[0];
   const bool sync = descs[count - 1].sync != 0, trace = descs[count - 1].enable_trace != 0;
+  // what an earlier, unrelated call of this thread left in the runtime's error slot is not
+  // this transfer's (the check at the end reads that slot)
+  (void)hipGetLastError();
   DeviceGuard guard(d.device);
   if (!guard.ok())
     return fail(FKV_ERR_RUNTIME, "cannot select HIP device %d", d.device);

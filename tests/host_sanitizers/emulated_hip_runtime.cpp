@@ -111,6 +111,25 @@ hipError_t remember(hipError_t e) {
   return e;
 }
 
+// Failures on request: after `after` more successful calls of a category the next `count`
+// calls of it fail (fkv_emulated_fail below).  What a real runtime does when memory, streams
+// or events run out, or a launch is refused.
+enum Category { kDeviceAlloc, kPinnedAlloc, kStreamCreate, kEventCreate, kCopy, kLaunch, kEventRecord,
+                kCategories };
+std::atomic<long> g_fail_after[kCategories];
+std::atomic<long> g_fail_count[kCategories];
+std::atomic<long> g_failed_calls{0};
+bool refused(Category c) {
+  if (g_fail_count[c].load(std::memory_order_relaxed) <= 0)
+    return false;
+  if (g_fail_after[c].fetch_sub(1) > 0)
+    return false;
+  if (g_fail_count[c].fetch_sub(1) <= 0)
+    return false;
+  g_failed_calls.fetch_add(1);
+  return true;
+}
+
 struct Runtime {
   std::mutex mu;
   // every live stream, the null stream first; shared, so that a device-wide wait can outlive
@@ -199,6 +218,8 @@ const char *hipGetErrorString(hipError_t e) {
   case hipErrorInvalidValue: return "invalid argument";
   case hipErrorOutOfMemory: return "out of memory";
   case hipErrorNotSupported: return "operation not supported";
+  case hipErrorLaunchFailure: return "launch failure";
+  case hipErrorInvalidHandle: return "invalid handle";
   default: return "emulated runtime error";
   }
 }
@@ -226,6 +247,8 @@ hipError_t hipDeviceGetPCIBusId(char *id, int len, int device) {
 }
 
 hipError_t hipStreamCreateWithFlags(hipStream_t *s, unsigned int) {
+  if (refused(kStreamCreate))
+    return remember(hipErrorOutOfMemory);
   auto made = std::make_shared<ihipStream_t>();
   *s = made.get();
   std::lock_guard<std::mutex> lk(rt().mu);
@@ -261,6 +284,8 @@ hipError_t hipStreamSynchronize(hipStream_t s) {
 hipError_t hipStreamQuery(hipStream_t s) { return of(s)->is_idle() ? hipSuccess : hipErrorNotReady; }
 
 hipError_t hipEventCreateWithFlags(hipEvent_t *e, unsigned int) {
+  if (refused(kEventCreate))
+    return remember(hipErrorOutOfMemory);
   *e = new ihipEvent_t();
   return hipSuccess;
 }
@@ -279,6 +304,8 @@ hipError_t hipEventDestroy(hipEvent_t e) {
 hipError_t hipEventRecord(hipEvent_t e, hipStream_t s) {
   if (!e)
     return remember(hipErrorInvalidHandle);
+  if (refused(kEventRecord))
+    return remember(hipErrorLaunchFailure);
   uint64_t gen;
   {
     std::lock_guard<std::mutex> lk(e->mu);
@@ -345,12 +372,12 @@ hipError_t hipEventElapsedTime(float *ms, hipEvent_t a, hipEvent_t b) {
 }
 
 hipError_t hipMalloc(void **p, size_t size) {
-  *p = allocate(size, false);
+  *p = refused(kDeviceAlloc) ? nullptr : allocate(size, false);
   return *p ? hipSuccess : remember(hipErrorOutOfMemory);
 }
 hipError_t hipFree(void *p) { return release(p, false); }
 hipError_t hipHostMalloc(void **p, size_t size, unsigned int) {
-  *p = allocate(size, true);
+  *p = refused(kPinnedAlloc) ? nullptr : allocate(size, true);
   return *p ? hipSuccess : remember(hipErrorOutOfMemory);
 }
 hipError_t hipHostFree(void *p) { return release(p, true); }
@@ -400,6 +427,8 @@ hipError_t hipMemGetAddressRange(hipDeviceptr_t *base, size_t *size, hipDevicept
 }
 
 hipError_t hipMemcpyAsync(void *dst, const void *src, size_t n, hipMemcpyKind, hipStream_t s) {
+  if (refused(kCopy))
+    return remember(hipErrorLaunchFailure);
   of(s)->push([dst, src, n] { std::memcpy(dst, src, n); });
   return hipSuccess;
 }
@@ -412,6 +441,8 @@ hipError_t hipMemcpy2DAsync(void *dst, size_t dpitch, const void *src, size_t sp
                             size_t height, hipMemcpyKind, hipStream_t s) {
   if (width > dpitch || width > spitch)
     return remember(hipErrorInvalidPitchValue);
+  if (refused(kCopy))
+    return remember(hipErrorLaunchFailure);
   of(s)->push([=] { copy_2d(dst, dpitch, src, spitch, width, height); });
   return hipSuccess;
 }
@@ -457,6 +488,8 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_wor
   if (a.num_blocks < 0 || a.lk < 0 || a.lk > kCopyMaxLK || a.chunk_bytes < 0 || num_workgroups < 1 ||
       threads_per_workgroup < 1)
     return fail(FKV_ERR_RUNTIME, "emulated copy kernel: bad launch");
+  if (refused(kLaunch))
+    return fail(FKV_ERR_RUNTIME, "emulated copy kernel: launch refused");
   g_launches.fetch_add(1);
   stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);
   of(stream)->push([a] { copy_rows(a); });
@@ -467,6 +500,8 @@ int launch_copy_jobs(const CopyKernelArgs *jobs, int njobs, int num_workgroups,
                      int threads_per_workgroup, hipStream_t stream) {
   if (njobs < 1 || njobs > kCopyMaxJobs)
     return fail(FKV_ERR_RUNTIME, "copy kernel: %d jobs in one launch (1..%d)", njobs, kCopyMaxJobs);
+  if (refused(kLaunch))
+    return fail(FKV_ERR_RUNTIME, "emulated copy kernel: launch refused");
   std::vector<CopyKernelArgs> all(jobs, jobs + njobs);
   stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);
   of(stream)->push([all] {
@@ -479,6 +514,8 @@ int launch_copy_jobs(const CopyKernelArgs *jobs, int njobs, int num_workgroups,
 uint64_t safety_net_ranges_of_current_device() { return 0; }
 
 int launch_plan_upload(void *device_dst, const void *pinned_src, size_t bytes, hipStream_t stream) {
+  if (refused(kLaunch))
+    return fail(FKV_ERR_RUNTIME, "emulated plan upload: launch refused");
   of(stream)->push([=] { std::memcpy(device_dst, pinned_src, bytes); });
   return FKV_OK;
 }
@@ -499,6 +536,17 @@ int common_vector_width(const uint64_t *vals, int n) {
 }
 
 } // namespace fkv
+
+// Test hook: the next `count` calls of `category` (0 device allocation, 1 pinned allocation,
+// 2 stream creation, 3 event creation, 4 copy, 5 kernel launch, 6 event record) fail once
+// `after` more of them have succeeded; count 0 switches it off.  Returns the calls refused so far.
+extern "C" long fkv_emulated_fail(int category, long after, long count) {
+  if (category >= 0 && category < kCategories) {
+    g_fail_after[category].store(after);
+    g_fail_count[category].store(count);
+  }
+  return g_failed_calls.load();
+}
 
 // Entry points of the library that live beside its kernels: not part of what runs here.
 extern "C" {

@@ -39,6 +39,7 @@ int fkv_oracle_tp_rank_plan(int rank, int num_gpus, int num_kv_heads, int is_hos
                             int layer_id, int layer_granularity, int num_blocks,
                             int64_t gpu_chunk_size, int64_t cpu_block_stride, int64_t cpu_tp_stride,
                             fkv_oracle_rank_plan *out);
+long fkv_emulated_fail(int category, long after, long count); // emulated_hip_runtime.cpp
 int fkv_oracle_transfer(int backend, const uint64_t *tensor_ptrs, int64_t num_layers_total,
                         int64_t gpu_kv_stride, int64_t gpu_block_stride, int64_t gpu_layer_stride,
                         int64_t gpu_off, uint8_t *cpu_ptr, int64_t cpu_kv_stride,
@@ -395,9 +396,26 @@ void transfer_case(uint64_t seed) {
     d.ce.enable_memcpy2d = rng() & 1;
     d.ce.gather_threads = pick(0, 4);
     d.ce.gather_nt = rng() & 1;
-    REQUIRE(fkv_transfer_kv_blocks(&d, st) == FKV_OK, "seed %llu rep %d: transfer",
-            (unsigned long long)seed, rep);
+    // every third transfer with the runtime refusing something part-way: it may fail, and what
+    // it leaves behind is the starting point of the next one
+    const bool inject = rep % 3 == 2;
+    if (inject)
+      fkv_emulated_fail(pick(0, 6), pick(0, 6), pick(1, 2));
+    const int rc = fkv_transfer_kv_blocks(&d, st);
     REQUIRE(hipStreamSynchronize(st) == hipSuccess, "sync");
+    for (int c = 0; c < 7; ++c)
+      fkv_emulated_fail(c, 0, 0);
+    REQUIRE(rc == FKV_OK || inject, "seed %llu rep %d: transfer", (unsigned long long)seed, rep);
+    if (rc != FKV_OK) {
+      { // the library's own streams included
+        void *probe = nullptr;
+        REQUIRE(hipMalloc(&probe, 64) == hipSuccess && hipFree(probe) == hipSuccess, "drain");
+      }
+      for (int l = 0; l < s.L; ++l)
+        std::memcpy(model[l].data(), dev[l], (size_t)s.layer_bytes());
+      std::memcpy(host_model.data(), host, host_model.size());
+      continue;
+    }
     for (int l = d.start_layer_id; l < d.start_layer_id + d.num_layers; ++l)
       for (int k = 0; k < s.kv; ++k)
         for (int q = 0; q < n; ++q) {
@@ -683,6 +701,119 @@ void concurrent_case(uint64_t seed) {
   REQUIRE(hipHostFree(host) == hipSuccess, "host free");
 }
 
+// The runtime runs out of something part-way: allocations, streams, events, copies, launches
+// and event records are refused at seeded points during layerwise restores on every route.
+// A refused call either is made up for (the kernel path needs no staging memory) or fails the
+// restore; it never hangs, corrupts or leaks into the next restore, which must be whole.
+void failure_case(uint64_t seed) {
+  std::mt19937_64 rng(seed);
+  auto pick = [&](int lo, int hi) { return lo + (int)(rng() % (uint64_t)(hi - lo + 1)); };
+  Shape s{};
+  s.ranks = pick(1, 2);
+  s.L = pick(2, 10);
+  s.kv = pick(1, 2);
+  s.NG = pick(6, 24);
+  s.NC = pick(6, 24);
+  s.chunk = 16 * pick(1, 64);
+  s.blockfirst = rng() & 1;
+  uint8_t *host = nullptr;
+  REQUIRE(hipHostMalloc((void **)&host, (size_t)s.host_bytes(), 0) == hipSuccess, "host pool");
+  std::vector<std::vector<uint8_t *>> dev(s.ranks);
+  std::vector<uint64_t> ptrs;
+  for (int r = 0; r < s.ranks; ++r)
+    for (int l = 0; l < s.L; ++l) {
+      uint8_t *d = nullptr;
+      REQUIRE(hipMalloc((void **)&d, (size_t)s.layer_bytes()) == hipSuccess, "engine tensor");
+      fill(rng, d, (size_t)s.layer_bytes());
+      dev[r].push_back(d);
+      ptrs.push_back((uint64_t)(uintptr_t)d);
+    }
+  std::vector<int32_t> fds;
+  for (int i = 0; i < s.ranks * s.L; ++i)
+    fds.push_back(eventfd(0, EFD_NONBLOCK));
+  std::vector<int64_t> kvs(s.ranks, s.gpu_kv_stride()), bs(s.ranks, s.gpu_block_stride()),
+      ls(s.ranks, s.layer_bytes()), cs(s.ranks, s.chunk), devs(s.ranks, 0);
+  fkv_layerwise_params p{};
+  p.num_gpus = s.ranks;
+  p.num_tensors_per_gpu = s.L;
+  p.gpu_block_ptrs_flat = ptrs.data();
+  p.cpu_blocks_ptr = host;
+  p.num_layers = s.L;
+  p.tp_size = s.ranks;
+  p.gpu_kv_strides = kvs.data();
+  p.gpu_block_strides = bs.data();
+  p.gpu_layer_strides = ls.data();
+  p.gpu_chunk_sizes = cs.data();
+  p.gpu_device_ids = devs.data();
+  p.layer_eventfds = fds.data();
+  p.num_layer_eventfds = (int32_t)fds.size();
+  fkv_ce_config_default(&p.ce);
+  p.ce.is_blockfirst = s.blockfirst;
+  fkv_layerwise *g = nullptr;
+  REQUIRE(fkv_layerwise_create(&p, &g) == FKV_OK, "create");
+  for (int rep = 0; rep < 6; ++rep) {
+    const int route = pick(1, 3);
+    std::vector<std::pair<std::string, int>> pol = {
+        {"model_seed", 0}, {"gather_threads", 3}, {"gather_first_by_kernel", pick(0, 1)},
+        {"kernel_alt_stream_kb", 4096}};
+    if (route == 1) { pol.push_back({"staged_restore", 0}); pol.push_back({"staged_gather", 0}); }
+    if (route == 2) { pol.push_back({"staged_restore", 2}); pol.push_back({"staged_gather", 0}); }
+    if (route == 3) { pol.push_back({"staged_restore", 0}); pol.push_back({"staged_gather", 3}); }
+    set_policy(pol);
+    const int n = pick(1, std::min(s.NG, s.NC));
+    std::vector<int64_t> gids(s.NG), cids(s.NC);
+    std::iota(gids.begin(), gids.end(), 0);
+    std::iota(cids.begin(), cids.end(), 0);
+    std::shuffle(gids.begin(), gids.end(), rng);
+    std::shuffle(cids.begin(), cids.end(), rng);
+    gids.resize(n);
+    cids.resize(n);
+    const int gran = pick(1, 3), use_ce = (rng() % 4) == 0;
+    const int notify = (rng() & 1) ? FKV_NOTIFY_POLLING : FKV_NOTIFY_HOSTFUNC;
+    const bool inject = rep % 2 == 0;
+    fill(rng, host, (size_t)s.host_bytes());
+    if (inject)
+      fkv_emulated_fail(pick(0, 6), pick(0, 12), pick(1, 3));
+    const int rc = fkv_layerwise_transfer(g, gids.data(), cids.data(), n, s.cpu_block_stride(),
+                                          s.cpu_kv_stride(), s.cpu_layer_stride(),
+                                          s.cpu_block_stride(), 4, use_ce, s.L, gran, s.kv, 1, 0,
+                                          "sharded", notify, 0);
+    const int src = fkv_layerwise_synchronize(g);
+    for (int c = 0; c < 7; ++c)
+      fkv_emulated_fail(c, 0, 0);
+    if (!inject)
+      REQUIRE(rc == FKV_OK && src == FKV_OK, "seed %llu rep %d: a clean restore failed (route %d)",
+              (unsigned long long)seed, rep, route);
+    if (rc == FKV_OK && src == FKV_OK) {
+      // whole: every rank has every block of every layer, and every layer was announced once
+      for (int r = 0; r < s.ranks; ++r)
+        for (int l = 0; l < s.L; ++l)
+          for (int k = 0; k < s.kv; ++k)
+            for (int q = 0; q < n; ++q)
+              REQUIRE(std::memcmp(dev[r][l] + k * s.gpu_kv_stride() + gids[q] * s.chunk,
+                                  host + cids[q] * s.cpu_block_stride() + l * s.cpu_layer_stride() +
+                                      k * s.cpu_kv_stride(), (size_t)s.chunk) == 0,
+                      "seed %llu rep %d: rank %d layer %d block %d differs after a restore that "
+                      "reported success (route %d, injected %d)", (unsigned long long)seed, rep, r, l,
+                      q, route, (int)inject);
+      for (int fd : fds)
+        REQUIRE(drain(fd) == 1, "seed %llu rep %d: a layer was not announced exactly once",
+                (unsigned long long)seed, rep);
+    } else {
+      for (int fd : fds)
+        REQUIRE(drain(fd) <= 1, "seed %llu rep %d: a layer was announced twice",
+                (unsigned long long)seed, rep);
+    }
+  }
+  fkv_layerwise_destroy(g);
+  for (int fd : fds)
+    close(fd);
+  for (auto &rank : dev)
+    for (uint8_t *d : rank)
+      REQUIRE(hipFree(d) == hipSuccess, "free");
+  REQUIRE(hipHostFree(host) == hipSuccess, "host free");
+}
+
 } // namespace
 
 int main(int argc, char **argv) {
@@ -694,6 +825,9 @@ int main(int argc, char **argv) {
   for (int i = 0; i < transfers; ++i)
     concurrent_case(10000 + i);
   for (int i = 0; i < restores; ++i)
+    failure_case(12000 + i);
+  const long refused_calls = fkv_emulated_fail(-1, 0, 0);
+  for (int i = 0; i < restores; ++i)
     layerwise_case(9000 + i);
   // four ranks that share their KV, rows gathered by host threads, asked for on the copy
   // engine: the launching thread serves four staging rings and eight copy streams
@@ -703,6 +837,7 @@ int main(int argc, char **argv) {
   for (int i = 0; i < restores / 2; ++i)
     layerwise_case(11000 + i, four);
   printf("ok: %d groups of layerwise restores, %d sets of transfers, %d thread groups and %d bursts "
-         "of concurrent calls over the emulated runtime\n", restores, transfers, transfers, transfers);
+         "of concurrent calls over the emulated runtime; %ld runtime calls refused on request\n",
+         restores, transfers, transfers, transfers, refused_calls);
   return 0;
 }

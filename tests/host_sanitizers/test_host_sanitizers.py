@@ -117,7 +117,10 @@ def test_whole_host_side_over_an_emulated_runtime_under_sanitizers(tmp_path, san
     pageable pools, both notify modes with eventfds, consumers gated per layer, restores that
     give up part-way; plain puts and gets on the kernel path and through every copy-engine
     strategy; the thread group of a tensor-parallel engine in every shared-KV mode and with
-    head slices (against the oracle's rank plan); puts and gets from several threads at once:
+    head slices (against the oracle's rank plan); puts and gets from several threads at once;
+    restores and transfers during which the runtime refuses allocations, streams, events,
+    copies, launches or event records at seeded points (they fail or are made up for, and the
+    next one is whole):
     the library's host code as it is shipped, over a HIP runtime made of threads, every byte
     against a plain model.  The library keeps per-stream events and staging memory until the
     process ends, so leak checking is off for this program."""
@@ -128,6 +131,7 @@ def test_whole_host_side_over_an_emulated_runtime_under_sanitizers(tmp_path, san
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
     assert ("ok: 80 groups of layerwise restores, 40 sets of transfers, 40 thread groups and "
             "40 bursts of concurrent calls") in r.stdout
+    assert "runtime calls refused on request" in r.stdout
 
 
 @pytest.mark.parametrize("sanitizer", SANITIZERS)
