@@ -535,11 +535,30 @@ void tp_case(uint64_t seed) {
     const int layer_id = pick(0, s.L - 1), gran = pick(1, s.L - layer_id);
     const int use_ce = s.chunk % 8 == 0 ? pick(0, 1) : 0;
     const int designated = pick(0, n - 1);
+    // every third call with the runtime refusing something in one of the rank threads
+    const bool inject = rep % 3 == 2;
+    if (inject)
+      fkv_emulated_fail(pick(0, 6), pick(0, 4), pick(1, 2));
     const int rc = fkv_tp_group_transfer(g, gids.data(), cids.data(), nb, cpu_kv_stride,
                                          cpu_layer_stride, cpu_block_stride, cpu_tp_stride, 4, h2d,
                                          use_ce, layer_id, gran, s.kv, heads, mode.c_str(), designated);
-    REQUIRE(rc == FKV_OK, "seed %llu rep %d: tp transfer (mode %s h2d %d ce %d)",
+    for (int c = 0; c < 7; ++c)
+      fkv_emulated_fail(c, 0, 0);
+    REQUIRE(rc == FKV_OK || inject, "seed %llu rep %d: tp transfer (mode %s h2d %d ce %d)",
             (unsigned long long)seed, rep, mode.c_str(), h2d, use_ce);
+    if (rc != FKV_OK) {
+      { // whatever the ranks left in flight
+        void *probe = nullptr;
+        REQUIRE(hipMalloc(&probe, 64) == hipSuccess && hipFree(probe) == hipSuccess, "drain");
+      }
+      for (int r = 0; r < n; ++r)
+        for (int l = 0; l < s.L; ++l)
+          std::memcpy(model[r][l].data(), dev[r][l], (size_t)s.layer_bytes());
+      std::memcpy(host_model.data(), host, host_model.size());
+      if (!h2d && shared && mode == "rank_rotate")
+        ++puts; // the writer moves on with every put that was asked for
+      continue;
+    }
     for (int r = 0; r < n; ++r) {
       fkv_oracle_rank_plan plan{};
       REQUIRE(fkv_oracle_tp_rank_plan(r, n, heads, h2d, mode.c_str(), designated, puts % n, layer_id,
