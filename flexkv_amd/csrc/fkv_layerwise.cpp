@@ -41,6 +41,7 @@
 #include <sys/eventfd.h>
 #include <unistd.h>
 
+#include <exception>
 #include <atomic>
 #include <condition_variable>
 #include <cstring>
@@ -1046,8 +1047,13 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
     g->poller_stop.store(false, std::memory_order_release);
     // Nobody listens when no eventfd table was given: in-process consumers wait
     // on the batch events directly, so there is nothing to poll for.
-    if (num_batches > 0 && !g->eventfds.empty())
-      g->poller = std::thread([g] { g->poll_loop(); });
+    if (num_batches > 0 && !g->eventfds.empty()) {
+      try {
+        g->poller = std::thread([g] { g->poll_loop(); });
+      } catch (const std::exception &) {
+        g->poll_loop(); // no thread to be had: the calling thread announces the layers, and blocks for it
+      }
+    }
   } else {
     // announce every batch as soon as all GPUs have finished it, in order
     for (int b = 0; b < num_batches; ++b) {

@@ -31,6 +31,7 @@
 #include <sys/uio.h>
 #include <unistd.h>
 
+#include <exception>
 #include <algorithm>
 #include <atomic>
 #include <cerrno>
@@ -375,8 +376,13 @@ void run_threads(const Plan &plan, bool is_read, int num_threads, Outcome *out) 
     }
   };
   std::vector<std::thread> pool;
-  for (int t = 1; t < num_threads; ++t)
-    pool.emplace_back(work);
+  for (int t = 1; t < num_threads; ++t) {
+    try {
+      pool.emplace_back(work);
+    } catch (const std::exception &) { // no more threads to be had: those there are do the work
+      break;
+    }
+  }
   work();
   for (auto &t : pool)
     t.join();

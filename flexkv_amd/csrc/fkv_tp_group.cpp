@@ -8,6 +8,7 @@
 // cross-rank logic is the placement rule in fkv_tp_rank_plan_compute().
 #include "fkv_internal.h"
 
+#include <exception>
 #include <condition_variable>
 #include <cstring>
 #include <deque>
@@ -214,8 +215,15 @@ int fkv_tp_group_create(const fkv_tp_group_params *p, fkv_tp_group **out) {
   for (int i = 0; i < p->num_gpus; ++i)
     g->lanes.push_back(std::make_unique<fkv_tp_group::Lane>());
   fkv_tp_group *raw = g.get();
-  for (int i = 0; i < p->num_gpus; ++i)
-    raw->lanes[i]->th = std::thread([raw, i] { raw->lane_loop(i); });
+  try {
+    for (int i = 0; i < p->num_gpus; ++i)
+      raw->lanes[i]->th = std::thread([raw, i] { raw->lane_loop(i); });
+  } catch (const std::exception &e) { // nothing may cross the C ABI
+    const std::string what = e.what();
+    fkv_tp_group_destroy(g.release()); // stops and joins the threads that did start
+    return fail(FKV_ERR_RUNTIME, "fkv_tp_group_create: cannot start the rank threads: %s",
+                what.c_str());
+  }
   *out = g.release();
   return FKV_OK;
 }
