@@ -1091,7 +1091,7 @@ extern "C" {
 int fkv_ce_analyze(const int64_t *gpu_block_ids, const int64_t *cpu_block_ids,
                    int32_t num_blocks, int64_t cpu_block_stride, int64_t chunk_size,
                    int64_t gpu_block_stride, fkv_ce_analysis *out, fkv_ce_segment *segments,
-                   int32_t segment_capacity) {
+                   int32_t segment_capacity) try {
   fkv::clear_error();
   if (!out || num_blocks < 0 || (num_blocks > 0 && (!gpu_block_ids || !cpu_block_ids)))
     return fkv::fail(FKV_ERR_INVALID_ARG, "fkv_ce_analyze: bad arguments");
@@ -1103,11 +1103,15 @@ int fkv_ce_analyze(const int64_t *gpu_block_ids, const int64_t *cpu_block_ids,
     for (int i = 0; i < (int)an.segs.size() && i < segment_capacity; ++i)
       segments[i] = an.segs[i];
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 int fkv_ce_choose_path(const fkv_ce_analysis *analysis, const fkv_ce_config *cfg,
-                       int64_t chunk_size, int32_t is_host_to_device, int32_t is_full_block) {
+                       int64_t chunk_size, int32_t is_host_to_device, int32_t is_full_block) try {
   return fkv::choose(*analysis, *cfg, chunk_size, is_host_to_device != 0, is_full_block != 0);
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 } // extern "C"

@@ -32,6 +32,22 @@ int fail(int code, const char *fmt, ...) {
   return code;
 }
 void clear_error() { t_last_error.clear(); }
+
+int caught(const char *where) noexcept {
+  try {
+    try {
+      throw;
+    } catch (const std::bad_alloc &) {
+      return fail(FKV_ERR_RUNTIME, "%s: out of host memory", where);
+    } catch (const std::exception &e) {
+      return fail(FKV_ERR_RUNTIME, "%s: %s", where, e.what());
+    } catch (...) {
+      return fail(FKV_ERR_RUNTIME, "%s: unknown exception", where);
+    }
+  } catch (...) { // not even the text could be kept
+    return FKV_ERR_RUNTIME;
+  }
+}
 void set_last_path(int path) { t_last_path = path; }
 
 Stats &stats() {
@@ -696,7 +712,7 @@ void fkv_ce_config_default(fkv_ce_config *cfg) {
 }
 
 int fkv_choose_engine(const fkv_transfer_desc *desc, int32_t *use_ce, double *est_kernel_ms,
-                      double *est_ce_ms) {
+                      double *est_ce_ms) try {
   fkv::clear_error();
   if (!desc || !use_ce)
     return fkv::fail(FKV_ERR_INVALID_ARG, "fkv_choose_engine: null argument");
@@ -711,6 +727,8 @@ int fkv_choose_engine(const fkv_transfer_desc *desc, int32_t *use_ce, double *es
   if (est_ce_ms)
     *est_ce_ms = tc * 1e3;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 void fkv_get_stats(fkv_stats *out) {
@@ -1021,7 +1039,7 @@ int transfer_descs(const fkv_transfer_desc *descs, int count, hipStream_t stream
 
 extern "C" {
 
-int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream_v) {
+int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream_v) try {
   using namespace fkv;
   clear_error();
   if (!desc)
@@ -1031,9 +1049,11 @@ int fkv_transfer_kv_blocks(const fkv_transfer_desc *desc, void *stream_v) {
   if (desc->num_blocks == 0 || desc->num_layers == 0)
     return FKV_OK;
   return transfer_descs(desc, 1, static_cast<hipStream_t>(stream_v));
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_transfer_kv_blocks_multi(const fkv_transfer_desc *descs, int32_t count, void *stream_v) {
+int fkv_transfer_kv_blocks_multi(const fkv_transfer_desc *descs, int32_t count, void *stream_v) try {
   using namespace fkv;
   clear_error();
   if (count < 0 || (count > 0 && !descs))
@@ -1055,6 +1075,8 @@ int fkv_transfer_kv_blocks_multi(const fkv_transfer_desc *descs, int32_t count, 
   work.back().sync = descs[count - 1].sync;
   work.back().enable_trace = descs[count - 1].enable_trace;
   return transfer_descs(work.data(), (int)work.size(), static_cast<hipStream_t>(stream_v));
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 } // extern "C"

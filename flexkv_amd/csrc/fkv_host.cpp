@@ -43,7 +43,7 @@ int64_t fkv_host_register_plan(size_t bytes, size_t chunk_bytes, size_t *offsets
   return n;
 }
 
-int fkv_host_alloc(size_t bytes, void **out) {
+int fkv_host_alloc(size_t bytes, void **out) try {
   fkv::clear_error();
   if (!out || bytes == 0)
     return fkv::fail(FKV_ERR_INVALID_ARG, "fkv_host_alloc: bad arguments");
@@ -56,17 +56,21 @@ int fkv_host_alloc(size_t bytes, void **out) {
   }
   *out = p;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_host_free(void *ptr) {
+int fkv_host_free(void *ptr) try {
   fkv::clear_error();
   if (!ptr)
     return FKV_OK;
   FKV_HIP_TRY(hipHostFree(ptr));
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_host_register(void *ptr, size_t bytes, size_t chunk_bytes) {
+int fkv_host_register(void *ptr, size_t bytes, size_t chunk_bytes) try {
   fkv::clear_error();
   if (!ptr || bytes == 0)
     return fkv::fail(FKV_ERR_INVALID_ARG, "fkv_host_register: bad arguments");
@@ -87,9 +91,11 @@ int fkv_host_register(void *ptr, size_t bytes, size_t chunk_bytes) {
     }
   }
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_host_unregister(void *ptr, size_t bytes, size_t chunk_bytes) {
+int fkv_host_unregister(void *ptr, size_t bytes, size_t chunk_bytes) try {
   fkv::clear_error();
   if (!ptr || bytes == 0)
     return fkv::fail(FKV_ERR_INVALID_ARG, "fkv_host_unregister: bad arguments");
@@ -107,10 +113,12 @@ int fkv_host_unregister(void *ptr, size_t bytes, size_t chunk_bytes) {
     return fkv::fail(FKV_ERR_RUNTIME, "hipHostUnregister failed for %d of %lld pieces", bad,
                      (long long)n);
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 int fkv_measure_link_peak(int32_t device, size_t bytes, int32_t reps, int32_t direction,
-                          double *best_gbps, double *median_gbps) {
+                          double *best_gbps, double *median_gbps) try {
   using namespace fkv;
   clear_error();
   if (bytes == 0 || reps < 1 || !best_gbps)
@@ -170,6 +178,8 @@ int fkv_measure_link_peak(int32_t device, size_t bytes, int32_t reps, int32_t di
   if (median_gbps)
     *median_gbps = rates[rates.size() / 2];
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 } // extern "C"

@@ -17,6 +17,9 @@ namespace fkv {
 // ---- errors -------------------------------------------------------------
 // Records the message for fkv_last_error() on this thread and returns `code`.
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+// For the catch-all handler of an entry point: turns the exception in flight into a status
+// and an error text.  No C++ exception crosses the C ABI.
+int caught(const char *where) noexcept;
 void clear_error();
 
 #define FKV_HIP_TRY(expr)                                                      \

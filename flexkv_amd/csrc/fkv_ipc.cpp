@@ -35,7 +35,7 @@ std::string key_of(const uint8_t *handle, int device) {
 extern "C" {
 
 int fkv_ipc_export(const void *device_ptr, uint8_t *handle_out, int64_t *offset_out,
-                   int64_t *allocation_bytes_out) {
+                   int64_t *allocation_bytes_out) try {
   using namespace fkv;
   clear_error();
   if (!device_ptr || !handle_out || !offset_out)
@@ -51,9 +51,11 @@ int fkv_ipc_export(const void *device_ptr, uint8_t *handle_out, int64_t *offset_
   if (allocation_bytes_out)
     *allocation_bytes_out = (int64_t)size;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_ipc_open(const uint8_t *handle, int32_t device, void **base_out) {
+int fkv_ipc_open(const uint8_t *handle, int32_t device, void **base_out) try {
   using namespace fkv;
   clear_error();
   if (!handle || !base_out)
@@ -80,9 +82,11 @@ int fkv_ipc_open(const uint8_t *handle, int32_t device, void **base_out) {
   ++m.refs;
   *base_out = m.base;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_ipc_close(void *base) {
+int fkv_ipc_close(void *base) try {
   using namespace fkv;
   clear_error();
   if (!base)
@@ -103,6 +107,8 @@ int fkv_ipc_close(void *base) {
     return FKV_OK;
   }
   return fail(FKV_ERR_INVALID_ARG, "fkv_ipc_close: %p was not opened by fkv_ipc_open", base);
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 } // extern "C"

@@ -763,7 +763,7 @@ __global__ __launch_bounds__(1024) void fkv_hbm_yardstick_kernel(const hbm_vec *
 } // namespace fkv
 
 extern "C" int fkv_measure_hbm_rate(int32_t device, size_t bytes, int32_t reps, int32_t mode,
-                                    double *best_gbps, double *median_gbps) {
+                                    double *best_gbps, double *median_gbps) try {
   using namespace fkv;
   clear_error();
   if (bytes < (1u << 20) || reps < 1 || mode < 0 || mode > 2 || !best_gbps)
@@ -827,10 +827,12 @@ extern "C" int fkv_measure_hbm_rate(int32_t device, size_t bytes, int32_t reps, 
   if (median_gbps)
     *median_gbps = rates[rates.size() / 2];
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 extern "C" int fkv_streams_run_concurrently(int32_t device, void *stream_a, void *stream_b,
-                                            int32_t *concurrent) {
+                                            int32_t *concurrent) try {
   using namespace fkv;
   clear_error();
   if (!concurrent)
@@ -868,4 +870,6 @@ extern "C" int fkv_streams_run_concurrently(int32_t device, void *stream_a, void
   }
   *concurrent = two < 1.5 * one ? 1 : 0;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }

@@ -234,7 +234,22 @@ struct fkv_layerwise {
   void notify(const Batch &b) const { notify_layers(b.start_layer, b.layers); }
 
   void poll_loop() {
-    const int status = fkv::poll_batches_in_order(
+    int status;
+    try {
+      status = poll_batches();
+    } catch (...) { // as a device error would: the layers behind it are not announced
+      status = (int)hipErrorUnknown;
+    }
+    if (status != (int)hipSuccess) {
+      // A real device error: the layers behind it were not announced; the next call
+      // on the group reports it.
+      int none = 0;
+      restore_error.compare_exchange_strong(none, status);
+    }
+  }
+
+  int poll_batches() {
+    return fkv::poll_batches_in_order(
         batches.size(), num_gpus, (int)hipSuccess, (int)hipErrorNotReady,
         [this](size_t b, int g) {
           // an event that has not been recorded yet reads as complete
@@ -248,12 +263,6 @@ struct fkv_layerwise {
           return (int)e;
         },
         [this](size_t b) { notify(*batches[b]); }, poller_stop);
-    if (status != (int)hipSuccess) {
-      // A real device error: the layers behind it were not announced; the next call
-      // on the group reports it.
-      int none = 0;
-      restore_error.compare_exchange_strong(none, status);
-    }
   }
 
   // The launching thread ends by itself: it waits for nothing but copies that are
@@ -601,7 +610,7 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
 
 extern "C" {
 
-int fkv_layerwise_create(const fkv_layerwise_params *p, fkv_layerwise **out) {
+int fkv_layerwise_create(const fkv_layerwise_params *p, fkv_layerwise **out) try {
   using namespace fkv;
   clear_error();
   if (!p || !out || p->num_gpus < 1 || p->num_tensors_per_gpu < 1 || p->num_layers < 1 ||
@@ -630,9 +639,11 @@ int fkv_layerwise_create(const fkv_layerwise_params *p, fkv_layerwise **out) {
   FKV_TRY(finish_create(g, p->gpu_device_ids, p->layer_eventfds, p->num_layer_eventfds));
   *out = g.release();
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_layerwise_create_multi_group(const fkv_layerwise_mg_params *p, fkv_layerwise **out) {
+int fkv_layerwise_create_multi_group(const fkv_layerwise_mg_params *p, fkv_layerwise **out) try {
   using namespace fkv;
   clear_error();
   if (!p || !out || p->num_gpus < 1 || p->num_original_layers < 1 || p->tp_size < 1 ||
@@ -661,10 +672,12 @@ int fkv_layerwise_create_multi_group(const fkv_layerwise_mg_params *p, fkv_layer
   FKV_TRY(finish_create(g, p->gpu_device_ids, p->layer_eventfds, p->num_layer_eventfds));
   *out = g.release();
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 int fkv_layerwise_init_swa(fkv_layerwise *g, const fkv_layer_group *swa,
-                           void *swa_cpu_blocks_ptr) {
+                           void *swa_cpu_blocks_ptr) try {
   using namespace fkv;
   clear_error();
   if (!g || !swa || !swa_cpu_blocks_ptr)
@@ -686,12 +699,14 @@ int fkv_layerwise_init_swa(fkv_layerwise *g, const fkv_layer_group *swa,
   g->has_swa = true;
   g->swa_multi_group = false;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 int fkv_layerwise_init_swa_multi_group(fkv_layerwise *g, const fkv_layer_group *groups,
                                        int32_t num_groups, const int32_t *member_offsets,
                                        const fkv_layer_member *members,
-                                       void *swa_cpu_blocks_ptr) {
+                                       void *swa_cpu_blocks_ptr) try {
   using namespace fkv;
   clear_error();
   if (!g || !groups || num_groups < 1)
@@ -725,9 +740,11 @@ int fkv_layerwise_init_swa_multi_group(fkv_layerwise *g, const fkv_layer_group *
   g->has_swa = true;
   g->swa_multi_group = true;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call) {
+int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call) try {
   using namespace fkv;
   clear_error();
   if (!g || !call)
@@ -1016,7 +1033,12 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
       }
     auto feed = [g] {
       const EngineChoice how{g->feed_use_ce, g->feed_num_cta};
-      const int frc = launch_batches(g, g->feed_lanes, how, true, FKV_OK);
+      int frc;
+      try {
+        frc = launch_batches(g, g->feed_lanes, how, true, FKV_OK);
+      } catch (...) { // a thread of the library ends with a status, not with std::terminate
+        frc = caught("launching thread of a layerwise restore");
+      }
       if (frc != FKV_OK) {
         g->feed_rc = frc; // read by others only after they have joined this thread
         g->feed_error = fkv_last_error();
@@ -1113,6 +1135,8 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
   }
   (void)hipSetDevice(restore.device());
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
@@ -1122,7 +1146,7 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
                            int32_t transfer_cta_num, int32_t use_ce_transfer,
                            int32_t num_layers, int32_t layer_granularity, int32_t kv_dim,
                            int32_t num_kv_heads, int32_t counter_id, const char *mode,
-                           int32_t notify_mode, int32_t enable_trace) {
+                           int32_t notify_mode, int32_t enable_trace) try {
   fkv_layerwise_call c{};
   c.gpu_block_ids = gpu_block_ids;
   c.cpu_block_ids = cpu_block_ids;
@@ -1143,10 +1167,12 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
   c.enable_trace = enable_trace;
   c.kv_shared_across_ranks_mode = mode;
   return fkv_layerwise_transfer_call(g, &c);
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 int fkv_layerwise_wait_layer(fkv_layerwise *g, int32_t gpu_index, int32_t layer,
-                             void *consumer_stream) {
+                             void *consumer_stream) try {
   using namespace fkv;
   clear_error();
   if (!g || gpu_index < 0 || gpu_index >= g->num_gpus)
@@ -1168,9 +1194,11 @@ int fkv_layerwise_wait_layer(fkv_layerwise *g, int32_t gpu_index, int32_t layer,
   FKV_HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(consumer_stream),
                                  g->batches[b]->done[gpu_index], 0));
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_layerwise_synchronize(fkv_layerwise *g) {
+int fkv_layerwise_synchronize(fkv_layerwise *g) try {
   using namespace fkv;
   clear_error();
   if (!g)
@@ -1183,10 +1211,12 @@ int fkv_layerwise_synchronize(fkv_layerwise *g) {
   }
   (void)hipSetDevice(restore.device());
   return g->take_restore_error("fkv_layerwise_synchronize");
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 int fkv_layerwise_batch_times_ms(fkv_layerwise *g, float *out_ms, int32_t capacity,
-                                 int32_t *num_batches) {
+                                 int32_t *num_batches) try {
   using namespace fkv;
   clear_error();
   if (!g || !num_batches)
@@ -1199,6 +1229,8 @@ int fkv_layerwise_batch_times_ms(fkv_layerwise *g, float *out_ms, int32_t capaci
   for (int b = 0; b < (int)g->batches.size() && b < capacity; ++b)
     FKV_HIP_TRY(hipEventElapsedTime(&out_ms[b], g->started, g->batches[b]->done[0]));
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 void fkv_layerwise_destroy(fkv_layerwise *g) {

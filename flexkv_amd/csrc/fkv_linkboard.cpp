@@ -211,17 +211,19 @@ int resolve_device(int32_t device) {
 } // namespace fkv
 
 extern "C" int fkv_link_activity_post(int32_t device, int32_t is_host_to_device,
-                                      int64_t expected_us) {
+                                      int64_t expected_us) try {
   using namespace fkv;
   clear_error();
   if (expected_us < 0)
     return fail(FKV_ERR_INVALID_ARG, "fkv_link_activity_post: negative duration");
   link_board_post(resolve_device(device), is_host_to_device != 0, expected_us * 1000);
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 extern "C" int fkv_link_activity_elsewhere(int32_t device, int32_t is_host_to_device,
-                                           int32_t window_ms, int32_t *busy) {
+                                           int32_t window_ms, int32_t *busy) try {
   using namespace fkv;
   clear_error();
   if (!busy)
@@ -231,4 +233,6 @@ extern "C" int fkv_link_activity_elsewhere(int32_t device, int32_t is_host_to_de
               ? 1
               : 0;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }

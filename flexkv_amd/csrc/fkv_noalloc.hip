@@ -116,7 +116,7 @@ const int64_t *device_view_of(const int64_t *p) {
 
 } // namespace
 
-extern "C" int fkv_transfer_kv_blocks_noalloc(const fkv_transfer_desc *desc, void *stream_v) {
+extern "C" int fkv_transfer_kv_blocks_noalloc(const fkv_transfer_desc *desc, void *stream_v) try {
   using namespace fkv;
   clear_error();
   if (!desc)
@@ -184,4 +184,6 @@ extern "C" int fkv_transfer_kv_blocks_noalloc(const fkv_transfer_desc *desc, voi
   if (d.sync)
     FKV_HIP_TRY(hipStreamSynchronize(stream));
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }

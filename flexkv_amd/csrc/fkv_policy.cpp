@@ -377,7 +377,7 @@ fkv_launch_policy policy_peek(int device) {
 
 extern "C" {
 
-int fkv_launch_policy_get(int32_t device, fkv_launch_policy *out) {
+int fkv_launch_policy_get(int32_t device, fkv_launch_policy *out) try {
   using namespace fkv;
   clear_error();
   if (!out)
@@ -386,9 +386,11 @@ int fkv_launch_policy_get(int32_t device, fkv_launch_policy *out) {
   FKV_TRY(resolve(device, &dev));
   *out = policy_of(dev);
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_launch_policy_set(int32_t device, const fkv_launch_policy *in) {
+int fkv_launch_policy_set(int32_t device, const fkv_launch_policy *in) try {
   using namespace fkv;
   clear_error();
   if (!in)
@@ -402,19 +404,23 @@ int fkv_launch_policy_set(int32_t device, const fkv_launch_policy *in) {
   sanitize(p, t.derived);
   t.current = p;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_launch_policy_seed(int32_t device) {
+int fkv_launch_policy_seed(int32_t device) try {
   using namespace fkv;
   clear_error();
   int dev = 0;
   FKV_TRY(resolve(device, &dev));
   (void)policy_of_seeded(dev);
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 int fkv_launch_policy_seeded(const fkv_launch_policy *in, double d2h_gbps, double h2d_gbps,
-                             double copy_overhead_us, fkv_launch_policy *out) {
+                             double copy_overhead_us, fkv_launch_policy *out) try {
   using namespace fkv;
   clear_error();
   if (!in || !out)
@@ -424,9 +430,11 @@ int fkv_launch_policy_seeded(const fkv_launch_policy *in, double d2h_gbps, doubl
   seed_from_measurement(p, d2h_gbps, h2d_gbps, copy_overhead_us);
   *out = p;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_launch_policy_reset(int32_t device) {
+int fkv_launch_policy_reset(int32_t device) try {
   using namespace fkv;
   clear_error();
   int dev = 0;
@@ -436,6 +444,8 @@ int fkv_launch_policy_reset(int32_t device) {
   DevicePolicy &t = tables()[dev];
   t.current = t.derived;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 } // extern "C"

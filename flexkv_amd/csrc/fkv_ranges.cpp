@@ -62,18 +62,22 @@ Range::~Range() {
 } // namespace fkv
 
 extern "C" {
-int fkv_range_push(const char *label) {
+int fkv_range_push(const char *label) try {
   const Markers &m = markers();
   if (!m.push || !label)
     return 0;
   m.push(label);
   return 1;
+} catch (...) {
+  return fkv::caught(__func__);
 }
-int fkv_range_pop(void) {
+int fkv_range_pop(void) try {
   const Markers &m = markers();
   if (!m.pop)
     return 0;
   m.pop();
   return 1;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 }

@@ -511,7 +511,7 @@ bool direct_io_possible(const SsdCall &c) {
 extern "C" {
 
 int fkv_ssd_locate(int64_t ssd_block_id, int32_t round_robin, int32_t num_devices,
-                   int32_t files_per_device, int32_t *device, int32_t *file, int64_t *block_in_file) {
+                   int32_t files_per_device, int32_t *device, int32_t *file, int64_t *block_in_file) try {
   fkv::clear_error();
   if (ssd_block_id < 0 || round_robin < 1 || num_devices < 1 || files_per_device < 1 || !device ||
       !file || !block_in_file)
@@ -521,10 +521,12 @@ int fkv_ssd_locate(int64_t ssd_block_id, int32_t round_robin, int32_t num_device
   *file = p.file;
   *block_in_file = p.in_file;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 int fkv_ssd_open(const char *const *paths, int32_t num_devices, int32_t files_per_device,
-                 int32_t iouring_entries, int32_t iouring_flags, fkv_ssd_ctx **out) {
+                 int32_t iouring_entries, int32_t iouring_flags, fkv_ssd_ctx **out) try {
   fkv::clear_error();
   if (!paths || !out || num_devices < 1 || files_per_device < 1)
     return fail(FKV_ERR_INVALID_ARG, "fkv_ssd_open: bad arguments");
@@ -560,6 +562,8 @@ int fkv_ssd_open(const char *const *paths, int32_t num_devices, int32_t files_pe
   ctx->write_ioprio = ioprio_value(kIoprioBE, 4);
   *out = ctx.release();
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 int fkv_ssd_uses_iouring(const fkv_ssd_ctx *ctx) { return ctx && ctx->ring ? 1 : 0; }
@@ -573,7 +577,7 @@ int fkv_ssd_transfer(fkv_ssd_ctx *ctx, int32_t start_layer, int32_t num_layers, 
                      int32_t num_blocks, int64_t cpu_layer_stride, int64_t cpu_kv_stride,
                      int64_t ssd_layer_stride, int64_t ssd_kv_stride, int64_t chunk_size,
                      int64_t block_stride, int32_t is_read, int32_t round_robin,
-                     int32_t num_threads_per_device, int32_t kv_dim, int32_t ssd_io_opt) {
+                     int32_t num_threads_per_device, int32_t kv_dim, int32_t ssd_io_opt) try {
   fkv::clear_error();
   if (!ctx)
     return fail(FKV_ERR_INVALID_ARG, "fkv_ssd_transfer: null context");
@@ -613,6 +617,8 @@ int fkv_ssd_transfer(fkv_ssd_ctx *ctx, int32_t start_layer, int32_t num_layers, 
                 out.failed.load(), plan.requests.size(), is_read ? "read" : "write",
                 std::strerror(out.err.load()));
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 int64_t fkv_ssd_plan(int32_t num_devices, int32_t files_per_device, int32_t start_layer,

@@ -487,7 +487,7 @@ extern "C" int fkv_staged_restore_plan(const int64_t *cpu_block_ids, int32_t num
                                        const fkv_launch_policy *policy, int32_t *staged,
                                        int32_t *num_runs, int64_t *total_rows,
                                        fkv_staged_run *runs, int32_t run_capacity,
-                                       int64_t *row_of_position) {
+                                       int64_t *row_of_position) try {
   using namespace fkv;
   clear_error();
   if (!policy || !staged || num_blocks < 0 || (num_blocks > 0 && !cpu_block_ids))
@@ -510,6 +510,8 @@ extern "C" int fkv_staged_restore_plan(const int64_t *cpu_block_ids, int32_t num
     for (int pos = 0; pos < num_blocks; ++pos)
       row_of_position[pos] = pos;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 namespace fkv {

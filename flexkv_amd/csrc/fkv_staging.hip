@@ -166,7 +166,7 @@ __global__ void fkv_chunk_ptrs_kernel(void **__restrict__ out, const uint64_t *_
 
 extern "C" {
 
-int fkv_staging_transfer(const fkv_staging_transfer_desc *dp, void *stream_v) {
+int fkv_staging_transfer(const fkv_staging_transfer_desc *dp, void *stream_v) try {
   using namespace fkv;
   clear_error();
   if (!dp)
@@ -263,9 +263,11 @@ int fkv_staging_transfer(const fkv_staging_transfer_desc *dp, void *stream_v) {
   if (d.sync)
     FKV_HIP_TRY(hipStreamSynchronize(stream));
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_build_gpu_chunk_ptrs(const fkv_chunk_ptrs_desc *dp, void *stream_v) {
+int fkv_build_gpu_chunk_ptrs(const fkv_chunk_ptrs_desc *dp, void *stream_v) try {
   using namespace fkv;
   clear_error();
   if (!dp)
@@ -338,6 +340,8 @@ int fkv_build_gpu_chunk_ptrs(const fkv_chunk_ptrs_desc *dp, void *stream_v) {
   if (d.sync)
     FKV_HIP_TRY(hipStreamSynchronize(stream));
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 } // extern "C"

@@ -43,7 +43,7 @@ extern "C" int fkv_tp_rank_plan_compute(int32_t rank, int32_t num_gpus, int32_t 
                                         int32_t layer_id, int32_t layer_granularity,
                                         int32_t num_blocks, int64_t gpu_chunk_size,
                                         int64_t cpu_block_stride, int64_t cpu_tp_stride,
-                                        fkv_tp_rank_plan *out) {
+                                        fkv_tp_rank_plan *out) try {
   if (!out || num_gpus < 1 || rank < 0 || rank >= num_gpus)
     return fkv::fail(FKV_ERR_INVALID_ARG, "fkv_tp_rank_plan_compute: bad rank %d of %d", rank,
                      num_gpus);
@@ -96,6 +96,8 @@ extern "C" int fkv_tp_rank_plan_compute(int32_t rank, int32_t num_gpus, int32_t 
   }
   *out = p;
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 struct fkv_tp_group {
@@ -159,7 +161,7 @@ struct Completion {
 
 extern "C" {
 
-int fkv_tp_group_create(const fkv_tp_group_params *p, fkv_tp_group **out) {
+int fkv_tp_group_create(const fkv_tp_group_params *p, fkv_tp_group **out) try {
   using namespace fkv;
   clear_error();
   if (!p || !out || p->num_gpus < 1 || p->num_tensors_per_gpu < 1 || !p->gpu_block_ptrs_flat ||
@@ -226,9 +228,11 @@ int fkv_tp_group_create(const fkv_tp_group_params *p, fkv_tp_group **out) {
   }
   *out = g.release();
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
-int fkv_tp_group_update_gpu_block_ptrs(fkv_tp_group *g, const uint64_t *ptrs, int64_t count) {
+int fkv_tp_group_update_gpu_block_ptrs(fkv_tp_group *g, const uint64_t *ptrs, int64_t count) try {
   using namespace fkv;
   clear_error();
   if (!g || !ptrs)
@@ -243,6 +247,8 @@ int fkv_tp_group_update_gpu_block_ptrs(fkv_tp_group *g, const uint64_t *ptrs, in
   (void)hipSetDevice(restore.device());
   g->gpu_ptrs.assign(ptrs, ptrs + count);
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 int fkv_tp_group_transfer(fkv_tp_group *g, const int64_t *gpu_block_ids,
@@ -252,7 +258,7 @@ int fkv_tp_group_transfer(fkv_tp_group *g, const int64_t *gpu_block_ids,
                           int32_t transfer_num_cta, int32_t is_host_to_device,
                           int32_t use_ce_transfer, int32_t layer_id, int32_t layer_granularity,
                           int32_t kv_dim, int32_t num_kv_heads, const char *mode,
-                          int32_t designated_rank) {
+                          int32_t designated_rank) try {
   using namespace fkv;
   clear_error();
   if (!g)
@@ -327,6 +333,8 @@ int fkv_tp_group_transfer(fkv_tp_group *g, const int64_t *gpu_block_ids,
   if (done.status != FKV_OK) // csrc/tp_transfer_thread_group.cpp:378-380
     return fail(done.status, "tp_group_transfer failed: %s", done.message.c_str());
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }
 
 void fkv_tp_group_destroy(fkv_tp_group *g) {

@@ -16,7 +16,7 @@
 
 using namespace fkv;
 
-extern "C" int fkv_layout_transform(const fkv_layout_transform_desc *dp, void *stream_v) {
+extern "C" int fkv_layout_transform(const fkv_layout_transform_desc *dp, void *stream_v) try {
   clear_error();
   if (!dp)
     return fail(FKV_ERR_INVALID_ARG, "fkv_layout_transform: null descriptor");
@@ -106,4 +106,6 @@ extern "C" int fkv_layout_transform(const fkv_layout_transform_desc *dp, void *s
   if (d.sync)
     FKV_HIP_TRY(hipStreamSynchronize(stream));
   return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
 }

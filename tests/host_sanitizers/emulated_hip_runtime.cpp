@@ -32,6 +32,7 @@
 #include <map>
 #include <memory>
 #include <mutex>
+#include <new>
 #include <thread>
 #include <vector>
 
@@ -115,7 +116,7 @@ hipError_t remember(hipError_t e) {
 // calls of it fail (fkv_emulated_fail below).  What a real runtime does when memory, streams
 // or events run out, or a launch is refused.
 enum Category { kDeviceAlloc, kPinnedAlloc, kStreamCreate, kEventCreate, kCopy, kLaunch, kEventRecord,
-                kCategories };
+                kThrow, kCategories };
 std::atomic<long> g_fail_after[kCategories];
 std::atomic<long> g_fail_count[kCategories];
 std::atomic<long> g_failed_calls{0};
@@ -490,6 +491,8 @@ int launch_copy_kernel(CopyKernelArgs a, int num_workgroups, int threads_per_wor
     return fail(FKV_ERR_RUNTIME, "emulated copy kernel: bad launch");
   if (refused(kLaunch))
     return fail(FKV_ERR_RUNTIME, "emulated copy kernel: launch refused");
+  if (refused(kThrow)) // as if the library had run out of host memory at this point
+    throw std::bad_alloc();
   g_launches.fetch_add(1);
   stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);
   of(stream)->push([a] { copy_rows(a); });
@@ -538,8 +541,9 @@ int common_vector_width(const uint64_t *vals, int n) {
 } // namespace fkv
 
 // Test hook: the next `count` calls of `category` (0 device allocation, 1 pinned allocation,
-// 2 stream creation, 3 event creation, 4 copy, 5 kernel launch, 6 event record) fail once
-// `after` more of them have succeeded; count 0 switches it off.  Returns the calls refused so far.
+// 2 stream creation, 3 event creation, 4 copy, 5 kernel launch, 6 event record; 7: a kernel
+// launch throws std::bad_alloc, as an allocation of the library's own might) fail once `after`
+// more of them have succeeded; count 0 switches it off.  Returns the calls refused so far.
 extern "C" long fkv_emulated_fail(int category, long after, long count) {
   if (category >= 0 && category < kCategories) {
     g_fail_after[category].store(after);

@@ -400,10 +400,10 @@ void transfer_case(uint64_t seed) {
     // it leaves behind is the starting point of the next one
     const bool inject = rep % 3 == 2;
     if (inject)
-      fkv_emulated_fail(pick(0, 6), pick(0, 6), pick(1, 2));
+      fkv_emulated_fail(pick(0, 7), pick(0, 6), pick(1, 2));
     const int rc = fkv_transfer_kv_blocks(&d, st);
     REQUIRE(hipStreamSynchronize(st) == hipSuccess, "sync");
-    for (int c = 0; c < 7; ++c)
+    for (int c = 0; c < 8; ++c)
       fkv_emulated_fail(c, 0, 0);
     REQUIRE(rc == FKV_OK || inject, "seed %llu rep %d: transfer", (unsigned long long)seed, rep);
     if (rc != FKV_OK) {
@@ -538,11 +538,11 @@ void tp_case(uint64_t seed) {
     // every third call with the runtime refusing something in one of the rank threads
     const bool inject = rep % 3 == 2;
     if (inject)
-      fkv_emulated_fail(pick(0, 6), pick(0, 4), pick(1, 2));
+      fkv_emulated_fail(pick(0, 7), pick(0, 4), pick(1, 2));
     const int rc = fkv_tp_group_transfer(g, gids.data(), cids.data(), nb, cpu_kv_stride,
                                          cpu_layer_stride, cpu_block_stride, cpu_tp_stride, 4, h2d,
                                          use_ce, layer_id, gran, s.kv, heads, mode.c_str(), designated);
-    for (int c = 0; c < 7; ++c)
+    for (int c = 0; c < 8; ++c)
       fkv_emulated_fail(c, 0, 0);
     REQUIRE(rc == FKV_OK || inject, "seed %llu rep %d: tp transfer (mode %s h2d %d ce %d)",
             (unsigned long long)seed, rep, mode.c_str(), h2d, use_ce);
@@ -792,13 +792,13 @@ void failure_case(uint64_t seed) {
     const bool inject = rep % 2 == 0;
     fill(rng, host, (size_t)s.host_bytes());
     if (inject)
-      fkv_emulated_fail(pick(0, 6), pick(0, 12), pick(1, 3));
+      fkv_emulated_fail(pick(0, 7), pick(0, 12), pick(1, 3));
     const int rc = fkv_layerwise_transfer(g, gids.data(), cids.data(), n, s.cpu_block_stride(),
                                           s.cpu_kv_stride(), s.cpu_layer_stride(),
                                           s.cpu_block_stride(), 4, use_ce, s.L, gran, s.kv, 1, 0,
                                           "sharded", notify, 0);
     const int src = fkv_layerwise_synchronize(g);
-    for (int c = 0; c < 7; ++c)
+    for (int c = 0; c < 8; ++c)
       fkv_emulated_fail(c, 0, 0);
     if (!inject)
       REQUIRE(rc == FKV_OK && src == FKV_OK, "seed %llu rep %d: a clean restore failed (route %d)",

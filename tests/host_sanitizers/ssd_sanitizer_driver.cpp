@@ -7,6 +7,7 @@
 namespace fkv {
 int fail(int code, const char *fmt, ...) { va_list ap; va_start(ap, fmt); vfprintf(stderr, fmt, ap); va_end(ap); fputc('\n', stderr); return code; }
 void clear_error() {}
+int caught(const char *where) noexcept { fprintf(stderr, "%s: exception\n", where); return 2; }
 }
 int main() {
   std::mt19937_64 rng(7);
