@@ -345,9 +345,10 @@ int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &
                       bool several_gpus = false);
 // The choice alone (no device): kRouteKernel, kRouteRuns (fills `segs` and `total_rows`)
 // or kRouteGathered.
+// `free_commands`: up to so many copy commands a batch are taken whatever the batch's size.
 int staged_route(const int64_t *cpu_ids, int num_blocks, int64_t row_bytes, int pieces,
                  const fkv_launch_policy &pol, std::vector<StagedPlan::Seg> *segs,
-                 int64_t *total_rows);
+                 int64_t *total_rows, int free_commands = 0);
 // Host threads a gathered restore uses under `pol` on this machine (>= 1).
 int gather_threads_of(const fkv_launch_policy &pol);
 // Layers [l0, l0 + nl) of a kRouteGathered plan: gathers the rows on the calling thread

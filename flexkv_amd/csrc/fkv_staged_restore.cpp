@@ -139,7 +139,7 @@ int ring_prepare(StagedRing &ring, int slots, size_t bytes) {
 // per run and batch.  Returns false when the restore stays on the kernel path.
 bool staged_layout(const int64_t *cpu_ids, int num_blocks, int64_t row_bytes, int pieces,
                    const fkv_launch_policy &pol, std::vector<StagedPlan::Seg> *segs,
-                   int64_t *total_rows_out) {
+                   int64_t *total_rows_out, int free_commands = 0) {
   segs->clear();
   *total_rows_out = 0;
   if (pol.staged_restore == 0 || num_blocks <= 0 || row_bytes <= 0 || pieces < 1)
@@ -181,7 +181,7 @@ bool staged_layout(const int64_t *cpu_ids, int num_blocks, int64_t row_bytes, in
   const int64_t total_rows = (int64_t)ids.size() + extra_rows;
   if (total_rows * row_bytes > (int64_t)pol.staged_max_mb << 20)
     return false;
-  if (pol.staged_restore == 1) {
+  if (pol.staged_restore == 1 && nsegs * pieces > free_commands) {
     // the copy commands of a batch against the batch's time on the link
     const double batch_us = useful / (std::max(1, pol.link_gbps_estimate) * 1e3);
     if ((double)(nsegs * pieces) * pol.staged_copy_overhead_us >
@@ -223,8 +223,8 @@ constexpr double kGatherPieceNs = 50.0;
 
 int staged_route(const int64_t *cpu_ids, int num_blocks, int64_t row_bytes, int pieces,
                  const fkv_launch_policy &pol, std::vector<StagedPlan::Seg> *segs,
-                 int64_t *total_rows) {
-  if (staged_layout(cpu_ids, num_blocks, row_bytes, pieces, pol, segs, total_rows))
+                 int64_t *total_rows, int free_commands) {
+  if (staged_layout(cpu_ids, num_blocks, row_bytes, pieces, pol, segs, total_rows, free_commands))
     return kRouteRuns;
   segs->clear();
   *total_rows = 0;
@@ -294,8 +294,18 @@ int staged_plan_build(const fkv_transfer_desc &d, int batch_layers, StagedRing &
   const int64_t batch_row_bytes = (int64_t)lk * d.chunk_size; // of one block, all pieces
   const int pieces = out->kind == 0 ? 1 : out->kind == 1 ? nl : lk;
   int64_t total_rows = 0;
+  // Asked for on the copy engine, the alternative to a staged batch is not a kernel launch but
+  // a copy-engine strategy, which issues at least as many copy commands and a compaction
+  // launch besides (46-56 us a layer at the small and medium scale of the notify
+  // microbenchmark, against 15-28 us staged): few commands are always worth it there, and
+  // more while they cost no more than the bytes themselves.
+  int free_commands = 0;
+  if (!kernel_allowed) {
+    free_commands = 4;
+    pol.staged_overhead_pct = std::max(pol.staged_overhead_pct, 100);
+  }
   out->route = staged_route(d.cpu_block_ids, d.num_blocks, batch_row_bytes, pieces, pol, &out->segs,
-                            &total_rows);
+                            &total_rows, free_commands);
   if (out->route == kRouteKernel)
     return FKV_OK;
   const bool gathered = out->route == kRouteGathered;
