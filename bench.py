@@ -492,7 +492,8 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=F
                 first_layer_ms=_median(firsts), compute_ms=compute_ms,
                 compute_overlapped_ms=_median(busy), stall_ms=_median(stalls),
                 compute_reps_per_layer=reps, layer_bytes=layer_bytes,
-                restore_alone_ms=restore_alone_ms)
+                restore_alone_ms=restore_alone_ms,
+                restore_alone_runs_ms=[round(x, 3) for x in alone])
 
 
 def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, verify=True):
@@ -1238,6 +1239,7 @@ def overlap_record(r, B, link):
             "restore_plus_compute_ms": round(r["total_ms"], 3),
             "restore_next_to_compute_ms": round(r["restore_ms"], 3),
             "first_layer_ms": round(r["first_layer_ms"], 3),
+            "restore_alone_runs_ms": r.get("restore_alone_runs_ms"),
             "compute_per_layer_ms": round(r["compute_ms"] / r["layers"], 3),
             "compute_units_per_layer": r["compute_reps_per_layer"],
             "exposed_ms": round(exposed, 3),
@@ -1298,6 +1300,32 @@ def measure_config(name, args, torch, device, link, steps, warmup):
                     "blocks": w.num_blocks, "bytes_per_direction": B, "steps": steps,
                     "warmup": warmup}
             frag.update(measure_layerwise(w, args, torch, device, link, steps, warmup))
+            # the same restore asked for on the copy engine, and out of a host pool the device
+            # cannot read (ordinary pageable memory): both go through gathered rows as well
+            variants = {}
+            short = max(2, min(steps, 5))
+            ce_args = argparse.Namespace(**{**vars(args), "use_ce": True})
+            variants["with_use_ce_transfer"] = measure_layerwise(w, ce_args, torch, device, link,
+                                                                 short, 2)
+            pinned = w.host
+            try:
+                w.host = torch.empty(pinned.numel(), dtype=pinned.dtype)   # pageable
+                w.host.copy_(pinned)
+                variants["pageable_host_pool"] = measure_layerwise(w, ce_args, torch, device, link,
+                                                                   short, 2, fill_host=False)
+            finally:
+                w.host = pinned
+            frag["variants"] = {
+                k: {"route": v["path"], "restore_alone_ms": v["layerwise"]["restore_alone_ms"],
+                    "restore_alone_GBps": v["layerwise"]["restore_alone_GBps"],
+                    "restore_plus_compute_ms": v["layerwise"]["restore_plus_compute_ms"],
+                    "compute_alone_ms": v["layerwise"]["compute_alone_ms"],
+                    "first_layer_ms": v["layerwise"]["first_layer_ms"],
+                    "restore_alone_runs_ms": v["layerwise"].get("restore_alone_runs_ms"),
+                    "host_gather_thread_ms_per_restore":
+                        v["layerwise"].get("host_gather_thread_ms_per_restore"),
+                    "bit_exact": v.get("bit_exact"), "steps": short}
+                for k, v in variants.items()}
             out["fragmented_record"] = frag
     else:  # c4
         r = run_concurrent(w, torch, steps, warmup, args.num_cta, args.streams_per_direction,
@@ -1318,14 +1346,19 @@ def measure_config(name, args, torch, device, link, steps, warmup):
     return out
 
 
-def measure_layerwise(w, args, torch, device, link, steps, warmup):
-    """c3 / c3f: the fields of a layerwise-restore record."""
+def measure_layerwise(w, args, torch, device, link, steps, warmup, fill_host=True):
+    """c3 / c3f: the fields of a layerwise-restore record.  `fill_host=False`: the host pool
+    already holds the engine's blocks (a pageable copy of a pool filled before, which the
+    kernel path could not write)."""
     import flexkv_amd.c_ext as c_ext
     B = w.bytes_per_direction
     # fill the host cache with the blocks to restore, then erase them on the GPU
-    w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=args.num_cta, sync=True)
     gi = w.gpu_ids.to(device)
-    saved = [w.gpu_rows(l, 0).index_select(0, gi) for l in range(w.L)]
+    if fill_host:
+        w.transfer(w.gpu_ids, w.cpu_ids, False, transfer_num_cta=args.num_cta, sync=True)
+        saved = [w.gpu_rows(l, 0).index_select(0, gi) for l in range(w.L)]
+    else:   # the engine's blocks are what an earlier restore out of the same bytes left
+        saved = [w.gpu_rows(l, 0).index_select(0, gi) for l in range(w.L)]
     for l in range(w.L):
         w.gpu_rows(l, 0).index_fill_(0, gi, 0)
     c_ext.reset_stats()
