@@ -370,7 +370,8 @@ def verify_round_trip(w, torch, num_cta):
     return bool(ok)
 
 
-def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=False, use_ce=False):
+def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=False, use_ce=False,
+                  name_compute_stream=True):
     """c3: per-layer restore with a dummy per-layer compute kernel on a second
     stream gated on each layer's event.  `layer_spans` brackets every layer's
     compute with two timing events; torch creates them with default flags, and
@@ -397,6 +398,8 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=F
     # time: fused attention (default; what a restored layer feeds), a 2048^3 GEMM
     # chain, or a streaming elementwise kernel.
     comp = torch.cuda.Stream()
+    # the engine names its forward stream: the group's own streams keep off its hardware queue
+    sharing = grp.set_compute_stream(comp) if name_compute_stream else None
     ev = lambda: torch.cuda.Event(enable_timing=True)
     target_ms = layer_bytes / 55e9 * 1e3
     if dummy == "sdpa":
@@ -493,7 +496,8 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=F
                 compute_overlapped_ms=_median(busy), stall_ms=_median(stalls),
                 compute_reps_per_layer=reps, layer_bytes=layer_bytes,
                 restore_alone_ms=restore_alone_ms,
-                restore_alone_runs_ms=[round(x, 3) for x in alone])
+                restore_alone_runs_ms=[round(x, 3) for x in alone],
+                group_streams_on_compute_queue=sharing)
 
 
 def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, verify=True):
@@ -1240,6 +1244,8 @@ def overlap_record(r, B, link):
             "restore_next_to_compute_ms": round(r["restore_ms"], 3),
             "first_layer_ms": round(r["first_layer_ms"], 3),
             "restore_alone_runs_ms": r.get("restore_alone_runs_ms"),
+            # after fkv_layerwise_set_compute_stream; None: the compute stream was not named
+            "group_streams_on_compute_queue": r.get("group_streams_on_compute_queue"),
             "compute_per_layer_ms": round(r["compute_ms"] / r["layers"], 3),
             "compute_units_per_layer": r["compute_reps_per_layer"],
             "exposed_ms": round(exposed, 3),

@@ -253,6 +253,7 @@ SIGNATURES = {
                                          c_int32, c_int32, c_int32, c_int32, c_int32,
                                          c_int32, c_int32, c_char_p, c_int32, c_int32]),
     "fkv_layerwise_wait_layer": (c_int32, [c_void_p, c_int32, c_int32, c_void_p]),
+    "fkv_layerwise_set_compute_stream": (c_int32, [c_void_p, c_int32, c_void_p, POINTER(c_int32)]),
     "fkv_layerwise_synchronize": (c_int32, [c_void_p]),
     "fkv_layerwise_batch_times_ms": (c_int32, [c_void_p, POINTER(c_float), c_int32,
                                                POINTER(c_int32)]),

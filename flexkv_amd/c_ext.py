@@ -1048,6 +1048,19 @@ class LayerwiseTransferGroup:
         handle = int((stream or torch.cuda.current_stream()).cuda_stream)
         check(_L.fkv_layerwise_wait_layer(self._h, int(gpu_index), int(layer), handle))
 
+    def set_compute_stream(self, stream: Optional["torch.cuda.Stream"] = None,
+                           gpu_index: int = 0) -> int:
+        """Names the stream the engine's forward pass runs on (default: torch's current
+        stream) next to this group's restores.  The group then keeps its own streams off
+        that stream's hardware queue; on a shared queue a restore is added to the forward
+        pass instead of hidden behind it.  Waits for ``stream``; call it at set-up.
+        Returns how many of the group's streams still share the queue (normally 0)."""
+        handle = int((stream or torch.cuda.current_stream()).cuda_stream)
+        left = ctypes.c_int32(0)
+        check(_L.fkv_layerwise_set_compute_stream(self._h, int(gpu_index), handle,
+                                                  ctypes.byref(left)))
+        return int(left.value)
+
     def synchronize(self) -> None:
         check(_L.fkv_layerwise_synchronize(self._h))
 

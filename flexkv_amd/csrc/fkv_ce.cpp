@@ -97,6 +97,7 @@ struct StageSet {
   // second DMA stream + the events that fork it off / join it back into the
   // caller's stream
   hipStream_t aux = nullptr;
+  int device = -1; // of `aux`: the key this set is kept under
   hipEvent_t fork = nullptr, join = nullptr;
   // the per-buffer events of a pipelined GATHER_DIRECT: compaction launches stay on the
   // caller's stream, copies run on `aux`
@@ -105,7 +106,7 @@ struct StageSet {
   bool ensure_fan() {
     if (aux && fork && join)
       return true;
-    if ((!aux && hipStreamCreateWithFlags(&aux, hipStreamNonBlocking) != hipSuccess) ||
+    if ((!aux && pooled_stream_acquire(device, true, &aux) != hipSuccess) ||
         (!fork && hipEventCreateWithFlags(&fork, hipEventDisableTiming) != hipSuccess) ||
         (!join && hipEventCreateWithFlags(&join, hipEventDisableTiming) != hipSuccess)) {
       (void)hipGetLastError();
@@ -127,8 +128,10 @@ struct StageSet {
     return ok;
   }
   ~StageSet() {
-    if (aux)
-      (void)hipStreamDestroy(aux);
+    if (aux) { // to the next thread that stages on this device
+      (void)hipStreamSynchronize(aux);
+      pooled_stream_release(device, true, aux);
+    }
     for (hipEvent_t e : {fork, join, kernel_done[0], kernel_done[1], copied[0], copied[1]})
       if (e)
         (void)hipEventDestroy(e);
@@ -150,7 +153,9 @@ struct StageSet {
 };
 StageSet &stage_set(int device) {
   thread_local std::unordered_map<int, StageSet> sets;
-  return sets[device];
+  StageSet &s = sets[device];
+  s.device = device;
+  return s;
 }
 
 // Device staging of at least `bytes`; nullptr when HBM is exhausted (callers

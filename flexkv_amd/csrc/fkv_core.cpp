@@ -79,6 +79,40 @@ DeviceGuard::~DeviceGuard() {
     (void)hipSetDevice(prev_);
 }
 
+// ---- pooled streams ---------------------------------------------------------
+namespace {
+struct StreamPool {
+  std::mutex mu;
+  std::map<std::pair<int, bool>, std::vector<hipStream_t>> idle;
+};
+StreamPool &stream_pool() {
+  static StreamPool *p = new StreamPool(); // never destructed, see pooled_stream_acquire
+  return *p;
+}
+} // namespace
+
+hipError_t pooled_stream_acquire(int device, bool non_blocking, hipStream_t *out) {
+  {
+    StreamPool &p = stream_pool();
+    std::lock_guard<std::mutex> lk(p.mu);
+    auto &v = p.idle[{device, non_blocking}];
+    if (!v.empty()) {
+      *out = v.back();
+      v.pop_back();
+      return hipSuccess;
+    }
+  }
+  return non_blocking ? hipStreamCreateWithFlags(out, hipStreamNonBlocking) : hipStreamCreate(out);
+}
+
+void pooled_stream_release(int device, bool non_blocking, hipStream_t stream) {
+  if (!stream)
+    return;
+  StreamPool &p = stream_pool();
+  std::lock_guard<std::mutex> lk(p.mu);
+  p.idle[{device, non_blocking}].push_back(stream);
+}
+
 // ---- plan memory ---------------------------------------------------------
 namespace {
 bool env_flag(const char *name) {

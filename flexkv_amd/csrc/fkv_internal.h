@@ -17,6 +17,14 @@ namespace fkv {
 // ---- errors -------------------------------------------------------------
 // Records the message for fkv_last_error() on this thread and returns `code`.
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+// Streams of the library's groups (layerwise restore, thread group): taken from a pool per
+// device and kind and given back, idle, when the group ends.  A process that makes and ends
+// groups by the hundred (a test session, an engine that re-creates its connectors) creates a
+// handful of streams instead of thousands; pooled streams are never destroyed, like plan
+// memory (tearing runtime objects down from a static destructor is unsafe).  The device must
+// be current.
+hipError_t pooled_stream_acquire(int device, bool non_blocking, hipStream_t *out);
+void pooled_stream_release(int device, bool non_blocking, hipStream_t stream);
 // For the catch-all handler of an entry point: turns the exception in flight into a status
 // and an error text.  No C++ exception crosses the C ABI.
 int caught(const char *where) noexcept;

@@ -368,15 +368,20 @@ int finish_create(std::unique_ptr<fkv_layerwise> &g, const int64_t *gpu_device_i
     g->device_ids.push_back((int)gpu_device_ids[i]);
   DeviceGuard restore(-1);
   g->streams.assign(g->num_gpus, nullptr);
+  g->dma_streams.assign(g->num_gpus, nullptr);
+  g->dma_streams2.assign(g->num_gpus, nullptr);
+  g->dma_turn.assign(g->num_gpus, 0u);
+  g->alt_streams.assign(g->num_gpus, nullptr);
+  g->alt_join.assign(g->num_gpus, nullptr);
   for (int i = 0; i < g->num_gpus; ++i) {
     hipError_t e = hipSetDevice(g->device_ids[i]);
     if (e == hipSuccess)
-      e = hipStreamCreateWithFlags(&g->streams[i], hipStreamNonBlocking);
+      e = pooled_stream_acquire(g->device_ids[i], true, &g->streams[i]);
     if (e != hipSuccess) {
       (void)hipGetLastError();
       for (int k = 0; k < i; ++k) {
         (void)hipSetDevice(g->device_ids[k]);
-        (void)hipStreamDestroy(g->streams[k]);
+        pooled_stream_release(g->device_ids[k], true, g->streams[k]);
       }
       (void)hipSetDevice(restore.device());
       return fail(FKV_ERR_RUNTIME, "stream creation on device %d failed: %s", g->device_ids[i],
@@ -450,19 +455,19 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
     two_dma_streams[i] = pol.staged_dma_streams >= 2;
     if (!direct || pol.kernel_alt_stream_kb <= 0 || num_batches < kAltMinBatches || rc != FKV_OK)
       continue;
-    if ((int)g->alt_streams.size() < g->num_gpus) {
-      g->alt_streams.resize(g->num_gpus, nullptr);
-      g->alt_join.resize(g->num_gpus, nullptr);
-    }
     (void)hipSetDevice(g->device_ids[i]);
     if (!g->alt_streams[i] &&
-        (hipStreamCreateWithFlags(&g->alt_streams[i], hipStreamNonBlocking) != hipSuccess ||
-         hipEventCreateWithFlags(&g->alt_join[i], hipEventDisableTiming) != hipSuccess)) {
+        pooled_stream_acquire(g->device_ids[i], true, &g->alt_streams[i]) != hipSuccess) {
       (void)hipGetLastError(); // everything on the one stream then
+      g->alt_streams[i] = nullptr;
       continue;
     }
-    if (!g->alt_join[i])
-      continue; // an earlier call could not create it
+    if (!g->alt_join[i] &&
+        hipEventCreateWithFlags(&g->alt_join[i], hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      g->alt_join[i] = nullptr;
+      continue;
+    }
     alt_max_bytes[i] = (int64_t)pol.kernel_alt_stream_kb * 1024;
   }
   std::vector<char> alt_used(g->num_gpus, 0);
@@ -936,11 +941,6 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
       continue;
     lane.plans.resize(g->num_gpus);
     lane.staged.resize(g->num_gpus);
-    if ((int)g->dma_streams.size() < g->num_gpus) {
-      g->dma_streams.resize(g->num_gpus, nullptr);
-      g->dma_streams2.resize(g->num_gpus, nullptr);
-      g->dma_turn.resize(g->num_gpus, 0u);
-    }
     const int layers = g->multi_group || lane.src != &g->groups[0] ? lane.src->num_layers
                                                                    : c.num_layers;
     const int lane_index = (int)(&lane - lanes.data());
@@ -965,12 +965,12 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
                              g->streams[i], &lane.staged[i], lane.plans[i].host_visible,
                              /*kernel_allowed=*/direct, /*several_gpus=*/g->num_gpus > 1);
       if (rc == FKV_OK && lane.staged[i].usable && !g->dma_streams[i]) {
-        hipError_t e = hipStreamCreateWithFlags(&g->dma_streams[i], hipStreamNonBlocking);
+        hipError_t e = pooled_stream_acquire(g->device_ids[i], true, &g->dma_streams[i]);
         if (e != hipSuccess) {
           (void)hipGetLastError();
           g->dma_streams[i] = nullptr;
           staged_plan_release(&lane.staged[i], g->streams[i]); // kernel path then
-        } else if (hipStreamCreateWithFlags(&g->dma_streams2[i], hipStreamNonBlocking) !=
+        } else if (pooled_stream_acquire(g->device_ids[i], true, &g->dma_streams2[i]) !=
                    hipSuccess) {
           (void)hipGetLastError();
           g->dma_streams2[i] = nullptr; // all copies on the first then
@@ -1198,6 +1198,101 @@ int fkv_layerwise_wait_layer(fkv_layerwise *g, int32_t gpu_index, int32_t layer,
   return fkv::caught(__func__);
 }
 
+int fkv_layerwise_set_compute_stream(fkv_layerwise *g, int32_t gpu_index, void *compute_stream,
+                                     int32_t *streams_sharing) try {
+  using namespace fkv;
+  clear_error();
+  if (!g)
+    return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_set_compute_stream: null group");
+  if (gpu_index < 0 || gpu_index >= g->num_gpus)
+    return fail(FKV_ERR_INVALID_ARG, "fkv_layerwise_set_compute_stream: gpu_index %d of %d GPUs",
+                gpu_index, g->num_gpus);
+  g->retire_previous(); // the streams below are swapped: nothing may be in flight on them
+  const int i = gpu_index, device = g->device_ids[i];
+  DeviceGuard guard(device);
+  if (!guard.ok())
+    return fail(FKV_ERR_RUNTIME, "cannot select HIP device %d", device);
+  // Every stream of the group on this GPU, also those a restore would only make when it
+  // first needs them: probing then would wait for the engine's stream in mid-service.
+  // A candidate that shares the engine's queue is held back until the end, so that the
+  // next one from the pool, or a new one, is another stream.
+  //
+  // Beyond that, where the queues allow: the scatter stream and the two copy streams on
+  // three queues of their own (a batch's copy, its scatter and the next batch's copy are in
+  // flight together), the second kernel stream off the first one's.
+  const hipStream_t compute = static_cast<hipStream_t>(compute_stream);
+  constexpr int kCandidates = 8;
+  std::vector<hipStream_t> held_back;
+  int sharing = 0, rc = FKV_OK;
+  struct Own {
+    hipStream_t *stream;
+    std::vector<hipStream_t *> apart_from; // wished for, not required
+  };
+  const Own owns[] = {{&g->streams[i], {}},
+                      {&g->dma_streams[i], {&g->streams[i]}},
+                      {&g->dma_streams2[i], {&g->streams[i], &g->dma_streams[i]}},
+                      {&g->alt_streams[i], {&g->streams[i]}}};
+  // 2: next to the engine's stream and to those of ours it should be apart from,
+  // 1: next to the engine's stream only, 0: shares the engine's queue
+  auto rank_of = [&](hipStream_t candidate, const Own &o, int *rank) -> int {
+    int32_t concurrent = 0;
+    FKV_TRY(fkv_streams_run_concurrently(device, compute, candidate, &concurrent));
+    *rank = concurrent ? 2 : 0;
+    for (hipStream_t *other : o.apart_from) {
+      if (*rank != 2 || !*other)
+        break;
+      FKV_TRY(fkv_streams_run_concurrently(device, *other, candidate, &concurrent));
+      if (!concurrent)
+        *rank = 1;
+    }
+    return FKV_OK;
+  };
+  for (const Own &o : owns) {
+    hipStream_t best = nullptr;
+    int best_rank = -1;
+    for (int attempt = 0; attempt < kCandidates && best_rank < 2; ++attempt) {
+      if (best_rank == 1 && attempt >= kCandidates / 2)
+        break; // good enough
+      hipStream_t candidate = *o.stream;
+      *o.stream = nullptr;
+      if (!candidate && pooled_stream_acquire(device, true, &candidate) != hipSuccess) {
+        (void)hipGetLastError();
+        break;
+      }
+      int rank = 0;
+      rc = rank_of(candidate, o, &rank);
+      if (rc != FKV_OK || rank <= best_rank) {
+        held_back.push_back(candidate);
+        if (rc != FKV_OK)
+          break;
+        continue;
+      }
+      if (best)
+        held_back.push_back(best);
+      best = candidate;
+      best_rank = rank;
+    }
+    *o.stream = best; // none: a restore makes the stream when it needs it, as without this call
+    if (best && best_rank == 0)
+      ++sharing;
+    if (rc != FKV_OK)
+      break;
+  }
+  if (!g->streams[i] && !held_back.empty()) { // the group always has its first stream
+    g->streams[i] = held_back.back();
+    held_back.pop_back();
+  }
+  for (hipStream_t s : held_back)
+    pooled_stream_release(device, true, s);
+  if (!g->streams[i]) // cannot be: the group was made with one and gives it up only for another
+    return fail(FKV_ERR_RUNTIME, "fkv_layerwise_set_compute_stream: no stream left for GPU %d", i);
+  if (streams_sharing)
+    *streams_sharing = sharing;
+  return rc;
+} catch (...) {
+  return fkv::caught(__func__);
+}
+
 int fkv_layerwise_synchronize(fkv_layerwise *g) try {
   using namespace fkv;
   clear_error();
@@ -1249,17 +1344,19 @@ void fkv_layerwise_destroy(fkv_layerwise *g) {
   g->crew.reset();
   for (int i = 0; i < g->num_gpus; ++i) {
     (void)hipSetDevice(g->device_ids[i]);
+    // every stream is idle (retire_previous), so the next group of the process may have it
     if (i < (int)g->dma_streams.size())
       for (hipStream_t s : {g->dma_streams[i], g->dma_streams2[i]})
-        if (s)
-          (void)hipStreamDestroy(s);
+        fkv::pooled_stream_release(g->device_ids[i], true, s);
     if (i < (int)g->alt_streams.size()) {
-      if (g->alt_streams[i])
-        (void)hipStreamDestroy(g->alt_streams[i]);
+      if (g->alt_streams[i]) {
+        (void)hipStreamSynchronize(g->alt_streams[i]);
+        fkv::pooled_stream_release(g->device_ids[i], true, g->alt_streams[i]);
+      }
       if (g->alt_join[i])
         (void)hipEventDestroy(g->alt_join[i]);
     }
-    (void)hipStreamDestroy(g->streams[i]);
+    fkv::pooled_stream_release(g->device_ids[i], true, g->streams[i]);
   }
   (void)hipSetDevice(restore.device());
   (void)hipGetLastError();

@@ -200,12 +200,12 @@ int fkv_tp_group_create(const fkv_tp_group_params *p, fkv_tp_group **out) try {
     for (int i = 0; i < p->num_gpus; ++i) {
       hipError_t e = hipSetDevice(g->device_ids[i]);
       if (e == hipSuccess)
-        e = hipStreamCreate(&g->streams[i]);
+        e = pooled_stream_acquire(g->device_ids[i], false, &g->streams[i]);
       if (e != hipSuccess) {
         (void)hipGetLastError();
         for (int k = 0; k < i; ++k) {
           (void)hipSetDevice(g->device_ids[k]);
-          (void)hipStreamDestroy(g->streams[k]);
+          pooled_stream_release(g->device_ids[k], false, g->streams[k]);
         }
         (void)hipSetDevice(restore.device());
         return fail(FKV_ERR_RUNTIME, "stream creation on device %d failed: %s", g->device_ids[i],
@@ -354,7 +354,7 @@ void fkv_tp_group_destroy(fkv_tp_group *g) {
   for (int i = 0; i < g->num_gpus; ++i) {
     (void)hipSetDevice(g->device_ids[i]);
     (void)hipStreamSynchronize(g->streams[i]);
-    (void)hipStreamDestroy(g->streams[i]);
+    fkv::pooled_stream_release(g->device_ids[i], false, g->streams[i]);
   }
   (void)hipSetDevice(restore.device());
   (void)hipGetLastError();

@@ -422,6 +422,23 @@ int fkv_layerwise_transfer(fkv_layerwise *g, const int64_t *gpu_block_ids,
  * (flexkv/integration/sglang/comm.py:705-744); the reference has no such call. */
 int fkv_layerwise_wait_layer(fkv_layerwise *g, int32_t gpu_index, int32_t layer,
                              void *consumer_stream);
+/* Names the stream on which the engine computes next to this group's restores on GPU
+ * `gpu_index` (a hipStream_t, or NULL for the null stream).  A process has few hardware
+ * queues (4 unless GPU_MAX_HW_QUEUES says otherwise) and the runtime spreads streams over
+ * them; two streams on one queue run one after the other.  A restore whose scatter or copy
+ * stream shares the queue of the engine's forward pass is therefore not hidden behind the
+ * forward pass but added to it (61 layers of 36 MiB next to 0.6 ms of attention per layer:
+ * 89 ms instead of 42).  The call swaps every stream the group uses on that GPU for one
+ * that was seen to run next to `compute_stream` (two short timed launches per candidate,
+ * about 3 ms each; up to 8 candidates per stream) and, where the queues allow, puts the
+ * scatter stream and the two copy streams on queues of their own; `streams_sharing` (may be NULL)
+ * receives how many of the group's streams still share the queue afterwards, 0 in the
+ * normal case.  It waits for the group's previous restore and for `compute_stream`: call
+ * it when the group is set up, and again if the engine changes its stream.  No
+ * counterpart in the reference, whose restore streams (csrc/layerwise.cpp:629, 822) land on a
+ * queue by the order of creation. */
+int fkv_layerwise_set_compute_stream(fkv_layerwise *g, int32_t gpu_index, void *compute_stream,
+                                     int32_t *streams_sharing);
 /* Block the host until the most recent transfer has finished on all GPUs and
  * every notification has been written. */
 int fkv_layerwise_synchronize(fkv_layerwise *g);

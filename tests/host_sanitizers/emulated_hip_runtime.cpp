@@ -44,6 +44,7 @@ struct ihipStream_t {
   std::condition_variable wake, idle;
   std::deque<std::function<void()>> queue;
   bool busy = false, quit = false;
+  int hardware_queue = 0; // streams are dealt over four, the null stream sits on the first
   std::thread worker;
   ihipStream_t() : worker([this] { run(); }) {}
   ~ihipStream_t() {
@@ -252,6 +253,8 @@ hipError_t hipStreamCreateWithFlags(hipStream_t *s, unsigned int) {
     return remember(hipErrorOutOfMemory);
   auto made = std::make_shared<ihipStream_t>();
   *s = made.get();
+  static std::atomic<int> dealt{0};
+  made->hardware_queue = ++dealt % 4;
   std::lock_guard<std::mutex> lk(rt().mu);
   if (rt().streams.empty())
     rt().streams.push_back(std::make_shared<ihipStream_t>());
@@ -557,8 +560,12 @@ extern "C" {
 int fkv_measure_hbm_rate(int32_t, size_t, int32_t, int32_t, double *, double *) {
   return fkv::fail(FKV_ERR_UNSUPPORTED, "emulated runtime: no HBM to measure");
 }
-int fkv_streams_run_concurrently(int32_t, void *, void *, int32_t *) {
-  return fkv::fail(FKV_ERR_UNSUPPORTED, "emulated runtime: no hardware queues");
+int fkv_streams_run_concurrently(int32_t, void *a, void *b, int32_t *concurrent) {
+  if (!concurrent)
+    return fkv::fail(FKV_ERR_INVALID_ARG, "fkv_streams_run_concurrently: null result pointer");
+  *concurrent = of(static_cast<hipStream_t>(a))->hardware_queue !=
+                of(static_cast<hipStream_t>(b))->hardware_queue;
+  return FKV_OK;
 }
 int fkv_transfer_kv_blocks_noalloc(const fkv_transfer_desc *, void *) {
   return fkv::fail(FKV_ERR_UNSUPPORTED, "emulated runtime: the entry point lives beside the kernels");

@@ -209,6 +209,15 @@ void layerwise_case(uint64_t seed, const Pinned &fix = Pinned()) {
   REQUIRE(hipStreamCreateWithFlags(&consumer, hipStreamNonBlocking) == hipSuccess, "stream");
   std::vector<uint8_t> seen((size_t)s.layer_bytes()); // what the consumer copies out of layer l
   for (int rep = 0; rep < 3; ++rep) {
+    // the engine names its stream: at set-up, or between two restores
+    if (rng() % 3 == 0) {
+      int32_t sharing = -1;
+      const int named = fkv_layerwise_set_compute_stream(g, pick(0, s.ranks - 1),
+                                                         (rng() & 1) ? consumer : nullptr, &sharing);
+      REQUIRE(named == FKV_OK && sharing == 0,
+              "seed %llu rep %d: set_compute_stream rc %d, %d streams share the queue",
+              (unsigned long long)seed, rep, named, sharing);
+    }
     fill(rng, t.host, (size_t)s.host_bytes());
     const int n = pick(0, std::min(s.NG, pool_blocks));
     std::vector<int64_t> gids(s.NG), cids(pool_blocks);
@@ -793,6 +802,8 @@ void failure_case(uint64_t seed) {
     fill(rng, host, (size_t)s.host_bytes());
     if (inject)
       fkv_emulated_fail(pick(0, 7), pick(0, 12), pick(1, 3));
+    if (rng() % 4 == 0) // may be refused part-way; the group keeps a stream per GPU either way
+      (void)fkv_layerwise_set_compute_stream(g, pick(0, s.ranks - 1), nullptr, nullptr);
     const int rc = fkv_layerwise_transfer(g, gids.data(), cids.data(), n, s.cpu_block_stride(),
                                           s.cpu_kv_stride(), s.cpu_layer_stride(),
                                           s.cpu_block_stride(), 4, use_ce, s.L, gran, s.kv, 1, 0,

@@ -466,3 +466,86 @@ def test_seeded_random_restores(gpu_device, seed):
             s.oracle_transfer(gids, cids, True, num_layers=layers)
             dev.assert_matches_reference(f"restore {rep}")
     grp.close()
+
+
+@pytest.mark.parametrize("route", ["kernel", "copy_engines", "gathered"])
+def test_named_compute_stream_keeps_the_restore_beside_the_forward_pass(gpu_device, route):
+    """Streams of a process share a few hardware queues, and two streams on one queue run
+    one after the other.  Once the engine has named its forward stream, the group's own
+    streams sit on other queues: for eight forward streams in a row (torch hands them out
+    over all queues, the null stream among them) no stream of the group shares the queue, a
+    restore with a per-layer consumer gated on wait_layer still equals the oracle, and a
+    restore next to a forward pass of about its own length takes well under the two
+    one after the other."""
+    from flexkv_amd.c_ext import get_stats, launch_policy, reset_stats
+    L, NG, NC, n, chunk = 16, 320, 320, 256, 32768
+    s = KVSetup(VLLM, L, 2, NG, NC, chunk, "BLOCKFIRST", seed=71)
+    dev = s.to_device(gpu_device)
+    grp = group_of(s, dev)
+    rng = np.random.default_rng(72)
+    gids = rng.permutation(NG)[:n].astype(np.int64)
+    cids = host_ids(rng, NC, n, "one_run" if route == "copy_engines" else "scattered")
+    s.oracle_transfer(gids, cids, True)
+    ev = lambda: torch.cuda.Event(enable_timing=True)  # noqa: E731
+    e = torch.empty(0, dtype=torch.int64)
+
+    def launch():
+        grp.layerwise_transfer(
+            e, e, 0, 0, 0, 0, 0, torch.as_tensor(gids), torch.as_tensor(cids), s.cpu_kv_stride,
+            s.cpu_layer_stride, s.cpu_block_stride, s.chunk, s.cpu_kv_stride, s.cpu_layer_stride,
+            s.cpu_block_stride, 4, False, L, 1, s.kv_dim, 1, counter_id=0,
+            kv_shared_across_ranks_mode="sharded", notify_mode="polling")
+
+    with launch_policy(**ROUTES[route]):
+        launch()            # buffers, code objects
+        grp.synchronize()
+        launch()
+        grp.synchronize()
+        restore_ms = grp.batch_times_ms()[-1]
+        cycles = 200_000
+        streams = [torch.cuda.default_stream()] + [torch.cuda.Stream() for _ in range(7)]
+        for k, comp in enumerate(streams):
+            assert grp.set_compute_stream(comp) == 0, k
+            with torch.cuda.stream(comp):   # a forward pass of about the restore's length
+                torch.cuda._sleep(cycles)
+                a, b = ev(), ev()
+                a.record(comp)
+                for _ in range(L):
+                    torch.cuda._sleep(cycles)
+                b.record(comp)
+                b.synchronize()
+                if k == 0:
+                    cycles = max(1000, int(cycles * restore_ms / max(a.elapsed_time(b), 1e-3)))
+                a, b = ev(), ev()
+                a.record(comp)
+                for _ in range(L):
+                    torch.cuda._sleep(cycles)
+                b.record(comp)
+                b.synchronize()
+                forward_ms = a.elapsed_time(b)
+            for t in dev.gpu:
+                t.zero_()
+            torch.cuda.synchronize()
+            reset_stats()
+            t0, t1 = ev(), ev()
+            with torch.cuda.stream(comp):
+                t0.record(comp)
+            launch()
+            with torch.cuda.stream(comp):
+                for l in range(L):
+                    grp.wait_layer(l, comp)
+                    torch.cuda._sleep(cycles)
+                t1.record(comp)
+            grp.synchronize()
+            t1.synchronize()
+            both_ms = t0.elapsed_time(t1)
+            st = get_stats()
+            assert (st["staged_batches"] > 0) == (route != "kernel"), st
+            assert (st["gathered_batches"] > 0) == (route == "gathered"), st
+            got = [t.cpu() for t in dev.gpu]
+            for l in range(L):
+                want = torch.from_numpy(s.gpu_ref[l].view(np.uint8).reshape(2, NG, -1)[:, gids])
+                have = got[l].view(torch.uint8).reshape(2, NG, -1)[:, torch.as_tensor(gids)]
+                assert torch.equal(have, want), (k, l)
+            assert both_ms < 0.8 * (restore_ms + forward_ms), (k, both_ms, restore_ms, forward_ms)
+    grp.close()
