@@ -17,7 +17,10 @@
 //    ThreadSanitizer sees exactly the ordering a HIP program may rely on: work that is not
 //    ordered by stream order, an event or a synchronize shows up as a race.
 //  * The copy kernel stand-ins do what the kernels do (rows of `chunk_bytes` between base
-//    tables and block ids) with memcpy, on the stream's thread.
+//    tables and block ids) with memcpy, on the stream's thread.  With
+//    FKV_KERNELS_FROM_SOURCE there are no stand-ins: the library's kernel sources are
+//    compiled for the CPU device model (cpu_device_model.h) and a launch runs the kernel
+//    itself, workgroup by workgroup, every work-item on a host thread.
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
@@ -468,6 +471,179 @@ hipError_t hipIpcCloseMemHandle(void *) { return remember(hipErrorNotSupported);
 
 } // extern "C"
 
+#ifdef FKV_KERNELS_FROM_SOURCE
+// ---- the library's kernels, from their own sources (cpu_device_model.h) ---------------
+#include "cpu_device_model.h"
+namespace cpu_device_model {
+thread_local Index thread_index, block_index;
+thread_local Extent block_extent, grid_extent;
+
+namespace {
+// The work-items of the workgroup that is running: a crew of host threads that lives as
+// long as the process and grows to the largest workgroup seen.
+struct Crew {
+  std::mutex mu;
+  // members wait for work in sets of 64, so that a small workgroup does not wake the members
+  // a large one once needed
+  static constexpr unsigned kSet = 64, kSets = 1024 / kSet;
+  std::condition_variable start[kSets], done, barrier_cv;
+  uint64_t workgroups_run = 0;
+  std::vector<std::thread> members;
+  uint64_t round = 0;        // a new workgroup
+  unsigned size = 0;         // work-items of that workgroup
+  unsigned finished = 0;
+  // the barrier: work-items that have left the kernel no longer take part
+  unsigned waiting = 0, left = 0;
+  uint64_t barrier_round = 0;
+  const std::function<void()> *work_item = nullptr;
+  Index block;
+  Extent block_extent, grid_extent;
+  bool quit = false;
+  std::vector<unsigned char> lds;
+  unsigned xcc = 0;
+
+  ~Crew() {
+    {
+      std::lock_guard<std::mutex> lk(mu);
+      quit = true;
+    }
+    for (auto &cv : start)
+      cv.notify_all();
+    for (auto &t : members)
+      t.join();
+  }
+  void member(unsigned id) {
+    uint64_t seen = 0;
+    for (;;) {
+      {
+        std::unique_lock<std::mutex> lk(mu);
+        start[id / kSet].wait(lk, [&] { return quit || (round != seen && id < size); });
+        if (quit)
+          return;
+        seen = round;
+        thread_index = Index{id % block_extent.x, id / block_extent.x % block_extent.y,
+                             id / (block_extent.x * block_extent.y)};
+        block_index = block;
+        cpu_device_model::block_extent = block_extent;
+        cpu_device_model::grid_extent = grid_extent;
+      }
+      (*work_item)();
+      {
+        std::lock_guard<std::mutex> lk(mu);
+        ++left; // a barrier the others wait at may be complete now
+        if (waiting > 0 && waiting + left == size) {
+          waiting = 0;
+          ++barrier_round;
+          barrier_cv.notify_all();
+        }
+        if (++finished == size)
+          done.notify_all();
+      }
+    }
+  }
+  void run_workgroup(const std::function<void()> &item, Index at, Extent block_ext, Extent grid_ext) {
+    std::unique_lock<std::mutex> lk(mu);
+    const unsigned n = block_ext.x * block_ext.y * block_ext.z;
+    while (members.size() < n) {
+      const unsigned id = (unsigned)members.size();
+      members.emplace_back([this, id] { member(id); });
+    }
+    work_item = &item;
+    block = at;
+    block_extent = block_ext;
+    grid_extent = grid_ext;
+    size = n;
+    finished = waiting = left = 0;
+    ++round;
+    ++workgroups_run;
+    for (unsigned set = 0; set * kSet < n; ++set)
+      start[set].notify_all();
+    done.wait(lk, [&] { return finished == size; });
+    size = 0;
+  }
+  void barrier() {
+    std::unique_lock<std::mutex> lk(mu);
+    if (++waiting + left == size) {
+      waiting = 0;
+      ++barrier_round;
+      barrier_cv.notify_all();
+      return;
+    }
+    const uint64_t mine = barrier_round;
+    barrier_cv.wait(lk, [&] { return barrier_round != mine; });
+  }
+};
+Crew &crew() {
+  static Crew c;
+  return c;
+}
+std::mutex g_device; // one launch at a time owns the crew and the kernels' __shared__ variables
+std::atomic<unsigned> g_launch_number{0};
+} // namespace
+
+void sync_threads() { crew().barrier(); }
+void *dynamic_lds() { return crew().lds.data(); }
+unsigned xcc_id() { return crew().xcc; }
+void nap() { std::this_thread::yield(); }
+
+void launch(hipStream_t stream, dim3 grid, dim3 block, size_t lds_bytes, std::function<void()> work_item) {
+  const uint64_t threads = (uint64_t)block.x * block.y * block.z;
+  if (threads == 0 || threads > 1024 || grid.x == 0 || grid.y == 0 || grid.z == 0 ||
+      lds_bytes > 160 * 1024) {
+    remember(hipErrorInvalidConfiguration);
+    return;
+  }
+  if (refused(kLaunch)) {
+    remember(hipErrorLaunchFailure);
+    return;
+  }
+  if (refused(kThrow)) // as if the library had run out of host memory at this point
+    throw std::bad_alloc();
+  const unsigned number = g_launch_number.fetch_add(1);
+  of(stream)->push([=] {
+    std::lock_guard<std::mutex> device(g_device);
+    Crew &c = crew();
+    // exactly as large as asked for: an access beyond it is one the device would not forgive either
+    c.lds.assign(lds_bytes, 0xA5);
+    c.lds.shrink_to_fit();
+    const Extent block_ext{block.x, block.y, block.z}, grid_ext{grid.x, grid.y, grid.z};
+    for (unsigned z = 0; z < grid.z; ++z)
+      for (unsigned y = 0; y < grid.y; ++y)
+        for (unsigned x = 0; x < grid.x; ++x) {
+          c.xcc = (x + number * 3) % 8;
+          c.run_workgroup(work_item, Index{x, y, z}, block_ext, grid_ext);
+        }
+  });
+}
+} // namespace cpu_device_model
+
+// Workgroups of the library's kernels that have run from their sources in this process.
+extern "C" unsigned long long fkv_emulated_workgroups_run() {
+  auto &c = cpu_device_model::crew();
+  std::lock_guard<std::mutex> lk(c.mu);
+  return c.workgroups_run;
+}
+
+extern "C" {
+// A __device__ variable of a kernel source is a variable of this process.
+hipError_t hipGetSymbolAddress(void **out, const void *symbol) {
+  if (!out || !symbol)
+    return remember(hipErrorInvalidSymbol);
+  *out = const_cast<void *>(symbol);
+  return hipSuccess;
+}
+hipError_t hipStreamIsCapturing(hipStream_t, hipStreamCaptureStatus *status) { // no graphs here
+  *status = hipStreamCaptureStatusNone;
+  return hipSuccess;
+}
+hipError_t hipMemcpyFromSymbol(void *dst, const void *symbol, size_t bytes, size_t offset,
+                               hipMemcpyKind) {
+  rt().drain_all();
+  std::memcpy(dst, static_cast<const unsigned char *>(symbol) + offset, bytes);
+  return hipSuccess;
+}
+}
+#else
 // ---- the library's kernels, on the stream's thread ------------------------------------
 namespace fkv {
 
@@ -543,6 +719,12 @@ int common_vector_width(const uint64_t *vals, int n) {
 
 } // namespace fkv
 
+#endif // FKV_KERNELS_FROM_SOURCE
+
+#ifndef FKV_KERNELS_FROM_SOURCE
+extern "C" unsigned long long fkv_emulated_workgroups_run() { return 0; }
+#endif
+
 // Test hook: the next `count` calls of `category` (0 device allocation, 1 pinned allocation,
 // 2 stream creation, 3 event creation, 4 copy, 5 kernel launch, 6 event record; 7: a kernel
 // launch throws std::bad_alloc, as an allocation of the library's own might) fail once `after`
@@ -567,6 +749,7 @@ int fkv_streams_run_concurrently(int32_t, void *a, void *b, int32_t *concurrent)
                 of(static_cast<hipStream_t>(b))->hardware_queue;
   return FKV_OK;
 }
+#ifndef FKV_KERNELS_FROM_SOURCE
 int fkv_transfer_kv_blocks_noalloc(const fkv_transfer_desc *, void *) {
   return fkv::fail(FKV_ERR_UNSUPPORTED, "emulated runtime: the entry point lives beside the kernels");
 }
@@ -576,4 +759,5 @@ int fkv_build_gpu_chunk_ptrs(const fkv_chunk_ptrs_desc *, void *) {
 int fkv_staging_transfer(const fkv_staging_transfer_desc *, void *) {
   return fkv::fail(FKV_ERR_UNSUPPORTED, "emulated runtime: the entry point lives beside the kernels");
 }
+#endif
 }

@@ -40,6 +40,7 @@ int fkv_oracle_tp_rank_plan(int rank, int num_gpus, int num_kv_heads, int is_hos
                             int64_t gpu_chunk_size, int64_t cpu_block_stride, int64_t cpu_tp_stride,
                             fkv_oracle_rank_plan *out);
 long fkv_emulated_fail(int category, long after, long count); // emulated_hip_runtime.cpp
+unsigned long long fkv_emulated_workgroups_run();             // 0: the kernels are stand-ins
 int fkv_oracle_transfer(int backend, const uint64_t *tensor_ptrs, int64_t num_layers_total,
                         int64_t gpu_kv_stride, int64_t gpu_block_stride, int64_t gpu_layer_stride,
                         int64_t gpu_off, uint8_t *cpu_ptr, int64_t cpu_kv_stride,
@@ -869,5 +870,7 @@ int main(int argc, char **argv) {
   printf("ok: %d groups of layerwise restores, %d sets of transfers, %d thread groups and %d bursts "
          "of concurrent calls over the emulated runtime; %ld runtime calls refused on request\n",
          restores, transfers, transfers, transfers, refused_calls);
+  if (fkv_emulated_workgroups_run())
+    printf("kernels from their sources: %llu workgroups\n", fkv_emulated_workgroups_run());
   return 0;
 }

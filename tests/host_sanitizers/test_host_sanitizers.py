@@ -71,43 +71,91 @@ LIBRARY_HOST_SOURCES = ["fkv_core", "fkv_ce", "fkv_host", "fkv_host_copy", "fkv_
                         "fkv_linkboard", "fkv_policy", "fkv_staged_restore"]
 
 
-_LIBRARY_OBJECTS = {}   # sanitizer flags -> objects of the library over the emulated runtime
+LIBRARY_KERNEL_SOURCES = ["fkv_kernels", "fkv_noalloc", "fkv_staging"]
+
+_LIBRARY_OBJECTS = {}   # sanitizer flags -> objects of the library's host code
+_DEVICE_OBJECTS = {}    # (sanitizer flags, kernels from source) -> emulated runtime and kernels
 
 
 def _compile(cmd):
     subprocess.run(cmd, check=True, capture_output=True, text=True)
 
 
-def build_over_emulated_runtime(tmp_path, driver, sanitizer, defines=()):
+def kernel_source_as_cpp(name, where):
+    """A kernel source of the library as a C++ file for the CPU device model
+    (cpu_device_model.h, included first): the three places where the device language has no
+    C++ spelling are rewritten, each checked to be there as often as expected, so that a
+    change of the source that this would miss fails here instead."""
+    text = open(os.path.join(ROOT, "flexkv_amd", "csrc", name + ".hip")).read()
+
+    def rewrite(old, new, count):
+        nonlocal text
+        assert text.count(old) == count, (name, old, text.count(old))
+        text = text.replace(old, new)
+
+    if name == "fkv_kernels":
+        # dynamically sized LDS: one array per workgroup, handed out by the model
+        rewrite("extern __shared__ uint64_t lds[];",
+                "uint64_t *lds = static_cast<uint64_t *>(cpu_device_model::dynamic_lds());", 2)
+        rewrite('asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(v));',
+                "v = cpu_device_model::xcc_id();", 1)
+        # the two entry points that time the device keep their stand-ins
+        rewrite("int fkv_streams_run_concurrently(", "int fkv_streams_run_concurrently_timed(", 1)
+        rewrite("int fkv_measure_hbm_rate(", "int fkv_measure_hbm_rate_timed(", 1)
+    path = os.path.join(where, name + ".cpp")
+    with open(path, "w") as f:
+        f.write(text)
+    return path
+
+
+def build_over_emulated_runtime(tmp_path, driver, sanitizer, defines=(), kernels_from_source=False):
     """Every host translation unit of the library, the emulated HIP runtime (streams as
-    threads, events as counters, the kernels as memcpy loops), the oracle's C file (the model
-    of the thread-group cases) and a driver, compiled with the sanitizer and linked into one
-    program.  The library's objects are built once per sanitizer and test session."""
+    threads, events as counters), the oracle's C file (the model of the thread-group cases)
+    and a driver, compiled with the sanitizer and linked into one program.  The kernels are
+    memcpy loops of the emulated runtime, or (`kernels_from_source`) the library's own kernel
+    sources compiled for the CPU device model: every work-item a host thread, so that the
+    sanitizer sees the addresses the kernels compute.  Objects are built once per sanitizer
+    and test session."""
     from concurrent.futures import ThreadPoolExecutor
+    import tempfile
     csrc = os.path.join(ROOT, "flexkv_amd", "csrc")
     flags = [CLANG, "-std=c++17", "-O1", "-g", *sanitizer, "-fno-omit-frame-pointer", "-mavx2",
              "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", "-I" + os.path.join(ROOT, "include"),
-             "-I" + csrc]
+             "-I" + csrc, "-I" + HERE]
     key = tuple(sanitizer)
+    jobs = []
     if key not in _LIBRARY_OBJECTS:
-        import tempfile
         where = tempfile.mkdtemp(prefix="fkv_emulated_", dir=str(tmp_path.parent))
         units = [os.path.join(csrc, f + ".cpp") for f in LIBRARY_HOST_SOURCES]
-        units.append(os.path.join(HERE, "emulated_hip_runtime.cpp"))
         objects = [os.path.join(where, os.path.basename(u)[:-4] + ".o") for u in units]
-        jobs = [flags + ["-c", u, "-o", o] for u, o in zip(units, objects)]
+        jobs += [flags + ["-c", u, "-o", o] for u, o in zip(units, objects)]
         oracle = os.path.join(where, "fkv_oracle.o")
         jobs.append([shutil.which("clang", path=os.path.dirname(CLANG)) or "clang", "-O1", "-g",
                      *sanitizer, "-fno-omit-frame-pointer", "-c",
                      os.path.join(ROOT, "oracle", "fkv_oracle.c"), "-o", oracle])
+        _LIBRARY_OBJECTS[key] = objects + [oracle]
+    if (key, kernels_from_source) not in _DEVICE_OBJECTS:
+        where = tempfile.mkdtemp(prefix="fkv_device_", dir=str(tmp_path.parent))
+        mode = ["-DFKV_KERNELS_FROM_SOURCE"] if kernels_from_source else []
+        objects = [os.path.join(where, "emulated_hip_runtime.o")]
+        jobs.append(flags + mode + ["-c", os.path.join(HERE, "emulated_hip_runtime.cpp"),
+                                    "-o", objects[0]])
+        if kernels_from_source:
+            for name in LIBRARY_KERNEL_SOURCES:
+                objects.append(os.path.join(where, name + ".o"))
+                jobs.append(flags + mode + ["-include", os.path.join(HERE, "cpu_device_model.h"),
+                                            "-c", kernel_source_as_cpp(name, where),
+                                            "-o", objects[-1]])
+        _DEVICE_OBJECTS[(key, kernels_from_source)] = objects
+    if jobs:
         with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 2)) as pool:
             list(pool.map(_compile, jobs))
-        _LIBRARY_OBJECTS[key] = objects + [oracle]
     source = driver if os.path.isabs(driver) else os.path.join(HERE, driver)
     obj = str(tmp_path / "driver.o")
     _compile(flags + [*defines, "-c", source, "-o", obj])
     exe = str(tmp_path / "driver")
-    _compile([CLANG, *sanitizer, *_LIBRARY_OBJECTS[key], obj, "-o", exe, "-pthread", "-ldl"])
+    _compile([CLANG, *sanitizer, *_LIBRARY_OBJECTS[key],
+              *_DEVICE_OBJECTS[(key, kernels_from_source)], obj, "-o", exe, "-pthread", "-ldl"])
     return exe
 
 
@@ -154,3 +202,34 @@ def test_native_consumers_over_an_emulated_runtime_under_sanitizers(tmp_path, sa
         r = subprocess.run([exe, *args], capture_output=True, text=True, env=env, timeout=900)
         assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
         assert expect in r.stdout, r.stdout[-2000:]
+
+
+@pytest.mark.parametrize("sanitizer", SANITIZERS)
+def test_kernel_sources_on_a_cpu_device_model_under_sanitizers(tmp_path, sanitizer):
+    """The same two programs with the library's kernels compiled from their own sources for a
+    CPU model of the device (cpu_device_model.h: a workgroup is a crew of host threads,
+    __syncthreads a barrier, the atomics host atomics, XCD ids dealt in turn with a start that
+    moves from launch to launch): AddressSanitizer checks every address the gather/scatter
+    kernel computes on every route (whole slices, short last slices, packed chunks, several
+    jobs in one launch, fixed shares, claimed ranges, launches confined to some XCDs and their
+    safety net), ThreadSanitizer the order among work-items; the launch shaping, the plan
+    upload, the entry point that allocates nothing and the compressed-staging kernels run as
+    shipped (35 cases of the ABI driver instead of 33)."""
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:verify_asan_link_order=0",
+               TSAN_OPTIONS="halt_on_error=1", TMPDIR=str(tmp_path))
+    sub = tmp_path / "restores"
+    sub.mkdir()
+    exe = build_over_emulated_runtime(sub, "layerwise_emulated_driver.cpp", sanitizer,
+                                      kernels_from_source=True)
+    r = subprocess.run([exe, "16", "8"], capture_output=True, text=True, env=env, timeout=900)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
+    assert "ok: 16 groups of layerwise restores, 8 sets of transfers" in r.stdout
+    assert "kernels from their sources:" in r.stdout
+    sub = tmp_path / "abi"
+    sub.mkdir()
+    exe = build_over_emulated_runtime(
+        sub, os.path.join(ROOT, "tests", "native", "abi_roundtrip_driver.cpp"), sanitizer,
+        defines=("-DFKV_EMULATED_RUNTIME", "-DFKV_KERNELS_FROM_SOURCE"), kernels_from_source=True)
+    r = subprocess.run([exe], capture_output=True, text=True, env=env, timeout=900)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
+    assert "ok: 35 cases through the C ABI" in r.stdout, r.stdout[-2000:]

@@ -508,7 +508,8 @@ int main() {
     ++cases;
   }
 
-#ifndef FKV_EMULATED_RUNTIME // the next two sections are about the kernels themselves
+// the next two sections are about the kernels themselves: not with stand-ins for them
+#if !defined(FKV_EMULATED_RUNTIME) || defined(FKV_KERNELS_FROM_SOURCE)
   // ---- launch policy: every way a launch shares out its work, and the entry point that
   //      allocates nothing, on the same descriptor ----
   {
