@@ -179,7 +179,7 @@ ihipStream_t *of(hipStream_t s) { return s ? s : rt().null_stream(); }
 void *allocate(size_t size, bool pinned) {
   // 2 MiB alignment, as the runtime gives large allocations
   void *p = nullptr;
-  if (posix_memalign(&p, (size_t)2 << 20, std::max<size_t>(size, 64)) != 0)
+  if (posix_memalign(&p, (size_t)2 << 20, std::max<size_t>(size, 1)) != 0)
     return nullptr;
   std::lock_guard<std::mutex> lk(rt().mu);
   rt().memory[(uintptr_t)p] = Runtime::Block{std::max<size_t>(size, 64), pinned, false};

@@ -233,3 +233,24 @@ def test_kernel_sources_on_a_cpu_device_model_under_sanitizers(tmp_path, sanitiz
     r = subprocess.run([exe], capture_output=True, text=True, env=env, timeout=900)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
     assert "ok: 35 cases through the C ABI" in r.stdout, r.stdout[-2000:]
+
+
+@pytest.mark.parametrize("sanitizer,launches", [(SANITIZERS[0].values[0], 60),
+                                                (SANITIZERS[1].values[0], 30)],
+                         ids=["asan-ubsan", "tsan"])
+def test_gather_scatter_kernel_shapes_on_a_cpu_device_model(tmp_path, sanitizer, launches):
+    """The gather/scatter kernel by itself, launched through the library's own shaping code
+    with seeded arguments over the space of shapes (vector widths 1-16, whole slices, a short
+    last slice, packed chunks, the deep unroll, up to 1024 (layer, kv) pairs, more positions
+    than an id tile, with and without id lists, both store kinds, fixed shares, claimed ranges,
+    confined launches with dirty counters, one to four jobs a launch).  Tables, id lists and
+    chunk regions are allocations of exactly the size the kernel may touch, so one vector too
+    far is a sanitizer report; every destination byte is compared with a plain model.
+    400 launches of the same program were run once by hand (clean); the suite runs fewer."""
+    exe = build_over_emulated_runtime(tmp_path, "copy_kernel_model_driver.cpp", sanitizer,
+                                      kernels_from_source=True)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:verify_asan_link_order=0",
+               TSAN_OPTIONS="halt_on_error=1", TMPDIR=str(tmp_path))
+    r = subprocess.run([exe, str(launches)], capture_output=True, text=True, env=env, timeout=900)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
+    assert "ok: %d launches of the gather/scatter kernel on the CPU device model" % launches in r.stdout
