@@ -503,8 +503,9 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=F
 def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, verify=True):
     """c4: 32 D2H puts and 32 H2D gets issued at once from 64 threads.  Each
     direction has its own set of streams (one per request by default); the
-    process has 4 hardware queues, so with more than 2 streams per direction
-    puts and gets also share queues and partly serialize."""
+    process has a few hardware queues (GPU_MAX_HW_QUEUES: 4 by HIP's default, see
+    --hw-queues), so with more streams per direction than half of them puts and gets
+    also share queues and partly serialize."""
     reqs = w.requests
     per_dir = max(1, min(streams_per_direction, len(reqs) // 2))
     pool = [[torch.cuda.Stream() for _ in range(per_dir)] for _ in range(2)]
@@ -1343,6 +1344,7 @@ def measure_config(name, args, torch, device, link, steps, warmup):
         out.update(value=round(agg, 3), ms_per_step=round(_median(r["walls"]) * 1e3, 3),
                    aggregate_GBps=round(agg, 3), requests=64,
                    streams_per_direction=args.streams_per_direction,
+                   hardware_queues=int(os.environ.get("GPU_MAX_HW_QUEUES", "4")),
                    total_blocks=sum(r["blocks"]), aggregate_bytes=r["total_bytes"],
                    p50_latency_ms=round(r["p50_ms"], 3), p99_latency_ms=round(r["p99_ms"], 3),
                    bidir_link_peak_GBps=round(bidir, 3), frac_of_bidir_link=round(agg / bidir, 4),
@@ -1460,6 +1462,9 @@ def main():
     ap.add_argument("--other-steps", type=int, default=10,
                     help="all: timed steps of the configurations next to the headline one "
                          "(3 warm-up steps each)")
+    ap.add_argument("--hw-queues", type=int, default=0, choices=range(0, 33), metavar="0..32",
+                    help="GPU_MAX_HW_QUEUES of this process (HIP's default is 4; 0, the default "
+                         "here, leaves the environment as it is)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     args = ap.parse_args()
@@ -1468,6 +1473,15 @@ def main():
               "link per GPU and has no cross-GPU step); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    # Hardware queues of the process: the runtime reads this when it starts.  HIP's default is
+    # 4, the reference's platform gives a process 8 (CUDA_DEVICE_MAX_CONNECTIONS).  With 64
+    # requests in flight on 64 streams the 4 make puts and gets queue up behind each other
+    # (c4: 86.8 GB/s in sum with 4, 93.3 with 8 or 16); a layerwise restore next to compute is
+    # the other way round (c3: 42 ms with 4; with 8, 52 ms in every second or third run,
+    # although no stream of the restore shares the compute stream's queue).  Left as the
+    # environment has it unless asked for.
+    if args.hw_queues > 0:
+        os.environ["GPU_MAX_HW_QUEUES"] = str(args.hw_queues)
     import torch
     import flexkv_amd.c_ext as c_ext  # fails loudly if libfkv_hip.so is missing
     if args.config == "ssd":  # host pool <-> files: no GPU work in this one
@@ -1692,6 +1706,7 @@ def main():
                                  "c3_fragmented and c4 are under `configs`, each with its own "
                                  "steps / warmup"}
     out["link_peak"] = link_rec
+    out["hardware_queues"] = int(os.environ.get("GPU_MAX_HW_QUEUES", "4"))   # of this process
     pol = c_ext.get_launch_policy()
     out["launch_policy"] = {k: pol[k] for k in (
         "model_seeded", "model_link_mbps", "model_kernel_d2h_mbps", "model_kernel_h2d_mbps",
