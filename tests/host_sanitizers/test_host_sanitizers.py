@@ -221,9 +221,9 @@ def test_kernel_sources_on_a_cpu_device_model_under_sanitizers(tmp_path, sanitiz
     sub.mkdir()
     exe = build_over_emulated_runtime(sub, "layerwise_emulated_driver.cpp", sanitizer,
                                       kernels_from_source=True)
-    r = subprocess.run([exe, "16", "8"], capture_output=True, text=True, env=env, timeout=900)
+    r = subprocess.run([exe, "10", "6"], capture_output=True, text=True, env=env, timeout=900)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
-    assert "ok: 16 groups of layerwise restores, 8 sets of transfers" in r.stdout
+    assert "ok: 10 groups of layerwise restores, 6 sets of transfers" in r.stdout
     assert "kernels from their sources:" in r.stdout
     sub = tmp_path / "abi"
     sub.mkdir()
@@ -235,8 +235,8 @@ def test_kernel_sources_on_a_cpu_device_model_under_sanitizers(tmp_path, sanitiz
     assert "ok: 35 cases through the C ABI" in r.stdout, r.stdout[-2000:]
 
 
-@pytest.mark.parametrize("sanitizer,launches", [(SANITIZERS[0].values[0], 60),
-                                                (SANITIZERS[1].values[0], 30)],
+@pytest.mark.parametrize("sanitizer,launches", [(SANITIZERS[0].values[0], 40),
+                                                (SANITIZERS[1].values[0], 20)],
                          ids=["asan-ubsan", "tsan"])
 def test_gather_scatter_kernel_shapes_on_a_cpu_device_model(tmp_path, sanitizer, launches):
     """The gather/scatter kernel by itself, launched through the library's own shaping code
