@@ -140,6 +140,17 @@ struct PlanPool {
   // Slots are never freed: the pool outlives every stream that may still read
   // them, and tearing HIP objects down from a static destructor is unsafe.
   std::vector<PlanSlot *> slots;
+  // The claim counters of a device's slots are cut from chunks that are allocated and
+  // cleared for many slots at once: clearing is a copy the host waits for, and under load
+  // that wait is long and holds up every thread that needs a slot (a process with four
+  // hardware queues has the null stream on the queue of some transfer stream: 64 requests
+  // in flight, one new slot, 24 ms during which no thread launched anything).  The first
+  // slot of a device pays for it, when nothing of the library is in flight there.
+  struct CounterChunk {
+    uint64_t *base = nullptr;
+    int handed_out = 0; // slots that have their counters from this chunk
+  };
+  std::map<int, CounterChunk> counter_chunks; // by device: the chunk that still has room
 };
 PlanPool &pool() {
   static PlanPool *p = new PlanPool();
@@ -147,6 +158,34 @@ PlanPool &pool() {
 }
 constexpr size_t kPlanMinBytes = 64 * 1024;
 constexpr int kPlanCounters = 1024;
+constexpr int kPlanSlotsPerChunk = 256; // as many as the pool holds before it waits for the oldest
+
+// kPlanCounters counters for a new slot of `device` (current); p.mu is held.
+uint64_t *counters_for_new_slot(PlanPool &p, int device) {
+  PlanPool::CounterChunk &chunk = p.counter_chunks[device];
+  if (!chunk.base || chunk.handed_out == kPlanSlotsPerChunk) {
+    // Cleared for tidiness and against a leftover whose high half happens to be the number
+    // of the first launch that uses it; a launch takes a counter over whatever else it
+    // holds (Shares::adopt).  A copy that has finished when it returns: a hipMemset on the
+    // null stream can still be under way when the first kernel on a non-blocking stream
+    // claims from the counters.
+    const size_t count = (size_t)kPlanCounters * kPlanSlotsPerChunk;
+    // FKV_TEST_DIRTY_COUNTERS=1 (tests): start them with garbage instead
+    static const std::vector<uint64_t> zeros(
+        count, env_flag("FKV_TEST_DIRTY_COUNTERS") ? 0xdeadbeef00000007ull : 0u);
+    void *c = nullptr;
+    if (hipMalloc(&c, count * sizeof(uint64_t)) != hipSuccess ||
+        hipMemcpy(c, zeros.data(), count * sizeof(uint64_t), hipMemcpyHostToDevice) != hipSuccess) {
+      (void)hipGetLastError();
+      if (c)
+        (void)hipFree(c);
+      return nullptr;
+    }
+    chunk.base = static_cast<uint64_t *>(c); // an exhausted chunk stays with its slots
+    chunk.handed_out = 0;
+  }
+  return chunk.base + (size_t)kPlanCounters * chunk.handed_out++;
+}
 
 bool slot_grow(PlanSlot *s, size_t bytes) {
   if (s->cap >= bytes)
@@ -214,26 +253,13 @@ PlanSlot *plan_acquire(int device, size_t bytes) {
         fail(FKV_ERR_RUNTIME, "plan memory: hipEventCreate failed");
         return nullptr;
       }
-      // Zeroed for tidiness only, by a copy that has finished when it returns (a
-      // hipMemset on the null stream can still be under way when the first kernel on
-      // a non-blocking stream claims from the counters): a launch takes a counter
-      // over whatever it holds, see Shares::adopt.
-      void *c = nullptr;
-      const size_t cbytes = (size_t)kPlanCounters * sizeof(uint64_t);
-      // FKV_TEST_DIRTY_COUNTERS=1 (tests): start them with garbage instead
-      static const std::vector<uint64_t> zeros(
-          (size_t)kPlanCounters, env_flag("FKV_TEST_DIRTY_COUNTERS") ? 0xdeadbeef00000007ull : 0u);
-      if (hipMalloc(&c, cbytes) != hipSuccess ||
-          hipMemcpy(c, zeros.data(), cbytes, hipMemcpyHostToDevice) != hipSuccess) {
-        (void)hipGetLastError();
-        if (c)
-          (void)hipFree(c);
+      pick->counters = counters_for_new_slot(p, device);
+      if (!pick->counters) {
         (void)hipEventDestroy(pick->done);
         delete pick;
         fail(FKV_ERR_RUNTIME, "plan memory: cannot allocate the claim counters");
         return nullptr;
       }
-      pick->counters = static_cast<uint64_t *>(c);
       p.slots.push_back(pick);
     }
     pick->busy = true;
