@@ -1474,12 +1474,11 @@ def main():
         sys.exit(2)
 
     # Hardware queues of the process: the runtime reads this when it starts.  HIP's default is
-    # 4, the reference's platform gives a process 8 (CUDA_DEVICE_MAX_CONNECTIONS).  With 64
-    # requests in flight on 64 streams the 4 make puts and gets queue up behind each other
-    # (c4: 86.8 GB/s in sum with 4, 93.3 with 8 or 16); a layerwise restore next to compute is
-    # the other way round (c3: 42 ms with 4; with 8, 52 ms in every second or third run,
-    # although no stream of the restore shares the compute stream's queue).  Left as the
-    # environment has it unless asked for.
+    # 4, the reference's platform gives a process 8 (CUDA_DEVICE_MAX_CONNECTIONS).  c4 reaches
+    # the same 93 GB/s with 2, 4, 8 and 16; a layerwise restore next to compute wants the
+    # default (c3: 42 ms with 4; with 8, 52 ms in every second or third run, although no
+    # stream of the restore shares the compute stream's queue).  Left as the environment has
+    # it unless asked for.
     if args.hw_queues > 0:
         os.environ["GPU_MAX_HW_QUEUES"] = str(args.hw_queues)
     import torch

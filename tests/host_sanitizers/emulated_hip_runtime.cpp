@@ -124,6 +124,7 @@ enum Category { kDeviceAlloc, kPinnedAlloc, kStreamCreate, kEventCreate, kCopy, 
 std::atomic<long> g_fail_after[kCategories];
 std::atomic<long> g_fail_count[kCategories];
 std::atomic<long> g_failed_calls{0};
+std::atomic<long> g_host_waited_copies{0}; // hipMemcpy calls: the host waits for each
 bool refused(Category c) {
   if (g_fail_count[c].load(std::memory_order_relaxed) <= 0)
     return false;
@@ -440,6 +441,7 @@ hipError_t hipMemcpyAsync(void *dst, const void *src, size_t n, hipMemcpyKind, h
   return hipSuccess;
 }
 hipError_t hipMemcpy(void *dst, const void *src, size_t n, hipMemcpyKind) {
+  g_host_waited_copies.fetch_add(1);
   rt().null_stream()->drain();
   std::memcpy(dst, src, n);
   return hipSuccess;
@@ -724,6 +726,10 @@ int common_vector_width(const uint64_t *vals, int n) {
 #ifndef FKV_KERNELS_FROM_SOURCE
 extern "C" unsigned long long fkv_emulated_workgroups_run() { return 0; }
 #endif
+
+// Copies the host has waited for since the process started (hipMemcpy): a library that
+// makes one per request under load holds every thread up for as long as the device is busy.
+extern "C" long fkv_emulated_host_waited_copies() { return g_host_waited_copies.load(); }
 
 // Test hook: the next `count` calls of `category` (0 device allocation, 1 pinned allocation,
 // 2 stream creation, 3 event creation, 4 copy, 5 kernel launch, 6 event record; 7: a kernel

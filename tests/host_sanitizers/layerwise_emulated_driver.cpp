@@ -41,6 +41,7 @@ int fkv_oracle_tp_rank_plan(int rank, int num_gpus, int num_kv_heads, int is_hos
                             fkv_oracle_rank_plan *out);
 long fkv_emulated_fail(int category, long after, long count); // emulated_hip_runtime.cpp
 unsigned long long fkv_emulated_workgroups_run();             // 0: the kernels are stand-ins
+long fkv_emulated_host_waited_copies();                        // hipMemcpy calls so far
 int fkv_oracle_transfer(int backend, const uint64_t *tensor_ptrs, int64_t num_layers_total,
                         int64_t gpu_kv_stride, int64_t gpu_block_stride, int64_t gpu_layer_stride,
                         int64_t gpu_off, uint8_t *cpu_ptr, int64_t cpu_kv_stride,
@@ -659,6 +660,7 @@ void concurrent_case(uint64_t seed) {
     }
   std::vector<std::thread> pool;
   std::atomic<int> failures{0};
+  const long waited_before = fkv_emulated_host_waited_copies();
   for (int t = 0; t < threads; ++t)
     pool.emplace_back([&, t] {
       hipStream_t st = nullptr;
@@ -703,6 +705,12 @@ void concurrent_case(uint64_t seed) {
   for (auto &th : pool)
     th.join();
   REQUIRE(failures.load() == 0, "seed %llu: %d calls failed", (unsigned long long)seed, failures.load());
+  // Plan memory, counters and staging were set up by the transfers before this case: with
+  // requests in flight the library makes no copy that the host waits for (it would wait for
+  // the device's queue, with locks held that every other request needs).
+  REQUIRE(fkv_emulated_host_waited_copies() == waited_before,
+          "seed %llu: %ld host-waited copies during concurrent requests", (unsigned long long)seed,
+          fkv_emulated_host_waited_copies() - waited_before);
   for (int t = 0; t < threads; ++t)
     for (const Op &op : script[t])
       for (int l = 0; l < s.L; ++l)
