@@ -1347,6 +1347,7 @@ def measure_config(name, args, torch, device, link, steps, warmup):
                    hardware_queues=int(os.environ.get("GPU_MAX_HW_QUEUES", "4")),
                    total_blocks=sum(r["blocks"]), aggregate_bytes=r["total_bytes"],
                    p50_latency_ms=round(r["p50_ms"], 3), p99_latency_ms=round(r["p99_ms"], 3),
+                   burst_ms=[round(x * 1e3, 2) for x in r["walls"]],   # every timed burst
                    bidir_link_peak_GBps=round(bidir, 3), frac_of_bidir_link=round(agg / bidir, 4),
                    frac_of_sum_of_one_way_peaks=round(agg / (link["d2h"] + link["h2d"]), 4))
     del w
@@ -1465,6 +1466,10 @@ def main():
     ap.add_argument("--hw-queues", type=int, default=0, choices=range(0, 33), metavar="0..32",
                     help="GPU_MAX_HW_QUEUES of this process (HIP's default is 4; 0, the default "
                          "here, leaves the environment as it is)")
+    ap.add_argument("--sequence", default=None, metavar="CFG,CFG,...",
+                    help="all: after the headline configuration measure only these, in this "
+                         "order (NAME+ce: through the copy-engine strategies), without the "
+                         "worker sub-record, and print them")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     args = ap.parse_args()
@@ -1669,9 +1674,20 @@ def main():
         return {k: ce[k] for k in ("d2h_GBps", "h2d_GBps", "d2h_frac_of_link", "h2d_frac_of_link",
                                    "d2h_ms_median", "d2h_ms_min", "h2d_ms_median", "h2d_ms_min",
                                    "d2h_ms_steps", "h2d_ms_steps", "path_taken", "steps")}
-    if not args.use_ce:
+    if not args.use_ce and not args.sequence:
         records[head]["copy_engine"] = copy_engine_record(head, min(3, args.steps))
     args.with_fragmented = True
+    if args.sequence:   # a study of what one configuration leaves behind for the next
+        for name in args.sequence.split(","):
+            if name.endswith("+ce"):   # the same blocks through the copy-engine strategies
+                records[name + "_in_sequence"] = copy_engine_record(name[:-3], min(5, args.other_steps))
+                continue
+            records[name + "_in_sequence"] = measure_config(
+                name, args, torch, device, link, 20 if name == "c4" else args.other_steps,
+                1 if name == "c4" else 3)
+            records[name + "_in_sequence"].pop("fragmented_record", None)
+        print(json.dumps({"sequence": args.sequence, "configs": records}))
+        return
     for name in ("c0", "c2", "c3", "c4"):
         # c4's latency percentiles want repetitions: 20 bursts of its 64 requests
         records[name] = measure_config(name, args, torch, device, link,

@@ -534,6 +534,7 @@ int device_staging_copy(const fkv_transfer_desc &d, int it0, int nit, int p0, in
     PlanSlot *slot = plan_acquire(device, 2 * tab + ids);
     if (!slot)
       return FKV_ERR_RUNTIME;
+    PlanSlotHold hold{slot, stream};
     uint8_t *h = plan_host(slot);
     uint64_t *gbase = reinterpret_cast<uint64_t *>(h);
     uint64_t *sbase = reinterpret_cast<uint64_t *>(h + tab);
@@ -570,7 +571,6 @@ int device_staging_copy(const fkv_transfer_desc &d, int it0, int nit, int p0, in
       a.unroll = pol.hbm_unroll;
       rc = launch_copy_kernel(a, kStagingWorkgroups, kStagingThreads, stream);
     }
-    plan_release(slot, stream, false);
     if (rc != FKV_OK)
       return rc;
   }

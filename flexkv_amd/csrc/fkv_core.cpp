@@ -278,6 +278,15 @@ PlanSlot *plan_acquire(int device, size_t bytes) {
   return pick;
 }
 
+void plan_pool_counts(int *slots, int *handed_out) {
+  PlanPool &p = pool();
+  std::lock_guard<std::mutex> lk(p.mu);
+  *slots = (int)p.slots.size();
+  *handed_out = 0;
+  for (const PlanSlot *s : p.slots)
+    *handed_out += s->busy ? 1 : 0;
+}
+
 uint8_t *plan_host(PlanSlot *s) { return s->host; }
 uint64_t *plan_counters(PlanSlot *s, int count) {
   return count <= kPlanCounters ? s->counters : nullptr;
@@ -711,9 +720,8 @@ int run_kernel_path(const fkv_transfer_desc &d, hipStream_t stream) {
   set_last_path(FKV_PATH_KERNEL);
   KernelPlan plan;
   FKV_TRY(kernel_plan_build(d, stream, &plan));
-  int rc = kernel_plan_launch(plan, 0, d.num_layers, stream);
-  kernel_plan_release(&plan, stream);
-  return rc;
+  KernelPlanHold hold{&plan, stream};
+  return kernel_plan_launch(plan, 0, d.num_layers, stream);
 }
 
 int validate(const fkv_transfer_desc &d) {
@@ -975,6 +983,15 @@ int order_after(hipStream_t from, hipStream_t to, int device, int which) {
 int run_kernel_path_multi(const fkv_transfer_desc *descs, int count, hipStream_t stream) {
   fkv::set_last_path(FKV_PATH_KERNEL);
   std::vector<fkv::KernelPlan> plans(count);
+  struct GiveBack { // also when a launch throws
+    std::vector<fkv::KernelPlan> &plans;
+    hipStream_t stream;
+    ~GiveBack() {
+      for (fkv::KernelPlan &p : plans)
+        if (p.slot)
+          fkv::kernel_plan_release(&p, stream);
+    }
+  } give_back{plans, stream};
   int rc = FKV_OK, built = 0;
   for (; built < count && rc == FKV_OK; ++built)
     rc = fkv::kernel_plan_build(descs[built], stream, &plans[built]);
@@ -991,8 +1008,6 @@ int run_kernel_path_multi(const fkv_transfer_desc *descs, int count, hipStream_t
     }
     rc = fkv::kernel_plans_launch(group, first, layers, n, stream);
   }
-  for (int i = 0; i < built; ++i)
-    fkv::kernel_plan_release(&plans[i], stream);
   return rc;
 }
 

@@ -215,6 +215,9 @@ int common_vector_width(const uint64_t *vals, int n);
 struct PlanSlot;
 // Returns nullptr (and sets the error) on allocation failure.
 PlanSlot *plan_acquire(int device, size_t bytes);
+// Slots the pool holds, and how many of them are handed out at the moment (acquired and not
+// yet released): after every user has finished, none.
+void plan_pool_counts(int *slots, int *handed_out);
 uint8_t *plan_host(PlanSlot *s);
 // `count` claim counters in device memory that belong to the slot
 // (CopyKernelArgs::claim), or nullptr when a slot holds fewer.
@@ -250,6 +253,24 @@ struct KernelPlan {
   bool recorded = false; // the launches are being recorded into a graph: shaped once for every
                          // replay, without a look at what the link is doing right now
   uint64_t *claims = nullptr; // a claim counter per layer of the plan, device memory
+};
+void kernel_plan_release(KernelPlan *p, hipStream_t stream);
+// Give plan memory back when the scope ends, by whichever way it ends.
+struct KernelPlanHold {
+  KernelPlan *plan;
+  hipStream_t stream;
+  ~KernelPlanHold() {
+    if (plan && plan->slot)
+      kernel_plan_release(plan, stream);
+  }
+};
+struct PlanSlotHold {
+  PlanSlot *slot;
+  hipStream_t stream;
+  ~PlanSlotHold() {
+    if (slot)
+      plan_release(slot, stream, false);
+  }
 };
 // Link-bound launches of the last while, per device and direction (see fkv_core.cpp).
 bool link_direction_busy(int device, bool h2d, hipStream_t launching_stream);

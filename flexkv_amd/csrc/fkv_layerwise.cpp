@@ -471,6 +471,7 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
     alt_max_bytes[i] = (int64_t)pol.kernel_alt_stream_kb * 1024;
   }
   std::vector<char> alt_used(g->num_gpus, 0);
+  try { // an exception ends the launches like an error: the plans below are given back either way
   for (int b = 0; b < num_batches && rc == FKV_OK; ++b) {
     if (give_up_at > 0 && b == give_up_at - 1) {
       rc = fail(FKV_ERR_RUNTIME, "layerwise restore made to give up before batch %d (test_fail_restore_batch)", b);
@@ -566,6 +567,9 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
     }
     if (rc == FKV_OK)
       g->gate.publish(b + 1);
+  }
+  } catch (...) {
+    rc = caught("launches of a layerwise restore");
   }
   // The second stream joins the first: what follows on `streams` (the release of the plan
   // memory, a synchronize, the next call) is behind every batch.
@@ -936,6 +940,7 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
   // copy command per block and layer: 8.7 GB/s on 512 blocks of 72 KiB).
   const EngineChoice choice{c.use_ce_transfer, c.transfer_cta_num};
   const bool direct = choice.use_ce_transfer == 0;
+  try { // an exception part-way ends the call like an error: launch_batches gives back what was built
   for (Lane &lane : lanes) {
     if (!lane.used || rc != FKV_OK)
       continue;
@@ -987,6 +992,9 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
                     d.cpu_ptr);
       }
     }
+  }
+  } catch (...) {
+    rc = caught("plans of a layerwise restore");
   }
   // Staging memory that several restores in a row had no use for goes back (a group
   // with many lanes would otherwise hold buffers for every route it ever took).

@@ -204,13 +204,10 @@ int fkv_staging_transfer(const fkv_staging_transfer_desc *dp, void *stream_v) tr
   PlanSlot *slot = plan_acquire(device, ids_bytes);
   if (!slot)
     return FKV_ERR_RUNTIME;
+  PlanSlotHold hold{slot, stream};
   std::memcpy(plan_host(slot), d.cpu_block_ids, ids_bytes);
   uint8_t *dv = nullptr;
-  int rc = plan_publish(slot, ids_bytes, /*mirror=*/true, stream, &dv);
-  if (rc != FKV_OK) {
-    plan_release(slot, stream, false);
-    return rc;
-  }
+  FKV_TRY(plan_publish(slot, ids_bytes, /*mirror=*/true, stream, &dv));
   StagingKernelArgs a{};
   a.staging = static_cast<uint8_t *>(d.staging);
   a.staging_stride = d.staging_stride;
@@ -256,7 +253,6 @@ int fkv_staging_transfer(const fkv_staging_transfer_desc *dp, void *stream_v) tr
     FKV_LAUNCH_STAGING(false, false);
 #undef FKV_LAUNCH_STAGING
   hipError_t e = hipGetLastError();
-  plan_release(slot, stream, false);
   if (e != hipSuccess)
     return fail(FKV_ERR_RUNTIME, "staging transfer launch failed: %s", hipGetErrorString(e));
   stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);
@@ -310,6 +306,7 @@ int fkv_build_gpu_chunk_ptrs(const fkv_chunk_ptrs_desc *dp, void *stream_v) try 
   PlanSlot *slot = plan_acquire(device, tab + ids_bytes);
   if (!slot)
     return FKV_ERR_RUNTIME;
+  PlanSlotHold hold{slot, stream};
   uint8_t *h = plan_host(slot);
   uint64_t *base = reinterpret_cast<uint64_t *>(h);
   for (int64_t l = 0; l <= last_layer; ++l)
@@ -333,7 +330,6 @@ int fkv_build_gpu_chunk_ptrs(const fkv_chunk_ptrs_desc *dp, void *stream_v) try 
     if (e != hipSuccess)
       rc = fail(FKV_ERR_RUNTIME, "chunk pointer launch failed: %s", hipGetErrorString(e));
   }
-  plan_release(slot, stream, false);
   if (rc != FKV_OK)
     return rc;
   stats().kernel_launches.fetch_add(1, std::memory_order_relaxed);

@@ -60,6 +60,7 @@ extern "C" int fkv_layout_transform(const fkv_layout_transform_desc *dp, void *s
     PlanSlot *slot = plan_acquire(device, 2 * tab + ids);
     if (!slot)
       return FKV_ERR_RUNTIME;
+    PlanSlotHold hold{slot, stream};
     uint8_t *h = plan_host(slot);
     uint64_t *gbase = reinterpret_cast<uint64_t *>(h);
     uint64_t *bbase = reinterpret_cast<uint64_t *>(h + tab);
@@ -97,7 +98,6 @@ extern "C" int fkv_layout_transform(const fkv_layout_transform_desc *dp, void *s
       a.xcd_mask = 0;
       rc = launch_copy_kernel(a, workgroups, threads, stream);
     }
-    plan_release(slot, stream, false);
     if (rc != FKV_OK)
       return rc;
   }

@@ -23,6 +23,10 @@
 
 #include "fkv_transfer.h"
 
+namespace fkv {
+void plan_pool_counts(int *slots, int *handed_out); // fkv_core.cpp: the pool of plan memory
+}
+
 // the CPU restatement of the reference's rank placement and byte loop (oracle/fkv_oracle.c)
 extern "C" {
 typedef struct {
@@ -878,6 +882,10 @@ int main(int argc, char **argv) {
   printf("ok: %d groups of layerwise restores, %d sets of transfers, %d thread groups and %d bursts "
          "of concurrent calls over the emulated runtime; %ld runtime calls refused on request\n",
          restores, transfers, transfers, transfers, refused_calls);
+  int plan_slots = 0, plan_slots_out = 0;
+  fkv::plan_pool_counts(&plan_slots, &plan_slots_out);
+  REQUIRE(plan_slots_out == 0, "%d of %d plan slots were never given back", plan_slots_out, plan_slots);
+  printf("plan pool: %d slots, all given back\n", plan_slots);
   if (fkv_emulated_workgroups_run())
     printf("kernels from their sources: %llu workgroups\n", fkv_emulated_workgroups_run());
   return 0;
