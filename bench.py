@@ -566,8 +566,13 @@ def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, v
         ok = w.verify_host_image(w.gpu_ids, w.cpu_ids) and all(
             bool(w.gpu_rows(l, 0).index_select(0, reqs[1][0].to(w.device)).any())
             for l in (0, w.L - 1))
+    from flexkv_amd.c_ext import get_stats
+    st = get_stats()
     return dict(walls=walls, p99_ms=p99, p50_ms=_median(all_lat), total_bytes=total_bytes,
-                blocks=[int(g.numel()) for g, _ in reqs], bit_exact=ok)
+                blocks=[int(g.numel()) for g, _ in reqs], bit_exact=ok,
+                # slots of the library's plan pool after the bursts, and how often a request
+                # had to wait for the oldest user of one since the counters were last reset
+                plan_memory={k: st[k] for k in ("plan_slots", "plan_slots_in_use", "plan_slot_waits")})
 
 
 def run_groups(torch, device, num_cta, reps=30):
@@ -1348,6 +1353,7 @@ def measure_config(name, args, torch, device, link, steps, warmup):
                    total_blocks=sum(r["blocks"]), aggregate_bytes=r["total_bytes"],
                    p50_latency_ms=round(r["p50_ms"], 3), p99_latency_ms=round(r["p99_ms"], 3),
                    burst_ms=[round(x * 1e3, 2) for x in r["walls"]],   # every timed burst
+                   plan_memory=r["plan_memory"],
                    bidir_link_peak_GBps=round(bidir, 3), frac_of_bidir_link=round(agg / bidir, 4),
                    frac_of_sum_of_one_way_peaks=round(agg / (link["d2h"] + link["h2d"]), 4))
     del w
@@ -1665,7 +1671,17 @@ def main():
     # most bytes per step through the plain gather/scatter call (8 GiB each way).
     # c0, c2, c3 and c4 follow with `--other-steps` timed steps each.
     head = "c1"
-    records = {head: measure_config(head, args, torch, device, link, args.steps, args.warmup)}
+    records = {}
+    if not args.sequence:
+        # c4 first: its 64 requests share the link between the directions, and that balance is
+        # the one figure here that depends on what the process has done before (93 GB/s in a
+        # fresh process or after any one other configuration, 85-90 GB/s at the end of the whole
+        # sequence, where one direction finishes its requests 20-30 ms before the other; the
+        # one-direction figures do not move with the order).  `--sequence ...,c4` measures it
+        # behind configurations of choice.
+        records["c4"] = measure_config("c4", args, torch, device, link, 20, 1)
+        records["c4"]["position_in_run"] = "first"
+    records[head] = measure_config(head, args, torch, device, link, args.steps, args.warmup)
 
     def copy_engine_record(name, steps):
         # the same blocks through the copy-engine strategies (the library's choice among them)
@@ -1688,11 +1704,8 @@ def main():
             records[name + "_in_sequence"].pop("fragmented_record", None)
         print(json.dumps({"sequence": args.sequence, "configs": records}))
         return
-    for name in ("c0", "c2", "c3", "c4"):
-        # c4's latency percentiles want repetitions: 20 bursts of its 64 requests
-        records[name] = measure_config(name, args, torch, device, link,
-                                       20 if name == "c4" else args.other_steps,
-                                       1 if name == "c4" else 3)
+    for name in ("c0", "c2", "c3"):
+        records[name] = measure_config(name, args, torch, device, link, args.other_steps, 3)
         if name in ("c0", "c2") and not args.use_ce:
             records[name]["copy_engine"] = copy_engine_record(name, min(5, args.other_steps))
     records["c3_fragmented"] = records["c3"].pop("fragmented_record")

@@ -175,7 +175,9 @@ class Stats(Structure):
                 ("staging_bytes_device", c_uint64), ("staging_bytes_host", c_uint64),
                 ("confined_launches", c_uint64), ("safety_net_ranges", c_uint64),
                 ("staged_batches", c_uint64), ("gathered_batches", c_uint64),
-                ("gather_busy_us", c_uint64), ("second_stream_batches", c_uint64)]
+                ("gather_busy_us", c_uint64), ("second_stream_batches", c_uint64),
+                ("plan_slots", c_uint64), ("plan_slots_in_use", c_uint64),
+                ("plan_slot_waits", c_uint64)]
 
 
 class LaunchPolicy(Structure):
@@ -320,8 +322,8 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.fkv_abi_version() != 4:
-        raise ImportError(f"{LIB_PATH}: ABI version {lib.fkv_abi_version()} != 4")
+    if lib.fkv_abi_version() != 5:
+        raise ImportError(f"{LIB_PATH}: ABI version {lib.fkv_abi_version()} != 5")
     _lib = lib
     return lib
 

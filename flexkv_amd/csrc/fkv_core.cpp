@@ -265,6 +265,7 @@ PlanSlot *plan_acquire(int device, size_t bytes) {
     pick->busy = true;
   }
   if (pick->event_pending) {
+    stats().plan_slot_waits.fetch_add(1, std::memory_order_relaxed);
     (void)hipEventSynchronize(pick->done);
     pick->event_pending = false;
   }
@@ -817,6 +818,11 @@ void fkv_get_stats(fkv_stats *out) {
   out->staged_batches = s.staged_batches.load();
   out->gathered_batches = s.gathered_batches.load();
   out->second_stream_batches = s.second_stream_batches.load();
+  int slots = 0, in_use = 0;
+  fkv::plan_pool_counts(&slots, &in_use);
+  out->plan_slots = (uint64_t)slots;
+  out->plan_slots_in_use = (uint64_t)in_use;
+  out->plan_slot_waits = s.plan_slot_waits.load();
   out->gather_busy_us = s.gather_busy_ns.load() / 1000;
 }
 void fkv_reset_stats(void) {
@@ -832,6 +838,7 @@ void fkv_reset_stats(void) {
   s.staged_batches = 0;
   s.gathered_batches = 0;
   s.second_stream_batches = 0;
+  s.plan_slot_waits = 0;
   s.gather_busy_ns = 0;
 }
 

@@ -75,7 +75,8 @@ constexpr unsigned kTimingEventNoFence = hipEventDisableSystemFence;
 struct Stats {
   std::atomic<uint64_t> calls{0}, bytes_h2d{0}, bytes_d2h{0}, kernel_launches{0},
       dma_copies{0}, staging_bytes_device{0}, staging_bytes_host{0}, confined_launches{0},
-      staged_batches{0}, gathered_batches{0}, gather_busy_ns{0}, second_stream_batches{0};
+      staged_batches{0}, gathered_batches{0}, gather_busy_ns{0}, second_stream_batches{0},
+      plan_slot_waits{0};
 };
 Stats &stats();
 

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define FKV_ABI_VERSION 4 /* 4: fkv_stats grew by second_stream_batches; 3: fkv_stats grew by gathered_batches and gather_busy_us, fkv_launch_policy by the host-gather and link-seeding fields; 2: fkv_stats grew by staged_batches; launch policy, no-alloc transfer, staging and HBM-rate entry points added */
+#define FKV_ABI_VERSION 5 /* 5: fkv_stats grew by plan_slots, plan_slots_in_use and plan_slot_waits; 4: fkv_stats grew by second_stream_batches; 3: fkv_stats grew by gathered_batches and gather_busy_us, fkv_launch_policy by the host-gather and link-seeding fields; 2: fkv_stats grew by staged_batches; launch policy, no-alloc transfer, staging and HBM-rate entry points added */
 
 /* status codes */
 #define FKV_OK 0
@@ -589,6 +589,12 @@ typedef struct fkv_stats {
   uint64_t gather_busy_us;    /* time host threads spent gathering such rows, summed over threads */
   uint64_t second_stream_batches; /* layer batches of a layerwise restore by kernel that were launched
                                  on the group's second stream (kernel_alt_stream_kb of the policy) */
+  /* plan memory (the tables a launch reads: pinned slots with a device mirror, recycled behind
+   * events): slots the pool holds and slots in use right now (not reset by fkv_reset_stats),
+   * and how often a caller had to wait for the oldest user because the pool was at its limit */
+  uint64_t plan_slots;
+  uint64_t plan_slots_in_use;
+  uint64_t plan_slot_waits;
 } fkv_stats;
 void fkv_get_stats(fkv_stats *out);
 void fkv_reset_stats(void);
