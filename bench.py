@@ -399,7 +399,9 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=F
     # chain, or a streaming elementwise kernel.
     comp = torch.cuda.Stream()
     # the engine names its forward stream: the group's own streams keep off its hardware queue
+    t_name = time.perf_counter()
     sharing = grp.set_compute_stream(comp) if name_compute_stream else None
+    naming_ms = (time.perf_counter() - t_name) * 1e3
     ev = lambda: torch.cuda.Event(enable_timing=True)
     target_ms = layer_bytes / 55e9 * 1e3
     if dummy == "sdpa":
@@ -497,7 +499,7 @@ def run_layerwise(w, torch, steps, warmup, num_cta, notify, dummy, layer_spans=F
                 compute_reps_per_layer=reps, layer_bytes=layer_bytes,
                 restore_alone_ms=restore_alone_ms,
                 restore_alone_runs_ms=[round(x, 3) for x in alone],
-                group_streams_on_compute_queue=sharing)
+                group_streams_on_compute_queue=sharing, naming_ms=round(naming_ms, 1))
 
 
 def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, verify=True):
@@ -1252,6 +1254,7 @@ def overlap_record(r, B, link):
             "restore_alone_runs_ms": r.get("restore_alone_runs_ms"),
             # after fkv_layerwise_set_compute_stream; None: the compute stream was not named
             "group_streams_on_compute_queue": r.get("group_streams_on_compute_queue"),
+            "set_compute_stream_ms": r.get("naming_ms"),   # once, at set-up: the probes
             "compute_per_layer_ms": round(r["compute_ms"] / r["layers"], 3),
             "compute_units_per_layer": r["compute_reps_per_layer"],
             "exposed_ms": round(exposed, 3),

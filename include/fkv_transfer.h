@@ -429,8 +429,9 @@ int fkv_layerwise_wait_layer(fkv_layerwise *g, int32_t gpu_index, int32_t layer,
  * stream shares the queue of the engine's forward pass is therefore not hidden behind the
  * forward pass but added to it (61 layers of 36 MiB next to 0.6 ms of attention per layer:
  * 89 ms instead of 42).  The call swaps every stream the group uses on that GPU for one
- * that was seen to run next to `compute_stream` (two short timed launches per candidate,
- * about 3 ms each; up to 8 candidates per stream) and, where the queues allow, puts the
+ * that was seen to run next to `compute_stream` (eleven timed launches of 0.3 ms per pair of
+ * streams probed, up to 8 candidates per stream; 50 ms for the whole call on a device with
+ * four queues) and, where the queues allow, puts the
  * scatter stream and the two copy streams on queues of their own; `streams_sharing` (may be NULL)
  * receives how many of the group's streams still share the queue afterwards, 0 in the
  * normal case.  It waits for the group's previous restore and for `compute_stream`: call
