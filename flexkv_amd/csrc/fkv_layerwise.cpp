@@ -472,102 +472,102 @@ int launch_batches(fkv_layerwise *g, std::vector<Lane> &lanes, const EngineChoic
   }
   std::vector<char> alt_used(g->num_gpus, 0);
   try { // an exception ends the launches like an error: the plans below are given back either way
-  for (int b = 0; b < num_batches && rc == FKV_OK; ++b) {
-    if (give_up_at > 0 && b == give_up_at - 1) {
-      rc = fail(FKV_ERR_RUNTIME, "layerwise restore made to give up before batch %d (test_fail_restore_batch)", b);
-      break;
-    }
-    fkv_layerwise::Batch &batch = *g->batches[b];
-    for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
-      (void)hipSetDevice(g->device_ids[i]);
-      // the members of one batch that go by kernel go out together: up to kCopyMaxJobs per launch
-      const KernelPlan *plans[kCopyMaxJobs];
-      int first[kCopyMaxJobs], count[kCopyMaxJobs];
-      std::vector<const Item *> by_kernel, by_strategy;
-      auto account = [&](const Item &it) {
-        const Lane &lane = lanes[it.lane];
-        stats().calls.fetch_add(1, std::memory_order_relaxed);
-        stats().bytes_h2d.fetch_add((uint64_t)lane.num_blocks * it.layers * lane.kv_dim *
-                                        (uint64_t)lane.src->chunk_sizes[i],
-                                    std::memory_order_relaxed);
-      };
-      for (const Item &it : batch.items) {
+    for (int b = 0; b < num_batches && rc == FKV_OK; ++b) {
+      if (give_up_at > 0 && b == give_up_at - 1) {
+        rc = fail(FKV_ERR_RUNTIME, "layerwise restore made to give up before batch %d (test_fail_restore_batch)", b);
+        break;
+      }
+      fkv_layerwise::Batch &batch = *g->batches[b];
+      for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
+        (void)hipSetDevice(g->device_ids[i]);
+        // the members of one batch that go by kernel go out together: up to kCopyMaxJobs per launch
+        const KernelPlan *plans[kCopyMaxJobs];
+        int first[kCopyMaxJobs], count[kCopyMaxJobs];
+        std::vector<const Item *> by_kernel, by_strategy;
+        auto account = [&](const Item &it) {
+          const Lane &lane = lanes[it.lane];
+          stats().calls.fetch_add(1, std::memory_order_relaxed);
+          stats().bytes_h2d.fetch_add((uint64_t)lane.num_blocks * it.layers * lane.kv_dim *
+                                          (uint64_t)lane.src->chunk_sizes[i],
+                                      std::memory_order_relaxed);
+        };
+        for (const Item &it : batch.items) {
+          if (rc != FKV_OK)
+            break;
+          Lane &lane = lanes[it.lane];
+          const StagedPlan *sp =
+              i < (int)lane.staged.size() && lane.staged[i].usable ? &lane.staged[i] : nullptr;
+          if (!sp || (b == 0 && sp->first_by_kernel)) {
+            (direct ? by_kernel : by_strategy).push_back(&it);
+            continue;
+          }
+          // gathered batches are enqueued one by one as their rows become ready: nothing to hide
+          // there, and next to other work of the process the second stream cost 1 % (c3 with
+          // scattered host blocks behind c3 in one process: 42.3 ms against 41.9 ms)
+          const bool second = two_dma_streams[i] && g->dma_streams2[i] && sp->route == kRouteRuns &&
+                              (g->dma_turn[i]++ & 1u);
+          const hipStream_t dma = second ? g->dma_streams2[i] : g->dma_streams[i];
+          if (sp->route == kRouteGathered)
+            rc = gathered_launch(*sp, g->rings[{it.lane, i}], g->pinned_rings[{it.lane, i}],
+                                 *g->crew, lane.plans[i], it.start_layer, it.layers, dma,
+                                 g->streams[i]);
+          else
+            rc = staged_launch(*sp, g->rings[{it.lane, i}], lane.plans[i], it.start_layer, it.layers,
+                               dma, g->streams[i]);
+          if (rc == FKV_OK)
+            account(it);
+        }
+        // a small batch that goes by kernel as a whole: every other one on the second stream,
+        // from the third on (the first one has the link to itself and lands as early as it can)
+        hipStream_t batch_stream = g->streams[i];
+        if (alt_max_bytes[i] > 0 && b >= 2 && !(b & 1) && !by_kernel.empty() &&
+            by_kernel.size() == batch.items.size()) {
+          int64_t bytes = 0;
+          for (const Item *it : by_kernel) {
+            const Lane &lane = lanes[it->lane];
+            bytes += (int64_t)lane.num_blocks * it->layers * lane.kv_dim * lane.src->chunk_sizes[i];
+          }
+          // the second stream starts behind the first batch, which is behind the plan uploads
+          if (bytes <= alt_max_bytes[i] &&
+              (alt_used[i] ||
+               hipStreamWaitEvent(g->alt_streams[i], g->batches[0]->done[i], 0) == hipSuccess)) {
+            batch_stream = g->alt_streams[i];
+            alt_used[i] = 1;
+            stats().second_stream_batches.fetch_add(1, std::memory_order_relaxed);
+          } else {
+            (void)hipGetLastError();
+          }
+        }
+        for (size_t k = 0; k < by_kernel.size() && rc == FKV_OK; k += kCopyMaxJobs) {
+          const int n = (int)std::min<size_t>(kCopyMaxJobs, by_kernel.size() - k);
+          for (int j = 0; j < n; ++j) {
+            const Item &it = *by_kernel[k + j];
+            plans[j] = &lanes[it.lane].plans[i];
+            first[j] = it.start_layer;
+            count[j] = it.layers;
+          }
+          rc = kernel_plans_launch(plans, first, count, n, batch_stream);
+          for (int j = 0; j < n && rc == FKV_OK; ++j)
+            account(*by_kernel[k + j]);
+        }
+        for (size_t k = 0; k < by_strategy.size() && rc == FKV_OK; ++k) {
+          const Item &it = *by_strategy[k];
+          fkv_transfer_desc d = describe(g, lanes[it.lane], i, it.start_layer, it.layers, choice);
+          rc = fkv_transfer_kv_blocks(&d, g->streams[i]); // does its own accounting
+          (void)hipSetDevice(g->device_ids[i]);
+        }
         if (rc != FKV_OK)
           break;
-        Lane &lane = lanes[it.lane];
-        const StagedPlan *sp =
-            i < (int)lane.staged.size() && lane.staged[i].usable ? &lane.staged[i] : nullptr;
-        if (!sp || (b == 0 && sp->first_by_kernel)) {
-          (direct ? by_kernel : by_strategy).push_back(&it);
-          continue;
-        }
-        // gathered batches are enqueued one by one as their rows become ready: nothing to hide
-        // there, and next to other work of the process the second stream cost 1 % (c3 with
-        // scattered host blocks behind c3 in one process: 42.3 ms against 41.9 ms)
-        const bool second = two_dma_streams[i] && g->dma_streams2[i] && sp->route == kRouteRuns &&
-                            (g->dma_turn[i]++ & 1u);
-        const hipStream_t dma = second ? g->dma_streams2[i] : g->dma_streams[i];
-        if (sp->route == kRouteGathered)
-          rc = gathered_launch(*sp, g->rings[{it.lane, i}], g->pinned_rings[{it.lane, i}],
-                               *g->crew, lane.plans[i], it.start_layer, it.layers, dma,
-                               g->streams[i]);
-        else
-          rc = staged_launch(*sp, g->rings[{it.lane, i}], lane.plans[i], it.start_layer, it.layers,
-                             dma, g->streams[i]);
-        if (rc == FKV_OK)
-          account(it);
-      }
-      // a small batch that goes by kernel as a whole: every other one on the second stream,
-      // from the third on (the first one has the link to itself and lands as early as it can)
-      hipStream_t batch_stream = g->streams[i];
-      if (alt_max_bytes[i] > 0 && b >= 2 && !(b & 1) && !by_kernel.empty() &&
-          by_kernel.size() == batch.items.size()) {
-        int64_t bytes = 0;
-        for (const Item *it : by_kernel) {
-          const Lane &lane = lanes[it->lane];
-          bytes += (int64_t)lane.num_blocks * it->layers * lane.kv_dim * lane.src->chunk_sizes[i];
-        }
-        // the second stream starts behind the first batch, which is behind the plan uploads
-        if (bytes <= alt_max_bytes[i] &&
-            (alt_used[i] ||
-             hipStreamWaitEvent(g->alt_streams[i], g->batches[0]->done[i], 0) == hipSuccess)) {
-          batch_stream = g->alt_streams[i];
-          alt_used[i] = 1;
-          stats().second_stream_batches.fetch_add(1, std::memory_order_relaxed);
-        } else {
+        hipError_t e = hipEventRecord(batch.done[i], batch_stream);
+        if (e != hipSuccess) {
           (void)hipGetLastError();
+          rc = fail(FKV_ERR_RUNTIME, "layerwise_transfer failed on GPU %d: %s", i,
+                    hipGetErrorString(e));
         }
       }
-      for (size_t k = 0; k < by_kernel.size() && rc == FKV_OK; k += kCopyMaxJobs) {
-        const int n = (int)std::min<size_t>(kCopyMaxJobs, by_kernel.size() - k);
-        for (int j = 0; j < n; ++j) {
-          const Item &it = *by_kernel[k + j];
-          plans[j] = &lanes[it.lane].plans[i];
-          first[j] = it.start_layer;
-          count[j] = it.layers;
-        }
-        rc = kernel_plans_launch(plans, first, count, n, batch_stream);
-        for (int j = 0; j < n && rc == FKV_OK; ++j)
-          account(*by_kernel[k + j]);
-      }
-      for (size_t k = 0; k < by_strategy.size() && rc == FKV_OK; ++k) {
-        const Item &it = *by_strategy[k];
-        fkv_transfer_desc d = describe(g, lanes[it.lane], i, it.start_layer, it.layers, choice);
-        rc = fkv_transfer_kv_blocks(&d, g->streams[i]); // does its own accounting
-        (void)hipSetDevice(g->device_ids[i]);
-      }
-      if (rc != FKV_OK)
-        break;
-      hipError_t e = hipEventRecord(batch.done[i], batch_stream);
-      if (e != hipSuccess) {
-        (void)hipGetLastError();
-        rc = fail(FKV_ERR_RUNTIME, "layerwise_transfer failed on GPU %d: %s", i,
-                  hipGetErrorString(e));
-      }
+      if (rc == FKV_OK)
+        g->gate.publish(b + 1);
     }
-    if (rc == FKV_OK)
-      g->gate.publish(b + 1);
-  }
   } catch (...) {
     rc = caught("launches of a layerwise restore");
   }
@@ -941,58 +941,58 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
   const EngineChoice choice{c.use_ce_transfer, c.transfer_cta_num};
   const bool direct = choice.use_ce_transfer == 0;
   try { // an exception part-way ends the call like an error: launch_batches gives back what was built
-  for (Lane &lane : lanes) {
-    if (!lane.used || rc != FKV_OK)
-      continue;
-    lane.plans.resize(g->num_gpus);
-    lane.staged.resize(g->num_gpus);
-    const int layers = g->multi_group || lane.src != &g->groups[0] ? lane.src->num_layers
-                                                                   : c.num_layers;
-    const int lane_index = (int)(&lane - lanes.data());
-    for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
-      fkv_transfer_desc d = describe(g, lane, i, 0, layers, choice);
-      rc = validate(d);
-      if (rc != FKV_OK)
-        break;
-      (void)hipSetDevice(g->device_ids[i]);
-      // A host pool the device cannot read (ordinary pageable memory) still serves a
-      // restore whose rows host threads gather; only the kernel path itself needs more.
-      rc = kernel_plan_build(d, g->streams[i], &lane.plans[i], /*host_optional=*/true);
-      if (rc != FKV_OK) {
-        if (direct)
-          break;
-        clear_error(); // the copy-engine strategies need no plan
-        rc = FKV_OK;
+    for (Lane &lane : lanes) {
+      if (!lane.used || rc != FKV_OK)
         continue;
-      }
-      rc = staged_plan_build(d, g->multi_group ? 1 : c.layer_granularity,
-                             g->rings[{lane_index, i}], g->pinned_rings[{lane_index, i}],
-                             g->streams[i], &lane.staged[i], lane.plans[i].host_visible,
-                             /*kernel_allowed=*/direct, /*several_gpus=*/g->num_gpus > 1);
-      if (rc == FKV_OK && lane.staged[i].usable && !g->dma_streams[i]) {
-        hipError_t e = pooled_stream_acquire(g->device_ids[i], true, &g->dma_streams[i]);
-        if (e != hipSuccess) {
-          (void)hipGetLastError();
-          g->dma_streams[i] = nullptr;
-          staged_plan_release(&lane.staged[i], g->streams[i]); // kernel path then
-        } else if (pooled_stream_acquire(g->device_ids[i], true, &g->dma_streams2[i]) !=
-                   hipSuccess) {
-          (void)hipGetLastError();
-          g->dma_streams2[i] = nullptr; // all copies on the first then
+      lane.plans.resize(g->num_gpus);
+      lane.staged.resize(g->num_gpus);
+      const int layers = g->multi_group || lane.src != &g->groups[0] ? lane.src->num_layers
+                                                                     : c.num_layers;
+      const int lane_index = (int)(&lane - lanes.data());
+      for (int i = 0; i < g->num_gpus && rc == FKV_OK; ++i) {
+        fkv_transfer_desc d = describe(g, lane, i, 0, layers, choice);
+        rc = validate(d);
+        if (rc != FKV_OK)
+          break;
+        (void)hipSetDevice(g->device_ids[i]);
+        // A host pool the device cannot read (ordinary pageable memory) still serves a
+        // restore whose rows host threads gather; only the kernel path itself needs more.
+        rc = kernel_plan_build(d, g->streams[i], &lane.plans[i], /*host_optional=*/true);
+        if (rc != FKV_OK) {
+          if (direct)
+            break;
+          clear_error(); // the copy-engine strategies need no plan
+          rc = FKV_OK;
+          continue;
+        }
+        rc = staged_plan_build(d, g->multi_group ? 1 : c.layer_granularity,
+                               g->rings[{lane_index, i}], g->pinned_rings[{lane_index, i}],
+                               g->streams[i], &lane.staged[i], lane.plans[i].host_visible,
+                               /*kernel_allowed=*/direct, /*several_gpus=*/g->num_gpus > 1);
+        if (rc == FKV_OK && lane.staged[i].usable && !g->dma_streams[i]) {
+          hipError_t e = pooled_stream_acquire(g->device_ids[i], true, &g->dma_streams[i]);
+          if (e != hipSuccess) {
+            (void)hipGetLastError();
+            g->dma_streams[i] = nullptr;
+            staged_plan_release(&lane.staged[i], g->streams[i]); // kernel path then
+          } else if (pooled_stream_acquire(g->device_ids[i], true, &g->dma_streams2[i]) !=
+                     hipSuccess) {
+            (void)hipGetLastError();
+            g->dma_streams2[i] = nullptr; // all copies on the first then
+          }
+        }
+        if (rc == FKV_OK && !lane.staged[i].usable) {
+          if (!direct) // the strategies of the copy-engine path take it from here
+            kernel_plan_release(&lane.plans[i], g->streams[i]);
+          else if (!lane.plans[i].host_visible)
+            rc = fail(FKV_ERR_INVALID_ARG,
+                      "cpu_tensor at %p is not device-visible (allocate it pinned or register it "
+                      "before a kernel transfer), and the restore cannot go through gathered rows "
+                      "either (staged_gather of the launch policy, batch size)",
+                      d.cpu_ptr);
         }
       }
-      if (rc == FKV_OK && !lane.staged[i].usable) {
-        if (!direct) // the strategies of the copy-engine path take it from here
-          kernel_plan_release(&lane.plans[i], g->streams[i]);
-        else if (!lane.plans[i].host_visible)
-          rc = fail(FKV_ERR_INVALID_ARG,
-                    "cpu_tensor at %p is not device-visible (allocate it pinned or register it "
-                    "before a kernel transfer), and the restore cannot go through gathered rows "
-                    "either (staged_gather of the launch policy, batch size)",
-                    d.cpu_ptr);
-      }
     }
-  }
   } catch (...) {
     rc = caught("plans of a layerwise restore");
   }
