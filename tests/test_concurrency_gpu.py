@@ -48,6 +48,10 @@ def test_random_transfers_from_six_threads(gpu_device, chunk):
     assert not errors, errors
     assert min(counts) > 5, counts
     dev.assert_matches_reference(f"{sum(counts)} concurrent transfers, chunk {chunk}")
+    # every plan went back to the pool, and the pool never made a request wait for a slot
+    from flexkv_amd.c_ext import get_stats
+    st = get_stats()
+    assert st["plan_slots"] > 0 and st["plan_slots_in_use"] == 0, st
 
 
 
