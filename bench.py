@@ -1489,10 +1489,8 @@ def main():
 
     # Hardware queues of the process: the runtime reads this when it starts.  HIP's default is
     # 4, the reference's platform gives a process 8 (CUDA_DEVICE_MAX_CONNECTIONS).  c4 reaches
-    # the same 93 GB/s with 2, 4, 8 and 16; a layerwise restore next to compute wants the
-    # default (c3: 42 ms with 4; with 8, 52 ms in every second or third run, although no
-    # stream of the restore shares the compute stream's queue).  Left as the environment has
-    # it unless asked for.
+    # the same 93 GB/s with 2, 4, 8 and 16, c3 its 42 ms with 4 and 8 once the group knows the
+    # compute stream.  Left as the environment has it unless asked for.
     if args.hw_queues > 0:
         os.environ["GPU_MAX_HW_QUEUES"] = str(args.hw_queues)
     import torch

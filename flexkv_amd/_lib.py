@@ -271,6 +271,7 @@ SIGNATURES = {
     "fkv_ssd_close": (None, [c_void_p]),
     "fkv_layout_transform": (c_int32, [POINTER(LayoutTransformDesc), c_void_p]),
     "fkv_streams_run_concurrently": (c_int32, [c_int32, c_void_p, c_void_p, POINTER(c_int32)]),
+    "fkv_streams_hand_over_us": (c_int32, [c_int32, c_void_p, c_void_p, POINTER(ctypes.c_double)]),
     "fkv_link_activity_post": (c_int32, [c_int32, c_int32, c_int64]),
     "fkv_link_activity_elsewhere": (c_int32, [c_int32, c_int32, c_int32, POINTER(c_int32)]),
     "fkv_range_push": (c_int32, [c_char_p]),

@@ -334,6 +334,15 @@ def streams_run_concurrently(stream_a, stream_b, device: int = -1) -> bool:
     return bool(out.value)
 
 
+def streams_hand_over_us(stream_a, stream_b, device: int = -1) -> float:
+    """Microseconds an event takes from one torch stream to the other and back on the
+    device (a chain of waits enqueued ahead of time).  Synchronises both."""
+    out = ctypes.c_double(0.0)
+    check(_L.fkv_streams_hand_over_us(int(device), ctypes.c_void_p(stream_a.cuda_stream),
+                                      ctypes.c_void_p(stream_b.cuda_stream), ctypes.byref(out)))
+    return float(out.value)
+
+
 def link_activity_post(is_host_to_device: bool, expected_us: int, device: int = -1) -> None:
     """Tell the other processes that use this GPU that this one keeps the host link
     busy in one direction for about `expected_us` more.  The library posts its own

@@ -873,3 +873,73 @@ extern "C" int fkv_streams_run_concurrently(int32_t device, void *stream_a, void
 } catch (...) {
   return fkv::caught(__func__);
 }
+
+extern "C" int fkv_streams_hand_over_us(int32_t device, void *stream_a, void *stream_b,
+                                        double *round_trip_us) try {
+  using namespace fkv;
+  clear_error();
+  if (!round_trip_us)
+    return fail(FKV_ERR_INVALID_ARG, "fkv_streams_hand_over_us: null result pointer");
+  DeviceGuard guard(device);
+  if (!guard.ok())
+    return fail(FKV_ERR_RUNTIME, "cannot select HIP device %d", device);
+  hipStream_t a = static_cast<hipStream_t>(stream_a), b = static_cast<hipStream_t>(stream_b);
+  constexpr int kRoundTrips = 16;
+  constexpr long long kGateTicks = 200000; // 2 ms: the whole chain is enqueued before it may start
+  hipEvent_t t0 = nullptr, t1 = nullptr, there[kRoundTrips] = {}, back[kRoundTrips] = {};
+  auto cleanup = [&] {
+    for (hipEvent_t e : {t0, t1})
+      if (e)
+        (void)hipEventDestroy(e);
+    for (int k = 0; k < kRoundTrips; ++k)
+      for (hipEvent_t e : {there[k], back[k]})
+        if (e)
+          (void)hipEventDestroy(e);
+  };
+#define HO_TRY(expr)                                                                      \
+  do {                                                                                    \
+    hipError_t e_ = (expr);                                                               \
+    if (e_ != hipSuccess) {                                                               \
+      (void)hipStreamSynchronize(a);                                                      \
+      (void)hipStreamSynchronize(b);                                                      \
+      cleanup();                                                                          \
+      (void)hipGetLastError();                                                            \
+      return fail(FKV_ERR_RUNTIME, "fkv_streams_hand_over_us: %s", hipGetErrorString(e_)); \
+    }                                                                                     \
+  } while (0)
+  HO_TRY(hipEventCreate(&t0));
+  HO_TRY(hipEventCreate(&t1));
+  for (int k = 0; k < kRoundTrips; ++k) {
+    HO_TRY(hipEventCreateWithFlags(&there[k], kBookkeepingEvent));
+    HO_TRY(hipEventCreateWithFlags(&back[k], kBookkeepingEvent));
+  }
+  double best = 1e30;
+  for (int rep = 0; rep < 2; ++rep) { // the first one carries whatever is set up on first use
+    HO_TRY(hipStreamSynchronize(a));
+    HO_TRY(hipStreamSynchronize(b));
+    hipLaunchKernelGGL(fkv_wait_kernel, dim3(1), dim3(64), 0, a, kGateTicks, nullptr);
+    HO_TRY(hipGetLastError());
+    HO_TRY(hipEventRecord(t0, a));
+    for (int k = 0; k < kRoundTrips; ++k) {
+      hipLaunchKernelGGL(fkv_wait_kernel, dim3(1), dim3(64), 0, a, 0ll, nullptr);
+      HO_TRY(hipEventRecord(there[k], a));
+      HO_TRY(hipStreamWaitEvent(b, there[k], 0));
+      hipLaunchKernelGGL(fkv_wait_kernel, dim3(1), dim3(64), 0, b, 0ll, nullptr);
+      HO_TRY(hipEventRecord(back[k], b));
+      HO_TRY(hipStreamWaitEvent(a, back[k], 0));
+    }
+    HO_TRY(hipGetLastError());
+    HO_TRY(hipEventRecord(t1, a));
+    HO_TRY(hipEventSynchronize(t1));
+    HO_TRY(hipStreamSynchronize(b));
+    float ms = 0;
+    HO_TRY(hipEventElapsedTime(&ms, t0, t1));
+    best = std::min(best, (double)ms * 1e3 / kRoundTrips);
+  }
+#undef HO_TRY
+  cleanup();
+  *round_trip_us = best;
+  return FKV_OK;
+} catch (...) {
+  return fkv::caught(__func__);
+}

@@ -1240,17 +1240,36 @@ int fkv_layerwise_set_compute_stream(fkv_layerwise *g, int32_t gpu_index, void *
                       {&g->dma_streams[i], {&g->streams[i]}},
                       {&g->dma_streams2[i], {&g->streams[i], &g->dma_streams[i]}},
                       {&g->alt_streams[i], {&g->streams[i]}}};
-  // 2: next to the engine's stream and to those of ours it should be apart from,
-  // 1: next to the engine's stream only, 0: shares the engine's queue
-  auto rank_of = [&](hipStream_t candidate, const Own &o, int *rank) -> int {
+  // Two streams go together when their kernels run at the same time and an event gets from
+  // one to the other and back about as fast as from a stream to itself: with more than four
+  // hardware queues some pairs pass the first test and take four times as long for the
+  // second, and a restore hands an event over per layer (61 layers next to compute: 52 ms
+  // instead of 42).
+  double own_round_trip_us = 0;
+  FKV_TRY(fkv_streams_hand_over_us(device, compute, compute, &own_round_trip_us));
+  const double slow_us = 2 * own_round_trip_us + 10;
+  auto go_together = [&](hipStream_t x, hipStream_t y, bool *yes) -> int {
     int32_t concurrent = 0;
-    FKV_TRY(fkv_streams_run_concurrently(device, compute, candidate, &concurrent));
-    *rank = concurrent ? 2 : 0;
+    FKV_TRY(fkv_streams_run_concurrently(device, x, y, &concurrent));
+    *yes = concurrent != 0;
+    if (*yes) {
+      double us = 0;
+      FKV_TRY(fkv_streams_hand_over_us(device, x, y, &us));
+      *yes = us < slow_us;
+    }
+    return FKV_OK;
+  };
+  // 2: goes together with the engine's stream and with those of ours it should be apart
+  // from, 1: with the engine's stream only, 0: shares the engine's queue or hardware
+  auto rank_of = [&](hipStream_t candidate, const Own &o, int *rank) -> int {
+    bool yes = false;
+    FKV_TRY(go_together(compute, candidate, &yes));
+    *rank = yes ? 2 : 0;
     for (hipStream_t *other : o.apart_from) {
       if (*rank != 2 || !*other)
         break;
-      FKV_TRY(fkv_streams_run_concurrently(device, *other, candidate, &concurrent));
-      if (!concurrent)
+      FKV_TRY(go_together(*other, candidate, &yes));
+      if (!yes)
         *rank = 1;
     }
     return FKV_OK;

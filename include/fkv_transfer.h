@@ -429,9 +429,10 @@ int fkv_layerwise_wait_layer(fkv_layerwise *g, int32_t gpu_index, int32_t layer,
  * stream shares the queue of the engine's forward pass is therefore not hidden behind the
  * forward pass but added to it (61 layers of 36 MiB next to 0.6 ms of attention per layer:
  * 89 ms instead of 42).  The call swaps every stream the group uses on that GPU for one
- * that was seen to run next to `compute_stream` (eleven timed launches of 0.3 ms per pair of
- * streams probed, up to 8 candidates per stream; 50 ms for the whole call on a device with
- * four queues) and, where the queues allow, puts the
+ * that was seen to run next to `compute_stream` and to exchange events with it at the normal
+ * latency (fkv_streams_run_concurrently and fkv_streams_hand_over_us per pair of streams
+ * probed, up to 8 candidates per stream; 100 ms for the whole call on a device with four
+ * queues) and, where the queues allow, puts the
  * scatter stream and the two copy streams on queues of their own; `streams_sharing` (may be NULL)
  * receives how many of the group's streams still share the queue afterwards, 0 in the
  * normal case.  It waits for the group's previous restore and for `compute_stream`: call
@@ -867,6 +868,15 @@ int fkv_range_pop(void);
  * than 1.5x the single one.  No counterpart in the reference. */
 int fkv_streams_run_concurrently(int32_t device, void *stream_a, void *stream_b,
                                  int32_t *concurrent);
+/* How long an event takes from one stream to another and back on the device: a chain of 16
+ * round trips (tiny kernel, record, wait on the other stream, tiny kernel, record, wait) is
+ * enqueued behind a 2 ms gate kernel and timed with events; *round_trip_us is the time per
+ * round trip, the better of two runs.  Streams on different hardware queues normally take
+ * 27 us; with more than four queues some pairs take 120 us although their kernels run at the
+ * same time (they share hardware further down), and a restore that hands an event to the
+ * engine's stream per layer loses that time per layer.  Synchronises both streams.  No
+ * counterpart in the reference. */
+int fkv_streams_hand_over_us(int32_t device, void *stream_a, void *stream_b, double *round_trip_us);
 
 /* Link activity across processes.  A put and a get that run at the same time are
  * kept on different XCDs; so that this also works when they come from different

@@ -755,6 +755,12 @@ int fkv_streams_run_concurrently(int32_t, void *a, void *b, int32_t *concurrent)
                 of(static_cast<hipStream_t>(b))->hardware_queue;
   return FKV_OK;
 }
+int fkv_streams_hand_over_us(int32_t, void *, void *, double *round_trip_us) {
+  if (!round_trip_us)
+    return fkv::fail(FKV_ERR_INVALID_ARG, "fkv_streams_hand_over_us: null result pointer");
+  *round_trip_us = 25.0; // every pair of the emulated device hands over alike
+  return FKV_OK;
+}
 #ifndef FKV_KERNELS_FROM_SOURCE
 int fkv_transfer_kv_blocks_noalloc(const fkv_transfer_desc *, void *) {
   return fkv::fail(FKV_ERR_UNSUPPORTED, "emulated runtime: the entry point lives beside the kernels");

@@ -99,9 +99,10 @@ def kernel_source_as_cpp(name, where):
                 "uint64_t *lds = static_cast<uint64_t *>(cpu_device_model::dynamic_lds());", 2)
         rewrite('asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(v));',
                 "v = cpu_device_model::xcc_id();", 1)
-        # the two entry points that time the device keep their stand-ins
+        # the three entry points that time the device keep their stand-ins
         rewrite("int fkv_streams_run_concurrently(", "int fkv_streams_run_concurrently_timed(", 1)
         rewrite("int fkv_measure_hbm_rate(", "int fkv_measure_hbm_rate_timed(", 1)
+        rewrite("int fkv_streams_hand_over_us(", "int fkv_streams_hand_over_us_timed(", 1)
     path = os.path.join(where, name + ".cpp")
     with open(path, "w") as f:
         f.write(text)
