@@ -290,6 +290,28 @@ def test_streams_run_concurrently_tells_hardware_queue_sharing(gpu_device):
     assert all(not table[i][i] for i in range(6))
 
 
+def test_streams_hand_over_us_times_an_event_chain_on_the_device(gpu_device):
+    """The round trip of an event between two streams, timed on the device: a stream with
+    itself gives the floor, another stream is at least as slow and (on different hardware
+    queues of a device with four of them) within a few times the floor; the streams are left
+    idle and usable.  Which pairs are slow is a property of the box: printed, not asserted."""
+    import torch
+    from flexkv_amd.c_ext import streams_hand_over_us
+    streams = [torch.cuda.Stream() for _ in range(5)]
+    floor = streams_hand_over_us(streams[0], streams[0])
+    assert 1.0 < floor < 500.0, floor
+    pairs = [streams_hand_over_us(streams[0], b) for b in streams[1:]]
+    print("event round trips in microseconds: same stream %.1f, others" % floor,
+          [round(p, 1) for p in pairs])
+    assert all(0.5 * floor < p < 2000.0 for p in pairs), (floor, pairs)
+    x = torch.zeros(8, device=gpu_device)
+    for s in streams:
+        with torch.cuda.stream(s):
+            x.add_(1)
+    torch.cuda.synchronize()
+    assert float(x[0]) == 5.0
+
+
 def test_a_put_in_another_process_confines_the_gets_of_this_one(gpu_device):
     """Two processes on one GPU: a child keeps posting puts, and the gets of this
     process (too small to keep to home XCDs by themselves) confine themselves
