@@ -194,7 +194,7 @@ def test_native_consumers_over_an_emulated_runtime_under_sanitizers(tmp_path, sa
     native = os.path.join(ROOT, "tests", "native")
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:verify_asan_link_order=0",
                TSAN_OPTIONS="halt_on_error=1", TMPDIR=str(tmp_path))
-    for source, args, expect in (("abi_roundtrip_driver.cpp", [], "ok: 33 cases through the C ABI"),
+    for source, args, expect in (("abi_roundtrip_driver.cpp", [], "ok: 34 cases through the C ABI"),
                                  ("two_way_driver.cpp", ["0.3", "8"], "ok: puts alone")):
         sub = tmp_path / source[:-4]
         sub.mkdir()
@@ -215,7 +215,7 @@ def test_kernel_sources_on_a_cpu_device_model_under_sanitizers(tmp_path, sanitiz
     jobs in one launch, fixed shares, claimed ranges, launches confined to some XCDs and their
     safety net), ThreadSanitizer the order among work-items; the launch shaping, the plan
     upload, the entry point that allocates nothing and the compressed-staging kernels run as
-    shipped (35 cases of the ABI driver instead of 33)."""
+    shipped (36 cases of the ABI driver instead of 34)."""
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:verify_asan_link_order=0",
                TSAN_OPTIONS="halt_on_error=1", TMPDIR=str(tmp_path))
     sub = tmp_path / "restores"
@@ -233,7 +233,7 @@ def test_kernel_sources_on_a_cpu_device_model_under_sanitizers(tmp_path, sanitiz
         defines=("-DFKV_EMULATED_RUNTIME", "-DFKV_KERNELS_FROM_SOURCE"), kernels_from_source=True)
     r = subprocess.run([exe], capture_output=True, text=True, env=env, timeout=900)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
-    assert "ok: 35 cases through the C ABI" in r.stdout, r.stdout[-2000:]
+    assert "ok: 36 cases through the C ABI" in r.stdout, r.stdout[-2000:]
 
 
 @pytest.mark.parametrize("sanitizer,launches", [(SANITIZERS[0].values[0], 40),

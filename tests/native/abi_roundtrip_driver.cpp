@@ -334,6 +334,50 @@ int main() {
       }
     FKV_OK_OR_DIE(fkv_launch_policy_reset(-1));
     ++cases;
+    // an engine in the same process: it names the stream of its forward pass once, then gates
+    // every layer's work on that stream with fkv_layerwise_wait_layer
+    {
+      hipStream_t forward = nullptr;
+      HIP_OK(hipStreamCreateWithFlags(&forward, hipStreamNonBlocking));
+      int32_t sharing = -1;
+      double round_trip_us = -1;
+      FKV_OK_OR_DIE(fkv_layerwise_set_compute_stream(lw, 0, forward, &sharing));
+      FKV_OK_OR_DIE(fkv_streams_hand_over_us(-1, forward, stream, &round_trip_us));
+      if (sharing != 0 || round_trip_us <= 0 ||
+          fkv_layerwise_set_compute_stream(lw, 1, forward, nullptr) == FKV_OK ||
+          fkv_layerwise_set_compute_stream(nullptr, 0, forward, nullptr) == FKV_OK) {
+        fprintf(stderr, "set_compute_stream: %d streams share the queue, round trip %.1f us\n", sharing,
+                round_trip_us);
+        return 1;
+      }
+      std::vector<int64_t> g = pick(rng, N, 27), c = pick(rng, NH, 27);
+      FKV_OK_OR_DIE(fkv_layerwise_transfer(lw, g.data(), c.data(), 27, CBS, CKS, CLS, CBS, 4, 0, L, 1,
+                                           KV, 8, 0, "sharded", 0, 0));
+      std::vector<std::vector<uint8_t>> seen(L, std::vector<uint8_t>((size_t)KV * GKS));
+      for (int l = 0; l < L; ++l) { // layer l as the forward stream sees it once it may go on
+        FKV_OK_OR_DIE(fkv_layerwise_wait_layer(lw, 0, l, forward));
+        HIP_OK(hipMemcpyAsync(seen[l].data(), dev[l], seen[l].size(), hipMemcpyDeviceToHost, forward));
+      }
+      HIP_OK(hipStreamSynchronize(forward));
+      FKV_OK_OR_DIE(fkv_layerwise_synchronize(lw));
+      m.put(g, c, true);
+      for (int l = 0; l < L; ++l)
+        if (memcmp(seen[l].data(), m.gpu[l].data(), seen[l].size()) != 0) {
+          fprintf(stderr, "layer %d was not whole when the forward stream went on\n", l);
+          return 1;
+        }
+      if (check("layerwise restore next to a named forward stream"))
+        return 1;
+      for (int l = 0; l < L; ++l) {
+        uint64_t v = 0;
+        if (read(fds[l], &v, 8) != 8 || v != 1) {
+          fprintf(stderr, "named forward stream: layer %d was not announced\n", l);
+          return 1;
+        }
+      }
+      HIP_OK(hipStreamDestroy(forward));
+      ++cases;
+    }
     fkv_layerwise_destroy(lw);
     for (int fd : fds)
       close(fd);

@@ -16,7 +16,7 @@ def test_native_consumer_of_the_c_abi(gpu_device):
     assert os.path.exists(exe), f"{exe} is missing: run make -C tests/native"
     r = subprocess.run([exe], capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-6000:]
-    assert "ok: 35 cases through the C ABI" in r.stdout, r.stdout
+    assert "ok: 36 cases through the C ABI" in r.stdout, r.stdout
 
 
 def test_two_threads_of_a_native_program_put_and_get_at_once(gpu_device):
