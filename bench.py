@@ -1482,6 +1482,14 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     args = ap.parse_args()
+    if args.sequence:
+        known = {"c0", "c1", "c2", "c3", "c4"}
+        bad = [n for n in args.sequence.split(",")
+               if (n[:-3] if n.endswith("+ce") else n) not in known
+               or (n.endswith("+ce") and n[:-3] not in ("c0", "c1", "c2"))]
+        if bad:
+            ap.error("--sequence: unknown configuration(s) %s (c0..c4, and c0+ce, c1+ce, c2+ce)"
+                     % ", ".join(bad))
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the transfer path crosses one host "
               "link per GPU and has no cross-GPU step); run with --gpus 1", file=sys.stderr)
