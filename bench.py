@@ -536,7 +536,9 @@ def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, v
                         rows.index_fill_(0, idx, 0)
         torch.cuda.synchronize()
 
-    def worker(i, barrier, record):
+    starts = []     # per timed burst: when each request thread got to its call, sorted
+
+    def worker(i, barrier, record, began):
         gi, ci = reqs[i]
         with torch.cuda.stream(streams[i]):
             barrier.wait()
@@ -544,10 +546,12 @@ def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, v
             w.transfer(gi, ci, h2d=(i % 2 == 1), transfer_num_cta=num_cta, sync=True)
             if record:
                 lat[i].append((time.perf_counter() - t0) * 1e3)
+            began[i] = t0
 
     for it in range(warmup + steps):
         barrier = threading.Barrier(len(reqs) + 1)
-        threads = [threading.Thread(target=worker, args=(i, barrier, it >= warmup))
+        began = [0.0] * len(reqs)
+        threads = [threading.Thread(target=worker, args=(i, barrier, it >= warmup, began))
                    for i in range(len(reqs))]
         for th in threads:
             th.start()
@@ -558,6 +562,7 @@ def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, v
             th.join()
         if it >= warmup:
             walls.append(time.perf_counter() - t0)
+            starts.append(sorted((b - t0) * 1e3 for b in began))
     all_lat = sorted(x for l in lat for x in l)
     p99 = all_lat[min(len(all_lat) - 1, int(0.99 * len(all_lat)))]
     total_bytes = sum(int(g.numel()) for g, _ in reqs) * w.L * w.kv_dim * w.chunk
@@ -574,7 +579,13 @@ def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, v
                 blocks=[int(g.numel()) for g, _ in reqs], bit_exact=ok,
                 # slots of the library's plan pool after the bursts, and how often a request
                 # had to wait for the oldest user of one since the counters were last reset
-                plan_memory={k: st[k] for k in ("plan_slots", "plan_slots_in_use", "plan_slot_waits")})
+                plan_memory={k: st[k] for k in ("plan_slots", "plan_slots_in_use", "plan_slot_waits")},
+                # the 64 threads do not get to their calls at once: the interpreter hands its
+                # lock from thread to thread.  Milliseconds after the start of a burst at which
+                # half, nine tenths and all of them had made their call (medians over bursts).
+                call_starts_ms={"half": round(_median([s[len(s) // 2] for s in starts]), 2),
+                                "nine_tenths": round(_median([s[len(s) * 9 // 10] for s in starts]), 2),
+                                "all": round(_median([s[-1] for s in starts]), 2)})
 
 
 def run_groups(torch, device, num_cta, reps=30):
@@ -1356,7 +1367,7 @@ def measure_config(name, args, torch, device, link, steps, warmup):
                    total_blocks=sum(r["blocks"]), aggregate_bytes=r["total_bytes"],
                    p50_latency_ms=round(r["p50_ms"], 3), p99_latency_ms=round(r["p99_ms"], 3),
                    burst_ms=[round(x * 1e3, 2) for x in r["walls"]],   # every timed burst
-                   plan_memory=r["plan_memory"],
+                   plan_memory=r["plan_memory"], call_starts_ms=r["call_starts_ms"],
                    bidir_link_peak_GBps=round(bidir, 3), frac_of_bidir_link=round(agg / bidir, 4),
                    frac_of_sum_of_one_way_peaks=round(agg / (link["d2h"] + link["h2d"]), 4))
     del w
@@ -1682,12 +1693,12 @@ def main():
     head = "c1"
     records = {}
     if not args.sequence:
-        # c4 first: its 64 requests share the link between the directions, and that balance is
-        # the one figure here that depends on what the process has done before (93 GB/s in a
-        # fresh process or after any one other configuration, 85-90 GB/s at the end of the whole
-        # sequence, where one direction finishes its requests 20-30 ms before the other; the
-        # one-direction figures do not move with the order).  `--sequence ...,c4` measures it
-        # behind configurations of choice.
+        # c4 first (it used to be the one figure that moved with its place in the run: 64
+        # waiting threads kept 13 of the box's 16 cores busy inside the runtime's waits, the
+        # threads that still had to submit their request got to it up to 50 ms late, and how
+        # late depended on what the process had done before; the library now lets only two
+        # waiters wait that way).  `--sequence ...,c4` measures it behind configurations of
+        # choice.
         records["c4"] = measure_config("c4", args, torch, device, link, 20, 1)
         records["c4"]["position_in_run"] = "first"
     records[head] = measure_config(head, args, torch, device, link, args.steps, args.warmup)

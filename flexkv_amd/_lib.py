@@ -211,7 +211,7 @@ class LaunchPolicy(Structure):
                 ("model_seed", c_int32), ("model_seeded", c_int32),
                 ("staged_scatter_threads", c_int32), ("test_fail_restore_batch", c_int32),
                 ("staged_dma_streams", c_int32), ("kernel_alt_stream_kb", c_int32),
-                ("reserved", c_int32 * 1)]
+                ("quiet_wait_us", c_int32)]
 
 
 # name -> (restype, argtypes); the complete export list of include/fkv_transfer.h

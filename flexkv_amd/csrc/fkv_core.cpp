@@ -13,6 +13,7 @@
 #include <cstring>
 #include <memory>
 #include <mutex>
+#include <thread>
 
 namespace fkv {
 
@@ -77,6 +78,75 @@ DeviceGuard::DeviceGuard(int device) : device_(device) {
 DeviceGuard::~DeviceGuard() {
   if (switched_)
     (void)hipSetDevice(prev_);
+}
+
+// ---- waits that leave the cores alone ------------------------------------------
+namespace {
+// Threads of the process that are waiting for device work inside the library right now.
+std::atomic<int> g_waiting{0};
+struct Waiting {
+  int others; // that were waiting already when this one came
+  Waiting() : others(g_waiting.fetch_add(1, std::memory_order_relaxed)) {}
+  ~Waiting() { g_waiting.fetch_sub(1, std::memory_order_relaxed); }
+};
+// As many waits as this may use the runtime's own, which returns soonest and costs a core
+// each: a worker that waits for one transfer at a time loses nothing, and a process with 64
+// requests in flight keeps two cores busy instead of thirteen.
+constexpr int kRuntimeWaits = 2;
+} // namespace
+
+hipError_t quiet_event_wait(hipEvent_t event, int device, int64_t expected_ns) {
+  const int limit_us = policy_peek(device).quiet_wait_us;
+  Waiting here;
+  if (limit_us <= 0 || here.others < kRuntimeWaits)
+    return hipEventSynchronize(event);
+  using clock = std::chrono::steady_clock;
+  const auto t0 = clock::now();
+  // Where the work is expected to end: sleep up to shortly before that, look closely around
+  // it, and fall back to longer and longer sleeps when it takes longer (work of others
+  // queued ahead, traffic the other way).
+  constexpr int64_t kCloseNs = 80 * 1000;
+  const auto close_from = t0 + std::chrono::nanoseconds(std::max<int64_t>(0, expected_ns - kCloseNs));
+  const auto close_until = t0 + std::chrono::nanoseconds(std::max<int64_t>(30 * 1000, expected_ns + kCloseNs));
+  int nap_us = 20;
+  for (;;) {
+    const hipError_t q = hipEventQuery(event);
+    if (q != hipErrorNotReady)
+      return q;
+    (void)hipGetLastError(); // "not ready" is no error of the caller's
+    const auto now = clock::now();
+    if (now < close_from) {
+      std::this_thread::sleep_for((close_from - now) / 2 + std::chrono::microseconds(10));
+    } else if (now < close_until) {
+      // spinning: the end is near
+    } else {
+      std::this_thread::sleep_for(std::chrono::microseconds(nap_us));
+      nap_us = std::min(nap_us * 2, limit_us);
+    }
+  }
+}
+
+hipError_t quiet_stream_wait(hipStream_t stream, int device) {
+  constexpr int kMaxDevices = 64;
+  if (device < 0 || device >= kMaxDevices || policy_peek(device).quiet_wait_us <= 0 ||
+      g_waiting.load(std::memory_order_relaxed) < kRuntimeWaits) {
+    Waiting here;
+    return hipStreamSynchronize(stream);
+  }
+  // one event per thread and device; with the system-scope fence, since the host may read
+  // what the stream wrote
+  thread_local hipEvent_t mine[kMaxDevices] = {};
+  hipEvent_t &ev = mine[device];
+  if (!ev && hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+    (void)hipGetLastError();
+    ev = nullptr;
+    return hipStreamSynchronize(stream);
+  }
+  if (hipEventRecord(ev, stream) != hipSuccess) {
+    (void)hipGetLastError();
+    return hipStreamSynchronize(stream);
+  }
+  return quiet_event_wait(ev, device, 0);
 }
 
 // ---- pooled streams ---------------------------------------------------------
@@ -1099,10 +1169,14 @@ int transfer_descs(const fkv_transfer_desc *descs, int count, hipStream_t stream
 
   if (sync) {
     auto t0 = std::chrono::steady_clock::now();
+    // alone on the link the transfer takes bytes / link rate (the policy's figure, re-based on
+    // a measurement of the device where one has been made; 3 % taken off)
+    const int64_t expected_ns =
+        (int64_t)((double)bytes * 1000.0 / std::max(1, policy_peek(device).model_link_mbps) * 0.97);
     if (done)
-      FKV_HIP_TRY(hipEventSynchronize(done));
+      FKV_HIP_TRY(quiet_event_wait(done, device, expected_ns));
     else
-      FKV_HIP_TRY(hipStreamSynchronize(stream));
+      FKV_HIP_TRY(quiet_stream_wait(stream, device));
     if (trace) {
       double ms = std::chrono::duration<double, std::milli>(
                       std::chrono::steady_clock::now() - t0)

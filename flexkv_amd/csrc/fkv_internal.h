@@ -25,6 +25,17 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 // be current.
 hipError_t pooled_stream_acquire(int device, bool non_blocking, hipStream_t *out);
 void pooled_stream_release(int device, bool non_blocking, hipStream_t stream);
+// Waits of the host for device work.  The runtime's own (hipEventSynchronize,
+// hipStreamSynchronize, also on events made for blocking waits) keep a core busy for as long
+// as they last; these poll instead when quiet_wait_us of the device's launch policy says so
+// and two threads of the process are already waiting the runtime's way:
+// a spin of 30 us for work that is nearly done, then sleeps that double from 20 us up to
+// that limit; with `expected_ns` (how long the work takes when nothing else holds it up, 0 =
+// unknown) the thread sleeps towards that moment first and spins for the 80 us either side of
+// it.  `event` must have been recorded.  The stream form records an event of the calling
+// thread behind what the stream holds and waits for that.
+hipError_t quiet_event_wait(hipEvent_t event, int device, int64_t expected_ns = 0);
+hipError_t quiet_stream_wait(hipStream_t stream, int device);
 // For the catch-all handler of an entry point: turns the exception in flight into a status
 // and an error text.  No C++ exception crosses the C ABI.
 int caught(const char *where) noexcept;

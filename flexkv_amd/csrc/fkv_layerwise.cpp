@@ -1091,7 +1091,7 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
         return launch_failure();
       for (int i = 0; i < g->num_gpus; ++i) {
         (void)hipSetDevice(g->device_ids[i]);
-        hipError_t e = hipEventSynchronize(g->batches[b]->done[i]);
+        hipError_t e = quiet_event_wait(g->batches[b]->done[i], g->device_ids[i], 0);
         if (e != hipSuccess) {
           (void)hipGetLastError();
           (void)hipSetDevice(restore.device());
@@ -1104,7 +1104,7 @@ int fkv_layerwise_transfer_call(fkv_layerwise *g, const fkv_layerwise_call *call
     g->join_feeder();
     for (int i = 0; i < g->num_gpus; ++i) { // csrc/layerwise.cpp:1249-1256, 1634-1642
       (void)hipSetDevice(g->device_ids[i]);
-      hipError_t e = hipStreamSynchronize(g->streams[i]);
+      hipError_t e = quiet_stream_wait(g->streams[i], g->device_ids[i]);
       if (e != hipSuccess) {
         (void)hipGetLastError();
         (void)hipSetDevice(restore.device());
@@ -1331,7 +1331,7 @@ int fkv_layerwise_synchronize(fkv_layerwise *g) try {
   DeviceGuard restore(-1);
   for (int i = 0; i < g->num_gpus; ++i) {
     FKV_HIP_TRY(hipSetDevice(g->device_ids[i]));
-    FKV_HIP_TRY(hipStreamSynchronize(g->streams[i]));
+    FKV_HIP_TRY(quiet_stream_wait(g->streams[i], g->device_ids[i]));
   }
   (void)hipSetDevice(restore.device());
   return g->take_restore_error("fkv_layerwise_synchronize");

@@ -40,6 +40,7 @@ const EnvField kEnv[] = {
     FKV_FIELD("FKV_STAGED_GATHER", staged_gather),
     FKV_FIELD("FKV_GATHER_THREADS", gather_threads),
     FKV_FIELD("FKV_MODEL_SEED", model_seed),
+    FKV_FIELD("FKV_QUIET_WAIT_US", quiet_wait_us),
 };
 #undef FKV_FIELD
 
@@ -170,6 +171,7 @@ void sanitize(fkv_launch_policy &p, const fkv_launch_policy &derived) {
   p.test_fail_restore_batch = clampi(p.test_fail_restore_batch, 0, 1 << 20);
   p.staged_dma_streams = clampi(p.staged_dma_streams, 1, 2);
   p.kernel_alt_stream_kb = clampi(p.kernel_alt_stream_kb, 0, 1 << 20);
+  p.quiet_wait_us = clampi(p.quiet_wait_us, 0, 10000);
 }
 
 // The table of a device with the XCDs `present`, environment applied.
@@ -239,6 +241,7 @@ fkv_launch_policy defaults_for(uint32_t present) {
   p.staged_scatter_threads = 256;
   p.staged_dma_streams = 2;
   p.kernel_alt_stream_kb = 4096;
+  p.quiet_wait_us = 100;
   for (const EnvField &f : kEnv) {
     const char *v = std::getenv(f.name);
     if (v && *v) // decimal, 0x.. or 0.. as written

@@ -242,7 +242,7 @@ int fkv_tp_group_update_gpu_block_ptrs(fkv_tp_group *g, const uint64_t *ptrs, in
   DeviceGuard restore(-1);
   for (int i = 0; i < g->num_gpus; ++i) { // no transfer may still read the old table
     FKV_HIP_TRY(hipSetDevice(g->device_ids[i]));
-    FKV_HIP_TRY(hipStreamSynchronize(g->streams[i]));
+    FKV_HIP_TRY(fkv::quiet_stream_wait(g->streams[i], g->device_ids[i]));
   }
   (void)hipSetDevice(restore.device());
   g->gpu_ptrs.assign(ptrs, ptrs + count);

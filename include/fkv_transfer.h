@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define FKV_ABI_VERSION 5 /* 5: fkv_stats grew by plan_slots, plan_slots_in_use and plan_slot_waits; 4: fkv_stats grew by second_stream_batches; 3: fkv_stats grew by gathered_batches and gather_busy_us, fkv_launch_policy by the host-gather and link-seeding fields; 2: fkv_stats grew by staged_batches; launch policy, no-alloc transfer, staging and HBM-rate entry points added */
+#define FKV_ABI_VERSION 5 /* 5: fkv_stats grew by plan_slots, plan_slots_in_use and plan_slot_waits, the last reserved slot of fkv_launch_policy became quiet_wait_us; 4: fkv_stats grew by second_stream_batches; 3: fkv_stats grew by gathered_batches and gather_busy_us, fkv_launch_policy by the host-gather and link-seeding fields; 2: fkv_stats grew by staged_batches; launch policy, no-alloc transfer, staging and HBM-rate entry points added */
 
 /* status codes */
 #define FKV_OK 0
@@ -796,7 +796,19 @@ typedef struct fkv_launch_policy {
                                  on one stream lie 8 us apart, next to 18 us of link time for
                                  1 MiB); events, notifications and wait_layer stay per batch and
                                  in order.  Default 4096; 0 = one stream */
-  int32_t reserved[1];
+  int32_t quiet_wait_us;        /* how a call waits for its transfer (sync = 1, the thread group, the
+                                 layerwise restore in HOSTFUNC mode, fkv_layerwise_synchronize): the
+                                 runtime's own waits keep a core busy for as long as they last (a
+                                 synchronous 9 ms transfer costs 9 ms of CPU time, 64 waiting
+                                 requests 13 of 16 cores, and the threads that still have to submit
+                                 theirs wait for a core).  > 0 (default 100): while two threads of the
+                                 process are already waiting the runtime's way, further ones poll
+                                 their event instead: they sleep towards the moment the transfer
+                                 would end alone on the link, spin for the 80 us around it, and
+                                 after that sleep for spells that double from 20 us up to this many
+                                 microseconds (2 % of a core each; such a wait ends up to that much
+                                 later).  A caller that waits for one transfer at a time sees no
+                                 difference.  0 = always the runtime's wait */
 } fkv_launch_policy;
 /* The table of `device` (-1 = current).  The first call for a device runs the probe kernel. */
 int fkv_launch_policy_get(int32_t device, fkv_launch_policy *out);
