@@ -89,3 +89,44 @@ def test_first_launches_of_a_fresh_process(gpu_device, dirty):
         r = subprocess.run([sys.executable, "-c", script, root], capture_output=True, text=True,
                            timeout=170, env=env)
         assert r.returncode == 0 and r.stdout.split()[-1:] == ["ok"], r.stdout + r.stderr
+
+
+def test_waiting_requests_leave_the_cores_alone(gpu_device):
+    """The runtime's waits keep a core busy each.  With eight threads waiting for their
+    synchronous transfers at once the library lets two of them wait that way and the others
+    poll with sleeps: the process uses well under half of the eight cores it would otherwise
+    (with quiet_wait_us = 0, the runtime's wait for everybody, it uses most of them: printed,
+    the box decides).  The bytes are checked against the oracle afterwards."""
+    from flexkv_amd.c_ext import launch_policy
+    threads, per, rounds = 8, 64, 12
+    s = KVSetup(VLLM, 4, 2, threads * per, threads * per, 65536, "BLOCKFIRST", seed=5)
+    dev = s.to_device(gpu_device)
+    ids = [np.arange(t * per, (t + 1) * per, dtype=np.int64) for t in range(threads)]
+
+    def burst(h2d):
+        barrier = threading.Barrier(threads + 1)
+
+        def work(t):
+            st = torch.cuda.Stream()
+            with torch.cuda.stream(st):
+                barrier.wait()
+                for _ in range(rounds):
+                    dev.transfer(ids[t], ids[t], is_h2d=h2d, sync=True)
+        workers = [threading.Thread(target=work, args=(t,)) for t in range(threads)]
+        [w.start() for w in workers]
+        barrier.wait()
+        cpu0, t0 = time.process_time(), time.perf_counter()
+        [w.join() for w in workers]
+        return (time.process_time() - cpu0) / (time.perf_counter() - t0)
+
+    burst(False)                                   # streams, plans, lanes
+    cores = max(burst(False), burst(True))
+    with launch_policy(quiet_wait_us=0):
+        spinning = max(burst(False), burst(True))
+    print("cores busy with eight waiting threads: %.1f, with the runtime's wait for all: %.1f"
+          % (cores, spinning))
+    assert cores < 4.0, (cores, spinning)
+    for t in range(threads):
+        s.oracle_transfer(ids[t], ids[t], False)
+        s.oracle_transfer(ids[t], ids[t], True)
+    dev.assert_matches_reference("eight threads of synchronous transfers")
