@@ -537,6 +537,7 @@ def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, v
         torch.cuda.synchronize()
 
     starts = []     # per timed burst: when each request thread got to its call, sorted
+    cores = []      # per timed burst: CPU time of the process / wall time
 
     def worker(i, barrier, record, began):
         gi, ci = reqs[i]
@@ -558,10 +559,12 @@ def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, v
         torch.cuda.synchronize()
         barrier.wait()
         t0 = time.perf_counter()
+        cpu0 = time.process_time()
         for th in threads:
             th.join()
         if it >= warmup:
             walls.append(time.perf_counter() - t0)
+            cores.append((time.process_time() - cpu0) / walls[-1])
             starts.append(sorted((b - t0) * 1e3 for b in began))
     all_lat = sorted(x for l in lat for x in l)
     p99 = all_lat[min(len(all_lat) - 1, int(0.99 * len(all_lat)))]
@@ -583,6 +586,7 @@ def run_concurrent(w, torch, steps, warmup, num_cta, streams_per_direction=32, v
                 # the 64 threads do not get to their calls at once: the interpreter hands its
                 # lock from thread to thread.  Milliseconds after the start of a burst at which
                 # half, nine tenths and all of them had made their call (medians over bursts).
+                host_cores_busy=round(_median(cores), 2),   # of the whole process, during a burst
                 call_starts_ms={"half": round(_median([s[len(s) // 2] for s in starts]), 2),
                                 "nine_tenths": round(_median([s[len(s) * 9 // 10] for s in starts]), 2),
                                 "all": round(_median([s[-1] for s in starts]), 2)})
@@ -1368,6 +1372,7 @@ def measure_config(name, args, torch, device, link, steps, warmup):
                    p50_latency_ms=round(r["p50_ms"], 3), p99_latency_ms=round(r["p99_ms"], 3),
                    burst_ms=[round(x * 1e3, 2) for x in r["walls"]],   # every timed burst
                    plan_memory=r["plan_memory"], call_starts_ms=r["call_starts_ms"],
+                   host_cores_busy=r["host_cores_busy"],
                    bidir_link_peak_GBps=round(bidir, 3), frac_of_bidir_link=round(agg / bidir, 4),
                    frac_of_sum_of_one_way_peaks=round(agg / (link["d2h"] + link["h2d"]), 4))
     del w
