@@ -96,9 +96,10 @@ constexpr int kRuntimeWaits = 2;
 } // namespace
 
 hipError_t quiet_event_wait(hipEvent_t event, int device, int64_t expected_ns) {
-  const int limit_us = policy_peek(device).quiet_wait_us;
+  const int setting = policy_peek(device).quiet_wait_us;
+  const int limit_us = setting < 0 ? -setting : setting;
   Waiting here;
-  if (limit_us <= 0 || here.others < kRuntimeWaits)
+  if (setting == 0 || (setting > 0 && here.others < kRuntimeWaits))
     return hipEventSynchronize(event);
   using clock = std::chrono::steady_clock;
   const auto t0 = clock::now();
@@ -128,8 +129,8 @@ hipError_t quiet_event_wait(hipEvent_t event, int device, int64_t expected_ns) {
 
 hipError_t quiet_stream_wait(hipStream_t stream, int device) {
   constexpr int kMaxDevices = 64;
-  if (device < 0 || device >= kMaxDevices || policy_peek(device).quiet_wait_us <= 0 ||
-      g_waiting.load(std::memory_order_relaxed) < kRuntimeWaits) {
+  const int setting = device < 0 || device >= kMaxDevices ? 0 : policy_peek(device).quiet_wait_us;
+  if (setting == 0 || (setting > 0 && g_waiting.load(std::memory_order_relaxed) < kRuntimeWaits)) {
     Waiting here;
     return hipStreamSynchronize(stream);
   }

@@ -171,7 +171,7 @@ void sanitize(fkv_launch_policy &p, const fkv_launch_policy &derived) {
   p.test_fail_restore_batch = clampi(p.test_fail_restore_batch, 0, 1 << 20);
   p.staged_dma_streams = clampi(p.staged_dma_streams, 1, 2);
   p.kernel_alt_stream_kb = clampi(p.kernel_alt_stream_kb, 0, 1 << 20);
-  p.quiet_wait_us = clampi(p.quiet_wait_us, 0, 10000);
+  p.quiet_wait_us = clampi(p.quiet_wait_us, -10000, 10000);
 }
 
 // The table of a device with the XCDs `present`, environment applied.

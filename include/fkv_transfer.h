@@ -808,7 +808,10 @@ typedef struct fkv_launch_policy {
                                  after that sleep for spells that double from 20 us up to this many
                                  microseconds (2 % of a core each; such a wait ends up to that much
                                  later).  A caller that waits for one transfer at a time sees no
-                                 difference.  0 = always the runtime's wait */
+                                 difference.  < 0: every waiting thread polls, with -value as the
+                                 limit (a worker then costs 2 % of a core while it waits instead of a
+                                 whole one, and its 9.4 ms op ends up to 0.1 ms later).  0 = always
+                                 the runtime's wait */
 } fkv_launch_policy;
 /* The table of `device` (-1 = current).  The first call for a device runs the probe kernel. */
 int fkv_launch_policy_get(int32_t device, fkv_launch_policy *out);

@@ -126,6 +126,16 @@ def test_waiting_requests_leave_the_cores_alone(gpu_device):
     print("cores busy with eight waiting threads: %.1f, with the runtime's wait for all: %.1f"
           % (cores, spinning))
     assert cores < 4.0, (cores, spinning)
+    # a negative setting makes every waiter poll: one thread waiting for its transfers then
+    # leaves its core alone too
+    with launch_policy(quiet_wait_us=-100):
+        cpu0, t0 = time.process_time(), time.perf_counter()
+        for _ in range(40):
+            dev.transfer(np.arange(threads * per, dtype=np.int64),
+                         np.arange(threads * per, dtype=np.int64), is_h2d=False, sync=True)
+        alone = (time.process_time() - cpu0) / (time.perf_counter() - t0)
+    print("one waiting thread, every waiter polling: %.2f cores" % alone)
+    assert alone < 0.6, alone
     for t in range(threads):
         s.oracle_transfer(ids[t], ids[t], False)
         s.oracle_transfer(ids[t], ids[t], True)
