@@ -93,13 +93,17 @@ struct Waiting {
 // each: a worker that waits for one transfer at a time loses nothing, and a process with 64
 // requests in flight keeps two cores busy instead of thirteen.
 constexpr int kRuntimeWaits = 2;
+// ... unless the work is known to take this long: polling then costs a few parts in a
+// thousand (a sleep towards the expected end, a spin of at most 160 us around it), and a
+// transfer of gigabytes no longer holds a core for its whole length.
+constexpr int64_t kLongWaitNs = 20 * 1000 * 1000;
 } // namespace
 
 hipError_t quiet_event_wait(hipEvent_t event, int device, int64_t expected_ns) {
   const int setting = policy_peek(device).quiet_wait_us;
   const int limit_us = setting < 0 ? -setting : setting;
   Waiting here;
-  if (setting == 0 || (setting > 0 && here.others < kRuntimeWaits))
+  if (setting == 0 || (setting > 0 && here.others < kRuntimeWaits && expected_ns < kLongWaitNs))
     return hipEventSynchronize(event);
   using clock = std::chrono::steady_clock;
   const auto t0 = clock::now();

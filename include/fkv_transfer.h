@@ -808,7 +808,9 @@ typedef struct fkv_launch_policy {
                                  after that sleep for spells that double from 20 us up to this many
                                  microseconds (2 % of a core each; such a wait ends up to that much
                                  later).  A caller that waits for one transfer at a time sees no
-                                 difference.  < 0: every waiting thread polls, with -value as the
+                                 difference, except that a transfer expected to take 20 ms or more
+                                 (1.1 GB) is polled for as well, at a cost of a few parts in a
+                                 thousand.  < 0: every waiting thread polls, with -value as the
                                  limit (a worker then costs 2 % of a core while it waits instead of a
                                  whole one, and its 9.4 ms op ends up to 0.1 ms later).  0 = always
                                  the runtime's wait */
