@@ -121,7 +121,10 @@ hipError_t quiet_event_wait(hipEvent_t event, int device, int64_t expected_ns) {
     (void)hipGetLastError(); // "not ready" is no error of the caller's
     const auto now = clock::now();
     if (now < close_from) {
-      std::this_thread::sleep_for((close_from - now) / 2 + std::chrono::microseconds(10));
+      // never long at a stretch: a core that has slept for tens of milliseconds can take
+      // milliseconds to come back (seen on a virtual machine: +2 to +5 ms on a 188 ms wait)
+      std::this_thread::sleep_for(std::min<clock::duration>(
+          (close_from - now) / 2 + std::chrono::microseconds(10), std::chrono::milliseconds(1)));
     } else if (now < close_until) {
       // spinning: the end is near
     } else {

@@ -31,8 +31,8 @@ void pooled_stream_release(int device, bool non_blocking, hipStream_t stream);
 // and two threads of the process are already waiting the runtime's way:
 // a spin of 30 us for work that is nearly done, then sleeps that double from 20 us up to
 // that limit; with `expected_ns` (how long the work takes when nothing else holds it up, 0 =
-// unknown) the thread sleeps towards that moment first and spins for the 80 us either side of
-// it.  `event` must have been recorded.  The stream form records an event of the calling
+// unknown) the thread sleeps towards that moment first, a millisecond at a time at most, and
+// spins for the 80 us either side of it.  `event` must have been recorded.  The stream form records an event of the calling
 // thread behind what the stream holds and waits for that.
 hipError_t quiet_event_wait(hipEvent_t event, int device, int64_t expected_ns = 0);
 hipError_t quiet_stream_wait(hipStream_t stream, int device);
