@@ -26,6 +26,9 @@ Beyond those (the callers and formats either side of the path):
   worker  c0-shaped put/get ops through a transfer worker process (pipe + shared op pool)
   groups  whole-block ops of a model with three layer groups: one call per group against
           one call for all; chunk sizes that are no whole number of slices
+Studies: --sequence CFG,CFG,... measures configurations of choice one behind the other in one
+process (what one leaves behind for the next), --policy FIELD=VALUE sets a field of the
+library's launch policy first, --hw-queues N the hardware queues of the process.
 """
 from __future__ import annotations
 
